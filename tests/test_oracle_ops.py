@@ -1,0 +1,334 @@
+"""Pins the oracle's operators: the reference tests' own known-answer vectors, an
+independent numpy formulation (explicit zero-point padding + window view), the
+zero-point fold form the GPU kernels use, and structural invariants."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
+UNIT = dict(multiplier=1 << 30, shift=1)  # real multiplier 1.0
+
+
+def np_requant(acc, q):
+    """Vectorised exact requant in Python integers (independent of the C code)."""
+    out = np.empty(acc.shape, np.uint8)
+    flat, o = acc.reshape(-1).tolist(), out.reshape(-1)
+    ls, rs = max(q.shift, 0), max(-q.shift, 0)
+    for i, a in enumerate(flat):
+        x = a << ls
+        p = x * q.multiplier
+        v = (p + (1 << 30)) >> 31                     # round half up
+        half = (1 << rs) >> 1
+        r = (abs(v) + half) >> rs if rs else abs(v)   # round half away from zero
+        r = -r if v < 0 else r
+        o[i] = min(max(r + q.zp_out, q.act_min), q.act_max)
+    return out
+
+
+def np_conv_acc(x, w, bias, s, zp_in, zp_w):
+    """Pads with zp_in, builds windows, contracts in int64. NCHW, groups supported."""
+    xp = np.pad(x.astype(np.int64), ((0, 0), (0, 0), (s.pad_t, s.pad_b), (s.pad_l, s.pad_r)), constant_values=zp_in) - zp_in
+    wz = w.astype(np.int64) - zp_w
+    ho, wo = O.conv_out_hw(s)
+    g, cig, cog = s.groups, s.c // s.groups, s.cout // s.groups
+    acc = np.zeros((s.n, s.cout, ho, wo), np.int64)
+    for ky in range(s.kh):
+        for kx in range(s.kw):
+            y0, x0 = ky * s.dil_h, kx * s.dil_w
+            win = xp[:, :, y0:y0 + (ho - 1) * s.stride_h + 1:s.stride_h, x0:x0 + (wo - 1) * s.stride_w + 1:s.stride_w]
+            for gi in range(g):
+                acc[:, gi * cog:(gi + 1) * cog] += np.einsum(
+                    "nchw,oc->nohw", win[:, gi * cig:(gi + 1) * cig], wz[gi * cog:(gi + 1) * cog, :, ky, kx])
+    return (acc + bias.astype(np.int64)[None, :, None, None]).astype(np.int32)
+
+
+def rand_case(rng, n, c, h, w, cout, kh, kw, **kw_):
+    s = O.conv_shape(n, c, h, w, cout, kh, kw, **kw_)
+    x = rng.integers(0, 256, (n, c, h, w), dtype=np.uint8)
+    wt = rng.integers(0, 256, (cout, c // s.groups, kh, kw), dtype=np.uint8)
+    b = rng.integers(-1000, 1001, cout).astype(np.int32)
+    return s, x, wt, b
+
+
+# --------------------------------------------------------------------- KATs
+
+@pytest.mark.parametrize("kat", KATS["conv"], ids=lambda k: k["name"])
+def test_conv_reference_kat(kat):
+    n, h, w, c = kat["in_dims"]
+    cout, kh, kw, _ = kat["w_dims"]
+    x = np.array(kat["input"], np.uint8).reshape(n, h, w, c).transpose(0, 3, 1, 2)
+    wt = np.array(kat["weight"], np.uint8).reshape(cout, kh, kw, c).transpose(0, 3, 1, 2)
+    bias = np.array(kat["bias"], np.int32)
+    t, b, l, r = kat["pad_tblr"]
+    s = O.conv_shape(n, c, h, w, cout, kh, kw, stride=tuple(kat["stride"]), pad=(t, b, l, r))
+    q = O.raw_quant(**UNIT)
+    if kat["relu"]:
+        q.act_min, q.act_max = O.act_range_u8(O.ACT_RELU, 1.0, 0)
+    out = O.conv2d(x, wt, bias, s, q)
+    on, oh, ow, oc = kat["out_dims"]
+    want = np.clip(np.array(kat["expect"]).reshape(on, oh, ow, oc).transpose(0, 3, 1, 2), 0, 255)
+    assert np.array_equal(out, want.astype(np.uint8))
+    # halve the multiplier: every non-negative expected value e becomes (e+1)//2, unsaturated for e <= 510
+    qh = O.raw_quant(multiplier=1 << 30, shift=0, act_min=q.act_min, act_max=q.act_max)
+    e = np.array(kat["expect"]).reshape(on, oh, ow, oc).transpose(0, 3, 1, 2)
+    half = np.sign(e) * ((np.abs(e) + 1) // 2)
+    assert np.array_equal(O.conv2d(x, wt, bias, s, qh), np.clip(half, q.act_min, 255).astype(np.uint8))
+
+
+def test_conv_perchannel_u8_kat():
+    k = KATS["conv_perchannel_u8"]
+    n, c, h, w = k["in_dims_nchw"]
+    cout, kh, kw, cin = k["w_dims_ohwi"]
+    x = np.array(k["input"], np.uint8).reshape(n, c, h, w)
+    wt = np.array(k["weight_i8"], np.int8).reshape(cout, kh, kw, cin).transpose(0, 3, 1, 2)
+    mults, shifts = [], []
+    for ws in k["w_scales"]:
+        m = float(np.float32(k["in_scale"])) * float(np.float32(ws)) / float(np.float32(k["out_scale"]))
+        qm, sh = O.quantize_multiplier(m)
+        mults.append(qm)
+        shifts.append(sh)
+    s = O.conv_shape(n, c, h, w, cout, kh, kw)
+    q = O.raw_quant(zp_in=k["in_zp"], zp_w=0, zp_out=k["out_zp"])
+    out = O.conv2d_perchannel(x, wt, np.array(k["bias"], np.int32), s, q, mults, shifts)
+    assert out.reshape(-1).tolist() == k["expect"]
+
+
+def test_relu_u8_kat():
+    """A quantized ReLU is a clamp at the zero point: values below zp come out as zp."""
+    k = KATS["relu_u8"]
+    lo, hi = O.act_range_u8(O.ACT_RELU, 1.0, k["zp"])
+    q = O.raw_quant(zp_in=k["zp"], zp_w=0, zp_out=k["zp"], act_min=lo, act_max=hi, **UNIT)
+    x = np.array(k["input"], np.uint8).reshape(1, 1, 1, 4)
+    one = np.array([1], np.uint8).reshape(1, 1, 1, 1)
+    out = O.conv2d(x, one, np.zeros(1, np.int32), O.conv_shape(1, 1, 1, 4, 1, 1, 1), q)
+    assert out.reshape(-1).tolist() == k["expect"]
+
+
+@pytest.mark.parametrize("kat", KATS["depthwise"], ids=lambda k: k["name"])
+def test_depthwise_reference_kat(kat):
+    n, c, h, w = kat["in_dims"]
+    cout, _, kh, kw = kat["w_dims"]
+    zp_w, zp_out = 16, 40  # weights go down to -16, outputs down to -36
+    x = np.array(kat["input"], np.uint8).reshape(n, c, h, w)
+    wt = (np.array(kat["weight"]) + zp_w).astype(np.uint8).reshape(cout, 1, kh, kw)
+    s = O.conv_shape(n, c, h, w, cout, kh, kw, stride=tuple(kat["stride"]), dm=kat["dm"])
+    q = O.raw_quant(zp_w=zp_w, zp_out=zp_out, **UNIT)
+    out, acc = O.dwconv2d(x, wt, np.array(kat["bias"], np.int32), s, q, want_acc=True)
+    assert list(out.shape) == kat["out_dims"]
+    assert acc.reshape(-1).tolist() == kat["expect"]
+    assert out.reshape(-1).tolist() == [e + zp_out for e in kat["expect"]]
+    # same vector with zp_out = 0: negatives clamp to 0
+    q0 = O.raw_quant(zp_w=zp_w, **UNIT)
+    assert O.dwconv2d(x, wt, np.array(kat["bias"], np.int32), s, q0).reshape(-1).tolist() == [max(e, 0) for e in kat["expect"]]
+
+
+@pytest.mark.parametrize("kat", KATS["fc"], ids=lambda k: k["name"])
+def test_fc_reference_kat(kat):
+    zp_a = 10  # inputs go down to -10
+    a = (np.array(kat["input"]) + zp_a).astype(np.uint8).reshape(kat["m"], kat["k"])
+    w = np.array(kat["weight"], np.uint8).reshape(kat["n"], kat["k"])
+    q = O.raw_quant(zp_in=zp_a, **UNIT)
+    out = O.fc(a, w, np.array(kat["bias"], np.int32), q)
+    assert out.reshape(-1).tolist() == kat["expect"]
+
+
+@pytest.mark.parametrize("kat", KATS["deconv_float"], ids=lambda k: k["name"])
+def test_deconv_index_math_reference_float_kat(kat):
+    n, c, h, w = kat["in_dims"]
+    cin, cog, kh, kw = kat["w_dims"]
+    g = kat["groups"]
+    t, r, b, l = kat["pad_trbl"]
+    s = O.conv_shape(n, c, h, w, cog * g, kh, kw, stride=tuple(kat["stride"]), pad=(t, b, l, r), groups=g)
+    assert cin == c
+    out = O.deconv2d_f64(np.array(kat["input"]).reshape(n, c, h, w), np.array(kat["weight"]).reshape(cin, cog, kh, kw),
+                         np.array(kat["bias"]), s)
+    assert list(out.shape) == kat["out_dims"]
+    # the reference compares at 1e-4 absolute (deconvolution_test.cpp:24); its data carries six digits
+    assert np.max(np.abs(out.reshape(-1) - np.array(kat["expect"]))) < 1e-4
+
+
+# ------------------------------------------------ independent formulations
+
+CONV_CASES = [
+    dict(n=2, c=3, h=7, w=9, cout=5, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=4, h=8, w=8, cout=6, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),
+    dict(n=1, c=6, h=9, w=7, cout=4, kh=3, kw=2, dil=(2, 1), pad=(2, 2, 0, 1), groups=2),
+    dict(n=3, c=8, h=5, w=5, cout=8, kh=1, kw=1),
+    dict(n=1, c=2, h=6, w=6, cout=3, kh=5, kw=5, pad=(2, 2, 2, 2), stride=(1, 2)),
+    dict(n=1, c=1, h=3, w=3, cout=1, kh=3, kw=3, pad=(3, 3, 3, 3)),  # windows that lie wholly in the padding
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_conv_vs_numpy_windows_and_fold_form(case):
+    rng = np.random.default_rng(11)
+    s, x, wt, b = rand_case(rng, **case)
+    zp_in, zp_w = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+    q = O.make_quant(0.02, zp_in, 0.005, zp_w, 0.05, int(rng.integers(0, 256)), O.ACT_RELU6, True)
+    out, acc = O.conv2d(x, wt, b, s, q, want_acc=True)
+    want_acc = np_conv_acc(x, wt, b, s, zp_in, zp_w)
+    assert np.array_equal(acc, want_acc)
+    assert np.array_equal(out, np_requant(want_acc, q))
+    # fold form used by the GPU kernels (groups == 1 only): with a' = a-128, w' = w-128,
+    # za = zp_in-128, zw = zp_w-128 and padding filled with za:
+    # sum (a-zp_in)(w-zp_w) = sum a'w' - zw*sum_k a' - za*sum_k w' + K*za*zw
+    if s.groups == 1:
+        za, zw = zp_in - 128, zp_w - 128
+        s0 = O.conv_shape(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, stride=(s.stride_h, s.stride_w),
+                          pad=(s.pad_t, s.pad_b, s.pad_l, s.pad_r), dil=(s.dil_h, s.dil_w))
+        zero_b = np.zeros(s.cout, np.int32)
+        xs, ws = x.astype(np.int64) - 128, wt.astype(np.int64) - 128
+        # np_conv_acc with "zero points" za/0 on pre-shifted data gives sum a'w' with za-filled padding
+        xp = np.pad(xs, ((0, 0), (0, 0), (s.pad_t, s.pad_b), (s.pad_l, s.pad_r)), constant_values=za)
+        ho, wo = O.conv_out_hw(s0)
+        dot = np.zeros((s.n, s.cout, ho, wo), np.int64)
+        rowsum = np.zeros((s.n, 1, ho, wo), np.int64)
+        for ky in range(s.kh):
+            for kx in range(s.kw):
+                y0, x0 = ky * s.dil_h, kx * s.dil_w
+                win = xp[:, :, y0:y0 + (ho - 1) * s.stride_h + 1:s.stride_h, x0:x0 + (wo - 1) * s.stride_w + 1:s.stride_w]
+                dot += np.einsum("nchw,oc->nohw", win, ws[:, :, ky, kx])
+                rowsum += win.sum(axis=1, keepdims=True)
+        k_total = s.c * s.kh * s.kw
+        colsum = ws.reshape(s.cout, -1).sum(axis=1)
+        folded = dot - zw * rowsum - za * colsum[None, :, None, None] + k_total * za * zw + b[None, :, None, None]
+        assert np.array_equal(folded.astype(np.int32), acc)
+        del zero_b
+
+
+def test_depthwise_equals_grouped_conv():
+    rng = np.random.default_rng(12)
+    for dm, stride, pad in ((1, (1, 1), (1, 1, 1, 1)), (2, (2, 2), (0, 1, 0, 1)), (3, (1, 2), (1, 0, 2, 1))):
+        c, h, w = 5, 9, 8
+        x = rng.integers(0, 256, (2, c, h, w), dtype=np.uint8)
+        wt = rng.integers(0, 256, (c * dm, 1, 3, 3), dtype=np.uint8)
+        b = rng.integers(-500, 500, c * dm).astype(np.int32)
+        q = O.make_quant(0.1, 7, 0.02, 200, 0.3, 99)
+        sd = O.conv_shape(2, c, h, w, c * dm, 3, 3, stride=stride, pad=pad, dm=dm)
+        sg = O.conv_shape(2, c, h, w, c * dm, 3, 3, stride=stride, pad=pad, groups=c)
+        o1, a1 = O.dwconv2d(x, wt, b, sd, q, want_acc=True)
+        o2, a2 = O.conv2d(x, wt, b, sg, q, want_acc=True)
+        assert np.array_equal(a1, a2) and np.array_equal(o1, o2)
+
+
+def test_fc_equals_1x1_conv_and_numpy():
+    rng = np.random.default_rng(13)
+    m, k, n = 7, 37, 11
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    w = rng.integers(0, 256, (n, k), dtype=np.uint8)
+    b = rng.integers(-1000, 1000, n).astype(np.int32)
+    q = O.make_quant(0.01, 3, 0.002, 128, 0.08, 0)
+    out, acc = O.fc(a, w, b, q, want_acc=True)
+    want = (a.astype(np.int64) - 3) @ (w.astype(np.int64) - 128).T + b
+    assert np.array_equal(acc, want.astype(np.int32))
+    s = O.conv_shape(m, k, 1, 1, n, 1, 1)
+    oc = O.conv2d(a.reshape(m, k, 1, 1), w.reshape(n, k, 1, 1), b, s, q)
+    assert np.array_equal(oc.reshape(m, n), out)
+    # 1x1 conv over pixels == FC over the pixel-major matrix
+    x = rng.integers(0, 256, (2, k, 3, 4), dtype=np.uint8)
+    s2 = O.conv_shape(2, k, 3, 4, n, 1, 1)
+    oc2 = O.conv2d(x, w.reshape(n, k, 1, 1), b, s2, q)
+    of = O.fc(O.nchw2nhwc(x).reshape(-1, k), w, b, q).reshape(2, 3, 4, n)
+    assert np.array_equal(O.nhwc2nchw(of), oc2)
+
+
+DECONV_CASES = [
+    dict(n=2, c=4, h=3, w=5, cout=6, kh=4, kw=4, stride=(2, 2), pad=(1, 1, 1, 1)),
+    dict(n=1, c=6, h=4, w=4, cout=4, kh=3, kw=3, stride=(3, 3), pad=(1, 1, 1, 1), groups=2),
+    dict(n=1, c=3, h=5, w=4, cout=2, kh=2, kw=3, stride=(1, 2), pad=(0, 1, 1, 0)),
+    dict(n=1, c=2, h=3, w=3, cout=2, kh=3, kw=3, stride=(1, 1), pad=(0, 0, 0, 0)),
+]
+
+
+@pytest.mark.parametrize("case", DECONV_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_deconv_gather_equals_scatter(case):
+    rng = np.random.default_rng(14)
+    s = O.conv_shape(**case)
+    x = rng.integers(0, 256, (s.n, s.c, s.h, s.w), dtype=np.uint8)
+    wt = rng.integers(0, 256, (s.c, s.cout // s.groups, s.kh, s.kw), dtype=np.uint8)
+    b = rng.integers(-1000, 1000, s.cout).astype(np.int32)
+    q = O.make_quant(0.03, 131, 0.01, 77, 0.9, 5)
+    o1, a1 = O.deconv2d(x, wt, b, s, q, want_acc=True)
+    o2, a2 = O.deconv2d(x, wt, b, s, q, want_acc=True, scatter=True)
+    assert np.array_equal(a1, a2) and np.array_equal(o1, o2)
+    assert a1.std() > 0
+
+
+def test_deconv_stride1_equals_conv_with_flipped_transposed_kernel():
+    rng = np.random.default_rng(15)
+    n, c, h, w, cout, k, p = 2, 3, 6, 5, 4, 3, 1
+    x = rng.integers(0, 256, (n, c, h, w), dtype=np.uint8)
+    wd = rng.integers(0, 256, (c, cout, k, k), dtype=np.uint8)
+    b = rng.integers(-100, 100, cout).astype(np.int32)
+    q = O.make_quant(0.05, 12, 0.02, 140, 0.7, 33)
+    od, ad = O.deconv2d(x, wd, b, O.conv_shape(n, c, h, w, cout, k, k, pad=(p, p, p, p)), q, want_acc=True)
+    wc = np.ascontiguousarray(wd.transpose(1, 0, 2, 3)[:, :, ::-1, ::-1])
+    pc = k - 1 - p
+    oc, ac = O.conv2d(x, wc, b, O.conv_shape(n, c, h, w, cout, k, k, pad=(pc, pc, pc, pc)), q, want_acc=True)
+    assert np.array_equal(ad, ac) and np.array_equal(od, oc)
+
+
+# ------------------------------------------------------------- invariants
+
+def test_input_at_zero_point_gives_requant_of_bias():
+    rng = np.random.default_rng(16)
+    s, _, wt, b = rand_case(rng, 1, 4, 6, 6, 5, 3, 3, pad=(1, 1, 1, 1))
+    q = O.make_quant(0.5, 77, 0.5, 13, 0.25, 100)
+    x = np.full((1, 4, 6, 6), 77, np.uint8)
+    out, acc = O.conv2d(x, wt, b, s, q, want_acc=True)
+    assert np.array_equal(acc, np.broadcast_to(b[None, :, None, None], acc.shape))
+    x2 = rng.integers(0, 256, (1, 4, 6, 6), dtype=np.uint8)
+    w2 = np.full(wt.shape, 13, np.uint8)
+    _, acc2 = O.conv2d(x2, w2, b, s, q, want_acc=True)
+    assert np.array_equal(acc2, np.broadcast_to(b[None, :, None, None], acc2.shape))
+
+
+def test_layout_round_trip_and_index_form():
+    rng = np.random.default_rng(17)
+    x = rng.integers(0, 256, (3, 5, 4, 7), dtype=np.uint8)
+    y = O.nchw2nhwc(x)
+    assert np.array_equal(y, x.transpose(0, 2, 3, 1))
+    assert np.array_equal(O.nhwc2nchw(y), x)
+
+
+def test_output_dim_formulas():
+    assert O.lib.eo_conv_out_dim(56, 1, 1, 3, 1, 1) == 56
+    assert O.lib.eo_conv_out_dim(56, 1, 1, 3, 1, 2) == 28
+    assert O.lib.eo_conv_out_dim(224, 0, 1, 3, 1, 2) == 112
+    assert O.lib.eo_conv_out_dim(7, 2, 2, 3, 2, 1) == 7
+    assert O.lib.eo_deconv_out_dim(32, 1, 1, 4, 2) == 64
+    assert O.lib.eo_deconv_out_dim(3, 0, 0, 3, 3) == 9
+
+
+def test_empty_shapes_do_not_touch_memory():
+    s = O.conv_shape(0, 4, 6, 6, 5, 3, 3)
+    q = O.raw_quant()
+    out = O.conv2d(np.zeros((0, 4, 6, 6), np.uint8), np.zeros((5, 4, 3, 3), np.uint8), np.zeros(5, np.int32), s, q)
+    assert out.size == 0
+    assert O.fc(np.zeros((0, 8), np.uint8), np.zeros((3, 8), np.uint8), np.zeros(3, np.int32), q).size == 0
+
+
+def test_add_closed_forms():
+    """parity unpinned by reference vectors: equal scales, out scale = in scale -> plain integer add."""
+    q = O.make_add_quant(0.5, 10, 0.5, 20, 0.5, 5)
+    a = np.arange(0, 200, dtype=np.uint8)
+    b = np.arange(200, 0, -1, dtype=np.uint8)
+    want = np.clip((a.astype(int) - 10) + (b.astype(int) - 20) + 5, 0, 255)
+    assert np.array_equal(O.add(a, b, q), want.astype(np.uint8))
+    # out scale twice the input scale halves the sum (ties away from zero after the two-stage rounding)
+    q2 = O.make_add_quant(0.5, 0, 0.5, 0, 1.0, 0)
+    assert O.add(np.array([4, 5, 7], np.uint8), np.array([2, 2, 2], np.uint8), q2).tolist() == [3, 4, 5]
+
+
+def test_avgpool_closed_forms():
+    """parity unpinned by reference vectors: (sum + n/2) / n over the clipped window."""
+    x = np.arange(16, dtype=np.uint8).reshape(1, 1, 4, 4)
+    assert O.avgpool(x, 2, 2, stride=(2, 2)).reshape(-1).tolist() == [3, 5, 11, 13]  # 2.5->3, 4.5->5, ...
+    assert O.avgpool(x, 4, 4).reshape(-1).tolist() == [8]  # 7.5 -> 8
+    # padded window counts only in-image taps
+    o = O.avgpool(x, 3, 3, stride=(1, 1), pad=(1, 1, 1, 1))
+    assert o[0, 0, 0, 0] == (0 + 1 + 4 + 5 + 2) // 4
