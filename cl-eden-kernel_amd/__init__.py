@@ -1,0 +1,257 @@
+"""ctypes binding of libedenhip.so (the C ABI in include/eden_hip.h) for the test
+and benchmark harnesses.  The product's host layer is the C++ operator classes
+under host/; this module only makes the same C ABI callable from Python.
+
+There is no CPU fallback: a missing library raises on import of `lib`, and a
+missing or non-gfx950 GPU makes `init()` raise."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libedenhip.so")
+
+EH_OK = 0
+ACT_NONE, ACT_RELU, ACT_RELU1, ACT_RELU6 = 0, 1, 2, 3
+NCHW, NHWC = 0, 1
+W_OIHW, W_OHWI, W_IOHW = 0, 1, 2
+
+
+class EdenHipError(RuntimeError):
+    pass
+
+
+class Requant(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("zp_in", "zp_w", "zp_out", "multiplier", "shift", "act_min", "act_max")]
+
+    def as_tuple(self):
+        return tuple(getattr(self, n) for n, _ in self._fields_)
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("n", "c", "h", "w", "cout", "kh", "kw", "stride_h", "stride_w",
+                 "pad_t", "pad_b", "pad_l", "pad_r", "dil_h", "dil_w", "groups",
+                 "depth_multiplier", "layout", "weight_layout")]
+
+
+EXPORTS = {
+    # name: (restype, argtypes)
+    "eh_quantize_multiplier": (None, [C.c_double, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "eh_conv_multiplier": (C.c_int, [C.c_float] * 4 + [C.POINTER(C.c_double)]),
+    "eh_act_range_u8": (None, [C.c_int, C.c_float, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "eh_make_requant": (None, [C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_float, C.c_float, C.c_int32,
+                               C.c_int, C.c_int, C.POINTER(Requant)]),
+    "eh_conv_out_dim": (C.c_int32, [C.c_int32] * 6),
+    "eh_deconv_out_dim": (C.c_int32, [C.c_int32] * 5),
+    "eh_init": (C.c_int, [C.c_int]),
+    "eh_device_name": (C.c_int, [C.c_char_p, C.c_size_t]),
+    "eh_malloc": (C.c_int, [C.POINTER(C.c_void_p), C.c_size_t]),
+    "eh_free": (C.c_int, [C.c_void_p]),
+    "eh_memset": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]),
+    "eh_h2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "eh_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "eh_d2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "eh_stream_sync": (C.c_int, [C.c_void_p]),
+    "eh_last_error": (C.c_char_p, []),
+    "eh_transpose_u8_nchw2nhwc": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int32] * 4 + [C.c_void_p]),
+    "eh_transpose_u8_nhwc2nchw": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int32] * 4 + [C.c_void_p]),
+    "eh_conv2d_u8_plan": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(ConvDesc), C.c_void_p, C.c_void_p,
+                                    C.POINTER(Requant), C.c_void_p]),
+    "eh_conv2d_u8_repack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_conv2d_u8_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_conv2d_u8_destroy": (C.c_int, [C.c_void_p]),
+    "eh_dwconv2d_u8_plan": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(ConvDesc), C.c_void_p, C.c_void_p,
+                                      C.POINTER(Requant), C.c_void_p]),
+    "eh_dwconv2d_u8_repack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_dwconv2d_u8_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_dwconv2d_u8_destroy": (C.c_int, [C.c_void_p]),
+    "eh_fc_u8_plan": (C.c_int, [C.POINTER(C.c_void_p), C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
+                                C.POINTER(Requant), C.c_void_p]),
+    "eh_fc_u8_repack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_fc_u8_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_fc_u8_destroy": (C.c_int, [C.c_void_p]),
+    "eh_deconv2d_u8_plan": (C.c_int, [C.POINTER(C.c_void_p), C.POINTER(ConvDesc), C.c_void_p, C.c_void_p,
+                                      C.POINTER(Requant), C.c_void_p]),
+    "eh_deconv2d_u8_repack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_deconv2d_u8_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
+    "eh_deconv2d_u8_destroy": (C.c_int, [C.c_void_p]),
+    "eh_event_create": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "eh_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eh_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "eh_event_destroy": (C.c_int, [C.c_void_p]),
+}
+
+_lib = None
+
+
+def load():
+    """Loads libedenhip.so and types every export; raises if the library or a symbol is missing."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise EdenHipError("%s is not built: run `python cl-eden-kernel_amd/build.py`" % LIB_PATH)
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def check(rc):
+    if rc != EH_OK:
+        raise EdenHipError("eden_hip status %d: %s" % (rc, load().eh_last_error().decode()))
+
+
+def init(device=0):
+    check(load().eh_init(device))
+
+
+def device_name():
+    buf = C.create_string_buffer(256)
+    check(load().eh_device_name(buf, 256))
+    return buf.value.decode()
+
+
+def make_requant(s_in, zp_in, s_w, zp_w, s_out, zp_out, act=ACT_NONE, act_enabled=False, s_bias=None):
+    if s_bias is None:
+        s_bias = float(np.float32(s_in) * np.float32(s_w))
+    q = Requant()
+    load().eh_make_requant(s_in, zp_in, s_w, zp_w, s_bias, s_out, zp_out, act, int(act_enabled), C.byref(q))
+    return q
+
+
+def conv_desc(n, c, h, w, cout, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, dm=1,
+              layout=NCHW, weight_layout=W_OIHW):
+    """pad = (top, bottom, left, right)"""
+    return ConvDesc(n, c, h, w, cout, kh, kw, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3],
+                    dil[0], dil[1], groups, dm, layout, weight_layout)
+
+
+class DeviceBuffer:
+    """A device allocation made through the C ABI, with host copies in and out."""
+
+    def __init__(self, nbytes=None, host=None):
+        lib = load()
+        if host is not None:
+            host = np.ascontiguousarray(host)
+            nbytes = host.nbytes
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        check(lib.eh_malloc(C.byref(p), self.nbytes))
+        self.ptr = p
+        if host is not None and self.nbytes:
+            check(lib.eh_h2d(self.ptr, host.ctypes.data_as(C.c_void_p), self.nbytes, None))
+            check(lib.eh_stream_sync(None))
+
+    def download(self, shape, dtype=np.uint8):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        lib = load()
+        if out.nbytes:
+            check(lib.eh_d2h(out.ctypes.data_as(C.c_void_p), self.ptr, out.nbytes, None))
+        check(lib.eh_stream_sync(None))
+        return out
+
+    def free(self):
+        if self.ptr is not None:
+            load().eh_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class _Plan:
+    _kind = ""
+
+    def __init__(self):
+        self.handle = C.c_void_p()
+        self._keep = []
+
+    def run(self, d_in, d_out, q, stream=None):
+        check(getattr(load(), "eh_%s_u8_run" % self._kind)(self.handle, d_in.ptr, d_out.ptr, C.byref(q), stream))
+
+    def repack(self, d_w, d_b, q, stream=None):
+        check(getattr(load(), "eh_%s_u8_repack" % self._kind)(self.handle, d_w.ptr, d_b.ptr if d_b else None,
+                                                            C.byref(q), stream))
+
+    def destroy(self):
+        if self.handle:
+            getattr(load(), "eh_%s_u8_destroy" % self._kind)(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class ConvPlan(_Plan):
+    _kind = "conv2d"
+
+    def __init__(self, desc, d_w, d_b, q, stream=None):
+        super().__init__()
+        self.desc = desc
+        check(load().eh_conv2d_u8_plan(C.byref(self.handle), C.byref(desc), d_w.ptr, d_b.ptr if d_b else None,
+                                       C.byref(q), stream))
+
+
+class DwConvPlan(_Plan):
+    _kind = "dwconv2d"
+
+    def __init__(self, desc, d_w, d_b, q, stream=None):
+        super().__init__()
+        self.desc = desc
+        check(load().eh_dwconv2d_u8_plan(C.byref(self.handle), C.byref(desc), d_w.ptr, d_b.ptr if d_b else None,
+                                         C.byref(q), stream))
+
+
+class DeconvPlan(_Plan):
+    _kind = "deconv2d"
+
+    def __init__(self, desc, d_w, d_b, q, stream=None):
+        super().__init__()
+        self.desc = desc
+        check(load().eh_deconv2d_u8_plan(C.byref(self.handle), C.byref(desc), d_w.ptr, d_b.ptr if d_b else None,
+                                         C.byref(q), stream))
+
+
+class FcPlan(_Plan):
+    _kind = "fc"
+
+    def __init__(self, m, k, n, d_w, d_b, q, stream=None):
+        super().__init__()
+        self.m, self.k, self.n = m, k, n
+        check(load().eh_fc_u8_plan(C.byref(self.handle), m, k, n, d_w.ptr, d_b.ptr if d_b else None, C.byref(q), stream))
+
+
+class Event:
+    def __init__(self):
+        self.h = C.c_void_p()
+        check(load().eh_event_create(C.byref(self.h)))
+
+    def record(self, stream=None):
+        check(load().eh_event_record(self.h, stream))
+
+    def elapsed_ms_since(self, start):
+        ms = C.c_float()
+        check(load().eh_event_elapsed_ms(start.h, self.h, C.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            load().eh_event_destroy(self.h)
+        except Exception:
+            pass
+
+
+def sync(stream=None):
+    check(load().eh_stream_sync(stream))

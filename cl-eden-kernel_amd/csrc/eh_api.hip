@@ -1,0 +1,939 @@
+// C ABI of libedenhip.so: host arithmetic, device buffers, and the operator
+// plans (packed weights + folded bias + k-tables) behind eden_hip.h.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <new>
+#include <vector>
+
+#include "eh_internal.h"
+
+namespace eh {
+
+// ------------------------------------------------------------------ errors
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return EH_DEVICE_FAILURE;
+}
+
+int check_requant(const eh_requant *q) {
+    EH_REQUIRE(q != nullptr, "requant parameters are null");
+    EH_REQUIRE(q->multiplier >= 0, "requant multiplier %d is negative", q->multiplier);
+    EH_REQUIRE(q->shift >= -31 && q->shift <= 30, "requant shift %d outside [-31, 30]", q->shift);
+    EH_REQUIRE(q->zp_in >= 0 && q->zp_in <= 255 && q->zp_w >= 0 && q->zp_w <= 255,
+               "uint8 zero points (%d, %d) outside [0, 255]", q->zp_in, q->zp_w);
+    EH_REQUIRE(q->act_min >= 0 && q->act_max <= 255 && q->act_min <= q->act_max, "activation range [%d, %d] invalid",
+               q->act_min, q->act_max);
+    return EH_OK;
+}
+
+namespace {
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+inline int round_up(int v, int a) { return (v + a - 1) / a * a; }
+
+template <typename T>
+int dev_alloc(T **p, size_t count) {
+    *p = nullptr;
+    if (count == 0) count = 1;
+    EH_HIP(hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T)));
+    return EH_OK;
+}
+
+template <typename T>
+void dev_free(T *&p) {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+}
+
+// One GEMM the operator decomposes into: a convolution group or a
+// deconvolution output phase.
+struct GemmPart {
+    int8_t *b = nullptr;
+    int32_t *colsum = nullptr;
+    int32_t *folded = nullptr;
+    KUnit *ktab = nullptr;
+    int32_t *tap_off = nullptr;
+    int32_t n = 0, n_pad = 0, k = 0, k_pad = 0, vec = 1, taps = 0, cin = 0;
+    int64_t so = 0, sc = 0;   // source weight strides (out channel, in channel)
+    int64_t w_base = 0;       // element offset of this part in the source weights
+    int32_t bias_base = 0;    // first output channel
+    GemmProblem proto{};      // geometry; pointers and quantization filled per run
+
+    void release() {
+        dev_free(b);
+        dev_free(colsum);
+        dev_free(folded);
+        dev_free(ktab);
+        dev_free(tap_off);
+    }
+};
+
+int pick_vec(int cig, int pixel_stride) {
+    if ((cig & 15) == 0 && (pixel_stride & 15) == 0) return 16;
+    if ((cig & 3) == 0 && (pixel_stride & 3) == 0) return 4;
+    return 1;
+}
+
+// Allocates a part's device arrays and uploads its tables.  `units` holds one
+// KUnit per `vec` bytes of the real reduction length; padding units are added here.
+int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream) {
+    g.k_pad = round_up(g.k > 0 ? g.k : 1, 64);
+    g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
+    KUnit pad;
+    pad.offset = 0;
+    pad.dy = INT16_MIN;
+    pad.dx = 0;
+    units.resize((size_t)g.k_pad / g.vec, pad);
+    int rc;
+    if ((rc = dev_alloc(&g.b, (size_t)g.n_pad * g.k_pad))) return rc;
+    if ((rc = dev_alloc(&g.colsum, (size_t)g.n_pad))) return rc;
+    if ((rc = dev_alloc(&g.folded, (size_t)g.n_pad))) return rc;
+    if ((rc = dev_alloc(&g.ktab, units.size()))) return rc;
+    if ((rc = dev_alloc(&g.tap_off, tap_off.size()))) return rc;
+    EH_HIP(hipMemcpyAsync(g.ktab, units.data(), units.size() * sizeof(KUnit), hipMemcpyHostToDevice, stream));
+    if (!tap_off.empty())
+        EH_HIP(hipMemcpyAsync(g.tap_off, tap_off.data(), tap_off.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+    // the host vectors die with the caller's frame: make sure the copies have left them
+    EH_HIP(hipStreamSynchronize(stream));
+    g.proto.ktab = g.ktab;
+    g.proto.k = g.k;
+    g.proto.k_pad = g.k_pad;
+    g.proto.vec = g.vec;
+    g.proto.n = g.n;
+    return EH_OK;
+}
+
+int pack_part(GemmPart &g, const uint8_t *weight, hipStream_t stream) {
+    PackProblem pp;
+    pp.w = weight + g.w_base;
+    pp.bias = nullptr;
+    pp.b = g.b;
+    pp.colsum = g.colsum;
+    pp.n = g.n;
+    pp.n_pad = g.n_pad;
+    pp.cin = g.cin > 0 ? g.cin : 1;
+    pp.taps = g.taps;
+    pp.k = g.k;
+    pp.k_pad = g.k_pad;
+    pp.so = g.so;
+    pp.sc = g.sc;
+    pp.tap_off = g.tap_off;
+    return launch_pack_weights(pp, stream);
+}
+
+// Shared state of the three GEMM-shaped operators.
+struct GemmOp {
+    std::vector<GemmPart> parts;
+    int32_t *bias_copy = nullptr;  // the operator's own copy of the int32 bias
+    int32_t cout = 0;
+    eh_requant q{};
+    bool folded_valid = false;
+    // NCHW boundary: the kernels compute channels-last, so planar tensors pass
+    // through these two staging images
+    uint8_t *stage_in = nullptr, *stage_out = nullptr;
+    int32_t layout = EH_NHWC;
+    int32_t in_n = 0, in_c = 0, in_hw = 0, out_hw = 0;
+    size_t in_bytes = 0;
+
+    void release() {
+        for (auto &g : parts) g.release();
+        parts.clear();
+        dev_free(bias_copy);
+        dev_free(stage_in);
+        dev_free(stage_out);
+    }
+
+    int set_weights(const void *weight, const void *bias, hipStream_t stream) {
+        EH_REQUIRE(weight != nullptr, "weight pointer is null");
+        for (auto &g : parts) {
+            int rc = pack_part(g, static_cast<const uint8_t *>(weight), stream);
+            if (rc) return rc;
+        }
+        if (bias)
+            EH_HIP(hipMemcpyAsync(bias_copy, bias, (size_t)cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
+        else
+            EH_HIP(hipMemsetAsync(bias_copy, 0, (size_t)cout * sizeof(int32_t), stream));
+        folded_valid = false;
+        return EH_OK;
+    }
+
+    int refold(const eh_requant &nq, hipStream_t stream) {
+        if (folded_valid && nq.zp_in == q.zp_in && nq.zp_w == q.zp_w) {
+            q = nq;
+            return EH_OK;
+        }
+        for (auto &g : parts) {
+            int rc = launch_fold_bias(bias_copy + g.bias_base, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, nq.zp_w,
+                                      stream);
+            if (rc) return rc;
+        }
+        q = nq;
+        folded_valid = true;
+        return EH_OK;
+    }
+
+    int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream) {
+        EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
+        int rc = check_requant(nq);
+        if (rc) return rc;
+        if ((rc = refold(*nq, stream))) return rc;
+        const uint8_t *in = static_cast<const uint8_t *>(input);
+        uint8_t *out = static_cast<uint8_t *>(output);
+        if (layout == EH_NCHW) {
+            if ((rc = launch_nchw2nhwc(in, stage_in, in_n, in_c, in_hw, stream))) return rc;
+            in = stage_in;
+            out = stage_out;
+        }
+        for (auto &g : parts) {
+            GemmProblem p = g.proto;
+            EH_REQUIRE((reinterpret_cast<uintptr_t>(in) & (uintptr_t)(g.vec - 1)) == 0,
+                       "input pointer is not aligned to %d bytes", g.vec);
+            p.a = in;
+            p.b = g.b;
+            p.bias = g.folded;
+            p.out = out + g.bias_base;
+            p.zw = q.zp_w - 128;
+            p.fill = (uint32_t)q.zp_in * 0x01010101u;
+            p.rq = make_requant_dev(q);
+            if ((rc = launch_igemm(p, stream))) return rc;
+        }
+        if (layout == EH_NCHW) {
+            if ((rc = launch_nhwc2nchw(stage_out, static_cast<uint8_t *>(output), in_n, cout, out_hw, stream))) return rc;
+        }
+        return EH_OK;
+    }
+};
+
+int check_desc_common(const eh_conv_desc *d) {
+    EH_REQUIRE(d != nullptr, "descriptor is null");
+    EH_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->cout > 0, "bad tensor extents n=%d c=%d h=%d w=%d cout=%d",
+               d->n, d->c, d->h, d->w, d->cout);
+    EH_REQUIRE(d->kh > 0 && d->kw > 0 && d->stride_h > 0 && d->stride_w > 0, "bad kernel/stride");
+    EH_REQUIRE(d->pad_t >= 0 && d->pad_b >= 0 && d->pad_l >= 0 && d->pad_r >= 0, "negative padding");
+    EH_REQUIRE(d->layout == EH_NCHW || d->layout == EH_NHWC, "unknown layout %d", d->layout);
+    EH_REQUIRE((int64_t)d->n * d->c * d->h * d->w < (1ll << 31), "input larger than 2 GiB is not supported");
+    EH_REQUIRE(d->h < 32000 && d->w < 32000, "spatial extent too large");
+    return EH_OK;
+}
+
+}  // namespace
+}  // namespace eh
+
+using namespace eh;
+
+struct eh_conv_plan {
+    GemmOp op;
+    eh_conv_desc d;
+};
+struct eh_fc_plan {
+    GemmOp op;
+    int32_t m, k, n;
+};
+struct eh_deconv_plan {
+    GemmOp op;
+    eh_conv_desc d;
+};
+struct eh_dwconv_plan {
+    eh_conv_desc d;
+    int32_t ho = 0, wo = 0, cout = 0, taps = 0;
+    uint8_t *w_copy = nullptr;
+    int32_t *bias_copy = nullptr;
+    int32_t *w_pair = nullptr;
+    int32_t *bias_folded = nullptr;
+    eh_requant q{};
+    bool packed_valid = false;
+};
+
+extern "C" {
+
+// ------------------------------------------------------------ host arithmetic
+
+void eh_quantize_multiplier(double real_multiplier, int32_t *quantized_multiplier, int32_t *shift) {
+    if (real_multiplier == 0.) {
+        *quantized_multiplier = 0;
+        *shift = 0;
+        return;
+    }
+    int exponent = 0;
+    const double significand = frexp(real_multiplier, &exponent);
+    int64_t fixed = (int64_t)round(significand * 2147483648.0);
+    if (fixed == 2147483648ll) {
+        fixed /= 2;
+        ++exponent;
+    }
+    *quantized_multiplier = (int32_t)fixed;
+    *shift = exponent;
+}
+
+int eh_conv_multiplier(float input_scale, float filter_scale, float bias_scale, float output_scale, double *multiplier) {
+    const double product = (double)input_scale * (double)filter_scale;
+    const double bs = (double)bias_scale;
+    if (!(fabs(product - bs) <= 1e-6 * (product < bs ? product : bs))) return EH_FAILURE;
+    if (!(product >= 0)) return EH_FAILURE;
+    *multiplier = product / (double)output_scale;
+    return EH_OK;
+}
+
+void eh_act_range_u8(int activation, float scale, int32_t zero_point, int32_t *act_min, int32_t *act_max) {
+    auto quantize = [scale, zero_point](float f) { return zero_point + (int32_t)round((double)(f / scale)); };
+    int32_t lo = 0, hi = 255;
+    if (activation == EH_ACT_RELU) {
+        lo = quantize(0.0f) > lo ? quantize(0.0f) : lo;
+    } else if (activation == EH_ACT_RELU6) {
+        lo = quantize(0.0f) > lo ? quantize(0.0f) : lo;
+        hi = quantize(6.0f) < hi ? quantize(6.0f) : hi;
+    } else if (activation == EH_ACT_RELU1) {
+        lo = quantize(-1.0f) > lo ? quantize(-1.0f) : lo;
+        hi = quantize(1.0f) < hi ? quantize(1.0f) : hi;
+    }
+    *act_min = lo;
+    *act_max = hi;
+}
+
+void eh_make_requant(float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp, float bias_scale,
+                     float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out) {
+    double m = 0.0;  // stays 0 when the bias scale check fails, as in the reference's callers
+    (void)eh_conv_multiplier(input_scale, filter_scale, bias_scale, output_scale, &m);
+    eh_quantize_multiplier(m, &out->multiplier, &out->shift);
+    if (out->shift < -31) {
+        // |acc * M| < 2^31 * 2^-32 rounds to 0 for every int32 accumulator
+        out->multiplier = 0;
+        out->shift = 0;
+    }
+    out->zp_in = input_zp;
+    out->zp_w = filter_zp;
+    out->zp_out = output_zp;
+    if (activation_enabled) {
+        eh_act_range_u8(activation, output_scale, output_zp, &out->act_min, &out->act_max);
+    } else {
+        out->act_min = 0;
+        out->act_max = 255;
+    }
+}
+
+int32_t eh_conv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t dilation, int32_t stride) {
+    return (in + pad_a + pad_b - (dilation * (kernel - 1) + 1) + stride) / stride;
+}
+
+int32_t eh_deconv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t stride) {
+    return in * stride + kernel - stride - pad_a - pad_b;
+}
+
+// ------------------------------------------------------------ runtime
+
+const char *eh_last_error(void) { return g_error; }
+
+int eh_init(int device) {
+    int count = 0;
+    EH_HIP(hipGetDeviceCount(&count));
+    EH_REQUIRE(device >= 0 && device < count, "device %d not present (%d visible)", device, count);
+    EH_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    EH_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+        return EH_FAILURE;
+    }
+    return EH_OK;
+}
+
+int eh_device_name(char *dst, size_t cap) {
+    EH_REQUIRE(dst != nullptr && cap > 0, "bad destination");
+    int dev = 0;
+    EH_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    EH_HIP(hipGetDeviceProperties(&prop, dev));
+    snprintf(dst, cap, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return EH_OK;
+}
+
+int eh_malloc(void **ptr, size_t bytes) {
+    EH_REQUIRE(ptr != nullptr, "null result pointer");
+    *ptr = nullptr;
+    const size_t padded = (bytes + 255) / 256 * 256 + 256;
+    EH_HIP(hipMalloc(ptr, padded));
+    hipError_t e = hipMemset(*ptr, 0, padded);
+    if (e != hipSuccess) {
+        (void)hipFree(*ptr);
+        *ptr = nullptr;
+        return hip_fail(e, "hipMemset");
+    }
+    return EH_OK;
+}
+
+int eh_free(void *ptr) {
+    if (ptr) EH_HIP(hipFree(ptr));
+    return EH_OK;
+}
+
+int eh_memset(void *ptr, int value, size_t bytes, void *stream) {
+    if (bytes) EH_HIP(hipMemsetAsync(ptr, value, bytes, as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_h2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes) EH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_d2h(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes) EH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes) EH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_stream_sync(void *stream) {
+    EH_HIP(hipStreamSynchronize(as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_event_create(void **event) {
+    EH_REQUIRE(event != nullptr, "null result pointer");
+    hipEvent_t e;
+    EH_HIP(hipEventCreate(&e));
+    *event = e;
+    return EH_OK;
+}
+
+int eh_event_record(void *event, void *stream) {
+    EH_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_event_elapsed_ms(void *start, void *stop, float *ms) {
+    EH_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(stop)));
+    EH_HIP(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop)));
+    return EH_OK;
+}
+
+int eh_event_destroy(void *event) {
+    if (event) EH_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+    return EH_OK;
+}
+
+// ------------------------------------------------------------ layout
+
+int eh_transpose_u8_nchw2nhwc(const void *src, void *dst, int32_t n, int32_t c, int32_t h, int32_t w, void *stream) {
+    EH_REQUIRE(n >= 0 && c >= 0 && h >= 0 && w >= 0, "negative extent");
+    if ((int64_t)n * c * h * w == 0) return EH_OK;
+    EH_REQUIRE(src != nullptr && dst != nullptr && src != dst, "bad pointers");
+    EH_REQUIRE((int64_t)h * w < (1ll << 31), "plane too large");
+    return launch_nchw2nhwc(static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), n, c, h * w, as_stream(stream));
+}
+
+int eh_transpose_u8_nhwc2nchw(const void *src, void *dst, int32_t n, int32_t c, int32_t h, int32_t w, void *stream) {
+    EH_REQUIRE(n >= 0 && c >= 0 && h >= 0 && w >= 0, "negative extent");
+    if ((int64_t)n * c * h * w == 0) return EH_OK;
+    EH_REQUIRE(src != nullptr && dst != nullptr && src != dst, "bad pointers");
+    EH_REQUIRE((int64_t)h * w < (1ll << 31), "plane too large");
+    return launch_nhwc2nchw(static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), n, c, h * w, as_stream(stream));
+}
+
+// ------------------------------------------------------------ convolution
+
+static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t stream) {
+    GemmOp &op = pl->op;
+    const int G = d->groups, cig = d->c / G, cog = d->cout / G;
+    const int ho = eh_conv_out_dim(d->h, d->pad_t, d->pad_b, d->kh, d->dil_h, d->stride_h);
+    const int wo = eh_conv_out_dim(d->w, d->pad_l, d->pad_r, d->kw, d->dil_w, d->stride_w);
+    EH_REQUIRE(ho > 0 && wo > 0, "convolution output is empty (%d x %d)", ho, wo);
+    EH_REQUIRE((int64_t)d->n * ho * wo < (1ll << 31), "too many output pixels");
+    EH_REQUIRE((int64_t)d->n * ho * wo * d->cout < (1ll << 31) * 2, "output larger than 4 GiB is not supported");
+    op.cout = d->cout;
+    op.layout = d->layout;
+    op.in_n = d->n;
+    op.in_c = d->c;
+    op.in_hw = d->h * d->w;
+    op.out_hw = ho * wo;
+    int rc;
+    if ((rc = dev_alloc(&op.bias_copy, (size_t)d->cout))) return rc;
+    if (d->layout == EH_NCHW) {
+        if ((rc = dev_alloc(&op.stage_in, (size_t)d->n * d->c * d->h * d->w + 256))) return rc;
+        if ((rc = dev_alloc(&op.stage_out, (size_t)d->n * d->cout * ho * wo + 256))) return rc;
+    }
+    const int taps = d->kh * d->kw;
+    op.parts.resize(G);
+    for (int g = 0; g < G; ++g) {
+        GemmPart &part = op.parts[g];
+        part.n = cog;
+        part.cin = cig;
+        part.taps = taps;
+        part.k = taps * cig;
+        part.vec = pick_vec(cig, d->c);
+        part.bias_base = g * cog;
+        if (d->weight_layout == EH_W_OIHW) {
+            part.so = (int64_t)cig * taps;
+            part.sc = taps;
+        } else {
+            part.so = (int64_t)taps * cig;
+            part.sc = 1;
+        }
+        part.w_base = (int64_t)g * cog * part.so;
+        std::vector<int32_t> tap_off(taps);
+        for (int t = 0; t < taps; ++t) tap_off[t] = d->weight_layout == EH_W_OIHW ? t : t * cig;
+        std::vector<KUnit> units;
+        for (int k = 0; k < part.k; k += part.vec) {
+            const int t = k / cig, c = k - t * cig;
+            const int ky = t / d->kw, kx = t - ky * d->kw;
+            KUnit u;
+            u.dy = (int16_t)(ky * d->dil_h);
+            u.dx = (int16_t)(kx * d->dil_w);
+            u.offset = (u.dy * d->w + u.dx) * d->c + g * cig + c;
+            units.push_back(u);
+        }
+        GemmProblem &p = part.proto;
+        p.m = d->n * ho * wo;
+        p.h = d->h;
+        p.w = d->w;
+        p.cin = d->c;
+        p.ho = ho;
+        p.wo = wo;
+        p.stride_h = d->stride_h;
+        p.stride_w = d->stride_w;
+        p.y_base = -d->pad_t;
+        p.x_base = -d->pad_l;
+        p.out_h = ho;
+        p.out_w = wo;
+        p.out_sy = 1;
+        p.out_sx = 1;
+        p.out_y0 = 0;
+        p.out_x0 = 0;
+        p.ldc = d->cout;
+        if ((rc = finish_part(part, units, tap_off, stream))) return rc;
+    }
+    return EH_OK;
+}
+
+int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
+                      const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan pointer");
+    *plan = nullptr;
+    int rc = check_desc_common(desc);
+    if (rc) return rc;
+    if ((rc = check_requant(q))) return rc;
+    EH_REQUIRE(desc->dil_h > 0 && desc->dil_w > 0, "bad dilation");
+    EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
+               "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
+    EH_REQUIRE(desc->weight_layout == EH_W_OIHW || desc->weight_layout == EH_W_OHWI, "bad convolution weight layout %d",
+               desc->weight_layout);
+    EH_REQUIRE(desc->weight_layout == EH_W_OIHW || desc->groups == 1, "OHWI weights support groups == 1 only");
+    EH_REQUIRE(desc->kh * desc->dil_h < 32000 && desc->kw * desc->dil_w < 32000, "kernel extent too large");
+    eh_conv_plan *pl = new (std::nothrow) eh_conv_plan();
+    EH_REQUIRE(pl != nullptr, "out of host memory");
+    pl->d = *desc;
+    if (desc->n > 0) {
+        rc = conv_plan_build(pl, desc, as_stream(stream));
+        if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
+        if (!rc) rc = pl->op.refold(*q, as_stream(stream));
+        if (rc) {
+            pl->op.release();
+            delete pl;
+            return rc;
+        }
+    }
+    *plan = pl;
+    return EH_OK;
+}
+
+int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    int rc = check_requant(q);
+    if (rc) return rc;
+    if (plan->d.n == 0) return EH_OK;
+    if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
+    return plan->op.refold(*q, as_stream(stream));
+}
+
+int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    if (plan->d.n == 0) return check_requant(q);  // zero-size early-out, as CLConvolution::execute does
+    return plan->op.run(input, output, q, as_stream(stream));
+}
+
+int eh_conv2d_u8_destroy(eh_conv_plan *plan) {
+    if (plan) {
+        plan->op.release();
+        delete plan;
+    }
+    return EH_OK;
+}
+
+// ------------------------------------------------------------ fully connected
+
+int eh_fc_u8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, const void *weight, const void *bias,
+                  const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan pointer");
+    *plan = nullptr;
+    EH_REQUIRE(m >= 0 && k > 0 && n > 0, "bad extents m=%d k=%d n=%d", m, k, n);
+    EH_REQUIRE((int64_t)m * k < (1ll << 31), "input larger than 2 GiB is not supported");
+    int rc = check_requant(q);
+    if (rc) return rc;
+    eh_fc_plan *pl = new (std::nothrow) eh_fc_plan();
+    EH_REQUIRE(pl != nullptr, "out of host memory");
+    pl->m = m;
+    pl->k = k;
+    pl->n = n;
+    GemmOp &op = pl->op;
+    op.cout = n;
+    op.layout = EH_NHWC;
+    hipStream_t s = as_stream(stream);
+    rc = dev_alloc(&op.bias_copy, (size_t)n);
+    if (!rc) {
+        op.parts.resize(1);
+        GemmPart &part = op.parts[0];
+        part.n = n;
+        part.cin = k;
+        part.taps = 1;
+        part.k = k;
+        part.vec = pick_vec(k, k);
+        part.so = k;
+        part.sc = 1;
+        std::vector<int32_t> tap_off(1, 0);
+        std::vector<KUnit> units;
+        for (int kk = 0; kk < k; kk += part.vec) {
+            KUnit u;
+            u.dy = 0;
+            u.dx = 0;
+            u.offset = kk;
+            units.push_back(u);
+        }
+        GemmProblem &p = part.proto;
+        p.m = m;
+        p.h = 1;
+        p.w = 1;
+        p.cin = k;
+        p.ho = 1;
+        p.wo = 1;
+        p.stride_h = 1;
+        p.stride_w = 1;
+        p.y_base = 0;
+        p.x_base = 0;
+        p.out_h = 1;
+        p.out_w = 1;
+        p.out_sy = 1;
+        p.out_sx = 1;
+        p.out_y0 = 0;
+        p.out_x0 = 0;
+        p.ldc = n;
+        rc = finish_part(part, units, tap_off, s);
+    }
+    if (!rc) rc = op.set_weights(weight, bias, s);
+    if (!rc) rc = op.refold(*q, s);
+    if (rc) {
+        op.release();
+        delete pl;
+        return rc;
+    }
+    *plan = pl;
+    return EH_OK;
+}
+
+int eh_fc_u8_repack(eh_fc_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    int rc = check_requant(q);
+    if (rc) return rc;
+    if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
+    return plan->op.refold(*q, as_stream(stream));
+}
+
+int eh_fc_u8_run(eh_fc_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    if (plan->m == 0) return check_requant(q);
+    return plan->op.run(input, output, q, as_stream(stream));
+}
+
+int eh_fc_u8_destroy(eh_fc_plan *plan) {
+    if (plan) {
+        plan->op.release();
+        delete plan;
+    }
+    return EH_OK;
+}
+
+// ------------------------------------------------------------ deconvolution
+// A transposed convolution with stride s splits into s_h * s_w independent
+// stride-1 convolutions, one per output phase (oy + pad_t) mod s_h,
+// (ox + pad_l) mod s_w: phase (py, px) uses the taps ky = py + s_h*ty,
+// kx = px + s_w*tx and writes every s-th output pixel.  Each phase is one
+// implicit GEMM with the epilogue fused, so the reference's int32 col buffer
+// (N*Hi*Wi*Cout*kh*kw*4 bytes, CLDeconvolutionQuantized.cpp:99-103) never exists.
+
+static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStream_t stream) {
+    GemmOp &op = pl->op;
+    const int G = d->groups, cig = d->c / G, cog = d->cout / G;
+    const int oh = eh_deconv_out_dim(d->h, d->pad_t, d->pad_b, d->kh, d->stride_h);
+    const int ow = eh_deconv_out_dim(d->w, d->pad_l, d->pad_r, d->kw, d->stride_w);
+    EH_REQUIRE(oh > 0 && ow > 0, "deconvolution output is empty (%d x %d)", oh, ow);
+    EH_REQUIRE((int64_t)d->n * oh * ow * d->cout < (1ll << 31) * 2, "output larger than 4 GiB is not supported");
+    op.cout = d->cout;
+    op.layout = d->layout;
+    op.in_n = d->n;
+    op.in_c = d->c;
+    op.in_hw = d->h * d->w;
+    op.out_hw = oh * ow;
+    int rc;
+    if ((rc = dev_alloc(&op.bias_copy, (size_t)d->cout))) return rc;
+    if (d->layout == EH_NCHW) {
+        if ((rc = dev_alloc(&op.stage_in, (size_t)d->n * d->c * d->h * d->w + 256))) return rc;
+        if ((rc = dev_alloc(&op.stage_out, (size_t)d->n * d->cout * oh * ow + 256))) return rc;
+    }
+    const int sh = d->stride_h, sw = d->stride_w;
+    for (int g = 0; g < G; ++g)
+        for (int py = 0; py < sh; ++py)
+            for (int px = 0; px < sw; ++px) {
+                const int oy0 = ((py - d->pad_t) % sh + sh) % sh, ox0 = ((px - d->pad_l) % sw + sw) % sw;
+                if (oy0 >= oh || ox0 >= ow) continue;
+                const int ho_p = (oh - oy0 + sh - 1) / sh, wo_p = (ow - ox0 + sw - 1) / sw;
+                const int nty = py < d->kh ? (d->kh - py + sh - 1) / sh : 0;
+                const int ntx = px < d->kw ? (d->kw - px + sw - 1) / sw : 0;
+                const int by = (oy0 + d->pad_t - py) / sh, bx = (ox0 + d->pad_l - px) / sw;
+                op.parts.emplace_back();
+                GemmPart &part = op.parts.back();
+                part.n = cog;
+                part.cin = cig;
+                part.taps = nty * ntx;
+                part.k = part.taps * cig;
+                part.vec = pick_vec(cig, d->c);
+                part.bias_base = g * cog;
+                std::vector<int32_t> tap_off(part.taps > 0 ? part.taps : 0);
+                if (d->weight_layout == EH_W_IOHW) {
+                    part.so = (int64_t)d->kh * d->kw;
+                    part.sc = (int64_t)cog * d->kh * d->kw;
+                    part.w_base = (int64_t)g * cig * cog * d->kh * d->kw;
+                } else {  // OHWI, groups == 1
+                    part.so = (int64_t)d->kh * d->kw * d->c;
+                    part.sc = 1;
+                    part.w_base = 0;
+                }
+                for (int ty = 0; ty < nty; ++ty)
+                    for (int tx = 0; tx < ntx; ++tx) {
+                        const int ky = py + sh * ty, kx = px + sw * tx;
+                        tap_off[ty * ntx + tx] = d->weight_layout == EH_W_IOHW ? ky * d->kw + kx : (ky * d->kw + kx) * d->c;
+                    }
+                std::vector<KUnit> units;
+                for (int k = 0; k < part.k; k += part.vec) {
+                    const int t = k / cig, c = k - t * cig;
+                    const int ty = t / ntx, tx = t - ty * ntx;
+                    KUnit u;
+                    u.dy = (int16_t)(by - ty);
+                    u.dx = (int16_t)(bx - tx);
+                    u.offset = (u.dy * d->w + u.dx) * d->c + g * cig + c;
+                    units.push_back(u);
+                }
+                GemmProblem &p = part.proto;
+                p.m = d->n * ho_p * wo_p;
+                p.h = d->h;
+                p.w = d->w;
+                p.cin = d->c;
+                p.ho = ho_p;
+                p.wo = wo_p;
+                p.stride_h = 1;
+                p.stride_w = 1;
+                p.y_base = 0;
+                p.x_base = 0;
+                p.out_h = oh;
+                p.out_w = ow;
+                p.out_sy = sh;
+                p.out_sx = sw;
+                p.out_y0 = oy0;
+                p.out_x0 = ox0;
+                p.ldc = d->cout;
+                if ((rc = finish_part(part, units, tap_off, stream))) return rc;
+            }
+    return EH_OK;
+}
+
+int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
+                        const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan pointer");
+    *plan = nullptr;
+    int rc = check_desc_common(desc);
+    if (rc) return rc;
+    if ((rc = check_requant(q))) return rc;
+    EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
+               "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
+    EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->weight_layout == EH_W_OHWI, "bad deconvolution weight layout %d",
+               desc->weight_layout);
+    EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->groups == 1, "OHWI weights support groups == 1 only");
+    eh_deconv_plan *pl = new (std::nothrow) eh_deconv_plan();
+    EH_REQUIRE(pl != nullptr, "out of host memory");
+    pl->d = *desc;
+    if (desc->n > 0) {
+        rc = deconv_plan_build(pl, desc, as_stream(stream));
+        if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
+        if (!rc) rc = pl->op.refold(*q, as_stream(stream));
+        if (rc) {
+            pl->op.release();
+            delete pl;
+            return rc;
+        }
+    }
+    *plan = pl;
+    return EH_OK;
+}
+
+int eh_deconv2d_u8_repack(eh_deconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    int rc = check_requant(q);
+    if (rc) return rc;
+    if (plan->d.n == 0) return EH_OK;
+    if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
+    return plan->op.refold(*q, as_stream(stream));
+}
+
+int eh_deconv2d_u8_run(eh_deconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    if (plan->d.n == 0) return check_requant(q);
+    return plan->op.run(input, output, q, as_stream(stream));
+}
+
+int eh_deconv2d_u8_destroy(eh_deconv_plan *plan) {
+    if (plan) {
+        plan->op.release();
+        delete plan;
+    }
+    return EH_OK;
+}
+
+// ------------------------------------------------------------ depthwise
+
+static void dw_release(eh_dwconv_plan *pl) {
+    dev_free(pl->w_copy);
+    dev_free(pl->bias_copy);
+    dev_free(pl->w_pair);
+    dev_free(pl->bias_folded);
+}
+
+static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
+    EH_REQUIRE(weight != nullptr, "weight pointer is null");
+    EH_HIP(hipMemcpyAsync(pl->w_copy, weight, (size_t)pl->cout * pl->taps, hipMemcpyDeviceToDevice, stream));
+    if (bias)
+        EH_HIP(hipMemcpyAsync(pl->bias_copy, bias, (size_t)pl->cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
+    else
+        EH_HIP(hipMemsetAsync(pl->bias_copy, 0, (size_t)pl->cout * sizeof(int32_t), stream));
+    pl->packed_valid = false;
+    return EH_OK;
+}
+
+static int dw_refold(eh_dwconv_plan *pl, const eh_requant &q, hipStream_t stream) {
+    if (!(pl->packed_valid && q.zp_in == pl->q.zp_in && q.zp_w == pl->q.zp_w)) {
+        int rc = launch_dw_pack(pl->w_copy, pl->bias_copy, pl->w_pair, pl->bias_folded, pl->cout, pl->taps, q.zp_in,
+                                q.zp_w, stream);
+        if (rc) return rc;
+        pl->packed_valid = true;
+    }
+    pl->q = q;
+    return EH_OK;
+}
+
+int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
+                        const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan pointer");
+    *plan = nullptr;
+    int rc = check_desc_common(desc);
+    if (rc) return rc;
+    if ((rc = check_requant(q))) return rc;
+    EH_REQUIRE(desc->dil_h > 0 && desc->dil_w > 0, "bad dilation");
+    EH_REQUIRE(desc->depth_multiplier > 0, "bad depth multiplier %d", desc->depth_multiplier);
+    EH_REQUIRE(desc->cout == desc->c * desc->depth_multiplier, "depthwise cout %d != c %d * depth multiplier %d", desc->cout,
+               desc->c, desc->depth_multiplier);
+    EH_REQUIRE(desc->weight_layout == EH_W_OIHW, "depthwise weights are [C*dm][1][kh][kw]");
+    eh_dwconv_plan *pl = new (std::nothrow) eh_dwconv_plan();
+    EH_REQUIRE(pl != nullptr, "out of host memory");
+    pl->d = *desc;
+    pl->ho = eh_conv_out_dim(desc->h, desc->pad_t, desc->pad_b, desc->kh, desc->dil_h, desc->stride_h);
+    pl->wo = eh_conv_out_dim(desc->w, desc->pad_l, desc->pad_r, desc->kw, desc->dil_w, desc->stride_w);
+    pl->cout = desc->cout;
+    pl->taps = desc->kh * desc->kw;
+    if (pl->ho <= 0 || pl->wo <= 0) {
+        delete pl;
+        set_error("depthwise output is empty");
+        return EH_INVALID_PARAMS;
+    }
+    hipStream_t s = as_stream(stream);
+    rc = dev_alloc(&pl->w_copy, (size_t)pl->cout * pl->taps);
+    if (!rc) rc = dev_alloc(&pl->bias_copy, (size_t)pl->cout);
+    if (!rc) rc = dev_alloc(&pl->w_pair, (size_t)((pl->taps + 1) / 2) * pl->cout);
+    if (!rc) rc = dev_alloc(&pl->bias_folded, (size_t)pl->cout + 4);
+    if (!rc) rc = dw_set_weights(pl, weight, bias, s);
+    if (!rc) rc = dw_refold(pl, *q, s);
+    if (rc) {
+        dw_release(pl);
+        delete pl;
+        return rc;
+    }
+    *plan = pl;
+    return EH_OK;
+}
+
+int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    int rc = check_requant(q);
+    if (rc) return rc;
+    if ((rc = dw_set_weights(plan, weight, bias, as_stream(stream)))) return rc;
+    return dw_refold(plan, *q, as_stream(stream));
+}
+
+int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    int rc = check_requant(q);
+    if (rc) return rc;
+    const eh_conv_desc &d = plan->d;
+    if (d.n == 0) return EH_OK;
+    EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
+    hipStream_t s = as_stream(stream);
+    if ((rc = dw_refold(plan, *q, s))) return rc;
+    DwProblem p;
+    p.in = static_cast<const uint8_t *>(input);
+    p.w = plan->w_copy;
+    p.bias = plan->bias_copy;
+    p.w_pair = plan->w_pair;
+    p.bias_folded = plan->bias_folded;
+    p.out = static_cast<uint8_t *>(output);
+    p.n = d.n;
+    p.c = d.c;
+    p.h = d.h;
+    p.w_ = d.w;
+    p.cout = plan->cout;
+    p.dm = d.depth_multiplier;
+    p.kh = d.kh;
+    p.kw = d.kw;
+    p.stride_h = d.stride_h;
+    p.stride_w = d.stride_w;
+    p.pad_t = d.pad_t;
+    p.pad_l = d.pad_l;
+    p.dil_h = d.dil_h;
+    p.dil_w = d.dil_w;
+    p.ho = plan->ho;
+    p.wo = plan->wo;
+    p.zp_in = q->zp_in;
+    p.zp_w = q->zp_w;
+    p.rq = make_requant_dev(*q);
+    return d.layout == EH_NHWC ? launch_dwconv_nhwc(p, s) : launch_dwconv_nchw(p, s);
+}
+
+int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan) {
+    if (plan) {
+        dw_release(plan);
+        delete plan;
+    }
+    return EH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,150 @@
+// Internal declarations shared by the translation units of libedenhip.so.
+// gfx950 (MI355X) only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "eden_hip.h"
+
+namespace eh {
+
+// ---------------------------------------------------------------- errors
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+int hip_fail(hipError_t e, const char *what);  // records the text, returns EH_DEVICE_FAILURE
+
+#define EH_HIP(call)                                          \
+    do {                                                      \
+        hipError_t eh_e_ = (call);                            \
+        if (eh_e_ != hipSuccess) return ::eh::hip_fail(eh_e_, #call); \
+    } while (0)
+
+#define EH_REQUIRE(cond, ...)               \
+    do {                                    \
+        if (!(cond)) {                      \
+            ::eh::set_error(__VA_ARGS__);   \
+            return EH_INVALID_PARAMS;       \
+        }                                   \
+    } while (0)
+
+// ---------------------------------------------------------------- requant
+// Integer requantization as the reference's generic kernels do it
+// (gpu/common/CLKernels.hpp:120-170): saturating rounding doubling high mul,
+// rounding divide by a power of two, output zero point, activation clamp.
+struct RequantDev {
+    int32_t multiplier;
+    int32_t left_shift;
+    int32_t right_shift;
+    int32_t zp_out;
+    int32_t act_min;
+    int32_t act_max;
+};
+
+__device__ __forceinline__ int32_t requant_core(int32_t acc, const RequantDev &r) {
+    // x * (1 << ls) wraps like the int32 multiply of the reference kernels
+    const int32_t x = (int32_t)((uint32_t)acc << r.left_shift);
+    // (ab + nudge) / 2^31 with nudge = ab >= 0 ? 2^30 : 1 - 2^30 and C truncation
+    // is floor((ab + 2^30) / 2^31) for every ab; the multiplier is never
+    // INT32_MIN (the host rejects negative multipliers), so no saturation case.
+    const int64_t ab = (int64_t)x * (int64_t)r.multiplier;
+    const int32_t v = (int32_t)((ab + (1ll << 30)) >> 31);
+    const int32_t mask = (int32_t)((1u << r.right_shift) - 1u);
+    const int32_t rem = v & mask;
+    const int32_t thr = (mask >> 1) + (v < 0 ? 1 : 0);
+    return (v >> r.right_shift) + (rem > thr ? 1 : 0);
+}
+
+__device__ __forceinline__ uint32_t requant_u8(int32_t acc, const RequantDev &r) {
+    int32_t v = requant_core(acc, r) + r.zp_out;
+    v = v < r.act_min ? r.act_min : v;
+    v = v > r.act_max ? r.act_max : v;
+    return (uint32_t)v;
+}
+
+inline RequantDev make_requant_dev(const eh_requant &q) {
+    RequantDev r;
+    r.multiplier = q.multiplier;
+    r.left_shift = q.shift > 0 ? q.shift : 0;
+    r.right_shift = q.shift > 0 ? 0 : -q.shift;
+    r.zp_out = q.zp_out;
+    r.act_min = q.act_min;
+    r.act_max = q.act_max;
+    return r;
+}
+
+int check_requant(const eh_requant *q);
+
+// ---------------------------------------------------------------- implicit GEMM
+// One row of the k-table describes one load unit (VEC bytes) of the reduction
+// axis: where it sits relative to the top-left input pixel of an output pixel.
+struct KUnit {
+    int32_t offset;  // (dy * W + dx) * Cin + c, in bytes
+    int16_t dy;
+    int16_t dx;
+};
+
+struct GemmProblem {
+    const uint8_t *a;     // activations: NHWC image or [M][K] matrix
+    const int8_t *b;      // packed weights [n_pad][k_pad], value = w - 128
+    const int32_t *bias;  // [n_pad] bias with the zero-point terms folded in
+    const KUnit *ktab;    // [k_pad / vec]
+    uint8_t *out;
+    int32_t m, n;           // GEMM extents (n = output channels)
+    int32_t k, k_pad;       // real and padded reduction length
+    int32_t vec;            // bytes per load unit of A: 16, 4 or 1
+    // input geometry: row m -> (img, oy, ox) over (ho, wo); top-left tap at
+    // (oy * stride_h + y_base, ox * stride_w + x_base)
+    int32_t h, w, cin;
+    int32_t ho, wo;
+    int32_t stride_h, stride_w, y_base, x_base;
+    // output addressing: ((img * out_h + oy * out_sy + out_y0) * out_w + ox * out_sx + out_x0) * ldc + col
+    int32_t out_h, out_w, out_sy, out_sx, out_y0, out_x0, ldc;
+    int32_t zw;        // zp_w - 128: coefficient of the per-row activation sum
+    uint32_t fill;     // input zero point replicated in 4 bytes (value of an out-of-image tap)
+    RequantDev rq;
+};
+
+int launch_igemm(const GemmProblem &p, hipStream_t stream);
+// tile extents the launcher will pick for (m, n): packed weights are padded to them
+int igemm_n_tile(int32_t m, int32_t n, int32_t k);
+
+// ---------------------------------------------------------------- packing
+struct PackProblem {
+    const uint8_t *w;      // source weights (uint8)
+    const int32_t *bias;   // source bias [n] or null
+    int8_t *b;             // [n_pad][k_pad]
+    int32_t *colsum;       // [n_pad]  sum_k (w - 128)
+    int32_t n, n_pad, cin, taps, k, k_pad;
+    // source index of (out channel o, in channel c, tap t) = o*so + c*sc + tap_off[t]
+    int64_t so, sc;
+    const int32_t *tap_off;  // device [taps]
+};
+int launch_pack_weights(const PackProblem &p, hipStream_t stream);
+// folded[n] = bias[n] - za * colsum[n] + k * za * zw   (za = zp_in - 128, zw = zp_w - 128)
+int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad,
+                     int32_t k, int32_t zp_in, int32_t zp_w, hipStream_t stream);
+
+// ---------------------------------------------------------------- depthwise
+struct DwProblem {
+    const uint8_t *in;
+    const uint8_t *w;            // raw weights [cout][kh*kw] (uint8)
+    const int32_t *bias;         // raw bias [cout] or null
+    const int32_t *w_pair;       // [ceil(taps/2)][cout]: (w[2p]-zp_w) | (w[2p+1]-zp_w) << 16 as int16 halves
+    const int32_t *bias_folded;  // [cout]: bias - zp_in * sum_t (w - zp_w)
+    uint8_t *out;
+    int32_t n, c, h, w_, cout, dm;
+    int32_t kh, kw, stride_h, stride_w, pad_t, pad_l, dil_h, dil_w;
+    int32_t ho, wo;
+    int32_t zp_in, zp_w;
+    RequantDev rq;
+};
+int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
+                   int32_t taps, int32_t zp_in, int32_t zp_w, hipStream_t stream);
+int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream);
+int launch_dwconv_nchw(const DwProblem &p, hipStream_t stream);
+
+// ---------------------------------------------------------------- layout
+int launch_nchw2nhwc(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);
+int launch_nhwc2nchw(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);
+
+}  // namespace eh

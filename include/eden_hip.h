@@ -1,0 +1,182 @@
+/*
+ * eden_hip.h — C ABI of the MI355X (gfx950) backend for the quantized operator
+ * path of the EDEN/ENN userdriver: Convolution, DepthwiseConvolution,
+ * FullyConnected and Deconvolution on asymmetric uint8 tensors with int32 bias
+ * and fixed-point requantization, plus layout conversion and device buffers.
+ *
+ * The reference has no C ABI: its operator classes call the OpenCL runtime
+ * directly.  Each entry point below names the reference interface it stands in
+ * for (paths relative to the reference repository root).  The C++ operator
+ * classes under cl-eden-kernel_amd/host/ are the only intended callers.
+ *
+ * Conventions: every function returns EH_OK (0) or a negative eh_status; no
+ * exceptions and no C++ types cross this boundary; device pointers are plain
+ * `void *` owned by the caller unless a plan allocated them; `stream` is a
+ * hipStream_t passed as `void *` (NULL = the default stream); all launches are
+ * asynchronous on that stream.  eh_last_error() gives the text of the last
+ * failure on the calling thread.
+ */
+#ifndef EDEN_HIP_H_
+#define EDEN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum eh_status {
+    EH_OK = 0,
+    EH_FAILURE = -1,        /* Status::FAILURE        (operator_interfaces/common/Common.hpp:113-119) */
+    EH_DEVICE_FAILURE = -2, /* Status::CL_FAILURE: the device runtime reported an error               */
+    EH_INVALID_PARAMS = -3  /* Status::INVALID_PARAMS                                                  */
+} eh_status;
+
+/* ActivationInfo::ActivationType (operator_interfaces/common/ActivationInfo.hpp:5-12) */
+typedef enum eh_activation { EH_ACT_NONE = 0, EH_ACT_RELU = 1, EH_ACT_RELU1 = 2, EH_ACT_RELU6 = 3 } eh_activation;
+
+/* DataOrder (operator_interfaces/common/Common.hpp:20-25) */
+typedef enum eh_layout { EH_NCHW = 0, EH_NHWC = 1 } eh_layout;
+
+/* Weight element order.  OIHW is the reference's default [Cout][Cin/g][kh][kw];
+ * OHWI is its androidNN order [Cout][kh][kw][Cin]
+ * (gpu/operators/cl_optimized_impls/CLDeconvolutionQuantized.cpp:39-46);
+ * IOHW is the deconvolution order [Cin][Cout/g][kh][kw] (gpu/op_test/deconv_guard.h:53-69). */
+typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh_weight_layout;
+
+/* Integer requantization parameters of one operator execution: what
+ * CLGEMMConvolutionQuantized::execute derives from its tensors
+ * (gpu/operators/cl_optimized_impls/CLGEMMConvolutionQuantized.cpp:137-171). */
+typedef struct eh_requant {
+    int32_t zp_in;      /* input tensor zero point, 0..255  */
+    int32_t zp_w;       /* weight tensor zero point, 0..255 */
+    int32_t zp_out;     /* output tensor zero point         */
+    int32_t multiplier; /* Q31 significand, >= 0            */
+    int32_t shift;      /* > 0 left shift, < 0 right shift  */
+    int32_t act_min;    /* clamp range in the quantized domain */
+    int32_t act_max;
+} eh_requant;
+
+/* Geometry of a convolution-like operator.  Input dims are (n, c, h, w) whatever
+ * the memory order; `layout` says how input and output bytes are ordered.
+ * Mirrors ConvolutionParameters / DepthwiseConvolutionParameters /
+ * DeconvolutionParameters (gpu/operators/CLConvolution.hpp:31-44,
+ * CLDepthwiseConvolution.hpp:18-29, CLDeconvolution.hpp:20-31). */
+typedef struct eh_conv_desc {
+    int32_t n, c, h, w;
+    int32_t cout;
+    int32_t kh, kw;
+    int32_t stride_h, stride_w;
+    int32_t pad_t, pad_b, pad_l, pad_r;
+    int32_t dil_h, dil_w;
+    int32_t groups;           /* convolution / deconvolution */
+    int32_t depth_multiplier; /* depthwise only              */
+    int32_t layout;           /* eh_layout of input and output */
+    int32_t weight_layout;    /* eh_weight_layout              */
+} eh_conv_desc;
+
+/* ---- host arithmetic (pure CPU, usable without a GPU) ------------------- */
+
+/* QuantizeMultiplier (gpu/operators/cl_quantized_utils/QuantizationUtil.cpp:8-21) */
+void eh_quantize_multiplier(double real_multiplier, int32_t *quantized_multiplier, int32_t *shift);
+/* GetQuantizedConvolutionMultipler (gpu/operators/cl_quantized_utils/KernelUtil.cpp:7-25):
+ * EH_FAILURE leaves *multiplier untouched. */
+int eh_conv_multiplier(float input_scale, float filter_scale, float bias_scale, float output_scale, double *multiplier);
+/* CalculateActivationRangeUint8 (gpu/operators/cl_quantized_utils/KernelUtil.cpp:27-60) */
+void eh_act_range_u8(int activation, float scale, int32_t zero_point, int32_t *act_min, int32_t *act_max);
+/* The whole derivation an operator's execute() performs, including the
+ * reference's behaviour of continuing with multiplier 0 when the bias scale
+ * does not match (CLGEMMConvolutionQuantized.cpp:163-166). */
+void eh_make_requant(float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp, float bias_scale,
+                     float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out);
+/* output extents: CLConvolution.cpp:99-104 and CLDeconvolution.cpp:82-87 */
+int32_t eh_conv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t dilation, int32_t stride);
+int32_t eh_deconv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t stride);
+
+/* ---- runtime and device buffers ------------------------------------------
+ * Stand in for CLRuntime::initialize / allocBuffer / releaseBuffer /
+ * writeBuffer / readBuffer / copyBuffer and clFinish
+ * (gpu/common/CLRuntime.cpp:1339-1372,1409-1416; CLRuntime.hpp:59-110). */
+int eh_init(int device);
+int eh_device_name(char *dst, size_t cap);
+int eh_malloc(void **ptr, size_t bytes);             /* zero-initialised, 256-byte aligned */
+int eh_free(void *ptr);
+int eh_memset(void *ptr, int value, size_t bytes, void *stream);
+int eh_h2d(void *dst, const void *src, size_t bytes, void *stream);
+int eh_d2h(void *dst, const void *src, size_t bytes, void *stream);
+int eh_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int eh_stream_sync(void *stream);
+const char *eh_last_error(void);
+
+/* ---- layout conversion -----------------------------------------------------
+ * nchw2nhwc_uint8 / nhwc2nchw_uint8 (gpu/common/CLKernels.hpp:429-491) as
+ * driven by CLRuntime::NCHW2NHWC / NHWC2NCHW (gpu/common/CLRuntime.cpp:1477-1619). */
+int eh_transpose_u8_nchw2nhwc(const void *src, void *dst, int32_t n, int32_t c, int32_t h, int32_t w, void *stream);
+int eh_transpose_u8_nhwc2nchw(const void *src, void *dst, int32_t n, int32_t c, int32_t h, int32_t w, void *stream);
+
+/* ---- operators -------------------------------------------------------------
+ * A plan owns everything initialize() prepares once: packed int8 weights, the
+ * bias with the zero-point terms folded in, and scratch.  `*_plan` reads the
+ * weights and bias from device memory on `stream`; `*_run` enqueues one
+ * execution.  Passing a requant whose zero points differ from the plan's
+ * re-folds the bias first (the reference reads quantization parameters from
+ * the tensors on every execute).  `*_repack` is the weights-as-input case:
+ * the reference re-packs non-constant weights on every execute. */
+typedef struct eh_conv_plan eh_conv_plan;
+typedef struct eh_dwconv_plan eh_dwconv_plan;
+typedef struct eh_fc_plan eh_fc_plan;
+typedef struct eh_deconv_plan eh_deconv_plan;
+
+/* CLConvolution::initialize / execute / release, uint8 branch
+ * (gpu/operators/CLConvolution.cpp:139-218,458-550) with the work of
+ * CLGEMMConvolutionQuantized and CLQuantizedDirectConvolution
+ * (gpu/operators/cl_optimized_impls/CLGEMMConvolutionQuantized.cpp:33-280,
+ * CLQuantizedDirectConvolution.cpp:30-249) and their kernels. */
+int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
+                      const eh_requant *q, void *stream);
+int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
+int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
+int eh_conv2d_u8_destroy(eh_conv_plan *plan);
+
+/* CLDepthwiseConvolution::initialize / execute / release, uint8 branch
+ * (gpu/operators/CLDepthwiseConvolution.cpp:88-200,388-425;
+ * cl_optimized_impls/CLDepthwiseConvolutionQuantized.cpp:82-674). */
+int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
+                        const eh_requant *q, void *stream);
+int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
+int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
+int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
+
+/* CLFullyConnected::initialize / execute / release (gpu/operators/CLFullyConnected.cpp:22-150):
+ * input [m][k], weight [n][k], bias [n], output [m][n]
+ * (gpu/op_test/fullyconnected_test.cpp:93-105), computed in the convolution's
+ * integer pipeline rather than the reference's float detour. */
+int eh_fc_u8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, const void *weight, const void *bias,
+                  const eh_requant *q, void *stream);
+int eh_fc_u8_repack(eh_fc_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
+int eh_fc_u8_run(eh_fc_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
+int eh_fc_u8_destroy(eh_fc_plan *plan);
+
+/* CLDeconvolution::initialize / execute / release, uint8 branch
+ * (gpu/operators/CLDeconvolution.cpp:36-272;
+ * cl_optimized_impls/CLDeconvolutionQuantized.cpp:18-288).  Output extent is
+ * in*stride + k - stride - pads. */
+int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
+                        const eh_requant *q, void *stream);
+int eh_deconv2d_u8_repack(eh_deconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
+int eh_deconv2d_u8_run(eh_deconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
+int eh_deconv2d_u8_destroy(eh_deconv_plan *plan);
+
+/* Timing aid for harnesses: runs `fn`-independent HIP event pairs on `stream`.
+ * eh_event_* wrap hipEventCreate / Record / ElapsedTime so that a harness can
+ * time the stream the kernels are launched on without linking HIP itself. */
+int eh_event_create(void **event);
+int eh_event_record(void *event, void *stream);
+int eh_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronises on `stop` */
+int eh_event_destroy(void *event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EDEN_HIP_H_ */

@@ -1,0 +1,96 @@
+"""Shared helpers of the GPU parity tests: run one operator through the C ABI and
+through the CPU oracle on the same seeded tensors."""
+import importlib
+
+import numpy as np
+
+import oracle_lib as O
+
+eden = importlib.import_module("cl-eden-kernel_amd")
+synth = importlib.import_module("cl-eden-kernel_amd.synth")
+
+
+def to_eh_requant(q):
+    return eden.Requant(*q.as_tuple())
+
+
+def assert_same_host_quant(args, kwargs):
+    """The product's own parameter derivation must agree with the oracle's."""
+    a = eden.make_requant(*args, **kwargs).as_tuple()
+    b = O.make_quant(*args, **kwargs).as_tuple()
+    assert a == b, (a, b)
+
+
+def gpu_conv(x_nchw, w, bias, s, q, layout=eden.NCHW, weight_layout=eden.W_OIHW, runs=1):
+    """x_nchw: uint8 NCHW array; w in OIHW; returns NCHW uint8 output of the GPU path."""
+    ho, wo = O.conv_out_hw(s)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, (s.stride_h, s.stride_w),
+                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), s.groups, 1, layout, weight_layout)
+    x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
+    w_dev = w if weight_layout == eden.W_OIHW else w.transpose(0, 2, 3, 1)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), eden.DeviceBuffer(host=bias)
+    d_o = eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
+    plan = eden.ConvPlan(desc, d_w, d_b, q)
+    for _ in range(runs):
+        plan.run(d_x, d_o, q)
+    if layout == eden.NCHW:
+        out = d_o.download((s.n, s.cout, ho, wo))
+    else:
+        out = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+    plan.destroy()
+    return np.ascontiguousarray(out)
+
+
+def gpu_dwconv(x_nchw, w, bias, s, q, layout=eden.NCHW):
+    ho, wo = O.conv_out_hw(s)
+    cout = s.c * max(s.dm, 1)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, cout, s.kh, s.kw, (s.stride_h, s.stride_w),
+                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), 1, max(s.dm, 1), layout, eden.W_OIHW)
+    x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=bias)
+    d_o = eden.DeviceBuffer(nbytes=s.n * cout * ho * wo)
+    plan = eden.DwConvPlan(desc, d_w, d_b, q)
+    plan.run(d_x, d_o, q)
+    if layout == eden.NCHW:
+        out = d_o.download((s.n, cout, ho, wo))
+    else:
+        out = d_o.download((s.n, ho, wo, cout)).transpose(0, 3, 1, 2)
+    plan.destroy()
+    return np.ascontiguousarray(out)
+
+
+def gpu_deconv(x_nchw, w_iohw, bias, s, q, layout=eden.NCHW, weight_layout=eden.W_IOHW):
+    ho, wo = O.deconv_out_hw(s)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, (s.stride_h, s.stride_w),
+                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (1, 1), s.groups, 1, layout, weight_layout)
+    x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
+    w_dev = w_iohw if weight_layout == eden.W_IOHW else w_iohw.transpose(1, 2, 3, 0)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), eden.DeviceBuffer(host=bias)
+    d_o = eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
+    plan = eden.DeconvPlan(desc, d_w, d_b, q)
+    plan.run(d_x, d_o, q)
+    if layout == eden.NCHW:
+        out = d_o.download((s.n, s.cout, ho, wo))
+    else:
+        out = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+    plan.destroy()
+    return np.ascontiguousarray(out)
+
+
+def gpu_fc(a, w, bias, q):
+    m, k = a.shape
+    n = w.shape[0]
+    d_a, d_w, d_b = eden.DeviceBuffer(host=a), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=bias)
+    d_o = eden.DeviceBuffer(nbytes=m * n)
+    plan = eden.FcPlan(m, k, n, d_w, d_b, q)
+    plan.run(d_a, d_o, q)
+    out = d_o.download((m, n))
+    plan.destroy()
+    return out
+
+
+def diff_report(got, want):
+    bad = np.argwhere(got != want)
+    return "%d of %d differ; first at %s: got %s want %s" % (
+        len(bad), got.size, bad[0].tolist() if len(bad) else None,
+        got[tuple(bad[0])] if len(bad) else None, want[tuple(bad[0])] if len(bad) else None)

@@ -1,0 +1,98 @@
+"""CPU-side checks of the C ABI library: it loads, exports every symbol the
+header declares, and its host arithmetic (no GPU involved) matches the golden
+vectors written from the reference's own code and the oracle."""
+import ctypes as C
+import json
+import os
+import re
+
+import numpy as np
+
+import oracle_lib as O
+from harness import eden
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLD = json.load(open(os.path.join(ROOT, "tests", "golden", "arith_vectors.json")))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "eden_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(eh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = eden.load()
+    names = declared_symbols()
+    assert len(names) >= 35
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(names) == set(eden.EXPORTS), set(names) ^ set(eden.EXPORTS)
+
+
+def test_product_host_arithmetic_matches_golden_vectors():
+    lib = eden.load()
+    for mhex, q, s in GOLD["quantize_multiplier"]:
+        qq, ss = C.c_int32(), C.c_int32()
+        lib.eh_quantize_multiplier(float.fromhex(mhex), C.byref(qq), C.byref(ss))
+        assert (qq.value, ss.value) == (q, s)
+    for a, b, c, d, status, mhex in GOLD["conv_multiplier"]:
+        m = C.c_double(-1.0)
+        st = lib.eh_conv_multiplier(float.fromhex(a), float.fromhex(b), float.fromhex(c), float.fromhex(d), C.byref(m))
+        assert (st != 0) == (status != 0) and m.value.hex() == mhex
+    for act, shex, zp, lo, hi in GOLD["act_range_u8"]:
+        l, h = C.c_int32(), C.c_int32()
+        lib.eh_act_range_u8(act, float.fromhex(shex), zp, C.byref(l), C.byref(h))
+        assert (l.value, h.value) == (lo, hi)
+
+
+def test_make_requant_matches_oracle_and_handles_bias_scale_mismatch():
+    rng = np.random.default_rng(21)
+    for _ in range(500):
+        s_in, s_w, s_out = [float(np.float32(x)) for x in np.exp(rng.uniform(np.log(1e-3), np.log(2.0), 3))]
+        zi, zw, zo = [int(v) for v in rng.integers(0, 256, 3)]
+        act, en = int(rng.integers(0, 4)), bool(rng.integers(0, 2))
+        a = eden.make_requant(s_in, zi, s_w, zw, s_out, zo, act, en).as_tuple()
+        b = O.make_quant(s_in, zi, s_w, zw, s_out, zo, act, en).as_tuple()
+        assert a == b
+    q = eden.make_requant(0.5, 0, 0.5, 0, 1.0, 7, s_bias=1.0)  # bias scale != s_in * s_w
+    assert (q.multiplier, q.shift) == (0, 0)
+
+
+def test_output_dim_formulas_match_oracle():
+    lib = eden.load()
+    rng = np.random.default_rng(22)
+    for _ in range(300):
+        i, pa, pb, k, d, s = [int(v) for v in (rng.integers(1, 300), rng.integers(0, 4), rng.integers(0, 4),
+                                                rng.integers(1, 8), rng.integers(1, 3), rng.integers(1, 4))]
+        assert lib.eh_conv_out_dim(i, pa, pb, k, d, s) == O.lib.eo_conv_out_dim(i, pa, pb, k, d, s)
+        assert lib.eh_deconv_out_dim(i, pa, pb, k, s) == O.lib.eo_deconv_out_dim(i, pa, pb, k, s)
+
+
+def test_parameter_errors_are_reported_without_a_gpu():
+    lib = eden.load()
+    plan = C.c_void_p()
+    desc = eden.conv_desc(1, 4, 4, 4, 4, 3, 3)
+    bad_q = eden.Requant(0, 0, 0, -5, 0, 0, 255)  # negative multiplier
+    rc = lib.eh_conv2d_u8_plan(C.byref(plan), C.byref(desc), None, None, C.byref(bad_q), None)
+    assert rc == -3 and b"multiplier" in lib.eh_last_error()
+    q = eden.Requant(0, 0, 0, 1 << 30, 1, 0, 255)
+    desc = eden.conv_desc(1, 4, 4, 4, 6, 3, 3, groups=4)  # groups do not divide cout
+    assert lib.eh_conv2d_u8_plan(C.byref(plan), C.byref(desc), None, None, C.byref(q), None) == -3
+    desc = eden.conv_desc(1, 4, 4, 4, 9, 3, 3, dm=2)  # cout != c * dm
+    assert lib.eh_dwconv2d_u8_plan(C.byref(plan), C.byref(desc), None, None, C.byref(q), None) == -3
+    assert lib.eh_fc_u8_plan(C.byref(plan), 4, 0, 4, None, None, C.byref(q), None) == -3
+    q = eden.Requant(0, 0, 0, 1 << 30, -40, 0, 255)  # shift out of range
+    assert lib.eh_fc_u8_plan(C.byref(plan), 4, 4, 4, None, None, C.byref(q), None) == -3
+    q = eden.Requant(300, 0, 0, 1 << 30, 0, 0, 255)  # zero point outside uint8
+    assert lib.eh_fc_u8_plan(C.byref(plan), 4, 4, 4, None, None, C.byref(q), None) == -3
+
+
+def test_synthetic_generators_match_the_c_harness():
+    from harness import synth
+    assert np.array_equal(synth.fill_u8((4097,), 0xEDE2), O.fill_u8((4097,), 0xEDE2))
+    assert np.array_equal(synth.fill_u8((333,), 9, 3, 17), O.fill_u8((333,), 9, 3, 17))
+    assert np.array_equal(synth.fill_i32((999,), 0xEDE3, -1000, 1000), O.fill_i32((999,), 0xEDE3, -1000, 1000))
+    a = synth.fill_u8_normal((50000,), 0xEDE4, 128, 20)
+    assert np.array_equal(a, O.fill_u8_normal((50000,), 0xEDE4, 128, 20))
+    assert abs(a.mean() - 128) < 0.5 and abs(a.std() - 20) < 0.5

@@ -1,0 +1,379 @@
+"""GPU parity: every operator, called through the C ABI, must reproduce the CPU
+oracle bit for bit (uint8 outputs; integer work, so the tolerance is zero)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from harness import (diff_report, eden, gpu_conv, gpu_deconv, gpu_dwconv, gpu_fc, synth, to_eh_requant)
+
+pytestmark = pytest.mark.gpu
+
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
+SEED = 0xEDE2
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    eden.init(0)
+    print("device:", eden.device_name(), flush=True)
+
+
+def quant(s_in=0.02, zp_in=128, s_w=0.005, zp_w=120, s_out=0.05, zp_out=0, act=O.ACT_NONE, en=False):
+    q = O.make_quant(s_in, zp_in, s_w, zp_w, s_out, zp_out, act, en)
+    assert eden.make_requant(s_in, zp_in, s_w, zp_w, s_out, zp_out, act, en).as_tuple() == q.as_tuple()
+    return q
+
+
+def centred_quant(acc, zp_in, zp_w, act_min=0, act_max=255):
+    """Integer requant parameters that spread the given accumulators over the uint8 range
+    (about 40 output steps per standard deviation, mean at 128), so that a parity case
+    exercises rounding and both clamps instead of a saturated constant."""
+    sd = float(acc.std()) or 1.0
+    qm, sh = O.quantize_multiplier(40.0 / sd)
+    zp_out = int(128 - round(float(acc.mean()) * 40.0 / sd))
+    return O.raw_quant(zp_in=zp_in, zp_w=zp_w, zp_out=zp_out, multiplier=qm, shift=sh, act_min=act_min, act_max=act_max)
+
+
+def conv_tensors(s, seed, w_normal=False):
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), seed)
+    wshape = (s.cout, s.c // s.groups, s.kh, s.kw)
+    w = synth.fill_u8_normal(wshape, seed + 1, 128, 20) if w_normal else synth.fill_u8(wshape, seed + 1)
+    b = synth.fill_i32((s.cout,), seed + 2, -1000, 1000)
+    return x, w, b
+
+
+# ----------------------------------------------------------------- fully connected
+
+FC_CASES = [
+    # m, k, n, zp_a, zp_w
+    (1, 64, 16, 3, 128),
+    (7, 37, 11, 3, 128),       # byte-granular loads, ragged tiles
+    (33, 100, 70, 250, 0),     # 4-byte loads, extreme zero points
+    (64, 64, 64, 0, 255),
+    (130, 256, 200, 128, 128),  # both shifted zero points vanish
+    (256, 1024, 512, 77, 201),
+    (300, 4096, 96, 3, 130),
+    (5, 4100, 1000, 10, 20),   # classifier-like: k not a multiple of 64, n = 1000
+]
+
+
+@pytest.mark.parametrize("m,k,n,zp_a,zp_w", FC_CASES)
+def test_fc_matches_oracle(m, k, n, zp_a, zp_w):
+    print("fc", m, k, n, zp_a, zp_w, flush=True)
+    a = synth.fill_u8((m, k), SEED + m)
+    w = synth.fill_u8((n, k), SEED + k)
+    b = synth.fill_i32((n,), SEED + n, -1000, 1000)
+    _, acc = O.fc(a, w, b, O.raw_quant(zp_in=zp_a, zp_w=zp_w), want_acc=True)
+    q = centred_quant(acc, zp_a, zp_w)
+    want = O.fc(a, w, b, q)
+    got = gpu_fc(a, w, b, to_eh_requant(q))
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 10  # the case exercises the requant range, not a saturated constant
+
+
+def test_fc_config2_full_size():
+    """M=256, K=4096, N=4096; uint8 activations zp 3; weights clip(N(128,20)) zp 128; scales 0.01/0.002/0.08."""
+    m, k, n = 256, 4096, 4096
+    print("fc config2", flush=True)
+    a = synth.fill_u8((m, k), SEED + 16 * 2 + 0)
+    w = synth.fill_u8_normal((n, k), SEED + 16 * 2 + 1, 128, 20)
+    b = synth.fill_i32((n,), SEED + 16 * 2 + 2, -1000, 1000)
+    q = quant(0.01, 3, 0.002, 128, 0.08, 0)
+    assert (q.multiplier, q.shift) == (1099511680, -11)
+    want, acc = O.fc(a, w, b, q, want_acc=True)
+    got = gpu_fc(a, w, b, to_eh_requant(q))
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert O.count_fastpath_overflow(acc, q) == 0
+    assert len(np.unique(want)) > 20
+
+
+@pytest.mark.parametrize("kat", KATS["fc"], ids=lambda k: k["name"])
+def test_fc_reference_kat_on_gpu(kat):
+    zp_a = 10
+    a = (np.array(kat["input"]) + zp_a).astype(np.uint8).reshape(kat["m"], kat["k"])
+    w = np.array(kat["weight"], np.uint8).reshape(kat["n"], kat["k"])
+    q = O.raw_quant(zp_in=zp_a)
+    got = gpu_fc(a, w, np.array(kat["bias"], np.int32), to_eh_requant(q))
+    assert got.reshape(-1).tolist() == kat["expect"]
+
+
+# ----------------------------------------------------------------- convolution
+
+CONV_CASES = [
+    # n, c, h, w, cout, kh, kw, kwargs
+    dict(n=1, c=64, h=56, w=56, cout=64, kh=3, kw=3, pad=(1, 1, 1, 1)),                    # config 1 shape
+    dict(n=2, c=3, h=17, w=19, cout=8, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),       # 3 channels: byte loads
+    dict(n=2, c=24, h=14, w=14, cout=144, kh=1, kw=1),                                       # pointwise expand, 4-byte loads
+    dict(n=1, c=32, h=9, w=11, cout=20, kh=5, kw=3, pad=(2, 2, 1, 1), dil=(1, 2)),          # dilation, cout % 16 != 0
+    dict(n=3, c=16, h=8, w=8, cout=24, kh=3, kw=3, stride=(1, 2), pad=(1, 1, 0, 2)),
+    dict(n=1, c=32, h=10, w=10, cout=48, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2),           # grouped
+    dict(n=1, c=12, h=6, w=6, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=3),             # grouped, 4-byte loads
+    dict(n=1, c=16, h=3, w=3, cout=16, kh=3, kw=3, pad=(3, 3, 3, 3)),                       # windows wholly in the padding
+    dict(n=4, c=128, h=7, w=7, cout=256, kh=1, kw=1),
+    dict(n=1, c=160, h=7, w=7, cout=960, kh=1, kw=1),
+]
+
+
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_conv_matches_oracle(case, layout):
+    print("conv", case, layout, flush=True)
+    s = O.conv_shape(**case)
+    x, w, b = conv_tensors(s, SEED + s.c + s.cout)
+    _, acc = O.conv2d(x, w, b, s, O.raw_quant(zp_in=131, zp_w=120), want_acc=True)
+    q = centred_quant(acc, 131, 120, act_min=20, act_max=230)
+    want = O.conv2d(x, w, b, s, q)
+    got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=layout)
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 10
+
+
+def test_conv_config1_exact_and_fastpath_census():
+    """N=1, Cin=64, 56x56, Cout=64, 3x3 s1 p1; in zp128 s0.02; w zp120 s0.005; out zp0 s0.05; ReLU."""
+    s = O.conv_shape(1, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 16 * 1)
+    q = quant(0.02, 128, 0.005, 120, 0.05, 0, O.ACT_RELU, True)
+    assert (q.multiplier, q.shift) == (1099511562, -8)
+    want, acc = O.conv2d(x, w, b, s, q, want_acc=True)
+    got = gpu_conv(x, w, b, s, to_eh_requant(q), runs=2)
+    assert np.array_equal(got, want), diff_report(got, want)
+    # the reference routes this shape to its mul_hi/rhadd kernel; that rounding is the same function
+    # unless acc << 2 overflows, which does not happen on these inputs
+    assert O.count_fastpath_overflow(acc, q) == 0
+
+
+def test_conv_ohwi_weights_equal_oihw():
+    s = O.conv_shape(2, 16, 9, 9, 32, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 5)
+    q = quant(0.02, 100, 0.005, 90, 0.04, 10)
+    want = O.conv2d(x, w, b, s, q)
+    got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC, weight_layout=eden.W_OHWI)
+    assert np.array_equal(got, want), diff_report(got, want)
+
+
+@pytest.mark.parametrize("kat", KATS["conv"], ids=lambda k: k["name"])
+def test_conv_reference_kat_on_gpu(kat):
+    n, h, w, c = kat["in_dims"]
+    cout, kh, kw, _ = kat["w_dims"]
+    x = np.array(kat["input"], np.uint8).reshape(n, h, w, c).transpose(0, 3, 1, 2)
+    wt = np.array(kat["weight"], np.uint8).reshape(cout, kh, kw, c).transpose(0, 3, 1, 2)
+    t, b, l, r = kat["pad_tblr"]
+    s = O.conv_shape(n, c, h, w, cout, kh, kw, stride=tuple(kat["stride"]), pad=(t, b, l, r))
+    q = O.raw_quant()
+    got = gpu_conv(np.ascontiguousarray(x), np.ascontiguousarray(wt), np.array(kat["bias"], np.int32), s, to_eh_requant(q))
+    on, oh, ow, oc = kat["out_dims"]
+    want = np.clip(np.array(kat["expect"]).reshape(on, oh, ow, oc).transpose(0, 3, 1, 2), 0, 255).astype(np.uint8)
+    assert np.array_equal(got, want)
+
+
+def test_requant_edge_multipliers_through_conv():
+    """Left shifts (M >= 1), M == 0 and large right shifts through the fused epilogue."""
+    s = O.conv_shape(1, 16, 6, 6, 16, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 9)
+    for m_real, zp_out in ((1.0, 128), (3.0, 128), (0.0, 9), (2.0 ** -20, 100), (0.74, 128), (1e-9, 50)):
+        qm, sh = O.quantize_multiplier(m_real)
+        q = O.raw_quant(zp_in=130, zp_w=127, zp_out=zp_out, multiplier=qm, shift=max(sh, -31))
+        if sh < -31:
+            q.multiplier, q.shift = 0, 0
+        want = O.conv2d(x, w, b, s, q)
+        got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
+        assert np.array_equal(got, want), (m_real, diff_report(got, want))
+
+
+def test_negative_half_ties_round_like_the_oracle():
+    """Accumulators chosen so that acc * M lands exactly on .5 for both signs and both rounding stages."""
+    k, n = 16, 16
+    a = np.zeros((64, k), np.uint8)
+    a[:, 0] = np.arange(64)              # a - zp_a = -32 .. 31 with zp 32
+    w = np.zeros((n, k), np.uint8)
+    w[:, 0] = 1
+    bias = np.zeros(n, np.int32)
+    for m_real in (0.5, 0.25, 0.125, 0.375):
+        qm, sh = O.quantize_multiplier(m_real)
+        q = O.raw_quant(zp_in=32, zp_w=0, zp_out=128, multiplier=qm, shift=sh)
+        want = O.fc(a, w, bias, q)
+        got = gpu_fc(a, w, bias, to_eh_requant(q))
+        assert np.array_equal(got, want), (m_real, diff_report(got, want))
+
+
+def test_plan_refolds_when_zero_points_change_and_repacks_new_weights():
+    s = O.conv_shape(1, 16, 8, 8, 16, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 11)
+    desc = eden.conv_desc(1, 16, 8, 8, 16, 3, 3, pad=(1, 1, 1, 1), layout=eden.NCHW)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+    d_o = eden.DeviceBuffer(nbytes=16 * 64)
+    q1 = quant(0.02, 128, 0.005, 120, 0.05, 0)
+    plan = eden.ConvPlan(desc, d_w, d_b, to_eh_requant(q1))
+    plan.run(d_x, d_o, to_eh_requant(q1))
+    assert np.array_equal(d_o.download((1, 16, 8, 8)), O.conv2d(x, w, b, s, q1))
+    q2 = quant(0.02, 7, 0.005, 201, 0.05, 30)  # tensors re-quantized: zero points read at execute time
+    plan.run(d_x, d_o, to_eh_requant(q2))
+    assert np.array_equal(d_o.download((1, 16, 8, 8)), O.conv2d(x, w, b, s, q2))
+    w2 = synth.fill_u8(w.shape, SEED + 99)
+    b2 = synth.fill_i32(b.shape, SEED + 98, -50, 50)
+    d_w2, d_b2 = eden.DeviceBuffer(host=w2), eden.DeviceBuffer(host=b2)
+    plan.repack(d_w2, d_b2, to_eh_requant(q2))  # weights as a run-time input
+    plan.run(d_x, d_o, to_eh_requant(q2))
+    assert np.array_equal(d_o.download((1, 16, 8, 8)), O.conv2d(x, w2, b2, s, q2))
+    plan.destroy()
+
+
+# ----------------------------------------------------------------- depthwise
+
+DW_CASES = [
+    dict(n=2, c=144, h=56, w=56, cout=144, kh=3, kw=3, stride=(2, 2), pad=(1, 1, 1, 1)),   # config 3 geometry, 2 images
+    dict(n=1, c=32, h=12, w=12, cout=32, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=8, h=9, w=7, cout=16, kh=3, kw=3, pad=(1, 1, 1, 1), dm=2),                  # depth multiplier
+    dict(n=2, c=5, h=10, w=10, cout=5, kh=5, kw=5, pad=(2, 2, 2, 2), dil=(1, 1)),           # odd channel count
+    dict(n=1, c=16, h=11, w=13, cout=16, kh=3, kw=3, stride=(1, 1), pad=(2, 2, 2, 2), dil=(2, 2)),
+    dict(n=1, c=4, h=5, w=5, cout=4, kh=2, kw=2),
+]
+
+
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("case", DW_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_depthwise_matches_oracle(case, layout):
+    print("dw", case, layout, flush=True)
+    s = O.conv_shape(**case)
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 40)
+    w = synth.fill_u8((s.cout, 1, s.kh, s.kw), SEED + 41)
+    b = synth.fill_i32((s.cout,), SEED + 42, -1000, 1000)
+    _, acc = O.dwconv2d(x, w, b, s, O.raw_quant(zp_in=37, zp_w=201), want_acc=True)
+    q = centred_quant(acc, 37, 201, act_min=10, act_max=240)
+    want = O.dwconv2d(x, w, b, s, q)
+    got = gpu_dwconv(x, w, b, s, to_eh_requant(q), layout=layout)
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 10
+
+
+@pytest.mark.parametrize("kat", KATS["depthwise"], ids=lambda k: k["name"])
+def test_depthwise_reference_kat_on_gpu(kat):
+    n, c, h, w = kat["in_dims"]
+    cout, _, kh, kw = kat["w_dims"]
+    zp_w, zp_out = 16, 40
+    x = np.array(kat["input"], np.uint8).reshape(n, c, h, w)
+    wt = (np.array(kat["weight"]) + zp_w).astype(np.uint8).reshape(cout, 1, kh, kw)
+    s = O.conv_shape(n, c, h, w, cout, kh, kw, stride=tuple(kat["stride"]), dm=kat["dm"])
+    q = O.raw_quant(zp_w=zp_w, zp_out=zp_out)
+    for layout in (eden.NCHW, eden.NHWC):
+        got = gpu_dwconv(x, wt, np.array(kat["bias"], np.int32), s, to_eh_requant(q), layout=layout)
+        assert got.reshape(-1).tolist() == [e + zp_out for e in kat["expect"]]
+
+
+def test_mobilenet_block_config3():
+    """Pointwise 24->144 (ReLU6) then depthwise 3x3 s2 p1 (ReLU6), channels-last, zero points drawn from the seed."""
+    n = 4
+    zps = synth.fill_u8((6,), SEED + 16 * 3 + 9).tolist()
+    x = synth.fill_u8((n, 24, 56, 56), SEED + 16 * 3)
+    w1 = synth.fill_u8((144, 24, 1, 1), SEED + 16 * 3 + 1)
+    b1 = synth.fill_i32((144,), SEED + 16 * 3 + 2, -1000, 1000)
+    w2 = synth.fill_u8((144, 1, 3, 3), SEED + 16 * 3 + 3)
+    b2 = synth.fill_i32((144,), SEED + 16 * 3 + 4, -1000, 1000)
+    q1 = quant(0.02, zps[0], 0.004, zps[1], 0.03, zps[2] // 4, O.ACT_RELU6, True)
+    q2 = quant(0.03, zps[2] // 4, 0.006, zps[3], 0.025, zps[4] // 4, O.ACT_RELU6, True)
+    s1 = O.conv_shape(n, 24, 56, 56, 144, 1, 1)
+    s2 = O.conv_shape(n, 144, 56, 56, 144, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1))
+    mid = O.conv2d(x, w1, b1, s1, q1)
+    want = O.dwconv2d(mid, w2, b2, s2, q2)
+    got_mid = gpu_conv(x, w1, b1, s1, to_eh_requant(q1), layout=eden.NHWC)
+    assert np.array_equal(got_mid, mid), diff_report(got_mid, mid)
+    got = gpu_dwconv(got_mid, w2, b2, s2, to_eh_requant(q2), layout=eden.NHWC)
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 1 and mid.std() > 1
+
+
+# ----------------------------------------------------------------- deconvolution
+
+DECONV_CASES = [
+    dict(n=2, c=16, h=5, w=7, cout=8, kh=4, kw=4, stride=(2, 2), pad=(1, 1, 1, 1)),
+    dict(n=1, c=6, h=4, w=4, cout=4, kh=3, kw=3, stride=(3, 3), pad=(1, 1, 1, 1), groups=2),
+    dict(n=1, c=3, h=5, w=4, cout=2, kh=2, kw=3, stride=(1, 2), pad=(0, 1, 1, 0)),
+    dict(n=1, c=32, h=6, w=6, cout=40, kh=3, kw=3, stride=(2, 2), pad=(0, 0, 0, 0)),       # kernel not a multiple of stride
+    dict(n=1, c=16, h=4, w=4, cout=16, kh=2, kw=2, stride=(3, 3), pad=(0, 0, 0, 0)),       # phases without any tap
+    dict(n=1, c=8, h=3, w=3, cout=8, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("case", DECONV_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_deconv_matches_oracle(case, layout):
+    print("deconv", case, layout, flush=True)
+    s = O.conv_shape(**case)
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 60)
+    w = synth.fill_u8((s.c, s.cout // s.groups, s.kh, s.kw), SEED + 61)
+    b = synth.fill_i32((s.cout,), SEED + 62, -1000, 1000)
+    _, acc = O.deconv2d(x, w, b, s, O.raw_quant(zp_in=131, zp_w=77), want_acc=True)
+    q = centred_quant(acc, 131, 77)
+    want = O.deconv2d(x, w, b, s, q)
+    got = gpu_deconv(x, w, b, s, to_eh_requant(q), layout=layout)
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 10
+
+
+def test_deconv_ohwi_weights():
+    s = O.conv_shape(1, 16, 5, 5, 12, 4, 4, stride=(2, 2), pad=(1, 1, 1, 1))
+    x = synth.fill_u8((1, 16, 5, 5), SEED + 63)
+    w = synth.fill_u8((16, 12, 4, 4), SEED + 64)
+    b = synth.fill_i32((12,), SEED + 65, -100, 100)
+    q = quant(0.03, 131, 0.01, 77, 0.3, 5)
+    want = O.deconv2d(x, w, b, s, q)
+    got = gpu_deconv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC, weight_layout=eden.W_OHWI)
+    assert np.array_equal(got, want), diff_report(got, want)
+
+
+def test_deconv_config4_full_size():
+    """N=8, Cin=256, 32x32 -> Cout=128, 4x4 s2 p1 -> 64x64."""
+    s = O.conv_shape(8, 256, 32, 32, 128, 4, 4, stride=(2, 2), pad=(1, 1, 1, 1))
+    x = synth.fill_u8((8, 256, 32, 32), SEED + 16 * 4)
+    w = synth.fill_u8((256, 128, 4, 4), SEED + 16 * 4 + 1)
+    b = synth.fill_i32((128,), SEED + 16 * 4 + 2, -1000, 1000)
+    q = quant(0.02, 121, 0.005, 133, 0.35, 128)
+    assert q.shift < 0
+    want = O.deconv2d(x, w, b, s, q)
+    got = gpu_deconv(x, w, b, s, to_eh_requant(q))
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 5
+
+
+# ----------------------------------------------------------------- layout
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (2, 3, 5, 7), (1, 64, 56, 56), (3, 24, 17, 9), (2, 144, 28, 28),
+                                   (1, 1000, 1, 1), (2, 130, 1, 67)])
+def test_layout_conversion(shape):
+    n, c, h, w = shape
+    x = synth.fill_u8(shape, SEED + 70)
+    d_x = eden.DeviceBuffer(host=x)
+    d_y = eden.DeviceBuffer(nbytes=x.size)
+    d_z = eden.DeviceBuffer(nbytes=x.size)
+    lib = eden.load()
+    eden.check(lib.eh_transpose_u8_nchw2nhwc(d_x.ptr, d_y.ptr, n, c, h, w, None))
+    y = d_y.download((n, h, w, c))
+    assert np.array_equal(y, O.nchw2nhwc(x))
+    eden.check(lib.eh_transpose_u8_nhwc2nchw(d_y.ptr, d_z.ptr, n, c, h, w, None))
+    assert np.array_equal(d_z.download(shape), x)
+
+
+# ----------------------------------------------------------------- size-independent properties at full size
+
+def test_fc_full_size_properties():
+    m, k, n = 256, 4096, 4096
+    q = quant(0.01, 3, 0.002, 128, 0.08, 0)
+    b = synth.fill_i32((n,), SEED + 80, -100000, 100000)
+    w = synth.fill_u8((n, k), SEED + 81)
+    # inputs at their zero point: every output is requant(bias), whatever the weights
+    a = np.full((m, k), 3, np.uint8)
+    got = gpu_fc(a, w, b, to_eh_requant(q))
+    row = np.array([O.lib.eo_requant(int(v), q) for v in b], np.uint8)
+    assert np.array_equal(got, np.broadcast_to(row, (m, n)))
+    # weights at their zero point: same
+    a = synth.fill_u8((m, k), SEED + 82)
+    got = gpu_fc(a, np.full((n, k), 128, np.uint8), b, to_eh_requant(q))
+    assert np.array_equal(got, np.broadcast_to(row, (m, n)))
+    # permuting the reduction axis of both operands changes nothing
+    perm = np.argsort(synth.splitmix64(SEED + 83, k))
+    got1 = gpu_fc(a, w, b, to_eh_requant(q))
+    got2 = gpu_fc(np.ascontiguousarray(a[:, perm]), np.ascontiguousarray(w[:, perm]), b, to_eh_requant(q))
+    assert np.array_equal(got1, got2)
