@@ -54,7 +54,13 @@ EXPORTS = {
     "eh_h2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "eh_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "eh_d2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "eh_stream_create": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "eh_stream_destroy": (C.c_int, [C.c_void_p]),
     "eh_stream_sync": (C.c_int, [C.c_void_p]),
+    "eh_graph_begin": (C.c_int, [C.c_void_p]),
+    "eh_graph_end": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "eh_graph_launch": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eh_graph_destroy": (C.c_int, [C.c_void_p]),
     "eh_last_error": (C.c_char_p, []),
     "eh_transpose_u8_nchw2nhwc": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int32] * 4 + [C.c_void_p]),
     "eh_transpose_u8_nhwc2nchw": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int32] * 4 + [C.c_void_p]),
@@ -249,6 +255,43 @@ class Event:
     def __del__(self):
         try:
             load().eh_event_destroy(self.h)
+        except Exception:
+            pass
+
+
+class Stream:
+    def __init__(self):
+        self.h = C.c_void_p()
+        check(load().eh_stream_create(C.byref(self.h)))
+
+    def sync(self):
+        check(load().eh_stream_sync(self.h))
+
+    def __del__(self):
+        try:
+            load().eh_stream_destroy(self.h)
+        except Exception:
+            pass
+
+
+class Graph:
+    """Captures whatever `record(stream_handle)` launches and replays it."""
+
+    def __init__(self, stream, record):
+        self.h = C.c_void_p()
+        check(load().eh_graph_begin(stream.h))
+        try:
+            record(stream.h)
+        finally:
+            rc = load().eh_graph_end(stream.h, C.byref(self.h))
+        check(rc)
+
+    def launch(self, stream):
+        check(load().eh_graph_launch(self.h, stream.h))
+
+    def __del__(self):
+        try:
+            load().eh_graph_destroy(self.h)
         except Exception:
             pass
 

@@ -403,6 +403,49 @@ int eh_stream_sync(void *stream) {
     return EH_OK;
 }
 
+int eh_stream_create(void **stream) {
+    EH_REQUIRE(stream != nullptr, "null result pointer");
+    hipStream_t s;
+    EH_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return EH_OK;
+}
+
+int eh_stream_destroy(void *stream) {
+    if (stream) EH_HIP(hipStreamDestroy(as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_graph_begin(void *stream) {
+    EH_REQUIRE(stream != nullptr, "graph capture needs a stream made by eh_stream_create");
+    EH_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return EH_OK;
+}
+
+int eh_graph_end(void *stream, void **graph) {
+    EH_REQUIRE(stream != nullptr && graph != nullptr, "null argument");
+    *graph = nullptr;
+    hipGraph_t g = nullptr;
+    EH_HIP(hipStreamEndCapture(as_stream(stream), &g));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    *graph = exec;
+    return EH_OK;
+}
+
+int eh_graph_launch(void *graph, void *stream) {
+    EH_REQUIRE(graph != nullptr, "null graph");
+    EH_HIP(hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph), as_stream(stream)));
+    return EH_OK;
+}
+
+int eh_graph_destroy(void *graph) {
+    if (graph) EH_HIP(hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph)));
+    return EH_OK;
+}
+
 int eh_event_create(void **event) {
     EH_REQUIRE(event != nullptr, "null result pointer");
     hipEvent_t e;

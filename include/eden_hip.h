@@ -106,8 +106,21 @@ int eh_memset(void *ptr, int value, size_t bytes, void *stream);
 int eh_h2d(void *dst, const void *src, size_t bytes, void *stream);
 int eh_d2h(void *dst, const void *src, size_t bytes, void *stream);
 int eh_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int eh_stream_create(void **stream);                 /* default priority, non-blocking w.r.t. the null stream */
+int eh_stream_destroy(void *stream);
 int eh_stream_sync(void *stream);
 const char *eh_last_error(void);
+
+/* Replay of a fixed launch sequence.  The reference submits a whole subgraph to
+ * one in-order queue and flushes once (gpu/gpu_userdriver.cc:78-112); on HIP the
+ * same sequence is captured once and replayed as a graph, which removes the
+ * per-kernel launch cost of short layers.  Capture needs a stream made by
+ * eh_stream_create; only `*_run` and the transposes may be called between
+ * begin and end (no allocation, no plan creation, no eh_memset). */
+int eh_graph_begin(void *stream);
+int eh_graph_end(void *stream, void **graph);
+int eh_graph_launch(void *graph, void *stream);
+int eh_graph_destroy(void *graph);
 
 /* ---- layout conversion -----------------------------------------------------
  * nchw2nhwc_uint8 / nhwc2nchw_uint8 (gpu/common/CLKernels.hpp:429-491) as
