@@ -143,6 +143,7 @@ struct GemmOp {
     // NCHW boundary: the kernels compute channels-last, so planar tensors pass
     // through these two staging images
     uint8_t *stage_in = nullptr, *stage_out = nullptr;
+    uint8_t *fillbuf = nullptr;  // 16 x input zero point, 16 x 0x80: what out-of-image / padding chunks read
     int32_t layout = EH_NHWC;
     int32_t in_n = 0, in_c = 0, in_hw = 0, out_hw = 0;
     size_t in_bytes = 0;
@@ -153,10 +154,15 @@ struct GemmOp {
         dev_free(bias_copy);
         dev_free(stage_in);
         dev_free(stage_out);
+        dev_free(fillbuf);
     }
 
     int set_weights(const void *weight, const void *bias, hipStream_t stream) {
         EH_REQUIRE(weight != nullptr, "weight pointer is null");
+        if (!fillbuf) {
+            int rc = dev_alloc(&fillbuf, 256);
+            if (rc) return rc;
+        }
         for (auto &g : parts) {
             int rc = pack_part(g, static_cast<const uint8_t *>(weight), stream);
             if (rc) return rc;
@@ -176,7 +182,7 @@ struct GemmOp {
         }
         for (auto &g : parts) {
             int rc = launch_fold_bias(bias_copy + g.bias_base, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, nq.zp_w,
-                                      stream);
+                                      fillbuf, stream);
             if (rc) return rc;
         }
         q = nq;
@@ -203,6 +209,7 @@ struct GemmOp {
             p.a = in;
             p.b = g.b;
             p.bias = g.folded;
+            p.fillbuf = fillbuf;
             p.out = out + g.bias_base;
             p.zw = q.zp_w - 128;
             p.fill = (uint32_t)q.zp_in * 0x01010101u;

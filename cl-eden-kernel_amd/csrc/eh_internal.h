@@ -85,7 +85,9 @@ struct KUnit {
 
 struct GemmProblem {
     const uint8_t *a;     // activations: NHWC image or [M][K] matrix
-    const int8_t *b;      // packed weights [n_pad][k_pad], value = w - 128
+    const int8_t *b;      // packed weights, value = w - 128, in 1 KiB blocks [n_pad/16][k_pad/64][16 rows][64]
+                          // with the four 16-byte chunks of a row swizzled by (row >> 1) & 3
+    const uint8_t *fillbuf;  // 32 bytes: 16 x input zero point, then 16 x 0x80
     const int32_t *bias;  // [n_pad] bias with the zero-point terms folded in
     const KUnit *ktab;    // [k_pad / vec]
     uint8_t *out;
@@ -105,6 +107,13 @@ struct GemmProblem {
 };
 
 int launch_igemm(const GemmProblem &p, hipStream_t stream);
+int launch_igemm_dma(const GemmProblem &p, hipStream_t stream);  // vec == 16 and a k-table that fits LDS
+size_t igemm_dma_ktab_limit();
+// byte offset of reduction chunk `kc16` (16-byte units) of packed row `n`
+__host__ __device__ inline size_t packed_b_offset(int n, int kc16, int k_tiles) {
+    const int r = n & 15, c = kc16 & 3;
+    return ((size_t)(n >> 4) * k_tiles + (kc16 >> 2)) * 1024 + r * 64 + ((c ^ ((r >> 1) & 3)) << 4);
+}
 // tile extents the launcher will pick for (m, n): packed weights are padded to them
 int igemm_n_tile(int32_t m, int32_t n, int32_t k);
 
@@ -121,8 +130,9 @@ struct PackProblem {
 };
 int launch_pack_weights(const PackProblem &p, hipStream_t stream);
 // folded[n] = bias[n] - za * colsum[n] + k * za * zw   (za = zp_in - 128, zw = zp_w - 128)
+// also refreshes the 32-byte fill constant when `fillbuf` is not null
 int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad,
-                     int32_t k, int32_t zp_in, int32_t zp_w, hipStream_t stream);
+                     int32_t k, int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, hipStream_t stream);
 
 // ---------------------------------------------------------------- depthwise
 struct DwProblem {

@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
             const int t = k / p.cin, c = k - t * p.cin;
             v = (int32_t)p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]] - 128;
         }
-        p.b[(size_t)o * p.k_pad + k] = (int8_t)v;
+        p.b[packed_b_offset(o, k >> 4, p.k_pad >> 6) + (k & 15)] = (int8_t)v;
         sum += v;
     }
     partial[threadIdx.x] = sum;
@@ -36,8 +36,9 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
 }
 
 __global__ void fold_bias_kernel(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad,
-                                 int32_t k, int32_t za, int32_t zw) {
+                                 int32_t k, int32_t za, int32_t zw, uint8_t *fillbuf) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (fillbuf && i < 32) fillbuf[i] = i < 16 ? (uint8_t)(za + 128) : (uint8_t)0x80;
     if (i >= n_pad) return;
     int32_t v = 0;
     if (i < n) v = (bias ? bias[i] : 0) - za * colsum[i] + k * za * zw;
@@ -108,10 +109,10 @@ int launch_pack_weights(const PackProblem &p, hipStream_t stream) {
 }
 
 int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad, int32_t k,
-                     int32_t zp_in, int32_t zp_w, hipStream_t stream) {
+                     int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, hipStream_t stream) {
     if (n_pad <= 0) return EH_OK;
     hipLaunchKernelGGL(fold_bias_kernel, dim3((n_pad + 255) / 256), dim3(256), 0, stream, bias, colsum, folded, n, n_pad,
-                       k, zp_in - 128, zp_w - 128);
+                       k, zp_in - 128, zp_w - 128, fillbuf);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }
