@@ -66,6 +66,7 @@ struct GemmPart {
     KUnit *ktab = nullptr;
     int32_t *tap_off = nullptr;
     int32_t n = 0, n_pad = 0, k = 0, k_pad = 0, vec = 1, taps = 0, cin = 0;
+    GemmConfig cfg;
     int64_t so = 0, sc = 0;   // source weight strides (out channel, in channel)
     int64_t w_base = 0;       // element offset of this part in the source weights
     int32_t bias_base = 0;    // first output channel
@@ -89,7 +90,11 @@ int pick_vec(int cig, int pixel_stride) {
 // Allocates a part's device arrays and uploads its tables.  `units` holds one
 // KUnit per `vec` bytes of the real reduction length; padding units are added here.
 int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream) {
-    g.k_pad = round_up(g.k > 0 ? g.k : 1, 64);
+    // the kernel shape is fixed here because the packed weight layout depends on it
+    g.cfg = GemmConfig();
+    if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
+        g.cfg = igemm_dma_select(g.proto.m, g.n, g.k);
+    g.k_pad = round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
     g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
     KUnit pad;
     pad.offset = 0;
@@ -112,6 +117,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     g.proto.k_pad = g.k_pad;
     g.proto.vec = g.vec;
     g.proto.n = g.n;
+    g.proto.cfg = g.cfg;
     return EH_OK;
 }
 
@@ -121,6 +127,7 @@ int pack_part(GemmPart &g, const uint8_t *weight, hipStream_t stream) {
     pp.bias = nullptr;
     pp.b = g.b;
     pp.colsum = g.colsum;
+    pp.cfg = g.cfg;
     pp.n = g.n;
     pp.n_pad = g.n_pad;
     pp.cin = g.cin > 0 ? g.cin : 1;

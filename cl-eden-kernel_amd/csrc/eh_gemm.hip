@@ -149,7 +149,6 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_u8_kernel(const GemmProbl
             a_base[i] = 0;
         }
     }
-    const int b_k_tiles = p.k_pad / BK;
 
     v16i acc[FM][FN];
 #pragma unroll
@@ -172,7 +171,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_u8_kernel(const GemmProbl
         for (int i = 0; i < A_CHUNKS; ++i) ra[i] = load_a_chunk<VEC>(p, a_base[i], a_iy0[i], a_ix0[i], kt * 4 + kc);
 #pragma unroll
         for (int i = 0; i < B_CHUNKS; ++i)
-            rb[i] = *reinterpret_cast<const uint4 *>(p.b + packed_b_offset(n0 + lrow + i * ROWS_PER_PASS, kt * 4 + kc, b_k_tiles));
+            rb[i] = *reinterpret_cast<const uint4 *>(p.b + (size_t)(n0 + lrow + i * ROWS_PER_PASS) * p.k_pad + kt * BK + kc * 16);
     };
     auto store_stage = [&](int buf) {
         uint8_t *as = lds + buf * STAGE_BYTES;
@@ -289,7 +288,7 @@ int launch_igemm(const GemmProblem &p, hipStream_t stream) {
     if (p.m <= 0 || p.n <= 0) return EH_OK;
     EH_REQUIRE(p.k_pad % BK == 0 && p.k_pad > 0, "igemm: padded reduction length %d is not a multiple of %d", p.k_pad, BK);
     EH_REQUIRE(p.vec == 16 || p.vec == 4 || p.vec == 1, "igemm: bad load unit %d", p.vec);
-    if (p.vec == 16 && (size_t)(p.k_pad / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit()) return launch_igemm_dma(p, stream);
+    if (p.cfg.id != GEMM_STAGED) return launch_igemm_dma(p, stream);
     // Pick the largest tile that still spreads the problem over the 256 CUs.
     const long tiles128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
     const long tiles64 = (long)((p.m + 63) / 64) * ((p.n + 63) / 64);

@@ -1,16 +1,23 @@
-// Implicit-GEMM uint8 kernels for gfx950 whose operands go from HBM/L2 straight
+// Implicit-GEMM uint8 kernel for gfx950 whose operands go from HBM/L2 straight
 // into LDS (global_load_lds_dwordx4), several reduction stages ahead of the
 // matrix cores, with no register staging.  Used whenever the input channels come
 // in 16-byte units; the register-staged kernel in eh_gemm.hip covers the rest.
 //
-// LDS image of one stage: rows of 64 reduction bytes, 16 rows per 1 KiB block,
-// the four 16-byte chunks of a row XOR-swizzled by (row >> 1) & 3 so that the
-// 32x32x32 MFMA fragment reads (32 rows x 16 bytes per half wave) are free of
-// bank conflicts.  A wave-wide LDS-DMA instruction writes lane i at base + 16*i,
-// so lane i fetches the global chunk that belongs in slot i: packed weights are
-// stored in exactly this order (a linear 1 KiB copy per instruction), activation
-// lanes compute their own addresses (implicit im2col), and lanes whose tap falls
-// outside the image fetch from a 16-byte constant holding the input zero point.
+// One stage holds a SLAB-byte slice of the reduction axis (128 or 256 bytes, so
+// every activation row is fetched in whole 128-byte cache lines) for BM
+// activation rows and BN weight rows.  LDS rows are SLAB bytes; the 16-byte
+// chunks of a row are XOR-swizzled by the row index so that the 32x32x32 MFMA
+// fragment reads (32 rows x 16 bytes per half wave) are free of bank conflicts.
+// A wave-wide LDS-DMA instruction writes lane i at base + 16*i, so lane i
+// fetches the global chunk that belongs in slot i: packed weights are stored in
+// exactly this order (a linear 1 KiB copy per instruction), activation lanes
+// compute their own addresses (implicit im2col), and lanes whose tap falls
+// outside the image fetch a 16-byte constant holding the input zero point.
+//
+// The 4 waves of a workgroup are arranged WGM x WGN x WGK.  WGK > 1 splits the
+// slab along the reduction axis between waves (each wave still owns the whole
+// BM/WGM x BN/WGN sub-tile): for problems with few output tiles this keeps LDS
+// traffic per MFMA low; the partial tiles meet in LDS at the end (exact: int32).
 //
 // Activations stay uint8 in LDS; the -128 shift is one XOR per fragment register
 // on the way to the MFMA, and the per-row activation sums needed when
@@ -25,12 +32,9 @@ typedef __attribute__((address_space(3))) uint8_t lds_byte;
 
 namespace {
 
-constexpr int BK = 64;
 constexpr int16_t KPAD_MARK = INT16_MIN;
 
-__device__ __forceinline__ uint32_t lds_offset(const void *p) {
-    return (uint32_t)(uintptr_t)(lds_byte *)p;
-}
+__device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(uintptr_t)(lds_byte *)p; }
 
 // One wave copies 64 x 16 bytes: lane i's 16 bytes land at lds_base + 16 * i.
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_base_uniform) {
@@ -61,7 +65,7 @@ __device__ __forceinline__ int sum_bytes_signed(v4i v, int acc) {
 // Where one activation row (one output pixel) starts in the input image.
 struct RowRef {
     int base;  // byte offset of the top-left tap (may be negative: the tap may lie in the padding)
-    int iy0, ix0;
+    int yx;    // (iy0 << 16) | (ix0 & 0xFFFF), both signed 16-bit
 };
 
 __device__ __forceinline__ RowRef make_row(const GemmProblem &p, int m, int plane) {
@@ -69,46 +73,52 @@ __device__ __forceinline__ RowRef make_row(const GemmProblem &p, int m, int plan
     if (m < p.m) {
         const int img = m / plane, rem = m - img * plane;
         const int oy = rem / p.wo, ox = rem - oy * p.wo;
-        r.iy0 = oy * p.stride_h + p.y_base;
-        r.ix0 = ox * p.stride_w + p.x_base;
-        r.base = ((img * p.h + r.iy0) * p.w + r.ix0) * p.cin;
+        const int iy0 = oy * p.stride_h + p.y_base, ix0 = ox * p.stride_w + p.x_base;
+        r.base = ((img * p.h + iy0) * p.w + ix0) * p.cin;
+        r.yx = (int)(((uint32_t)iy0 << 16) | ((uint32_t)ix0 & 0xFFFFu));
     } else {  // rows past M: every tap is "outside", they read the constant
-        r.iy0 = -(1 << 20);
-        r.ix0 = -(1 << 20);
         r.base = 0;
+        r.yx = (int)0x80008000u;
     }
     return r;
 }
 
 __device__ __forceinline__ const uint8_t *a_chunk_address(const GemmProblem &p, const RowRef &r, const KUnit ku) {
-    const int iy = r.iy0 + ku.dy, ix = r.ix0 + ku.dx;
-    if (ku.dy == KPAD_MARK) return p.fillbuf + 16;  // reduction padding: 0x80 bytes, i.e. zero after the shift
-    if ((unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w) return p.a + (r.base + ku.offset);
-    return p.fillbuf;  // spatial padding: the input zero point
+    const int iy = (r.yx >> 16) + ku.dy, ix = (int)(short)(r.yx & 0xFFFF) + ku.dx;
+    const bool inside = (unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w;
+    // reduction padding reads 0x80 bytes (zero after the shift); spatial padding reads the input zero point
+    const uintptr_t image = reinterpret_cast<uintptr_t>(p.a) + (intptr_t)(r.base + ku.offset);
+    const uintptr_t constant = reinterpret_cast<uintptr_t>(p.fillbuf) + (ku.dy == KPAD_MARK ? 16 : 0);
+    return reinterpret_cast<const uint8_t *>(inside && ku.dy != KPAD_MARK ? image : constant);
 }
 
-__device__ __forceinline__ int frag_offset(int row, int chunk) { return row * 64 + ((chunk ^ ((row >> 1) & 3)) << 4); }
-
-// ---------------------------------------------------------------------------
-// Cooperative kernel: 2 x 2 waves share a BM x BN tile; one barrier per stage.
-// ---------------------------------------------------------------------------
-template <int BM, int BN, int STAGES>
-__global__ __launch_bounds__(256) void igemm_dma_tile_kernel(const GemmProblem p, const int tiles_m, const int tiles_n) {
-    constexpr int WTM = BM / 2, WTN = BN / 2;
+template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES>
+__global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, const int tiles_m, const int tiles_n) {
+    static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
+    constexpr int CPR = SLAB / 16;            // 16-byte chunks per LDS row
+    constexpr int RPB = 1024 / SLAB;          // rows per 1 KiB DMA block
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int FM = WTM / 32, FN = WTN / 32;
-    constexpr int A_LOADS = BM / 64, B_LOADS = BN / 64;  // wave-wide DMA instructions per wave per stage
+    constexpr int KSTEPS = SLAB / WGK / 32;   // 32-byte MFMA steps per wave per stage
+    constexpr int A_LOADS = BM / RPB / 4, B_LOADS = BN / RPB / 4;  // DMA instructions per wave per stage
     constexpr int LPS = A_LOADS + B_LOADS;
-    constexpr int STAGE_BYTES = (BM + BN) * BK;
-    constexpr int OUT_ROW = BN + 16;
-    static_assert(BM % 64 == 0 && BN % 64 == 0, "tile extents are multiples of 64");
+    constexpr int STAGE_BYTES = (BM + BN) * SLAB;
+    constexpr int OUT_ROW = BN + 16;          // bytes per row of the staged uint8 tile
+    constexpr int PART_ROW = BN + 16;         // int32 per row of a partial tile
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KSTEPS >= 1, "wave tile is made of 32x32x32 MFMA steps");
+    static_assert(BM % (RPB * 4) == 0 && BN % (RPB * 4) == 0, "whole DMA blocks per wave");
     static_assert((STAGES - 2) * LPS <= 63, "vmcnt is a 6-bit counter");
     static_assert(BM * OUT_ROW <= STAGES * STAGE_BYTES, "output staging reuses the operand stages");
+    static_assert(WGK == 1 || WGK * BM * PART_ROW * 4 <= STAGES * STAGE_BYTES, "partial tiles reuse the operand stages");
 
     __shared__ __align__(1024) uint8_t stages[STAGES * STAGE_BYTES];
-    __shared__ int32_t rowsum_s[BM];
+    __shared__ int32_t rowsum_s[WGK * 2][BM];
     extern __shared__ __align__(8) uint8_t ktab_s_raw[];
     KUnit *ktab_s = reinterpret_cast<KUnit *>(ktab_s_raw);
 
+    // Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2.
+    // Give every XCD a contiguous run of tiles, ordered m-fastest, so that the
+    // workgroups that share a weight tile share an L2.
     int tile = blockIdx.x;
     const int total = tiles_m * tiles_n;
     if ((total & 7) == 0) tile = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
@@ -117,32 +127,37 @@ __global__ __launch_bounds__(256) void igemm_dma_tile_kernel(const GemmProblem p
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave & 1, wn = wave >> 1;
-    const int k_tiles = p.k_pad / BK;
+    const int wm = wave % WGM, wn = (wave / WGM) % WGN, wk = wave / (WGM * WGN);
+    const int k_slabs = p.k_pad / SLAB;
 
-    for (int i = tid; i < k_tiles * 4; i += 256) ktab_s[i] = p.ktab[i];
+    for (int i = tid; i < k_slabs * CPR; i += 256) ktab_s[i] = p.ktab[i];
 
-    // this lane's slot in a DMA block: row (lane >> 2) of 16, physical chunk lane & 3
-    const int slot_row = lane >> 2;
-    const int my_chunk = (lane & 3) ^ ((slot_row >> 1) & 3);
+    // this lane's slot in a DMA block: row (lane / CPR), physical chunk lane % CPR
+    const int slot_row = lane / CPR;
+    const int my_chunk = (lane % CPR) ^ ((wave * RPB + slot_row) & (CPR - 1));
     const int plane = p.ho * p.wo;
     RowRef rows[A_LOADS];
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) rows[i] = make_row(p, m0 + (i * 4 + wave) * 16 + slot_row, plane);
-    const int8_t *b_src = p.b + ((size_t)(n0 >> 4) * k_tiles) * 1024 + lane * 16;
+    for (int i = 0; i < A_LOADS; ++i) rows[i] = make_row(p, m0 + (i * 4 + wave) * RPB + slot_row, plane);
+    const int8_t *b_src = p.b + ((size_t)(n0 / RPB) * k_slabs) * 1024 + lane * 16;
     const uint32_t lds0 = lds_offset(stages);
     __syncthreads();
 
-    auto issue = [&](int kt) {
-        const uint32_t sbase = lds0 + (kt % STAGES) * STAGE_BYTES;
-        const KUnit ku = ktab_s[kt * 4 + my_chunk];
+    // Workgroups walk the reduction axis from different starting slabs (the int32
+    // sum does not care about the order), which spreads the chip's requests over
+    // the L2 channels instead of marching through them in lockstep.
+    const int rot = (int)((blockIdx.x >> 3) * 5u % (unsigned)k_slabs);
+    auto issue = [&](int seq) {
+        int ks = seq + rot;
+        if (ks >= k_slabs) ks -= k_slabs;
+        const uint32_t sbase = lds0 + (seq % STAGES) * STAGE_BYTES;
+        const KUnit ku = ktab_s[ks * CPR + my_chunk];
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i)
-            dma16(a_chunk_address(p, rows[i], ku), sbase + ((i * 4 + wave) << 10));
+        for (int i = 0; i < A_LOADS; ++i) dma16(a_chunk_address(p, rows[i], ku), sbase + ((i * 4 + wave) << 10));
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i) {
             const int blk = i * 4 + wave;
-            dma16(b_src + ((size_t)blk * k_tiles + kt) * 1024, sbase + BM * BK + (blk << 10));
+            dma16(b_src + ((size_t)blk * k_slabs + ks) * 1024, sbase + BM * SLAB + (blk << 10));
         }
     };
 
@@ -160,32 +175,33 @@ __global__ __launch_bounds__(256) void igemm_dma_tile_kernel(const GemmProblem p
 
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
-        if (s < k_tiles) issue(s);
+        if (s < k_slabs) issue(s);
 
     const int frow = lane & 31, fhalf = lane >> 5;
-    for (int kt = 0; kt < k_tiles; ++kt) {
-        // loads of the stages after kt may stay in flight; in the tail just drain
-        if (k_tiles - 1 - kt >= STAGES - 2)
+    for (int seq = 0; seq < k_slabs; ++seq) {
+        // loads of the stages after this one may stay in flight; in the tail just drain
+        if (k_slabs - 1 - seq >= STAGES - 2)
             wait_vmcnt<(STAGES - 2) * LPS>();
         else
             wait_vmcnt<0>();
-        __syncthreads();
-        if (kt + STAGES - 1 < k_tiles) issue(kt + STAGES - 1);
-        const uint8_t *as = stages + (kt % STAGES) * STAGE_BYTES;
-        const uint8_t *bs = as + BM * BK;
+        __syncthreads();  // this stage has landed for every wave; the stage refilled next is no longer read
+        if (seq + STAGES - 1 < k_slabs) issue(seq + STAGES - 1);
+        const uint8_t *as = stages + (seq % STAGES) * STAGE_BYTES;
+        const uint8_t *bs = as + BM * SLAB;
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        for (int kk = 0; kk < KSTEPS; ++kk) {
+            const int chunk = wk * (CPR / WGK) + kk * 2 + fhalf;
             v4i af[FM], bf[FN];
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
                 const int row = wm * WTM + i * 32 + frow;
-                af[i] = xor128(*reinterpret_cast<const v4i *>(as + frag_offset(row, kk * 2 + fhalf)));
+                af[i] = xor128(*reinterpret_cast<const v4i *>(as + row * SLAB + ((chunk ^ (row & (CPR - 1))) << 4)));
                 if (need_rowsum) rowsum[i] = sum_bytes_signed(af[i], rowsum[i]);
             }
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const int row = wn * WTN + j * 32 + frow;
-                bf[j] = *reinterpret_cast<const v4i *>(bs + frag_offset(row, kk * 2 + fhalf));
+                bf[j] = *reinterpret_cast<const v4i *>(bs + row * SLAB + ((chunk ^ (row & (CPR - 1))) << 4));
             }
 #pragma unroll
             for (int i = 0; i < FM; ++i)
@@ -199,233 +215,147 @@ __global__ __launch_bounds__(256) void igemm_dma_tile_kernel(const GemmProblem p
     if (p.zw != 0) {
         if (wn == 0) {
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                const int s = rowsum[i] + __shfl_xor(rowsum[i], 32);
-                if (fhalf == 0) rowsum_s[wm * WTM + i * 32 + frow] = s;
-            }
+            for (int i = 0; i < FM; ++i) rowsum_s[wk * 2 + fhalf][wm * WTM + i * 32 + frow] = rowsum[i];
         }
-    } else {
-        for (int i = tid; i < BM; i += 256) rowsum_s[i] = 0;
     }
     __syncthreads();  // row sums visible; every wave is done with the operand stages
-
-    uint8_t *cs = stages;
     const RequantDev rq = p.rq;
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-        const int nl = wn * WTN + j * 32 + frow;
-        const int32_t bias = p.bias[n0 + nl];
+    const bool wide = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+
+    if constexpr (WGK == 1) {
+        uint8_t *cs = stages;
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
-                const int32_t v = acc[i][j][r] + bias - p.zw * rowsum_s[ml];
-                cs[ml * OUT_ROW + nl] = (uint8_t)requant_u8(v, rq);
+                const int corr = p.zw != 0 ? p.zw * (rowsum_s[0][ml] + rowsum_s[1][ml]) : 0;
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    const int nl = wn * WTN + j * 32 + frow;
+                    cs[ml * OUT_ROW + nl] = (uint8_t)requant_u8(acc[i][j][r] + p.bias[n0 + nl] - corr, rq);
+                }
             }
         }
-    }
-    __syncthreads();
-
-    constexpr int CHUNKS_PER_ROW = BN / 16;
-    const bool wide = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-    for (int q = tid; q < BM * CHUNKS_PER_ROW; q += 256) {
-        const int ml = q / CHUNKS_PER_ROW, nl = (q - ml * CHUNKS_PER_ROW) * 16;
-        const int m = m0 + ml, n = n0 + nl;
-        if (m >= p.m || n >= p.n) continue;
-        const int img = m / plane, r = m - img * plane;
-        const int oy = r / p.wo, ox = r - oy * p.wo;
-        const size_t pix = ((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0);
-        uint8_t *dst = p.out + pix * p.ldc + n;
-        const uint8_t *src = cs + ml * OUT_ROW + nl;
-        if (wide && n + 16 <= p.n) {
-            *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
-        } else {
-            const int cnt = p.n - n < 16 ? p.n - n : 16;
-            for (int t = 0; t < cnt; ++t) dst[t] = src[t];
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Split-reduction kernel for problems with few output tiles: the four waves of a
-// workgroup share one 64 x 64 output tile and each takes every fourth 64-byte
-// slice of the reduction axis through its own private LDS ring, so the main loop
-// has no barrier at all; the four partial tiles meet in LDS at the end.
-// ---------------------------------------------------------------------------
-template <int STAGES>
-__global__ __launch_bounds__(256) void igemm_dma_splitk_kernel(const GemmProblem p, const int tiles_m, const int tiles_n) {
-    constexpr int BM = 64, BN = 64, FM = 2, FN = 2;
-    constexpr int LPS = 8;  // 4 activation + 4 weight DMA instructions per stage
-    constexpr int STAGE_BYTES = (BM + BN) * BK;
-    constexpr int RING_BYTES = STAGES * STAGE_BYTES;
-    constexpr int PART_ROW = BN + 4;  // int32 elements per row of a partial tile
-    static_assert((STAGES - 2) * LPS <= 63, "vmcnt is a 6-bit counter");
-    static_assert(4 * RING_BYTES >= 4 * BM * PART_ROW * 4, "partial tiles reuse the rings");
-
-    __shared__ __align__(1024) uint8_t rings[4 * RING_BYTES];
-    __shared__ int32_t rowsum_s[8][BM];
-    extern __shared__ __align__(8) uint8_t ktab_s_raw[];
-    KUnit *ktab_s = reinterpret_cast<KUnit *>(ktab_s_raw);
-
-    int tile = blockIdx.x;
-    const int total = tiles_m * tiles_n;
-    if ((total & 7) == 0) tile = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
-    const int tm = tile % tiles_m, tn = tile / tiles_m;
-    const int m0 = tm * BM, n0 = tn * BN;
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int k_tiles = p.k_pad / BK;
-    for (int i = tid; i < k_tiles * 4; i += 256) ktab_s[i] = p.ktab[i];
-
-    const int slot_row = lane >> 2;
-    const int my_chunk = (lane & 3) ^ ((slot_row >> 1) & 3);
-    const int plane = p.ho * p.wo;
-    RowRef rows[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rows[i] = make_row(p, m0 + i * 16 + slot_row, plane);
-    const int8_t *b_src = p.b + ((size_t)(n0 >> 4) * k_tiles) * 1024 + lane * 16;
-    uint8_t *ring = rings + wave * RING_BYTES;
-    const uint32_t lds0 = lds_offset(ring);
-    __syncthreads();
-
-    // this wave's slices: kt = wave, wave + 4, ...
-    const int my_tiles = (k_tiles - wave + 3) >> 2;
-    auto issue = [&](int it) {
-        const int kt = wave + (it << 2);
-        const uint32_t sbase = lds0 + (it % STAGES) * STAGE_BYTES;
-        const KUnit ku = ktab_s[kt * 4 + my_chunk];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(a_chunk_address(p, rows[i], ku), sbase + (i << 10));
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(b_src + ((size_t)i * k_tiles + kt) * 1024, sbase + BM * BK + (i << 10));
-    };
-
-    v16i acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-    int rowsum[FM] = {0, 0};
-    const bool need_rowsum = p.zw != 0;
-
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s)
-        if (s < my_tiles) issue(s);
-
-    const int frow = lane & 31, fhalf = lane >> 5;
-    for (int it = 0; it < my_tiles; ++it) {
-        if (my_tiles - 1 - it >= STAGES - 2)
-            wait_vmcnt<(STAGES - 2) * LPS>();
-        else
-            wait_vmcnt<0>();
-        // The stage refilled below was read in the previous iteration by this same
-        // wave; its LDS reads have returned (their values fed the MFMAs already issued).
-        if (it + STAGES - 1 < my_tiles) issue(it + STAGES - 1);
-        const uint8_t *as = ring + (it % STAGES) * STAGE_BYTES;
-        const uint8_t *bs = as + BM * BK;
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            v4i af[FM], bf[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                af[i] = xor128(*reinterpret_cast<const v4i *>(as + frag_offset(i * 32 + frow, kk * 2 + fhalf)));
-                if (need_rowsum) rowsum[i] = sum_bytes_signed(af[i], rowsum[i]);
+        __syncthreads();
+        constexpr int CHUNKS_PER_ROW = BN / 16;
+        for (int q = tid; q < BM * CHUNKS_PER_ROW; q += 256) {
+            const int ml = q / CHUNKS_PER_ROW, nl = (q - ml * CHUNKS_PER_ROW) * 16;
+            const int m = m0 + ml, n = n0 + nl;
+            if (m >= p.m || n >= p.n) continue;
+            const int img = m / plane, r = m - img * plane;
+            const int oy = r / p.wo, ox = r - oy * p.wo;
+            const size_t pix = ((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0);
+            uint8_t *dst = p.out + pix * p.ldc + n;
+            const uint8_t *src = cs + ml * OUT_ROW + nl;
+            if (wide && n + 16 <= p.n) {
+                *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
+            } else {
+                const int cnt = p.n - n < 16 ? p.n - n : 16;
+                for (int t = 0; t < cnt; ++t) dst[t] = src[t];
             }
-#pragma unroll
-            for (int j = 0; j < FN; ++j) bf[j] = *reinterpret_cast<const v4i *>(bs + frag_offset(j * 32 + frow, kk * 2 + fhalf));
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
-    }
-
-    // ---- meet in LDS
-    __syncthreads();  // every wave has finished reading its ring
-    int32_t *part = reinterpret_cast<int32_t *>(rings) + wave * BM * PART_ROW;
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ml = i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
-                part[ml * PART_ROW + j * 32 + frow] = acc[i][j][r];
-            }
-#pragma unroll
-    for (int i = 0; i < FM; ++i) rowsum_s[wave * 2 + fhalf][i * 32 + frow] = rowsum[i];
-    __syncthreads();
-
-    // thread -> row tid / 4, sixteen columns starting at (tid & 3) * 16
-    const int ml = tid >> 2, nl = (tid & 3) * 16;
-    const int m = m0 + ml, n = n0 + nl;
-    if (m >= p.m || n >= p.n) return;
-    int rs = 0;
-    if (need_rowsum) {
-#pragma unroll
-        for (int w = 0; w < 8; ++w) rs += rowsum_s[w][ml];
-    }
-    const int32_t *pr = reinterpret_cast<const int32_t *>(rings) + ml * PART_ROW + nl;
-    const RequantDev rq = p.rq;
-    uint32_t packed[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const int4 s0 = *reinterpret_cast<const int4 *>(pr + g * 4);
-        const int4 s1 = *reinterpret_cast<const int4 *>(pr + g * 4 + BM * PART_ROW);
-        const int4 s2 = *reinterpret_cast<const int4 *>(pr + g * 4 + 2 * BM * PART_ROW);
-        const int4 s3 = *reinterpret_cast<const int4 *>(pr + g * 4 + 3 * BM * PART_ROW);
-        const int4 bb = *reinterpret_cast<const int4 *>(p.bias + n + g * 4);
-        const int corr = p.zw * rs;
-        const uint32_t o0 = requant_u8(s0.x + s1.x + s2.x + s3.x + bb.x - corr, rq);
-        const uint32_t o1 = requant_u8(s0.y + s1.y + s2.y + s3.y + bb.y - corr, rq);
-        const uint32_t o2 = requant_u8(s0.z + s1.z + s2.z + s3.z + bb.z - corr, rq);
-        const uint32_t o3 = requant_u8(s0.w + s1.w + s2.w + s3.w + bb.w - corr, rq);
-        packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
-    }
-    const int img = m / plane, r = m - img * plane;
-    const int oy = r / p.wo, ox = r - oy * p.wo;
-    const size_t pix = ((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0);
-    uint8_t *dst = p.out + pix * p.ldc + n;
-    const bool wide = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-    if (wide && n + 16 <= p.n) {
-        *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     } else {
-        const int cnt = p.n - n < 16 ? p.n - n : 16;
-        for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+        // the WGK partial tiles meet in LDS
+        int32_t *part = reinterpret_cast<int32_t *>(stages) + wk * BM * PART_ROW;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
+                    part[ml * PART_ROW + wn * WTN + j * 32 + frow] = acc[i][j][r];
+                }
+        __syncthreads();
+        // a quad of lanes covers 16 consecutive columns of one row per step
+        constexpr int QUADS_PER_ROW = BN / 16;
+        for (int q = tid >> 2; q < BM * QUADS_PER_ROW; q += 64) {
+            const int ml = q / QUADS_PER_ROW, nl = (q - ml * QUADS_PER_ROW) * 16 + (tid & 3) * 4;
+            const int m = m0 + ml, n = n0 + nl;
+            if (m >= p.m || n >= p.n) continue;
+            int corr = 0;
+            if (p.zw != 0) {
+#pragma unroll
+                for (int w = 0; w < WGK * 2; ++w) corr += rowsum_s[w][ml];
+                corr *= p.zw;
+            }
+            const int32_t *pr = reinterpret_cast<const int32_t *>(stages) + ml * PART_ROW + nl;
+            int4 s = *reinterpret_cast<const int4 *>(pr);
+#pragma unroll
+            for (int w = 1; w < WGK; ++w) {
+                const int4 t = *reinterpret_cast<const int4 *>(pr + w * BM * PART_ROW);
+                s.x += t.x;
+                s.y += t.y;
+                s.z += t.z;
+                s.w += t.w;
+            }
+            const int4 bb = *reinterpret_cast<const int4 *>(p.bias + n);
+            const uint32_t o0 = requant_u8(s.x + bb.x - corr, rq), o1 = requant_u8(s.y + bb.y - corr, rq);
+            const uint32_t o2 = requant_u8(s.z + bb.z - corr, rq), o3 = requant_u8(s.w + bb.w - corr, rq);
+            const uint32_t packed = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+            const int img = m / plane, r = m - img * plane;
+            const int oy = r / p.wo, ox = r - oy * p.wo;
+            const size_t pix = ((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0);
+            uint8_t *dst = p.out + pix * p.ldc + n;
+            if (wide && n + 4 <= p.n) {
+                *reinterpret_cast<uint32_t *>(dst) = packed;
+            } else {
+                const int cnt = p.n - n < 4 ? p.n - n : 4;
+                for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed >> (8 * t));
+            }
+        }
     }
 }
 
-template <int BM, int BN, int STAGES>
-int launch_tile(const GemmProblem &p, hipStream_t stream) {
+template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES>
+int launch_cfg(const GemmProblem &p, hipStream_t stream) {
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
-    hipLaunchKernelGGL((igemm_dma_tile_kernel<BM, BN, STAGES>), dim3(tiles_m * tiles_n), dim3(256), ktab_bytes, stream, p,
-                       tiles_m, tiles_n);
+    hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES>), dim3(tiles_m * tiles_n), dim3(256),
+                       ktab_bytes, stream, p, tiles_m, tiles_n);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }
 
 }  // namespace
 
-size_t igemm_dma_ktab_limit() { return 16384; }
+// Which kernel shape serves an (m, n, k) problem whose activations come in
+// 16-byte channel units.  The packed weight layout depends on the slab, so the
+// choice is made once, when the weights are packed.
+GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k) {
+    GemmConfig c;
+    const long t256 = (long)((m + 255) / 256) * ((n + 127) / 128);
+    const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
+    const long t128x64 = (long)((m + 127) / 128) * ((n + 63) / 64);
+    if (n > 64 && t256 >= 240) {
+        c.id = GEMM_DMA_256x128;
+        c.slab = 128;
+    } else if (n > 64 && t128 >= 200) {
+        c.id = GEMM_DMA_128x128;
+        c.slab = 128;
+    } else if (n <= 64 && t128x64 >= 200) {
+        c.id = GEMM_DMA_128x64;
+        c.slab = 128;
+    } else {
+        c.id = GEMM_DMA_64x64_SPLITK;
+        c.slab = 256;
+    }
+    (void)k;
+    return c;
+}
 
 int launch_igemm_dma(const GemmProblem &p, hipStream_t stream) {
-    const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
-    EH_REQUIRE(p.vec == 16 && ktab_bytes <= igemm_dma_ktab_limit(), "igemm_dma: unsupported problem");
-    const long t256 = (long)((p.m + 255) / 256) * ((p.n + 127) / 128);
-    const long t128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
-    if (p.n > 64 && t256 >= 256) return launch_tile<256, 128, 3>(p, stream);
-    if (p.n > 64 && t128 >= 192) return launch_tile<128, 128, 3>(p, stream);
-    const int tiles_m = (p.m + 63) / 64, tiles_n = (p.n + 63) / 64;
-    hipLaunchKernelGGL((igemm_dma_splitk_kernel<4>), dim3(tiles_m * tiles_n), dim3(256), ktab_bytes, stream, p, tiles_m,
-                       tiles_n);
-    EH_HIP(hipGetLastError());
-    return EH_OK;
+    EH_REQUIRE(p.vec == 16 && p.k_pad % p.cfg.slab == 0, "igemm_dma: unsupported problem");
+    switch (p.cfg.id) {
+        case GEMM_DMA_256x128: return launch_cfg<256, 128, 2, 2, 1, 128, 3>(p, stream);
+        case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 4>(p, stream);
+        case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 4>(p, stream);
+        case GEMM_DMA_64x64_SPLITK: return launch_cfg<64, 64, 1, 1, 4, 256, 4>(p, stream);
+        default: break;
+    }
+    set_error("igemm_dma: unknown configuration %d", p.cfg.id);
+    return EH_INVALID_PARAMS;
 }
 
 }  // namespace eh

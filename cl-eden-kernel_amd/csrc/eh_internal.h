@@ -83,10 +83,23 @@ struct KUnit {
     int16_t dx;
 };
 
+// Kernel shape chosen for a problem when its weights are packed.
+enum GemmConfigId {
+    GEMM_STAGED = 0,            // register-staged kernel, any channel count; weights row-major [n_pad][k_pad]
+    GEMM_DMA_256x128 = 1,       // direct-to-LDS kernels; weights in swizzled 1 KiB blocks (see packed_b_offset)
+    GEMM_DMA_128x128 = 2,
+    GEMM_DMA_128x64 = 3,
+    GEMM_DMA_64x64_SPLITK = 4,
+};
+struct GemmConfig {
+    int32_t id = GEMM_STAGED;
+    int32_t slab = 64;  // reduction bytes per stage; k_pad is a multiple of it
+};
+
 struct GemmProblem {
     const uint8_t *a;     // activations: NHWC image or [M][K] matrix
-    const int8_t *b;      // packed weights, value = w - 128, in 1 KiB blocks [n_pad/16][k_pad/64][16 rows][64]
-                          // with the four 16-byte chunks of a row swizzled by (row >> 1) & 3
+    const int8_t *b;      // packed weights, value = w - 128, laid out for cfg (see packed_b_offset)
+    GemmConfig cfg;
     const uint8_t *fillbuf;  // 32 bytes: 16 x input zero point, then 16 x 0x80
     const int32_t *bias;  // [n_pad] bias with the zero-point terms folded in
     const KUnit *ktab;    // [k_pad / vec]
@@ -108,11 +121,17 @@ struct GemmProblem {
 
 int launch_igemm(const GemmProblem &p, hipStream_t stream);
 int launch_igemm_dma(const GemmProblem &p, hipStream_t stream);  // vec == 16 and a k-table that fits LDS
-size_t igemm_dma_ktab_limit();
-// byte offset of reduction chunk `kc16` (16-byte units) of packed row `n`
-__host__ __device__ inline size_t packed_b_offset(int n, int kc16, int k_tiles) {
-    const int r = n & 15, c = kc16 & 3;
-    return ((size_t)(n >> 4) * k_tiles + (kc16 >> 2)) * 1024 + r * 64 + ((c ^ ((r >> 1) & 3)) << 4);
+GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k);
+inline size_t igemm_dma_ktab_limit() { return 12288; }
+// Byte offset of reduction chunk `kc16` (16-byte units) of packed weight row `n`.
+// Direct-to-LDS layouts: 1 KiB blocks of (1024 / slab) rows x slab bytes, ordered
+// [row block][slab index], the 16-byte chunks of a row XOR-swizzled by the row index.
+__host__ __device__ inline size_t packed_b_offset(const GemmConfig &cfg, int n, int kc16, int k_pad) {
+    if (cfg.id == GEMM_STAGED) return (size_t)n * k_pad + (size_t)kc16 * 16;
+    const int cpr = cfg.slab / 16, rpb = 1024 / cfg.slab;
+    const int c = kc16 % cpr;
+    return ((size_t)(n / rpb) * (k_pad / cfg.slab) + kc16 / cpr) * 1024 + (size_t)(n % rpb) * cfg.slab +
+           ((c ^ (n & (cpr - 1))) << 4);
 }
 // tile extents the launcher will pick for (m, n): packed weights are padded to them
 int igemm_n_tile(int32_t m, int32_t n, int32_t k);
@@ -123,6 +142,7 @@ struct PackProblem {
     const int32_t *bias;   // source bias [n] or null
     int8_t *b;             // [n_pad][k_pad]
     int32_t *colsum;       // [n_pad]  sum_k (w - 128)
+    GemmConfig cfg;
     int32_t n, n_pad, cin, taps, k, k_pad;
     // source index of (out channel o, in channel c, tap t) = o*so + c*sc + tap_off[t]
     int64_t so, sc;

@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
             const int t = k / p.cin, c = k - t * p.cin;
             v = (int32_t)p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]] - 128;
         }
-        p.b[packed_b_offset(o, k >> 4, p.k_pad >> 6) + (k & 15)] = (int8_t)v;
+        p.b[packed_b_offset(p.cfg, o, k >> 4, p.k_pad) + (k & 15)] = (int8_t)v;
         sum += v;
     }
     partial[threadIdx.x] = sum;
