@@ -187,7 +187,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, conv, dw, pw, deconv")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (got --gpus %d); no multi-GPU figure exists" % args.gpus,
@@ -201,7 +201,8 @@ def main():
     stream = eden.Stream()
     use_graph = not args.no_graph
 
-    families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload)
+    families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
+                    fcbig=lambda e, s: fc_workload(e, s, 8192, 4096, 4096), conv64=lambda e, s: conv_workload(e, s, 64))
     if args.only:
         work = families[args.only](eden, synth)
         wall, ev = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph)

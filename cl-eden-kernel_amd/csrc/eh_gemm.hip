@@ -282,7 +282,7 @@ int launch_tile(const GemmProblem &p, hipStream_t stream) {
 
 }  // namespace
 
-int igemm_n_tile(int32_t, int32_t, int32_t) { return 128; }
+int igemm_n_tile(int32_t, int32_t, int32_t) { return 256; }
 
 int launch_igemm(const GemmProblem &p, hipStream_t stream) {
     if (p.m <= 0 || p.n <= 0) return EH_OK;

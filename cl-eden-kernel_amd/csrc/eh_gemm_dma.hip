@@ -22,6 +22,8 @@
 // Activations stay uint8 in LDS; the -128 shift is one XOR per fragment register
 // on the way to the MFMA, and the per-row activation sums needed when
 // zp_w != 128 are v_dot4 accumulations over the same fragment registers.
+#include <type_traits>
+
 #include "eh_internal.h"
 
 namespace eh {
@@ -93,7 +95,7 @@ __device__ __forceinline__ const uint8_t *a_chunk_address(const GemmProblem &p, 
 }
 
 template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES>
-__global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, const int tiles_m, const int tiles_n) {
+__global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, const int tiles_m, const int tiles_n, const int gm) {
     static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
     constexpr int CPR = SLAB / 16;            // 16-byte chunks per LDS row
     constexpr int RPB = 1024 / SLAB;          // rows per 1 KiB DMA block
@@ -116,13 +118,18 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     extern __shared__ __align__(8) uint8_t ktab_s_raw[];
     KUnit *ktab_s = reinterpret_cast<KUnit *>(ktab_s_raw);
 
-    // Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2.
-    // Give every XCD a contiguous run of tiles, ordered m-fastest, so that the
-    // workgroups that share a weight tile share an L2.
-    int tile = blockIdx.x;
-    const int total = tiles_m * tiles_n;
-    if ((total & 7) == 0) tile = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
-    const int tm = tile % tiles_m, tn = tile / tiles_m;
+    // Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2,
+    // and an XCD runs 32 of these workgroups at a time (one per CU).  Tiles are
+    // therefore handed out in groups of 32 that form a gm x gn rectangle of the
+    // output: the workgroups of a group walk the reduction axis in step, so every
+    // activation slab is pulled into that L2 once for gn tiles and every weight
+    // slab once for gm tiles.
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int group = (j >> 5) * 8 + xcd, within = j & 31;
+    const int groups_m = (tiles_m + gm - 1) / gm;
+    const int gi = group % groups_m, gj = group / groups_m;
+    const int tm = gi * gm + within % gm, tn = gj * (32 / gm) + within / gm;
+    if (tm >= tiles_m || tn >= tiles_n) return;
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -143,22 +150,23 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     const uint32_t lds0 = lds_offset(stages);
     __syncthreads();
 
-    // Workgroups walk the reduction axis from different starting slabs (the int32
-    // sum does not care about the order), which spreads the chip's requests over
-    // the L2 channels instead of marching through them in lockstep.
-    const int rot = (int)((blockIdx.x >> 3) * 5u % (unsigned)k_slabs);
-    auto issue = [&](int seq) {
-        int ks = seq + rot;
-        if (ks >= k_slabs) ks -= k_slabs;
+    // The DMA instructions of a stage are spread over the MFMA steps of the stage
+    // before it, so that their address arithmetic fills the issue slots the matrix
+    // pipe leaves free instead of running ahead of it as one serial block.
+    auto issue_part = [&](int seq, const KUnit ku, auto first, auto last) {
         const uint32_t sbase = lds0 + (seq % STAGES) * STAGE_BYTES;
-        const KUnit ku = ktab_s[ks * CPR + my_chunk];
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) dma16(a_chunk_address(p, rows[i], ku), sbase + ((i * 4 + wave) << 10));
-#pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) {
-            const int blk = i * 4 + wave;
-            dma16(b_src + ((size_t)blk * k_slabs + ks) * 1024, sbase + BM * SLAB + (blk << 10));
+        for (int idx = decltype(first)::value; idx < decltype(last)::value; ++idx) {
+            if (idx < A_LOADS) {
+                dma16(a_chunk_address(p, rows[idx], ku), sbase + ((idx * 4 + wave) << 10));
+            } else {
+                const int blk = (idx - A_LOADS) * 4 + wave;
+                dma16(b_src + ((size_t)blk * k_slabs + seq) * 1024, sbase + BM * SLAB + (blk << 10));
+            }
         }
+    };
+    auto issue = [&](int seq) {
+        issue_part(seq, ktab_s[seq * CPR + my_chunk], std::integral_constant<int, 0>{}, std::integral_constant<int, LPS>{});
     };
 
     v16i acc[FM][FN];
@@ -185,11 +193,13 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         else
             wait_vmcnt<0>();
         __syncthreads();  // this stage has landed for every wave; the stage refilled next is no longer read
-        if (seq + STAGES - 1 < k_slabs) issue(seq + STAGES - 1);
+        const int next = seq + STAGES - 1;
+        const bool more = next < k_slabs;
+        const KUnit ku = ktab_s[(more ? next : 0) * CPR + my_chunk];
         const uint8_t *as = stages + (seq % STAGES) * STAGE_BYTES;
         const uint8_t *bs = as + BM * SLAB;
-#pragma unroll
-        for (int kk = 0; kk < KSTEPS; ++kk) {
+        auto step = [&](auto kk_c) {
+            constexpr int kk = decltype(kk_c)::value;
             const int chunk = wk * (CPR / WGK) + kk * 2 + fhalf;
             v4i af[FM], bf[FN];
 #pragma unroll
@@ -203,12 +213,20 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
                 const int row = wn * WTN + j * 32 + frow;
                 bf[j] = *reinterpret_cast<const v4i *>(bs + row * SLAB + ((chunk ^ (row & (CPR - 1))) << 4));
             }
+            if (more)
+                issue_part(next, ku, std::integral_constant<int, kk * LPS / KSTEPS>{},
+                           std::integral_constant<int, (kk + 1) * LPS / KSTEPS>{});
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
+        };
+        step(std::integral_constant<int, 0>{});
+        if constexpr (KSTEPS > 1) step(std::integral_constant<int, 1>{});
+        if constexpr (KSTEPS > 2) step(std::integral_constant<int, 2>{});
+        if constexpr (KSTEPS > 3) step(std::integral_constant<int, 3>{});
+        static_assert(KSTEPS <= 4, "at most four MFMA steps per stage");
     }
 
     // ---- epilogue
@@ -311,9 +329,24 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
 template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES>
 int launch_cfg(const GemmProblem &p, hipStream_t stream) {
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    // group shape gm x (32 / gm): least operand rows per group among the shapes that fit the tile grid
+    int gm = 1;
+    long best = -1;
+    for (int cand = 1; cand <= 32; cand *= 2) {
+        const int gn = 32 / cand;
+        const long cost = (long)(cand < tiles_m ? cand : tiles_m) * BM + (long)(gn < tiles_n ? gn : tiles_n) * BN;
+        const long waste = (long)((tiles_m + cand - 1) / cand) * ((tiles_n + gn - 1) / gn);  // groups launched
+        const long score = cost * waste;
+        if (best < 0 || score < best) {
+            best = score;
+            gm = cand;
+        }
+    }
+    const int groups = ((tiles_m + gm - 1) / gm) * ((tiles_n + 32 / gm - 1) / (32 / gm));
+    const int grid = ((groups + 7) / 8) * 8 * 32;
     const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
-    hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES>), dim3(tiles_m * tiles_n), dim3(256),
-                       ktab_bytes, stream, p, tiles_m, tiles_n);
+    hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES>), dim3(grid), dim3(256), ktab_bytes, stream, p,
+                       tiles_m, tiles_n, gm);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }
@@ -328,7 +361,11 @@ GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k) {
     const long t256 = (long)((m + 255) / 256) * ((n + 127) / 128);
     const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
     const long t128x64 = (long)((m + 127) / 128) * ((n + 63) / 64);
-    if (n > 64 && t256 >= 240) {
+    const long t256x256 = (long)((m + 255) / 256) * ((n + 255) / 256);
+    if (n > 128 && t256x256 >= 240) {
+        c.id = GEMM_DMA_256x256;
+        c.slab = 128;
+    } else if (n > 64 && t256 >= 240) {
         c.id = GEMM_DMA_256x128;
         c.slab = 128;
     } else if (n > 64 && t128 >= 200) {
@@ -348,6 +385,7 @@ GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k) {
 int launch_igemm_dma(const GemmProblem &p, hipStream_t stream) {
     EH_REQUIRE(p.vec == 16 && p.k_pad % p.cfg.slab == 0, "igemm_dma: unsupported problem");
     switch (p.cfg.id) {
+        case GEMM_DMA_256x256: return launch_cfg<256, 256, 2, 2, 1, 128, 2>(p, stream);
         case GEMM_DMA_256x128: return launch_cfg<256, 128, 2, 2, 1, 128, 3>(p, stream);
         case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 4>(p, stream);
         case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 4>(p, stream);

@@ -90,6 +90,7 @@ enum GemmConfigId {
     GEMM_DMA_128x128 = 2,
     GEMM_DMA_128x64 = 3,
     GEMM_DMA_64x64_SPLITK = 4,
+    GEMM_DMA_256x256 = 5,
 };
 struct GemmConfig {
     int32_t id = GEMM_STAGED;

@@ -74,6 +74,46 @@ def test_fc_matches_oracle(m, k, n, zp_a, zp_w):
     assert want.std() > 10  # the case exercises the requant range, not a saturated constant
 
 
+# shapes chosen to land on each large-tile kernel configuration (by tile count), ragged in m and n
+BIG_FC_CASES = [
+    (16384 - 37, 128, 1024 - 24, 9, 77),    # 256 x 256 tiles
+    (65536 - 5, 128, 128 - 16, 200, 128),   # 256 x 128 tiles
+    (16384 - 100, 192, 256, 128, 3),        # 128 x 128 tiles
+    (32768 - 3, 64, 64 - 8, 17, 250),       # 128 x 64 tiles
+]
+
+
+@pytest.mark.parametrize("m,k,n,zp_a,zp_w", BIG_FC_CASES)
+def test_fc_large_tile_configurations(m, k, n, zp_a, zp_w):
+    print("fc big", m, k, n, flush=True)
+    a = synth.fill_u8((m, k), SEED + 7)
+    w = synth.fill_u8((n, k), SEED + 8)
+    b = synth.fill_i32((n,), SEED + 9, -1000, 1000)
+    _, acc = O.fc(a[:512], w, b, O.raw_quant(zp_in=zp_a, zp_w=zp_w), want_acc=True)
+    q = centred_quant(acc, zp_a, zp_w)
+    want = O.fc(a, w, b, q)
+    got = gpu_fc(a, w, b, to_eh_requant(q))
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 10
+
+
+def test_conv_batched_large_tiles():
+    """3x3 convolution at batch 16 (50176 output pixels): the cooperative-tile kernels with padding taps."""
+    s = O.conv_shape(16, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 21)
+    q = quant(0.02, 128, 0.005, 120, 0.05, 0, O.ACT_RELU, True)
+    want = O.conv2d(x, w, b, s, q)
+    got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
+    assert np.array_equal(got, want), diff_report(got, want)
+    s = O.conv_shape(4, 32, 56, 56, 192, 3, 3, stride=(1, 1), pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 22)
+    _, acc = O.conv2d(x[:1], w, b, O.conv_shape(1, 32, 56, 56, 192, 3, 3, pad=(1, 1, 1, 1)), O.raw_quant(zp_in=131, zp_w=120), want_acc=True)
+    q = centred_quant(acc, 131, 120)
+    want = O.conv2d(x, w, b, s, q)
+    got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
+    assert np.array_equal(got, want), diff_report(got, want)
+
+
 def test_fc_config2_full_size():
     """M=256, K=4096, N=4096; uint8 activations zp 3; weights clip(N(128,20)) zp 128; scales 0.01/0.002/0.08."""
     m, k, n = 256, 4096, 4096
