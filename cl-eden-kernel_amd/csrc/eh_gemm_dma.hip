@@ -19,6 +19,11 @@
 // BM/WGM x BN/WGN sub-tile): for problems with few output tiles this keeps LDS
 // traffic per MFMA low; the partial tiles meet in LDS at the end (exact: int32).
 //
+// The MFMA is issued with the weight fragment as its row operand, so a lane ends
+// up holding, for ONE output pixel, groups of four consecutive output channels:
+// four requantized bytes pack into one 32-bit store to the channels-last output
+// with no LDS round trip, and the per-pixel terms are per-lane scalars.
+//
 // Activations stay uint8 in LDS; the -128 shift is one XOR per fragment register
 // on the way to the MFMA, and the per-row activation sums needed when
 // zp_w != 128 are v_dot4 accumulations over the same fragment registers.
@@ -73,8 +78,8 @@ struct RowRef {
 __device__ __forceinline__ RowRef make_row(const GemmProblem &p, int m, int plane) {
     RowRef r;
     if (m < p.m) {
-        const int img = m / plane, rem = m - img * plane;
-        const int oy = rem / p.wo, ox = rem - oy * p.wo;
+        const int img = (int)fastdiv((uint32_t)m, p.div_plane), rem = m - img * plane;
+        const int oy = (int)fastdiv((uint32_t)rem, p.div_wo), ox = rem - oy * p.wo;
         const int iy0 = oy * p.stride_h + p.y_base, ix0 = ox * p.stride_w + p.x_base;
         r.base = ((img * p.h + iy0) * p.w + ix0) * p.cin;
         r.yx = (int)(((uint32_t)iy0 << 16) | ((uint32_t)ix0 & 0xFFFFu));
@@ -94,7 +99,14 @@ __device__ __forceinline__ const uint8_t *a_chunk_address(const GemmProblem &p, 
     return reinterpret_cast<const uint8_t *>(inside && ku.dy != KPAD_MARK ? image : constant);
 }
 
-template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES>
+// byte offset of output pixel m (row of the GEMM) in the channels-last output
+__device__ __forceinline__ size_t out_pixel_offset(const GemmProblem &p, int m, int plane) {
+    const int img = (int)fastdiv((uint32_t)m, p.div_plane), rem = m - img * plane;
+    const int oy = (int)fastdiv((uint32_t)rem, p.div_wo), ox = rem - oy * p.wo;
+    return (((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0)) * (size_t)p.ldc;
+}
+
+template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES, bool DENSE>
 __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, const int tiles_m, const int tiles_n, const int gm) {
     static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
     constexpr int CPR = SLAB / 16;            // 16-byte chunks per LDS row
@@ -105,16 +117,17 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     constexpr int A_LOADS = BM / RPB / 4, B_LOADS = BN / RPB / 4;  // DMA instructions per wave per stage
     constexpr int LPS = A_LOADS + B_LOADS;
     constexpr int STAGE_BYTES = (BM + BN) * SLAB;
-    constexpr int OUT_ROW = BN + 16;          // bytes per row of the staged uint8 tile
-    constexpr int PART_ROW = BN + 16;         // int32 per row of a partial tile
+    constexpr int PART_ROW = BN + 4;          // int32 per row of a partial tile: 8 consecutive rows cover all banks
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KSTEPS >= 1, "wave tile is made of 32x32x32 MFMA steps");
     static_assert(BM % (RPB * 4) == 0 && BN % (RPB * 4) == 0, "whole DMA blocks per wave");
     static_assert((STAGES - 2) * LPS <= 63, "vmcnt is a 6-bit counter");
-    static_assert(BM * OUT_ROW <= STAGES * STAGE_BYTES, "output staging reuses the operand stages");
     static_assert(WGK == 1 || WGK * BM * PART_ROW * 4 <= STAGES * STAGE_BYTES, "partial tiles reuse the operand stages");
+    static_assert(WGK == 1 || (BM == 64 && BN == 64 && WGM == 1 && WGN == 1), "the split-reduction epilogue is written for one 64x64 tile");
 
     __shared__ __align__(1024) uint8_t stages[STAGES * STAGE_BYTES];
     __shared__ int32_t rowsum_s[WGK * 2][BM];
+    __shared__ __align__(16) int32_t bias_s[BN];  // read in the epilogue from LDS: a global load there would have to
+                                                   // wait for the stores issued before it (one counter for both)
     extern __shared__ __align__(8) uint8_t ktab_s_raw[];
     KUnit *ktab_s = reinterpret_cast<KUnit *>(ktab_s_raw);
 
@@ -133,40 +146,62 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
+    for (int i = tid; i < BN; i += 256) bias_s[i] = p.bias[n0 + i];
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = (wave / WGM) % WGN, wk = wave / (WGM * WGN);
     const int k_slabs = p.k_pad / SLAB;
 
-    for (int i = tid; i < k_slabs * CPR; i += 256) ktab_s[i] = p.ktab[i];
+    if constexpr (!DENSE)
+        for (int i = tid; i < k_slabs * CPR; i += 256) ktab_s[i] = p.ktab[i];
 
     // this lane's slot in a DMA block: row (lane / CPR), physical chunk lane % CPR
     const int slot_row = lane / CPR;
     const int my_chunk = (lane % CPR) ^ ((wave * RPB + slot_row) & (CPR - 1));
     const int plane = p.ho * p.wo;
-    RowRef rows[A_LOADS];
+    RowRef rows[DENSE ? 1 : A_LOADS];
+    const uint8_t *a_ptr[DENSE ? A_LOADS : 1];  // dense: where this lane's chunk of the next slab sits, per row
+    if constexpr (DENSE) {
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) rows[i] = make_row(p, m0 + (i * 4 + wave) * RPB + slot_row, plane);
-    const int8_t *b_src = p.b + ((size_t)(n0 / RPB) * k_slabs) * 1024 + lane * 16;
+        for (int i = 0; i < A_LOADS; ++i) {
+            int m = m0 + (i * 4 + wave) * RPB + slot_row;
+            m = m < p.m ? m : p.m - 1;  // rows past M re-read the last row; their results are never stored
+            a_ptr[i] = p.a + (size_t)m * p.cin + my_chunk * 16;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) rows[i] = make_row(p, m0 + (i * 4 + wave) * RPB + slot_row, plane);
+    }
+    const int8_t *b_ptr[B_LOADS];  // where this lane's 16 bytes of the next slab sit, per weight block
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) b_ptr[i] = p.b + ((size_t)(n0 / RPB + i * 4 + wave) * k_slabs) * 1024 + lane * 16;
     const uint32_t lds0 = lds_offset(stages);
     __syncthreads();
 
     // The DMA instructions of a stage are spread over the MFMA steps of the stage
     // before it, so that their address arithmetic fills the issue slots the matrix
-    // pipe leaves free instead of running ahead of it as one serial block.
+    // pipe leaves free instead of running ahead of it as one serial block.  Stages
+    // are issued in order, so the weight (and dense activation) pointers just advance.
     auto issue_part = [&](int seq, const KUnit ku, auto first, auto last) {
         const uint32_t sbase = lds0 + (seq % STAGES) * STAGE_BYTES;
 #pragma unroll
         for (int idx = decltype(first)::value; idx < decltype(last)::value; ++idx) {
             if (idx < A_LOADS) {
-                dma16(a_chunk_address(p, rows[idx], ku), sbase + ((idx * 4 + wave) << 10));
+                if constexpr (DENSE) {
+                    dma16(a_ptr[idx], sbase + ((idx * 4 + wave) << 10));
+                    a_ptr[idx] += SLAB;
+                } else {
+                    dma16(a_chunk_address(p, rows[idx], ku), sbase + ((idx * 4 + wave) << 10));
+                }
             } else {
-                const int blk = (idx - A_LOADS) * 4 + wave;
-                dma16(b_src + ((size_t)blk * k_slabs + seq) * 1024, sbase + BM * SLAB + (blk << 10));
+                const int bi = idx - A_LOADS;
+                dma16(b_ptr[bi], sbase + BM * SLAB + ((bi * 4 + wave) << 10));
+                b_ptr[bi] += 1024;
             }
         }
     };
     auto issue = [&](int seq) {
-        issue_part(seq, ktab_s[seq * CPR + my_chunk], std::integral_constant<int, 0>{}, std::integral_constant<int, LPS>{});
+        issue_part(seq, DENSE ? KUnit() : ktab_s[seq * CPR + my_chunk], std::integral_constant<int, 0>{},
+                   std::integral_constant<int, LPS>{});
     };
 
     v16i acc[FM][FN];
@@ -195,7 +230,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         __syncthreads();  // this stage has landed for every wave; the stage refilled next is no longer read
         const int next = seq + STAGES - 1;
         const bool more = next < k_slabs;
-        const KUnit ku = ktab_s[(more ? next : 0) * CPR + my_chunk];
+        const KUnit ku = DENSE ? KUnit() : ktab_s[(more ? next : 0) * CPR + my_chunk];
         const uint8_t *as = stages + (seq % STAGES) * STAGE_BYTES;
         const uint8_t *bs = as + BM * SLAB;
         auto step = [&](auto kk_c) {
@@ -220,7 +255,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
             for (int i = 0; i < FM; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
         };
         step(std::integral_constant<int, 0>{});
         if constexpr (KSTEPS > 1) step(std::integral_constant<int, 1>{});
@@ -229,7 +264,8 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         static_assert(KSTEPS <= 4, "at most four MFMA steps per stage");
     }
 
-    // ---- epilogue
+    // ---- epilogue.  acc[i][j][r] belongs to pixel row i*32 + (lane & 31) and channel
+    // j*32 + 8*(r >> 2) + 4*(lane >> 5) + (r & 3) of this wave's sub-tile.
     if (p.zw != 0) {
         if (wn == 0) {
 #pragma unroll
@@ -238,96 +274,103 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     }
     __syncthreads();  // row sums visible; every wave is done with the operand stages
     const RequantDev rq = p.rq;
-    const bool wide = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+    const bool aligned4 = (p.ldc & 3) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 3) == 0);
 
     if constexpr (WGK == 1) {
-        uint8_t *cs = stages;
+        size_t row_off[FM];
+        int corr[FM];
+        bool row_ok[FM];
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
+            const int ml = wm * WTM + i * 32 + frow, m = m0 + ml;
+            row_ok[i] = m < p.m;
+            row_off[i] = row_ok[i] ? out_pixel_offset(p, m, plane) : 0;
+            corr[i] = p.zw != 0 ? p.zw * (rowsum_s[0][ml] + rowsum_s[1][ml]) : 0;
+        }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
-                const int corr = p.zw != 0 ? p.zw * (rowsum_s[0][ml] + rowsum_s[1][ml]) : 0;
+        for (int j = 0; j < FN; ++j) {
 #pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    const int nl = wn * WTN + j * 32 + frow;
-                    cs[ml * OUT_ROW + nl] = (uint8_t)requant_u8(acc[i][j][r] + p.bias[n0 + nl] - corr, rq);
+            for (int g = 0; g < 4; ++g) {
+                const int nl = wn * WTN + j * 32 + g * 8 + fhalf * 4, n = n0 + nl;
+                const int4 bb = *reinterpret_cast<const int4 *>(bias_s + nl);
+#pragma unroll
+                for (int i = 0; i < FM; ++i) {
+                    const uint32_t o0 = requant_u8(acc[i][j][g * 4 + 0] + bb.x - corr[i], rq);
+                    const uint32_t o1 = requant_u8(acc[i][j][g * 4 + 1] + bb.y - corr[i], rq);
+                    const uint32_t o2 = requant_u8(acc[i][j][g * 4 + 2] + bb.z - corr[i], rq);
+                    const uint32_t o3 = requant_u8(acc[i][j][g * 4 + 3] + bb.w - corr[i], rq);
+                    const uint32_t packed = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+                    if (!row_ok[i] || n >= p.n) continue;
+                    uint8_t *dst = p.out + row_off[i] + n;
+                    if (aligned4 && n + 4 <= p.n) {
+                        *reinterpret_cast<uint32_t *>(dst) = packed;
+                    } else {
+                        const int cnt = p.n - n < 4 ? p.n - n : 4;
+                        for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed >> (8 * t));
+                    }
                 }
             }
         }
-        __syncthreads();
-        constexpr int CHUNKS_PER_ROW = BN / 16;
-        for (int q = tid; q < BM * CHUNKS_PER_ROW; q += 256) {
-            const int ml = q / CHUNKS_PER_ROW, nl = (q - ml * CHUNKS_PER_ROW) * 16;
-            const int m = m0 + ml, n = n0 + nl;
-            if (m >= p.m || n >= p.n) continue;
-            const int img = m / plane, r = m - img * plane;
-            const int oy = r / p.wo, ox = r - oy * p.wo;
-            const size_t pix = ((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0);
-            uint8_t *dst = p.out + pix * p.ldc + n;
-            const uint8_t *src = cs + ml * OUT_ROW + nl;
-            if (wide && n + 16 <= p.n) {
-                *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
-            } else {
-                const int cnt = p.n - n < 16 ? p.n - n : 16;
-                for (int t = 0; t < cnt; ++t) dst[t] = src[t];
-            }
-        }
     } else {
-        // the WGK partial tiles meet in LDS
+        // the WGK partial tiles meet in LDS: [wk][pixel row][channel], rows padded so that
+        // eight consecutive rows of 16-byte accesses fall in distinct banks
         int32_t *part = reinterpret_cast<int32_t *>(stages) + wk * BM * PART_ROW;
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
-                    part[ml * PART_ROW + wn * WTN + j * 32 + frow] = acc[i][j][r];
+                for (int g = 0; g < 4; ++g) {
+                    int4 v;
+                    v.x = acc[i][j][g * 4 + 0];
+                    v.y = acc[i][j][g * 4 + 1];
+                    v.z = acc[i][j][g * 4 + 2];
+                    v.w = acc[i][j][g * 4 + 3];
+                    *reinterpret_cast<int4 *>(part + (i * 32 + frow) * PART_ROW + j * 32 + g * 8 + fhalf * 4) = v;
                 }
         __syncthreads();
-        // a quad of lanes covers 16 consecutive columns of one row per step
-        constexpr int QUADS_PER_ROW = BN / 16;
-        for (int q = tid >> 2; q < BM * QUADS_PER_ROW; q += 64) {
-            const int ml = q / QUADS_PER_ROW, nl = (q - ml * QUADS_PER_ROW) * 16 + (tid & 3) * 4;
-            const int m = m0 + ml, n = n0 + nl;
-            if (m >= p.m || n >= p.n) continue;
-            int corr = 0;
-            if (p.zw != 0) {
+        // thread -> pixel row tid & 63, sixteen channels starting at (tid >> 6) * 16
+        const int ml = tid & 63, nl = (tid >> 6) * 16;
+        const int m = m0 + ml, n = n0 + nl;
+        if (m >= p.m || n >= p.n) return;
+        int corr = 0;
+        if (p.zw != 0) {
 #pragma unroll
-                for (int w = 0; w < WGK * 2; ++w) corr += rowsum_s[w][ml];
-                corr *= p.zw;
-            }
-            const int32_t *pr = reinterpret_cast<const int32_t *>(stages) + ml * PART_ROW + nl;
-            int4 s = *reinterpret_cast<const int4 *>(pr);
+            for (int w = 0; w < WGK * 2; ++w) corr += rowsum_s[w][ml];
+            corr *= p.zw;
+        }
+        const int32_t *pr = reinterpret_cast<const int32_t *>(stages) + ml * PART_ROW + nl;
+        uint32_t packed[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            int4 s4 = *reinterpret_cast<const int4 *>(pr + g * 4);
 #pragma unroll
             for (int w = 1; w < WGK; ++w) {
-                const int4 t = *reinterpret_cast<const int4 *>(pr + w * BM * PART_ROW);
-                s.x += t.x;
-                s.y += t.y;
-                s.z += t.z;
-                s.w += t.w;
+                const int4 t = *reinterpret_cast<const int4 *>(pr + g * 4 + w * BM * PART_ROW);
+                s4.x += t.x;
+                s4.y += t.y;
+                s4.z += t.z;
+                s4.w += t.w;
             }
-            const int4 bb = *reinterpret_cast<const int4 *>(p.bias + n);
-            const uint32_t o0 = requant_u8(s.x + bb.x - corr, rq), o1 = requant_u8(s.y + bb.y - corr, rq);
-            const uint32_t o2 = requant_u8(s.z + bb.z - corr, rq), o3 = requant_u8(s.w + bb.w - corr, rq);
-            const uint32_t packed = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
-            const int img = m / plane, r = m - img * plane;
-            const int oy = r / p.wo, ox = r - oy * p.wo;
-            const size_t pix = ((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0);
-            uint8_t *dst = p.out + pix * p.ldc + n;
-            if (wide && n + 4 <= p.n) {
-                *reinterpret_cast<uint32_t *>(dst) = packed;
-            } else {
-                const int cnt = p.n - n < 4 ? p.n - n : 4;
-                for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed >> (8 * t));
-            }
+            const int4 bb = *reinterpret_cast<const int4 *>(bias_s + nl + g * 4);
+            const uint32_t o0 = requant_u8(s4.x + bb.x - corr, rq), o1 = requant_u8(s4.y + bb.y - corr, rq);
+            const uint32_t o2 = requant_u8(s4.z + bb.z - corr, rq), o3 = requant_u8(s4.w + bb.w - corr, rq);
+            packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+        }
+        uint8_t *dst = p.out + out_pixel_offset(p, m, plane) + n;
+        const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+        if (aligned16 && n + 16 <= p.n) {
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+        } else {
+            const int cnt = p.n - n < 16 ? p.n - n : 16;
+            for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
         }
     }
 }
 
 template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES>
 int launch_cfg(const GemmProblem &p, hipStream_t stream) {
+    static_assert(STAGES * (BM + BN) * SLAB + WGK * 2 * BM * 4 + BN * 4 <= 160 * 1024 - 12288, "LDS budget with the largest k-table");
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     // group shape gm x (32 / gm): least operand rows per group among the shapes that fit the tile grid
     int gm = 1;
@@ -345,8 +388,12 @@ int launch_cfg(const GemmProblem &p, hipStream_t stream) {
     const int groups = ((tiles_m + gm - 1) / gm) * ((tiles_n + 32 / gm - 1) / (32 / gm));
     const int grid = ((groups + 7) / 8) * 8 * 32;
     const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
-    hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES>), dim3(grid), dim3(256), ktab_bytes, stream, p,
-                       tiles_m, tiles_n, gm);
+    if (p.dense)
+        hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true>), dim3(grid), dim3(256), 0, stream,
+                           p, tiles_m, tiles_n, gm);
+    else
+        hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false>), dim3(grid), dim3(256), ktab_bytes,
+                           stream, p, tiles_m, tiles_n, gm);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }
@@ -387,8 +434,8 @@ int launch_igemm_dma(const GemmProblem &p, hipStream_t stream) {
     switch (p.cfg.id) {
         case GEMM_DMA_256x256: return launch_cfg<256, 256, 2, 2, 1, 128, 2>(p, stream);
         case GEMM_DMA_256x128: return launch_cfg<256, 128, 2, 2, 1, 128, 3>(p, stream);
-        case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 4>(p, stream);
-        case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 4>(p, stream);
+        case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 2>(p, stream);
+        case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 3>(p, stream);
         case GEMM_DMA_64x64_SPLITK: return launch_cfg<64, 64, 1, 1, 4, 256, 4>(p, stream);
         default: break;
     }

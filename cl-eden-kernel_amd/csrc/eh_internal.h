@@ -35,6 +35,8 @@ struct RequantDev {
     int32_t multiplier;
     int32_t left_shift;
     int32_t right_shift;
+    int32_t mask;  // (1 << right_shift) - 1
+    int32_t half;  // mask >> 1
     int32_t zp_out;
     int32_t act_min;
     int32_t act_max;
@@ -46,11 +48,11 @@ __device__ __forceinline__ int32_t requant_core(int32_t acc, const RequantDev &r
     // (ab + nudge) / 2^31 with nudge = ab >= 0 ? 2^30 : 1 - 2^30 and C truncation
     // is floor((ab + 2^30) / 2^31) for every ab; the multiplier is never
     // INT32_MIN (the host rejects negative multipliers), so no saturation case.
-    const int64_t ab = (int64_t)x * (int64_t)r.multiplier;
-    const int32_t v = (int32_t)((ab + (1ll << 30)) >> 31);
-    const int32_t mask = (int32_t)((1u << r.right_shift) - 1u);
-    const int32_t rem = v & mask;
-    const int32_t thr = (mask >> 1) + (v < 0 ? 1 : 0);
+    const int64_t ab = (int64_t)x * (int64_t)r.multiplier + (1ll << 30);
+    const int32_t v = (int32_t)(ab >> 31);
+    // rounding divide by 2^rs: remainder > (mask >> 1) + (v < 0)
+    const int32_t rem = v & r.mask;
+    const int32_t thr = r.half - (v >> 31);
     return (v >> r.right_shift) + (rem > thr ? 1 : 0);
 }
 
@@ -66,11 +68,28 @@ inline RequantDev make_requant_dev(const eh_requant &q) {
     r.multiplier = q.multiplier;
     r.left_shift = q.shift > 0 ? q.shift : 0;
     r.right_shift = q.shift > 0 ? 0 : -q.shift;
+    r.mask = (int32_t)((1u << r.right_shift) - 1u);
+    r.half = r.mask >> 1;
     r.zp_out = q.zp_out;
     r.act_min = q.act_min;
     r.act_max = q.act_max;
     return r;
 }
+
+// floor(n / d) for 0 <= n < 2^31 as (umulhi(mul, n) + n) >> shift
+struct FastDiv {
+    uint32_t mul = 1;
+    uint32_t shift = 0;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    f.shift = l;
+    f.mul = (uint32_t)((((1ull << 32) * ((1ull << l) - d)) / d + 1) & 0xFFFFFFFFull);
+    return f;
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) { return (__umulhi(f.mul, n) + n) >> f.shift; }
 
 int check_requant(const eh_requant *q);
 
@@ -115,6 +134,8 @@ struct GemmProblem {
     int32_t stride_h, stride_w, y_base, x_base;
     // output addressing: ((img * out_h + oy * out_sy + out_y0) * out_w + ox * out_sx + out_x0) * ldc + col
     int32_t out_h, out_w, out_sy, out_sx, out_y0, out_x0, ldc;
+    FastDiv div_plane, div_wo;  // row decode: m / (ho * wo), rem / wo
+    int32_t dense;     // 1: a plain [m][k] matrix with row stride cin and k a multiple of the slab (no taps, no padding)
     int32_t zw;        // zp_w - 128: coefficient of the per-row activation sum
     uint32_t fill;     // input zero point replicated in 4 bytes (value of an out-of-image tap)
     RequantDev rq;
