@@ -1,0 +1,488 @@
+// Operator classes of the HIP userdriver backend for the quantized path:
+// Convolution, DepthwiseConvolution, FullyConnected, Deconvolution on uint8 tensors.
+//
+// Each class keeps the reference operator surface: constructed from
+// (runtime, precision); initialize({input, weight, bias}, {output}, parameters);
+// execute(); release(); every call returns Status and logs instead of throwing.
+// Reference counterparts: CLConvolution (src/userdriver/gpu/operators/CLConvolution.hpp:31-66,
+// CLConvolution.cpp:34-550), CLDepthwiseConvolution (CLDepthwiseConvolution.hpp:18-38,
+// .cpp:88-425), CLFullyConnected (CLFullyConnected.hpp:21-35, .cpp:22-150),
+// CLDeconvolution (CLDeconvolution.hpp:20-40, .cpp:36-272).
+//
+// Behaviour kept from the reference: quantization parameters are read from the
+// tensors on every execute(); constant weights are packed once in initialize(),
+// weights that are run-time inputs (is_const() == false) are re-packed on every
+// execute(); a bias scale that does not match input_scale * filter_scale leaves
+// the multiplier at zero (every output is the clamped output zero point); an
+// empty weight or input tensor makes initialize()/execute() succeed without work;
+// in channels-last mode (isNCHW == false) a tensor's Dim4 holds (n, h, w, c)
+// positionally; in androidNN mode the weight Dim4 holds (out, kh, kw, in).
+// Not offered here: per-channel quantized weights, INT8 precision, float
+// precisions, texture storage (initialize() returns FAILURE for them).
+#pragma once
+
+#include <memory>
+#include <vector>
+
+#include "ActivationInfo.hpp"
+#include "HipTensor.hpp"
+
+namespace enn {
+namespace ud {
+namespace hip {
+
+#define INPUT_INDEX 0
+#define WEIGHT_INDEX 1
+#define BIAS_INDEX 2
+#define OUTPUT_INDEX 0
+
+struct Parameters {
+    virtual ~Parameters() {}
+};
+
+struct ConvolutionParameters : public Parameters {
+    Pad4 padding = {0, 0, 0, 0};
+    Dim2 dilation = {1, 1};
+    Dim2 stride = {1, 1};
+    uint32_t group_size = 1;
+    uint32_t axis = 0;
+    bool per_channel_quant = false;
+    bool androidNN = false;
+    bool isNCHW = true;
+    StorageType storage_type = StorageType::BUFFER;
+    bool openAibWino = false;
+    std::shared_ptr<ActivationInfo> activation_info = std::make_shared<ActivationInfo>();
+    std::vector<float> scales;
+};
+
+struct DepthwiseConvolutionParameters : public Parameters {
+    Pad4 padding = {0, 0, 0, 0};
+    Dim2 dilation = {1, 1};
+    Dim2 stride = {1, 1};
+    uint32_t depth_multiplier = 1;
+    bool per_channel_quant = false;
+    bool androidNN = false;
+    bool isNCHW = true;
+    StorageType storage_type = StorageType::BUFFER;
+    std::shared_ptr<ActivationInfo> activation_info = std::make_shared<ActivationInfo>();
+    std::vector<float> scales;
+};
+
+struct FullyConnectedParameters : public Parameters {
+    bool androidNN = false;
+    StorageType storage_type = StorageType::BUFFER;
+    std::shared_ptr<ActivationInfo> activation_info = std::make_shared<ActivationInfo>();
+};
+
+struct DeconvolutionParameters : public Parameters {
+    Pad4 padding = {0, 0, 0, 0};
+    Dim2 stride = {1, 1};
+    uint32_t group_size = 1;
+    bool weights_as_input = false;
+    bool per_channel_quant = false;
+    bool androidNN = false;
+    bool isNCHW = true;
+    bool openAibWino = false;
+    std::shared_ptr<ActivationInfo> activation_info = std::make_shared<ActivationInfo>();
+    std::vector<float> scales;
+};
+
+namespace detail {
+
+inline int toEhActivation(const ActivationInfo &a) {
+    switch (a.activation()) {
+        case ActivationInfo::ActivationType::RELU: return EH_ACT_RELU;
+        case ActivationInfo::ActivationType::RELU1: return EH_ACT_RELU1;
+        case ActivationInfo::ActivationType::RELU6: return EH_ACT_RELU6;
+        default: return EH_ACT_NONE;
+    }
+}
+
+// What the reference's quantized operators compute at the top of execute()
+// (cl_optimized_impls/CLGEMMConvolutionQuantized.cpp:137-171).
+inline eh_requant requantFromTensors(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &w,
+                                     const std::shared_ptr<HipTensor> &bias, const std::shared_ptr<HipTensor> &out,
+                                     const ActivationInfo &act) {
+    eh_requant q;
+    eh_make_requant(in->getScale(), in->getZeroPoint(), w->getScale(), w->getZeroPoint(), bias->getScale(), out->getScale(),
+                    out->getZeroPoint(), toEhActivation(act), act.isEnabled() ? 1 : 0, &q);
+    return q;
+}
+
+inline bool uint8Tensors(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &w,
+                         const std::shared_ptr<HipTensor> &bias, const std::shared_ptr<HipTensor> &out) {
+    return in->getDataType() == DataType::UINT8 && w->getDataType() == DataType::UINT8 &&
+           bias->getDataType() == DataType::INT32 && out->getDataType() == DataType::UINT8;
+}
+
+}  // namespace detail
+
+class HipConvolution {
+public:
+    HipConvolution(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision)
+        : runtime_(runtime), precision_(precision) {}
+    ~HipConvolution() { release(); }
+
+    Status initialize(std::vector<std::shared_ptr<ITensor>> inputs, std::vector<std::shared_ptr<ITensor>> outputs,
+                      std::shared_ptr<Parameters> parameters) {
+        CHECK_EXPR_RETURN_FAILURE(inputs.size() >= 3 && outputs.size() >= 1, "HipConvolution: needs {input, weight, bias} and {output}");
+        input_ = std::static_pointer_cast<HipTensor>(inputs.at(INPUT_INDEX));
+        weight_ = std::static_pointer_cast<HipTensor>(inputs.at(WEIGHT_INDEX));
+        bias_ = std::static_pointer_cast<HipTensor>(inputs.at(BIAS_INDEX));
+        output_ = std::static_pointer_cast<HipTensor>(outputs.at(OUTPUT_INDEX));
+        parameters_ = std::dynamic_pointer_cast<ConvolutionParameters>(parameters);
+        CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipConvolution: parameters are not ConvolutionParameters");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->activation_info != nullptr, "HipConvolution: null activation info");
+        activation_info_ = *parameters_->activation_info;
+        weights_as_input_ = !weight_->is_const();
+        bias_as_input_ = !bias_->is_const();
+
+        if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;  // zero-sized: nothing to prepare
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipConvolution: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipConvolution: no texture storage");
+        CHECK_EXPR_RETURN_FAILURE(!parameters_->per_channel_quant, "HipConvolution: per-channel quantization is not offered");
+        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipConvolution: expects uint8 input/weight/output and int32 bias");
+
+        Dim4 in = input_->getDim(), wd = weight_->getDim();
+        if (!parameters_->isNCHW) in = convertDimToNCHW(in);
+        const bool ohwi = parameters_->androidNN || !parameters_->isNCHW;  // weight Dim4 = (out, kh, kw, in)
+        const uint32_t cout = wd.n, kh = ohwi ? wd.c : wd.h, kw = ohwi ? wd.h : wd.w, cin_g = ohwi ? wd.w : wd.c;
+        CHECK_EXPR_RETURN_FAILURE(cin_g != 0 && in.c % cin_g == 0, "HipConvolution: weight channels %u do not divide input channels %u", cin_g, in.c);
+        const uint32_t groups = ohwi ? in.c / cin_g : parameters_->group_size;
+        CHECK_EXPR_RETURN_FAILURE(groups != 0 && in.c == cin_g * groups, "HipConvolution: group size %u does not match the weight shape", groups);
+
+        eh_conv_desc d;
+        d.n = (int32_t)in.n;
+        d.c = (int32_t)in.c;
+        d.h = (int32_t)in.h;
+        d.w = (int32_t)in.w;
+        d.cout = (int32_t)cout;
+        d.kh = (int32_t)kh;
+        d.kw = (int32_t)kw;
+        d.stride_h = (int32_t)parameters_->stride.h;
+        d.stride_w = (int32_t)parameters_->stride.w;
+        d.pad_t = (int32_t)parameters_->padding.t;
+        d.pad_b = (int32_t)parameters_->padding.b;
+        d.pad_l = (int32_t)parameters_->padding.l;
+        d.pad_r = (int32_t)parameters_->padding.r;
+        d.dil_h = (int32_t)parameters_->dilation.h;
+        d.dil_w = (int32_t)parameters_->dilation.w;
+        d.groups = (int32_t)groups;
+        d.depth_multiplier = 1;
+        d.layout = parameters_->isNCHW ? EH_NCHW : EH_NHWC;
+        d.weight_layout = ohwi ? EH_W_OHWI : EH_W_OIHW;
+        desc_ = d;
+        const int32_t ho = eh_conv_out_dim(d.h, d.pad_t, d.pad_b, d.kh, d.dil_h, d.stride_h);
+        const int32_t wo = eh_conv_out_dim(d.w, d.pad_l, d.pad_r, d.kw, d.dil_w, d.stride_w);
+        CHECK_EXPR_RETURN_FAILURE((int64_t)output_->getTotalSizeFromDims() == (int64_t)d.n * d.cout * ho * wo,
+                                  "HipConvolution: output tensor has %u elements, the geometry gives %lld", output_->getTotalSizeFromDims(),
+                                  (long long)d.n * d.cout * ho * wo);
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        const int rc = eh_conv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::initialize: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status execute() {
+        if (plan_ == nullptr) {  // zero-sized operator
+            CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipConvolution::execute before initialize");
+            return Status::SUCCESS;
+        }
+        if (input_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        if (weights_as_input_ || bias_as_input_) {
+            const int rc = eh_conv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute (repack): %s", eh_last_error());
+        }
+        const int rc = eh_conv2d_u8_run(plan_, input_->getDataPtr(), output_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status release() {
+        if (plan_) {
+            (void)runtime_->synchronize();
+            eh_conv2d_u8_destroy(plan_);
+            plan_ = nullptr;
+        }
+        return Status::SUCCESS;
+    }
+
+private:
+    std::shared_ptr<HipRuntime> runtime_;
+    PrecisionType precision_;
+    std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
+    std::shared_ptr<ConvolutionParameters> parameters_;
+    ActivationInfo activation_info_;
+    bool weights_as_input_ = false, bias_as_input_ = false;
+    eh_conv_desc desc_{};
+    eh_conv_plan *plan_ = nullptr;
+};
+
+class HipDepthwiseConvolution {
+public:
+    HipDepthwiseConvolution(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision)
+        : runtime_(runtime), precision_(precision) {}
+    ~HipDepthwiseConvolution() { release(); }
+
+    Status initialize(std::vector<std::shared_ptr<ITensor>> inputs, std::vector<std::shared_ptr<ITensor>> outputs,
+                      std::shared_ptr<Parameters> parameters) {
+        CHECK_EXPR_RETURN_FAILURE(inputs.size() >= 3 && outputs.size() >= 1, "HipDepthwiseConvolution: needs {input, weight, bias} and {output}");
+        input_ = std::static_pointer_cast<HipTensor>(inputs.at(INPUT_INDEX));
+        weight_ = std::static_pointer_cast<HipTensor>(inputs.at(WEIGHT_INDEX));
+        bias_ = std::static_pointer_cast<HipTensor>(inputs.at(BIAS_INDEX));
+        output_ = std::static_pointer_cast<HipTensor>(outputs.at(OUTPUT_INDEX));
+        parameters_ = std::dynamic_pointer_cast<DepthwiseConvolutionParameters>(parameters);
+        CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipDepthwiseConvolution: parameters are not DepthwiseConvolutionParameters");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->activation_info != nullptr, "HipDepthwiseConvolution: null activation info");
+        activation_info_ = *parameters_->activation_info;
+        weights_as_input_ = !weight_->is_const() || !bias_->is_const();
+
+        if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipDepthwiseConvolution: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipDepthwiseConvolution: no texture storage");
+        CHECK_EXPR_RETURN_FAILURE(!parameters_->per_channel_quant, "HipDepthwiseConvolution: per-channel quantization is not offered");
+        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDepthwiseConvolution: expects uint8 input/weight/output and int32 bias");
+
+        Dim4 in = input_->getDim();
+        if (!parameters_->isNCHW) in = convertDimToNCHW(in);
+        const Dim4 wd = weight_->getDim();  // [C * depth_multiplier][1][kh][kw]
+        eh_conv_desc d;
+        d.n = (int32_t)in.n;
+        d.c = (int32_t)in.c;
+        d.h = (int32_t)in.h;
+        d.w = (int32_t)in.w;
+        d.cout = (int32_t)(in.c * parameters_->depth_multiplier);
+        d.kh = (int32_t)wd.h;
+        d.kw = (int32_t)wd.w;
+        d.stride_h = (int32_t)parameters_->stride.h;
+        d.stride_w = (int32_t)parameters_->stride.w;
+        d.pad_t = (int32_t)parameters_->padding.t;
+        d.pad_b = (int32_t)parameters_->padding.b;
+        d.pad_l = (int32_t)parameters_->padding.l;
+        d.pad_r = (int32_t)parameters_->padding.r;
+        d.dil_h = (int32_t)parameters_->dilation.h;
+        d.dil_w = (int32_t)parameters_->dilation.w;
+        d.groups = 1;
+        d.depth_multiplier = (int32_t)parameters_->depth_multiplier;
+        d.layout = parameters_->isNCHW ? EH_NCHW : EH_NHWC;
+        d.weight_layout = EH_W_OIHW;
+        CHECK_EXPR_RETURN_FAILURE(wd.n == (uint32_t)d.cout && wd.c == 1, "HipDepthwiseConvolution: weight shape [%u %u %u %u] is not [C*dm][1][kh][kw]", wd.n, wd.c, wd.h, wd.w);
+        desc_ = d;
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        const int rc = eh_dwconv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDepthwiseConvolution::initialize: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status execute() {
+        if (plan_ == nullptr) {
+            CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipDepthwiseConvolution::execute before initialize");
+            return Status::SUCCESS;
+        }
+        if (input_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        if (weights_as_input_) {
+            const int rc = eh_dwconv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDepthwiseConvolution::execute (repack): %s", eh_last_error());
+        }
+        const int rc = eh_dwconv2d_u8_run(plan_, input_->getDataPtr(), output_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDepthwiseConvolution::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status release() {
+        if (plan_) {
+            (void)runtime_->synchronize();
+            eh_dwconv2d_u8_destroy(plan_);
+            plan_ = nullptr;
+        }
+        return Status::SUCCESS;
+    }
+
+private:
+    std::shared_ptr<HipRuntime> runtime_;
+    PrecisionType precision_;
+    std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
+    std::shared_ptr<DepthwiseConvolutionParameters> parameters_;
+    ActivationInfo activation_info_;
+    bool weights_as_input_ = false;
+    eh_conv_desc desc_{};
+    eh_dwconv_plan *plan_ = nullptr;
+};
+
+class HipFullyConnected {
+public:
+    HipFullyConnected(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision)
+        : runtime_(runtime), precision_(precision) {}
+    ~HipFullyConnected() { release(); }
+
+    Status initialize(const std::vector<std::shared_ptr<ITensor>> &input_tensors,
+                      const std::vector<std::shared_ptr<ITensor>> &output_tensors, const std::shared_ptr<Parameters> parameters) {
+        CHECK_EXPR_RETURN_FAILURE(input_tensors.size() >= 3 && output_tensors.size() >= 1, "HipFullyConnected: needs {input, weight, bias} and {output}");
+        input_ = std::static_pointer_cast<HipTensor>(input_tensors.at(INPUT_INDEX));
+        weight_ = std::static_pointer_cast<HipTensor>(input_tensors.at(WEIGHT_INDEX));
+        bias_ = std::static_pointer_cast<HipTensor>(input_tensors.at(BIAS_INDEX));
+        output_ = std::static_pointer_cast<HipTensor>(output_tensors.at(OUTPUT_INDEX));
+        parameters_ = std::dynamic_pointer_cast<FullyConnectedParameters>(parameters);
+        CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipFullyConnected: parameters are not FullyConnectedParameters");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->activation_info != nullptr, "HipFullyConnected: null activation info");
+        activation_info_ = *parameters_->activation_info;
+        weights_as_input_ = !weight_->is_const() || !bias_->is_const();
+
+        if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipFullyConnected: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipFullyConnected: no texture storage");
+        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipFullyConnected: expects uint8 input/weight/output and int32 bias");
+        // weight [units][k]; the input is flattened to [size / k][k]
+        // (CLFullyConnected.cpp:46-57: in androidNN mode the batch is whatever the element count gives)
+        const Dim4 wd = weight_->getDim();
+        const uint32_t units = wd.n, k = wd.c * wd.h * wd.w;
+        CHECK_EXPR_RETURN_FAILURE(k != 0 && input_->getTotalSizeFromDims() % k == 0, "HipFullyConnected: input of %u elements is not a multiple of k = %u", input_->getTotalSizeFromDims(), k);
+        const uint32_t m = input_->getTotalSizeFromDims() / k;
+        CHECK_EXPR_RETURN_FAILURE(parameters_->androidNN || m == input_->getDim().n, "HipFullyConnected: input batch %u does not match %u rows of k = %u", input_->getDim().n, m, k);
+        CHECK_EXPR_RETURN_FAILURE(output_->getTotalSizeFromDims() == m * units, "HipFullyConnected: output has %u elements, expected %u", output_->getTotalSizeFromDims(), m * units);
+        m_ = (int32_t)m;
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        const int rc = eh_fc_u8_plan(&plan_, (int32_t)m, (int32_t)k, (int32_t)units, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipFullyConnected::initialize: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status execute() {
+        if (plan_ == nullptr) {
+            CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipFullyConnected::execute before initialize");
+            return Status::SUCCESS;
+        }
+        if (m_ == 0) return Status::SUCCESS;
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        if (weights_as_input_) {
+            const int rc = eh_fc_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipFullyConnected::execute (repack): %s", eh_last_error());
+        }
+        const int rc = eh_fc_u8_run(plan_, input_->getDataPtr(), output_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipFullyConnected::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status release() {
+        if (plan_) {
+            (void)runtime_->synchronize();
+            eh_fc_u8_destroy(plan_);
+            plan_ = nullptr;
+        }
+        return Status::SUCCESS;
+    }
+
+private:
+    std::shared_ptr<HipRuntime> runtime_;
+    PrecisionType precision_;
+    std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
+    std::shared_ptr<FullyConnectedParameters> parameters_;
+    ActivationInfo activation_info_;
+    bool weights_as_input_ = false;
+    int32_t m_ = 0;
+    eh_fc_plan *plan_ = nullptr;
+};
+
+class HipDeconvolution {
+public:
+    HipDeconvolution(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision)
+        : runtime_(runtime), precision_(precision) {}
+    ~HipDeconvolution() { release(); }
+
+    Status initialize(std::vector<std::shared_ptr<ITensor>> inputs_tensors, std::vector<std::shared_ptr<ITensor>> outputs_tensors,
+                      std::shared_ptr<Parameters> parameters) {
+        CHECK_EXPR_RETURN_FAILURE(inputs_tensors.size() >= 3 && outputs_tensors.size() >= 1, "HipDeconvolution: needs {input, weight, bias} and {output}");
+        input_ = std::static_pointer_cast<HipTensor>(inputs_tensors.at(INPUT_INDEX));
+        weight_ = std::static_pointer_cast<HipTensor>(inputs_tensors.at(WEIGHT_INDEX));
+        bias_ = std::static_pointer_cast<HipTensor>(inputs_tensors.at(BIAS_INDEX));
+        output_ = std::static_pointer_cast<HipTensor>(outputs_tensors.at(OUTPUT_INDEX));
+        parameters_ = std::dynamic_pointer_cast<DeconvolutionParameters>(parameters);
+        CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipDeconvolution: parameters are not DeconvolutionParameters");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->activation_info != nullptr, "HipDeconvolution: null activation info");
+        activation_info_ = *parameters_->activation_info;
+        weights_as_input_ = parameters_->weights_as_input || !weight_->is_const() || !bias_->is_const();
+
+        if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipDeconvolution: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(!parameters_->per_channel_quant, "HipDeconvolution: per-channel quantization is not offered");
+        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDeconvolution: expects uint8 input/weight/output and int32 bias");
+
+        Dim4 in = input_->getDim();
+        if (!parameters_->isNCHW) in = convertDimToNCHW(in);
+        const Dim4 wd = weight_->getDim();
+        const bool nn = parameters_->androidNN;  // weight Dim4 = (out, kh, kw, in); otherwise (in, out / groups, kh, kw)
+        const uint32_t groups = nn ? 1 : parameters_->group_size;
+        eh_conv_desc d;
+        d.n = (int32_t)in.n;
+        d.c = (int32_t)in.c;
+        d.h = (int32_t)in.h;
+        d.w = (int32_t)in.w;
+        d.cout = (int32_t)(nn ? wd.n : wd.c * groups);
+        d.kh = (int32_t)(nn ? wd.c : wd.h);
+        d.kw = (int32_t)(nn ? wd.h : wd.w);
+        d.stride_h = (int32_t)parameters_->stride.h;
+        d.stride_w = (int32_t)parameters_->stride.w;
+        d.pad_t = (int32_t)parameters_->padding.t;
+        d.pad_b = (int32_t)parameters_->padding.b;
+        d.pad_l = (int32_t)parameters_->padding.l;
+        d.pad_r = (int32_t)parameters_->padding.r;
+        d.dil_h = 1;
+        d.dil_w = 1;
+        d.groups = (int32_t)groups;
+        d.depth_multiplier = 1;
+        d.layout = parameters_->isNCHW ? EH_NCHW : EH_NHWC;
+        d.weight_layout = nn ? EH_W_OHWI : EH_W_IOHW;
+        CHECK_EXPR_RETURN_FAILURE((nn ? wd.w : wd.n) == in.c, "HipDeconvolution: weight input channels %u do not match the input's %u", nn ? wd.w : wd.n, in.c);
+        desc_ = d;
+        const int32_t oh = eh_deconv_out_dim(d.h, d.pad_t, d.pad_b, d.kh, d.stride_h);
+        const int32_t ow = eh_deconv_out_dim(d.w, d.pad_l, d.pad_r, d.kw, d.stride_w);
+        CHECK_EXPR_RETURN_FAILURE((int64_t)output_->getTotalSizeFromDims() == (int64_t)d.n * d.cout * oh * ow,
+                                  "HipDeconvolution: output tensor has %u elements, the geometry gives %lld", output_->getTotalSizeFromDims(),
+                                  (long long)d.n * d.cout * oh * ow);
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        const int rc = eh_deconv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDeconvolution::initialize: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status execute() {
+        if (plan_ == nullptr) {
+            CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipDeconvolution::execute before initialize");
+            return Status::SUCCESS;
+        }
+        if (input_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
+        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        if (weights_as_input_) {
+            const int rc = eh_deconv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDeconvolution::execute (repack): %s", eh_last_error());
+        }
+        const int rc = eh_deconv2d_u8_run(plan_, input_->getDataPtr(), output_->getDataPtr(), &q, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDeconvolution::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status release() {
+        if (plan_) {
+            (void)runtime_->synchronize();
+            eh_deconv2d_u8_destroy(plan_);
+            plan_ = nullptr;
+        }
+        return Status::SUCCESS;
+    }
+
+private:
+    std::shared_ptr<HipRuntime> runtime_;
+    PrecisionType precision_;
+    std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
+    std::shared_ptr<DeconvolutionParameters> parameters_;
+    ActivationInfo activation_info_;
+    bool weights_as_input_ = false;
+    eh_conv_desc desc_{};
+    eh_deconv_plan *plan_ = nullptr;
+};
+
+}  // namespace hip
+}  // namespace ud
+}  // namespace enn

@@ -1,0 +1,210 @@
+// Tensor of the HIP userdriver backend: dims, data order, element type and the
+// per-tensor quantization parameters (scale, zero point) the operators read at
+// execute time, over a HipBuffer.
+//
+// Mirrors CLTensor (src/userdriver/gpu/common/CLTensor.hpp:40-152 constructors:
+// a shape-only tensor is a run-time input/output, a tensor built from host data is
+// a constant; CLTensor.cpp:181-225 layout conversion; destructor :268-276).
+#pragma once
+
+#include <cstring>
+#include <string>
+#include <typeinfo>
+#include <vector>
+
+#include "HipRuntime.hpp"
+#include "ITensor.hpp"
+
+namespace enn {
+namespace ud {
+namespace hip {
+
+template <typename T> struct data_type_of;
+template <> struct data_type_of<uint8_t> { static constexpr DataType value = DataType::UINT8; };
+template <> struct data_type_of<int8_t> { static constexpr DataType value = DataType::INT8; };
+template <> struct data_type_of<int32_t> { static constexpr DataType value = DataType::INT32; };
+template <> struct data_type_of<float> { static constexpr DataType value = DataType::FLOAT; };
+
+class HipTensor : public ITensor {
+public:
+    // run-time tensor (input, output, intermediate)
+    HipTensor(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision, const DataType &data_type,
+              const Dim4 &dim, const DataOrder &data_order = DataOrder::NCHW, const float &scale = 1.0f,
+              const int32_t &zero_point = 0, const BufferType &buffer_type = BufferType::DEDICATED,
+              const StorageType &storage_type = StorageType::BUFFER, const uint32_t buffer_data_type = 0,
+              const int32_t buffer_index = UNDEFINED)
+        : runtime_(runtime), precision_(precision), data_type_(data_type), dims_(dim), vdims_({dim.n, dim.c, dim.h, dim.w}),
+          order_(data_order), scale_(scale), zero_point_(zero_point), buffer_type_(buffer_type), storage_type_(storage_type),
+          buffer_data_type_(buffer_data_type), buffer_index_(buffer_index), is_const_(false) {
+        buf_ = runtime_->getBuffer(precision_, data_type_, dims_, buffer_type_, storage_type_);
+    }
+
+    // constant tensor (weights, bias): uploaded at construction
+    template <typename T>
+    HipTensor(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision, T *data, const Dim4 &dims,
+              const DataOrder &data_order = DataOrder::NCHW, const float &scale = 1.0f, const int32_t &zero_point = 0,
+              const BufferType &buffer_type = BufferType::DEDICATED, const StorageType &storage_type = StorageType::BUFFER,
+              const uint32_t buffer_data_type = 0, const int32_t buffer_index = UNDEFINED)
+        : runtime_(runtime), precision_(precision), data_type_(data_type_of<typename std::remove_const<T>::type>::value),
+          dims_(dims), vdims_({dims.n, dims.c, dims.h, dims.w}), order_(data_order), scale_(scale), zero_point_(zero_point),
+          buffer_type_(buffer_type), storage_type_(storage_type), buffer_data_type_(buffer_data_type),
+          buffer_index_(buffer_index), is_const_(true) {
+        buf_ = std::make_shared<HipBuffer>(getNumOfBytes());
+        buf_->assignBuffer(runtime_->allocBuffer(getNumOfBytes(), false));
+        if (getNumOfBytes())
+            (void)runtime_->writeBuffer(buf_->getDataPtr(), data, getTypeBytes(data_type_, precision_), getTotalSizeFromDims(),
+                                        true);
+    }
+
+    ~HipTensor() override {
+        if (buf_ && buf_.use_count() == 1 && buf_->getDataPtr() != nullptr) (void)runtime_->releaseBuffer(buf_);
+    }
+
+    size_t getNumOfBytes() override { return getTypeBytes(data_type_, precision_) * (size_t)getTotalSizeFromDims(); }
+    DataType getDataType() override { return data_type_; }
+    PrecisionType getPrecisionType() override { return precision_; }
+    const Dim4 &getDim() override { return dims_; }
+    const NDims &getDims() override { return vdims_; }
+    uint32_t getDims(const int32_t &idx) override { return idx >= 0 && (size_t)idx < vdims_.size() ? vdims_[idx] : 0; }
+    uint32_t getNumOfDims() override { return (uint32_t)vdims_.size(); }
+    uint32_t getTotalSizeFromDims() override { return getTensorSizeFromDims(vdims_); }
+    DataOrder getDataOrder() override { return order_; }
+    float getScale() override { return scale_; }
+    int32_t getZeroPoint() override { return zero_point_; }
+    void setZeroPoint(int32_t zero_point) override { zero_point_ = zero_point; }
+    void setScale(float scale) override { scale_ = scale; }
+    void set_buffer_index(int32_t index) override { buffer_index_ = index; }
+    int32_t get_buffer_index() override { return buffer_index_; }
+    void set_buffer_type(uint32_t type) override { buffer_data_type_ = type; }
+    uint32_t get_buffer_type() override { return buffer_data_type_; }
+    void set_buffer_ptr(void *addr) override { raw_buffer = addr; }
+    bool is_const() override { return is_const_; }
+
+    void *getDataPtr() { return buf_ ? buf_->getDataPtr() : nullptr; }
+    std::shared_ptr<HipBuffer> getBuffer() { return buf_; }
+    BufferType getBufferType() const { return buffer_type_; }
+
+    // Host -> device, converting the element order on the way when asked to
+    // (the reference reorders host NHWC data into its planar device tensors).
+    Status writeData(DataPtr data, bool blocking = true, DataOrderChangeType type = DataOrderChangeType::OTHER) override {
+        CHECK_EXPR_RETURN_FAILURE(getDataPtr() != nullptr || getNumOfBytes() == 0, "HipTensor::writeData: no device buffer");
+        if (getNumOfBytes() == 0) return Status::SUCCESS;
+        if (type == DataOrderChangeType::OTHER)
+            return runtime_->writeBuffer(getDataPtr(), data, getTypeBytes(data_type_, precision_), getTotalSizeFromDims(),
+                                         blocking);
+        CHECK_EXPR_RETURN_FAILURE(getTypeBytes(data_type_, precision_) == 1, "layout conversion is byte tensors only");
+        CHECK_EXPR_RETURN_FAILURE(type == DataOrderChangeType::NHWC2NCHW || type == DataOrderChangeType::NCHW2NHWC,
+                                  "HipTensor::writeData: unsupported order change");
+        void *tmp = runtime_->allocBuffer(getNumOfBytes(), false);
+        CHECK_EXPR_RETURN_FAILURE(tmp != nullptr, "HipTensor::writeData: staging allocation failed");
+        Status st = runtime_->writeBuffer(tmp, data, 1, getTotalSizeFromDims(), true);
+        if (st == Status::SUCCESS)
+            st = type == DataOrderChangeType::NHWC2NCHW ? runtime_->NHWC2NCHW(tmp, getDataPtr(), dims_)
+                                                        : runtime_->NCHW2NHWC(tmp, getDataPtr(), dims_);
+        auto holder = std::make_shared<HipBuffer>(getNumOfBytes());
+        holder->assignBuffer(tmp);
+        (void)runtime_->releaseBuffer(holder);  // synchronises first
+        return st;
+    }
+
+    Status readData(DataPtr data, bool blocking = true, DataOrderChangeType type = DataOrderChangeType::OTHER,
+                    void *event = nullptr) override {
+        (void)event;
+        if (getNumOfBytes() == 0) return Status::SUCCESS;
+        CHECK_EXPR_RETURN_FAILURE(getDataPtr() != nullptr, "HipTensor::readData: no device buffer");
+        if (type == DataOrderChangeType::OTHER)
+            return runtime_->readBuffer(data, getDataPtr(), getTypeBytes(data_type_, precision_), getTotalSizeFromDims(), blocking);
+        CHECK_EXPR_RETURN_FAILURE(getTypeBytes(data_type_, precision_) == 1, "layout conversion is byte tensors only");
+        CHECK_EXPR_RETURN_FAILURE(type == DataOrderChangeType::NHWC2NCHW || type == DataOrderChangeType::NCHW2NHWC,
+                                  "HipTensor::readData: unsupported order change");
+        void *tmp = runtime_->allocBuffer(getNumOfBytes(), false);
+        CHECK_EXPR_RETURN_FAILURE(tmp != nullptr, "HipTensor::readData: staging allocation failed");
+        Status st = type == DataOrderChangeType::NHWC2NCHW ? runtime_->NHWC2NCHW(getDataPtr(), tmp, dims_)
+                                                           : runtime_->NCHW2NHWC(getDataPtr(), tmp, dims_);
+        if (st == Status::SUCCESS) st = runtime_->readBuffer(data, tmp, 1, getTotalSizeFromDims(), true);
+        auto holder = std::make_shared<HipBuffer>(getNumOfBytes());
+        holder->assignBuffer(tmp);
+        (void)runtime_->releaseBuffer(holder);
+        return st;
+    }
+
+    Status reconfigure(const PrecisionType &precision, const DataOrder &order, const Dim4 &dims, const float &scale,
+                       const int32_t &offset) override {
+        precision_ = precision;
+        order_ = order;
+        scale_ = scale;
+        zero_point_ = offset;
+        return reconfigureDim(dims);
+    }
+    Status reconfigure(const PrecisionType &precision, const DataOrder &order, const NDims &ndim, const float &scale,
+                       const int32_t &offset) override {
+        precision_ = precision;
+        order_ = order;
+        scale_ = scale;
+        zero_point_ = offset;
+        return reconfigureDims(ndim);
+    }
+    Status reconfigureDim(const Dim4 &dims) override {
+        dims_ = dims;
+        vdims_ = {dims.n, dims.c, dims.h, dims.w};
+        return Status::SUCCESS;
+    }
+    Status reconfigureDims(const NDims &ndim) override {
+        vdims_ = ndim;
+        dims_ = extendToDim4(ndim);
+        return Status::SUCCESS;
+    }
+    Status reconfigureDimAndBuffer(const Dim4 &dims) override {
+        reconfigureDim(dims);
+        return growBuffer();
+    }
+    Status reconfigureDimsAndBuffer(const NDims &dims) override {
+        reconfigureDims(dims);
+        return growBuffer();
+    }
+    Status reorder(const DataOrder &order) override {
+        order_ = order;
+        return Status::SUCCESS;
+    }
+    void queryTensorInfo() override {
+        std::fprintf(stderr, "HipTensor dims [%u %u %u %u] order %d type %d scale %g zp %d const %d\n", dims_.n, dims_.c, dims_.h,
+                     dims_.w, (int)order_, (int)data_type_, (double)scale_, zero_point_, (int)is_const_);
+    }
+    void dumpTensorData(std::string file_name) override {
+        std::vector<char> host(getNumOfBytes());
+        if (readData(host.data()) != Status::SUCCESS) return;
+        if (FILE *f = std::fopen(file_name.c_str(), "wb")) {
+            std::fwrite(host.data(), 1, host.size(), f);
+            std::fclose(f);
+        }
+    }
+    Status resetInterBuffer() override { return runtime_->resetInterBuffer(buf_); }
+
+private:
+    Status growBuffer() {
+        if (buf_ && buf_->getDataPtr() && buf_->getBytes() >= getNumOfBytes()) return Status::SUCCESS;
+        if (buf_ && buf_->getDataPtr()) (void)runtime_->releaseBuffer(buf_);
+        buf_ = std::make_shared<HipBuffer>(getNumOfBytes());
+        buf_->assignBuffer(runtime_->allocBuffer(getNumOfBytes(), true));
+        return buf_->getDataPtr() || getNumOfBytes() == 0 ? Status::SUCCESS : Status::FAILURE;
+    }
+
+    std::shared_ptr<HipRuntime> runtime_;
+    PrecisionType precision_;
+    DataType data_type_;
+    Dim4 dims_;
+    NDims vdims_;
+    DataOrder order_;
+    float scale_;
+    int32_t zero_point_;
+    BufferType buffer_type_;
+    StorageType storage_type_;
+    uint32_t buffer_data_type_;
+    int32_t buffer_index_;
+    bool is_const_;
+    std::shared_ptr<HipBuffer> buf_;
+};
+
+}  // namespace hip
+}  // namespace ud
+}  // namespace enn

@@ -1,0 +1,570 @@
+// Operator-level tests of the HIP userdriver backend, shaped like the reference's
+// op tests (src/userdriver/gpu/op_test/convolution_test.cpp:16-267,
+// fullyconnected_test.cpp:12-120): build tensors from host arrays, initialize /
+// execute / release an operator, read the output back and compare it, here bit for
+// bit against the CPU oracle.  The oracle (oracle/eden_oracle.h) is linked into
+// this test program only; the operator classes never see it.
+//
+//   ud_op_test              run everything (needs the GPU)
+//   ud_op_test --host-only  buffer-pool bookkeeping and argument checks that touch no device
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "HipOperators.hpp"
+#include "eden_oracle.h"
+#include "userdriver_operator.hpp"
+
+using namespace enn::ud;
+using namespace enn::ud::hip;
+
+static int g_failed = 0, g_run = 0;
+#define EXPECT(cond)                                                                    \
+    do {                                                                                \
+        if (!(cond)) {                                                                  \
+            std::printf("    EXPECT failed at line %d: %s\n", __LINE__, #cond);        \
+            ok = false;                                                                 \
+        }                                                                               \
+    } while (0)
+
+static void run_test(const char *name, const std::function<bool()> &fn) {
+    std::printf("[ RUN  ] %s\n", name);
+    std::fflush(stdout);
+    ++g_run;
+    const bool ok = fn();
+    if (!ok) ++g_failed;
+    std::printf("[ %s ] %s\n", ok ? " OK " : "FAIL", name);
+    std::fflush(stdout);
+}
+
+static std::vector<uint8_t> rand_u8(size_t n, uint64_t seed, int lo = 0, int hi = 255) {
+    std::vector<uint8_t> v(n);
+    eo_fill_u8(v.data(), (int64_t)n, seed, lo, hi);
+    return v;
+}
+static std::vector<int32_t> rand_i32(size_t n, uint64_t seed, int lo, int hi) {
+    std::vector<int32_t> v(n);
+    eo_fill_i32(v.data(), (int64_t)n, seed, lo, hi);
+    return v;
+}
+static bool same(const std::vector<uint8_t> &a, const std::vector<uint8_t> &b) {
+    if (a.size() != b.size()) return false;
+    size_t bad = 0, first = 0;
+    for (size_t i = 0; i < a.size(); ++i)
+        if (a[i] != b[i] && bad++ == 0) first = i;
+    if (bad) std::printf("    %zu of %zu bytes differ; first at %zu: got %u want %u\n", bad, a.size(), first, a[first], b[first]);
+    return bad == 0;
+}
+static bool varied(const std::vector<uint8_t> &v) {
+    int seen[256] = {0}, distinct = 0;
+    for (uint8_t x : v)
+        if (!seen[x]++) ++distinct;
+    return distinct > 8;
+}
+static std::vector<uint8_t> nchw_to_nhwc(const std::vector<uint8_t> &x, int n, int c, int h, int w) {
+    std::vector<uint8_t> y(x.size());
+    eo_nchw2nhwc_u8(x.data(), y.data(), n, c, h, w);
+    return y;
+}
+static std::vector<uint8_t> nhwc_to_nchw(const std::vector<uint8_t> &x, int n, int c, int h, int w) {
+    std::vector<uint8_t> y(x.size());
+    eo_nhwc2nchw_u8(x.data(), y.data(), n, c, h, w);
+    return y;
+}
+static eo_conv_shape shape(int n, int c, int h, int w, int cout, int kh, int kw, int sh = 1, int sw = 1, int pt = 0, int pb = 0,
+                           int pl = 0, int pr = 0, int dh = 1, int dw = 1, int groups = 1, int dm = 1) {
+    eo_conv_shape s = {n, c, h, w, cout, kh, kw, sh, sw, pt, pb, pl, pr, dh, dw, groups, dm};
+    return s;
+}
+
+static const PrecisionType U8 = PrecisionType::UINT8;
+struct Quant {
+    float s_in, s_w, s_out;
+    int zp_in, zp_w, zp_out;
+    float s_bias() const { return s_in * s_w; }  // float32 product, as a converter would store it
+};
+
+// ---------------------------------------------------------------- convolution
+
+static bool conv_case(const std::shared_ptr<HipRuntime> &rt, const eo_conv_shape &s, const Quant &qt, ActivationInfo act,
+                      bool nchw, bool androidNN, uint64_t seed) {
+    bool ok = true;
+    const int ho = eo_conv_out_dim(s.h, s.pad_t, s.pad_b, s.kh, s.dil_h, s.stride_h);
+    const int wo = eo_conv_out_dim(s.w, s.pad_l, s.pad_r, s.kw, s.dil_w, s.stride_w);
+    const int cig = s.c / s.groups;
+    auto x = rand_u8((size_t)s.n * s.c * s.h * s.w, seed);
+    auto w = rand_u8((size_t)s.cout * cig * s.kh * s.kw, seed + 1);
+    auto b = rand_i32(s.cout, seed + 2, -1000, 1000);
+    eo_quant q;
+    eo_make_quant(qt.s_in, qt.zp_in, qt.s_w, qt.zp_w, qt.s_bias(), qt.s_out, qt.zp_out, (int)act.activation(), act.isEnabled(), &q);
+    std::vector<uint8_t> want((size_t)s.n * s.cout * ho * wo);
+    eo_conv2d_u8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr);
+
+    // tensors as the model hands them over: planar, or channels-last with positional dims
+    const bool ohwi = androidNN || !nchw;
+    Dim4 in_dim = nchw ? Dim4{(uint32_t)s.n, (uint32_t)s.c, (uint32_t)s.h, (uint32_t)s.w}
+                       : Dim4{(uint32_t)s.n, (uint32_t)s.h, (uint32_t)s.w, (uint32_t)s.c};
+    Dim4 out_dim = nchw ? Dim4{(uint32_t)s.n, (uint32_t)s.cout, (uint32_t)ho, (uint32_t)wo}
+                        : Dim4{(uint32_t)s.n, (uint32_t)ho, (uint32_t)wo, (uint32_t)s.cout};
+    Dim4 w_dim = ohwi ? Dim4{(uint32_t)s.cout, (uint32_t)s.kh, (uint32_t)s.kw, (uint32_t)cig}
+                      : Dim4{(uint32_t)s.cout, (uint32_t)cig, (uint32_t)s.kh, (uint32_t)s.kw};
+    std::vector<uint8_t> w_dev = ohwi ? nchw_to_nhwc(w, s.cout, cig, s.kh, s.kw) : w;
+    const DataOrder order = nchw ? DataOrder::NCHW : DataOrder::NHWC;
+    std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, in_dim, order, qt.s_in, qt.zp_in);
+    std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w_dev.data(), w_dim, order, qt.s_w, qt.zp_w);
+    std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, (uint32_t)s.cout, 1, 1}, DataOrder::NCHW, qt.s_bias(), 0);
+    std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, out_dim, order, qt.s_out, qt.zp_out);
+
+    auto params = std::make_shared<ConvolutionParameters>();
+    params->padding = {(uint32_t)s.pad_t, (uint32_t)s.pad_r, (uint32_t)s.pad_b, (uint32_t)s.pad_l};
+    params->dilation = {(uint32_t)s.dil_h, (uint32_t)s.dil_w};
+    params->stride = {(uint32_t)s.stride_h, (uint32_t)s.stride_w};
+    params->group_size = s.groups;
+    params->androidNN = androidNN;
+    params->isNCHW = nchw;
+    params->activation_info = std::make_shared<ActivationInfo>(act);
+
+    HipConvolution conv(rt, U8);
+    EXPECT(conv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+    rt->assignBufferPool();
+    std::vector<uint8_t> x_dev = nchw ? x : nchw_to_nhwc(x, s.n, s.c, s.h, s.w);
+    EXPECT(input->writeData(x_dev.data()) == Status::SUCCESS);
+    EXPECT(conv.execute() == Status::SUCCESS);
+    std::vector<uint8_t> got(want.size());
+    EXPECT(output->readData(got.data()) == Status::SUCCESS);
+    if (!nchw) got = nhwc_to_nchw(got, s.n, s.cout, ho, wo);
+    EXPECT(same(got, want));
+    EXPECT(varied(want));
+    EXPECT(conv.release() == Status::SUCCESS);
+    return ok;
+}
+
+// ---------------------------------------------------------------- tests
+
+static int gpu_tests() {
+    auto rt = std::make_shared<HipRuntime>();
+    if (rt->initialize(0) != Status::SUCCESS || rt->initializeQueue() != Status::SUCCESS) {
+        std::printf("cannot initialise the GPU runtime: %s\n", eh_last_error());
+        return 2;
+    }
+    const Quant q1 = {0.02f, 0.005f, 0.05f, 128, 120, 0};
+
+    run_test("Convolution.Config1_3x3_64to64_56x56_nchw_relu", [&] {
+        return conv_case(rt, shape(1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1), q1, ActivationInfo(ActivationInfo::ActivationType::RELU, true), true, false, 0xEDF2);
+    });
+    run_test("Convolution.ChannelsLast_androidNN_weights_stride2", [&] {
+        return conv_case(rt, shape(2, 32, 15, 17, 48, 3, 3, 2, 2, 0, 1, 0, 1), {0.02f, 0.005f, 0.04f, 100, 131, 7}, ActivationInfo(ActivationInfo::ActivationType::RELU6, true), false, true, 11);
+    });
+    run_test("Convolution.Planar_androidNN_weights", [&] {
+        return conv_case(rt, shape(1, 16, 9, 9, 24, 3, 3, 1, 1, 1, 1, 1, 1), {0.02f, 0.005f, 0.02f, 100, 131, 7}, ActivationInfo(), true, true, 12);
+    });
+    run_test("Convolution.Grouped_dilated_3_channel_groups", [&] {
+        return conv_case(rt, shape(1, 12, 10, 10, 12, 3, 3, 1, 1, 2, 2, 2, 2, 2, 2, 3), {0.02f, 0.005f, 0.08f, 120, 131, 128}, ActivationInfo(), true, false, 13);
+    });
+    run_test("Convolution.Pointwise_24_to_144_channels_last", [&] {
+        return conv_case(rt, shape(2, 24, 28, 28, 144, 1, 1), {0.02f, 0.004f, 0.03f, 77, 140, 3}, ActivationInfo(ActivationInfo::ActivationType::RELU6, true), false, false, 14);
+    });
+
+    run_test("Convolution.BiasScaleMismatch_gives_clamped_zero_point", [&] {
+        bool ok = true;
+        auto x = rand_u8(1 * 16 * 6 * 6, 21), w = rand_u8(16 * 16 * 9, 22);
+        auto b = rand_i32(16, 23, -1000, 1000);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 16, 6, 6}, DataOrder::NCHW, 0.02f, 128);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{16, 16, 3, 3}, DataOrder::NCHW, 0.005f, 120);
+        // an int32 bias built without quantization parameters keeps scale 1.0 (gpu_op_constructor.cc:2032-2039)
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 16, 1, 1});
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 16, 6, 6}, DataOrder::NCHW, 0.05f, 42);
+        auto params = std::make_shared<ConvolutionParameters>();
+        params->padding = {1, 1, 1, 1};
+        HipConvolution conv(rt, U8);
+        EXPECT(conv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+        EXPECT(conv.execute() == Status::SUCCESS);
+        std::vector<uint8_t> got(16 * 36);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        for (uint8_t v : got) EXPECT(v == 42);
+        return ok;
+    });
+
+    run_test("Convolution.QuantParamsAreReadAtExecute_and_WeightsAsInput", [&] {
+        bool ok = true;
+        const eo_conv_shape s = shape(1, 16, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1);
+        auto x = rand_u8(16 * 64, 31), w = rand_u8(16 * 16 * 9, 32), w2 = rand_u8(16 * 16 * 9, 33);
+        auto b = rand_i32(16, 34, -1000, 1000);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 16, 8, 8}, DataOrder::NCHW, 0.02f, 128);
+        // weights as a run-time input: a shape-only tensor that is written afterwards
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{16, 16, 3, 3}, DataOrder::NCHW, 0.005f, 120);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 16, 1, 1}, DataOrder::NCHW, 0.02f * 0.005f, 0);
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 16, 8, 8}, DataOrder::NCHW, 0.05f, 10);
+        EXPECT(!weight->is_const() && bias->is_const());
+        auto params = std::make_shared<ConvolutionParameters>();
+        params->padding = {1, 1, 1, 1};
+        HipConvolution conv(rt, U8);
+        EXPECT(weight->writeData(w.data()) == Status::SUCCESS);
+        EXPECT(conv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+        std::vector<uint8_t> got(16 * 64), want(16 * 64);
+        eo_quant q;
+        auto check = [&](const std::vector<uint8_t> &wt, float s_out, int zp_in, int zp_out) {
+            eo_make_quant(0.02f, zp_in, 0.005f, 120, 0.02f * 0.005f, s_out, zp_out, 0, 0, &q);
+            eo_conv2d_u8(x.data(), wt.data(), b.data(), want.data(), &s, &q, nullptr);
+            EXPECT(conv.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(got, want));
+        };
+        check(w, 0.05f, 128, 10);
+        input->setZeroPoint(99);   // the tensors are re-quantized between runs
+        output->setScale(0.07f);
+        output->setZeroPoint(20);
+        check(w, 0.07f, 99, 20);
+        EXPECT(weight->writeData(w2.data()) == Status::SUCCESS);  // new weights arrive as data
+        check(w2, 0.07f, 99, 20);
+        return ok;
+    });
+
+    run_test("DepthwiseConvolution.Config3_geometry_channels_last_and_planar", [&] {
+        bool ok = true;
+        for (int nchw = 0; nchw < 2; ++nchw) {
+            const eo_conv_shape s = shape(2, 144, 56, 56, 144, 3, 3, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1);
+            const int ho = 28, wo = 28;
+            auto x = rand_u8((size_t)2 * 144 * 56 * 56, 41), w = rand_u8(144 * 9, 42);
+            auto b = rand_i32(144, 43, -1000, 1000);
+            eo_quant q;
+            eo_make_quant(0.03f, 17, 0.006f, 140, 0.03f * 0.006f, 0.025f, 9, EO_ACT_RELU6, 1, &q);
+            std::vector<uint8_t> want((size_t)2 * 144 * ho * wo), got(want.size());
+            eo_dwconv2d_u8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr);
+            const DataOrder order = nchw ? DataOrder::NCHW : DataOrder::NHWC;
+            const Dim4 in_dim = nchw ? Dim4{2, 144, 56, 56} : Dim4{2, 56, 56, 144};
+            const Dim4 out_dim = nchw ? Dim4{2, 144, 28, 28} : Dim4{2, 28, 28, 144};
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, in_dim, order, 0.03f, 17);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{144, 1, 3, 3}, DataOrder::NCHW, 0.006f, 140);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 144, 1, 1}, DataOrder::NCHW, 0.03f * 0.006f, 0);
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, out_dim, order, 0.025f, 9);
+            auto params = std::make_shared<DepthwiseConvolutionParameters>();
+            params->padding = {1, 1, 1, 1};
+            params->stride = {2, 2};
+            params->isNCHW = nchw != 0;
+            params->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU6, true);
+            HipDepthwiseConvolution dw(rt, U8);
+            EXPECT(dw.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+            auto x_dev = nchw ? x : nchw_to_nhwc(x, 2, 144, 56, 56);
+            EXPECT(input->writeData(x_dev.data()) == Status::SUCCESS);
+            EXPECT(dw.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            if (!nchw) got = nhwc_to_nchw(got, 2, 144, ho, wo);
+            EXPECT(same(got, want));
+            EXPECT(varied(want));
+            EXPECT(dw.release() == Status::SUCCESS);
+        }
+        return ok;
+    });
+
+    run_test("DepthwiseConvolution.DepthMultiplier2", [&] {
+        bool ok = true;
+        const eo_conv_shape s = shape(1, 8, 9, 7, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 2);
+        auto x = rand_u8(8 * 63, 51), w = rand_u8(16 * 9, 52);
+        auto b = rand_i32(16, 53, -100, 100);
+        eo_quant q;
+        eo_make_quant(0.03f, 17, 0.006f, 140, 0.03f * 0.006f, 0.02f, 128, 0, 0, &q);
+        std::vector<uint8_t> want(16 * 63), got(16 * 63);
+        eo_dwconv2d_u8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 8, 9, 7}, DataOrder::NCHW, 0.03f, 17);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{16, 1, 3, 3}, DataOrder::NCHW, 0.006f, 140);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 16, 1, 1}, DataOrder::NCHW, 0.03f * 0.006f, 0);
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 16, 9, 7}, DataOrder::NCHW, 0.02f, 128);
+        auto params = std::make_shared<DepthwiseConvolutionParameters>();
+        params->padding = {1, 1, 1, 1};
+        params->depth_multiplier = 2;
+        HipDepthwiseConvolution dw(rt, U8);
+        EXPECT(dw.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+        EXPECT(dw.execute() == Status::SUCCESS);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        EXPECT(same(got, want));
+        return ok;
+    });
+
+    run_test("FullyConnected.Config2_M256_K4096_N4096", [&] {
+        bool ok = true;
+        const int m = 256, k = 4096, n = 4096;
+        auto a = rand_u8((size_t)m * k, 0xEDE2 + 32);
+        std::vector<uint8_t> w((size_t)n * k);
+        eo_fill_u8_normal(w.data(), (int64_t)w.size(), 0xEDE2 + 33, 128, 20);
+        auto b = rand_i32(n, 0xEDE2 + 34, -1000, 1000);
+        eo_quant q;
+        eo_make_quant(0.01f, 3, 0.002f, 128, 0.01f * 0.002f, 0.08f, 0, 0, 0, &q);
+        EXPECT(q.multiplier == 1099511680 && q.shift == -11);
+        std::vector<uint8_t> want((size_t)m * n), got((size_t)m * n);
+        eo_fc_u8(a.data(), w.data(), b.data(), want.data(), m, k, n, &q, nullptr);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)m, (uint32_t)k, 1, 1}, DataOrder::NCHW, 0.01f, 3);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{(uint32_t)n, (uint32_t)k, 1, 1}, DataOrder::NCHW, 0.002f, 128);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{(uint32_t)n, 1, 1, 1}, DataOrder::NCHW, 0.01f * 0.002f, 0);
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)m, (uint32_t)n, 1, 1}, DataOrder::NCHW, 0.08f, 0);
+        HipFullyConnected fc(rt, U8);
+        EXPECT(fc.initialize({input, weight, bias}, {output}, std::make_shared<FullyConnectedParameters>()) == Status::SUCCESS);
+        EXPECT(input->writeData(a.data()) == Status::SUCCESS);
+        EXPECT(fc.execute() == Status::SUCCESS);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        EXPECT(same(got, want));
+        EXPECT(varied(want));
+        EXPECT(fc.release() == Status::SUCCESS);
+        return ok;
+    });
+
+    run_test("FullyConnected.AndroidNN_flattens_a_4D_input", [&] {
+        bool ok = true;
+        const int k = 4 * 5 * 6, n = 5;  // input [6][4][5][6] read as 6 rows of 120
+        auto a = rand_u8((size_t)6 * k, 61), w = rand_u8((size_t)n * k, 62);
+        auto b = rand_i32(n, 63, -100, 100);
+        eo_quant q;
+        eo_make_quant(0.5f, 100, 0.25f, 90, 0.125f, 40.0f, 128, EO_ACT_RELU1, 1, &q);
+        std::vector<uint8_t> want(6 * n), got(6 * n);
+        eo_fc_u8(a.data(), w.data(), b.data(), want.data(), 6, k, n, &q, nullptr);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{6, 4, 5, 6}, DataOrder::NCHW, 0.5f, 100);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{(uint32_t)n, (uint32_t)k, 1, 1}, DataOrder::NCHW, 0.25f, 90);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{(uint32_t)n, 1, 1, 1}, DataOrder::NCHW, 0.125f, 0);
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{6, (uint32_t)n, 1, 1}, DataOrder::NCHW, 40.0f, 128);
+        auto params = std::make_shared<FullyConnectedParameters>();
+        params->androidNN = true;
+        params->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU1, true);
+        HipFullyConnected fc(rt, U8);
+        EXPECT(fc.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        EXPECT(input->writeData(a.data()) == Status::SUCCESS);
+        EXPECT(fc.execute() == Status::SUCCESS);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        EXPECT(same(got, want));
+        return ok;
+    });
+
+    run_test("FullyConnected.ReferenceSimpleTest_vector", [&] {
+        // src/userdriver/gpu/op_test/fullyconnected_test.cpp:135-149, inputs shifted by a zero point of 10
+        bool ok = true;
+        const int in_raw[20] = {1, 2, 3, 4, 5, 6, 7, 8, -9, -10, 1, 2, 3, 4, 5, 6, 7, -8, 9, -10};
+        std::vector<uint8_t> a(20), w(30);
+        for (int i = 0; i < 20; ++i) a[i] = (uint8_t)(in_raw[i] + 10);
+        for (int i = 0; i < 30; ++i) w[i] = (uint8_t)(i % 10 + 1);
+        std::vector<int32_t> b = {1, 2, 3};
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{2, 10, 1, 1}, DataOrder::NCHW, 1.0f, 10);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{3, 10, 1, 1}, DataOrder::NCHW, 1.0f, 0);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{3, 1, 1, 1}, DataOrder::NCHW, 1.0f, 0);
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{2, 3, 1, 1}, DataOrder::NCHW, 1.0f, 0);
+        HipFullyConnected fc(rt, U8);
+        EXPECT(fc.initialize({input, weight, bias}, {output}, std::make_shared<FullyConnectedParameters>()) == Status::SUCCESS);
+        EXPECT(input->writeData(a.data()) == Status::SUCCESS);
+        EXPECT(fc.execute() == Status::SUCCESS);
+        std::vector<uint8_t> got(6);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        const uint8_t expect[6] = {24, 25, 26, 58, 59, 60};
+        for (int i = 0; i < 6; ++i) EXPECT(got[i] == expect[i]);
+        return ok;
+    });
+
+    run_test("Deconvolution.Config4_4x4_stride2_256to128", [&] {
+        bool ok = true;
+        const eo_conv_shape s = shape(8, 256, 32, 32, 128, 4, 4, 2, 2, 1, 1, 1, 1);
+        auto x = rand_u8((size_t)8 * 256 * 1024, 0xEDE2 + 64), w = rand_u8((size_t)256 * 128 * 16, 0xEDE2 + 65);
+        auto b = rand_i32(128, 0xEDE2 + 66, -1000, 1000);
+        eo_quant q;
+        eo_make_quant(0.02f, 121, 0.005f, 133, 0.02f * 0.005f, 0.35f, 128, 0, 0, &q);
+        std::vector<uint8_t> want((size_t)8 * 128 * 4096), got(want.size());
+        eo_deconv2d_u8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{8, 256, 32, 32}, DataOrder::NCHW, 0.02f, 121);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{256, 128, 4, 4}, DataOrder::NCHW, 0.005f, 133);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 128, 1, 1}, DataOrder::NCHW, 0.02f * 0.005f, 0);
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{8, 128, 64, 64}, DataOrder::NCHW, 0.35f, 128);
+        auto params = std::make_shared<DeconvolutionParameters>();
+        params->padding = {1, 1, 1, 1};
+        params->stride = {2, 2};
+        HipDeconvolution deconv(rt, U8);
+        EXPECT(deconv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+        EXPECT(deconv.execute() == Status::SUCCESS);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        EXPECT(same(got, want));
+        EXPECT(varied(want));
+        EXPECT(deconv.release() == Status::SUCCESS);
+        return ok;
+    });
+
+    run_test("Deconvolution.AndroidNN_weight_order_channels_last_grouped_planar", [&] {
+        bool ok = true;
+        {  // androidNN: weight Dim4 = (out, kh, kw, in), channels-last tensors
+            const eo_conv_shape s = shape(1, 16, 5, 6, 12, 3, 3, 2, 2, 0, 0, 0, 0);
+            const int oh = eo_deconv_out_dim(5, 0, 0, 3, 2), ow = eo_deconv_out_dim(6, 0, 0, 3, 2);
+            auto x = rand_u8(16 * 30, 71), w = rand_u8(16 * 12 * 9, 72);  // w in [in][out][kh][kw]
+            auto b = rand_i32(12, 73, -100, 100);
+            eo_quant q;
+            eo_make_quant(0.03f, 131, 0.01f, 77, 0.03f * 0.01f, 0.3f, 5, 0, 0, &q);
+            std::vector<uint8_t> want((size_t)12 * oh * ow), got(want.size());
+            eo_deconv2d_u8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr);
+            std::vector<uint8_t> w_nn((size_t)12 * 9 * 16);
+            for (int ic = 0; ic < 16; ++ic)
+                for (int oc = 0; oc < 12; ++oc)
+                    for (int t = 0; t < 9; ++t) w_nn[((size_t)oc * 9 + t) * 16 + ic] = w[((size_t)ic * 12 + oc) * 9 + t];
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 5, 6, 16}, DataOrder::NHWC, 0.03f, 131);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w_nn.data(), Dim4{12, 3, 3, 16}, DataOrder::NHWC, 0.01f, 77);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 12, 1, 1}, DataOrder::NCHW, 0.03f * 0.01f, 0);
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, (uint32_t)oh, (uint32_t)ow, 12}, DataOrder::NHWC, 0.3f, 5);
+            auto params = std::make_shared<DeconvolutionParameters>();
+            params->stride = {2, 2};
+            params->androidNN = true;
+            params->isNCHW = false;
+            HipDeconvolution deconv(rt, U8);
+            EXPECT(deconv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+            auto x_dev = nchw_to_nhwc(x, 1, 16, 5, 6);
+            EXPECT(input->writeData(x_dev.data()) == Status::SUCCESS);
+            EXPECT(deconv.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(nhwc_to_nchw(got, 1, 12, oh, ow), want));
+        }
+        {  // grouped, planar
+            const eo_conv_shape s = shape(1, 6, 4, 4, 4, 3, 3, 3, 3, 1, 1, 1, 1, 1, 1, 2);
+            const int oh = eo_deconv_out_dim(4, 1, 1, 3, 3);
+            auto x = rand_u8(6 * 16, 74), w = rand_u8(6 * 2 * 9, 75);
+            auto b = rand_i32(4, 76, -100, 100);
+            eo_quant q;
+            eo_make_quant(0.03f, 131, 0.01f, 77, 0.03f * 0.01f, 0.1f, 128, 0, 0, &q);
+            std::vector<uint8_t> want((size_t)4 * oh * oh), got(want.size());
+            eo_deconv2d_u8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr);
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 6, 4, 4}, DataOrder::NCHW, 0.03f, 131);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{6, 2, 3, 3}, DataOrder::NCHW, 0.01f, 77);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 4, 1, 1}, DataOrder::NCHW, 0.03f * 0.01f, 0);
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 4, (uint32_t)oh, (uint32_t)oh}, DataOrder::NCHW, 0.1f, 128);
+            auto params = std::make_shared<DeconvolutionParameters>();
+            params->padding = {1, 1, 1, 1};
+            params->stride = {3, 3};
+            params->group_size = 2;
+            HipDeconvolution deconv(rt, U8);
+            EXPECT(deconv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+            EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+            EXPECT(deconv.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(got, want));
+        }
+        return ok;
+    });
+
+    run_test("Tensor.HostOrderConversion_on_write_and_read", [&] {
+        bool ok = true;
+        auto x = rand_u8(2 * 5 * 6 * 7, 81);  // planar host data
+        HipTensor t(rt, U8, DataType::UINT8, Dim4{2, 5, 6, 7});
+        auto x_nhwc = nchw_to_nhwc(x, 2, 5, 6, 7);
+        EXPECT(t.writeData(x_nhwc.data(), true, DataOrderChangeType::NHWC2NCHW) == Status::SUCCESS);
+        std::vector<uint8_t> got(x.size());
+        EXPECT(t.readData(got.data()) == Status::SUCCESS);
+        EXPECT(same(got, x));
+        EXPECT(t.readData(got.data(), true, DataOrderChangeType::NCHW2NHWC) == Status::SUCCESS);
+        EXPECT(same(got, x_nhwc));
+        return ok;
+    });
+
+    run_test("OperatorList.Pointwise_then_depthwise_over_pooled_buffers", [&] {
+        // the block of configuration 3 as an operator list: tensors between operators come from
+        // the inter-operator pool and are materialised by assignBufferPool(), as OpenSubGraph does
+        bool ok = true;
+        const int n = 2;
+        auto x = rand_u8((size_t)n * 56 * 56 * 24, 91);  // channels-last
+        auto w1 = rand_u8(144 * 24, 92), w2 = rand_u8(144 * 9, 93);
+        auto b1 = rand_i32(144, 94, -1000, 1000), b2 = rand_i32(144, 95, -1000, 1000);
+        const eo_conv_shape s1 = shape(n, 24, 56, 56, 144, 1, 1), s2 = shape(n, 144, 56, 56, 144, 3, 3, 2, 2, 1, 1, 1, 1);
+        eo_quant q1o, q2o;
+        eo_make_quant(0.02f, 120, 0.004f, 131, 0.02f * 0.004f, 0.03f, 4, EO_ACT_RELU6, 1, &q1o);
+        eo_make_quant(0.03f, 4, 0.006f, 140, 0.03f * 0.006f, 0.025f, 9, EO_ACT_RELU6, 1, &q2o);
+        auto x_nchw = nhwc_to_nchw(x, n, 24, 56, 56);
+        std::vector<uint8_t> mid((size_t)n * 144 * 56 * 56), want((size_t)n * 144 * 28 * 28), got(want.size());
+        eo_conv2d_u8(x_nchw.data(), w1.data(), b1.data(), mid.data(), &s1, &q1o, nullptr);
+        eo_dwconv2d_u8(mid.data(), w2.data(), b2.data(), want.data(), &s2, &q2o, nullptr);
+
+        std::shared_ptr<ITensor> in = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)n, 56, 56, 24}, DataOrder::NHWC, 0.02f, 120, BufferType::INTER_SHARED_NEW);
+        std::shared_ptr<ITensor> mid_t = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)n, 56, 56, 144}, DataOrder::NHWC, 0.03f, 4, BufferType::INTER_SHARED_REUSE);
+        std::shared_ptr<ITensor> out = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)n, 28, 28, 144}, DataOrder::NHWC, 0.025f, 9, BufferType::INTER_SHARED_REUSE);
+        auto w1n = nchw_to_nhwc(w1, 144, 24, 1, 1);
+        std::shared_ptr<ITensor> w1_t = std::make_shared<HipTensor>(rt, U8, w1n.data(), Dim4{144, 1, 1, 24}, DataOrder::NHWC, 0.004f, 131);
+        std::shared_ptr<ITensor> b1_t = std::make_shared<HipTensor>(rt, U8, b1.data(), Dim4{1, 144, 1, 1}, DataOrder::NCHW, 0.02f * 0.004f, 0);
+        std::shared_ptr<ITensor> w2_t = std::make_shared<HipTensor>(rt, U8, w2.data(), Dim4{144, 1, 3, 3}, DataOrder::NCHW, 0.006f, 140);
+        std::shared_ptr<ITensor> b2_t = std::make_shared<HipTensor>(rt, U8, b2.data(), Dim4{1, 144, 1, 1}, DataOrder::NCHW, 0.03f * 0.006f, 0);
+        EXPECT(std::static_pointer_cast<HipTensor>(mid_t)->getDataPtr() == nullptr);  // pooled: not there yet
+
+        auto p1 = std::make_shared<ConvolutionParameters>();
+        p1->isNCHW = false;
+        p1->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU6, true);
+        auto p2 = std::make_shared<DepthwiseConvolutionParameters>();
+        p2->isNCHW = false;
+        p2->padding = {1, 1, 1, 1};
+        p2->stride = {2, 2};
+        p2->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU6, true);
+        auto conv = std::make_shared<HipConvolution>(rt, U8);
+        auto dw = std::make_shared<HipDepthwiseConvolution>(rt, U8);
+        EXPECT(conv->initialize({in, w1_t, b1_t}, {mid_t}, p1) == Status::SUCCESS);
+        EXPECT(dw->initialize({mid_t, w2_t, b2_t}, {out}, p2) == Status::SUCCESS);
+        UDOperators ops = std::make_shared<std::vector<std::shared_ptr<UDOperator>>>();
+        ops->push_back(std::make_shared<EnnUDOperator<HipConvolution>>("CONV_2D", 0, UDTensors{in}, UDTensors{mid_t}, UDTensors{w1_t, b1_t}, conv));
+        ops->push_back(std::make_shared<EnnUDOperator<HipDepthwiseConvolution>>("DEPTHWISE_CONV_2D", 1, UDTensors{mid_t}, UDTensors{out}, UDTensors{w2_t, b2_t}, dw));
+        EXPECT(rt->assignBufferPool() == Status::SUCCESS);
+        EXPECT(std::static_pointer_cast<HipTensor>(mid_t)->getDataPtr() != nullptr);
+        EXPECT(in->writeData(x.data()) == Status::SUCCESS);
+        for (auto &op : *ops) EXPECT(op->execute(nullptr) == ENN_RET_SUCCESS);
+        EXPECT(out->readData(got.data()) == Status::SUCCESS);
+        EXPECT(same(nhwc_to_nchw(got, n, 144, 28, 28), want));
+        for (auto &op : *ops) EXPECT(op->release() == ENN_RET_SUCCESS);
+        return ok;
+    });
+
+    std::printf("%d of %d GPU operator tests failed\n", g_failed, g_run);
+    return g_failed ? 1 : 0;
+}
+
+static int host_tests() {
+    // none of these reaches the device: pooled buffers are only sized until assignBufferPool()
+    auto rt = std::make_shared<HipRuntime>();
+    run_test("BufferPool.InterSharedReuseTakesOverAReleasedBuffer", [&] {
+        bool ok = true;
+        auto a = rt->getBuffer(U8, DataType::UINT8, Dim4{1, 8, 4, 4}, BufferType::INTER_SHARED_NEW);
+        auto b = rt->getBuffer(U8, DataType::UINT8, Dim4{1, 8, 8, 8}, BufferType::INTER_SHARED_REUSE);
+        EXPECT(a != b && rt->interPoolSize() == 2);  // nothing released yet: REUSE had to open a new one
+        EXPECT(rt->resetInterBuffer(a) == Status::SUCCESS);
+        auto c = rt->getBuffer(U8, DataType::UINT8, Dim4{1, 16, 8, 8}, BufferType::INTER_SHARED_REUSE);
+        EXPECT(c == a && a->getBytes() == 1024);  // taken over and grown to the larger request
+        auto d = rt->getBuffer(U8, DataType::UINT8, Dim4{1, 1, 2, 2}, BufferType::INTER_SHARED_REUSE);
+        EXPECT(d != a && d != b && rt->interPoolSize() == 3);
+        EXPECT(rt->resetInterBuffer(std::make_shared<HipBuffer>(4)) == Status::FAILURE);
+        EXPECT(a->getDataPtr() == nullptr);  // deferred until assignBufferPool
+        return ok;
+    });
+    run_test("BufferPool.IntraSharedIsSizedToTheLargestRequest", [&] {
+        bool ok = true;
+        auto a = rt->getBuffer(U8, DataType::INT32, Dim4{1, 1, 1, 100}, BufferType::INTRA_SHARED);  // 400 B
+        auto b = rt->getBuffer(U8, DataType::INT32, Dim4{1, 1, 1, 50}, BufferType::INTRA_SHARED);   // both live: two buffers
+        EXPECT(a != b && rt->intraPoolSize() == 2);
+        EXPECT(rt->resetIntraBuffer() == Status::SUCCESS);  // next operator
+        auto c = rt->getBuffer(U8, DataType::INT32, Dim4{1, 1, 1, 80}, BufferType::INTRA_SHARED);
+        EXPECT(c == a);  // the free one that is already large enough
+        auto d = rt->getBuffer(U8, DataType::INT32, Dim4{1, 1, 1, 300}, BufferType::INTRA_SHARED);
+        EXPECT(d == b && rt->intraPoolSize() == 2);  // the remaining free one, grown to 1200 B
+        return ok;
+    });
+    run_test("Types.LayoutHelpersAndTypeBytes", [&] {
+        bool ok = true;
+        const Dim4 nhwc = {2, 7, 9, 3};
+        const Dim4 nchw = convertDimToNCHW(nhwc);
+        EXPECT(nchw.n == 2 && nchw.c == 3 && nchw.h == 7 && nchw.w == 9);
+        EXPECT(isDimsSame(convertDimToNHWC(nchw), nhwc));
+        EXPECT(getTypeBytes(DataType::UINT8, U8) == 1 && getTypeBytes(DataType::INT32, U8) == 4);
+        EXPECT(getTypeBytes(DataType::FLOAT, PrecisionType::FP16) == 2);
+        EXPECT(getTensorSizeFromDims(extendToDim4({5, 6})) == 30 && getTensorSizeFromDims(extendToDim4({})) == 0);
+        EXPECT(alignTo(1025, 1024) == 2048);
+        EXPECT((int)Status::INVALID_PARAMS == 3 && (int)BufferType::INTRA_SHARED == 3 && (int)PrecisionType::UINT8 == 5 &&
+               (int)DataType::UINT8 == 4 && (int)DataOrder::NHWC == 1);
+        return ok;
+    });
+    std::printf("%d of %d host-only tests failed\n", g_failed, g_run);
+    return g_failed ? 1 : 0;
+}
+
+int main(int argc, char **argv) {
+    if (argc > 1 && std::strcmp(argv[1], "--host-only") == 0) return host_tests();
+    const int rc = host_tests();
+    return rc ? rc : gpu_tests();
+}

@@ -1,0 +1,33 @@
+"""Runs the C++ operator-level tests (cl-eden-kernel_amd/host/ud_op_test.cpp): the Hip*
+operator classes, tensors and buffer manager that mirror the reference's operator API,
+checked bit for bit against the CPU oracle inside the test program."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "cl-eden-kernel_amd", "ud_op_test")
+
+
+def _binary():
+    if not os.path.exists(BIN):
+        import importlib
+        importlib.import_module("cl-eden-kernel_amd.build").build_all()
+    return BIN
+
+
+def test_host_side_buffer_pool_and_types():
+    r = subprocess.run([_binary(), "--host-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout
+    assert "0 of 3 host-only tests failed" in r.stdout
+
+
+@pytest.mark.gpu
+def test_operator_classes_on_gpu():
+    r = subprocess.run([_binary()], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    print(r.stdout, flush=True)
+    assert r.returncode == 0, r.stdout[-4000:]
+    assert "FAIL" not in r.stdout
+    assert "GPU operator tests failed" in r.stdout
