@@ -147,6 +147,15 @@ def deconv_workload(eden, synth, n=8):
                 bytes=n * 256 * 1024 + 256 * 128 * 16 + 512 + n * 128 * 4096, bound="mfma")
 
 
+def copy_workload(eden, synth, mib=64):
+    """A plain device-to-device copy of known size: the yardstick the HBM byte counters are scaled by."""
+    nbytes = mib << 20
+    src, dst = eden.DeviceBuffer(nbytes=nbytes), eden.DeviceBuffer(nbytes=nbytes)
+    lib = eden.load()
+    return dict(name="copy_%dMiB" % mib, launch=lambda s: eden.check(lib.eh_d2d(dst.ptr, src.ptr, nbytes, s)),
+                keep=(src, dst), ops=0.0, bytes=2 * nbytes, bound="hbm")
+
+
 def roofline(work, event_s, steps):
     per_launch = event_s / steps
     if work["bound"] == "mfma":
@@ -202,7 +211,8 @@ def main():
     use_graph = not args.no_graph
 
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
-                    fcbig=lambda e, s: fc_workload(e, s, 8192, 4096, 4096), conv64=lambda e, s: conv_workload(e, s, 64))
+                    fcbig=lambda e, s: fc_workload(e, s, 8192, 4096, 4096), conv64=lambda e, s: conv_workload(e, s, 64),
+                    copy=copy_workload)
     if args.only:
         work = families[args.only](eden, synth)
         wall, ev = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph)
