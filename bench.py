@@ -23,9 +23,10 @@ sys.path.insert(0, ROOT)
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 SEED = 0xEDE2
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
-# scaled by a copy kernel of known size; see profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc (FETCH_SIZE 12348.1 KiB x 1.999,
+# WRITE_SIZE 1024 KiB x 1.000, the factors being what the same counters read on a 64 MiB copy):
+# profiles/igemm_dma_64x64_splitk__fc_m256_k4096_n4096.md
+MEASURED_TRAFFIC_BYTES = 25279996 + 1048576
 
 
 def time_steps(eden, stream, launch, steps, warmup, use_graph=True, chunk=50):
