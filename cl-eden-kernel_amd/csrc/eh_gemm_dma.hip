@@ -28,6 +28,7 @@
 // on the way to the MFMA, and the per-row activation sums needed when
 // zp_w != 128 are v_dot4 accumulations over the same fragment registers.
 #include <type_traits>
+#include <utility>
 
 #include "eh_internal.h"
 
@@ -46,6 +47,13 @@ __device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t
 // One wave copies 64 x 16 bytes: lane i's 16 bytes land at lds_base + 16 * i.
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_base_uniform) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_base_uniform) : "memory");
+}
+
+// The same with the address split into a wave-uniform base and a 32-bit per-lane offset.
+__device__ __forceinline__ void dma16_off(const void *base_uniform, uint32_t lane_offset, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base_uniform),
+                 "s"(lds_base_uniform)
+                 : "memory");
 }
 
 template <int N>
@@ -106,7 +114,17 @@ __device__ __forceinline__ size_t out_pixel_offset(const GemmProblem &p, int m, 
     return (((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0)) * (size_t)p.ldc;
 }
 
-template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES, bool DENSE>
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), unrolled at compile time
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES, bool DENSE, bool ROWSUM>
 __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, const int tiles_m, const int tiles_n, const int gm) {
     static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
     constexpr int CPR = SLAB / 16;            // 16-byte chunks per LDS row
@@ -118,11 +136,17 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     constexpr int LPS = A_LOADS + B_LOADS;
     constexpr int STAGE_BYTES = (BM + BN) * SLAB;
     constexpr int PART_ROW = BN + 4;          // int32 per row of a partial tile: 8 consecutive rows cover all banks
-    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KSTEPS >= 1, "wave tile is made of 32x32x32 MFMA steps");
+    constexpr int NMF = FM * FN;              // MFMAs per step
+    constexpr int NREADS = FM + FN;           // fragment reads per step
+    constexpr int RPS = (NREADS + NMF - 1) / NMF;                    // fragment reads placed behind one MFMA
+    constexpr int WINDOW = STAGES == 2 ? KSTEPS / 2 : KSTEPS;        // steps over which the DMA of one stage is issued
+    constexpr int DPS = (LPS + WINDOW * NMF - 1) / (WINDOW * NMF);   // DMA instructions placed behind one MFMA
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KSTEPS >= 2 && KSTEPS % 2 == 0, "wave tile is made of 32x32x32 MFMA steps; fragment registers alternate between two sets");
     static_assert(BM % (RPB * 4) == 0 && BN % (RPB * 4) == 0, "whole DMA blocks per wave");
-    static_assert((STAGES - 2) * LPS <= 63, "vmcnt is a 6-bit counter");
+    static_assert((STAGES - 1) * LPS <= 63, "vmcnt is a 6-bit counter");
     static_assert(WGK == 1 || WGK * BM * PART_ROW * 4 <= STAGES * STAGE_BYTES, "partial tiles reuse the operand stages");
     static_assert(WGK == 1 || (BM == 64 && BN == 64 && WGM == 1 && WGN == 1), "the split-reduction epilogue is written for one 64x64 tile");
+    static_assert(WTM % CPR == 0 && WTN % CPR == 0, "every fragment row of a lane has the same swizzle");
 
     __shared__ __align__(1024) uint8_t stages[STAGES * STAGE_BYTES];
     __shared__ int32_t rowsum_s[WGK * 2][BM];
@@ -146,62 +170,53 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    for (int i = tid; i < BN; i += 256) bias_s[i] = p.bias[n0 + i];
+    // issued first and consumed after the main loop: by then it has long arrived
+    static_assert(BN <= 256, "one bias value per thread");
+    const int32_t bias_reg = tid < BN ? p.bias[n0 + tid] : 0;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = (wave / WGM) % WGN, wk = wave / (WGM * WGN);
     const int k_slabs = p.k_pad / SLAB;
 
-    if constexpr (!DENSE)
-        for (int i = tid; i < k_slabs * CPR; i += 256) ktab_s[i] = p.ktab[i];
-
-    // this lane's slot in a DMA block: row (lane / CPR), physical chunk lane % CPR
+    // ---- operand fetch.  This lane's slot in a DMA block: row (lane / CPR), physical chunk lane % CPR.
     const int slot_row = lane / CPR;
     const int my_chunk = (lane % CPR) ^ ((wave * RPB + slot_row) & (CPR - 1));
     const int plane = p.ho * p.wo;
     RowRef rows[DENSE ? 1 : A_LOADS];
-    const uint8_t *a_ptr[DENSE ? A_LOADS : 1];  // dense: where this lane's chunk of the next slab sits, per row
+    uint32_t a_voff[DENSE ? A_LOADS : 1];  // dense: where this lane's chunk sits in the activation matrix, per DMA block
+    const uint8_t *a_base = p.a;           // dense: uniform, advances by one slab per issued stage
     if constexpr (DENSE) {
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) {
             int m = m0 + (i * 4 + wave) * RPB + slot_row;
             m = m < p.m ? m : p.m - 1;  // rows past M re-read the last row; their results are never stored
-            a_ptr[i] = p.a + (size_t)m * p.cin + my_chunk * 16;
+            a_voff[i] = (uint32_t)m * (uint32_t)p.cin + my_chunk * 16;
         }
     } else {
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) rows[i] = make_row(p, m0 + (i * 4 + wave) * RPB + slot_row, plane);
     }
-    const int8_t *b_ptr[B_LOADS];  // where this lane's 16 bytes of the next slab sit, per weight block
+    const int8_t *b_base[B_LOADS];  // uniform: the packed 1 KiB blocks of this wave's weight rows, slab 0
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) b_ptr[i] = p.b + ((size_t)(n0 / RPB + i * 4 + wave) * k_slabs) * 1024 + lane * 16;
-    const uint32_t lds0 = lds_offset(stages);
-    __syncthreads();
+    for (int i = 0; i < B_LOADS; ++i) b_base[i] = p.b + ((size_t)(n0 / RPB + i * 4 + wave) * k_slabs) * 1024;
+    uint32_t b_voff = lane * 16;    // advances by one block per issued stage
+    const uint32_t wave_lds = lds_offset(stages) + (wave << 10);
 
-    // The DMA instructions of a stage are spread over the MFMA steps of the stage
-    // before it, so that their address arithmetic fills the issue slots the matrix
-    // pipe leaves free instead of running ahead of it as one serial block.  Stages
-    // are issued in order, so the weight (and dense activation) pointers just advance.
-    auto issue_part = [&](int seq, const KUnit ku, auto first, auto last) {
-        const uint32_t sbase = lds0 + (seq % STAGES) * STAGE_BYTES;
-#pragma unroll
-        for (int idx = decltype(first)::value; idx < decltype(last)::value; ++idx) {
-            if (idx < A_LOADS) {
-                if constexpr (DENSE) {
-                    dma16(a_ptr[idx], sbase + ((idx * 4 + wave) << 10));
-                    a_ptr[idx] += SLAB;
-                } else {
-                    dma16(a_chunk_address(p, rows[idx], ku), sbase + ((idx * 4 + wave) << 10));
-                }
-            } else {
-                const int bi = idx - A_LOADS;
-                dma16(b_ptr[bi], sbase + BM * SLAB + ((bi * 4 + wave) << 10));
-                b_ptr[bi] += 1024;
-            }
+    auto issue_piece = [&](auto idx_c, const uint32_t stage_off, const KUnit ku) {
+        constexpr int idx = decltype(idx_c)::value;
+        if constexpr (idx < A_LOADS) {
+            const uint32_t dst = wave_lds + stage_off + idx * 4096;
+            if constexpr (DENSE)
+                dma16_off(a_base, a_voff[idx], dst);
+            else
+                dma16(a_chunk_address(p, rows[idx], ku), dst);
+        } else {
+            constexpr int bi = idx - A_LOADS;
+            dma16_off(b_base[bi], b_voff, wave_lds + stage_off + BM * SLAB + bi * 4096);
         }
     };
-    auto issue = [&](int seq) {
-        issue_part(seq, DENSE ? KUnit() : ktab_s[seq * CPR + my_chunk], std::integral_constant<int, 0>{},
-                   std::integral_constant<int, LPS>{});
+    auto advance_slab = [&]() {
+        if constexpr (DENSE) a_base += SLAB;
+        b_voff += 1024;
     };
 
     v16i acc[FM][FN];
@@ -214,65 +229,152 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     int rowsum[FM];
 #pragma unroll
     for (int i = 0; i < FM; ++i) rowsum[i] = 0;
-    const bool need_rowsum = p.zw != 0 && wn == 0;
 
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s)
-        if (s < k_slabs) issue(s);
-
-    const int frow = lane & 31, fhalf = lane >> 5;
-    for (int seq = 0; seq < k_slabs; ++seq) {
-        // loads of the stages after this one may stay in flight; in the tail just drain
-        if (k_slabs - 1 - seq >= STAGES - 2)
-            wait_vmcnt<(STAGES - 2) * LPS>();
-        else
-            wait_vmcnt<0>();
-        __syncthreads();  // this stage has landed for every wave; the stage refilled next is no longer read
-        const int next = seq + STAGES - 1;
-        const bool more = next < k_slabs;
-        const KUnit ku = DENSE ? KUnit() : ktab_s[(more ? next : 0) * CPR + my_chunk];
-        const uint8_t *as = stages + (seq % STAGES) * STAGE_BYTES;
-        const uint8_t *bs = as + BM * SLAB;
-        auto step = [&](auto kk_c) {
-            constexpr int kk = decltype(kk_c)::value;
-            const int chunk = wk * (CPR / WGK) + kk * 2 + fhalf;
-            v4i af[FM], bf[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                const int row = wm * WTM + i * 32 + frow;
-                af[i] = xor128(*reinterpret_cast<const v4i *>(as + row * SLAB + ((chunk ^ (row & (CPR - 1))) << 4)));
-                if (need_rowsum) rowsum[i] = sum_bytes_signed(af[i], rowsum[i]);
-            }
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                const int row = wn * WTN + j * 32 + frow;
-                bf[j] = *reinterpret_cast<const v4i *>(bs + row * SLAB + ((chunk ^ (row & (CPR - 1))) << 4));
-            }
-            if (more)
-                issue_part(next, ku, std::integral_constant<int, kk * LPS / KSTEPS>{},
-                           std::integral_constant<int, (kk + 1) * LPS / KSTEPS>{});
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
-        };
-        step(std::integral_constant<int, 0>{});
-        if constexpr (KSTEPS > 1) step(std::integral_constant<int, 1>{});
-        if constexpr (KSTEPS > 2) step(std::integral_constant<int, 2>{});
-        if constexpr (KSTEPS > 3) step(std::integral_constant<int, 3>{});
-        static_assert(KSTEPS <= 4, "at most four MFMA steps per stage");
+    // ---- prologue: every stage buffer is filled.  The table-driven path sends the weight
+    // blocks of the first stage ahead, so the copy of the k-table to LDS runs under their latency.
+    if constexpr (!DENSE) {
+        static_for<B_LOADS>([&](auto bi) { issue_piece(std::integral_constant<int, A_LOADS + decltype(bi)::value>{}, 0u, KUnit()); });
+        for (int i = tid; i < k_slabs * CPR; i += 256) ktab_s[i] = p.ktab[i];
+        __syncthreads();
+        const KUnit ku = ktab_s[my_chunk];
+        static_for<A_LOADS>([&](auto ai) { issue_piece(ai, 0u, ku); });
+        advance_slab();
     }
+#pragma unroll
+    for (int s = DENSE ? 0 : 1; s < STAGES; ++s) {
+        if (s < k_slabs) {
+            KUnit ku = KUnit();
+            if constexpr (!DENSE) ku = ktab_s[s * CPR + my_chunk];
+            static_for<LPS>([&](auto idx) { issue_piece(idx, (uint32_t)(s * STAGE_BYTES), ku); });
+            advance_slab();
+        }
+    }
+
+    // ---- main loop.  A SIMD runs one wave here and issues its instructions in order, one
+    // per four clocks, while an MFMA occupies the matrix pipe for 32: the pipe stays busy only
+    // if the other work of a step (fragment reads for the following step, the DMA of a later
+    // stage, the signed shift of the activation fragments) is issued in the shadow of the
+    // MFMAs, a few instructions behind each one.  The order below is written out slot by slot
+    // and fenced, because the compiler otherwise gathers the MFMAs of a step into one block.
+    //
+    // Fragment registers alternate between two sets, so a stage buffer has been read completely
+    // one step before its MFMAs end.  In the last step of slab s every wave waits for its own
+    // DMA of slab s+1 and meets the others at a barrier; behind that barrier slab s+1 is visible
+    // to all and the buffer of slab s is free, so the DMA of slab s+STAGES is issued into it
+    // from that step on.
+    const int frow = lane & 31, fhalf = lane >> 5;
+    v4i af[2][FM], bf[2][FN];
+    // read number r of a step, in order of first use: A0, B0 .. B(FN-1), A1 .. A(FM-1)
+    auto read_frag = [&](auto r_c, auto buf_c, const uint8_t *stage, const int chunk_base) {
+        constexpr int r = decltype(r_c)::value, buf = decltype(buf_c)::value;
+        const int chunk = wk * (CPR / WGK) + chunk_base + fhalf;
+        if constexpr (r == 0 || r > FN) {
+            constexpr int i = r == 0 ? 0 : r - FN;
+            const int row = wm * WTM + i * 32 + frow;
+            af[buf][i] = *reinterpret_cast<const v4i *>(stage + row * SLAB + ((chunk ^ (row & (CPR - 1))) << 4));
+        } else {
+            constexpr int jj = r - 1;
+            const int row = wn * WTN + jj * 32 + frow;
+            bf[buf][jj] = *reinterpret_cast<const v4i *>(stage + BM * SLAB + row * SLAB + ((chunk ^ (row & (CPR - 1))) << 4));
+        }
+    };
+    auto flip = [&](auto buf_c, auto i_c) {
+        constexpr int buf = decltype(buf_c)::value, i = decltype(i_c)::value;
+        af[buf][i] = xor128(af[buf][i]);
+        if constexpr (ROWSUM) rowsum[i] = sum_bytes_signed(af[buf][i], rowsum[i]);
+    };
+    typedef std::integral_constant<int, 0> c0;
+    typedef std::integral_constant<int, -1> no_wait;
+
+    uint32_t rd_off = 0;  // byte offset of the stage being multiplied
+    // fetch_c: read the fragments of the following step; issue_c: this step carries DMA;
+    // wait_c: vmcnt bound to wait for before crossing into the next slab (-1: no crossing wait)
+    auto step = [&](auto kk_c, auto fetch_c, auto issue_c, auto wait_c, const uint32_t next_off, const KUnit ku) {
+        constexpr int kk = decltype(kk_c)::value;
+        constexpr bool fetch = decltype(fetch_c)::value, issue = decltype(issue_c)::value;
+        constexpr int waitn = decltype(wait_c)::value;
+        constexpr int cur = kk & 1, nxt = cur ^ 1;
+        constexpr bool cross = kk == KSTEPS - 1;  // the following step belongs to the next slab
+        constexpr int w = (kk + 1) % KSTEPS;      // position of this step in the DMA window, which opens at the crossing
+        typedef std::integral_constant<int, cur> cur_c;
+        typedef std::integral_constant<int, nxt> nxt_c;
+        static_for<NMF>([&](auto q_c) {
+            constexpr int q = decltype(q_c)::value, i = q / FN, jj = q % FN;
+            acc[i][jj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[cur][jj], af[cur][i], acc[i][jj], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (fetch) {
+                if constexpr (cross && q == 0) {
+                    wait_vmcnt<waitn>();
+                    __syncthreads();
+                }
+                static_for<RPS>([&](auto t_c) {
+                    constexpr int r = q * RPS + decltype(t_c)::value;
+                    if constexpr (r < NREADS) {
+                        if constexpr (cross)
+                            read_frag(std::integral_constant<int, r>{}, nxt_c{}, stages + next_off, 0);
+                        else
+                            read_frag(std::integral_constant<int, r>{}, nxt_c{}, stages + rd_off, (kk + 1) * 2);
+                    }
+                });
+            }
+            if constexpr (issue && w < WINDOW) {
+                static_for<DPS>([&](auto t_c) {
+                    constexpr int idx = (w * NMF + q) * DPS + decltype(t_c)::value;
+                    // the buffer being refilled is the one whose last fragments were read a step ago
+                    if constexpr (idx < LPS) issue_piece(std::integral_constant<int, idx>{}, cross ? rd_off : next_off, ku);
+                });
+            }
+            if constexpr (q == NMF - 1) {
+                if constexpr (fetch) flip(nxt_c{}, c0{});
+            } else if constexpr ((q + 1) % FN == 0) {
+                flip(cur_c{}, std::integral_constant<int, (q + 1) / FN>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    typedef std::true_type yes;
+    typedef std::false_type no;
+
+    if (k_slabs >= STAGES)
+        wait_vmcnt<(STAGES - 1) * LPS>();
+    else
+        wait_vmcnt<0>();
+    __syncthreads();
+    static_for<NREADS>([&](auto r_c) { read_frag(r_c, c0{}, stages, 0); });
+    flip(c0{}, c0{});
+    // steps 0 .. KSTEPS-2 of slab 0
+    static_for<KSTEPS - 1>([&](auto kk_c) { step(kk_c, yes{}, no{}, no_wait{}, 0u, KUnit()); });
+    // iteration `it`: last step of slab it, then steps 0 .. KSTEPS-2 of slab it+1
+    int it = 0;
+    for (; it < k_slabs - STAGES; ++it) {
+        KUnit ku = KUnit();
+        if constexpr (!DENSE) ku = ktab_s[(it + STAGES) * CPR + my_chunk];
+        const uint32_t freed = rd_off;
+        const uint32_t next_off = rd_off + STAGE_BYTES == STAGES * STAGE_BYTES ? 0u : rd_off + STAGE_BYTES;
+        step(std::integral_constant<int, KSTEPS - 1>{}, yes{}, yes{}, std::integral_constant<int, (STAGES - 2) * LPS>{}, next_off, ku);
+        rd_off = next_off;
+        // in the steps after the crossing, `freed` is what the crossing step called rd_off
+        static_for<KSTEPS - 1>([&](auto kk_c) { step(kk_c, yes{}, yes{}, no_wait{}, freed, ku); });
+        advance_slab();
+    }
+    for (; it < k_slabs - 1; ++it) {  // the last stages are in flight: nothing more to issue
+        const uint32_t next_off = rd_off + STAGE_BYTES == STAGES * STAGE_BYTES ? 0u : rd_off + STAGE_BYTES;
+        step(std::integral_constant<int, KSTEPS - 1>{}, yes{}, no{}, c0{}, next_off, KUnit());
+        rd_off = next_off;
+        static_for<KSTEPS - 1>([&](auto kk_c) { step(kk_c, yes{}, no{}, no_wait{}, 0u, KUnit()); });
+    }
+    step(std::integral_constant<int, KSTEPS - 1>{}, no{}, no{}, no_wait{}, 0u, KUnit());
 
     // ---- epilogue.  acc[i][j][r] belongs to pixel row i*32 + (lane & 31) and channel
     // j*32 + 8*(r >> 2) + 4*(lane >> 5) + (r & 3) of this wave's sub-tile.
-    if (p.zw != 0) {
+    if constexpr (ROWSUM) {
         if (wn == 0) {
 #pragma unroll
             for (int i = 0; i < FM; ++i) rowsum_s[wk * 2 + fhalf][wm * WTM + i * 32 + frow] = rowsum[i];
         }
     }
-    __syncthreads();  // row sums visible; every wave is done with the operand stages
+    if (tid < BN) bias_s[tid] = bias_reg;
+    __syncthreads();  // row sums and bias visible; every wave is done with the operand stages
     const RequantDev rq = p.rq;
     const bool aligned4 = (p.ldc & 3) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 3) == 0);
 
@@ -285,7 +387,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
             const int ml = wm * WTM + i * 32 + frow, m = m0 + ml;
             row_ok[i] = m < p.m;
             row_off[i] = row_ok[i] ? out_pixel_offset(p, m, plane) : 0;
-            corr[i] = p.zw != 0 ? p.zw * (rowsum_s[0][ml] + rowsum_s[1][ml]) : 0;
+            corr[i] = ROWSUM ? p.zw * (rowsum_s[0][ml] + rowsum_s[1][ml]) : 0;
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
@@ -334,7 +436,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         const int m = m0 + ml, n = n0 + nl;
         if (m >= p.m || n >= p.n) return;
         int corr = 0;
-        if (p.zw != 0) {
+        if constexpr (ROWSUM) {
 #pragma unroll
             for (int w = 0; w < WGK * 2; ++w) corr += rowsum_s[w][ml];
             corr *= p.zw;
@@ -388,12 +490,22 @@ int launch_cfg(const GemmProblem &p, hipStream_t stream) {
     const int groups = ((tiles_m + gm - 1) / gm) * ((tiles_n + 32 / gm - 1) / (32 / gm));
     const int grid = ((groups + 7) / 8) * 8 * 32;
     const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
-    if (p.dense)
-        hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true>), dim3(grid), dim3(256), 0, stream,
-                           p, tiles_m, tiles_n, gm);
-    else
-        hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false>), dim3(grid), dim3(256), ktab_bytes,
-                           stream, p, tiles_m, tiles_n, gm);
+    // the per-row activation sums are only carried when the weight zero point is not 128
+    if (p.dense) {
+        if (p.zw != 0)
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true, true>), dim3(grid), dim3(256), 0,
+                               stream, p, tiles_m, tiles_n, gm);
+        else
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true, false>), dim3(grid), dim3(256), 0,
+                               stream, p, tiles_m, tiles_n, gm);
+    } else {
+        if (p.zw != 0)
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false, true>), dim3(grid), dim3(256),
+                               ktab_bytes, stream, p, tiles_m, tiles_n, gm);
+        else
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false, false>), dim3(grid), dim3(256),
+                               ktab_bytes, stream, p, tiles_m, tiles_n, gm);
+    }
     EH_HIP(hipGetLastError());
     return EH_OK;
 }
