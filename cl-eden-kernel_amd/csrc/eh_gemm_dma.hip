@@ -19,10 +19,11 @@
 // BM/WGM x BN/WGN sub-tile): for problems with few output tiles this keeps LDS
 // traffic per MFMA low; the partial tiles meet in LDS at the end (exact: int32).
 //
-// The MFMA is issued with the weight fragment as its row operand, so a lane ends
-// up holding, for ONE output pixel, groups of four consecutive output channels:
-// four requantized bytes pack into one 32-bit store to the channels-last output
-// with no LDS round trip, and the per-pixel terms are per-lane scalars.
+// The MFMA is issued with the weight fragment as its row operand and the packed
+// weight rows of every 32-channel block are permuted, so a lane ends up holding,
+// for ONE output pixel, sixteen consecutive output channels: sixteen requantized
+// bytes go out in one 16-byte store to the channels-last output with no LDS round
+// trip, and the per-pixel terms are per-lane scalars.
 //
 // Activations stay uint8 in LDS; the -128 shift is one XOR per fragment register
 // on the way to the MFMA, and the per-row activation sums needed when
@@ -365,8 +366,8 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     }
     step(std::integral_constant<int, KSTEPS - 1>{}, no{}, no{}, no_wait{}, 0u, KUnit());
 
-    // ---- epilogue.  acc[i][j][r] belongs to pixel row i*32 + (lane & 31) and channel
-    // j*32 + 8*(r >> 2) + 4*(lane >> 5) + (r & 3) of this wave's sub-tile.
+    // ---- epilogue.  acc[i][j][r] belongs to pixel row i*32 + (lane & 31) and, with the row
+    // permutation of the packed weights, channel j*32 + 16*(lane >> 5) + r of this wave's sub-tile.
     if constexpr (ROWSUM) {
         if (wn == 0) {
 #pragma unroll
@@ -376,43 +377,59 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     if (tid < BN) bias_s[tid] = bias_reg;
     __syncthreads();  // row sums and bias visible; every wave is done with the operand stages
     const RequantDev rq = p.rq;
-    const bool aligned4 = (p.ldc & 3) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 3) == 0);
 
     if constexpr (WGK == 1) {
         size_t row_off[FM];
-        int corr[FM];
+        int ncorr[FM];
         bool row_ok[FM];
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             const int ml = wm * WTM + i * 32 + frow, m = m0 + ml;
             row_ok[i] = m < p.m;
             row_off[i] = row_ok[i] ? out_pixel_offset(p, m, plane) : 0;
-            corr[i] = ROWSUM ? p.zw * (rowsum_s[0][ml] + rowsum_s[1][ml]) : 0;
+            ncorr[i] = ROWSUM ? -p.zw * (rowsum_s[0][ml] + rowsum_s[1][ml]) : 0;
         }
+        // whole tiles with 16-byte aligned rows (the usual case) store without any per-store test
+        const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+        auto emit = [&](auto checked_c) {
+            constexpr bool checked = decltype(checked_c)::value;
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
+            for (int j = 0; j < FN; ++j) {
+                const int nl = wn * WTN + j * 32 + fhalf * 16, n = n0 + nl;  // this lane's 16 consecutive channels
+                int4 bb[4];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int nl = wn * WTN + j * 32 + g * 8 + fhalf * 4, n = n0 + nl;
-                const int4 bb = *reinterpret_cast<const int4 *>(bias_s + nl);
+                for (int g = 0; g < 4; ++g) bb[g] = *reinterpret_cast<const int4 *>(bias_s + nl + g * 4);
 #pragma unroll
                 for (int i = 0; i < FM; ++i) {
-                    const uint32_t o0 = requant_u8(acc[i][j][g * 4 + 0] + bb.x - corr[i], rq);
-                    const uint32_t o1 = requant_u8(acc[i][j][g * 4 + 1] + bb.y - corr[i], rq);
-                    const uint32_t o2 = requant_u8(acc[i][j][g * 4 + 2] + bb.z - corr[i], rq);
-                    const uint32_t o3 = requant_u8(acc[i][j][g * 4 + 3] + bb.w - corr[i], rq);
-                    const uint32_t packed = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
-                    if (!row_ok[i] || n >= p.n) continue;
+                    uint32_t packed[4];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const uint32_t o0 = requant_u8(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], rq);
+                        const uint32_t o1 = requant_u8(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], rq);
+                        const uint32_t o2 = requant_u8(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], rq);
+                        const uint32_t o3 = requant_u8(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], rq);
+                        packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+                    }
                     uint8_t *dst = p.out + row_off[i] + n;
-                    if (aligned4 && n + 4 <= p.n) {
-                        *reinterpret_cast<uint32_t *>(dst) = packed;
+                    if constexpr (!checked) {
+                        *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+                        __builtin_amdgcn_sched_barrier(0);  // one fragment at a time: keeps the accumulators where they are
                     } else {
-                        const int cnt = p.n - n < 4 ? p.n - n : 4;
-                        for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed >> (8 * t));
+                        if (!row_ok[i] || n >= p.n) continue;
+                        if (aligned16 && n + 16 <= p.n) {
+                            *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+                        } else {
+                            const int cnt = p.n - n < 16 ? p.n - n : 16;
+                            for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+                        }
                     }
                 }
             }
-        }
+        };
+        if (aligned16 && m0 + BM <= p.m && n0 + BN <= p.n)
+            emit(std::false_type{});
+        else
+            emit(std::true_type{});
     } else {
         // the WGK partial tiles meet in LDS: [wk][pixel row][channel], rows padded so that
         // eight consecutive rows of 16-byte accesses fall in distinct banks
@@ -428,7 +445,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
                     v.y = acc[i][j][g * 4 + 1];
                     v.z = acc[i][j][g * 4 + 2];
                     v.w = acc[i][j][g * 4 + 3];
-                    *reinterpret_cast<int4 *>(part + (i * 32 + frow) * PART_ROW + j * 32 + g * 8 + fhalf * 4) = v;
+                    *reinterpret_cast<int4 *>(part + (i * 32 + frow) * PART_ROW + j * 32 + fhalf * 16 + g * 4) = v;
                 }
         __syncthreads();
         // thread -> pixel row tid & 63, sixteen channels starting at (tid >> 6) * 16

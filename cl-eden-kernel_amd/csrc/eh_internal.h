@@ -148,8 +148,13 @@ inline size_t igemm_dma_ktab_limit() { return 12288; }
 // Byte offset of reduction chunk `kc16` (16-byte units) of packed weight row `n`.
 // Direct-to-LDS layouts: 1 KiB blocks of (1024 / slab) rows x slab bytes, ordered
 // [row block][slab index], the 16-byte chunks of a row XOR-swizzled by the row index.
+// Within every block of 32 output channels the rows are permuted (channel
+// 16h + 4g + t sits in row 8g + 4h + t): a lane of the 32x32x32 MFMA holds result
+// rows 8g + 4h + t (h = lane / 32), which this way are 16 consecutive channels.
 __host__ __device__ inline size_t packed_b_offset(const GemmConfig &cfg, int n, int kc16, int k_pad) {
     if (cfg.id == GEMM_STAGED) return (size_t)n * k_pad + (size_t)kc16 * 16;
+    const int ch = n & 31;
+    n = (n & ~31) | (((ch & 15) >> 2) << 3) | ((ch >> 4) << 2) | (ch & 3);
     const int cpr = cfg.slab / 16, rpb = 1024 / cfg.slab;
     const int c = kc16 % cpr;
     return ((size_t)(n / rpb) * (k_pad / cfg.slab) + kc16 / cpr) * 1024 + (size_t)(n % rpb) * cfg.slab +
