@@ -92,7 +92,11 @@ int pick_vec(int cig, int pixel_stride) {
 int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream) {
     // the kernel shape is fixed here because the packed weight layout depends on it
     g.cfg = GemmConfig();
-    if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
+    if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 &&
+        igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base)) {
+        g.cfg.id = GEMM_THIN;
+        g.cfg.slab = 32;
+    } else if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
         g.cfg = igemm_dma_select(g.proto.m, g.n, g.k);
     g.k_pad = round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
     g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));

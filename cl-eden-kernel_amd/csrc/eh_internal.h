@@ -110,6 +110,7 @@ enum GemmConfigId {
     GEMM_DMA_128x64 = 3,
     GEMM_DMA_64x64_SPLITK = 4,
     GEMM_DMA_256x256 = 5,
+    GEMM_THIN = 6,              // one-tap problems with at most 64 reduction bytes; weights in MFMA fragment order
 };
 struct GemmConfig {
     int32_t id = GEMM_STAGED;
@@ -145,6 +146,9 @@ int launch_igemm(const GemmProblem &p, hipStream_t stream);
 int launch_igemm_dma(const GemmProblem &p, hipStream_t stream);  // vec == 16 and a k-table that fits LDS
 GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k);
 inline size_t igemm_dma_ktab_limit() { return 12288; }
+int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
+bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, int32_t channel_offset, int32_t y_base,
+                        int32_t x_base);
 // Byte offset of reduction chunk `kc16` (16-byte units) of packed weight row `n`.
 // Direct-to-LDS layouts: 1 KiB blocks of (1024 / slab) rows x slab bytes, ordered
 // [row block][slab index], the 16-byte chunks of a row XOR-swizzled by the row index.
@@ -155,6 +159,8 @@ __host__ __device__ inline size_t packed_b_offset(const GemmConfig &cfg, int n, 
     if (cfg.id == GEMM_STAGED) return (size_t)n * k_pad + (size_t)kc16 * 16;
     const int ch = n & 31;
     n = (n & ~31) | (((ch & 15) >> 2) << 3) | ((ch >> 4) << 2) | (ch & 3);
+    // fragment order: [32-channel block][32-byte step][lane = 32 * (chunk & 1) + row][16 bytes]
+    if (cfg.id == GEMM_THIN) return ((((size_t)(n >> 5) * (k_pad / 32) + (kc16 >> 1)) * 2 + (kc16 & 1)) * 32 + (n & 31)) * 16;
     const int cpr = cfg.slab / 16, rpb = 1024 / cfg.slab;
     const int c = kc16 % cpr;
     return ((size_t)(n / rpb) * (k_pad / cfg.slab) + kc16 / cpr) * 1024 + (size_t)(n % rpb) * cfg.slab +

@@ -57,6 +57,8 @@ FC_CASES = [
     (256, 1024, 512, 77, 201),
     (300, 4096, 96, 3, 130),
     (5, 4100, 1000, 10, 20),   # classifier-like: k not a multiple of 64, n = 1000
+    (1000, 24, 144, 128, 5),   # at most 64 reduction bytes: the fragment-direct kernel
+    (129, 56, 17, 250, 128),
 ]
 
 
@@ -154,6 +156,12 @@ CONV_CASES = [
     dict(n=1, c=16, h=3, w=3, cout=16, kh=3, kw=3, pad=(3, 3, 3, 3)),                       # windows wholly in the padding
     dict(n=4, c=128, h=7, w=7, cout=256, kh=1, kw=1),
     dict(n=1, c=160, h=7, w=7, cout=960, kh=1, kw=1),
+    # one tap and at most 64 reduction bytes: the fragment-direct kernel
+    dict(n=3, c=8, h=9, w=7, cout=20, kh=1, kw=1),                                          # half-filled fragments, ragged channels
+    dict(n=2, c=40, h=13, w=13, cout=240, kh=1, kw=1, stride=(2, 2)),                       # two steps, strided rows
+    dict(n=2, c=64, h=12, w=12, cout=32, kh=1, kw=1),
+    dict(n=1, c=48, h=10, w=10, cout=96, kh=1, kw=1, groups=2),                             # 24-byte rows inside 48-byte pixels
+    dict(n=5, c=16, h=33, w=5, cout=96, kh=1, kw=1, stride=(1, 2)),
 ]
 
 
