@@ -37,13 +37,30 @@ class ConvDesc(C.Structure):
                  "depth_multiplier", "layout", "weight_layout")]
 
 
+class AddRequant(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("zp_a", "zp_b", "zp_out", "left_shift", "mult_a", "shift_a", "mult_b", "shift_b", "mult_out", "shift_out",
+                 "act_min", "act_max")]
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("n", "c", "h", "w", "kh", "kw", "stride_h", "stride_w", "pad_t", "pad_b", "pad_l", "pad_r", "layout",
+                 "act_min", "act_max")]
+
+
 EXPORTS = {
     # name: (restype, argtypes)
     "eh_quantize_multiplier": (None, [C.c_double, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "eh_conv_multiplier": (C.c_int, [C.c_float] * 4 + [C.POINTER(C.c_double)]),
     "eh_act_range_u8": (None, [C.c_int, C.c_float, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "eh_requant_apply": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]),
     "eh_make_requant": (None, [C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_float, C.c_float, C.c_int32,
                                C.c_int, C.c_int, C.POINTER(Requant)]),
+    "eh_make_add_requant": (None, [C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_int, C.c_int,
+                                   C.POINTER(AddRequant)]),
+    "eh_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(AddRequant), C.c_void_p]),
+    "eh_avgpool_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PoolDesc), C.c_void_p]),
     "eh_conv_out_dim": (C.c_int32, [C.c_int32] * 6),
     "eh_deconv_out_dim": (C.c_int32, [C.c_int32] * 5),
     "eh_init": (C.c_int, [C.c_int]),
@@ -128,6 +145,38 @@ def make_requant(s_in, zp_in, s_w, zp_w, s_out, zp_out, act=ACT_NONE, act_enable
     q = Requant()
     load().eh_make_requant(s_in, zp_in, s_w, zp_w, s_bias, s_out, zp_out, act, int(act_enabled), C.byref(q))
     return q
+
+
+def make_add_requant(s_a, zp_a, s_b, zp_b, s_out, zp_out, act=ACT_NONE, act_enabled=False):
+    q = AddRequant()
+    load().eh_make_add_requant(s_a, zp_a, s_b, zp_b, s_out, zp_out, act, int(act_enabled), C.byref(q))
+    return q
+
+
+def add_u8(a, b, out, count, q, stream=None):
+    """a, b, out: DeviceBuffer or raw device addresses."""
+    check(load().eh_add_u8(_addr(a), _addr(b), _addr(out), count, C.byref(q), stream))
+
+
+def avgpool_u8(src, dst, n, c, h, w, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), layout=None, act_min=0, act_max=255,
+               stream=None):
+    d = PoolDesc(n, c, h, w, kh, kw, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3],
+                 NCHW if layout is None else layout, act_min, act_max)
+    check(load().eh_avgpool_u8(_addr(src), _addr(dst), C.byref(d), stream))
+
+
+def _addr(x):
+    return x.ptr if hasattr(x, "ptr") else x
+
+
+def requant_apply(q, acc, two_step=False):
+    """Host evaluation of the kernels' requantization of int32 accumulators; returns (uint8 array, used_single_shift)."""
+    acc = np.ascontiguousarray(acc, np.int32)
+    out = np.empty(acc.shape, np.uint8)
+    used = C.c_int32(0)
+    check(load().eh_requant_apply(C.addressof(q), acc.ctypes.data, out.ctypes.data, acc.size, 1 if two_step else 0,
+                                  C.addressof(used)))
+    return out, bool(used.value)
 
 
 def conv_desc(n, c, h, w, cout, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, dm=1,

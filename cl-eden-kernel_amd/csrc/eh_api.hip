@@ -284,6 +284,20 @@ struct eh_dwconv_plan {
 
 extern "C" {
 
+int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int64_t count, int32_t form,
+                                int32_t *single_shift) {
+    int rc = check_requant(q);
+    if (rc) return rc;
+    EH_REQUIRE(count >= 0 && (count == 0 || (acc && out)), "requant_apply: null array");
+    EH_REQUIRE(form == 0 || form == 1, "requant_apply: form %d", form);
+    const RequantDev r = make_requant_dev(*q);
+    const bool fast = form == 0 && r.fast;
+    if (single_shift) *single_shift = fast ? 1 : 0;
+    for (int64_t i = 0; i < count; ++i) out[i] = (uint8_t)(fast ? requant_u8_fast(acc[i], r) : requant_u8(acc[i], r));
+    return EH_OK;
+}
+
+
 // ------------------------------------------------------------ host arithmetic
 
 void eh_quantize_multiplier(double real_multiplier, int32_t *quantized_multiplier, int32_t *shift) {

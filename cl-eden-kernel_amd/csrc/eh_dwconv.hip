@@ -76,8 +76,13 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
             acc3 = dot2(pair_bytes<3>(lo, hi), w4.w, acc3);
         }
     }
-    const uint32_t o = requant_u8(acc0, p.rq) | (requant_u8(acc1, p.rq) << 8) | (requant_u8(acc2, p.rq) << 16) |
-                       (requant_u8(acc3, p.rq) << 24);
+    uint32_t o;
+    if (p.rq.fast)
+        o = requant_u8_fast(acc0, p.rq) | (requant_u8_fast(acc1, p.rq) << 8) | (requant_u8_fast(acc2, p.rq) << 16) |
+            (requant_u8_fast(acc3, p.rq) << 24);
+    else
+        o = requant_u8(acc0, p.rq) | (requant_u8(acc1, p.rq) << 8) | (requant_u8(acc2, p.rq) << 16) |
+            (requant_u8(acc3, p.rq) << 24);
     *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) = o;
 }
 

@@ -1,0 +1,251 @@
+// Quantized residual Add and AveragePool on uint8 tensors (gfx950): the two
+// operators a quantized MobileNet-style network needs between its convolutions.
+// Both are plain HBM streaming kernels.
+//
+// Add follows the reference's quantized add (parameter derivation
+// gpu/operators/cl_optimized_impls/CLAddQuantized.cpp:70-115, kernel
+// gpu/operators/cl_kernels/AddKernelsQauntized.cpp:135-215): both inputs are
+// shifted left by 20 bits, brought to a common scale by a Q31 multiplier and a
+// rounding right shift each, summed, rescaled to the output the same way, offset
+// and clamped.  AveragePool follows gpu/operators/cl_kernels/AveragepoolKernels.cpp:8-44:
+// the window is clipped to the image, (sum + count / 2) / count, clamp.
+#include "eh_internal.h"
+
+namespace eh {
+namespace {
+
+struct AddDev {
+    int32_t zp_a, zp_b, zp_out, left_shift;
+    int32_t mult_a, rs_a, mult_b, rs_b, mult_out, rs_out;
+    int32_t act_min, act_max;
+};
+
+// SaturatingRoundingDoublingHighMul for a non-negative multiplier (no saturation case), then
+// RoundingDivideByPOT
+__device__ __forceinline__ int32_t mul_round_shift(int32_t x, int32_t mult, int32_t rs) {
+    const int64_t ab = (int64_t)x * (int64_t)mult + (1ll << 30);
+    const int32_t v = (int32_t)(ab >> 31);
+    const int32_t mask = (int32_t)((1u << rs) - 1u);
+    const int32_t rem = v & mask;
+    const int32_t thr = (mask >> 1) - (v >> 31);
+    return (v >> rs) + (rem > thr ? 1 : 0);
+}
+
+__device__ __forceinline__ uint32_t add_one(uint32_t a, uint32_t b, const AddDev &q) {
+    const int32_t va = (int32_t)(((uint32_t)((int32_t)a - q.zp_a)) << q.left_shift);
+    const int32_t vb = (int32_t)(((uint32_t)((int32_t)b - q.zp_b)) << q.left_shift);
+    const int32_t sa = mul_round_shift(va, q.mult_a, q.rs_a);
+    const int32_t sb = mul_round_shift(vb, q.mult_b, q.rs_b);
+    int32_t r = mul_round_shift(sa + sb, q.mult_out, q.rs_out) + q.zp_out;
+    r = r < q.act_min ? q.act_min : r;
+    r = r > q.act_max ? q.act_max : r;
+    return (uint32_t)r;
+}
+
+__device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b, const AddDev &q) {
+    return add_one(a & 255u, b & 255u, q) | (add_one((a >> 8) & 255u, (b >> 8) & 255u, q) << 8) |
+           (add_one((a >> 16) & 255u, (b >> 16) & 255u, q) << 16) | (add_one(a >> 24, b >> 24, q) << 24);
+}
+
+// 16 bytes per thread where the three pointers allow it, bytes for the tail
+__global__ __launch_bounds__(256) void add_u8_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
+                                                     uint8_t *__restrict__ out, const int64_t count, const int64_t vec_count,
+                                                     const AddDev q) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < vec_count) {
+        const uint4 va = reinterpret_cast<const uint4 *>(a)[i], vb = reinterpret_cast<const uint4 *>(b)[i];
+        uint4 r;
+        r.x = add_word(va.x, vb.x, q);
+        r.y = add_word(va.y, vb.y, q);
+        r.z = add_word(va.z, vb.z, q);
+        r.w = add_word(va.w, vb.w, q);
+        reinterpret_cast<uint4 *>(out)[i] = r;
+    } else {
+        const int64_t j = vec_count * 16 + (i - vec_count);
+        if (j < count) out[j] = (uint8_t)add_one(a[j], b[j], q);
+    }
+}
+
+struct PoolDev {
+    int32_t n, c, h, w, ho, wo, kh, kw, stride_h, stride_w, pad_t, pad_l, act_min, act_max;
+};
+
+// channels-last: a thread owns four consecutive channels of one output pixel (c % 4 == 0)
+__global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                                const PoolDev p, const int64_t total) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int cq = p.c >> 2;
+    const int c4 = (int)(idx % cq);
+    int64_t r = idx / cq;
+    const int ox = (int)(r % p.wo);
+    r /= p.wo;
+    const int oy = (int)(r % p.ho), img = (int)(r / p.ho);
+    int y0 = oy * p.stride_h - p.pad_t, x0 = ox * p.stride_w - p.pad_l;
+    const int y1 = y0 + p.kh < p.h ? y0 + p.kh : p.h, x1 = x0 + p.kw < p.w ? x0 + p.kw : p.w;
+    y0 = y0 < 0 ? 0 : y0;
+    x0 = x0 < 0 ? 0 : x0;
+    const int cnt = (y1 - y0) * (x1 - x0);
+    int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    for (int y = y0; y < y1; ++y)
+        for (int x = x0; x < x1; ++x) {
+            const uint32_t v = *reinterpret_cast<const uint32_t *>(in + (((size_t)img * p.h + y) * p.w + x) * p.c + c4 * 4);
+            s0 += v & 255u;
+            s1 += (v >> 8) & 255u;
+            s2 += (v >> 16) & 255u;
+            s3 += v >> 24;
+        }
+    auto fin = [&](int s) -> uint32_t {
+        int v = cnt > 0 ? (s + cnt / 2) / cnt : 0;
+        v = v < p.act_min ? p.act_min : v;
+        v = v > p.act_max ? p.act_max : v;
+        return (uint32_t)v;
+    };
+    *reinterpret_cast<uint32_t *>(out + idx * 4) = fin(s0) | (fin(s1) << 8) | (fin(s2) << 16) | (fin(s3) << 24);
+}
+
+// one output element per thread, either layout
+template <bool NHWC>
+__global__ __launch_bounds__(256) void avgpool_scalar_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                             const PoolDev p, const int64_t total) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    int ch, ox, oy, img;
+    int64_t r = idx;
+    if (NHWC) {
+        ch = (int)(r % p.c);
+        r /= p.c;
+        ox = (int)(r % p.wo);
+        r /= p.wo;
+        oy = (int)(r % p.ho);
+        img = (int)(r / p.ho);
+    } else {
+        ox = (int)(r % p.wo);
+        r /= p.wo;
+        oy = (int)(r % p.ho);
+        r /= p.ho;
+        ch = (int)(r % p.c);
+        img = (int)(r / p.c);
+    }
+    int y0 = oy * p.stride_h - p.pad_t, x0 = ox * p.stride_w - p.pad_l;
+    const int y1 = y0 + p.kh < p.h ? y0 + p.kh : p.h, x1 = x0 + p.kw < p.w ? x0 + p.kw : p.w;
+    y0 = y0 < 0 ? 0 : y0;
+    x0 = x0 < 0 ? 0 : x0;
+    const int cnt = (y1 - y0) * (x1 - x0);
+    int s = 0;
+    for (int y = y0; y < y1; ++y)
+        for (int x = x0; x < x1; ++x)
+            s += NHWC ? in[(((size_t)img * p.h + y) * p.w + x) * p.c + ch] : in[(((size_t)img * p.c + ch) * p.h + y) * p.w + x];
+    int v = cnt > 0 ? (s + cnt / 2) / cnt : 0;
+    v = v < p.act_min ? p.act_min : v;
+    v = v > p.act_max ? p.act_max : v;
+    out[idx] = (uint8_t)v;
+}
+
+}  // namespace
+}  // namespace eh
+
+using namespace eh;
+
+extern "C" {
+
+void eh_make_add_requant(float scale_a, int32_t zp_a, float scale_b, int32_t zp_b, float scale_out, int32_t zp_out,
+                         int activation, int activation_enabled, eh_add_requant *out) {
+    out->zp_a = zp_a;
+    out->zp_b = zp_b;
+    out->zp_out = zp_out;
+    out->left_shift = 20;
+    const float mx = scale_a > scale_b ? scale_a : scale_b;  // the maximum is taken in float, then widened
+    const double twice_max = 2 * (double)mx;
+    eh_quantize_multiplier((double)scale_a / twice_max, &out->mult_a, &out->shift_a);
+    eh_quantize_multiplier((double)scale_b / twice_max, &out->mult_b, &out->shift_b);
+    eh_quantize_multiplier(twice_max / ((double)(1 << out->left_shift) * (double)scale_out), &out->mult_out, &out->shift_out);
+    out->act_min = 0;
+    out->act_max = 255;
+    if (activation_enabled) eh_act_range_u8(activation, scale_out, zp_out, &out->act_min, &out->act_max);
+}
+
+int eh_add_u8(const void *a, const void *b, void *out, int64_t count, const eh_add_requant *q, void *stream) {
+    EH_REQUIRE(q != nullptr, "add: null parameters");
+    EH_REQUIRE(count >= 0, "add: negative count");
+    if (count == 0) return EH_OK;
+    EH_REQUIRE(a && b && out, "add: null tensor");
+    EH_REQUIRE(q->mult_a >= 0 && q->mult_b >= 0 && q->mult_out >= 0, "add: negative multiplier");
+    EH_REQUIRE(q->left_shift >= 0 && q->left_shift <= 23, "add: left shift %d outside [0, 23]", q->left_shift);
+    EH_REQUIRE(q->shift_a >= -31 && q->shift_b >= -31 && q->shift_out >= -31, "add: shift below -31");
+    EH_REQUIRE(q->act_min >= 0 && q->act_max <= 255 && q->act_min <= q->act_max, "add: activation range [%d, %d] invalid",
+               q->act_min, q->act_max);
+    AddDev d;
+    d.zp_a = q->zp_a;
+    d.zp_b = q->zp_b;
+    d.zp_out = q->zp_out;
+    d.left_shift = q->left_shift;
+    d.mult_a = q->mult_a;
+    d.mult_b = q->mult_b;
+    d.mult_out = q->mult_out;
+    // a positive shift (a multiplier of 1 or more) is applied as no shift, as the reference kernel's fall-through does
+    d.rs_a = q->shift_a < 0 ? -q->shift_a : 0;
+    d.rs_b = q->shift_b < 0 ? -q->shift_b : 0;
+    d.rs_out = q->shift_out < 0 ? -q->shift_out : 0;
+    d.act_min = q->act_min;
+    d.act_max = q->act_max;
+    const bool wide = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const int64_t vec_count = wide ? count / 16 : 0;
+    const int64_t threads = vec_count + (count - vec_count * 16);
+    const int64_t blocks = (threads + 255) / 256;
+    EH_REQUIRE(blocks < (1ll << 31), "add: tensor too large");
+    hipLaunchKernelGGL(add_u8_kernel, dim3((unsigned)blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), static_cast<uint8_t *>(out), count,
+                       vec_count, d);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
+
+int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *stream) {
+    EH_REQUIRE(desc != nullptr, "avgpool: null descriptor");
+    const eh_pool_desc &d = *desc;
+    EH_REQUIRE(d.n >= 0 && d.c >= 0 && d.h >= 0 && d.w >= 0, "avgpool: negative extent");
+    EH_REQUIRE(d.kh > 0 && d.kw > 0 && d.stride_h > 0 && d.stride_w > 0, "avgpool: bad window or stride");
+    EH_REQUIRE(d.pad_t >= 0 && d.pad_b >= 0 && d.pad_l >= 0 && d.pad_r >= 0, "avgpool: negative padding");
+    EH_REQUIRE(d.layout == EH_NCHW || d.layout == EH_NHWC, "avgpool: bad layout %d", d.layout);
+    EH_REQUIRE(d.act_min >= 0 && d.act_max <= 255 && d.act_min <= d.act_max, "avgpool: activation range [%d, %d] invalid",
+               d.act_min, d.act_max);
+    if ((int64_t)d.n * d.c * d.h * d.w == 0) return EH_OK;
+    PoolDev p;
+    p.n = d.n;
+    p.c = d.c;
+    p.h = d.h;
+    p.w = d.w;
+    p.ho = (d.h + d.pad_t + d.pad_b - d.kh) / d.stride_h + 1;
+    p.wo = (d.w + d.pad_l + d.pad_r - d.kw) / d.stride_w + 1;
+    EH_REQUIRE(d.h + d.pad_t + d.pad_b >= d.kh && d.w + d.pad_l + d.pad_r >= d.kw, "avgpool: window larger than the padded image");
+    p.kh = d.kh;
+    p.kw = d.kw;
+    p.stride_h = d.stride_h;
+    p.stride_w = d.stride_w;
+    p.pad_t = d.pad_t;
+    p.pad_l = d.pad_l;
+    p.act_min = d.act_min;
+    p.act_max = d.act_max;
+    EH_REQUIRE(in && out, "avgpool: null tensor");
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int64_t outputs = (int64_t)d.n * d.c * p.ho * p.wo;
+    const bool vec4 = d.layout == EH_NHWC && (d.c & 3) == 0 &&
+                      ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 3) == 0;
+    const int64_t total = vec4 ? outputs / 4 : outputs;
+    const int64_t blocks = (total + 255) / 256;
+    EH_REQUIRE(blocks < (1ll << 31), "avgpool: tensor too large");
+    if (vec4)
+        hipLaunchKernelGGL(avgpool_nhwc_vec4_kernel, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint8_t *>(in),
+                           static_cast<uint8_t *>(out), p, total);
+    else if (d.layout == EH_NHWC)
+        hipLaunchKernelGGL(avgpool_scalar_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s,
+                           static_cast<const uint8_t *>(in), static_cast<uint8_t *>(out), p, total);
+    else
+        hipLaunchKernelGGL(avgpool_scalar_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s,
+                           static_cast<const uint8_t *>(in), static_cast<uint8_t *>(out), p, total);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
+
+}  // extern "C"

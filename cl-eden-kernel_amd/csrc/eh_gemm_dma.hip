@@ -391,8 +391,8 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         }
         // whole tiles with 16-byte aligned rows (the usual case) store without any per-store test
         const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-        auto emit = [&](auto checked_c) {
-            constexpr bool checked = decltype(checked_c)::value;
+        auto emit = [&](auto checked_c, auto fast_c) {
+            constexpr bool checked = decltype(checked_c)::value, fast = decltype(fast_c)::value;
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const int nl = wn * WTN + j * 32 + fhalf * 16, n = n0 + nl;  // this lane's 16 consecutive channels
@@ -404,10 +404,10 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
                     uint32_t packed[4];
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
-                        const uint32_t o0 = requant_u8(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], rq);
-                        const uint32_t o1 = requant_u8(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], rq);
-                        const uint32_t o2 = requant_u8(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], rq);
-                        const uint32_t o3 = requant_u8(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], rq);
+                        const uint32_t o0 = requant_u8_as<fast>(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], rq);
+                        const uint32_t o1 = requant_u8_as<fast>(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], rq);
+                        const uint32_t o2 = requant_u8_as<fast>(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], rq);
+                        const uint32_t o3 = requant_u8_as<fast>(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], rq);
                         packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
                     }
                     uint8_t *dst = p.out + row_off[i] + n;
@@ -426,10 +426,11 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
                 }
             }
         };
-        if (aligned16 && m0 + BM <= p.m && n0 + BN <= p.n)
-            emit(std::false_type{});
+        // edge tiles and unusual requantization parameters take the general code
+        if (rq.fast && aligned16 && m0 + BM <= p.m && n0 + BN <= p.n)
+            emit(std::false_type{}, std::true_type{});
         else
-            emit(std::true_type{});
+            emit(std::true_type{}, std::false_type{});
     } else {
         // the WGK partial tiles meet in LDS: [wk][pixel row][channel], rows padded so that
         // eight consecutive rows of 16-byte accesses fall in distinct banks
@@ -460,6 +461,8 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         }
         const int32_t *pr = reinterpret_cast<const int32_t *>(stages) + ml * PART_ROW + nl;
         uint32_t packed[4];
+        auto reduce = [&](auto fast_c) {
+            constexpr bool fast = decltype(fast_c)::value;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             int4 s4 = *reinterpret_cast<const int4 *>(pr + g * 4);
@@ -472,10 +475,15 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
                 s4.w += t.w;
             }
             const int4 bb = *reinterpret_cast<const int4 *>(bias_s + nl + g * 4);
-            const uint32_t o0 = requant_u8(s4.x + bb.x - corr, rq), o1 = requant_u8(s4.y + bb.y - corr, rq);
-            const uint32_t o2 = requant_u8(s4.z + bb.z - corr, rq), o3 = requant_u8(s4.w + bb.w - corr, rq);
+            const uint32_t o0 = requant_u8_as<fast>(s4.x + bb.x - corr, rq), o1 = requant_u8_as<fast>(s4.y + bb.y - corr, rq);
+            const uint32_t o2 = requant_u8_as<fast>(s4.z + bb.z - corr, rq), o3 = requant_u8_as<fast>(s4.w + bb.w - corr, rq);
             packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
         }
+        };
+        if (rq.fast)
+            reduce(std::true_type{});
+        else
+            reduce(std::false_type{});
         uint8_t *dst = p.out + out_pixel_offset(p, m, plane) + n;
         const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
         if (aligned16 && n + 16 <= p.n) {

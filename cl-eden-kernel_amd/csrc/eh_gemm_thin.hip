@@ -19,7 +19,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 namespace {
 
-template <int KSTEPS, bool ROWSUM>
+template <int KSTEPS, bool ROWSUM, bool FAST>
 __global__ __launch_bounds__(256) void thin_gemm_kernel(const GemmProblem p, const int n_blocks) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, half = lane >> 5;
@@ -65,30 +65,47 @@ __global__ __launch_bounds__(256) void thin_gemm_kernel(const GemmProblem p, con
     const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
     const v4i *bfrag = reinterpret_cast<const v4i *>(p.b) + lane;
 
-#pragma unroll 2
-    for (int nb = 0; nb < n_blocks; ++nb) {
-        v16i acc;
+    // four channel blocks at a time: all their weight fragments and bias values are requested
+    // before the first is used, so one memory latency covers the group
+    constexpr int NBU = 4;
+    for (int nb0 = 0; nb0 < n_blocks; nb0 += NBU) {
+        v4i bf[NBU][KSTEPS];
+        int4 bb[NBU][4];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0;
+        for (int u = 0; u < NBU; ++u) {
+            const int nb = nb0 + u < n_blocks ? nb0 + u : n_blocks - 1;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks)
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bfrag[(nb * KSTEPS + ks) * 64], af[ks], acc, 0, 0, 0);
-        const int n = nb * 32 + half * 16;  // this lane's 16 consecutive channels
-        uint32_t packed[4];
+            for (int ks = 0; ks < KSTEPS; ++ks) bf[u][ks] = bfrag[(nb * KSTEPS + ks) * 64];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int4 bb = *reinterpret_cast<const int4 *>(p.bias + n + g * 4);
-            const uint32_t o0 = requant_u8(acc[g * 4 + 0] + bb.x + ncorr, rq), o1 = requant_u8(acc[g * 4 + 1] + bb.y + ncorr, rq);
-            const uint32_t o2 = requant_u8(acc[g * 4 + 2] + bb.z + ncorr, rq), o3 = requant_u8(acc[g * 4 + 3] + bb.w + ncorr, rq);
-            packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+            for (int g = 0; g < 4; ++g) bb[u][g] = *reinterpret_cast<const int4 *>(p.bias + nb * 32 + half * 16 + g * 4);
         }
-        if (!row_ok || n >= p.n) continue;
-        uint8_t *dst = p.out + out_off + n;
-        if (aligned16 && n + 16 <= p.n) {
-            *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
-        } else {
-            const int cnt = p.n - n < 16 ? p.n - n : 16;
-            for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+#pragma unroll
+        for (int u = 0; u < NBU; ++u) {
+            const int nb = nb0 + u;
+            if (nb >= n_blocks) break;
+            v16i acc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[i] = 0;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[u][ks], af[ks], acc, 0, 0, 0);
+            const int n = nb * 32 + half * 16;  // this lane's 16 consecutive channels
+            uint32_t packed[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t o0 = requant_u8_as<FAST>(acc[g * 4 + 0] + bb[u][g].x + ncorr, rq);
+                const uint32_t o1 = requant_u8_as<FAST>(acc[g * 4 + 1] + bb[u][g].y + ncorr, rq);
+                const uint32_t o2 = requant_u8_as<FAST>(acc[g * 4 + 2] + bb[u][g].z + ncorr, rq);
+                const uint32_t o3 = requant_u8_as<FAST>(acc[g * 4 + 3] + bb[u][g].w + ncorr, rq);
+                packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+            }
+            if (!row_ok || n >= p.n) continue;
+            uint8_t *dst = p.out + out_off + n;
+            if (aligned16 && n + 16 <= p.n) {
+                *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+            } else {
+                const int cnt = p.n - n < 16 ? p.n - n : 16;
+                for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+            }
         }
     }
 }
@@ -97,10 +114,17 @@ template <int KSTEPS>
 int launch_steps(const GemmProblem &p, hipStream_t stream) {
     const int n_blocks = (p.n + 31) / 32;
     const dim3 grid((p.m + 127) / 128);
-    if (p.zw != 0)
-        hipLaunchKernelGGL((thin_gemm_kernel<KSTEPS, true>), grid, dim3(256), 0, stream, p, n_blocks);
-    else
-        hipLaunchKernelGGL((thin_gemm_kernel<KSTEPS, false>), grid, dim3(256), 0, stream, p, n_blocks);
+    if (p.zw != 0) {
+        if (p.rq.fast)
+            hipLaunchKernelGGL((thin_gemm_kernel<KSTEPS, true, true>), grid, dim3(256), 0, stream, p, n_blocks);
+        else
+            hipLaunchKernelGGL((thin_gemm_kernel<KSTEPS, true, false>), grid, dim3(256), 0, stream, p, n_blocks);
+    } else {
+        if (p.rq.fast)
+            hipLaunchKernelGGL((thin_gemm_kernel<KSTEPS, false, true>), grid, dim3(256), 0, stream, p, n_blocks);
+        else
+            hipLaunchKernelGGL((thin_gemm_kernel<KSTEPS, false, false>), grid, dim3(256), 0, stream, p, n_blocks);
+    }
     EH_HIP(hipGetLastError());
     return EH_OK;
 }

@@ -40,9 +40,14 @@ struct RequantDev {
     int32_t zp_out;
     int32_t act_min;
     int32_t act_max;
+    // single-shift form (see requant_u8_fast); valid when `fast` is set
+    int32_t fast;
+    int32_t fast_shift;        // right_shift - 1
+    uint32_t pos_lo, pos_hi;   // 64-bit rounding term for accumulators >= 0
+    uint32_t neg_lo, neg_hi;   // the same for accumulators < 0
 };
 
-__device__ __forceinline__ int32_t requant_core(int32_t acc, const RequantDev &r) {
+__host__ __device__ __forceinline__ int32_t requant_core(int32_t acc, const RequantDev &r) {
     // x * (1 << ls) wraps like the int32 multiply of the reference kernels
     const int32_t x = (int32_t)((uint32_t)acc << r.left_shift);
     // (ab + nudge) / 2^31 with nudge = ab >= 0 ? 2^30 : 1 - 2^30 and C truncation
@@ -56,11 +61,37 @@ __device__ __forceinline__ int32_t requant_core(int32_t acc, const RequantDev &r
     return (v >> r.right_shift) + (rem > thr ? 1 : 0);
 }
 
-__device__ __forceinline__ uint32_t requant_u8(int32_t acc, const RequantDev &r) {
+__host__ __device__ __forceinline__ uint32_t requant_u8(int32_t acc, const RequantDev &r) {
     int32_t v = requant_core(acc, r) + r.zp_out;
     v = v < r.act_min ? r.act_min : v;
     v = v > r.act_max ? r.act_max : v;
     return (uint32_t)v;
+}
+
+// The same function in one multiply-add and one shift, for left_shift == 0 and
+// 1 <= right_shift <= 21.  With v = floor((xM + 2^30) / 2^31), h = 2^(rs-1) and
+// s = -(v < 0), the rounding divide is floor((v + h + s) / 2^rs), and since h + s
+// is an integer the two floors merge:
+//     result + zp = floor((xM + 2^30 + (h + s + zp * 2^rs) * 2^31) / 2^(31 + rs)).
+// s may be taken from the sign of x: where x < 0 but v = 0 (-2^30 <= xM < 0) the
+// numerator stays inside [0, 2^(30 + rs)), so the result is 0 either way.  The
+// quotient by 2^(31 + rs) with rs >= 1 only needs the high word of the sum.
+__host__ __device__ __forceinline__ uint32_t requant_u8_fast(int32_t x, const RequantDev &r) {
+    const bool neg = x < 0;
+    const uint64_t term = ((uint64_t)(neg ? r.neg_hi : r.pos_hi) << 32) | (neg ? r.neg_lo : r.pos_lo);
+    const int64_t t = (int64_t)x * (int64_t)r.multiplier + (int64_t)term;
+    int32_t v = (int32_t)(t >> 32) >> r.fast_shift;
+    v = v < r.act_min ? r.act_min : v;
+    v = v > r.act_max ? r.act_max : v;
+    return (uint32_t)v;
+}
+
+template <bool FAST>
+__host__ __device__ __forceinline__ uint32_t requant_u8_as(int32_t acc, const RequantDev &r) {
+    if constexpr (FAST)
+        return requant_u8_fast(acc, r);
+    else
+        return requant_u8(acc, r);
 }
 
 inline RequantDev make_requant_dev(const eh_requant &q) {
@@ -73,6 +104,19 @@ inline RequantDev make_requant_dev(const eh_requant &q) {
     r.zp_out = q.zp_out;
     r.act_min = q.act_min;
     r.act_max = q.act_max;
+    // |xM| < 2^62 and the rounding term stays below 2^(42 + rs): no 64-bit overflow up to rs = 20
+    r.fast = (r.left_shift == 0 && r.right_shift >= 1 && r.right_shift <= 20 && q.multiplier >= 0 && q.zp_out >= -1024 &&
+              q.zp_out <= 1024)
+                 ? 1
+                 : 0;
+    r.fast_shift = r.fast ? r.right_shift - 1 : 0;
+    const int rs = r.fast ? r.right_shift : 1;
+    const int64_t pos = (1ll << 30) + (1ll << (30 + rs)) + (int64_t)q.zp_out * (1ll << (31 + rs));
+    const int64_t neg = pos - (1ll << 31);
+    r.pos_lo = (uint32_t)((uint64_t)pos & 0xFFFFFFFFull);
+    r.pos_hi = (uint32_t)((uint64_t)pos >> 32);
+    r.neg_lo = (uint32_t)((uint64_t)neg & 0xFFFFFFFFull);
+    r.neg_hi = (uint32_t)((uint64_t)neg >> 32);
     return r;
 }
 

@@ -58,6 +58,28 @@ typedef struct eh_requant {
     int32_t act_max;
 } eh_requant;
 
+/* Parameters of a quantized element-wise add: what CLAddQuantized::execute derives
+ * from its three tensors (gpu/operators/cl_optimized_impls/CLAddQuantized.cpp:70-115). */
+typedef struct eh_add_requant {
+    int32_t zp_a, zp_b, zp_out;
+    int32_t left_shift;           /* 20 */
+    int32_t mult_a, shift_a;      /* scale_a / (2 max(scale_a, scale_b)) */
+    int32_t mult_b, shift_b;
+    int32_t mult_out, shift_out;  /* 2 max(scale_a, scale_b) / (2^left_shift scale_out) */
+    int32_t act_min, act_max;
+} eh_add_requant;
+
+/* Geometry of an average pool (Pool2DParameters, gpu/common/CLParameter.hpp:25-34);
+ * the clamp range is what CLAveragepool::averagepool_quant derives from the output
+ * tensor (gpu/operators/CLAveragepool.cpp:175-198), see eh_act_range_u8. */
+typedef struct eh_pool_desc {
+    int32_t n, c, h, w;
+    int32_t kh, kw, stride_h, stride_w;
+    int32_t pad_t, pad_b, pad_l, pad_r;
+    int32_t layout;               /* EH_NCHW or EH_NHWC, input and output alike */
+    int32_t act_min, act_max;
+} eh_pool_desc;
+
 /* Geometry of a convolution-like operator.  Input dims are (n, c, h, w) whatever
  * the memory order; `layout` says how input and output bytes are ordered.
  * Mirrors ConvolutionParameters / DepthwiseConvolutionParameters /
@@ -90,6 +112,15 @@ void eh_act_range_u8(int activation, float scale, int32_t zero_point, int32_t *a
  * does not match (CLGEMMConvolutionQuantized.cpp:163-166). */
 void eh_make_requant(float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp, float bias_scale,
                      float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out);
+/* The requantization every kernel epilogue applies to an int32 accumulator (bias
+ * and zero-point terms already added): MultiplyByQuantizedMultiplier, output
+ * zero point, activation clamp (gpu/common/CLKernels.hpp:120-170), evaluated on
+ * the host with the same source the kernels compile.  form 0 evaluates it the
+ * way the kernels would for these parameters (a single 64-bit multiply-add and
+ * shift where that is exact, *single_shift reports which), form 1 always takes
+ * the two-step reference order. */
+int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int64_t count, int32_t form,
+                     int32_t *single_shift);
 /* output extents: CLConvolution.cpp:99-104 and CLDeconvolution.cpp:82-87 */
 int32_t eh_conv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t dilation, int32_t stride);
 int32_t eh_deconv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t stride);
@@ -127,6 +158,19 @@ int eh_graph_destroy(void *graph);
  * driven by CLRuntime::NCHW2NHWC / NHWC2NCHW (gpu/common/CLRuntime.cpp:1477-1619). */
 int eh_transpose_u8_nchw2nhwc(const void *src, void *dst, int32_t n, int32_t c, int32_t h, int32_t w, void *stream);
 int eh_transpose_u8_nhwc2nchw(const void *src, void *dst, int32_t n, int32_t c, int32_t h, int32_t w, void *stream);
+
+/* ---- element-wise add and average pool --------------------------------------
+ * The two operators between the convolutions of a quantized residual network.
+ * eh_make_add_requant is host arithmetic (CLAddQuantized.cpp:70-115); eh_add_u8 is
+ * the quantized add kernel (gpu/operators/cl_kernels/AddKernelsQauntized.cpp:135-215)
+ * over `count` bytes of two equally shaped tensors; eh_avgpool_u8 is
+ * avepooling_tflite_INT8 (gpu/operators/cl_kernels/AveragepoolKernels.cpp:8-44):
+ * windows clipped to the image, (sum + count / 2) / count, clamp.  Both are
+ * asynchronous on `stream` and may be captured in a graph. */
+void eh_make_add_requant(float scale_a, int32_t zp_a, float scale_b, int32_t zp_b, float scale_out, int32_t zp_out,
+                         int activation, int activation_enabled, eh_add_requant *out);
+int eh_add_u8(const void *a, const void *b, void *out, int64_t count, const eh_add_requant *q, void *stream);
+int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *stream);
 
 /* ---- operators -------------------------------------------------------------
  * A plan owns everything initialize() prepares once: packed int8 weights, the

@@ -231,6 +231,31 @@ def test_requant_edge_multipliers_through_conv():
         assert np.array_equal(got, want), (m_real, diff_report(got, want))
 
 
+def test_two_step_requant_in_every_kernel_family():
+    """Multipliers above 1 and right shifts beyond 20 take the general two-step epilogue: the fragment-direct
+    kernel, the direct-to-LDS tiles (whole tiles included), the register-staged kernel and depthwise."""
+    for m_real, zp_out in ((1.5, 128), (2.0 ** -24, 77)):
+        qm, sh = O.quantize_multiplier(m_real)
+        for m, k, n in ((200, 32, 48), (512, 256, 256), (70, 100, 40)):
+            a = (synth.fill_u8((m, k), SEED + 31 + m) % 5 + 126).astype(np.uint8)   # small accumulators: outputs spread at M = 1.5
+            w = (synth.fill_u8((n, k), SEED + 32 + m) % 5 + 126).astype(np.uint8)
+            b = synth.fill_i32((n,), SEED + 33, -20, 20)
+            q = O.raw_quant(zp_in=128, zp_w=127, zp_out=zp_out, multiplier=qm, shift=sh)
+            want = O.fc(a, w, b, q)
+            got = gpu_fc(a, w, b, to_eh_requant(q))
+            assert np.array_equal(got, want), (m_real, m, k, n, diff_report(got, want))
+            if m_real > 1:
+                assert want.std() > 5
+        s = O.conv_shape(2, 16, 9, 9, 16, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), groups=16)
+        x = (synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 34) % 5 + 126).astype(np.uint8)
+        w = (synth.fill_u8((s.c, 1, 3, 3), SEED + 35) % 5 + 126).astype(np.uint8)
+        b = synth.fill_i32((s.c,), SEED + 36, -20, 20)
+        q = O.raw_quant(zp_in=128, zp_w=127, zp_out=zp_out, multiplier=qm, shift=sh)
+        want = O.dwconv2d(x, w, b, s, q)
+        got = gpu_dwconv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
+        assert np.array_equal(got, want), (m_real, diff_report(got, want))
+
+
 def test_negative_half_ties_round_like_the_oracle():
     """Accumulators chosen so that acc * M lands exactly on .5 for both signs and both rounding stages."""
     k, n = 16, 16
