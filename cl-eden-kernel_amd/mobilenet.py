@@ -1,0 +1,206 @@
+"""MobileNetV2-1.0 (224x224x3, 1000 classes) as a list of quantized uint8
+operators over the C ABI: convolution, depthwise convolution, pointwise
+convolution, residual Add, AveragePool and FullyConnected, per-tensor
+asymmetric quantization, ReLU6 as a clamp in the quantized domain.
+
+The operator list plays the part of the reference's OperationConstructor /
+OperationExecutor pair (src/userdriver/gpu/gpu_op_constructor.cc:1797-1850,
+gpu_userdriver.cc:78-112): build every operator once, then execute them in
+order on one stream, here captured into one HIP graph.
+
+Weights are random (there is no checkpoint): uint8 clip(round(N(zp_w, 20)))
+with a per-layer weight zero point, int32 uniform bias.  Scales are chosen
+analytically from the layer shapes so that activations neither die nor saturate
+on their way through the 53 convolutions:
+  * a ReLU6 output tensor has zero point 0 and scale 6/255, so ReLU6 is the
+    whole uint8 range, and the layer's weight scale is set so that the
+    pre-activation has a standard deviation of about 64 output steps;
+  * a linear (projection / classifier) output has zero point 128 and about 30
+    steps of standard deviation;
+  * a residual sum is rescaled back to about 30 steps.
+`layers()` is pure data (no GPU): tests evaluate the same list with the oracle.
+"""
+import math
+
+import numpy as np
+
+from . import synth
+
+SEED = 0xEDE2 + 16 * 5
+
+# (expansion t, output channels c, repeats n, stride s)
+BOTTLENECKS = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1))
+
+W_SD = 20                 # standard deviation of the weight bytes around their zero point
+RELU6_SCALE = 6.0 / 255   # ReLU6 == [0, 255] at zero point 0
+RELU_RMS = 45.0           # root mean square of clip(N(0, 64), 0, 255)
+LINEAR_SD = 30.0
+INPUT_SCALE, INPUT_ZP = 0.02, 128
+INPUT_RMS = 74.0          # of uniform bytes around 128
+
+
+def layers(image=224):
+    """The operator list.  Tensors are numbered; tensor 0 is the network input.  Returns
+    (tensors, ops): tensors[i] = dict(h, w, c, scale, zp, rms), ops = list of dicts."""
+    tensors = [dict(h=image, w=image, c=3, scale=INPUT_SCALE, zp=INPUT_ZP, rms=INPUT_RMS)]
+    ops = []
+
+    def conv(src, cout, k, stride, relu6, depthwise=False):
+        t = tensors[src]
+        idx = len(ops)
+        pad = (k - 1) // 2
+        ho, wo = (t["h"] + 2 * pad - k) // stride + 1, (t["w"] + 2 * pad - k) // stride + 1
+        fan_in = k * k * (1 if depthwise else t["c"])
+        acc_sd = math.sqrt(fan_in) * W_SD * t["rms"]
+        if relu6:
+            out_scale, out_zp, out_sd, out_rms = RELU6_SCALE, 0, 64.0, RELU_RMS
+        else:
+            out_scale, out_zp, out_sd, out_rms = 0.05, 128, LINEAR_SD, LINEAR_SD
+        w_scale = (out_sd / acc_sd) * out_scale / t["scale"]
+        tensors.append(dict(h=ho, w=wo, c=cout, scale=out_scale, zp=out_zp, rms=out_rms))
+        ops.append(dict(op="dw" if depthwise else "conv", src=src, dst=len(tensors) - 1, k=k, stride=stride, pad=pad,
+                        cout=cout, relu6=relu6, w_scale=w_scale, w_zp=120 + idx % 16, w_seed=SEED + 3 * idx,
+                        b_seed=SEED + 3 * idx + 1, b_range=max(1, int(acc_sd / 4))))
+        return len(tensors) - 1
+
+    cur = conv(0, 32, 3, 2, True)
+    for t_exp, c, n, s in BOTTLENECKS:
+        for rep in range(n):
+            block_in = cur
+            cin = tensors[cur]["c"]
+            x = cur
+            if t_exp != 1:
+                x = conv(x, cin * t_exp, 1, 1, True)
+            x = conv(x, tensors[x]["c"], 3, s if rep == 0 else 1, True, depthwise=True)
+            x = conv(x, c, 1, 1, False)
+            if rep > 0 and cin == c:   # stride 1 and equal shapes: residual connection
+                a, b = tensors[block_in], tensors[x]
+                real_sd = math.hypot(a["rms"] * a["scale"], b["rms"] * b["scale"])
+                tensors.append(dict(h=b["h"], w=b["w"], c=c, scale=real_sd / LINEAR_SD, zp=128, rms=LINEAR_SD))
+                ops.append(dict(op="add", a=block_in, b=x, dst=len(tensors) - 1))
+                x = len(tensors) - 1
+            cur = x
+    cur = conv(cur, 1280, 1, 1, True)
+    t = tensors[cur]
+    tensors.append(dict(h=1, w=1, c=t["c"], scale=t["scale"], zp=t["zp"], rms=30.0))
+    ops.append(dict(op="avgpool", src=cur, dst=len(tensors) - 1, k=t["h"]))
+    cur = len(tensors) - 1
+    t = tensors[cur]
+    idx = len(ops)
+    acc_sd = math.sqrt(t["c"]) * W_SD * t["rms"]
+    tensors.append(dict(h=1, w=1, c=1000, scale=0.05, zp=128, rms=LINEAR_SD))
+    ops.append(dict(op="fc", src=cur, dst=len(tensors) - 1, cout=1000, w_scale=(LINEAR_SD / acc_sd) * 0.05 / t["scale"],
+                    w_zp=128, w_seed=SEED + 3 * idx, b_seed=SEED + 3 * idx + 1, b_range=max(1, int(acc_sd / 4))))
+    return tensors, ops
+
+
+def op_weights(op, cin):
+    """(weights, bias) of a conv / dw / fc operator: OIHW uint8 (depthwise: [C, 1, k, k]; fc: [N, K]) and int32."""
+    if op["op"] == "fc":
+        shape = (op["cout"], cin)
+    elif op["op"] == "dw":
+        shape = (op["cout"], 1, op["k"], op["k"])
+    else:
+        shape = (op["cout"], cin, op["k"], op["k"])
+    w = synth.fill_u8_normal(shape, op["w_seed"], op["w_zp"], W_SD)
+    b = synth.fill_i32((op["cout"],), op["b_seed"], -op["b_range"], op["b_range"])
+    return w, b
+
+
+def network_input(batch, image=224):
+    """uint8 uniform[0, 255], channels-last [batch, image, image, 3]"""
+    return synth.fill_u8((batch, image, image, 3), SEED + 9999)
+
+
+def macs_per_image(image=224):
+    tensors, ops = layers(image)
+    total = 0
+    for op in ops:
+        if op["op"] in ("conv", "dw", "fc"):
+            d = tensors[op["dst"]]
+            cin = tensors[op["src"]]["c"]
+            k2 = op.get("k", 1) ** 2
+            total += d["h"] * d["w"] * d["c"] * k2 * (1 if op["op"] == "dw" else cin)
+    return total
+
+
+def compulsory_bytes_per_image(image=224):
+    """activations in and out of every operator, once each (weights excluded: they are shared by the batch)"""
+    tensors, ops = layers(image)
+    size = lambda i: tensors[i]["h"] * tensors[i]["w"] * tensors[i]["c"]
+    total = 0
+    for op in ops:
+        srcs = [op["a"], op["b"]] if op["op"] == "add" else [op["src"]]
+        total += sum(size(i) for i in srcs) + size(op["dst"])
+    return total
+
+
+class MobileNetV2:
+    """The operator list instantiated on the GPU for one batch size.  Activations are channels-last."""
+
+    def __init__(self, eden, batch, image=224, stream=None):
+        self.eden, self.batch, self.image = eden, batch, image
+        self.tensors, self.ops = layers(image)
+        self.buffers = [eden.DeviceBuffer(nbytes=batch * t["h"] * t["w"] * t["c"]) for t in self.tensors]
+        self.steps = []
+        self._keep = []
+        for op in self.ops:
+            kind = op["op"]
+            if kind == "add":
+                a, b, d = (self.tensors[op[k]] for k in ("a", "b", "dst"))
+                q = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
+                count = batch * d["h"] * d["w"] * d["c"]
+                self.steps.append(("add", (self.buffers[op["a"]], self.buffers[op["b"]], self.buffers[op["dst"]], count, q)))
+                continue
+            s, d = self.tensors[op["src"]], self.tensors[op["dst"]]
+            if kind == "avgpool":
+                self.steps.append(("avgpool", (self.buffers[op["src"]], self.buffers[op["dst"]], s, op["k"])))
+                continue
+            w, b = op_weights(op, s["c"])
+            d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+            self._keep += [d_w, d_b]
+            act = eden.ACT_RELU6 if op.get("relu6") else eden.ACT_NONE
+            q = eden.make_requant(s["scale"], s["zp"], op["w_scale"], op["w_zp"], d["scale"], d["zp"], act, bool(op.get("relu6")))
+            if kind == "fc":
+                plan = eden.FcPlan(batch, s["c"], op["cout"], d_w, d_b, q, stream)
+            else:
+                pad = (op["pad"],) * 4
+                if kind == "dw":
+                    desc = eden.conv_desc(batch, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, pad,
+                                          (1, 1), 1, 1, eden.NHWC, eden.W_OIHW)
+                    plan = eden.DwConvPlan(desc, d_w, d_b, q, stream)
+                else:
+                    desc = eden.conv_desc(batch, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, pad,
+                                          (1, 1), 1, 1, eden.NHWC, eden.W_OIHW)
+                    plan = eden.ConvPlan(desc, d_w, d_b, q, stream)
+            self.steps.append(("plan", (plan, self.buffers[op["src"]], self.buffers[op["dst"]], q)))
+        eden.sync(stream)
+
+    def set_input(self, x_nhwc):
+        x = np.ascontiguousarray(x_nhwc, np.uint8)
+        assert x.shape == (self.batch, self.image, self.image, 3)
+        lib = self.eden.load()
+        self.eden.check(lib.eh_h2d(self.buffers[0].ptr, x.ctypes.data, x.nbytes, None))
+        self.eden.sync()
+
+    def run(self, stream=None):
+        """Enqueues every operator in order on `stream` (a raw handle or None)."""
+        eden = self.eden
+        for kind, args in self.steps:
+            if kind == "plan":
+                plan, src, dst, q = args
+                plan.run(src, dst, q, stream)
+            elif kind == "add":
+                a, b, dst, count, q = args
+                eden.add_u8(a, b, dst, count, q, stream)
+            else:
+                src, dst, s, k = args
+                eden.avgpool_u8(src, dst, self.batch, s["c"], s["h"], s["w"], k, k, layout=eden.NHWC, stream=stream)
+
+    def tensor(self, index):
+        """Downloads tensor `index` as [batch, h, w, c]."""
+        t = self.tensors[index]
+        return self.buffers[index].download((self.batch, t["h"], t["w"], t["c"]))
+
+    def logits(self):
+        return self.tensor(len(self.tensors) - 1).reshape(self.batch, -1)

@@ -1,0 +1,90 @@
+"""MobileNetV2-1.0 uint8 (BASELINE configs[4] at a small batch): every operator of the GPU operator list against
+the oracle evaluating the same list, bit-exact tensor by tensor."""
+import importlib
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from harness import eden, to_eh_requant
+
+mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_forward(x_nhwc, image):
+    """All tensors of the network, NCHW, computed by the oracle from the same operator list."""
+    tensors, ops = mobilenet.layers(image)
+    vals = [np.ascontiguousarray(x_nhwc.transpose(0, 3, 1, 2))]
+    n = x_nhwc.shape[0]
+    for op in ops:
+        kind = op["op"]
+        if kind == "add":
+            a, b, d = (tensors[op[k]] for k in ("a", "b", "dst"))
+            q = O.make_add_quant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
+            vals.append(O.add(vals[op["a"]], vals[op["b"]], q))
+            continue
+        s, d = tensors[op["src"]], tensors[op["dst"]]
+        x = vals[op["src"]]
+        if kind == "avgpool":
+            vals.append(O.avgpool(x, op["k"], op["k"]))
+            continue
+        w, b = mobilenet.op_weights(op, s["c"])
+        act = O.ACT_RELU6 if op.get("relu6") else O.ACT_NONE
+        q = O.make_quant(s["scale"], s["zp"], op["w_scale"], op["w_zp"], d["scale"], d["zp"], act, bool(op.get("relu6")))
+        if kind == "fc":
+            vals.append(O.fc(x.reshape(n, -1), w, b, q).reshape(n, -1, 1, 1))
+        elif kind == "dw":
+            shape = O.conv_shape(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4,
+                                 groups=s["c"])
+            vals.append(O.dwconv2d(x, w, b, shape, q))
+        else:
+            shape = O.conv_shape(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4)
+            vals.append(O.conv2d(x, w, b, shape, q))
+    return tensors, ops, vals
+
+
+@pytest.mark.parametrize("batch,image", [(2, 224), (3, 96)])
+def test_mobilenet_v2_matches_oracle_tensor_by_tensor(batch, image):
+    print("mobilenet", batch, image, flush=True)
+    x = mobilenet.network_input(batch, image)
+    tensors, ops, want = oracle_forward(x, image)
+    net = mobilenet.MobileNetV2(eden, batch, image)
+    net.set_input(x)
+    net.run()
+    eden.sync()
+    for op in ops:
+        i = op["dst"]
+        got = net.tensor(i).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, want[i]), (op["op"], i, tensors[i], int((got != want[i]).sum()))
+    logits = want[-1].reshape(batch, -1)
+    # the network is alive: no operator's output has collapsed to a constant or to the clamps
+    for op in ops:
+        v = want[op["dst"]]
+        assert v.std() > 8, (op["op"], op["dst"], float(v.std()))
+        assert np.mean((v == 0) | (v == 255)) < 0.8, (op["op"], op["dst"])
+    assert len(np.unique(logits)) > 40
+    assert not np.array_equal(logits[0], logits[1])
+
+
+def test_mobilenet_v2_graph_replay_equals_eager():
+    """The whole operator list captured once; every replay (with eager work between replays) gives the eager logits."""
+    batch, image = 2, 96
+    x = mobilenet.network_input(batch, image)
+    net = mobilenet.MobileNetV2(eden, batch, image)
+    net.set_input(x)
+    net.run()
+    eden.sync()
+    eager = net.logits().copy()
+    stream = eden.Stream()
+    graph = eden.Graph(stream, lambda s: net.run(s))
+    lib = eden.load()
+    for rep in range(3):
+        eden.check(lib.eh_memset(net.buffers[-1].ptr, 0, eager.size, None))
+        eden.sync()
+        graph.launch(stream)
+        stream.sync()
+        assert np.array_equal(net.logits(), eager), rep
+        net.run()           # eager work between the replays
+        eden.sync()
