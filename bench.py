@@ -148,6 +148,16 @@ def deconv_workload(eden, synth, n=8):
                 bytes=n * 256 * 1024 + 256 * 128 * 16 + 512 + n * 128 * 4096, bound="mfma")
 
 
+def mbv2_workload(eden, synth, batch=64):
+    """BASELINE.json configs[4]: MobileNetV2-1.0 uint8 at 224x224x3, batch 64, the whole operator list per step."""
+    mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+    net = mobilenet.MobileNetV2(eden, batch)
+    net.set_input(mobilenet.network_input(batch))
+    return dict(name="mobilenet_v2_1.0_224_u8_batch%d" % batch, launch=lambda s: net.run(s), keep=net,
+                ops=2.0 * mobilenet.macs_per_image() * batch, bytes=mobilenet.compulsory_bytes_per_image() * batch,
+                bound="hbm", images=batch, chunk=4)
+
+
 def copy_workload(eden, synth, mib=64):
     """A plain device-to-device copy of known size: the yardstick the HBM byte counters are scaled by."""
     nbytes = mib << 20
@@ -197,7 +207,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv, mbv2, copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (got --gpus %d); no multi-GPU figure exists" % args.gpus,
@@ -213,12 +223,15 @@ def main():
 
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
                     fcbig=lambda e, s: fc_workload(e, s, 8192, 4096, 4096), conv64=lambda e, s: conv_workload(e, s, 64),
-                    copy=copy_workload)
+                    copy=copy_workload, mbv2=mbv2_workload)
     if args.only:
         work = families[args.only](eden, synth)
-        wall, ev = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph)
-        print(json.dumps(dict(workload=work["name"], steps=args.steps, ms_per_step=wall / args.steps * 1e3,
-                              roofline=roofline(work, ev, args.steps))))
+        wall, ev = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph, work.get("chunk", 50))
+        line = dict(workload=work["name"], steps=args.steps, ms_per_step=wall / args.steps * 1e3,
+                    roofline=roofline(work, ev, args.steps))
+        if "images" in work:
+            line["images_per_s"] = round(work["images"] * args.steps / wall, 1)
+        print(json.dumps(line))
         return
 
     work = fc_workload(eden, synth)
@@ -249,11 +262,14 @@ def main():
         others = []
         for make, steps in ((conv_workload, 2000), (lambda e, s: conv_workload(e, s, 64), 300), (pw_workload, 500),
                             (dw_workload, 1000), (deconv_workload, 500),
-                            (lambda e, s: fc_workload(e, s, 8192, 4096, 4096), 100)):
+                            (lambda e, s: fc_workload(e, s, 8192, 4096, 4096), 100), (mbv2_workload, 40)):
             w2 = make(eden, synth)
-            wall2, ev2 = time_steps(eden, stream, w2["launch"], steps, max(10, steps // 10), use_graph)
-            others.append(dict(workload=w2["name"], steps=steps, tops=round(w2["ops"] * steps / wall2 / 1e12, 2),
-                               roofline=roofline(w2, ev2, steps)))
+            wall2, ev2 = time_steps(eden, stream, w2["launch"], steps, max(10, steps // 10), use_graph, w2.get("chunk", 50))
+            entry = dict(workload=w2["name"], steps=steps, tops=round(w2["ops"] * steps / wall2 / 1e12, 2),
+                         roofline=roofline(w2, ev2, steps))
+            if "images" in w2:
+                entry["images_per_s"] = round(w2["images"] * steps / wall2, 1)
+            others.append(entry)
             del w2
         result["others"] = others
     print(json.dumps(result))

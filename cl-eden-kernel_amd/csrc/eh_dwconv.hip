@@ -86,6 +86,82 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
     *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) = o;
 }
 
+// 3x3, dilation 1, stride S in both directions: a thread owns four adjacent channels of FOUR
+// horizontally adjacent output pixels.  The 3 x (3 * S + 3) input pixels they need are loaded
+// once (every load is issued before the first use, from clamped in-image addresses; taps
+// outside the image are then replaced by the input zero point), so the address arithmetic, the
+// weight and bias loads and the border tests are shared by sixteen outputs.
+template <int S>
+__global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
+                                                               const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
+    constexpr int TW = 4, IW = (TW - 1) * S + 3;
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    // idx -> (image, output row, tile of four output columns, channel quad), channel quad fastest;
+    // all offsets fit 32 bits (the launcher checks the tensor sizes)
+    const uint32_t cq_count = (uint32_t)p.c >> 2;
+    uint32_t r = fastdiv(idx, div_cq);
+    const uint32_t cq = idx - r * cq_count;
+    const uint32_t r2 = fastdiv(r, div_tiles);
+    const int tx = (int)(r - r2 * (uint32_t)tiles_x);
+    const uint32_t img = fastdiv(r2, div_ho);
+    const int oy = (int)(r2 - img * (uint32_t)p.ho);
+    const int ox0 = tx * TW;
+    const int iy0 = oy * S - p.pad_t, ix0 = ox0 * S - p.pad_l;
+    const uint32_t fill = (uint32_t)p.zp_in * 0x01010101u;
+    const uint32_t base = img * (uint32_t)(p.h * p.w_ * p.c) + cq * 4u;
+
+    uint32_t col_off[IW];
+    bool col_ok[IW];
+#pragma unroll
+    for (int x = 0; x < IW; ++x) {
+        const int ix = ix0 + x;
+        col_ok[x] = (unsigned)ix < (unsigned)p.w_;
+        const int ixc = ix < 0 ? 0 : (ix >= p.w_ ? p.w_ - 1 : ix);
+        col_off[x] = base + (uint32_t)ixc * (uint32_t)p.c;
+    }
+    uint32_t in[3][IW];
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+        const int iy = iy0 + ky;
+        const bool row_ok = (unsigned)iy < (unsigned)p.h;
+        const int iyc = iy < 0 ? 0 : (iy >= p.h ? p.h - 1 : iy);
+        const uint32_t row_off = (uint32_t)iyc * (uint32_t)(p.w_ * p.c);
+#pragma unroll
+        for (int x = 0; x < IW; ++x) {
+            const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in + (row_off + col_off[x]));
+            in[ky][x] = row_ok && col_ok[x] ? v : fill;
+        }
+    }
+    int4 w4[5];
+#pragma unroll
+    for (int pr = 0; pr < 5; ++pr) w4[pr] = *reinterpret_cast<const int4 *>(p.w_pair + ((uint32_t)pr * (uint32_t)p.cout + cq * 4u));
+    const int4 b4 = *reinterpret_cast<const int4 *>(p.bias_folded + cq * 4u);
+    uint8_t *dst = p.out + (((img * (uint32_t)p.ho + (uint32_t)oy) * (uint32_t)p.wo + (uint32_t)ox0) * (uint32_t)p.cout + cq * 4u);
+    const RequantDev rq = p.rq;
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        int acc0 = b4.x, acc1 = b4.y, acc2 = b4.z, acc3 = b4.w;
+#pragma unroll
+        for (int pr = 0; pr < 5; ++pr) {
+            const int t0 = 2 * pr, t1 = 2 * pr + 1;
+            const uint32_t lo = in[t0 / 3][j * S + t0 % 3];
+            const uint32_t hi = t1 < 9 ? in[t1 / 3][j * S + t1 % 3] : 0u;
+            acc0 = dot2(pair_bytes<0>(lo, hi), w4[pr].x, acc0);
+            acc1 = dot2(pair_bytes<1>(lo, hi), w4[pr].y, acc1);
+            acc2 = dot2(pair_bytes<2>(lo, hi), w4[pr].z, acc2);
+            acc3 = dot2(pair_bytes<3>(lo, hi), w4[pr].w, acc3);
+        }
+        uint32_t o;
+        if (rq.fast)
+            o = requant_u8_fast(acc0, rq) | (requant_u8_fast(acc1, rq) << 8) | (requant_u8_fast(acc2, rq) << 16) |
+                (requant_u8_fast(acc3, rq) << 24);
+        else
+            o = requant_u8(acc0, rq) | (requant_u8(acc1, rq) << 8) | (requant_u8(acc2, rq) << 16) | (requant_u8(acc3, rq) << 24);
+        if (ox0 + j < p.wo) *reinterpret_cast<uint32_t *>(dst + (uint32_t)j * (uint32_t)p.cout) = o;
+    }
+}
+
 // One output element per thread; any depth multiplier, dilation, channel count.
 // NHWC = true: channel fastest.  NHWC = false: planar NCHW, x fastest.
 template <bool NHWC>
@@ -158,7 +234,22 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
     if (outs <= 0) return EH_OK;
     const bool vec = p.dm == 1 && (p.c & 3) == 0 && (reinterpret_cast<uintptr_t>(p.in) & 3) == 0 &&
                      (reinterpret_cast<uintptr_t>(p.out) & 3) == 0;
-    if (vec) {
+    const bool tile3x3 = vec && p.kh == 3 && p.kw == 3 && p.dil_h == 1 && p.dil_w == 1 && p.stride_h == p.stride_w &&
+                         (p.stride_h == 1 || p.stride_h == 2) && (size_t)p.n * p.h * p.w_ * p.c < (1ull << 31) &&
+                         (size_t)p.n * p.ho * p.wo * p.cout < (1ull << 31);
+    if (tile3x3) {
+        const int tiles_x = (p.wo + 3) / 4;
+        const long total = (long)p.n * p.ho * tiles_x * (p.c >> 2);
+        const long blocks = (total + 255) / 256;
+        EH_REQUIRE(total < (1l << 31), "depthwise: grid too large");
+        const FastDiv d_cq = make_fastdiv((uint32_t)(p.c >> 2)), d_t = make_fastdiv((uint32_t)tiles_x), d_ho = make_fastdiv((uint32_t)p.ho);
+        if (p.stride_h == 1)
+            hipLaunchKernelGGL((dw3x3_nhwc_tile4_kernel<1>), dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total,
+                               tiles_x, d_cq, d_t, d_ho);
+        else
+            hipLaunchKernelGGL((dw3x3_nhwc_tile4_kernel<2>), dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total,
+                               tiles_x, d_cq, d_t, d_ho);
+    } else if (vec) {
         const long total = outs / 4;
         const long blocks = (total + 255) / 256;
         EH_REQUIRE(blocks < (1l << 31), "depthwise: grid too large");

@@ -303,6 +303,13 @@ DW_CASES = [
     dict(n=2, c=5, h=10, w=10, cout=5, kh=5, kw=5, pad=(2, 2, 2, 2), dil=(1, 1)),           # odd channel count
     dict(n=1, c=16, h=11, w=13, cout=16, kh=3, kw=3, stride=(1, 1), pad=(2, 2, 2, 2), dil=(2, 2)),
     dict(n=1, c=4, h=5, w=5, cout=4, kh=2, kw=2),
+    # 3x3 tiles of four output pixels: widths that are not multiples of four, every border, both strides
+    dict(n=2, c=16, h=7, w=7, cout=16, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=24, h=14, w=13, cout=24, kh=3, kw=3, stride=(2, 2), pad=(1, 1, 1, 1)),
+    dict(n=1, c=8, h=6, w=9, cout=8, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),
+    dict(n=1, c=8, h=5, w=6, cout=8, kh=3, kw=3, pad=(2, 2, 2, 2)),
+    dict(n=3, c=960, h=7, w=7, cout=960, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=12, h=3, w=1, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1)),
 ]
 
 
