@@ -96,6 +96,11 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base)) {
         g.cfg.id = GEMM_THIN;
         g.cfg.slab = 32;
+    } else if (g.cin == 3 && g.proto.cin == 3 && g.taps == 9 && g.k == 27 && units.size() == 27 && units[26].dy == 2 &&
+               units[26].dx == 2 && units[12].dy == 1 && units[12].dx == 1 && units[0].offset == 0) {
+        // three channels, 3x3 taps, dilation 1: the first layer of image networks
+        g.cfg.id = GEMM_C3K3;
+        g.cfg.slab = 32;
     } else if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
         g.cfg = igemm_dma_select(g.proto.m, g.n, g.k);
     g.k_pad = round_up(g.k > 0 ? g.k : 1, g.cfg.slab);

@@ -87,14 +87,29 @@ __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *_
     x0 = x0 < 0 ? 0 : x0;
     const int cnt = (y1 - y0) * (x1 - x0);
     int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
-    for (int y = y0; y < y1; ++y)
-        for (int x = x0; x < x1; ++x) {
-            const uint32_t v = *reinterpret_cast<const uint32_t *>(in + (((size_t)img * p.h + y) * p.w + x) * p.c + c4 * 4);
-            s0 += v & 255u;
-            s1 += (v >> 8) & 255u;
-            s2 += (v >> 16) & 255u;
-            s3 += v >> 24;
+    auto take = [&](uint32_t v) {
+        s0 += v & 255u;
+        s1 += (v >> 8) & 255u;
+        s2 += (v >> 16) & 255u;
+        s3 += v >> 24;
+    };
+    // eight window pixels are requested before the first is summed: a global pool is one long chain of loads otherwise
+    for (int y = y0; y < y1; ++y) {
+        const uint8_t *row = in + ((size_t)img * p.h + y) * p.w * p.c + c4 * 4;
+        int x = x0;
+        for (; x + 8 <= x1; x += 8) {
+            uint32_t v[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) v[t] = *reinterpret_cast<const uint32_t *>(row + (size_t)(x + t) * p.c);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) take(v[t]);
         }
+        uint32_t v[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v[t] = x + t < x1 ? *reinterpret_cast<const uint32_t *>(row + (size_t)(x + t) * p.c) : 0u;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) take(v[t]);
+    }
     auto fin = [&](int s) -> uint32_t {
         int v = cnt > 0 ? (s + cnt / 2) / cnt : 0;
         v = v < p.act_min ? p.act_min : v;

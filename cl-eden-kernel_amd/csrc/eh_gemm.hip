@@ -287,6 +287,7 @@ int igemm_n_tile(int32_t, int32_t, int32_t) { return 256; }
 int launch_igemm(const GemmProblem &p, hipStream_t stream) {
     if (p.m <= 0 || p.n <= 0) return EH_OK;
     if (p.cfg.id == GEMM_THIN) return launch_igemm_thin(p, stream);
+    if (p.cfg.id == GEMM_C3K3) return launch_conv_c3k3(p, stream);
     EH_REQUIRE(p.k_pad % BK == 0 && p.k_pad > 0, "igemm: padded reduction length %d is not a multiple of %d", p.k_pad, BK);
     EH_REQUIRE(p.vec == 16 || p.vec == 4 || p.vec == 1, "igemm: bad load unit %d", p.vec);
     if (p.cfg.id != GEMM_STAGED) return launch_igemm_dma(p, stream);

@@ -67,8 +67,9 @@ __global__ __launch_bounds__(256) void thin_gemm_kernel(const GemmProblem p, con
 
     // four channel blocks at a time: all their weight fragments and bias values are requested
     // before the first is used, so one memory latency covers the group
+    // (blockIdx.y splits the channel blocks between workgroups when there are few pixels)
     constexpr int NBU = 4;
-    for (int nb0 = 0; nb0 < n_blocks; nb0 += NBU) {
+    for (int nb0 = blockIdx.y * NBU; nb0 < n_blocks; nb0 += gridDim.y * NBU) {
         v4i bf[NBU][KSTEPS];
         int4 bb[NBU][4];
 #pragma unroll
@@ -113,7 +114,11 @@ __global__ __launch_bounds__(256) void thin_gemm_kernel(const GemmProblem p, con
 template <int KSTEPS>
 int launch_steps(const GemmProblem &p, hipStream_t stream) {
     const int n_blocks = (p.n + 31) / 32;
-    const dim3 grid((p.m + 127) / 128);
+    // enough waves to fill 256 CUs several times over: with few pixels the channel blocks are spread over grid.y too
+    const int row_groups = (p.m + 127) / 128, n_groups = (n_blocks + 3) / 4;
+    int split = 1;
+    while (split < n_groups && (long)row_groups * split < 2048) ++split;
+    const dim3 grid(row_groups, split);
     if (p.zw != 0) {
         if (p.rq.fast)
             hipLaunchKernelGGL((thin_gemm_kernel<KSTEPS, true, true>), grid, dim3(256), 0, stream, p, n_blocks);

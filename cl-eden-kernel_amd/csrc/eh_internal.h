@@ -155,6 +155,7 @@ enum GemmConfigId {
     GEMM_DMA_64x64_SPLITK = 4,
     GEMM_DMA_256x256 = 5,
     GEMM_THIN = 6,              // one-tap problems with at most 64 reduction bytes; weights in MFMA fragment order
+    GEMM_C3K3 = 7,              // 3 input channels, 3x3 taps (first layers); weights row-major [n_pad][32]
 };
 struct GemmConfig {
     int32_t id = GEMM_STAGED;
@@ -191,6 +192,7 @@ int launch_igemm_dma(const GemmProblem &p, hipStream_t stream);  // vec == 16 an
 GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k);
 inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
+int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
 bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, int32_t channel_offset, int32_t y_base,
                         int32_t x_base);
 // Byte offset of reduction chunk `kc16` (16-byte units) of packed weight row `n`.
@@ -200,7 +202,7 @@ bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, i
 // 16h + 4g + t sits in row 8g + 4h + t): a lane of the 32x32x32 MFMA holds result
 // rows 8g + 4h + t (h = lane / 32), which this way are 16 consecutive channels.
 __host__ __device__ inline size_t packed_b_offset(const GemmConfig &cfg, int n, int kc16, int k_pad) {
-    if (cfg.id == GEMM_STAGED) return (size_t)n * k_pad + (size_t)kc16 * 16;
+    if (cfg.id == GEMM_STAGED || cfg.id == GEMM_C3K3) return (size_t)n * k_pad + (size_t)kc16 * 16;
     const int ch = n & 31;
     n = (n & ~31) | (((ch & 15) >> 2) << 3) | ((ch >> 4) << 2) | (ch & 3);
     // fragment order: [32-channel block][32-byte step][lane = 32 * (chunk & 1) + row][16 bytes]

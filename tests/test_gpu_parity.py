@@ -162,6 +162,11 @@ CONV_CASES = [
     dict(n=2, c=64, h=12, w=12, cout=32, kh=1, kw=1),
     dict(n=1, c=48, h=10, w=10, cout=96, kh=1, kw=1, groups=2),                             # 24-byte rows inside 48-byte pixels
     dict(n=5, c=16, h=33, w=5, cout=96, kh=1, kw=1, stride=(1, 2)),
+    # three channels, 3x3: the first-layer kernel (unaligned 12-byte reads; byte path at the two ends of the tensor)
+    dict(n=2, c=3, h=32, w=32, cout=32, kh=3, kw=3, stride=(2, 2), pad=(1, 1, 1, 1)),
+    dict(n=1, c=3, h=9, w=10, cout=20, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=3, c=3, h=5, w=3, cout=16, kh=3, kw=3, pad=(2, 0, 0, 2)),
+    dict(n=1, c=3, h=3, w=3, cout=5, kh=3, kw=3),
 ]
 
 
