@@ -93,7 +93,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     // the kernel shape is fixed here because the packed weight layout depends on it
     g.cfg = GemmConfig();
     if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 &&
-        igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base)) {
+        igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base, g.proto.m, g.n)) {
         g.cfg.id = GEMM_THIN;
         g.cfg.slab = 32;
     } else if (g.cin == 3 && g.proto.cin == 3 && g.taps == 9 && g.k == 27 && units.size() == 27 && units[26].dy == 2 &&
@@ -122,6 +122,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     // the host vectors die with the caller's frame: make sure the copies have left them
     EH_HIP(hipStreamSynchronize(stream));
     g.proto.ktab = g.ktab;
+    g.proto.a_offset = units.empty() ? 0 : units[0].offset;
     g.proto.k = g.k;
     g.proto.k_pad = g.k_pad;
     g.proto.vec = g.vec;

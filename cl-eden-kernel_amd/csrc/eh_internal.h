@@ -154,7 +154,7 @@ enum GemmConfigId {
     GEMM_DMA_128x64 = 3,
     GEMM_DMA_64x64_SPLITK = 4,
     GEMM_DMA_256x256 = 5,
-    GEMM_THIN = 6,              // one-tap problems with at most 64 reduction bytes; weights in MFMA fragment order
+    GEMM_THIN = 6,              // one-tap problems short of work for tiles; weights in MFMA fragment order
     GEMM_C3K3 = 7,              // 3 input channels, 3x3 taps (first layers); weights row-major [n_pad][32]
 };
 struct GemmConfig {
@@ -183,6 +183,7 @@ struct GemmProblem {
     FastDiv div_plane, div_wo;  // row decode: m / (ho * wo), rem / wo
     int32_t dense;     // 1: a plain [m][k] matrix with row stride cin and k a multiple of the slab (no taps, no padding)
     int32_t zw;        // zp_w - 128: coefficient of the per-row activation sum
+    int32_t a_offset;  // one-tap problems: byte offset of the (group's) first channel within a pixel
     uint32_t fill;     // input zero point replicated in 4 bytes (value of an out-of-image tap)
     RequantDev rq;
 };
@@ -194,7 +195,7 @@ inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
 bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, int32_t channel_offset, int32_t y_base,
-                        int32_t x_base);
+                        int32_t x_base, int64_t m, int64_t n);
 // Byte offset of reduction chunk `kc16` (16-byte units) of packed weight row `n`.
 // Direct-to-LDS layouts: 1 KiB blocks of (1024 / slab) rows x slab bytes, ordered
 // [row block][slab index], the 16-byte chunks of a row XOR-swizzled by the row index.

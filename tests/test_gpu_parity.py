@@ -76,12 +76,18 @@ def test_fc_matches_oracle(m, k, n, zp_a, zp_w):
     assert want.std() > 10  # the case exercises the requant range, not a saturated constant
 
 
-# shapes chosen to land on each large-tile kernel configuration (by tile count), ragged in m and n
+# shapes chosen to land on each large-tile kernel configuration (by tile count), ragged in m and n, and with
+# enough multiply-adds (over 1.5e9) that the one-tap latency kernel does not take them
 BIG_FC_CASES = [
     (16384 - 37, 128, 1024 - 24, 9, 77),    # 256 x 256 tiles
-    (65536 - 5, 128, 128 - 16, 200, 128),   # 256 x 128 tiles
-    (16384 - 100, 192, 256, 128, 3),        # 128 x 128 tiles
-    (32768 - 3, 64, 64 - 8, 17, 250),       # 128 x 64 tiles
+    (65536 - 5, 256, 128 - 16, 200, 128),   # 256 x 128 tiles
+    (16384 - 100, 384, 256, 128, 3),        # 128 x 128 tiles
+    (32768 - 3, 896, 64 - 8, 17, 250),      # 128 x 64 tiles
+    # the one-tap kernel with a long reduction loop and every channel-group width
+    (3000, 96, 576, 77, 120),
+    (3136 - 7, 256, 320, 0, 131),
+    (520, 200, 24, 250, 5),
+    (12544, 144, 40, 3, 128),
 ]
 
 
