@@ -299,7 +299,8 @@ int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int6
     const RequantDev r = make_requant_dev(*q);
     const bool fast = form == 0 && r.fast;
     if (single_shift) *single_shift = fast ? 1 : 0;
-    for (int64_t i = 0; i < count; ++i) out[i] = (uint8_t)(fast ? requant_u8_fast(acc[i], r) : requant_u8(acc[i], r));
+    for (int64_t i = 0; i < count; ++i)
+        out[i] = (uint8_t)(!fast ? requant_u8(acc[i], r) : r.fast == 2 ? requant_u8_fast_relu(acc[i], r) : requant_u8_fast(acc[i], r));
     return EH_OK;
 }
 

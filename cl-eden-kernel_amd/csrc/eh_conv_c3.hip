@@ -11,6 +11,8 @@
 //
 // Stands in for the reference's direct convolution kernels on this shape
 // (gpu/operators/cl_kernels/DirectConvolutionKernel.cpp, 3x3 uint8 variants).
+#include <type_traits>
+
 #include "eh_internal.h"
 
 namespace eh {
@@ -81,6 +83,8 @@ __global__ __launch_bounds__(256) void conv_c3k3_kernel(const GemmProblem p, con
     }
     const RequantDev rq = p.rq;
     uint32_t packed[4];
+    auto produce = [&](auto mode_c) {
+    constexpr int mode = decltype(mode_c)::value;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         uint32_t o[4];
@@ -91,10 +95,17 @@ __global__ __launch_bounds__(256) void conv_c3k3_kernel(const GemmProblem p, con
             int acc = p.bias[n] + ncorr;
 #pragma unroll
             for (int i = 0; i < 7; ++i) acc = __builtin_amdgcn_sdot4((int)A[i], wrow[i], acc, false);
-            o[t] = requant_u8_as<FAST>(acc, rq);
+            o[t] = requant_u8_as<mode>(acc, rq);
         }
         packed[g] = o[0] | (o[1] << 8) | (o[2] << 16) | (o[3] << 24);
     }
+    };
+    if constexpr (!FAST)
+        produce(std::integral_constant<int, 0>{});
+    else if (rq.fast == 2)
+        produce(std::integral_constant<int, 2>{});
+    else
+        produce(std::integral_constant<int, 1>{});
     uint8_t *dst = p.out + (((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0)) * (size_t)p.ldc + n0;
     const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
     if (aligned16 && n0 + 16 <= p.n) {

@@ -153,7 +153,10 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p
             acc3 = dot2(pair_bytes<3>(lo, hi), w4[pr].w, acc3);
         }
         uint32_t o;
-        if (rq.fast)
+        if (rq.fast == 2)
+            o = requant_u8_fast_relu(acc0, rq) | (requant_u8_fast_relu(acc1, rq) << 8) | (requant_u8_fast_relu(acc2, rq) << 16) |
+                (requant_u8_fast_relu(acc3, rq) << 24);
+        else if (rq.fast)
             o = requant_u8_fast(acc0, rq) | (requant_u8_fast(acc1, rq) << 8) | (requant_u8_fast(acc2, rq) << 16) |
                 (requant_u8_fast(acc3, rq) << 24);
         else

@@ -392,7 +392,8 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         // whole tiles with 16-byte aligned rows (the usual case) store without any per-store test
         const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
         auto emit = [&](auto checked_c, auto fast_c) {
-            constexpr bool checked = decltype(checked_c)::value, fast = decltype(fast_c)::value;
+            constexpr bool checked = decltype(checked_c)::value;
+            constexpr int fast = decltype(fast_c)::value;
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const int nl = wn * WTN + j * 32 + fhalf * 16, n = n0 + nl;  // this lane's 16 consecutive channels
@@ -427,10 +428,14 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
             }
         };
         // edge tiles and unusual requantization parameters take the general code
-        if (rq.fast && aligned16 && m0 + BM <= p.m && n0 + BN <= p.n)
-            emit(std::false_type{}, std::true_type{});
-        else
-            emit(std::true_type{}, std::false_type{});
+        if (rq.fast && aligned16 && m0 + BM <= p.m && n0 + BN <= p.n) {
+            if (rq.fast == 2)
+                emit(std::false_type{}, std::integral_constant<int, 2>{});
+            else
+                emit(std::false_type{}, std::integral_constant<int, 1>{});
+        } else {
+            emit(std::true_type{}, std::integral_constant<int, 0>{});
+        }
     } else {
         // the WGK partial tiles meet in LDS: [wk][pixel row][channel], rows padded so that
         // eight consecutive rows of 16-byte accesses fall in distinct banks
@@ -462,7 +467,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
         const int32_t *pr = reinterpret_cast<const int32_t *>(stages) + ml * PART_ROW + nl;
         uint32_t packed[4];
         auto reduce = [&](auto fast_c) {
-            constexpr bool fast = decltype(fast_c)::value;
+            constexpr int fast = decltype(fast_c)::value;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             int4 s4 = *reinterpret_cast<const int4 *>(pr + g * 4);
@@ -480,10 +485,12 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
             packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
         }
         };
-        if (rq.fast)
-            reduce(std::true_type{});
+        if (rq.fast == 2)
+            reduce(std::integral_constant<int, 2>{});
+        else if (rq.fast == 1)
+            reduce(std::integral_constant<int, 1>{});
         else
-            reduce(std::false_type{});
+            reduce(std::integral_constant<int, 0>{});
         uint8_t *dst = p.out + out_pixel_offset(p, m, plane) + n;
         const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
         if (aligned16 && n + 16 <= p.n) {

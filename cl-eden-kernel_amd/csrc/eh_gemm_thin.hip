@@ -14,6 +14,8 @@
 // The weight fragment is the row operand and its rows are permuted within a
 // 32-channel block (see packed_b_offset), so a lane ends up with 16 consecutive
 // output channels of its pixel: requantize, pack, one 16-byte store.
+#include <type_traits>
+
 #include "eh_internal.h"
 
 namespace eh {
@@ -128,14 +130,23 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                 for (int t = 0; t < KU; ++t) acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bfs[t][u], afs[t], acc[0], 0, 0, 0);
             }
             uint32_t packed[4];
+            auto quantize = [&](auto mode_c) {
+                constexpr int mode = decltype(mode_c)::value;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const uint32_t o0 = requant_u8_as<FAST>(acc[ai][g * 4 + 0] + bb[u][g].x + ncorr, rq);
-                const uint32_t o1 = requant_u8_as<FAST>(acc[ai][g * 4 + 1] + bb[u][g].y + ncorr, rq);
-                const uint32_t o2 = requant_u8_as<FAST>(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, rq);
-                const uint32_t o3 = requant_u8_as<FAST>(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, rq);
-                packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
-            }
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t o0 = requant_u8_as<mode>(acc[ai][g * 4 + 0] + bb[u][g].x + ncorr, rq);
+                    const uint32_t o1 = requant_u8_as<mode>(acc[ai][g * 4 + 1] + bb[u][g].y + ncorr, rq);
+                    const uint32_t o2 = requant_u8_as<mode>(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, rq);
+                    const uint32_t o3 = requant_u8_as<mode>(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, rq);
+                    packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+                }
+            };
+            if constexpr (!FAST)
+                quantize(std::integral_constant<int, 0>{});
+            else if (rq.fast == 2)
+                quantize(std::integral_constant<int, 2>{});
+            else
+                quantize(std::integral_constant<int, 1>{});
             if (!row_ok || n >= p.n) continue;
             uint8_t *dst = p.out + out_off + n;
             if (aligned16 && n + 16 <= p.n) {

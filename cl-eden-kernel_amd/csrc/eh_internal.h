@@ -40,7 +40,7 @@ struct RequantDev {
     int32_t zp_out;
     int32_t act_min;
     int32_t act_max;
-    // single-shift form (see requant_u8_fast); valid when `fast` is set
+    // single-shift form (see requant_u8_fast); valid when `fast` is set (2: the sign test may be skipped too)
     int32_t fast;
     int32_t fast_shift;        // right_shift - 1
     uint32_t pos_lo, pos_hi;   // 64-bit rounding term for accumulators >= 0
@@ -86,9 +86,32 @@ __host__ __device__ __forceinline__ uint32_t requant_u8_fast(int32_t x, const Re
     return (uint32_t)v;
 }
 
-template <bool FAST>
+// Where the clamp floor is not below the output zero point (a fused ReLU-type activation),
+// every negative accumulator ends on the floor whichever way its tie is broken (the quotient
+// with the non-negative rounding term is still <= 0), so the sign test can go.
+__host__ __device__ __forceinline__ uint32_t requant_u8_fast_relu(int32_t x, const RequantDev &r) {
+    const int64_t term = (int64_t)(((uint64_t)r.pos_hi << 32) | r.pos_lo);
+    const int64_t t = (int64_t)x * (int64_t)r.multiplier + term;
+    int32_t v = (int32_t)(t >> 32) >> r.fast_shift;
+#if defined(__HIP_DEVICE_COMPILE__)
+    // act_min <= act_max always holds, so the clamp is a median of three (one instruction; the
+    // compiler cannot assume the ordering and would emit max + min)
+    int32_t o;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(o) : "v"(v), "s"(r.act_min), "v"(r.act_max));
+    return (uint32_t)o;
+#else
+    v = v < r.act_min ? r.act_min : v;
+    v = v > r.act_max ? r.act_max : v;
+    return (uint32_t)v;
+#endif
+}
+
+// MODE 0: two-step reference order; 1: single shift; 2: single shift without the sign test
+template <int MODE>
 __host__ __device__ __forceinline__ uint32_t requant_u8_as(int32_t acc, const RequantDev &r) {
-    if constexpr (FAST)
+    if constexpr (MODE == 2)
+        return requant_u8_fast_relu(acc, r);
+    else if constexpr (MODE == 1)
         return requant_u8_fast(acc, r);
     else
         return requant_u8(acc, r);
@@ -109,6 +132,7 @@ inline RequantDev make_requant_dev(const eh_requant &q) {
               q.zp_out <= 1024)
                  ? 1
                  : 0;
+    if (r.fast && q.act_min >= q.zp_out) r.fast = 2;
     r.fast_shift = r.fast ? r.right_shift - 1 : 0;
     const int rs = r.fast ? r.right_shift : 1;
     const int64_t pos = (1ll << 30) + (1ll << (30 + rs)) + (int64_t)q.zp_out * (1ll << (31 + rs));
