@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include <new>
+#include <algorithm>
 #include <vector>
 
 #include "eh_internal.h"
@@ -89,7 +90,8 @@ int pick_vec(int cig, int pixel_stride) {
 
 // Allocates a part's device arrays and uploads its tables.  `units` holds one
 // KUnit per `vec` bytes of the real reduction length; padding units are added here.
-int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream) {
+int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream,
+                int siblings = 1) {
     // the kernel shape is fixed here because the packed weight layout depends on it
     g.cfg = GemmConfig();
     if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 &&
@@ -102,7 +104,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         g.cfg.id = GEMM_C3K3;
         g.cfg.slab = 32;
     } else if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
-        g.cfg = igemm_dma_select(g.proto.m, g.n, g.k);
+        g.cfg = igemm_dma_select(g.proto.m, g.n, g.k, siblings);
     g.k_pad = round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
     g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
     KUnit pad;
@@ -227,6 +229,8 @@ struct GemmOp {
             in = stage_in;
             out = stage_out;
         }
+        std::vector<GemmProblem> problems;
+        problems.reserve(parts.size());
         for (auto &g : parts) {
             GemmProblem p = g.proto;
             EH_REQUIRE((reinterpret_cast<uintptr_t>(in) & (uintptr_t)(g.vec - 1)) == 0,
@@ -239,8 +243,9 @@ struct GemmOp {
             p.zw = q.zp_w - 128;
             p.fill = (uint32_t)q.zp_in * 0x01010101u;
             p.rq = make_requant_dev(q);
-            if ((rc = launch_igemm(p, stream))) return rc;
+            problems.push_back(p);
         }
+        if ((rc = launch_igemm_batch(problems.data(), (int)problems.size(), stream))) return rc;
         if (layout == EH_NCHW) {
             if ((rc = launch_nhwc2nchw(stage_out, static_cast<uint8_t *>(output), in_n, cout, out_hw, stream))) return rc;
         }
@@ -605,7 +610,7 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
         p.out_y0 = 0;
         p.out_x0 = 0;
         p.ldc = d->cout;
-        if ((rc = finish_part(part, units, tap_off, stream))) return rc;
+        if ((rc = finish_part(part, units, tap_off, stream, std::min(G, (int)GemmBatch::MAX)))) return rc;
     }
     return EH_OK;
 }
@@ -844,7 +849,9 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                 p.out_y0 = oy0;
                 p.out_x0 = ox0;
                 p.ldc = d->cout;
-                if ((rc = finish_part(part, units, tap_off, stream))) return rc;
+                // phases (and groups) of equal shape share launches: choose the tile shape for the joint tile count
+                const int siblings = (d->kh % sh == 0 && d->kw % sw == 0) ? std::min(G * sh * sw, (int)GemmBatch::MAX) : 1;
+                if ((rc = finish_part(part, units, tap_off, stream, siblings))) return rc;
             }
     return EH_OK;
 }

@@ -290,7 +290,7 @@ int launch_igemm(const GemmProblem &p, hipStream_t stream) {
     if (p.cfg.id == GEMM_C3K3) return launch_conv_c3k3(p, stream);
     EH_REQUIRE(p.k_pad % BK == 0 && p.k_pad > 0, "igemm: padded reduction length %d is not a multiple of %d", p.k_pad, BK);
     EH_REQUIRE(p.vec == 16 || p.vec == 4 || p.vec == 1, "igemm: bad load unit %d", p.vec);
-    if (p.cfg.id != GEMM_STAGED) return launch_igemm_dma(p, stream);
+    if (p.cfg.id != GEMM_STAGED) return launch_igemm_dma(&p, 1, stream);
     // Pick the largest tile that still spreads the problem over the 256 CUs.
     const long tiles128 = (long)((p.m + 127) / 128) * ((p.n + 127) / 128);
     const long tiles64 = (long)((p.m + 63) / 64) * ((p.n + 63) / 64);
@@ -299,6 +299,29 @@ int launch_igemm(const GemmProblem &p, hipStream_t stream) {
         return launch_tile<128, 64, 2, 2>(p, stream);
     }
     return launch_tile<64, 64, 2, 2>(p, stream);
+}
+
+int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream) {
+    int i = 0;
+    while (i < count) {
+        const GemmProblem &p = ps[i];
+        int run = 1;
+        const bool dma = p.cfg.id != GEMM_STAGED && p.cfg.id != GEMM_THIN && p.cfg.id != GEMM_C3K3 && p.m > 0 && p.n > 0;
+        if (dma)
+            while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == p.cfg.id && ps[i + run].m == p.m &&
+                   ps[i + run].n == p.n && ps[i + run].k_pad == p.k_pad && ps[i + run].dense == p.dense && ps[i + run].zw == p.zw)
+                ++run;
+        int rc;
+        if (dma && run > 1) {
+            EH_REQUIRE(p.k_pad % 64 == 0 && p.k_pad > 0, "igemm: padded reduction length %d", p.k_pad);
+            rc = launch_igemm_dma(ps + i, run, stream);
+        } else {
+            rc = launch_igemm(p, stream);
+        }
+        if (rc) return rc;
+        i += run;
+    }
+    return EH_OK;
 }
 
 }  // namespace eh

@@ -126,7 +126,8 @@ __device__ __forceinline__ void static_for(F &&f) {
 }
 
 template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES, bool DENSE, bool ROWSUM>
-__global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, const int tiles_m, const int tiles_n, const int gm) {
+__global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, const int count, const int tiles_m, const int tiles_n,
+                                                        const int gm, const int gn) {
     static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
     constexpr int CPR = SLAB / 16;            // 16-byte chunks per LDS row
     constexpr int RPB = 1024 / SLAB;          // rows per 1 KiB DMA block
@@ -156,17 +157,27 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
     extern __shared__ __align__(8) uint8_t ktab_s_raw[];
     KUnit *ktab_s = reinterpret_cast<KUnit *>(ktab_s_raw);
 
-    // Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2,
-    // and an XCD runs 32 of these workgroups at a time (one per CU).  Tiles are
-    // therefore handed out in groups of 32 that form a gm x gn rectangle of the
-    // output: the workgroups of a group walk the reduction axis in step, so every
-    // activation slab is pulled into that L2 once for gn tiles and every weight
-    // slab once for gm tiles.
+    // Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2, and an
+    // XCD runs up to 32 of these workgroups at a time (one per CU).  Tiles are therefore
+    // handed out in groups that form a gm x gn rectangle of the output (32 tiles, fewer when
+    // the whole launch has too few tiles to give every XCD a group): the workgroups of a
+    // group walk the reduction axis in step, so every activation slab is pulled into that
+    // L2 once for gn tiles and every weight slab once for gm tiles.  Equally shaped
+    // problems of one operator (convolution groups, deconvolution phases) share a launch:
+    // their groups are numbered one problem after the other.
+    const int gs = gm * gn;
     const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-    const int group = (j >> 5) * 8 + xcd, within = j & 31;
-    const int groups_m = (tiles_m + gm - 1) / gm;
-    const int gi = group % groups_m, gj = group / groups_m;
-    const int tm = gi * gm + within % gm, tn = gj * (32 / gm) + within / gm;
+    const int jg = __builtin_amdgcn_readfirstlane(j / gs);
+    const int group_all = jg * 8 + xcd, within = j - jg * gs;
+    const int groups_m = (tiles_m + gm - 1) / gm, groups_n = (tiles_n + gn - 1) / gn;
+    // (the divisions run on the vector unit: tell the compiler their results are wave-uniform)
+    const int which = __builtin_amdgcn_readfirstlane(group_all / (groups_m * groups_n));
+    const int group = group_all - which * (groups_m * groups_n);
+    if (which >= count) return;
+    const GemmProblem &p = batch.p[which];
+    const int gj = __builtin_amdgcn_readfirstlane(group / groups_m), gi = group - gj * groups_m;
+    const int wj = __builtin_amdgcn_readfirstlane(within / gm), wi = within - wj * gm;
+    const int tm = gi * gm + wi, tn = gj * gn + wj;
     if (tm >= tiles_m || tn >= tiles_n) return;
     const int m0 = tm * BM, n0 = tn * BN;
 
@@ -423,6 +434,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
                             const int cnt = p.n - n < 16 ? p.n - n : 16;
                             for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
                         }
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
@@ -503,14 +515,20 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmProblem p, con
 }
 
 template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES>
-int launch_cfg(const GemmProblem &p, hipStream_t stream) {
+int launch_cfg(const GemmProblem *ps, int count, hipStream_t stream) {
+    const GemmProblem &p = ps[0];
+    GemmBatch batch;
+    for (int i = 0; i < count; ++i) batch.p[i] = ps[i];
     static_assert(STAGES * (BM + BN) * SLAB + WGK * 2 * BM * 4 + BN * 4 <= 160 * 1024 - 12288, "LDS budget with the largest k-table");
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
-    // group shape gm x (32 / gm): least operand rows per group among the shapes that fit the tile grid
+    // group size: 32 tiles, or fewer (a power of two) when that is needed to give each of the 8 XCDs a group
+    int gs = 32;
+    while (gs > 1 && (long)tiles_m * tiles_n * count < 8l * gs) gs >>= 1;
+    // group shape gm x gn: least operand rows per group among the shapes that fit the tile grid
     int gm = 1;
     long best = -1;
-    for (int cand = 1; cand <= 32; cand *= 2) {
-        const int gn = 32 / cand;
+    for (int cand = 1; cand <= gs; cand *= 2) {
+        const int gn = gs / cand;
         const long cost = (long)(cand < tiles_m ? cand : tiles_m) * BM + (long)(gn < tiles_n ? gn : tiles_n) * BN;
         const long waste = (long)((tiles_m + cand - 1) / cand) * ((tiles_n + gn - 1) / gn);  // groups launched
         const long score = cost * waste;
@@ -519,24 +537,25 @@ int launch_cfg(const GemmProblem &p, hipStream_t stream) {
             gm = cand;
         }
     }
-    const int groups = ((tiles_m + gm - 1) / gm) * ((tiles_n + 32 / gm - 1) / (32 / gm));
-    const int grid = ((groups + 7) / 8) * 8 * 32;
+    const int gn = gs / gm;
+    const int groups = ((tiles_m + gm - 1) / gm) * ((tiles_n + gn - 1) / gn) * count;
+    const int grid = ((groups + 7) / 8) * 8 * gs;
     const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
     // the per-row activation sums are only carried when the weight zero point is not 128
     if (p.dense) {
         if (p.zw != 0)
             hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true, true>), dim3(grid), dim3(256), 0,
-                               stream, p, tiles_m, tiles_n, gm);
+                               stream, batch, count, tiles_m, tiles_n, gm, gn);
         else
             hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true, false>), dim3(grid), dim3(256), 0,
-                               stream, p, tiles_m, tiles_n, gm);
+                               stream, batch, count, tiles_m, tiles_n, gm, gn);
     } else {
         if (p.zw != 0)
             hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false, true>), dim3(grid), dim3(256),
-                               ktab_bytes, stream, p, tiles_m, tiles_n, gm);
+                               ktab_bytes, stream, batch, count, tiles_m, tiles_n, gm, gn);
         else
             hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false, false>), dim3(grid), dim3(256),
-                               ktab_bytes, stream, p, tiles_m, tiles_n, gm);
+                               ktab_bytes, stream, batch, count, tiles_m, tiles_n, gm, gn);
     }
     EH_HIP(hipGetLastError());
     return EH_OK;
@@ -547,12 +566,13 @@ int launch_cfg(const GemmProblem &p, hipStream_t stream) {
 // Which kernel shape serves an (m, n, k) problem whose activations come in
 // 16-byte channel units.  The packed weight layout depends on the slab, so the
 // choice is made once, when the weights are packed.
-GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k) {
+// `siblings` equally shaped problems share one launch (convolution groups, deconvolution phases).
+GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k, int32_t siblings) {
     GemmConfig c;
-    const long t256 = (long)((m + 255) / 256) * ((n + 127) / 128);
-    const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
-    const long t128x64 = (long)((m + 127) / 128) * ((n + 63) / 64);
-    const long t256x256 = (long)((m + 255) / 256) * ((n + 255) / 256);
+    const long t256 = (long)((m + 255) / 256) * ((n + 127) / 128) * siblings;
+    const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128) * siblings;
+    const long t128x64 = (long)((m + 127) / 128) * ((n + 63) / 64) * siblings;
+    const long t256x256 = (long)((m + 255) / 256) * ((n + 255) / 256) * siblings;
     if (n > 128 && t256x256 >= 240) {
         c.id = GEMM_DMA_256x256;
         c.slab = 128;
@@ -573,14 +593,21 @@ GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k) {
     return c;
 }
 
-int launch_igemm_dma(const GemmProblem &p, hipStream_t stream) {
-    EH_REQUIRE(p.vec == 16 && p.k_pad % p.cfg.slab == 0, "igemm_dma: unsupported problem");
+int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream) {
+    const GemmProblem &p = ps[0];
+    EH_REQUIRE(count >= 1 && count <= GemmBatch::MAX, "igemm_dma: batch of %d", count);
+    for (int i = 0; i < count; ++i) {
+        EH_REQUIRE(ps[i].vec == 16 && ps[i].k_pad % ps[i].cfg.slab == 0, "igemm_dma: unsupported problem");
+        EH_REQUIRE(ps[i].cfg.id == p.cfg.id && ps[i].m == p.m && ps[i].n == p.n && ps[i].k_pad == p.k_pad &&
+                       ps[i].dense == p.dense && ps[i].zw == p.zw,
+                   "igemm_dma: a batch must hold equally shaped problems");
+    }
     switch (p.cfg.id) {
-        case GEMM_DMA_256x256: return launch_cfg<256, 256, 2, 2, 1, 128, 2>(p, stream);
-        case GEMM_DMA_256x128: return launch_cfg<256, 128, 2, 2, 1, 128, 3>(p, stream);
-        case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 2>(p, stream);
-        case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 3>(p, stream);
-        case GEMM_DMA_64x64_SPLITK: return launch_cfg<64, 64, 1, 1, 4, 256, 4>(p, stream);
+        case GEMM_DMA_256x256: return launch_cfg<256, 256, 2, 2, 1, 128, 2>(ps, count, stream);
+        case GEMM_DMA_256x128: return launch_cfg<256, 128, 2, 2, 1, 128, 3>(ps, count, stream);
+        case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 2>(ps, count, stream);
+        case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 3>(ps, count, stream);
+        case GEMM_DMA_64x64_SPLITK: return launch_cfg<64, 64, 1, 1, 4, 256, 4>(ps, count, stream);
         default: break;
     }
     set_error("igemm_dma: unknown configuration %d", p.cfg.id);

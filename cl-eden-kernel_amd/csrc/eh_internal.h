@@ -212,9 +212,16 @@ struct GemmProblem {
     RequantDev rq;
 };
 
+// Equally shaped problems of one operator that go out as one launch (kernel argument).
+struct GemmBatch {
+    static constexpr int MAX = 4;
+    GemmProblem p[MAX];
+};
 int launch_igemm(const GemmProblem &p, hipStream_t stream);
-int launch_igemm_dma(const GemmProblem &p, hipStream_t stream);  // vec == 16 and a k-table that fits LDS
-GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k);
+// `count` problems in order; consecutive equally shaped ones that the direct-to-LDS kernels serve share launches
+int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream);
+int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream);  // vec == 16 and a k-table that fits LDS
+GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k, int32_t siblings);
 inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
