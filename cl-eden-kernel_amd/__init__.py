@@ -61,6 +61,7 @@ EXPORTS = {
                                    C.POINTER(AddRequant)]),
     "eh_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(AddRequant), C.c_void_p]),
     "eh_avgpool_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PoolDesc), C.c_void_p]),
+    "eh_probe_mfma_i8": (C.c_int, [C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
     "eh_conv_out_dim": (C.c_int32, [C.c_int32] * 6),
     "eh_deconv_out_dim": (C.c_int32, [C.c_int32] * 5),
     "eh_init": (C.c_int, [C.c_int]),
@@ -167,6 +168,13 @@ def avgpool_u8(src, dst, n, c, h, w, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), la
 
 def _addr(x):
     return x.ptr if hasattr(x, "ptr") else x
+
+
+def probe_mfma_i8(iterations=100000, toggling_operands=True):
+    """Sustained int8 MFMA rate of the device in TOP/s (registers only)."""
+    tops = C.c_double(0)
+    check(load().eh_probe_mfma_i8(iterations, int(toggling_operands), C.byref(tops)))
+    return tops.value
 
 
 def requant_apply(q, acc, two_step=False):

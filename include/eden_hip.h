@@ -153,6 +153,14 @@ int eh_graph_end(void *stream, void **graph);
 int eh_graph_launch(void *graph, void *stream);
 int eh_graph_destroy(void *graph);
 
+/* ---- machine probe -----------------------------------------------------------
+ * Sustained rate (TOP/s, 1 op = 1 multiply or 1 add) of v_mfma_i32_32x32x32_i8 issued
+ * from registers on every SIMD of the device, with constant operands or with operands
+ * whose bits toggle like data (the clock the device sustains differs).  The measured
+ * ceiling the benchmark prints beside the published peak; no counterpart in the
+ * reference.  Synchronous; allocates and frees a small device buffer. */
+int eh_probe_mfma_i8(int32_t iterations, int32_t toggling_operands, double *tops);
+
 /* ---- layout conversion -----------------------------------------------------
  * nchw2nhwc_uint8 / nhwc2nchw_uint8 (gpu/common/CLKernels.hpp:429-491) as
  * driven by CLRuntime::NCHW2NHWC / NHWC2NCHW (gpu/common/CLRuntime.cpp:1477-1619). */
