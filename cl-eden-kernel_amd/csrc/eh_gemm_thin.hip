@@ -26,7 +26,8 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 namespace {
 
 template <int NBU, int KU, bool ROWSUM, bool FAST>
-__global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps) {
+__global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps,
+                                                          const int stage_out) {
     // KU: reduction steps whose loads are in flight together; NBU: channel blocks per wave
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, half = lane >> 5;
@@ -47,6 +48,11 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
     const RequantDev rq = p.rq;
     const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
     const v4i *bfrag = reinterpret_cast<const v4i *>(p.b) + lane;
+    // stage_out: the 32 pixels of a wave are 32 * N contiguous output bytes (plain channels-last rows, N a
+    // multiple of 8, one workgroup row per pixel block): the wave collects its rows in LDS and writes them
+    // as one linear run of 16-byte pieces, whole cache lines instead of a 32-byte piece per pixel and block
+    extern __shared__ __align__(16) uint8_t out_stage[];
+    uint8_t *wave_stage = out_stage + (size_t)wave * 32 * p.n;
 
     // blockIdx.y spreads the channel-block groups over workgroups when there are few pixels
     for (int nb0 = blockIdx.y * NBU; nb0 < n_blocks; nb0 += gridDim.y * NBU) {
@@ -147,6 +153,14 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                 quantize(std::integral_constant<int, 2>{});
             else
                 quantize(std::integral_constant<int, 1>{});
+            if (stage_out) {
+                if (n < p.n) {
+                    uint2 *dst2 = reinterpret_cast<uint2 *>(wave_stage + r * p.n + n);
+                    dst2[0] = make_uint2(packed[0], packed[1]);
+                    if (n + 8 < p.n) dst2[1] = make_uint2(packed[2], packed[3]);
+                }
+                continue;
+            }
             if (!row_ok || n >= p.n) continue;
             uint8_t *dst = p.out + out_off + n;
             if (aligned16 && n + 16 <= p.n) {
@@ -154,6 +168,20 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
             } else {
                 const int cnt = p.n - n < 16 ? p.n - n : 16;
                 for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+            }
+        }
+    }
+    if (stage_out) {
+        __syncthreads();
+        const int m_wave = (blockIdx.x * 4 + wave) * 32;
+        const int rows = p.m - m_wave < 32 ? p.m - m_wave : 32;
+        const int bytes = rows > 0 ? rows * p.n : 0;  // a multiple of 8
+        uint8_t *dst = p.out + (size_t)m_wave * p.n;   // 16-byte aligned: m_wave is a multiple of 32
+        for (int off = lane * 16; off < bytes; off += 64 * 16) {
+            if (off + 16 <= bytes) {
+                *reinterpret_cast<uint4 *>(dst + off) = *reinterpret_cast<const uint4 *>(wave_stage + off);
+            } else {
+                *reinterpret_cast<uint2 *>(dst + off) = *reinterpret_cast<const uint2 *>(wave_stage + off);
             }
         }
     }
@@ -167,16 +195,22 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     int split = 1;
     while (split < n_groups && (long)row_groups * split < 2048) ++split;
     const dim3 grid(row_groups, split);
+    // rows of one pixel block contiguous in the output (see the kernel): identity pixel mapping, no channel offset
+    const bool linear = split == 1 && p.ldc == p.n && (p.n & 7) == 0 && p.n <= 384 && p.out_sy == 1 && p.out_sx == 1 &&
+                        p.out_y0 == 0 && p.out_x0 == 0 && p.out_h == p.ho && p.out_w == p.wo &&
+                        (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
+    const int stage_out = linear ? 1 : 0;
+    const size_t lds = linear ? (size_t)4 * 32 * p.n : 0;
     if (p.zw != 0) {
         if (p.rq.fast)
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, true>), grid, dim3(256), 0, stream, p, n_blocks, ksteps);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
         else
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, false>), grid, dim3(256), 0, stream, p, n_blocks, ksteps);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
     } else {
         if (p.rq.fast)
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, true>), grid, dim3(256), 0, stream, p, n_blocks, ksteps);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
         else
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, false>), grid, dim3(256), 0, stream, p, n_blocks, ksteps);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
     }
     EH_HIP(hipGetLastError());
     return EH_OK;
