@@ -39,6 +39,7 @@ enum class BufferType {
 };
 
 enum class StorageType { BUFFER = 0, TEXTURE = 1, SIZE };
+enum class ComputeType { TFLite = 0, Caffe, SIZE };
 
 enum { N_NCHW = 0, C_NCHW = 1, H_NCHW = 2, W_NCHW = 3 };
 enum { N_NHWC = 0, H_NHWC = 1, W_NHWC = 2, C_NHWC = 3 };

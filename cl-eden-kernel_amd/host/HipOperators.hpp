@@ -7,7 +7,10 @@
 // Reference counterparts: CLConvolution (src/userdriver/gpu/operators/CLConvolution.hpp:31-66,
 // CLConvolution.cpp:34-550), CLDepthwiseConvolution (CLDepthwiseConvolution.hpp:18-38,
 // .cpp:88-425), CLFullyConnected (CLFullyConnected.hpp:21-35, .cpp:22-150),
-// CLDeconvolution (CLDeconvolution.hpp:20-40, .cpp:36-272).
+// CLDeconvolution (CLDeconvolution.hpp:20-40, .cpp:36-272); and the two operators a residual
+// network needs between them: CLAdd on its quantized path (CLAdd.hpp:21-66,
+// cl_optimized_impls/CLAddQuantized.cpp:67-166) and CLAveragepool (CLAveragepool.hpp:15-60,
+// CLAveragepool.cpp:175-230, parameters gpu/common/CLParameter.hpp:25-34).
 //
 // Behaviour kept from the reference: quantization parameters are read from the
 // tensors on every execute(); constant weights are packed once in initialize(),
@@ -85,6 +88,28 @@ struct DeconvolutionParameters : public Parameters {
     bool openAibWino = false;
     std::shared_ptr<ActivationInfo> activation_info = std::make_shared<ActivationInfo>();
     std::vector<float> scales;
+};
+
+// AddParameters (gpu/operators/CLAdd.hpp:21-28) and Pool2DParameters (gpu/common/CLParameter.hpp:25-34):
+// the activation is held by value there
+struct AddParameters : public Parameters {
+    ActivationInfo activation_info = ActivationInfo();
+    bool pot_scale_int16 = false;
+    std::vector<float> coeff = {};
+    bool androidNN = false;
+    bool isNCHW = false;
+    StorageType storage_type = StorageType::BUFFER;
+};
+
+struct Pool2DParameters : public Parameters {
+    Pad4 padding = {0, 0, 0, 0};
+    Dim2 stride = {1, 1};
+    Dim2 filter = {1, 1};
+    ActivationInfo activation_info = ActivationInfo();
+    bool androidNN = false;
+    bool isNCHW = true;
+    StorageType storage_type = StorageType::BUFFER;
+    ComputeType compute_type = ComputeType::TFLite;
 };
 
 namespace detail {
@@ -481,6 +506,118 @@ private:
     bool weights_as_input_ = false;
     eh_conv_desc desc_{};
     eh_deconv_plan *plan_ = nullptr;
+};
+
+// Element-wise sum of two equally shaped uint8 tensors, requantized to the output tensor's
+// scale (quantization parameters are read from the three tensors at every execute()).
+// Broadcasting, coefficients and the int16 power-of-two variant are not offered here.
+class HipAdd {
+public:
+    HipAdd(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision) : runtime_(runtime), precision_(precision) {}
+
+    Status initialize(const std::vector<std::shared_ptr<ITensor>> &input_tensors,
+                      const std::vector<std::shared_ptr<ITensor>> &output_tensors, const std::shared_ptr<Parameters> parameters) {
+        CHECK_EXPR_RETURN_FAILURE(input_tensors.size() == 2 && output_tensors.size() >= 1, "HipAdd: needs two inputs and one output");
+        a_ = std::static_pointer_cast<HipTensor>(input_tensors.at(0));
+        b_ = std::static_pointer_cast<HipTensor>(input_tensors.at(1));
+        output_ = std::static_pointer_cast<HipTensor>(output_tensors.at(0));
+        parameters_ = std::dynamic_pointer_cast<AddParameters>(parameters);
+        CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipAdd: parameters are not AddParameters");
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipAdd: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipAdd: no texture storage");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->coeff.empty() && !parameters_->pot_scale_int16, "HipAdd: coefficients / int16 scaling are not offered");
+        CHECK_EXPR_RETURN_FAILURE(a_->getDataType() == DataType::UINT8 && b_->getDataType() == DataType::UINT8 &&
+                                      output_->getDataType() == DataType::UINT8, "HipAdd: expects uint8 tensors");
+        CHECK_EXPR_RETURN_FAILURE(a_->getTotalSizeFromDims() == b_->getTotalSizeFromDims() &&
+                                      a_->getTotalSizeFromDims() == output_->getTotalSizeFromDims(), "HipAdd: shapes differ (no broadcast)");
+        ready_ = true;
+        return Status::SUCCESS;
+    }
+
+    Status execute() {
+        CHECK_EXPR_RETURN_FAILURE(ready_, "HipAdd::execute before initialize");
+        eh_add_requant q;
+        eh_make_add_requant(a_->getScale(), a_->getZeroPoint(), b_->getScale(), b_->getZeroPoint(), output_->getScale(),
+                            output_->getZeroPoint(), detail::toEhActivation(parameters_->activation_info),
+                            parameters_->activation_info.isEnabled() ? 1 : 0, &q);
+        const int rc = eh_add_u8(a_->getDataPtr(), b_->getDataPtr(), output_->getDataPtr(), (int64_t)output_->getTotalSizeFromDims(), &q,
+                                 runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipAdd::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status release() { return Status::SUCCESS; }
+
+private:
+    std::shared_ptr<HipRuntime> runtime_;
+    PrecisionType precision_;
+    std::shared_ptr<HipTensor> a_, b_, output_;
+    std::shared_ptr<AddParameters> parameters_;
+    bool ready_ = false;
+};
+
+// Average pool on a uint8 tensor: windows clipped to the image, (sum + count / 2) / count, clamp to
+// the activation range of the output tensor.  Input and output share one scale and zero point.
+class HipAveragepool {
+public:
+    HipAveragepool(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision)
+        : runtime_(runtime), precision_(precision) {}
+
+    Status initialize(const std::vector<std::shared_ptr<ITensor>> &input_tensors,
+                      const std::vector<std::shared_ptr<ITensor>> &output_tensors, const std::shared_ptr<Parameters> parameters) {
+        CHECK_EXPR_RETURN_FAILURE(input_tensors.size() >= 1 && output_tensors.size() >= 1, "HipAveragepool: needs an input and an output");
+        input_ = std::static_pointer_cast<HipTensor>(input_tensors.at(0));
+        output_ = std::static_pointer_cast<HipTensor>(output_tensors.at(0));
+        parameters_ = std::dynamic_pointer_cast<Pool2DParameters>(parameters);
+        CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipAveragepool: parameters are not Pool2DParameters");
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipAveragepool: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipAveragepool: no texture storage");
+        CHECK_EXPR_RETURN_FAILURE(parameters_->compute_type == ComputeType::TFLite, "HipAveragepool: only the TFLite window rule");
+        CHECK_EXPR_RETURN_FAILURE(input_->getDataType() == DataType::UINT8 && output_->getDataType() == DataType::UINT8,
+                                  "HipAveragepool: expects uint8 tensors");
+        const Dim4 id = input_->getDim();
+        const bool nchw = parameters_->isNCHW;
+        d_.n = (int32_t)id.n;
+        d_.c = (int32_t)(nchw ? id.c : id.w);  // channels-last tensors hold (n, h, w, c) positionally
+        d_.h = (int32_t)(nchw ? id.h : id.c);
+        d_.w = (int32_t)(nchw ? id.w : id.h);
+        d_.kh = (int32_t)parameters_->filter.h;
+        d_.kw = (int32_t)parameters_->filter.w;
+        d_.stride_h = (int32_t)parameters_->stride.h;
+        d_.stride_w = (int32_t)parameters_->stride.w;
+        d_.pad_t = (int32_t)parameters_->padding.t;
+        d_.pad_b = (int32_t)parameters_->padding.b;
+        d_.pad_l = (int32_t)parameters_->padding.l;
+        d_.pad_r = (int32_t)parameters_->padding.r;
+        d_.layout = nchw ? EH_NCHW : EH_NHWC;
+        CHECK_EXPR_RETURN_FAILURE(d_.kh > 0 && d_.kw > 0 && d_.stride_h > 0 && d_.stride_w > 0, "HipAveragepool: bad window or stride");
+        const int32_t ho = (d_.h + d_.pad_t + d_.pad_b - d_.kh) / d_.stride_h + 1, wo = (d_.w + d_.pad_l + d_.pad_r - d_.kw) / d_.stride_w + 1;
+        CHECK_EXPR_RETURN_FAILURE((uint64_t)output_->getTotalSizeFromDims() == (uint64_t)d_.n * d_.c * ho * wo,
+                                  "HipAveragepool: output has %u elements, expected %d x %d x %d x %d", output_->getTotalSizeFromDims(), d_.n, d_.c, ho, wo);
+        ready_ = true;
+        return Status::SUCCESS;
+    }
+
+    Status execute() {
+        CHECK_EXPR_RETURN_FAILURE(ready_, "HipAveragepool::execute before initialize");
+        eh_pool_desc d = d_;
+        // the range comes from the activation type alone, as in CLAveragepool::averagepool_quant (CLAveragepool.cpp:183-198)
+        eh_act_range_u8(detail::toEhActivation(parameters_->activation_info), output_->getScale(), output_->getZeroPoint(), &d.act_min,
+                        &d.act_max);
+        const int rc = eh_avgpool_u8(input_->getDataPtr(), output_->getDataPtr(), &d, runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipAveragepool::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    Status release() { return Status::SUCCESS; }
+
+private:
+    std::shared_ptr<HipRuntime> runtime_;
+    PrecisionType precision_;
+    std::shared_ptr<HipTensor> input_, output_;
+    std::shared_ptr<Pool2DParameters> parameters_;
+    eh_pool_desc d_{};
+    bool ready_ = false;
 };
 
 }  // namespace hip

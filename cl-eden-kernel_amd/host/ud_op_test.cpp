@@ -512,6 +512,88 @@ static int gpu_tests() {
         return ok;
     });
 
+    run_test("Add.Residual_sum_of_two_tensors_with_different_scales", [&] {
+        bool ok = true;
+        const Dim4 dim = {2, 28, 28, 32};  // channels-last, positional
+        const size_t count = (size_t)2 * 28 * 28 * 32;
+        auto a = rand_u8(count, 301), b = rand_u8(count, 302);
+        std::shared_ptr<ITensor> ta = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, dim, DataOrder::NHWC, 0.0235f, 3);
+        std::shared_ptr<ITensor> tb = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, dim, DataOrder::NHWC, 0.011f, 250);
+        std::shared_ptr<ITensor> to = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, dim, DataOrder::NHWC, 0.03f, 77);
+        auto params = std::make_shared<AddParameters>();
+        HipAdd add(rt, U8);
+        EXPECT(add.initialize({ta, tb}, {to}, params) == Status::SUCCESS);
+        rt->assignBufferPool();
+        EXPECT(ta->writeData(a.data()) == Status::SUCCESS);
+        EXPECT(tb->writeData(b.data()) == Status::SUCCESS);
+        EXPECT(add.execute() == Status::SUCCESS);
+        std::vector<uint8_t> got(count), want(count);
+        EXPECT(to->readData(got.data()) == Status::SUCCESS);
+        eo_add_quant q;
+        eo_make_add_quant(0.0235f, 3, 0.011f, 250, 0.03f, 77, 0, 0, &q);
+        eo_add_u8(a.data(), b.data(), want.data(), (int64_t)count, &q);
+        EXPECT(same(got, want));
+        EXPECT(varied(want));
+        // a fused ReLU6 narrows the clamp
+        params->activation_info = ActivationInfo(ActivationInfo::ActivationType::RELU6, true);
+        EXPECT(add.execute() == Status::SUCCESS);
+        EXPECT(to->readData(got.data()) == Status::SUCCESS);
+        eo_make_add_quant(0.0235f, 3, 0.011f, 250, 0.03f, 77, (int)ActivationInfo::ActivationType::RELU6, 1, &q);
+        eo_add_u8(a.data(), b.data(), want.data(), (int64_t)count, &q);
+        EXPECT(same(got, want));
+        return ok;
+    });
+
+    run_test("Averagepool.Global_7x7_channels_last_and_padded_3x3_planar", [&] {
+        bool ok = true;
+        {
+            const int n = 3, c = 1280, h = 7, w = 7;
+            auto x = rand_u8((size_t)n * c * h * w, 311);  // planar for the oracle
+            std::vector<uint8_t> want((size_t)n * c);
+            eo_avgpool_u8(x.data(), want.data(), n, c, h, w, 7, 7, 1, 1, 0, 0, 0, 0, 0, 255);
+            std::shared_ptr<ITensor> ti = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)n, (uint32_t)h, (uint32_t)w, (uint32_t)c}, DataOrder::NHWC, 0.0235f, 0);
+            std::shared_ptr<ITensor> to = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)n, 1, 1, (uint32_t)c}, DataOrder::NHWC, 0.0235f, 0);
+            auto params = std::make_shared<Pool2DParameters>();
+            params->filter = {7, 7};
+            params->isNCHW = false;
+            HipAveragepool pool(rt, U8);
+            EXPECT(pool.initialize({ti}, {to}, params) == Status::SUCCESS);
+            rt->assignBufferPool();
+            auto x_nhwc = nchw_to_nhwc(x, n, c, h, w);
+            EXPECT(ti->writeData(x_nhwc.data()) == Status::SUCCESS);
+            EXPECT(pool.execute() == Status::SUCCESS);
+            std::vector<uint8_t> got(want.size());
+            EXPECT(to->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(got, want));
+            EXPECT(varied(want));
+        }
+        {
+            const int n = 2, c = 5, h = 9, w = 11;
+            auto x = rand_u8((size_t)n * c * h * w, 312);
+            const int ho = (h + 2 - 3) / 2 + 1, wo = (w + 2 - 3) / 2 + 1;
+            std::vector<uint8_t> want((size_t)n * c * ho * wo);
+            int32_t lo, hi;
+            eo_act_range_u8((int)ActivationInfo::ActivationType::RELU1, 0.01f, 100, &lo, &hi);
+            eo_avgpool_u8(x.data(), want.data(), n, c, h, w, 3, 3, 2, 2, 1, 1, 1, 1, lo, hi);
+            std::shared_ptr<ITensor> ti = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)n, (uint32_t)c, (uint32_t)h, (uint32_t)w}, DataOrder::NCHW, 0.01f, 100);
+            std::shared_ptr<ITensor> to = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{(uint32_t)n, (uint32_t)c, (uint32_t)ho, (uint32_t)wo}, DataOrder::NCHW, 0.01f, 100);
+            auto params = std::make_shared<Pool2DParameters>();
+            params->filter = {3, 3};
+            params->stride = {2, 2};
+            params->padding = {1, 1, 1, 1};
+            params->activation_info = ActivationInfo(ActivationInfo::ActivationType::RELU1, true);
+            HipAveragepool pool(rt, U8);
+            EXPECT(pool.initialize({ti}, {to}, params) == Status::SUCCESS);
+            rt->assignBufferPool();
+            EXPECT(ti->writeData(x.data()) == Status::SUCCESS);
+            EXPECT(pool.execute() == Status::SUCCESS);
+            std::vector<uint8_t> got(want.size());
+            EXPECT(to->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(got, want));
+        }
+        return ok;
+    });
+
     std::printf("%d of %d GPU operator tests failed\n", g_failed, g_run);
     return g_failed ? 1 : 0;
 }
