@@ -83,6 +83,10 @@ BIG_FC_CASES = [
     (65536 - 5, 256, 128 - 16, 200, 128),   # 256 x 128 tiles
     (16384 - 100, 384, 256, 128, 3),        # 128 x 128 tiles
     (32768 - 3, 896, 64 - 8, 17, 250),      # 128 x 64 tiles
+    # more tiles than the device holds workgroups at once, with reductions shorter and longer than the stage count
+    (20000 - 3, 128, 1024, 5, 140),         # 256 x 256, one slab per tile
+    (80000 - 11, 384, 64, 128, 100),        # 128 x 64, three slabs
+    (140000 - 1, 256, 128 - 8, 30, 128),    # 256 x 128, two slabs
     # the one-tap kernel with a long reduction loop and every channel-group width
     (3000, 96, 576, 77, 120),
     (3136 - 7, 256, 320, 0, 131),
@@ -120,6 +124,21 @@ def test_conv_batched_large_tiles():
     want = O.conv2d(x, w, b, s, q)
     got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
     assert np.array_equal(got, want), diff_report(got, want)
+
+
+@pytest.mark.parametrize("cin,cout", [(16, 64), (32, 64), (64, 128)])
+def test_conv_more_tiles_than_workgroups(cin, cout):
+    """3x3 convolution at batch 24 (75264 output pixels): more tiles than the device holds workgroups at once, with
+    the k-table path and reductions of 2, 3 and 5 slabs against 2 or 3 stages."""
+    print("conv many tiles", cin, cout, flush=True)
+    s = O.conv_shape(24, cin, 56, 56, cout, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 23 + cin)
+    _, acc = O.conv2d(x[:1], w, b, O.conv_shape(1, cin, 56, 56, cout, 3, 3, pad=(1, 1, 1, 1)), O.raw_quant(zp_in=131, zp_w=120), want_acc=True)
+    q = centred_quant(acc, 131, 120)
+    want = O.conv2d(x, w, b, s, q)
+    got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
+    assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 10
 
 
 def test_fc_config2_full_size():
