@@ -16,6 +16,7 @@ EH_OK = 0
 ACT_NONE, ACT_RELU, ACT_RELU1, ACT_RELU6 = 0, 1, 2, 3
 NCHW, NHWC = 0, 1
 W_OIHW, W_OHWI, W_IOHW = 0, 1, 2
+W_SIGNED = 0x100  # or-ed into a convolution's weight layout: int8 weight bytes
 
 
 class EdenHipError(RuntimeError):
@@ -62,6 +63,9 @@ EXPORTS = {
     "eh_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(AddRequant), C.c_void_p]),
     "eh_avgpool_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PoolDesc), C.c_void_p]),
     "eh_probe_mfma_i8": (C.c_int, [C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
+    "eh_make_requant_perchannel": (None, [C.c_float, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32, C.c_int, C.c_int,
+                                          C.POINTER(Requant), C.c_void_p, C.c_void_p]),
+    "eh_conv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "eh_conv_out_dim": (C.c_int32, [C.c_int32] * 6),
     "eh_deconv_out_dim": (C.c_int32, [C.c_int32] * 5),
     "eh_init": (C.c_int, [C.c_int]),
@@ -265,6 +269,24 @@ class ConvPlan(_Plan):
         self.desc = desc
         check(load().eh_conv2d_u8_plan(C.byref(self.handle), C.byref(desc), d_w.ptr, d_b.ptr if d_b else None,
                                        C.byref(q), stream))
+
+    def set_perchannel(self, multipliers, shifts, stream=None):
+        """One multiplier / shift per output channel from now on (None, None: back to the Requant's pair)."""
+        if multipliers is None:
+            check(load().eh_conv2d_u8_set_perchannel(self.handle, None, None, 0, stream))
+            return
+        m, s = np.ascontiguousarray(multipliers, np.int32), np.ascontiguousarray(shifts, np.int32)
+        check(load().eh_conv2d_u8_set_perchannel(self.handle, m.ctypes.data, s.ctypes.data, m.size, stream))
+
+
+def make_requant_perchannel(s_in, zp_in, filter_scales, s_out, zp_out, act=ACT_NONE, act_enabled=False):
+    """(Requant, multipliers, shifts) as the per-channel quantized convolution derives them at execute()."""
+    scales = np.ascontiguousarray(filter_scales, np.float32)
+    mult, shift = np.zeros(scales.size, np.int32), np.zeros(scales.size, np.int32)
+    q = Requant()
+    load().eh_make_requant_perchannel(s_in, zp_in, scales.ctypes.data, scales.size, s_out, zp_out, act, int(act_enabled),
+                                      C.byref(q), mult.ctypes.data, shift.ctypes.data)
+    return q, mult, shift
 
 
 class DwConvPlan(_Plan):

@@ -28,8 +28,14 @@ int hip_fail(hipError_t e, const char *what) {
     return EH_DEVICE_FAILURE;
 }
 
-int check_requant(const eh_requant *q) {
+int check_requant(const eh_requant *q, bool signed_weights) {
     EH_REQUIRE(q != nullptr, "requant parameters are null");
+    if (signed_weights) {
+        EH_REQUIRE(q->zp_w >= -128 && q->zp_w <= 127, "int8 weight zero point %d outside [-128, 127]", q->zp_w);
+        eh_requant u = *q;
+        u.zp_w += 128;
+        return check_requant(&u, false);
+    }
     EH_REQUIRE(q->multiplier >= 0, "requant multiplier %d is negative", q->multiplier);
     EH_REQUIRE(q->shift >= -31 && q->shift <= 30, "requant shift %d outside [-31, 30]", q->shift);
     EH_REQUIRE(q->zp_in >= 0 && q->zp_in <= 255 && q->zp_w >= 0 && q->zp_w <= 255,
@@ -141,9 +147,10 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     return EH_OK;
 }
 
-int pack_part(GemmPart &g, const uint8_t *weight, hipStream_t stream) {
+int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t stream) {
     PackProblem pp;
     pp.w = weight + g.w_base;
+    pp.w_signed = w_signed ? 1 : 0;
     pp.bias = nullptr;
     pp.b = g.b;
     pp.colsum = g.colsum;
@@ -174,6 +181,34 @@ struct GemmOp {
     int32_t layout = EH_NHWC;
     int32_t in_n = 0, in_c = 0, in_hw = 0, out_hw = 0;
     size_t in_bytes = 0;
+    // int8 weights (value = byte as signed; zp_w is then an int8 zero point) and one multiplier / shift per
+    // output channel instead of the requant's single pair
+    bool w_signed = false;
+    int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;
+
+    int zp_w_u8(const eh_requant &r) const { return r.zp_w + (w_signed ? 128 : 0); }  // zero point of the equivalent uint8 weights
+
+    int set_perchannel(const int32_t *multipliers, const int32_t *shifts, int32_t count, hipStream_t stream) {
+        if (multipliers == nullptr && shifts == nullptr) {
+            EH_HIP(hipStreamSynchronize(stream));
+            dev_free(pc_multiplier);
+            dev_free(pc_shift);
+            return EH_OK;
+        }
+        EH_REQUIRE(multipliers != nullptr && shifts != nullptr && count == cout, "per-channel arrays must hold %d entries (got %d)", cout, count);
+        for (int32_t i = 0; i < count; ++i)
+            EH_REQUIRE(multipliers[i] >= 0 && shifts[i] >= -31 && shifts[i] <= 30, "per-channel multiplier/shift %d out of range", i);
+        int rc;
+        // padded so that the kernels may read whole channel blocks
+        if (!pc_multiplier && (rc = dev_alloc(&pc_multiplier, (size_t)cout + 512))) return rc;
+        if (!pc_shift && (rc = dev_alloc(&pc_shift, (size_t)cout + 512))) return rc;
+        EH_HIP(hipMemsetAsync(pc_multiplier, 0, ((size_t)cout + 512) * sizeof(int32_t), stream));
+        EH_HIP(hipMemsetAsync(pc_shift, 0, ((size_t)cout + 512) * sizeof(int32_t), stream));
+        EH_HIP(hipMemcpyAsync(pc_multiplier, multipliers, (size_t)cout * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+        EH_HIP(hipMemcpyAsync(pc_shift, shifts, (size_t)cout * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+        EH_HIP(hipStreamSynchronize(stream));  // the host arrays are the caller's
+        return EH_OK;
+    }
 
     void release() {
         for (auto &g : parts) g.release();
@@ -182,6 +217,8 @@ struct GemmOp {
         dev_free(stage_in);
         dev_free(stage_out);
         dev_free(fillbuf);
+        dev_free(pc_multiplier);
+        dev_free(pc_shift);
     }
 
     int set_weights(const void *weight, const void *bias, hipStream_t stream) {
@@ -191,7 +228,7 @@ struct GemmOp {
             if (rc) return rc;
         }
         for (auto &g : parts) {
-            int rc = pack_part(g, static_cast<const uint8_t *>(weight), stream);
+            int rc = pack_part(g, static_cast<const uint8_t *>(weight), w_signed, stream);
             if (rc) return rc;
         }
         if (bias)
@@ -203,12 +240,12 @@ struct GemmOp {
     }
 
     int refold(const eh_requant &nq, hipStream_t stream) {
-        if (folded_valid && nq.zp_in == q.zp_in && nq.zp_w == q.zp_w) {
+        if (folded_valid && nq.zp_in == q.zp_in && nq.zp_w == q.zp_w) {  // (w_signed is fixed per plan)
             q = nq;
             return EH_OK;
         }
         for (auto &g : parts) {
-            int rc = launch_fold_bias(bias_copy + g.bias_base, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, nq.zp_w,
+            int rc = launch_fold_bias(bias_copy + g.bias_base, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, zp_w_u8(nq),
                                       fillbuf, stream);
             if (rc) return rc;
         }
@@ -219,7 +256,7 @@ struct GemmOp {
 
     int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream) {
         EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
-        int rc = check_requant(nq);
+        int rc = check_requant(nq, w_signed);
         if (rc) return rc;
         if ((rc = refold(*nq, stream))) return rc;
         const uint8_t *in = static_cast<const uint8_t *>(input);
@@ -240,9 +277,14 @@ struct GemmOp {
             p.bias = g.folded;
             p.fillbuf = fillbuf;
             p.out = out + g.bias_base;
-            p.zw = q.zp_w - 128;
+            p.zw = zp_w_u8(q) - 128;
             p.fill = (uint32_t)q.zp_in * 0x01010101u;
             p.rq = make_requant_dev(q);
+            if (pc_multiplier) {
+                p.rq.pc_multiplier = pc_multiplier + g.bias_base;
+                p.rq.pc_shift = pc_shift + g.bias_base;
+                p.rq.fast = 0;  // the kernels' per-channel code sits on their general path
+            }
             problems.push_back(p);
         }
         if ((rc = launch_igemm_batch(problems.data(), (int)problems.size(), stream))) return rc;
@@ -373,6 +415,25 @@ void eh_make_requant(float input_scale, int32_t input_zp, float filter_scale, in
         out->act_min = 0;
         out->act_max = 255;
     }
+}
+
+void eh_make_requant_perchannel(float input_scale, int32_t input_zp, const float *filter_scales, int32_t channels,
+                                float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out,
+                                int32_t *multipliers, int32_t *shifts) {
+    out->zp_in = input_zp;
+    out->zp_w = 0;
+    out->zp_out = output_zp;
+    out->multiplier = 0;
+    out->shift = 0;
+    for (int32_t i = 0; i < channels; ++i) {
+        // the bias scale handed to the check is input_scale * scales[i] by construction, so it always passes
+        double m = 0.0;
+        (void)eh_conv_multiplier(input_scale, filter_scales[i], input_scale * filter_scales[i], output_scale, &m);
+        eh_quantize_multiplier(m, &multipliers[i], &shifts[i]);
+    }
+    out->act_min = 0;
+    out->act_max = 255;
+    if (activation_enabled) eh_act_range_u8(activation, output_scale, output_zp, &out->act_min, &out->act_max);
 }
 
 int32_t eh_conv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t dilation, int32_t stride) {
@@ -621,7 +682,11 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
     *plan = nullptr;
     int rc = check_desc_common(desc);
     if (rc) return rc;
-    if ((rc = check_requant(q))) return rc;
+    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0;
+    eh_conv_desc plain = *desc;
+    plain.weight_layout &= ~EH_W_SIGNED;
+    desc = &plain;
+    if ((rc = check_requant(q, w_signed))) return rc;
     EH_REQUIRE(desc->dil_h > 0 && desc->dil_w > 0, "bad dilation");
     EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
                "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
@@ -632,6 +697,7 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
     eh_conv_plan *pl = new (std::nothrow) eh_conv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
+    pl->op.w_signed = w_signed;
     if (desc->n > 0) {
         rc = conv_plan_build(pl, desc, as_stream(stream));
         if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
@@ -646,9 +712,16 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
     return EH_OK;
 }
 
+int eh_conv2d_u8_set_perchannel(eh_conv_plan *plan, const int32_t *multipliers, const int32_t *shifts, int32_t count,
+                                void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    if (plan->d.n == 0) return EH_OK;
+    return plan->op.set_perchannel(multipliers, shifts, count, as_stream(stream));
+}
+
 int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q);
+    int rc = check_requant(q, plan->op.w_signed);
     if (rc) return rc;
     if (plan->d.n == 0) return EH_OK;
     if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
@@ -657,7 +730,7 @@ int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias
 
 int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    if (plan->d.n == 0) return check_requant(q);  // zero-size early-out, as CLConvolution::execute does
+    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed);  // zero-size early-out, as CLConvolution::execute does
     return plan->op.run(input, output, q, as_stream(stream));
 }
 

@@ -95,7 +95,8 @@ __global__ __launch_bounds__(256) void conv_c3k3_kernel(const GemmProblem p, con
             int acc = p.bias[n] + ncorr;
 #pragma unroll
             for (int i = 0; i < 7; ++i) acc = __builtin_amdgcn_sdot4((int)A[i], wrow[i], acc, false);
-            o[t] = requant_u8_as<mode>(acc, rq);
+            o[t] = mode == 0 && rq.pc_multiplier ? requant_u8_channel(acc, rq.pc_multiplier[n], rq.pc_shift[n], rq)
+                                                 : requant_u8_as<mode>(acc, rq);
         }
         packed[g] = o[0] | (o[1] << 8) | (o[2] << 16) | (o[3] << 24);
     }

@@ -234,13 +234,15 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_u8_kernel(const GemmProbl
     for (int j = 0; j < FN; ++j) {
         const int nl = wn * WTN + j * 32 + (lane & 31);
         const int32_t bias = p.bias[n0 + nl];
+        const bool per_channel = rq.pc_multiplier != nullptr;
+        const int32_t ch_mult = per_channel ? rq.pc_multiplier[n0 + nl] : 0, ch_shift = per_channel ? rq.pc_shift[n0 + nl] : 0;
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 const int32_t v = acc[i][j][r] + bias - p.zw * rowsum_s[ml];
-                cs[ml * OUT_ROW + nl] = (uint8_t)requant_u8(v, rq);
+                cs[ml * OUT_ROW + nl] = (uint8_t)(per_channel ? requant_u8_channel(v, ch_mult, ch_shift, rq) : requant_u8(v, rq));
             }
         }
     }

@@ -416,10 +416,22 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
                     uint32_t packed[4];
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
-                        const uint32_t o0 = requant_u8_as<fast>(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], rq);
-                        const uint32_t o1 = requant_u8_as<fast>(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], rq);
-                        const uint32_t o2 = requant_u8_as<fast>(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], rq);
-                        const uint32_t o3 = requant_u8_as<fast>(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], rq);
+                        uint32_t o0, o1, o2, o3;
+                        if (checked && rq.pc_multiplier) {  // per-channel parameters (always the checked path)
+                            const int32_t *pm = rq.pc_multiplier + n + g * 4;
+                            const int4 cm = make_int4(pm[0], pm[1], pm[2], pm[3]);
+                            const int32_t *ps = rq.pc_shift + n + g * 4;
+                            const int4 cs = make_int4(ps[0], ps[1], ps[2], ps[3]);
+                            o0 = requant_u8_channel(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], cm.x, cs.x, rq);
+                            o1 = requant_u8_channel(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], cm.y, cs.y, rq);
+                            o2 = requant_u8_channel(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], cm.z, cs.z, rq);
+                            o3 = requant_u8_channel(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], cm.w, cs.w, rq);
+                        } else {
+                            o0 = requant_u8_as<fast>(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], rq);
+                            o1 = requant_u8_as<fast>(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], rq);
+                            o2 = requant_u8_as<fast>(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], rq);
+                            o3 = requant_u8_as<fast>(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], rq);
+                        }
                         packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
                     }
                     uint8_t *dst = p.out + row_off[i] + n;
@@ -492,8 +504,20 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
                 s4.w += t.w;
             }
             const int4 bb = *reinterpret_cast<const int4 *>(bias_s + nl + g * 4);
-            const uint32_t o0 = requant_u8_as<fast>(s4.x + bb.x - corr, rq), o1 = requant_u8_as<fast>(s4.y + bb.y - corr, rq);
-            const uint32_t o2 = requant_u8_as<fast>(s4.z + bb.z - corr, rq), o3 = requant_u8_as<fast>(s4.w + bb.w - corr, rq);
+            uint32_t o0, o1, o2, o3;
+            if (fast == 0 && rq.pc_multiplier) {
+                const int32_t *pm = rq.pc_multiplier + n + g * 4;
+                            const int4 cm = make_int4(pm[0], pm[1], pm[2], pm[3]);
+                const int32_t *ps = rq.pc_shift + n + g * 4;
+                            const int4 cs = make_int4(ps[0], ps[1], ps[2], ps[3]);
+                o0 = requant_u8_channel(s4.x + bb.x - corr, cm.x, cs.x, rq);
+                o1 = requant_u8_channel(s4.y + bb.y - corr, cm.y, cs.y, rq);
+                o2 = requant_u8_channel(s4.z + bb.z - corr, cm.z, cs.z, rq);
+                o3 = requant_u8_channel(s4.w + bb.w - corr, cm.w, cs.w, rq);
+            } else {
+                o0 = requant_u8_as<fast>(s4.x + bb.x - corr, rq), o1 = requant_u8_as<fast>(s4.y + bb.y - corr, rq);
+                o2 = requant_u8_as<fast>(s4.z + bb.z - corr, rq), o3 = requant_u8_as<fast>(s4.w + bb.w - corr, rq);
+            }
             packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
         }
         };

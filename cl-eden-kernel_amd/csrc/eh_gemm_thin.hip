@@ -140,10 +140,22 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                 constexpr int mode = decltype(mode_c)::value;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const uint32_t o0 = requant_u8_as<mode>(acc[ai][g * 4 + 0] + bb[u][g].x + ncorr, rq);
-                    const uint32_t o1 = requant_u8_as<mode>(acc[ai][g * 4 + 1] + bb[u][g].y + ncorr, rq);
-                    const uint32_t o2 = requant_u8_as<mode>(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, rq);
-                    const uint32_t o3 = requant_u8_as<mode>(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, rq);
+                    uint32_t o0, o1, o2, o3;
+                    if (mode == 0 && rq.pc_multiplier) {  // per-channel parameters (the padded arrays cover whole blocks)
+                        const int32_t *pm = rq.pc_multiplier + n + g * 4;
+                            const int4 cm = make_int4(pm[0], pm[1], pm[2], pm[3]);
+                        const int32_t *ps = rq.pc_shift + n + g * 4;
+                            const int4 cs = make_int4(ps[0], ps[1], ps[2], ps[3]);
+                        o0 = requant_u8_channel(acc[ai][g * 4 + 0] + bb[u][g].x + ncorr, cm.x, cs.x, rq);
+                        o1 = requant_u8_channel(acc[ai][g * 4 + 1] + bb[u][g].y + ncorr, cm.y, cs.y, rq);
+                        o2 = requant_u8_channel(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, cm.z, cs.z, rq);
+                        o3 = requant_u8_channel(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, cm.w, cs.w, rq);
+                    } else {
+                        o0 = requant_u8_as<mode>(acc[ai][g * 4 + 0] + bb[u][g].x + ncorr, rq);
+                        o1 = requant_u8_as<mode>(acc[ai][g * 4 + 1] + bb[u][g].y + ncorr, rq);
+                        o2 = requant_u8_as<mode>(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, rq);
+                        o3 = requant_u8_as<mode>(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, rq);
+                    }
                     packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
                 }
             };

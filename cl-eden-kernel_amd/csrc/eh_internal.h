@@ -45,6 +45,10 @@ struct RequantDev {
     int32_t fast_shift;        // right_shift - 1
     uint32_t pos_lo, pos_hi;   // 64-bit rounding term for accumulators >= 0
     uint32_t neg_lo, neg_hi;   // the same for accumulators < 0
+    // per-output-channel quantization (int8 weights with one scale per channel): device arrays indexed by the
+    // problem's own channel number, or null; when set they replace multiplier and shift above
+    const int32_t *pc_multiplier;
+    const int32_t *pc_shift;
 };
 
 __host__ __device__ __forceinline__ int32_t requant_core(int32_t acc, const RequantDev &r) {
@@ -63,6 +67,23 @@ __host__ __device__ __forceinline__ int32_t requant_core(int32_t acc, const Requ
 
 __host__ __device__ __forceinline__ uint32_t requant_u8(int32_t acc, const RequantDev &r) {
     int32_t v = requant_core(acc, r) + r.zp_out;
+    v = v < r.act_min ? r.act_min : v;
+    v = v > r.act_max ? r.act_max : v;
+    return (uint32_t)v;
+}
+
+// One multiplier and shift per output channel (conv_per_channel_quantized,
+// gpu/operators/cl_kernels/ConvolutionKernels.cpp:1317-1375): the two-step order with the
+// channel's own parameters; shift > 0 is a left shift of the accumulator, as above.
+__host__ __device__ __forceinline__ uint32_t requant_u8_channel(int32_t acc, int32_t multiplier, int32_t shift, const RequantDev &r) {
+    const int32_t ls = shift > 0 ? shift : 0, rs = shift > 0 ? 0 : -shift;
+    const int32_t x = (int32_t)((uint32_t)acc << ls);
+    const int64_t ab = (int64_t)x * (int64_t)multiplier + (1ll << 30);
+    int32_t v = (int32_t)(ab >> 31);
+    const int32_t mask = (int32_t)((1u << rs) - 1u);
+    const int32_t rem = v & mask;
+    const int32_t thr = (mask >> 1) - (v >> 31);
+    v = (v >> rs) + (rem > thr ? 1 : 0) + r.zp_out;
     v = v < r.act_min ? r.act_min : v;
     v = v > r.act_max ? r.act_max : v;
     return (uint32_t)v;
@@ -137,6 +158,8 @@ inline RequantDev make_requant_dev(const eh_requant &q) {
     const int rs = r.fast ? r.right_shift : 1;
     const int64_t pos = (1ll << 30) + (1ll << (30 + rs)) + (int64_t)q.zp_out * (1ll << (31 + rs));
     const int64_t neg = pos - (1ll << 31);
+    r.pc_multiplier = nullptr;
+    r.pc_shift = nullptr;
     r.pos_lo = (uint32_t)((uint64_t)pos & 0xFFFFFFFFull);
     r.pos_hi = (uint32_t)((uint64_t)pos >> 32);
     r.neg_lo = (uint32_t)((uint64_t)neg & 0xFFFFFFFFull);
@@ -159,7 +182,7 @@ inline FastDiv make_fastdiv(uint32_t d) {
 }
 __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) { return (__umulhi(f.mul, n) + n) >> f.shift; }
 
-int check_requant(const eh_requant *q);
+int check_requant(const eh_requant *q, bool signed_weights = false);
 
 // ---------------------------------------------------------------- implicit GEMM
 // One row of the k-table describes one load unit (VEC bytes) of the reduction
@@ -249,7 +272,8 @@ int igemm_n_tile(int32_t m, int32_t n, int32_t k);
 
 // ---------------------------------------------------------------- packing
 struct PackProblem {
-    const uint8_t *w;      // source weights (uint8)
+    const uint8_t *w;      // source weights (uint8, or int8 when w_signed)
+    int32_t w_signed;      // the bytes are int8 values (per-channel quantized weights): packed as they are, not minus 128
     const int32_t *bias;   // source bias [n] or null
     int8_t *b;             // [n_pad][k_pad]
     int32_t *colsum;       // [n_pad]  sum_k (w - 128)

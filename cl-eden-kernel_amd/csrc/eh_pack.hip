@@ -21,7 +21,8 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
         int32_t v = 0;
         if (o < p.n && k < p.k) {
             const int t = k / p.cin, c = k - t * p.cin;
-            v = (int32_t)p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]] - 128;
+            const uint8_t raw = p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]];
+            v = p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw - 128;
         }
         p.b[packed_b_offset(p.cfg, o, k >> 4, p.k_pad) + (k & 15)] = (int8_t)v;
         sum += v;

@@ -44,6 +44,10 @@ typedef enum eh_layout { EH_NCHW = 0, EH_NHWC = 1 } eh_layout;
  * (gpu/operators/cl_optimized_impls/CLDeconvolutionQuantized.cpp:39-46);
  * IOHW is the deconvolution order [Cin][Cout/g][kh][kw] (gpu/op_test/deconv_guard.h:53-69). */
 typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh_weight_layout;
+/* Or-ed into eh_conv_desc.weight_layout (convolution only): the weight bytes are int8 values, as the
+ * per-channel quantized convolution takes them (CLConvolutionPerChannelQuantized.cpp:73-159);
+ * eh_requant.zp_w is then an int8 zero point in [-128, 127] (0 in the reference). */
+#define EH_W_SIGNED 0x100
 
 /* Integer requantization parameters of one operator execution: what
  * CLGEMMConvolutionQuantized::execute derives from its tensors
@@ -121,6 +125,12 @@ void eh_make_requant(float input_scale, int32_t input_zp, float filter_scale, in
  * the two-step reference order. */
 int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int64_t count, int32_t form,
                      int32_t *single_shift);
+/* What CLConvolutionPerChannelQuantized::execute derives (CLConvolutionPerChannelQuantized.cpp:88-121):
+ * one (multiplier, shift) per output channel from input_scale * filter_scales[i] / output_scale, and
+ * the clamp range; out->multiplier / out->shift are unused in per-channel mode. */
+void eh_make_requant_perchannel(float input_scale, int32_t input_zp, const float *filter_scales, int32_t channels,
+                                float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out,
+                                int32_t *multipliers, int32_t *shifts);
 /* output extents: CLConvolution.cpp:99-104 and CLDeconvolution.cpp:82-87 */
 int32_t eh_conv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t dilation, int32_t stride);
 int32_t eh_deconv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t kernel, int32_t stride);
@@ -200,6 +210,11 @@ typedef struct eh_deconv_plan eh_deconv_plan;
  * CLQuantizedDirectConvolution.cpp:30-249) and their kernels. */
 int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
                       const eh_requant *q, void *stream);
+/* Per-channel mode (conv_per_channel_quantized, gpu/operators/cl_kernels/ConvolutionKernels.cpp:1317-1375):
+ * `count` == cout host arrays of multipliers and shifts replace the requant's single pair on every
+ * following run; two null pointers return to per-tensor mode.  Copies synchronously. */
+int eh_conv2d_u8_set_perchannel(eh_conv_plan *plan, const int32_t *multipliers, const int32_t *shifts, int32_t count,
+                                void *stream);
 int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
 int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
 int eh_conv2d_u8_destroy(eh_conv_plan *plan);

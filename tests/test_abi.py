@@ -59,6 +59,23 @@ def test_make_requant_matches_oracle_and_handles_bias_scale_mismatch():
     assert (q.multiplier, q.shift) == (0, 0)
 
 
+def test_make_requant_perchannel_matches_per_channel_oracle_multipliers():
+    """One (multiplier, shift) per filter scale: float(in_scale) * float(filter_scale) / float(out_scale) in double, as
+    the per-channel convolution computes them when it runs (cl_operators/CLConvolutionPerChannelQuantized.cpp:96-115)."""
+    rng = np.random.default_rng(23)
+    for _ in range(50):
+        s_in, s_out = [float(np.float32(x)) for x in np.exp(rng.uniform(np.log(1e-3), np.log(2.0), 2))]
+        scales = np.exp(rng.uniform(np.log(1e-4), np.log(1.0), int(rng.integers(1, 70)))).astype(np.float32)
+        zi, zo = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+        act, en = int(rng.integers(0, 4)), bool(rng.integers(0, 2))
+        q, mult, shift = eden.make_requant_perchannel(s_in, zi, scales, s_out, zo, act, en)
+        want = [O.quantize_multiplier(s_in * float(ws) / s_out) for ws in scales]
+        assert list(zip(mult.tolist(), shift.tolist())) == want
+        lo, hi = O.act_range_u8(act, s_out, zo) if en else (0, 255)
+        assert (q.zp_in, q.zp_w, q.zp_out, q.act_min, q.act_max) == (zi, 0, zo, lo, hi)
+        assert (q.multiplier, q.shift) == (0, 0)  # the per-tensor pair is unused in this mode
+
+
 def test_output_dim_formulas_match_oracle():
     lib = eden.load()
     rng = np.random.default_rng(22)
