@@ -66,6 +66,8 @@ EXPORTS = {
     "eh_make_requant_perchannel": (None, [C.c_float, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32, C.c_int, C.c_int,
                                           C.POINTER(Requant), C.c_void_p, C.c_void_p]),
     "eh_conv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "eh_dwconv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "eh_deconv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "eh_conv_out_dim": (C.c_int32, [C.c_int32] * 6),
     "eh_deconv_out_dim": (C.c_int32, [C.c_int32] * 5),
     "eh_init": (C.c_int, [C.c_int]),
@@ -254,6 +256,16 @@ class _Plan:
             getattr(load(), "eh_%s_u8_destroy" % self._kind)(self.handle)
             self.handle = C.c_void_p()
 
+    def set_perchannel(self, multipliers, shifts, stream=None):
+        """One multiplier / shift per output channel from now on (None, None: back to the Requant's pair).
+        Convolution, depthwise convolution and deconvolution plans."""
+        fn = getattr(load(), "eh_%s_u8_set_perchannel" % self._kind)
+        if multipliers is None:
+            check(fn(self.handle, None, None, 0, stream))
+            return
+        m, s = np.ascontiguousarray(multipliers, np.int32), np.ascontiguousarray(shifts, np.int32)
+        check(fn(self.handle, m.ctypes.data, s.ctypes.data, m.size, stream))
+
     def __del__(self):
         try:
             self.destroy()
@@ -270,13 +282,6 @@ class ConvPlan(_Plan):
         check(load().eh_conv2d_u8_plan(C.byref(self.handle), C.byref(desc), d_w.ptr, d_b.ptr if d_b else None,
                                        C.byref(q), stream))
 
-    def set_perchannel(self, multipliers, shifts, stream=None):
-        """One multiplier / shift per output channel from now on (None, None: back to the Requant's pair)."""
-        if multipliers is None:
-            check(load().eh_conv2d_u8_set_perchannel(self.handle, None, None, 0, stream))
-            return
-        m, s = np.ascontiguousarray(multipliers, np.int32), np.ascontiguousarray(shifts, np.int32)
-        check(load().eh_conv2d_u8_set_perchannel(self.handle, m.ctypes.data, s.ctypes.data, m.size, stream))
 
 
 def make_requant_perchannel(s_in, zp_in, filter_scales, s_out, zp_out, act=ACT_NONE, act_enabled=False):

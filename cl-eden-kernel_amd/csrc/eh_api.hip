@@ -168,6 +168,12 @@ int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t str
 }
 
 // Shared state of the three GEMM-shaped operators.
+static int check_perchannel(const int32_t *multipliers, const int32_t *shifts, int32_t count) {
+    for (int32_t i = 0; i < count; ++i)
+        EH_REQUIRE(multipliers[i] >= 0 && shifts[i] >= -31 && shifts[i] <= 30, "per-channel multiplier/shift %d out of range", i);
+    return EH_OK;
+}
+
 struct GemmOp {
     std::vector<GemmPart> parts;
     int32_t *bias_copy = nullptr;  // the operator's own copy of the int32 bias
@@ -196,9 +202,8 @@ struct GemmOp {
             return EH_OK;
         }
         EH_REQUIRE(multipliers != nullptr && shifts != nullptr && count == cout, "per-channel arrays must hold %d entries (got %d)", cout, count);
-        for (int32_t i = 0; i < count; ++i)
-            EH_REQUIRE(multipliers[i] >= 0 && shifts[i] >= -31 && shifts[i] <= 30, "per-channel multiplier/shift %d out of range", i);
-        int rc;
+        int rc = check_perchannel(multipliers, shifts, count);
+        if (rc) return rc;
         // padded so that the kernels may read whole channel blocks
         if (!pc_multiplier && (rc = dev_alloc(&pc_multiplier, (size_t)cout + 512))) return rc;
         if (!pc_shift && (rc = dev_alloc(&pc_shift, (size_t)cout + 512))) return rc;
@@ -333,6 +338,8 @@ struct eh_dwconv_plan {
     int32_t *bias_folded = nullptr;
     eh_requant q{};
     bool packed_valid = false;
+    bool w_signed = false;
+    int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;  // [cout + 4] once per-channel pairs are set
 };
 
 extern "C" {
@@ -935,7 +942,11 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
     *plan = nullptr;
     int rc = check_desc_common(desc);
     if (rc) return rc;
-    if ((rc = check_requant(q))) return rc;
+    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0;
+    eh_conv_desc plain = *desc;
+    plain.weight_layout &= ~EH_W_SIGNED;
+    desc = &plain;
+    if ((rc = check_requant(q, w_signed))) return rc;
     EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
                "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
     EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->weight_layout == EH_W_OHWI, "bad deconvolution weight layout %d",
@@ -944,6 +955,7 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
     eh_deconv_plan *pl = new (std::nothrow) eh_deconv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
+    pl->op.w_signed = w_signed;
     if (desc->n > 0) {
         rc = deconv_plan_build(pl, desc, as_stream(stream));
         if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
@@ -958,9 +970,16 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
     return EH_OK;
 }
 
+int eh_deconv2d_u8_set_perchannel(eh_deconv_plan *plan, const int32_t *multipliers, const int32_t *shifts, int32_t count,
+                                  void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    if (plan->d.n == 0) return EH_OK;
+    return plan->op.set_perchannel(multipliers, shifts, count, as_stream(stream));
+}
+
 int eh_deconv2d_u8_repack(eh_deconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q);
+    int rc = check_requant(q, plan->op.w_signed);
     if (rc) return rc;
     if (plan->d.n == 0) return EH_OK;
     if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
@@ -969,7 +988,7 @@ int eh_deconv2d_u8_repack(eh_deconv_plan *plan, const void *weight, const void *
 
 int eh_deconv2d_u8_run(eh_deconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    if (plan->d.n == 0) return check_requant(q);
+    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed);
     return plan->op.run(input, output, q, as_stream(stream));
 }
 
@@ -988,6 +1007,8 @@ static void dw_release(eh_dwconv_plan *pl) {
     dev_free(pl->bias_copy);
     dev_free(pl->w_pair);
     dev_free(pl->bias_folded);
+    dev_free(pl->pc_multiplier);
+    dev_free(pl->pc_shift);
 }
 
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
@@ -1004,7 +1025,7 @@ static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bi
 static int dw_refold(eh_dwconv_plan *pl, const eh_requant &q, hipStream_t stream) {
     if (!(pl->packed_valid && q.zp_in == pl->q.zp_in && q.zp_w == pl->q.zp_w)) {
         int rc = launch_dw_pack(pl->w_copy, pl->bias_copy, pl->w_pair, pl->bias_folded, pl->cout, pl->taps, q.zp_in,
-                                q.zp_w, stream);
+                                q.zp_w, pl->w_signed ? 1 : 0, stream);
         if (rc) return rc;
         pl->packed_valid = true;
     }
@@ -1018,7 +1039,11 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     *plan = nullptr;
     int rc = check_desc_common(desc);
     if (rc) return rc;
-    if ((rc = check_requant(q))) return rc;
+    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0;
+    eh_conv_desc plain = *desc;
+    plain.weight_layout &= ~EH_W_SIGNED;
+    desc = &plain;
+    if ((rc = check_requant(q, w_signed))) return rc;
     EH_REQUIRE(desc->dil_h > 0 && desc->dil_w > 0, "bad dilation");
     EH_REQUIRE(desc->depth_multiplier > 0, "bad depth multiplier %d", desc->depth_multiplier);
     EH_REQUIRE(desc->cout == desc->c * desc->depth_multiplier, "depthwise cout %d != c %d * depth multiplier %d", desc->cout,
@@ -1027,6 +1052,7 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     eh_dwconv_plan *pl = new (std::nothrow) eh_dwconv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
+    pl->w_signed = w_signed;
     pl->ho = eh_conv_out_dim(desc->h, desc->pad_t, desc->pad_b, desc->kh, desc->dil_h, desc->stride_h);
     pl->wo = eh_conv_out_dim(desc->w, desc->pad_l, desc->pad_r, desc->kw, desc->dil_w, desc->stride_w);
     pl->cout = desc->cout;
@@ -1052,9 +1078,35 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     return EH_OK;
 }
 
+int eh_dwconv2d_u8_set_perchannel(eh_dwconv_plan *plan, const int32_t *multipliers, const int32_t *shifts, int32_t count,
+                                  void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    if (multipliers == nullptr || shifts == nullptr) {
+        EH_REQUIRE(multipliers == nullptr && shifts == nullptr, "per-channel: one of the two arrays is null");
+        EH_HIP(hipStreamSynchronize(as_stream(stream)));  // a queued run may still read the arrays
+        dev_free(plan->pc_multiplier);
+        dev_free(plan->pc_shift);
+        plan->pc_multiplier = plan->pc_shift = nullptr;
+        return EH_OK;
+    }
+    EH_REQUIRE(count == plan->cout, "per-channel: %d pairs for %d output channels", count, plan->cout);
+    int rc = check_perchannel(multipliers, shifts, count);
+    if (rc) return rc;
+    hipStream_t s = as_stream(stream);
+    const size_t padded = (size_t)plan->cout + 4;
+    if (!plan->pc_multiplier && (rc = dev_alloc(&plan->pc_multiplier, padded))) return rc;
+    if (!plan->pc_shift && (rc = dev_alloc(&plan->pc_shift, padded))) return rc;
+    EH_HIP(hipMemsetAsync(plan->pc_multiplier, 0, padded * sizeof(int32_t), s));
+    EH_HIP(hipMemsetAsync(plan->pc_shift, 0, padded * sizeof(int32_t), s));
+    EH_HIP(hipMemcpyAsync(plan->pc_multiplier, multipliers, (size_t)count * sizeof(int32_t), hipMemcpyHostToDevice, s));
+    EH_HIP(hipMemcpyAsync(plan->pc_shift, shifts, (size_t)count * sizeof(int32_t), hipMemcpyHostToDevice, s));
+    EH_HIP(hipStreamSynchronize(s));  // the host arrays may go away after the call
+    return EH_OK;
+}
+
 int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q);
+    int rc = check_requant(q, plan->w_signed);
     if (rc) return rc;
     if ((rc = dw_set_weights(plan, weight, bias, as_stream(stream)))) return rc;
     return dw_refold(plan, *q, as_stream(stream));
@@ -1062,7 +1114,7 @@ int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *
 
 int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q);
+    int rc = check_requant(q, plan->w_signed);
     if (rc) return rc;
     const eh_conv_desc &d = plan->d;
     if (d.n == 0) return EH_OK;
@@ -1094,7 +1146,13 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     p.wo = plan->wo;
     p.zp_in = q->zp_in;
     p.zp_w = q->zp_w;
+    p.w_signed = plan->w_signed ? 1 : 0;
     p.rq = make_requant_dev(*q);
+    if (plan->pc_multiplier) {
+        p.rq.pc_multiplier = plan->pc_multiplier;
+        p.rq.pc_shift = plan->pc_shift;
+        p.rq.fast = 0;
+    }
     return d.layout == EH_NHWC ? launch_dwconv_nhwc(p, s) : launch_dwconv_nchw(p, s);
 }
 

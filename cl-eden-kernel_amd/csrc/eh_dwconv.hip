@@ -29,6 +29,26 @@ __device__ __forceinline__ uint32_t pair_bytes(uint32_t lo, uint32_t hi) {
     return __builtin_amdgcn_perm(hi, lo, sel);
 }
 
+// Four adjacent channels' accumulators to four output bytes.  `ch` is the first channel: with one
+// multiplier and shift per channel (depthwise_conv_per_channel,
+// gpu/operators/cl_kernels/DepthwiseconvolutionKernels.cpp:1323-1371) the four pairs are read from there.
+template <bool PC = true>
+__device__ __forceinline__ uint32_t requant4(int acc0, int acc1, int acc2, int acc3, const RequantDev &rq, uint32_t ch) {
+    if (PC && rq.pc_multiplier) {
+        const int4 m = *reinterpret_cast<const int4 *>(rq.pc_multiplier + ch);
+        const int4 s = *reinterpret_cast<const int4 *>(rq.pc_shift + ch);
+        return requant_u8_channel(acc0, m.x, s.x, rq) | (requant_u8_channel(acc1, m.y, s.y, rq) << 8) |
+               (requant_u8_channel(acc2, m.z, s.z, rq) << 16) | (requant_u8_channel(acc3, m.w, s.w, rq) << 24);
+    }
+    if (rq.fast == 2)
+        return requant_u8_fast_relu(acc0, rq) | (requant_u8_fast_relu(acc1, rq) << 8) | (requant_u8_fast_relu(acc2, rq) << 16) |
+               (requant_u8_fast_relu(acc3, rq) << 24);
+    if (rq.fast)
+        return requant_u8_fast(acc0, rq) | (requant_u8_fast(acc1, rq) << 8) | (requant_u8_fast(acc2, rq) << 16) |
+               (requant_u8_fast(acc3, rq) << 24);
+    return requant_u8(acc0, rq) | (requant_u8(acc1, rq) << 8) | (requant_u8(acc2, rq) << 16) | (requant_u8(acc3, rq) << 24);
+}
+
 template <int KH, int KW>
 __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, const long total) {
     const long idx = (long)blockIdx.x * 256 + threadIdx.x;
@@ -76,14 +96,7 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
             acc3 = dot2(pair_bytes<3>(lo, hi), w4.w, acc3);
         }
     }
-    uint32_t o;
-    if (p.rq.fast)
-        o = requant_u8_fast(acc0, p.rq) | (requant_u8_fast(acc1, p.rq) << 8) | (requant_u8_fast(acc2, p.rq) << 16) |
-            (requant_u8_fast(acc3, p.rq) << 24);
-    else
-        o = requant_u8(acc0, p.rq) | (requant_u8(acc1, p.rq) << 8) | (requant_u8(acc2, p.rq) << 16) |
-            (requant_u8(acc3, p.rq) << 24);
-    *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) = o;
+    *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) = requant4(acc0, acc1, acc2, acc3, p.rq, (uint32_t)cq * 4u);
 }
 
 // 3x3, dilation 1, stride S in both directions: a thread owns four adjacent channels of FOUR
@@ -91,7 +104,7 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
 // once (every load is issued before the first use, from clamped in-image addresses; taps
 // outside the image are then replaced by the input zero point), so the address arithmetic, the
 // weight and bias loads and the border tests are shared by sixteen outputs.
-template <int S>
+template <int S, bool PC>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
     constexpr int TW = 4, IW = (TW - 1) * S + 3;
@@ -152,15 +165,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p
             acc2 = dot2(pair_bytes<2>(lo, hi), w4[pr].z, acc2);
             acc3 = dot2(pair_bytes<3>(lo, hi), w4[pr].w, acc3);
         }
-        uint32_t o;
-        if (rq.fast == 2)
-            o = requant_u8_fast_relu(acc0, rq) | (requant_u8_fast_relu(acc1, rq) << 8) | (requant_u8_fast_relu(acc2, rq) << 16) |
-                (requant_u8_fast_relu(acc3, rq) << 24);
-        else if (rq.fast)
-            o = requant_u8_fast(acc0, rq) | (requant_u8_fast(acc1, rq) << 8) | (requant_u8_fast(acc2, rq) << 16) |
-                (requant_u8_fast(acc3, rq) << 24);
-        else
-            o = requant_u8(acc0, rq) | (requant_u8(acc1, rq) << 8) | (requant_u8(acc2, rq) << 16) | (requant_u8(acc3, rq) << 24);
+        const uint32_t o = requant4<PC>(acc0, acc1, acc2, acc3, rq, cq * 4u);
         if (ox0 + j < p.wo) *reinterpret_cast<uint32_t *>(dst + (uint32_t)j * (uint32_t)p.cout) = o;
     }
 }
@@ -199,22 +204,28 @@ __global__ __launch_bounds__(256) void dw_scalar_kernel(const DwProblem p, const
             const size_t a_idx = NHWC ? (((size_t)img * p.h + iy) * p.w_ + ix) * p.c + ic
                                       : (((size_t)img * p.c + ic) * p.h + iy) * p.w_ + ix;
             const int32_t a = (int32_t)p.in[a_idx] - p.zp_in;
-            const int32_t w = (int32_t)p.w[((size_t)oc * p.kh + ky) * p.kw + kx] - p.zp_w;
+            const uint8_t raw = p.w[((size_t)oc * p.kh + ky) * p.kw + kx];
+            const int32_t w = (p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw) - p.zp_w;
             acc += a * w;
         }
     }
-    p.out[idx] = (uint8_t)requant_u8(acc, p.rq);
+    p.out[idx] = (uint8_t)(p.rq.pc_multiplier ? requant_u8_channel(acc, p.rq.pc_multiplier[oc], p.rq.pc_shift[oc], p.rq)
+                                               : requant_u8(acc, p.rq));
 }
 
 __global__ void dw_pack_kernel(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
-                               int32_t taps, int32_t zp_in, int32_t zp_w) {
+                               int32_t taps, int32_t zp_in, int32_t zp_w, int32_t w_signed) {
     const int oc = blockIdx.x * blockDim.x + threadIdx.x;
     if (oc >= cout) return;
     int32_t sum = 0;
     const int pairs = (taps + 1) >> 1;
     for (int pr = 0; pr < pairs; ++pr) {
-        const int32_t lo = (int32_t)w[(size_t)oc * taps + 2 * pr] - zp_w;
-        const int32_t hi = 2 * pr + 1 < taps ? (int32_t)w[(size_t)oc * taps + 2 * pr + 1] - zp_w : 0;
+        auto value = [&](int t) {
+            const uint8_t raw = w[(size_t)oc * taps + t];
+            return (w_signed ? (int32_t)(int8_t)raw : (int32_t)raw) - zp_w;
+        };
+        const int32_t lo = value(2 * pr);
+        const int32_t hi = 2 * pr + 1 < taps ? value(2 * pr + 1) : 0;
         sum += lo + hi;
         w_pair[(size_t)pr * cout + oc] = (int32_t)(((uint32_t)lo & 0xFFFFu) | ((uint32_t)hi << 16));
     }
@@ -224,10 +235,10 @@ __global__ void dw_pack_kernel(const uint8_t *w, const int32_t *bias, int32_t *w
 }  // namespace
 
 int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
-                   int32_t taps, int32_t zp_in, int32_t zp_w, hipStream_t stream) {
+                   int32_t taps, int32_t zp_in, int32_t zp_w, int32_t w_signed, hipStream_t stream) {
     if (cout <= 0) return EH_OK;
     hipLaunchKernelGGL(dw_pack_kernel, dim3((cout + 127) / 128), dim3(128), 0, stream, w, bias, w_pair, bias_folded, cout,
-                       taps, zp_in, zp_w);
+                       taps, zp_in, zp_w, w_signed);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }
@@ -246,12 +257,9 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
         const long blocks = (total + 255) / 256;
         EH_REQUIRE(total < (1l << 31), "depthwise: grid too large");
         const FastDiv d_cq = make_fastdiv((uint32_t)(p.c >> 2)), d_t = make_fastdiv((uint32_t)tiles_x), d_ho = make_fastdiv((uint32_t)p.ho);
-        if (p.stride_h == 1)
-            hipLaunchKernelGGL((dw3x3_nhwc_tile4_kernel<1>), dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total,
-                               tiles_x, d_cq, d_t, d_ho);
-        else
-            hipLaunchKernelGGL((dw3x3_nhwc_tile4_kernel<2>), dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total,
-                               tiles_x, d_cq, d_t, d_ho);
+        auto kernel = p.stride_h == 1 ? (p.rq.pc_multiplier ? dw3x3_nhwc_tile4_kernel<1, true> : dw3x3_nhwc_tile4_kernel<1, false>)
+                                      : (p.rq.pc_multiplier ? dw3x3_nhwc_tile4_kernel<2, true> : dw3x3_nhwc_tile4_kernel<2, false>);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total, tiles_x, d_cq, d_t, d_ho);
     } else if (vec) {
         const long total = outs / 4;
         const long blocks = (total + 255) / 256;

@@ -292,7 +292,7 @@ int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded
 // ---------------------------------------------------------------- depthwise
 struct DwProblem {
     const uint8_t *in;
-    const uint8_t *w;            // raw weights [cout][kh*kw] (uint8)
+    const uint8_t *w;            // raw weights [cout][kh*kw] (uint8, or int8 bytes when w_signed)
     const int32_t *bias;         // raw bias [cout] or null
     const int32_t *w_pair;       // [ceil(taps/2)][cout]: (w[2p]-zp_w) | (w[2p+1]-zp_w) << 16 as int16 halves
     const int32_t *bias_folded;  // [cout]: bias - zp_in * sum_t (w - zp_w)
@@ -301,10 +301,11 @@ struct DwProblem {
     int32_t kh, kw, stride_h, stride_w, pad_t, pad_l, dil_h, dil_w;
     int32_t ho, wo;
     int32_t zp_in, zp_w;
-    RequantDev rq;
+    int32_t w_signed;            // weight bytes are int8
+    RequantDev rq;               // rq.pc_multiplier / rq.pc_shift: [cout + 4] when set
 };
 int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
-                   int32_t taps, int32_t zp_in, int32_t zp_w, hipStream_t stream);
+                   int32_t taps, int32_t zp_in, int32_t zp_w, int32_t w_signed, hipStream_t stream);
 int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream);
 int launch_dwconv_nchw(const DwProblem &p, hipStream_t stream);
 

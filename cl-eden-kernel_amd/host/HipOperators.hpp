@@ -134,6 +134,37 @@ inline eh_requant requantFromTensors(const std::shared_ptr<HipTensor> &in, const
     return q;
 }
 
+// Per-channel mode: int8 weights and one filter scale per output channel
+// (cl_optimized_impls/CLConvolutionPerChannelQuantized.cpp:96-120,
+// CLDepthwiseConvolutionPerChannelQuantized.cpp:133-160, CLDeconvolutionPerChannelQuantized.cpp:147-179).
+// The pairs are derived from the tensors' scales at every execute(), as there; the plan is only told when they change.
+struct PerChannelState {
+    std::vector<int32_t> multipliers, shifts;  // what the plan holds
+    bool sent = false;
+
+    // weight_zp: the convolution ignores the filter's zero point, the depthwise convolution and the
+    // deconvolution subtract it.  range_always: the deconvolution derives the activation range even
+    // for a disabled activation.
+    eh_requant derive(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &out, const ActivationInfo &act,
+                      const std::vector<float> &scales, int32_t weight_zp, bool range_always, std::vector<int32_t> *m,
+                      std::vector<int32_t> *s) const {
+        eh_requant q;
+        m->assign(scales.size(), 0);
+        s->assign(scales.size(), 0);
+        eh_make_requant_perchannel(in->getScale(), in->getZeroPoint(), scales.data(), (int32_t)scales.size(), out->getScale(),
+                                   out->getZeroPoint(), toEhActivation(act), (range_always || act.isEnabled()) ? 1 : 0, &q, m->data(),
+                                   s->data());
+        q.zp_w = weight_zp;
+        return q;
+    }
+};
+
+inline bool perChannelTensors(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &w,
+                              const std::shared_ptr<HipTensor> &bias, const std::shared_ptr<HipTensor> &out) {
+    return in->getDataType() == DataType::UINT8 && w->getDataType() == DataType::INT8 &&
+           bias->getDataType() == DataType::INT32 && out->getDataType() == DataType::UINT8;
+}
+
 inline bool uint8Tensors(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &w,
                          const std::shared_ptr<HipTensor> &bias, const std::shared_ptr<HipTensor> &out) {
     return in->getDataType() == DataType::UINT8 && w->getDataType() == DataType::UINT8 &&
@@ -165,8 +196,11 @@ public:
         if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;  // zero-sized: nothing to prepare
         CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipConvolution: only the UINT8 path exists on this backend");
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipConvolution: no texture storage");
-        CHECK_EXPR_RETURN_FAILURE(!parameters_->per_channel_quant, "HipConvolution: per-channel quantization is not offered");
-        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipConvolution: expects uint8 input/weight/output and int32 bias");
+        per_channel_ = parameters_->per_channel_quant;
+        if (per_channel_)
+            CHECK_EXPR_RETURN_FAILURE(detail::perChannelTensors(input_, weight_, bias_, output_), "HipConvolution: per-channel mode expects uint8 input/output, int8 weight and int32 bias");
+        else
+            CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipConvolution: expects uint8 input/weight/output and int32 bias");
 
         Dim4 in = input_->getDim(), wd = weight_->getDim();
         if (!parameters_->isNCHW) in = convertDimToNCHW(in);
@@ -202,9 +236,15 @@ public:
         CHECK_EXPR_RETURN_FAILURE((int64_t)output_->getTotalSizeFromDims() == (int64_t)d.n * d.cout * ho * wo,
                                   "HipConvolution: output tensor has %u elements, the geometry gives %lld", output_->getTotalSizeFromDims(),
                                   (long long)d.n * d.cout * ho * wo);
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        if (per_channel_) {
+            CHECK_EXPR_RETURN_FAILURE(parameters_->scales.size() == (size_t)desc_.cout, "HipConvolution: %zu filter scales for %d output channels", parameters_->scales.size(), desc_.cout);
+            desc_.weight_layout |= EH_W_SIGNED;
+        }
+        eh_requant q;
+        CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipConvolution::initialize: requantization parameters");
         const int rc = eh_conv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
         CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::initialize: %s", eh_last_error());
+        if (per_channel_) CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipConvolution::initialize: per-channel pairs");
         return Status::SUCCESS;
     }
 
@@ -214,7 +254,8 @@ public:
             return Status::SUCCESS;
         }
         if (input_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        eh_requant q;
+        CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipConvolution::execute: requantization parameters");
         if (weights_as_input_ || bias_as_input_) {
             const int rc = eh_conv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute (repack): %s", eh_last_error());
@@ -234,6 +275,27 @@ public:
     }
 
 private:
+    // The requantization parameters of this execution, read from the tensors now; in per-channel mode
+    // also hands the plan the channel pairs when they differ from the ones it holds.
+    Status currentRequant(eh_requant *q) {
+        if (!per_channel_) {
+            *q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+            return Status::SUCCESS;
+        }
+        std::vector<int32_t> m, s;
+        *q = pc_.derive(input_, output_, activation_info_, parameters_->scales, 0, false, &m, &s);
+        if (plan_ != nullptr && (!pc_.sent || m != pc_.multipliers || s != pc_.shifts)) {
+            const int rc = eh_conv2d_u8_set_perchannel(plan_, m.data(), s.data(), (int32_t)m.size(), runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution: %s", eh_last_error());
+            pc_.multipliers = m;
+            pc_.shifts = s;
+            pc_.sent = true;
+        }
+        return Status::SUCCESS;
+    }
+
+    bool per_channel_ = false;
+    detail::PerChannelState pc_;
     std::shared_ptr<HipRuntime> runtime_;
     PrecisionType precision_;
     std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
@@ -266,8 +328,11 @@ public:
         if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
         CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipDepthwiseConvolution: only the UINT8 path exists on this backend");
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipDepthwiseConvolution: no texture storage");
-        CHECK_EXPR_RETURN_FAILURE(!parameters_->per_channel_quant, "HipDepthwiseConvolution: per-channel quantization is not offered");
-        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDepthwiseConvolution: expects uint8 input/weight/output and int32 bias");
+        per_channel_ = parameters_->per_channel_quant;
+        if (per_channel_)
+            CHECK_EXPR_RETURN_FAILURE(detail::perChannelTensors(input_, weight_, bias_, output_), "HipDepthwiseConvolution: per-channel mode expects uint8 input/output, int8 weight and int32 bias");
+        else
+            CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDepthwiseConvolution: expects uint8 input/weight/output and int32 bias");
 
         Dim4 in = input_->getDim();
         if (!parameters_->isNCHW) in = convertDimToNCHW(in);
@@ -294,9 +359,15 @@ public:
         d.weight_layout = EH_W_OIHW;
         CHECK_EXPR_RETURN_FAILURE(wd.n == (uint32_t)d.cout && wd.c == 1, "HipDepthwiseConvolution: weight shape [%u %u %u %u] is not [C*dm][1][kh][kw]", wd.n, wd.c, wd.h, wd.w);
         desc_ = d;
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        if (per_channel_) {
+            CHECK_EXPR_RETURN_FAILURE(parameters_->scales.size() == (size_t)desc_.cout, "HipDepthwiseConvolution: %zu filter scales for %d output channels", parameters_->scales.size(), desc_.cout);
+            desc_.weight_layout |= EH_W_SIGNED;
+        }
+        eh_requant q;
+        CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDepthwiseConvolution::initialize: requantization parameters");
         const int rc = eh_dwconv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
         CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDepthwiseConvolution::initialize: %s", eh_last_error());
+        if (per_channel_) CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDepthwiseConvolution::initialize: per-channel pairs");
         return Status::SUCCESS;
     }
 
@@ -306,7 +377,8 @@ public:
             return Status::SUCCESS;
         }
         if (input_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        eh_requant q;
+        CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDepthwiseConvolution::execute: requantization parameters");
         if (weights_as_input_) {
             const int rc = eh_dwconv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDepthwiseConvolution::execute (repack): %s", eh_last_error());
@@ -326,6 +398,27 @@ public:
     }
 
 private:
+    // The requantization parameters of this execution, read from the tensors now; in per-channel mode
+    // also hands the plan the channel pairs when they differ from the ones it holds.
+    Status currentRequant(eh_requant *q) {
+        if (!per_channel_) {
+            *q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+            return Status::SUCCESS;
+        }
+        std::vector<int32_t> m, s;
+        *q = pc_.derive(input_, output_, activation_info_, parameters_->scales, weight_->getZeroPoint(), false, &m, &s);
+        if (plan_ != nullptr && (!pc_.sent || m != pc_.multipliers || s != pc_.shifts)) {
+            const int rc = eh_dwconv2d_u8_set_perchannel(plan_, m.data(), s.data(), (int32_t)m.size(), runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDepthwiseConvolution: %s", eh_last_error());
+            pc_.multipliers = m;
+            pc_.shifts = s;
+            pc_.sent = true;
+        }
+        return Status::SUCCESS;
+    }
+
+    bool per_channel_ = false;
+    detail::PerChannelState pc_;
     std::shared_ptr<HipRuntime> runtime_;
     PrecisionType precision_;
     std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
@@ -431,8 +524,11 @@ public:
 
         if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
         CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipDeconvolution: only the UINT8 path exists on this backend");
-        CHECK_EXPR_RETURN_FAILURE(!parameters_->per_channel_quant, "HipDeconvolution: per-channel quantization is not offered");
-        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDeconvolution: expects uint8 input/weight/output and int32 bias");
+        per_channel_ = parameters_->per_channel_quant;
+        if (per_channel_)
+            CHECK_EXPR_RETURN_FAILURE(detail::perChannelTensors(input_, weight_, bias_, output_), "HipDeconvolution: per-channel mode expects uint8 input/output, int8 weight and int32 bias");
+        else
+            CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDeconvolution: expects uint8 input/weight/output and int32 bias");
 
         Dim4 in = input_->getDim();
         if (!parameters_->isNCHW) in = convertDimToNCHW(in);
@@ -466,9 +562,15 @@ public:
         CHECK_EXPR_RETURN_FAILURE((int64_t)output_->getTotalSizeFromDims() == (int64_t)d.n * d.cout * oh * ow,
                                   "HipDeconvolution: output tensor has %u elements, the geometry gives %lld", output_->getTotalSizeFromDims(),
                                   (long long)d.n * d.cout * oh * ow);
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        if (per_channel_) {
+            CHECK_EXPR_RETURN_FAILURE(parameters_->scales.size() == (size_t)desc_.cout, "HipDeconvolution: %zu filter scales for %d output channels", parameters_->scales.size(), desc_.cout);
+            desc_.weight_layout |= EH_W_SIGNED;
+        }
+        eh_requant q;
+        CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDeconvolution::initialize: requantization parameters");
         const int rc = eh_deconv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
         CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDeconvolution::initialize: %s", eh_last_error());
+        if (per_channel_) CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDeconvolution::initialize: per-channel pairs");
         return Status::SUCCESS;
     }
 
@@ -478,7 +580,8 @@ public:
             return Status::SUCCESS;
         }
         if (input_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        eh_requant q;
+        CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDeconvolution::execute: requantization parameters");
         if (weights_as_input_) {
             const int rc = eh_deconv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDeconvolution::execute (repack): %s", eh_last_error());
@@ -498,6 +601,27 @@ public:
     }
 
 private:
+    // The requantization parameters of this execution, read from the tensors now; in per-channel mode
+    // also hands the plan the channel pairs when they differ from the ones it holds.
+    Status currentRequant(eh_requant *q) {
+        if (!per_channel_) {
+            *q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+            return Status::SUCCESS;
+        }
+        std::vector<int32_t> m, s;
+        *q = pc_.derive(input_, output_, activation_info_, parameters_->scales, weight_->getZeroPoint(), true, &m, &s);
+        if (plan_ != nullptr && (!pc_.sent || m != pc_.multipliers || s != pc_.shifts)) {
+            const int rc = eh_deconv2d_u8_set_perchannel(plan_, m.data(), s.data(), (int32_t)m.size(), runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDeconvolution: %s", eh_last_error());
+            pc_.multipliers = m;
+            pc_.shifts = s;
+            pc_.sent = true;
+        }
+        return Status::SUCCESS;
+    }
+
+    bool per_channel_ = false;
+    detail::PerChannelState pc_;
     std::shared_ptr<HipRuntime> runtime_;
     PrecisionType precision_;
     std::shared_ptr<HipTensor> input_, output_, weight_, bias_;

@@ -594,6 +594,197 @@ static int gpu_tests() {
         return ok;
     });
 
+
+    // ------------------------------------------------------------ per-channel quantization
+    run_test("Convolution.PerChannel_reference_uint8_vector", [&] {
+        // src/userdriver/gpu/gpu_userdriver_test.cc:474-576: int8 weights in (out, kh, kw, in) order,
+        // one filter scale per output channel, expected output bit for bit
+        bool ok = true;
+        std::vector<uint8_t> x = {138, 138, 138, 108, 108, 108};
+        std::vector<int8_t> w = {1, 2, 1, 2, 1, 2};
+        std::vector<int32_t> b = {4, 4, 4};
+        const uint8_t expect[9] = {121, 121, 121, 118, 118, 118, 115, 115, 115};
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 2, 3, 1}, DataOrder::NCHW, 0.5f, 128);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{3, 1, 1, 2}, DataOrder::NCHW, 0.0f, 0);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{3, 1, 1, 1});
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 3, 3, 1}, DataOrder::NCHW, 1.0f, 128);
+        auto params = std::make_shared<ConvolutionParameters>();
+        params->androidNN = true;
+        params->per_channel_quant = true;
+        params->scales = {0.5f, 0.75f, 1.0f};
+        HipConvolution conv(rt, U8);
+        EXPECT(conv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+        EXPECT(conv.execute() == Status::SUCCESS);
+        std::vector<uint8_t> got(9);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        for (int i = 0; i < 9; ++i) EXPECT(got[i] == expect[i]);
+        return ok;
+    });
+
+    // pairs as the per-channel operators derive them: (double)in_scale * (double)filter_scale / (double)out_scale
+    auto channel_pairs = [](float s_in, const std::vector<float> &scales, float s_out, std::vector<int32_t> *m, std::vector<int32_t> *sh) {
+        m->resize(scales.size());
+        sh->resize(scales.size());
+        for (size_t i = 0; i < scales.size(); ++i)
+            eo_quantize_multiplier((double)s_in * (double)scales[i] / (double)s_out, &(*m)[i], &(*sh)[i]);
+    };
+    auto channel_scales = [](int count, uint64_t seed, float base) {
+        auto r = rand_u8(count, seed);
+        std::vector<float> v(count);
+        for (int i = 0; i < count; ++i) v[i] = base * (1.0f + 19.0f * r[i] / 255.0f);
+        return v;
+    };
+    auto to_i8 = [](const std::vector<uint8_t> &v) {
+        std::vector<int8_t> o(v.size());
+        for (size_t i = 0; i < v.size(); ++i) o[i] = (int8_t)((int)v[i] - 128);
+        return o;
+    };
+
+    run_test("Convolution.PerChannel_channels_last_relu6_and_scales_read_at_execute", [&] {
+        bool ok = true;
+        const eo_conv_shape s = shape(2, 32, 12, 12, 48, 3, 3, 1, 1, 1, 1, 1, 1);
+        auto x = rand_u8((size_t)2 * 32 * 144, 201);
+        auto w = to_i8(rand_u8((size_t)48 * 32 * 9, 202));
+        auto b = rand_i32(48, 203, -1000, 1000);
+        auto scales = channel_scales(48, 204, 0.001f);
+        const float s_in = 0.02f, s_out = 0.6f;
+        std::vector<int8_t> w_ohwi(w.size());
+        for (int o = 0; o < 48; ++o)
+            for (int c = 0; c < 32; ++c)
+                for (int t = 0; t < 9; ++t) w_ohwi[((size_t)o * 9 + t) * 32 + c] = w[((size_t)o * 32 + c) * 9 + t];
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{2, 12, 12, 32}, DataOrder::NHWC, s_in, 117);
+        // the filter's own zero point is not used by the per-channel convolution
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w_ohwi.data(), Dim4{48, 3, 3, 32}, DataOrder::NHWC, 0.0f, 5);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 48, 1, 1});
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{2, 12, 12, 48}, DataOrder::NHWC, s_out, 20);
+        auto params = std::make_shared<ConvolutionParameters>();
+        params->padding = {1, 1, 1, 1};
+        params->isNCHW = false;
+        params->per_channel_quant = true;
+        params->scales = scales;
+        params->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU6, true);
+        HipConvolution conv(rt, U8);
+        EXPECT(conv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        auto x_dev = nchw_to_nhwc(x, 2, 32, 12, 12);
+        EXPECT(input->writeData(x_dev.data()) == Status::SUCCESS);
+        std::vector<uint8_t> want((size_t)2 * 48 * 144), got(want.size());
+        for (int round = 0; round < 2; ++round) {
+            if (round == 1)
+                for (auto &v : params->scales) v *= 1.7f;  // the next execute() must derive new pairs
+            std::vector<int32_t> m, sh;
+            channel_pairs(s_in, params->scales, s_out, &m, &sh);
+            eo_quant q = {117, 0, 20, 0, 0, 0, 0};
+            eo_act_range_u8(EO_ACT_RELU6, s_out, 20, &q.act_min, &q.act_max);
+            eo_conv2d_u8_perchannel(x.data(), w.data(), b.data(), want.data(), &s, &q, m.data(), sh.data(), nullptr);
+            EXPECT(conv.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(nhwc_to_nchw(got, 2, 48, 12, 12), want));
+            EXPECT(varied(want));
+        }
+        return ok;
+    });
+
+    run_test("DepthwiseConvolution.PerChannel_3x3_stride2_channels_last_and_planar_multiplier2", [&] {
+        bool ok = true;
+        for (int variant = 0; variant < 2; ++variant) {
+            const bool nchw = variant == 1;
+            const int c = nchw ? 6 : 32, dm = nchw ? 2 : 1, cout = c * dm, h = 13, wdt = 11;
+            const eo_conv_shape s = shape(2, c, h, wdt, cout, 3, 3, 2, 2, 1, 1, 1, 1, 1, 1, 1, dm);
+            const int ho = eo_conv_out_dim(h, 1, 1, 3, 1, 2), wo = eo_conv_out_dim(wdt, 1, 1, 3, 1, 2);
+            auto x = rand_u8((size_t)2 * c * h * wdt, 211 + variant);
+            auto w = to_i8(rand_u8((size_t)cout * 9, 213 + variant));
+            auto b = rand_i32(cout, 215, -500, 500);
+            auto scales = channel_scales(cout, 216, 0.002f);
+            const float s_in = 0.02f, s_out = 0.25f;
+            std::vector<int32_t> m, sh;
+            channel_pairs(s_in, scales, s_out, &m, &sh);
+            eo_quant q = {117, -3, 131, 0, 0, 0, 255};  // the filter's zero point is subtracted here
+            std::vector<uint8_t> want((size_t)2 * cout * ho * wo), got(want.size());
+            eo_dwconv2d_u8_perchannel(x.data(), w.data(), b.data(), want.data(), &s, &q, m.data(), sh.data(), nullptr);
+            const DataOrder order = nchw ? DataOrder::NCHW : DataOrder::NHWC;
+            Dim4 in_dim = nchw ? Dim4{2, (uint32_t)c, (uint32_t)h, (uint32_t)wdt} : Dim4{2, (uint32_t)h, (uint32_t)wdt, (uint32_t)c};
+            Dim4 out_dim = nchw ? Dim4{2, (uint32_t)cout, (uint32_t)ho, (uint32_t)wo} : Dim4{2, (uint32_t)ho, (uint32_t)wo, (uint32_t)cout};
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, in_dim, order, s_in, 117);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{(uint32_t)cout, 1, 3, 3}, DataOrder::NCHW, 0.0f, -3);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, (uint32_t)cout, 1, 1});
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, out_dim, order, s_out, 131);
+            auto params = std::make_shared<DepthwiseConvolutionParameters>();
+            params->padding = {1, 1, 1, 1};
+            params->stride = {2, 2};
+            params->depth_multiplier = dm;
+            params->isNCHW = nchw;
+            params->per_channel_quant = true;
+            params->scales = scales;
+            HipDepthwiseConvolution dw(rt, U8);
+            EXPECT(dw.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+            auto x_dev = nchw ? x : nchw_to_nhwc(x, 2, c, h, wdt);
+            EXPECT(input->writeData(x_dev.data()) == Status::SUCCESS);
+            EXPECT(dw.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(nchw ? got : nhwc_to_nchw(got, 2, cout, ho, wo), want));
+            EXPECT(varied(want));
+        }
+        return ok;
+    });
+
+    run_test("Deconvolution.PerChannel_4x4_stride2_planar_range_derived_for_a_disabled_activation", [&] {
+        bool ok = true;
+        const eo_conv_shape s = shape(2, 32, 9, 7, 24, 4, 4, 2, 2, 1, 1, 1, 1);
+        const int oh = eo_deconv_out_dim(9, 1, 1, 4, 2), ow = eo_deconv_out_dim(7, 1, 1, 4, 2);
+        auto x = rand_u8((size_t)2 * 32 * 63, 221);
+        auto w = to_i8(rand_u8((size_t)32 * 24 * 16, 222));
+        auto b = rand_i32(24, 223, -500, 500);
+        auto scales = channel_scales(24, 224, 0.001f);
+        const float s_in = 0.02f, s_out = 0.3f;
+        std::vector<int32_t> m, sh;
+        channel_pairs(s_in, scales, s_out, &m, &sh);
+        eo_quant q = {117, 2, 100, 0, 0, 0, 255};
+        // CLDeconvolutionPerChannelQuantized.cpp:162-175 derives the range without asking isEnabled()
+        eo_act_range_u8(EO_ACT_RELU, s_out, 100, &q.act_min, &q.act_max);
+        std::vector<uint8_t> want((size_t)2 * 24 * oh * ow), got(want.size());
+        eo_deconv2d_u8_perchannel(x.data(), w.data(), b.data(), want.data(), &s, &q, m.data(), sh.data(), nullptr);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{2, 32, 9, 7}, DataOrder::NCHW, s_in, 117);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{32, 24, 4, 4}, DataOrder::NCHW, 0.0f, 2);
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 24, 1, 1});
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{2, 24, (uint32_t)oh, (uint32_t)ow}, DataOrder::NCHW, s_out, 100);
+        auto params = std::make_shared<DeconvolutionParameters>();
+        params->padding = {1, 1, 1, 1};
+        params->stride = {2, 2};
+        params->per_channel_quant = true;
+        params->scales = scales;
+        params->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU, false);
+        HipDeconvolution deconv(rt, U8);
+        EXPECT(deconv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+        EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+        EXPECT(deconv.execute() == Status::SUCCESS);
+        EXPECT(output->readData(got.data()) == Status::SUCCESS);
+        EXPECT(same(got, want));
+        EXPECT(varied(want));
+        return ok;
+    });
+
+    run_test("PerChannel.ScaleCountAndWeightTypeAreChecked", [&] {
+        bool ok = true;
+        std::vector<int8_t> w(8 * 8 * 9, 1);
+        std::vector<uint8_t> wu(8 * 8 * 9, 1);
+        std::vector<int32_t> b(8, 0);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 8, 6, 6}, DataOrder::NCHW, 0.5f, 0);
+        std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, U8, w.data(), Dim4{8, 8, 3, 3});
+        std::shared_ptr<ITensor> weight_u8 = std::make_shared<HipTensor>(rt, U8, wu.data(), Dim4{8, 8, 3, 3});
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, U8, b.data(), Dim4{1, 8, 1, 1});
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, U8, DataType::UINT8, Dim4{1, 8, 4, 4}, DataOrder::NCHW, 1.0f, 0);
+        auto params = std::make_shared<ConvolutionParameters>();
+        params->per_channel_quant = true;
+        params->scales = std::vector<float>(7, 0.5f);
+        HipConvolution short_scales(rt, U8), wrong_type(rt, U8), int8_without_flag(rt, U8);
+        EXPECT(short_scales.initialize({input, weight, bias}, {output}, params) == Status::FAILURE);
+        params->scales = std::vector<float>(8, 0.5f);
+        EXPECT(wrong_type.initialize({input, weight_u8, bias}, {output}, params) == Status::FAILURE);
+        EXPECT(int8_without_flag.initialize({input, weight, bias}, {output}, std::make_shared<ConvolutionParameters>()) == Status::FAILURE);
+        return ok;
+    });
+
     std::printf("%d of %d GPU operator tests failed\n", g_failed, g_run);
     return g_failed ? 1 : 0;
 }

@@ -44,8 +44,10 @@ typedef enum eh_layout { EH_NCHW = 0, EH_NHWC = 1 } eh_layout;
  * (gpu/operators/cl_optimized_impls/CLDeconvolutionQuantized.cpp:39-46);
  * IOHW is the deconvolution order [Cin][Cout/g][kh][kw] (gpu/op_test/deconv_guard.h:53-69). */
 typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh_weight_layout;
-/* Or-ed into eh_conv_desc.weight_layout (convolution only): the weight bytes are int8 values, as the
- * per-channel quantized convolution takes them (CLConvolutionPerChannelQuantized.cpp:73-159);
+/* Or-ed into eh_conv_desc.weight_layout (convolution, depthwise convolution, deconvolution): the weight
+ * bytes are int8 values, as the per-channel quantized operators take them
+ * (CLConvolutionPerChannelQuantized.cpp:73-159, cl_kernels/DepthwiseconvolutionKernels.cpp:2323-2340,
+ * cl_kernels/DeconvolutionKernels.cpp:449-454);
  * eh_requant.zp_w is then an int8 zero point in [-128, 127] (0 in the reference). */
 #define EH_W_SIGNED 0x100
 
@@ -224,6 +226,11 @@ int eh_conv2d_u8_destroy(eh_conv_plan *plan);
  * cl_optimized_impls/CLDepthwiseConvolutionQuantized.cpp:82-674). */
 int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
                         const eh_requant *q, void *stream);
+/* Per-channel mode of the depthwise convolution
+ * (cl_optimized_impls/CLDepthwiseConvolutionPerChannelQuantized.cpp:133-153,
+ * cl_kernels/DepthwiseconvolutionKernels.cpp:1323-1371); arguments as eh_conv2d_u8_set_perchannel. */
+int eh_dwconv2d_u8_set_perchannel(eh_dwconv_plan *plan, const int32_t *multipliers, const int32_t *shifts, int32_t count,
+                                  void *stream);
 int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
 int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
 int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
@@ -244,6 +251,11 @@ int eh_fc_u8_destroy(eh_fc_plan *plan);
  * in*stride + k - stride - pads. */
 int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
                         const eh_requant *q, void *stream);
+/* Per-channel mode of the deconvolution
+ * (cl_optimized_impls/CLDeconvolutionPerChannelQuantized.cpp:147-176,
+ * cl_kernels/DeconvolutionKernels.cpp:200-249); arguments as eh_conv2d_u8_set_perchannel. */
+int eh_deconv2d_u8_set_perchannel(eh_deconv_plan *plan, const int32_t *multipliers, const int32_t *shifts, int32_t count,
+                                  void *stream);
 int eh_deconv2d_u8_repack(eh_deconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
 int eh_deconv2d_u8_run(eh_deconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
 int eh_deconv2d_u8_destroy(eh_deconv_plan *plan);

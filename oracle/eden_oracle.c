@@ -230,8 +230,9 @@ void eo_conv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *
 
 /* cl_kernels/DepthwiseconvolutionKernels.cpp:1273-1321; weights [C*dm][1][kh][kw],
  * output channel c*dm+d reads input channel c. */
-void eo_dwconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
-                    const eo_conv_shape *s, const eo_quant *q, int32_t *acc_out) {
+static void dw_core(const uint8_t *in, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
+                    const eo_conv_shape *s, const eo_quant *q, const int32_t *multipliers,
+                    const int32_t *shifts, int32_t *acc_out) {
     const int32_t Ho = eo_conv_out_dim(s->h, s->pad_t, s->pad_b, s->kh, s->dil_h, s->stride_h);
     const int32_t Wo = eo_conv_out_dim(s->w, s->pad_l, s->pad_r, s->kw, s->dil_w, s->stride_w);
     const int32_t dm = s->dm > 0 ? s->dm : 1;
@@ -250,17 +251,38 @@ void eo_dwconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, ui
             const uint8_t *src = in + ((int64_t)n * s->c + ic) * s->h * s->w;
             for (int32_t ky = 0; ky < s->kh; ++ky)
                 for (int32_t kx = 0; kx < s->kw; ++kx) {
-                    const int32_t wv = (int32_t)w[((int64_t)oc * s->kh + ky) * s->kw + kx] - q->zp_w;
+                    const int64_t wi = ((int64_t)oc * s->kh + ky) * s->kw + kx;
+                    const int32_t wv = w_is_signed ? (int32_t)((const int8_t *)w)[wi] - q->zp_w
+                                                   : (int32_t)((const uint8_t *)w)[wi] - q->zp_w;
                     accumulate_tap(acc, src, wv, q->zp_in, s->h, s->w, Ho, Wo,
                                    ky * s->dil_h - s->pad_t, kx * s->dil_w - s->pad_l,
                                    s->stride_h, s->stride_w);
                 }
+            eo_quant ql = *q;
+            if (multipliers) {
+                ql.multiplier = multipliers[oc];
+                ql.shift = shifts[oc];
+            }
             uint8_t *dst = out + job * plane;
-            for (int64_t i = 0; i < plane; ++i) dst[i] = eo_requant(acc[i], q);
+            for (int64_t i = 0; i < plane; ++i) dst[i] = eo_requant(acc[i], &ql);
             if (acc_out) memcpy(acc_out + job * plane, acc, sizeof(int32_t) * (size_t)plane);
         }
         free(acc);
     }
+}
+
+void eo_dwconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
+                    const eo_conv_shape *s, const eo_quant *q, int32_t *acc_out) {
+    dw_core(in, w, 0, bias, out, s, q, NULL, NULL, acc_out);
+}
+
+/* cl_kernels/DepthwiseconvolutionKernels.cpp:1323-1371 (int8 weight bytes, the multiplier and
+ * shift of output channel c*dm+d), driven by
+ * cl_optimized_impls/CLDepthwiseConvolutionPerChannelQuantized.cpp:133-153. */
+void eo_dwconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
+                               const eo_conv_shape *s, const eo_quant *q,
+                               const int32_t *multipliers, const int32_t *shifts, int32_t *acc_out) {
+    dw_core(in, w, 1, bias, out, s, q, multipliers, shifts, acc_out);
 }
 
 /* Layout a[m][k], w[n][k], out[m][n]: src/userdriver/gpu/op_test/fullyconnected_test.cpp:93-105.
@@ -327,8 +349,9 @@ void eo_deconv2d_f64(const double *in, const double *w, const double *bias, doub
     }
 }
 
-void eo_deconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
-                    const eo_conv_shape *s, const eo_quant *q, int32_t *acc_out) {
+static void deconv_core(const uint8_t *in, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
+                        const eo_conv_shape *s, const eo_quant *q, const int32_t *multipliers,
+                        const int32_t *shifts, int32_t *acc_out) {
     const int32_t Ho = eo_deconv_out_dim(s->h, s->pad_t, s->pad_b, s->kh, s->stride_h);
     const int32_t Wo = eo_deconv_out_dim(s->w, s->pad_l, s->pad_r, s->kw, s->stride_w);
     const int64_t n_in = (int64_t)s->n * s->c * s->h * s->w;
@@ -340,18 +363,39 @@ void eo_deconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, ui
     double *db = (double *)malloc(sizeof(double) * (size_t)s->cout);
     double *dout = (double *)malloc(sizeof(double) * (size_t)n_out);
     for (int64_t i = 0; i < n_in; ++i) din[i] = (double)((int32_t)in[i] - q->zp_in);
-    for (int64_t i = 0; i < n_w; ++i) dw[i] = (double)((int32_t)w[i] - q->zp_w);
+    for (int64_t i = 0; i < n_w; ++i)
+        dw[i] = (double)((w_is_signed ? (int32_t)((const int8_t *)w)[i] : (int32_t)((const uint8_t *)w)[i]) - q->zp_w);
     for (int32_t i = 0; i < s->cout; ++i) db[i] = bias ? (double)bias[i] : 0.0;
     eo_deconv2d_f64(din, dw, db, dout, s);
     for (int64_t i = 0; i < n_out; ++i) {
         const int32_t acc = (int32_t)dout[i];
-        out[i] = eo_requant(acc, q);
+        eo_quant ql = *q;
+        if (multipliers) {
+            const int32_t oc = (int32_t)((i / ((int64_t)Ho * Wo)) % s->cout);
+            ql.multiplier = multipliers[oc];
+            ql.shift = shifts[oc];
+        }
+        out[i] = eo_requant(acc, &ql);
         if (acc_out) acc_out[i] = acc;
     }
     free(din);
     free(dw);
     free(db);
     free(dout);
+}
+
+void eo_deconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
+                    const eo_conv_shape *s, const eo_quant *q, int32_t *acc_out) {
+    deconv_core(in, w, 0, bias, out, s, q, NULL, NULL, acc_out);
+}
+
+/* cl_kernels/DeconvolutionKernels.cpp:200-249 (the gather with the pair of channel
+ * get_global_id(0) % channels) over int8 weight bytes (:449-454), driven by
+ * cl_optimized_impls/CLDeconvolutionPerChannelQuantized.cpp:147-176. */
+void eo_deconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
+                               const eo_conv_shape *s, const eo_quant *q,
+                               const int32_t *multipliers, const int32_t *shifts, int32_t *acc_out) {
+    deconv_core(in, w, 1, bias, out, s, q, multipliers, shifts, acc_out);
 }
 
 /* Scatter form: col = W^T x A (cl_kernels/DeconvolutionKernels.cpp:24-60), then

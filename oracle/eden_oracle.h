@@ -20,6 +20,11 @@
  *   eo_fc_u8                 pinned: reference KAT, equality with 1x1 conv
  *   eo_deconv2d_u8           pinned: reference KATs (integer data), scatter form == gather form,
  *                                    stride-1 deconv == conv with flipped kernel
+ *   eo_conv2d_u8_perchannel  pinned: the reference's uint8 per-channel KAT
+ *   eo_dwconv2d_u8_perchannel / eo_deconv2d_u8_perchannel
+ *                            pinned by reduction: channel c of the result equals channel c of the per-tensor
+ *                                    function above run on the weight bytes + 128 with weight zero point + 128
+ *                                    and channel c's (multiplier, shift); no reference vector exists for them
  *   eo_nchw2nhwc_u8 / eo_nhwc2nchw_u8  pinned: round trip + index closed form
  *   eo_add_u8 / eo_avgpool_u8           parity unpinned by reference vectors (closed-form checks only)
  */
@@ -81,6 +86,12 @@ void eo_conv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *
                              const int32_t *multipliers, const int32_t *shifts, int32_t *acc);
 void eo_dwconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
                     const eo_conv_shape *s, const eo_quant *q, int32_t *acc);
+void eo_dwconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
+                               const eo_conv_shape *s, const eo_quant *q,
+                               const int32_t *multipliers, const int32_t *shifts, int32_t *acc);
+void eo_deconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
+                               const eo_conv_shape *s, const eo_quant *q,
+                               const int32_t *multipliers, const int32_t *shifts, int32_t *acc);
 void eo_fc_u8(const uint8_t *a, const uint8_t *w, const int32_t *bias, uint8_t *out,
               int32_t m, int32_t k, int32_t n, const eo_quant *q, int32_t *acc);
 /* gather form (each output pixel sums its contributing taps) */

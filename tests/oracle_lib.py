@@ -57,6 +57,8 @@ def _load():
         "eo_conv2d_u8": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp]),
         "eo_conv2d_u8_perchannel": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp, vp, vp]),
         "eo_dwconv2d_u8": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp]),
+        "eo_dwconv2d_u8_perchannel": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp, vp, vp]),
+        "eo_deconv2d_u8_perchannel": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp, vp, vp]),
         "eo_fc_u8": (None, [vp, vp, vp, vp, i32, i32, i32, P(Quant), vp]),
         "eo_deconv2d_u8": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp]),
         "eo_deconv2d_u8_scatter": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp]),
@@ -182,6 +184,24 @@ def dwconv2d(x, w, bias, s, q, want_acc=False):
     acc = np.zeros(out.shape, np.int32) if want_acc else None
     lib.eo_dwconv2d_u8(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), C.byref(s), C.byref(q), _ptr(acc))
     return (out, acc) if want_acc else out
+
+
+def dwconv2d_perchannel(x, w_i8, bias, s, q, multipliers, shifts):
+    x, w, bias = _c(x, np.uint8), _c(w_i8, np.int8), _c(bias, np.int32)
+    m, sh = _c(multipliers, np.int32), _c(shifts, np.int32)
+    ho, wo = conv_out_hw(s)
+    out = np.zeros((s.n, s.c * max(s.dm, 1), ho, wo), np.uint8)
+    lib.eo_dwconv2d_u8_perchannel(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), C.byref(s), C.byref(q), _ptr(m), _ptr(sh), None)
+    return out
+
+
+def deconv2d_perchannel(x, w_i8, bias, s, q, multipliers, shifts):
+    x, w, bias = _c(x, np.uint8), _c(w_i8, np.int8), _c(bias, np.int32)
+    m, sh = _c(multipliers, np.int32), _c(shifts, np.int32)
+    ho, wo = deconv_out_hw(s)
+    out = np.zeros((s.n, s.cout, ho, wo), np.uint8)
+    lib.eo_deconv2d_u8_perchannel(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), C.byref(s), C.byref(q), _ptr(m), _ptr(sh), None)
+    return out
 
 
 def fc(a, w, bias, q, want_acc=False):

@@ -88,3 +88,105 @@ def test_perchannel_conv_matches_oracle(case, layout):
     want2 = O.conv2d_perchannel(x, w, b, s, oq2, np.full(s.cout, mults[0], np.int32), np.full(s.cout, shifts[0], np.int32))
     _, uniform = gpu_conv_perchannel(x, w, b, s, q2, mults, shifts, layout)
     assert np.array_equal(uniform, want2)
+
+
+def _pairs_for(s_in, w_scales, s_out):
+    q, mults, shifts = eden.make_requant_perchannel(s_in, 117, w_scales, s_out, 131, eden.ACT_NONE, False)
+    return q, mults, shifts
+
+
+DW_PC_CASES = [
+    dict(n=2, c=32, h=15, w=14, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),              # 3x3 tile kernel, stride 1
+    dict(n=2, c=24, h=15, w=17, cout=24, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),              # 3x3 tile kernel, stride 2
+    dict(n=1, c=16, h=12, w=12, cout=16, kh=5, kw=5, stride=(1, 1), pad=(2, 2, 2, 2)),              # four-channel kernel
+    dict(n=1, c=16, h=12, w=12, cout=16, kh=3, kw=3, stride=(1, 1), pad=(2, 2, 2, 2), dil=(2, 2)),  # four-channel kernel, 3x3 dilated
+    dict(n=2, c=5, h=9, w=8, cout=10, kh=3, kw=3, stride=(2, 1), pad=(1, 0, 1, 1), dm=2),           # one output per thread
+]
+
+
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("case", DW_PC_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_perchannel_depthwise_matches_oracle(case, layout):
+    print("per-channel depthwise", case, layout, flush=True)
+    s = O.conv_shape(**case)
+    cout = s.c * max(s.dm, 1)
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 21)
+    w = (synth.fill_u8((cout, 1, s.kh, s.kw), SEED + 22).astype(np.int16) - 128).astype(np.int8)
+    b = synth.fill_i32((cout,), SEED + 23, -500, 500)
+    w_scales = (0.002 * (1.0 + 29.0 * synth.fill_u8((cout,), SEED + 24) / 255.0)).astype(np.float32)
+    s_out = float(0.02 * float(w_scales.max()) * 74.0 * 74.0 * np.sqrt(s.kh * s.kw) / 60.0)
+    for zp_w in (0, -9):
+        q, mults, shifts = _pairs_for(0.02, w_scales, s_out)
+        q.zp_w = zp_w
+        oq = O.raw_quant(zp_in=117, zp_w=zp_w, zp_out=131)
+        want = O.dwconv2d_perchannel(x, w, b, s, oq, mults, shifts)
+        desc = eden.conv_desc(s.n, s.c, s.h, s.w, cout, s.kh, s.kw, (s.stride_h, s.stride_w),
+                              (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), 1, max(s.dm, 1), layout,
+                              eden.W_OIHW | eden.W_SIGNED)
+        ho, wo = O.conv_out_hw(s)
+        x_dev = x if layout == eden.NCHW else x.transpose(0, 2, 3, 1)
+        d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+        d_o = eden.DeviceBuffer(nbytes=s.n * cout * ho * wo)
+        plan = eden.DwConvPlan(desc, d_w, d_b, q)
+        plan.set_perchannel(mults, shifts)
+        plan.run(d_x, d_o, q)
+        got = d_o.download((s.n, cout, ho, wo)) if layout == eden.NCHW else d_o.download((s.n, ho, wo, cout)).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, want), int((got != want).sum())
+        assert want.std() > 4
+        # back to one pair: int8 weights, per-tensor requant
+        plan.set_perchannel(None, None)
+        q1 = eden.Requant(117, zp_w, 131, int(mults[1]), int(shifts[1]), 0, 255)
+        plan.run(d_x, d_o, q1)
+        got = d_o.download((s.n, cout, ho, wo)) if layout == eden.NCHW else d_o.download((s.n, ho, wo, cout)).transpose(0, 3, 1, 2)
+        want = O.dwconv2d_perchannel(x, w, b, s, oq, np.full(cout, mults[1], np.int32), np.full(cout, shifts[1], np.int32))
+        assert np.array_equal(got, want)
+        plan.destroy()
+
+
+DECONV_PC_CASES = [
+    dict(n=2, c=64, h=14, w=14, cout=32, kh=2, kw=2, stride=(2, 2)),                       # four equal phases in one launch
+    dict(n=1, c=24, h=7, w=9, cout=40, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),       # unequal phases
+    dict(n=2, c=12, h=6, w=5, cout=8, kh=4, kw=4, stride=(2, 2), pad=(1, 1, 1, 1), groups=2),
+    dict(n=1, c=16, h=8, w=8, cout=16, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("case", DECONV_PC_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_perchannel_deconv_matches_oracle(case, layout):
+    print("per-channel deconvolution", case, layout, flush=True)
+    s = O.conv_shape(**case)
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 31)
+    w = (synth.fill_u8((s.c, s.cout // s.groups, s.kh, s.kw), SEED + 32).astype(np.int16) - 128).astype(np.int8)
+    b = synth.fill_i32((s.cout,), SEED + 33, -500, 500)
+    w_scales = (0.002 * (1.0 + 29.0 * synth.fill_u8((s.cout,), SEED + 34) / 255.0)).astype(np.float32)
+    taps = max(1, (s.kh // s.stride_h) * (s.kw // s.stride_w))
+    s_out = float(0.02 * float(w_scales.max()) * 74.0 * 74.0 * np.sqrt(taps * s.c // s.groups) / 60.0)
+    q, mults, shifts = _pairs_for(0.02, w_scales, s_out)
+    oq = O.raw_quant(zp_in=117, zp_w=0, zp_out=131)
+    want = O.deconv2d_perchannel(x, w, b, s, oq, mults, shifts)
+    ho, wo = O.deconv_out_hw(s)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, (s.stride_h, s.stride_w),
+                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (1, 1), s.groups, 1, layout, eden.W_IOHW | eden.W_SIGNED)
+    x_dev = x if layout == eden.NCHW else x.transpose(0, 2, 3, 1)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+    d_o = eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
+    plan = eden.DeconvPlan(desc, d_w, d_b, q)
+    plan.set_perchannel(mults, shifts)
+    plan.run(d_x, d_o, q)
+    got = d_o.download((s.n, s.cout, ho, wo)) if layout == eden.NCHW else d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+    plan.destroy()
+    assert np.array_equal(got, want), int((got != want).sum())
+    assert want.std() > 4
+
+
+def test_perchannel_argument_errors():
+    desc = eden.conv_desc(1, 8, 6, 6, 8, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, 1, eden.NHWC, eden.W_OIHW | eden.W_SIGNED)
+    w = np.zeros((8, 1, 3, 3), np.int8)
+    q = eden.Requant(0, 0, 0, 1 << 30, -3, 0, 255)
+    plan = eden.DwConvPlan(desc, eden.DeviceBuffer(host=w), None, q)
+    with pytest.raises(eden.EdenHipError):
+        plan.set_perchannel(np.ones(7, np.int32), np.zeros(7, np.int32))       # wrong count
+    with pytest.raises(eden.EdenHipError):
+        plan.set_perchannel(np.full(8, -1, np.int32), np.zeros(8, np.int32))   # negative multiplier
+    plan.destroy()

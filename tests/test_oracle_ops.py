@@ -332,3 +332,39 @@ def test_avgpool_closed_forms():
     # padded window counts only in-image taps
     o = O.avgpool(x, 3, 3, stride=(1, 1), pad=(1, 1, 1, 1))
     assert o[0, 0, 0, 0] == (0 + 1 + 4 + 5 + 2) // 4
+
+
+def _perchannel_pairs(rng, cout):
+    mults = rng.integers(1 << 30, (1 << 31) - 1, cout).astype(np.int32)
+    shifts = rng.integers(-12, -4, cout).astype(np.int32)
+    return mults, shifts
+
+
+@pytest.mark.parametrize("kind", ["conv", "dw", "deconv"])
+def test_perchannel_forms_reduce_to_the_per_tensor_functions(kind):
+    """Channel c of a per-channel result is channel c of the pinned per-tensor function run on the same weights
+    read as uint8 (byte + 128, zero point + 128) with channel c's multiplier and shift."""
+    rng = np.random.default_rng(77 + len(kind))
+    if kind == "dw":
+        s = O.conv_shape(2, 5, 9, 8, 10, 3, 3, stride=(2, 1), pad=(1, 0, 1, 1), dm=2)
+        w_shape, fn, fn_pc = (10, 1, 3, 3), O.dwconv2d, O.dwconv2d_perchannel
+    elif kind == "deconv":
+        s = O.conv_shape(2, 6, 5, 4, 8, 3, 3, stride=(2, 2), pad=(1, 0, 1, 0), groups=2)
+        w_shape, fn, fn_pc = (6, 4, 3, 3), O.deconv2d, O.deconv2d_perchannel
+    else:
+        s = O.conv_shape(2, 6, 7, 6, 8, 3, 2, stride=(1, 2), pad=(1, 1, 0, 1), groups=2)
+        w_shape, fn, fn_pc = (8, 3, 3, 2), O.conv2d, O.conv2d_perchannel
+    cout = 10 if kind == "dw" else 8
+    x = rng.integers(0, 256, (s.n, s.c, s.h, s.w)).astype(np.uint8)
+    w = rng.integers(-128, 128, w_shape).astype(np.int8)
+    bias = rng.integers(-3000, 3000, cout).astype(np.int32)
+    mults, shifts = _perchannel_pairs(rng, cout)
+    for zp_w in (0, -7):
+        q = O.raw_quant(zp_in=101, zp_w=zp_w, zp_out=120, act_min=3, act_max=250)
+        got = fn_pc(x, w, bias, s, q, mults, shifts)
+        assert got.std() > 10
+        w_u8 = (w.astype(np.int16) + 128).astype(np.uint8)
+        for c in range(cout):
+            qc = O.raw_quant(zp_in=101, zp_w=zp_w + 128, zp_out=120, multiplier=int(mults[c]), shift=int(shifts[c]),
+                             act_min=3, act_max=250)
+            assert np.array_equal(got[:, c], fn(x, w_u8, bias, s, qc)[:, c]), (kind, c)
