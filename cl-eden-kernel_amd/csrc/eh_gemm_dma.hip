@@ -402,30 +402,35 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
         }
         // whole tiles with 16-byte aligned rows (the usual case) store without any per-store test
         const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-        auto emit = [&](auto checked_c, auto fast_c) {
+        auto emit = [&](auto checked_c, auto fast_c, auto pc_c) {
             constexpr bool checked = decltype(checked_c)::value;
             constexpr int fast = decltype(fast_c)::value;
+            constexpr bool pc = decltype(pc_c)::value;  // one multiplier and shift per channel
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const int nl = wn * WTN + j * 32 + fhalf * 16, n = n0 + nl;  // this lane's 16 consecutive channels
                 int4 bb[4];
 #pragma unroll
                 for (int g = 0; g < 4; ++g) bb[g] = *reinterpret_cast<const int4 *>(bias_s + nl + g * 4);
+                int4 cm[pc ? 4 : 1], cs[pc ? 4 : 1];
+                if constexpr (pc) {  // the arrays are padded past the last channel block
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        cm[g] = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + g * 4);
+                        cs[g] = *reinterpret_cast<const int4 *>(rq.pc_shift + n + g * 4);
+                    }
+                }
 #pragma unroll
                 for (int i = 0; i < FM; ++i) {
                     uint32_t packed[4];
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
                         uint32_t o0, o1, o2, o3;
-                        if (checked && rq.pc_multiplier) {  // per-channel parameters (always the checked path)
-                            const int32_t *pm = rq.pc_multiplier + n + g * 4;
-                            const int4 cm = make_int4(pm[0], pm[1], pm[2], pm[3]);
-                            const int32_t *ps = rq.pc_shift + n + g * 4;
-                            const int4 cs = make_int4(ps[0], ps[1], ps[2], ps[3]);
-                            o0 = requant_u8_channel(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], cm.x, cs.x, rq);
-                            o1 = requant_u8_channel(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], cm.y, cs.y, rq);
-                            o2 = requant_u8_channel(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], cm.z, cs.z, rq);
-                            o3 = requant_u8_channel(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], cm.w, cs.w, rq);
+                        if constexpr (pc) {
+                            o0 = requant_u8_channel(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], cm[g].x, cs[g].x, rq);
+                            o1 = requant_u8_channel(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], cm[g].y, cs[g].y, rq);
+                            o2 = requant_u8_channel(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], cm[g].z, cs[g].z, rq);
+                            o3 = requant_u8_channel(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], cm[g].w, cs[g].w, rq);
                         } else {
                             o0 = requant_u8_as<fast>(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], rq);
                             o1 = requant_u8_as<fast>(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], rq);
@@ -452,13 +457,15 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
             }
         };
         // edge tiles and unusual requantization parameters take the general code
-        if (rq.fast && aligned16 && m0 + BM <= p.m && n0 + BN <= p.n) {
+        if (rq.pc_multiplier) {
+            emit(std::true_type{}, std::integral_constant<int, 0>{}, std::true_type{});
+        } else if (rq.fast && aligned16 && m0 + BM <= p.m && n0 + BN <= p.n) {
             if (rq.fast == 2)
-                emit(std::false_type{}, std::integral_constant<int, 2>{});
+                emit(std::false_type{}, std::integral_constant<int, 2>{}, std::false_type{});
             else
-                emit(std::false_type{}, std::integral_constant<int, 1>{});
+                emit(std::false_type{}, std::integral_constant<int, 1>{}, std::false_type{});
         } else {
-            emit(std::true_type{}, std::integral_constant<int, 0>{});
+            emit(std::true_type{}, std::integral_constant<int, 0>{}, std::false_type{});
         }
     } else {
         // the WGK partial tiles meet in LDS: [wk][pixel row][channel], rows padded so that
