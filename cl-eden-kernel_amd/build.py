@@ -1,6 +1,7 @@
 """Builds libedenhip.so (HIP kernels + C ABI) and libedenhip_ud.so's test driver
 for gfx950 with hipcc.  Everything is built in-tree; nothing is installed."""
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -19,14 +20,47 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-W
              "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
 
 
+RESOURCES = os.path.join(OBJ, "kernel_resources.txt")
+
+
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # the host pass of hipcc does not know the packed-fp32 feature and says so once per file: harmless
-    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    lines = [l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l]
+    remarks, rest, after_remark = [], [], False
+    for l in lines:
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            remarks.append(l)
+            after_remark = True
+        elif after_remark and re.match(r"^\s*(\d+\s*)?\|", l):
+            pass  # the source line and caret the compiler prints under a remark
+        else:
+            rest.append(l)
+            after_remark = False
+    out = "\n".join(rest)
     if r.returncode != 0:
         raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
     if out.strip():
         print(out)
+    return remarks
+
+
+def _resource_table(remarks):
+    """'kernel vgprs agprs scratch_bytes_per_lane waves_per_simd' lines from the compiler's resource remarks"""
+    rows, cur = [], None
+    for l in remarks:
+        m = re.search(r"Function Name: (\S+)", l)
+        if m:
+            cur = {"name": m.group(1)}
+            rows.append(cur)
+            continue
+        for key, pat in (("vgprs", r" VGPRs: (\d+)"), ("agprs", r"AGPRs: (\d+)"), ("scratch", r"ScratchSize \[bytes/lane\]: (\d+)"),
+                         ("occupancy", r"Occupancy \[waves/SIMD\]: (\d+)")):
+            m = re.search(pat, l)
+            if m and cur is not None:
+                cur[key] = int(m.group(1))
+    return ["%s %d %d %d %d" % (r["name"], r.get("vgprs", -1), r.get("agprs", -1), r.get("scratch", -1), r.get("occupancy", -1))
+            for r in rows]
 
 
 def build_lib(jobs=8):
@@ -34,8 +68,14 @@ def build_lib(jobs=8):
     srcs = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
     objs = [os.path.join(OBJ, f[:-4] + ".o") for f in srcs]
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        list(ex.map(lambda so: _run([HIPCC, *HIP_FLAGS, "-c", os.path.join(CSRC, so[0]), "-o", so[1]]), zip(srcs, objs)))
+        remarks = list(ex.map(lambda so: _run([HIPCC, *HIP_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c",
+                                               os.path.join(CSRC, so[0]), "-o", so[1]]), zip(srcs, objs)))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
+    # registers, spill bytes and occupancy of every kernel, for the test that guards the hot kernels' budgets
+    with open(RESOURCES, "w") as f:
+        for src, r in zip(srcs, remarks):
+            for row in _resource_table(r):
+                f.write(src + " " + row + "\n")
     return LIB
 
 
