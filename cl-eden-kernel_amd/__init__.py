@@ -17,6 +17,7 @@ ACT_NONE, ACT_RELU, ACT_RELU1, ACT_RELU6 = 0, 1, 2, 3
 NCHW, NHWC = 0, 1
 W_OIHW, W_OHWI, W_IOHW = 0, 1, 2
 W_SIGNED = 0x100  # or-ed into a convolution's weight layout: int8 weight bytes
+IO_SIGNED = 0x200  # or-ed into a convolution's tensor layout: int8 input and output (zero points and range in [-128, 127])
 
 
 class EdenHipError(RuntimeError):
@@ -55,6 +56,9 @@ EXPORTS = {
     "eh_quantize_multiplier": (None, [C.c_double, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "eh_conv_multiplier": (C.c_int, [C.c_float] * 4 + [C.POINTER(C.c_double)]),
     "eh_act_range_u8": (None, [C.c_int, C.c_float, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "eh_act_range_s8": (None, [C.c_int, C.c_float, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "eh_make_requant_s8": (None, [C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_float, C.c_float, C.c_int32,
+                                  C.c_int, C.c_int, C.POINTER(Requant)]),
     "eh_requant_apply": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]),
     "eh_make_requant": (None, [C.c_float, C.c_int32, C.c_float, C.c_int32, C.c_float, C.c_float, C.c_int32,
                                C.c_int, C.c_int, C.POINTER(Requant)]),
@@ -99,6 +103,8 @@ EXPORTS = {
     "eh_dwconv2d_u8_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
     "eh_dwconv2d_u8_destroy": (C.c_int, [C.c_void_p]),
     "eh_fc_u8_plan": (C.c_int, [C.POINTER(C.c_void_p), C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
+                                C.POINTER(Requant), C.c_void_p]),
+    "eh_fc_q8_plan": (C.c_int, [C.POINTER(C.c_void_p), C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
                                 C.POINTER(Requant), C.c_void_p]),
     "eh_fc_u8_repack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
     "eh_fc_u8_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
@@ -151,6 +157,15 @@ def make_requant(s_in, zp_in, s_w, zp_w, s_out, zp_out, act=ACT_NONE, act_enable
         s_bias = float(np.float32(s_in) * np.float32(s_w))
     q = Requant()
     load().eh_make_requant(s_in, zp_in, s_w, zp_w, s_bias, s_out, zp_out, act, int(act_enabled), C.byref(q))
+    return q
+
+
+def make_requant_s8(s_in, zp_in, s_w, zp_w, s_out, zp_out, act=ACT_NONE, act_enabled=False, s_bias=None):
+    """INT8 precision (IO_SIGNED plans): zero points and the activation range are int8 values."""
+    if s_bias is None:
+        s_bias = float(np.float32(s_in) * np.float32(s_w))
+    q = Requant()
+    load().eh_make_requant_s8(s_in, zp_in, s_w, zp_w, s_bias, s_out, zp_out, act, int(act_enabled), C.byref(q))
     return q
 
 
@@ -317,10 +332,14 @@ class DeconvPlan(_Plan):
 class FcPlan(_Plan):
     _kind = "fc"
 
-    def __init__(self, m, k, n, d_w, d_b, q, stream=None):
+    def __init__(self, m, k, n, d_w, d_b, q, stream=None, flags=0):
+        """flags: any of W_SIGNED | IO_SIGNED"""
         super().__init__()
         self.m, self.k, self.n = m, k, n
-        check(load().eh_fc_u8_plan(C.byref(self.handle), m, k, n, d_w.ptr, d_b.ptr if d_b else None, C.byref(q), stream))
+        if flags:
+            check(load().eh_fc_q8_plan(C.byref(self.handle), m, k, n, flags, d_w.ptr, d_b.ptr if d_b else None, C.byref(q), stream))
+        else:
+            check(load().eh_fc_u8_plan(C.byref(self.handle), m, k, n, d_w.ptr, d_b.ptr if d_b else None, C.byref(q), stream))
 
 
 class Event:

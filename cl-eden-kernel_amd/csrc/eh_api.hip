@@ -28,13 +28,32 @@ int hip_fail(hipError_t e, const char *what) {
     return EH_DEVICE_FAILURE;
 }
 
-int check_requant(const eh_requant *q, bool signed_weights) {
+// int8 tensors are computed as their uint8 equivalents: every stored value, zero point and clamp bound + 128
+// (SIGNED_TO_UNSIGNED in gpu/operators/cl_kernels/DepthwiseconvolutionKernels.cpp:2410-2411, and the zero points
+// + 128 of cl_optimized_impls/CLDepthwiseConvolutionQuantized.cpp:207-211)
+static eh_requant io_as_uint8(const eh_requant &q) {
+    eh_requant u = q;
+    u.zp_in += 128;
+    u.zp_out += 128;
+    u.act_min += 128;
+    u.act_max += 128;
+    return u;
+}
+
+int check_requant(const eh_requant *q, bool signed_weights, bool signed_io) {
     EH_REQUIRE(q != nullptr, "requant parameters are null");
     if (signed_weights) {
         EH_REQUIRE(q->zp_w >= -128 && q->zp_w <= 127, "int8 weight zero point %d outside [-128, 127]", q->zp_w);
         eh_requant u = *q;
         u.zp_w += 128;
-        return check_requant(&u, false);
+        return check_requant(&u, false, signed_io);
+    }
+    if (signed_io) {
+        EH_REQUIRE(q->zp_in >= -128 && q->zp_in <= 127, "int8 input zero point %d outside [-128, 127]", q->zp_in);
+        EH_REQUIRE(q->act_min >= -128 && q->act_max <= 127 && q->act_min <= q->act_max, "int8 activation range [%d, %d] invalid",
+                   q->act_min, q->act_max);
+        const eh_requant u = io_as_uint8(*q);
+        return check_requant(&u, false, false);
     }
     EH_REQUIRE(q->multiplier >= 0, "requant multiplier %d is negative", q->multiplier);
     EH_REQUIRE(q->shift >= -31 && q->shift <= 30, "requant shift %d outside [-31, 30]", q->shift);
@@ -190,6 +209,7 @@ struct GemmOp {
     // int8 weights (value = byte as signed; zp_w is then an int8 zero point) and one multiplier / shift per
     // output channel instead of the requant's single pair
     bool w_signed = false;
+    bool io_signed = false;  // input and output tensors hold int8 values
     int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;
 
     int zp_w_u8(const eh_requant &r) const { return r.zp_w + (w_signed ? 128 : 0); }  // zero point of the equivalent uint8 weights
@@ -244,14 +264,16 @@ struct GemmOp {
         return EH_OK;
     }
 
-    int refold(const eh_requant &nq, hipStream_t stream) {
-        if (folded_valid && nq.zp_in == q.zp_in && nq.zp_w == q.zp_w) {  // (w_signed is fixed per plan)
+    // `caller_q` as the caller states it; `q` keeps the uint8-equivalent input/output side
+    int refold(const eh_requant &caller_q, hipStream_t stream) {
+        const eh_requant nq = io_signed ? io_as_uint8(caller_q) : caller_q;
+        if (folded_valid && nq.zp_in == q.zp_in && nq.zp_w == q.zp_w) {  // (w_signed and io_signed are fixed per plan)
             q = nq;
             return EH_OK;
         }
         for (auto &g : parts) {
             int rc = launch_fold_bias(bias_copy + g.bias_base, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, zp_w_u8(nq),
-                                      fillbuf, stream);
+                                      fillbuf, io_signed ? 0x80 : 0, stream);
             if (rc) return rc;
         }
         q = nq;
@@ -261,7 +283,7 @@ struct GemmOp {
 
     int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream) {
         EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
-        int rc = check_requant(nq, w_signed);
+        int rc = check_requant(nq, w_signed, io_signed);
         if (rc) return rc;
         if ((rc = refold(*nq, stream))) return rc;
         const uint8_t *in = static_cast<const uint8_t *>(input);
@@ -283,7 +305,9 @@ struct GemmOp {
             p.fillbuf = fillbuf;
             p.out = out + g.bias_base;
             p.zw = zp_w_u8(q) - 128;
-            p.fill = (uint32_t)q.zp_in * 0x01010101u;
+            p.out_xor = io_signed ? 0x80808080u : 0u;
+            p.a_xor = 0x80808080u ^ p.out_xor;
+            p.fill = ((uint32_t)q.zp_in * 0x01010101u) ^ p.out_xor;
             p.rq = make_requant_dev(q);
             if (pc_multiplier) {
                 p.rq.pc_multiplier = pc_multiplier + g.bias_base;
@@ -338,7 +362,7 @@ struct eh_dwconv_plan {
     int32_t *bias_folded = nullptr;
     eh_requant q{};
     bool packed_valid = false;
-    bool w_signed = false;
+    bool w_signed = false, io_signed = false;
     int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;  // [cout + 4] once per-channel pairs are set
 };
 
@@ -387,9 +411,9 @@ int eh_conv_multiplier(float input_scale, float filter_scale, float bias_scale, 
     return EH_OK;
 }
 
-void eh_act_range_u8(int activation, float scale, int32_t zero_point, int32_t *act_min, int32_t *act_max) {
+static void act_range(int activation, float scale, int32_t zero_point, int32_t lo, int32_t hi, int32_t *act_min,
+                      int32_t *act_max) {
     auto quantize = [scale, zero_point](float f) { return zero_point + (int32_t)round((double)(f / scale)); };
-    int32_t lo = 0, hi = 255;
     if (activation == EH_ACT_RELU) {
         lo = quantize(0.0f) > lo ? quantize(0.0f) : lo;
     } else if (activation == EH_ACT_RELU6) {
@@ -401,6 +425,22 @@ void eh_act_range_u8(int activation, float scale, int32_t zero_point, int32_t *a
     }
     *act_min = lo;
     *act_max = hi;
+}
+
+void eh_act_range_u8(int activation, float scale, int32_t zero_point, int32_t *act_min, int32_t *act_max) {
+    act_range(activation, scale, zero_point, 0, 255, act_min, act_max);
+}
+
+void eh_act_range_s8(int activation, float scale, int32_t zero_point, int32_t *act_min, int32_t *act_max) {
+    act_range(activation, scale, zero_point, -128, 127, act_min, act_max);
+}
+
+void eh_make_requant_s8(float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp, float bias_scale,
+                        float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out) {
+    eh_make_requant(input_scale, input_zp, filter_scale, filter_zp, bias_scale, output_scale, output_zp, activation, 0, out);
+    out->act_min = -128;
+    out->act_max = 127;
+    if (activation_enabled) eh_act_range_s8(activation, output_scale, output_zp, &out->act_min, &out->act_max);
 }
 
 void eh_make_requant(float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp, float bias_scale,
@@ -687,13 +727,15 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
                       const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan pointer");
     *plan = nullptr;
-    int rc = check_desc_common(desc);
-    if (rc) return rc;
-    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0;
+    EH_REQUIRE(desc != nullptr, "descriptor is null");
+    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
     eh_conv_desc plain = *desc;
     plain.weight_layout &= ~EH_W_SIGNED;
+    plain.layout &= ~EH_IO_SIGNED;
     desc = &plain;
-    if ((rc = check_requant(q, w_signed))) return rc;
+    int rc = check_desc_common(desc);
+    if (rc) return rc;
+    if ((rc = check_requant(q, w_signed, io_signed))) return rc;
     EH_REQUIRE(desc->dil_h > 0 && desc->dil_w > 0, "bad dilation");
     EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
                "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
@@ -705,6 +747,7 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
     pl->op.w_signed = w_signed;
+    pl->op.io_signed = io_signed;
     if (desc->n > 0) {
         rc = conv_plan_build(pl, desc, as_stream(stream));
         if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
@@ -728,7 +771,7 @@ int eh_conv2d_u8_set_perchannel(eh_conv_plan *plan, const int32_t *multipliers, 
 
 int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q, plan->op.w_signed);
+    int rc = check_requant(q, plan->op.w_signed, plan->op.io_signed);
     if (rc) return rc;
     if (plan->d.n == 0) return EH_OK;
     if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
@@ -737,7 +780,7 @@ int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias
 
 int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed);  // zero-size early-out, as CLConvolution::execute does
+    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);  // zero-size early-out, as CLConvolution::execute does
     return plan->op.run(input, output, q, as_stream(stream));
 }
 
@@ -753,11 +796,18 @@ int eh_conv2d_u8_destroy(eh_conv_plan *plan) {
 
 int eh_fc_u8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, const void *weight, const void *bias,
                   const eh_requant *q, void *stream) {
+    return eh_fc_q8_plan(plan, m, k, n, 0, weight, bias, q, stream);
+}
+
+int eh_fc_q8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, int32_t flags, const void *weight, const void *bias,
+                  const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan pointer");
     *plan = nullptr;
     EH_REQUIRE(m >= 0 && k > 0 && n > 0, "bad extents m=%d k=%d n=%d", m, k, n);
     EH_REQUIRE((int64_t)m * k < (1ll << 31), "input larger than 2 GiB is not supported");
-    int rc = check_requant(q);
+    EH_REQUIRE((flags & ~(EH_W_SIGNED | EH_IO_SIGNED)) == 0, "unknown flags 0x%x", flags);
+    const bool w_signed = (flags & EH_W_SIGNED) != 0, io_signed = (flags & EH_IO_SIGNED) != 0;
+    int rc = check_requant(q, w_signed, io_signed);
     if (rc) return rc;
     eh_fc_plan *pl = new (std::nothrow) eh_fc_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
@@ -765,6 +815,8 @@ int eh_fc_u8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, const void
     pl->k = k;
     pl->n = n;
     GemmOp &op = pl->op;
+    op.w_signed = w_signed;
+    op.io_signed = io_signed;
     op.cout = n;
     op.layout = EH_NHWC;
     hipStream_t s = as_stream(stream);
@@ -821,7 +873,7 @@ int eh_fc_u8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, const void
 
 int eh_fc_u8_repack(eh_fc_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q);
+    int rc = check_requant(q, plan->op.w_signed, plan->op.io_signed);
     if (rc) return rc;
     if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
     return plan->op.refold(*q, as_stream(stream));
@@ -829,7 +881,7 @@ int eh_fc_u8_repack(eh_fc_plan *plan, const void *weight, const void *bias, cons
 
 int eh_fc_u8_run(eh_fc_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    if (plan->m == 0) return check_requant(q);
+    if (plan->m == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);
     return plan->op.run(input, output, q, as_stream(stream));
 }
 
@@ -940,13 +992,15 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
                         const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan pointer");
     *plan = nullptr;
-    int rc = check_desc_common(desc);
-    if (rc) return rc;
-    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0;
+    EH_REQUIRE(desc != nullptr, "descriptor is null");
+    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
     eh_conv_desc plain = *desc;
     plain.weight_layout &= ~EH_W_SIGNED;
+    plain.layout &= ~EH_IO_SIGNED;
     desc = &plain;
-    if ((rc = check_requant(q, w_signed))) return rc;
+    int rc = check_desc_common(desc);
+    if (rc) return rc;
+    if ((rc = check_requant(q, w_signed, io_signed))) return rc;
     EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
                "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
     EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->weight_layout == EH_W_OHWI, "bad deconvolution weight layout %d",
@@ -956,6 +1010,7 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
     pl->op.w_signed = w_signed;
+    pl->op.io_signed = io_signed;
     if (desc->n > 0) {
         rc = deconv_plan_build(pl, desc, as_stream(stream));
         if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
@@ -979,7 +1034,7 @@ int eh_deconv2d_u8_set_perchannel(eh_deconv_plan *plan, const int32_t *multiplie
 
 int eh_deconv2d_u8_repack(eh_deconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q, plan->op.w_signed);
+    int rc = check_requant(q, plan->op.w_signed, plan->op.io_signed);
     if (rc) return rc;
     if (plan->d.n == 0) return EH_OK;
     if ((rc = plan->op.set_weights(weight, bias, as_stream(stream)))) return rc;
@@ -988,7 +1043,7 @@ int eh_deconv2d_u8_repack(eh_deconv_plan *plan, const void *weight, const void *
 
 int eh_deconv2d_u8_run(eh_deconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed);
+    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);
     return plan->op.run(input, output, q, as_stream(stream));
 }
 
@@ -1022,7 +1077,8 @@ static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bi
     return EH_OK;
 }
 
-static int dw_refold(eh_dwconv_plan *pl, const eh_requant &q, hipStream_t stream) {
+static int dw_refold(eh_dwconv_plan *pl, const eh_requant &caller_q, hipStream_t stream) {
+    const eh_requant q = pl->io_signed ? io_as_uint8(caller_q) : caller_q;  // pl->q: the uint8-equivalent input/output side
     if (!(pl->packed_valid && q.zp_in == pl->q.zp_in && q.zp_w == pl->q.zp_w)) {
         int rc = launch_dw_pack(pl->w_copy, pl->bias_copy, pl->w_pair, pl->bias_folded, pl->cout, pl->taps, q.zp_in,
                                 q.zp_w, pl->w_signed ? 1 : 0, stream);
@@ -1037,13 +1093,15 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
                         const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan pointer");
     *plan = nullptr;
-    int rc = check_desc_common(desc);
-    if (rc) return rc;
-    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0;
+    EH_REQUIRE(desc != nullptr, "descriptor is null");
+    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
     eh_conv_desc plain = *desc;
     plain.weight_layout &= ~EH_W_SIGNED;
+    plain.layout &= ~EH_IO_SIGNED;
     desc = &plain;
-    if ((rc = check_requant(q, w_signed))) return rc;
+    int rc = check_desc_common(desc);
+    if (rc) return rc;
+    if ((rc = check_requant(q, w_signed, io_signed))) return rc;
     EH_REQUIRE(desc->dil_h > 0 && desc->dil_w > 0, "bad dilation");
     EH_REQUIRE(desc->depth_multiplier > 0, "bad depth multiplier %d", desc->depth_multiplier);
     EH_REQUIRE(desc->cout == desc->c * desc->depth_multiplier, "depthwise cout %d != c %d * depth multiplier %d", desc->cout,
@@ -1053,6 +1111,7 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
     pl->w_signed = w_signed;
+    pl->io_signed = io_signed;
     pl->ho = eh_conv_out_dim(desc->h, desc->pad_t, desc->pad_b, desc->kh, desc->dil_h, desc->stride_h);
     pl->wo = eh_conv_out_dim(desc->w, desc->pad_l, desc->pad_r, desc->kw, desc->dil_w, desc->stride_w);
     pl->cout = desc->cout;
@@ -1106,7 +1165,7 @@ int eh_dwconv2d_u8_set_perchannel(eh_dwconv_plan *plan, const int32_t *multiplie
 
 int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q, plan->w_signed);
+    int rc = check_requant(q, plan->w_signed, plan->io_signed);
     if (rc) return rc;
     if ((rc = dw_set_weights(plan, weight, bias, as_stream(stream)))) return rc;
     return dw_refold(plan, *q, as_stream(stream));
@@ -1114,7 +1173,7 @@ int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *
 
 int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q, plan->w_signed);
+    int rc = check_requant(q, plan->w_signed, plan->io_signed);
     if (rc) return rc;
     const eh_conv_desc &d = plan->d;
     if (d.n == 0) return EH_OK;
@@ -1144,10 +1203,11 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     p.dil_w = d.dil_w;
     p.ho = plan->ho;
     p.wo = plan->wo;
-    p.zp_in = q->zp_in;
-    p.zp_w = q->zp_w;
+    p.zp_in = plan->q.zp_in;
+    p.zp_w = plan->q.zp_w;
     p.w_signed = plan->w_signed ? 1 : 0;
-    p.rq = make_requant_dev(*q);
+    p.io_flip = plan->io_signed ? 0x80808080u : 0u;
+    p.rq = make_requant_dev(plan->q);
     if (plan->pc_multiplier) {
         p.rq.pc_multiplier = plan->pc_multiplier;
         p.rq.pc_shift = plan->pc_shift;

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void conv_c3k3_kernel(const GemmProblem p, con
     A[5] = __builtin_amdgcn_alignbyte(seg[2][1], seg[2][0], 2);
     A[6] = __builtin_amdgcn_alignbyte(seg[2][2], seg[2][1], 2);
 #pragma unroll
-    for (int i = 0; i < 7; ++i) A[i] ^= 0x80808080u;
+    for (int i = 0; i < 7; ++i) A[i] ^= p.a_xor;
     A[6] &= 0x00FFFFFFu;
     int ncorr = 0;
     if constexpr (ROWSUM) {
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void conv_c3k3_kernel(const GemmProblem p, con
             o[t] = mode == 0 && rq.pc_multiplier ? requant_u8_channel(acc, rq.pc_multiplier[n], rq.pc_shift[n], rq)
                                                  : requant_u8_as<mode>(acc, rq);
         }
-        packed[g] = o[0] | (o[1] << 8) | (o[2] << 16) | (o[3] << 24);
+        packed[g] = (o[0] | (o[1] << 8) | (o[2] << 16) | (o[3] << 24)) ^ p.out_xor;
     }
     };
     if constexpr (!FAST)

@@ -11,6 +11,8 @@
 // channel are paired into a 16-bit dot product (v_dot2_i32_i16) against
 // weights stored as (w - zp_w) int16 pairs; the input zero point is folded
 // into the bias: sum (a - zi)(w - zw) = sum a (w - zw) - zi * sum (w - zw).
+#include <type_traits>
+
 #include "eh_internal.h"
 
 namespace eh {
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
         const int ky = t / kw, kx = t - ky * kw;
         const int iy = iy0 + ky * p.dil_h, ix = ix0 + kx * p.dil_w;
         if ((unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w_)
-            return *reinterpret_cast<const uint32_t *>(src + ((size_t)iy * p.w_ + ix) * p.c);
+            return *reinterpret_cast<const uint32_t *>(src + ((size_t)iy * p.w_ + ix) * p.c) ^ p.io_flip;
         return fill;
     };
 
@@ -96,7 +98,8 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
             acc3 = dot2(pair_bytes<3>(lo, hi), w4.w, acc3);
         }
     }
-    *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) = requant4(acc0, acc1, acc2, acc3, p.rq, (uint32_t)cq * 4u);
+    *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) =
+        requant4(acc0, acc1, acc2, acc3, p.rq, (uint32_t)cq * 4u) ^ p.io_flip;
 }
 
 // 3x3, dilation 1, stride S in both directions: a thread owns four adjacent channels of FOUR
@@ -104,7 +107,7 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
 // once (every load is issued before the first use, from clamped in-image addresses; taps
 // outside the image are then replaced by the input zero point), so the address arithmetic, the
 // weight and bias loads and the border tests are shared by sixteen outputs.
-template <int S, bool PC>
+template <int S, bool PC, bool FLIP>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
     constexpr int TW = 4, IW = (TW - 1) * S + 3;
@@ -143,7 +146,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p
 #pragma unroll
         for (int x = 0; x < IW; ++x) {
             const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in + (row_off + col_off[x]));
-            in[ky][x] = row_ok && col_ok[x] ? v : fill;
+            in[ky][x] = row_ok && col_ok[x] ? (FLIP ? v ^ 0x80808080u : v) : fill;
         }
     }
     int4 w4[5];
@@ -165,7 +168,8 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p
             acc2 = dot2(pair_bytes<2>(lo, hi), w4[pr].z, acc2);
             acc3 = dot2(pair_bytes<3>(lo, hi), w4[pr].w, acc3);
         }
-        const uint32_t o = requant4<PC>(acc0, acc1, acc2, acc3, rq, cq * 4u);
+        uint32_t o = requant4<PC>(acc0, acc1, acc2, acc3, rq, cq * 4u);
+        if (FLIP) o ^= 0x80808080u;
         if (ox0 + j < p.wo) *reinterpret_cast<uint32_t *>(dst + (uint32_t)j * (uint32_t)p.cout) = o;
     }
 }
@@ -203,14 +207,14 @@ __global__ __launch_bounds__(256) void dw_scalar_kernel(const DwProblem p, const
             if ((unsigned)ix >= (unsigned)p.w_) continue;
             const size_t a_idx = NHWC ? (((size_t)img * p.h + iy) * p.w_ + ix) * p.c + ic
                                       : (((size_t)img * p.c + ic) * p.h + iy) * p.w_ + ix;
-            const int32_t a = (int32_t)p.in[a_idx] - p.zp_in;
+            const int32_t a = (int32_t)(p.in[a_idx] ^ (p.io_flip & 0xFFu)) - p.zp_in;
             const uint8_t raw = p.w[((size_t)oc * p.kh + ky) * p.kw + kx];
             const int32_t w = (p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw) - p.zp_w;
             acc += a * w;
         }
     }
-    p.out[idx] = (uint8_t)(p.rq.pc_multiplier ? requant_u8_channel(acc, p.rq.pc_multiplier[oc], p.rq.pc_shift[oc], p.rq)
-                                               : requant_u8(acc, p.rq));
+    p.out[idx] = (uint8_t)((p.rq.pc_multiplier ? requant_u8_channel(acc, p.rq.pc_multiplier[oc], p.rq.pc_shift[oc], p.rq)
+                                                : requant_u8(acc, p.rq)) ^ (p.io_flip & 0xFFu));
 }
 
 __global__ void dw_pack_kernel(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
@@ -257,8 +261,14 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
         const long blocks = (total + 255) / 256;
         EH_REQUIRE(total < (1l << 31), "depthwise: grid too large");
         const FastDiv d_cq = make_fastdiv((uint32_t)(p.c >> 2)), d_t = make_fastdiv((uint32_t)tiles_x), d_ho = make_fastdiv((uint32_t)p.ho);
-        auto kernel = p.stride_h == 1 ? (p.rq.pc_multiplier ? dw3x3_nhwc_tile4_kernel<1, true> : dw3x3_nhwc_tile4_kernel<1, false>)
-                                      : (p.rq.pc_multiplier ? dw3x3_nhwc_tile4_kernel<2, true> : dw3x3_nhwc_tile4_kernel<2, false>);
+        // per-channel pairs and int8 tensors are compile-time variants: the plain uint8 kernel pays for neither
+        const bool pc = p.rq.pc_multiplier != nullptr, flip = p.io_flip != 0;
+        auto pick = [&](auto stride_c) {
+            constexpr int S = decltype(stride_c)::value;
+            return pc ? (flip ? dw3x3_nhwc_tile4_kernel<S, true, true> : dw3x3_nhwc_tile4_kernel<S, true, false>)
+                      : (flip ? dw3x3_nhwc_tile4_kernel<S, false, true> : dw3x3_nhwc_tile4_kernel<S, false, false>);
+        };
+        auto kernel = p.stride_h == 1 ? pick(std::integral_constant<int, 1>{}) : pick(std::integral_constant<int, 2>{});
         hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total, tiles_x, d_cq, d_t, d_ho);
     } else if (vec) {
         const long total = outs / 4;

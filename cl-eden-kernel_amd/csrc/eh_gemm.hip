@@ -31,11 +31,11 @@ constexpr int BK = 64;        // reduction bytes per LDS stage
 constexpr int LDS_ROW = 80;   // 64 data bytes + 16 pad: 16-byte accesses from 8 consecutive rows hit 32 distinct banks
 constexpr int16_t KPAD_MARK = INT16_MIN;
 
-__device__ __forceinline__ uint4 xor128(uint4 v) {
-    v.x ^= 0x80808080u;
-    v.y ^= 0x80808080u;
-    v.z ^= 0x80808080u;
-    v.w ^= 0x80808080u;
+__device__ __forceinline__ uint4 xor128(uint4 v, uint32_t x) {
+    v.x ^= x;
+    v.y ^= x;
+    v.z ^= x;
+    v.w ^= x;
     return v;
 }
 
@@ -55,7 +55,7 @@ __device__ __forceinline__ uint4 load_a_chunk(const GemmProblem &p, int base, in
         const KUnit ku = p.ktab[unit16];
         const int iy = iy0 + ku.dy, ix = ix0 + ku.dx;
         if (ku.dy == KPAD_MARK) {
-            v = make_uint4(0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u);
+            v = make_uint4(p.a_xor, p.a_xor, p.a_xor, p.a_xor);
         } else if ((unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w) {
             v = *reinterpret_cast<const uint4 *>(p.a + (base + ku.offset));
         } else {
@@ -68,7 +68,7 @@ __device__ __forceinline__ uint4 load_a_chunk(const GemmProblem &p, int base, in
             const KUnit ku = p.ktab[unit16 * 4 + j];
             const int iy = iy0 + ku.dy, ix = ix0 + ku.dx;
             if (ku.dy == KPAD_MARK) {
-                d[j] = 0x80808080u;
+                d[j] = p.a_xor;
             } else if ((unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w) {
                 d[j] = *reinterpret_cast<const uint32_t *>(p.a + (base + ku.offset));
             } else {
@@ -84,7 +84,7 @@ __device__ __forceinline__ uint4 load_a_chunk(const GemmProblem &p, int base, in
             const int iy = iy0 + ku.dy, ix = ix0 + ku.dx;
             uint32_t b;
             if (ku.dy == KPAD_MARK) {
-                b = 0x80u;
+                b = p.a_xor & 0xFFu;
             } else if ((unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w) {
                 b = p.a[base + ku.offset];
             } else {
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_u8_kernel(const GemmProbl
         uint8_t *bs = as + BM * LDS_ROW;
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
-            const uint4 v = xor128(ra[i]);
+            const uint4 v = xor128(ra[i], p.a_xor);
             if (need_rowsum) rowsum[i] = sum_bytes_signed(v, rowsum[i]);
             *reinterpret_cast<uint4 *>(as + (lrow + i * ROWS_PER_PASS) * LDS_ROW + kc * 16) = v;
         }
@@ -242,7 +242,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_u8_kernel(const GemmProbl
             for (int r = 0; r < 16; ++r) {
                 const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 const int32_t v = acc[i][j][r] + bias - p.zw * rowsum_s[ml];
-                cs[ml * OUT_ROW + nl] = (uint8_t)(per_channel ? requant_u8_channel(v, ch_mult, ch_shift, rq) : requant_u8(v, rq));
+                cs[ml * OUT_ROW + nl] =
+                    (uint8_t)((per_channel ? requant_u8_channel(v, ch_mult, ch_shift, rq) : requant_u8(v, rq)) ^ (p.out_xor & 0xFFu));
             }
         }
     }

@@ -62,11 +62,11 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-__device__ __forceinline__ v4i xor128(v4i v) {
-    v.x ^= (int)0x80808080u;
-    v.y ^= (int)0x80808080u;
-    v.z ^= (int)0x80808080u;
-    v.w ^= (int)0x80808080u;
+__device__ __forceinline__ v4i xor128(v4i v, int x) {
+    v.x ^= x;
+    v.y ^= x;
+    v.z ^= x;
+    v.w ^= x;
     return v;
 }
 
@@ -188,6 +188,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = (wave / WGM) % WGN, wk = wave / (WGM * WGN);
     const int k_slabs = p.k_pad / SLAB;
+    const int a_xor = (int)p.a_xor;  // stored activation bytes -> int8 operands (uniform)
 
     // ---- operand fetch.  This lane's slot in a DMA block: row (lane / CPR), physical chunk lane % CPR.
     const int slot_row = lane / CPR;
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
     };
     auto flip = [&](auto buf_c, auto i_c) {
         constexpr int buf = decltype(buf_c)::value, i = decltype(i_c)::value;
-        af[buf][i] = xor128(af[buf][i]);
+        af[buf][i] = xor128(af[buf][i], a_xor);
         if constexpr (ROWSUM) rowsum[i] = sum_bytes_signed(af[buf][i], rowsum[i]);
     };
     typedef std::integral_constant<int, 0> c0;
@@ -437,7 +438,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
                             o2 = requant_u8_as<fast>(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], rq);
                             o3 = requant_u8_as<fast>(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], rq);
                         }
-                        packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+                        packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
                     }
                     uint8_t *dst = p.out + row_off[i] + n;
                     if constexpr (!checked) {
@@ -525,7 +526,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
                 o0 = requant_u8_as<fast>(s4.x + bb.x - corr, rq), o1 = requant_u8_as<fast>(s4.y + bb.y - corr, rq);
                 o2 = requant_u8_as<fast>(s4.z + bb.z - corr, rq), o3 = requant_u8_as<fast>(s4.w + bb.w - corr, rq);
             }
-            packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+            packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
         }
         };
         if (rq.fast == 2)

@@ -72,14 +72,14 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         v4i afs[SINGLE ? KU : 1], bfs[SINGLE ? KU : 1][SINGLE ? NBU : 1];
         int rowsum = 0;
         for (int ks0 = 0; ks0 < (SINGLE ? 1 : ksteps); ks0 += KU) {
-            // reduction bytes past K read as 0x80, which the signed shift turns into 0; steps past the
+            // reduction bytes past K read as the byte that the sign flip turns into 0; steps past the
             // last one therefore multiply by zero whatever weight block they re-read
             uint2 lo[KU], hi[KU];
             v4i bf[KU][NBU];
 #pragma unroll
             for (int t = 0; t < KU; ++t) {
                 const int kb = (ks0 + t) * 32 + half * 16;
-                lo[t] = make_uint2(0x80808080u, 0x80808080u);
+                lo[t] = make_uint2(p.a_xor, p.a_xor);
                 hi[t] = lo[t];
                 if (row_ok && kb < p.k) lo[t] = *reinterpret_cast<const uint2 *>(arow + (ks0 + t) * 32);
                 if (row_ok && kb + 8 < p.k) hi[t] = *reinterpret_cast<const uint2 *>(arow + (ks0 + t) * 32 + 8);
@@ -98,10 +98,10 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
 #pragma unroll
             for (int t = 0; t < KU; ++t) {
                 v4i af;
-                af.x = (int)(lo[t].x ^ 0x80808080u);
-                af.y = (int)(lo[t].y ^ 0x80808080u);
-                af.z = (int)(hi[t].x ^ 0x80808080u);
-                af.w = (int)(hi[t].y ^ 0x80808080u);
+                af.x = (int)(lo[t].x ^ p.a_xor);
+                af.y = (int)(lo[t].y ^ p.a_xor);
+                af.z = (int)(hi[t].x ^ p.a_xor);
+                af.w = (int)(hi[t].y ^ p.a_xor);
                 if constexpr (ROWSUM) {
                     rowsum = __builtin_amdgcn_sdot4(af.x, 0x01010101, rowsum, false);
                     rowsum = __builtin_amdgcn_sdot4(af.y, 0x01010101, rowsum, false);
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                         o2 = requant_u8_as<mode>(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, rq);
                         o3 = requant_u8_as<mode>(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, rq);
                     }
-                    packed[g] = o0 | (o1 << 8) | (o2 << 16) | (o3 << 24);
+                    packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
                 }
             };
             if constexpr (!FAST)

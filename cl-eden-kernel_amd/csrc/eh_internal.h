@@ -182,7 +182,8 @@ inline FastDiv make_fastdiv(uint32_t d) {
 }
 __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) { return (__umulhi(f.mul, n) + n) >> f.shift; }
 
-int check_requant(const eh_requant *q, bool signed_weights = false);
+// signed_weights: zp_w is an int8 zero point; signed_io: zp_in, zp_out and the activation range are int8 values
+int check_requant(const eh_requant *q, bool signed_weights = false, bool signed_io = false);
 
 // ---------------------------------------------------------------- implicit GEMM
 // One row of the k-table describes one load unit (VEC bytes) of the reduction
@@ -213,7 +214,7 @@ struct GemmProblem {
     const uint8_t *a;     // activations: NHWC image or [M][K] matrix
     const int8_t *b;      // packed weights, value = w - 128, laid out for cfg (see packed_b_offset)
     GemmConfig cfg;
-    const uint8_t *fillbuf;  // 32 bytes: 16 x input zero point, then 16 x 0x80
+    const uint8_t *fillbuf;  // 32 bytes: 16 x input zero point byte, then 16 x the byte that a_xor turns into 0
     const int32_t *bias;  // [n_pad] bias with the zero-point terms folded in
     const KUnit *ktab;    // [k_pad / vec]
     uint8_t *out;
@@ -231,7 +232,10 @@ struct GemmProblem {
     int32_t dense;     // 1: a plain [m][k] matrix with row stride cin and k a multiple of the slab (no taps, no padding)
     int32_t zw;        // zp_w - 128: coefficient of the per-row activation sum
     int32_t a_offset;  // one-tap problems: byte offset of the (group's) first channel within a pixel
-    uint32_t fill;     // input zero point replicated in 4 bytes (value of an out-of-image tap)
+    uint32_t fill;     // input zero point byte as it is stored, replicated in 4 bytes (value of an out-of-image tap)
+    // int8 tensors (PrecisionType::INT8) run as their uint8 equivalents (value + 128, zero points + 128):
+    uint32_t a_xor;    // turns four stored activation bytes into int8 MFMA operands: 0x80808080 for uint8 data, 0 for int8
+    uint32_t out_xor;  // turns four uint8 results into the stored bytes: 0 for uint8 data, 0x80808080 for int8
     RequantDev rq;
 };
 
@@ -287,7 +291,7 @@ int launch_pack_weights(const PackProblem &p, hipStream_t stream);
 // folded[n] = bias[n] - za * colsum[n] + k * za * zw   (za = zp_in - 128, zw = zp_w - 128)
 // also refreshes the 32-byte fill constant when `fillbuf` is not null
 int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad,
-                     int32_t k, int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, hipStream_t stream);
+                     int32_t k, int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, int32_t io_flip, hipStream_t stream);
 
 // ---------------------------------------------------------------- depthwise
 struct DwProblem {
@@ -302,6 +306,7 @@ struct DwProblem {
     int32_t ho, wo;
     int32_t zp_in, zp_w;
     int32_t w_signed;            // weight bytes are int8
+    uint32_t io_flip;            // 0x80808080 when input and output hold int8 values (computed as value + 128), else 0
     RequantDev rq;               // rq.pc_multiplier / rq.pc_shift: [cout + 4] when set
 };
 int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,

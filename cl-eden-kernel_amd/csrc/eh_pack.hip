@@ -37,9 +37,10 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
 }
 
 __global__ void fold_bias_kernel(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad,
-                                 int32_t k, int32_t za, int32_t zw, uint8_t *fillbuf) {
+                                 int32_t k, int32_t za, int32_t zw, uint8_t *fillbuf, int32_t io_flip) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (fillbuf && i < 32) fillbuf[i] = i < 16 ? (uint8_t)(za + 128) : (uint8_t)0x80;
+    // bytes as the input tensor stores them: int8 tensors (io_flip = 0x80) hold value - 128
+    if (fillbuf && i < 32) fillbuf[i] = (uint8_t)((i < 16 ? za + 128 : 0x80) ^ io_flip);
     if (i >= n_pad) return;
     int32_t v = 0;
     if (i < n) v = (bias ? bias[i] : 0) - za * colsum[i] + k * za * zw;
@@ -110,10 +111,10 @@ int launch_pack_weights(const PackProblem &p, hipStream_t stream) {
 }
 
 int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad, int32_t k,
-                     int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, hipStream_t stream) {
+                     int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, int32_t io_flip, hipStream_t stream) {
     if (n_pad <= 0) return EH_OK;
     hipLaunchKernelGGL(fold_bias_kernel, dim3((n_pad + 255) / 256), dim3(256), 0, stream, bias, colsum, folded, n, n_pad,
-                       k, zp_in - 128, zp_w - 128, fillbuf);
+                       k, zp_in - 128, zp_w - 128, fillbuf, io_flip);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }

@@ -50,6 +50,11 @@ typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh
  * cl_kernels/DeconvolutionKernels.cpp:449-454);
  * eh_requant.zp_w is then an int8 zero point in [-128, 127] (0 in the reference). */
 #define EH_W_SIGNED 0x100
+/* Or-ed into eh_conv_desc.layout: the input and output tensors hold int8 values (PrecisionType::INT8: the
+ * SIGNED* kernels, e.g. gpu/operators/cl_optimized_impls/CLGEMMConvolutionQuantized.cpp:47,110-114,226-241);
+ * eh_requant.zp_in, zp_out, act_min and act_max are then int8 values in [-128, 127].  The reference pairs this
+ * precision with int8 weights (EH_W_SIGNED); the two flags are independent here. */
+#define EH_IO_SIGNED 0x200
 
 /* Integer requantization parameters of one operator execution: what
  * CLGEMMConvolutionQuantized::execute derives from its tensors
@@ -113,11 +118,17 @@ void eh_quantize_multiplier(double real_multiplier, int32_t *quantized_multiplie
 int eh_conv_multiplier(float input_scale, float filter_scale, float bias_scale, float output_scale, double *multiplier);
 /* CalculateActivationRangeUint8 (gpu/operators/cl_quantized_utils/KernelUtil.cpp:27-60) */
 void eh_act_range_u8(int activation, float scale, int32_t zero_point, int32_t *act_min, int32_t *act_max);
+/* CalculateActivationRangeInt8 (gpu/operators/cl_quantized_utils/KernelUtil.cpp:62-71) */
+void eh_act_range_s8(int activation, float scale, int32_t zero_point, int32_t *act_min, int32_t *act_max);
 /* The whole derivation an operator's execute() performs, including the
  * reference's behaviour of continuing with multiplier 0 when the bias scale
  * does not match (CLGEMMConvolutionQuantized.cpp:163-166). */
 void eh_make_requant(float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp, float bias_scale,
                      float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out);
+/* The same for PrecisionType::INT8 (EH_IO_SIGNED plans): range [-128, 127] or CalculateActivationRangeInt8
+ * (gpu/operators/cl_optimized_impls/CLGEMMConvolutionQuantized.cpp:224-241). */
+void eh_make_requant_s8(float input_scale, int32_t input_zp, float filter_scale, int32_t filter_zp, float bias_scale,
+                        float output_scale, int32_t output_zp, int activation, int activation_enabled, eh_requant *out);
 /* The requantization every kernel epilogue applies to an int32 accumulator (bias
  * and zero-point terms already added): MultiplyByQuantizedMultiplier, output
  * zero point, activation clamp (gpu/common/CLKernels.hpp:120-170), evaluated on
@@ -240,6 +251,10 @@ int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
  * (gpu/op_test/fullyconnected_test.cpp:93-105), computed in the convolution's
  * integer pipeline rather than the reference's float detour. */
 int eh_fc_u8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, const void *weight, const void *bias,
+                  const eh_requant *q, void *stream);
+/* The same with `flags` = any of EH_W_SIGNED | EH_IO_SIGNED: int8 weights and/or int8 input and output
+ * (PrecisionType::INT8 takes the quantized path too, cl_optimized_impls/CLBaseFullyConnected.cpp:88,147-148). */
+int eh_fc_q8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, int32_t flags, const void *weight, const void *bias,
                   const eh_requant *q, void *stream);
 int eh_fc_u8_repack(eh_fc_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
 int eh_fc_u8_run(eh_fc_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);

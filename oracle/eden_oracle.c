@@ -58,8 +58,18 @@ static int32_t quantize_real(float f, float scale, int32_t zp) {
     return zp + (int32_t)round((double)(f / scale));
 }
 
+static void act_range(int act, float scale, int32_t zp, int32_t qmin, int32_t qmax, int32_t *amin, int32_t *amax);
+
 void eo_act_range_u8(int act, float scale, int32_t zp, int32_t *amin, int32_t *amax) {
-    const int32_t qmin = 0, qmax = 255;
+    act_range(act, scale, zp, 0, 255, amin, amax);
+}
+
+/* src/userdriver/gpu/operators/cl_quantized_utils/KernelUtil.cpp:62-71: the same clamps over [-128, 127] */
+void eo_act_range_s8(int act, float scale, int32_t zp, int32_t *amin, int32_t *amax) {
+    act_range(act, scale, zp, -128, 127, amin, amax);
+}
+
+static void act_range(int act, float scale, int32_t zp, int32_t qmin, int32_t qmax, int32_t *amin, int32_t *amax) {
     if (act == EO_ACT_RELU) {
         const int32_t lo = quantize_real(0.0f, scale, zp);
         *amin = qmin > lo ? qmin : lo;
@@ -134,6 +144,18 @@ void eo_make_quant(float s_in, int32_t zp_in, float s_w, int32_t zp_w, float s_b
     }
 }
 
+/* INT8 precision: cl_optimized_impls/CLGEMMConvolutionQuantized.cpp:224-241 */
+void eo_make_quant_s8(float s_in, int32_t zp_in, float s_w, int32_t zp_w, float s_bias,
+                      float s_out, int32_t zp_out, int act, int act_enabled, eo_quant *q) {
+    eo_make_quant(s_in, zp_in, s_w, zp_w, s_bias, s_out, zp_out, act, 0, q);
+    if (act_enabled) {
+        eo_act_range_s8(act, s_out, zp_out, &q->act_min, &q->act_max);
+    } else {
+        q->act_min = -128;
+        q->act_max = 127;
+    }
+}
+
 /* src/userdriver/gpu/operators/CLConvolution.cpp:99-104 */
 int32_t eo_conv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t k, int32_t dil, int32_t stride) {
     return (in + pad_a + pad_b - (dil * (k - 1) + 1) + stride) / stride;
@@ -153,7 +175,7 @@ int32_t eo_deconv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t k, i
  * taps follow src/userdriver/gpu/op_test/convolution_guard.h:118-144 and
  * cl_kernels/ConvolutionKernels.cpp:1321-1350; a skipped tap is the same as
  * a tap that reads zp_in (cl_optimized_impls/CLPadConvert.cpp:185). */
-static void accumulate_tap(int32_t *plane, const uint8_t *src, int32_t wv, int32_t zp_in,
+static void accumulate_tap(int32_t *plane, const uint8_t *src, int in_is_signed, int32_t wv, int32_t zp_in,
                            int32_t H, int32_t W, int32_t Ho, int32_t Wo,
                            int32_t oy_off, int32_t ox_off, int32_t sh, int32_t sw) {
     /* iy = oy*sh + oy_off, ix = ox*sw + ox_off */
@@ -167,11 +189,16 @@ static void accumulate_tap(int32_t *plane, const uint8_t *src, int32_t wv, int32
         if (ox_off > W - 1) ox1 = 0;
         const uint8_t *row = src + (int64_t)iy * W;
         int32_t *dst = plane + (int64_t)oy * Wo;
-        for (int32_t ox = ox0; ox < ox1; ++ox) dst[ox] += ((int32_t)row[ox * sw + ox_off] - zp_in) * wv;
+        if (in_is_signed) {
+            const int8_t *srow = (const int8_t *)row;
+            for (int32_t ox = ox0; ox < ox1; ++ox) dst[ox] += ((int32_t)srow[ox * sw + ox_off] - zp_in) * wv;
+        } else {
+            for (int32_t ox = ox0; ox < ox1; ++ox) dst[ox] += ((int32_t)row[ox * sw + ox_off] - zp_in) * wv;
+        }
     }
 }
 
-static void conv_core(const uint8_t *in, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
+static void conv_core(const uint8_t *in, int in_is_signed, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
                       const eo_conv_shape *s, const eo_quant *q, const int32_t *multipliers,
                       const int32_t *shifts, int32_t *acc_out) {
     const int32_t Ho = eo_conv_out_dim(s->h, s->pad_t, s->pad_b, s->kh, s->dil_h, s->stride_h);
@@ -195,7 +222,7 @@ static void conv_core(const uint8_t *in, const void *w, int w_is_signed, const i
                         const int64_t wi = (((int64_t)oc * Cig + ic) * s->kh + ky) * s->kw + kx;
                         const int32_t wv = w_is_signed ? (int32_t)((const int8_t *)w)[wi] - q->zp_w
                                                        : (int32_t)((const uint8_t *)w)[wi] - q->zp_w;
-                        accumulate_tap(acc, src, wv, q->zp_in, s->h, s->w, Ho, Wo,
+                        accumulate_tap(acc, src, in_is_signed, wv, q->zp_in, s->h, s->w, Ho, Wo,
                                        ky * s->dil_h - s->pad_t, kx * s->dil_w - s->pad_l,
                                        s->stride_h, s->stride_w);
                     }
@@ -217,7 +244,7 @@ static void conv_core(const uint8_t *in, const void *w, int w_is_signed, const i
  * :1317-1375 (naive per-channel form); weights [Cout][Cin/g][kh][kw]. */
 void eo_conv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
                   const eo_conv_shape *s, const eo_quant *q, int32_t *acc) {
-    conv_core(in, w, 0, bias, out, s, q, NULL, NULL, acc);
+    conv_core(in, 0, w, 0, bias, out, s, q, NULL, NULL, acc);
 }
 
 /* cl_kernels/ConvolutionKernels.cpp:1317-1375: int8 weights, one multiplier
@@ -225,12 +252,12 @@ void eo_conv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint
 void eo_conv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
                              const eo_conv_shape *s, const eo_quant *q,
                              const int32_t *multipliers, const int32_t *shifts, int32_t *acc) {
-    conv_core(in, w, 1, bias, out, s, q, multipliers, shifts, acc);
+    conv_core(in, 0, w, 1, bias, out, s, q, multipliers, shifts, acc);
 }
 
 /* cl_kernels/DepthwiseconvolutionKernels.cpp:1273-1321; weights [C*dm][1][kh][kw],
  * output channel c*dm+d reads input channel c. */
-static void dw_core(const uint8_t *in, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
+static void dw_core(const uint8_t *in, int in_is_signed, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
                     const eo_conv_shape *s, const eo_quant *q, const int32_t *multipliers,
                     const int32_t *shifts, int32_t *acc_out) {
     const int32_t Ho = eo_conv_out_dim(s->h, s->pad_t, s->pad_b, s->kh, s->dil_h, s->stride_h);
@@ -254,7 +281,7 @@ static void dw_core(const uint8_t *in, const void *w, int w_is_signed, const int
                     const int64_t wi = ((int64_t)oc * s->kh + ky) * s->kw + kx;
                     const int32_t wv = w_is_signed ? (int32_t)((const int8_t *)w)[wi] - q->zp_w
                                                    : (int32_t)((const uint8_t *)w)[wi] - q->zp_w;
-                    accumulate_tap(acc, src, wv, q->zp_in, s->h, s->w, Ho, Wo,
+                    accumulate_tap(acc, src, in_is_signed, wv, q->zp_in, s->h, s->w, Ho, Wo,
                                    ky * s->dil_h - s->pad_t, kx * s->dil_w - s->pad_l,
                                    s->stride_h, s->stride_w);
                 }
@@ -273,7 +300,7 @@ static void dw_core(const uint8_t *in, const void *w, int w_is_signed, const int
 
 void eo_dwconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
                     const eo_conv_shape *s, const eo_quant *q, int32_t *acc_out) {
-    dw_core(in, w, 0, bias, out, s, q, NULL, NULL, acc_out);
+    dw_core(in, 0, w, 0, bias, out, s, q, NULL, NULL, acc_out);
 }
 
 /* cl_kernels/DepthwiseconvolutionKernels.cpp:1323-1371 (int8 weight bytes, the multiplier and
@@ -282,7 +309,7 @@ void eo_dwconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, ui
 void eo_dwconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
                                const eo_conv_shape *s, const eo_quant *q,
                                const int32_t *multipliers, const int32_t *shifts, int32_t *acc_out) {
-    dw_core(in, w, 1, bias, out, s, q, multipliers, shifts, acc_out);
+    dw_core(in, 0, w, 1, bias, out, s, q, multipliers, shifts, acc_out);
 }
 
 /* Layout a[m][k], w[n][k], out[m][n]: src/userdriver/gpu/op_test/fullyconnected_test.cpp:93-105.
@@ -349,7 +376,7 @@ void eo_deconv2d_f64(const double *in, const double *w, const double *bias, doub
     }
 }
 
-static void deconv_core(const uint8_t *in, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
+static void deconv_core(const uint8_t *in, int in_is_signed, const void *w, int w_is_signed, const int32_t *bias, uint8_t *out,
                         const eo_conv_shape *s, const eo_quant *q, const int32_t *multipliers,
                         const int32_t *shifts, int32_t *acc_out) {
     const int32_t Ho = eo_deconv_out_dim(s->h, s->pad_t, s->pad_b, s->kh, s->stride_h);
@@ -362,7 +389,8 @@ static void deconv_core(const uint8_t *in, const void *w, int w_is_signed, const
     double *dw = (double *)malloc(sizeof(double) * (size_t)(n_w > 0 ? n_w : 1));
     double *db = (double *)malloc(sizeof(double) * (size_t)s->cout);
     double *dout = (double *)malloc(sizeof(double) * (size_t)n_out);
-    for (int64_t i = 0; i < n_in; ++i) din[i] = (double)((int32_t)in[i] - q->zp_in);
+    for (int64_t i = 0; i < n_in; ++i)
+        din[i] = (double)((in_is_signed ? (int32_t)((const int8_t *)in)[i] : (int32_t)in[i]) - q->zp_in);
     for (int64_t i = 0; i < n_w; ++i)
         dw[i] = (double)((w_is_signed ? (int32_t)((const int8_t *)w)[i] : (int32_t)((const uint8_t *)w)[i]) - q->zp_w);
     for (int32_t i = 0; i < s->cout; ++i) db[i] = bias ? (double)bias[i] : 0.0;
@@ -386,7 +414,7 @@ static void deconv_core(const uint8_t *in, const void *w, int w_is_signed, const
 
 void eo_deconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, uint8_t *out,
                     const eo_conv_shape *s, const eo_quant *q, int32_t *acc_out) {
-    deconv_core(in, w, 0, bias, out, s, q, NULL, NULL, acc_out);
+    deconv_core(in, 0, w, 0, bias, out, s, q, NULL, NULL, acc_out);
 }
 
 /* cl_kernels/DeconvolutionKernels.cpp:200-249 (the gather with the pair of channel
@@ -395,7 +423,39 @@ void eo_deconv2d_u8(const uint8_t *in, const uint8_t *w, const int32_t *bias, ui
 void eo_deconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
                                const eo_conv_shape *s, const eo_quant *q,
                                const int32_t *multipliers, const int32_t *shifts, int32_t *acc_out) {
-    deconv_core(in, w, 1, bias, out, s, q, multipliers, shifts, acc_out);
+    deconv_core(in, 0, w, 1, bias, out, s, q, multipliers, shifts, acc_out);
+}
+
+/* PrecisionType::INT8: int8 input, weight and output bytes, zero points and clamp bounds in [-128, 127] (the
+ * SIGNED* kernels: cl_kernels/ConvolutionKernels.cpp SIGNEDquantizedGemmBlocked,
+ * cl_kernels/DepthwiseconvolutionKernels.cpp:2410-2450, cl_kernels/DeconvolutionKernels.cpp:340-440).  The
+ * arithmetic is the uint8 one on the signed values; `multipliers` may be NULL (per-tensor). */
+void eo_conv2d_s8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const eo_conv_shape *s,
+                  const eo_quant *q, const int32_t *multipliers, const int32_t *shifts) {
+    conv_core((const uint8_t *)in, 1, w, 1, bias, (uint8_t *)out, s, q, multipliers, shifts, NULL);
+}
+
+void eo_dwconv2d_s8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const eo_conv_shape *s,
+                    const eo_quant *q, const int32_t *multipliers, const int32_t *shifts) {
+    dw_core((const uint8_t *)in, 1, w, 1, bias, (uint8_t *)out, s, q, multipliers, shifts, NULL);
+}
+
+void eo_deconv2d_s8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const eo_conv_shape *s,
+                    const eo_quant *q, const int32_t *multipliers, const int32_t *shifts) {
+    deconv_core((const uint8_t *)in, 1, w, 1, bias, (uint8_t *)out, s, q, multipliers, shifts, NULL);
+}
+
+void eo_fc_s8(const int8_t *a, const int8_t *w, const int32_t *bias, int8_t *out, int32_t m, int32_t k, int32_t n,
+              const eo_quant *q) {
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int32_t i = 0; i < m; ++i)
+        for (int32_t j = 0; j < n; ++j) {
+            const int8_t *ar = a + (int64_t)i * k, *wr = w + (int64_t)j * k;
+            int32_t acc = 0;
+            for (int32_t t = 0; t < k; ++t) acc += ((int32_t)ar[t] - q->zp_in) * ((int32_t)wr[t] - q->zp_w);
+            acc += bias ? bias[j] : 0;
+            out[(int64_t)i * n + j] = (int8_t)eo_requant(acc, q);
+        }
 }
 
 /* Scatter form: col = W^T x A (cl_kernels/DeconvolutionKernels.cpp:24-60), then

@@ -25,6 +25,10 @@
  *                            pinned by reduction: channel c of the result equals channel c of the per-tensor
  *                                    function above run on the weight bytes + 128 with weight zero point + 128
  *                                    and channel c's (multiplier, shift); no reference vector exists for them
+ *   eo_act_range_s8          pinned: reference build + golden vectors
+ *   eo_conv2d_s8 / eo_dwconv2d_s8 / eo_deconv2d_s8 / eo_fc_s8
+ *                            pinned by reduction: the result + 128 equals the uint8 function above on every byte,
+ *                                    zero point and clamp bound + 128; no reference vector exists for them
  *   eo_nchw2nhwc_u8 / eo_nhwc2nchw_u8  pinned: round trip + index closed form
  *   eo_add_u8 / eo_avgpool_u8           parity unpinned by reference vectors (closed-form checks only)
  */
@@ -65,6 +69,7 @@ typedef struct eo_conv_shape {
 void    eo_quantize_multiplier(double m, int32_t *q, int32_t *shift);
 int     eo_conv_multiplier(float s_in, float s_w, float s_bias, float s_out, double *m);
 void    eo_act_range_u8(int act, float scale, int32_t zp, int32_t *amin, int32_t *amax);
+void    eo_act_range_s8(int act, float scale, int32_t zp, int32_t *amin, int32_t *amax);
 int32_t eo_srdhm(int32_t a, int32_t b);
 int32_t eo_rdivpot(int32_t x, int32_t exponent);
 int32_t eo_mbqm(int32_t x, int32_t q, int32_t shift);
@@ -72,6 +77,9 @@ uint8_t eo_requant(int32_t acc, const eo_quant *q);
 /* fill an eo_quant from tensor scales exactly as an operator's execute() does */
 void    eo_make_quant(float s_in, int32_t zp_in, float s_w, int32_t zp_w, float s_bias,
                       float s_out, int32_t zp_out, int act, int act_enabled, eo_quant *q);
+
+void    eo_make_quant_s8(float s_in, int32_t zp_in, float s_w, int32_t zp_w, float s_bias,
+                         float s_out, int32_t zp_out, int act, int act_enabled, eo_quant *q);
 
 /* output-size formulas */
 int32_t eo_conv_out_dim(int32_t in, int32_t pad_a, int32_t pad_b, int32_t k, int32_t dil, int32_t stride);
@@ -92,6 +100,15 @@ void eo_dwconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t
 void eo_deconv2d_u8_perchannel(const uint8_t *in, const int8_t *w, const int32_t *bias, uint8_t *out,
                                const eo_conv_shape *s, const eo_quant *q,
                                const int32_t *multipliers, const int32_t *shifts, int32_t *acc);
+/* INT8 precision: int8 bytes everywhere, parameters in [-128, 127]; multipliers/shifts NULL = per-tensor */
+void eo_conv2d_s8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const eo_conv_shape *s,
+                  const eo_quant *q, const int32_t *multipliers, const int32_t *shifts);
+void eo_dwconv2d_s8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const eo_conv_shape *s,
+                    const eo_quant *q, const int32_t *multipliers, const int32_t *shifts);
+void eo_deconv2d_s8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const eo_conv_shape *s,
+                    const eo_quant *q, const int32_t *multipliers, const int32_t *shifts);
+void eo_fc_s8(const int8_t *a, const int8_t *w, const int32_t *bias, int8_t *out, int32_t m, int32_t k, int32_t n,
+              const eo_quant *q);
 void eo_fc_u8(const uint8_t *a, const uint8_t *w, const int32_t *bias, uint8_t *out,
               int32_t m, int32_t k, int32_t n, const eo_quant *q, int32_t *acc);
 /* gather form (each output pixel sums its contributing taps) */

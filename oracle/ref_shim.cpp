@@ -15,6 +15,7 @@ namespace gpu {
 // header also pulls in the OpenCL tensor class, which this shim does not need
 Status GetQuantizedConvolutionMultipler(double, double, double, double, double *);
 void CalculateActivationRangeUint8(ActivationInfo::ActivationType, float, int32_t, int32_t *, int32_t *);
+void CalculateActivationRangeInt8(ActivationInfo::ActivationType, float, int32_t, int32_t *, int32_t *);
 }  // namespace gpu
 }  // namespace ud
 }  // namespace enn
@@ -33,6 +34,10 @@ int ref_conv_multiplier(float s_in, float s_w, float s_bias, float s_out, double
 
 void ref_act_range_u8(int act, float scale, int32_t zp, int32_t *amin, int32_t *amax) {
     enn::ud::gpu::CalculateActivationRangeUint8(static_cast<ActivationInfo::ActivationType>(act), scale, zp, amin, amax);
+}
+
+void ref_act_range_s8(int act, float scale, int32_t zp, int32_t *amin, int32_t *amax) {
+    enn::ud::gpu::CalculateActivationRangeInt8(static_cast<ActivationInfo::ActivationType>(act), scale, zp, amin, amax);
 }
 
 int32_t ref_srdhm(int32_t a, int32_t b) { return gemmlowp::SaturatingRoundingDoublingHighMul(a, b); }

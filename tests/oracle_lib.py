@@ -47,6 +47,12 @@ def _load():
         "eo_quantize_multiplier": (None, [f64, P(i32), P(i32)]),
         "eo_conv_multiplier": (C.c_int, [f32, f32, f32, f32, P(f64)]),
         "eo_act_range_u8": (None, [C.c_int, f32, i32, P(i32), P(i32)]),
+        "eo_act_range_s8": (None, [C.c_int, f32, i32, P(i32), P(i32)]),
+        "eo_make_quant_s8": (None, [f32, i32, f32, i32, f32, f32, i32, C.c_int, C.c_int, P(Quant)]),
+        "eo_conv2d_s8": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp, vp]),
+        "eo_dwconv2d_s8": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp, vp]),
+        "eo_deconv2d_s8": (None, [vp, vp, vp, vp, P(ConvShape), P(Quant), vp, vp]),
+        "eo_fc_s8": (None, [vp, vp, vp, vp, i32, i32, i32, P(Quant)]),
         "eo_srdhm": (i32, [i32, i32]),
         "eo_rdivpot": (i32, [i32, i32]),
         "eo_mbqm": (i32, [i32, i32, i32]),
@@ -99,6 +105,8 @@ def load_ref():
     ref.ref_conv_multiplier.restype = C.c_int
     ref.ref_act_range_u8.argtypes = [C.c_int, f32, i32, P(i32), P(i32)]
     ref.ref_act_range_u8.restype = None
+    ref.ref_act_range_s8.argtypes = [C.c_int, f32, i32, P(i32), P(i32)]
+    ref.ref_act_range_s8.restype = None
     for n in ("ref_srdhm", "ref_rdivpot"):
         getattr(ref, n).argtypes = [i32, i32]
         getattr(ref, n).restype = i32
@@ -121,6 +129,52 @@ def act_range_u8(act, scale, zp):
     lo, hi = C.c_int32(), C.c_int32()
     lib.eo_act_range_u8(act, scale, zp, C.byref(lo), C.byref(hi))
     return lo.value, hi.value
+
+
+def act_range_s8(act, scale, zp):
+    lo, hi = C.c_int32(), C.c_int32()
+    lib.eo_act_range_s8(act, scale, zp, C.byref(lo), C.byref(hi))
+    return lo.value, hi.value
+
+
+def make_quant_s8(s_in, zp_in, s_w, zp_w, s_out, zp_out, act=ACT_NONE, act_enabled=False, s_bias=None):
+    """INT8 precision: zero points and the activation range are int8 values"""
+    q = Quant()
+    if s_bias is None:
+        s_bias = float(np.float32(s_in) * np.float32(s_w))
+    lib.eo_make_quant_s8(s_in, zp_in, s_w, zp_w, s_bias, s_out, zp_out, act, int(act_enabled), C.byref(q))
+    return q
+
+
+def _s8_op(fn, x, w, bias, s, q, out_shape, multipliers, shifts):
+    x, w, bias = _c(x, np.int8), _c(w, np.int8), _c(bias, np.int32)
+    out = np.zeros(out_shape, np.int8)
+    m = _c(multipliers, np.int32) if multipliers is not None else None
+    sh = _c(shifts, np.int32) if shifts is not None else None
+    fn(_ptr(x), _ptr(w), _ptr(bias), _ptr(out), C.byref(s), C.byref(q), _ptr(m), _ptr(sh))
+    return out
+
+
+def conv2d_s8(x, w, bias, s, q, multipliers=None, shifts=None):
+    ho, wo = conv_out_hw(s)
+    return _s8_op(lib.eo_conv2d_s8, x, w, bias, s, q, (s.n, s.cout, ho, wo), multipliers, shifts)
+
+
+def dwconv2d_s8(x, w, bias, s, q, multipliers=None, shifts=None):
+    ho, wo = conv_out_hw(s)
+    return _s8_op(lib.eo_dwconv2d_s8, x, w, bias, s, q, (s.n, s.c * max(s.dm, 1), ho, wo), multipliers, shifts)
+
+
+def deconv2d_s8(x, w, bias, s, q, multipliers=None, shifts=None):
+    ho, wo = deconv_out_hw(s)
+    return _s8_op(lib.eo_deconv2d_s8, x, w, bias, s, q, (s.n, s.cout, ho, wo), multipliers, shifts)
+
+
+def fc_s8(a, w, bias, q):
+    a, w, bias = _c(a, np.int8), _c(w, np.int8), _c(bias, np.int32)
+    out = np.zeros((a.shape[0], w.shape[0]), np.int8)
+    lib.eo_fc_s8(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), a.shape[0], a.shape[1], w.shape[0], C.byref(q))
+    return out
 
 
 def make_quant(s_in, zp_in, s_w, zp_w, s_out, zp_out, act=ACT_NONE, act_enabled=False, s_bias=None):

@@ -55,6 +55,14 @@ def test_make_requant_matches_oracle_and_handles_bias_scale_mismatch():
         a = eden.make_requant(s_in, zi, s_w, zw, s_out, zo, act, en).as_tuple()
         b = O.make_quant(s_in, zi, s_w, zw, s_out, zo, act, en).as_tuple()
         assert a == b
+        a = eden.make_requant_s8(s_in, zi - 128, s_w, zw - 128, s_out, zo - 128, act, en).as_tuple()
+        b = O.make_quant_s8(s_in, zi - 128, s_w, zw - 128, s_out, zo - 128, act, en).as_tuple()
+        assert a == b
+    lib = eden.load()
+    for act, shex, zp, lo, hi in GOLD["act_range_s8"]:
+        l, h = C.c_int32(), C.c_int32()
+        lib.eh_act_range_s8(act, float.fromhex(shex), zp, C.byref(l), C.byref(h))
+        assert (l.value, h.value) == (lo, hi)
     q = eden.make_requant(0.5, 0, 0.5, 0, 1.0, 7, s_bias=1.0)  # bias scale != s_in * s_w
     assert (q.multiplier, q.shift) == (0, 0)
 

@@ -80,6 +80,14 @@ def test_act_range_closed_forms_and_golden():
     assert O.act_range_u8(O.ACT_RELU1, 0.0625, 128) == (112, 144)
     for act, shex, zp, lo, hi in GOLD["act_range_u8"]:
         assert O.act_range_u8(act, float.fromhex(shex), zp) == (lo, hi)
+    # int8 limits: RELU6 at scale 0.05 from zero point -128 ends at -128 + 120
+    assert O.act_range_s8(O.ACT_RELU6, float(np.float32(0.05)), -128) == (-128, -8)
+    assert O.act_range_s8(O.ACT_NONE, 0.05, 3) == (-128, 127)
+    for act, shex, zp, lo, hi in GOLD["act_range_s8"]:
+        assert O.act_range_s8(act, float.fromhex(shex), zp) == (lo, hi)
+        # the int8 range is the uint8 range of the zero point + 128, moved down by 128
+        ulo, uhi = O.act_range_u8(act, float.fromhex(shex), zp + 128)
+        assert (ulo - 128, uhi - 128) == (lo, hi)
 
 
 def test_srdhm_identities():
@@ -203,3 +211,5 @@ def test_against_reference_build_live():
         lo, hi = C.c_int32(), C.c_int32()
         ref.ref_act_range_u8(act, scale, zp, C.byref(lo), C.byref(hi))
         assert O.act_range_u8(act, scale, zp) == (lo.value, hi.value)
+        ref.ref_act_range_s8(act, scale, zp - 128, C.byref(lo), C.byref(hi))
+        assert O.act_range_s8(act, scale, zp - 128) == (lo.value, hi.value)

@@ -368,3 +368,37 @@ def test_perchannel_forms_reduce_to_the_per_tensor_functions(kind):
             qc = O.raw_quant(zp_in=101, zp_w=zp_w + 128, zp_out=120, multiplier=int(mults[c]), shift=int(shifts[c]),
                              act_min=3, act_max=250)
             assert np.array_equal(got[:, c], fn(x, w_u8, bias, s, qc)[:, c]), (kind, c)
+
+
+@pytest.mark.parametrize("kind", ["conv", "dw", "deconv", "fc"])
+def test_int8_precision_forms_reduce_to_the_uint8_functions(kind):
+    """An INT8-precision operator is the uint8 operator on every byte, zero point and clamp bound + 128, with the
+    result moved back by 128 (SIGNED_TO_UNSIGNED / UNSIGNED_TO_SIGNED, cl_kernels/DepthwiseconvolutionKernels.cpp:2410-2411)."""
+    rng = np.random.default_rng(99 + len(kind))
+    q8 = O.raw_quant(zp_in=-20, zp_w=3, zp_out=-7, multiplier=1518500250, shift=-8, act_min=-50, act_max=60)
+    qu = O.raw_quant(zp_in=108, zp_w=131, zp_out=121, multiplier=1518500250, shift=-8, act_min=78, act_max=188)
+    up = lambda a: (a.astype(np.int16) + 128).astype(np.uint8)
+    if kind == "fc":
+        a = rng.integers(-128, 128, (7, 40)).astype(np.int8)
+        w = rng.integers(-128, 128, (9, 40)).astype(np.int8)
+        b = rng.integers(-3000, 3000, 9).astype(np.int32)
+        got = O.fc_s8(a, w, b, q8)
+        want = O.fc(up(a), up(w), b, qu)
+    else:
+        if kind == "dw":
+            s = O.conv_shape(2, 5, 9, 8, 10, 3, 3, stride=(2, 1), pad=(1, 0, 1, 1), dm=2)
+            w_shape, f8, fu = (10, 1, 3, 3), O.dwconv2d_s8, O.dwconv2d
+        elif kind == "deconv":
+            s = O.conv_shape(2, 6, 5, 4, 8, 3, 3, stride=(2, 2), pad=(1, 0, 1, 0), groups=2)
+            w_shape, f8, fu = (6, 4, 3, 3), O.deconv2d_s8, O.deconv2d
+        else:
+            s = O.conv_shape(2, 6, 7, 6, 8, 3, 2, stride=(1, 2), pad=(1, 1, 0, 1), groups=2)
+            w_shape, f8, fu = (8, 3, 3, 2), O.conv2d_s8, O.conv2d
+        x = rng.integers(-128, 128, (s.n, s.c, s.h, s.w)).astype(np.int8)
+        w = rng.integers(-128, 128, w_shape).astype(np.int8)
+        b = rng.integers(-3000, 3000, w_shape[0] if kind != "deconv" else 8).astype(np.int32)
+        got = f8(x, w, b, s, q8)
+        want = fu(up(x), up(w), b, s, qu)
+    assert got.dtype == np.int8 and got.std() > 10
+    assert got.min() == -50 and got.max() == 60  # both clamp bounds are reached
+    assert np.array_equal(up(got), want)
