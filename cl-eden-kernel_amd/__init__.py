@@ -182,6 +182,7 @@ def add_u8(a, b, out, count, q, stream=None):
 
 def avgpool_u8(src, dst, n, c, h, w, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), layout=None, act_min=0, act_max=255,
                stream=None):
+    """layout | IO_SIGNED: int8 tensors (range within [-128, 127], mean rounded half away from zero)"""
     d = PoolDesc(n, c, h, w, kh, kw, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3],
                  NCHW if layout is None else layout, act_min, act_max)
     check(load().eh_avgpool_u8(_addr(src), _addr(dst), C.byref(d), stream))

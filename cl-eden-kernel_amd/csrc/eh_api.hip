@@ -5,8 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
-#include <new>
 #include <algorithm>
+#include <new>
 #include <vector>
 
 #include "eh_internal.h"
@@ -193,6 +193,21 @@ static int check_perchannel(const int32_t *multipliers, const int32_t *shifts, i
     return EH_OK;
 }
 
+// The per-channel arrays with `pad` zero entries behind them (kernels read whole channel blocks), written by one
+// blocking copy each from a padded host image, once the stream's earlier work that may still read the arrays is
+// done.  (A memset of the whole array followed by an asynchronous copy of its head from pageable memory left
+// zeros in place of some pairs now and then.)
+static int upload_padded_pairs(int32_t *d_mult, int32_t *d_shift, const int32_t *multipliers, const int32_t *shifts,
+                               int32_t count, int32_t pad, hipStream_t stream) {
+    std::vector<int32_t> image((size_t)count + pad, 0);
+    EH_HIP(hipStreamSynchronize(stream));
+    std::copy(multipliers, multipliers + count, image.begin());
+    EH_HIP(hipMemcpy(d_mult, image.data(), image.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+    std::copy(shifts, shifts + count, image.begin());
+    EH_HIP(hipMemcpy(d_shift, image.data(), image.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+    return EH_OK;
+}
+
 struct GemmOp {
     std::vector<GemmPart> parts;
     int32_t *bias_copy = nullptr;  // the operator's own copy of the int32 bias
@@ -208,6 +223,7 @@ struct GemmOp {
     size_t in_bytes = 0;
     // int8 weights (value = byte as signed; zp_w is then an int8 zero point) and one multiplier / shift per
     // output channel instead of the requant's single pair
+    bool has_bias = true;
     bool w_signed = false;
     bool io_signed = false;  // input and output tensors hold int8 values
     int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;
@@ -227,12 +243,7 @@ struct GemmOp {
         // padded so that the kernels may read whole channel blocks
         if (!pc_multiplier && (rc = dev_alloc(&pc_multiplier, (size_t)cout + 512))) return rc;
         if (!pc_shift && (rc = dev_alloc(&pc_shift, (size_t)cout + 512))) return rc;
-        EH_HIP(hipMemsetAsync(pc_multiplier, 0, ((size_t)cout + 512) * sizeof(int32_t), stream));
-        EH_HIP(hipMemsetAsync(pc_shift, 0, ((size_t)cout + 512) * sizeof(int32_t), stream));
-        EH_HIP(hipMemcpyAsync(pc_multiplier, multipliers, (size_t)cout * sizeof(int32_t), hipMemcpyHostToDevice, stream));
-        EH_HIP(hipMemcpyAsync(pc_shift, shifts, (size_t)cout * sizeof(int32_t), hipMemcpyHostToDevice, stream));
-        EH_HIP(hipStreamSynchronize(stream));  // the host arrays are the caller's
-        return EH_OK;
+        return upload_padded_pairs(pc_multiplier, pc_shift, multipliers, shifts, cout, 512, stream);
     }
 
     void release() {
@@ -256,10 +267,8 @@ struct GemmOp {
             int rc = pack_part(g, static_cast<const uint8_t *>(weight), w_signed, stream);
             if (rc) return rc;
         }
-        if (bias)
-            EH_HIP(hipMemcpyAsync(bias_copy, bias, (size_t)cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
-        else
-            EH_HIP(hipMemsetAsync(bias_copy, 0, (size_t)cout * sizeof(int32_t), stream));
+        has_bias = bias != nullptr;  // no bias: the fold kernel takes zeros (no memset, so that a caller may capture this)
+        if (bias) EH_HIP(hipMemcpyAsync(bias_copy, bias, (size_t)cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
         folded_valid = false;
         return EH_OK;
     }
@@ -272,7 +281,7 @@ struct GemmOp {
             return EH_OK;
         }
         for (auto &g : parts) {
-            int rc = launch_fold_bias(bias_copy + g.bias_base, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, zp_w_u8(nq),
+            int rc = launch_fold_bias(has_bias ? bias_copy + g.bias_base : nullptr, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, zp_w_u8(nq),
                                       fillbuf, io_signed ? 0x80 : 0, stream);
             if (rc) return rc;
         }
@@ -362,7 +371,7 @@ struct eh_dwconv_plan {
     int32_t *bias_folded = nullptr;
     eh_requant q{};
     bool packed_valid = false;
-    bool w_signed = false, io_signed = false;
+    bool w_signed = false, io_signed = false, has_bias = true;
     int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;  // [cout + 4] once per-channel pairs are set
 };
 
@@ -1069,10 +1078,8 @@ static void dw_release(eh_dwconv_plan *pl) {
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
     EH_REQUIRE(weight != nullptr, "weight pointer is null");
     EH_HIP(hipMemcpyAsync(pl->w_copy, weight, (size_t)pl->cout * pl->taps, hipMemcpyDeviceToDevice, stream));
-    if (bias)
-        EH_HIP(hipMemcpyAsync(pl->bias_copy, bias, (size_t)pl->cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
-    else
-        EH_HIP(hipMemsetAsync(pl->bias_copy, 0, (size_t)pl->cout * sizeof(int32_t), stream));
+    pl->has_bias = bias != nullptr;
+    if (bias) EH_HIP(hipMemcpyAsync(pl->bias_copy, bias, (size_t)pl->cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
     pl->packed_valid = false;
     return EH_OK;
 }
@@ -1080,7 +1087,7 @@ static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bi
 static int dw_refold(eh_dwconv_plan *pl, const eh_requant &caller_q, hipStream_t stream) {
     const eh_requant q = pl->io_signed ? io_as_uint8(caller_q) : caller_q;  // pl->q: the uint8-equivalent input/output side
     if (!(pl->packed_valid && q.zp_in == pl->q.zp_in && q.zp_w == pl->q.zp_w)) {
-        int rc = launch_dw_pack(pl->w_copy, pl->bias_copy, pl->w_pair, pl->bias_folded, pl->cout, pl->taps, q.zp_in,
+        int rc = launch_dw_pack(pl->w_copy, pl->has_bias ? pl->bias_copy : nullptr, pl->w_pair, pl->bias_folded, pl->cout, pl->taps, q.zp_in,
                                 q.zp_w, pl->w_signed ? 1 : 0, stream);
         if (rc) return rc;
         pl->packed_valid = true;
@@ -1152,15 +1159,10 @@ int eh_dwconv2d_u8_set_perchannel(eh_dwconv_plan *plan, const int32_t *multiplie
     int rc = check_perchannel(multipliers, shifts, count);
     if (rc) return rc;
     hipStream_t s = as_stream(stream);
-    const size_t padded = (size_t)plan->cout + 4;
+    const size_t padded = (size_t)plan->cout + 4;  // the four-channel kernels read whole quads
     if (!plan->pc_multiplier && (rc = dev_alloc(&plan->pc_multiplier, padded))) return rc;
     if (!plan->pc_shift && (rc = dev_alloc(&plan->pc_shift, padded))) return rc;
-    EH_HIP(hipMemsetAsync(plan->pc_multiplier, 0, padded * sizeof(int32_t), s));
-    EH_HIP(hipMemsetAsync(plan->pc_shift, 0, padded * sizeof(int32_t), s));
-    EH_HIP(hipMemcpyAsync(plan->pc_multiplier, multipliers, (size_t)count * sizeof(int32_t), hipMemcpyHostToDevice, s));
-    EH_HIP(hipMemcpyAsync(plan->pc_shift, shifts, (size_t)count * sizeof(int32_t), hipMemcpyHostToDevice, s));
-    EH_HIP(hipStreamSynchronize(s));  // the host arrays may go away after the call
-    return EH_OK;
+    return upload_padded_pairs(plan->pc_multiplier, plan->pc_shift, multipliers, shifts, count, 4, s);
 }
 
 int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream) {
@@ -1183,7 +1185,7 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     DwProblem p;
     p.in = static_cast<const uint8_t *>(input);
     p.w = plan->w_copy;
-    p.bias = plan->bias_copy;
+    p.bias = plan->has_bias ? plan->bias_copy : nullptr;
     p.w_pair = plan->w_pair;
     p.bias_folded = plan->bias_folded;
     p.out = static_cast<uint8_t *>(output);

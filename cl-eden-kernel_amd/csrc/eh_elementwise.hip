@@ -68,7 +68,26 @@ __global__ __launch_bounds__(256) void add_u8_kernel(const uint8_t *__restrict__
 
 struct PoolDev {
     int32_t n, c, h, w, ho, wo, kh, kw, stride_h, stride_w, pad_t, pad_l, act_min, act_max;
+    uint32_t flip;  // 0x80808080 for int8 tensors: stored byte ^ 0x80 = value + 128
 };
+
+// Window sum over (value + 128 for int8 tensors) to the stored output byte.  uint8: (sum + n/2) / n.  int8: the sum of
+// the signed values, rounded half away from zero (SIGNEDavepooling_tflite,
+// gpu/operators/cl_kernels/AveragepoolKernels.cpp:70-74), which differs from the uint8 rule at negative ties.
+__device__ __forceinline__ uint32_t pool_finish(int s, int cnt, const PoolDev &p) {
+    int v = 0;
+    if (cnt > 0) {
+        if (p.flip) {
+            s -= 128 * cnt;
+            v = s > 0 ? (s + cnt / 2) / cnt : (s - cnt / 2) / cnt;
+        } else {
+            v = (s + cnt / 2) / cnt;
+        }
+    }
+    v = v < p.act_min ? p.act_min : v;
+    v = v > p.act_max ? p.act_max : v;
+    return (uint32_t)v & 255u;
+}
 
 // channels-last: a thread owns four consecutive channels of one output pixel (c % 4 == 0)
 __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
@@ -88,6 +107,7 @@ __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *_
     const int cnt = (y1 - y0) * (x1 - x0);
     int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
     auto take = [&](uint32_t v) {
+        v ^= p.flip;
         s0 += v & 255u;
         s1 += (v >> 8) & 255u;
         s2 += (v >> 16) & 255u;
@@ -106,17 +126,12 @@ __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *_
         }
         uint32_t v[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) v[t] = x + t < x1 ? *reinterpret_cast<const uint32_t *>(row + (size_t)(x + t) * p.c) : 0u;
+        for (int t = 0; t < 8; ++t) v[t] = x + t < x1 ? *reinterpret_cast<const uint32_t *>(row + (size_t)(x + t) * p.c) : p.flip;
 #pragma unroll
         for (int t = 0; t < 8; ++t) take(v[t]);
     }
-    auto fin = [&](int s) -> uint32_t {
-        int v = cnt > 0 ? (s + cnt / 2) / cnt : 0;
-        v = v < p.act_min ? p.act_min : v;
-        v = v > p.act_max ? p.act_max : v;
-        return (uint32_t)v;
-    };
-    *reinterpret_cast<uint32_t *>(out + idx * 4) = fin(s0) | (fin(s1) << 8) | (fin(s2) << 16) | (fin(s3) << 24);
+    *reinterpret_cast<uint32_t *>(out + idx * 4) = pool_finish(s0, cnt, p) | (pool_finish(s1, cnt, p) << 8) |
+                                                   (pool_finish(s2, cnt, p) << 16) | (pool_finish(s3, cnt, p) << 24);
 }
 
 // one output element per thread, either layout
@@ -150,11 +165,9 @@ __global__ __launch_bounds__(256) void avgpool_scalar_kernel(const uint8_t *__re
     int s = 0;
     for (int y = y0; y < y1; ++y)
         for (int x = x0; x < x1; ++x)
-            s += NHWC ? in[(((size_t)img * p.h + y) * p.w + x) * p.c + ch] : in[(((size_t)img * p.c + ch) * p.h + y) * p.w + x];
-    int v = cnt > 0 ? (s + cnt / 2) / cnt : 0;
-    v = v < p.act_min ? p.act_min : v;
-    v = v > p.act_max ? p.act_max : v;
-    out[idx] = (uint8_t)v;
+            s += (NHWC ? in[(((size_t)img * p.h + y) * p.w + x) * p.c + ch] : in[(((size_t)img * p.c + ch) * p.h + y) * p.w + x]) ^
+                 (p.flip & 255u);
+    out[idx] = (uint8_t)pool_finish(s, cnt, p);
 }
 
 }  // namespace
@@ -218,13 +231,15 @@ int eh_add_u8(const void *a, const void *b, void *out, int64_t count, const eh_a
 
 int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *stream) {
     EH_REQUIRE(desc != nullptr, "avgpool: null descriptor");
-    const eh_pool_desc &d = *desc;
+    eh_pool_desc d = *desc;
+    const bool io_signed = (d.layout & EH_IO_SIGNED) != 0;
+    d.layout &= ~EH_IO_SIGNED;
     EH_REQUIRE(d.n >= 0 && d.c >= 0 && d.h >= 0 && d.w >= 0, "avgpool: negative extent");
     EH_REQUIRE(d.kh > 0 && d.kw > 0 && d.stride_h > 0 && d.stride_w > 0, "avgpool: bad window or stride");
     EH_REQUIRE(d.pad_t >= 0 && d.pad_b >= 0 && d.pad_l >= 0 && d.pad_r >= 0, "avgpool: negative padding");
     EH_REQUIRE(d.layout == EH_NCHW || d.layout == EH_NHWC, "avgpool: bad layout %d", d.layout);
-    EH_REQUIRE(d.act_min >= 0 && d.act_max <= 255 && d.act_min <= d.act_max, "avgpool: activation range [%d, %d] invalid",
-               d.act_min, d.act_max);
+    EH_REQUIRE(d.act_min >= (io_signed ? -128 : 0) && d.act_max <= (io_signed ? 127 : 255) && d.act_min <= d.act_max,
+               "avgpool: activation range [%d, %d] invalid", d.act_min, d.act_max);
     if ((int64_t)d.n * d.c * d.h * d.w == 0) return EH_OK;
     PoolDev p;
     p.n = d.n;
@@ -242,6 +257,7 @@ int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *str
     p.pad_l = d.pad_l;
     p.act_min = d.act_min;
     p.act_max = d.act_max;
+    p.flip = io_signed ? 0x80808080u : 0u;
     EH_REQUIRE(in && out, "avgpool: null tensor");
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const int64_t outputs = (int64_t)d.n * d.c * p.ho * p.wo;

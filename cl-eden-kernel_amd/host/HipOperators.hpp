@@ -134,6 +134,30 @@ inline eh_requant requantFromTensors(const std::shared_ptr<HipTensor> &in, const
     return q;
 }
 
+// PrecisionType::INT8: every tensor holds int8 bytes and the parameters are int8 values (the SIGNED* kernels,
+// cl_optimized_impls/CLGEMMConvolutionQuantized.cpp:47,224-241)
+inline eh_requant requantFromTensors(const PrecisionType &precision, const std::shared_ptr<HipTensor> &in,
+                                     const std::shared_ptr<HipTensor> &w, const std::shared_ptr<HipTensor> &bias,
+                                     const std::shared_ptr<HipTensor> &out, const ActivationInfo &act) {
+    if (precision != PrecisionType::INT8) return requantFromTensors(in, w, bias, out, act);
+    eh_requant q;
+    eh_make_requant_s8(in->getScale(), in->getZeroPoint(), w->getScale(), w->getZeroPoint(), bias->getScale(), out->getScale(),
+                       out->getZeroPoint(), toEhActivation(act), act.isEnabled() ? 1 : 0, &q);
+    return q;
+}
+
+inline bool quantizedPrecision(const PrecisionType &p) { return p == PrecisionType::UINT8 || p == PrecisionType::INT8; }
+
+// data types of {input, weight, bias, output} for a precision: uint8 everywhere (int8 weights in per-channel
+// mode), or int8 everywhere
+inline bool tensorTypesMatch(const PrecisionType &precision, bool per_channel, const std::shared_ptr<HipTensor> &in,
+                             const std::shared_ptr<HipTensor> &w, const std::shared_ptr<HipTensor> &bias,
+                             const std::shared_ptr<HipTensor> &out) {
+    const DataType io = precision == PrecisionType::INT8 ? DataType::INT8 : DataType::UINT8;
+    const DataType wt = (precision == PrecisionType::INT8 || per_channel) ? DataType::INT8 : DataType::UINT8;
+    return in->getDataType() == io && w->getDataType() == wt && bias->getDataType() == DataType::INT32 && out->getDataType() == io;
+}
+
 // Per-channel mode: int8 weights and one filter scale per output channel
 // (cl_optimized_impls/CLConvolutionPerChannelQuantized.cpp:96-120,
 // CLDepthwiseConvolutionPerChannelQuantized.cpp:133-160, CLDeconvolutionPerChannelQuantized.cpp:147-179).
@@ -145,9 +169,9 @@ struct PerChannelState {
     // weight_zp: the convolution ignores the filter's zero point, the depthwise convolution and the
     // deconvolution subtract it.  range_always: the deconvolution derives the activation range even
     // for a disabled activation.
-    eh_requant derive(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &out, const ActivationInfo &act,
-                      const std::vector<float> &scales, int32_t weight_zp, bool range_always, std::vector<int32_t> *m,
-                      std::vector<int32_t> *s) const {
+    eh_requant derive(const PrecisionType &precision, const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &out,
+                      const ActivationInfo &act, const std::vector<float> &scales, int32_t weight_zp, bool range_always,
+                      std::vector<int32_t> *m, std::vector<int32_t> *s) const {
         eh_requant q;
         m->assign(scales.size(), 0);
         s->assign(scales.size(), 0);
@@ -155,21 +179,14 @@ struct PerChannelState {
                                    out->getZeroPoint(), toEhActivation(act), (range_always || act.isEnabled()) ? 1 : 0, &q, m->data(),
                                    s->data());
         q.zp_w = weight_zp;
+        if (precision == PrecisionType::INT8) {
+            q.act_min = -128;
+            q.act_max = 127;
+            if (range_always || act.isEnabled()) eh_act_range_s8(toEhActivation(act), out->getScale(), out->getZeroPoint(), &q.act_min, &q.act_max);
+        }
         return q;
     }
 };
-
-inline bool perChannelTensors(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &w,
-                              const std::shared_ptr<HipTensor> &bias, const std::shared_ptr<HipTensor> &out) {
-    return in->getDataType() == DataType::UINT8 && w->getDataType() == DataType::INT8 &&
-           bias->getDataType() == DataType::INT32 && out->getDataType() == DataType::UINT8;
-}
-
-inline bool uint8Tensors(const std::shared_ptr<HipTensor> &in, const std::shared_ptr<HipTensor> &w,
-                         const std::shared_ptr<HipTensor> &bias, const std::shared_ptr<HipTensor> &out) {
-    return in->getDataType() == DataType::UINT8 && w->getDataType() == DataType::UINT8 &&
-           bias->getDataType() == DataType::INT32 && out->getDataType() == DataType::UINT8;
-}
 
 }  // namespace detail
 
@@ -194,13 +211,11 @@ public:
         bias_as_input_ = !bias_->is_const();
 
         if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;  // zero-sized: nothing to prepare
-        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipConvolution: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(detail::quantizedPrecision(precision_), "HipConvolution: only the UINT8 and INT8 paths exist on this backend");
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipConvolution: no texture storage");
         per_channel_ = parameters_->per_channel_quant;
-        if (per_channel_)
-            CHECK_EXPR_RETURN_FAILURE(detail::perChannelTensors(input_, weight_, bias_, output_), "HipConvolution: per-channel mode expects uint8 input/output, int8 weight and int32 bias");
-        else
-            CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipConvolution: expects uint8 input/weight/output and int32 bias");
+        CHECK_EXPR_RETURN_FAILURE(detail::tensorTypesMatch(precision_, per_channel_, input_, weight_, bias_, output_),
+                                  "HipConvolution: tensor data types do not fit the precision (uint8 tensors, int8 weights in per-channel mode; int8 tensors for INT8)");
 
         Dim4 in = input_->getDim(), wd = weight_->getDim();
         if (!parameters_->isNCHW) in = convertDimToNCHW(in);
@@ -239,6 +254,10 @@ public:
         if (per_channel_) {
             CHECK_EXPR_RETURN_FAILURE(parameters_->scales.size() == (size_t)desc_.cout, "HipConvolution: %zu filter scales for %d output channels", parameters_->scales.size(), desc_.cout);
             desc_.weight_layout |= EH_W_SIGNED;
+        }
+        if (precision_ == PrecisionType::INT8) {
+            desc_.weight_layout |= EH_W_SIGNED;
+            desc_.layout |= EH_IO_SIGNED;
         }
         eh_requant q;
         CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipConvolution::initialize: requantization parameters");
@@ -279,11 +298,11 @@ private:
     // also hands the plan the channel pairs when they differ from the ones it holds.
     Status currentRequant(eh_requant *q) {
         if (!per_channel_) {
-            *q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+            *q = detail::requantFromTensors(precision_, input_, weight_, bias_, output_, activation_info_);
             return Status::SUCCESS;
         }
         std::vector<int32_t> m, s;
-        *q = pc_.derive(input_, output_, activation_info_, parameters_->scales, 0, false, &m, &s);
+        *q = pc_.derive(precision_, input_, output_, activation_info_, parameters_->scales, 0, false, &m, &s);
         if (plan_ != nullptr && (!pc_.sent || m != pc_.multipliers || s != pc_.shifts)) {
             const int rc = eh_conv2d_u8_set_perchannel(plan_, m.data(), s.data(), (int32_t)m.size(), runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution: %s", eh_last_error());
@@ -326,13 +345,11 @@ public:
         weights_as_input_ = !weight_->is_const() || !bias_->is_const();
 
         if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
-        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipDepthwiseConvolution: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(detail::quantizedPrecision(precision_), "HipDepthwiseConvolution: only the UINT8 and INT8 paths exist on this backend");
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipDepthwiseConvolution: no texture storage");
         per_channel_ = parameters_->per_channel_quant;
-        if (per_channel_)
-            CHECK_EXPR_RETURN_FAILURE(detail::perChannelTensors(input_, weight_, bias_, output_), "HipDepthwiseConvolution: per-channel mode expects uint8 input/output, int8 weight and int32 bias");
-        else
-            CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDepthwiseConvolution: expects uint8 input/weight/output and int32 bias");
+        CHECK_EXPR_RETURN_FAILURE(detail::tensorTypesMatch(precision_, per_channel_, input_, weight_, bias_, output_),
+                                  "HipDepthwiseConvolution: tensor data types do not fit the precision (uint8 tensors, int8 weights in per-channel mode; int8 tensors for INT8)");
 
         Dim4 in = input_->getDim();
         if (!parameters_->isNCHW) in = convertDimToNCHW(in);
@@ -362,6 +379,10 @@ public:
         if (per_channel_) {
             CHECK_EXPR_RETURN_FAILURE(parameters_->scales.size() == (size_t)desc_.cout, "HipDepthwiseConvolution: %zu filter scales for %d output channels", parameters_->scales.size(), desc_.cout);
             desc_.weight_layout |= EH_W_SIGNED;
+        }
+        if (precision_ == PrecisionType::INT8) {
+            desc_.weight_layout |= EH_W_SIGNED;
+            desc_.layout |= EH_IO_SIGNED;
         }
         eh_requant q;
         CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDepthwiseConvolution::initialize: requantization parameters");
@@ -402,11 +423,11 @@ private:
     // also hands the plan the channel pairs when they differ from the ones it holds.
     Status currentRequant(eh_requant *q) {
         if (!per_channel_) {
-            *q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+            *q = detail::requantFromTensors(precision_, input_, weight_, bias_, output_, activation_info_);
             return Status::SUCCESS;
         }
         std::vector<int32_t> m, s;
-        *q = pc_.derive(input_, output_, activation_info_, parameters_->scales, weight_->getZeroPoint(), false, &m, &s);
+        *q = pc_.derive(precision_, input_, output_, activation_info_, parameters_->scales, weight_->getZeroPoint(), false, &m, &s);
         if (plan_ != nullptr && (!pc_.sent || m != pc_.multipliers || s != pc_.shifts)) {
             const int rc = eh_dwconv2d_u8_set_perchannel(plan_, m.data(), s.data(), (int32_t)m.size(), runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDepthwiseConvolution: %s", eh_last_error());
@@ -449,9 +470,10 @@ public:
         weights_as_input_ = !weight_->is_const() || !bias_->is_const();
 
         if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
-        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipFullyConnected: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(detail::quantizedPrecision(precision_), "HipFullyConnected: only the UINT8 and INT8 paths exist on this backend");
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipFullyConnected: no texture storage");
-        CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipFullyConnected: expects uint8 input/weight/output and int32 bias");
+        CHECK_EXPR_RETURN_FAILURE(detail::tensorTypesMatch(precision_, false, input_, weight_, bias_, output_),
+                                  "HipFullyConnected: expects uint8 (INT8 precision: int8) input/weight/output and int32 bias");
         // weight [units][k]; the input is flattened to [size / k][k]
         // (CLFullyConnected.cpp:46-57: in androidNN mode the batch is whatever the element count gives)
         const Dim4 wd = weight_->getDim();
@@ -461,8 +483,9 @@ public:
         CHECK_EXPR_RETURN_FAILURE(parameters_->androidNN || m == input_->getDim().n, "HipFullyConnected: input batch %u does not match %u rows of k = %u", input_->getDim().n, m, k);
         CHECK_EXPR_RETURN_FAILURE(output_->getTotalSizeFromDims() == m * units, "HipFullyConnected: output has %u elements, expected %u", output_->getTotalSizeFromDims(), m * units);
         m_ = (int32_t)m;
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
-        const int rc = eh_fc_u8_plan(&plan_, (int32_t)m, (int32_t)k, (int32_t)units, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+        const eh_requant q = detail::requantFromTensors(precision_, input_, weight_, bias_, output_, activation_info_);
+        const int32_t flags = precision_ == PrecisionType::INT8 ? (EH_W_SIGNED | EH_IO_SIGNED) : 0;
+        const int rc = eh_fc_q8_plan(&plan_, (int32_t)m, (int32_t)k, (int32_t)units, flags, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
         CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipFullyConnected::initialize: %s", eh_last_error());
         return Status::SUCCESS;
     }
@@ -473,7 +496,7 @@ public:
             return Status::SUCCESS;
         }
         if (m_ == 0) return Status::SUCCESS;
-        const eh_requant q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+        const eh_requant q = detail::requantFromTensors(precision_, input_, weight_, bias_, output_, activation_info_);
         if (weights_as_input_) {
             const int rc = eh_fc_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipFullyConnected::execute (repack): %s", eh_last_error());
@@ -523,12 +546,10 @@ public:
         weights_as_input_ = parameters_->weights_as_input || !weight_->is_const() || !bias_->is_const();
 
         if (weight_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
-        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipDeconvolution: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(detail::quantizedPrecision(precision_), "HipDeconvolution: only the UINT8 and INT8 paths exist on this backend");
         per_channel_ = parameters_->per_channel_quant;
-        if (per_channel_)
-            CHECK_EXPR_RETURN_FAILURE(detail::perChannelTensors(input_, weight_, bias_, output_), "HipDeconvolution: per-channel mode expects uint8 input/output, int8 weight and int32 bias");
-        else
-            CHECK_EXPR_RETURN_FAILURE(detail::uint8Tensors(input_, weight_, bias_, output_), "HipDeconvolution: expects uint8 input/weight/output and int32 bias");
+        CHECK_EXPR_RETURN_FAILURE(detail::tensorTypesMatch(precision_, per_channel_, input_, weight_, bias_, output_),
+                                  "HipDeconvolution: tensor data types do not fit the precision (uint8 tensors, int8 weights in per-channel mode; int8 tensors for INT8)");
 
         Dim4 in = input_->getDim();
         if (!parameters_->isNCHW) in = convertDimToNCHW(in);
@@ -565,6 +586,10 @@ public:
         if (per_channel_) {
             CHECK_EXPR_RETURN_FAILURE(parameters_->scales.size() == (size_t)desc_.cout, "HipDeconvolution: %zu filter scales for %d output channels", parameters_->scales.size(), desc_.cout);
             desc_.weight_layout |= EH_W_SIGNED;
+        }
+        if (precision_ == PrecisionType::INT8) {
+            desc_.weight_layout |= EH_W_SIGNED;
+            desc_.layout |= EH_IO_SIGNED;
         }
         eh_requant q;
         CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDeconvolution::initialize: requantization parameters");
@@ -605,11 +630,11 @@ private:
     // also hands the plan the channel pairs when they differ from the ones it holds.
     Status currentRequant(eh_requant *q) {
         if (!per_channel_) {
-            *q = detail::requantFromTensors(input_, weight_, bias_, output_, activation_info_);
+            *q = detail::requantFromTensors(precision_, input_, weight_, bias_, output_, activation_info_);
             return Status::SUCCESS;
         }
         std::vector<int32_t> m, s;
-        *q = pc_.derive(input_, output_, activation_info_, parameters_->scales, weight_->getZeroPoint(), true, &m, &s);
+        *q = pc_.derive(precision_, input_, output_, activation_info_, parameters_->scales, weight_->getZeroPoint(), true, &m, &s);
         if (plan_ != nullptr && (!pc_.sent || m != pc_.multipliers || s != pc_.shifts)) {
             const int rc = eh_deconv2d_u8_set_perchannel(plan_, m.data(), s.data(), (int32_t)m.size(), runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipDeconvolution: %s", eh_last_error());
@@ -694,11 +719,12 @@ public:
         output_ = std::static_pointer_cast<HipTensor>(output_tensors.at(0));
         parameters_ = std::dynamic_pointer_cast<Pool2DParameters>(parameters);
         CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipAveragepool: parameters are not Pool2DParameters");
-        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipAveragepool: only the UINT8 path exists on this backend");
+        CHECK_EXPR_RETURN_FAILURE(detail::quantizedPrecision(precision_), "HipAveragepool: only the UINT8 and INT8 paths exist on this backend");
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipAveragepool: no texture storage");
         CHECK_EXPR_RETURN_FAILURE(parameters_->compute_type == ComputeType::TFLite, "HipAveragepool: only the TFLite window rule");
-        CHECK_EXPR_RETURN_FAILURE(input_->getDataType() == DataType::UINT8 && output_->getDataType() == DataType::UINT8,
-                                  "HipAveragepool: expects uint8 tensors");
+        const DataType io = precision_ == PrecisionType::INT8 ? DataType::INT8 : DataType::UINT8;
+        CHECK_EXPR_RETURN_FAILURE(input_->getDataType() == io && output_->getDataType() == io,
+                                  "HipAveragepool: expects uint8 tensors (INT8 precision: int8)");
         const Dim4 id = input_->getDim();
         const bool nchw = parameters_->isNCHW;
         d_.n = (int32_t)id.n;
@@ -713,7 +739,7 @@ public:
         d_.pad_b = (int32_t)parameters_->padding.b;
         d_.pad_l = (int32_t)parameters_->padding.l;
         d_.pad_r = (int32_t)parameters_->padding.r;
-        d_.layout = nchw ? EH_NCHW : EH_NHWC;
+        d_.layout = (nchw ? EH_NCHW : EH_NHWC) | (precision_ == PrecisionType::INT8 ? EH_IO_SIGNED : 0);
         CHECK_EXPR_RETURN_FAILURE(d_.kh > 0 && d_.kw > 0 && d_.stride_h > 0 && d_.stride_w > 0, "HipAveragepool: bad window or stride");
         const int32_t ho = (d_.h + d_.pad_t + d_.pad_b - d_.kh) / d_.stride_h + 1, wo = (d_.w + d_.pad_l + d_.pad_r - d_.kw) / d_.stride_w + 1;
         CHECK_EXPR_RETURN_FAILURE((uint64_t)output_->getTotalSizeFromDims() == (uint64_t)d_.n * d_.c * ho * wo,
@@ -726,8 +752,9 @@ public:
         CHECK_EXPR_RETURN_FAILURE(ready_, "HipAveragepool::execute before initialize");
         eh_pool_desc d = d_;
         // the range comes from the activation type alone, as in CLAveragepool::averagepool_quant (CLAveragepool.cpp:183-198)
-        eh_act_range_u8(detail::toEhActivation(parameters_->activation_info), output_->getScale(), output_->getZeroPoint(), &d.act_min,
-                        &d.act_max);
+        (precision_ == PrecisionType::INT8 ? eh_act_range_s8 : eh_act_range_u8)(detail::toEhActivation(parameters_->activation_info),
+                                                                                output_->getScale(), output_->getZeroPoint(),
+                                                                                &d.act_min, &d.act_max);
         const int rc = eh_avgpool_u8(input_->getDataPtr(), output_->getDataPtr(), &d, runtime_->stream());
         CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipAveragepool::execute: %s", eh_last_error());
         return Status::SUCCESS;

@@ -7,6 +7,7 @@
 //
 //   ud_op_test              run everything (needs the GPU)
 //   ud_op_test --host-only  buffer-pool bookkeeping and argument checks that touch no device
+//   ud_op_test --filter T   only the tests whose name contains T
 #include <cstdio>
 #include <cstring>
 #include <functional>
@@ -21,6 +22,7 @@ using namespace enn::ud;
 using namespace enn::ud::hip;
 
 static int g_failed = 0, g_run = 0;
+static const char *g_filter = nullptr;  // --filter TEXT: run only the tests whose name contains TEXT
 #define EXPECT(cond)                                                                    \
     do {                                                                                \
         if (!(cond)) {                                                                  \
@@ -30,6 +32,7 @@ static int g_failed = 0, g_run = 0;
     } while (0)
 
 static void run_test(const char *name, const std::function<bool()> &fn) {
+    if (g_filter && !std::strstr(name, g_filter)) return;
     std::printf("[ RUN  ] %s\n", name);
     std::fflush(stdout);
     ++g_run;
@@ -54,7 +57,14 @@ static bool same(const std::vector<uint8_t> &a, const std::vector<uint8_t> &b) {
     size_t bad = 0, first = 0;
     for (size_t i = 0; i < a.size(); ++i)
         if (a[i] != b[i] && bad++ == 0) first = i;
-    if (bad) std::printf("    %zu of %zu bytes differ; first at %zu: got %u want %u\n", bad, a.size(), first, a[first], b[first]);
+    if (bad) {
+        std::printf("    %zu of %zu bytes differ; first at %zu: got %u want %u\n", bad, a.size(), first, a[first], b[first]);
+        std::printf("    got :");
+        for (size_t i = first; i < a.size() && i < first + 16; ++i) std::printf(" %3u", a[i]);
+        std::printf("\n    want:");
+        for (size_t i = first; i < b.size() && i < first + 16; ++i) std::printf(" %3u", b[i]);
+        std::printf("\n");
+    }
     return bad == 0;
 }
 static bool varied(const std::vector<uint8_t> &v) {
@@ -785,6 +795,167 @@ static int gpu_tests() {
         return ok;
     });
 
+
+    // ------------------------------------------------------------ INT8 precision
+    const PrecisionType S8 = PrecisionType::INT8;
+    run_test("Int8.Convolution_channels_last_relu_and_planar_grouped", [&] {
+        bool ok = true;
+        for (int variant = 0; variant < 2; ++variant) {
+            const bool nchw = variant == 1;
+            const eo_conv_shape s = nchw ? shape(1, 12, 10, 10, 12, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 3) : shape(2, 32, 12, 12, 48, 3, 3, 2, 2, 1, 1, 1, 1);
+            const int cig = s.c / s.groups;
+            const int ho = eo_conv_out_dim(s.h, s.pad_t, s.pad_b, s.kh, 1, s.stride_h), wo = eo_conv_out_dim(s.w, s.pad_l, s.pad_r, s.kw, 1, s.stride_w);
+            auto x = to_i8(rand_u8((size_t)s.n * s.c * s.h * s.w, 301 + variant));
+            auto w = to_i8(rand_u8((size_t)s.cout * cig * 9, 303 + variant));
+            auto b = rand_i32(s.cout, 305, -1000, 1000);
+            const float s_in = 0.02f, s_w = 0.005f, s_out = 0.2f;
+            eo_quant q;
+            eo_make_quant_s8(s_in, -9, s_w, 4, s_in * s_w, s_out, -20, EO_ACT_RELU, 1, &q);
+            std::vector<int8_t> want((size_t)s.n * s.cout * ho * wo), got(want.size());
+            eo_conv2d_s8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr, nullptr);
+            const DataOrder order = nchw ? DataOrder::NCHW : DataOrder::NHWC;
+            Dim4 in_dim = nchw ? Dim4{(uint32_t)s.n, (uint32_t)s.c, (uint32_t)s.h, (uint32_t)s.w} : Dim4{(uint32_t)s.n, (uint32_t)s.h, (uint32_t)s.w, (uint32_t)s.c};
+            Dim4 out_dim = nchw ? Dim4{(uint32_t)s.n, (uint32_t)s.cout, (uint32_t)ho, (uint32_t)wo} : Dim4{(uint32_t)s.n, (uint32_t)ho, (uint32_t)wo, (uint32_t)s.cout};
+            Dim4 w_dim = nchw ? Dim4{(uint32_t)s.cout, (uint32_t)cig, 3, 3} : Dim4{(uint32_t)s.cout, 3, 3, (uint32_t)cig};
+            std::vector<int8_t> w_dev = w;
+            if (!nchw)
+                for (int o = 0; o < s.cout; ++o)
+                    for (int c = 0; c < cig; ++c)
+                        for (int t = 0; t < 9; ++t) w_dev[((size_t)o * 9 + t) * cig + c] = w[((size_t)o * cig + c) * 9 + t];
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, S8, DataType::INT8, in_dim, order, s_in, -9);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, S8, w_dev.data(), w_dim, order, s_w, 4);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, S8, b.data(), Dim4{1, (uint32_t)s.cout, 1, 1}, DataOrder::NCHW, s_in * s_w, 0);
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, S8, DataType::INT8, out_dim, order, s_out, -20);
+            auto params = std::make_shared<ConvolutionParameters>();
+            params->padding = {1, 1, 1, 1};
+            params->stride = {(uint32_t)s.stride_h, (uint32_t)s.stride_w};
+            params->group_size = s.groups;
+            params->isNCHW = nchw;
+            params->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU, true);
+            HipConvolution conv(rt, S8);
+            EXPECT(conv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+            std::vector<int8_t> x_dev = x;
+            if (!nchw) {
+                auto t = nchw_to_nhwc(std::vector<uint8_t>(x.begin(), x.end()), s.n, s.c, s.h, s.w);
+                x_dev.assign(t.begin(), t.end());
+            }
+            EXPECT(input->writeData(x_dev.data()) == Status::SUCCESS);
+            EXPECT(conv.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            std::vector<uint8_t> g8(got.begin(), got.end()), w8(want.begin(), want.end());
+            if (!nchw) g8 = nhwc_to_nchw(g8, s.n, s.cout, ho, wo);
+            EXPECT(same(g8, w8));
+            EXPECT(varied(w8));
+        }
+        return ok;
+    });
+
+    run_test("Int8.Depthwise_FullyConnected_Deconvolution_Averagepool", [&] {
+        bool ok = true;
+        const float s_in = 0.02f, s_w = 0.005f;
+        {  // depthwise 3x3 stride 1, channels-last
+            const int c = 16, h = 9, wd = 10;
+            const eo_conv_shape s = shape(2, c, h, wd, c, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1);
+            auto x = to_i8(rand_u8((size_t)2 * c * h * wd, 311)), w = to_i8(rand_u8((size_t)c * 9, 312));
+            auto b = rand_i32(c, 313, -300, 300);
+            eo_quant q;
+            eo_make_quant_s8(s_in, 7, s_w, -2, s_in * s_w, 0.05f, -128, EO_ACT_RELU6, 1, &q);
+            std::vector<int8_t> want((size_t)2 * c * h * wd), got(want.size());
+            eo_dwconv2d_s8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr, nullptr);
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{2, (uint32_t)h, (uint32_t)wd, (uint32_t)c}, DataOrder::NHWC, s_in, 7);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, S8, w.data(), Dim4{(uint32_t)c, 1, 3, 3}, DataOrder::NCHW, s_w, -2);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, S8, b.data(), Dim4{1, (uint32_t)c, 1, 1}, DataOrder::NCHW, s_in * s_w, 0);
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{2, (uint32_t)h, (uint32_t)wd, (uint32_t)c}, DataOrder::NHWC, 0.05f, -128);
+            auto params = std::make_shared<DepthwiseConvolutionParameters>();
+            params->padding = {1, 1, 1, 1};
+            params->isNCHW = false;
+            params->activation_info = std::make_shared<ActivationInfo>(ActivationInfo::ActivationType::RELU6, true);
+            HipDepthwiseConvolution dw(rt, S8);
+            EXPECT(dw.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+            auto t = nchw_to_nhwc(std::vector<uint8_t>(x.begin(), x.end()), 2, c, h, wd);
+            EXPECT(input->writeData(t.data()) == Status::SUCCESS);
+            EXPECT(dw.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(nhwc_to_nchw(std::vector<uint8_t>(got.begin(), got.end()), 2, c, h, wd), std::vector<uint8_t>(want.begin(), want.end())));
+            EXPECT(varied(std::vector<uint8_t>(want.begin(), want.end())));
+        }
+        {  // fully connected
+            const int m = 33, k = 200, n = 70;
+            auto a = to_i8(rand_u8((size_t)m * k, 321)), w = to_i8(rand_u8((size_t)n * k, 322));
+            auto b = rand_i32(n, 323, -1000, 1000);
+            eo_quant q;
+            eo_make_quant_s8(s_in, -3, s_w, 0, s_in * s_w, 0.6f, 11, 0, 0, &q);
+            std::vector<int8_t> want((size_t)m * n), got(want.size());
+            eo_fc_s8(a.data(), w.data(), b.data(), want.data(), m, k, n, &q);
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{(uint32_t)m, (uint32_t)k, 1, 1}, DataOrder::NCHW, s_in, -3);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, S8, w.data(), Dim4{(uint32_t)n, (uint32_t)k, 1, 1}, DataOrder::NCHW, s_w, 0);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, S8, b.data(), Dim4{(uint32_t)n, 1, 1, 1}, DataOrder::NCHW, s_in * s_w, 0);
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{(uint32_t)m, (uint32_t)n, 1, 1}, DataOrder::NCHW, 0.6f, 11);
+            HipFullyConnected fc(rt, S8);
+            EXPECT(fc.initialize({input, weight, bias}, {output}, std::make_shared<FullyConnectedParameters>()) == Status::SUCCESS);
+            EXPECT(input->writeData(a.data()) == Status::SUCCESS);
+            EXPECT(fc.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(std::vector<uint8_t>(got.begin(), got.end()), std::vector<uint8_t>(want.begin(), want.end())));
+            EXPECT(varied(std::vector<uint8_t>(want.begin(), want.end())));
+        }
+        {  // deconvolution 2x2 stride 2, planar
+            const eo_conv_shape s = shape(1, 24, 6, 5, 16, 2, 2, 2, 2);
+            auto x = to_i8(rand_u8((size_t)24 * 30, 331)), w = to_i8(rand_u8((size_t)24 * 16 * 4, 332));
+            auto b = rand_i32(16, 333, -500, 500);
+            eo_quant q;
+            eo_make_quant_s8(s_in, 5, s_w, 1, s_in * s_w, 0.12f, -4, 0, 0, &q);
+            std::vector<int8_t> want((size_t)16 * 12 * 10), got(want.size());
+            eo_deconv2d_s8(x.data(), w.data(), b.data(), want.data(), &s, &q, nullptr, nullptr);
+            std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{1, 24, 6, 5}, DataOrder::NCHW, s_in, 5);
+            std::shared_ptr<ITensor> weight = std::make_shared<HipTensor>(rt, S8, w.data(), Dim4{24, 16, 2, 2}, DataOrder::NCHW, s_w, 1);
+            std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, S8, b.data(), Dim4{1, 16, 1, 1}, DataOrder::NCHW, s_in * s_w, 0);
+            std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{1, 16, 12, 10}, DataOrder::NCHW, 0.12f, -4);
+            auto params = std::make_shared<DeconvolutionParameters>();
+            params->stride = {2, 2};
+            HipDeconvolution deconv(rt, S8);
+            EXPECT(deconv.initialize({input, weight, bias}, {output}, params) == Status::SUCCESS);
+            EXPECT(input->writeData(x.data()) == Status::SUCCESS);
+            EXPECT(deconv.execute() == Status::SUCCESS);
+            EXPECT(output->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(std::vector<uint8_t>(got.begin(), got.end()), std::vector<uint8_t>(want.begin(), want.end())));
+            EXPECT(varied(std::vector<uint8_t>(want.begin(), want.end())));
+        }
+        {  // average pool 3x3 stride 2 with padding, planar
+            auto x = to_i8(rand_u8((size_t)2 * 6 * 9 * 9, 341));
+            std::vector<int8_t> want((size_t)2 * 6 * 5 * 5), got(want.size());
+            eo_avgpool_s8(x.data(), want.data(), 2, 6, 9, 9, 3, 3, 2, 2, 1, 1, 1, 1, -128, 127);
+            std::shared_ptr<ITensor> ti = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{2, 6, 9, 9}, DataOrder::NCHW, 0.1f, 3);
+            std::shared_ptr<ITensor> to = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{2, 6, 5, 5}, DataOrder::NCHW, 0.1f, 3);
+            auto params = std::make_shared<Pool2DParameters>();
+            params->padding = {1, 1, 1, 1};
+            params->stride = {2, 2};
+            params->filter = {3, 3};
+            HipAveragepool pool(rt, S8);
+            EXPECT(pool.initialize({ti}, {to}, params) == Status::SUCCESS);
+            EXPECT(ti->writeData(x.data()) == Status::SUCCESS);
+            EXPECT(pool.execute() == Status::SUCCESS);
+            EXPECT(to->readData(got.data()) == Status::SUCCESS);
+            EXPECT(same(std::vector<uint8_t>(got.begin(), got.end()), std::vector<uint8_t>(want.begin(), want.end())));
+        }
+        return ok;
+    });
+
+    run_test("Int8.TensorTypesMustFitThePrecision", [&] {
+        bool ok = true;
+        std::vector<uint8_t> wu(8 * 8 * 9, 1);
+        std::vector<int32_t> b(8, 0);
+        std::shared_ptr<ITensor> input = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{1, 8, 6, 6}, DataOrder::NCHW, 0.5f, 0);
+        std::shared_ptr<ITensor> weight_u8 = std::make_shared<HipTensor>(rt, S8, wu.data(), Dim4{8, 8, 3, 3});
+        std::shared_ptr<ITensor> bias = std::make_shared<HipTensor>(rt, S8, b.data(), Dim4{1, 8, 1, 1});
+        std::shared_ptr<ITensor> output = std::make_shared<HipTensor>(rt, S8, DataType::INT8, Dim4{1, 8, 4, 4}, DataOrder::NCHW, 1.0f, 0);
+        HipConvolution conv(rt, S8);
+        EXPECT(conv.initialize({input, weight_u8, bias}, {output}, std::make_shared<ConvolutionParameters>()) == Status::FAILURE);
+        HipConvolution fp(rt, PrecisionType::FP16);
+        EXPECT(fp.initialize({input, weight_u8, bias}, {output}, std::make_shared<ConvolutionParameters>()) == Status::FAILURE);
+        return ok;
+    });
+
     std::printf("%d of %d GPU operator tests failed\n", g_failed, g_run);
     return g_failed ? 1 : 0;
 }
@@ -837,6 +1008,7 @@ static int host_tests() {
 }
 
 int main(int argc, char **argv) {
+    if (argc > 2 && std::strcmp(argv[1], "--filter") == 0) g_filter = argv[2];
     if (argc > 1 && std::strcmp(argv[1], "--host-only") == 0) return host_tests();
     const int rc = host_tests();
     return rc ? rc : gpu_tests();

@@ -196,7 +196,10 @@ int eh_transpose_u8_nhwc2nchw(const void *src, void *dst, int32_t n, int32_t c, 
  * the quantized add kernel (gpu/operators/cl_kernels/AddKernelsQauntized.cpp:135-215)
  * over `count` bytes of two equally shaped tensors; eh_avgpool_u8 is
  * avepooling_tflite_INT8 (gpu/operators/cl_kernels/AveragepoolKernels.cpp:8-44):
- * windows clipped to the image, (sum + count / 2) / count, clamp.  Both are
+ * windows clipped to the image, (sum + count / 2) / count, clamp; with EH_IO_SIGNED or-ed into
+ * eh_pool_desc.layout it is SIGNEDavepooling_tflite_INT8 (:64-85): int8 bytes, a clamp range within
+ * [-128, 127], the signed mean rounded half away from zero.  The int8 Add of the reference
+ * (SIGNEDeltwiseAddQuantized, AddKernelsQauntized.cpp:97-127) is a float kernel and is not offered.  Both are
  * asynchronous on `stream` and may be captured in a graph. */
 void eh_make_add_requant(float scale_a, int32_t zp_a, float scale_b, int32_t zp_b, float scale_out, int32_t zp_out,
                          int activation, int activation_enabled, eh_add_requant *out);

@@ -611,6 +611,33 @@ void eo_avgpool_u8(const uint8_t *in, uint8_t *out, int32_t n, int32_t c, int32_
             }
 }
 
+/* cl_kernels/AveragepoolKernels.cpp:8-38 with the int8 rounding of :70-74: the signed sum is rounded half away from
+ * zero by C's truncating division. */
+void eo_avgpool_s8(const int8_t *in, int8_t *out, int32_t n, int32_t c, int32_t h, int32_t w,
+                   int32_t kh, int32_t kw, int32_t stride_h, int32_t stride_w,
+                   int32_t pad_t, int32_t pad_b, int32_t pad_l, int32_t pad_r,
+                   int32_t act_min, int32_t act_max) {
+    const int32_t Ho = (h + pad_t + pad_b - kh) / stride_h + 1;
+    const int32_t Wo = (w + pad_l + pad_r - kw) / stride_w + 1;
+    for (int64_t p = 0; p < (int64_t)n * c; ++p)
+        for (int32_t oy = 0; oy < Ho; ++oy)
+            for (int32_t ox = 0; ox < Wo; ++ox) {
+                int32_t y0 = oy * stride_h - pad_t, x0 = ox * stride_w - pad_l;
+                int32_t y1 = y0 + kh < h ? y0 + kh : h, x1 = x0 + kw < w ? x0 + kw : w;
+                if (y0 < 0) y0 = 0;
+                if (x0 < 0) x0 = 0;
+                const int32_t cnt = (y1 - y0) * (x1 - x0);
+                int32_t sum = 0;
+                for (int32_t y = y0; y < y1; ++y)
+                    for (int32_t x = x0; x < x1; ++x) sum += in[(p * h + y) * w + x];
+                int32_t v = 0;
+                if (cnt > 0) v = sum > 0 ? (sum + cnt / 2) / cnt : (sum - cnt / 2) / cnt;
+                if (v < act_min) v = act_min;
+                if (v > act_max) v = act_max;
+                out[(p * Ho + oy) * Wo + ox] = (int8_t)v;
+            }
+}
+
 /* ------------------------------------------------------------------------ */
 /* seeded data                                                              */
 /* ------------------------------------------------------------------------ */

@@ -30,7 +30,8 @@
  *                            pinned by reduction: the result + 128 equals the uint8 function above on every byte,
  *                                    zero point and clamp bound + 128; no reference vector exists for them
  *   eo_nchw2nhwc_u8 / eo_nhwc2nchw_u8  pinned: round trip + index closed form
- *   eo_add_u8 / eo_avgpool_u8           parity unpinned by reference vectors (closed-form checks only)
+ *   eo_add_u8 / eo_avgpool_u8 / eo_avgpool_s8
+ *                            parity unpinned by reference vectors (closed-form checks only)
  */
 #ifndef EDEN_ORACLE_H_
 #define EDEN_ORACLE_H_
@@ -142,6 +143,10 @@ void eo_make_add_quant(float s_a, int32_t zp_a, float s_b, int32_t zp_b, float s
                        int act, int act_enabled, eo_add_quant *q);
 void eo_add_u8(const uint8_t *a, const uint8_t *b, uint8_t *out, int64_t count, const eo_add_quant *q);
 void eo_avgpool_u8(const uint8_t *in, uint8_t *out, int32_t n, int32_t c, int32_t h, int32_t w,
+                   int32_t kh, int32_t kw, int32_t stride_h, int32_t stride_w,
+                   int32_t pad_t, int32_t pad_b, int32_t pad_l, int32_t pad_r,
+                   int32_t act_min, int32_t act_max);
+void eo_avgpool_s8(const int8_t *in, int8_t *out, int32_t n, int32_t c, int32_t h, int32_t w,
                    int32_t kh, int32_t kw, int32_t stride_h, int32_t stride_w,
                    int32_t pad_t, int32_t pad_b, int32_t pad_l, int32_t pad_r,
                    int32_t act_min, int32_t act_max);

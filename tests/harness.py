@@ -28,7 +28,7 @@ def gpu_conv(x_nchw, w, bias, s, q, layout=eden.NCHW, weight_layout=eden.W_OIHW,
                           (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), s.groups, 1, layout, weight_layout)
     x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
     w_dev = w if weight_layout == eden.W_OIHW else w.transpose(0, 2, 3, 1)
-    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), eden.DeviceBuffer(host=bias)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), (eden.DeviceBuffer(host=bias) if bias is not None else None)
     d_o = eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
     plan = eden.ConvPlan(desc, d_w, d_b, q)
     for _ in range(runs):
@@ -47,7 +47,7 @@ def gpu_dwconv(x_nchw, w, bias, s, q, layout=eden.NCHW):
     desc = eden.conv_desc(s.n, s.c, s.h, s.w, cout, s.kh, s.kw, (s.stride_h, s.stride_w),
                           (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), 1, max(s.dm, 1), layout, eden.W_OIHW)
     x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
-    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=bias)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), (eden.DeviceBuffer(host=bias) if bias is not None else None)
     d_o = eden.DeviceBuffer(nbytes=s.n * cout * ho * wo)
     plan = eden.DwConvPlan(desc, d_w, d_b, q)
     plan.run(d_x, d_o, q)
@@ -65,7 +65,7 @@ def gpu_deconv(x_nchw, w_iohw, bias, s, q, layout=eden.NCHW, weight_layout=eden.
                           (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (1, 1), s.groups, 1, layout, weight_layout)
     x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
     w_dev = w_iohw if weight_layout == eden.W_IOHW else w_iohw.transpose(1, 2, 3, 0)
-    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), eden.DeviceBuffer(host=bias)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), (eden.DeviceBuffer(host=bias) if bias is not None else None)
     d_o = eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
     plan = eden.DeconvPlan(desc, d_w, d_b, q)
     plan.run(d_x, d_o, q)
@@ -80,7 +80,7 @@ def gpu_deconv(x_nchw, w_iohw, bias, s, q, layout=eden.NCHW, weight_layout=eden.
 def gpu_fc(a, w, bias, q):
     m, k = a.shape
     n = w.shape[0]
-    d_a, d_w, d_b = eden.DeviceBuffer(host=a), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=bias)
+    d_a, d_w, d_b = eden.DeviceBuffer(host=a), eden.DeviceBuffer(host=w), (eden.DeviceBuffer(host=bias) if bias is not None else None)
     d_o = eden.DeviceBuffer(nbytes=m * n)
     plan = eden.FcPlan(m, k, n, d_w, d_b, q)
     plan.run(d_a, d_o, q)

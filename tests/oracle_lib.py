@@ -76,6 +76,7 @@ def _load():
         "eo_make_add_quant": (None, [f32, i32, f32, i32, f32, i32, C.c_int, C.c_int, P(AddQuant)]),
         "eo_add_u8": (None, [vp, vp, vp, i64, P(AddQuant)]),
         "eo_avgpool_u8": (None, [vp, vp] + [i32] * 14),
+        "eo_avgpool_s8": (None, [vp, vp] + [i32] * 14),
         "eo_splitmix64": (u64, [u64, u64]),
         "eo_fill_u8": (None, [vp, i64, u64, i32, i32]),
         "eo_fill_i32": (None, [vp, i64, u64, i32, i32]),
@@ -328,6 +329,17 @@ def avgpool(x, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), act_min=0, act_max=255):
     wo = (w + pad[2] + pad[3] - kw) // stride[1] + 1
     out = np.zeros((n, c, ho, wo), np.uint8)
     lib.eo_avgpool_u8(_ptr(x), _ptr(out), n, c, h, w, kh, kw, stride[0], stride[1],
+                      pad[0], pad[1], pad[2], pad[3], act_min, act_max)
+    return out
+
+
+def avgpool_s8(x, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), act_min=-128, act_max=127):
+    x = _c(x, np.int8)
+    n, c, h, w = x.shape
+    ho = (h + pad[0] + pad[1] - kh) // stride[0] + 1
+    wo = (w + pad[2] + pad[3] - kw) // stride[1] + 1
+    out = np.zeros((n, c, ho, wo), np.int8)
+    lib.eo_avgpool_s8(_ptr(x), _ptr(out), n, c, h, w, kh, kw, stride[0], stride[1],
                       pad[0], pad[1], pad[2], pad[3], act_min, act_max)
     return out
 

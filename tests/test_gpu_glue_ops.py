@@ -88,3 +88,23 @@ def test_avgpool_matches_oracle(case, layout):
     got = d_out.download((n, ho, wo, c)).transpose(0, 3, 1, 2) if nhwc else d_out.download(want.shape)
     assert np.array_equal(got, want)
     assert want.std() > 1
+
+
+@pytest.mark.parametrize("layout", ["nchw", "nhwc"])
+@pytest.mark.parametrize("case", POOL_CASES, ids=lambda c: "x".join(str(v) for v in c[:6]))
+def test_avgpool_int8_matches_oracle(case, layout):
+    print("avgpool int8", case, layout, flush=True)
+    n, c, h, w, kh, kw, stride, pad, (lo, hi) = case
+    lo, hi = lo - 128, hi - 128
+    x = (synth.fill_u8((n, c, h, w), SEED + c + h + 1).astype(np.int16) - 128).astype(np.int8)
+    x[0, 0, :2, :2] = np.array([[-1, 0], [0, -1]], np.int8)  # a negative tie in the first window
+    want = O.avgpool_s8(x, kh, kw, stride, pad, lo, hi)
+    nhwc = layout == "nhwc"
+    src = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if nhwc else x
+    d_in = eden.DeviceBuffer(host=src)
+    d_out = eden.DeviceBuffer(nbytes=want.size)
+    eden.avgpool_u8(d_in, d_out, n, c, h, w, kh, kw, stride, pad, (eden.NHWC if nhwc else eden.NCHW) | eden.IO_SIGNED, lo, hi)
+    ho, wo = want.shape[2:]
+    got = d_out.download((n, ho, wo, c)).transpose(0, 3, 1, 2) if nhwc else d_out.download(want.shape)
+    assert np.array_equal(np.ascontiguousarray(got).view(np.int8), want)
+    assert want.std() > 1

@@ -487,3 +487,37 @@ def test_fc_full_size_properties():
     got1 = gpu_fc(a, w, b, to_eh_requant(q))
     got2 = gpu_fc(np.ascontiguousarray(a[:, perm]), np.ascontiguousarray(w[:, perm]), b, to_eh_requant(q))
     assert np.array_equal(got1, got2)
+
+
+def test_operators_without_a_bias_tensor():
+    """A null bias pointer is a bias of zeros in every operator; setting a bias later through repack is honoured."""
+    q = O.raw_quant(zp_in=117, zp_w=131, zp_out=128, multiplier=1518500250, shift=-9)
+    eq = to_eh_requant(q)
+    s = O.conv_shape(2, 32, 9, 9, 48, 3, 3, pad=(1, 1, 1, 1))
+    x, w = synth.fill_u8((2, 32, 9, 9), SEED + 901), synth.fill_u8_normal((48, 32, 3, 3), SEED + 902, 131, 20)
+    zeros = np.zeros(48, np.int32)
+    assert np.array_equal(gpu_conv(x, w, None, s, eq, eden.NHWC), O.conv2d(x, w, zeros, s, q))
+    sd = O.conv_shape(2, 16, 9, 9, 16, 3, 3, pad=(1, 1, 1, 1), dm=1)
+    wd = synth.fill_u8_normal((16, 1, 3, 3), SEED + 903, 131, 40)
+    xd = synth.fill_u8((2, 16, 9, 9), SEED + 904)
+    qd = O.raw_quant(zp_in=117, zp_w=131, zp_out=128, multiplier=1518500250, shift=-6)
+    for layout in (eden.NHWC, eden.NCHW):
+        assert np.array_equal(gpu_dwconv(xd, wd, None, sd, to_eh_requant(qd), layout), O.dwconv2d(xd, wd, np.zeros(16, np.int32), sd, qd))
+    st = O.conv_shape(1, 32, 5, 5, 24, 2, 2, stride=(2, 2))
+    wt = synth.fill_u8_normal((32, 24, 2, 2), SEED + 905, 131, 20)
+    xt = synth.fill_u8((1, 32, 5, 5), SEED + 906)
+    assert np.array_equal(gpu_deconv(xt, wt, None, st, eq, eden.NHWC), O.deconv2d(xt, wt, np.zeros(24, np.int32), st, q))
+    a, wf = synth.fill_u8((9, 96), SEED + 907), synth.fill_u8_normal((40, 96), SEED + 908, 131, 20)
+    assert np.array_equal(gpu_fc(a, wf, None, eq), O.fc(a, wf, np.zeros(40, np.int32), q))
+    # repack: none -> some -> none
+    b = synth.fill_i32((48,), SEED + 909, -4000, 4000)
+    desc = eden.conv_desc(2, 32, 9, 9, 48, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, 1, eden.NHWC, eden.W_OIHW)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x.transpose(0, 2, 3, 1)), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+    d_o = eden.DeviceBuffer(nbytes=2 * 48 * 81)
+    plan = eden.ConvPlan(desc, d_w, None, eq)
+    for bias_buf, bias_host in ((d_b, b), (None, zeros)):
+        plan.repack(d_w, bias_buf, eq)
+        plan.run(d_x, d_o, eq)
+        got = d_o.download((2, 9, 9, 48)).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, O.conv2d(x, w, bias_host, s, q))
+    plan.destroy()

@@ -334,6 +334,31 @@ def test_avgpool_closed_forms():
     assert o[0, 0, 0, 0] == (0 + 1 + 4 + 5 + 2) // 4
 
 
+def test_avgpool_int8_rounds_half_away_from_zero():
+    """parity unpinned by reference vectors.  The int8 pool rounds the signed mean half away from zero, so it is not
+    the uint8 pool on bytes + 128: (-1 + 0) / 2 gives -1 there, while (127 + 128 + 1) / 2 - 128 gives 0."""
+    x = np.array([-1, 0, 1, 2, -3, -4, -5, -8], np.int8).reshape(1, 1, 2, 4)
+    assert O.avgpool_s8(x, 1, 2, stride=(1, 2)).reshape(-1).tolist() == [-1, 2, -4, -7]  # -0.5, 1.5, -3.5, -6.5
+    assert O.avgpool_s8(x, 2, 4).reshape(-1).tolist() == [-2]  # -18 / 8 = -2.25
+    assert O.avgpool_s8(x, 2, 4, act_min=-1, act_max=5).reshape(-1).tolist() == [-1]
+    rng = np.random.default_rng(5)
+    y = rng.integers(-128, 128, (2, 3, 9, 7)).astype(np.int8)
+    got = O.avgpool_s8(y, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1)).astype(np.int64)
+    # against exact rational arithmetic: |got - mean| <= 1/2, ties away from zero
+    from fractions import Fraction
+    for n in range(2):
+        for c in range(3):
+            for oy in range(got.shape[2]):
+                for ox in range(got.shape[3]):
+                    ys = [v for v in range(oy * 2 - 1, oy * 2 + 2) if 0 <= v < 9]
+                    xs = [v for v in range(ox * 2 - 1, ox * 2 + 2) if 0 <= v < 7]
+                    mean = Fraction(int(sum(int(y[n, c, a, b]) for a in ys for b in xs)), len(ys) * len(xs))
+                    g = int(got[n, c, oy, ox])
+                    assert abs(g - mean) <= Fraction(1, 2)
+                    if abs(g - mean) == Fraction(1, 2):
+                        assert abs(g) > abs(mean)
+
+
 def _perchannel_pairs(rng, cout):
     mults = rng.integers(1 << 30, (1 << 31) - 1, cout).astype(np.int32)
     shifts = rng.integers(-12, -4, cout).astype(np.int32)
