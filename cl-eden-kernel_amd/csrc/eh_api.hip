@@ -333,12 +333,14 @@ struct GemmOp {
     }
 };
 
-int check_desc_common(const eh_conv_desc *d) {
+int check_desc_common(const eh_conv_desc *d, bool negative_tail_padding = false) {
     EH_REQUIRE(d != nullptr, "descriptor is null");
     EH_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->cout > 0, "bad tensor extents n=%d c=%d h=%d w=%d cout=%d",
                d->n, d->c, d->h, d->w, d->cout);
     EH_REQUIRE(d->kh > 0 && d->kw > 0 && d->stride_h > 0 && d->stride_w > 0, "bad kernel/stride");
-    EH_REQUIRE(d->pad_t >= 0 && d->pad_b >= 0 && d->pad_l >= 0 && d->pad_r >= 0, "negative padding");
+    // a transposed convolution may state a negative bottom / right padding: it only enlarges the output
+    // (cl_optimized_impls/CLDeconvolutionQuantized.cpp:254-256 uses the top / left values alone)
+    EH_REQUIRE(d->pad_t >= 0 && d->pad_l >= 0 && (negative_tail_padding || (d->pad_b >= 0 && d->pad_r >= 0)), "negative padding");
     EH_REQUIRE(d->layout == EH_NCHW || d->layout == EH_NHWC, "unknown layout %d", d->layout);
     EH_REQUIRE((int64_t)d->n * d->c * d->h * d->w < (1ll << 31), "input larger than 2 GiB is not supported");
     EH_REQUIRE(d->h < 32000 && d->w < 32000, "spatial extent too large");
@@ -1007,7 +1009,7 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
     plain.weight_layout &= ~EH_W_SIGNED;
     plain.layout &= ~EH_IO_SIGNED;
     desc = &plain;
-    int rc = check_desc_common(desc);
+    int rc = check_desc_common(desc, true);
     if (rc) return rc;
     if ((rc = check_requant(q, w_signed, io_signed))) return rc;
     EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
@@ -1077,7 +1079,12 @@ static void dw_release(eh_dwconv_plan *pl) {
 
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
     EH_REQUIRE(weight != nullptr, "weight pointer is null");
-    EH_HIP(hipMemcpyAsync(pl->w_copy, weight, (size_t)pl->cout * pl->taps, hipMemcpyDeviceToDevice, stream));
+    if (pl->d.weight_layout == EH_W_OHWI) {  // [taps][cout] -> [cout][taps]
+        int rc = launch_nhwc2nchw(static_cast<const uint8_t *>(weight), pl->w_copy, 1, pl->cout, pl->taps, stream);
+        if (rc) return rc;
+    } else {
+        EH_HIP(hipMemcpyAsync(pl->w_copy, weight, (size_t)pl->cout * pl->taps, hipMemcpyDeviceToDevice, stream));
+    }
     pl->has_bias = bias != nullptr;
     if (bias) EH_HIP(hipMemcpyAsync(pl->bias_copy, bias, (size_t)pl->cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
     pl->packed_valid = false;
@@ -1113,7 +1120,8 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     EH_REQUIRE(desc->depth_multiplier > 0, "bad depth multiplier %d", desc->depth_multiplier);
     EH_REQUIRE(desc->cout == desc->c * desc->depth_multiplier, "depthwise cout %d != c %d * depth multiplier %d", desc->cout,
                desc->c, desc->depth_multiplier);
-    EH_REQUIRE(desc->weight_layout == EH_W_OIHW, "depthwise weights are [C*dm][1][kh][kw]");
+    EH_REQUIRE(desc->weight_layout == EH_W_OIHW || desc->weight_layout == EH_W_OHWI,
+               "depthwise weights are [C*dm][1][kh][kw] (OIHW) or [1][kh][kw][C*dm] (OHWI)");
     eh_dwconv_plan *pl = new (std::nothrow) eh_dwconv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;

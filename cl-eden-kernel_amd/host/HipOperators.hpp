@@ -353,7 +353,11 @@ public:
 
         Dim4 in = input_->getDim();
         if (!parameters_->isNCHW) in = convertDimToNCHW(in);
-        const Dim4 wd = weight_->getDim();  // [C * depth_multiplier][1][kh][kw]
+        // [C * depth_multiplier][1][kh][kw]; androidNN models hold [1][kh][kw][C * depth_multiplier]
+        // (gpu/operators/CLDepthwiseConvolution.cpp:128-131,146)
+        Dim4 wd = weight_->getDim();
+        const bool hwo = parameters_->androidNN;
+        if (hwo) wd = Dim4{wd.w, wd.n, wd.c, wd.h};
         eh_conv_desc d;
         d.n = (int32_t)in.n;
         d.c = (int32_t)in.c;
@@ -373,7 +377,7 @@ public:
         d.groups = 1;
         d.depth_multiplier = (int32_t)parameters_->depth_multiplier;
         d.layout = parameters_->isNCHW ? EH_NCHW : EH_NHWC;
-        d.weight_layout = EH_W_OIHW;
+        d.weight_layout = hwo ? EH_W_OHWI : EH_W_OIHW;
         CHECK_EXPR_RETURN_FAILURE(wd.n == (uint32_t)d.cout && wd.c == 1, "HipDepthwiseConvolution: weight shape [%u %u %u %u] is not [C*dm][1][kh][kw]", wd.n, wd.c, wd.h, wd.w);
         desc_ = d;
         if (per_channel_) {
@@ -659,7 +663,8 @@ private:
 
 // Element-wise sum of two equally shaped uint8 tensors, requantized to the output tensor's
 // scale (quantization parameters are read from the three tensors at every execute()).
-// Broadcasting, coefficients and the int16 power-of-two variant are not offered here.
+// Broadcasting and the int16 power-of-two variant are not offered here; coefficients are ignored, as the
+// reference's quantized path ignores them.
 class HipAdd {
 public:
     HipAdd(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision) : runtime_(runtime), precision_(precision) {}
@@ -674,7 +679,8 @@ public:
         CHECK_EXPR_RETURN_FAILURE(parameters_ != nullptr, "HipAdd: parameters are not AddParameters");
         CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipAdd: only the UINT8 path exists on this backend");
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipAdd: no texture storage");
-        CHECK_EXPR_RETURN_FAILURE(parameters_->coeff.empty() && !parameters_->pot_scale_int16, "HipAdd: coefficients / int16 scaling are not offered");
+        // coefficients belong to the float kernels: the quantized path never reads them (gpu/operators/CLAdd.cpp:159-163)
+        CHECK_EXPR_RETURN_FAILURE(!parameters_->pot_scale_int16, "HipAdd: int16 scaling is not offered");
         CHECK_EXPR_RETURN_FAILURE(a_->getDataType() == DataType::UINT8 && b_->getDataType() == DataType::UINT8 &&
                                       output_->getDataType() == DataType::UINT8, "HipAdd: expects uint8 tensors");
         CHECK_EXPR_RETURN_FAILURE(a_->getTotalSizeFromDims() == b_->getTotalSizeFromDims() &&

@@ -14,6 +14,7 @@
 #include <string>
 #include <vector>
 
+#include "HipOpConstructor.hpp"
 #include "HipOperators.hpp"
 #include "eden_oracle.h"
 #include "userdriver_operator.hpp"
@@ -956,6 +957,184 @@ static int gpu_tests() {
         return ok;
     });
 
+
+    // ------------------------------------------------------------ construction from TFLite options
+    auto fmap = [](const char *name, NDims shape, int32_t index, float scale, int32_t zp, TFlite::TensorType type = TFlite::TensorType_UINT8) {
+        auto t = std::make_shared<TensorDesc>();
+        t->name = name;
+        t->shape = shape;
+        t->data_type = type;
+        t->scale = scale;
+        t->zero_point = zp;
+        t->buffer_index = index;
+        return t;
+    };
+    auto param = [](const char *name, NDims shape, const void *data, TFlite::TensorType type, float scale, int32_t zp) {
+        auto t = std::make_shared<TensorDesc>();
+        t->name = name;
+        t->shape = shape;
+        t->data_type = type;
+        t->scale = scale;
+        t->zero_point = zp;
+        t->is_const = true;
+        t->data = data;
+        return t;
+    };
+    auto op_desc = [](const char *name, uint64_t id, TFlite::BuiltinOperator code, std::vector<std::shared_ptr<TensorDesc>> in,
+                      std::vector<std::shared_ptr<TensorDesc>> out, std::shared_ptr<void> option) {
+        OperatorDesc d;
+        d.name = name;
+        d.id = id;
+        d.code = code;
+        d.in_tensors = in;
+        d.out_tensors = out;
+        d.option = option;
+        return d;
+    };
+
+    run_test("OpConstructor.AndroidNN_channels_last_residual_network_with_SAME_padding", [&] {
+        // input 1x16x16x8 -> conv 3x3 s2 SAME relu6 (16) -> depthwise 3x3 SAME relu6 -> conv 1x1 -> add(conv1) -> pool 8x8 -> fc 10
+        bool ok = true;
+        const float s0 = 0.02f, sw = 0.004f, s1 = 6.0f / 255, s2 = 6.0f / 255, s3 = 0.05f, s4 = 0.06f, s5 = 0.06f, s6 = 0.1f;
+        auto x = rand_u8(16 * 16 * 8, 401);                                  // NHWC
+        auto w1 = rand_u8(16 * 9 * 8, 402), wd = rand_u8(9 * 16, 403), w3 = rand_u8(16 * 16, 404), wf = rand_u8(10 * 16, 405);
+        auto b1 = rand_i32(16, 406, -500, 500), bd = rand_i32(16, 407, -500, 500), b3 = rand_i32(16, 408, -500, 500), bf = rand_i32(10, 409, -500, 500);
+        // ---- oracle, planar
+        auto xn = nhwc_to_nchw(x, 1, 8, 16, 16);
+        auto w1o = nhwc_to_nchw(w1, 16, 8, 3, 3);                            // [o][kh][kw][i] -> [o][i][kh][kw]
+        std::vector<uint8_t> wdo(16 * 9);
+        for (int t = 0; t < 9; ++t)
+            for (int c = 0; c < 16; ++c) wdo[c * 9 + t] = wd[t * 16 + c];    // [1][kh][kw][c] -> [c][1][kh][kw]
+        eo_quant q;
+        std::vector<uint8_t> t1(16 * 64), t2(16 * 64), t3(16 * 64), t4(16 * 64), t5(16), want(10), got(10);
+        eo_conv_shape c1 = shape(1, 8, 16, 16, 16, 3, 3, 2, 2, 0, 1, 0, 1);  // SAME, TF rule: the extra row and column go last
+        eo_make_quant(s0, 128, sw, 120, s0 * sw, s1, 0, EO_ACT_RELU6, 1, &q);
+        eo_conv2d_u8(xn.data(), w1o.data(), b1.data(), t1.data(), &c1, &q, nullptr);
+        eo_conv_shape c2 = shape(1, 16, 8, 8, 16, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1);
+        eo_make_quant(s1, 0, sw, 131, s1 * sw, s2, 0, EO_ACT_RELU6, 1, &q);
+        eo_dwconv2d_u8(t1.data(), wdo.data(), bd.data(), t2.data(), &c2, &q, nullptr);
+        eo_conv_shape c3 = shape(1, 16, 8, 8, 16, 1, 1);
+        eo_make_quant(s2, 0, sw, 125, s2 * sw, s3, 128, 0, 0, &q);
+        eo_conv2d_u8(t2.data(), w3.data(), b3.data(), t3.data(), &c3, &q, nullptr);
+        eo_add_quant aq;
+        eo_make_add_quant(s1, 0, s3, 128, s4, 100, 0, 0, &aq);
+        eo_add_u8(t1.data(), t3.data(), t4.data(), 16 * 64, &aq);
+        eo_avgpool_u8(t4.data(), t5.data(), 1, 16, 8, 8, 8, 8, 1, 1, 0, 0, 0, 0, 0, 255);
+        eo_make_quant(s5, 100, sw, 128, s5 * sw, s6, 128, 0, 0, &q);
+        eo_fc_u8(t5.data(), wf.data(), bf.data(), want.data(), 1, 16, 10, &q, nullptr);
+        // ---- the list
+        const TFlite::TensorType I32 = TFlite::TensorType_INT32, U8T = TFlite::TensorType_UINT8;
+        auto f0 = fmap("in", {1, 16, 16, 8}, 0, s0, 128), f1 = fmap("c1", {1, 8, 8, 16}, 1, s1, 0), f2 = fmap("dw", {1, 8, 8, 16}, 2, s2, 0);
+        auto f3 = fmap("pw", {1, 8, 8, 16}, 3, s3, 128), f4 = fmap("sum", {1, 8, 8, 16}, 4, s4, 100), f5 = fmap("pool", {1, 1, 1, 16}, 5, s5, 100);
+        auto f6 = fmap("logits", {1, 10}, 6, s6, 128);
+        auto conv_opt = std::make_shared<TFlite::Conv2DOptions>();
+        conv_opt->stride_h = conv_opt->stride_w = 2;
+        conv_opt->fused_activation_function = TFlite::ActivationFunctionType_RELU6;
+        auto dw_opt = std::make_shared<TFlite::DepthwiseConv2DOptions>();
+        dw_opt->fused_activation_function = TFlite::ActivationFunctionType_RELU6;
+        auto pw_opt = std::make_shared<TFlite::Conv2DOptions>();
+        auto pool_opt = std::make_shared<TFlite::Pool2DOptions>();
+        pool_opt->filter_height = pool_opt->filter_width = 8;
+        OperatorListDesc list;
+        list.legacy_model = TFlite::LegacyModel_ANDROID_NN;
+        list.operators = {
+            op_desc("CONV_2D", 1, TFlite::BuiltinOperator_CONV_2D,
+                    {f0, param("w1", {16, 3, 3, 8}, w1.data(), U8T, sw, 120), param("b1", {16}, b1.data(), I32, s0 * sw, 0)}, {f1}, conv_opt),
+            op_desc("DEPTHWISE_CONV_2D", 2, TFlite::BuiltinOperator_DEPTHWISE_CONV_2D,
+                    {f1, param("wd", {1, 3, 3, 16}, wd.data(), U8T, sw, 131), param("bd", {16}, bd.data(), I32, s1 * sw, 0)}, {f2}, dw_opt),
+            op_desc("CONV_2D", 3, TFlite::BuiltinOperator_CONV_2D,
+                    {f2, param("w3", {16, 1, 1, 16}, w3.data(), U8T, sw, 125), param("b3", {16}, b3.data(), I32, s2 * sw, 0)}, {f3}, pw_opt),
+            op_desc("ADD", 4, TFlite::BuiltinOperator_ADD, {f1, f3}, {f4}, std::make_shared<TFlite::AddOptions>()),
+            op_desc("AVERAGE_POOL_2D", 5, TFlite::BuiltinOperator_AVERAGE_POOL_2D, {f4}, {f5}, pool_opt),
+            op_desc("FULLY_CONNECTED", 6, TFlite::BuiltinOperator_FULLY_CONNECTED,
+                    {f5, param("wf", {10, 16}, wf.data(), U8T, sw, 128), param("bf", {10}, bf.data(), I32, s5 * sw, 0)}, {f6},
+                    std::make_shared<TFlite::FullyConnectedOptions>()),
+        };
+        OperationConstructor built(rt);
+        EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
+        EXPECT(built.operators && built.operators->size() == 6);
+        EXPECT(built.in_tensors.size() == 1 && built.out_tensors.size() == 1);
+        OperationExecutor executor(rt);
+        for (int round = 0; round < 2; ++round) {  // a second execution reuses the pooled buffers
+            std::fill(got.begin(), got.end(), 0);
+            EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
+            EXPECT(same(got, want));
+        }
+        EXPECT(varied(t4));
+        for (auto &o : *built.operators) EXPECT(o->release() == ENN_RET_SUCCESS);
+        return ok;
+    });
+
+    run_test("OpConstructor.Planar_models_Tensorflow_and_Caffe_padding_rules_and_transposed_convolution", [&] {
+        bool ok = true;
+        const float s0 = 0.02f, sw = 0.004f, s1 = 0.08f, s2 = 0.3f;
+        auto x = rand_u8(8 * 15 * 15, 411), w1 = rand_u8(12 * 8 * 9, 412), w2 = rand_u8(12 * 6 * 4, 413);
+        auto b1 = rand_i32(12, 414, -500, 500), b2 = rand_i32(6, 415, -500, 500);
+        for (int variant = 0; variant < 2; ++variant) {
+            const bool caffe = variant == 1;
+            // 15 -> 8 with 3x3 stride 2 needs 2 rows of padding: one each side under either rule; 14 -> 7 would differ.
+            // Use stride 2 on 15 (symmetric) for the convolution and let the 2x2 stride-2 deconvolution (8 -> 16) follow.
+            eo_quant q;
+            std::vector<uint8_t> t1(12 * 64), want(6 * 256), got(want.size());
+            eo_conv_shape c1 = shape(1, 8, 15, 15, 12, 3, 3, 2, 2, 1, 1, 1, 1);
+            eo_make_quant(s0, 128, sw, 120, s0 * sw, s1, 128, 0, 0, &q);
+            eo_conv2d_u8(x.data(), w1.data(), b1.data(), t1.data(), &c1, &q, nullptr);
+            eo_conv_shape c2 = shape(1, 12, 8, 8, 6, 2, 2, 2, 2);
+            eo_make_quant(s1, 128, sw, 130, s1 * sw, s2, 128, EO_ACT_RELU, 1, &q);
+            eo_deconv2d_u8(t1.data(), w2.data(), b2.data(), want.data(), &c2, &q, nullptr);
+            auto f0 = fmap("in", {1, 8, 15, 15}, 0, s0, 128), f1 = fmap("c1", {1, 12, 8, 8}, 1, s1, 128), f2 = fmap("up", {1, 6, 16, 16}, 2, s2, 128);
+            auto conv_opt = std::make_shared<TFlite::Conv2DOptions>();
+            conv_opt->stride_h = conv_opt->stride_w = 2;
+            auto up_opt = std::make_shared<TFlite::TransposeConvOptions>();
+            up_opt->stride_h = up_opt->stride_w = 2;
+            up_opt->fused_activation_function = TFlite::ActivationFunctionType_RELU;
+            OperatorListDesc list;
+            list.legacy_model = caffe ? TFlite::LegacyModel_CAFFE : TFlite::LegacyModel_TENSORFLOW;
+            list.operators = {
+                op_desc("CONV_2D", 1, TFlite::BuiltinOperator_CONV_2D,
+                        {f0, param("w1", {12, 8, 3, 3}, w1.data(), TFlite::TensorType_UINT8, sw, 120),
+                         param("b1", {12}, b1.data(), TFlite::TensorType_INT32, s0 * sw, 0)}, {f1}, conv_opt),
+                op_desc("TRANSPOSE_CONV", 2, TFlite::BuiltinOperator_TRANSPOSE_CONV,
+                        {f1, param("w2", {12, 6, 2, 2}, w2.data(), TFlite::TensorType_UINT8, sw, 130),
+                         param("b2", {6}, b2.data(), TFlite::TensorType_INT32, s1 * sw, 0)}, {f2}, up_opt),
+            };
+            OperationConstructor built(rt);
+            EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
+            OperationExecutor executor(rt);
+            EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
+            EXPECT(same(got, want));
+            EXPECT(varied(want));
+        }
+        return ok;
+    });
+
+    run_test("OpConstructor.Int8_tensors_select_INT8_precision_and_per_channel_scales_select_that_mode", [&] {
+        bool ok = true;
+        const eo_conv_shape s = shape(1, 16, 9, 9, 24, 3, 3, 1, 1, 1, 1, 1, 1);
+        auto x = to_i8(rand_u8(16 * 81, 421)), w = to_i8(rand_u8(24 * 16 * 9, 422));
+        auto b = rand_i32(24, 423, -500, 500);
+        auto scales = channel_scales(24, 424, 0.002f);
+        std::vector<int32_t> m, sh;
+        channel_pairs(0.02f, scales, 0.3f, &m, &sh);
+        eo_quant q = {-5, 0, 3, 0, 0, -128, 127};
+        std::vector<int8_t> want(24 * 81), got(want.size());
+        eo_conv2d_s8(x.data(), w.data(), b.data(), want.data(), &s, &q, m.data(), sh.data());
+        auto f0 = fmap("in", {1, 16, 9, 9}, 0, 0.02f, -5, TFlite::TensorType_INT8), f1 = fmap("out", {1, 24, 9, 9}, 1, 0.3f, 3, TFlite::TensorType_INT8);
+        auto wt = param("w", {24, 16, 3, 3}, w.data(), TFlite::TensorType_INT8, 0.0f, 0);
+        wt->per_channel_scales = scales;
+        OperatorListDesc list;
+        list.legacy_model = TFlite::LegacyModel_TENSORFLOW_NCHW;
+        list.operators = {op_desc("CONV_2D", 1, TFlite::BuiltinOperator_CONV_2D, {f0, wt, param("b", {24}, b.data(), TFlite::TensorType_INT32, 1.0f, 0)},
+                                  {f1}, std::make_shared<TFlite::Conv2DOptions>())};
+        OperationConstructor built(rt);
+        EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
+        OperationExecutor executor(rt);
+        EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
+        EXPECT(same(std::vector<uint8_t>(got.begin(), got.end()), std::vector<uint8_t>(want.begin(), want.end())));
+        EXPECT(varied(std::vector<uint8_t>(want.begin(), want.end())));
+        return ok;
+    });
+
     std::printf("%d of %d GPU operator tests failed\n", g_failed, g_run);
     return g_failed ? 1 : 0;
 }
@@ -1003,6 +1182,41 @@ static int host_tests() {
                (int)DataType::UINT8 == 4 && (int)DataOrder::NHWC == 1);
         return ok;
     });
+    run_test("OpConstructor.PaddingLayoutAndPrecisionRules", [&] {
+        bool ok = true;
+        typedef OperationConstructor OC;
+        Pad4 p;
+        // VALID: nothing
+        OC::get_padding(TFlite::LegacyModel_TENSORFLOW, TFlite::Padding_VALID, p, {1, 3, 224, 224}, {1, 32, 111, 111}, {32, 3, 3, 3}, {2, 2}, {1, 1}, false, true);
+        EXPECT(p.t == 0 && p.b == 0 && p.l == 0 && p.r == 0);
+        // SAME, 224 -> 112 with 3x3 stride 2 needs one row: TensorFlow puts it last, Caffe pads both sides with the ceiling
+        OC::get_padding(TFlite::LegacyModel_TENSORFLOW, TFlite::Padding_SAME, p, {1, 3, 224, 224}, {1, 32, 112, 112}, {32, 3, 3, 3}, {2, 2}, {1, 1}, false, true);
+        EXPECT(p.t == 0 && p.b == 1 && p.l == 0 && p.r == 1);
+        OC::get_padding(TFlite::LegacyModel_CAFFE, TFlite::Padding_SAME, p, {1, 3, 224, 224}, {1, 32, 112, 112}, {32, 3, 3, 3}, {2, 2}, {1, 1}, false, true);
+        EXPECT(p.t == 1 && p.b == 1 && p.l == 1 && p.r == 1);
+        // channels-last extents and (out, kh, kw, in) filters
+        OC::get_padding(TFlite::LegacyModel_TENSORFLOW_NHWC, TFlite::Padding_SAME, p, {1, 20, 30, 8}, {1, 20, 30, 16}, {16, 5, 3, 8}, {1, 1}, {1, 1}, false, false);
+        EXPECT(p.t == 2 && p.b == 2 && p.l == 1 && p.r == 1);
+        // androidNN with planar data still reads the filter as (out, kh, kw, in)
+        OC::get_padding(TFlite::LegacyModel_ANDROID_NN, TFlite::Padding_SAME, p, {1, 8, 20, 30}, {1, 16, 20, 30}, {16, 5, 3, 8}, {1, 1}, {1, 1}, false, true);
+        EXPECT(p.t == 2 && p.b == 2 && p.l == 1 && p.r == 1);
+        // dilation: the reference widens the filter width by dilation.h and the height by dilation.w
+        OC::get_padding(TFlite::LegacyModel_TENSORFLOW, TFlite::Padding_SAME, p, {1, 4, 20, 20}, {1, 4, 20, 20}, {4, 4, 3, 3}, {1, 1}, {2, 1}, false, true);
+        EXPECT(p.l == 2 && p.r == 2 && p.t == 1 && p.b == 1);
+        // transposed convolution: input and output trade places (8 -> 16, 4x4 stride 2 needs 2 in all)
+        OC::get_padding(TFlite::LegacyModel_TENSORFLOW, TFlite::Padding_SAME, p, {1, 12, 8, 8}, {1, 6, 16, 16}, {12, 6, 4, 4}, {2, 2}, {1, 1}, true, true);
+        EXPECT(p.t == 1 && p.b == 1 && p.l == 1 && p.r == 1);
+        // androidNN transposed convolution whose output (18) exceeds (in - 1) * stride + k = 16... no: smaller needed than given -> negative tail
+        OC::get_padding(TFlite::LegacyModel_ANDROID_NN, TFlite::Padding_SAME, p, {1, 8, 8, 12}, {1, 18, 18, 6}, {6, 2, 2, 12}, {2, 2}, {1, 1}, true, false);
+        EXPECT((int32_t)p.b == -2 && (int32_t)p.r == -2 && p.t == 0 && p.l == 0);
+        EXPECT(OC::is_nchw_layout(TFlite::LegacyModel_CAFFE) && OC::is_nchw_layout(TFlite::LegacyModel_TENSORFLOW) &&
+               OC::is_nchw_layout(TFlite::LegacyModel_ANDROID_NN) && !OC::is_nchw_layout(TFlite::LegacyModel_TENSORFLOW_NHWC) &&
+               !OC::is_nchw_layout(TFlite::LegacyModel_CAFFE_NHWC));
+        EXPECT(OC::get_precision(TFlite::TensorType_UINT8) == PrecisionType::UINT8 && OC::get_precision(TFlite::TensorType_INT8) == PrecisionType::INT8 &&
+               OC::get_precision(TFlite::TensorType_FLOAT32) == PrecisionType::FP32 && OC::get_precision(TFlite::TensorType_INT32) == PrecisionType::FP16);
+        return ok;
+    });
+
     std::printf("%d of %d host-only tests failed\n", g_failed, g_run);
     return g_failed ? 1 : 0;
 }

@@ -41,7 +41,8 @@ typedef enum eh_layout { EH_NCHW = 0, EH_NHWC = 1 } eh_layout;
 
 /* Weight element order.  OIHW is the reference's default [Cout][Cin/g][kh][kw];
  * OHWI is its androidNN order [Cout][kh][kw][Cin]
- * (gpu/operators/cl_optimized_impls/CLDeconvolutionQuantized.cpp:39-46);
+ * (gpu/operators/cl_optimized_impls/CLDeconvolutionQuantized.cpp:39-46), for a depthwise
+ * convolution [1][kh][kw][C*dm] (gpu/operators/CLDepthwiseConvolution.cpp:128-131,146);
  * IOHW is the deconvolution order [Cin][Cout/g][kh][kw] (gpu/op_test/deconv_guard.h:53-69). */
 typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh_weight_layout;
 /* Or-ed into eh_conv_desc.weight_layout (convolution, depthwise convolution, deconvolution): the weight
