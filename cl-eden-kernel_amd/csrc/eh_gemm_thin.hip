@@ -3,17 +3,20 @@
 // (pointwise expansions such as 24 -> 144), or a small pixel count (the late
 // layers of an image network, classifier heads).
 //
-// Such layers are bound by memory or by latency, not by the matrix cores, so
-// nothing is staged in LDS and no workgroup-wide step exists: a wave owns 32
-// output pixels and a group of 32-channel blocks, every lane fetches 16 reduction
-// bytes of its pixel per 32-byte step straight into the 32x32x32 MFMA fragment
-// layout (the bytes of a wave are one contiguous span when the pixels are), and
-// the weights, packed in fragment order, are read per block and step as one
-// coalesced 1 KiB wave load that stays in L2.  Four steps' worth of loads are
-// requested before the first MFMA of the group.
+// Such layers are bound by memory, by the requantization arithmetic or by latency,
+// not by the matrix cores.  A workgroup copies the weights of its channel range
+// (packed in MFMA fragment order, 1 KiB per 32-channel block and 32-byte step) and
+// their bias into LDS once; each of its waves then walks 32-pixel blocks: every lane
+// fetches 16 reduction bytes of its pixel per step straight into the 32x32x32 MFMA
+// fragment layout (the bytes of a wave are one contiguous span when the pixels are),
+// with the next block's bytes requested before the current block's arithmetic, and
+// finishes the range's channel blocks against the weights in LDS.  The activations
+// are read once per channel range, the weights once per workgroup.
 // The weight fragment is the row operand and its rows are permuted within a
 // 32-channel block (see packed_b_offset), so a lane ends up with 16 consecutive
 // output channels of its pixel: requantize, pack, one 16-byte store.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "eh_internal.h"
@@ -25,175 +28,209 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 namespace {
 
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+
+// NBU: channel blocks a wave finishes per pass; KU: reduction steps whose loads are in flight together.
+// Grid: x = workgroups along the pixel rows (each wave walks 32-row blocks with stride gridDim.x * 4),
+// y = channel ranges of `nbw` blocks.
 template <int NBU, int KU, bool ROWSUM, bool FAST>
-__global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps,
-                                                          const int stage_out) {
-    // KU: reduction steps whose loads are in flight together; NBU: channel blocks per wave
+__global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps, const int nbw,
+                                                          const int row_blocks) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, half = lane >> 5;
-    const int m = (blockIdx.x * 4 + wave) * 32 + r;
-    const bool row_ok = m < p.m;
     const int plane = p.ho * p.wo;
+    const int nb_first = blockIdx.y * nbw;
+    const int nb_count = n_blocks - nb_first < nbw ? n_blocks - nb_first : nbw;  // blocks of this range that exist
 
-    // this lane's pixel: where its reduction bytes start, where its outputs go
-    size_t in_off = 0, out_off = 0;
-    if (row_ok) {
-        const int img = (int)fastdiv((uint32_t)m, p.div_plane), rem = m - img * plane;
-        const int oy = (int)fastdiv((uint32_t)rem, p.div_wo), ox = rem - oy * p.wo;
-        in_off = ((size_t)(img * p.h + oy * p.stride_h + p.y_base) * p.w + (ox * p.stride_w + p.x_base)) * (size_t)p.cin +
-                 (size_t)p.a_offset;
-        out_off = (((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0)) * (size_t)p.ldc;
+    // this range's weights (fragment order: 1 KiB per block and step) and bias, once per workgroup
+    extern __shared__ __align__(16) uint8_t lds_raw[];
+    v4i *b_s = reinterpret_cast<v4i *>(lds_raw);                                  // [nbw][ksteps][64 lanes]
+    int32_t *bias_s = reinterpret_cast<int32_t *>(lds_raw + (size_t)nbw * ksteps * 1024);  // [nbw * 32]
+    {
+        const v4i *src = reinterpret_cast<const v4i *>(p.b) + (size_t)nb_first * ksteps * 64;
+        const int pieces = nb_count * ksteps * 64;
+        for (int i = threadIdx.x; i < pieces; i += 256) b_s[i] = src[i];
+        for (int i = threadIdx.x; i < nb_count * 32; i += 256) bias_s[i] = p.bias[nb_first * 32 + i];
     }
-    const uint8_t *arow = p.a + in_off + half * 16;
+    __syncthreads();
+
     const RequantDev rq = p.rq;
-    const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-    const v4i *bfrag = reinterpret_cast<const v4i *>(p.b) + lane;
-    // stage_out: the 32 pixels of a wave are 32 * N contiguous output bytes (plain channels-last rows, N a
-    // multiple of 8, one workgroup row per pixel block): the wave collects its rows in LDS and writes them
-    // as one linear run of 16-byte pieces, whole cache lines instead of a 32-byte piece per pixel and block
-    extern __shared__ __align__(16) uint8_t out_stage[];
-    uint8_t *wave_stage = out_stage + (size_t)wave * 32 * p.n;
+    const bool wide = (p.ldc & 3) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 3) == 0);  // dword-aligned rows: vector stores
+    const int rb_stride = gridDim.x * 4;
+    constexpr bool SINGLE = KU < 4;  // the whole reduction is one group of KU steps (the launcher guarantees ksteps <= KU)
 
-    // blockIdx.y spreads the channel-block groups over workgroups when there are few pixels
-    for (int nb0 = blockIdx.y * NBU; nb0 < n_blocks; nb0 += gridDim.y * NBU) {
-        const v4i *bblk[NBU];
-        int4 bb[NBU][4];
-#pragma unroll
-        for (int u = 0; u < NBU; ++u) {
-            const int nb = nb0 + u < n_blocks ? nb0 + u : n_blocks - 1;
-            bblk[u] = bfrag + (size_t)nb * ksteps * 64;
-#pragma unroll
-            for (int g = 0; g < 4; ++g) bb[u][g] = *reinterpret_cast<const int4 *>(p.bias + nb * 32 + half * 16 + g * 4);
+    // where the lane's pixel of row block `rb` reads and writes
+    auto locate = [&](int rb, bool &ok, size_t &in_off, size_t &out_off) {
+        const int m = rb * 32 + r;
+        ok = rb < row_blocks && m < p.m;
+        in_off = 0;
+        out_off = 0;
+        if (ok) {
+            const int img = (int)fastdiv((uint32_t)m, p.div_plane), rem = m - img * plane;
+            const int oy = (int)fastdiv((uint32_t)rem, p.div_wo), ox = rem - oy * p.wo;
+            in_off = ((size_t)(img * p.h + oy * p.stride_h + p.y_base) * p.w + (ox * p.stride_w + p.x_base)) * (size_t)p.cin +
+                     (size_t)p.a_offset + half * 16;
+            out_off = (((size_t)img * p.out_h + (oy * p.out_sy + p.out_y0)) * p.out_w + (ox * p.out_sx + p.out_x0)) * (size_t)p.ldc;
         }
-        // SINGLE: the whole reduction is one group of KU steps, so each channel block's accumulator
-        // can be formed right before it is requantized instead of all NBU living side by side
-        constexpr bool SINGLE = KU < 4;
-        v16i acc[SINGLE ? 1 : NBU];
-        v4i afs[SINGLE ? KU : 1], bfs[SINGLE ? KU : 1][SINGLE ? NBU : 1];
-        int rowsum = 0;
-        for (int ks0 = 0; ks0 < (SINGLE ? 1 : ksteps); ks0 += KU) {
-            // reduction bytes past K read as the byte that the sign flip turns into 0; steps past the
-            // last one therefore multiply by zero whatever weight block they re-read
-            uint2 lo[KU], hi[KU];
-            v4i bf[KU][NBU];
-#pragma unroll
-            for (int t = 0; t < KU; ++t) {
-                const int kb = (ks0 + t) * 32 + half * 16;
-                lo[t] = make_uint2(p.a_xor, p.a_xor);
-                hi[t] = lo[t];
-                if (row_ok && kb < p.k) lo[t] = *reinterpret_cast<const uint2 *>(arow + (ks0 + t) * 32);
-                if (row_ok && kb + 8 < p.k) hi[t] = *reinterpret_cast<const uint2 *>(arow + (ks0 + t) * 32 + 8);
-                const int ks = ks0 + t < ksteps ? ks0 + t : ksteps - 1;
-#pragma unroll
-                for (int u = 0; u < NBU; ++u) bf[t][u] = bblk[u][ks * 64];
-            }
-            if constexpr (!SINGLE) {
-                if (ks0 == 0) {
-#pragma unroll
-                    for (int u = 0; u < NBU; ++u)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) acc[u][i] = 0;
-                }
-            }
-#pragma unroll
-            for (int t = 0; t < KU; ++t) {
-                v4i af;
-                af.x = (int)(lo[t].x ^ p.a_xor);
-                af.y = (int)(lo[t].y ^ p.a_xor);
-                af.z = (int)(hi[t].x ^ p.a_xor);
-                af.w = (int)(hi[t].y ^ p.a_xor);
-                if constexpr (ROWSUM) {
-                    rowsum = __builtin_amdgcn_sdot4(af.x, 0x01010101, rowsum, false);
-                    rowsum = __builtin_amdgcn_sdot4(af.y, 0x01010101, rowsum, false);
-                    rowsum = __builtin_amdgcn_sdot4(af.z, 0x01010101, rowsum, false);
-                    rowsum = __builtin_amdgcn_sdot4(af.w, 0x01010101, rowsum, false);
-                }
-                if constexpr (SINGLE) {
-                    afs[t] = af;
-#pragma unroll
-                    for (int u = 0; u < NBU; ++u) bfs[t][u] = bf[t][u];
-                } else {
-#pragma unroll
-                    for (int u = 0; u < NBU; ++u) acc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[t][u], af, acc[u], 0, 0, 0);
-                }
-            }
-        }
-        int ncorr = 0;
+    };
+    // 16 reduction bytes of step ks; bytes past K read as the byte that the sign flip turns into 0
+    auto load_a = [&](bool ok, size_t in_off, int ks, uint2 &lo, uint2 &hi) {
+        const int kb = ks * 32 + half * 16;
+        lo = make_uint2(p.a_xor, p.a_xor);
+        hi = lo;
+        if (ok && kb < p.k) lo = *reinterpret_cast<const uint2 *>(p.a + in_off + ks * 32);
+        if (ok && kb + 8 < p.k) hi = *reinterpret_cast<const uint2 *>(p.a + in_off + ks * 32 + 8);
+    };
+    auto to_fragment = [&](uint2 lo, uint2 hi, int &rowsum) {
+        v4i af;
+        af.x = (int)(lo.x ^ p.a_xor);
+        af.y = (int)(lo.y ^ p.a_xor);
+        af.z = (int)(hi.x ^ p.a_xor);
+        af.w = (int)(hi.y ^ p.a_xor);
         if constexpr (ROWSUM) {
-            rowsum += __shfl_xor(rowsum, 32);  // the other half of this pixel's reduction bytes
-            ncorr = -p.zw * rowsum;
+            rowsum = __builtin_amdgcn_sdot4(af.x, 0x01010101, rowsum, false);
+            rowsum = __builtin_amdgcn_sdot4(af.y, 0x01010101, rowsum, false);
+            rowsum = __builtin_amdgcn_sdot4(af.z, 0x01010101, rowsum, false);
+            rowsum = __builtin_amdgcn_sdot4(af.w, 0x01010101, rowsum, false);
         }
+        return af;
+    };
+    // 16 accumulators of one channel block -> 16 output bytes of the lane's pixel
+    auto finish_block = [&](const v16i &acc, int nb_local, int ncorr, bool ok, size_t out_off) {
+        const int n = (nb_first + nb_local) * 32 + half * 16;  // this lane's 16 consecutive channels
+        const int32_t *bsrc = bias_s + nb_local * 32 + half * 16;
+        uint32_t packed[4];
+        auto quantize = [&](auto mode_c) {
+            constexpr int mode = decltype(mode_c)::value;
 #pragma unroll
-        for (int u = 0; u < NBU; ++u) {
-            const int nb = nb0 + u;
-            if (nb >= n_blocks) break;
-            const int n = nb * 32 + half * 16;  // this lane's 16 consecutive channels
-            const int ai = SINGLE ? 0 : u;
-            if constexpr (SINGLE) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) acc[0][i] = 0;
-#pragma unroll
-                for (int t = 0; t < KU; ++t) acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bfs[t][u], afs[t], acc[0], 0, 0, 0);
+            for (int g = 0; g < 4; ++g) {
+                const int4 bb = *reinterpret_cast<const int4 *>(bsrc + g * 4);
+                uint32_t o0, o1, o2, o3;
+                if (mode == 0 && rq.pc_multiplier) {  // per-channel parameters (the padded arrays cover whole blocks)
+                    const int4 cm = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + g * 4);
+                    const int4 cs = *reinterpret_cast<const int4 *>(rq.pc_shift + n + g * 4);
+                    o0 = requant_u8_channel(acc[g * 4 + 0] + bb.x + ncorr, cm.x, cs.x, rq);
+                    o1 = requant_u8_channel(acc[g * 4 + 1] + bb.y + ncorr, cm.y, cs.y, rq);
+                    o2 = requant_u8_channel(acc[g * 4 + 2] + bb.z + ncorr, cm.z, cs.z, rq);
+                    o3 = requant_u8_channel(acc[g * 4 + 3] + bb.w + ncorr, cm.w, cs.w, rq);
+                } else {
+                    o0 = requant_u8_as<mode>(acc[g * 4 + 0] + bb.x + ncorr, rq);
+                    o1 = requant_u8_as<mode>(acc[g * 4 + 1] + bb.y + ncorr, rq);
+                    o2 = requant_u8_as<mode>(acc[g * 4 + 2] + bb.z + ncorr, rq);
+                    o3 = requant_u8_as<mode>(acc[g * 4 + 3] + bb.w + ncorr, rq);
+                }
+                packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
             }
-            uint32_t packed[4];
-            auto quantize = [&](auto mode_c) {
-                constexpr int mode = decltype(mode_c)::value;
+        };
+        if constexpr (!FAST)
+            quantize(std::integral_constant<int, 0>{});
+        else if (rq.fast == 2)
+            quantize(std::integral_constant<int, 2>{});
+        else
+            quantize(std::integral_constant<int, 1>{});
+        if (!ok || n >= p.n) return;
+        uint8_t *dst = p.out + out_off + n;
+        const int cnt = p.n - n;
+        if (wide && cnt >= 16) {
+            *reinterpret_cast<u32x4_a4 *>(dst) = u32x4_a4{packed[0], packed[1], packed[2], packed[3]};
+        } else if (wide && cnt == 8) {
+            *reinterpret_cast<u32x2_a4 *>(dst) = u32x2_a4{packed[0], packed[1]};
+        } else {
+            const int c = cnt < 16 ? cnt : 16;
+            for (int t = 0; t < c; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+        }
+    };
+
+    if constexpr (SINGLE) {
+        // the pixel block's reduction bytes sit in registers for all of its channel blocks; the next
+        // block's bytes are requested before this one's arithmetic starts
+        bool ok, ok_next;
+        size_t in_off, out_off, in_next, out_next;
+        uint2 lo[KU], hi[KU], lo_next[KU], hi_next[KU];
+        int rb = blockIdx.x * 4 + wave;
+        locate(rb, ok, in_off, out_off);
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    uint32_t o0, o1, o2, o3;
-                    if (mode == 0 && rq.pc_multiplier) {  // per-channel parameters (the padded arrays cover whole blocks)
-                        const int32_t *pm = rq.pc_multiplier + n + g * 4;
-                            const int4 cm = make_int4(pm[0], pm[1], pm[2], pm[3]);
-                        const int32_t *ps = rq.pc_shift + n + g * 4;
-                            const int4 cs = make_int4(ps[0], ps[1], ps[2], ps[3]);
-                        o0 = requant_u8_channel(acc[ai][g * 4 + 0] + bb[u][g].x + ncorr, cm.x, cs.x, rq);
-                        o1 = requant_u8_channel(acc[ai][g * 4 + 1] + bb[u][g].y + ncorr, cm.y, cs.y, rq);
-                        o2 = requant_u8_channel(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, cm.z, cs.z, rq);
-                        o3 = requant_u8_channel(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, cm.w, cs.w, rq);
-                    } else {
-                        o0 = requant_u8_as<mode>(acc[ai][g * 4 + 0] + bb[u][g].x + ncorr, rq);
-                        o1 = requant_u8_as<mode>(acc[ai][g * 4 + 1] + bb[u][g].y + ncorr, rq);
-                        o2 = requant_u8_as<mode>(acc[ai][g * 4 + 2] + bb[u][g].z + ncorr, rq);
-                        o3 = requant_u8_as<mode>(acc[ai][g * 4 + 3] + bb[u][g].w + ncorr, rq);
+        for (int t = 0; t < KU; ++t) load_a(ok, in_off, t, lo[t], hi[t]);
+        for (; rb < row_blocks; rb += rb_stride) {
+            locate(rb + rb_stride, ok_next, in_next, out_next);
+#pragma unroll
+            for (int t = 0; t < KU; ++t) load_a(ok_next, in_next, t, lo_next[t], hi_next[t]);
+            v4i af[KU];
+            int rowsum = 0;
+#pragma unroll
+            for (int t = 0; t < KU; ++t) af[t] = to_fragment(lo[t], hi[t], rowsum);
+            int ncorr = 0;
+            if constexpr (ROWSUM) {
+                rowsum += __shfl_xor(rowsum, 32);  // the other half of this pixel's reduction bytes
+                ncorr = -p.zw * rowsum;
+            }
+            for (int nb0 = 0; nb0 < nb_count; nb0 += NBU) {
+                v4i bf[NBU][KU];
+#pragma unroll
+                for (int u = 0; u < NBU; ++u) {
+                    const int nb = nb0 + u < nb_count ? nb0 + u : nb_count - 1;
+#pragma unroll
+                    for (int t = 0; t < KU; ++t) bf[u][t] = b_s[(nb * ksteps + (t < ksteps ? t : ksteps - 1)) * 64 + lane];
+                }
+#pragma unroll
+                for (int u = 0; u < NBU; ++u) {
+                    if (nb0 + u >= nb_count) break;
+                    v16i acc;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[i] = 0;
+#pragma unroll
+                    for (int t = 0; t < KU; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[u][t], af[t], acc, 0, 0, 0);
+                    finish_block(acc, nb0 + u, ncorr, ok, out_off);
+                }
+            }
+            ok = ok_next;
+            in_off = in_next;
+            out_off = out_next;
+#pragma unroll
+            for (int t = 0; t < KU; ++t) {
+                lo[t] = lo_next[t];
+                hi[t] = hi_next[t];
+            }
+        }
+    } else {
+        for (int rb = blockIdx.x * 4 + wave; rb < row_blocks; rb += rb_stride) {
+            bool ok;
+            size_t in_off, out_off;
+            locate(rb, ok, in_off, out_off);
+            for (int nb0 = 0; nb0 < nb_count; nb0 += NBU) {
+                v16i acc[NBU];
+#pragma unroll
+                for (int u = 0; u < NBU; ++u)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[u][i] = 0;
+                int rowsum = 0;
+                for (int ks0 = 0; ks0 < ksteps; ks0 += KU) {
+                    // steps past the last one read bytes that flip to 0, so they multiply whatever weights they re-read by zero
+                    uint2 lo[KU], hi[KU];
+#pragma unroll
+                    for (int t = 0; t < KU; ++t) load_a(ok, in_off, ks0 + t, lo[t], hi[t]);
+#pragma unroll
+                    for (int t = 0; t < KU; ++t) {
+                        const v4i af = to_fragment(lo[t], hi[t], rowsum);
+                        const int ks = ks0 + t < ksteps ? ks0 + t : ksteps - 1;
+#pragma unroll
+                        for (int u = 0; u < NBU; ++u) {
+                            const int nb = nb0 + u < nb_count ? nb0 + u : nb_count - 1;
+                            acc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b_s[(nb * ksteps + ks) * 64 + lane], af, acc[u], 0, 0, 0);
+                        }
                     }
-                    packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
                 }
-            };
-            if constexpr (!FAST)
-                quantize(std::integral_constant<int, 0>{});
-            else if (rq.fast == 2)
-                quantize(std::integral_constant<int, 2>{});
-            else
-                quantize(std::integral_constant<int, 1>{});
-            if (stage_out) {
-                if (n < p.n) {
-                    uint2 *dst2 = reinterpret_cast<uint2 *>(wave_stage + r * p.n + n);
-                    dst2[0] = make_uint2(packed[0], packed[1]);
-                    if (n + 8 < p.n) dst2[1] = make_uint2(packed[2], packed[3]);
+                int ncorr = 0;
+                if constexpr (ROWSUM) {
+                    rowsum += __shfl_xor(rowsum, 32);
+                    ncorr = -p.zw * rowsum;
                 }
-                continue;
-            }
-            if (!row_ok || n >= p.n) continue;
-            uint8_t *dst = p.out + out_off + n;
-            if (aligned16 && n + 16 <= p.n) {
-                *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
-            } else {
-                const int cnt = p.n - n < 16 ? p.n - n : 16;
-                for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
-            }
-        }
-    }
-    if (stage_out) {
-        __syncthreads();
-        const int m_wave = (blockIdx.x * 4 + wave) * 32;
-        const int rows = p.m - m_wave < 32 ? p.m - m_wave : 32;
-        const int bytes = rows > 0 ? rows * p.n : 0;  // a multiple of 8
-        uint8_t *dst = p.out + (size_t)m_wave * p.n;   // 16-byte aligned: m_wave is a multiple of 32
-        for (int off = lane * 16; off < bytes; off += 64 * 16) {
-            if (off + 16 <= bytes) {
-                *reinterpret_cast<uint4 *>(dst + off) = *reinterpret_cast<const uint4 *>(wave_stage + off);
-            } else {
-                *reinterpret_cast<uint2 *>(dst + off) = *reinterpret_cast<const uint2 *>(wave_stage + off);
+#pragma unroll
+                for (int u = 0; u < NBU; ++u) {
+                    if (nb0 + u >= nb_count) break;
+                    finish_block(acc[u], nb0 + u, ncorr, ok, out_off);
+                }
             }
         }
     }
@@ -202,27 +239,33 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
 template <int NBU, int KU>
 int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     const int n_blocks = (p.n + 31) / 32, ksteps = p.k_pad / 32;
-    // enough waves to fill 256 CUs several times over: with few pixels the channel-block groups are spread over grid.y too
-    const int row_groups = (p.m + 127) / 128, n_groups = (n_blocks + NBU - 1) / NBU;
-    int split = 1;
-    while (split < n_groups && (long)row_groups * split < 2048) ++split;
-    const dim3 grid(row_groups, split);
-    // rows of one pixel block contiguous in the output (see the kernel): identity pixel mapping, no channel offset
-    const bool linear = split == 1 && p.ldc == p.n && (p.n & 7) == 0 && p.n <= 384 && p.out_sy == 1 && p.out_sx == 1 &&
-                        p.out_y0 == 0 && p.out_x0 == 0 && p.out_h == p.ho && p.out_w == p.wo &&
-                        (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
-    const int stage_out = linear ? 1 : 0;
-    const size_t lds = linear ? (size_t)4 * 32 * p.n : 0;
+    const int row_blocks = (p.m + 31) / 32;
+    // Channel ranges: as few as the LDS budget for the weights allows (32 KiB, so that several workgroups share a CU),
+    // more when the pixel rows alone do not give every SIMD a few waves.
+    const int groups_total = (n_blocks + NBU - 1) / NBU;
+    int nbw_max = (32 / ksteps) / NBU * NBU;
+    if (nbw_max < NBU) nbw_max = NBU;
+    int ranges = (n_blocks + nbw_max - 1) / nbw_max;
+    while (ranges < groups_total && (long)row_blocks * ranges < 2048) ++ranges;
+    const int nbw = (groups_total + ranges - 1) / ranges * NBU;
+    ranges = (n_blocks + nbw - 1) / nbw;
+    int row_wgs = (row_blocks + 3) / 4;
+    static const int tune_wgs = getenv("EH_THIN_WGS") ? atoi(getenv("EH_THIN_WGS")) : 1024;
+    const int wg_target = tune_wgs / ranges > 0 ? tune_wgs / ranges : 1;  // four workgroups per CU over the whole launch
+    if (row_wgs > wg_target) row_wgs = wg_target;
+    const dim3 grid(row_wgs, ranges);
+    const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t);
+    EH_REQUIRE(lds <= 64 * 1024, "igemm_thin: %zu bytes of LDS for the weights", lds);
     if (p.zw != 0) {
         if (p.rq.fast)
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
         else
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
     } else {
         if (p.rq.fast)
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
         else
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, stage_out);
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
     }
     EH_HIP(hipGetLastError());
     return EH_OK;
