@@ -43,17 +43,17 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
     const int nb_first = blockIdx.y * nbw;
     const int nb_count = n_blocks - nb_first < nbw ? n_blocks - nb_first : nbw;  // blocks of this range that exist
 
-    // this range's weights (fragment order: 1 KiB per block and step) and bias, once per workgroup
+    // this range's weights (fragment order: 1 KiB per block and step) and bias live in LDS, copied once per workgroup
     extern __shared__ __align__(16) uint8_t lds_raw[];
     v4i *b_s = reinterpret_cast<v4i *>(lds_raw);                                  // [nbw][ksteps][64 lanes]
     int32_t *bias_s = reinterpret_cast<int32_t *>(lds_raw + (size_t)nbw * ksteps * 1024);  // [nbw * 32]
-    {
+    auto stage_weights = [&]() {
         const v4i *src = reinterpret_cast<const v4i *>(p.b) + (size_t)nb_first * ksteps * 64;
         const int pieces = nb_count * ksteps * 64;
         for (int i = threadIdx.x; i < pieces; i += 256) b_s[i] = src[i];
         for (int i = threadIdx.x; i < nb_count * 32; i += 256) bias_s[i] = p.bias[nb_first * 32 + i];
-    }
-    __syncthreads();
+        __syncthreads();
+    };
 
     const RequantDev rq = p.rq;
     const bool wide = (p.ldc & 3) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 3) == 0);  // dword-aligned rows: vector stores
@@ -152,6 +152,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         locate(rb, ok, in_off, out_off);
 #pragma unroll
         for (int t = 0; t < KU; ++t) load_a(ok, in_off, t, lo[t], hi[t]);
+        stage_weights();  // after the first activation loads are on their way: the two latencies overlap
         for (; rb < row_blocks; rb += rb_stride) {
             locate(rb + rb_stride, ok_next, in_next, out_next);
 #pragma unroll
@@ -194,6 +195,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
             }
         }
     } else {
+        stage_weights();
         for (int rb = blockIdx.x * 4 + wave; rb < row_blocks; rb += rb_stride) {
             bool ok;
             size_t in_off, out_off;
