@@ -151,7 +151,7 @@ def deconv_workload(eden, synth, n=8):
 def mbv2_workload(eden, synth, batch=64):
     """BASELINE.json configs[4]: MobileNetV2-1.0 uint8 at 224x224x3, batch 64, the whole operator list per step."""
     mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
-    net = mobilenet.MobileNetV2(eden, batch)
+    net = mobilenet.MobileNetV2(eden, batch, fuse_add=True)  # residual adds inside the projection convolutions' launches
     net.set_input(mobilenet.network_input(batch))
     return dict(name="mobilenet_v2_1.0_224_u8_batch%d" % batch, launch=lambda s: net.run(s), keep=net,
                 ops=2.0 * mobilenet.macs_per_image() * batch, bytes=mobilenet.compulsory_bytes_per_image() * batch,

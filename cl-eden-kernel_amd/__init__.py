@@ -69,6 +69,9 @@ EXPORTS = {
     "eh_probe_mfma_i8": (C.c_int, [C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
     "eh_make_requant_perchannel": (None, [C.c_float, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32, C.c_int, C.c_int,
                                           C.POINTER(Requant), C.c_void_p, C.c_void_p]),
+    "eh_conv2d_u8_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(AddRequant),
+                                       C.c_void_p]),
+    "eh_conv2d_u8_fuses_add": (C.c_int, [C.c_void_p]),
     "eh_conv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "eh_dwconv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "eh_deconv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
@@ -308,6 +311,15 @@ def make_requant_perchannel(s_in, zp_in, filter_scales, s_out, zp_out, act=ACT_N
     load().eh_make_requant_perchannel(s_in, zp_in, scales.ctypes.data, scales.size, s_out, zp_out, act, int(act_enabled),
                                       C.byref(q), mult.ctypes.data, shift.ctypes.data)
     return q, mult, shift
+
+
+def _conv_run_add(self, d_in, d_residual, d_out, q, aq, stream=None):
+    """d_out = add(d_residual, convolution(d_in)) with the add parameters `aq` (the residual is the first operand)"""
+    check(load().eh_conv2d_u8_run_add(self.handle, d_in.ptr, d_residual.ptr, d_out.ptr, C.byref(q), C.byref(aq), stream))
+
+
+ConvPlan.run_add = _conv_run_add
+ConvPlan.fuses_add = lambda self: bool(load().eh_conv2d_u8_fuses_add(self.handle))
 
 
 class DwConvPlan(_Plan):

@@ -290,10 +290,21 @@ struct GemmOp {
         return EH_OK;
     }
 
-    int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream) {
+    // the one-tap kernel and the split-reduction epilogue of the tiled kernel can add a residual tensor
+    bool fuses_add() const {
+        bool fuse = layout == EH_NHWC && !io_signed && !parts.empty();
+        for (auto &g : parts) fuse = fuse && (g.cfg.id == GEMM_THIN || g.cfg.id == GEMM_DMA_64x64_SPLITK);
+        return fuse;
+    }
+
+    // residual != null: output = add(residual, result) with `radd`; `fused` tells whether the kernels did it
+    int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream, const uint8_t *residual = nullptr,
+            const AddDev *radd = nullptr, bool *fused = nullptr) {
         EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
         int rc = check_requant(nq, w_signed, io_signed);
         if (rc) return rc;
+        const bool fuse = residual != nullptr && fuses_add();
+        if (fused) *fused = fuse;
         if ((rc = refold(*nq, stream))) return rc;
         const uint8_t *in = static_cast<const uint8_t *>(input);
         uint8_t *out = static_cast<uint8_t *>(output);
@@ -318,6 +329,8 @@ struct GemmOp {
             p.a_xor = 0x80808080u ^ p.out_xor;
             p.fill = ((uint32_t)q.zp_in * 0x01010101u) ^ p.out_xor;
             p.rq = make_requant_dev(q);
+            p.residual = fuse ? residual + g.bias_base : nullptr;
+            if (fuse) p.radd = *radd;
             if (pc_multiplier) {
                 p.rq.pc_multiplier = pc_multiplier + g.bias_base;
                 p.rq.pc_shift = pc_shift + g.bias_base;
@@ -794,6 +807,28 @@ int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const 
     if (plan->d.n == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);  // zero-size early-out, as CLConvolution::execute does
     return plan->op.run(input, output, q, as_stream(stream));
 }
+
+int eh_conv2d_u8_run_add(eh_conv_plan *plan, const void *input, const void *residual, void *output, const eh_requant *q,
+                         const eh_add_requant *aq, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    EH_REQUIRE(!plan->op.io_signed, "run_add: int8 tensors are not offered (the reference's int8 add is a float kernel)");
+    int rc = check_add_requant(aq);
+    if (rc) return rc;
+    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);
+    EH_REQUIRE(residual != nullptr, "run_add: residual pointer is null");
+    const AddDev radd = make_add_dev(*aq);
+    bool fused = false;
+    if ((rc = plan->op.run(input, output, q, as_stream(stream), static_cast<const uint8_t *>(residual), &radd, &fused))) return rc;
+    if (fused) return EH_OK;
+    // kernels without the fused epilogue: the convolution's own result, then the add in place
+    const eh_conv_desc &d = plan->d;
+    const int64_t count = (int64_t)d.n * d.cout * eh_conv_out_dim(d.h, d.pad_t, d.pad_b, d.kh, d.dil_h, d.stride_h) *
+                          eh_conv_out_dim(d.w, d.pad_l, d.pad_r, d.kw, d.dil_w, d.stride_w);
+    return launch_add_u8(static_cast<const uint8_t *>(residual), static_cast<const uint8_t *>(output),
+                         static_cast<uint8_t *>(output), count, radd, as_stream(stream));
+}
+
+int eh_conv2d_u8_fuses_add(const eh_conv_plan *plan) { return plan != nullptr && plan->op.fuses_add() ? 1 : 0; }
 
 int eh_conv2d_u8_destroy(eh_conv_plan *plan) {
     if (plan) {

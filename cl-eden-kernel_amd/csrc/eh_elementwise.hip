@@ -14,39 +14,6 @@
 namespace eh {
 namespace {
 
-struct AddDev {
-    int32_t zp_a, zp_b, zp_out, left_shift;
-    int32_t mult_a, rs_a, mult_b, rs_b, mult_out, rs_out;
-    int32_t act_min, act_max;
-};
-
-// SaturatingRoundingDoublingHighMul for a non-negative multiplier (no saturation case), then
-// RoundingDivideByPOT
-__device__ __forceinline__ int32_t mul_round_shift(int32_t x, int32_t mult, int32_t rs) {
-    const int64_t ab = (int64_t)x * (int64_t)mult + (1ll << 30);
-    const int32_t v = (int32_t)(ab >> 31);
-    const int32_t mask = (int32_t)((1u << rs) - 1u);
-    const int32_t rem = v & mask;
-    const int32_t thr = (mask >> 1) - (v >> 31);
-    return (v >> rs) + (rem > thr ? 1 : 0);
-}
-
-__device__ __forceinline__ uint32_t add_one(uint32_t a, uint32_t b, const AddDev &q) {
-    const int32_t va = (int32_t)(((uint32_t)((int32_t)a - q.zp_a)) << q.left_shift);
-    const int32_t vb = (int32_t)(((uint32_t)((int32_t)b - q.zp_b)) << q.left_shift);
-    const int32_t sa = mul_round_shift(va, q.mult_a, q.rs_a);
-    const int32_t sb = mul_round_shift(vb, q.mult_b, q.rs_b);
-    int32_t r = mul_round_shift(sa + sb, q.mult_out, q.rs_out) + q.zp_out;
-    r = r < q.act_min ? q.act_min : r;
-    r = r > q.act_max ? q.act_max : r;
-    return (uint32_t)r;
-}
-
-__device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b, const AddDev &q) {
-    return add_one(a & 255u, b & 255u, q) | (add_one((a >> 8) & 255u, (b >> 8) & 255u, q) << 8) |
-           (add_one((a >> 16) & 255u, (b >> 16) & 255u, q) << 16) | (add_one(a >> 24, b >> 24, q) << 24);
-}
-
 // 16 bytes per thread where the three pointers allow it, bytes for the tail
 __global__ __launch_bounds__(256) void add_u8_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
                                                      uint8_t *__restrict__ out, const int64_t count, const int64_t vec_count,
@@ -171,6 +138,29 @@ __global__ __launch_bounds__(256) void avgpool_scalar_kernel(const uint8_t *__re
 }
 
 }  // namespace
+
+int check_add_requant(const eh_add_requant *q) {
+    EH_REQUIRE(q != nullptr, "add: null parameters");
+    EH_REQUIRE(q->mult_a >= 0 && q->mult_b >= 0 && q->mult_out >= 0, "add: negative multiplier");
+    EH_REQUIRE(q->left_shift >= 0 && q->left_shift <= 23, "add: left shift %d outside [0, 23]", q->left_shift);
+    EH_REQUIRE(q->shift_a >= -31 && q->shift_b >= -31 && q->shift_out >= -31, "add: shift below -31");
+    EH_REQUIRE(q->act_min >= 0 && q->act_max <= 255 && q->act_min <= q->act_max, "add: activation range [%d, %d] invalid",
+               q->act_min, q->act_max);
+    return EH_OK;
+}
+
+int launch_add_u8(const uint8_t *a, const uint8_t *b, uint8_t *out, int64_t count, const AddDev &d, hipStream_t stream) {
+    if (count <= 0) return EH_OK;
+    const bool wide = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const int64_t vec_count = wide ? count / 16 : 0;
+    const int64_t threads = vec_count + (count - vec_count * 16);
+    const int64_t blocks = (threads + 255) / 256;
+    EH_REQUIRE(blocks < (1ll << 31), "add: tensor too large");
+    hipLaunchKernelGGL(add_u8_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a, b, out, count, vec_count, d);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
+
 }  // namespace eh
 
 using namespace eh;
@@ -198,35 +188,10 @@ int eh_add_u8(const void *a, const void *b, void *out, int64_t count, const eh_a
     EH_REQUIRE(count >= 0, "add: negative count");
     if (count == 0) return EH_OK;
     EH_REQUIRE(a && b && out, "add: null tensor");
-    EH_REQUIRE(q->mult_a >= 0 && q->mult_b >= 0 && q->mult_out >= 0, "add: negative multiplier");
-    EH_REQUIRE(q->left_shift >= 0 && q->left_shift <= 23, "add: left shift %d outside [0, 23]", q->left_shift);
-    EH_REQUIRE(q->shift_a >= -31 && q->shift_b >= -31 && q->shift_out >= -31, "add: shift below -31");
-    EH_REQUIRE(q->act_min >= 0 && q->act_max <= 255 && q->act_min <= q->act_max, "add: activation range [%d, %d] invalid",
-               q->act_min, q->act_max);
-    AddDev d;
-    d.zp_a = q->zp_a;
-    d.zp_b = q->zp_b;
-    d.zp_out = q->zp_out;
-    d.left_shift = q->left_shift;
-    d.mult_a = q->mult_a;
-    d.mult_b = q->mult_b;
-    d.mult_out = q->mult_out;
-    // a positive shift (a multiplier of 1 or more) is applied as no shift, as the reference kernel's fall-through does
-    d.rs_a = q->shift_a < 0 ? -q->shift_a : 0;
-    d.rs_b = q->shift_b < 0 ? -q->shift_b : 0;
-    d.rs_out = q->shift_out < 0 ? -q->shift_out : 0;
-    d.act_min = q->act_min;
-    d.act_max = q->act_max;
-    const bool wide = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-    const int64_t vec_count = wide ? count / 16 : 0;
-    const int64_t threads = vec_count + (count - vec_count * 16);
-    const int64_t blocks = (threads + 255) / 256;
-    EH_REQUIRE(blocks < (1ll << 31), "add: tensor too large");
-    hipLaunchKernelGGL(add_u8_kernel, dim3((unsigned)blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
-                       static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), static_cast<uint8_t *>(out), count,
-                       vec_count, d);
-    EH_HIP(hipGetLastError());
-    return EH_OK;
+    int rc = check_add_requant(q);
+    if (rc) return rc;
+    return launch_add_u8(static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), static_cast<uint8_t *>(out), count,
+                         make_add_dev(*q), reinterpret_cast<hipStream_t>(stream));
 }
 
 int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *stream) {

@@ -535,8 +535,25 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
             reduce(std::integral_constant<int, 1>{});
         else
             reduce(std::integral_constant<int, 0>{});
-        uint8_t *dst = p.out + out_pixel_offset(p, m, plane) + n;
+        const size_t out_off = out_pixel_offset(p, m, plane) + n;
+        uint8_t *dst = p.out + out_off;
         const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+        if (p.residual) {  // out = add(residual, result); only this split-reduction epilogue offers it
+            const uint8_t *res = p.residual + out_off;
+            if (aligned16 && n + 16 <= p.n && (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) {
+                const uint4 rv = *reinterpret_cast<const uint4 *>(res);
+                packed[0] = add_word(rv.x, packed[0], p.radd);
+                packed[1] = add_word(rv.y, packed[1], p.radd);
+                packed[2] = add_word(rv.z, packed[2], p.radd);
+                packed[3] = add_word(rv.w, packed[3], p.radd);
+            } else {
+                const int cnt = p.n - n < 16 ? p.n - n : 16;
+                for (int t = 0; t < cnt; ++t) {
+                    const uint32_t v = add_one(res[t], (packed[t >> 2] >> (8 * (t & 3))) & 255u, p.radd);
+                    packed[t >> 2] = (packed[t >> 2] & ~(255u << (8 * (t & 3)))) | (v << (8 * (t & 3)));
+                }
+            }
+        }
         if (aligned16 && n + 16 <= p.n) {
             *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
         } else {

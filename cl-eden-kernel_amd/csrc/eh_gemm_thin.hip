@@ -132,6 +132,22 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         if (!ok || n >= p.n) return;
         uint8_t *dst = p.out + out_off + n;
         const int cnt = p.n - n;
+        if (p.residual) {  // out = add(residual, result); the residual tensor is addressed like the output
+            const uint8_t *res = p.residual + out_off + n;
+            if (wide && cnt >= 16) {
+                const u32x4_a4 rv = *reinterpret_cast<const u32x4_a4 *>(res);
+                packed[0] = add_word(rv.x, packed[0], p.radd);
+                packed[1] = add_word(rv.y, packed[1], p.radd);
+                packed[2] = add_word(rv.z, packed[2], p.radd);
+                packed[3] = add_word(rv.w, packed[3], p.radd);
+            } else {
+                const int c = cnt < 16 ? cnt : 16;
+                for (int t = 0; t < c; ++t) {
+                    const uint32_t v = add_one(res[t], (packed[t >> 2] >> (8 * (t & 3))) & 255u, p.radd);
+                    packed[t >> 2] = (packed[t >> 2] & ~(255u << (8 * (t & 3)))) | (v << (8 * (t & 3)));
+                }
+            }
+        }
         if (wide && cnt >= 16) {
             *reinterpret_cast<u32x4_a4 *>(dst) = u32x4_a4{packed[0], packed[1], packed[2], packed[3]};
         } else if (wide && cnt == 8) {

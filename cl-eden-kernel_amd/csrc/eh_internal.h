@@ -185,6 +185,65 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) { retu
 // signed_weights: zp_w is an int8 zero point; signed_io: zp_in, zp_out and the activation range are int8 values
 int check_requant(const eh_requant *q, bool signed_weights = false, bool signed_io = false);
 
+// ---------------------------------------------------------------- quantized add
+// The reference's quantized add (gpu/operators/cl_kernels/AddKernelsQauntized.cpp:135-215): both inputs shifted
+// left, brought to a common scale by a Q31 multiplier and a rounding right shift each, summed, rescaled, offset,
+// clamped.  Lives here because the GEMM epilogues can apply it to their result and a residual tensor.
+struct AddDev {
+    int32_t zp_a, zp_b, zp_out, left_shift;
+    int32_t mult_a, rs_a, mult_b, rs_b, mult_out, rs_out;
+    int32_t act_min, act_max;
+};
+
+// SaturatingRoundingDoublingHighMul for a non-negative multiplier (no saturation case), then
+// RoundingDivideByPOT
+__host__ __device__ __forceinline__ int32_t mul_round_shift(int32_t x, int32_t mult, int32_t rs) {
+    const int64_t ab = (int64_t)x * (int64_t)mult + (1ll << 30);
+    const int32_t v = (int32_t)(ab >> 31);
+    const int32_t mask = (int32_t)((1u << rs) - 1u);
+    const int32_t rem = v & mask;
+    const int32_t thr = (mask >> 1) - (v >> 31);
+    return (v >> rs) + (rem > thr ? 1 : 0);
+}
+
+__host__ __device__ __forceinline__ uint32_t add_one(uint32_t a, uint32_t b, const AddDev &q) {
+    const int32_t va = (int32_t)(((uint32_t)((int32_t)a - q.zp_a)) << q.left_shift);
+    const int32_t vb = (int32_t)(((uint32_t)((int32_t)b - q.zp_b)) << q.left_shift);
+    const int32_t sa = mul_round_shift(va, q.mult_a, q.rs_a);
+    const int32_t sb = mul_round_shift(vb, q.mult_b, q.rs_b);
+    int32_t r = mul_round_shift(sa + sb, q.mult_out, q.rs_out) + q.zp_out;
+    r = r < q.act_min ? q.act_min : r;
+    r = r > q.act_max ? q.act_max : r;
+    return (uint32_t)r;
+}
+
+__host__ __device__ __forceinline__ uint32_t add_word(uint32_t a, uint32_t b, const AddDev &q) {
+    return add_one(a & 255u, b & 255u, q) | (add_one((a >> 8) & 255u, (b >> 8) & 255u, q) << 8) |
+           (add_one((a >> 16) & 255u, (b >> 16) & 255u, q) << 16) | (add_one(a >> 24, b >> 24, q) << 24);
+}
+
+
+inline AddDev make_add_dev(const eh_add_requant &q) {
+    AddDev d;
+    d.zp_a = q.zp_a;
+    d.zp_b = q.zp_b;
+    d.zp_out = q.zp_out;
+    d.left_shift = q.left_shift;
+    d.mult_a = q.mult_a;
+    d.mult_b = q.mult_b;
+    d.mult_out = q.mult_out;
+    // a positive shift (a multiplier of 1 or more) is applied as no shift, as the reference kernel's fall-through does
+    d.rs_a = q.shift_a < 0 ? -q.shift_a : 0;
+    d.rs_b = q.shift_b < 0 ? -q.shift_b : 0;
+    d.rs_out = q.shift_out < 0 ? -q.shift_out : 0;
+    d.act_min = q.act_min;
+    d.act_max = q.act_max;
+    return d;
+}
+int check_add_requant(const eh_add_requant *q);
+// out = add(a, b) over `count` bytes on `stream` (out may be a or b)
+int launch_add_u8(const uint8_t *a, const uint8_t *b, uint8_t *out, int64_t count, const AddDev &d, hipStream_t stream);
+
 // ---------------------------------------------------------------- implicit GEMM
 // One row of the k-table describes one load unit (VEC bytes) of the reduction
 // axis: where it sits relative to the top-left input pixel of an output pixel.
@@ -236,6 +295,10 @@ struct GemmProblem {
     // int8 tensors (PrecisionType::INT8) run as their uint8 equivalents (value + 128, zero points + 128):
     uint32_t a_xor;    // turns four stored activation bytes into int8 MFMA operands: 0x80808080 for uint8 data, 0 for int8
     uint32_t out_xor;  // turns four uint8 results into the stored bytes: 0 for uint8 data, 0x80808080 for int8
+    // fused residual add (one-tap and split-reduction kernels only): out = add(residual, result) with `radd`;
+    // `residual` is addressed like `out`.  Null: plain convolution.
+    const uint8_t *residual;
+    AddDev radd;
     RequantDev rq;
 };
 

@@ -136,17 +136,36 @@ def compulsory_bytes_per_image(image=224):
 
 
 class MobileNetV2:
-    """The operator list instantiated on the GPU for one batch size.  Activations are channels-last."""
+    """The operator list instantiated on the GPU for one batch size.  Activations are channels-last.
 
-    def __init__(self, eden, batch, image=224, stream=None):
+    fuse_add: a residual Add whose second operand is the projection convolution right before it (and nothing else
+    reads that projection) runs inside that convolution's launch (`ConvPlan.run_add`); the projection's own tensor
+    is then never written.  Results are the same bit for bit."""
+
+    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False):
         self.eden, self.batch, self.image = eden, batch, image
         self.tensors, self.ops = layers(image)
         self.buffers = [eden.DeviceBuffer(nbytes=batch * t["h"] * t["w"] * t["c"]) for t in self.tensors]
         self.steps = []
         self._keep = []
+        self.unwritten = set()  # tensors a fused step skips
+        readers = {}
         for op in self.ops:
+            for key in ("src", "a", "b"):
+                if key in op:
+                    readers[op[key]] = readers.get(op[key], 0) + 1
+        for index, op in enumerate(self.ops):
             kind = op["op"]
             if kind == "add":
+                prev = self.steps[-1] if self.steps else None
+                if (fuse_add and prev and prev[0] == "plan" and self.ops[index - 1]["op"] == "conv" and
+                        self.ops[index - 1]["dst"] == op["b"] and readers.get(op["b"], 0) == 1):
+                    a, b, d = (self.tensors[op[k]] for k in ("a", "b", "dst"))
+                    q_add = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
+                    plan, src, _, q = prev[1]
+                    self.steps[-1] = ("plan_add", (plan, src, self.buffers[op["a"]], self.buffers[op["dst"]], q, q_add))
+                    self.unwritten.add(op["b"])
+                    continue
                 a, b, d = (self.tensors[op[k]] for k in ("a", "b", "dst"))
                 q = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
                 count = batch * d["h"] * d["w"] * d["c"]
@@ -190,6 +209,9 @@ class MobileNetV2:
             if kind == "plan":
                 plan, src, dst, q = args
                 plan.run(src, dst, q, stream)
+            elif kind == "plan_add":
+                plan, src, residual, dst, q, q_add = args
+                plan.run_add(src, residual, dst, q, q_add, stream)
             elif kind == "add":
                 a, b, dst, count, q = args
                 eden.add_u8(a, b, dst, count, q, stream)

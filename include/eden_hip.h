@@ -234,6 +234,16 @@ int eh_conv2d_u8_set_perchannel(eh_conv_plan *plan, const int32_t *multipliers, 
                                 void *stream);
 int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
 int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
+/* Convolution followed by the quantized residual add, output = add(residual, convolution) with `aq` as eh_add_u8
+ * applies it (the residual is the add's first operand; it has the output's shape and layout and must not be the
+ * output buffer).  Bit for bit what eh_conv2d_u8_run into a temporary followed by eh_add_u8 gives; the one-tap and
+ * split-reduction GEMM kernels add in their epilogue, other kernels run the add as a second launch in place.  No
+ * counterpart in the reference, whose operator list runs CLConvolution and CLAdd one after the other
+ * (gpu/gpu_op_executor.cc:56-103); offered for uint8 tensors only. */
+int eh_conv2d_u8_run_add(eh_conv_plan *plan, const void *input, const void *residual, void *output, const eh_requant *q,
+                         const eh_add_requant *aq, void *stream);
+/* 1 when eh_conv2d_u8_run_add on this plan is a single launch (the add happens in the kernel's epilogue), else 0 */
+int eh_conv2d_u8_fuses_add(const eh_conv_plan *plan);
 int eh_conv2d_u8_destroy(eh_conv_plan *plan);
 
 /* CLDepthwiseConvolution::initialize / execute / release, uint8 branch

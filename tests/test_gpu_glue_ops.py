@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from harness import eden, synth
+from harness import eden, synth, to_eh_requant
 
 pytestmark = pytest.mark.gpu
 
@@ -108,3 +108,51 @@ def test_avgpool_int8_matches_oracle(case, layout):
     got = d_out.download((n, ho, wo, c)).transpose(0, 3, 1, 2) if nhwc else d_out.download(want.shape)
     assert np.array_equal(np.ascontiguousarray(got).view(np.int8), want)
     assert want.std() > 1
+
+
+RUN_ADD_CASES = [
+    # one-tap kernel (fused), split-reduction tiles (fused), 128 x 128 tiles and the register-staged kernel (second launch)
+    dict(n=2, c=144, h=14, w=14, cout=24, kh=1, kw=1, fused=True),
+    dict(n=2, c=32, h=9, w=9, cout=40, kh=1, kw=1, fused=True),
+    dict(n=4, c=384, h=14, w=14, cout=64, kh=1, kw=1, fused=True),
+    dict(n=2, c=576, h=7, w=7, cout=96, kh=1, kw=1, fused=True),
+    dict(n=32, c=264, h=28, w=28, cout=256, kh=1, kw=1, fused=False),
+    dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2, fused=False),
+]
+
+
+@pytest.mark.parametrize("layout", ["nhwc", "nchw"])
+@pytest.mark.parametrize("case", RUN_ADD_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_conv_with_residual_add_equals_conv_then_add(case, layout):
+    print("conv + add", case, layout, flush=True)
+    case = dict(case)
+    fused = case.pop("fused")
+    s = O.conv_shape(**case)
+    ho, wo = O.conv_out_hw(s)
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 500 + s.c)
+    w = synth.fill_u8_normal((s.cout, s.c // s.groups, s.kh, s.kw), SEED + 501, 131, 20)
+    b = synth.fill_i32((s.cout,), SEED + 502, -500, 500)
+    res = synth.fill_u8((s.n, s.cout, ho, wo), SEED + 503)
+    fan = (s.c // s.groups) * s.kh * s.kw
+    s_out = float(0.02 * 0.005 * 74.0 * 20.0 * np.sqrt(fan) / 30.0)
+    for act, en in ((O.ACT_NONE, False), (O.ACT_RELU, True)):
+        q = O.make_quant(0.02, 117, 0.005, 131, s_out, 128, act, en)
+        aq = O.make_add_quant(0.031, 120, s_out, 128, 0.05, 125, O.ACT_NONE, False)
+        want = O.add(res, O.conv2d(x, w, b, s, q), aq)
+        nhwc = layout == "nhwc"
+        desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, (s.stride_h, s.stride_w), (s.pad_t, s.pad_b, s.pad_l, s.pad_r),
+                              (1, 1), s.groups, 1, eden.NHWC if nhwc else eden.NCHW, eden.W_OIHW)
+        to_dev = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))) if nhwc else (lambda a: a)
+        d_x, d_w, d_b = eden.DeviceBuffer(host=to_dev(x)), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+        d_r, d_o = eden.DeviceBuffer(host=to_dev(res)), eden.DeviceBuffer(nbytes=want.size)
+        plan = eden.ConvPlan(desc, d_w, d_b, to_eh_requant(q))
+        assert plan.fuses_add() == (fused and nhwc)
+        plan.run_add(d_x, d_r, d_o, to_eh_requant(q), to_eh_add(aq))
+        got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2) if nhwc else d_o.download(want.shape)
+        assert np.array_equal(got, want), int((got != want).sum())
+        # the plan still runs without the add
+        plan.run(d_x, d_o, to_eh_requant(q))
+        got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2) if nhwc else d_o.download(want.shape)
+        assert np.array_equal(got, O.conv2d(x, w, b, s, q))
+        plan.destroy()
+    assert want.std() > 4
