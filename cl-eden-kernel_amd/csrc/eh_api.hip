@@ -195,8 +195,7 @@ static int check_perchannel(const int32_t *multipliers, const int32_t *shifts, i
 
 // The per-channel arrays with `pad` zero entries behind them (kernels read whole channel blocks), written by one
 // blocking copy each from a padded host image, once the stream's earlier work that may still read the arrays is
-// done.  (A memset of the whole array followed by an asynchronous copy of its head from pageable memory left
-// zeros in place of some pairs now and then.)
+// done.
 static int upload_padded_pairs(int32_t *d_mult, int32_t *d_shift, const int32_t *multipliers, const int32_t *shifts,
                                int32_t count, int32_t pad, hipStream_t stream) {
     std::vector<int32_t> image((size_t)count + pad, 0);
@@ -548,7 +547,11 @@ int eh_malloc(void **ptr, size_t bytes) {
     *ptr = nullptr;
     const size_t padded = (bytes + 255) / 256 * 256 + 256;
     EH_HIP(hipMalloc(ptr, padded));
+    // The fill is queued on the null stream and hipMemset may return before it has run; the streams this library
+    // hands out do not synchronize with the null stream, so the caller's first write on such a stream could otherwise
+    // be overtaken by the zeros.  Wait for the fill.
     hipError_t e = hipMemset(*ptr, 0, padded);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
     if (e != hipSuccess) {
         (void)hipFree(*ptr);
         *ptr = nullptr;

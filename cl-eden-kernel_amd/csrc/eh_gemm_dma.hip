@@ -146,11 +146,13 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KSTEPS >= 2 && KSTEPS % 2 == 0, "wave tile is made of 32x32x32 MFMA steps; fragment registers alternate between two sets");
     static_assert(BM % (RPB * 4) == 0 && BN % (RPB * 4) == 0, "whole DMA blocks per wave");
     static_assert((STAGES - 1) * LPS <= 63, "vmcnt is a 6-bit counter");
-    static_assert(WGK == 1 || WGK * BM * PART_ROW * 4 <= STAGES * STAGE_BYTES, "partial tiles reuse the operand stages");
+    // the WGK partial tiles of the split reduction reuse the operand stages; with two stages they need a little more
+    constexpr int PARTIAL_BYTES = WGK == 1 ? 0 : WGK * BM * PART_ROW * 4;
+    constexpr int STAGE_AREA = STAGES * STAGE_BYTES > PARTIAL_BYTES ? STAGES * STAGE_BYTES : PARTIAL_BYTES;
     static_assert(WGK == 1 || (BM == 64 && BN == 64 && WGM == 1 && WGN == 1), "the split-reduction epilogue is written for one 64x64 tile");
     static_assert(WTM % CPR == 0 && WTN % CPR == 0, "every fragment row of a lane has the same swizzle");
 
-    __shared__ __align__(1024) uint8_t stages[STAGES * STAGE_BYTES];
+    __shared__ __align__(1024) uint8_t stages[STAGE_AREA];
     __shared__ int32_t rowsum_s[WGK * 2][BM];
     __shared__ __align__(16) int32_t bias_s[BN];  // read in the epilogue from LDS: a global load there would have to
                                                    // wait for the stores issued before it (one counter for both)
@@ -656,7 +658,14 @@ int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream) {
         case GEMM_DMA_256x128: return launch_cfg<256, 128, 2, 2, 1, 128, 3>(ps, count, stream);
         case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 2>(ps, count, stream);
         case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 3>(ps, count, stream);
-        case GEMM_DMA_64x64_SPLITK: return launch_cfg<64, 64, 1, 1, 4, 256, 4>(ps, count, stream);
+        case GEMM_DMA_64x64_SPLITK: {
+            // Two stages take half the LDS, so two workgroups share a CU: for reductions of one or two slabs (deeper
+            // staging has nothing to prefetch) and for launches with more tiles than CUs (the second workgroup's
+            // prologue and epilogue hide behind the first one's loop instead of forming a second round).
+            const long tiles = (long)((p.m + 63) / 64) * ((p.n + 63) / 64) * count;
+            if (p.k_pad / 256 <= 2 || tiles > 256) return launch_cfg<64, 64, 1, 1, 4, 256, 2>(ps, count, stream);
+            return launch_cfg<64, 64, 1, 1, 4, 256, 4>(ps, count, stream);
+        }
         default: break;
     }
     set_error("igemm_dma: unknown configuration %d", p.cfg.id);

@@ -15,8 +15,6 @@
 // The weight fragment is the row operand and its rows are permuted within a
 // 32-channel block (see packed_b_offset), so a lane ends up with 16 consecutive
 // output channels of its pixel: requantize, pack, one 16-byte store.
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "eh_internal.h"
@@ -264,12 +262,11 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     int nbw_max = (32 / ksteps) / NBU * NBU;
     if (nbw_max < NBU) nbw_max = NBU;
     int ranges = (n_blocks + nbw_max - 1) / nbw_max;
-    while (ranges < groups_total && (long)row_blocks * ranges < 2048) ++ranges;
+    while (ranges < groups_total && (long)row_blocks * ranges < 4096) ++ranges;
     const int nbw = (groups_total + ranges - 1) / ranges * NBU;
     ranges = (n_blocks + nbw - 1) / nbw;
     int row_wgs = (row_blocks + 3) / 4;
-    static const int tune_wgs = getenv("EH_THIN_WGS") ? atoi(getenv("EH_THIN_WGS")) : 1024;
-    const int wg_target = tune_wgs / ranges > 0 ? tune_wgs / ranges : 1;  // four workgroups per CU over the whole launch
+    const int wg_target = 1024 / ranges > 0 ? 1024 / ranges : 1;  // four workgroups per CU over the whole launch
     if (row_wgs > wg_target) row_wgs = wg_target;
     const dim3 grid(row_wgs, ranges);
     const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t);

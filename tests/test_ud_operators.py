@@ -28,6 +28,8 @@ def test_host_side_buffer_pool_and_types():
 def test_operator_classes_on_gpu():
     r = subprocess.run([_binary()], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
     print(r.stdout, flush=True)
-    assert r.returncode == 0, r.stdout[-4000:]
-    assert "FAIL" not in r.stdout
+    # on failure show what is not a plain RUN / OK line: the failed expectations and the first mismatching bytes
+    notable = "\n".join(l for l in r.stdout.splitlines() if not l.startswith(("[ RUN", "[  OK")))
+    assert r.returncode == 0, notable[-4000:]
+    assert "FAIL" not in r.stdout, notable[-4000:]
     assert "GPU operator tests failed" in r.stdout
