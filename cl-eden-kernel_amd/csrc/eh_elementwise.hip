@@ -56,14 +56,19 @@ __device__ __forceinline__ uint32_t pool_finish(int s, int cnt, const PoolDev &p
     return (uint32_t)v & 255u;
 }
 
-// channels-last: a thread owns four consecutive channels of one output pixel (c % 4 == 0)
+// channels-last: ROWS threads (adjacent lanes) own four consecutive channels of one output pixel (c % 4 == 0) and
+// share the window's rows; ROWS = 8 serves launches with few outputs and tall windows (a global pool is one long
+// chain of dependent loads otherwise), ROWS = 1 the rest
+template <int ROWS>
 __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
                                                                 const PoolDev p, const int64_t total) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= total) return;
+    const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t idx = tid / ROWS;
+    const int part = (int)(tid % ROWS);
+    const bool live = idx < total;  // whole groups of ROWS lanes are live or not; all lanes reach the shuffles
     const int cq = p.c >> 2;
-    const int c4 = (int)(idx % cq);
-    int64_t r = idx / cq;
+    const int c4 = live ? (int)(idx % cq) : 0;
+    int64_t r = live ? idx / cq : 0;
     const int ox = (int)(r % p.wo);
     r /= p.wo;
     const int oy = (int)(r % p.ho), img = (int)(r / p.ho);
@@ -80,8 +85,8 @@ __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *_
         s2 += (v >> 16) & 255u;
         s3 += v >> 24;
     };
-    // eight window pixels are requested before the first is summed: a global pool is one long chain of loads otherwise
-    for (int y = y0; y < y1; ++y) {
+    // eight window pixels are requested before the first is summed
+    for (int y = y0 + part; y < y1 && live; y += ROWS) {
         const uint8_t *row = in + ((size_t)img * p.h + y) * p.w * p.c + c4 * 4;
         int x = x0;
         for (; x + 8 <= x1; x += 8) {
@@ -97,8 +102,16 @@ __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *_
 #pragma unroll
         for (int t = 0; t < 8; ++t) take(v[t]);
     }
-    *reinterpret_cast<uint32_t *>(out + idx * 4) = pool_finish(s0, cnt, p) | (pool_finish(s1, cnt, p) << 8) |
-                                                   (pool_finish(s2, cnt, p) << 16) | (pool_finish(s3, cnt, p) << 24);
+#pragma unroll
+    for (int step = 1; step < ROWS; step <<= 1) {
+        s0 += __shfl_xor(s0, step);
+        s1 += __shfl_xor(s1, step);
+        s2 += __shfl_xor(s2, step);
+        s3 += __shfl_xor(s3, step);
+    }
+    if (live && part == 0)
+        *reinterpret_cast<uint32_t *>(out + idx * 4) = pool_finish(s0, cnt, p) | (pool_finish(s1, cnt, p) << 8) |
+                                                       (pool_finish(s2, cnt, p) << 16) | (pool_finish(s3, cnt, p) << 24);
 }
 
 // one output element per thread, either layout
@@ -229,10 +242,14 @@ int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *str
     const bool vec4 = d.layout == EH_NHWC && (d.c & 3) == 0 &&
                       ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 3) == 0;
     const int64_t total = vec4 ? outputs / 4 : outputs;
-    const int64_t blocks = (total + 255) / 256;
+    const bool split_rows = vec4 && total < 256 * 1024 && d.kh >= 4;  // few threads, tall windows: eight lanes per output
+    const int64_t blocks = ((split_rows ? total * 8 : total) + 255) / 256;
     EH_REQUIRE(blocks < (1ll << 31), "avgpool: tensor too large");
-    if (vec4)
-        hipLaunchKernelGGL(avgpool_nhwc_vec4_kernel, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint8_t *>(in),
+    if (split_rows)
+        hipLaunchKernelGGL(avgpool_nhwc_vec4_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint8_t *>(in),
+                           static_cast<uint8_t *>(out), p, total);
+    else if (vec4)
+        hipLaunchKernelGGL(avgpool_nhwc_vec4_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint8_t *>(in),
                            static_cast<uint8_t *>(out), p, total);
     else if (d.layout == EH_NHWC)
         hipLaunchKernelGGL(avgpool_scalar_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s,

@@ -69,6 +69,8 @@ POOL_CASES = [
     (1, 5, 6, 6, 2, 2, (2, 2), (0, 0, 0, 0), (10, 200)),          # odd channel count: scalar kernels
     (2, 16, 8, 8, 5, 3, (1, 2), (2, 2, 1, 1), (0, 255)),
     (1, 4, 3, 3, 3, 3, (1, 1), (2, 2, 2, 2), (0, 255)),           # some windows hold a single pixel
+    (2, 24, 13, 12, 13, 12, (1, 1), (0, 0, 0, 0), (0, 255)),      # more window rows than the lanes that share them
+    (24, 64, 40, 40, 5, 5, (1, 1), (2, 2, 2, 2), (0, 255)),       # tall windows, many outputs: one lane per output
 ]
 
 
