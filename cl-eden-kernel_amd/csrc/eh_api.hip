@@ -387,6 +387,11 @@ struct eh_dwconv_plan {
     bool packed_valid = false;
     bool w_signed = false, io_signed = false, has_bias = true;
     int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;  // [cout + 4] once per-channel pairs are set
+    // 3x3 channels-last plans: the 8-bit dot product form of the weights, usable while every w - zp_w fits int8
+    int32_t *w_trip = nullptr, *bias_trip = nullptr;
+    bool range_known = false;   // w_lo / w_hi hold the extremes of the weight bytes (in the caller's own domain)
+    int32_t w_lo = 0, w_hi = 0;
+    bool trip_valid = false;    // w_trip / bias_trip match the current zero points
 };
 
 extern "C" {
@@ -1113,6 +1118,8 @@ static void dw_release(eh_dwconv_plan *pl) {
     dev_free(pl->bias_folded);
     dev_free(pl->pc_multiplier);
     dev_free(pl->pc_shift);
+    dev_free(pl->w_trip);
+    dev_free(pl->bias_trip);
 }
 
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
@@ -1126,6 +1133,8 @@ static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bi
     pl->has_bias = bias != nullptr;
     if (bias) EH_HIP(hipMemcpyAsync(pl->bias_copy, bias, (size_t)pl->cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
     pl->packed_valid = false;
+    pl->range_known = false;  // the plan call looks at the bytes once; weights replaced later keep the 16-bit form
+    pl->trip_valid = false;
     return EH_OK;
 }
 
@@ -1135,6 +1144,13 @@ static int dw_refold(eh_dwconv_plan *pl, const eh_requant &caller_q, hipStream_t
         int rc = launch_dw_pack(pl->w_copy, pl->has_bias ? pl->bias_copy : nullptr, pl->w_pair, pl->bias_folded, pl->cout, pl->taps, q.zp_in,
                                 q.zp_w, pl->w_signed ? 1 : 0, stream);
         if (rc) return rc;
+        pl->trip_valid = false;
+        if (pl->w_trip && pl->range_known && pl->w_lo - q.zp_w >= -128 && pl->w_hi - q.zp_w <= 127) {
+            rc = launch_dw_pack_trip(pl->w_copy, pl->has_bias ? pl->bias_copy : nullptr, pl->w_trip, pl->bias_trip, pl->cout, q.zp_in,
+                                     q.zp_w, pl->w_signed ? 1 : 0, stream);
+            if (rc) return rc;
+            pl->trip_valid = true;
+        }
         pl->packed_valid = true;
     }
     pl->q = q;
@@ -1179,7 +1195,31 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     if (!rc) rc = dev_alloc(&pl->bias_copy, (size_t)pl->cout);
     if (!rc) rc = dev_alloc(&pl->w_pair, (size_t)((pl->taps + 1) / 2) * pl->cout);
     if (!rc) rc = dev_alloc(&pl->bias_folded, (size_t)pl->cout + 4);
+    const bool tile_form = pl->d.layout == EH_NHWC && pl->d.kh == 3 && pl->d.kw == 3 && pl->d.depth_multiplier == 1;
+    if (!rc && tile_form) {
+        rc = dev_alloc(&pl->w_trip, (size_t)3 * pl->cout);
+        if (!rc) rc = dev_alloc(&pl->bias_trip, (size_t)pl->cout + 4);
+    }
     if (!rc) rc = dw_set_weights(pl, weight, bias, s);
+    if (!rc && tile_form && pl->cout > 0) {
+        // the extremes of the weight bytes decide, per zero point, whether the 8-bit dot product form applies
+        std::vector<uint8_t> host((size_t)pl->cout * 9);
+        hipError_t e = hipMemcpyAsync(host.data(), pl->w_copy, host.size(), hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        if (e != hipSuccess) {
+            rc = hip_fail(e, "depthwise: weight download");
+        } else {
+            int lo = 255, hi = -128;
+            for (uint8_t b : host) {
+                const int v = pl->w_signed ? (int)(int8_t)b : (int)b;
+                lo = v < lo ? v : lo;
+                hi = v > hi ? v : hi;
+            }
+            pl->w_lo = lo;
+            pl->w_hi = hi;
+            pl->range_known = true;
+        }
+    }
     if (!rc) rc = dw_refold(pl, *q, s);
     if (rc) {
         dw_release(pl);
@@ -1254,6 +1294,8 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     p.zp_in = plan->q.zp_in;
     p.zp_w = plan->q.zp_w;
     p.w_signed = plan->w_signed ? 1 : 0;
+    p.w_trip = plan->trip_valid ? plan->w_trip : nullptr;
+    p.bias_trip = plan->bias_trip;
     p.io_flip = plan->io_signed ? 0x80808080u : 0u;
     p.rq = make_requant_dev(plan->q);
     if (plan->pc_multiplier) {

@@ -174,6 +174,88 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p
     }
 }
 
+// byte J of three rows' words into bytes 0, 1, 2 of one word (byte 3 zero): the three vertical taps of one channel
+template <int J>
+__device__ __forceinline__ uint32_t column_bytes(uint32_t r0, uint32_t r1, uint32_t r2) {
+    constexpr uint32_t sel01 = (0x0cu << 24) | (0x0cu << 16) | ((4u + J) << 8) | (uint32_t)J;
+    constexpr uint32_t sel2 = (0x0cu << 24) | ((4u + J) << 16) | (1u << 8) | 0u;
+    return __builtin_amdgcn_perm(r2, __builtin_amdgcn_perm(r1, r0, sel01), sel2);
+}
+
+// The same tile with 8-bit dot products, for weights whose differences w - zp_w all fit int8 (per-tensor
+// requantization): activations as a - 128, the three vertical taps of a channel and column gathered into one word
+// once and used by every output that touches the column (v_dot4_i32_i8 against the column's three weights), the
+// term (zp_in - 128) * sum (w - zp_w) folded into the bias.  Six instructions per output for the taps instead of ten.
+template <int S, bool FLIP>
+__global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
+                                                                    const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
+    constexpr int TW = 4, IW = (TW - 1) * S + 3;
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t cq_count = (uint32_t)p.c >> 2;
+    uint32_t r = fastdiv(idx, div_cq);
+    const uint32_t cq = idx - r * cq_count;
+    const uint32_t r2 = fastdiv(r, div_tiles);
+    const int tx = (int)(r - r2 * (uint32_t)tiles_x);
+    const uint32_t img = fastdiv(r2, div_ho);
+    const int oy = (int)(r2 - img * (uint32_t)p.ho);
+    const int ox0 = tx * TW;
+    const int iy0 = oy * S - p.pad_t, ix0 = ox0 * S - p.pad_l;
+    const uint32_t fill = ((uint32_t)p.zp_in * 0x01010101u) ^ 0x80808080u;  // the input zero point minus 128
+    const uint32_t base = img * (uint32_t)(p.h * p.w_ * p.c) + cq * 4u;
+
+    uint32_t col_off[IW];
+    bool col_ok[IW];
+#pragma unroll
+    for (int x = 0; x < IW; ++x) {
+        const int ix = ix0 + x;
+        col_ok[x] = (unsigned)ix < (unsigned)p.w_;
+        const int ixc = ix < 0 ? 0 : (ix >= p.w_ ? p.w_ - 1 : ix);
+        col_off[x] = base + (uint32_t)ixc * (uint32_t)p.c;
+    }
+    uint32_t in[3][IW];
+#pragma unroll
+    for (int ky = 0; ky < 3; ++ky) {
+        const int iy = iy0 + ky;
+        const bool row_ok = (unsigned)iy < (unsigned)p.h;
+        const int iyc = iy < 0 ? 0 : (iy >= p.h ? p.h - 1 : iy);
+        const uint32_t row_off = (uint32_t)iyc * (uint32_t)(p.w_ * p.c);
+#pragma unroll
+        for (int x = 0; x < IW; ++x) {
+            const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in + (row_off + col_off[x]));
+            in[ky][x] = row_ok && col_ok[x] ? (FLIP ? v : v ^ 0x80808080u) : fill;  // int8 tensors hold a - 128 already
+        }
+    }
+    int4 wk[3];
+#pragma unroll
+    for (int kx = 0; kx < 3; ++kx) wk[kx] = *reinterpret_cast<const int4 *>(p.w_trip + ((uint32_t)kx * (uint32_t)p.cout + cq * 4u));
+    const int4 b4 = *reinterpret_cast<const int4 *>(p.bias_trip + cq * 4u);
+    uint32_t col[IW][4];
+#pragma unroll
+    for (int x = 0; x < IW; ++x) {
+        col[x][0] = column_bytes<0>(in[0][x], in[1][x], in[2][x]);
+        col[x][1] = column_bytes<1>(in[0][x], in[1][x], in[2][x]);
+        col[x][2] = column_bytes<2>(in[0][x], in[1][x], in[2][x]);
+        col[x][3] = column_bytes<3>(in[0][x], in[1][x], in[2][x]);
+    }
+    uint8_t *dst = p.out + (((img * (uint32_t)p.ho + (uint32_t)oy) * (uint32_t)p.wo + (uint32_t)ox0) * (uint32_t)p.cout + cq * 4u);
+    const RequantDev rq = p.rq;
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        int acc0 = b4.x, acc1 = b4.y, acc2 = b4.z, acc3 = b4.w;
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+            acc0 = __builtin_amdgcn_sdot4((int)col[j * S + kx][0], wk[kx].x, acc0, false);
+            acc1 = __builtin_amdgcn_sdot4((int)col[j * S + kx][1], wk[kx].y, acc1, false);
+            acc2 = __builtin_amdgcn_sdot4((int)col[j * S + kx][2], wk[kx].z, acc2, false);
+            acc3 = __builtin_amdgcn_sdot4((int)col[j * S + kx][3], wk[kx].w, acc3, false);
+        }
+        uint32_t o = requant4<false>(acc0, acc1, acc2, acc3, rq, cq * 4u);
+        if (FLIP) o ^= 0x80808080u;
+        if (ox0 + j < p.wo) *reinterpret_cast<uint32_t *>(dst + (uint32_t)j * (uint32_t)p.cout) = o;
+    }
+}
+
 // One output element per thread; any depth multiplier, dilation, channel count.
 // NHWC = true: channel fastest.  NHWC = false: planar NCHW, x fastest.
 template <bool NHWC>
@@ -236,6 +318,26 @@ __global__ void dw_pack_kernel(const uint8_t *w, const int32_t *bias, int32_t *w
     bias_folded[oc] = (bias ? bias[oc] : 0) - zp_in * sum;
 }
 
+// 3x3 weights [cout][9] -> w_trip[kx][cout]: the three vertical taps (w - zp_w, each known to fit int8) of column kx
+// in bytes 0..2; bias_trip[c] = bias - (zp_in - 128) * sum (w - zp_w)
+__global__ void dw_pack_trip_kernel(const uint8_t *w, const int32_t *bias, int32_t *w_trip, int32_t *bias_trip, int32_t cout,
+                                    int32_t zp_in, int32_t zp_w, int32_t w_signed) {
+    const int oc = blockIdx.x * blockDim.x + threadIdx.x;
+    if (oc >= cout) return;
+    int32_t sum = 0;
+    for (int kx = 0; kx < 3; ++kx) {
+        uint32_t word = 0;
+        for (int ky = 0; ky < 3; ++ky) {
+            const uint8_t raw = w[(size_t)oc * 9 + ky * 3 + kx];
+            const int32_t v = (w_signed ? (int32_t)(int8_t)raw : (int32_t)raw) - zp_w;
+            sum += v;
+            word |= ((uint32_t)v & 255u) << (8 * ky);
+        }
+        w_trip[(size_t)kx * cout + oc] = (int32_t)word;
+    }
+    bias_trip[oc] = (bias ? bias[oc] : 0) - (zp_in - 128) * sum;
+}
+
 }  // namespace
 
 int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
@@ -243,6 +345,15 @@ int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32
     if (cout <= 0) return EH_OK;
     hipLaunchKernelGGL(dw_pack_kernel, dim3((cout + 127) / 128), dim3(128), 0, stream, w, bias, w_pair, bias_folded, cout,
                        taps, zp_in, zp_w, w_signed);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
+
+int launch_dw_pack_trip(const uint8_t *w, const int32_t *bias, int32_t *w_trip, int32_t *bias_trip, int32_t cout, int32_t zp_in,
+                        int32_t zp_w, int32_t w_signed, hipStream_t stream) {
+    if (cout <= 0) return EH_OK;
+    hipLaunchKernelGGL(dw_pack_trip_kernel, dim3((cout + 127) / 128), dim3(128), 0, stream, w, bias, w_trip, bias_trip, cout, zp_in, zp_w,
+                       w_signed);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }
@@ -269,6 +380,9 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
                       : (flip ? dw3x3_nhwc_tile4_kernel<S, false, true> : dw3x3_nhwc_tile4_kernel<S, false, false>);
         };
         auto kernel = p.stride_h == 1 ? pick(std::integral_constant<int, 1>{}) : pick(std::integral_constant<int, 2>{});
+        if (p.w_trip && !pc)  // every w - zp_w fits int8: the 8-bit dot product form
+            kernel = p.stride_h == 1 ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true> : dw3x3_nhwc_tile4_dot4_kernel<1, false>)
+                                     : (flip ? dw3x3_nhwc_tile4_dot4_kernel<2, true> : dw3x3_nhwc_tile4_dot4_kernel<2, false>);
         hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total, tiles_x, d_cq, d_t, d_ho);
     } else if (vec) {
         const long total = outs / 4;

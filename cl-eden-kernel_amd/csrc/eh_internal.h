@@ -363,6 +363,10 @@ struct DwProblem {
     const int32_t *bias;         // raw bias [cout] or null
     const int32_t *w_pair;       // [ceil(taps/2)][cout]: (w[2p]-zp_w) | (w[2p+1]-zp_w) << 16 as int16 halves
     const int32_t *bias_folded;  // [cout]: bias - zp_in * sum_t (w - zp_w)
+    // 3x3 weights whose differences w - zp_w all fit int8 (else null): [3 columns][cout] words holding a column's
+    // three vertical taps in bytes 0..2, and the bias with (zp_in - 128) * sum_t (w - zp_w) folded in
+    const int32_t *w_trip;
+    const int32_t *bias_trip;
     uint8_t *out;
     int32_t n, c, h, w_, cout, dm;
     int32_t kh, kw, stride_h, stride_w, pad_t, pad_l, dil_h, dil_w;
@@ -374,6 +378,8 @@ struct DwProblem {
 };
 int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
                    int32_t taps, int32_t zp_in, int32_t zp_w, int32_t w_signed, hipStream_t stream);
+int launch_dw_pack_trip(const uint8_t *w, const int32_t *bias, int32_t *w_trip, int32_t *bias_trip, int32_t cout, int32_t zp_in,
+                        int32_t zp_w, int32_t w_signed, hipStream_t stream);
 int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream);
 int launch_dwconv_nchw(const DwProblem &p, hipStream_t stream);
 

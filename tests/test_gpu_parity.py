@@ -359,6 +359,39 @@ def test_depthwise_matches_oracle(case, layout):
     assert want.std() > 10
 
 
+DW_INT8_RANGE_CASES = [c for c in DW_CASES if c["kh"] == 3 and c.get("dm", 1) == 1 and c.get("dil", (1, 1)) == (1, 1)]
+
+
+@pytest.mark.parametrize("case", DW_INT8_RANGE_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_depthwise_3x3_weights_within_int8_of_their_zero_point(case):
+    """Channels-last 3x3 plans whose w - zp_w all fit int8 run the 8-bit dot product kernel; a zero point that
+    pushes one weight out of that range at run time sends the same plan back to the 16-bit form, and back again."""
+    print("dw int8 range", case, flush=True)
+    s = O.conv_shape(**case)
+    zp_w = 140
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 43)
+    w = (12 + synth.fill_u8((s.cout, 1, 3, 3), SEED + 44).astype(np.int32) % 244).astype(np.uint8)   # 12 .. 255
+    w.reshape(-1)[0], w.reshape(-1)[1] = 12, 255                                                       # zp_w - 128 and the top
+    b = synth.fill_i32((s.cout,), SEED + 45, -1000, 1000)
+    quants = []
+    for z in (zp_w, zp_w + 1, zp_w):   # 12 - 141 = -129 does not fit
+        _, acc = O.dwconv2d(x, w, b, s, O.raw_quant(zp_in=37, zp_w=z), want_acc=True)
+        quants.append(centred_quant(acc, 37, z, act_min=5, act_max=250))
+    ho, wo = O.conv_out_hw(s)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, 3, 3, (s.stride_h, s.stride_w), (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (1, 1), 1, 1,
+                          eden.NHWC, eden.W_OIHW)
+    d_x = eden.DeviceBuffer(host=np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+    d_w, d_b, d_o = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b), eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
+    plan = eden.DwConvPlan(desc, d_w, d_b, to_eh_requant(quants[0]))
+    for q in quants:
+        plan.run(d_x, d_o, to_eh_requant(q))
+        got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+        want = O.dwconv2d(x, w, b, s, q)
+        assert np.array_equal(got, want), diff_report(got, want)
+        assert want.std() > 10
+    plan.destroy()
+
+
 @pytest.mark.parametrize("kat", KATS["depthwise"], ids=lambda k: k["name"])
 def test_depthwise_reference_kat_on_gpu(kat):
     n, c, h, w = kat["in_dims"]
