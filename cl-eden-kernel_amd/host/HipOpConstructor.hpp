@@ -148,8 +148,17 @@ public:
                     tensors_used_[t->buffer_index]++;  // init_inter_buffer
                 }
         }
-        for (const auto &op : list.operators) {
+        for (size_t index = 0; index < list.operators.size(); ++index) {
+            const auto &op = list.operators[index];
             EnnReturn rc = ENN_RET_FAILED;
+            if (fuse_residual_adds && index + 1 < list.operators.size() && fusable_add(op, list.operators[index + 1])) {
+                if (create_conv_with_add(op, list.operators[index + 1]) != ENN_RET_SUCCESS) {
+                    ERROR_PRINT("OperationConstructor: building %s with its residual add failed\n", op.name.c_str());
+                    return ENN_RET_FAILED;
+                }
+                ++index;  // the Add went into the convolution's launch
+                continue;
+            }
             switch (op.code) {
                 case TFlite::BuiltinOperator_CONV_2D: rc = create_conv(op); break;
                 case TFlite::BuiltinOperator_DEPTHWISE_CONV_2D: rc = create_depthwise(op); break;
@@ -169,6 +178,11 @@ public:
 
     UDOperators operators;
     UDTensors in_tensors, out_tensors;  // feature maps no operator of the list writes / reads
+    // A uint8 ADD right behind the CONV_2D that produces one of its operands, where nothing else reads that
+    // operand, runs inside the convolution's launch (HipConvolution::fuseResidualAdd); the list then holds one
+    // operator less than the description.  The reference builds one operator per description
+    // (gpu_op_constructor.cc:63-383); set to false for that.
+    bool fuse_residual_adds = true;
 
     // ---- helpers, public because tests pin them against hand-computed cases
 
@@ -366,6 +380,47 @@ private:
         p->per_channel_quant = !op.in_tensors[1]->per_channel_scales.empty();
         p->scales = op.in_tensors[1]->per_channel_scales;
         return finish<HipConvolution>(op, precision, in, out, p);
+    }
+
+    // `add` consumes `conv`'s only output, nothing else does, both are uint8 per-tensor, and the sum is not
+    // written over one of the tensors the fused launch still reads
+    bool fusable_add(const OperatorDesc &conv, const OperatorDesc &add) const {
+        if (conv.code != TFlite::BuiltinOperator_CONV_2D || add.code != TFlite::BuiltinOperator_ADD) return false;
+        if (conv.out_tensors.size() != 1 || conv.in_tensors.size() < 3 || add.in_tensors.size() != 2 || add.out_tensors.size() != 1 ||
+            !conv.option || !add.option)
+            return false;
+        const auto &produced = conv.out_tensors[0];
+        const bool first = add.in_tensors[0]->buffer_index == produced->buffer_index && !add.in_tensors[0]->is_const;
+        const bool second = add.in_tensors[1]->buffer_index == produced->buffer_index && !add.in_tensors[1]->is_const;
+        if (first == second) return false;  // neither, or the convolution added to itself
+        const auto &other = add.in_tensors[first ? 1 : 0];
+        if (other->is_const) return false;
+        const auto readers = tensors_used_.find(produced->buffer_index);
+        if (readers == tensors_used_.end() || readers->second != 1) return false;
+        if (!conv.in_tensors[1]->per_channel_scales.empty()) return false;
+        for (const auto &t : {produced, other, add.out_tensors[0], conv.in_tensors[0]})
+            if (t->data_type != TFlite::TensorType_UINT8) return false;
+        if (produced->shape != other->shape || produced->shape != add.out_tensors[0]->shape) return false;
+        const int32_t sum = add.out_tensors[0]->buffer_index;
+        return sum != other->buffer_index && sum != produced->buffer_index && sum != conv.in_tensors[0]->buffer_index;
+    }
+
+    // The Add's tensors are made first: its output then cannot be given the storage of a feature map the
+    // convolution still reads (the convolution's input may see its last reader here and be handed back to the pool
+    // once the convolution's own tensors are made).
+    EnnReturn create_conv_with_add(const OperatorDesc &conv, const OperatorDesc &add) {
+        const PrecisionType precision = get_precision(add.out_tensors[0]->data_type);
+        UDTensors add_in, add_out;
+        if (!convert_to_tensors(add, precision, add_in, add_out)) return ENN_RET_FAILED;
+        if (create_conv(conv) != ENN_RET_SUCCESS) return ENN_RET_FAILED;
+        auto wrapper = std::dynamic_pointer_cast<EnnUDOperator<HipConvolution>>(operators->back());
+        if (!wrapper) return ENN_RET_FAILED;
+        const bool conv_first = add.in_tensors[0]->buffer_index == conv.out_tensors[0]->buffer_index;
+        const auto *o = options_of<TFlite::AddOptions>(add);
+        return wrapper->getOp()->fuseResidualAdd(add_in[conv_first ? 1 : 0], add_out[0],
+                                                          to_activation(o->fused_activation_function)) == Status::SUCCESS
+                   ? ENN_RET_SUCCESS
+                   : ENN_RET_FAILED;
     }
 
     EnnReturn create_depthwise(const OperatorDesc &op) {

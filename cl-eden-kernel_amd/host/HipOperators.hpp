@@ -279,8 +279,37 @@ public:
             const int rc = eh_conv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute (repack): %s", eh_last_error());
         }
+        if (residual_) {  // output = add(residual, this convolution), as the CLAdd behind it would compute it
+            eh_add_requant aq;
+            eh_make_add_requant(residual_->getScale(), residual_->getZeroPoint(), output_->getScale(), output_->getZeroPoint(),
+                                sum_->getScale(), sum_->getZeroPoint(), detail::toEhActivation(add_activation_),
+                                add_activation_.isEnabled() ? 1 : 0, &aq);
+            const int rc = eh_conv2d_u8_run_add(plan_, input_->getDataPtr(), residual_->getDataPtr(), sum_->getDataPtr(), &q, &aq,
+                                                runtime_->stream());
+            CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute (with residual add): %s", eh_last_error());
+            return Status::SUCCESS;
+        }
         const int rc = eh_conv2d_u8_run(plan_, input_->getDataPtr(), output_->getDataPtr(), &q, runtime_->stream());
         CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    // From now on execute() stores add(residual, convolution) in `sum` and leaves this operator's own output tensor
+    // unwritten: the quantized CLAdd that follows this convolution in an operator list, taken into its launch
+    // (gpu/operators/CLAdd.cpp:159-163; the sum of the two rescaled operands does not depend on their order).  The
+    // output tensor still supplies the scale and zero point the convolution requantizes to.  UINT8, per-tensor.
+    Status fuseResidualAdd(std::shared_ptr<ITensor> residual, std::shared_ptr<ITensor> sum, const ActivationInfo &add_activation) {
+        CHECK_EXPR_RETURN_FAILURE(plan_ != nullptr, "HipConvolution::fuseResidualAdd before initialize");
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8 && !per_channel_, "HipConvolution::fuseResidualAdd: UINT8 per-tensor only");
+        auto r = std::static_pointer_cast<HipTensor>(residual), t = std::static_pointer_cast<HipTensor>(sum);
+        CHECK_EXPR_RETURN_FAILURE(r && t && r->getDataType() == DataType::UINT8 && t->getDataType() == DataType::UINT8,
+                                  "HipConvolution::fuseResidualAdd: expects uint8 tensors");
+        CHECK_EXPR_RETURN_FAILURE(r->getTotalSizeFromDims() == output_->getTotalSizeFromDims() &&
+                                      t->getTotalSizeFromDims() == output_->getTotalSizeFromDims() && r != t,
+                                  "HipConvolution::fuseResidualAdd: shapes differ");
+        residual_ = r;
+        sum_ = t;
+        add_activation_ = add_activation;
         return Status::SUCCESS;
     }
 
@@ -318,6 +347,8 @@ private:
     std::shared_ptr<HipRuntime> runtime_;
     PrecisionType precision_;
     std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
+    std::shared_ptr<HipTensor> residual_, sum_;  // set by fuseResidualAdd
+    ActivationInfo add_activation_;
     std::shared_ptr<ConvolutionParameters> parameters_;
     ActivationInfo activation_info_;
     bool weights_as_input_ = false, bias_as_input_ = false;

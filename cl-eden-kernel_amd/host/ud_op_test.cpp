@@ -1050,18 +1050,29 @@ static int gpu_tests() {
                     {f5, param("wf", {10, 16}, wf.data(), U8T, sw, 128), param("bf", {10}, bf.data(), I32, s5 * sw, 0)}, {f6},
                     std::make_shared<TFlite::FullyConnectedOptions>()),
         };
-        OperationConstructor built(rt);
-        EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
-        EXPECT(built.operators && built.operators->size() == 6);
-        EXPECT(built.in_tensors.size() == 1 && built.out_tensors.size() == 1);
-        OperationExecutor executor(rt);
-        for (int round = 0; round < 2; ++round) {  // a second execution reuses the pooled buffers
-            std::fill(got.begin(), got.end(), 0);
-            EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
-            EXPECT(same(got, want));
+        for (const int variant : {0, 1, 2}) {  // the Add inside the 1x1 convolution's launch (either operand order), or an operator of its own
+            const bool fuse = variant != 2;
+            if (variant == 1) {  // the convolution as the Add's first operand: the oracle adds in that order too
+                list.operators[3] = op_desc("ADD", 4, TFlite::BuiltinOperator_ADD, {f3, f1}, {f4}, std::make_shared<TFlite::AddOptions>());
+                eo_make_add_quant(s3, 128, s1, 0, s4, 100, 0, 0, &aq);
+                std::vector<uint8_t> t4b(t4.size());
+                eo_add_u8(t3.data(), t1.data(), t4b.data(), 16 * 64, &aq);
+                EXPECT(same(t4b, t4));  // the quantized sum does not depend on the operand order
+            }
+            OperationConstructor built(rt);
+            built.fuse_residual_adds = fuse;
+            EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
+            EXPECT(built.operators && built.operators->size() == (fuse ? 5u : 6u));
+            EXPECT(built.in_tensors.size() == 1 && built.out_tensors.size() == 1);
+            OperationExecutor executor(rt);
+            for (int round = 0; round < 2; ++round) {  // a second execution reuses the pooled buffers
+                std::fill(got.begin(), got.end(), 0);
+                EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
+                EXPECT(same(got, want));
+            }
+            for (auto &o : *built.operators) EXPECT(o->release() == ENN_RET_SUCCESS);
         }
         EXPECT(varied(t4));
-        for (auto &o : *built.operators) EXPECT(o->release() == ENN_RET_SUCCESS);
         return ok;
     });
 
