@@ -106,6 +106,24 @@ def test_int8_depthwise_matches_oracle(case, layout):
         assert want.std() > 4
 
 
+@pytest.mark.parametrize("case", DW_CASES[:2], ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_int8_depthwise_weights_within_int8_of_their_zero_point(case):
+    """channels-last 3x3 with every w - zp_w inside int8: the 8-bit dot product kernel on int8 tensors"""
+    print("int8 depthwise, narrow weights", case, flush=True)
+    s = O.conv_shape(**case)
+    x = s8((s.n, s.c, s.h, s.w), SEED + 54)
+    w = (synth.fill_u8((s.c, 1, 3, 3), SEED + 55).astype(np.int16) % 200 - 100).astype(np.int8)
+    w.reshape(-1)[0], w.reshape(-1)[1] = -125, 127    # zp_w - 128 and the top of the range
+    b = synth.fill_i32((s.c,), SEED + 56, -500, 500)
+    ho, wo = O.conv_out_hw(s)
+    for act, enabled in ((eden.ACT_NONE, False), (eden.ACT_RELU6, True)):
+        q, oq = quant_pair(9, act, enabled, zp_out=-128 if enabled else -3)
+        want = O.dwconv2d_s8(x, w, b, s, oq)
+        got = run_conv(eden.DwConvPlan, None, x, w, b, s, q, (s.n, s.c, ho, wo), eden.NHWC, eden.W_OIHW)
+        assert np.array_equal(got, want), int((got != want).sum())
+        assert want.std() > 4
+
+
 DECONV_CASES = [
     dict(n=2, c=64, h=14, w=14, cout=32, kh=2, kw=2, stride=(2, 2)),
     dict(n=1, c=24, h=7, w=9, cout=40, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),
