@@ -186,10 +186,12 @@ __device__ __forceinline__ uint32_t column_bytes(uint32_t r0, uint32_t r1, uint3
 // requantization): activations as a - 128, the three vertical taps of a channel and column gathered into one word
 // once and used by every output that touches the column (v_dot4_i32_i8 against the column's three weights), the
 // term (zp_in - 128) * sum (w - zp_w) folded into the bias.  Six instructions per output for the taps instead of ten.
-template <int S, bool FLIP>
+// TW output pixels per thread: four, or eight for stride 1 on rows that are whole tiles of eight (the column words and
+// the index arithmetic are then shared by twice as many outputs).
+template <int S, bool FLIP, int TW = 4>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                     const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
-    constexpr int TW = 4, IW = (TW - 1) * S + 3;
+    constexpr int IW = (TW - 1) * S + 3;
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
     if (idx >= total) return;
     const uint32_t cq_count = (uint32_t)p.c >> 2;
@@ -383,6 +385,17 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
         if (p.w_trip && !pc)  // every w - zp_w fits int8: the 8-bit dot product form
             kernel = p.stride_h == 1 ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true> : dw3x3_nhwc_tile4_dot4_kernel<1, false>)
                                      : (flip ? dw3x3_nhwc_tile4_dot4_kernel<2, true> : dw3x3_nhwc_tile4_dot4_kernel<2, false>);
+        if (p.w_trip && !pc && p.stride_h == 1 && (p.wo & 7) == 0 && total >= (1l << 20)) {
+            // large stride-1 layers with rows of whole eight-pixel tiles: eight outputs per thread
+            const int tiles8 = p.wo / 8;
+            const long total8 = (long)p.n * p.ho * tiles8 * (p.c >> 2);
+            const FastDiv d_t8 = make_fastdiv((uint32_t)tiles8);
+            auto kernel8 = flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true, 8> : dw3x3_nhwc_tile4_dot4_kernel<1, false, 8>;
+            hipLaunchKernelGGL(kernel8, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, stream, p, (uint32_t)total8, tiles8, d_cq, d_t8,
+                               d_ho);
+            EH_HIP(hipGetLastError());
+            return EH_OK;
+        }
         hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total, tiles_x, d_cq, d_t, d_ho);
     } else if (vec) {
         const long total = outs / 4;

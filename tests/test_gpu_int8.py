@@ -106,7 +106,8 @@ def test_int8_depthwise_matches_oracle(case, layout):
         assert want.std() > 4
 
 
-@pytest.mark.parametrize("case", DW_CASES[:2], ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+@pytest.mark.parametrize("case", DW_CASES[:2] + [dict(n=40, c=64, h=64, w=64, cout=64, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1))],
+                         ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
 def test_int8_depthwise_weights_within_int8_of_their_zero_point(case):
     """channels-last 3x3 with every w - zp_w inside int8: the 8-bit dot product kernel on int8 tensors"""
     print("int8 depthwise, narrow weights", case, flush=True)

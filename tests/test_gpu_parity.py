@@ -359,7 +359,11 @@ def test_depthwise_matches_oracle(case, layout):
     assert want.std() > 10
 
 
-DW_INT8_RANGE_CASES = [c for c in DW_CASES if c["kh"] == 3 and c.get("dm", 1) == 1 and c.get("dil", (1, 1)) == (1, 1)]
+DW_INT8_RANGE_CASES = [c for c in DW_CASES if c["kh"] == 3 and c.get("dm", 1) == 1 and c.get("dil", (1, 1)) == (1, 1)] + [
+    # large stride-1 layers whose rows are whole eight-pixel tiles: eight outputs per thread
+    dict(n=44, c=32, h=112, w=112, cout=32, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=70, c=16, h=37, w=112, cout=16, kh=3, kw=3, pad=(0, 1, 2, 0)),
+]
 
 
 @pytest.mark.parametrize("case", DW_INT8_RANGE_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
