@@ -192,6 +192,10 @@ CONV_CASES = [
     dict(n=1, c=3, h=9, w=10, cout=20, kh=3, kw=3, pad=(1, 1, 1, 1)),
     dict(n=3, c=3, h=5, w=3, cout=16, kh=3, kw=3, pad=(2, 0, 0, 2)),
     dict(n=1, c=3, h=3, w=3, cout=5, kh=3, kw=3),
+    # 32 channels and more: its matrix-core form (two channel blocks with a ragged second one, a single output pixel)
+    dict(n=2, c=3, h=13, w=9, cout=40, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=3, c=3, h=21, w=23, cout=64, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),
+    dict(n=1, c=3, h=3, w=3, cout=72, kh=3, kw=3),
 ]
 
 
