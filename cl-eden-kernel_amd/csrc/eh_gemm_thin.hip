@@ -32,7 +32,7 @@ typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
 // NBU: channel blocks a wave finishes per pass; KU: reduction steps whose loads are in flight together.
 // Grid: x = workgroups along the pixel rows (each wave walks 32-row blocks with stride gridDim.x * 4),
 // y = channel ranges of `nbw` blocks.
-template <int NBU, int KU, bool ROWSUM, bool FAST>
+template <int NBU, int KU, bool ROWSUM, bool FAST, bool RES>
 __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps, const int nbw,
                                                           const int row_blocks) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         if (!ok || n >= p.n) return;
         uint8_t *dst = p.out + out_off + n;
         const int cnt = p.n - n;
-        if (p.residual) {  // out = add(residual, result); the residual tensor is addressed like the output
+        if constexpr (RES) {  // out = add(residual, result); the residual tensor is addressed like the output
             const uint8_t *res = p.residual + out_off + n;
             if (wide && cnt >= 16) {
                 const u32x4_a4 rv = *reinterpret_cast<const u32x4_a4 *>(res);
@@ -271,16 +271,28 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     const dim3 grid(row_wgs, ranges);
     const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t);
     EH_REQUIRE(lds <= 64 * 1024, "igemm_thin: %zu bytes of LDS for the weights", lds);
+    // row sums, the single-shift requantization and the fused residual add are compile-time variants: a launch pays for
+    // none of the code it does not use
+    auto launch = [&](auto rowsum_c, auto fast_c, auto res_c) {
+        hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, decltype(rowsum_c)::value, decltype(fast_c)::value, decltype(res_c)::value>), grid,
+                           dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
+    };
+    auto with_res = [&](auto rowsum_c, auto fast_c) {
+        if (p.residual)
+            launch(rowsum_c, fast_c, std::true_type{});
+        else
+            launch(rowsum_c, fast_c, std::false_type{});
+    };
     if (p.zw != 0) {
         if (p.rq.fast)
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
+            with_res(std::true_type{}, std::true_type{});
         else
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, true, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
+            with_res(std::true_type{}, std::false_type{});
     } else {
         if (p.rq.fast)
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, true>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
+            with_res(std::false_type{}, std::true_type{});
         else
-            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, false, false>), grid, dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
+            with_res(std::false_type{}, std::false_type{});
     }
     EH_HIP(hipGetLastError());
     return EH_OK;
