@@ -45,12 +45,33 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
     extern __shared__ __align__(16) uint8_t lds_raw[];
     v4i *b_s = reinterpret_cast<v4i *>(lds_raw);                                  // [nbw][ksteps][64 lanes]
     int32_t *bias_s = reinterpret_cast<int32_t *>(lds_raw + (size_t)nbw * ksteps * 1024);  // [nbw * 32]
+    // fused residual add: the rescaled value of every possible residual byte and of every possible result byte, so that
+    // an output costs two lookups and one rescaling instead of three rescalings
+    int32_t *add_a_s = bias_s + nbw * 32, *add_b_s = add_a_s + 256;  // [256] each, only with RES
     auto stage_weights = [&]() {
         const v4i *src = reinterpret_cast<const v4i *>(p.b) + (size_t)nb_first * ksteps * 64;
         const int pieces = nb_count * ksteps * 64;
         for (int i = threadIdx.x; i < pieces; i += 256) b_s[i] = src[i];
         for (int i = threadIdx.x; i < nb_count * 32; i += 256) bias_s[i] = p.bias[nb_first * 32 + i];
+        if constexpr (RES) {
+            const int byte = threadIdx.x;  // 256 threads, 256 byte values
+            add_a_s[byte] = mul_round_shift((int32_t)((uint32_t)(byte - p.radd.zp_a) << p.radd.left_shift), p.radd.mult_a, p.radd.rs_a);
+            add_b_s[byte] = mul_round_shift((int32_t)((uint32_t)(byte - p.radd.zp_b) << p.radd.left_shift), p.radd.mult_b, p.radd.rs_b);
+        }
         __syncthreads();
+    };
+    // add_word with the two tables (the same arithmetic: the tables hold what add_one computes first)
+    auto add_word_lut = [&](uint32_t a, uint32_t b) {
+        uint32_t out = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int32_t sum = add_a_s[(a >> (8 * i)) & 255u] + add_b_s[(b >> (8 * i)) & 255u];
+            int32_t v = mul_round_shift(sum, p.radd.mult_out, p.radd.rs_out) + p.radd.zp_out;
+            v = v < p.radd.act_min ? p.radd.act_min : v;
+            v = v > p.radd.act_max ? p.radd.act_max : v;
+            out |= (uint32_t)v << (8 * i);
+        }
+        return out;
     };
 
     const RequantDev rq = p.rq;
@@ -134,10 +155,10 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
             const uint8_t *res = p.residual + out_off + n;
             if (wide && cnt >= 16) {
                 const u32x4_a4 rv = *reinterpret_cast<const u32x4_a4 *>(res);
-                packed[0] = add_word(rv.x, packed[0], p.radd);
-                packed[1] = add_word(rv.y, packed[1], p.radd);
-                packed[2] = add_word(rv.z, packed[2], p.radd);
-                packed[3] = add_word(rv.w, packed[3], p.radd);
+                packed[0] = add_word_lut(rv.x, packed[0]);
+                packed[1] = add_word_lut(rv.y, packed[1]);
+                packed[2] = add_word_lut(rv.z, packed[2]);
+                packed[3] = add_word_lut(rv.w, packed[3]);
             } else {
                 const int c = cnt < 16 ? cnt : 16;
                 for (int t = 0; t < c; ++t) {
@@ -269,7 +290,7 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     const int wg_target = 1024 / ranges > 0 ? 1024 / ranges : 1;  // four workgroups per CU over the whole launch
     if (row_wgs > wg_target) row_wgs = wg_target;
     const dim3 grid(row_wgs, ranges);
-    const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t);
+    const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t) + (p.residual ? 2 * 256 * sizeof(int32_t) : 0);
     EH_REQUIRE(lds <= 64 * 1024, "igemm_thin: %zu bytes of LDS for the weights", lds);
     // row sums, the single-shift requantization and the fused residual add are compile-time variants: a launch pays for
     // none of the code it does not use
