@@ -193,7 +193,13 @@ static int check_perchannel(const int32_t *multipliers, const int32_t *shifts, i
     return EH_OK;
 }
 
-// The per-channel arrays with `pad` zero entries behind them (kernels read whole channel blocks), written by one
+static bool all_pairs_fast(const int32_t *multipliers, const int32_t *shifts, int32_t count, int32_t max_shift = -1) {
+    for (int32_t i = 0; i < count; ++i)
+        if (!channel_pair_is_fast(multipliers[i], shifts[i], max_shift)) return false;
+    return true;
+}
+
+// The per-channel arrays with `pad` entries behind them (kernels read whole channel blocks), written by one
 // blocking copy each from a padded host image, once the stream's earlier work that may still read the arrays is
 // done.
 static int upload_padded_pairs(int32_t *d_mult, int32_t *d_shift, const int32_t *multipliers, const int32_t *shifts,
@@ -203,6 +209,7 @@ static int upload_padded_pairs(int32_t *d_mult, int32_t *d_shift, const int32_t 
     std::copy(multipliers, multipliers + count, image.begin());
     EH_HIP(hipMemcpy(d_mult, image.data(), image.size() * sizeof(int32_t), hipMemcpyHostToDevice));
     std::copy(shifts, shifts + count, image.begin());
+    std::fill(image.begin() + count, image.end(), -2);  // the padding pairs stay inside the single-shift form's range
     EH_HIP(hipMemcpy(d_shift, image.data(), image.size() * sizeof(int32_t), hipMemcpyHostToDevice));
     return EH_OK;
 }
@@ -226,6 +233,7 @@ struct GemmOp {
     bool w_signed = false;
     bool io_signed = false;  // input and output tensors hold int8 values
     int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;
+    bool pc_fast = false;  // every channel's pair is inside the range of the kernels' per-channel single-shift form
 
     int zp_w_u8(const eh_requant &r) const { return r.zp_w + (w_signed ? 128 : 0); }  // zero point of the equivalent uint8 weights
 
@@ -242,6 +250,7 @@ struct GemmOp {
         // padded so that the kernels may read whole channel blocks
         if (!pc_multiplier && (rc = dev_alloc(&pc_multiplier, (size_t)cout + 512))) return rc;
         if (!pc_shift && (rc = dev_alloc(&pc_shift, (size_t)cout + 512))) return rc;
+        pc_fast = all_pairs_fast(multipliers, shifts, cout, -2);  // the table form's rounding term needs rs >= 2
         return upload_padded_pairs(pc_multiplier, pc_shift, multipliers, shifts, cout, 512, stream);
     }
 
@@ -333,7 +342,10 @@ struct GemmOp {
             if (pc_multiplier) {
                 p.rq.pc_multiplier = pc_multiplier + g.bias_base;
                 p.rq.pc_shift = pc_shift + g.bias_base;
-                p.rq.fast = 0;  // the kernels' per-channel code sits on their general path
+                // the one-tap and the direct-to-LDS kernels have the single-shift form per channel; the others'
+                // per-channel code sits on their general path
+                const bool has_form = g.cfg.id != GEMM_STAGED && g.cfg.id != GEMM_C3K3;
+                p.rq.fast = (pc_fast && has_form) ? channel_fast_mode(q) : 0;
             }
             problems.push_back(p);
         }
@@ -387,6 +399,7 @@ struct eh_dwconv_plan {
     bool packed_valid = false;
     bool w_signed = false, io_signed = false, has_bias = true;
     int32_t *pc_multiplier = nullptr, *pc_shift = nullptr;  // [cout + 4] once per-channel pairs are set
+    bool pc_fast = false;  // every pair is inside the single-shift form's range
     // 3x3 channels-last plans: the 8-bit dot product form of the weights, usable while every w - zp_w fits int8
     int32_t *w_trip = nullptr, *bias_trip = nullptr;
     bool range_known = false;   // w_lo / w_hi hold the extremes of the weight bytes (in the caller's own domain)
@@ -1248,6 +1261,7 @@ int eh_dwconv2d_u8_set_perchannel(eh_dwconv_plan *plan, const int32_t *multiplie
     const size_t padded = (size_t)plan->cout + 4;  // the four-channel kernels read whole quads
     if (!plan->pc_multiplier && (rc = dev_alloc(&plan->pc_multiplier, padded))) return rc;
     if (!plan->pc_shift && (rc = dev_alloc(&plan->pc_shift, padded))) return rc;
+    plan->pc_fast = all_pairs_fast(multipliers, shifts, count);
     return upload_padded_pairs(plan->pc_multiplier, plan->pc_shift, multipliers, shifts, count, 4, s);
 }
 
@@ -1301,7 +1315,7 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     if (plan->pc_multiplier) {
         p.rq.pc_multiplier = plan->pc_multiplier;
         p.rq.pc_shift = plan->pc_shift;
-        p.rq.fast = 0;
+        p.rq.fast = plan->pc_fast ? channel_fast_mode(plan->q) : 0;
     }
     return d.layout == EH_NHWC ? launch_dwconv_nhwc(p, s) : launch_dwconv_nchw(p, s);
 }

@@ -31,17 +31,28 @@ __device__ __forceinline__ uint32_t pair_bytes(uint32_t lo, uint32_t hi) {
     return __builtin_amdgcn_perm(hi, lo, sel);
 }
 
-// Four adjacent channels' accumulators to four output bytes.  `ch` is the first channel: with one
-// multiplier and shift per channel (depthwise_conv_per_channel,
-// gpu/operators/cl_kernels/DepthwiseconvolutionKernels.cpp:1323-1371) the four pairs are read from there.
-template <bool PC = true>
-__device__ __forceinline__ uint32_t requant4(int acc0, int acc1, int acc2, int acc3, const RequantDev &rq, uint32_t ch) {
+// The per-channel multipliers and shifts of four adjacent channels, read once per thread.
+struct ChannelQuad {
+    int4 m, s;
+};
+template <bool PC>
+__device__ __forceinline__ ChannelQuad load_channel_quad(const RequantDev &rq, uint32_t ch) {
+    ChannelQuad q{};
     if (PC && rq.pc_multiplier) {
-        const int4 m = *reinterpret_cast<const int4 *>(rq.pc_multiplier + ch);
-        const int4 s = *reinterpret_cast<const int4 *>(rq.pc_shift + ch);
-        return requant_u8_channel(acc0, m.x, s.x, rq) | (requant_u8_channel(acc1, m.y, s.y, rq) << 8) |
-               (requant_u8_channel(acc2, m.z, s.z, rq) << 16) | (requant_u8_channel(acc3, m.w, s.w, rq) << 24);
+        q.m = *reinterpret_cast<const int4 *>(rq.pc_multiplier + ch);
+        q.s = *reinterpret_cast<const int4 *>(rq.pc_shift + ch);
     }
+    return q;
+}
+
+// Four adjacent channels' accumulators to four output bytes.  With one multiplier and shift per channel
+// (depthwise_conv_per_channel, gpu/operators/cl_kernels/DepthwiseconvolutionKernels.cpp:1323-1371) the four pairs
+// come in `cq`.
+template <bool PC = true>
+__device__ __forceinline__ uint32_t requant4(int acc0, int acc1, int acc2, int acc3, const RequantDev &rq, const ChannelQuad &cq) {
+    if (PC && rq.pc_multiplier)  // the two-step order; the single-shift form per channel is the dot product kernel's
+        return requant_u8_channel(acc0, cq.m.x, cq.s.x, rq) | (requant_u8_channel(acc1, cq.m.y, cq.s.y, rq) << 8) |
+               (requant_u8_channel(acc2, cq.m.z, cq.s.z, rq) << 16) | (requant_u8_channel(acc3, cq.m.w, cq.s.w, rq) << 24);
     if (rq.fast == 2)
         return requant_u8_fast_relu(acc0, rq) | (requant_u8_fast_relu(acc1, rq) << 8) | (requant_u8_fast_relu(acc2, rq) << 16) |
                (requant_u8_fast_relu(acc3, rq) << 24);
@@ -49,6 +60,15 @@ __device__ __forceinline__ uint32_t requant4(int acc0, int acc1, int acc2, int a
         return requant_u8_fast(acc0, rq) | (requant_u8_fast(acc1, rq) << 8) | (requant_u8_fast(acc2, rq) << 16) |
                (requant_u8_fast(acc3, rq) << 24);
     return requant_u8(acc0, rq) | (requant_u8(acc1, rq) << 8) | (requant_u8(acc2, rq) << 16) | (requant_u8(acc3, rq) << 24);
+}
+
+// the per-channel single-shift form alone (rq.fast is 1 or 2)
+__device__ __forceinline__ uint32_t requant4_channel_fast(int acc0, int acc1, int acc2, int acc3, const RequantDev &rq, const ChannelQuad &cq) {
+    if (rq.fast == 2)
+        return requant_u8_channel_fast<2>(acc0, cq.m.x, cq.s.x, rq) | (requant_u8_channel_fast<2>(acc1, cq.m.y, cq.s.y, rq) << 8) |
+               (requant_u8_channel_fast<2>(acc2, cq.m.z, cq.s.z, rq) << 16) | (requant_u8_channel_fast<2>(acc3, cq.m.w, cq.s.w, rq) << 24);
+    return requant_u8_channel_fast<1>(acc0, cq.m.x, cq.s.x, rq) | (requant_u8_channel_fast<1>(acc1, cq.m.y, cq.s.y, rq) << 8) |
+           (requant_u8_channel_fast<1>(acc2, cq.m.z, cq.s.z, rq) << 16) | (requant_u8_channel_fast<1>(acc3, cq.m.w, cq.s.w, rq) << 24);
 }
 
 template <int KH, int KW>
@@ -99,7 +119,7 @@ __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, co
         }
     }
     *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) =
-        requant4(acc0, acc1, acc2, acc3, p.rq, (uint32_t)cq * 4u) ^ p.io_flip;
+        requant4(acc0, acc1, acc2, acc3, p.rq, load_channel_quad<true>(p.rq, (uint32_t)cq * 4u)) ^ p.io_flip;
 }
 
 // 3x3, dilation 1, stride S in both directions: a thread owns four adjacent channels of FOUR
@@ -168,7 +188,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p
             acc2 = dot2(pair_bytes<2>(lo, hi), w4[pr].z, acc2);
             acc3 = dot2(pair_bytes<3>(lo, hi), w4[pr].w, acc3);
         }
-        uint32_t o = requant4<PC>(acc0, acc1, acc2, acc3, rq, cq * 4u);
+        uint32_t o = requant4<PC>(acc0, acc1, acc2, acc3, rq, load_channel_quad<PC>(rq, cq * 4u));
         if (FLIP) o ^= 0x80808080u;
         if (ox0 + j < p.wo) *reinterpret_cast<uint32_t *>(dst + (uint32_t)j * (uint32_t)p.cout) = o;
     }
@@ -188,7 +208,8 @@ __device__ __forceinline__ uint32_t column_bytes(uint32_t r0, uint32_t r1, uint3
 // term (zp_in - 128) * sum (w - zp_w) folded into the bias.  Six instructions per output for the taps instead of ten.
 // TW output pixels per thread: four, or eight for stride 1 on rows that are whole tiles of eight (the column words and
 // the index arithmetic are then shared by twice as many outputs).
-template <int S, bool FLIP, int TW = 4>
+// PC: one multiplier and shift per channel, all inside the single-shift form's range (p.rq.fast != 0).
+template <int S, bool FLIP, int TW = 4, bool PC = false>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                     const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
     constexpr int IW = (TW - 1) * S + 3;
@@ -242,6 +263,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
     }
     uint8_t *dst = p.out + (((img * (uint32_t)p.ho + (uint32_t)oy) * (uint32_t)p.wo + (uint32_t)ox0) * (uint32_t)p.cout + cq * 4u);
     const RequantDev rq = p.rq;
+    const ChannelQuad quad = load_channel_quad<PC>(rq, cq * 4u);
 #pragma unroll
     for (int j = 0; j < TW; ++j) {
         int acc0 = b4.x, acc1 = b4.y, acc2 = b4.z, acc3 = b4.w;
@@ -252,7 +274,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
             acc2 = __builtin_amdgcn_sdot4((int)col[j * S + kx][2], wk[kx].z, acc2, false);
             acc3 = __builtin_amdgcn_sdot4((int)col[j * S + kx][3], wk[kx].w, acc3, false);
         }
-        uint32_t o = requant4<false>(acc0, acc1, acc2, acc3, rq, cq * 4u);
+        uint32_t o = PC ? requant4_channel_fast(acc0, acc1, acc2, acc3, rq, quad) : requant4<false>(acc0, acc1, acc2, acc3, rq, quad);
         if (FLIP) o ^= 0x80808080u;
         if (ox0 + j < p.wo) *reinterpret_cast<uint32_t *>(dst + (uint32_t)j * (uint32_t)p.cout) = o;
     }
@@ -382,15 +404,21 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
                       : (flip ? dw3x3_nhwc_tile4_kernel<S, false, true> : dw3x3_nhwc_tile4_kernel<S, false, false>);
         };
         auto kernel = p.stride_h == 1 ? pick(std::integral_constant<int, 1>{}) : pick(std::integral_constant<int, 2>{});
-        if (p.w_trip && !pc)  // every w - zp_w fits int8: the 8-bit dot product form
-            kernel = p.stride_h == 1 ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true> : dw3x3_nhwc_tile4_dot4_kernel<1, false>)
-                                     : (flip ? dw3x3_nhwc_tile4_dot4_kernel<2, true> : dw3x3_nhwc_tile4_dot4_kernel<2, false>);
-        if (p.w_trip && !pc && p.stride_h == 1 && (p.wo & 7) == 0 && total >= (1l << 20)) {
+        auto pick_dot4 = [&](auto s_tag, auto tw_tag) {
+            constexpr int S = decltype(s_tag)::value, TW = decltype(tw_tag)::value;
+            return pc ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, true> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, true>)
+                      : (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, false> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, false>);
+        };
+        using tw4 = std::integral_constant<int, 4>;
+        const bool dot4 = p.w_trip && (!pc || p.rq.fast);
+        if (dot4)  // every w - zp_w fits int8: the 8-bit dot product form
+            kernel = p.stride_h == 1 ? pick_dot4(std::integral_constant<int, 1>{}, tw4{}) : pick_dot4(std::integral_constant<int, 2>{}, tw4{});
+        if (dot4 && p.stride_h == 1 && (p.wo & 7) == 0 && total >= (1l << 20)) {
             // large stride-1 layers with rows of whole eight-pixel tiles: eight outputs per thread
             const int tiles8 = p.wo / 8;
             const long total8 = (long)p.n * p.ho * tiles8 * (p.c >> 2);
             const FastDiv d_t8 = make_fastdiv((uint32_t)tiles8);
-            auto kernel8 = flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true, 8> : dw3x3_nhwc_tile4_dot4_kernel<1, false, 8>;
+            auto kernel8 = pick_dot4(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{});
             hipLaunchKernelGGL(kernel8, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, stream, p, (uint32_t)total8, tiles8, d_cq, d_t8,
                                d_ho);
             EH_HIP(hipGetLastError());

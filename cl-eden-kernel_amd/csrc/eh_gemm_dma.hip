@@ -429,7 +429,12 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
                         uint32_t o0, o1, o2, o3;
-                        if constexpr (pc) {
+                        if constexpr (pc && fast != 0) {  // every channel's pair inside the single-shift form's range
+                            o0 = requant_u8_channel_fast<fast>(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], cm[g].x, cs[g].x, rq);
+                            o1 = requant_u8_channel_fast<fast>(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], cm[g].y, cs[g].y, rq);
+                            o2 = requant_u8_channel_fast<fast>(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], cm[g].z, cs[g].z, rq);
+                            o3 = requant_u8_channel_fast<fast>(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], cm[g].w, cs[g].w, rq);
+                        } else if constexpr (pc) {
                             o0 = requant_u8_channel(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], cm[g].x, cs[g].x, rq);
                             o1 = requant_u8_channel(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], cm[g].y, cs[g].y, rq);
                             o2 = requant_u8_channel(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], cm[g].z, cs[g].z, rq);
@@ -461,7 +466,14 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
         };
         // edge tiles and unusual requantization parameters take the general code
         if (rq.pc_multiplier) {
-            emit(std::true_type{}, std::integral_constant<int, 0>{}, std::true_type{});
+            // (the 256 x 256 tile has no registers to spare for the per-channel terms: two-step order there)
+            constexpr bool pc_single_shift = !(BM == 256 && BN == 256);
+            if (pc_single_shift && rq.fast == 2)
+                emit(std::true_type{}, std::integral_constant<int, pc_single_shift ? 2 : 0>{}, std::true_type{});
+            else if (pc_single_shift && rq.fast == 1)
+                emit(std::true_type{}, std::integral_constant<int, pc_single_shift ? 1 : 0>{}, std::true_type{});
+            else
+                emit(std::true_type{}, std::integral_constant<int, 0>{}, std::true_type{});
         } else if (rq.fast && aligned16 && m0 + BM <= p.m && n0 + BN <= p.n) {
             if (rq.fast == 2)
                 emit(std::false_type{}, std::integral_constant<int, 2>{}, std::false_type{});
@@ -515,15 +527,22 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
             }
             const int4 bb = *reinterpret_cast<const int4 *>(bias_s + nl + g * 4);
             uint32_t o0, o1, o2, o3;
-            if (fast == 0 && rq.pc_multiplier) {
+            if (rq.pc_multiplier) {
                 const int32_t *pm = rq.pc_multiplier + n + g * 4;
-                            const int4 cm = make_int4(pm[0], pm[1], pm[2], pm[3]);
+                const int4 cm = make_int4(pm[0], pm[1], pm[2], pm[3]);
                 const int32_t *ps = rq.pc_shift + n + g * 4;
-                            const int4 cs = make_int4(ps[0], ps[1], ps[2], ps[3]);
-                o0 = requant_u8_channel(s4.x + bb.x - corr, cm.x, cs.x, rq);
-                o1 = requant_u8_channel(s4.y + bb.y - corr, cm.y, cs.y, rq);
-                o2 = requant_u8_channel(s4.z + bb.z - corr, cm.z, cs.z, rq);
-                o3 = requant_u8_channel(s4.w + bb.w - corr, cm.w, cs.w, rq);
+                const int4 cs = make_int4(ps[0], ps[1], ps[2], ps[3]);
+                if constexpr (fast != 0) {
+                    o0 = requant_u8_channel_fast<fast>(s4.x + bb.x - corr, cm.x, cs.x, rq);
+                    o1 = requant_u8_channel_fast<fast>(s4.y + bb.y - corr, cm.y, cs.y, rq);
+                    o2 = requant_u8_channel_fast<fast>(s4.z + bb.z - corr, cm.z, cs.z, rq);
+                    o3 = requant_u8_channel_fast<fast>(s4.w + bb.w - corr, cm.w, cs.w, rq);
+                } else {
+                    o0 = requant_u8_channel(s4.x + bb.x - corr, cm.x, cs.x, rq);
+                    o1 = requant_u8_channel(s4.y + bb.y - corr, cm.y, cs.y, rq);
+                    o2 = requant_u8_channel(s4.z + bb.z - corr, cm.z, cs.z, rq);
+                    o3 = requant_u8_channel(s4.w + bb.w - corr, cm.w, cs.w, rq);
+                }
             } else {
                 o0 = requant_u8_as<fast>(s4.x + bb.x - corr, rq), o1 = requant_u8_as<fast>(s4.y + bb.y - corr, rq);
                 o2 = requant_u8_as<fast>(s4.z + bb.z - corr, rq), o3 = requant_u8_as<fast>(s4.w + bb.w - corr, rq);

@@ -32,7 +32,10 @@ typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
 // NBU: channel blocks a wave finishes per pass; KU: reduction steps whose loads are in flight together.
 // Grid: x = workgroups along the pixel rows (each wave walks 32-row blocks with stride gridDim.x * 4),
 // y = channel ranges of `nbw` blocks.
-template <int NBU, int KU, bool ROWSUM, bool FAST, bool RES>
+// QM: how results are requantized.  0: the two-step order (one pair, or one per channel read from global memory);
+// 1: the single-shift form with the requant's one pair; 2: the single-shift form with one pair per channel, whose
+// multiplier, shift and rounding term sit in LDS beside the bias.
+template <int NBU, int KU, bool ROWSUM, int QM, bool RES>
 __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps, const int nbw,
                                                           const int row_blocks) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -47,12 +50,23 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
     int32_t *bias_s = reinterpret_cast<int32_t *>(lds_raw + (size_t)nbw * ksteps * 1024);  // [nbw * 32]
     // fused residual add: the rescaled value of every possible residual byte and of every possible result byte, so that
     // an output costs two lookups and one rescaling instead of three rescalings
-    int32_t *add_a_s = bias_s + nbw * 32, *add_b_s = add_a_s + 256;  // [256] each, only with RES
+    // per-channel single-shift tables, only with QM == 2: multiplier, right shift - 1, high word of the rounding term
+    int32_t *pcm_s = bias_s + nbw * 32, *pcf_s = pcm_s + nbw * 32, *pch_s = pcf_s + nbw * 32;
+    int32_t *add_a_s = bias_s + (QM == 2 ? 4 : 1) * nbw * 32, *add_b_s = add_a_s + 256;  // [256] each, only with RES
     auto stage_weights = [&]() {
         const v4i *src = reinterpret_cast<const v4i *>(p.b) + (size_t)nb_first * ksteps * 64;
         const int pieces = nb_count * ksteps * 64;
         for (int i = threadIdx.x; i < pieces; i += 256) b_s[i] = src[i];
         for (int i = threadIdx.x; i < nb_count * 32; i += 256) bias_s[i] = p.bias[nb_first * 32 + i];
+        if constexpr (QM == 2) {
+            // rounding term 2^30 + (1 + 2 zp_out) 2^(30 + rs) for rs >= 2: low word 2^30, high word (1 + 2 zp_out) 2^(rs - 2)
+            for (int i = threadIdx.x; i < nb_count * 32; i += 256) {
+                const int32_t rs = -p.rq.pc_shift[nb_first * 32 + i];
+                pcm_s[i] = p.rq.pc_multiplier[nb_first * 32 + i];
+                pcf_s[i] = rs - 1;
+                pch_s[i] = (int32_t)((uint32_t)(1 + 2 * p.rq.zp_out) << (rs - 2));
+            }
+        }
         if constexpr (RES) {
             const int byte = threadIdx.x;  // 256 threads, 256 byte values
             add_a_s[byte] = mul_round_shift((int32_t)((uint32_t)(byte - p.radd.zp_a) << p.radd.left_shift), p.radd.mult_a, p.radd.rs_a);
@@ -126,7 +140,16 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
             for (int g = 0; g < 4; ++g) {
                 const int4 bb = *reinterpret_cast<const int4 *>(bsrc + g * 4);
                 uint32_t o0, o1, o2, o3;
-                if (mode == 0 && rq.pc_multiplier) {  // per-channel parameters (the padded arrays cover whole blocks)
+                if constexpr (QM == 2) {
+                    const int tab = nb_local * 32 + half * 16 + g * 4;
+                    const int4 cm = *reinterpret_cast<const int4 *>(pcm_s + tab);
+                    const int4 cf = *reinterpret_cast<const int4 *>(pcf_s + tab);
+                    const int4 ch = *reinterpret_cast<const int4 *>(pch_s + tab);
+                    o0 = requant_u8_channel_table<mode>(acc[g * 4 + 0] + bb.x + ncorr, cm.x, cf.x, ch.x, rq);
+                    o1 = requant_u8_channel_table<mode>(acc[g * 4 + 1] + bb.y + ncorr, cm.y, cf.y, ch.y, rq);
+                    o2 = requant_u8_channel_table<mode>(acc[g * 4 + 2] + bb.z + ncorr, cm.z, cf.z, ch.z, rq);
+                    o3 = requant_u8_channel_table<mode>(acc[g * 4 + 3] + bb.w + ncorr, cm.w, cf.w, ch.w, rq);
+                } else if (mode == 0 && rq.pc_multiplier) {  // per-channel parameters (the padded arrays cover whole blocks)
                     const int4 cm = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + g * 4);
                     const int4 cs = *reinterpret_cast<const int4 *>(rq.pc_shift + n + g * 4);
                     o0 = requant_u8_channel(acc[g * 4 + 0] + bb.x + ncorr, cm.x, cs.x, rq);
@@ -142,7 +165,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                 packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
             }
         };
-        if constexpr (!FAST)
+        if constexpr (QM == 0)
             quantize(std::integral_constant<int, 0>{});
         else if (rq.fast == 2)
             quantize(std::integral_constant<int, 2>{});
@@ -290,31 +313,34 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     const int wg_target = 1024 / ranges > 0 ? 1024 / ranges : 1;  // four workgroups per CU over the whole launch
     if (row_wgs > wg_target) row_wgs = wg_target;
     const dim3 grid(row_wgs, ranges);
-    const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t) + (p.residual ? 2 * 256 * sizeof(int32_t) : 0);
+    const bool pc_fast = p.rq.fast && p.rq.pc_multiplier;
+    const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t) * (pc_fast ? 4 : 1) +
+                       (p.residual ? 2 * 256 * sizeof(int32_t) : 0);
     EH_REQUIRE(lds <= 64 * 1024, "igemm_thin: %zu bytes of LDS for the weights", lds);
     // row sums, the single-shift requantization and the fused residual add are compile-time variants: a launch pays for
     // none of the code it does not use
-    auto launch = [&](auto rowsum_c, auto fast_c, auto res_c) {
-        hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, decltype(rowsum_c)::value, decltype(fast_c)::value, decltype(res_c)::value>), grid,
+    auto launch = [&](auto rowsum_c, auto qm_c, auto res_c) {
+        hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(res_c)::value>), grid,
                            dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
     };
-    auto with_res = [&](auto rowsum_c, auto fast_c) {
+    auto with_res = [&](auto rowsum_c, auto qm_c) {
         if (p.residual)
-            launch(rowsum_c, fast_c, std::true_type{});
+            launch(rowsum_c, qm_c, std::true_type{});
         else
-            launch(rowsum_c, fast_c, std::false_type{});
+            launch(rowsum_c, qm_c, std::false_type{});
     };
-    if (p.zw != 0) {
-        if (p.rq.fast)
-            with_res(std::true_type{}, std::true_type{});
+    auto with_qm = [&](auto rowsum_c) {
+        if (pc_fast)
+            with_res(rowsum_c, std::integral_constant<int, 2>{});
+        else if (p.rq.fast)
+            with_res(rowsum_c, std::integral_constant<int, 1>{});
         else
-            with_res(std::true_type{}, std::false_type{});
-    } else {
-        if (p.rq.fast)
-            with_res(std::false_type{}, std::true_type{});
-        else
-            with_res(std::false_type{}, std::false_type{});
-    }
+            with_res(rowsum_c, std::integral_constant<int, 0>{});
+    };
+    if (p.zw != 0)
+        with_qm(std::true_type{});
+    else
+        with_qm(std::false_type{});
     EH_HIP(hipGetLastError());
     return EH_OK;
 }

@@ -127,6 +127,51 @@ __host__ __device__ __forceinline__ uint32_t requant_u8_fast_relu(int32_t x, con
 #endif
 }
 
+// The single-shift form with a channel's own multiplier and shift (-20 <= shift <= -1; the host sets `fast` on a
+// per-channel problem only when every channel is in that range).  The rounding term 2^30 + (1 + 2 zp) 2^(30 + rs)
+// depends on the channel alone, so a thread that keeps its channels across many outputs computes it once.
+// MODE 2 skips the sign test as requant_u8_fast_relu does.
+template <int MODE>
+__host__ __device__ __forceinline__ uint32_t requant_u8_channel_fast(int32_t x, int32_t multiplier, int32_t shift, const RequantDev &r) {
+    const int32_t rs = -shift;
+    const int64_t pos = (1ll << 30) + (int64_t)(1 + 2 * r.zp_out) * (1ll << (30 + rs));
+    const int64_t term = (MODE != 2 && x < 0) ? pos - (1ll << 31) : pos;
+    const int64_t t = (int64_t)x * (int64_t)multiplier + term;
+    int32_t v = (int32_t)(t >> 32) >> (rs - 1);
+    v = v < r.act_min ? r.act_min : v;
+    v = v > r.act_max ? r.act_max : v;
+    return (uint32_t)v;
+}
+
+// The same with the channel's terms from a table: `fs` = rs - 1 and `pos_hi` = (1 + 2 zp) 2^(rs - 2), the high word
+// of the rounding term, whose low word is 2^30 for every rs >= 2.  For a negative accumulator the term is 2^31
+// less: the low word gains bit 31 and the high word lends one.
+template <int MODE>
+__host__ __device__ __forceinline__ uint32_t requant_u8_channel_table(int32_t x, int32_t multiplier, int32_t fs, int32_t pos_hi,
+                                                                      const RequantDev &r) {
+    uint32_t lo = 0x40000000u;
+    int32_t hi = pos_hi;
+    if (MODE != 2) {
+        lo |= (uint32_t)x & 0x80000000u;
+        hi += x >> 31;
+    }
+    const int64_t t = (int64_t)x * (int64_t)multiplier + (int64_t)(((uint64_t)(uint32_t)hi << 32) | lo);
+    int32_t v = (int32_t)(t >> 32) >> fs;
+    v = v < r.act_min ? r.act_min : v;
+    v = v > r.act_max ? r.act_max : v;
+    return (uint32_t)v;
+}
+
+// whether the single-shift form covers a channel's pair
+inline bool channel_pair_is_fast(int32_t multiplier, int32_t shift, int32_t max_shift = -1) {
+    return multiplier >= 0 && shift <= max_shift && shift >= -20;
+}
+// `fast` of a per-channel problem whose pairs all pass channel_pair_is_fast
+inline int32_t channel_fast_mode(const eh_requant &q) {
+    if (q.zp_out < -1024 || q.zp_out > 1024) return 0;
+    return q.act_min >= q.zp_out ? 2 : 1;
+}
+
 // MODE 0: two-step reference order; 1: single shift; 2: single shift without the sign test
 template <int MODE>
 __host__ __device__ __forceinline__ uint32_t requant_u8_as(int32_t acc, const RequantDev &r) {

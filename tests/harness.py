@@ -14,6 +14,13 @@ def to_eh_requant(q):
     return eden.Requant(*q.as_tuple())
 
 
+def to_eh_add(q):
+    r = eden.AddRequant()
+    for f, _ in eden.AddRequant._fields_:
+        setattr(r, f, getattr(q, f))
+    return r
+
+
 def assert_same_host_quant(args, kwargs):
     """The product's own parameter derivation must agree with the oracle's."""
     a = eden.make_requant(*args, **kwargs).as_tuple()

@@ -3,18 +3,11 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from harness import eden, synth, to_eh_requant
+from harness import eden, synth, to_eh_add, to_eh_requant
 
 pytestmark = pytest.mark.gpu
 
 SEED = 0xEDE2 + 16 * 7
-
-
-def to_eh_add(q):
-    r = eden.AddRequant()
-    for f, _ in eden.AddRequant._fields_:
-        setattr(r, f, getattr(q, f))
-    return r
 
 
 def gpu_add(a, b, q, offset=0):

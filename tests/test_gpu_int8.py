@@ -125,6 +125,36 @@ def test_int8_depthwise_weights_within_int8_of_their_zero_point(case):
         assert want.std() > 4
 
 
+DW_PC_S8_CASES = [
+    dict(n=2, c=32, h=15, w=14, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),     # four outputs per thread, stride 1
+    dict(n=2, c=24, h=15, w=17, cout=24, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),     # four outputs per thread, stride 2
+    dict(n=44, c=32, h=112, w=112, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),  # eight outputs per thread
+]
+
+
+@pytest.mark.parametrize("case", DW_PC_S8_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_int8_perchannel_depthwise_dot_product_form(case):
+    """The full-integer depthwise layer of a TFLite model: int8 tensors, int8 weights at zero point 0 and one
+    multiplier / shift per channel.  Every weight fits int8 about its zero point by construction, so channels-last
+    3x3 plans run the 8-bit dot product kernel's per-channel variant."""
+    print("int8 per-channel depthwise", case, flush=True)
+    s = O.conv_shape(**case)
+    x, w = s8((s.n, s.c, s.h, s.w), SEED + 91), s8((s.c, 1, 3, 3), SEED + 92)
+    w.reshape(-1)[0], w.reshape(-1)[1] = -128, 127
+    b = synth.fill_i32((s.c,), SEED + 93, -500, 500)
+    w_scales = (0.002 * (1.0 + 29.0 * synth.fill_u8((s.c,), SEED + 94) / 255.0)).astype(np.float32)
+    s_out = float(0.02 * float(w_scales.max()) * 74.0 * 74.0 * 3.0 / 60.0)
+    q, mults, shifts = eden.make_requant_perchannel(0.02, -20, w_scales, s_out, 5)
+    q.act_min, q.act_max = -128, 127
+    assert q.zp_w == 0 and len(set(mults.tolist())) > 4
+    oq = O.raw_quant(zp_in=-20, zp_w=0, zp_out=5, act_min=-128, act_max=127)
+    want = O.dwconv2d_s8(x, w, b, s, oq, mults, shifts)
+    ho, wo = O.conv_out_hw(s)
+    got = run_conv(eden.DwConvPlan, None, x, w, b, s, q, (s.n, s.c, ho, wo), eden.NHWC, eden.W_OIHW, (mults, shifts))
+    assert np.array_equal(got, want), int((got != want).sum())
+    assert want.std() > 4
+
+
 DECONV_CASES = [
     dict(n=2, c=64, h=14, w=14, cout=32, kh=2, kw=2, stride=(2, 2)),
     dict(n=1, c=24, h=7, w=9, cout=40, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from harness import eden, synth, to_eh_requant
+from harness import eden, synth, to_eh_add, to_eh_requant
 
 pytestmark = pytest.mark.gpu
 
@@ -82,12 +82,74 @@ def test_perchannel_conv_matches_oracle(case, layout):
     got, uniform = gpu_conv_perchannel(x, w, b, s, q, mults, shifts, layout)
     assert np.array_equal(got, want), int((got != want).sum())
     assert want.std() > 4
+    # a clamp floor at the output zero point (fused ReLU): the kernels' single-shift form drops its sign test
+    q.act_min = 131
+    oq_relu = O.raw_quant(zp_in=117, zp_w=0, zp_out=131, act_min=131)
+    got, _ = gpu_conv_perchannel(x, w, b, s, q, mults, shifts, layout)
+    assert np.array_equal(got, O.conv2d_perchannel(x, w, b, s, oq_relu, mults, shifts))
     # per-tensor mode on the same plan: int8 weights with the requant's own pair
     q2 = eden.Requant(117, 0, 131, int(mults[0]), int(shifts[0]), 0, 255)
     oq2 = O.raw_quant(zp_in=117, zp_w=0, zp_out=131, multiplier=int(mults[0]), shift=int(shifts[0]))
     want2 = O.conv2d_perchannel(x, w, b, s, oq2, np.full(s.cout, mults[0], np.int32), np.full(s.cout, shifts[0], np.int32))
     _, uniform = gpu_conv_perchannel(x, w, b, s, q2, mults, shifts, layout)
     assert np.array_equal(uniform, want2)
+
+
+ONE_TAP_PC_CASES = [
+    dict(n=3, c=16, h=20, w=21, cout=96, kh=1, kw=1),    # one reduction step, three channel blocks
+    dict(n=2, c=64, h=15, w=15, cout=24, kh=1, kw=1),    # two steps, a ragged channel block
+    dict(n=2, c=96, h=14, w=14, cout=40, kh=1, kw=1),    # reduction walked in groups of steps
+    dict(n=1, c=144, h=9, w=9, cout=200, kh=1, kw=1),    # several channel ranges
+]
+
+
+@pytest.mark.parametrize("case", ONE_TAP_PC_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_perchannel_one_tap_kernel_single_shift_forms(case):
+    """Channels-last 1x1 layers with every channel's shift in -20 .. -2 requantize from the per-channel tables in LDS:
+    with and without the sign test (fused ReLU or not), with and without the row-sum term (zp_w != 0 or 0), with the
+    fused residual add, and back on the two-step order when one channel's shift leaves the range."""
+    print("per-channel one-tap", case, flush=True)
+    s = O.conv_shape(**case)
+    ho, wo = O.conv_out_hw(s)
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 71)
+    w = (synth.fill_u8((s.cout, s.c, 1, 1), SEED + 72).astype(np.int16) - 128).astype(np.int8)
+    b = synth.fill_i32((s.cout,), SEED + 73, -5000, 5000)
+    res = synth.fill_u8((s.n, s.cout, ho, wo), SEED + 74)
+    w_scales = (0.002 * (1.0 + 29.0 * synth.fill_u8((s.cout,), SEED + 75) / 255.0)).astype(np.float32)
+    s_out = float(0.02 * float(w_scales.max()) * 74.0 * 74.0 * np.sqrt(s.c) / 60.0)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), 1, 1, eden.NHWC, eden.W_OIHW | eden.W_SIGNED)
+    d_x, d_w, d_b = eden.DeviceBuffer(host=x.transpose(0, 2, 3, 1)), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+    d_r = eden.DeviceBuffer(host=np.ascontiguousarray(res.transpose(0, 2, 3, 1)))
+    d_o = eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
+    aq = O.make_add_quant(0.031, 120, s_out, 131, 0.05, 125, O.ACT_NONE, False)
+    plan = None
+    for zp_w in (0, -7):
+        for act_min, zp_out in ((0, 131), (131, 131), (3, 0)):     # sign test needed / ReLU at the zero point / ReLU6-like floor
+            q, mults, shifts = eden.make_requant_perchannel(0.02, 117, w_scales, s_out, zp_out, eden.ACT_NONE, False)
+            q.zp_w, q.act_min = zp_w, act_min
+            assert shifts.max() <= -2 and shifts.min() >= -20
+            oq = O.raw_quant(zp_in=117, zp_w=zp_w, zp_out=zp_out, act_min=act_min)
+            want = O.conv2d_perchannel(x, w, b, s, oq, mults, shifts)
+            if plan is None:
+                plan = eden.ConvPlan(desc, d_w, d_b, q)
+            plan.set_perchannel(mults, shifts)
+            plan.run(d_x, d_o, q)
+            got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+            assert np.array_equal(got, want), (zp_w, act_min, int((got != want).sum()))
+            if zp_out == 131:
+                plan.run_add(d_x, d_r, d_o, q, to_eh_add(aq))
+                got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+                assert np.array_equal(got, O.add(res, want, aq))
+    assert want.std() > 4
+    # shifts the tables do not cover: -1 (the rounding term's low word differs) and 0
+    for odd in (-1, 0):
+        odd_shifts = shifts.copy()
+        odd_shifts[s.cout // 2] = odd
+        plan.set_perchannel(mults, odd_shifts)
+        plan.run(d_x, d_o, q)
+        got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, O.conv2d_perchannel(x, w, b, s, oq, mults, odd_shifts))
+    plan.destroy()
 
 
 def _pairs_for(s_in, w_scales, s_out):
@@ -101,6 +163,7 @@ DW_PC_CASES = [
     dict(n=1, c=16, h=12, w=12, cout=16, kh=5, kw=5, stride=(1, 1), pad=(2, 2, 2, 2)),              # four-channel kernel
     dict(n=1, c=16, h=12, w=12, cout=16, kh=3, kw=3, stride=(1, 1), pad=(2, 2, 2, 2), dil=(2, 2)),  # four-channel kernel, 3x3 dilated
     dict(n=2, c=5, h=9, w=8, cout=10, kh=3, kw=3, stride=(2, 1), pad=(1, 0, 1, 1), dm=2),           # one output per thread
+    dict(n=44, c=32, h=112, w=112, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),           # 3x3 tile kernel, eight outputs per thread
 ]
 
 
@@ -133,6 +196,13 @@ def test_perchannel_depthwise_matches_oracle(case, layout):
         got = d_o.download((s.n, cout, ho, wo)) if layout == eden.NCHW else d_o.download((s.n, ho, wo, cout)).transpose(0, 3, 1, 2)
         assert np.array_equal(got, want), int((got != want).sum())
         assert want.std() > 4
+        # two pairs outside the range of the kernels' single-shift form: the whole plan takes the two-step order
+        odd_shifts = shifts.copy()
+        odd_shifts[0], odd_shifts[1] = 0, -21
+        plan.set_perchannel(mults, odd_shifts)
+        plan.run(d_x, d_o, q)
+        got = d_o.download((s.n, cout, ho, wo)) if layout == eden.NCHW else d_o.download((s.n, ho, wo, cout)).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, O.dwconv2d_perchannel(x, w, b, s, oq, mults, odd_shifts))
         # back to one pair: int8 weights, per-tensor requant
         plan.set_perchannel(None, None)
         q1 = eden.Requant(117, zp_w, 131, int(mults[1]), int(shifts[1]), 0, 255)
