@@ -148,12 +148,14 @@ def deconv_workload(eden, synth, n=8):
                 bytes=n * 256 * 1024 + 256 * 128 * 16 + 512 + n * 128 * 4096, bound="mfma")
 
 
-def mbv2_workload(eden, synth, batch=64):
-    """BASELINE.json configs[4]: MobileNetV2-1.0 uint8 at 224x224x3, batch 64, the whole operator list per step."""
+def mbv2_workload(eden, synth, batch=64, per_channel=False):
+    """BASELINE.json configs[4]: MobileNetV2-1.0 uint8 at 224x224x3, batch 64, the whole operator list per step.
+    per_channel: int8 weights with one scale per output channel in the convolutions."""
     mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
-    net = mobilenet.MobileNetV2(eden, batch, fuse_add=True)  # residual adds inside the projection convolutions' launches
+    # residual adds inside the projection convolutions' launches
+    net = mobilenet.MobileNetV2(eden, batch, fuse_add=True, per_channel=per_channel)
     net.set_input(mobilenet.network_input(batch))
-    return dict(name="mobilenet_v2_1.0_224_u8_batch%d" % batch, launch=lambda s: net.run(s), keep=net,
+    return dict(name="mobilenet_v2_1.0_224_u8%s_batch%d" % ("_perchannel_w" if per_channel else "", batch), launch=lambda s: net.run(s), keep=net,
                 ops=2.0 * mobilenet.macs_per_image() * batch, bytes=mobilenet.compulsory_bytes_per_image() * batch,
                 bound="hbm", images=batch, chunk=4)
 
@@ -207,7 +209,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv, mbv2, copy")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv, mbv2, mbv2pc, copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (got --gpus %d); no multi-GPU figure exists" % args.gpus,
@@ -223,7 +225,8 @@ def main():
 
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
                     fcbig=lambda e, s: fc_workload(e, s, 8192, 4096, 4096), conv64=lambda e, s: conv_workload(e, s, 64),
-                    copy=copy_workload, mbv2=mbv2_workload)
+                    copy=copy_workload, mbv2=mbv2_workload,
+                    mbv2pc=lambda e, s: mbv2_workload(e, s, per_channel=True))
     if args.only:
         work = families[args.only](eden, synth)
         wall, ev = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph, work.get("chunk", 50))

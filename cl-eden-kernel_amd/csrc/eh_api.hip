@@ -414,8 +414,24 @@ int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int6
     int rc = check_requant(q);
     if (rc) return rc;
     EH_REQUIRE(count >= 0 && (count == 0 || (acc && out)), "requant_apply: null array");
-    EH_REQUIRE(form == 0 || form == 1, "requant_apply: form %d", form);
+    EH_REQUIRE(form >= 0 && form <= 3, "requant_apply: form %d", form);
     const RequantDev r = make_requant_dev(*q);
+    if (form >= 2) {  // the per-channel single-shift forms, with the requant's pair as the channel's
+        EH_REQUIRE(channel_pair_is_fast(q->multiplier, q->shift, form == 3 ? -2 : -1) && channel_fast_mode(*q) != 0,
+                   "requant_apply: multiplier %d, shift %d, zero point %d are outside form %d", q->multiplier, q->shift, q->zp_out, form);
+        const int mode = channel_fast_mode(*q), rs = -q->shift;
+        if (single_shift) *single_shift = 1;
+        for (int64_t i = 0; i < count; ++i) {
+            uint32_t v;
+            if (form == 2)
+                v = mode == 2 ? requant_u8_channel_fast<2>(acc[i], q->multiplier, q->shift, r) : requant_u8_channel_fast<1>(acc[i], q->multiplier, q->shift, r);
+            else
+                v = mode == 2 ? requant_u8_channel_table<2>(acc[i], q->multiplier, rs - 1, channel_table_pos_hi(q->zp_out, rs), r)
+                              : requant_u8_channel_table<1>(acc[i], q->multiplier, rs - 1, channel_table_pos_hi(q->zp_out, rs), r);
+            out[i] = (uint8_t)v;
+        }
+        return EH_OK;
+    }
     const bool fast = form == 0 && r.fast;
     if (single_shift) *single_shift = fast ? 1 : 0;
     for (int64_t i = 0; i < count; ++i)

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                 const int32_t rs = -p.rq.pc_shift[nb_first * 32 + i];
                 pcm_s[i] = p.rq.pc_multiplier[nb_first * 32 + i];
                 pcf_s[i] = rs - 1;
-                pch_s[i] = (int32_t)((uint32_t)(1 + 2 * p.rq.zp_out) << (rs - 2));
+                pch_s[i] = channel_table_pos_hi(p.rq.zp_out, rs);
             }
         }
         if constexpr (RES) {

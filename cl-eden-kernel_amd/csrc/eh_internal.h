@@ -162,6 +162,11 @@ __host__ __device__ __forceinline__ uint32_t requant_u8_channel_table(int32_t x,
     return (uint32_t)v;
 }
 
+// high word of the table form's rounding term for a right shift rs >= 2
+__host__ __device__ __forceinline__ int32_t channel_table_pos_hi(int32_t zp_out, int32_t rs) {
+    return (int32_t)((uint32_t)(1 + 2 * zp_out) << (rs - 2));
+}
+
 // whether the single-shift form covers a channel's pair
 inline bool channel_pair_is_fast(int32_t multiplier, int32_t shift, int32_t max_shift = -1) {
     return multiplier >= 0 && shift <= max_shift && shift >= -20;

@@ -107,6 +107,17 @@ def op_weights(op, cin):
     return w, b
 
 
+def op_weights_perchannel(op, cin):
+    """(int8 weights, bias, float32 scale per output channel) of a conv / dw operator in the per-channel form
+    (int8 weights at zero point 0, as TFLite's full-integer converter writes them): clip(round(N(0, 20))) and the
+    layer's weight scale times a factor in [0.5, 2] per channel."""
+    shape = (op["cout"], 1 if op["op"] == "dw" else cin, op["k"], op["k"])
+    w = (synth.fill_u8_normal(shape, op["w_seed"], 128, W_SD).astype(np.int16) - 128).clip(-127, 127).astype(np.int8)
+    b = synth.fill_i32((op["cout"],), op["b_seed"], -op["b_range"], op["b_range"])
+    factor = 0.5 + 1.5 * synth.fill_u8((op["cout"],), op["w_seed"] + 2).astype(np.float32) / 255.0
+    return w, b, (np.float32(op["w_scale"]) * factor).astype(np.float32)
+
+
 def network_input(batch, image=224):
     """uint8 uniform[0, 255], channels-last [batch, image, image, 3]"""
     return synth.fill_u8((batch, image, image, 3), SEED + 9999)
@@ -140,9 +151,12 @@ class MobileNetV2:
 
     fuse_add: a residual Add whose second operand is the projection convolution right before it (and nothing else
     reads that projection) runs inside that convolution's launch (`ConvPlan.run_add`); the projection's own tensor
-    is then never written.  Results are the same bit for bit."""
+    is then never written.  Results are the same bit for bit.
 
-    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False):
+    per_channel: convolutions and depthwise convolutions take int8 weights with one scale per output channel
+    (`op_weights_perchannel`); tensors stay uint8 and the classifier keeps its per-tensor uint8 weights."""
+
+    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False, per_channel=False):
         self.eden, self.batch, self.image = eden, batch, image
         self.tensors, self.ops = layers(image)
         self.buffers = [eden.DeviceBuffer(nbytes=batch * t["h"] * t["w"] * t["c"]) for t in self.tensors]
@@ -175,23 +189,33 @@ class MobileNetV2:
             if kind == "avgpool":
                 self.steps.append(("avgpool", (self.buffers[op["src"]], self.buffers[op["dst"]], s, op["k"])))
                 continue
-            w, b = op_weights(op, s["c"])
+            act = eden.ACT_RELU6 if op.get("relu6") else eden.ACT_NONE
+            pairs = None
+            if per_channel and kind != "fc":
+                w, b, w_scales = op_weights_perchannel(op, s["c"])
+                q, mults, shifts = eden.make_requant_perchannel(s["scale"], s["zp"], w_scales, d["scale"], d["zp"], act,
+                                                                bool(op.get("relu6")))
+                pairs = (mults, shifts)
+            else:
+                w, b = op_weights(op, s["c"])
+                q = eden.make_requant(s["scale"], s["zp"], op["w_scale"], op["w_zp"], d["scale"], d["zp"], act, bool(op.get("relu6")))
+            w_layout = eden.W_OIHW | (eden.W_SIGNED if pairs else 0)
             d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
             self._keep += [d_w, d_b]
-            act = eden.ACT_RELU6 if op.get("relu6") else eden.ACT_NONE
-            q = eden.make_requant(s["scale"], s["zp"], op["w_scale"], op["w_zp"], d["scale"], d["zp"], act, bool(op.get("relu6")))
             if kind == "fc":
                 plan = eden.FcPlan(batch, s["c"], op["cout"], d_w, d_b, q, stream)
             else:
                 pad = (op["pad"],) * 4
                 if kind == "dw":
                     desc = eden.conv_desc(batch, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, pad,
-                                          (1, 1), 1, 1, eden.NHWC, eden.W_OIHW)
+                                          (1, 1), 1, 1, eden.NHWC, w_layout)
                     plan = eden.DwConvPlan(desc, d_w, d_b, q, stream)
                 else:
                     desc = eden.conv_desc(batch, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, pad,
-                                          (1, 1), 1, 1, eden.NHWC, eden.W_OIHW)
+                                          (1, 1), 1, 1, eden.NHWC, w_layout)
                     plan = eden.ConvPlan(desc, d_w, d_b, q, stream)
+                if pairs:
+                    plan.set_perchannel(*pairs)
             self.steps.append(("plan", (plan, self.buffers[op["src"]], self.buffers[op["dst"]], q)))
         eden.sync(stream)
 

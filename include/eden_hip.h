@@ -136,7 +136,12 @@ void eh_make_requant_s8(float input_scale, int32_t input_zp, float filter_scale,
  * the host with the same source the kernels compile.  form 0 evaluates it the
  * way the kernels would for these parameters (a single 64-bit multiply-add and
  * shift where that is exact, *single_shift reports which), form 1 always takes
- * the two-step reference order. */
+ * the two-step reference order.  Forms 2 and 3 are the single-shift forms the
+ * kernels use with one multiplier and shift per channel (conv_per_channel_quantized,
+ * gpu/operators/cl_kernels/ConvolutionKernels.cpp:1317-1375), q's pair standing for
+ * the channel's: 2 with the rounding term computed from the shift (-20 <= shift <= -1),
+ * 3 with it taken from a per-channel table (-20 <= shift <= -2); parameters outside
+ * those ranges are an error, as the kernels then take the two-step order. */
 int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int64_t count, int32_t form,
                      int32_t *single_shift);
 /* What CLConvolutionPerChannelQuantized::execute derives (CLConvolutionPerChannelQuantized.cpp:88-121):

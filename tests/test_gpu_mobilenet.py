@@ -13,7 +13,7 @@ mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
 pytestmark = pytest.mark.gpu
 
 
-def oracle_forward(x_nhwc, image):
+def oracle_forward(x_nhwc, image, per_channel=False):
     """All tensors of the network, NCHW, computed by the oracle from the same operator list."""
     tensors, ops = mobilenet.layers(image)
     vals = [np.ascontiguousarray(x_nhwc.transpose(0, 3, 1, 2))]
@@ -30,8 +30,20 @@ def oracle_forward(x_nhwc, image):
         if kind == "avgpool":
             vals.append(O.avgpool(x, op["k"], op["k"]))
             continue
-        w, b = mobilenet.op_weights(op, s["c"])
         act = O.ACT_RELU6 if op.get("relu6") else O.ACT_NONE
+        if per_channel and kind != "fc":
+            w, b, w_scales = mobilenet.op_weights_perchannel(op, s["c"])
+            eq, mults, shifts = eden.make_requant_perchannel(s["scale"], s["zp"], w_scales, d["scale"], d["zp"], act, bool(op.get("relu6")))
+            q = O.raw_quant(zp_in=eq.zp_in, zp_w=0, zp_out=eq.zp_out, act_min=eq.act_min, act_max=eq.act_max)
+            lo, hi = O.act_range_u8(act if op.get("relu6") else O.ACT_NONE, d["scale"], d["zp"])
+            assert (eq.zp_in, eq.zp_out, eq.act_min, eq.act_max) == (s["zp"], d["zp"], lo, hi)
+            groups = s["c"] if kind == "dw" else 1
+            shape = O.conv_shape(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4,
+                                 groups=groups)
+            fn = O.dwconv2d_perchannel if kind == "dw" else O.conv2d_perchannel
+            vals.append(fn(x, w, b, shape, q, mults, shifts))
+            continue
+        w, b = mobilenet.op_weights(op, s["c"])
         q = O.make_quant(s["scale"], s["zp"], op["w_scale"], op["w_zp"], d["scale"], d["zp"], act, bool(op.get("relu6")))
         if kind == "fc":
             vals.append(O.fc(x.reshape(n, -1), w, b, q).reshape(n, -1, 1, 1))
@@ -92,3 +104,29 @@ def test_mobilenet_v2_graph_replay_equals_eager():
         assert np.array_equal(net.logits(), eager), rep
         net.run()           # eager work between the replays
         eden.sync()
+
+
+@pytest.mark.parametrize("batch,image", [(2, 224), (3, 96)])
+def test_mobilenet_v2_per_channel_weights_matches_oracle_tensor_by_tensor(batch, image):
+    """The same network with int8 weights and one scale per output channel in every convolution and depthwise
+    convolution (uint8 tensors, residual adds inside the projection convolutions)."""
+    print("mobilenet per-channel", batch, image, flush=True)
+    x = mobilenet.network_input(batch, image)
+    tensors, ops, want = oracle_forward(x, image, per_channel=True)
+    net = mobilenet.MobileNetV2(eden, batch, image, fuse_add=True, per_channel=True)
+    net.set_input(x)
+    net.run()
+    eden.sync()
+    assert len(net.unwritten) == 10
+    for op in ops:
+        i = op["dst"]
+        if i in net.unwritten:
+            continue
+        got = net.tensor(i).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, want[i]), (op["op"], i, tensors[i], int((got != want[i]).sum()))
+    for op in ops:
+        v = want[op["dst"]]
+        assert v.std() > 8, (op["op"], op["dst"], float(v.std()))
+        assert np.mean((v == 0) | (v == 255)) < 0.8, (op["op"], op["dst"])
+    logits = want[-1].reshape(batch, -1)
+    assert len(np.unique(logits)) > 40 and not np.array_equal(logits[0], logits[1])

@@ -69,3 +69,32 @@ def test_other_shifts_take_the_two_step_form(shift):
         got, single = eden.requant_apply(to_eh(q), acc)
         assert not single
         assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("rs", [1, 2, 3, 7, 8, 11, 16, 20])
+def test_per_channel_single_shift_forms_equal_oracle(rs):
+    """The two per-channel forms (rounding term from the shift in registers; from a table, for rs >= 2), with and
+    without the sign test (clamp floor below / at the output zero point)."""
+    rng = np.random.default_rng(3000 + rs)
+    for mult in MULTIPLIERS:
+        for zp_out, lo, hi in ((0, 0, 255), (128, 0, 255), (255, 20, 230), (3, 3, 3), (131, 131, 255), (5, 9, 255)):
+            q = O.raw_quant(zp_out=zp_out, multiplier=mult, shift=-rs, act_min=lo, act_max=hi)
+            acc = probe_accumulators(mult, rs, rng)
+            want = np.array([O.lib.eo_requant(int(a), q) for a in acc], np.uint8)
+            for form in ("registers", "table"):
+                if form == "table" and rs < 2:
+                    with pytest.raises(eden.EdenHipError):
+                        eden.requant_apply(to_eh(q), acc, channel_form=form)
+                    continue
+                got, single = eden.requant_apply(to_eh(q), acc, channel_form=form)
+                bad = np.nonzero(got != want)[0]
+                assert single and bad.size == 0, (form, mult, rs, zp_out, acc[bad[:5]], got[bad[:5]], want[bad[:5]])
+
+
+def test_per_channel_forms_refuse_shifts_outside_their_range():
+    acc = np.arange(-5, 5, dtype=np.int32)
+    for shift in (-21, 0, 1):
+        q = O.raw_quant(zp_out=7, multiplier=1 << 30, shift=shift)
+        for form in ("registers", "table"):
+            with pytest.raises(eden.EdenHipError):
+                eden.requant_apply(to_eh(q), acc, channel_form=form)
