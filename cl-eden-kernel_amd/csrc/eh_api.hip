@@ -342,9 +342,9 @@ struct GemmOp {
             if (pc_multiplier) {
                 p.rq.pc_multiplier = pc_multiplier + g.bias_base;
                 p.rq.pc_shift = pc_shift + g.bias_base;
-                // the one-tap and the direct-to-LDS kernels have the single-shift form per channel; the others'
-                // per-channel code sits on their general path
-                const bool has_form = g.cfg.id != GEMM_STAGED && g.cfg.id != GEMM_C3K3;
+                // every kernel but the register-staged one has the single-shift form per channel (the first-layer
+                // kernel for fewer than 32 channels ignores the flag)
+                const bool has_form = g.cfg.id != GEMM_STAGED;
                 p.rq.fast = (pc_fast && has_form) ? channel_fast_mode(q) : 0;
             }
             problems.push_back(p);

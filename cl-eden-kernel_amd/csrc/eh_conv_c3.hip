@@ -83,7 +83,8 @@ __device__ __forceinline__ void gather_c3k3(const GemmProblem &p, const uint32_t
     }
 }
 
-// Matrix-core form, per-tensor requantization.  Grid: x = 256 pixels per workgroup (64 per wave).
+// Matrix-core form.  Grid: x = 256 pixels per workgroup (64 per wave).  With one multiplier and shift per channel,
+// FAST means that every channel's pair is inside the single-shift form's range.
 template <bool ROWSUM, bool FAST>
 __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p, const uint32_t in_bytes) {
     const int lane = threadIdx.x & 63, r = lane & 31, half = lane >> 5;
@@ -138,6 +139,20 @@ __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const int4 bb = *reinterpret_cast<const int4 *>(p.bias + n + g * 4);
+                    if (rq.pc_multiplier) {  // (the arrays are padded past the last channel block)
+                        const int4 cm = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + g * 4);
+                        const int4 cs = *reinterpret_cast<const int4 *>(rq.pc_shift + n + g * 4);
+                        auto one = [&](int x, int32_t mult, int32_t shift) {
+                            if constexpr (mode == 0)
+                                return requant_u8_channel(x, mult, shift, rq);
+                            else
+                                return requant_u8_channel_fast<mode>(x, mult, shift, rq);
+                        };
+                        packed[g] = (one(acc[g * 4 + 0] + bb.x + ncorr, cm.x, cs.x) | (one(acc[g * 4 + 1] + bb.y + ncorr, cm.y, cs.y) << 8) |
+                                     (one(acc[g * 4 + 2] + bb.z + ncorr, cm.z, cs.z) << 16) | (one(acc[g * 4 + 3] + bb.w + ncorr, cm.w, cs.w) << 24)) ^
+                                    p.out_xor;
+                        continue;
+                    }
                     packed[g] = (requant_u8_as<mode>(acc[g * 4 + 0] + bb.x + ncorr, rq) | (requant_u8_as<mode>(acc[g * 4 + 1] + bb.y + ncorr, rq) << 8) |
                                  (requant_u8_as<mode>(acc[g * 4 + 2] + bb.z + ncorr, rq) << 16) |
                                  (requant_u8_as<mode>(acc[g * 4 + 3] + bb.w + ncorr, rq) << 24)) ^
@@ -269,8 +284,9 @@ int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream) {
     const int images = (p.m + p.ho * p.wo - 1) / (p.ho * p.wo);
     EH_REQUIRE(in_bytes * images < (1ull << 31), "conv_c3k3: input too large");
     const uint32_t total_bytes = (uint32_t)(in_bytes * images);
-    const bool rowsum = p.zw != 0, fast = p.rq.fast != 0;
-    if (p.n >= 32 && p.rq.pc_multiplier == nullptr) {  // the packed rows and the folded bias are padded to whole tiles of channels
+    const bool rowsum = p.zw != 0;
+    bool fast = p.rq.fast != 0;
+    if (p.n >= 32) {  // the packed rows and the folded bias are padded to whole tiles of channels
         const dim3 grid_m((p.m + 255) / 256);
         if (rowsum && fast)
             hipLaunchKernelGGL((conv_c3k3_mfma_kernel<true, true>), grid_m, dim3(256), 0, stream, p, total_bytes);
@@ -284,6 +300,7 @@ int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream) {
         return EH_OK;
     }
     const dim3 grid((p.m + 255) / 256, (p.n + 15) / 16);
+    if (p.rq.pc_multiplier) fast = false;  // this kernel's per-channel code is the two-step order
     if (rowsum && fast)
         hipLaunchKernelGGL((conv_c3k3_kernel<true, true>), grid, dim3(256), 0, stream, p, total_bytes);
     else if (rowsum)

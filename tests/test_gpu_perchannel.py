@@ -87,6 +87,12 @@ def test_perchannel_conv_matches_oracle(case, layout):
     oq_relu = O.raw_quant(zp_in=117, zp_w=0, zp_out=131, act_min=131)
     got, _ = gpu_conv_perchannel(x, w, b, s, q, mults, shifts, layout)
     assert np.array_equal(got, O.conv2d_perchannel(x, w, b, s, oq_relu, mults, shifts))
+    # one channel's shift outside the single-shift form's range: the whole launch takes the two-step order
+    odd_shifts = shifts.copy()
+    odd_shifts[s.cout // 3] = 0
+    got, _ = gpu_conv_perchannel(x, w, b, s, q, mults, odd_shifts, layout)
+    assert np.array_equal(got, O.conv2d_perchannel(x, w, b, s, oq_relu, mults, odd_shifts))
+    q.act_min = 0
     # per-tensor mode on the same plan: int8 weights with the requant's own pair
     q2 = eden.Requant(117, 0, 131, int(mults[0]), int(shifts[0]), 0, 255)
     oq2 = O.raw_quant(zp_in=117, zp_w=0, zp_out=131, multiplier=int(mults[0]), shift=int(shifts[0]))
