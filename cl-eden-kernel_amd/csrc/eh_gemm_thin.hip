@@ -129,38 +129,52 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         }
         return af;
     };
-    // 16 accumulators of one channel block -> 16 output bytes of the lane's pixel
+    // The accumulators start from the folded bias (plus `extra`, the pixel's row-sum term where it is known before the
+    // products): the matrix instruction adds to them, so the epilogue has no additions left to do.
+    auto start_block = [&](int nb_local, int extra) {
+        const int32_t *bsrc = bias_s + nb_local * 32 + half * 16;
+        v16i acc;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int4 bb = *reinterpret_cast<const int4 *>(bsrc + g * 4);
+            acc[g * 4 + 0] = bb.x + extra;
+            acc[g * 4 + 1] = bb.y + extra;
+            acc[g * 4 + 2] = bb.z + extra;
+            acc[g * 4 + 3] = bb.w + extra;
+        }
+        return acc;
+    };
+    // 16 accumulators of one channel block (bias included) -> 16 output bytes of the lane's pixel; `ncorr` is what
+    // is still to be added to each
     auto finish_block = [&](const v16i &acc, int nb_local, int ncorr, bool ok, size_t out_off) {
         const int n = (nb_first + nb_local) * 32 + half * 16;  // this lane's 16 consecutive channels
-        const int32_t *bsrc = bias_s + nb_local * 32 + half * 16;
         uint32_t packed[4];
         auto quantize = [&](auto mode_c) {
             constexpr int mode = decltype(mode_c)::value;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int4 bb = *reinterpret_cast<const int4 *>(bsrc + g * 4);
                 uint32_t o0, o1, o2, o3;
                 if constexpr (QM == 2) {
                     const int tab = nb_local * 32 + half * 16 + g * 4;
                     const int4 cm = *reinterpret_cast<const int4 *>(pcm_s + tab);
                     const int4 cf = *reinterpret_cast<const int4 *>(pcf_s + tab);
                     const int4 ch = *reinterpret_cast<const int4 *>(pch_s + tab);
-                    o0 = requant_u8_channel_table<mode>(acc[g * 4 + 0] + bb.x + ncorr, cm.x, cf.x, ch.x, rq);
-                    o1 = requant_u8_channel_table<mode>(acc[g * 4 + 1] + bb.y + ncorr, cm.y, cf.y, ch.y, rq);
-                    o2 = requant_u8_channel_table<mode>(acc[g * 4 + 2] + bb.z + ncorr, cm.z, cf.z, ch.z, rq);
-                    o3 = requant_u8_channel_table<mode>(acc[g * 4 + 3] + bb.w + ncorr, cm.w, cf.w, ch.w, rq);
+                    o0 = requant_u8_channel_table<mode>(acc[g * 4 + 0] + ncorr, cm.x, cf.x, ch.x, rq);
+                    o1 = requant_u8_channel_table<mode>(acc[g * 4 + 1] + ncorr, cm.y, cf.y, ch.y, rq);
+                    o2 = requant_u8_channel_table<mode>(acc[g * 4 + 2] + ncorr, cm.z, cf.z, ch.z, rq);
+                    o3 = requant_u8_channel_table<mode>(acc[g * 4 + 3] + ncorr, cm.w, cf.w, ch.w, rq);
                 } else if (mode == 0 && rq.pc_multiplier) {  // per-channel parameters (the padded arrays cover whole blocks)
                     const int4 cm = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + g * 4);
                     const int4 cs = *reinterpret_cast<const int4 *>(rq.pc_shift + n + g * 4);
-                    o0 = requant_u8_channel(acc[g * 4 + 0] + bb.x + ncorr, cm.x, cs.x, rq);
-                    o1 = requant_u8_channel(acc[g * 4 + 1] + bb.y + ncorr, cm.y, cs.y, rq);
-                    o2 = requant_u8_channel(acc[g * 4 + 2] + bb.z + ncorr, cm.z, cs.z, rq);
-                    o3 = requant_u8_channel(acc[g * 4 + 3] + bb.w + ncorr, cm.w, cs.w, rq);
+                    o0 = requant_u8_channel(acc[g * 4 + 0] + ncorr, cm.x, cs.x, rq);
+                    o1 = requant_u8_channel(acc[g * 4 + 1] + ncorr, cm.y, cs.y, rq);
+                    o2 = requant_u8_channel(acc[g * 4 + 2] + ncorr, cm.z, cs.z, rq);
+                    o3 = requant_u8_channel(acc[g * 4 + 3] + ncorr, cm.w, cs.w, rq);
                 } else {
-                    o0 = requant_u8_as<mode>(acc[g * 4 + 0] + bb.x + ncorr, rq);
-                    o1 = requant_u8_as<mode>(acc[g * 4 + 1] + bb.y + ncorr, rq);
-                    o2 = requant_u8_as<mode>(acc[g * 4 + 2] + bb.z + ncorr, rq);
-                    o3 = requant_u8_as<mode>(acc[g * 4 + 3] + bb.w + ncorr, rq);
+                    o0 = requant_u8_as<mode>(acc[g * 4 + 0] + ncorr, rq);
+                    o1 = requant_u8_as<mode>(acc[g * 4 + 1] + ncorr, rq);
+                    o2 = requant_u8_as<mode>(acc[g * 4 + 2] + ncorr, rq);
+                    o3 = requant_u8_as<mode>(acc[g * 4 + 3] + ncorr, rq);
                 }
                 packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
             }
@@ -235,12 +249,10 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
 #pragma unroll
                 for (int u = 0; u < NBU; ++u) {
                     if (nb0 + u >= nb_count) break;
-                    v16i acc;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[i] = 0;
+                    v16i acc = start_block(nb0 + u, ncorr);
 #pragma unroll
                     for (int t = 0; t < KU; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[u][t], af[t], acc, 0, 0, 0);
-                    finish_block(acc, nb0 + u, ncorr, ok, out_off);
+                    finish_block(acc, nb0 + u, 0, ok, out_off);
                 }
             }
             ok = ok_next;
@@ -261,9 +273,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
             for (int nb0 = 0; nb0 < nb_count; nb0 += NBU) {
                 v16i acc[NBU];
 #pragma unroll
-                for (int u = 0; u < NBU; ++u)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[u][i] = 0;
+                for (int u = 0; u < NBU; ++u) acc[u] = start_block(nb0 + u < nb_count ? nb0 + u : nb_count - 1, 0);
                 int rowsum = 0;
                 for (int ks0 = 0; ks0 < ksteps; ks0 += KU) {
                     // steps past the last one read bytes that flip to 0, so they multiply whatever weights they re-read by zero
