@@ -128,17 +128,23 @@ __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p
             // weight rows are stored plainly, [channel][32 bytes]: row `r` of the fragment is channel 16 h + 4 g + t of the block
             const int ch = nb * 32 + 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
             const v4i wf = *reinterpret_cast<const v4i *>(p.b + (size_t)ch * 32 + half * 16);
+            const int n = nb * 32 + half * 16;
+            // the accumulators start from the folded bias and the pixel's row-sum term: nothing left to add afterwards
             v16i acc;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[e] = 0;
+            for (int g = 0; g < 4; ++g) {
+                const int4 bb = *reinterpret_cast<const int4 *>(p.bias + n + g * 4);
+                acc[g * 4 + 0] = bb.x + ncorr;
+                acc[g * 4 + 1] = bb.y + ncorr;
+                acc[g * 4 + 2] = bb.z + ncorr;
+                acc[g * 4 + 3] = bb.w + ncorr;
+            }
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf, af[b], acc, 0, 0, 0);
-            const int n = nb * 32 + half * 16;
             uint32_t packed[4];
             auto produce = [&](auto mode_c) {
                 constexpr int mode = decltype(mode_c)::value;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int4 bb = *reinterpret_cast<const int4 *>(p.bias + n + g * 4);
                     if (rq.pc_multiplier) {  // (the arrays are padded past the last channel block)
                         const int4 cm = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + g * 4);
                         const int4 cs = *reinterpret_cast<const int4 *>(rq.pc_shift + n + g * 4);
@@ -148,14 +154,14 @@ __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p
                             else
                                 return requant_u8_channel_fast<mode>(x, mult, shift, rq);
                         };
-                        packed[g] = (one(acc[g * 4 + 0] + bb.x + ncorr, cm.x, cs.x) | (one(acc[g * 4 + 1] + bb.y + ncorr, cm.y, cs.y) << 8) |
-                                     (one(acc[g * 4 + 2] + bb.z + ncorr, cm.z, cs.z) << 16) | (one(acc[g * 4 + 3] + bb.w + ncorr, cm.w, cs.w) << 24)) ^
+                        packed[g] = (one(acc[g * 4 + 0], cm.x, cs.x) | (one(acc[g * 4 + 1], cm.y, cs.y) << 8) |
+                                     (one(acc[g * 4 + 2], cm.z, cs.z) << 16) | (one(acc[g * 4 + 3], cm.w, cs.w) << 24)) ^
                                     p.out_xor;
                         continue;
                     }
-                    packed[g] = (requant_u8_as<mode>(acc[g * 4 + 0] + bb.x + ncorr, rq) | (requant_u8_as<mode>(acc[g * 4 + 1] + bb.y + ncorr, rq) << 8) |
-                                 (requant_u8_as<mode>(acc[g * 4 + 2] + bb.z + ncorr, rq) << 16) |
-                                 (requant_u8_as<mode>(acc[g * 4 + 3] + bb.w + ncorr, rq) << 24)) ^
+                    packed[g] = (requant_u8_as<mode>(acc[g * 4 + 0], rq) | (requant_u8_as<mode>(acc[g * 4 + 1], rq) << 8) |
+                                 (requant_u8_as<mode>(acc[g * 4 + 2], rq) << 16) |
+                                 (requant_u8_as<mode>(acc[g * 4 + 3], rq) << 24)) ^
                                 p.out_xor;
                 }
             };
