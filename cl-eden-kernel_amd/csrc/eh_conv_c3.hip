@@ -154,14 +154,13 @@ __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p
                             else
                                 return requant_u8_channel_fast<mode>(x, mult, shift, rq);
                         };
-                        packed[g] = (one(acc[g * 4 + 0], cm.x, cs.x) | (one(acc[g * 4 + 1], cm.y, cs.y) << 8) |
-                                     (one(acc[g * 4 + 2], cm.z, cs.z) << 16) | (one(acc[g * 4 + 3], cm.w, cs.w) << 24)) ^
+                        packed[g] = pack_bytes(one(acc[g * 4 + 0], cm.x, cs.x), one(acc[g * 4 + 1], cm.y, cs.y),
+                                               one(acc[g * 4 + 2], cm.z, cs.z), one(acc[g * 4 + 3], cm.w, cs.w)) ^
                                     p.out_xor;
                         continue;
                     }
-                    packed[g] = (requant_u8_as<mode>(acc[g * 4 + 0], rq) | (requant_u8_as<mode>(acc[g * 4 + 1], rq) << 8) |
-                                 (requant_u8_as<mode>(acc[g * 4 + 2], rq) << 16) |
-                                 (requant_u8_as<mode>(acc[g * 4 + 3], rq) << 24)) ^
+                    packed[g] = pack_bytes(requant_u8_as<mode>(acc[g * 4 + 0], rq), requant_u8_as<mode>(acc[g * 4 + 1], rq),
+                                           requant_u8_as<mode>(acc[g * 4 + 2], rq), requant_u8_as<mode>(acc[g * 4 + 3], rq)) ^
                                 p.out_xor;
                 }
             };
@@ -263,7 +262,7 @@ __global__ __launch_bounds__(256) void conv_c3k3_kernel(const GemmProblem p, con
             o[t] = mode == 0 && rq.pc_multiplier ? requant_u8_channel(acc, rq.pc_multiplier[n], rq.pc_shift[n], rq)
                                                  : requant_u8_as<mode>(acc, rq);
         }
-        packed[g] = (o[0] | (o[1] << 8) | (o[2] << 16) | (o[3] << 24)) ^ p.out_xor;
+        packed[g] = pack_bytes(o[0], o[1], o[2], o[3]) ^ p.out_xor;
     }
     };
     if constexpr (!FAST)

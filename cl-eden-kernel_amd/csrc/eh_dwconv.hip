@@ -51,24 +51,23 @@ __device__ __forceinline__ ChannelQuad load_channel_quad(const RequantDev &rq, u
 template <bool PC = true>
 __device__ __forceinline__ uint32_t requant4(int acc0, int acc1, int acc2, int acc3, const RequantDev &rq, const ChannelQuad &cq) {
     if (PC && rq.pc_multiplier)  // the two-step order; the single-shift form per channel is the dot product kernel's
-        return requant_u8_channel(acc0, cq.m.x, cq.s.x, rq) | (requant_u8_channel(acc1, cq.m.y, cq.s.y, rq) << 8) |
-               (requant_u8_channel(acc2, cq.m.z, cq.s.z, rq) << 16) | (requant_u8_channel(acc3, cq.m.w, cq.s.w, rq) << 24);
+        return pack_bytes(requant_u8_channel(acc0, cq.m.x, cq.s.x, rq), requant_u8_channel(acc1, cq.m.y, cq.s.y, rq),
+                          requant_u8_channel(acc2, cq.m.z, cq.s.z, rq), requant_u8_channel(acc3, cq.m.w, cq.s.w, rq));
     if (rq.fast == 2)
-        return requant_u8_fast_relu(acc0, rq) | (requant_u8_fast_relu(acc1, rq) << 8) | (requant_u8_fast_relu(acc2, rq) << 16) |
-               (requant_u8_fast_relu(acc3, rq) << 24);
+        return pack_bytes(requant_u8_fast_relu(acc0, rq), requant_u8_fast_relu(acc1, rq),
+                          requant_u8_fast_relu(acc2, rq), requant_u8_fast_relu(acc3, rq));
     if (rq.fast)
-        return requant_u8_fast(acc0, rq) | (requant_u8_fast(acc1, rq) << 8) | (requant_u8_fast(acc2, rq) << 16) |
-               (requant_u8_fast(acc3, rq) << 24);
-    return requant_u8(acc0, rq) | (requant_u8(acc1, rq) << 8) | (requant_u8(acc2, rq) << 16) | (requant_u8(acc3, rq) << 24);
+        return pack_bytes(requant_u8_fast(acc0, rq), requant_u8_fast(acc1, rq), requant_u8_fast(acc2, rq), requant_u8_fast(acc3, rq));
+    return pack_bytes(requant_u8(acc0, rq), requant_u8(acc1, rq), requant_u8(acc2, rq), requant_u8(acc3, rq));
 }
 
 // the per-channel single-shift form alone (rq.fast is 1 or 2)
 __device__ __forceinline__ uint32_t requant4_channel_fast(int acc0, int acc1, int acc2, int acc3, const RequantDev &rq, const ChannelQuad &cq) {
     if (rq.fast == 2)
-        return requant_u8_channel_fast<2>(acc0, cq.m.x, cq.s.x, rq) | (requant_u8_channel_fast<2>(acc1, cq.m.y, cq.s.y, rq) << 8) |
-               (requant_u8_channel_fast<2>(acc2, cq.m.z, cq.s.z, rq) << 16) | (requant_u8_channel_fast<2>(acc3, cq.m.w, cq.s.w, rq) << 24);
-    return requant_u8_channel_fast<1>(acc0, cq.m.x, cq.s.x, rq) | (requant_u8_channel_fast<1>(acc1, cq.m.y, cq.s.y, rq) << 8) |
-           (requant_u8_channel_fast<1>(acc2, cq.m.z, cq.s.z, rq) << 16) | (requant_u8_channel_fast<1>(acc3, cq.m.w, cq.s.w, rq) << 24);
+        return pack_bytes(requant_u8_channel_fast<2>(acc0, cq.m.x, cq.s.x, rq), requant_u8_channel_fast<2>(acc1, cq.m.y, cq.s.y, rq),
+                          requant_u8_channel_fast<2>(acc2, cq.m.z, cq.s.z, rq), requant_u8_channel_fast<2>(acc3, cq.m.w, cq.s.w, rq));
+    return pack_bytes(requant_u8_channel_fast<1>(acc0, cq.m.x, cq.s.x, rq), requant_u8_channel_fast<1>(acc1, cq.m.y, cq.s.y, rq),
+                      requant_u8_channel_fast<1>(acc2, cq.m.z, cq.s.z, rq), requant_u8_channel_fast<1>(acc3, cq.m.w, cq.s.w, rq));
 }
 
 template <int KH, int KW>

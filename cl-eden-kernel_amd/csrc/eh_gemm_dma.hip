@@ -445,7 +445,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
                             o2 = requant_u8_as<fast>(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], rq);
                             o3 = requant_u8_as<fast>(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], rq);
                         }
-                        packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
+                        packed[g] = pack_bytes(o0, o1, o2, o3) ^ p.out_xor;
                     }
                     uint8_t *dst = p.out + row_off[i] + n;
                     if constexpr (!checked) {
@@ -547,7 +547,7 @@ __global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, c
                 o0 = requant_u8_as<fast>(s4.x + bb.x - corr, rq), o1 = requant_u8_as<fast>(s4.y + bb.y - corr, rq);
                 o2 = requant_u8_as<fast>(s4.z + bb.z - corr, rq), o3 = requant_u8_as<fast>(s4.w + bb.w - corr, rq);
             }
-            packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
+            packed[g] = pack_bytes(o0, o1, o2, o3) ^ p.out_xor;
         }
         };
         if (rq.fast == 2)

@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                     o2 = requant_u8_as<mode>(acc[g * 4 + 2] + ncorr, rq);
                     o3 = requant_u8_as<mode>(acc[g * 4 + 3] + ncorr, rq);
                 }
-                packed[g] = (o0 | (o1 << 8) | (o2 << 16) | (o3 << 24)) ^ p.out_xor;
+                packed[g] = pack_bytes(o0, o1, o2, o3) ^ p.out_xor;
             }
         };
         if constexpr (QM == 0)

@@ -177,7 +177,17 @@ inline int32_t channel_fast_mode(const eh_requant &q) {
     return q.act_min >= q.zp_out ? 2 : 1;
 }
 
-// MODE 0: two-step reference order; 1: single shift; 2: single shift without the sign test
+// Four values in 0 .. 255 to the four bytes of a word, lowest first: two byte permutes and one OR
+// (shift-and-OR takes four or five instructions).
+__host__ __device__ __forceinline__ uint32_t pack_bytes(uint32_t b0, uint32_t b1, uint32_t b2, uint32_t b3) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // v_perm_b32(S0, S1, sel): selector bytes 0..3 pick from S1, 4..7 from S0, 0x0c gives zero
+    return __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+#else
+    return b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+#endif
+}
+
 template <int MODE>
 __host__ __device__ __forceinline__ uint32_t requant_u8_as(int32_t acc, const RequantDev &r) {
     if constexpr (MODE == 2)
