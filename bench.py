@@ -269,7 +269,8 @@ def main():
         others = []
         for make, steps in ((conv_workload, 2000), (lambda e, s: conv_workload(e, s, 64), 300), (pw_workload, 500),
                             (dw_workload, 1000), (deconv_workload, 500),
-                            (lambda e, s: fc_workload(e, s, 8192, 4096, 4096), 100), (mbv2_workload, 40)):
+                            (lambda e, s: fc_workload(e, s, 8192, 4096, 4096), 100), (mbv2_workload, 40),
+                            (lambda e, s: mbv2_workload(e, s, per_channel=True), 40)):
             w2 = make(eden, synth)
             wall2, ev2 = time_steps(eden, stream, w2["launch"], steps, max(10, steps // 10), use_graph, w2.get("chunk", 50))
             entry = dict(workload=w2["name"], steps=steps, tops=round(w2["ops"] * steps / wall2 / 1e12, 2),
