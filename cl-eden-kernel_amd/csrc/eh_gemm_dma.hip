@@ -126,7 +126,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 }
 
 template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES, bool DENSE, bool ROWSUM>
-__global__ __launch_bounds__(256) void igemm_dma_kernel(const GemmBatch batch, const int count, const int tiles_m, const int tiles_n,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 && BN == 64 ? 3 : (BM == 128 && BN == 128 ? 2 : 1)))) void igemm_dma_kernel(const GemmBatch batch, const int count, const int tiles_m, const int tiles_n,
                                                         const int gm, const int gn) {
     static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
     constexpr int CPR = SLAB / 16;            // 16-byte chunks per LDS row
@@ -676,7 +676,7 @@ int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream) {
         case GEMM_DMA_256x256: return launch_cfg<256, 256, 2, 2, 1, 128, 2>(ps, count, stream);
         case GEMM_DMA_256x128: return launch_cfg<256, 128, 2, 2, 1, 128, 3>(ps, count, stream);
         case GEMM_DMA_128x128: return launch_cfg<128, 128, 2, 2, 1, 128, 2>(ps, count, stream);
-        case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 3>(ps, count, stream);
+        case GEMM_DMA_128x64: return launch_cfg<128, 64, 4, 1, 1, 128, 2>(ps, count, stream);
         case GEMM_DMA_64x64_SPLITK: {
             // Two stages take half the LDS, so two workgroups share a CU: for reductions of one or two slabs (deeper
             // staging has nothing to prefetch) and for launches with more tiles than CUs (the second workgroup's
