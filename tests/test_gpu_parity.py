@@ -196,6 +196,10 @@ CONV_CASES = [
     dict(n=2, c=3, h=13, w=9, cout=40, kh=3, kw=3, pad=(1, 1, 1, 1)),
     dict(n=3, c=3, h=21, w=23, cout=64, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),
     dict(n=1, c=3, h=3, w=3, cout=72, kh=3, kw=3),
+    # dilated taps through the direct-to-LDS tiles (16-byte channel units), alone and with stride and groups
+    dict(n=2, c=64, h=20, w=20, cout=64, kh=3, kw=3, pad=(2, 2, 2, 2), dil=(2, 2)),
+    dict(n=1, c=32, h=15, w=17, cout=32, kh=3, kw=3, stride=(2, 1), pad=(3, 3, 1, 1), dil=(3, 1), groups=2),
+    dict(n=3, c=16, h=12, w=9, cout=40, kh=2, kw=3, stride=(1, 2), pad=(0, 2, 2, 0), dil=(2, 3)),
 ]
 
 
@@ -344,6 +348,8 @@ DW_CASES = [
     dict(n=1, c=8, h=5, w=6, cout=8, kh=3, kw=3, pad=(2, 2, 2, 2)),
     dict(n=3, c=960, h=7, w=7, cout=960, kh=3, kw=3, pad=(1, 1, 1, 1)),
     dict(n=1, c=12, h=3, w=1, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=6, h=12, w=10, cout=12, kh=3, kw=2, stride=(2, 1), pad=(2, 2, 1, 1), dil=(2, 3), dm=2),   # dilation, stride and depth multiplier
+    dict(n=2, c=32, h=16, w=16, cout=32, kh=3, kw=3, stride=(2, 2), pad=(2, 2, 2, 2), dil=(2, 2)),
 ]
 
 
