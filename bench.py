@@ -169,6 +169,17 @@ def copy_workload(eden, synth, mib=64):
                 keep=(src, dst), ops=0.0, bytes=2 * nbytes, bound="hbm")
 
 
+def layout_workload(eden, synth, to_nhwc=True, n=64, c=96, h=112, w=112):
+    """NCHW <-> NHWC conversion of a feature map (MobileNetV2's largest, [64, 96, 112, 112]): bytes in + bytes out."""
+    nbytes = n * c * h * w
+    src, dst = eden.DeviceBuffer(host=synth.fill_u8((nbytes,), SEED + 90)), eden.DeviceBuffer(nbytes=nbytes)
+    lib = eden.load()
+    fn = lib.eh_transpose_u8_nchw2nhwc if to_nhwc else lib.eh_transpose_u8_nhwc2nchw
+    return dict(name="%s_n%d_c%d_%dx%d" % ("nchw2nhwc" if to_nhwc else "nhwc2nchw", n, c, h, w),
+                launch=lambda s: eden.check(fn(src.ptr, dst.ptr, n, c, h, w, s)),
+                keep=(src, dst), ops=0.0, bytes=2 * nbytes, bound="hbm")
+
+
 def roofline(work, event_s, steps):
     per_launch = event_s / steps
     if work["bound"] == "mfma":
@@ -209,7 +220,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv, mbv2, mbv2pc, copy")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv, mbv2, mbv2pc, copy, tonhwc, tonchw")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (got --gpus %d); no multi-GPU figure exists" % args.gpus,
@@ -225,7 +236,8 @@ def main():
 
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
                     fcbig=lambda e, s: fc_workload(e, s, 8192, 4096, 4096), conv64=lambda e, s: conv_workload(e, s, 64),
-                    copy=copy_workload, mbv2=mbv2_workload,
+                    copy=copy_workload, mbv2=mbv2_workload, tonhwc=layout_workload,
+                    tonchw=lambda e, s: layout_workload(e, s, to_nhwc=False),
                     mbv2pc=lambda e, s: mbv2_workload(e, s, per_channel=True))
     if args.only:
         work = families[args.only](eden, synth)
@@ -269,7 +281,9 @@ def main():
         others = []
         for make, steps in ((conv_workload, 2000), (lambda e, s: conv_workload(e, s, 64), 300), (pw_workload, 500),
                             (dw_workload, 1000), (deconv_workload, 500),
-                            (lambda e, s: fc_workload(e, s, 8192, 4096, 4096), 100), (mbv2_workload, 40),
+                            (lambda e, s: fc_workload(e, s, 8192, 4096, 4096), 100),
+                            (layout_workload, 200), (lambda e, s: layout_workload(e, s, to_nhwc=False), 200),
+                            (mbv2_workload, 40),
                             (lambda e, s: mbv2_workload(e, s, per_channel=True), 40)):
             w2 = make(eden, synth)
             wall2, ev2 = time_steps(eden, stream, w2["launch"], steps, max(10, steps // 10), use_graph, w2.get("chunk", 50))

@@ -92,9 +92,102 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t *__rest
     }
 }
 
+// The same transpose for extents that are multiples of 16 on both axes (most feature maps): 16 KiB tiles of
+// TR rows x TS columns, 16-byte global loads along S and 16-byte global stores along R, so a wave instruction
+// moves whole 128-byte lines on either side.  A thread brings four 16-byte chunks into LDS, then gathers a
+// block of 16 rows x 4 columns as sixteen dwords, transposes its four 4x4 byte blocks in registers (two
+// rounds of byte permutes) and stores, for each of its four columns, sixteen consecutive row bytes.
+// Three tile shapes: 128x128, 32x512 for few rows (NCHW -> NHWC with up to 32 channels) and 512x32 for few
+// columns (the way back).  The 16-byte chunks of an LDS row are XOR-swizzled by the 16-row group (the rows
+// themselves in the 32-column shape), which makes the dword gathers of a half wave fall on 32 distinct banks.
+__device__ __forceinline__ void transpose4x4_bytes(const uint32_t a0, const uint32_t a1, const uint32_t a2, const uint32_t a3,
+                                                   uint32_t out[4]) {
+    const uint32_t lo01 = __builtin_amdgcn_perm(a1, a0, 0x05010400u), hi01 = __builtin_amdgcn_perm(a1, a0, 0x07030602u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(a3, a2, 0x05010400u), hi23 = __builtin_amdgcn_perm(a3, a2, 0x07030602u);
+    out[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    out[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    out[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    out[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+template <int TR, int TS>
+__global__ __launch_bounds__(256) void transpose_u8_wide_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                                int32_t R, int32_t S) {
+    static_assert(TR * TS == 16384 && TR % 16 == 0 && TS % 16 == 0, "a 16 KiB tile, four chunks per thread");
+    constexpr int CPR = TS / 16;   // 16-byte chunks per tile row
+    constexpr int NRG = TR / 16;   // 16-row groups per tile
+    __shared__ __align__(16) uint8_t tile[TR * TS];
+    // where chunk c of row r sits in LDS
+    auto lds_pos = [](int r, int c) -> int {
+        if constexpr (TS == 32)
+            return ((r ^ ((r >> 4) & 3)) * CPR + c) * 16;
+        else if constexpr (NRG >= 8)
+            return (r * CPR + (c ^ ((r >> 4) & (CPR - 1)))) * 16;
+        else
+            return (r * CPR + (c ^ ((r >> 4) * (8 / NRG)))) * 16;
+    };
+    const size_t batch_off = (size_t)blockIdx.z * R * S;
+    src += batch_off;
+    dst += batch_off;
+    const int r0 = blockIdx.y * TR, s0 = blockIdx.x * TS;
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int idx = t + 256 * it, row = idx / CPR, c = idx % CPR;
+        const int gr = r0 + row, gs = s0 + 16 * c;
+        if (gr < R && gs < S)
+            *reinterpret_cast<uint4 *>(tile + lds_pos(row, c)) = *reinterpret_cast<const uint4 *>(src + (size_t)gr * S + gs);
+    }
+    __syncthreads();
+    // this thread's block: rows 16*rg .. 16*rg+15, columns 4*cg .. 4*cg+3
+    int rg, cg;
+    if constexpr (TS == 32) {
+        cg = t & 7;
+        rg = t >> 3;
+    } else {
+        rg = t % NRG;
+        cg = t / NRG;
+    }
+    const int gr = r0 + 16 * rg;
+    if (gr >= R) return;
+    uint32_t col[4][4];  // [column][row quad]
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t a[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const uint32_t *>(tile + lds_pos(16 * rg + 4 * q + i, cg >> 2) + (cg & 3) * 4);
+        uint32_t o[4];
+        transpose4x4_bytes(a[0], a[1], a[2], a[3], o);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) col[k][q] = o[k];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int gs = s0 + 4 * cg + k;
+        if (gs < S) *reinterpret_cast<uint4 *>(dst + (size_t)gs * R + gr) = make_uint4(col[k][0], col[k][1], col[k][2], col[k][3]);
+    }
+}
+
 int launch_transpose(const uint8_t *src, uint8_t *dst, int32_t batch, int32_t R, int32_t S, hipStream_t stream) {
     if (batch <= 0 || R <= 0 || S <= 0) return EH_OK;
     EH_REQUIRE(batch <= 65535, "transpose: batch %d exceeds the grid limit", batch);
+    if (R % 16 == 0 && S % 16 == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0) {
+        if (S <= 32 && (R + 511) / 512 <= 65535) {
+            hipLaunchKernelGGL((transpose_u8_wide_kernel<512, 32>), dim3(1, (R + 511) / 512, batch), dim3(256), 0, stream, src, dst, R, S);
+            EH_HIP(hipGetLastError());
+            return EH_OK;
+        }
+        if (R <= 32) {
+            hipLaunchKernelGGL((transpose_u8_wide_kernel<32, 512>), dim3((S + 511) / 512, 1, batch), dim3(256), 0, stream, src, dst, R, S);
+            EH_HIP(hipGetLastError());
+            return EH_OK;
+        }
+        if ((R + 127) / 128 <= 65535) {
+            hipLaunchKernelGGL((transpose_u8_wide_kernel<128, 128>), dim3((S + 127) / 128, (R + 127) / 128, batch), dim3(256), 0, stream, src, dst, R, S);
+            EH_HIP(hipGetLastError());
+            return EH_OK;
+        }
+    }
     const dim3 grid((S + TT - 1) / TT, (R + TT - 1) / TT, batch);
     hipLaunchKernelGGL(transpose_u8_kernel, grid, dim3(256), 0, stream, src, dst, R, S);
     EH_HIP(hipGetLastError());
