@@ -70,9 +70,14 @@ __device__ __forceinline__ uint32_t requant4_channel_fast(int acc0, int acc1, in
                       requant_u8_channel_fast<1>(acc2, cq.m.z, cq.s.z, rq), requant_u8_channel_fast<1>(acc3, cq.m.w, cq.s.w, rq));
 }
 
+// Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2.  Neighbouring output rows read
+// the same input rows, so every XCD takes one contiguous eighth of the block range (launch grids are whole
+// multiples of 8): a shared input row is then fetched from HBM into one L2 instead of two or three.
+__device__ __forceinline__ uint32_t xcd_contiguous_block() { return (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3); }
+
 template <int KH, int KW>
 __global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, const long total) {
-    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    const long idx = (long)xcd_contiguous_block() * 256 + threadIdx.x;
     if (idx >= total) return;
     const int cq_count = p.c >> 2;
     const int cq = (int)(idx % cq_count);
@@ -130,7 +135,7 @@ template <int S, bool PC, bool FLIP>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
     constexpr int TW = 4, IW = (TW - 1) * S + 3;
-    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t idx = xcd_contiguous_block() * 256u + threadIdx.x;
     if (idx >= total) return;
     // idx -> (image, output row, tile of four output columns, channel quad), channel quad fastest;
     // all offsets fit 32 bits (the launcher checks the tensor sizes)
@@ -212,7 +217,7 @@ template <int S, bool FLIP, int TW = 4, bool PC = false>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                     const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
     constexpr int IW = (TW - 1) * S + 3;
-    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t idx = xcd_contiguous_block() * 256u + threadIdx.x;
     if (idx >= total) return;
     const uint32_t cq_count = (uint32_t)p.c >> 2;
     uint32_t r = fastdiv(idx, div_cq);
@@ -418,20 +423,20 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
             const long total8 = (long)p.n * p.ho * tiles8 * (p.c >> 2);
             const FastDiv d_t8 = make_fastdiv((uint32_t)tiles8);
             auto kernel8 = pick_dot4(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{});
-            hipLaunchKernelGGL(kernel8, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, stream, p, (uint32_t)total8, tiles8, d_cq, d_t8,
+            hipLaunchKernelGGL(kernel8, dim3((unsigned)(((total8 + 255) / 256 + 7) / 8 * 8)), dim3(256), 0, stream, p, (uint32_t)total8, tiles8, d_cq, d_t8,
                                d_ho);
             EH_HIP(hipGetLastError());
             return EH_OK;
         }
-        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, (uint32_t)total, tiles_x, d_cq, d_t, d_ho);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)((blocks + 7) / 8 * 8)), dim3(256), 0, stream, p, (uint32_t)total, tiles_x, d_cq, d_t, d_ho);
     } else if (vec) {
         const long total = outs / 4;
         const long blocks = (total + 255) / 256;
         EH_REQUIRE(blocks < (1l << 31), "depthwise: grid too large");
         if (p.kh == 3 && p.kw == 3)
-            hipLaunchKernelGGL((dw_nhwc_vec4_kernel<3, 3>), dim3((unsigned)blocks), dim3(256), 0, stream, p, total);
+            hipLaunchKernelGGL((dw_nhwc_vec4_kernel<3, 3>), dim3((unsigned)((blocks + 7) / 8 * 8)), dim3(256), 0, stream, p, total);
         else
-            hipLaunchKernelGGL((dw_nhwc_vec4_kernel<0, 0>), dim3((unsigned)blocks), dim3(256), 0, stream, p, total);
+            hipLaunchKernelGGL((dw_nhwc_vec4_kernel<0, 0>), dim3((unsigned)((blocks + 7) / 8 * 8)), dim3(256), 0, stream, p, total);
     } else {
         const long blocks = (outs + 255) / 256;
         EH_REQUIRE(blocks < (1l << 31), "depthwise: grid too large");
