@@ -92,9 +92,10 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t *__rest
     }
 }
 
-// The same transpose for extents that are multiples of 16 on both axes (most feature maps): 16 KiB tiles of
+// The same transpose for extents that are multiples of 4 on both axes (most feature maps): 16 KiB tiles of
 // TR rows x TS columns, 16-byte global loads along S and 16-byte global stores along R, so a wave instruction
-// moves whole 128-byte lines on either side.  A thread brings four 16-byte chunks into LDS, then gathers a
+// moves whole 128-byte lines on either side when the extents are multiples of 16 (other multiples of 4 take
+// the same accesses at dword boundaries and finish rows and row groups with single dwords).  A thread brings four 16-byte chunks into LDS, then gathers a
 // block of 16 rows x 4 columns as sixteen dwords, transposes its four 4x4 byte blocks in registers (two
 // rounds of byte permutes) and stores, for each of its four columns, sixteen consecutive row bytes.
 // Three tile shapes: 128x128, 32x512 for few rows (NCHW -> NHWC with up to 32 channels) and 512x32 for few
@@ -109,6 +110,9 @@ __device__ __forceinline__ void transpose4x4_bytes(const uint32_t a0, const uint
     out[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
     out[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
 }
+
+// four dwords at a 4-byte aligned address (global memory takes a dwordx4 access at any dword boundary)
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 template <int TR, int TS>
 __global__ __launch_bounds__(256) void transpose_u8_wide_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
@@ -135,8 +139,18 @@ __global__ __launch_bounds__(256) void transpose_u8_wide_kernel(const uint8_t *_
     for (int it = 0; it < 4; ++it) {
         const int idx = t + 256 * it, row = idx / CPR, c = idx % CPR;
         const int gr = r0 + row, gs = s0 + 16 * c;
-        if (gr < R && gs < S)
-            *reinterpret_cast<uint4 *>(tile + lds_pos(row, c)) = *reinterpret_cast<const uint4 *>(src + (size_t)gr * S + gs);
+        if (gr < R && gs < S) {
+            const uint8_t *g = src + (size_t)gr * S + gs;
+            u32x4_a4 v = {0u, 0u, 0u, 0u};
+            if (gs + 16 <= S) {
+                v = *reinterpret_cast<const u32x4_a4 *>(g);
+            } else {  // the last chunk of a row whose length is a multiple of 4 only
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    if (gs + 4 * d < S) v[d] = *reinterpret_cast<const uint32_t *>(g + 4 * d);
+            }
+            *reinterpret_cast<uint4 *>(tile + lds_pos(row, c)) = make_uint4(v[0], v[1], v[2], v[3]);
+        }
     }
     __syncthreads();
     // this thread's block: rows 16*rg .. 16*rg+15, columns 4*cg .. 4*cg+3
@@ -164,14 +178,23 @@ __global__ __launch_bounds__(256) void transpose_u8_wide_kernel(const uint8_t *_
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int gs = s0 + 4 * cg + k;
-        if (gs < S) *reinterpret_cast<uint4 *>(dst + (size_t)gs * R + gr) = make_uint4(col[k][0], col[k][1], col[k][2], col[k][3]);
+        if (gs >= S) continue;
+        uint8_t *g = dst + (size_t)gs * R + gr;
+        if (gr + 16 <= R) {
+            const u32x4_a4 v = {col[k][0], col[k][1], col[k][2], col[k][3]};
+            *reinterpret_cast<u32x4_a4 *>(g) = v;
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (gr + 4 * q < R) *reinterpret_cast<uint32_t *>(g + 4 * q) = col[k][q];
+        }
     }
 }
 
 int launch_transpose(const uint8_t *src, uint8_t *dst, int32_t batch, int32_t R, int32_t S, hipStream_t stream) {
     if (batch <= 0 || R <= 0 || S <= 0) return EH_OK;
     EH_REQUIRE(batch <= 65535, "transpose: batch %d exceeds the grid limit", batch);
-    if (R % 16 == 0 && S % 16 == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0) {
+    if (R % 4 == 0 && S % 4 == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 3) == 0) {
         if (S <= 32 && (R + 511) / 512 <= 65535) {
             hipLaunchKernelGGL((transpose_u8_wide_kernel<512, 32>), dim3(1, (R + 511) / 512, batch), dim3(256), 0, stream, src, dst, R, S);
             EH_HIP(hipGetLastError());
