@@ -88,7 +88,10 @@ __device__ __forceinline__ void gather_c3k3(const GemmProblem &p, const uint32_t
 template <bool ROWSUM, bool FAST>
 __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p, const uint32_t in_bytes) {
     const int lane = threadIdx.x & 63, r = lane & 31, half = lane >> 5;
-    const int m_own = blockIdx.x * 256 + threadIdx.x;  // the pixel this lane gathers
+    // every XCD (workgroups are dispatched round-robin over the 8 of them) takes one contiguous eighth of the
+    // pixel range, so the input rows that neighbouring output rows share are fetched into one L2 only
+    const int block = (int)((blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3));
+    const int m_own = block * 256 + threadIdx.x;  // the pixel this lane gathers
     uint32_t A[7];
     gather_c3k3(p, in_bytes, m_own < p.m ? m_own : p.m - 1, A);
     if (m_own >= p.m) {
@@ -292,7 +295,7 @@ int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream) {
     const bool rowsum = p.zw != 0;
     bool fast = p.rq.fast != 0;
     if (p.n >= 32) {  // the packed rows and the folded bias are padded to whole tiles of channels
-        const dim3 grid_m((p.m + 255) / 256);
+        const dim3 grid_m(((p.m + 255) / 256 + 7) / 8 * 8);  // whole multiples of 8: see the kernel's block numbering
         if (rowsum && fast)
             hipLaunchKernelGGL((conv_c3k3_mfma_kernel<true, true>), grid_m, dim3(256), 0, stream, p, total_bytes);
         else if (rowsum)
