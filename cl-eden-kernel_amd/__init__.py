@@ -72,6 +72,8 @@ EXPORTS = {
     "eh_conv2d_u8_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(AddRequant),
                                        C.c_void_p]),
     "eh_conv2d_u8_fuses_add": (C.c_int, [C.c_void_p]),
+    "eh_conv2d_u8_kernels": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_int32]),
+    "eh_deconv2d_u8_kernels": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_int32]),
     "eh_conv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "eh_dwconv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "eh_deconv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
@@ -218,6 +220,19 @@ def conv_desc(n, c, h, w, cout, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1,
     """pad = (top, bottom, left, right)"""
     return ConvDesc(n, c, h, w, cout, kh, kw, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3],
                     dil[0], dil[1], groups, dm, layout, weight_layout)
+
+
+KERNEL_NAMES = ("staged", "dma_256x128", "dma_128x128", "dma_128x64", "dma_64x64_splitk", "dma_256x256", "one_tap", "c3k3")
+
+
+def conv_kernels(desc, deconv=False):
+    """Kernel family (a KERNEL_NAMES entry) per part of a convolution / deconvolution plan made from `desc`; no GPU."""
+    ids = (C.c_int32 * 64)()
+    fn = load().eh_deconv2d_u8_kernels if deconv else load().eh_conv2d_u8_kernels
+    count = fn(C.byref(desc), ids, 64)
+    if count < 0:
+        check(count)
+    return [KERNEL_NAMES[ids[i]] for i in range(min(count, 64))]
 
 
 class DeviceBuffer:

@@ -69,9 +69,14 @@ namespace {
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 inline int round_up(int v, int a) { return (v + a - 1) / a * a; }
 
+// Set while a descriptor is only being asked which kernels would serve it: geometry and kernel choice are
+// computed as for a plan, nothing is allocated or copied.
+static thread_local bool g_dry_run = false;
+
 template <typename T>
 int dev_alloc(T **p, size_t count) {
     *p = nullptr;
+    if (g_dry_run) return EH_OK;
     if (count == 0) count = 1;
     EH_HIP(hipMalloc(reinterpret_cast<void **>(p), count * sizeof(T)));
     return EH_OK;
@@ -120,7 +125,11 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     // the kernel shape is fixed here because the packed weight layout depends on it
     g.cfg = GemmConfig();
     if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 &&
-        igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base, g.proto.m, g.n)) {
+        igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base, g.proto.m, g.n) &&
+        // the one-tap kernel does not test its pixel against the image: every output pixel's tap must lie inside
+        // (bottom / right padding of a 1x1 convolution, or a deconvolution phase enlarged by a negative tail padding,
+        // go to the kernels that do)
+        (g.proto.ho - 1) * g.proto.stride_h < g.proto.h && (g.proto.wo - 1) * g.proto.stride_w < g.proto.w) {
         g.cfg.id = GEMM_THIN;
         g.cfg.slab = 32;
     } else if (g.cin == 3 && g.proto.cin == 3 && g.taps == 9 && g.k == 27 && units.size() == 27 && units[26].dy == 2 &&
@@ -143,11 +152,13 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     if ((rc = dev_alloc(&g.folded, (size_t)g.n_pad))) return rc;
     if ((rc = dev_alloc(&g.ktab, units.size()))) return rc;
     if ((rc = dev_alloc(&g.tap_off, tap_off.size()))) return rc;
-    EH_HIP(hipMemcpyAsync(g.ktab, units.data(), units.size() * sizeof(KUnit), hipMemcpyHostToDevice, stream));
-    if (!tap_off.empty())
-        EH_HIP(hipMemcpyAsync(g.tap_off, tap_off.data(), tap_off.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream));
-    // the host vectors die with the caller's frame: make sure the copies have left them
-    EH_HIP(hipStreamSynchronize(stream));
+    if (!g_dry_run) {
+        EH_HIP(hipMemcpyAsync(g.ktab, units.data(), units.size() * sizeof(KUnit), hipMemcpyHostToDevice, stream));
+        if (!tap_off.empty())
+            EH_HIP(hipMemcpyAsync(g.tap_off, tap_off.data(), tap_off.size() * sizeof(int32_t), hipMemcpyHostToDevice, stream));
+        // the host vectors die with the caller's frame: make sure the copies have left them
+        EH_HIP(hipStreamSynchronize(stream));
+    }
     g.proto.ktab = g.ktab;
     g.proto.a_offset = units.empty() ? 0 : units[0].offset;
     g.proto.k = g.k;
@@ -784,19 +795,15 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
     return EH_OK;
 }
 
-int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
-                      const eh_requant *q, void *stream) {
-    EH_REQUIRE(plan != nullptr, "null plan pointer");
-    *plan = nullptr;
+// `desc` with the two flag bits taken out, checked
+static int conv_desc_checked(const eh_conv_desc *desc, eh_conv_desc *plain) {
     EH_REQUIRE(desc != nullptr, "descriptor is null");
-    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
-    eh_conv_desc plain = *desc;
-    plain.weight_layout &= ~EH_W_SIGNED;
-    plain.layout &= ~EH_IO_SIGNED;
-    desc = &plain;
+    *plain = *desc;
+    plain->weight_layout &= ~EH_W_SIGNED;
+    plain->layout &= ~EH_IO_SIGNED;
+    desc = plain;
     int rc = check_desc_common(desc);
     if (rc) return rc;
-    if ((rc = check_requant(q, w_signed, io_signed))) return rc;
     EH_REQUIRE(desc->dil_h > 0 && desc->dil_w > 0, "bad dilation");
     EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
                "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
@@ -804,6 +811,38 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
                desc->weight_layout);
     EH_REQUIRE(desc->weight_layout == EH_W_OIHW || desc->groups == 1, "OHWI weights support groups == 1 only");
     EH_REQUIRE(desc->kh * desc->dil_h < 32000 && desc->kw * desc->dil_w < 32000, "kernel extent too large");
+    return EH_OK;
+}
+
+static int report_kernels(const GemmOp &op, int32_t *kernel_ids, int32_t cap) {
+    for (size_t i = 0; i < op.parts.size() && (int32_t)i < cap; ++i) kernel_ids[i] = op.parts[i].cfg.id;
+    return (int)op.parts.size();
+}
+
+int eh_conv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_t cap) {
+    EH_REQUIRE(kernel_ids != nullptr || cap == 0, "null result array");
+    eh_conv_desc plain;
+    int rc = conv_desc_checked(desc, &plain);
+    if (rc) return rc;
+    if (plain.n == 0) return 0;
+    eh_conv_plan pl;
+    g_dry_run = true;
+    rc = conv_plan_build(&pl, &plain, nullptr);
+    g_dry_run = false;
+    return rc ? rc : report_kernels(pl.op, kernel_ids, cap);
+}
+
+int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
+                      const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan pointer");
+    *plan = nullptr;
+    EH_REQUIRE(desc != nullptr, "descriptor is null");
+    const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
+    eh_conv_desc plain;
+    int rc = conv_desc_checked(desc, &plain);
+    if (rc) return rc;
+    desc = &plain;
+    if ((rc = check_requant(q, w_signed, io_signed))) return rc;
     eh_conv_plan *pl = new (std::nothrow) eh_conv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
@@ -1071,24 +1110,46 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
     return EH_OK;
 }
 
+static int deconv_desc_checked(const eh_conv_desc *desc, eh_conv_desc *plain) {
+    EH_REQUIRE(desc != nullptr, "descriptor is null");
+    *plain = *desc;
+    plain->weight_layout &= ~EH_W_SIGNED;
+    plain->layout &= ~EH_IO_SIGNED;
+    desc = plain;
+    int rc = check_desc_common(desc, true);
+    if (rc) return rc;
+    EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
+               "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
+    EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->weight_layout == EH_W_OHWI, "bad deconvolution weight layout %d",
+               desc->weight_layout);
+    EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->groups == 1, "OHWI weights support groups == 1 only");
+    return EH_OK;
+}
+
+int eh_deconv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_t cap) {
+    EH_REQUIRE(kernel_ids != nullptr || cap == 0, "null result array");
+    eh_conv_desc plain;
+    int rc = deconv_desc_checked(desc, &plain);
+    if (rc) return rc;
+    if (plain.n == 0) return 0;
+    eh_deconv_plan pl;
+    g_dry_run = true;
+    rc = deconv_plan_build(&pl, &plain, nullptr);
+    g_dry_run = false;
+    return rc ? rc : report_kernels(pl.op, kernel_ids, cap);
+}
+
 int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
                         const eh_requant *q, void *stream) {
     EH_REQUIRE(plan != nullptr, "null plan pointer");
     *plan = nullptr;
     EH_REQUIRE(desc != nullptr, "descriptor is null");
     const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
-    eh_conv_desc plain = *desc;
-    plain.weight_layout &= ~EH_W_SIGNED;
-    plain.layout &= ~EH_IO_SIGNED;
-    desc = &plain;
-    int rc = check_desc_common(desc, true);
+    eh_conv_desc plain;
+    int rc = deconv_desc_checked(desc, &plain);
     if (rc) return rc;
+    desc = &plain;
     if ((rc = check_requant(q, w_signed, io_signed))) return rc;
-    EH_REQUIRE(desc->groups > 0 && desc->c % desc->groups == 0 && desc->cout % desc->groups == 0,
-               "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
-    EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->weight_layout == EH_W_OHWI, "bad deconvolution weight layout %d",
-               desc->weight_layout);
-    EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->groups == 1, "OHWI weights support groups == 1 only");
     eh_deconv_plan *pl = new (std::nothrow) eh_deconv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;

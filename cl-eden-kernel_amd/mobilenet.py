@@ -8,9 +8,13 @@ OperationExecutor pair (src/userdriver/gpu/gpu_op_constructor.cc:1797-1850,
 gpu_userdriver.cc:78-112): build every operator once, then execute them in
 order on one stream, here captured into one HIP graph.
 
-Weights are random (there is no checkpoint): uint8 clip(round(N(zp_w, 20)))
-with a per-layer weight zero point, int32 uniform bias.  Scales are chosen
-analytically from the layer shapes so that activations neither die nor saturate
+Weights are random (there is no checkpoint).  The default form ("minmax") is
+what a post-training quantizer makes of random-init float weights: a zero-mean
+normal field per tensor, its minimum mapped to byte 0 and its maximum to byte
+255, the zero point where real 0 falls, so the bytes of every tensor span
+0 .. 255.  The "narrow" form (uint8 clip(round(N(zp_w, 20))) with a per-layer
+zero point, every byte within int8 reach of its zero point) is kept as a
+labelled extra.  Bias is int32 uniform.  Scales are chosen analytically from the layer shapes so that activations neither die nor saturate
 on their way through the 53 convolutions:
   * a ReLU6 output tensor has zero point 0 and scale 6/255, so ReLU6 is the
     whole uint8 range, and the layer's weight scale is set so that the
@@ -20,6 +24,7 @@ on their way through the 53 convolutions:
   * a residual sum is rescaled back to about 30 steps.
 `layers()` is pure data (no GPU): tests evaluate the same list with the oracle.
 """
+import functools
 import math
 
 import numpy as np
@@ -31,7 +36,8 @@ SEED = 0xEDE2 + 16 * 5
 # (expansion t, output channels c, repeats n, stride s)
 BOTTLENECKS = ((1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1))
 
-W_SD = 20                 # standard deviation of the weight bytes around their zero point
+W_SD = 20                 # "narrow" weights: standard deviation of the weight bytes around their zero point
+FIELD_SD = 65535          # standard deviation of the integer normal field the "minmax" weights are quantized from
 RELU6_SCALE = 6.0 / 255   # ReLU6 == [0, 255] at zero point 0
 RELU_RMS = 45.0           # root mean square of clip(N(0, 64), 0, 255)
 LINEAR_SD = 30.0
@@ -39,11 +45,32 @@ INPUT_SCALE, INPUT_ZP = 0.02, 128
 INPUT_RMS = 74.0          # of uniform bytes around 128
 
 
-def layers(image=224):
+@functools.lru_cache(maxsize=None)
+def _field_extremes(shape, seed):
+    g = synth.fill_normal_field(shape, seed)
+    return int(g.min()), int(g.max())
+
+
+def _minmax_bytes(g, lo, hi):
+    """round((g - lo) * 255 / (hi - lo)) in integer arithmetic"""
+    span = hi - lo
+    return ((2 * 255 * (g - lo) + span) // (2 * span)).astype(np.uint8)
+
+
+def layers(image=224, weights="minmax"):
     """The operator list.  Tensors are numbered; tensor 0 is the network input.  Returns
-    (tensors, ops): tensors[i] = dict(h, w, c, scale, zp, rms), ops = list of dicts."""
+    (tensors, ops): tensors[i] = dict(h, w, c, scale, zp, rms), ops = list of dicts.
+    weights: "minmax" (per-tensor min/max quantized, bytes span 0 .. 255) or "narrow"."""
+    assert weights in ("minmax", "narrow")
     tensors = [dict(h=image, w=image, c=3, scale=INPUT_SCALE, zp=INPUT_ZP, rms=INPUT_RMS)]
     ops = []
+
+    def weight_stats(shape, seed, narrow_zp):
+        """(zero point, standard deviation of the bytes around it) of an operator's weight tensor"""
+        if weights == "narrow":
+            return narrow_zp, float(W_SD)
+        lo, hi = _field_extremes(shape, seed)
+        return int((2 * 255 * (0 - lo) + (hi - lo)) // (2 * (hi - lo))), FIELD_SD * 255.0 / (hi - lo)
 
     def conv(src, cout, k, stride, relu6, depthwise=False):
         t = tensors[src]
@@ -51,7 +78,9 @@ def layers(image=224):
         pad = (k - 1) // 2
         ho, wo = (t["h"] + 2 * pad - k) // stride + 1, (t["w"] + 2 * pad - k) // stride + 1
         fan_in = k * k * (1 if depthwise else t["c"])
-        acc_sd = math.sqrt(fan_in) * W_SD * t["rms"]
+        w_seed = SEED + 3 * idx
+        w_zp, w_sd = weight_stats((cout, 1 if depthwise else t["c"], k, k), w_seed, 120 + idx % 16)
+        acc_sd = math.sqrt(fan_in) * w_sd * t["rms"]
         if relu6:
             out_scale, out_zp, out_sd, out_rms = RELU6_SCALE, 0, 64.0, RELU_RMS
         else:
@@ -59,7 +88,7 @@ def layers(image=224):
         w_scale = (out_sd / acc_sd) * out_scale / t["scale"]
         tensors.append(dict(h=ho, w=wo, c=cout, scale=out_scale, zp=out_zp, rms=out_rms))
         ops.append(dict(op="dw" if depthwise else "conv", src=src, dst=len(tensors) - 1, k=k, stride=stride, pad=pad,
-                        cout=cout, relu6=relu6, w_scale=w_scale, w_zp=120 + idx % 16, w_seed=SEED + 3 * idx,
+                        cout=cout, relu6=relu6, w_scale=w_scale, w_zp=w_zp, w_seed=w_seed, w_mode=weights,
                         b_seed=SEED + 3 * idx + 1, b_range=max(1, int(acc_sd / 4))))
         return len(tensors) - 1
 
@@ -87,10 +116,11 @@ def layers(image=224):
     cur = len(tensors) - 1
     t = tensors[cur]
     idx = len(ops)
-    acc_sd = math.sqrt(t["c"]) * W_SD * t["rms"]
+    w_zp, w_sd = weight_stats((1000, t["c"]), SEED + 3 * idx, 128)
+    acc_sd = math.sqrt(t["c"]) * w_sd * t["rms"]
     tensors.append(dict(h=1, w=1, c=1000, scale=0.05, zp=128, rms=LINEAR_SD))
     ops.append(dict(op="fc", src=cur, dst=len(tensors) - 1, cout=1000, w_scale=(LINEAR_SD / acc_sd) * 0.05 / t["scale"],
-                    w_zp=128, w_seed=SEED + 3 * idx, b_seed=SEED + 3 * idx + 1, b_range=max(1, int(acc_sd / 4))))
+                    w_zp=w_zp, w_seed=SEED + 3 * idx, w_mode=weights, b_seed=SEED + 3 * idx + 1, b_range=max(1, int(acc_sd / 4))))
     return tensors, ops
 
 
@@ -102,18 +132,31 @@ def op_weights(op, cin):
         shape = (op["cout"], 1, op["k"], op["k"])
     else:
         shape = (op["cout"], cin, op["k"], op["k"])
-    w = synth.fill_u8_normal(shape, op["w_seed"], op["w_zp"], W_SD)
+    if op["w_mode"] == "minmax":
+        w = _minmax_bytes(synth.fill_normal_field(shape, op["w_seed"]), *_field_extremes(shape, op["w_seed"]))
+    else:
+        w = synth.fill_u8_normal(shape, op["w_seed"], op["w_zp"], W_SD)
     b = synth.fill_i32((op["cout"],), op["b_seed"], -op["b_range"], op["b_range"])
     return w, b
 
 
 def op_weights_perchannel(op, cin):
     """(int8 weights, bias, float32 scale per output channel) of a conv / dw operator in the per-channel form
-    (int8 weights at zero point 0, as TFLite's full-integer converter writes them): clip(round(N(0, 20))) and the
-    layer's weight scale times a factor in [0.5, 2] per channel."""
+    (int8 weights at zero point 0, as TFLite's full-integer converter writes them).  "minmax": the operator's normal
+    field with every channel's largest magnitude mapped to 127 (bytes span -127 .. 127 in every channel), the
+    channel's scale following from it.  "narrow": clip(round(N(0, 20))) and the layer's weight scale times a factor
+    in [0.5, 2] per channel."""
     shape = (op["cout"], 1 if op["op"] == "dw" else cin, op["k"], op["k"])
-    w = (synth.fill_u8_normal(shape, op["w_seed"], 128, W_SD).astype(np.int16) - 128).clip(-127, 127).astype(np.int8)
     b = synth.fill_i32((op["cout"],), op["b_seed"], -op["b_range"], op["b_range"])
+    if op["w_mode"] == "minmax":
+        g = synth.fill_normal_field(shape, op["w_seed"]).reshape(op["cout"], -1)
+        top = np.maximum(np.abs(g).max(axis=1, keepdims=True), 1)
+        num = 2 * 127 * np.abs(g) + top
+        w = (np.sign(g) * (num // (2 * top))).astype(np.int8).reshape(shape)
+        lo, hi = _field_extremes(shape, op["w_seed"])
+        field_step = op["w_scale"] * 255.0 / (hi - lo)   # real value of one unit of the field
+        return w, b, (top.reshape(-1).astype(np.float64) * field_step / 127.0).astype(np.float32)
+    w = (synth.fill_u8_normal(shape, op["w_seed"], 128, W_SD).astype(np.int16) - 128).clip(-127, 127).astype(np.int8)
     factor = 0.5 + 1.5 * synth.fill_u8((op["cout"],), op["w_seed"] + 2).astype(np.float32) / 255.0
     return w, b, (np.float32(op["w_scale"]) * factor).astype(np.float32)
 
@@ -156,9 +199,9 @@ class MobileNetV2:
     per_channel: convolutions and depthwise convolutions take int8 weights with one scale per output channel
     (`op_weights_perchannel`); tensors stay uint8 and the classifier keeps its per-tensor uint8 weights."""
 
-    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False, per_channel=False):
+    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False, per_channel=False, weights="minmax"):
         self.eden, self.batch, self.image = eden, batch, image
-        self.tensors, self.ops = layers(image)
+        self.tensors, self.ops = layers(image, weights)
         self.buffers = [eden.DeviceBuffer(nbytes=batch * t["h"] * t["w"] * t["c"]) for t in self.tensors]
         self.steps = []
         self._keep = []

@@ -28,6 +28,17 @@ def fill_i32(shape, seed, lo, hi):
     return (r.astype(np.int64) + lo).astype(np.int32).reshape(shape)
 
 
+def fill_normal_field(shape, seed):
+    """int64 values close to N(0, 65535): a 12-term Irwin-Hall sum of 16-bit uniforms, centred (what float weights
+    drawn from a normal distribution look like before a quantizer sees them, in integer arithmetic)"""
+    count = int(np.prod(shape))
+    r = splitmix64(seed, count * 3).reshape(count, 3)
+    total = np.zeros(count, np.int64)
+    for sh in (0, 16, 32, 48):
+        total += ((r >> np.uint64(sh)) & np.uint64(0xFFFF)).astype(np.int64).sum(axis=1)
+    return (total - 6 * 65535).reshape(shape)
+
+
 def fill_u8_normal(shape, seed, mean, sd):
     """clip(round(N(mean, sd)), 0, 255): a 12-term Irwin-Hall sum of 16-bit uniforms in integer arithmetic."""
     count = int(np.prod(shape))

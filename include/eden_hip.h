@@ -232,6 +232,22 @@ typedef struct eh_deconv_plan eh_deconv_plan;
  * CLQuantizedDirectConvolution.cpp:30-249) and their kernels. */
 int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void *weight, const void *bias,
                       const eh_requant *q, void *stream);
+/* Which kernel family a plan made from `desc` would run, one eh_kernel_id per part (convolution group;
+ * deconvolution output phase and group), without a GPU: the choice CLConvolution::initialize makes among its
+ * implementations (gpu/operators/CLConvolution.cpp:139-218).  Writes at most `cap` ids, returns the number of
+ * parts or a negative eh_status. */
+typedef enum eh_kernel_id {
+    EH_KERNEL_STAGED = 0,         /* register-staged implicit GEMM, any channel count               */
+    EH_KERNEL_DMA_256x128 = 1,    /* direct-to-LDS implicit GEMM tiles                              */
+    EH_KERNEL_DMA_128x128 = 2,
+    EH_KERNEL_DMA_128x64 = 3,
+    EH_KERNEL_DMA_64x64_SPLITK = 4,
+    EH_KERNEL_DMA_256x256 = 5,
+    EH_KERNEL_ONE_TAP = 6,        /* 1x1 problems with short reductions or few pixels               */
+    EH_KERNEL_C3K3 = 7            /* 3x3 on three input channels (first layers)                     */
+} eh_kernel_id;
+int eh_conv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_t cap);
+int eh_deconv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_t cap);
 /* Per-channel mode (conv_per_channel_quantized, gpu/operators/cl_kernels/ConvolutionKernels.cpp:1317-1375):
  * `count` == cout host arrays of multipliers and shifts replace the requant's single pair on every
  * following run; two null pointers return to per-tensor mode.  Copies synchronously. */

@@ -121,3 +121,23 @@ def test_synthetic_generators_match_the_c_harness():
     a = synth.fill_u8_normal((50000,), 0xEDE4, 128, 20)
     assert np.array_equal(a, O.fill_u8_normal((50000,), 0xEDE4, 128, 20))
     assert abs(a.mean() - 128) < 0.5 and abs(a.std() - 20) < 0.5
+
+
+def test_one_tap_kernel_is_only_chosen_when_every_tap_lies_inside_the_image():
+    """The one-tap kernel does not test its pixel against the image, so a 1x1 convolution with bottom / right padding
+    and a deconvolution phase that a negative tail padding enlarges beyond the input must go to other kernels."""
+    nhwc = eden.NHWC
+    assert eden.conv_kernels(eden.conv_desc(2, 24, 14, 14, 144, 1, 1, layout=nhwc)) == ["one_tap"]
+    assert eden.conv_kernels(eden.conv_desc(2, 24, 14, 14, 144, 1, 1, stride=(2, 2), layout=nhwc)) == ["one_tap"]
+    for pad in ((0, 1, 0, 0), (0, 0, 0, 1), (0, 1, 0, 1), (0, 3, 0, 2)):
+        got = eden.conv_kernels(eden.conv_desc(2, 24, 14, 14, 144, 1, 1, pad=pad, layout=nhwc))
+        assert got != ["one_tap"], (pad, got)
+    # top / left padding never qualified (the tap of the first pixel lies outside)
+    assert eden.conv_kernels(eden.conv_desc(2, 24, 14, 14, 144, 1, 1, pad=(1, 0, 0, 0), layout=nhwc)) != ["one_tap"]
+    # stride 2 over an odd extent with one row of bottom padding: the last output row reads row 14 of 14
+    assert eden.conv_kernels(eden.conv_desc(1, 16, 13, 13, 32, 1, 1, stride=(2, 2), pad=(0, 2, 0, 2), layout=nhwc)) != ["one_tap"]
+    # transposed convolution, kernel <= stride: every phase is one tap
+    d = eden.conv_desc(1, 16, 6, 6, 32, 2, 2, stride=(2, 2), layout=nhwc, weight_layout=eden.W_IOHW)
+    assert eden.conv_kernels(d, deconv=True) == ["one_tap"] * 4
+    d = eden.conv_desc(1, 16, 6, 6, 32, 2, 2, stride=(2, 2), pad=(0, -2, 0, -2), layout=nhwc, weight_layout=eden.W_IOHW)
+    assert "one_tap" not in eden.conv_kernels(d, deconv=True)

@@ -1,5 +1,7 @@
-"""MobileNetV2-1.0 uint8 (BASELINE configs[4] at a small batch): every operator of the GPU operator list against
-the oracle evaluating the same list, bit-exact tensor by tensor."""
+"""MobileNetV2-1.0 uint8 (BASELINE configs[4]): every operator of the GPU operator list against the oracle
+evaluating the same list, bit-exact tensor by tensor, at small batches directly and at the full batch of 64 on an
+input made of an oracle-evaluated pair of images repeated 32 times."""
+import functools
 import importlib
 
 import numpy as np
@@ -13,9 +15,9 @@ mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
 pytestmark = pytest.mark.gpu
 
 
-def oracle_forward(x_nhwc, image, per_channel=False):
+def oracle_forward(x_nhwc, image, per_channel=False, weights="minmax"):
     """All tensors of the network, NCHW, computed by the oracle from the same operator list."""
-    tensors, ops = mobilenet.layers(image)
+    tensors, ops = mobilenet.layers(image, weights)
     vals = [np.ascontiguousarray(x_nhwc.transpose(0, 3, 1, 2))]
     n = x_nhwc.shape[0]
     for op in ops:
@@ -57,13 +59,30 @@ def oracle_forward(x_nhwc, image, per_channel=False):
     return tensors, ops, vals
 
 
+def assert_network_alive(ops, want, batch):
+    """no operator's output has collapsed to a constant or to the clamps"""
+    for op in ops:
+        v = want[op["dst"]]
+        assert v.std() > 8, (op["op"], op["dst"], float(v.std()))
+        assert np.mean((v == 0) | (v == 255)) < 0.8, (op["op"], op["dst"])
+    logits = want[-1].reshape(batch, -1)
+    assert len(np.unique(logits)) > 40
+    assert not np.array_equal(logits[0], logits[1])
+
+
+@pytest.mark.parametrize("weights", ["minmax", "narrow"])
 @pytest.mark.parametrize("fuse_add", [False, True], ids=["separate_adds", "fused_adds"])
 @pytest.mark.parametrize("batch,image", [(2, 224), (3, 96)])
-def test_mobilenet_v2_matches_oracle_tensor_by_tensor(batch, image, fuse_add):
-    print("mobilenet", batch, image, fuse_add, flush=True)
+def test_mobilenet_v2_matches_oracle_tensor_by_tensor(batch, image, fuse_add, weights):
+    print("mobilenet", batch, image, fuse_add, weights, flush=True)
     x = mobilenet.network_input(batch, image)
-    tensors, ops, want = oracle_forward(x, image)
-    net = mobilenet.MobileNetV2(eden, batch, image, fuse_add=fuse_add)
+    tensors, ops, want = oracle_forward(x, image, weights=weights)
+    if weights == "minmax":  # per-tensor min/max quantized: every weight tensor uses the whole byte range
+        for op in ops:
+            if "w_seed" in op:
+                w, _ = mobilenet.op_weights(op, tensors[op["src"]]["c"])
+                assert (w.min(), w.max()) == (0, 255)
+    net = mobilenet.MobileNetV2(eden, batch, image, fuse_add=fuse_add, weights=weights)
     net.set_input(x)
     net.run()
     eden.sync()
@@ -74,14 +93,39 @@ def test_mobilenet_v2_matches_oracle_tensor_by_tensor(batch, image, fuse_add):
             continue
         got = net.tensor(i).transpose(0, 3, 1, 2)
         assert np.array_equal(got, want[i]), (op["op"], i, tensors[i], int((got != want[i]).sum()))
-    logits = want[-1].reshape(batch, -1)
-    # the network is alive: no operator's output has collapsed to a constant or to the clamps
+    assert_network_alive(ops, want, batch)
+
+
+@functools.lru_cache(maxsize=None)
+def oracle_pair(per_channel, weights):
+    return oracle_forward(mobilenet.network_input(2), 224, per_channel, weights)
+
+
+@pytest.mark.parametrize("per_channel,weights", [(False, "minmax"), (False, "narrow"), (True, "minmax")],
+                         ids=["per_tensor_minmax", "per_tensor_narrow", "per_channel_minmax"])
+def test_mobilenet_v2_full_batch_64(per_channel, weights):
+    """The network exactly as the benchmark builds it (batch 64, which decides tile shapes, grids and the depthwise
+    tile width) on 32 repetitions of a pair of images: every tensor of every image must equal the oracle's tensor
+    for that image of the pair."""
+    print("mobilenet batch 64", per_channel, weights, flush=True)
+    batch = 64
+    tensors, ops, want = oracle_pair(per_channel, weights)
+    x = np.tile(mobilenet.network_input(2), (batch // 2, 1, 1, 1))
+    net = mobilenet.MobileNetV2(eden, batch, 224, fuse_add=True, per_channel=per_channel, weights=weights)
+    net.set_input(x)
+    stream = eden.Stream()
+    graph = eden.Graph(stream, lambda s: net.run(s))   # as the benchmark launches it
+    graph.launch(stream)
+    stream.sync()
     for op in ops:
-        v = want[op["dst"]]
-        assert v.std() > 8, (op["op"], op["dst"], float(v.std()))
-        assert np.mean((v == 0) | (v == 255)) < 0.8, (op["op"], op["dst"])
-    assert len(np.unique(logits)) > 40
-    assert not np.array_equal(logits[0], logits[1])
+        i = op["dst"]
+        if i in net.unwritten:
+            continue
+        got = net.tensor(i).transpose(0, 3, 1, 2)
+        pair = want[i]
+        for img in range(batch):
+            assert np.array_equal(got[img], pair[img % 2]), (op["op"], i, img, tensors[i], int((got[img] != pair[img % 2]).sum()))
+    assert_network_alive(ops, want, 2)
 
 
 def test_mobilenet_v2_graph_replay_equals_eager():
@@ -124,9 +168,4 @@ def test_mobilenet_v2_per_channel_weights_matches_oracle_tensor_by_tensor(batch,
             continue
         got = net.tensor(i).transpose(0, 3, 1, 2)
         assert np.array_equal(got, want[i]), (op["op"], i, tensors[i], int((got != want[i]).sum()))
-    for op in ops:
-        v = want[op["dst"]]
-        assert v.std() > 8, (op["op"], op["dst"], float(v.std()))
-        assert np.mean((v == 0) | (v == 255)) < 0.8, (op["op"], op["dst"])
-    logits = want[-1].reshape(batch, -1)
-    assert len(np.unique(logits)) > 40 and not np.array_equal(logits[0], logits[1])
+    assert_network_alive(ops, want, batch)

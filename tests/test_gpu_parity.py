@@ -187,6 +187,10 @@ CONV_CASES = [
     dict(n=2, c=64, h=12, w=12, cout=32, kh=1, kw=1),
     dict(n=1, c=48, h=10, w=10, cout=96, kh=1, kw=1, groups=2),                             # 24-byte rows inside 48-byte pixels
     dict(n=5, c=16, h=33, w=5, cout=96, kh=1, kw=1, stride=(1, 2)),
+    # one tap with bottom / right padding: output pixels whose only tap lies outside the image (they read the zero
+    # point); the one-tap kernel must not be chosen
+    dict(n=2, c=24, h=14, w=14, cout=144, kh=1, kw=1, pad=(0, 1, 0, 1)),
+    dict(n=3, c=16, h=13, w=13, cout=32, kh=1, kw=1, stride=(2, 2), pad=(0, 2, 0, 2)),
     # three channels, 3x3: the first-layer kernel (unaligned 12-byte reads; byte path at the two ends of the tensor)
     dict(n=2, c=3, h=32, w=32, cout=32, kh=3, kw=3, stride=(2, 2), pad=(1, 1, 1, 1)),
     dict(n=1, c=3, h=9, w=10, cout=20, kh=3, kw=3, pad=(1, 1, 1, 1)),
@@ -420,9 +424,11 @@ def test_depthwise_reference_kat_on_gpu(kat):
         assert got.reshape(-1).tolist() == [e + zp_out for e in kat["expect"]]
 
 
-def test_mobilenet_block_config3():
-    """Pointwise 24->144 (ReLU6) then depthwise 3x3 s2 p1 (ReLU6), channels-last, zero points drawn from the seed."""
-    n = 4
+@pytest.mark.parametrize("n", [4, 32], ids=["n4", "n32_full_size"])
+def test_mobilenet_block_config3(n):
+    """Pointwise 24->144 (ReLU6) then depthwise 3x3 s2 p1 (ReLU6), channels-last, zero points drawn from the seed;
+    n = 32 is the benchmark's own size (the batch decides tile shapes and the depthwise tile width)."""
+    print("config 3 block, n =", n, flush=True)
     zps = synth.fill_u8((6,), SEED + 16 * 3 + 9).tolist()
     x = synth.fill_u8((n, 24, 56, 56), SEED + 16 * 3)
     w1 = synth.fill_u8((144, 24, 1, 1), SEED + 16 * 3 + 1)
@@ -451,6 +457,9 @@ DECONV_CASES = [
     dict(n=1, c=32, h=6, w=6, cout=40, kh=3, kw=3, stride=(2, 2), pad=(0, 0, 0, 0)),       # kernel not a multiple of stride
     dict(n=1, c=16, h=4, w=4, cout=16, kh=2, kw=2, stride=(3, 3), pad=(0, 0, 0, 0)),       # phases without any tap
     dict(n=1, c=8, h=3, w=3, cout=8, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),
+    # kernel <= stride (every phase is one tap) with a negative tail padding: phases larger than the input
+    dict(n=2, c=16, h=6, w=6, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, -2, 0, -2)),
+    dict(n=2, c=16, h=6, w=6, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, 0, 0, 0)),
 ]
 
 

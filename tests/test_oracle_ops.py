@@ -324,6 +324,52 @@ def test_add_closed_forms():
     assert O.add(np.array([4, 5, 7], np.uint8), np.array([2, 2, 2], np.uint8), q2).tolist() == [3, 4, 5]
 
 
+ADD_UNEQUAL = [
+    # scale_a, zp_a, scale_b, zp_b, scale_out, zp_out
+    (0.047, 128, 0.0213, 100, 0.0611, 120),
+    (0.013, 7, 0.11, 201, 0.09, 64),
+    (0.4, 90, 0.031, 33, 0.45, 128),
+]
+
+
+@pytest.mark.parametrize("params", ADD_UNEQUAL, ids=lambda p: "sa%g_sb%g_so%g" % (p[0], p[2], p[4]))
+def test_add_unequal_scales_against_exact_rational_arithmetic(params):
+    """All 65,536 byte pairs: the three-multiplier fixed-point add stays within one step of the exactly rounded real
+    sum round((s_a (a - zp_a) + s_b (b - zp_b)) / s_out) + zp_out, equals it in at least 99 % of the pairs away from
+    the clamps, and an add with the two input multipliers exchanged (the mistake this test exists for) does not."""
+    from fractions import Fraction
+    s_a, zp_a, s_b, zp_b, s_out, zp_out = params
+    q = O.make_add_quant(s_a, zp_a, s_b, zp_b, s_out, zp_out)
+    a, b = np.meshgrid(np.arange(256, dtype=np.uint8), np.arange(256, dtype=np.uint8), indexing="ij")
+    got = O.add(a, b, q).astype(np.int64)
+    # exact: the float32 scales as rationals, rounding half away from zero
+    fa, fb, fo = (Fraction(float(np.float32(v))) for v in (s_a, s_b, s_out))
+    ra, rb = fa / fo, fb / fo
+    den = (ra.denominator * rb.denominator)
+    num = (a.astype(object) - zp_a) * (ra.numerator * rb.denominator) + (b.astype(object) - zp_b) * (rb.numerator * ra.denominator)  # Python integers
+    exact = np.array([[(abs(int(v)) * 2 + den) // (2 * den) * (1 if v >= 0 else -1) for v in row] for row in num], dtype=np.int64) + zp_out
+    inside = (exact > 0) & (exact < 255)
+    assert inside.mean() > 0.3                      # the case exercises the arithmetic, not the clamps
+    err = np.abs(got - np.clip(exact, 0, 255))
+    assert err.max() <= 1
+    assert (err[inside] == 0).mean() >= 0.99
+
+    # the mutant: multipliers (and shifts) of the two inputs exchanged
+    m = O.AddQuant()
+    for f, _ in O.AddQuant._fields_:
+        setattr(m, f, getattr(q, f))
+    m.mult_a, m.mult_b, m.shift_a, m.shift_b = q.mult_b, q.mult_a, q.shift_b, q.shift_a
+    bad = np.abs(O.add(a, b, m).astype(np.int64) - np.clip(exact, 0, 255))
+    assert bad.max() > 1 and (bad[inside] == 0).mean() < 0.9
+    # a second mutant: one more right shift on both inputs
+    m2 = O.AddQuant()
+    for f, _ in O.AddQuant._fields_:
+        setattr(m2, f, getattr(q, f))
+    m2.shift_a, m2.shift_b = q.shift_a - 1, q.shift_b - 1
+    bad2 = np.abs(O.add(a, b, m2).astype(np.int64) - np.clip(exact, 0, 255))
+    assert bad2.max() > 1
+
+
 def test_avgpool_closed_forms():
     """parity unpinned by reference vectors: (sum + n/2) / n over the clipped window."""
     x = np.arange(16, dtype=np.uint8).reshape(1, 1, 4, 4)
