@@ -72,6 +72,7 @@ EXPORTS = {
     "eh_conv2d_u8_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(AddRequant),
                                        C.c_void_p]),
     "eh_conv2d_u8_fuses_add": (C.c_int, [C.c_void_p]),
+    "eh_conv2d_u8_run_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
     "eh_conv2d_u8_kernels": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_int32]),
     "eh_deconv2d_u8_kernels": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_int32]),
     "eh_conv2d_u8_set_perchannel": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
@@ -334,6 +335,13 @@ def _conv_run_add(self, d_in, d_residual, d_out, q, aq, stream=None):
     check(load().eh_conv2d_u8_run_add(self.handle, d_in.ptr, d_residual.ptr, d_out.ptr, C.byref(q), C.byref(aq), stream))
 
 
+def _conv_run_static(self, d_in, d_out, q, stream=None):
+    """ConvPlan.run through the entry point that allocates nothing (planar plans stage in the library's static scratch)"""
+    check(load().eh_conv2d_u8_run_static(self.handle, d_in.ptr, d_out.ptr, C.byref(q), stream))
+
+
+STATIC_SCRATCH_BYTES = 32 << 20
+ConvPlan.run_static = _conv_run_static
 ConvPlan.run_add = _conv_run_add
 ConvPlan.fuses_add = lambda self: bool(load().eh_conv2d_u8_fuses_add(self.handle))
 

@@ -28,6 +28,31 @@ int hip_fail(hipError_t e, const char *what) {
     return EH_DEVICE_FAILURE;
 }
 
+// ------------------------------------------------------------------ static scratch
+// Device memory for the entry point that may not allocate (eh_conv2d_u8_run_static): one array per GPU, part of the
+// code object, held from the moment the library is loaded on a device until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; `static_scratch` asks once per device, with that device
+// current, and every later use (kernel arguments, copies) goes through the address it keeps.
+static __device__ __align__(256) uint8_t scratch[EH_STATIC_SCRATCH_BYTES];
+static constexpr int kMaxDevices = 64;
+static uint8_t *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until asked
+
+static int static_scratch(uint8_t **ptr) {
+    int dev = -1;
+    EH_HIP(hipGetDevice(&dev));
+    EH_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d is outside the static scratch table", dev);
+    uint8_t *p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p == nullptr) {
+        void *addr = nullptr;
+        EH_HIP(hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)));
+        EH_REQUIRE(addr != nullptr, "hipGetSymbolAddress returned a null address for the static scratch");
+        p = static_cast<uint8_t *>(addr);
+        __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);  // concurrent first calls store the same address
+    }
+    *ptr = p;
+    return EH_OK;
+}
+
 // int8 tensors are computed as their uint8 equivalents: every stored value, zero point and clamp bound + 128
 // (SIGNED_TO_UNSIGNED in gpu/operators/cl_kernels/DepthwiseconvolutionKernels.cpp:2410-2411, and the zero points
 // + 128 of cl_optimized_impls/CLDepthwiseConvolutionQuantized.cpp:207-211)
@@ -317,8 +342,14 @@ struct GemmOp {
     }
 
     // residual != null: output = add(residual, result) with `radd`; `fused` tells whether the kernels did it
+    // bytes of the two channels-last staging images of a planar plan (each with the slack the kernels' wide loads need)
+    size_t stage_in_bytes() const { return ((size_t)in_n * in_c * in_hw + 256 + 255) / 256 * 256; }
+    size_t stage_out_bytes() const { return ((size_t)in_n * cout * out_hw + 256 + 255) / 256 * 256; }
+    static constexpr int kInlineParts = 8;  // a run over at most this many parts allocates no host memory
+
+    // staging != null: a planar plan uses [staging, staging + stage_in_bytes() + stage_out_bytes()) instead of its own images
     int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream, const uint8_t *residual = nullptr,
-            const AddDev *radd = nullptr, bool *fused = nullptr) {
+            const AddDev *radd = nullptr, bool *fused = nullptr, uint8_t *staging = nullptr) {
         EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
         int rc = check_requant(nq, w_signed, io_signed);
         if (rc) return rc;
@@ -327,13 +358,17 @@ struct GemmOp {
         if ((rc = refold(*nq, stream))) return rc;
         const uint8_t *in = static_cast<const uint8_t *>(input);
         uint8_t *out = static_cast<uint8_t *>(output);
+        uint8_t *const st_in = staging ? staging : stage_in, *const st_out = staging ? staging + stage_in_bytes() : stage_out;
         if (layout == EH_NCHW) {
-            if ((rc = launch_nchw2nhwc(in, stage_in, in_n, in_c, in_hw, stream))) return rc;
-            in = stage_in;
-            out = stage_out;
+            if ((rc = launch_nchw2nhwc(in, st_in, in_n, in_c, in_hw, stream))) return rc;
+            in = st_in;
+            out = st_out;
         }
-        std::vector<GemmProblem> problems;
-        problems.reserve(parts.size());
+        GemmProblem inline_problems[kInlineParts];
+        std::vector<GemmProblem> many;
+        if (parts.size() > (size_t)kInlineParts) many.resize(parts.size());
+        GemmProblem *const problems = many.empty() ? inline_problems : many.data();
+        int filled = 0;
         for (auto &g : parts) {
             GemmProblem p = g.proto;
             EH_REQUIRE((reinterpret_cast<uintptr_t>(in) & (uintptr_t)(g.vec - 1)) == 0,
@@ -358,11 +393,11 @@ struct GemmOp {
                 const bool has_form = g.cfg.id != GEMM_STAGED;
                 p.rq.fast = (pc_fast && has_form) ? channel_fast_mode(q) : 0;
             }
-            problems.push_back(p);
+            problems[filled++] = p;
         }
-        if ((rc = launch_igemm_batch(problems.data(), (int)problems.size(), stream))) return rc;
+        if ((rc = launch_igemm_batch(problems, filled, stream))) return rc;
         if (layout == EH_NCHW) {
-            if ((rc = launch_nhwc2nchw(stage_out, static_cast<uint8_t *>(output), in_n, cout, out_hw, stream))) return rc;
+            if ((rc = launch_nhwc2nchw(st_out, static_cast<uint8_t *>(output), in_n, cout, out_hw, stream))) return rc;
         }
         return EH_OK;
     }
@@ -574,7 +609,8 @@ int eh_init(int device) {
         set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
         return EH_FAILURE;
     }
-    return EH_OK;
+    uint8_t *unused = nullptr;
+    return static_scratch(&unused);  // this device's address of the static scratch, asked for while the device is current
 }
 
 int eh_device_name(char *dst, size_t cap) {
@@ -739,8 +775,8 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
     int rc;
     if ((rc = dev_alloc(&op.bias_copy, (size_t)d->cout))) return rc;
     if (d->layout == EH_NCHW) {
-        if ((rc = dev_alloc(&op.stage_in, (size_t)d->n * d->c * d->h * d->w + 256))) return rc;
-        if ((rc = dev_alloc(&op.stage_out, (size_t)d->n * d->cout * ho * wo + 256))) return rc;
+        if ((rc = dev_alloc(&op.stage_in, op.stage_in_bytes()))) return rc;
+        if ((rc = dev_alloc(&op.stage_out, op.stage_out_bytes()))) return rc;
     }
     const int taps = d->kh * d->kw;
     op.parts.resize(G);
@@ -882,6 +918,25 @@ int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const 
     EH_REQUIRE(plan != nullptr, "null plan");
     if (plan->d.n == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);  // zero-size early-out, as CLConvolution::execute does
     return plan->op.run(input, output, q, as_stream(stream));
+}
+
+int eh_conv2d_u8_run_static(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    if (plan->d.n == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);
+    const GemmOp &op = plan->op;
+    EH_REQUIRE(op.parts.size() <= (size_t)GemmOp::kInlineParts, "run_static: %zu convolution groups, at most %d are supported",
+               op.parts.size(), GemmOp::kInlineParts);
+    uint8_t *staging = nullptr;
+    if (op.layout == EH_NCHW) {
+        const size_t need = op.stage_in_bytes() + op.stage_out_bytes();
+        EH_REQUIRE(need <= (size_t)EH_STATIC_SCRATCH_BYTES,
+                   "run_static: the channels-last staging of this plan takes %zu bytes, the static scratch holds %zu", need,
+                   (size_t)EH_STATIC_SCRATCH_BYTES);
+        int rc = static_scratch(&staging);
+        if (rc) return rc;
+    }
+    // every staging byte a kernel reads was written earlier in the same call, so nothing has to be cleared
+    return plan->op.run(input, output, q, as_stream(stream), nullptr, nullptr, nullptr, staging);
 }
 
 int eh_conv2d_u8_run_add(eh_conv_plan *plan, const void *input, const void *residual, void *output, const eh_requant *q,
@@ -1039,8 +1094,8 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
     int rc;
     if ((rc = dev_alloc(&op.bias_copy, (size_t)d->cout))) return rc;
     if (d->layout == EH_NCHW) {
-        if ((rc = dev_alloc(&op.stage_in, (size_t)d->n * d->c * d->h * d->w + 256))) return rc;
-        if ((rc = dev_alloc(&op.stage_out, (size_t)d->n * d->cout * oh * ow + 256))) return rc;
+        if ((rc = dev_alloc(&op.stage_in, op.stage_in_bytes()))) return rc;
+        if ((rc = dev_alloc(&op.stage_out, op.stage_out_bytes()))) return rc;
     }
     const int sh = d->stride_h, sw = d->stride_w;
     for (int g = 0; g < G; ++g)

@@ -255,6 +255,17 @@ int eh_conv2d_u8_set_perchannel(eh_conv_plan *plan, const int32_t *multipliers, 
                                 void *stream);
 int eh_conv2d_u8_repack(eh_conv_plan *plan, const void *weight, const void *bias, const eh_requant *q, void *stream);
 int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
+/* eh_conv2d_u8_run for callers that must not allocate (code under graph capture, tight serving loops, harnesses
+ * that forbid it): no counterpart in the reference.  Calls no hipMalloc / hipFree and allocates no host memory.  A
+ * planar (EH_NCHW) plan computes channels-last between two layout conversions; here the two channels-last staging
+ * images live in a static device array of EH_STATIC_SCRATCH_BYTES that each GPU holds from the moment the library
+ * is loaded on it, instead of in the plan's own buffers (an EH_NHWC plan needs no staging and runs as
+ * eh_conv2d_u8_run does).  Fails with EH_INVALID_PARAMS, launching nothing, when the staging
+ * (n*c*h*w + n*cout*ho*wo bytes, each rounded up to 256 plus 256) exceeds the array or the plan has more than
+ * 8 groups.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * threads) race; calls ordered on one stream do not.  Results are bit for bit those of eh_conv2d_u8_run. */
+#define EH_STATIC_SCRATCH_BYTES (32u << 20)
+int eh_conv2d_u8_run_static(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
 /* Convolution followed by the quantized residual add, output = add(residual, convolution) with `aq` as eh_add_u8
  * applies it (the residual is the add's first operand; it has the output's shape and layout and must not be the
  * output buffer).  Bit for bit what eh_conv2d_u8_run into a temporary followed by eh_add_u8 gives; the one-tap and
