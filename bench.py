@@ -4,13 +4,22 @@ Headline workload (BASELINE.json configs[1]): uint8 FullyConnected GEMM, M=256
 batch rows, K=4096, N=4096, zero points 3 / 128, scales 0.01 / 0.002 / 0.08,
 int32 bias, fixed-point requantization fused.  One step = one execution of the
 operator on device-resident tensors with pre-packed weights.  The other
-configurations are timed the same way and reported under "others".
+configurations are timed the same way and reported under "others"; the
+MobileNetV2 figure (BASELINE.json configs[4], the second half of the metric) is
+repeated at the top level as "images_per_s".
+
+Memory-bound workloads are timed twice: "warm" replays one set of buffers (every
+working set here is smaller than the 256 MB Infinity Cache, so the bytes come
+from that cache, not from HBM), "cold" rotates over enough buffer sets that a
+set has been evicted before it is used again.  The cold figure is the one the
+HBM roofline fraction is quoted on.
 
 Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this build uses one GPU."""
 import argparse
 import importlib
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -23,41 +32,63 @@ sys.path.insert(0, ROOT)
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA peak, TOP/s
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 SEED = 0xEDE2
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc (FETCH_SIZE 12348.6 KiB x 1.999,
-# WRITE_SIZE 1024 KiB x 1.000, the factors being what the same counters read on a 64 MiB copy):
-# profiles/igemm_dma_64x64_splitk__fc_m256_k4096_n4096.md
-MEASURED_TRAFFIC_BYTES = 25281004 + 1048576
+COLD_FOOTPRINT = 640 << 20   # bytes a rotating workload walks through before it comes back: 2.5 x the Infinity Cache
+HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "igemm_dma_64x64_splitk__fc_m256_k4096_n4096.md")
+MIN_TIMED_SECONDS = 0.02   # a timed region shorter than this is mostly host overhead: the K steps are then repeated
 
 
-def time_steps(eden, stream, launch, steps, warmup, use_graph=True, chunk=50):
-    """Runs `warmup` untimed and exactly `steps` timed executions of launch(stream_handle).
-    Returns (wall seconds, HIP-event seconds) for the timed region."""
-    for _ in range(warmup):
-        launch(stream.h)
+def time_steps(eden, stream, launch, steps, warmup, use_graph=True, chunk=50, sets=1):
+    """Runs `warmup` untimed and `steps` timed executions of launch(stream_handle, set_index), set_index walking
+    0 .. sets-1 round and round (workloads that rotate over several buffer sets to defeat the caches).  When the K
+    steps take less than MIN_TIMED_SECONDS the whole K-step region is repeated R times inside the timed region.
+    Returns (wall seconds per K steps, HIP-event seconds per K steps, R)."""
+    counter = [0]
+
+    def one(s):
+        launch(s, counter[0] % sets)
+        counter[0] += 1
+
+    for _ in range(max(warmup, sets)):
+        one(stream.h)
     stream.sync()
     graph = None
     chunk = max(1, min(chunk, steps))
-    if use_graph:
-        graph = eden.Graph(stream, lambda s: [launch(s) for _ in range(chunk)])
+    if sets > 1:
+        chunk = max(sets, chunk // sets * sets)  # a replay walks whole rounds of the buffer sets
+        steps = -(-steps // chunk) * chunk if use_graph else steps  # (callers pass whole rounds: see round_steps)
+    if use_graph and chunk <= steps:
+        counter[0] = 0
+        graph = eden.Graph(stream, lambda s: [one(s) for _ in range(chunk)])
         graph.launch(stream)  # first replay uploads the graph; keep it out of the timed region
         stream.sync()
+
+    def region():
+        done = 0
+        if graph is not None:
+            while done + chunk <= steps:
+                graph.launch(stream)
+                done += chunk
+        while done < steps:
+            one(stream.h)
+            done += 1
+
     e0, e1 = eden.Event(), eden.Event()
-    device_sync()
-    t0 = time.perf_counter()
-    e0.record(stream.h)
-    done = 0
-    if graph is not None:
-        while done + chunk <= steps:
-            graph.launch(stream)
-            done += chunk
-    while done < steps:
-        launch(stream.h)
-        done += 1
-    e1.record(stream.h)
-    stream.sync()
-    device_sync()
-    t1 = time.perf_counter()
-    return t1 - t0, e1.elapsed_ms_since(e0) * 1e-3
+    repeats, wall, ev = 1, 0.0, 0.0
+    while True:
+        device_sync()
+        t0 = time.perf_counter()
+        e0.record(stream.h)
+        for _ in range(repeats):
+            region()
+        e1.record(stream.h)
+        stream.sync()
+        device_sync()
+        wall = time.perf_counter() - t0
+        ev = e1.elapsed_ms_since(e0) * 1e-3
+        if wall >= MIN_TIMED_SECONDS or repeats >= 4096:
+            break
+        repeats = min(4096, max(repeats * 2, int(repeats * MIN_TIMED_SECONDS * 1.3 / max(wall, 1e-6)) + 1))
+    return wall / repeats, ev / repeats, repeats
 
 
 _torch = None
@@ -77,107 +108,138 @@ def device_sync():
     eden_mod.sync(None)
 
 
-def fc_workload(eden, synth, m=256, k=4096, n=4096):
+def round_steps(steps, sets, chunk=50):
+    """`steps` rounded up to whole graph replays of a rotating workload, so that no launch of the timed region comes from the host"""
+    if sets <= 1:
+        return steps
+    chunk = max(sets, min(chunk, steps) // sets * sets)
+    return -(-steps // chunk) * chunk
+
+
+def set_count(per_set_bytes, cold):
+    return max(2, -(-COLD_FOOTPRINT // per_set_bytes)) if cold else 1
+
+
+def fc_workload(eden, synth, m=256, k=4096, n=4096, cold=False):
+    """cold: every set has its own activations, weights (packed per plan) and output"""
     a = synth.fill_u8((m, k), SEED + 32)
     w = synth.fill_u8_normal((n, k), SEED + 33, 128, 20)
     b = synth.fill_i32((n,), SEED + 34, -1000, 1000)
     q = eden.make_requant(0.01, 3, 0.002, 128, 0.08, 0)
-    d_a, d_w, d_b = eden.DeviceBuffer(host=a), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
-    d_o = eden.DeviceBuffer(nbytes=m * n)
-    plan = eden.FcPlan(m, k, n, d_w, d_b, q)
-    keep = (d_a, d_w, d_b, d_o, plan)
-    return dict(name="fc_m%d_k%d_n%d" % (m, k, n), launch=lambda s: plan.run(d_a, d_o, q, s), keep=keep,
-                ops=2.0 * m * k * n, bytes=m * k + n * k + 4 * n + m * n, bound="mfma",
-                host=(a, w, b, q), out=d_o, out_shape=(m, n))
+    nbytes = m * k + n * k + 4 * n + m * n
+    sets = set_count(nbytes, cold)
+    d_b = eden.DeviceBuffer(host=b)
+    per_set = []
+    for _ in range(sets):
+        d_a, d_w, d_o = eden.DeviceBuffer(host=a), eden.DeviceBuffer(host=w), eden.DeviceBuffer(nbytes=m * n)
+        plan = eden.FcPlan(m, k, n, d_w, d_b, q)
+        if cold:
+            eden.sync()
+            d_w.free()   # the plan keeps its own packed copy; the raw weights are not read again
+        per_set.append((d_a, d_o, plan))
+    return dict(name="fc_m%d_k%d_n%d" % (m, k, n), launch=lambda s, i: per_set[i][2].run(per_set[i][0], per_set[i][1], q, s),
+                keep=(per_set, d_b), sets=sets, ops=2.0 * m * k * n, bytes=nbytes, bound="mfma",
+                host=(a, w, b, q), out=per_set[0][1], out_shape=(m, n))
 
 
-def conv_workload(eden, synth, n=1):
+def conv_workload(eden, synth, n=1, cold=False):
     desc = eden.conv_desc(n, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=eden.NHWC)
     x = synth.fill_u8((n, 56, 56, 64), SEED + 16)
     w = synth.fill_u8((64, 64, 3, 3), SEED + 17)
     b = synth.fill_i32((64,), SEED + 18, -1000, 1000)
     q = eden.make_requant(0.02, 128, 0.005, 120, 0.05, 0, eden.ACT_RELU, True)
-    d_x, d_w, d_b = eden.DeviceBuffer(host=x), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
-    d_o = eden.DeviceBuffer(nbytes=n * 56 * 56 * 64)
+    d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
     plan = eden.ConvPlan(desc, d_w, d_b, q)
-    return dict(name="conv3x3_n%d_c64_56x56_nhwc" % n, launch=lambda s: plan.run(d_x, d_o, q, s),
-                keep=(d_x, d_w, d_b, d_o, plan), ops=2.0 * n * 56 * 56 * 64 * 576,
-                bytes=2 * n * 56 * 56 * 64 + 64 * 576 + 256, bound="mfma")
+    nbytes = 2 * n * 56 * 56 * 64 + 64 * 576 + 256
+    sets = set_count(nbytes, cold)
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 56 * 56 * 64)) for _ in range(sets)]
+    return dict(name="conv3x3_n%d_c64_56x56_nhwc" % n, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 56 * 56 * 64 * 576, bytes=nbytes, bound="mfma")
 
 
-def dw_workload(eden, synth, n=32):
+def dw_workload(eden, synth, n=32, cold=False):
     desc = eden.conv_desc(n, 144, 56, 56, 144, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), dm=1, layout=eden.NHWC)
     x = synth.fill_u8((n, 56, 56, 144), SEED + 48)
     w = synth.fill_u8((144, 1, 3, 3), SEED + 49)
     b = synth.fill_i32((144,), SEED + 50, -1000, 1000)
     q = eden.make_requant(0.03, 17, 0.006, 140, 0.025, 9, eden.ACT_RELU6, True)
-    d_x, d_w, d_b = eden.DeviceBuffer(host=x), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
-    d_o = eden.DeviceBuffer(nbytes=n * 28 * 28 * 144)
+    d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
     plan = eden.DwConvPlan(desc, d_w, d_b, q)
-    return dict(name="dw3x3s2_n%d_c144_56x56_nhwc" % n, launch=lambda s: plan.run(d_x, d_o, q, s),
-                keep=(d_x, d_w, d_b, d_o, plan), ops=2.0 * n * 144 * 28 * 28 * 9,
-                bytes=n * 144 * 56 * 56 + 144 * 9 + 144 * 4 + n * 144 * 28 * 28, bound="hbm")
+    nbytes = n * 144 * 56 * 56 + 144 * 9 + 144 * 4 + n * 144 * 28 * 28
+    sets = set_count(nbytes, cold)
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 28 * 28 * 144)) for _ in range(sets)]
+    return dict(name="dw3x3s2_n%d_c144_56x56_nhwc" % n, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 144 * 28 * 28 * 9, bytes=nbytes, bound="hbm")
 
 
-def pw_workload(eden, synth, n=32):
+def pw_workload(eden, synth, n=32, cold=False):
     desc = eden.conv_desc(n, 24, 56, 56, 144, 1, 1, layout=eden.NHWC)
     x = synth.fill_u8((n, 56, 56, 24), SEED + 51)
     w = synth.fill_u8((144, 24, 1, 1), SEED + 52)
     b = synth.fill_i32((144,), SEED + 53, -1000, 1000)
     q = eden.make_requant(0.02, 120, 0.004, 131, 0.03, 4, eden.ACT_RELU6, True)
-    d_x, d_w, d_b = eden.DeviceBuffer(host=x), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
-    d_o = eden.DeviceBuffer(nbytes=n * 56 * 56 * 144)
+    d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
     plan = eden.ConvPlan(desc, d_w, d_b, q)
-    return dict(name="pw1x1_n%d_24to144_56x56_nhwc" % n, launch=lambda s: plan.run(d_x, d_o, q, s),
-                keep=(d_x, d_w, d_b, d_o, plan), ops=2.0 * n * 56 * 56 * 24 * 144,
-                bytes=n * 56 * 56 * 24 + 144 * 24 + 576 + n * 56 * 56 * 144, bound="hbm")
+    nbytes = n * 56 * 56 * 24 + 144 * 24 + 576 + n * 56 * 56 * 144
+    sets = set_count(nbytes, cold)
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 56 * 56 * 144)) for _ in range(sets)]
+    return dict(name="pw1x1_n%d_24to144_56x56_nhwc" % n, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 56 * 56 * 24 * 144, bytes=nbytes, bound="hbm")
 
 
-def deconv_workload(eden, synth, n=8):
+def deconv_workload(eden, synth, n=8, cold=False):
     desc = eden.conv_desc(n, 256, 32, 32, 128, 4, 4, stride=(2, 2), pad=(1, 1, 1, 1), layout=eden.NHWC,
                           weight_layout=eden.W_IOHW)
     x = synth.fill_u8((n, 32, 32, 256), SEED + 64)
     w = synth.fill_u8((256, 128, 4, 4), SEED + 65)
     b = synth.fill_i32((128,), SEED + 66, -1000, 1000)
     q = eden.make_requant(0.02, 121, 0.005, 133, 0.35, 128)
-    d_x, d_w, d_b = eden.DeviceBuffer(host=x), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
-    d_o = eden.DeviceBuffer(nbytes=n * 64 * 64 * 128)
+    d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
     plan = eden.DeconvPlan(desc, d_w, d_b, q)
-    return dict(name="deconv4x4s2_n%d_256to128_32x32_nhwc" % n, launch=lambda s: plan.run(d_x, d_o, q, s),
-                keep=(d_x, d_w, d_b, d_o, plan), ops=2.0 * n * 1024 * 256 * 2048,
-                bytes=n * 256 * 1024 + 256 * 128 * 16 + 512 + n * 128 * 4096, bound="mfma")
+    nbytes = n * 256 * 1024 + 256 * 128 * 16 + 512 + n * 128 * 4096
+    sets = set_count(nbytes, cold)
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 64 * 64 * 128)) for _ in range(sets)]
+    return dict(name="deconv4x4s2_n%d_256to128_32x32_nhwc" % n, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 1024 * 256 * 2048, bytes=nbytes, bound="mfma")
 
 
-def mbv2_workload(eden, synth, batch=64, per_channel=False):
+def mbv2_workload(eden, synth, batch=64, per_channel=False, weights="minmax", cold=False):
     """BASELINE.json configs[4]: MobileNetV2-1.0 uint8 at 224x224x3, batch 64, the whole operator list per step.
-    per_channel: int8 weights with one scale per output channel in the convolutions."""
+    weights: "minmax" = per-tensor min/max quantized random-init weights (bytes span 0 .. 255), the configuration
+    BASELINE.json names; "narrow" = N(zp, 20) bytes.  per_channel: int8 weights with one scale per output channel in
+    the convolutions.  A step streams every feature map once, more than the Infinity Cache holds (working_set)."""
     mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
     # residual adds inside the projection convolutions' launches
-    net = mobilenet.MobileNetV2(eden, batch, fuse_add=True, per_channel=per_channel)
+    net = mobilenet.MobileNetV2(eden, batch, fuse_add=True, per_channel=per_channel, weights=weights)
     net.set_input(mobilenet.network_input(batch))
-    return dict(name="mobilenet_v2_1.0_224_u8%s_batch%d" % ("_perchannel_w" if per_channel else "", batch), launch=lambda s: net.run(s), keep=net,
+    name = "mobilenet_v2_1.0_224_u8%s%s_batch%d" % ("_perchannel_w" if per_channel else "", "" if weights == "minmax" else "_narrow_w", batch)
+    return dict(name=name, launch=lambda s, i: net.run(s), keep=net, sets=1, net=net,
                 ops=2.0 * mobilenet.macs_per_image() * batch, bytes=mobilenet.compulsory_bytes_per_image() * batch,
-                bound="hbm", images=batch, chunk=4)
+                bound="hbm", images=batch, chunk=4, per_channel=per_channel, weights=weights,
+                working_set=sum(b.nbytes for i, b in enumerate(net.buffers) if i not in net.unwritten))
 
 
-def copy_workload(eden, synth, mib=64):
+def copy_workload(eden, synth, mib=64, cold=False):
     """A plain device-to-device copy of known size: the yardstick the HBM byte counters are scaled by."""
     nbytes = mib << 20
-    src, dst = eden.DeviceBuffer(nbytes=nbytes), eden.DeviceBuffer(nbytes=nbytes)
+    sets = set_count(2 * nbytes, cold)
+    bufs = [(eden.DeviceBuffer(nbytes=nbytes), eden.DeviceBuffer(nbytes=nbytes)) for _ in range(sets)]
     lib = eden.load()
-    return dict(name="copy_%dMiB" % mib, launch=lambda s: eden.check(lib.eh_d2d(dst.ptr, src.ptr, nbytes, s)),
-                keep=(src, dst), ops=0.0, bytes=2 * nbytes, bound="hbm")
+    return dict(name="copy_%dMiB" % mib, launch=lambda s, i: eden.check(lib.eh_d2d(bufs[i][1].ptr, bufs[i][0].ptr, nbytes, s)),
+                keep=bufs, sets=sets, ops=0.0, bytes=2 * nbytes, bound="hbm")
 
 
-def layout_workload(eden, synth, to_nhwc=True, n=64, c=96, h=112, w=112):
+def layout_workload(eden, synth, to_nhwc=True, n=64, c=96, h=112, w=112, cold=False):
     """NCHW <-> NHWC conversion of a feature map (MobileNetV2's largest, [64, 96, 112, 112]): bytes in + bytes out."""
     nbytes = n * c * h * w
-    src, dst = eden.DeviceBuffer(host=synth.fill_u8((nbytes,), SEED + 90)), eden.DeviceBuffer(nbytes=nbytes)
+    x = synth.fill_u8((nbytes,), SEED + 90)
+    sets = set_count(2 * nbytes, cold)
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=nbytes)) for _ in range(sets)]
     lib = eden.load()
     fn = lib.eh_transpose_u8_nchw2nhwc if to_nhwc else lib.eh_transpose_u8_nhwc2nchw
     return dict(name="%s_n%d_c%d_%dx%d" % ("nchw2nhwc" if to_nhwc else "nhwc2nchw", n, c, h, w),
-                launch=lambda s: eden.check(fn(src.ptr, dst.ptr, n, c, h, w, s)),
-                keep=(src, dst), ops=0.0, bytes=2 * nbytes, bound="hbm")
+                launch=lambda s, i: eden.check(fn(bufs[i][0].ptr, bufs[i][1].ptr, n, c, h, w, s)),
+                keep=bufs, sets=sets, ops=0.0, bytes=2 * nbytes, bound="hbm")
 
 
 def roofline(work, event_s, steps):
@@ -189,6 +251,18 @@ def roofline(work, event_s, steps):
     achieved = work["bytes"] / per_launch / 1e9
     return dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                 frac=round(achieved / HBM_PEAK_GBS, 4), us_per_launch=round(per_launch * 1e6, 3))
+
+
+def profiled_traffic():
+    """HBM bytes per launch of the headline kernel, read from the committed rocprofv3 summary (FETCH_SIZE and
+    WRITE_SIZE per dispatch, each scaled by what the same counter reads on a copy of known size); None without it."""
+    try:
+        text = open(HEADLINE_PROFILE).read()
+        fetch = re.search(r"FETCH_SIZE.*= (\d+) bytes per dispatch", text)
+        write = re.search(r"WRITE_SIZE.*= (\d+) bytes per dispatch", text)
+        return int(fetch.group(1)) + int(write.group(1))
+    except Exception:
+        return None
 
 
 def cpu_baseline(work):
@@ -212,6 +286,56 @@ def cpu_baseline(work):
                 sample="full workload (M=256, K=4096, N=4096) %d times, median %.4f s per run, %.1f s of CPU time in all; GPU output checked equal" % (len(times), t, sum(times)))
 
 
+def check_network(work):
+    """The checker's part of the MobileNetV2 line: the network object that is about to be timed (batch 64) runs 32
+    repetitions of a pair of images and every image's logits must equal the CPU oracle's for that image of the pair;
+    the oracle's own time for the pair is the CPU figure.  Raises SystemExit on a mismatch."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from harness import oracle_forward
+    mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+    net = work["net"]
+    pair = mobilenet.network_input(2)
+    t0 = time.perf_counter()
+    _, _, want = oracle_forward(pair, 224, work["per_channel"], work["weights"])
+    cpu_s = time.perf_counter() - t0
+    net.set_input(np.tile(pair, (net.batch // 2, 1, 1, 1)))
+    net.run()
+    eden_mod.sync(None)
+    got = net.logits()
+    ref = want[-1].reshape(2, -1)
+    for img in range(net.batch):
+        if not np.array_equal(got[img], ref[img % 2]):
+            raise SystemExit("bench: %s: logits of image %d differ from the CPU oracle" % (work["name"], img))
+    net.set_input(mobilenet.network_input(net.batch))
+    return round(2 / cpu_s, 2)
+
+
+def measure(eden, synth, stream, make, steps, warmup, use_graph, cold_too):
+    """One workload, warm and (for the memory-bound ones, when asked) cold."""
+    w = make(eden, synth)
+    wall, ev, reps = time_steps(eden, stream, w["launch"], steps, warmup, use_graph, w.get("chunk", 50))
+    entry = dict(workload=w["name"], steps=steps, tops=round(w["ops"] * steps / wall / 1e12, 2), roofline=roofline(w, ev, steps))
+    entry["roofline"]["buffers"] = "warm: one buffer set replayed (%.1f MB, below the 256 MB Infinity Cache)" % (w["bytes"] / 1e6)
+    if "images" in w:
+        entry["images_per_s"] = round(w["images"] * steps / wall, 1)
+        entry["roofline"]["buffers"] = "one step streams %.0f MB of feature maps (each written once and read by the next operators)" % (w["working_set"] / 1e6)
+    if reps > 1:
+        entry["timed_region_repeats"] = reps
+    del w
+    if cold_too:
+        c = make(eden, synth, cold=True)
+        steps = round_steps(steps, c["sets"], c.get("chunk", 50))
+        wall2, ev2, reps2 = time_steps(eden, stream, c["launch"], steps, warmup, use_graph, c.get("chunk", 50), c["sets"])
+        warm = entry["roofline"]
+        entry["roofline"] = roofline(c, ev2, steps)
+        entry["steps_cold"] = steps
+        entry["roofline"]["buffers"] = "cold: %d buffer sets in rotation (%.0f MB between two uses of a set)" % (c["sets"], c["sets"] * c["bytes"] / 1e6)
+        entry["roofline_warm"] = warm
+        entry["tops"] = round(c["ops"] * steps / wall2 / 1e12, 2)
+        del c
+    return entry
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -219,8 +343,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, pw, deconv, mbv2, mbv2pc, copy, tonhwc, tonchw")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the oracle check of the network")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2, mbv2narrow, mbv2pc, copy, tonhwc, tonchw")
+    ap.add_argument("--cold", action="store_true", help="with --only: rotate over buffer sets that together exceed the Infinity Cache")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (got --gpus %d); no multi-GPU figure exists" % args.gpus,
@@ -234,25 +359,34 @@ def main():
     stream = eden.Stream()
     use_graph = not args.no_graph
 
+    def shaped(fn, **fixed):
+        return lambda e, s, cold=False: fn(e, s, cold=cold, **fixed)
+
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
-                    fcbig=lambda e, s: fc_workload(e, s, 8192, 4096, 4096), conv64=lambda e, s: conv_workload(e, s, 64),
-                    copy=copy_workload, mbv2=mbv2_workload, tonhwc=layout_workload,
-                    tonchw=lambda e, s: layout_workload(e, s, to_nhwc=False),
-                    mbv2pc=lambda e, s: mbv2_workload(e, s, per_channel=True))
+                    fcbig=shaped(fc_workload, m=8192, k=4096, n=4096), conv64=shaped(conv_workload, n=64),
+                    dwbig=shaped(dw_workload, n=256), pwbig=shaped(pw_workload, n=256),
+                    copy=copy_workload, mbv2=mbv2_workload, mbv2narrow=shaped(mbv2_workload, weights="narrow"),
+                    tonhwc=layout_workload, tonchw=shaped(layout_workload, to_nhwc=False),
+                    mbv2pc=shaped(mbv2_workload, per_channel=True))
     if args.only:
-        work = families[args.only](eden, synth)
-        wall, ev = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph, work.get("chunk", 50))
-        line = dict(workload=work["name"], steps=args.steps, ms_per_step=wall / args.steps * 1e3,
-                    roofline=roofline(work, ev, args.steps))
+        work = families[args.only](eden, synth, cold=args.cold)
+        args.steps = round_steps(args.steps, work["sets"], work.get("chunk", 50))
+        wall, ev, reps = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph, work.get("chunk", 50), work["sets"])
+        line = dict(workload=work["name"], steps=args.steps, ms_per_step=wall / args.steps * 1e3, buffer_sets=work["sets"],
+                    timed_region_repeats=reps, roofline=roofline(work, ev, args.steps))
         if "images" in work:
             line["images_per_s"] = round(work["images"] * args.steps / wall, 1)
         print(json.dumps(line))
         return
 
     work = fc_workload(eden, synth)
-    wall, ev = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph)
+    wall, ev, reps = time_steps(eden, stream, work["launch"], args.steps, args.warmup, use_graph)
     rf = roofline(work, ev, args.steps)
-    rf["traffic"] = MEASURED_TRAFFIC_BYTES
+    rf["traffic"] = profiled_traffic()
+    launch_note = "hip graph replay" if use_graph else "host launches"
+    if reps > 1:
+        launch_note += "; the %d steps took under %d ms, so the timed region is %d repetitions of them and ms_per_step is its wall clock / (%d x %d)" % (
+            args.steps, int(MIN_TIMED_SECONDS * 1e3), reps, reps, args.steps)
     result = {
         "metric": "int8 TOPS per conv/FC layer + MobileNetV2-u8 images/sec, 1 GPU, % roofline",
         "value": round(work["ops"] * args.steps / wall / 1e12, 2),
@@ -268,7 +402,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "uint8 FullyConnected GEMM M=256 K=4096 N=4096 (BASELINE configs[1]), int32 bias, "
                                "fixed-point requant fused, weights pre-packed, tensors resident in HBM",
-                   "launch": "hip graph replay" if use_graph else "host launches"},
+                   "launch": launch_note},
         "roofline": rf,
     }
     # the ceilings measured on this device next to the published ones: int8 MFMA issued from registers only,
@@ -277,22 +411,32 @@ def main():
                                "mfma_i8_toggling_operands_tops": round(eden.probe_mfma_i8(200000, True), 1)}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(work)
+    del work
     if not args.no_others:
-        others = []
-        for make, steps in ((conv_workload, 2000), (lambda e, s: conv_workload(e, s, 64), 300), (pw_workload, 500),
-                            (dw_workload, 1000), (deconv_workload, 500),
-                            (lambda e, s: fc_workload(e, s, 8192, 4096, 4096), 100),
-                            (layout_workload, 200), (lambda e, s: layout_workload(e, s, to_nhwc=False), 200),
-                            (mbv2_workload, 40),
-                            (lambda e, s: mbv2_workload(e, s, per_channel=True), 40)):
-            w2 = make(eden, synth)
-            wall2, ev2 = time_steps(eden, stream, w2["launch"], steps, max(10, steps // 10), use_graph, w2.get("chunk", 50))
-            entry = dict(workload=w2["name"], steps=steps, tops=round(w2["ops"] * steps / wall2 / 1e12, 2),
-                         roofline=roofline(w2, ev2, steps))
-            if "images" in w2:
-                entry["images_per_s"] = round(w2["images"] * steps / wall2, 1)
-            others.append(entry)
-            del w2
+        # MobileNetV2 (BASELINE configs[4]): checked against the oracle before it is timed
+        net = mbv2_workload(eden, synth)
+        if not args.no_cpu:
+            result["cpu_baseline"]["mobilenet_v2_images_per_s"] = check_network(net)
+            result["cpu_baseline"]["mobilenet_v2_sample"] = "2 images (224x224x3) through the oracle's operator list; the batch-64 GPU network's logits checked equal on 32 repetitions of the pair"
+        wall2, ev2, reps2 = time_steps(eden, stream, net["launch"], 40, 4, use_graph, net["chunk"])
+        c5 = dict(workload=net["name"], steps=40, tops=round(net["ops"] * 40 / wall2 / 1e12, 2), roofline=roofline(net, ev2, 40),
+                  images_per_s=round(net["images"] * 40 / wall2, 1), checked_against_oracle=not args.no_cpu)
+        c5["roofline"]["buffers"] = "one step streams %.0f MB of feature maps (each written once and read by the next operators)" % (net["working_set"] / 1e6)
+        result["images_per_s"] = c5["images_per_s"]
+        result["config"]["images_per_s"] = ("MobileNetV2-1.0 uint8 224x224x3, batch 64, per-tensor min/max quantized random-init weights "
+                                            "(BASELINE configs[4]), one HIP graph replay per batch; ms per batch %.4f" % (wall2 / 40 * 1e3))
+        del net
+        others = [c5]
+        for make, steps, cold_too in ((conv_workload, 2000, False), (shaped(conv_workload, n=64), 300, False),
+                                      (pw_workload, 500, True), (dw_workload, 1000, True),
+                                      (shaped(pw_workload, n=256), 100, True), (shaped(dw_workload, n=256), 200, True),
+                                      (deconv_workload, 500, False), (fc_workload, 500, True),
+                                      (shaped(fc_workload, m=8192, k=4096, n=4096), 100, False),
+                                      (layout_workload, 200, True), (shaped(layout_workload, to_nhwc=False), 200, True),
+                                      (copy_workload, 200, True),
+                                      (shaped(mbv2_workload, weights="narrow"), 40, False),
+                                      (shaped(mbv2_workload, per_channel=True), 40, False)):
+            others.append(measure(eden, synth, stream, make, steps, max(4, steps // 10), use_graph, cold_too))
         result["others"] = others
     print(json.dumps(result))
 

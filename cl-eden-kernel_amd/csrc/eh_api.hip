@@ -143,6 +143,14 @@ int pick_vec(int cig, int pixel_stride) {
     return 1;
 }
 
+// whether the load units describe the nine taps of a 3x3 window at dilation 1, row by row, `per_tap` units each
+static bool units_are_3x3(const std::vector<KUnit> &units, int per_tap) {
+    if (per_tap <= 0 || units.size() != (size_t)9 * per_tap) return false;
+    for (int t = 0; t < 9; ++t)
+        if (units[(size_t)t * per_tap].dy != t / 3 || units[(size_t)t * per_tap].dx != t % 3) return false;
+    return true;
+}
+
 // Allocates a part's device arrays and uploads its tables.  `units` holds one
 // KUnit per `vec` bytes of the real reduction length; padding units are added here.
 int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream,
@@ -161,6 +169,12 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
                units[26].dx == 2 && units[12].dy == 1 && units[12].dx == 1 && units[0].offset == 0) {
         // three channels, 3x3 taps, dilation 1: the first layer of image networks
         g.cfg.id = GEMM_C3K3;
+        g.cfg.slab = 32;
+    } else if (g.vec == 16 && g.taps == 9 && g.k == 9 * g.cin && units.size() == (size_t)g.k / 16 && g.proto.stride_h == 1 &&
+               g.proto.stride_w == 1 && g.proto.out_sy == 1 && g.proto.out_sx == 1 && units_are_3x3(units, g.cin / 16) &&
+               conv3x3_patch_applies(g.cin, g.proto.cin, g.proto.wo, g.proto.ho)) {
+        // 3x3 taps at dilation 1 and stride 1 over all input channels: the patch-in-LDS kernel
+        g.cfg.id = GEMM_CONV3X3;
         g.cfg.slab = 32;
     } else if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
         g.cfg = igemm_dma_select(g.proto.m, g.n, g.k, siblings);

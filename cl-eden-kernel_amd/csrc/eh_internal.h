@@ -323,6 +323,7 @@ enum GemmConfigId {
     GEMM_DMA_256x256 = 5,
     GEMM_THIN = 6,              // one-tap problems short of work for tiles; weights in MFMA fragment order
     GEMM_C3K3 = 7,              // 3 input channels, 3x3 taps (first layers); weights row-major [n_pad][32]
+    GEMM_CONV3X3 = 8,           // 3x3 taps, stride 1, input patch staged in LDS once; weights in MFMA fragment order
 };
 struct GemmConfig {
     int32_t id = GEMM_STAGED;
@@ -375,6 +376,8 @@ GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k, int32_t siblings);
 inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
+int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream);
+bool conv3x3_patch_applies(int32_t cin_group, int32_t pixel_stride, int32_t wo, int32_t ho);
 bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, int32_t channel_offset, int32_t y_base,
                         int32_t x_base, int64_t m, int64_t n);
 // Byte offset of reduction chunk `kc16` (16-byte units) of packed weight row `n`.
@@ -388,7 +391,7 @@ __host__ __device__ inline size_t packed_b_offset(const GemmConfig &cfg, int n, 
     const int ch = n & 31;
     n = (n & ~31) | (((ch & 15) >> 2) << 3) | ((ch >> 4) << 2) | (ch & 3);
     // fragment order: [32-channel block][32-byte step][lane = 32 * (chunk & 1) + row][16 bytes]
-    if (cfg.id == GEMM_THIN) return ((((size_t)(n >> 5) * (k_pad / 32) + (kc16 >> 1)) * 2 + (kc16 & 1)) * 32 + (n & 31)) * 16;
+    if (cfg.id == GEMM_THIN || cfg.id == GEMM_CONV3X3) return ((((size_t)(n >> 5) * (k_pad / 32) + (kc16 >> 1)) * 2 + (kc16 & 1)) * 32 + (n & 31)) * 16;
     const int cpr = cfg.slab / 16, rpb = 1024 / cfg.slab;
     const int c = kc16 % cpr;
     return ((size_t)(n / rpb) * (k_pad / cfg.slab) + kc16 / cpr) * 1024 + (size_t)(n % rpb) * cfg.slab +

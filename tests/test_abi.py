@@ -141,3 +141,17 @@ def test_one_tap_kernel_is_only_chosen_when_every_tap_lies_inside_the_image():
     assert eden.conv_kernels(d, deconv=True) == ["one_tap"] * 4
     d = eden.conv_desc(1, 16, 6, 6, 32, 2, 2, stride=(2, 2), pad=(0, -2, 0, -2), layout=nhwc, weight_layout=eden.W_IOHW)
     assert "one_tap" not in eden.conv_kernels(d, deconv=True)
+
+
+def test_3x3_stride_1_convolutions_take_the_patch_kernel():
+    nhwc = eden.NHWC
+    assert eden.conv_kernels(eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    assert eden.conv_kernels(eden.conv_desc(64, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    assert eden.conv_kernels(eden.conv_desc(2, 128, 16, 16, 100, 3, 3, layout=eden.NCHW)) == ["conv3x3_patch"]
+    # stride 2, dilation 2, groups, 16-byte channel counts, tiny images: the implicit-GEMM kernels
+    for d in (eden.conv_desc(1, 64, 56, 56, 64, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), layout=nhwc),
+              eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(2, 2, 2, 2), dil=(2, 2), layout=nhwc),
+              eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), groups=2, layout=nhwc),
+              eden.conv_desc(1, 48, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc),
+              eden.conv_desc(4, 64, 7, 7, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)):
+        assert "conv3x3_patch" not in eden.conv_kernels(d)

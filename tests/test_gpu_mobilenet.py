@@ -8,55 +8,11 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from harness import eden, to_eh_requant
+from harness import eden, oracle_forward, to_eh_requant
 
 mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
 
 pytestmark = pytest.mark.gpu
-
-
-def oracle_forward(x_nhwc, image, per_channel=False, weights="minmax"):
-    """All tensors of the network, NCHW, computed by the oracle from the same operator list."""
-    tensors, ops = mobilenet.layers(image, weights)
-    vals = [np.ascontiguousarray(x_nhwc.transpose(0, 3, 1, 2))]
-    n = x_nhwc.shape[0]
-    for op in ops:
-        kind = op["op"]
-        if kind == "add":
-            a, b, d = (tensors[op[k]] for k in ("a", "b", "dst"))
-            q = O.make_add_quant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
-            vals.append(O.add(vals[op["a"]], vals[op["b"]], q))
-            continue
-        s, d = tensors[op["src"]], tensors[op["dst"]]
-        x = vals[op["src"]]
-        if kind == "avgpool":
-            vals.append(O.avgpool(x, op["k"], op["k"]))
-            continue
-        act = O.ACT_RELU6 if op.get("relu6") else O.ACT_NONE
-        if per_channel and kind != "fc":
-            w, b, w_scales = mobilenet.op_weights_perchannel(op, s["c"])
-            eq, mults, shifts = eden.make_requant_perchannel(s["scale"], s["zp"], w_scales, d["scale"], d["zp"], act, bool(op.get("relu6")))
-            q = O.raw_quant(zp_in=eq.zp_in, zp_w=0, zp_out=eq.zp_out, act_min=eq.act_min, act_max=eq.act_max)
-            lo, hi = O.act_range_u8(act if op.get("relu6") else O.ACT_NONE, d["scale"], d["zp"])
-            assert (eq.zp_in, eq.zp_out, eq.act_min, eq.act_max) == (s["zp"], d["zp"], lo, hi)
-            groups = s["c"] if kind == "dw" else 1
-            shape = O.conv_shape(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4,
-                                 groups=groups)
-            fn = O.dwconv2d_perchannel if kind == "dw" else O.conv2d_perchannel
-            vals.append(fn(x, w, b, shape, q, mults, shifts))
-            continue
-        w, b = mobilenet.op_weights(op, s["c"])
-        q = O.make_quant(s["scale"], s["zp"], op["w_scale"], op["w_zp"], d["scale"], d["zp"], act, bool(op.get("relu6")))
-        if kind == "fc":
-            vals.append(O.fc(x.reshape(n, -1), w, b, q).reshape(n, -1, 1, 1))
-        elif kind == "dw":
-            shape = O.conv_shape(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4,
-                                 groups=s["c"])
-            vals.append(O.dwconv2d(x, w, b, shape, q))
-        else:
-            shape = O.conv_shape(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4)
-            vals.append(O.conv2d(x, w, b, shape, q))
-    return tensors, ops, vals
 
 
 def assert_network_alive(ops, want, batch):

@@ -204,6 +204,14 @@ CONV_CASES = [
     dict(n=2, c=64, h=20, w=20, cout=64, kh=3, kw=3, pad=(2, 2, 2, 2), dil=(2, 2)),
     dict(n=1, c=32, h=15, w=17, cout=32, kh=3, kw=3, stride=(2, 1), pad=(3, 3, 1, 1), dil=(3, 1), groups=2),
     dict(n=3, c=16, h=12, w=9, cout=40, kh=2, kw=3, stride=(1, 2), pad=(0, 2, 2, 0), dil=(2, 3)),
+    # 3x3 at stride 1 over 32-byte channel steps: the patch-in-LDS kernel (ragged channel blocks, every padding,
+    # widths that are not multiples of 32, tiles whose last rows fall off the image, one and two channel blocks)
+    dict(n=2, c=32, h=20, w=17, cout=40, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=3, c=96, h=9, w=30, cout=72, kh=3, kw=3, pad=(0, 2, 2, 0)),
+    dict(n=1, c=128, h=16, w=16, cout=100, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=5, c=64, h=33, w=12, cout=64, kh=3, kw=3),
+    dict(n=2, c=64, h=14, w=70, cout=32, kh=3, kw=3, pad=(2, 2, 2, 2)),
+    dict(n=9, c=64, h=56, w=56, cout=16, kh=3, kw=3, pad=(1, 1, 1, 1)),
 ]
 
 
@@ -334,6 +342,20 @@ def test_plan_refolds_when_zero_points_change_and_repacks_new_weights():
     plan.run(d_x, d_o, to_eh_requant(q2))
     assert np.array_equal(d_o.download((1, 16, 8, 8)), O.conv2d(x, w2, b2, s, q2))
     plan.destroy()
+
+
+def test_conv3x3_batch_64_equals_oracle_pair():
+    """The benchmark's 3x3 convolution at its batch of 64 (the batch decides the tile height of the patch kernel), on
+    32 repetitions of a pair of images: every image must equal the oracle's result for that image of the pair."""
+    s2 = O.conv_shape(2, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s2, SEED + 16)
+    q = quant(0.02, 128, 0.005, 120, 0.05, 0, O.ACT_RELU, True)
+    want = O.conv2d(x, w, b, s2, q)
+    s64 = O.conv_shape(64, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1))
+    got = gpu_conv(np.tile(x, (32, 1, 1, 1)), w, b, s64, to_eh_requant(q), layout=eden.NHWC)
+    for img in range(64):
+        assert np.array_equal(got[img], want[img % 2]), (img, diff_report(got[img], want[img % 2]))
+    assert want.std() > 10
 
 
 # ----------------------------------------------------------------- depthwise
