@@ -462,6 +462,8 @@ struct eh_dwconv_plan {
     bool pc_fast = false;  // every pair is inside the single-shift form's range
     // 3x3 channels-last plans: the 8-bit dot product form of the weights, usable while every w - zp_w fits int8
     int32_t *w_trip = nullptr, *bias_trip = nullptr;
+    int32_t *w_fold = nullptr, *bias_fold = nullptr;  // the unsigned form of the same plans, for weights of any range
+    bool fold_valid = false;
     bool range_known = false;   // w_lo / w_hi hold the extremes of the weight bytes (in the caller's own domain)
     int32_t w_lo = 0, w_hi = 0;
     bool trip_valid = false;    // w_trip / bias_trip match the current zero points
@@ -1279,6 +1281,8 @@ static void dw_release(eh_dwconv_plan *pl) {
     dev_free(pl->pc_shift);
     dev_free(pl->w_trip);
     dev_free(pl->bias_trip);
+    dev_free(pl->w_fold);
+    dev_free(pl->bias_fold);
 }
 
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
@@ -1309,6 +1313,13 @@ static int dw_refold(eh_dwconv_plan *pl, const eh_requant &caller_q, hipStream_t
                                      q.zp_w, pl->w_signed ? 1 : 0, stream);
             if (rc) return rc;
             pl->trip_valid = true;
+        }
+        pl->fold_valid = false;
+        if (pl->w_fold && !pl->trip_valid) {
+            rc = launch_dw_pack_fold(pl->w_copy, pl->has_bias ? pl->bias_copy : nullptr, pl->w_fold, pl->bias_fold, pl->cout, q.zp_in,
+                                     q.zp_w + (pl->w_signed ? 128 : 0), pl->w_signed ? 1 : 0, stream);
+            if (rc) return rc;
+            pl->fold_valid = true;
         }
         pl->packed_valid = true;
     }
@@ -1358,6 +1369,8 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     if (!rc && tile_form) {
         rc = dev_alloc(&pl->w_trip, (size_t)3 * pl->cout);
         if (!rc) rc = dev_alloc(&pl->bias_trip, (size_t)pl->cout + 4);
+        if (!rc) rc = dev_alloc(&pl->w_fold, (size_t)3 * pl->cout);
+        if (!rc) rc = dev_alloc(&pl->bias_fold, (size_t)pl->cout + 4);
     }
     if (!rc) rc = dw_set_weights(pl, weight, bias, s);
     if (!rc && tile_form && pl->cout > 0) {
@@ -1456,6 +1469,8 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     p.w_signed = plan->w_signed ? 1 : 0;
     p.w_trip = plan->trip_valid ? plan->w_trip : nullptr;
     p.bias_trip = plan->bias_trip;
+    p.w_fold = plan->fold_valid ? plan->w_fold : nullptr;
+    p.bias_fold = plan->bias_fold;
     p.io_flip = plan->io_signed ? 0x80808080u : 0u;
     p.rq = make_requant_dev(plan->q);
     if (plan->pc_multiplier) {

@@ -213,7 +213,14 @@ __device__ __forceinline__ uint32_t column_bytes(uint32_t r0, uint32_t r1, uint3
 // TW output pixels per thread: four, or eight for stride 1 on rows that are whole tiles of eight (the column words and
 // the index arithmetic are then shared by twice as many outputs).
 // PC: one multiplier and shift per channel, all inside the single-shift form's range (p.rq.fast != 0).
-template <int S, bool FLIP, int TW = 4, bool PC = false>
+// FOLD: weights of any range.  The products are then unsigned dot products of the raw bytes a and w, and
+//     sum (a - za)(w - zw) = sum a w - zw * sum a - za * sum w + 9 za zw
+// with the last two terms folded into the bias and sum a (nine taps, those outside the image reading za) taken from
+// per-column sums that neighbouring outputs share: one more dot product per column and channel.  p.zp_w is then the
+// zero point of the uint8 values being multiplied (int8 weights: + 128).
+__device__ __forceinline__ int udot4(uint32_t a, uint32_t b, int acc) { return (int)__builtin_amdgcn_udot4(a, b, (uint32_t)acc, false); }
+
+template <int S, bool FLIP, int TW = 4, bool PC = false, bool FOLD = false>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                     const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
     constexpr int IW = (TW - 1) * S + 3;
@@ -228,7 +235,10 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
     const int oy = (int)(r2 - img * (uint32_t)p.ho);
     const int ox0 = tx * TW;
     const int iy0 = oy * S - p.pad_t, ix0 = ox0 * S - p.pad_l;
-    const uint32_t fill = ((uint32_t)p.zp_in * 0x01010101u) ^ 0x80808080u;  // the input zero point minus 128
+    // what a tap outside the image reads, as an operand of the form in use: the input zero point (FOLD) or that minus 128
+    const uint32_t fill = ((uint32_t)p.zp_in * 0x01010101u) ^ (FOLD ? 0u : 0x80808080u);
+    // uint8 tensors hold a, int8 tensors a - 128: the signed form wants a - 128, the unsigned one a
+    constexpr bool flip_loaded = FOLD ? FLIP : !FLIP;
     const uint32_t base = img * (uint32_t)(p.h * p.w_ * p.c) + cq * 4u;
 
     uint32_t col_off[IW];
@@ -250,20 +260,25 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
 #pragma unroll
         for (int x = 0; x < IW; ++x) {
             const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in + (row_off + col_off[x]));
-            in[ky][x] = row_ok && col_ok[x] ? (FLIP ? v : v ^ 0x80808080u) : fill;  // int8 tensors hold a - 128 already
+            in[ky][x] = row_ok && col_ok[x] ? (flip_loaded ? v ^ 0x80808080u : v) : fill;
         }
     }
     int4 wk[3];
 #pragma unroll
-    for (int kx = 0; kx < 3; ++kx) wk[kx] = *reinterpret_cast<const int4 *>(p.w_trip + ((uint32_t)kx * (uint32_t)p.cout + cq * 4u));
-    const int4 b4 = *reinterpret_cast<const int4 *>(p.bias_trip + cq * 4u);
+    for (int kx = 0; kx < 3; ++kx) wk[kx] = *reinterpret_cast<const int4 *>((FOLD ? p.w_fold : p.w_trip) + ((uint32_t)kx * (uint32_t)p.cout + cq * 4u));
+    const int4 b4 = *reinterpret_cast<const int4 *>((FOLD ? p.bias_fold : p.bias_trip) + cq * 4u);
     uint32_t col[IW][4];
+    int cs[FOLD ? IW : 1][4];  // FOLD: sum of the column's three bytes
 #pragma unroll
     for (int x = 0; x < IW; ++x) {
         col[x][0] = column_bytes<0>(in[0][x], in[1][x], in[2][x]);
         col[x][1] = column_bytes<1>(in[0][x], in[1][x], in[2][x]);
         col[x][2] = column_bytes<2>(in[0][x], in[1][x], in[2][x]);
         col[x][3] = column_bytes<3>(in[0][x], in[1][x], in[2][x]);
+        if constexpr (FOLD) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) cs[x][c] = udot4(col[x][c], 0x00010101u, 0);
+        }
     }
     uint8_t *dst = p.out + (((img * (uint32_t)p.ho + (uint32_t)oy) * (uint32_t)p.wo + (uint32_t)ox0) * (uint32_t)p.cout + cq * 4u);
     const RequantDev rq = p.rq;
@@ -273,10 +288,23 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
         int acc0 = b4.x, acc1 = b4.y, acc2 = b4.z, acc3 = b4.w;
 #pragma unroll
         for (int kx = 0; kx < 3; ++kx) {
-            acc0 = __builtin_amdgcn_sdot4((int)col[j * S + kx][0], wk[kx].x, acc0, false);
-            acc1 = __builtin_amdgcn_sdot4((int)col[j * S + kx][1], wk[kx].y, acc1, false);
-            acc2 = __builtin_amdgcn_sdot4((int)col[j * S + kx][2], wk[kx].z, acc2, false);
-            acc3 = __builtin_amdgcn_sdot4((int)col[j * S + kx][3], wk[kx].w, acc3, false);
+            if constexpr (FOLD) {
+                acc0 = udot4(col[j * S + kx][0], (uint32_t)wk[kx].x, acc0);
+                acc1 = udot4(col[j * S + kx][1], (uint32_t)wk[kx].y, acc1);
+                acc2 = udot4(col[j * S + kx][2], (uint32_t)wk[kx].z, acc2);
+                acc3 = udot4(col[j * S + kx][3], (uint32_t)wk[kx].w, acc3);
+            } else {
+                acc0 = __builtin_amdgcn_sdot4((int)col[j * S + kx][0], wk[kx].x, acc0, false);
+                acc1 = __builtin_amdgcn_sdot4((int)col[j * S + kx][1], wk[kx].y, acc1, false);
+                acc2 = __builtin_amdgcn_sdot4((int)col[j * S + kx][2], wk[kx].z, acc2, false);
+                acc3 = __builtin_amdgcn_sdot4((int)col[j * S + kx][3], wk[kx].w, acc3, false);
+            }
+        }
+        if constexpr (FOLD) {
+            acc0 -= p.zp_w * (cs[j * S][0] + cs[j * S + 1][0] + cs[j * S + 2][0]);
+            acc1 -= p.zp_w * (cs[j * S][1] + cs[j * S + 1][1] + cs[j * S + 2][1]);
+            acc2 -= p.zp_w * (cs[j * S][2] + cs[j * S + 1][2] + cs[j * S + 2][2]);
+            acc3 -= p.zp_w * (cs[j * S][3] + cs[j * S + 1][3] + cs[j * S + 2][3]);
         }
         uint32_t o = PC ? requant4_channel_fast(acc0, acc1, acc2, acc3, rq, quad) : requant4<false>(acc0, acc1, acc2, acc3, rq, quad);
         if (FLIP) o ^= 0x80808080u;
@@ -366,7 +394,36 @@ __global__ void dw_pack_trip_kernel(const uint8_t *w, const int32_t *bias, int32
     bias_trip[oc] = (bias ? bias[oc] : 0) - (zp_in - 128) * sum;
 }
 
+// 3x3 weights [cout][9] -> w_fold[kx][cout]: the three vertical taps of column kx as the uint8 values the unsigned
+// form multiplies (int8 weights: byte + 128, `zp_w` being their zero point + 128) in bytes 0..2;
+// bias_fold[c] = bias - zp_in * sum w + 9 * zp_in * zp_w
+__global__ void dw_pack_fold_kernel(const uint8_t *w, const int32_t *bias, int32_t *w_fold, int32_t *bias_fold, int32_t cout,
+                                    int32_t zp_in, int32_t zp_w, int32_t w_signed) {
+    const int oc = blockIdx.x * blockDim.x + threadIdx.x;
+    if (oc >= cout) return;
+    int32_t sum = 0;
+    for (int kx = 0; kx < 3; ++kx) {
+        uint32_t word = 0;
+        for (int ky = 0; ky < 3; ++ky) {
+            const uint32_t v = (uint32_t)w[(size_t)oc * 9 + ky * 3 + kx] ^ (w_signed ? 0x80u : 0u);
+            sum += (int32_t)v;
+            word |= v << (8 * ky);
+        }
+        w_fold[(size_t)kx * cout + oc] = (int32_t)word;
+    }
+    bias_fold[oc] = (bias ? bias[oc] : 0) - zp_in * sum + 9 * zp_in * zp_w;
+}
+
 }  // namespace
+
+int launch_dw_pack_fold(const uint8_t *w, const int32_t *bias, int32_t *w_fold, int32_t *bias_fold, int32_t cout, int32_t zp_in,
+                        int32_t zp_w_u8, int32_t w_signed, hipStream_t stream) {
+    if (cout <= 0) return EH_OK;
+    hipLaunchKernelGGL(dw_pack_fold_kernel, dim3((cout + 127) / 128), dim3(128), 0, stream, w, bias, w_fold, bias_fold, cout, zp_in,
+                       zp_w_u8, w_signed);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
 
 int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32_t *bias_folded, int32_t cout,
                    int32_t taps, int32_t zp_in, int32_t zp_w, int32_t w_signed, hipStream_t stream) {
@@ -386,7 +443,11 @@ int launch_dw_pack_trip(const uint8_t *w, const int32_t *bias, int32_t *w_trip, 
     return EH_OK;
 }
 
-int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
+int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
+    DwProblem p = caller_p;
+    const bool pc_two_step = p.rq.pc_multiplier != nullptr && !p.rq.fast;
+    if (p.w_trip || pc_two_step) p.w_fold = nullptr;  // the signed form where it applies; per-channel pairs outside the single-shift range use the 16-bit kernel
+    if (p.w_fold) p.zp_w += p.w_signed ? 128 : 0;     // zero point of the uint8 values the unsigned form multiplies
     const long outs = (long)p.n * p.ho * p.wo * p.cout;
     if (outs <= 0) return EH_OK;
     const bool vec = p.dm == 1 && (p.c & 3) == 0 && (reinterpret_cast<uintptr_t>(p.in) & 3) == 0 &&
@@ -408,14 +469,19 @@ int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream) {
                       : (flip ? dw3x3_nhwc_tile4_kernel<S, false, true> : dw3x3_nhwc_tile4_kernel<S, false, false>);
         };
         auto kernel = p.stride_h == 1 ? pick(std::integral_constant<int, 1>{}) : pick(std::integral_constant<int, 2>{});
+        // 8-bit dot products: the signed form where every w - zp_w fits int8, else the unsigned form for any weights
+        const bool fold = p.w_trip == nullptr;
         auto pick_dot4 = [&](auto s_tag, auto tw_tag) {
             constexpr int S = decltype(s_tag)::value, TW = decltype(tw_tag)::value;
+            if (fold)
+                return pc ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, true, true> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, true, true>)
+                          : (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, false, true> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, false, true>);
             return pc ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, true> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, true>)
                       : (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, false> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, false>);
         };
         using tw4 = std::integral_constant<int, 4>;
-        const bool dot4 = p.w_trip && (!pc || p.rq.fast);
-        if (dot4)  // every w - zp_w fits int8: the 8-bit dot product form
+        const bool dot4 = (p.w_trip || p.w_fold) && (!pc || p.rq.fast);
+        if (dot4)
             kernel = p.stride_h == 1 ? pick_dot4(std::integral_constant<int, 1>{}, tw4{}) : pick_dot4(std::integral_constant<int, 2>{}, tw4{});
         if (dot4 && p.stride_h == 1 && (p.wo & 7) == 0 && total >= (1l << 20)) {
             // large stride-1 layers with rows of whole eight-pixel tiles: eight outputs per thread

@@ -430,6 +430,10 @@ struct DwProblem {
     // three vertical taps in bytes 0..2, and the bias with (zp_in - 128) * sum_t (w - zp_w) folded in
     const int32_t *w_trip;
     const int32_t *bias_trip;
+    // 3x3 weights of any range for the unsigned dot product form (else null): [3 columns][cout] words of the uint8
+    // weight bytes (int8 weights: byte + 128), and the bias with -zp_in * sum w + 9 zp_in zp_w folded in
+    const int32_t *w_fold;
+    const int32_t *bias_fold;
     uint8_t *out;
     int32_t n, c, h, w_, cout, dm;
     int32_t kh, kw, stride_h, stride_w, pad_t, pad_l, dil_h, dil_w;
@@ -443,6 +447,8 @@ int launch_dw_pack(const uint8_t *w, const int32_t *bias, int32_t *w_pair, int32
                    int32_t taps, int32_t zp_in, int32_t zp_w, int32_t w_signed, hipStream_t stream);
 int launch_dw_pack_trip(const uint8_t *w, const int32_t *bias, int32_t *w_trip, int32_t *bias_trip, int32_t cout, int32_t zp_in,
                         int32_t zp_w, int32_t w_signed, hipStream_t stream);
+int launch_dw_pack_fold(const uint8_t *w, const int32_t *bias, int32_t *w_fold, int32_t *bias_fold, int32_t cout, int32_t zp_in,
+                        int32_t zp_w_u8, int32_t w_signed, hipStream_t stream);
 int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream);
 int launch_dwconv_nchw(const DwProblem &p, hipStream_t stream);
 
