@@ -88,6 +88,15 @@ EXPORTS = {
     "eh_h2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "eh_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "eh_d2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "eh_pool_create": (C.c_int, [C.POINTER(C.c_void_p)]),
+    "eh_pool_request": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t, C.POINTER(C.c_int32)]),
+    "eh_pool_reset_inter": (C.c_int, [C.c_void_p, C.c_int32]),
+    "eh_pool_reset_intra": (C.c_int, [C.c_void_p]),
+    "eh_pool_layout": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_int32)]),
+    "eh_pool_assign": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t)]),
+    "eh_pool_slot": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]),
+    "eh_pool_release": (C.c_int, [C.c_void_p, C.c_int32]),
+    "eh_pool_destroy": (C.c_int, [C.c_void_p]),
     "eh_stream_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "eh_stream_destroy": (C.c_int, [C.c_void_p]),
     "eh_stream_sync": (C.c_int, [C.c_void_p]),
@@ -269,6 +278,76 @@ class DeviceBuffer:
     def __del__(self):
         try:
             self.free()
+        except Exception:
+            pass
+
+
+POOL_INTER_NEW, POOL_INTER_REUSE, POOL_INTRA = 0, 1, 2
+
+
+class PooledBuffer:
+    """One slot of a BufferPool: sized at request time, addressed once the pool is assigned."""
+
+    def __init__(self, pool, slot):
+        self.pool, self.slot = pool, slot
+
+    @property
+    def ptr(self):
+        p = C.c_void_p()
+        check(load().eh_pool_slot(self.pool.h, self.slot, C.byref(p), None))
+        return p
+
+    @property
+    def nbytes(self):
+        n = C.c_size_t()
+        check(load().eh_pool_slot(self.pool.h, self.slot, None, C.byref(n)))
+        return n.value
+
+    def download(self, shape, dtype=np.uint8):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        lib = load()
+        if out.nbytes:
+            check(lib.eh_d2h(out.ctypes.data_as(C.c_void_p), self.ptr, out.nbytes, None))
+        check(lib.eh_stream_sync(None))
+        return out
+
+
+class BufferPool:
+    """The pooled-buffer protocol of an operator list (eh_pool_*): request / reset while the operators are built,
+    then one device allocation for all of them."""
+
+    def __init__(self):
+        self.h = C.c_void_p()
+        check(load().eh_pool_create(C.byref(self.h)))
+
+    def request(self, kind, nbytes):
+        slot = C.c_int32(-1)
+        check(load().eh_pool_request(self.h, kind, int(nbytes), C.byref(slot)))
+        return PooledBuffer(self, slot.value)
+
+    def reset_inter(self, buf):
+        check(load().eh_pool_reset_inter(self.h, buf.slot))
+
+    def reset_intra(self):
+        check(load().eh_pool_reset_intra(self.h))
+
+    def layout(self):
+        """(bytes an assignment would allocate, slots it would hold)"""
+        n, c = C.c_size_t(), C.c_int32()
+        check(load().eh_pool_layout(self.h, C.byref(n), C.byref(c)))
+        return n.value, c.value
+
+    def assign(self):
+        n = C.c_size_t()
+        check(load().eh_pool_assign(self.h, C.byref(n)))
+        return n.value
+
+    def __del__(self):
+        try:
+            if self.h:
+                load().eh_pool_destroy(self.h)
+                self.h = C.c_void_p()
         except Exception:
             pass
 

@@ -20,8 +20,9 @@
 // empty weight or input tensor makes initialize()/execute() succeed without work;
 // in channels-last mode (isNCHW == false) a tensor's Dim4 holds (n, h, w, c)
 // positionally; in androidNN mode the weight Dim4 holds (out, kh, kw, in).
-// Not offered here: per-channel quantized weights, INT8 precision, float
-// precisions, texture storage (initialize() returns FAILURE for them).
+// Per-channel quantized weights (per_channel_quant + scales) and INT8 precision are
+// offered as the reference offers them; float precisions and texture storage are not
+// (initialize() returns FAILURE for them).
 #pragma once
 
 #include <memory>

@@ -1,19 +1,21 @@
 // Device runtime and buffer manager of the HIP userdriver backend: hipMalloc-backed
 // buffers on one GPU behind the reference's pooling protocol.
 //
-// Mirrors CLRuntime's buffer manager (src/userdriver/gpu/common/CLRuntime.cpp:34-157
+// Same protocol as CLRuntime's buffer manager (src/userdriver/gpu/common/CLRuntime.cpp:34-157
 // getBuffer / assignBufferPool / resetIntraBuffer / resetInterBuffer, :1339-1372
 // allocBuffer with its 1024-byte head and 32-byte tail slack, :1409-1416
 // releaseBuffer) and its copy / layout entry points (CLRuntime.hpp:59-110,
-// CLRuntime.cpp:1477-1619).  One in-order stream stands in for the reference's
-// single in-order command queue (CLRuntime.cpp:920-928).
+// CLRuntime.cpp:1477-1619), built differently: the pooled buffers of an operator list
+// (INTER_SHARED_*, INTRA_SHARED) are slots of the library's eh_pool, which
+// assignBufferPool() lays out in one device allocation, so an operator list costs one
+// hipMalloc and none after it is built; DEDICATED buffers are allocations of their own.
+// One in-order stream stands in for the reference's single in-order command queue
+// (CLRuntime.cpp:920-928).
 #pragma once
 
-#include <algorithm>
 #include <map>
 #include <memory>
 #include <mutex>
-#include <tuple>
 #include <utility>
 #include <vector>
 
@@ -28,15 +30,17 @@ namespace hip {
 // A device allocation that may not exist yet (pooled buffers materialise in assignBufferPool).
 class HipBuffer {
 public:
-    explicit HipBuffer(size_t byte) : byte_(byte), buffer_(nullptr) {}
+    explicit HipBuffer(size_t byte, int32_t pool_slot = -1) : byte_(byte), buffer_(nullptr), pool_slot_(pool_slot) {}
     void assignBuffer(void *buffer) { buffer_ = buffer; }
     void setBytes(size_t byte) { byte_ = byte; }
     size_t getBytes() { return byte_; }
     void *getDataPtr() { return buffer_; }
+    int32_t poolSlot() const { return pool_slot_; }  // >= 0: lives in the runtime's pooled allocation
 
 private:
     size_t byte_;
     void *buffer_;
+    int32_t pool_slot_;
 };
 
 class HipRuntime {
@@ -44,6 +48,7 @@ public:
     HipRuntime() = default;
     ~HipRuntime() {
         for (auto &kv : allocations_) eh_free(kv.second);
+        if (pool_) eh_pool_destroy(pool_);
         if (stream_) eh_stream_destroy(stream_);
     }
     HipRuntime(const HipRuntime &) = delete;
@@ -74,79 +79,52 @@ public:
                 buffer->assignBuffer(allocBuffer(bytes, true));
                 return buffer;
             }
-            case BufferType::INTER_SHARED_NEW: {
-                auto buffer = std::make_shared<HipBuffer>(bytes);
-                inter_buffers_.push_back(std::make_pair(buffer, true));
-                return buffer;
-            }
-            case BufferType::INTER_SHARED_REUSE: {
-                for (auto &entry : inter_buffers_) {
-                    if (!entry.second) {  // released by resetInterBuffer: take it over, grown if needed
-                        if (entry.first->getBytes() < bytes) entry.first->setBytes(bytes);
-                        entry.second = true;
-                        return entry.first;
-                    }
-                }
-                auto buffer = std::make_shared<HipBuffer>(bytes);
-                inter_buffers_.push_back(std::make_pair(buffer, true));
-                return buffer;
-            }
-            case BufferType::INTRA_SHARED: {
-                for (auto &entry : intra_buffers_) {  // a free one that is already large enough
-                    if (!std::get<1>(entry) && std::get<0>(entry) >= bytes) {
-                        std::get<1>(entry) = true;
-                        return std::get<2>(entry);
-                    }
-                }
-                for (auto it = intra_buffers_.rbegin(); it != intra_buffers_.rend(); ++it) {  // the largest free one, grown
-                    if (!std::get<1>(*it)) {
-                        std::get<0>(*it) = bytes;
-                        std::get<1>(*it) = true;
-                        auto mem = std::get<2>(*it);
-                        sortIntra();
-                        return mem;
-                    }
-                }
-                auto buffer = std::make_shared<HipBuffer>(0);
-                intra_buffers_.push_back(std::make_tuple(bytes, true, buffer));
-                sortIntra();
-                return buffer;
-            }
+            case BufferType::INTER_SHARED_NEW: return pooled(EH_POOL_INTER_NEW, bytes);
+            case BufferType::INTER_SHARED_REUSE: return pooled(EH_POOL_INTER_REUSE, bytes);
+            case BufferType::INTRA_SHARED: return pooled(EH_POOL_INTRA, bytes);
             default: ERROR_PRINT("HipRuntime::getBuffer: unknown buffer type\n");
         }
         return nullptr;
     }
 
-    // Materialises every pooled buffer at its final size (intra: zero filled), then forgets the pools.
+    // Materialises every pooled buffer at its final size, all of them in ONE device allocation (the reference
+    // allocates each: CLRuntime.cpp:120-137), then forgets the pools.
     Status assignBufferPool() {
-        for (auto &entry : intra_buffers_) {
-            std::get<2>(entry)->setBytes(std::get<0>(entry));
-            std::get<2>(entry)->assignBuffer(allocBuffer(std::get<0>(entry), true));
+        if (!pool_) return Status::SUCCESS;
+        size_t arena = 0;
+        CHECK_EXPR_RETURN_FAILURE(eh_pool_assign(pool_, &arena) == EH_OK, "assignBufferPool: %s", eh_last_error());
+        last_arena_bytes_ = arena;
+        for (auto &kv : pending_) {
+            void *ptr = nullptr;
+            size_t bytes = 0;
+            CHECK_EXPR_RETURN_FAILURE(eh_pool_slot(pool_, kv.first, &ptr, &bytes) == EH_OK, "assignBufferPool: %s", eh_last_error());
+            kv.second.first->setBytes(bytes);
+            kv.second.first->assignBuffer(bytes ? ptr : nullptr);
         }
-        intra_buffers_.clear();
-        for (auto &entry : inter_buffers_) entry.first->assignBuffer(allocBuffer(entry.first->getBytes(), false));
-        inter_buffers_.clear();
+        pending_.clear();
         return Status::SUCCESS;
     }
 
     Status resetIntraBuffer() {
-        for (auto &entry : intra_buffers_) std::get<1>(entry) = false;
+        if (pool_) CHECK_EXPR_RETURN_FAILURE(eh_pool_reset_intra(pool_) == EH_OK, "resetIntraBuffer: %s", eh_last_error());
         return Status::SUCCESS;
     }
 
     Status resetInterBuffer(const std::shared_ptr<HipBuffer> buffer) {
-        for (auto &entry : inter_buffers_) {
-            if (entry.first == buffer) {
-                entry.second = false;
-                return Status::SUCCESS;
-            }
+        auto it = buffer ? pending_.find(buffer->poolSlot()) : pending_.end();
+        if (it == pending_.end() || it->second.first != buffer || it->second.second == EH_POOL_INTRA || !pool_ ||
+            eh_pool_reset_inter(pool_, it->first) != EH_OK) {
+            ERROR_PRINT("HipRuntime::resetInterBuffer: buffer not found\n");
+            return Status::FAILURE;
         }
-        ERROR_PRINT("HipRuntime::resetInterBuffer: buffer not found\n");
-        return Status::FAILURE;
+        return Status::SUCCESS;
     }
 
-    size_t interPoolSize() const { return inter_buffers_.size(); }
-    size_t intraPoolSize() const { return intra_buffers_.size(); }
+    // bytes of the single allocation the last assignBufferPool() made for its pooled buffers
+    size_t lastPoolAllocationBytes() const { return last_arena_bytes_; }
+
+    size_t interPoolSize() const { return countPending(false); }
+    size_t intraPoolSize() const { return countPending(true); }
 
     // 1024 bytes of slack in front, 32 behind, total rounded to 1024, as the reference pads every
     // allocation; the returned pointer is 1024-byte aligned.
@@ -168,6 +146,13 @@ public:
 
     Status releaseBuffer(std::shared_ptr<HipBuffer> buffer) {
         std::lock_guard<std::mutex> lock(mutex_);
+        if (buffer->poolSlot() >= 0) {  // a pooled buffer: its allocation goes when the last buffer in it is released
+            CHECK_EXPR_RETURN_FAILURE(pool_ != nullptr, "HipRuntime::releaseBuffer: no pool");
+            synchronizeLocked();
+            const int rc = eh_pool_release(pool_, buffer->poolSlot());
+            buffer->assignBuffer(nullptr);
+            return rc == EH_OK ? Status::SUCCESS : Status::CL_FAILURE;
+        }
         auto it = allocations_.find(buffer->getDataPtr());
         CHECK_EXPR_RETURN_FAILURE(it != allocations_.end(), "HipRuntime::releaseBuffer: unknown buffer");
         synchronizeLocked();
@@ -181,17 +166,18 @@ public:
         std::lock_guard<std::mutex> lock(mutex_);
         CHECK_EXPR_RETURN_FAILURE(eh_h2d(dst, src, type_bytes * (size_t)num, stream_) == EH_OK, "writeBuffer: %s",
                                   eh_last_error());
-        // the source is pageable host memory the caller may reuse at once: always wait
-        (void)blocking;
-        return synchronizeLocked();
+        // hipMemcpyAsync from pageable host memory returns once the source has been staged, so a non-blocking
+        // write may return here, as clEnqueueWriteBuffer(blocking = CL_FALSE) does after its copy of the source
+        return blocking ? synchronizeLocked() : Status::SUCCESS;
     }
 
     Status readBuffer(void *dst, const void *src, size_t type_bytes, uint32_t num, bool blocking) {
         std::lock_guard<std::mutex> lock(mutex_);
         CHECK_EXPR_RETURN_FAILURE(eh_d2h(dst, src, type_bytes * (size_t)num, stream_) == EH_OK, "readBuffer: %s",
                                   eh_last_error());
-        (void)blocking;
-        return synchronizeLocked();
+        // the destination is pageable host memory: the copy is complete only after the stream has drained, and a
+        // caller that asks for a non-blocking read must synchronize() before it looks (as with clEnqueueReadBuffer)
+        return blocking ? synchronizeLocked() : Status::SUCCESS;
     }
 
     Status copyBuffer(void *dst, const void *src, size_t bytes) {
@@ -221,14 +207,39 @@ private:
         CHECK_EXPR_RETURN_FAILURE(eh_stream_sync(stream_) == EH_OK, "synchronize: %s", eh_last_error());
         return Status::SUCCESS;
     }
-    void sortIntra() {
-        std::sort(intra_buffers_.begin(), intra_buffers_.end(),
-                  [](const IntraEntry &a, const IntraEntry &b) { return std::get<0>(a) < std::get<0>(b); });
+    // One pooled request: the library keeps the protocol's books (which slot a REUSE takes over, how large it has
+    // to be in the end); a slot that is taken over keeps its HipBuffer object, as the reference hands back the same
+    // CLBuffer.
+    std::shared_ptr<HipBuffer> pooled(int kind, size_t bytes) {
+        if (!pool_ && eh_pool_create(&pool_) != EH_OK) {
+            ERROR_PRINT("HipRuntime::getBuffer: %s\n", eh_last_error());
+            return nullptr;
+        }
+        int32_t slot = -1;
+        if (eh_pool_request(pool_, kind, bytes, &slot) != EH_OK) {
+            ERROR_PRINT("HipRuntime::getBuffer: %s\n", eh_last_error());
+            return nullptr;
+        }
+        size_t final_bytes = bytes;
+        (void)eh_pool_slot(pool_, slot, nullptr, &final_bytes);
+        auto it = pending_.find(slot);
+        if (it != pending_.end()) {
+            it->second.first->setBytes(final_bytes);
+            return it->second.first;
+        }
+        auto buffer = std::make_shared<HipBuffer>(final_bytes, slot);
+        pending_[slot] = std::make_pair(buffer, kind);
+        return buffer;
+    }
+    size_t countPending(bool intra) const {
+        size_t n = 0;
+        for (auto &kv : pending_) n += (kv.second.second == EH_POOL_INTRA) == intra ? 1 : 0;
+        return n;
     }
 
-    typedef std::tuple<size_t, bool, std::shared_ptr<HipBuffer>> IntraEntry;
-    std::vector<std::pair<std::shared_ptr<HipBuffer>, bool>> inter_buffers_;
-    std::vector<IntraEntry> intra_buffers_;
+    eh_pool *pool_ = nullptr;
+    std::map<int32_t, std::pair<std::shared_ptr<HipBuffer>, int>> pending_;  // slots requested since the last assignment
+    size_t last_arena_bytes_ = 0;
     std::map<void *, void *> allocations_;  // user pointer -> hipMalloc base
     std::mutex mutex_;
     void *stream_ = nullptr;

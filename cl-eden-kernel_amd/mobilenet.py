@@ -197,20 +197,54 @@ class MobileNetV2:
     is then never written.  Results are the same bit for bit.
 
     per_channel: convolutions and depthwise convolutions take int8 weights with one scale per output channel
-    (`op_weights_perchannel`); tensors stay uint8 and the classifier keeps its per-tensor uint8 weights."""
+    (`op_weights_perchannel`); tensors stay uint8 and the classifier keeps its per-tensor uint8 weights.
 
-    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False, per_channel=False, weights="minmax"):
+    pooled: feature maps live in the library's buffer pool as the reference's operator constructor places them
+    (gpu_op_constructor.cc:2157-2191): an operator's output is requested with INTER_SHARED_REUSE, then the inputs it
+    is the last reader of are handed back, and once the list is built one device allocation holds them all
+    (`pool_bytes`).  A feature map's storage is then taken over by later ones (the network input is kept), so only
+    the input and the logits can be read back after a run; without it every tensor keeps a buffer of its own (`tensor()` works for all)."""
+
+    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False, per_channel=False, weights="minmax", pooled=False):
         self.eden, self.batch, self.image = eden, batch, image
         self.tensors, self.ops = layers(image, weights)
-        self.buffers = [eden.DeviceBuffer(nbytes=batch * t["h"] * t["w"] * t["c"]) for t in self.tensors]
         self.steps = []
         self._keep = []
         self.unwritten = set()  # tensors a fused step skips
+        self.pooled = pooled
         readers = {}
         for op in self.ops:
             for key in ("src", "a", "b"):
                 if key in op:
                     readers[op[key]] = readers.get(op[key], 0) + 1
+        # a fused convolution + add never stores the projection's own tensor: find those before placing buffers
+        if fuse_add:
+            for index, op in enumerate(self.ops):
+                if (op["op"] == "add" and index > 0 and self.ops[index - 1]["op"] == "conv" and self.ops[index - 1]["dst"] == op["b"]
+                        and readers.get(op["b"], 0) == 1):
+                    self.unwritten.add(op["b"])
+        size = lambda i: batch * self.tensors[i]["h"] * self.tensors[i]["w"] * self.tensors[i]["c"]
+        if pooled:
+            self.pool = eden.BufferPool()
+            self.buffers = [None] * len(self.tensors)
+            self.buffers[0] = self.pool.request(eden.POOL_INTER_NEW, size(0))
+            left = dict(readers)
+            left[0] += 1   # the network input keeps its storage, so that a replay reads the same image again
+            for index, op in enumerate(self.ops):
+                if op["dst"] in self.unwritten:
+                    continue   # its reads happen in the add's launch, which is where its inputs are handed back
+                self.buffers[op["dst"]] = self.pool.request(eden.POOL_INTER_REUSE, size(op["dst"]))
+                reads = [op[k] for k in ("src", "a", "b") if k in op and op[k] not in self.unwritten]
+                if op["op"] == "add" and op["b"] in self.unwritten:
+                    reads.append(self.ops[index - 1]["src"])   # the fused launch reads the projection's input
+                for t in reads:
+                    left[t] -= 1
+                    if left[t] == 0:
+                        self.pool.reset_inter(self.buffers[t])
+            self.pool_bytes = self.pool.assign()
+        else:
+            self.buffers = [eden.DeviceBuffer(nbytes=size(i)) for i in range(len(self.tensors))]
+            self.pool_bytes = None
         for index, op in enumerate(self.ops):
             kind = op["op"]
             if kind == "add":
@@ -221,7 +255,6 @@ class MobileNetV2:
                     q_add = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
                     plan, src, _, q = prev[1]
                     self.steps[-1] = ("plan_add", (plan, src, self.buffers[op["a"]], self.buffers[op["dst"]], q, q_add))
-                    self.unwritten.add(op["b"])
                     continue
                 a, b, d = (self.tensors[op[k]] for k in ("a", "b", "dst"))
                 q = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])

@@ -171,6 +171,29 @@ int eh_stream_destroy(void *stream);
 int eh_stream_sync(void *stream);
 const char *eh_last_error(void);
 
+/* Pooled buffers of an operator list: CLRuntime::getBuffer with BufferType INTER_SHARED_NEW / INTER_SHARED_REUSE /
+ * INTRA_SHARED, resetInterBuffer, resetIntraBuffer and assignBufferPool (gpu/common/CLRuntime.cpp:34-157), as the
+ * operator constructor drives them (gpu/gpu_op_constructor.cc:2157-2191: an operator's outputs are requested with
+ * REUSE before the inputs it reads last are handed back).  A request returns a slot, sized but without memory;
+ * eh_pool_assign lays every slot requested since the last assignment out in ONE device allocation (each at a
+ * 1024-byte aligned address with the reference's 1024 bytes of slack in front and 32 behind, zero-filled) and, as the
+ * reference does, forgets the pools: later requests collect the next list.  eh_pool_layout reports what an
+ * assignment would allocate without allocating; eh_pool_slot gives a slot's address (null before its assignment)
+ * and final size; eh_pool_release is releaseBuffer for a pooled buffer (the allocation is freed with its last
+ * slot); eh_pool_destroy frees whatever is left.  Not thread-safe: one builder at a time, as under the reference's
+ * constructor mutex. */
+typedef struct eh_pool eh_pool;
+typedef enum eh_pool_kind { EH_POOL_INTER_NEW = 0, EH_POOL_INTER_REUSE = 1, EH_POOL_INTRA = 2 } eh_pool_kind;
+int eh_pool_create(eh_pool **pool);
+int eh_pool_request(eh_pool *pool, int kind, size_t bytes, int32_t *slot);
+int eh_pool_reset_inter(eh_pool *pool, int32_t slot);
+int eh_pool_reset_intra(eh_pool *pool);
+int eh_pool_layout(eh_pool *pool, size_t *arena_bytes, int32_t *slot_count);
+int eh_pool_assign(eh_pool *pool, size_t *arena_bytes);
+int eh_pool_slot(const eh_pool *pool, int32_t slot, void **ptr, size_t *bytes);
+int eh_pool_release(eh_pool *pool, int32_t slot);
+int eh_pool_destroy(eh_pool *pool);
+
 /* Replay of a fixed launch sequence.  The reference submits a whole subgraph to
  * one in-order queue and flushes once (gpu/gpu_userdriver.cc:78-112); on HIP the
  * same sequence is captured once and replayed as a graph, which removes the

@@ -7,6 +7,7 @@ import os
 import re
 
 import numpy as np
+import pytest
 
 import oracle_lib as O
 from harness import eden
@@ -155,3 +156,64 @@ def test_3x3_stride_1_convolutions_take_the_patch_kernel():
               eden.conv_desc(1, 48, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc),
               eden.conv_desc(4, 64, 7, 7, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)):
         assert "conv3x3_patch" not in eden.conv_kernels(d)
+
+
+def test_buffer_pool_protocol_without_a_gpu():
+    """request / reset / layout are host bookkeeping (CLRuntime.cpp:34-118, 147-157): a REUSE request takes over the
+    first feature map handed back and grows it, intra-operator scratch is sized to the largest request per slot, and
+    the layout is one allocation with 1024 bytes in front of and 32 behind every buffer, rounded to 1024."""
+    pool = eden.BufferPool()
+    a = pool.request(eden.POOL_INTER_NEW, 128)
+    b = pool.request(eden.POOL_INTER_REUSE, 512)          # nothing handed back yet: a new slot
+    assert b.slot != a.slot
+    pool.reset_inter(a)
+    c = pool.request(eden.POOL_INTER_REUSE, 1024)         # takes a over, grown
+    assert c.slot == a.slot and a.nbytes == 1024
+    d = pool.request(eden.POOL_INTER_REUSE, 16)
+    assert d.slot not in (a.slot, b.slot)
+    pool.reset_inter(b)
+    e = pool.request(eden.POOL_INTER_REUSE, 100)          # smaller than what b holds: b keeps its size
+    assert e.slot == b.slot and b.nbytes == 512
+    s1 = pool.request(eden.POOL_INTRA, 400)
+    s2 = pool.request(eden.POOL_INTRA, 200)
+    assert s1.slot != s2.slot
+    pool.reset_intra()
+    s3 = pool.request(eden.POOL_INTRA, 320)               # the free one that is already large enough
+    assert s3.slot == s1.slot and s1.nbytes == 400
+    s4 = pool.request(eden.POOL_INTRA, 1200)              # the remaining free one, grown
+    assert s4.slot == s2.slot and s2.nbytes == 1200
+    nbytes, slots = pool.layout()
+    assert slots == 5
+    pad = lambda n: (1024 + n + 32 + 1023) // 1024 * 1024
+    assert nbytes == pad(1024) + pad(512) + pad(16) + pad(400) + pad(1200)
+    assert a.ptr.value is None                            # no memory before the assignment
+    with pytest.raises(eden.EdenHipError):
+        pool.reset_inter(s1)                              # not a feature map
+
+
+def test_mobilenet_pool_is_a_fraction_of_one_buffer_per_tensor():
+    """Liveness reuse over the MobileNetV2 operator list (gpu_op_constructor.cc:2157-2191), on the host: replaying
+    the list's requests and releases through the pool gives far fewer buffers than tensors."""
+    import importlib
+    mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+    tensors, ops = mobilenet.layers(224)
+    batch = 64
+    size = lambda i: batch * tensors[i]["h"] * tensors[i]["w"] * tensors[i]["c"]
+    readers = {}
+    for op in ops:
+        for key in ("src", "a", "b"):
+            if key in op:
+                readers[op[key]] = readers.get(op[key], 0) + 1
+    pool = eden.BufferPool()
+    bufs = {0: pool.request(eden.POOL_INTER_NEW, size(0))}
+    for op in ops:
+        bufs[op["dst"]] = pool.request(eden.POOL_INTER_REUSE, size(op["dst"]))
+        for t in [op[k] for k in ("src", "a", "b") if k in op]:
+            readers[t] -= 1
+            if readers[t] == 0:
+                pool.reset_inter(bufs[t])
+        # an operator's output never shares storage with what it reads
+        assert all(bufs[op["dst"]].slot != bufs[op[k]].slot for k in ("src", "a", "b") if k in op)
+    nbytes, slots = pool.layout()
+    assert slots <= 4
+    assert nbytes < 0.45 * sum(size(i) for i in range(len(tensors)))

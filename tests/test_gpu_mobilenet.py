@@ -84,6 +84,27 @@ def test_mobilenet_v2_full_batch_64(per_channel, weights):
     assert_network_alive(ops, want, 2)
 
 
+@pytest.mark.parametrize("per_channel", [False, True], ids=["per_tensor", "per_channel"])
+def test_mobilenet_v2_on_pooled_buffers_batch_64(per_channel):
+    """The network as the benchmark runs it: feature maps in the library's buffer pool (liveness reuse, one device
+    allocation), batch 64, one graph replay; the logits of every image must equal the oracle's for its image of the
+    repeated pair, on two replays."""
+    batch = 64
+    tensors, ops, want = oracle_pair(per_channel, "minmax")
+    net = mobilenet.MobileNetV2(eden, batch, 224, fuse_add=True, per_channel=per_channel, pooled=True)
+    assert net.pool_bytes < 0.45 * sum(batch * t["h"] * t["w"] * t["c"] for t in tensors)
+    net.set_input(np.tile(mobilenet.network_input(2), (batch // 2, 1, 1, 1)))
+    stream = eden.Stream()
+    graph = eden.Graph(stream, lambda s: net.run(s))
+    ref = want[-1].reshape(2, -1)
+    for rep in range(2):
+        graph.launch(stream)
+        stream.sync()
+        got = net.logits()
+        for img in range(batch):
+            assert np.array_equal(got[img], ref[img % 2]), (rep, img)
+
+
 def test_mobilenet_v2_graph_replay_equals_eager():
     """The whole operator list captured once; every replay (with eager work between replays) gives the eager logits."""
     batch, image = 2, 96
