@@ -156,6 +156,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
     __shared__ int32_t rowsum_s[WGK * 2][BM];
     __shared__ __align__(16) int32_t bias_s[BN];  // read in the epilogue from LDS: a global load there would have to
                                                    // wait for the stores issued before it (one counter for both)
+    // fused residual add (split-reduction epilogue only): the rescaled value of every possible residual byte and of
+    // every possible result byte, so that an output costs two lookups and one rescaling instead of three rescalings
+    __shared__ int32_t add_lut_s[WGK == 1 ? 1 : 2][WGK == 1 ? 1 : 256];
     extern __shared__ __align__(8) uint8_t ktab_s_raw[];
     KUnit *ktab_s = reinterpret_cast<KUnit *>(ktab_s_raw);
 
@@ -167,26 +170,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
     // L2 once for gn tiles and every weight slab once for gm tiles.  Equally shaped
     // problems of one operator (convolution groups, deconvolution phases) share a launch:
     // their groups are numbered one problem after the other.
-    const int gs = gm * gn;
+    // Rectangles leave slots empty where they overhang the tile grid.  A launch with few tiles cannot afford that (the
+    // empty slots push real tiles into a second round of workgroups): gm == 0 selects a plain split instead, every XCD
+    // taking gn consecutive tiles of the problems' tiles in row-major order (neighbours share their activation rows).
     const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-    const int jg = __builtin_amdgcn_readfirstlane(j / gs);
-    const int group_all = jg * 8 + xcd, within = j - jg * gs;
-    const int groups_m = (tiles_m + gm - 1) / gm, groups_n = (tiles_n + gn - 1) / gn;
-    // (the divisions run on the vector unit: tell the compiler their results are wave-uniform)
-    const int which = __builtin_amdgcn_readfirstlane(group_all / (groups_m * groups_n));
-    const int group = group_all - which * (groups_m * groups_n);
-    if (which >= count) return;
+    int which, tm, tn;
+    if (gm == 0) {
+        const int t_all = xcd * gn + j;
+        const int per_problem = tiles_m * tiles_n;
+        which = __builtin_amdgcn_readfirstlane(t_all / per_problem);
+        const int t = t_all - which * per_problem;
+        tm = __builtin_amdgcn_readfirstlane(t / tiles_n);
+        tn = t - tm * tiles_n;
+        if (which >= count) return;
+    } else {
+        const int gs = gm * gn;
+        const int jg = __builtin_amdgcn_readfirstlane(j / gs);
+        const int group_all = jg * 8 + xcd, within = j - jg * gs;
+        const int groups_m = (tiles_m + gm - 1) / gm, groups_n = (tiles_n + gn - 1) / gn;
+        // (the divisions run on the vector unit: tell the compiler their results are wave-uniform)
+        which = __builtin_amdgcn_readfirstlane(group_all / (groups_m * groups_n));
+        const int group = group_all - which * (groups_m * groups_n);
+        if (which >= count) return;
+        const int gj = __builtin_amdgcn_readfirstlane(group / groups_m), gi = group - gj * groups_m;
+        const int wj = __builtin_amdgcn_readfirstlane(within / gm), wi = within - wj * gm;
+        tm = gi * gm + wi;
+        tn = gj * gn + wj;
+        if (tm >= tiles_m || tn >= tiles_n) return;
+    }
     const GemmProblem &p = batch.p[which];
-    const int gj = __builtin_amdgcn_readfirstlane(group / groups_m), gi = group - gj * groups_m;
-    const int wj = __builtin_amdgcn_readfirstlane(within / gm), wi = within - wj * gm;
-    const int tm = gi * gm + wi, tn = gj * gn + wj;
-    if (tm >= tiles_m || tn >= tiles_n) return;
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63;
     // issued first and consumed after the main loop: by then it has long arrived
     static_assert(BN <= 256, "one bias value per thread");
     const int32_t bias_reg = tid < BN ? p.bias[n0 + tid] : 0;
+    if constexpr (WGK != 1) {
+        if (p.residual) {  // 256 threads, 256 byte values; visible after the barriers that precede the epilogue
+            add_lut_s[0][tid] = mul_round_shift((int32_t)((uint32_t)(tid - p.radd.zp_a) << p.radd.left_shift), p.radd.mult_a, p.radd.rs_a);
+            add_lut_s[1][tid] = mul_round_shift((int32_t)((uint32_t)(tid - p.radd.zp_b) << p.radd.left_shift), p.radd.mult_b, p.radd.rs_b);
+        }
+    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = (wave / WGM) % WGN, wk = wave / (WGM * WGN);
     const int k_slabs = p.k_pad / SLAB;
@@ -563,10 +587,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
             const uint8_t *res = p.residual + out_off;
             if (aligned16 && n + 16 <= p.n && (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) {
                 const uint4 rv = *reinterpret_cast<const uint4 *>(res);
-                packed[0] = add_word(rv.x, packed[0], p.radd);
-                packed[1] = add_word(rv.y, packed[1], p.radd);
-                packed[2] = add_word(rv.z, packed[2], p.radd);
-                packed[3] = add_word(rv.w, packed[3], p.radd);
+                // add_word with the two tables (the same arithmetic: the tables hold what add_one computes first)
+                auto add_word_lut = [&](uint32_t a, uint32_t b) {
+                    uint32_t o = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int32_t sum = add_lut_s[0][(a >> (8 * i)) & 255u] + add_lut_s[1][(b >> (8 * i)) & 255u];
+                        int32_t v = mul_round_shift(sum, p.radd.mult_out, p.radd.rs_out) + p.radd.zp_out;
+                        v = v < p.radd.act_min ? p.radd.act_min : v;
+                        v = v > p.radd.act_max ? p.radd.act_max : v;
+                        o |= (uint32_t)v << (8 * i);
+                    }
+                    return o;
+                };
+                packed[0] = add_word_lut(rv.x, packed[0]);
+                packed[1] = add_word_lut(rv.y, packed[1]);
+                packed[2] = add_word_lut(rv.z, packed[2]);
+                packed[3] = add_word_lut(rv.w, packed[3]);
             } else {
                 const int cnt = p.n - n < 16 ? p.n - n : 16;
                 for (int t = 0; t < cnt; ++t) {
@@ -607,9 +644,17 @@ int launch_cfg(const GemmProblem *ps, int count, hipStream_t stream) {
             gm = cand;
         }
     }
-    const int gn = gs / gm;
+    int gn = gs / gm;
     const int groups = ((tiles_m + gm - 1) / gm) * ((tiles_n + gn - 1) / gn) * count;
-    const int grid = ((groups + 7) / 8) * 8 * gs;
+    int grid = ((groups + 7) / 8) * 8 * gs;
+    // rectangles that overhang the tile grid leave workgroup slots empty; where that costs a launch of up to a few
+    // rounds more than an eighth of its slots, split the tiles evenly over the XCDs instead
+    const long tiles_all = (long)tiles_m * tiles_n * count;
+    if (tiles_all <= 1024 && (long)grid * 8 > tiles_all * 9) {
+        gm = 0;
+        gn = (int)((tiles_all + 7) / 8);  // tiles per XCD
+        grid = gn * 8;
+    }
     const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
     // the per-row activation sums are only carried when the weight zero point is not 128
     if (p.dense) {
