@@ -35,9 +35,20 @@ typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
 // QM: how results are requantized.  0: the two-step order (one pair, or one per channel read from global memory);
 // 1: the single-shift form with the requant's one pair; 2: the single-shift form with one pair per channel, whose
 // multiplier, shift and rounding term sit in LDS beside the bias.
+// Output staging (stage_pitch != 0; launches whose workgroups own whole pixels of a densely stored output, no residual):
+// a lane's sixteen bytes go to a per-wave LDS image of the block's 32 pixels first, and the wave then writes that
+// image out as one contiguous span, 16 bytes per lane.  A pixel block's output is contiguous in memory (32 x ldc
+// bytes), but a lane holds 16 channels of one pixel, so storing from the accumulator layout makes every store
+// instruction touch 32 separate sectors of 32 bytes; from the image it writes whole 128-byte lines.
+struct ThinStage {
+    int32_t pitch;     // LDS bytes per pixel of the image (an odd number of 16-byte chunks), 0: store directly
+    int32_t offset;    // byte offset of the four waves' images in dynamic LDS
+    FastDiv div_cpp;   // chunks of 16 bytes per pixel: ldc / 16
+};
+
 template <int NBU, int KU, bool ROWSUM, int QM, bool RES>
 __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps, const int nbw,
-                                                          const int row_blocks) {
+                                                          const int row_blocks, const ThinStage stage) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, half = lane >> 5;
     const int plane = p.ho * p.wo;
@@ -185,6 +196,14 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
             quantize(std::integral_constant<int, 2>{});
         else
             quantize(std::integral_constant<int, 1>{});
+        if constexpr (!RES) {
+            if (stage.pitch) {  // (every channel block is whole here: the launcher asks for n % 16 == 0)
+                if (n < p.n)
+                    *reinterpret_cast<uint4 *>(lds_raw + stage.offset + (wave * 32 + r) * stage.pitch + n) =
+                        make_uint4(packed[0], packed[1], packed[2], packed[3]);
+                return;
+            }
+        }
         if (!ok || n >= p.n) return;
         uint8_t *dst = p.out + out_off + n;
         const int cnt = p.n - n;
@@ -211,6 +230,19 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         } else {
             const int c = cnt < 16 ? cnt : 16;
             for (int t = 0; t < c; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+        }
+    };
+
+    // writes the wave's staged image of row block `rb` out as one contiguous span
+    auto flush_stage = [&](int rb) {
+        const int first = rb * 32;
+        const int pixels = p.m - first < 32 ? p.m - first : 32;
+        const int cpp = p.ldc >> 4, chunks = pixels * cpp;
+        const uint8_t *img = lds_raw + stage.offset + wave * 32 * stage.pitch;
+        uint8_t *dst = p.out + (size_t)first * (size_t)p.ldc;
+        for (int c = lane; c < chunks; c += 64) {
+            const int px = (int)fastdiv((uint32_t)c, stage.div_cpp), col = c - px * cpp;
+            *reinterpret_cast<uint4 *>(dst + (size_t)c * 16) = *reinterpret_cast<const uint4 *>(img + px * stage.pitch + col * 16);
         }
     };
 
@@ -254,6 +286,9 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                     for (int t = 0; t < KU; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[u][t], af[t], acc, 0, 0, 0);
                     finish_block(acc, nb0 + u, 0, ok, out_off);
                 }
+            }
+            if constexpr (!RES) {
+                if (stage.pitch) flush_stage(rb);
             }
             ok = ok_next;
             in_off = in_next;
@@ -302,6 +337,9 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                     finish_block(acc[u], nb0 + u, ncorr, ok, out_off);
                 }
             }
+            if constexpr (!RES) {
+                if (stage.pitch) flush_stage(rb);
+            }
         }
     }
 }
@@ -316,6 +354,9 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     int nbw_max = (32 / ksteps) / NBU * NBU;
     if (nbw_max < NBU) nbw_max = NBU;
     int ranges = (n_blocks + nbw_max - 1) / nbw_max;
+    const bool dense_out = p.out_sy == 1 && p.out_sx == 1 && p.out_y0 == 0 && p.out_x0 == 0 && p.out_h == p.ho && p.out_w == p.wo;
+    const bool stageable = !p.residual && p.n == p.ldc && (p.n & 15) == 0 && p.n <= 256 && dense_out &&
+                           (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
     while (ranges < groups_total && (long)row_blocks * ranges < 4096) ++ranges;
     const int nbw = (groups_total + ranges - 1) / ranges * NBU;
     ranges = (n_blocks + nbw - 1) / nbw;
@@ -327,11 +368,22 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t) * (pc_fast ? 4 : 1) +
                        (p.residual ? 2 * 256 * sizeof(int32_t) : 0);
     EH_REQUIRE(lds <= 64 * 1024, "igemm_thin: %zu bytes of LDS for the weights", lds);
+    // Staged output where a workgroup owns whole, densely stored pixels of at most 256 bytes (wider pixels already fill
+    // whole lines per store, and the images would crowd the CU's LDS)
+    ThinStage stage{};
+    if (ranges == 1 && stageable) {
+        const int cpp = p.ldc / 16;
+        stage.pitch = (cpp | 1) * 16;
+        stage.offset = (int32_t)((lds + 15) / 16 * 16);
+        stage.div_cpp = make_fastdiv((uint32_t)cpp);
+        if ((size_t)stage.offset + 4u * 32u * stage.pitch > 64 * 1024) stage = ThinStage{};
+    }
+    const size_t lds_all = stage.pitch ? (size_t)stage.offset + 4u * 32u * stage.pitch : lds;
     // row sums, the single-shift requantization and the fused residual add are compile-time variants: a launch pays for
     // none of the code it does not use
     auto launch = [&](auto rowsum_c, auto qm_c, auto res_c) {
         hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(res_c)::value>), grid,
-                           dim3(256), lds, stream, p, n_blocks, ksteps, nbw, row_blocks);
+                           dim3(256), lds_all, stream, p, n_blocks, ksteps, nbw, row_blocks, stage);
     };
     auto with_res = [&](auto rowsum_c, auto qm_c) {
         if (p.residual)

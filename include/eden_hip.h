@@ -242,7 +242,14 @@ int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *str
  * execution.  Passing a requant whose zero points differ from the plan's
  * re-folds the bias first (the reference reads quantization parameters from
  * the tensors on every execute).  `*_repack` is the weights-as-input case:
- * the reference re-packs non-constant weights on every execute. */
+ * the reference re-packs non-constant weights on every execute.
+ *
+ * A plan belongs to ONE stream at a time, like the reference's operators on their single in-order queue: the
+ * re-fold and re-pack rewrite the plan's own device arrays in stream order, so work queued on another stream, or a
+ * captured graph, that still uses the plan must have finished (or must never be replayed again) before a `*_run`
+ * with other zero points, a `*_repack` or a `*_set_perchannel` on it.  In particular the zero points (and, in
+ * per-channel mode, the pairs) a plan was captured with have to stay the same for as long as the graph is replayed:
+ * `*_run` bakes them into the kernel arguments it records, while the folded bias they must match lives in the plan. */
 typedef struct eh_conv_plan eh_conv_plan;
 typedef struct eh_dwconv_plan eh_dwconv_plan;
 typedef struct eh_fc_plan eh_fc_plan;

@@ -187,6 +187,11 @@ CONV_CASES = [
     dict(n=2, c=64, h=12, w=12, cout=32, kh=1, kw=1),
     dict(n=1, c=48, h=10, w=10, cout=96, kh=1, kw=1, groups=2),                             # 24-byte rows inside 48-byte pixels
     dict(n=5, c=16, h=33, w=5, cout=96, kh=1, kw=1, stride=(1, 2)),
+    # ... whose output leaves through the per-wave LDS image: one 16-byte chunk per pixel, the widest pixel (256 bytes),
+    # a last pixel block of three pixels
+    dict(n=1, c=32, h=5, w=7, cout=16, kh=1, kw=1),
+    dict(n=2, c=32, h=9, w=9, cout=256, kh=1, kw=1),
+    dict(n=1, c=64, h=7, w=5, cout=208, kh=1, kw=1),
     # one tap with bottom / right padding: output pixels whose only tap lies outside the image (they read the zero
     # point); the one-tap kernel must not be chosen
     dict(n=2, c=24, h=14, w=14, cout=144, kh=1, kw=1, pad=(0, 1, 0, 1)),
