@@ -216,11 +216,12 @@ def probe_mfma_i8(iterations=100000, toggling_operands=True):
 
 def requant_apply(q, acc, two_step=False, channel_form=None):
     """Host evaluation of the kernels' requantization of int32 accumulators; returns (uint8 array, used_single_shift).
-    channel_form: "registers" or "table" evaluates the per-channel single-shift forms with q's pair as the channel's."""
+    channel_form: "registers" or "table" evaluates the per-channel single-shift forms with q's pair as the channel's;
+    "packed" the per-tensor single-shift form four outputs at a time with a row term folded into the rounding term."""
     acc = np.ascontiguousarray(acc, np.int32)
     out = np.empty(acc.shape, np.uint8)
     used = C.c_int32(0)
-    form = {None: 1 if two_step else 0, "registers": 2, "table": 3}[channel_form]
+    form = {None: 1 if two_step else 0, "registers": 2, "table": 3, "packed": 4}[channel_form]
     check(load().eh_requant_apply(C.addressof(q), acc.ctypes.data, out.ctypes.data, acc.size, form, C.addressof(used)))
     return out, bool(used.value)
 

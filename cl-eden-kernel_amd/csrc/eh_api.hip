@@ -476,9 +476,9 @@ int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int6
     int rc = check_requant(q);
     if (rc) return rc;
     EH_REQUIRE(count >= 0 && (count == 0 || (acc && out)), "requant_apply: null array");
-    EH_REQUIRE(form >= 0 && form <= 3, "requant_apply: form %d", form);
+    EH_REQUIRE(form >= 0 && form <= 4, "requant_apply: form %d", form);
     const RequantDev r = make_requant_dev(*q);
-    if (form >= 2) {  // the per-channel single-shift forms, with the requant's pair as the channel's
+    if (form == 2 || form == 3) {  // the per-channel single-shift forms, with the requant's pair as the channel's
         EH_REQUIRE(channel_pair_is_fast(q->multiplier, q->shift, form == 3 ? -2 : -1) && channel_fast_mode(*q) != 0,
                    "requant_apply: multiplier %d, shift %d, zero point %d are outside form %d", q->multiplier, q->shift, q->zp_out, form);
         const int mode = channel_fast_mode(*q), rs = -q->shift;
@@ -491,6 +491,18 @@ int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int6
                 v = mode == 2 ? requant_u8_channel_table<2>(acc[i], q->multiplier, rs - 1, channel_table_pos_hi(q->zp_out, rs), r)
                               : requant_u8_channel_table<1>(acc[i], q->multiplier, rs - 1, channel_table_pos_hi(q->zp_out, rs), r);
             out[i] = (uint8_t)v;
+        }
+        return EH_OK;
+    }
+    if (form == 4) {  // four at a time, a row term of up to +-4000 (varying with the group) held back from the accumulators
+        EH_REQUIRE(r.fast != 0, "requant_apply: multiplier %d, shift %d, zero point %d are outside form 4", q->multiplier, q->shift, q->zp_out);
+        if (single_shift) *single_shift = 1;
+        for (int64_t i = 0; i < count; i += 4) {
+            const int32_t extra = (int32_t)(((uint64_t)(i + 1) * 2654435761ull >> 13) % 8001) - 4000;
+            int32_t x[4];
+            for (int t = 0; t < 4; ++t) x[t] = (int32_t)((uint32_t)acc[i + t < count ? i + t : count - 1] - (uint32_t)extra);
+            const uint32_t w = r.fast == 2 ? requant4_fast<2>(x[0], x[1], x[2], x[3], extra, r) : requant4_fast<1>(x[0], x[1], x[2], x[3], extra, r);
+            for (int t = 0; t < 4 && i + t < count; ++t) out[i + t] = (uint8_t)(w >> (8 * t));
         }
         return EH_OK;
     }

@@ -181,15 +181,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
 #pragma unroll
             for (int g = 0; g < G; ++g) acc[g][nb] = b16;
         }
-        if constexpr (ROWSUM) {
-            // -(zp_w - 128) * sum of the pixel's 9 * C signed activations, known before the first product: the
-            // accumulators start from it, so the epilogue has nothing left to add
+        // -(zp_w - 128) * sum of the pixel's 9 * C signed activations.  The per-tensor single-shift forms take it inside
+        // their rounding term, in the epilogue (one multiply-add per pixel and no register held across the products);
+        // otherwise the accumulators start from it, so the epilogue has nothing left to add
+        constexpr bool late_corr = ROWSUM && QM != 0 && !PC;
+        auto pixel_term = [&](int g) {
+            int rs = 0;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) rs += *reinterpret_cast<const int *>(patch + base[g] + ((t / 3) * L.pc + t % 3) * L.pitch + p.cin);
+            return -p.zw * rs;
+        };
+        if constexpr (ROWSUM && !late_corr) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
-                int rs = 0;
-#pragma unroll
-                for (int t = 0; t < 9; ++t) rs += *reinterpret_cast<const int *>(patch + base[g] + ((t / 3) * L.pc + t % 3) * L.pitch + p.cin);
-                const int ncorr = -p.zw * rs;
+                const int ncorr = pixel_term(g);
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -234,6 +239,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             const int pidx = (g0 + 4 * g) * 32 + r;
             const bool ok = g < ng && pidx < pixels;
             uint8_t *const row = p.out + out_tile + (size_t)(ok ? pidx : 0) * (size_t)p.ldc;
+            int late = 0;
+            if constexpr (late_corr) late = pixel_term(g);
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 const int n = (nb_first + nb) * 32 + half * 16;
@@ -253,6 +260,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                             o0 = requant_u8_channel(x0, cm.x, cs.x, rq), o1 = requant_u8_channel(x1, cm.y, cs.y, rq);
                             o2 = requant_u8_channel(x2, cm.z, cs.z, rq), o3 = requant_u8_channel(x3, cm.w, cs.w, rq);
                         }
+                    } else if constexpr (QM != 0) {
+                        packed[q4] = requant4_fast<QM>(x0, x1, x2, x3, late, rq) ^ p.out_xor;
+                        continue;
                     } else {
                         o0 = requant_u8_as<QM>(x0, rq), o1 = requant_u8_as<QM>(x1, rq);
                         o2 = requant_u8_as<QM>(x2, rq), o3 = requant_u8_as<QM>(x3, rq);

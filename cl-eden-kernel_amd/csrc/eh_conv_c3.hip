@@ -162,9 +162,12 @@ __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p
                                     p.out_xor;
                         continue;
                     }
-                    packed[g] = pack_bytes(requant_u8_as<mode>(acc[g * 4 + 0], rq), requant_u8_as<mode>(acc[g * 4 + 1], rq),
-                                           requant_u8_as<mode>(acc[g * 4 + 2], rq), requant_u8_as<mode>(acc[g * 4 + 3], rq)) ^
-                                p.out_xor;
+                    if constexpr (mode != 0)
+                        packed[g] = requant4_fast<mode>(acc[g * 4 + 0], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3], 0, rq) ^ p.out_xor;
+                    else
+                        packed[g] = pack_bytes(requant_u8_as<mode>(acc[g * 4 + 0], rq), requant_u8_as<mode>(acc[g * 4 + 1], rq),
+                                               requant_u8_as<mode>(acc[g * 4 + 2], rq), requant_u8_as<mode>(acc[g * 4 + 3], rq)) ^
+                                    p.out_xor;
                 }
             };
             if constexpr (!FAST)

@@ -53,11 +53,8 @@ __device__ __forceinline__ uint32_t requant4(int acc0, int acc1, int acc2, int a
     if (PC && rq.pc_multiplier)  // the two-step order; the single-shift form per channel is the dot product kernel's
         return pack_bytes(requant_u8_channel(acc0, cq.m.x, cq.s.x, rq), requant_u8_channel(acc1, cq.m.y, cq.s.y, rq),
                           requant_u8_channel(acc2, cq.m.z, cq.s.z, rq), requant_u8_channel(acc3, cq.m.w, cq.s.w, rq));
-    if (rq.fast == 2)
-        return pack_bytes(requant_u8_fast_relu(acc0, rq), requant_u8_fast_relu(acc1, rq),
-                          requant_u8_fast_relu(acc2, rq), requant_u8_fast_relu(acc3, rq));
-    if (rq.fast)
-        return pack_bytes(requant_u8_fast(acc0, rq), requant_u8_fast(acc1, rq), requant_u8_fast(acc2, rq), requant_u8_fast(acc3, rq));
+    if (rq.fast == 2) return requant4_fast<2>(acc0, acc1, acc2, acc3, 0, rq);
+    if (rq.fast) return requant4_fast<1>(acc0, acc1, acc2, acc3, 0, rq);
     return pack_bytes(requant_u8(acc0, rq), requant_u8(acc1, rq), requant_u8(acc2, rq), requant_u8(acc3, rq));
 }
 

@@ -463,6 +463,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
                             o1 = requant_u8_channel(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], cm[g].y, cs[g].y, rq);
                             o2 = requant_u8_channel(acc[i][j][g * 4 + 2] + bb[g].z + ncorr[i], cm[g].z, cs[g].z, rq);
                             o3 = requant_u8_channel(acc[i][j][g * 4 + 3] + bb[g].w + ncorr[i], cm[g].w, cs[g].w, rq);
+                        } else if constexpr (fast != 0) {
+                            packed[g] = requant4_fast<fast>(acc[i][j][g * 4 + 0] + bb[g].x, acc[i][j][g * 4 + 1] + bb[g].y,
+                                                            acc[i][j][g * 4 + 2] + bb[g].z, acc[i][j][g * 4 + 3] + bb[g].w, ncorr[i], rq) ^
+                                        p.out_xor;
+                            continue;
                         } else {
                             o0 = requant_u8_as<fast>(acc[i][j][g * 4 + 0] + bb[g].x + ncorr[i], rq);
                             o1 = requant_u8_as<fast>(acc[i][j][g * 4 + 1] + bb[g].y + ncorr[i], rq);
@@ -567,6 +572,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
                     o2 = requant_u8_channel(s4.z + bb.z - corr, cm.z, cs.z, rq);
                     o3 = requant_u8_channel(s4.w + bb.w - corr, cm.w, cs.w, rq);
                 }
+            } else if constexpr (fast != 0) {
+                packed[g] = requant4_fast<fast>(s4.x + bb.x, s4.y + bb.y, s4.z + bb.z, s4.w + bb.w, -corr, rq) ^ p.out_xor;
+                continue;
             } else {
                 o0 = requant_u8_as<fast>(s4.x + bb.x - corr, rq), o1 = requant_u8_as<fast>(s4.y + bb.y - corr, rq);
                 o2 = requant_u8_as<fast>(s4.z + bb.z - corr, rq), o3 = requant_u8_as<fast>(s4.w + bb.w - corr, rq);

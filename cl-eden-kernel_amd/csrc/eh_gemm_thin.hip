@@ -142,7 +142,8 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
     };
     // The accumulators start from the folded bias (plus `extra`, the pixel's row-sum term where it is known before the
     // products): the matrix instruction adds to them, so the epilogue has no additions left to do.
-    auto start_block = [&](int nb_local, int extra) {
+    constexpr bool late_corr = ROWSUM && QM == 1;
+    auto start_block = [&](int nb_local, int extra = 0) {
         const int32_t *bsrc = bias_s + nb_local * 32 + half * 16;
         v16i acc;
 #pragma unroll
@@ -181,6 +182,9 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
                     o1 = requant_u8_channel(acc[g * 4 + 1] + ncorr, cm.y, cs.y, rq);
                     o2 = requant_u8_channel(acc[g * 4 + 2] + ncorr, cm.z, cs.z, rq);
                     o3 = requant_u8_channel(acc[g * 4 + 3] + ncorr, cm.w, cs.w, rq);
+                } else if constexpr (mode != 0) {
+                    packed[g] = requant4_fast<mode>(acc[g * 4 + 0], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3], ncorr, rq) ^ p.out_xor;
+                    continue;
                 } else {
                     o0 = requant_u8_as<mode>(acc[g * 4 + 0] + ncorr, rq);
                     o1 = requant_u8_as<mode>(acc[g * 4 + 1] + ncorr, rq);
@@ -281,10 +285,11 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
 #pragma unroll
                 for (int u = 0; u < NBU; ++u) {
                     if (nb0 + u >= nb_count) break;
-                    v16i acc = start_block(nb0 + u, ncorr);
+                    // (the single-shift forms take the pixel's term inside their rounding term: nothing to add per accumulator)
+                    v16i acc = late_corr ? start_block(nb0 + u) : start_block(nb0 + u, ncorr);
 #pragma unroll
                     for (int t = 0; t < KU; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[u][t], af[t], acc, 0, 0, 0);
-                    finish_block(acc, nb0 + u, 0, ok, out_off);
+                    finish_block(acc, nb0 + u, late_corr ? ncorr : 0, ok, out_off);
                 }
             }
             if constexpr (!RES) {

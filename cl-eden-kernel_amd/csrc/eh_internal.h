@@ -45,6 +45,7 @@ struct RequantDev {
     int32_t fast_shift;        // right_shift - 1
     uint32_t pos_lo, pos_hi;   // 64-bit rounding term for accumulators >= 0
     uint32_t neg_lo, neg_hi;   // the same for accumulators < 0
+    int32_t lo_scaled, hi_scaled;  // the clamp of the single-shift form applied before its shift (see requant4_fast)
     // per-output-channel quantization (int8 weights with one scale per channel): device arrays indexed by the
     // problem's own channel number, or null; when set they replace multiplier and shift above
     const int32_t *pc_multiplier;
@@ -124,6 +125,44 @@ __host__ __device__ __forceinline__ uint32_t requant_u8_fast_relu(int32_t x, con
     v = v < r.act_min ? r.act_min : v;
     v = v > r.act_max ? r.act_max : v;
     return (uint32_t)v;
+#endif
+}
+
+// Four outputs of the single-shift form, packed into one word, lowest byte first, in three instructions each (MODE 2)
+// or six (MODE 1).  `extra` is an addend that all four accumulators still lack (a pixel's row-sum term): it goes into
+// the 64-bit rounding term as extra * M, once for every call that shares it, instead of into each accumulator, and the
+// sign test of MODE 1 compares against -extra.  The clamp comes before the shift, on bounds scaled by 2^fs: floor is
+// monotone, so clamp(h >> fs, a, b) == clamp(h, a << fs, (b << fs) | (2^fs - 1)) >> fs.  What is left to shift is
+// non-negative and ends in 0 .. 255, so the shift writes its byte of the packed word directly (an SDWA destination
+// select that keeps the other bytes).  Needs 0 <= act_min <= act_max <= 255, which the operators' entry points check.
+template <int MODE>
+__host__ __device__ __forceinline__ uint32_t requant4_fast(int32_t x0, int32_t x1, int32_t x2, int32_t x3, int32_t extra, const RequantDev &r) {
+    static_assert(MODE == 1 || MODE == 2, "single-shift forms only");
+    const int64_t pos = (int64_t)(((uint64_t)r.pos_hi << 32) | r.pos_lo) + (int64_t)extra * (int64_t)r.multiplier;
+    const int64_t neg = pos - (1ll << 31);
+    const int32_t zero = -extra;  // (extra is a sum of at most a few thousand byte products: no overflow)
+    auto high = [&](int32_t x) {
+        const int64_t term = (MODE == 1 && x < zero) ? neg : pos;
+        const int32_t h = (int32_t)(((int64_t)x * (int64_t)r.multiplier + term) >> 32);
+#if defined(__HIP_DEVICE_COMPILE__)
+        int32_t o;
+        asm("v_med3_i32 %0, %1, %2, %3" : "=v"(o) : "v"(h), "s"(r.lo_scaled), "v"(r.hi_scaled));
+        return o;
+#else
+        return h < r.lo_scaled ? r.lo_scaled : h > r.hi_scaled ? r.hi_scaled : h;
+#endif
+    };
+    const int32_t h0 = high(x0), h1 = high(x1), h2 = high(x2), h3 = high(x3);
+#if defined(__HIP_DEVICE_COMPILE__)
+    uint32_t w;
+    asm("v_lshrrev_b32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(w) : "v"(r.fast_shift), "v"(h0));
+    asm("v_lshrrev_b32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(w) : "v"(r.fast_shift), "v"(h1));
+    asm("v_lshrrev_b32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(w) : "v"(r.fast_shift), "v"(h2));
+    asm("v_lshrrev_b32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(w) : "v"(r.fast_shift), "v"(h3));
+    return w;
+#else
+    const int fs = r.fast_shift;
+    return (uint32_t)(h0 >> fs) | ((uint32_t)(h1 >> fs) << 8) | ((uint32_t)(h2 >> fs) << 16) | ((uint32_t)(h3 >> fs) << 24);
 #endif
 }
 
@@ -220,6 +259,8 @@ inline RequantDev make_requant_dev(const eh_requant &q) {
     const int64_t neg = pos - (1ll << 31);
     r.pc_multiplier = nullptr;
     r.pc_shift = nullptr;
+    r.lo_scaled = (int32_t)((uint32_t)q.act_min << r.fast_shift);
+    r.hi_scaled = (int32_t)(((uint32_t)q.act_max << r.fast_shift) | ((1u << r.fast_shift) - 1u));
     r.pos_lo = (uint32_t)((uint64_t)pos & 0xFFFFFFFFull);
     r.pos_hi = (uint32_t)((uint64_t)pos >> 32);
     r.neg_lo = (uint32_t)((uint64_t)neg & 0xFFFFFFFFull);

@@ -141,7 +141,10 @@ void eh_make_requant_s8(float input_scale, int32_t input_zp, float filter_scale,
  * gpu/operators/cl_kernels/ConvolutionKernels.cpp:1317-1375), q's pair standing for
  * the channel's: 2 with the rounding term computed from the shift (-20 <= shift <= -1),
  * 3 with it taken from a per-channel table (-20 <= shift <= -2); parameters outside
- * those ranges are an error, as the kernels then take the two-step order. */
+ * those ranges are an error, as the kernels then take the two-step order.  Form 4 is
+ * the per-tensor single-shift form as the kernels' epilogues evaluate it: four accumulators
+ * at a time, the clamp applied before the shift, and a row term (here a value that varies
+ * with the group of four) kept out of the accumulators and folded into the rounding term. */
 int eh_requant_apply(const eh_requant *q, const int32_t *acc, uint8_t *out, int64_t count, int32_t form,
                      int32_t *single_shift);
 /* What CLConvolutionPerChannelQuantized::execute derives (CLConvolutionPerChannelQuantized.cpp:88-121):

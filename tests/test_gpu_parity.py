@@ -311,6 +311,40 @@ def test_two_step_requant_in_every_kernel_family():
         assert np.array_equal(got, want), (m_real, diff_report(got, want))
 
 
+@pytest.mark.parametrize("rs", [1, 2, 5, 8, 9, 12, 16, 20])
+def test_packed_single_shift_epilogue_every_kernel_family(rs):
+    """The epilogues' four-at-a-time single-shift form (clamp before the shift, the byte written by the shift, the row
+    term inside the rounding term) at small and large shifts, with and without the sign test, through the one-tap
+    kernel, the patch-in-LDS 3x3 kernel, the tiled GEMM (whole tiles and its split reduction) and depthwise."""
+    print("packed epilogue rs", rs, flush=True)
+    for mult, zp_out, lo, hi in ((1 << 30, 0, 0, 255), ((1 << 31) - 1, 131, 0, 255), (1518500250, 17, 17, 200)):
+        q = O.raw_quant(zp_in=131, zp_w=121, zp_out=zp_out, multiplier=mult, shift=-rs, act_min=lo, act_max=hi)
+        amp = 1 if rs > 6 else 0   # small accumulators for the small shifts, so that the outputs are not all clamped
+        def tensor(shape, seed, zp):
+            t = synth.fill_u8(shape, seed)
+            return t if amp else (t % (3 + rs) + zp - 1 - rs // 2).astype(np.uint8)
+        for s in (O.conv_shape(2, 16, 9, 7, 48, 1, 1), O.conv_shape(1, 32, 12, 12, 32, 3, 3, pad=(1, 1, 1, 1))):
+            x, w = tensor((s.n, s.c, s.h, s.w), SEED + rs, 131), tensor((s.cout, s.c, s.kh, s.kw), SEED + rs + 1, 121)
+            b = synth.fill_i32((s.cout,), SEED + rs + 2, -300, 300)
+            want = O.conv2d(x, w, b, s, q)
+            got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
+            assert np.array_equal(got, want), (rs, mult, s, diff_report(got, want))
+        for m, k, n in ((70, 256, 40), (512, 256, 256)):
+            a, w = tensor((m, k), SEED + rs + 3, 131), tensor((n, k), SEED + rs + 4, 121)
+            b = synth.fill_i32((n,), SEED + rs + 5, -300, 300)
+            want = O.fc(a, w, b, q)
+            got = gpu_fc(a, w, b, to_eh_requant(q))
+            assert np.array_equal(got, want), (rs, mult, m, k, n, diff_report(got, want))
+        s = O.conv_shape(2, 16, 9, 9, 16, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), groups=16)
+        x, w = tensor((s.n, s.c, s.h, s.w), SEED + rs + 6, 131), tensor((s.c, 1, 3, 3), SEED + rs + 7, 121)
+        b = synth.fill_i32((s.c,), SEED + rs + 8, -300, 300)
+        want = O.dwconv2d(x, w, b, s, q)
+        got = gpu_dwconv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC)
+        assert np.array_equal(got, want), (rs, mult, "dw", diff_report(got, want))
+        if rs in (1, 8):
+            assert len(np.unique(want)) > 8
+
+
 def test_negative_half_ties_round_like_the_oracle():
     """Accumulators chosen so that acc * M lands exactly on .5 for both signs and both rounding stages."""
     k, n = 16, 16

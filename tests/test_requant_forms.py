@@ -57,6 +57,12 @@ def test_single_shift_form_equals_oracle(rs):
             assert bad.size == 0, (mult, rs, zp_out, acc[bad[:5]], got[bad[:5]], want[bad[:5]])
             two, single = eden.requant_apply(to_eh(q), acc, two_step=True)
             assert not single and np.array_equal(two, want)
+            # the epilogues' packed evaluation: clamp before the shift, a row term inside the rounding term
+            near = acc[(acc > -2**31 + 5000) & (acc < 2**31 - 5000)]
+            packed, _ = eden.requant_apply(to_eh(q), near, channel_form="packed")
+            ref = np.array([O.lib.eo_requant(int(a), q) for a in near], np.uint8)
+            bad = np.nonzero(packed != ref)[0]
+            assert bad.size == 0, ("packed", mult, rs, zp_out, near[bad[:5]], packed[bad[:5]], ref[bad[:5]])
 
 
 @pytest.mark.parametrize("shift", [-31, -25, -21, 0, 1, 5])
