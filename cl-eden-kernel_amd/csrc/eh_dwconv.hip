@@ -238,26 +238,43 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
     constexpr bool flip_loaded = FOLD ? FLIP : !FLIP;
     const uint32_t base = img * (uint32_t)(p.h * p.w_ * p.c) + cq * 4u;
 
-    uint32_t col_off[IW];
-    bool col_ok[IW];
-#pragma unroll
-    for (int x = 0; x < IW; ++x) {
-        const int ix = ix0 + x;
-        col_ok[x] = (unsigned)ix < (unsigned)p.w_;
-        const int ixc = ix < 0 ? 0 : (ix >= p.w_ ? p.w_ - 1 : ix);
-        col_off[x] = base + (uint32_t)ixc * (uint32_t)p.c;
-    }
+    // (row pitch and pixel offsets stay below 2^24, which the launcher checks: 24-bit multiplies run at full rate,
+    // 32-bit ones at a quarter of it)
+    const int row_pitch = p.w_ * p.c;
     uint32_t in[3][IW];
+    const bool inside = iy0 >= 0 && iy0 + 2 < p.h && ix0 >= 0 && ix0 + IW - 1 < p.w_;
+    if (__builtin_amdgcn_ballot_w64(!inside) == 0) {
+        // every window of the wave lies inside the image (most waves): no clamps, no selects, offsets that differ
+        // between the loads by wave-uniform amounts; a wave with one window on the border takes the general path whole
+        const uint8_t *src = p.in + (base + (uint32_t)__mul24(iy0, row_pitch) + (uint32_t)__mul24(ix0, p.c));
 #pragma unroll
-    for (int ky = 0; ky < 3; ++ky) {
-        const int iy = iy0 + ky;
-        const bool row_ok = (unsigned)iy < (unsigned)p.h;
-        const int iyc = iy < 0 ? 0 : (iy >= p.h ? p.h - 1 : iy);
-        const uint32_t row_off = (uint32_t)iyc * (uint32_t)(p.w_ * p.c);
+        for (int ky = 0; ky < 3; ++ky)
+#pragma unroll
+            for (int x = 0; x < IW; ++x) {
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(src + (uint32_t)(ky * row_pitch + x * p.c));
+                in[ky][x] = flip_loaded ? v ^ 0x80808080u : v;
+            }
+    } else {
+        uint32_t col_off[IW];
+        bool col_ok[IW];
 #pragma unroll
         for (int x = 0; x < IW; ++x) {
-            const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in + (row_off + col_off[x]));
-            in[ky][x] = row_ok && col_ok[x] ? (flip_loaded ? v ^ 0x80808080u : v) : fill;
+            const int ix = ix0 + x;
+            col_ok[x] = (unsigned)ix < (unsigned)p.w_;
+            const int ixc = ix < 0 ? 0 : (ix >= p.w_ ? p.w_ - 1 : ix);
+            col_off[x] = base + (uint32_t)__mul24(ixc, p.c);
+        }
+#pragma unroll
+        for (int ky = 0; ky < 3; ++ky) {
+            const int iy = iy0 + ky;
+            const bool row_ok = (unsigned)iy < (unsigned)p.h;
+            const int iyc = iy < 0 ? 0 : (iy >= p.h ? p.h - 1 : iy);
+            const uint32_t row_off = (uint32_t)__mul24(iyc, row_pitch);
+#pragma unroll
+            for (int x = 0; x < IW; ++x) {
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in + (row_off + col_off[x]));
+                in[ky][x] = row_ok && col_ok[x] ? (flip_loaded ? v ^ 0x80808080u : v) : fill;
+            }
         }
     }
     int4 wk[3];
@@ -298,10 +315,11 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
             }
         }
         if constexpr (FOLD) {
-            acc0 -= p.zp_w * (cs[j * S][0] + cs[j * S + 1][0] + cs[j * S + 2][0]);
-            acc1 -= p.zp_w * (cs[j * S][1] + cs[j * S + 1][1] + cs[j * S + 2][1]);
-            acc2 -= p.zp_w * (cs[j * S][2] + cs[j * S + 1][2] + cs[j * S + 2][2]);
-            acc3 -= p.zp_w * (cs[j * S][3] + cs[j * S + 1][3] + cs[j * S + 2][3]);
+            // (nine bytes times a zero point of at most 383: a 24-bit multiply-add)
+            acc0 += __mul24(-p.zp_w, cs[j * S][0] + cs[j * S + 1][0] + cs[j * S + 2][0]);
+            acc1 += __mul24(-p.zp_w, cs[j * S][1] + cs[j * S + 1][1] + cs[j * S + 2][1]);
+            acc2 += __mul24(-p.zp_w, cs[j * S][2] + cs[j * S + 1][2] + cs[j * S + 2][2]);
+            acc3 += __mul24(-p.zp_w, cs[j * S][3] + cs[j * S + 1][3] + cs[j * S + 2][3]);
         }
         uint32_t o = PC ? requant4_channel_fast(acc0, acc1, acc2, acc3, rq, quad) : requant4<false>(acc0, acc1, acc2, acc3, rq, quad);
         if (FLIP) o ^= 0x80808080u;
@@ -477,7 +495,8 @@ int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
                       : (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, false> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, false>);
         };
         using tw4 = std::integral_constant<int, 4>;
-        const bool dot4 = (p.w_trip || p.w_fold) && (!pc || p.rq.fast);
+        // (the dot product kernels index rows and pixels with 24-bit multiplies)
+        const bool dot4 = (p.w_trip || p.w_fold) && (!pc || p.rq.fast) && (long)p.w_ * p.c < (1l << 23) && p.h < (1 << 23);
         if (dot4)
             kernel = p.stride_h == 1 ? pick_dot4(std::integral_constant<int, 1>{}, tw4{}) : pick_dot4(std::integral_constant<int, 2>{}, tw4{});
         if (dot4 && p.stride_h == 1 && (p.wo & 7) == 0 && total >= (1l << 20)) {
