@@ -232,6 +232,21 @@ def copy_workload(eden, synth, mib=64, cold=False):
                 keep=bufs, sets=sets, ops=0.0, bytes=2 * nbytes, bound="hbm")
 
 
+def stream_workload(eden, synth, mode=1, out_bytes=32 * 56 * 56 * 144, cold=False):
+    """A kernel that only moves bytes in the ratio of an HBM-bound layer (mode 1: one chunk read, six written, the
+    24 -> 144 pointwise layer; mode 2: four read, one written, the stride-2 depthwise layer; mode 0: copy): what the
+    device gives a launch of that size before any arithmetic."""
+    in_bytes = {0: out_bytes, 1: out_bytes // 6, 2: 4 * out_bytes}[mode]
+    sets = set_count(in_bytes + out_bytes, cold)
+    bufs = [(eden.DeviceBuffer(nbytes=in_bytes), eden.DeviceBuffer(nbytes=out_bytes)) for _ in range(sets)]
+    for src, _ in bufs:
+        eden.check(eden.load().eh_memset(src.ptr, 7, in_bytes, None))
+    lib = eden.load()
+    return dict(name="stream_%s_%.1fMB" % ({0: "copy", 1: "1to6", 2: "4to1"}[mode], (in_bytes + out_bytes) / 1e6),
+                launch=lambda s, i: eden.check(lib.eh_probe_stream(bufs[i][0].ptr, bufs[i][1].ptr, out_bytes, mode, s)),
+                keep=bufs, sets=sets, ops=0.0, bytes=in_bytes + out_bytes, bound="hbm")
+
+
 def layout_workload(eden, synth, to_nhwc=True, n=64, c=96, h=112, w=112, cold=False):
     """NCHW <-> NHWC conversion of a feature map (MobileNetV2's largest, [64, 96, 112, 112]): bytes in + bytes out."""
     nbytes = n * c * h * w
@@ -370,7 +385,10 @@ def main():
                     dwbig=shaped(dw_workload, n=256), pwbig=shaped(pw_workload, n=256),
                     copy=copy_workload, mbv2=mbv2_workload, mbv2narrow=shaped(mbv2_workload, weights="narrow"),
                     tonhwc=layout_workload, tonchw=shaped(layout_workload, to_nhwc=False),
-                    mbv2pc=shaped(mbv2_workload, per_channel=True))
+                    mbv2pc=shaped(mbv2_workload, per_channel=True),
+                    stream16=stream_workload, stream16big=shaped(stream_workload, out_bytes=256 * 56 * 56 * 144),
+                    stream41=shaped(stream_workload, mode=2, out_bytes=32 * 28 * 28 * 144),
+                    stream41big=shaped(stream_workload, mode=2, out_bytes=256 * 28 * 28 * 144))
     if args.only:
         work = families[args.only](eden, synth, cold=args.cold)
         args.steps = round_steps(args.steps, work["sets"], work.get("chunk", 50))
@@ -438,6 +456,9 @@ def main():
                                       (shaped(fc_workload, m=8192, k=4096, n=4096), 100, False),
                                       (layout_workload, 200, True), (shaped(layout_workload, to_nhwc=False), 200, True),
                                       (copy_workload, 200, True),
+                                      (stream_workload, 500, True), (shaped(stream_workload, out_bytes=256 * 56 * 56 * 144), 100, True),
+                                      (shaped(stream_workload, mode=2, out_bytes=32 * 28 * 28 * 144), 500, True),
+                                      (shaped(stream_workload, mode=2, out_bytes=256 * 28 * 28 * 144), 100, True),
                                       (shaped(mbv2_workload, weights="narrow"), 40, False),
                                       (shaped(mbv2_workload, per_channel=True), 40, False)):
             others.append(measure(eden, synth, stream, make, steps, max(4, steps // 10), use_graph, cold_too))

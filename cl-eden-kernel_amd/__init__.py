@@ -67,6 +67,7 @@ EXPORTS = {
     "eh_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(AddRequant), C.c_void_p]),
     "eh_avgpool_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PoolDesc), C.c_void_p]),
     "eh_probe_mfma_i8": (C.c_int, [C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
+    "eh_probe_stream": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]),
     "eh_make_requant_perchannel": (None, [C.c_float, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32, C.c_int, C.c_int,
                                           C.POINTER(Requant), C.c_void_p, C.c_void_p]),
     "eh_conv2d_u8_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(AddRequant),

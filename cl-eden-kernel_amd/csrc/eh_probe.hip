@@ -2,7 +2,8 @@
 // issue rate of the int8 MFMA this library uses, from registers only (no memory
 // traffic at all).  With operand bits that toggle like real data the sustained
 // clock under this load is lower than with constant operands, so both are
-// reported.  A measurement utility: it has no counterpart in the reference.
+// reported.  And what plain streaming kernels reach on the byte ratios of the HBM-bound layers.
+// Measurement utilities: they have no counterpart in the reference.
 #include "eh_internal.h"
 
 namespace eh {
@@ -28,10 +29,48 @@ __global__ __launch_bounds__(256) void mfma_i8_probe_kernel(const int iters, int
     sink[blockIdx.x * 256 + threadIdx.x] = c0[0] + c1[1] + c2[2] + c3[3];
 }
 
+// Streaming yardsticks for the HBM-bound kernels: 16 bytes per lane, whole lines per wave, nothing but the moves.
+// MODE 0: copy.  MODE 1: every source chunk is written six times (the byte ratio of a 24 -> 144 pointwise layer).
+// MODE 2: four source chunks are folded into one written chunk (the byte ratio of a stride-2 depthwise layer).
+template <int MODE>
+__global__ __launch_bounds__(256) void stream_probe_kernel(const uint4 *__restrict__ in, uint4 *__restrict__ out, const uint32_t n_out) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n_out; i += gridDim.x * 256u) {
+        if constexpr (MODE == 0) {
+            out[i] = in[i];
+        } else if constexpr (MODE == 1) {
+            const uint4 a = in[i / 6u];
+            out[i] = make_uint4(a.x + i, a.y, a.z, a.w);
+        } else {
+            const uint4 a = in[4u * i], b = in[4u * i + 1u], c = in[4u * i + 2u], d = in[4u * i + 3u];
+            out[i] = make_uint4(a.x ^ b.x ^ c.x ^ d.x, a.y ^ b.y ^ c.y ^ d.y, a.z ^ b.z ^ c.z ^ d.z, a.w ^ b.w ^ c.w ^ d.w);
+        }
+    }
+}
+
 }  // namespace
 }  // namespace eh
 
 using namespace eh;
+
+extern "C" int eh_probe_stream(const void *src, void *dst, int64_t out_bytes, int32_t mode, void *stream) {
+    EH_REQUIRE(src && dst && out_bytes > 0 && (out_bytes & 15) == 0 && out_bytes < (1ll << 35), "stream probe: %lld bytes", (long long)out_bytes);
+    EH_REQUIRE(mode >= 0 && mode <= 2, "stream probe: mode %d", mode);
+    EH_REQUIRE(((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0, "stream probe: unaligned pointers");
+    const uint32_t n_out = (uint32_t)(out_bytes / 16);
+    const uint32_t blocks = (n_out + 255u) / 256u;
+    const dim3 grid(blocks < 8192u ? blocks : 8192u);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint4 *in = static_cast<const uint4 *>(src);
+    uint4 *out = static_cast<uint4 *>(dst);
+    if (mode == 0)
+        hipLaunchKernelGGL(stream_probe_kernel<0>, grid, dim3(256), 0, st, in, out, n_out);
+    else if (mode == 1)
+        hipLaunchKernelGGL(stream_probe_kernel<1>, grid, dim3(256), 0, st, in, out, n_out);
+    else
+        hipLaunchKernelGGL(stream_probe_kernel<2>, grid, dim3(256), 0, st, in, out, n_out);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
 
 extern "C" int eh_probe_mfma_i8(int32_t iterations, int32_t toggling_operands, double *tops) {
     EH_REQUIRE(tops != nullptr && iterations > 0 && iterations <= (1 << 22), "probe: bad arguments");

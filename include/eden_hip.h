@@ -215,6 +215,12 @@ int eh_graph_destroy(void *graph);
  * ceiling the benchmark prints beside the published peak; no counterpart in the
  * reference.  Synchronous; allocates and frees a small device buffer. */
 int eh_probe_mfma_i8(int32_t iterations, int32_t toggling_operands, double *tops);
+/* A kernel that only moves bytes (16 per lane, whole lines per wave), launched on `stream`:
+ * the yardstick beside the HBM-bound kernels' figures.  mode 0 copies out_bytes; mode 1
+ * writes every 16-byte source chunk six times (reads out_bytes / 6: the ratio of a 24 -> 144
+ * pointwise layer); mode 2 folds four source chunks into each written one (reads
+ * 4 * out_bytes: the ratio of a stride-2 depthwise layer).  No counterpart in the reference. */
+int eh_probe_stream(const void *src, void *dst, int64_t out_bytes, int32_t mode, void *stream);
 
 /* ---- layout conversion -----------------------------------------------------
  * nchw2nhwc_uint8 / nhwc2nchw_uint8 (gpu/common/CLKernels.hpp:429-491) as
