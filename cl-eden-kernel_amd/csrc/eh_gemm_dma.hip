@@ -211,6 +211,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
             add_lut_s[1][tid] = mul_round_shift((int32_t)((uint32_t)(tid - p.radd.zp_b) << p.radd.left_shift), p.radd.mult_b, p.radd.rs_b);
         }
     }
+    // the sixteen residual bytes this thread's outputs will be added to travel under the whole main loop as well
+    uint4 res_reg = make_uint4(0, 0, 0, 0);
+    bool res_vec = false;
+    if constexpr (WGK != 1) {
+        if (p.residual) {
+            const int m = m0 + (tid & 63), n = n0 + (tid >> 6) * 16;
+            res_vec = m < p.m && n + 16 <= p.n && (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0) &&
+                      (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0;
+            if (res_vec) res_reg = *reinterpret_cast<const uint4 *>(p.residual + out_pixel_offset(p, m, p.ho * p.wo) + n);
+        }
+    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WGM, wn = (wave / WGM) % WGN, wk = wave / (WGM * WGN);
     const int k_slabs = p.k_pad / SLAB;
@@ -593,8 +604,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
         const bool aligned16 = (p.ldc & 15) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
         if (p.residual) {  // out = add(residual, result); only this split-reduction epilogue offers it
             const uint8_t *res = p.residual + out_off;
-            if (aligned16 && n + 16 <= p.n && (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) {
-                const uint4 rv = *reinterpret_cast<const uint4 *>(res);
+            if (res_vec) {
+                const uint4 rv = res_reg;
                 // add_word with the two tables (the same arithmetic: the tables hold what add_one computes first)
                 auto add_word_lut = [&](uint32_t a, uint32_t b) {
                     uint32_t o = 0;
