@@ -213,12 +213,16 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         const int cnt = p.n - n;
         if constexpr (RES) {  // out = add(residual, result); the residual tensor is addressed like the output
             const uint8_t *res = p.residual + out_off + n;
-            if (wide && cnt >= 16) {
-                const u32x4_a4 rv = *reinterpret_cast<const u32x4_a4 *>(res);
-                packed[0] = add_word_lut(rv.x, packed[0]);
-                packed[1] = add_word_lut(rv.y, packed[1]);
-                packed[2] = add_word_lut(rv.z, packed[2]);
-                packed[3] = add_word_lut(rv.w, packed[3]);
+            if (wide && (cnt >= 16 || cnt == 8)) {
+                // (a block's second half may hold eight channels only, as with 24 or 56 of them: its upper words are
+                // computed from zeros and never stored)
+                const u32x2_a4 lo = *reinterpret_cast<const u32x2_a4 *>(res);
+                u32x2_a4 hi = {0u, 0u};
+                if (cnt >= 16) hi = *reinterpret_cast<const u32x2_a4 *>(res + 8);
+                packed[0] = add_word_lut(lo.x, packed[0]);
+                packed[1] = add_word_lut(lo.y, packed[1]);
+                packed[2] = add_word_lut(hi.x, packed[2]);
+                packed[3] = add_word_lut(hi.y, packed[3]);
             } else {
                 const int c = cnt < 16 ? cnt : 16;
                 for (int t = 0; t < c; ++t) {
@@ -440,6 +444,10 @@ int launch_igemm_thin(const GemmProblem &p, hipStream_t stream) {
         if (n_blocks == 1) return launch_nbu<1, 2>(p, stream);
         if (n_blocks == 2) return launch_nbu<2, 2>(p, stream);
         return launch_nbu<4, 2>(p, stream);
+    }
+    if (p.k_pad <= 192) {  // one group of six steps: a row block's loads leave together
+        if (n_blocks == 1) return launch_nbu<1, 6>(p, stream);
+        return launch_nbu<2, 6>(p, stream);
     }
     if (n_blocks == 1) return launch_nbu<1, 4>(p, stream);
     return launch_nbu<2, 4>(p, stream);
