@@ -17,6 +17,8 @@
 // output channels of its pixel: requantize, pack, one 16-byte store.
 #include <type_traits>
 
+#include <atomic>
+
 #include "eh_internal.h"
 
 namespace eh {
@@ -44,6 +46,10 @@ struct ThinStage {
     int32_t pitch;     // LDS bytes per pixel of the image (an odd number of 16-byte chunks), 0: store directly
     int32_t offset;    // byte offset of the four waves' images in dynamic LDS
     FastDiv div_cpp;   // chunks of 16 bytes per pixel: ldc / 16
+    // 1: pixel m of the GEMM reads at m * cin and writes at m * ldc (stride 1, no offsets, dense output), every factor
+    // below 2^24 and every product below 2^32, so a lane finds its pixel with two full-rate multiplies instead of two
+    // divisions and a dozen 32- and 64-bit multiplies (which issue at a quarter of the rate)
+    int32_t linear;
 };
 
 template <int NBU, int KU, bool ROWSUM, int QM, bool RES>
@@ -110,7 +116,10 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         ok = rb < row_blocks && m < p.m;
         in_off = 0;
         out_off = 0;
-        if (ok) {
+        if (ok && stage.linear) {
+            in_off = (size_t)(__umul24((uint32_t)m, (uint32_t)p.cin) + (uint32_t)p.a_offset + (uint32_t)half * 16u);
+            out_off = (size_t)__umul24((uint32_t)m, (uint32_t)p.ldc);
+        } else if (ok) {
             const int img = (int)fastdiv((uint32_t)m, p.div_plane), rem = m - img * plane;
             const int oy = (int)fastdiv((uint32_t)rem, p.div_wo), ox = rem - oy * p.wo;
             in_off = ((size_t)(img * p.h + oy * p.stride_h + p.y_base) * p.w + (ox * p.stride_w + p.x_base)) * (size_t)p.cin +
@@ -369,10 +378,6 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     while (ranges < groups_total && (long)row_blocks * ranges < 4096) ++ranges;
     const int nbw = (groups_total + ranges - 1) / ranges * NBU;
     ranges = (n_blocks + nbw - 1) / nbw;
-    int row_wgs = (row_blocks + 3) / 4;
-    const int wg_target = 1024 / ranges > 0 ? 1024 / ranges : 1;  // four workgroups per CU over the whole launch
-    if (row_wgs > wg_target) row_wgs = wg_target;
-    const dim3 grid(row_wgs, ranges);
     const bool pc_fast = p.rq.fast && p.rq.pc_multiplier;
     const size_t lds = (size_t)nbw * ksteps * 1024 + (size_t)nbw * 32 * sizeof(int32_t) * (pc_fast ? 4 : 1) +
                        (p.residual ? 2 * 256 * sizeof(int32_t) : 0);
@@ -388,11 +393,32 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
         if ((size_t)stage.offset + 4u * 32u * stage.pitch > 64 * 1024) stage = ThinStage{};
     }
     const size_t lds_all = stage.pitch ? (size_t)stage.offset + 4u * 32u * stage.pitch : lds;
+    {
+        const long reach_in = (long)p.m * p.cin + p.a_offset + 16, reach_out = (long)p.m * p.ldc;
+        stage.linear = dense_out && p.stride_h == 1 && p.stride_w == 1 && p.y_base == 0 && p.x_base == 0 && p.h == p.ho && p.w == p.wo &&
+                       p.a_offset >= 0 && p.m < (1 << 24) && p.cin < (1 << 24) && p.ldc < (1 << 24) && reach_in < (1l << 32) &&
+                       reach_out < (1l << 32);
+    }
     // row sums, the single-shift requantization and the fused residual add are compile-time variants: a launch pays for
     // none of the code it does not use
     auto launch = [&](auto rowsum_c, auto qm_c, auto res_c) {
-        hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(res_c)::value>), grid,
-                           dim3(256), lds_all, stream, p, n_blocks, ksteps, nbw, row_blocks, stage);
+        auto kernel = direct_gemm_kernel<NBU, KU, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(res_c)::value>;
+        // The grid is persistent: as many workgroups as the device holds at once with this variant's registers and
+        // this launch's LDS (a wave has one pixel block in flight, so the bytes in flight grow with the waves), and
+        // at least four per CU.  The answer is kept per KiB of LDS.
+        static std::atomic<int> resident[65];
+        const size_t slot = (lds_all + 1023) / 1024;
+        int per_cu = resident[slot].load(std::memory_order_relaxed);
+        if (per_cu == 0) {
+            int n = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, lds_all) != hipSuccess || n < 1) n = 4;
+            per_cu = n < 4 ? 4 : (n > 8 ? 8 : n);
+            resident[slot].store(per_cu, std::memory_order_relaxed);
+        }
+        int row_wgs = (row_blocks + 3) / 4;
+        const int wg_target = 256 * per_cu / ranges > 0 ? 256 * per_cu / ranges : 1;
+        if (row_wgs > wg_target) row_wgs = wg_target;
+        hipLaunchKernelGGL(kernel, dim3(row_wgs, ranges), dim3(256), lds_all, stream, p, n_blocks, ksteps, nbw, row_blocks, stage);
     };
     auto with_res = [&](auto rowsum_c, auto qm_c) {
         if (p.residual)
