@@ -1,0 +1,81 @@
+"""Randomized differential sweep: a few hundred seeded random operator instances (shapes, strides, paddings, dilations,
+groups, layouts, zero points, clamp ranges, requantization scales) through the C ABI against the CPU oracle.  The
+hand-picked cases of test_gpu_parity.py aim at each kernel family's corners; this one aims at what nobody thought of.
+Bit-exact, as everywhere."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from harness import diff_report, eden, gpu_conv, gpu_deconv, gpu_dwconv, gpu_fc, synth, to_eh_requant
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_operator_instances_match_the_oracle(seed):
+    eden.init(0)
+    print("random sweep, seed", seed, flush=True)
+    rng = np.random.default_rng(seed)
+    N = 400
+    def centred(acc, zp_in, zp_w, lo, hi):
+        sd = float(acc.std()) or 1.0
+        qm, sh = O.quantize_multiplier(float(rng.choice([10.0, 40.0, 120.0])) / sd)
+        zp_out = int(np.clip(128 - round(float(acc.mean()) * 40.0 / sd), 0, 255))
+        return O.raw_quant(zp_in=zp_in, zp_w=zp_w, zp_out=zp_out, multiplier=qm, shift=sh, act_min=lo, act_max=hi)
+    ran = {}
+    for it in range(N):
+        kind = rng.choice(["conv", "conv1x1", "conv3x3", "dw", "fc", "deconv"], p=[0.25, 0.2, 0.15, 0.2, 0.1, 0.1])
+        zp_in, zp_w = int(rng.integers(0, 256)), int(rng.choice([128, int(rng.integers(0, 256))]))
+        lo = int(rng.choice([0, 0, int(rng.integers(0, 100))])); hi = int(rng.choice([255, 255, int(rng.integers(150, 256))]))
+        layout = eden.NHWC if rng.random() < 0.7 else eden.NCHW
+        tseed = int(rng.integers(1, 1 << 30))
+        try:
+            if kind == "fc":
+                m, k, n = int(rng.integers(1, 300)), int(rng.choice([8, 16, 24, 40, 64, 100, 128, 192, 256, 260, 512, 1000])), int(rng.integers(1, 300))
+                a = synth.fill_u8((m, k), tseed); w = synth.fill_u8((n, k), tseed + 1); b = synth.fill_i32((n,), tseed + 2, -1000, 1000)
+                _, acc = O.fc(a, w, b, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+                q = centred(acc, zp_in, zp_w, lo, hi)
+                want = O.fc(a, w, b, q); got = gpu_fc(a, w, b, to_eh_requant(q)); desc = (kind, m, k, n)
+            else:
+                n = int(rng.integers(1, 5))
+                if kind == "dw":
+                    c = int(rng.choice([4, 8, 12, 16, 32, 36, 144, 20, 7])); h, w_ = int(rng.integers(3, 30)), int(rng.integers(3, 30))
+                    k = int(rng.choice([3, 3, 3, 5, 2])); st = int(rng.choice([1, 2])); pads = tuple(int(v) for v in rng.integers(0, k, 4))
+                    s = O.conv_shape(n, c, h, w_, c, k, k, stride=(st, st), pad=pads, groups=c)
+                    if min(O.conv_out_hw(s)) < 1: continue
+                    x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((c, 1, k, k), tseed + 1); b = synth.fill_i32((c,), tseed + 2, -1000, 1000)
+                    _, acc = O.dwconv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+                    q = centred(acc, zp_in, zp_w, lo, hi)
+                    want = O.dwconv2d(x, w, b, s, q); got = gpu_dwconv(x, w, b, s, to_eh_requant(q), layout=layout); desc = (kind, s, layout)
+                elif kind == "deconv":
+                    c = int(rng.choice([8, 16, 32, 24])); cout = int(rng.choice([8, 16, 20, 32, 64])); h, w_ = int(rng.integers(2, 12)), int(rng.integers(2, 12))
+                    k = int(rng.choice([2, 3, 4])); st = int(rng.choice([1, 2])); pad = int(rng.integers(0, k))
+                    s = O.conv_shape(n, c, h, w_, cout, k, k, stride=(st, st), pad=(pad, pad, pad, pad))
+                    if min(O.deconv_out_hw(s)) < 1: continue
+                    x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((c, cout, k, k), tseed + 1); b = synth.fill_i32((cout,), tseed + 2, -1000, 1000)
+                    _, acc = O.deconv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+                    q = centred(acc, zp_in, zp_w, lo, hi)
+                    want = O.deconv2d(x, w, b, s, q); got = gpu_deconv(x, w, b, s, to_eh_requant(q), layout=layout); desc = (kind, s, layout)
+                else:
+                    if kind == "conv1x1":
+                        c = int(rng.choice([8, 16, 24, 32, 40, 64, 96, 144, 192, 320])); cout = int(rng.choice([8, 16, 24, 32, 48, 96, 144, 208, 256, 300])); k = 1
+                        h, w_ = int(rng.integers(1, 20)), int(rng.integers(1, 20)); st = int(rng.choice([1, 1, 2])); pads = (0, 0, 0, 0) if rng.random() < 0.8 else tuple(int(v) for v in rng.integers(0, 2, 4)); groups = 1; dil = 1
+                    elif kind == "conv3x3":
+                        c = int(rng.choice([32, 64, 96, 128])); cout = int(rng.choice([16, 32, 40, 64, 100])); k = 3
+                        h, w_ = int(rng.integers(6, 24)), int(rng.integers(8, 40)); st = 1; pads = tuple(int(v) for v in rng.integers(0, 3, 4)); groups = 1; dil = 1
+                    else:
+                        groups = int(rng.choice([1, 1, 1, 2, 4])); c = groups * int(rng.choice([1, 3, 4, 8, 16, 20])); cout = groups * int(rng.choice([1, 4, 8, 10, 16]))
+                        k = int(rng.choice([1, 2, 3, 5])); h, w_ = int(rng.integers(k, 20)), int(rng.integers(k, 20)); st = int(rng.choice([1, 2, 3])); pads = tuple(int(v) for v in rng.integers(0, k + 1, 4)); dil = int(rng.choice([1, 1, 2]))
+                    s = O.conv_shape(n, c, h, w_, cout, k, k, stride=(st, st), pad=pads, dil=(dil, dil), groups=groups)
+                    if min(O.conv_out_hw(s)) < 1: continue
+                    x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((cout, c // groups, k, k), tseed + 1); b = synth.fill_i32((cout,), tseed + 2, -1000, 1000)
+                    _, acc = O.conv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+                    q = centred(acc, zp_in, zp_w, lo, hi)
+                    want = O.conv2d(x, w, b, s, q); got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=layout); desc = (kind, s, layout)
+        except Exception as e:
+            raise AssertionError(("error", seed, it, kind, repr(e)[:300]))
+        ran[kind] = ran.get(kind, 0) + 1
+        if not np.array_equal(got, want):
+            bad += 1
+            print("MISMATCH", it, desc, q.as_tuple(), diff_report(got, want), flush=True)
+    assert sum(ran.values()) > 300 and all(ran.get(k, 0) > 10 for k in ("conv", "conv1x1", "conv3x3", "dw", "fc", "deconv")), ran
