@@ -203,6 +203,18 @@ __device__ __forceinline__ uint32_t column_bytes(uint32_t r0, uint32_t r1, uint3
     return __builtin_amdgcn_perm(r2, __builtin_amdgcn_perm(r1, r0, sel01), sel2);
 }
 
+// The same for the four channels of a column at once, in six permutes instead of eight: the first two rows are
+// interleaved pairwise (channels 0 and 1 in one word, 2 and 3 in the other), and each channel's word then takes its
+// pair and its byte of the third row.
+__device__ __forceinline__ void column_words(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t (&out)[4]) {
+    const uint32_t t01 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);  // r0.b0 r1.b0 r0.b1 r1.b1
+    const uint32_t t23 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);  // r0.b2 r1.b2 r0.b3 r1.b3
+    out[0] = __builtin_amdgcn_perm(r2, t01, 0x0c040100u);
+    out[1] = __builtin_amdgcn_perm(r2, t01, 0x0c050302u);
+    out[2] = __builtin_amdgcn_perm(r2, t23, 0x0c060100u);
+    out[3] = __builtin_amdgcn_perm(r2, t23, 0x0c070302u);
+}
+
 // The same tile with 8-bit dot products, for weights whose differences w - zp_w all fit int8 (per-tensor
 // requantization): activations as a - 128, the three vertical taps of a channel and column gathered into one word
 // once and used by every output that touches the column (v_dot4_i32_i8 against the column's three weights), the
@@ -285,10 +297,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
     int cs[FOLD ? IW : 1][4];  // FOLD: sum of the column's three bytes
 #pragma unroll
     for (int x = 0; x < IW; ++x) {
-        col[x][0] = column_bytes<0>(in[0][x], in[1][x], in[2][x]);
-        col[x][1] = column_bytes<1>(in[0][x], in[1][x], in[2][x]);
-        col[x][2] = column_bytes<2>(in[0][x], in[1][x], in[2][x]);
-        col[x][3] = column_bytes<3>(in[0][x], in[1][x], in[2][x]);
+        column_words(in[0][x], in[1][x], in[2][x], col[x]);
         if constexpr (FOLD) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) cs[x][c] = udot4(col[x][c], 0x00010101u, 0);
