@@ -151,3 +151,33 @@ def test_conv_with_residual_add_equals_conv_then_add(case, layout):
         assert np.array_equal(got, O.conv2d(x, w, b, s, q))
         plan.destroy()
     assert want.std() > 4
+
+
+def test_streaming_yardsticks_move_what_they_say():
+    """eh_probe_stream (the byte-moving kernels the HBM-bound figures are set against): copy, one chunk written six
+    times, four chunks folded into one; every 16-byte chunk of the output checked."""
+    lib = eden.load()
+    chunks = 6 * 1000 + 6          # output chunks; a multiple of 6, not of 256
+    out_bytes = chunks * 16
+    src = synth.fill_u8((4 * out_bytes,), SEED + 90)
+    d_in = eden.DeviceBuffer(host=src)
+    d_out = eden.DeviceBuffer(nbytes=out_bytes)
+    words = src.view(np.uint32).reshape(-1, 4)
+    # copy
+    eden.check(lib.eh_probe_stream(d_in.ptr, d_out.ptr, out_bytes, 0, None))
+    eden.sync()
+    assert np.array_equal(d_out.download((out_bytes,)), src[:out_bytes])
+    # 1 -> 6: chunk i of the output is chunk i / 6 of the input with i added to its first word
+    eden.check(lib.eh_probe_stream(d_in.ptr, d_out.ptr, out_bytes, 1, None))
+    eden.sync()
+    want = words[np.arange(chunks) // 6].copy()
+    want[:, 0] += np.arange(chunks, dtype=np.uint32)
+    assert np.array_equal(d_out.download((out_bytes,)).view(np.uint32).reshape(-1, 4), want)
+    # 4 -> 1: the xor of four consecutive input chunks
+    eden.check(lib.eh_probe_stream(d_in.ptr, d_out.ptr, out_bytes, 2, None))
+    eden.sync()
+    want = words[: 4 * chunks].reshape(chunks, 4, 4)
+    want = want[:, 0] ^ want[:, 1] ^ want[:, 2] ^ want[:, 3]
+    assert np.array_equal(d_out.download((out_bytes,)).view(np.uint32).reshape(-1, 4), want)
+    with pytest.raises(eden.EdenHipError):
+        eden.check(lib.eh_probe_stream(d_in.ptr, d_out.ptr, out_bytes + 8, 0, None))
