@@ -208,8 +208,9 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     g.proto.div_plane = make_fastdiv((uint32_t)(g.proto.ho * g.proto.wo));
     g.proto.div_wo = make_fastdiv((uint32_t)g.proto.wo);
     // a plain matrix: one tap at the pixel itself, unit stride, no padding, whole slabs
+    // (a reduction that ends inside its last slab is handled by the kernel: the chunks past the end read a constant)
     g.proto.dense = (g.taps == 1 && g.proto.stride_h == 1 && g.proto.stride_w == 1 && g.proto.y_base == 0 &&
-                     g.proto.x_base == 0 && g.proto.ho == g.proto.h && g.proto.wo == g.proto.w && g.k == g.k_pad &&
+                     g.proto.x_base == 0 && g.proto.ho == g.proto.h && g.proto.wo == g.proto.w && g.vec == 16 &&
                      g.cin == g.proto.cin && !units.empty() && units[0].dy == 0 && units[0].dx == 0 && units[0].offset == 0)
                         ? 1
                         : 0;

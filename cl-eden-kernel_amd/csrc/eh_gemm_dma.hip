@@ -125,7 +125,9 @@ __device__ __forceinline__ void static_for(F &&f) {
     static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
-template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES, bool DENSE, bool ROWSUM>
+// DENSE: 0 table-driven operand gather; 1 a plain matrix of whole slabs; 2 a plain matrix whose reduction ends inside
+// its last slab (the chunks past the end read a constant that the sign flip turns into 0).
+template <int BM, int BN, int WGM, int WGN, int WGK, int SLAB, int STAGES, int DENSE, bool ROWSUM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 && BN == 64 ? 3 : (BM == 128 && BN == 128 ? 2 : 1)))) void igemm_dma_kernel(const GemmBatch batch, const int count, const int tiles_m, const int tiles_n,
                                                         const int gm, const int gn) {
     static_assert(WGM * WGN * WGK == 4, "four waves per workgroup");
@@ -245,6 +247,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i) rows[i] = make_row(p, m0 + (i * 4 + wave) * RPB + slot_row, plane);
     }
+    // dense operands whose reduction is not whole slabs: which lanes' chunks lie past its end in the last slab
+    constexpr bool ragged = DENSE == 2;
+    const bool tail_lane = ragged && my_chunk * 16 >= p.k - (k_slabs - 1) * SLAB;
+    auto tail_unit = [&](int slab) {
+        KUnit ku = KUnit();
+        ku.dy = (int16_t)(ragged && slab == k_slabs - 1 ? 1 : 0);
+        return ku;
+    };
     const int8_t *b_base[B_LOADS];  // uniform: the packed 1 KiB blocks of this wave's weight rows, slab 0
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) b_base[i] = p.b + ((size_t)(n0 / RPB + i * 4 + wave) * k_slabs) * 1024;
@@ -255,9 +265,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
         constexpr int idx = decltype(idx_c)::value;
         if constexpr (idx < A_LOADS) {
             const uint32_t dst = wave_lds + stage_off + idx * 4096;
-            if constexpr (DENSE)
-                dma16_off(a_base, a_voff[idx], dst);
-            else
+            if constexpr (DENSE) {
+                // (ku.dy marks the last slab of a reduction that ends inside it: the chunks past its end read the
+                // constant that the sign flip turns into 0 instead of the next pixel's bytes)
+                if (DENSE == 1 || ku.dy == 0)
+                    dma16_off(a_base, a_voff[idx], dst);
+                else
+                    dma16(tail_lane ? p.fillbuf + 16 : a_base + a_voff[idx], dst);
+            } else
                 dma16(a_chunk_address(p, rows[idx], ku), dst);
         } else {
             constexpr int bi = idx - A_LOADS;
@@ -293,7 +308,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
 #pragma unroll
     for (int s = DENSE ? 0 : 1; s < STAGES; ++s) {
         if (s < k_slabs) {
-            KUnit ku = KUnit();
+            KUnit ku = tail_unit(s);
             if constexpr (!DENSE) ku = ktab_s[s * CPR + my_chunk];
             static_for<LPS>([&](auto idx) { issue_piece(idx, (uint32_t)(s * STAGE_BYTES), ku); });
             advance_slab();
@@ -397,7 +412,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
     // iteration `it`: last step of slab it, then steps 0 .. KSTEPS-2 of slab it+1
     int it = 0;
     for (; it < k_slabs - STAGES; ++it) {
-        KUnit ku = KUnit();
+        KUnit ku = tail_unit(it + STAGES);
         if constexpr (!DENSE) ku = ktab_s[(it + STAGES) * CPR + my_chunk];
         const uint32_t freed = rd_off;
         const uint32_t next_off = rd_off + STAGE_BYTES == STAGES * STAGE_BYTES ? 0u : rd_off + STAGE_BYTES;
@@ -676,19 +691,32 @@ int launch_cfg(const GemmProblem *ps, int count, hipStream_t stream) {
     }
     const size_t ktab_bytes = (size_t)(p.k_pad / 16) * sizeof(KUnit);
     // the per-row activation sums are only carried when the weight zero point is not 128
-    if (p.dense) {
+    // a plain matrix whose reduction ends inside its last slab has a kernel variant of its own where the 64 x 64 tile
+    // with the split reduction serves it (1x1 layers with 320 .. 960 input channels); elsewhere it is gathered by table
+    constexpr bool ragged_variant = BM == 64 && BN == 64;
+    const bool whole = p.k == p.k_pad;
+    if (p.dense && whole) {
         if (p.zw != 0)
-            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true, true>), dim3(grid), dim3(256), 0,
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, 1, true>), dim3(grid), dim3(256), 0,
                                stream, batch, count, tiles_m, tiles_n, gm, gn);
         else
-            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, true, false>), dim3(grid), dim3(256), 0,
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, 1, false>), dim3(grid), dim3(256), 0,
                                stream, batch, count, tiles_m, tiles_n, gm, gn);
+    } else if (p.dense && ragged_variant) {
+        if constexpr (ragged_variant) {
+            if (p.zw != 0)
+                hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, 2, true>), dim3(grid), dim3(256), 0,
+                                   stream, batch, count, tiles_m, tiles_n, gm, gn);
+            else
+                hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, 2, false>), dim3(grid), dim3(256), 0,
+                                   stream, batch, count, tiles_m, tiles_n, gm, gn);
+        }
     } else {
         if (p.zw != 0)
-            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false, true>), dim3(grid), dim3(256),
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, 0, true>), dim3(grid), dim3(256),
                                ktab_bytes, stream, batch, count, tiles_m, tiles_n, gm, gn);
         else
-            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, false, false>), dim3(grid), dim3(256),
+            hipLaunchKernelGGL((igemm_dma_kernel<BM, BN, WGM, WGN, WGK, SLAB, STAGES, 0, false>), dim3(grid), dim3(256),
                                ktab_bytes, stream, batch, count, tiles_m, tiles_n, gm, gn);
     }
     EH_HIP(hipGetLastError());
