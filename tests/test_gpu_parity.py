@@ -59,6 +59,10 @@ FC_CASES = [
     (5, 4100, 1000, 10, 20),   # classifier-like: k not a multiple of 64, n = 1000
     (1000, 24, 144, 128, 5),   # at most 64 reduction bytes: the fragment-direct kernel
     (129, 56, 17, 250, 128),
+    # plain matrices whose reduction ends inside the last 256-byte slab (the dense path with the zero constant)
+    (130, 272, 200, 77, 201),
+    (64, 1296, 130, 3, 128),
+    (200, 528, 64, 131, 120),
 ]
 
 
