@@ -37,22 +37,24 @@ __device__ __forceinline__ void gather_c3k3(const GemmProblem &p, const uint32_t
     const int oy = (int)fastdiv((uint32_t)rem, p.div_wo), ox = rem - oy * p.wo;
     const int iy0 = oy * p.stride_h + p.y_base, ix0 = ox * p.stride_w + p.x_base;
     const bool c0 = (unsigned)ix0 < (unsigned)p.w, c1 = (unsigned)(ix0 + 1) < (unsigned)p.w, c2 = (unsigned)(ix0 + 2) < (unsigned)p.w;
+    const int row_bytes = p.w * 3, a_row0 = ((img * p.h + iy0) * p.w + ix0) * 3;
     uint32_t seg[3][3];  // per kernel row: bytes 0..8 = 3 pixels x 3 channels, the rest zero
 #pragma unroll
     for (int ky = 0; ky < 3; ++ky) {
         const int iy = iy0 + ky;
         const bool row_ok = (unsigned)iy < (unsigned)p.h;
-        const long a = ((long)(img * p.h + iy) * p.w + ix0) * 3;
+        // (tensors stay below 2 GiB: 32-bit offsets, one multiplication chain per pixel instead of one per row)
+        const int a = a_row0 + ky * row_bytes;
         uint32_t d0 = 0, d1 = 0, d2 = 0;
         if (row_ok) {
-            if (a >= 0 && a + 12 <= (long)in_bytes) {
+            if (a >= 0 && (uint32_t)a + 12u <= in_bytes) {
                 d0 = *reinterpret_cast<const u32_unaligned *>(p.a + a);
                 d1 = *reinterpret_cast<const u32_unaligned *>(p.a + a + 4);
                 d2 = *reinterpret_cast<const u32_unaligned *>(p.a + a + 8);
             } else {  // the first pixel of the first image and the last of the last: byte by byte, inside the tensor
                 for (int j = 0; j < 9; ++j) {
-                    const long b = a + j;
-                    const uint32_t v = b >= 0 && b < (long)in_bytes ? p.a[b] : 0u;
+                    const int b = a + j;
+                    const uint32_t v = b >= 0 && (uint32_t)b < in_bytes ? p.a[b] : 0u;
                     if (j < 4) d0 |= v << (8 * j);
                     else if (j < 8) d1 |= v << (8 * (j - 4));
                     else d2 |= v;
