@@ -11,8 +11,16 @@ repeated at the top level as "images_per_s".
 Memory-bound workloads are timed twice: "warm" replays one set of buffers (every
 working set here is smaller than the 256 MB Infinity Cache, so the bytes come
 from that cache, not from HBM), "cold" rotates over enough buffer sets that a
-set has been evicted before it is used again.  The cold figure is the one the
-HBM roofline fraction is quoted on.
+set has been evicted before it is used again.  For the HBM-bound workloads
+under "others" the cold figure is the one the roofline fraction is quoted on
+(the warm one stands beside it as roofline_warm).  The headline (`value`,
+`roofline`) is the warm figure of the MFMA-bound GEMM; its cold figure stands at
+the top level as `roofline_cold`.
+
+The MobileNetV2 figure is given twice: `images_per_s` (operator plans over the
+C ABI, one graph replay per four batches) and `images_per_s_operator_api` (the
+network described as an operator list, built by the C++ OperationConstructor and
+run by the OperationExecutor, the level the reference binds its userdriver at).
 
 Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this build uses one GPU."""
 import argparse
@@ -222,6 +230,42 @@ def mbv2_workload(eden, synth, batch=64, per_channel=False, weights="minmax", co
                 pool_bytes=net.pool_bytes)
 
 
+def mbv2_userdriver(eden, batch=64, per_channel=False, list_id=0xC5):
+    """The same network through the operator API the reference binds: described as an operator list, opened by the C++
+    OperationConstructor on a HipComputeLibrary (HipConvolution ... operators, pooled feature maps), executed by the
+    OperationExecutor, which records the list into a HIP graph on its second execution and replays it.  Returns
+    (driver, list id, logits shape); the input tensor holds network_input(batch)."""
+    mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+    ud = importlib.import_module("cl-eden-kernel_amd.userdriver")
+    driver = ud.UserDriver(0)
+    ol, _, _, shape = mobilenet.operator_list(ud, list_id, batch, per_channel=per_channel)
+    driver.open_subgraph(ol)
+    driver.write_input(list_id, 0, mobilenet.network_input(batch))
+    return driver, list_id, shape
+
+
+def time_userdriver(eden, driver, list_id, steps, warmup):
+    """`steps` executions of the list's operators (OperationExecutor::execute, tensors resident), timed by wall clock
+    and by HIP events on the userdriver's own stream; repeated like time_steps when shorter than MIN_TIMED_SECONDS."""
+    driver.execute_operators(list_id, max(warmup, 3))   # the first runs operator by operator, the second records
+    driver.synchronize()
+    e0, e1 = eden.Event(), eden.Event()
+    repeats = 1
+    while True:
+        device_sync()
+        t0 = time.perf_counter()
+        e0.record(driver.stream)
+        driver.execute_operators(list_id, steps * repeats)
+        e1.record(driver.stream)
+        driver.synchronize()
+        device_sync()
+        wall = time.perf_counter() - t0
+        ev = e1.elapsed_ms_since(e0) * 1e-3
+        if wall >= MIN_TIMED_SECONDS or repeats >= 4096:
+            return wall / repeats, ev / repeats, repeats
+        repeats = min(4096, max(repeats * 2, int(repeats * MIN_TIMED_SECONDS * 1.3 / max(wall, 1e-6)) + 1))
+
+
 def copy_workload(eden, synth, mib=64, cold=False):
     """A plain device-to-device copy of known size: the yardstick the HBM byte counters are scaled by."""
     nbytes = mib << 20
@@ -304,28 +348,38 @@ def cpu_baseline(work):
                 sample="full workload (M=256, K=4096, N=4096) %d times, median %.4f s per run, %.1f s of CPU time in all; GPU output checked equal" % (len(times), t, sum(times)))
 
 
-def check_network(work):
-    """The checker's part of the MobileNetV2 line: the network object that is about to be timed (batch 64) runs 32
-    repetitions of a pair of images and every image's logits must equal the CPU oracle's for that image of the pair;
-    the oracle's own time for the pair is the CPU figure.  Raises SystemExit on a mismatch."""
+def check_network(work, userdriver=None):
+    """The checker's part of the MobileNetV2 line: the network object that is about to be timed (batch 64) runs eight
+    distinct images scattered over its batch positions (seeded, without a period) and the logits at every position
+    must equal the CPU oracle's for the image that sits there; so must the logits of the same batch run through the
+    userdriver's operator list when one is given.  The oracle's own time for the eight images is the CPU figure.
+    Raises SystemExit on a mismatch."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from harness import oracle_forward
+    from harness import oracle_forward, scattered_batch
     mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
     net = work["net"]
-    pair = mobilenet.network_input(2)
+    distinct = mobilenet.network_input(8)
     t0 = time.perf_counter()
-    _, _, want = oracle_forward(pair, 224, work["per_channel"], work["weights"])
+    _, _, want = oracle_forward(distinct, 224, work["per_channel"], work["weights"])
     cpu_s = time.perf_counter() - t0
-    net.set_input(np.tile(pair, (net.batch // 2, 1, 1, 1)))
+    where = scattered_batch(net.batch, 8)
+    x = np.ascontiguousarray(distinct[where])
+    ref = want[-1].reshape(8, -1)[where]
+    net.set_input(x)
     net.run()
     eden_mod.sync(None)
-    got = net.logits()
-    ref = want[-1].reshape(2, -1)
-    for img in range(net.batch):
-        if not np.array_equal(got[img], ref[img % 2]):
-            raise SystemExit("bench: %s: logits of image %d differ from the CPU oracle" % (work["name"], img))
+    if not np.array_equal(net.logits(), ref):
+        raise SystemExit("bench: %s: logits differ from the CPU oracle" % work["name"])
     net.set_input(mobilenet.network_input(net.batch))
-    return round(2 / cpu_s, 2)
+    if userdriver is not None:
+        driver, list_id, shape = userdriver
+        driver.write_input(list_id, 0, x)
+        driver.execute_operators(list_id, 3)   # direct, recorded, replayed: the replay's logits are the ones read
+        driver.synchronize()
+        if not np.array_equal(driver.read_output(list_id, 0, shape), ref):
+            raise SystemExit("bench: %s through the operator API: logits differ from the CPU oracle" % work["name"])
+        driver.write_input(list_id, 0, mobilenet.network_input(net.batch))
+    return round(8 / cpu_s, 2)
 
 
 def measure(eden, synth, stream, make, steps, warmup, use_graph, cold_too):
@@ -362,7 +416,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the oracle check of the network")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2, mbv2narrow, mbv2pc, copy, tonhwc, tonchw")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2, mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, copy, tonhwc, tonchw")
     ap.add_argument("--cold", action="store_true", help="with --only: rotate over buffer sets that together exceed the Infinity Cache")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -389,6 +443,17 @@ def main():
                     stream16=stream_workload, stream16big=shaped(stream_workload, out_bytes=256 * 56 * 56 * 144),
                     stream41=shaped(stream_workload, mode=2, out_bytes=32 * 28 * 28 * 144),
                     stream41big=shaped(stream_workload, mode=2, out_bytes=256 * 28 * 28 * 144))
+    if args.only in ("mbv2ud", "mbv2udpc"):
+        mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+        driver, list_id, _ = mbv2_userdriver(eden, per_channel=args.only == "mbv2udpc")
+        if args.no_graph:
+            driver.set_replay(False)
+        steps = min(args.steps, 200)
+        wall, ev, reps = time_userdriver(eden, driver, list_id, steps, max(3, min(args.warmup, 10)))
+        print(json.dumps(dict(workload="mobilenet_v2_1.0_224_u8_batch64 through OperationConstructor / OperationExecutor", steps=steps,
+                              ms_per_step=wall / steps * 1e3, us_per_step_by_events=ev / steps * 1e6, timed_region_repeats=reps,
+                              images_per_s=round(64 * steps / wall, 1), executor=driver.stats(list_id))))
+        return
     if args.only:
         work = families[args.only](eden, synth, cold=args.cold)
         args.steps = round_steps(args.steps, work["sets"], work.get("chunk", 50))
@@ -436,17 +501,34 @@ def main():
     if not args.no_others:
         # MobileNetV2 (BASELINE configs[4]): checked against the oracle before it is timed
         net = mbv2_workload(eden, synth)
+        via_api = mbv2_userdriver(eden)
         if not args.no_cpu:
-            result["cpu_baseline"]["mobilenet_v2_images_per_s"] = check_network(net)
-            result["cpu_baseline"]["mobilenet_v2_sample"] = "2 images (224x224x3) through the oracle's operator list; the batch-64 GPU network's logits checked equal on 32 repetitions of the pair"
+            result["cpu_baseline"]["mobilenet_v2_images_per_s"] = check_network(net, via_api)
+            result["cpu_baseline"]["mobilenet_v2_sample"] = ("8 images (224x224x3) through the oracle's operator list; the batch-64 GPU network's logits checked equal, through "
+                                                            "the C ABI and through the operator API, on those 8 images scattered over the 64 batch positions")
         wall2, ev2, reps2 = time_steps(eden, stream, net["launch"], 40, 4, use_graph, net["chunk"])
         c5 = dict(workload=net["name"], steps=40, tops=round(net["ops"] * 40 / wall2 / 1e12, 2), roofline=roofline(net, ev2, 40),
                   images_per_s=round(net["images"] * 40 / wall2, 1), checked_against_oracle=not args.no_cpu)
         c5["roofline"]["buffers"] = "one step streams %.0f MB of feature maps (each written once and read by the next operators) through a pool of %.0f MB" % (net["working_set"] / 1e6, net["pool_bytes"] / 1e6)
         c5["pool_bytes"] = net["pool_bytes"]
+        # the same network built by OperationConstructor from an operator-list description and run by OperationExecutor
+        if not use_graph:
+            via_api[0].set_replay(False)
+        wall3, ev3, reps3 = time_userdriver(eden, via_api[0], via_api[1], 40, 4)
+        api_stats = via_api[0].stats(via_api[1])
+        c5["operator_api"] = dict(path="eud_open_subgraph -> HipUserDriver -> OperationConstructor (HipComputeLibrary tensors and operators, pooled buffers) -> "
+                                       "OperationExecutor (recorded once, replayed)", images_per_s=round(net["images"] * 40 / wall3, 1),
+                                  us_per_batch_by_events=round(ev3 / 40 * 1e6, 1), executor=api_stats, checked_against_oracle=not args.no_cpu)
         result["images_per_s"] = c5["images_per_s"]
-        result["config"]["images_per_s"] = ("MobileNetV2-1.0 uint8 224x224x3, batch 64, per-tensor min/max quantized random-init weights "
-                                            "(BASELINE configs[4]), one HIP graph replay per batch; ms per batch %.4f" % (wall2 / 40 * 1e3))
+        result["images_per_s_operator_api"] = c5["operator_api"]["images_per_s"]
+        result["config"]["images_per_s"] = c5["images_per_s"]
+        result["config"]["images_per_s_operator_api"] = c5["operator_api"]["images_per_s"]
+        result["config"]["images_per_s_workload"] = ("MobileNetV2-1.0 uint8 224x224x3, batch 64, per-tensor min/max quantized random-init weights "
+                                                     "(BASELINE configs[4]); images_per_s: operator plans over the C ABI, one HIP graph replay per 4 batches, "
+                                                     "ms per batch %.4f; images_per_s_operator_api: the operator list opened and executed through the "
+                                                     "userdriver classes (OperationConstructor / OperationExecutor), ms per batch %.4f" % (wall2 / 40 * 1e3, wall3 / 40 * 1e3))
+        via_api[0].close()
+        del via_api
         del net
         others = [c5]
         for make, steps, cold_too in ((conv_workload, 2000, False), (shaped(conv_workload, n=64), 300, False),
@@ -463,6 +545,12 @@ def main():
                                       (shaped(mbv2_workload, per_channel=True), 40, False)):
             others.append(measure(eden, synth, stream, make, steps, max(4, steps // 10), use_graph, cold_too))
         result["others"] = others
+        # the headline workload on cold buffers (sets rotated so that nothing is found in the Infinity Cache), beside the
+        # warm figure `value` and `roofline` are measured on
+        for entry in others:
+            if entry["workload"] == "fc_m256_k4096_n4096" and "roofline_warm" in entry:
+                result["roofline_cold"] = entry["roofline"]
+    result["roofline"]["buffers"] = "warm: one set of tensors replayed; the 16 MiB of weights are found in the 256 MB Infinity Cache (roofline_cold: rotated sets)"
     print(json.dumps(result))
 
 

@@ -1,5 +1,6 @@
-"""Builds libedenhip.so (HIP kernels + C ABI) and libedenhip_ud.so's test driver
-for gfx950 with hipcc.  Everything is built in-tree; nothing is installed."""
+"""Builds libedenhip.so (HIP kernels + the operator-level C ABI, include/eden_hip.h) for gfx950 with hipcc, and
+libedenud.so (the C++ host classes behind the userdriver-level C ABI, include/eden_ud.h) with g++ against it.
+Everything is built in-tree; nothing is installed."""
 import os
 import re
 import subprocess
@@ -12,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 HOST = os.path.join(HERE, "host")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libedenhip.so")
-UD_TEST = os.path.join(HERE, "ud_op_test")
+UD_LIB = os.path.join(HERE, "libedenud.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -84,21 +85,16 @@ def build_lib(jobs=8):
     return LIB
 
 
-def build_ud_test():
-    """The C++ operator classes (header-only, host/) with their test driver, linked against libedenhip.so."""
-    src = os.path.join(HOST, "ud_op_test.cpp")
-    if not os.path.exists(src):
-        return None
-    _run(["g++", "-O2", "-std=c++17", "-Wall", "-I" + os.path.join(ROOT, "include"), "-I" + HOST,
-          "-I" + os.path.join(ROOT, "oracle"), src, "-o", UD_TEST,
-          "-L" + HERE, "-ledenhip", "-Wl,-rpath,$ORIGIN", "-L" + os.path.join(ROOT, "oracle"), "-loracle",
-          "-Wl,-rpath,$ORIGIN/../oracle"])
-    return UD_TEST
+def build_ud_lib():
+    """The userdriver level: host/*.hpp (header-only C++ classes) behind host/ud_c_api.cpp, linked against libedenhip.so."""
+    _run(["g++", "-O2", "-std=c++17", "-Wall", "-fPIC", "-shared", "-I" + os.path.join(ROOT, "include"), "-I" + HOST,
+          os.path.join(HOST, "ud_c_api.cpp"), "-o", UD_LIB, "-L" + HERE, "-ledenhip", "-Wl,-rpath,$ORIGIN"])
+    return UD_LIB
 
 
 def build_all():
     lib = build_lib()
-    build_ud_test()
+    build_ud_lib()
     return lib
 
 

@@ -171,7 +171,8 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         g.cfg.id = GEMM_C3K3;
         g.cfg.slab = 32;
     } else if (g.vec == 16 && g.taps == 9 && g.k == 9 * g.cin && units.size() == (size_t)g.k / 16 && g.proto.stride_h == 1 &&
-               g.proto.stride_w == 1 && g.proto.out_sy == 1 && g.proto.out_sx == 1 && units_are_3x3(units, g.cin / 16) &&
+               g.proto.stride_w == 1 && g.proto.out_sy == 1 && g.proto.out_sx == 1 && g.proto.out_y0 == 0 && g.proto.out_x0 == 0 &&
+               g.proto.out_h == g.proto.ho && g.proto.out_w == g.proto.wo && units_are_3x3(units, g.cin / 16) &&
                conv3x3_patch_applies(g.cin, g.proto.cin, g.proto.wo, g.proto.ho)) {
         // 3x3 taps at dilation 1 and stride 1 over all input channels: the patch-in-LDS kernel
         g.cfg.id = GEMM_CONV3X3;
@@ -638,6 +639,8 @@ int eh_init(int device) {
         set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
         return EH_FAILURE;
     }
+    int rc = conv3x3_patch_prepare();  // per-device kernel attributes, set here so that no launch has to
+    if (rc) return rc;
     uint8_t *unused = nullptr;
     return static_scratch(&unused);  // this device's address of the static scratch, asked for while the device is current
 }

@@ -23,6 +23,8 @@
 // per pixel from v_dot4 over the same fragments); a lane ends up with 16 consecutive channels of one pixel.
 #include <type_traits>
 
+#include <atomic>
+
 #include "eh_internal.h"
 
 namespace eh {
@@ -330,12 +332,6 @@ int launch_nb(const GemmProblem &p, const Conv3Launch &L, size_t lds, hipStream_
     const dim3 grid((unsigned)((L.tiles + 7) / 8 * 8), (unsigned)((n_blocks + NB - 1) / NB));
     auto launch_pc = [&](auto rowsum_c, auto qm_c, auto pc_c) {
         auto kernel = conv3x3_patch_kernel<NB, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(pc_c)::value>;
-        static bool raised = false;  // per kernel variant: dynamic LDS beyond 64 KiB has to be allowed once
-        if (lds > 64 * 1024 && !raised) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsMax);
-            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(conv3x3_patch_kernel)");
-            raised = true;
-        }
         hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, p, L);
         return (int)EH_OK;
     };
@@ -363,9 +359,43 @@ bool conv3x3_patch_applies(int32_t cin_group, int32_t pixel_stride, int32_t wo, 
     return conv3_lds_bytes(1, cin_group, wo, 1) <= kLdsMax;
 }
 
+// Allows every variant of the kernel its dynamic LDS beyond 64 KiB on the current device.  Done once per device when the
+// library is initialised on it, so that a launch (which may sit in a capture or in a caller that must not meet the
+// driver) is a launch and nothing else.
+static std::atomic<bool> g_conv3_prepared{false};
+
+int conv3x3_patch_prepare() {
+    int rc = EH_OK;
+    auto raise = [&](auto kernel) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsMax);
+        if (e != hipSuccess && rc == EH_OK) rc = hip_fail(e, "hipFuncSetAttribute(conv3x3_patch_kernel)");
+    };
+    auto each_pc = [&](auto nb_c, auto rowsum_c, auto qm_c) {
+        raise(conv3x3_patch_kernel<decltype(nb_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value, false>);
+        raise(conv3x3_patch_kernel<decltype(nb_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value, true>);
+    };
+    auto each_qm = [&](auto nb_c, auto rowsum_c) {
+        each_pc(nb_c, rowsum_c, std::integral_constant<int, 0>{});
+        each_pc(nb_c, rowsum_c, std::integral_constant<int, 1>{});
+        each_pc(nb_c, rowsum_c, std::integral_constant<int, 2>{});
+    };
+    auto each_rowsum = [&](auto nb_c) {
+        each_qm(nb_c, std::false_type{});
+        each_qm(nb_c, std::true_type{});
+    };
+    each_rowsum(std::integral_constant<int, 1>{});
+    each_rowsum(std::integral_constant<int, 2>{});
+    if (rc == EH_OK) g_conv3_prepared.store(true, std::memory_order_release);
+    return rc;
+}
+
 int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream) {
     EH_REQUIRE(p.k == 9 * p.cin && (p.cin & 31) == 0 && p.k_pad == p.k && p.stride_h == 1 && p.stride_w == 1,
                "conv3x3: unsupported problem (k %d, cin %d)", p.k, p.cin);
+    // the kernel addresses the output as one dense image per input image: no window, offset or stride on the output side
+    EH_REQUIRE(p.out_sy == 1 && p.out_sx == 1 && p.out_y0 == 0 && p.out_x0 == 0 && p.out_h == p.ho && p.out_w == p.wo,
+               "conv3x3: the output must be the whole dense image (window %d x %d at %d,%d step %d,%d for %d x %d)", p.out_h, p.out_w,
+               p.out_y0, p.out_x0, p.out_sy, p.out_sx, p.ho, p.wo);
     EH_REQUIRE((reinterpret_cast<uintptr_t>(p.a) & 15) == 0, "conv3x3: input pointer is not aligned to 16 bytes");
     const int n_img = p.m / (p.ho * p.wo);
     int th = 1, nb = 1;
@@ -383,6 +413,10 @@ int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream) {
     L.div_tiles = make_fastdiv((uint32_t)L.tiles_per_image);
     const size_t lds = conv3_lds_bytes(nb, p.cin, p.wo, th);
     EH_REQUIRE(lds <= kLdsMax, "conv3x3: %zu bytes of LDS", lds);
+    if (!g_conv3_prepared.load(std::memory_order_acquire)) {  // a caller that never went through eh_init
+        const int rc = conv3x3_patch_prepare();
+        if (rc) return rc;
+    }
     return nb == 2 ? launch_nb<2>(p, L, lds, stream) : launch_nb<1>(p, L, lds, stream);
 }
 

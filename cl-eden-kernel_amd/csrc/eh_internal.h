@@ -418,6 +418,7 @@ inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
 int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream);
+int conv3x3_patch_prepare();  // per device, from eh_init
 bool conv3x3_patch_applies(int32_t cin_group, int32_t pixel_stride, int32_t wo, int32_t ho);
 bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, int32_t channel_offset, int32_t y_base,
                         int32_t x_base, int64_t m, int64_t n);

@@ -44,7 +44,7 @@ struct eh_pool {
     size_t layout() {
         size_t at = 0;
         for (auto &s : slots) {
-            if (s.generation != generation) continue;
+            if (s.generation != generation || s.released) continue;  // a buffer released before assignment gets no memory
             s.offset = at + kHead;
             at += padded(s.bytes);
         }
@@ -73,7 +73,14 @@ int eh_pool_request(eh_pool *pool, int kind, size_t bytes, int32_t *slot) {
         s.live = true;
         s.generation = gen;
         (void)intra;
-        slots.push_back(s);
+        try {
+            slots.push_back(s);
+        } catch (const std::bad_alloc &) {
+            {
+            eh::set_error("out of host memory");
+            return EH_FAILURE;
+        }
+        }
         *slot = (int32_t)slots.size() - 1;
         return EH_OK;
     };
@@ -82,7 +89,7 @@ int eh_pool_request(eh_pool *pool, int kind, size_t bytes, int32_t *slot) {
         // the first buffer handed back by resetInterBuffer, grown if it is too small (CLRuntime.cpp:52-72)
         for (size_t i = 0; i < slots.size(); ++i) {
             Slot &s = slots[i];
-            if (s.generation == gen && s.kind != EH_POOL_INTRA && !s.live) {
+            if (s.generation == gen && s.kind != EH_POOL_INTRA && !s.live && !s.released) {
                 if (s.bytes < bytes) s.bytes = bytes;
                 s.live = true;
                 *slot = (int32_t)i;
@@ -96,13 +103,13 @@ int eh_pool_request(eh_pool *pool, int kind, size_t bytes, int32_t *slot) {
     int best = -1;
     for (size_t i = 0; i < slots.size(); ++i) {
         const Slot &s = slots[i];
-        if (s.generation == gen && s.kind == EH_POOL_INTRA && !s.live && s.bytes >= bytes && (best < 0 || s.bytes < slots[best].bytes))
+        if (s.generation == gen && s.kind == EH_POOL_INTRA && !s.live && !s.released && s.bytes >= bytes && (best < 0 || s.bytes < slots[best].bytes))
             best = (int)i;
     }
     if (best < 0) {
         for (size_t i = 0; i < slots.size(); ++i) {
             const Slot &s = slots[i];
-            if (s.generation == gen && s.kind == EH_POOL_INTRA && !s.live && (best < 0 || s.bytes > slots[best].bytes)) best = (int)i;
+            if (s.generation == gen && s.kind == EH_POOL_INTRA && !s.live && !s.released && (best < 0 || s.bytes > slots[best].bytes)) best = (int)i;
         }
         if (best >= 0) slots[best].bytes = bytes;
     }
@@ -115,7 +122,7 @@ int eh_pool_request(eh_pool *pool, int kind, size_t bytes, int32_t *slot) {
 int eh_pool_reset_inter(eh_pool *pool, int32_t slot) {
     EH_REQUIRE(pool != nullptr, "null pool");
     EH_REQUIRE(slot >= 0 && (size_t)slot < pool->slots.size() && pool->slots[slot].generation == pool->generation &&
-                   pool->slots[slot].kind != EH_POOL_INTRA,
+                   pool->slots[slot].kind != EH_POOL_INTRA && !pool->slots[slot].released,
                "resetInterBuffer: slot %d is not a pooled feature map of the list being built", slot);
     pool->slots[slot].live = false;
     return EH_OK;
@@ -132,7 +139,7 @@ int eh_pool_layout(eh_pool *pool, size_t *arena_bytes, int32_t *slot_count) {
     EH_REQUIRE(pool != nullptr, "null pool");
     const size_t total = pool->layout();
     int32_t count = 0;
-    for (auto &s : pool->slots) count += s.generation == pool->generation ? 1 : 0;
+    for (auto &s : pool->slots) count += (s.generation == pool->generation && !s.released) ? 1 : 0;
     if (arena_bytes) *arena_bytes = total;
     if (slot_count) *slot_count = count;
     return EH_OK;
@@ -143,12 +150,20 @@ int eh_pool_assign(eh_pool *pool, size_t *arena_bytes) {
     const size_t total = pool->layout();
     Arena arena;
     arena.bytes = total;
-    if (total > 0) {
+    // slots released before this assignment were left out of the layout and do not keep the allocation alive
+    for (auto &s : pool->slots) arena.live_slots += (s.generation == pool->generation && !s.released) ? 1 : 0;
+    try {
+        pool->arenas.resize((size_t)pool->generation + 1);
+    } catch (const std::bad_alloc &) {
+        {
+            eh::set_error("out of host memory");
+            return EH_FAILURE;
+        }
+    }
+    if (total > 0 && arena.live_slots > 0) {
         int rc = eh_malloc(&arena.base, total);  // zero-filled: the reference zero-fills its intra buffers (:124-129)
         if (rc) return rc;
     }
-    for (auto &s : pool->slots) arena.live_slots += s.generation == pool->generation ? 1 : 0;
-    pool->arenas.resize((size_t)pool->generation + 1);
     pool->arenas[pool->generation] = arena;
     ++pool->generation;  // the pools are forgotten: later requests start another list (:131-135)
     if (arena_bytes) *arena_bytes = total;

@@ -1,141 +1,62 @@
 // Operator construction from TFLite-style options, and the executor of the resulting list.
 //
 // Mirrors OperationConstructor / OperationExecutor of the reference
-// (src/userdriver/gpu/gpu_op_constructor.cc:63-383 CONV_2D / DEPTHWISE_CONV_2D / TRANSPOSE_CONV /
-// FULLY_CONNECTED, :789-860 AVERAGE_POOL_2D, :1166-1205 ADD, :1797-1850 open_oplist, :1884-2009
-// layout / precision / padding helpers, :2062-2191 tensor allocation with inter-buffer reuse;
-// src/userdriver/gpu/gpu_op_executor.cc:56-103) for the six operators this backend has.
+// (src/userdriver/gpu/gpu_op_constructor.h:33-56, gpu_op_constructor.cc:63-383 CONV_2D / DEPTHWISE_CONV_2D /
+// TRANSPOSE_CONV / FULLY_CONNECTED, :789-860 AVERAGE_POOL_2D, :1166-1205 ADD, :1797-1870 open_oplist / close_oplist,
+// :1884-2009 layout / precision / padding helpers, :2062-2191 tensor allocation with inter-buffer reuse;
+// src/userdriver/gpu/gpu_op_executor.h:31-44, gpu_op_executor.cc:56-103) for the six operators this backend has.
+// Both are built on a HipComputeLibrary, as the reference's are on its CLComputeLibrary: every tensor comes from
+// create_tensor / create_and_copy_tensor, every operator from create<Operator>(precision), pooled buffers are
+// materialised by assignBuffers().
 //
-// The reference reads flatbuffer tables (TFlite::Conv2DOptions, ...) out of a loaded model.  The
-// model loader is not part of this backend, so the option tables are plain structs with the
-// schema's field names (src/model/schema/nnc/v2/schema.fbs:547-567,580-606,659-695,953-962), and
-// OperatorDesc / TensorDesc stand where model::component::Operator / FeatureMap / Parameter do.
+// Where the executor differs: the reference enqueues every operator's kernels on one in-order queue at each execution
+// (one clFlush per subgraph).  Here a list whose operators only launch kernels is recorded into a HIP graph the second
+// time it runs with the same tensors and quantization parameters, and replayed from then on (one launch per execution
+// instead of one per kernel); anything that changes what was recorded (a tensor's scale or zero point, a buffer that
+// moved) makes the next execution run operator by operator again and re-record.
 #pragma once
 
 #include <map>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
-#include "HipOperators.hpp"
+#include "HipComputeLibrary.hpp"
+#include "ModelDesc.hpp"
 #include "userdriver_operator.hpp"
 
-namespace TFlite {
-
-enum Padding { Padding_SAME = 0, Padding_VALID = 1 };
-enum ActivationFunctionType {
-    ActivationFunctionType_NONE = 0,
-    ActivationFunctionType_RELU = 1,
-    ActivationFunctionType_RELU_N1_TO_1 = 2,
-    ActivationFunctionType_RELU6 = 3,
-};
-enum LegacyModel {
-    LegacyModel_CAFFE = 0,
-    LegacyModel_TENSORFLOW = 1,
-    LegacyModel_CAFFE_NCHW = 2,
-    LegacyModel_CAFFE_NHWC = 3,
-    LegacyModel_TENSORFLOW_NCHW = 4,
-    LegacyModel_TENSORFLOW_NHWC = 5,
-    LegacyModel_ANDROID_NN = 6,
-};
-enum TensorType { TensorType_FLOAT32 = 0, TensorType_FLOAT16 = 1, TensorType_INT32 = 2, TensorType_UINT8 = 3, TensorType_INT8 = 9 };
-enum BuiltinOperator {
-    BuiltinOperator_ADD = 0,
-    BuiltinOperator_AVERAGE_POOL_2D = 1,
-    BuiltinOperator_CONV_2D = 3,
-    BuiltinOperator_DEPTHWISE_CONV_2D = 4,
-    BuiltinOperator_FULLY_CONNECTED = 9,
-    BuiltinOperator_TRANSPOSE_CONV = 67,
-};
-
-struct Conv2DOptions {
-    Padding padding = Padding_SAME;
-    int32_t stride_w = 1, stride_h = 1;
-    ActivationFunctionType fused_activation_function = ActivationFunctionType_NONE;
-    int32_t dilation_w_factor = 1, dilation_h_factor = 1;
-    std::vector<int32_t> padding_value;  // androidNN: explicit {left, right, top, bottom}
-    bool use_nchw = false;               // androidNN
-};
-struct DepthwiseConv2DOptions {
-    Padding padding = Padding_SAME;
-    int32_t stride_w = 1, stride_h = 1;
-    int32_t depth_multiplier = 1;
-    ActivationFunctionType fused_activation_function = ActivationFunctionType_NONE;
-    int32_t dilation_w_factor = 1, dilation_h_factor = 1;
-    std::vector<int32_t> padding_value;
-    bool use_nchw = false;
-};
-struct TransposeConvOptions {
-    Padding padding = Padding_SAME;
-    int32_t stride_w = 1, stride_h = 1;
-    int32_t group = 1;
-    ActivationFunctionType fused_activation_function = ActivationFunctionType_NONE;
-    std::vector<int32_t> padding_value;
-    bool use_nchw = false;
-};
-struct Pool2DOptions {
-    Padding padding = Padding_VALID;
-    int32_t stride_w = 1, stride_h = 1;
-    int32_t filter_width = 1, filter_height = 1;
-    ActivationFunctionType fused_activation_function = ActivationFunctionType_NONE;
-    std::vector<int32_t> padding_value;
-    bool use_nchw = false;
-};
-struct FullyConnectedOptions {
-    ActivationFunctionType fused_activation_function = ActivationFunctionType_NONE;
-};
-struct AddOptions {
-    ActivationFunctionType fused_activation_function = ActivationFunctionType_NONE;
-    bool pot_scale_int16 = true;
-    std::vector<float> coeff;
-};
-
-}  // namespace TFlite
 
 namespace enn {
 namespace ud {
 namespace hip {
 
-// An edge of the model graph: a feature map (is_const false, buffer_index names its storage) or a
-// parameter (is_const true, data points at the host bytes).
-struct TensorDesc {
-    std::string name;
-    NDims shape;
-    TFlite::TensorType data_type = TFlite::TensorType_UINT8;
-    float scale = 1.0f;
-    int32_t zero_point = 0;
-    bool is_const = false;
-    const void *data = nullptr;
-    int32_t buffer_index = UNDEFINED;
-    std::vector<float> per_channel_scales;  // symmetric per-channel quantization of a filter; empty otherwise
-};
-
-struct OperatorDesc {
-    std::string name;
-    uint64_t id = 0;
-    TFlite::BuiltinOperator code = TFlite::BuiltinOperator_CONV_2D;
-    std::vector<std::shared_ptr<TensorDesc>> in_tensors, out_tensors;
-    std::shared_ptr<void> option;  // the TFlite::*Options struct that belongs to `code`
-};
-
-struct OperatorListDesc {
-    uint64_t id = 0;
-    TFlite::LegacyModel legacy_model = TFlite::LegacyModel_TENSORFLOW_NHWC;
-    std::vector<OperatorDesc> operators;
-};
-
 class OperationConstructor {
 public:
-    explicit OperationConstructor(std::shared_ptr<HipRuntime> runtime) : runtime_(runtime) {}
+    explicit OperationConstructor(std::shared_ptr<HipComputeLibrary> compute_library) : compute_library_(compute_library) {}
+    ~OperationConstructor() {
+        alloc_tensors_map_.clear();
+        tensors_used_.clear();
+    }
 
-    // Builds every operator of the list in order (tensors are created as the operators name them; a
-    // feature map's storage is handed back to the pool once its last reader has been built) and
-    // materialises the pooled buffers.
-    EnnReturn open_oplist(const OperatorListDesc &list) {
+    // IOperationConstructor (src/userdriver/common/IOperationConstructor.h:28-37)
+    EnnReturn initialize_ud_operators() {
         operators = std::make_shared<std::vector<std::shared_ptr<UDOperator>>>();
         in_tensors.clear();
         out_tensors.clear();
-        alloc_tensors_.clear();
+        return ENN_RET_SUCCESS;
+    }
+    const UDOperators &get_ud_operators() { return operators; }
+    const UDTensors &get_in_tensors() const { return in_tensors; }
+    const UDTensors &get_out_tensors() const { return out_tensors; }
+
+    // Builds every operator of the list in order (tensors are created as the operators name them; a
+    // feature map's storage is handed back to the pool once its last reader has been built), materialises
+    // the pooled buffers and waits for the device (gpu_op_constructor.cc:1797-1850).
+    EnnReturn open_oplist(const OperatorListDesc &list) {
+        std::lock_guard<std::mutex> lock_guard(mutex_constructor_);
+        if (!operators) initialize_ud_operators();
+        operator_list_id_ = list.id;
         tensors_used_.clear();
         produced_.clear();
         consumed_.clear();
@@ -154,26 +75,48 @@ public:
             if (fuse_residual_adds && index + 1 < list.operators.size() && fusable_add(op, list.operators[index + 1])) {
                 if (create_conv_with_add(op, list.operators[index + 1]) != ENN_RET_SUCCESS) {
                     ERROR_PRINT("OperationConstructor: building %s with its residual add failed\n", op.name.c_str());
-                    return ENN_RET_FAILED;
+                    return abandon();
                 }
                 ++index;  // the Add went into the convolution's launch
                 continue;
             }
-            switch (op.code) {
-                case TFlite::BuiltinOperator_CONV_2D: rc = create_conv(op); break;
-                case TFlite::BuiltinOperator_DEPTHWISE_CONV_2D: rc = create_depthwise(op); break;
-                case TFlite::BuiltinOperator_TRANSPOSE_CONV: rc = create_deconv(op); break;
-                case TFlite::BuiltinOperator_FULLY_CONNECTED: rc = create_fc(op); break;
-                case TFlite::BuiltinOperator_AVERAGE_POOL_2D: rc = create_avgpool(op); break;
-                case TFlite::BuiltinOperator_ADD: rc = create_add(op); break;
-                default: ERROR_PRINT("OperationConstructor: operator code %d is not offered\n", (int)op.code);
-            }
+            rc = create_ud_operator(op);
             if (rc != ENN_RET_SUCCESS) {
                 ERROR_PRINT("OperationConstructor: building %s failed\n", op.name.c_str());
-                return ENN_RET_FAILED;
+                return abandon();
             }
         }
-        return runtime_->assignBufferPool() == Status::SUCCESS ? ENN_RET_SUCCESS : ENN_RET_FAILED;
+        compute_library_->assignBuffers();
+        compute_library_->synchronize();
+        tensors_used_.clear();
+        produced_.clear();
+        consumed_.clear();
+        for (const auto &kv : alloc_tensors_map_[operator_list_id_])  // a pooled buffer that assignBuffers() could not place
+            if (kv.second->getNumOfBytes() != 0 && std::static_pointer_cast<HipTensor>(kv.second)->getDataPtr() == nullptr) {
+                ERROR_PRINT("OperationConstructor: feature map %d has no device memory after assignBuffers()\n", kv.first);
+                return ENN_RET_FAILED;
+            }
+        return ENN_RET_SUCCESS;
+    }
+
+    // Drops the constructor's own references to the list's feature maps (gpu_op_constructor.cc:1852-1870); the
+    // operators keep theirs until the userdriver forgets the list.
+    void close_oplist(const uint64_t &oplist_id) {
+        std::lock_guard<std::mutex> lock_guard(mutex_constructor_);
+        alloc_tensors_map_.erase(oplist_id);
+    }
+
+    EnnReturn create_ud_operator(const OperatorDesc &op) {
+        switch (op.code) {
+            case TFlite::BuiltinOperator_CONV_2D: return create_conv(op);
+            case TFlite::BuiltinOperator_DEPTHWISE_CONV_2D: return create_depthwise(op);
+            case TFlite::BuiltinOperator_TRANSPOSE_CONV: return create_deconv(op);
+            case TFlite::BuiltinOperator_FULLY_CONNECTED: return create_fc(op);
+            case TFlite::BuiltinOperator_AVERAGE_POOL_2D: return create_avgpool(op);
+            case TFlite::BuiltinOperator_ADD: return create_add(op);
+            default: ERROR_PRINT("OperationConstructor: operator code %d is not offered\n", (int)op.code);
+        }
+        return ENN_RET_FAILED;
     }
 
     UDOperators operators;
@@ -255,6 +198,16 @@ public:
     }
 
 private:
+    // a list that fails half way: its operators and tensors go, and the pooled buffers they asked for are given up
+    EnnReturn abandon() {
+        if (operators) operators->clear();
+        in_tensors.clear();
+        out_tensors.clear();
+        alloc_tensors_map_.erase(operator_list_id_);
+        compute_library_->abandonBuffers();
+        return ENN_RET_FAILED;
+    }
+
     static DataType to_data_type(TFlite::TensorType t) {
         switch (t) {
             case TFlite::TensorType_UINT8: return DataType::UINT8;
@@ -290,21 +243,29 @@ private:
         }
     }
 
+    // A feature map becomes a pooled run-time tensor, made once per buffer index of the list; a parameter becomes a
+    // constant tensor uploaded at once (gpu_op_constructor.cc:2062-2155).
     std::shared_ptr<ITensor> allocate_tensor(const std::shared_ptr<TensorDesc> &edge, const PrecisionType &precision,
-                                             const BufferType &buffer_type) {
+                                             const BufferType &buffer_type, const DataOrder &data_order = DataOrder::NCHW) {
         if (edge->shape.empty() || edge->shape.size() > 4) {
             ERROR_PRINT("OperationConstructor: tensor %s has %zu dimensions\n", edge->name.c_str(), edge->shape.size());
             return nullptr;
         }
-        const Dim4 dims = extendToDim4(edge->shape);
-        const DataType type = to_data_type(edge->data_type);
+        // operators read positional (n, c, h, w) extents from a four-entry shape, as the reference's CLTensor gives them
+        const Dim4 d4 = extendToDim4(edge->shape);
+        const NDims dims = {d4.n, d4.c, d4.h, d4.w};
         if (!edge->is_const) {
-            auto found = alloc_tensors_.find(edge->buffer_index);
-            if (found != alloc_tensors_.end()) return found->second;
-            std::shared_ptr<ITensor> tensor = std::make_shared<HipTensor>(runtime_, precision, type, dims, DataOrder::NCHW, edge->scale,
-                                                                          edge->zero_point, buffer_type, StorageType::BUFFER, 0,
-                                                                          edge->buffer_index);
-            alloc_tensors_[edge->buffer_index] = tensor;
+            auto &made = alloc_tensors_map_[operator_list_id_];
+            auto found = made.find(edge->buffer_index);
+            if (found != made.end()) return found->second;
+            std::shared_ptr<ITensor> tensor = compute_library_->create_tensor(edge->data_type, precision, dims, edge->buffer_index, buffer_type,
+                                                                              false, StorageType::BUFFER, data_order, edge->scale,
+                                                                              edge->zero_point);
+            if (tensor == nullptr) {
+                ERROR_PRINT("OperationConstructor: feature map %s could not be made\n", edge->name.c_str());
+                return nullptr;
+            }
+            made[edge->buffer_index] = tensor;
             if (!produced_.count(edge->buffer_index))
                 in_tensors.push_back(tensor);
             else if (!consumed_.count(edge->buffer_index))
@@ -315,19 +276,11 @@ private:
             ERROR_PRINT("OperationConstructor: parameter %s has no data\n", edge->name.c_str());
             return nullptr;
         }
-        switch (type) {
-            case DataType::UINT8:
-                return std::make_shared<HipTensor>(runtime_, precision, static_cast<const uint8_t *>(edge->data), dims, DataOrder::NCHW,
-                                                   edge->scale, edge->zero_point);
-            case DataType::INT8:
-                return std::make_shared<HipTensor>(runtime_, precision, static_cast<const int8_t *>(edge->data), dims, DataOrder::NCHW,
-                                                   edge->scale, edge->zero_point);
-            case DataType::INT32:
-                return std::make_shared<HipTensor>(runtime_, precision, static_cast<const int32_t *>(edge->data), dims, DataOrder::NCHW,
-                                                   edge->scale, edge->zero_point);
-            default: ERROR_PRINT("OperationConstructor: parameter %s has an unsupported type\n", edge->name.c_str());
-        }
-        return nullptr;
+        DataPtr data = const_cast<DataPtr>(edge->data);
+        auto tensor = compute_library_->create_and_copy_tensor(edge->data_type, data, precision, dims, UNDEFINED, buffer_type, false,
+                                                               StorageType::BUFFER, data_order, edge->scale, edge->zero_point);
+        if (tensor == nullptr) ERROR_PRINT("OperationConstructor: parameter %s could not be made\n", edge->name.c_str());
+        return tensor;
     }
 
     // outputs first (they may take over storage released by earlier operators), then inputs; an input
@@ -351,10 +304,9 @@ private:
     }
 
     template <typename Op, typename Params>
-    EnnReturn finish(const OperatorDesc &op, const PrecisionType &precision, const UDTensors &in, const UDTensors &out,
+    EnnReturn finish(const OperatorDesc &op, const std::shared_ptr<Op> &impl, const UDTensors &in, const UDTensors &out,
                      const std::shared_ptr<Params> &parameters) {
-        auto impl = std::make_shared<Op>(runtime_, precision);
-        if (impl->initialize(in, out, parameters) != Status::SUCCESS) return ENN_RET_FAILED;
+        if (impl == nullptr || impl->initialize(in, out, parameters) != Status::SUCCESS) return ENN_RET_FAILED;
         operators->push_back(std::make_shared<EnnUDOperator<Op>>(op.name, op.id, in, out, UDTensors(), impl));
         return ENN_RET_SUCCESS;
     }
@@ -364,11 +316,15 @@ private:
         return static_cast<const Options *>(op.option.get());
     }
 
-    EnnReturn create_conv(const OperatorDesc &op) {
+    // extra_in / extra_out: tensors of an Add taken into this convolution's launch; they ride at the end of the
+    // operator's tensor lists so that whoever walks the list (the executor's signature, a dump) sees them
+    EnnReturn create_conv(const OperatorDesc &op, const UDTensors &extra_in = UDTensors(), const UDTensors &extra_out = UDTensors()) {
         if (op.out_tensors.empty() || op.in_tensors.size() < 3 || !op.option) return ENN_RET_FAILED;
         const PrecisionType precision = get_precision(op.out_tensors[0]->data_type);
         UDTensors in, out;
         if (!convert_to_tensors(op, precision, in, out)) return ENN_RET_FAILED;
+        in.insert(in.end(), extra_in.begin(), extra_in.end());
+        out.insert(out.end(), extra_out.begin(), extra_out.end());
         const auto *o = options_of<TFlite::Conv2DOptions>(op);
         auto p = std::make_shared<ConvolutionParameters>();
         p->dilation = {(uint32_t)o->dilation_h_factor, (uint32_t)o->dilation_w_factor};
@@ -379,7 +335,7 @@ private:
         padding_of(*o, &p->padding, in, out, in[1]->getDims(), p->stride, p->dilation, false, p->isNCHW);
         p->per_channel_quant = !op.in_tensors[1]->per_channel_scales.empty();
         p->scales = op.in_tensors[1]->per_channel_scales;
-        return finish<HipConvolution>(op, precision, in, out, p);
+        return finish(op, compute_library_->createConvolution(precision), in, out, p);
     }
 
     // `add` consumes `conv`'s only output, nothing else does, both are uint8 per-tensor, and the sum is not
@@ -412,10 +368,10 @@ private:
         const PrecisionType precision = get_precision(add.out_tensors[0]->data_type);
         UDTensors add_in, add_out;
         if (!convert_to_tensors(add, precision, add_in, add_out)) return ENN_RET_FAILED;
-        if (create_conv(conv) != ENN_RET_SUCCESS) return ENN_RET_FAILED;
+        const bool conv_first = add.in_tensors[0]->buffer_index == conv.out_tensors[0]->buffer_index;
+        if (create_conv(conv, {add_in[conv_first ? 1 : 0]}, {add_out[0]}) != ENN_RET_SUCCESS) return ENN_RET_FAILED;
         auto wrapper = std::dynamic_pointer_cast<EnnUDOperator<HipConvolution>>(operators->back());
         if (!wrapper) return ENN_RET_FAILED;
-        const bool conv_first = add.in_tensors[0]->buffer_index == conv.out_tensors[0]->buffer_index;
         const auto *o = options_of<TFlite::AddOptions>(add);
         return wrapper->getOp()->fuseResidualAdd(add_in[conv_first ? 1 : 0], add_out[0],
                                                           to_activation(o->fused_activation_function)) == Status::SUCCESS
@@ -438,7 +394,7 @@ private:
         padding_of(*o, &p->padding, in, out, in[1]->getDims(), p->stride, p->dilation, false, p->isNCHW);
         p->per_channel_quant = !op.in_tensors[1]->per_channel_scales.empty();
         p->scales = op.in_tensors[1]->per_channel_scales;
-        return finish<HipDepthwiseConvolution>(op, precision, in, out, p);
+        return finish(op, compute_library_->createDepthwiseConvolution(precision), in, out, p);
     }
 
     EnnReturn create_deconv(const OperatorDesc &op) {
@@ -456,7 +412,7 @@ private:
         padding_of(*o, &p->padding, in, out, in[1]->getDims(), p->stride, Dim2{1, 1}, true, p->isNCHW);
         p->per_channel_quant = !op.in_tensors[1]->per_channel_scales.empty();
         p->scales = op.in_tensors[1]->per_channel_scales;
-        return finish<HipDeconvolution>(op, precision, in, out, p);
+        return finish(op, compute_library_->createDeconvolution(precision), in, out, p);
     }
 
     EnnReturn create_fc(const OperatorDesc &op) {
@@ -468,7 +424,7 @@ private:
         auto p = std::make_shared<FullyConnectedParameters>();
         p->androidNN = android_nn();
         p->activation_info = std::make_shared<ActivationInfo>(to_activation(o->fused_activation_function));
-        return finish<HipFullyConnected>(op, precision, in, out, p);
+        return finish(op, compute_library_->createFullyConnected(precision), in, out, p);
     }
 
     EnnReturn create_avgpool(const OperatorDesc &op) {
@@ -487,7 +443,7 @@ private:
         layout_of(*o, &p->androidNN, &p->isNCHW);
         // the pool takes explicit padding values from every model kind (gpu_op_constructor.cc:832-847)
         padding_of(*o, &p->padding, in, out, NDims{1, 1, p->filter.h, p->filter.w}, p->stride, Dim2{1, 1}, false, p->isNCHW, true);
-        return finish<HipAveragepool>(op, precision, in, out, p);
+        return finish(op, compute_library_->createAveragepool(precision), in, out, p);
     }
 
     EnnReturn create_add(const OperatorDesc &op) {
@@ -501,45 +457,148 @@ private:
         p->coeff = o->coeff.empty() ? std::vector<float>(in.size(), 1.0f) : o->coeff;
         p->androidNN = android_nn();
         p->isNCHW = false;
-        return finish<HipAdd>(op, precision, in, out, p);
+        return finish(op, compute_library_->createAdd(precision), in, out, p);
     }
 
-    std::shared_ptr<HipRuntime> runtime_;
+    std::shared_ptr<HipComputeLibrary> compute_library_;
+    std::mutex mutex_constructor_;
+    uint64_t operator_list_id_ = 0;
     TFlite::LegacyModel legacy_model_ = TFlite::LegacyModel_TENSORFLOW_NHWC;
-    std::map<int32_t, std::shared_ptr<ITensor>> alloc_tensors_;  // feature maps by buffer index
+    std::map<uint64_t, std::map<int32_t, std::shared_ptr<ITensor>>> alloc_tensors_map_;  // feature maps by list id and buffer index
     std::map<int32_t, int32_t> tensors_used_;                    // readers still to be built, by buffer index
     std::map<int32_t, bool> produced_, consumed_;
 };
 
-// Runs a built list: host bytes into the list's input tensors, every operator in order on the
-// runtime's stream, the list's output tensors back to the host (gpu_op_executor.cc:56-103).
+// Runs a built list: every operator in order on the compute library's stream (gpu_op_executor.cc:56-103).  Moving host
+// bytes into the list's inputs and out of its outputs is the userdriver's part (gpu_userdriver.cc:97-103).
+//
+// Record and replay.  A list is recorded when all of its operators are replayable() (they only enqueue kernels whose
+// arguments follow from their tensors).  What was recorded stays valid while every tensor of every operator keeps
+// its device address, scale and zero point: the executor keeps that signature per list, and an execution whose
+// signature differs runs operator by operator (which also lets the operators re-fold biases or send new per-channel
+// pairs, things that cannot be recorded), records at the next execution with that same signature, and replays after
+// that.  The recorded graph holds kernel launches and device-to-device copies only; buffers are cleared by fill
+// kernels, never by memset nodes.
 class OperationExecutor {
 public:
-    explicit OperationExecutor(std::shared_ptr<HipRuntime> runtime) : runtime_(runtime) {}
+    explicit OperationExecutor(std::shared_ptr<HipComputeLibrary> compute_library) : compute_library_(compute_library) {}
+    ~OperationExecutor() {
+        for (auto &kv : recorded_)
+            if (kv.second.graph) eh_graph_destroy(kv.second.graph);
+    }
+    OperationExecutor(const OperationExecutor &) = delete;
+    OperationExecutor &operator=(const OperationExecutor &) = delete;
 
-    EnnReturn execute(const OperationConstructor &built, const std::vector<const void *> &inputs, const std::vector<void *> &outputs) {
-        if (!built.operators || inputs.size() != built.in_tensors.size() || outputs.size() != built.out_tensors.size()) {
-            ERROR_PRINT("OperationExecutor: %zu inputs and %zu outputs given, the list has %zu and %zu\n", inputs.size(), outputs.size(),
-                        built.in_tensors.size(), built.out_tensors.size());
+    struct Counters {
+        uint64_t direct = 0;     // executions that ran operator by operator
+        uint64_t recordings = 0;
+        uint64_t replays = 0;
+    };
+
+    EnnReturn execute(UDOperators &operators, UDBuffers &buffers, const BufferTable &buffer_table) {
+        (void)buffers;
+        (void)buffer_table;
+        if (!operators) return ENN_RET_FAILED;
+        if (!replay) return run_in_order(operators);
+        Recorded &r = recorded_[operators.get()];
+        std::vector<uint64_t> now;
+        const bool can_record = signature(operators, &now);
+        if (!can_record || now != r.signature || r.state == State::DIRECT_ONLY) {
+            const bool changed = now != r.signature;
+            if (r.graph && changed) {
+                // what was recorded is stale; the operators are about to rewrite the arrays it reads
+                compute_library_->synchronize();
+                eh_graph_destroy(r.graph);
+                r.graph = nullptr;
+            }
+            if (changed) r.state = can_record ? State::WARM : State::DIRECT_ONLY;
+            r.signature = now;
+            return run_in_order(operators);
+        }
+        if (r.state == State::WARM) {  // second execution with this signature: record it
+            void *stream = compute_library_->runtime()->stream();
+            if (stream == nullptr || eh_graph_begin(stream) != EH_OK) {
+                r.state = State::DIRECT_ONLY;
+                return run_in_order(operators);
+            }
+            const EnnReturn ran = run_in_order(operators, false);
+            void *graph = nullptr;
+            const int ended = eh_graph_end(stream, &graph);  // always ends the capture, also after a failed operator
+            if (ran != ENN_RET_SUCCESS || ended != EH_OK || graph == nullptr) {
+                if (graph) eh_graph_destroy(graph);
+                ERROR_PRINT("OperationExecutor: the list could not be recorded (%s); it runs operator by operator\n", eh_last_error());
+                r.state = State::DIRECT_ONLY;
+                return run_in_order(operators);
+            }
+            r.graph = graph;
+            r.state = State::RECORDED;
+            ++counters_.recordings;
+        }
+        if (eh_graph_launch(r.graph, compute_library_->runtime()->stream()) != EH_OK) {
+            ERROR_PRINT("OperationExecutor: replay failed: %s\n", eh_last_error());
             return ENN_RET_FAILED;
         }
-        for (size_t i = 0; i < inputs.size(); ++i)
-            if (built.in_tensors[i]->writeData(const_cast<void *>(inputs[i])) != Status::SUCCESS) return ENN_RET_FAILED;
-        auto buffer = std::make_shared<UDBuffer>();
-        buffer->set_id(++execution_id_);
-        for (auto &op : *built.operators)
-            if (op->execute(buffer) != ENN_RET_SUCCESS) {
-                ERROR_PRINT("OperationExecutor: %s failed\n", op->getName().c_str());
-                return ENN_RET_FAILED;
-            }
-        for (size_t i = 0; i < outputs.size(); ++i)
-            if (built.out_tensors[i]->readData(outputs[i]) != Status::SUCCESS) return ENN_RET_FAILED;
+        ++counters_.replays;
         return ENN_RET_SUCCESS;
     }
 
+    // Forgets what was recorded for a list (the userdriver calls this when the list is closed, before its operators go).
+    void forget(const UDOperators &operators) {
+        auto it = recorded_.find(operators.get());
+        if (it == recorded_.end()) return;
+        if (it->second.graph) {
+            compute_library_->synchronize();
+            eh_graph_destroy(it->second.graph);
+        }
+        recorded_.erase(it);
+    }
+
+    const Counters &counters() const { return counters_; }
+    bool replay = true;  // false: every execution runs operator by operator, as the reference's does
+
 private:
-    std::shared_ptr<HipRuntime> runtime_;
-    uint64_t execution_id_ = 0;
+    enum class State { WARM, RECORDED, DIRECT_ONLY };
+    struct Recorded {
+        std::vector<uint64_t> signature;
+        void *graph = nullptr;
+        State state = State::WARM;
+    };
+
+    EnnReturn run_in_order(UDOperators &operators, bool count = true) {
+        if (count) ++counters_.direct;
+        for (auto &op : *operators)
+            if (op->execute(nullptr) != ENN_RET_SUCCESS) {
+                ERROR_PRINT("OperationExecutor: %s failed\n", op->getName().c_str());
+                return ENN_RET_FAILED;
+            }
+        return ENN_RET_SUCCESS;
+    }
+
+    // device address, scale and zero point of every tensor of every operator; false when an operator cannot be recorded
+    static bool signature(const UDOperators &operators, std::vector<uint64_t> *out) {
+        bool all = true;
+        out->clear();
+        out->reserve(operators->size() * 12);
+        auto add = [&](const std::shared_ptr<ITensor> &t) {
+            if (!t) return;
+            const float scale = t->getScale();
+            uint32_t bits;
+            std::memcpy(&bits, &scale, sizeof bits);
+            out->push_back(reinterpret_cast<uint64_t>(std::static_pointer_cast<HipTensor>(t)->getDataPtr()));
+            out->push_back(((uint64_t)bits << 32) | (uint32_t)t->getZeroPoint());
+        };
+        for (auto &op : *operators) {
+            all = all && op->replayable();
+            for (const auto &t : op->getInTensors()) add(t);
+            for (const auto &t : op->getOutTensors()) add(t);
+            out->push_back(0xED0ull);  // operator boundary
+        }
+        return all;
+    }
+
+    std::shared_ptr<HipComputeLibrary> compute_library_;
+    std::map<const void *, Recorded> recorded_;
+    Counters counters_;
 };
 
 }  // namespace hip

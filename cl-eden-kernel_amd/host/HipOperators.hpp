@@ -295,6 +295,10 @@ public:
         return Status::SUCCESS;
     }
 
+    // execute() only enqueues kernels unless the weights or bias are run-time inputs (they are then re-packed, which
+    // may read device memory back to choose a kernel form)
+    bool launchesOnly() const { return !weights_as_input_ && !bias_as_input_; }
+
     // From now on execute() stores add(residual, convolution) in `sum` and leaves this operator's own output tensor
     // unwritten: the quantized CLAdd that follows this convolution in an operator list, taken into its launch
     // (gpu/operators/CLAdd.cpp:159-163; the sum of the two rescaled operands does not depend on their order).  The
@@ -445,6 +449,7 @@ public:
         return Status::SUCCESS;
     }
 
+    bool launchesOnly() const { return !weights_as_input_; }  // a re-pack reads the weights back to choose the dot-product form
     Status release() {
         if (plan_) {
             (void)runtime_->synchronize();
@@ -542,6 +547,7 @@ public:
         return Status::SUCCESS;
     }
 
+    bool launchesOnly() const { return !weights_as_input_; }
     Status release() {
         if (plan_) {
             (void)runtime_->synchronize();
@@ -652,6 +658,7 @@ public:
         return Status::SUCCESS;
     }
 
+    bool launchesOnly() const { return !weights_as_input_; }
     Status release() {
         if (plan_) {
             (void)runtime_->synchronize();
@@ -733,6 +740,7 @@ public:
         return Status::SUCCESS;
     }
 
+    bool launchesOnly() const { return true; }
     Status release() { return Status::SUCCESS; }
 
 private:
@@ -798,6 +806,7 @@ public:
         return Status::SUCCESS;
     }
 
+    bool launchesOnly() const { return true; }
     Status release() { return Status::SUCCESS; }
 
 private:

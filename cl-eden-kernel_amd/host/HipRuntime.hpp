@@ -105,6 +105,16 @@ public:
         return Status::SUCCESS;
     }
 
+    // Gives up the pooled buffers requested since the last assignment (a list whose construction failed half way):
+    // they take no part in the next assignment and get no memory.
+    Status abandonPendingBuffers() {
+        Status st = Status::SUCCESS;
+        for (auto &kv : pending_)
+            if (pool_ && eh_pool_release(pool_, kv.first) != EH_OK) st = Status::FAILURE;
+        pending_.clear();
+        return st;
+    }
+
     Status resetIntraBuffer() {
         if (pool_) CHECK_EXPR_RETURN_FAILURE(eh_pool_reset_intra(pool_) == EH_OK, "resetIntraBuffer: %s", eh_last_error());
         return Status::SUCCESS;
@@ -166,9 +176,12 @@ public:
         std::lock_guard<std::mutex> lock(mutex_);
         CHECK_EXPR_RETURN_FAILURE(eh_h2d(dst, src, type_bytes * (size_t)num, stream_) == EH_OK, "writeBuffer: %s",
                                   eh_last_error());
-        // hipMemcpyAsync from pageable host memory returns once the source has been staged, so a non-blocking
-        // write may return here, as clEnqueueWriteBuffer(blocking = CL_FALSE) does after its copy of the source
-        return blocking ? synchronizeLocked() : Status::SUCCESS;
+        // The source is ordinary pageable memory that the caller may reuse as soon as this returns (the contract of
+        // clEnqueueWriteBuffer(blocking = CL_FALSE) is that the caller waits for the event; callers of the reference's
+        // writeData(false) do not, gpu_userdriver.cc:188-220).  That hipMemcpyAsync has staged a pageable source by the
+        // time it returns is what the runtime does today, not what the API promises, so both modes wait for the copy.
+        (void)blocking;
+        return synchronizeLocked();
     }
 
     Status readBuffer(void *dst, const void *src, size_t type_bytes, uint32_t num, bool blocking) {

@@ -39,6 +39,18 @@ public:
         buf_ = runtime_->getBuffer(precision_, data_type_, dims_, buffer_type_, storage_type_);
     }
 
+    // the same from a shape of any rank up to four (CLTensor.cpp:29-47): getDims() keeps the rank, getDim() is the
+    // shape padded with ones
+    HipTensor(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision, const DataType &data_type,
+              const NDims &ndim, const DataOrder &data_order = DataOrder::NCHW, const float &scale = 1.0f,
+              const int32_t &zero_point = 0, const BufferType &buffer_type = BufferType::DEDICATED,
+              const StorageType &storage_type = StorageType::BUFFER, const uint32_t buffer_data_type = 0,
+              const int32_t buffer_index = UNDEFINED)
+        : HipTensor(runtime, precision, data_type, extendToDim4(ndim), data_order, scale, zero_point, buffer_type, storage_type,
+                    buffer_data_type, buffer_index) {
+        vdims_ = ndim;
+    }
+
     // constant tensor (weights, bias): uploaded at construction
     template <typename T>
     HipTensor(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision, T *data, const Dim4 &dims,
@@ -54,6 +66,16 @@ public:
         if (getNumOfBytes())
             (void)runtime_->writeBuffer(buf_->getDataPtr(), data, getTypeBytes(data_type_, precision_), getTotalSizeFromDims(),
                                         true);
+    }
+
+    template <typename T>
+    HipTensor(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision, T *data, const NDims &ndim,
+              const DataOrder &data_order = DataOrder::NCHW, const float &scale = 1.0f, const int32_t &zero_point = 0,
+              const BufferType &buffer_type = BufferType::DEDICATED, const StorageType &storage_type = StorageType::BUFFER,
+              const uint32_t buffer_data_type = 0, const int32_t buffer_index = UNDEFINED)
+        : HipTensor(runtime, precision, data, extendToDim4(ndim), data_order, scale, zero_point, buffer_type, storage_type,
+                    buffer_data_type, buffer_index) {
+        vdims_ = ndim;
     }
 
     ~HipTensor() override {
@@ -107,6 +129,9 @@ public:
         return st;
     }
 
+    // Device -> host.  blocking == false only queues the copy: the host bytes are defined after the runtime's
+    // synchronize() (or a later blocking call on the same runtime), as with clEnqueueReadBuffer(CL_FALSE); reads that
+    // change the element order always block.
     Status readData(DataPtr data, bool blocking = true, DataOrderChangeType type = DataOrderChangeType::OTHER,
                     void *event = nullptr) override {
         (void)event;

@@ -34,6 +34,10 @@ public:
     virtual ~UDOperator() {}
     virtual EnnReturn execute(const std::shared_ptr<UDBuffer> &buffer) = 0;
     virtual EnnReturn release() = 0;
+    // Whether execute() does nothing but enqueue kernels whose arguments follow from the operator's tensors (their
+    // device addresses, scales and zero points): such an execution can be recorded once and replayed.  Not part of the
+    // reference's UDOperator; the list executor of this backend asks it.
+    virtual bool replayable() const { return false; }
     std::string getName() { return name_; }
     uint64_t getId() { return id_; }
     std::vector<std::shared_ptr<ITensor>> getInTensors() { return in_; }
@@ -59,6 +63,7 @@ public:
         return op_->execute() == Status::SUCCESS ? ENN_RET_SUCCESS : ENN_RET_FAILED;
     }
     EnnReturn release() override { return op_->release() == Status::SUCCESS ? ENN_RET_SUCCESS : ENN_RET_FAILED; }
+    bool replayable() const override { return op_->launchesOnly(); }
     std::shared_ptr<T> getOp() { return op_; }
 
 private:
@@ -66,6 +71,7 @@ private:
 };
 
 using UDOperators = std::shared_ptr<std::vector<std::shared_ptr<UDOperator>>>;
+using UDBuffers = std::vector<std::shared_ptr<UDBuffer>>;
 using UDTensors = std::vector<std::shared_ptr<ITensor>>;
 
 }  // namespace ud

@@ -189,6 +189,60 @@ def compulsory_bytes_per_image(image=224):
     return total
 
 
+def operator_list(ud, list_id, batch, image=224, per_channel=False, weights="minmax"):
+    """The same network as a description for the userdriver (`ud` = the userdriver module): an androidNN model with
+    channels-last data (use_nchw false), i.e. feature maps [batch, h, w, c], convolution filters [out, kh, kw, in] and
+    depthwise filters [1, kh, kw, c] as TFLite stores them, and the explicit padding values of layers() (its
+    symmetric padding is not what SAME gives a stride-2 layer).  Returns (OperatorList, input buffer index, output
+    buffer index, logits shape).  Buffer index i is tensor i of layers()."""
+    tensors, ops = layers(image, weights)
+    ol = ud.OperatorList(list_id, ud.MODEL_ANDROID_NN)
+    fm = {}
+
+    def feature_map(i):
+        if i not in fm:
+            t = tensors[i]
+            shape = (batch, t["h"], t["w"], t["c"])
+            fm[i] = ol.feature_map(i, shape, t["scale"], t["zp"])
+        return fm[i]
+
+    for n, op in enumerate(ops):
+        kind = op["op"]
+        if kind == "add":
+            ol.operator("ADD_%d" % n, ud.OP_ADD, [feature_map(op["a"]), feature_map(op["b"])], [feature_map(op["dst"])])
+            continue
+        s = tensors[op["src"]]
+        if kind == "avgpool":
+            ol.operator("AVERAGE_POOL_2D_%d" % n, ud.OP_AVERAGE_POOL_2D, [feature_map(op["src"])], [feature_map(op["dst"])],
+                        ud.options(padding=ud.PADDING_VALID, stride=(1, 1), filter=(op["k"], op["k"])))
+            continue
+        act = ud.ACT_RELU6 if op.get("relu6") else ud.ACT_NONE
+        bias_scale = float(np.float32(s["scale"]) * np.float32(op["w_scale"]))
+        if kind == "fc":
+            w, b = op_weights(op, s["c"])
+            wt = ol.parameter(w, op["w_scale"], op["w_zp"])
+            bt = ol.parameter(b, bias_scale, 0)
+            ol.operator("FULLY_CONNECTED_%d" % n, ud.OP_FULLY_CONNECTED, [feature_map(op["src"]), wt, bt], [feature_map(op["dst"])],
+                        ud.options(activation=act))
+            continue
+        if per_channel:
+            w, b, w_scales = op_weights_perchannel(op, s["c"])
+        else:
+            (w, b), w_scales = op_weights(op, s["c"]), None
+        if kind == "dw":
+            w = np.ascontiguousarray(w.transpose(1, 2, 3, 0))   # [C, 1, kh, kw] -> [1, kh, kw, C]
+        else:
+            w = np.ascontiguousarray(w.transpose(0, 2, 3, 1))   # [O, I, kh, kw] -> [O, kh, kw, I]
+        wt = ol.parameter(w, 0.0 if per_channel else op["w_scale"], 0 if per_channel else op["w_zp"], per_channel_scales=w_scales)
+        bt = ol.parameter(b, 1.0 if per_channel else bias_scale, 0)
+        pad = op["pad"]
+        opts = ud.options(padding=ud.PADDING_VALID, stride=(op["stride"],) * 2, activation=act, padding_value=(pad,) * 4)
+        code, name = (ud.OP_DEPTHWISE_CONV_2D, "DEPTHWISE_CONV_2D_%d") if kind == "dw" else (ud.OP_CONV_2D, "CONV_2D_%d")
+        ol.operator(name % n, code, [feature_map(op["src"]), wt, bt], [feature_map(op["dst"])], opts)
+    last = len(tensors) - 1
+    return ol, 0, last, (batch, tensors[last]["c"])
+
+
 class MobileNetV2:
     """The operator list instantiated on the GPU for one batch size.  Activations are channels-last.
 

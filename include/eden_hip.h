@@ -303,7 +303,10 @@ int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const 
  * eh_conv2d_u8_run does).  Fails with EH_INVALID_PARAMS, launching nothing, when the staging
  * (n*c*h*w + n*cout*ho*wo bytes, each rounded up to 256 plus 256) exceeds the array or the plan has more than
  * 8 groups.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
- * threads) race; calls ordered on one stream do not.  Results are bit for bit those of eh_conv2d_u8_run. */
+ * threads) race; calls ordered on one stream do not.  Results are bit for bit those of eh_conv2d_u8_run.  The first
+ * launch of a one-tap kernel variant at a given LDS size asks the driver once how many of its workgroups a CU holds
+ * (an occupancy query: no allocation, no stream operation, legal under capture); every later launch reads the cached
+ * answer. */
 #define EH_STATIC_SCRATCH_BYTES (32u << 20)
 int eh_conv2d_u8_run_static(eh_conv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
 /* Convolution followed by the quantized residual add, output = add(residual, convolution) with `aq` as eh_add_u8

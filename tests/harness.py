@@ -97,6 +97,19 @@ def gpu_fc(a, w, bias, q):
     return out
 
 
+def scattered_batch(batch, distinct=8, seed=2025):
+    """Which of `distinct` oracle-evaluated images sits at each of `batch` positions: seeded and without a period, so
+    that a kernel reading image i +- 1, 2, 4, 8 ... instead of image i cannot pass; the first two, the middle two and
+    the last two positions hold six different images and every image is used."""
+    rng = np.random.default_rng(seed)
+    while True:
+        idx = rng.integers(0, distinct, batch)
+        ends = [0, 1, batch // 2 - 1, batch // 2, batch - 2, batch - 1]
+        shifted_equal = any(np.array_equal(idx[k:], idx[:-k]) for k in (1, 2, 4, 8, 16, 32) if k < batch)
+        if len(set(idx[ends].tolist())) == min(6, distinct) and len(set(idx.tolist())) == distinct and not shifted_equal:
+            return idx
+
+
 def diff_report(got, want):
     bad = np.argwhere(got != want)
     return "%d of %d differ; first at %s: got %s want %s" % (
@@ -124,10 +137,9 @@ def oracle_forward(x_nhwc, image, per_channel=False, weights="minmax"):
         act = O.ACT_RELU6 if op.get("relu6") else O.ACT_NONE
         if per_channel and kind != "fc":
             w, b, w_scales = mobilenet.op_weights_perchannel(op, s["c"])
-            eq, mults, shifts = eden.make_requant_perchannel(s["scale"], s["zp"], w_scales, d["scale"], d["zp"], act, bool(op.get("relu6")))
-            q = O.raw_quant(zp_in=eq.zp_in, zp_w=0, zp_out=eq.zp_out, act_min=eq.act_min, act_max=eq.act_max)
+            mults, shifts = O.perchannel_pairs(s["scale"], w_scales, d["scale"])
             lo, hi = O.act_range_u8(act if op.get("relu6") else O.ACT_NONE, d["scale"], d["zp"])
-            assert (eq.zp_in, eq.zp_out, eq.act_min, eq.act_max) == (s["zp"], d["zp"], lo, hi)
+            q = O.raw_quant(zp_in=s["zp"], zp_w=0, zp_out=d["zp"], act_min=lo, act_max=hi)
             groups = s["c"] if kind == "dw" else 1
             shape = O.conv_shape(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4,
                                  groups=groups)

@@ -188,6 +188,14 @@ def make_quant(s_in, zp_in, s_w, zp_w, s_out, zp_out, act=ACT_NONE, act_enabled=
     return q
 
 
+def perchannel_pairs(s_in, filter_scales, s_out):
+    """One (multiplier, shift) per output channel as the per-channel operators derive them at execute()
+    (cl_optimized_impls/CLConvolutionPerChannelQuantized.cpp:88-97): the per-tensor derivation with the channel's
+    filter scale and the bias scale s_in * scale."""
+    pairs = [make_quant(s_in, 0, float(s), 0, s_out, 0) for s in np.asarray(filter_scales, np.float32)]
+    return np.array([q.multiplier for q in pairs], np.int32), np.array([q.shift for q in pairs], np.int32)
+
+
 def raw_quant(zp_in=0, zp_w=0, zp_out=0, multiplier=1 << 30, shift=1, act_min=0, act_max=255):
     """Explicit integer parameters; the default multiplier/shift is M == 1."""
     return Quant(zp_in, zp_w, zp_out, multiplier, shift, act_min, act_max)

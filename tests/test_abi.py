@@ -31,6 +31,36 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(eden.EXPORTS), set(names) ^ set(eden.EXPORTS)
 
 
+def test_userdriver_library_exports_every_declared_symbol_and_describes_a_list_without_a_gpu():
+    """libedenud.so (include/eden_ud.h): every declared entry point is exported and bound; describing an operator list
+    is host work, and its argument checks answer with an error text instead of crashing.  Nothing here computes."""
+    import importlib
+    ud = importlib.import_module("cl-eden-kernel_amd.userdriver")
+    lib = ud.load()
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "eden_ud.h")).read(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(eud_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) >= 20
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(names) == set(ud.EXPORTS), set(names) ^ set(ud.EXPORTS)
+    ol = ud.OperatorList(5, ud.MODEL_ANDROID_NN)
+    x = ol.feature_map(0, (1, 8, 8, 4), 0.1, 3)
+    y = ol.feature_map(1, (1, 8, 8, 6), 0.2, 5)
+    w = ol.parameter(np.zeros((6, 1, 1, 4), np.uint8), 0.01, 128)
+    b = ol.parameter(np.zeros(6, np.int32), 0.001, 0)
+    assert (x, y, w, b) == (0, 1, 2, 3)
+    ol.operator("CONV_2D", ud.OP_CONV_2D, [x, w, b], [y], ud.options())
+    with pytest.raises(ud.EdenUdError, match="unknown tensor"):
+        ol.operator("CONV_2D", ud.OP_CONV_2D, [x, 17, b], [y], ud.options())
+    with pytest.raises(ud.EdenUdError, match="not offered"):
+        ol.operator("SOFTMAX", 25, [x], [y], ud.options())
+    with pytest.raises(ud.EdenUdError):
+        ol.feature_map(2, (1, 2, 3, 4, 5), 0.1, 0)   # five extents
+    mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+    net, i, o, shape = mobilenet.operator_list(ud, 9, 2, 96)   # 64 operator descriptions, weights copied
+    assert (i, o, shape) == (0, 64, (2, 1000))
+
+
 def test_product_host_arithmetic_matches_golden_vectors():
     lib = eden.load()
     for mhex, q, s in GOLD["quantize_multiplier"]:
@@ -189,6 +219,37 @@ def test_buffer_pool_protocol_without_a_gpu():
     assert a.ptr.value is None                            # no memory before the assignment
     with pytest.raises(eden.EdenHipError):
         pool.reset_inter(s1)                              # not a feature map
+
+
+def test_buffer_pool_release_before_assignment_without_a_gpu():
+    """A pooled buffer released before its list is assigned (a tensor destroyed while the list is still being built)
+    takes no part in the layout, is not handed to later REUSE / INTRA requests, cannot be reset, and an assignment
+    whose every slot was released allocates nothing (so nothing here reaches the device)."""
+    lib = eden.load()
+    pool = eden.BufferPool()
+    a = pool.request(eden.POOL_INTER_NEW, 3000)
+    b = pool.request(eden.POOL_INTER_NEW, 500)
+    s = pool.request(eden.POOL_INTRA, 700)
+    pad = lambda n: (1024 + n + 32 + 1023) // 1024 * 1024
+    assert pool.layout() == (pad(3000) + pad(500) + pad(700), 3)
+    pool.reset_inter(a)
+    eden.check(lib.eh_pool_release(pool.h, a.slot))       # handed back AND released: must not be taken over
+    assert pool.layout() == (pad(500) + pad(700), 2)
+    c = pool.request(eden.POOL_INTER_REUSE, 100)
+    assert c.slot not in (a.slot, b.slot)
+    with pytest.raises(eden.EdenHipError):
+        pool.reset_inter(a)
+    with pytest.raises(eden.EdenHipError):
+        eden.check(lib.eh_pool_release(pool.h, a.slot))   # twice
+    pool.reset_intra()
+    eden.check(lib.eh_pool_release(pool.h, s.slot))
+    s2 = pool.request(eden.POOL_INTRA, 50)                # the released scratch slot is not reused either
+    assert s2.slot != s.slot
+    for buf in (b, c, s2):
+        eden.check(lib.eh_pool_release(pool.h, buf.slot))
+    assert pool.layout() == (0, 0)
+    assert pool.assign() == 0                             # nothing live: no device allocation is made
+    assert a.ptr.value is None and b.ptr.value is None
 
 
 def test_mobilenet_pool_is_a_fraction_of_one_buffer_per_tensor():

@@ -1,6 +1,6 @@
 """MobileNetV2-1.0 uint8 (BASELINE configs[4]): every operator of the GPU operator list against the oracle
 evaluating the same list, bit-exact tensor by tensor, at small batches directly and at the full batch of 64 on an
-input made of an oracle-evaluated pair of images repeated 32 times."""
+input made of eight distinct oracle-evaluated images scattered over the batch positions without a period."""
 import functools
 import importlib
 
@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from harness import eden, oracle_forward, to_eh_requant
+from harness import eden, oracle_forward, scattered_batch, to_eh_requant
 
 mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
 
@@ -52,21 +52,26 @@ def test_mobilenet_v2_matches_oracle_tensor_by_tensor(batch, image, fuse_add, we
     assert_network_alive(ops, want, batch)
 
 
+DISTINCT = 8
+
+
 @functools.lru_cache(maxsize=None)
-def oracle_pair(per_channel, weights):
-    return oracle_forward(mobilenet.network_input(2), 224, per_channel, weights)
+def oracle_images(per_channel, weights):
+    """the oracle's tensors for DISTINCT different images"""
+    return oracle_forward(mobilenet.network_input(DISTINCT), 224, per_channel, weights)
 
 
 @pytest.mark.parametrize("per_channel,weights", [(False, "minmax"), (False, "narrow"), (True, "minmax")],
                          ids=["per_tensor_minmax", "per_tensor_narrow", "per_channel_minmax"])
 def test_mobilenet_v2_full_batch_64(per_channel, weights):
     """The network exactly as the benchmark builds it (batch 64, which decides tile shapes, grids and the depthwise
-    tile width) on 32 repetitions of a pair of images: every tensor of every image must equal the oracle's tensor
-    for that image of the pair."""
+    tile width) on eight distinct images scattered over the 64 batch positions: every tensor of every batch position
+    must equal the oracle's tensor for the image that sits there."""
     print("mobilenet batch 64", per_channel, weights, flush=True)
     batch = 64
-    tensors, ops, want = oracle_pair(per_channel, weights)
-    x = np.tile(mobilenet.network_input(2), (batch // 2, 1, 1, 1))
+    tensors, ops, want = oracle_images(per_channel, weights)
+    where = scattered_batch(batch, DISTINCT)
+    x = mobilenet.network_input(DISTINCT)[where]
     net = mobilenet.MobileNetV2(eden, batch, 224, fuse_add=True, per_channel=per_channel, weights=weights)
     net.set_input(x)
     stream = eden.Stream()
@@ -78,31 +83,32 @@ def test_mobilenet_v2_full_batch_64(per_channel, weights):
         if i in net.unwritten:
             continue
         got = net.tensor(i).transpose(0, 3, 1, 2)
-        pair = want[i]
-        for img in range(batch):
-            assert np.array_equal(got[img], pair[img % 2]), (op["op"], i, img, tensors[i], int((got[img] != pair[img % 2]).sum()))
-    assert_network_alive(ops, want, 2)
+        expect = want[i][where]
+        if not np.array_equal(got, expect):
+            img = int(np.argwhere((got != expect).reshape(batch, -1).any(axis=1))[0, 0])
+            raise AssertionError((op["op"], i, img, int(where[img]), tensors[i], int((got[img] != expect[img]).sum())))
+    assert_network_alive(ops, want, DISTINCT)
 
 
 @pytest.mark.parametrize("per_channel", [False, True], ids=["per_tensor", "per_channel"])
 def test_mobilenet_v2_on_pooled_buffers_batch_64(per_channel):
     """The network as the benchmark runs it: feature maps in the library's buffer pool (liveness reuse, one device
-    allocation), batch 64, one graph replay; the logits of every image must equal the oracle's for its image of the
-    repeated pair, on two replays."""
+    allocation), batch 64, one graph replay; the logits at every batch position must equal the oracle's for the
+    image that sits there (eight distinct images, scattered), on two replays."""
     batch = 64
-    tensors, ops, want = oracle_pair(per_channel, "minmax")
+    tensors, ops, want = oracle_images(per_channel, "minmax")
+    where = scattered_batch(batch, DISTINCT)
     net = mobilenet.MobileNetV2(eden, batch, 224, fuse_add=True, per_channel=per_channel, pooled=True)
     assert net.pool_bytes < 0.45 * sum(batch * t["h"] * t["w"] * t["c"] for t in tensors)
-    net.set_input(np.tile(mobilenet.network_input(2), (batch // 2, 1, 1, 1)))
+    net.set_input(mobilenet.network_input(DISTINCT)[where])
     stream = eden.Stream()
     graph = eden.Graph(stream, lambda s: net.run(s))
-    ref = want[-1].reshape(2, -1)
+    ref = want[-1].reshape(DISTINCT, -1)[where]
     for rep in range(2):
         graph.launch(stream)
         stream.sync()
         got = net.logits()
-        for img in range(batch):
-            assert np.array_equal(got[img], ref[img % 2]), (rep, img)
+        assert np.array_equal(got, ref), (rep, np.argwhere((got != ref).any(axis=1)).ravel().tolist())
 
 
 def test_mobilenet_v2_graph_replay_equals_eager():

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from harness import (diff_report, eden, gpu_conv, gpu_deconv, gpu_dwconv, gpu_fc, synth, to_eh_requant)
+from harness import (diff_report, eden, gpu_conv, gpu_deconv, gpu_dwconv, gpu_fc, scattered_batch, synth, to_eh_requant)
 
 pytestmark = pytest.mark.gpu
 
@@ -387,18 +387,21 @@ def test_plan_refolds_when_zero_points_change_and_repacks_new_weights():
     plan.destroy()
 
 
-def test_conv3x3_batch_64_equals_oracle_pair():
+def test_conv3x3_batch_64_equals_oracle_on_scattered_distinct_images():
     """The benchmark's 3x3 convolution at its batch of 64 (the batch decides the tile height of the patch kernel), on
-    32 repetitions of a pair of images: every image must equal the oracle's result for that image of the pair."""
-    s2 = O.conv_shape(2, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1))
-    x, w, b = conv_tensors(s2, SEED + 16)
+    eight distinct images scattered over the batch positions without a period: every position must equal the
+    oracle's result for the image that sits there."""
+    s8 = O.conv_shape(8, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s8, SEED + 16)
     q = quant(0.02, 128, 0.005, 120, 0.05, 0, O.ACT_RELU, True)
-    want = O.conv2d(x, w, b, s2, q)
+    want = O.conv2d(x, w, b, s8, q)
+    where = scattered_batch(64, 8)
     s64 = O.conv_shape(64, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1))
-    got = gpu_conv(np.tile(x, (32, 1, 1, 1)), w, b, s64, to_eh_requant(q), layout=eden.NHWC)
+    got = gpu_conv(x[where], w, b, s64, to_eh_requant(q), layout=eden.NHWC)
     for img in range(64):
-        assert np.array_equal(got[img], want[img % 2]), (img, diff_report(got[img], want[img % 2]))
+        assert np.array_equal(got[img], want[where[img]]), (img, int(where[img]), diff_report(got[img], want[where[img]]))
     assert want.std() > 10
+    assert not np.array_equal(want[0], want[1])
 
 
 # ----------------------------------------------------------------- depthwise

@@ -23,6 +23,7 @@ def test_random_operator_instances_match_the_oracle(seed):
         zp_out = int(np.clip(128 - round(float(acc.mean()) * 40.0 / sd), 0, 255))
         return O.raw_quant(zp_in=zp_in, zp_w=zp_w, zp_out=zp_out, multiplier=qm, shift=sh, act_min=lo, act_max=hi)
     ran = {}
+    bad = 0
     for it in range(N):
         kind = rng.choice(["conv", "conv1x1", "conv3x3", "dw", "fc", "deconv"], p=[0.25, 0.2, 0.15, 0.2, 0.1, 0.1])
         zp_in, zp_w = int(rng.integers(0, 256)), int(rng.choice([128, int(rng.integers(0, 256))]))
@@ -78,4 +79,5 @@ def test_random_operator_instances_match_the_oracle(seed):
         if not np.array_equal(got, want):
             bad += 1
             print("MISMATCH", it, desc, q.as_tuple(), diff_report(got, want), flush=True)
+    assert bad == 0, "%d of %d random instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
     assert sum(ran.values()) > 300 and all(ran.get(k, 0) > 10 for k in ("conv", "conv1x1", "conv3x3", "dw", "fc", "deconv")), ran

@@ -1,0 +1,163 @@
+"""The operator list through the userdriver level (include/eden_ud.h -> HipUserDriver -> OperationConstructor /
+OperationExecutor -> HipComputeLibrary -> operator classes -> kernels): MobileNetV2 described as an operator list,
+opened, executed on host buffers and compared with the CPU oracle, bit for bit; the executor's record-and-replay is
+checked through its counters and by changing a tensor's quantization parameters between executions."""
+import functools
+import importlib
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from harness import eden, oracle_forward, scattered_batch
+
+mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
+ud = importlib.import_module("cl-eden-kernel_amd.userdriver")
+
+pytestmark = pytest.mark.gpu
+
+
+@functools.lru_cache(maxsize=None)
+def driver():
+    eden.init(0)
+    return ud.UserDriver(0)
+
+
+@functools.lru_cache(maxsize=None)
+def oracle_images(count, image, per_channel):
+    return oracle_forward(mobilenet.network_input(count, image), image, per_channel, "minmax")
+
+
+@pytest.mark.parametrize("batch,image,per_channel,fuse", [(2, 224, False, True), (3, 96, False, False), (2, 96, True, True)],
+                         ids=["b2_224_fused_adds", "b3_96_one_operator_per_description", "b2_96_per_channel"])
+def test_mobilenet_v2_through_open_execute_close(batch, image, per_channel, fuse):
+    print("userdriver mobilenet", batch, image, per_channel, fuse, flush=True)
+    d = driver()
+    list_id = 0x1000 + batch * 16 + image + (1 if per_channel else 0)
+    ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image, per_channel=per_channel)
+    d.open_subgraph(ol, fuse_residual_adds=fuse)
+    before = d.stats(list_id)
+    assert before["operators"] == (54 if fuse else 64)   # ten residual adds ride in their convolutions' launches
+    x = mobilenet.network_input(batch, image)
+    _, _, want = oracle_images(batch, image, per_channel)
+    ref = want[-1].reshape(batch, -1)
+    for rep in range(4):
+        got = np.zeros(shape, np.uint8)
+        d.execute_subgraph(list_id, {in_index: x, out_index: got})
+        assert np.array_equal(got, ref), (rep, int((got != ref).sum()))
+    after = d.stats(list_id)
+    # first execution operator by operator, second recorded, and replayed from then on
+    assert (after["direct"] - before["direct"], after["recordings"] - before["recordings"], after["replays"] - before["replays"]) == (1, 1, 3)
+    assert len(np.unique(ref)) > 40
+    d.close_subgraph(list_id)
+    with pytest.raises(ud.EdenUdError):
+        d.execute_subgraph(list_id, {in_index: x})   # closed
+
+
+def test_mobilenet_v2_batch_64_through_the_userdriver_on_scattered_images():
+    """BASELINE configs[4] as the benchmark runs it through the operator API: batch 64, eight distinct
+    oracle-evaluated images scattered over the batch positions, logits of every position equal to the oracle's."""
+    d = driver()
+    batch, list_id = 64, 0x6400
+    tensors, ops, want = oracle_forward(mobilenet.network_input(8), 224, False, "minmax")
+    where = scattered_batch(batch, 8)
+    ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch)
+    d.open_subgraph(ol)
+    s = d.stats(list_id)
+    assert 0 < s["pool_bytes"] < 0.45 * sum(batch * t["h"] * t["w"] * t["c"] for t in tensors)   # liveness reuse, one allocation
+    x = np.ascontiguousarray(mobilenet.network_input(8)[where])
+    ref = want[-1].reshape(8, -1)[where]
+    for rep in range(3):
+        got = np.zeros(shape, np.uint8)
+        d.execute_subgraph(list_id, {in_index: x, out_index: got})
+        assert np.array_equal(got, ref), (rep, np.argwhere((got != ref).any(axis=1)).ravel().tolist())
+    # the resident-tensor path the benchmark times: operators only, several executions queued, then one read
+    d.write_input(list_id, 0, x)
+    d.execute_operators(list_id, 5)
+    d.synchronize()
+    assert np.array_equal(d.read_output(list_id, 0, shape), ref)
+    d.close_subgraph(list_id)
+
+
+def test_quantization_parameters_changed_between_executions_are_honoured():
+    """The operators read scale and zero point from their tensors at every execution (the reference derives its
+    multiplier in execute()).  Changing the output tensor's parameters after the list has been recorded must not replay
+    the stale recording: the next execution runs operator by operator, the one after records again, and every result
+    equals the oracle's for the parameters in force."""
+    d = driver()
+    list_id = 0x77
+    rng = np.random.default_rng(3)
+    n, h, w, cin, cout = 2, 12, 10, 16, 24
+    x = rng.integers(0, 256, (n, h, w, cin)).astype(np.uint8)
+    wt = rng.integers(0, 256, (cout, 3, 3, cin)).astype(np.uint8)
+    b = rng.integers(-500, 500, cout).astype(np.int32)
+    s_in, s_w = 0.02, 0.005
+    ol = ud.OperatorList(list_id, ud.MODEL_ANDROID_NN)
+    fx = ol.feature_map(0, (n, h, w, cin), s_in, 128)
+    fy = ol.feature_map(1, (n, h, w, cout), 0.2, 100)
+    ol.operator("CONV_2D", ud.OP_CONV_2D, [fx, ol.parameter(wt, s_w, 121), ol.parameter(b, float(np.float32(s_in) * np.float32(s_w)), 0)], [fy],
+                ud.options(padding=ud.PADDING_SAME, activation=ud.ACT_RELU))
+    d.open_subgraph(ol)
+    shape_o = O.conv_shape(n, cin, h, w, cout, 3, 3, pad=(1, 1, 1, 1))
+
+    def expect(s_out, zp_out, zp_in):
+        q = O.make_quant(s_in, zp_in, s_w, 121, s_out, zp_out, O.ACT_RELU, True)
+        return O.conv2d(x.transpose(0, 3, 1, 2), wt.transpose(0, 3, 1, 2), b, shape_o, q).transpose(0, 2, 3, 1)
+
+    base = d.stats(list_id)
+    for s_out, zp_out, zp_in, runs in ((0.2, 100, 128, 3), (0.35, 17, 128, 3), (0.35, 17, 99, 2), (0.2, 100, 128, 2)):
+        d.set_quant(list_id, True, 0, s_out, zp_out)
+        d.set_quant(list_id, False, 0, s_in, zp_in)
+        want = expect(s_out, zp_out, zp_in)
+        for rep in range(runs):
+            got = np.zeros((n, h, w, cout), np.uint8)
+            d.execute_subgraph(list_id, {0: x, 1: got})
+            assert np.array_equal(got, want), (s_out, zp_out, zp_in, rep, int((got != want).sum()))
+        assert want.std() > 5
+    s = d.stats(list_id)
+    # per parameter set: one direct execution, one recording, the rest replays
+    assert (s["direct"] - base["direct"], s["recordings"] - base["recordings"], s["replays"] - base["replays"]) == (4, 4, 6)
+    d.set_replay(False)   # the reference's behaviour: every execution operator by operator
+    got = np.zeros((n, h, w, cout), np.uint8)
+    d.execute_subgraph(list_id, {0: x, 1: got})
+    assert np.array_equal(got, expect(0.2, 100, 128))
+    assert d.stats(list_id)["direct"] == s["direct"] + 1
+    d.set_replay(True)
+    d.close_subgraph(list_id)
+
+
+def test_two_lists_open_at_once_and_error_paths():
+    d = driver()
+    rng = np.random.default_rng(5)
+    lists = {}
+    for list_id, (m, k, nn) in ((0x201, (5, 64, 40)), (0x202, (9, 128, 16))):
+        a = rng.integers(0, 256, (m, k)).astype(np.uint8)
+        wt = rng.integers(0, 256, (nn, k)).astype(np.uint8)
+        b = rng.integers(-500, 500, nn).astype(np.int32)
+        ol = ud.OperatorList(list_id, ud.MODEL_TENSORFLOW)
+        fx, fy = ol.feature_map(0, (m, k), 0.01, 3), ol.feature_map(1, (m, nn), 0.08, 7)
+        ol.operator("FULLY_CONNECTED", ud.OP_FULLY_CONNECTED, [fx, ol.parameter(wt, 0.002, 128), ol.parameter(b, float(np.float32(0.01) * np.float32(0.002)), 0)], [fy])
+        d.open_subgraph(ol)
+        lists[list_id] = (a, O.fc(a, wt, b, O.make_quant(0.01, 3, 0.002, 128, 0.08, 7)), ol)
+    with pytest.raises(ud.EdenUdError):
+        d.open_subgraph(lists[0x201][2])   # open already
+    for _ in range(3):   # interleaved executions of both lists, each with its own recording
+        for list_id, (a, want, _) in lists.items():
+            got = np.zeros(want.shape, np.uint8)
+            d.execute_subgraph(list_id, {0: a, 1: got})
+            assert np.array_equal(got, want)
+    small = np.zeros(3, np.uint8)
+    with pytest.raises(ud.EdenUdError):
+        d.execute_subgraph(0x201, {0: small})   # input buffer smaller than the tensor
+    for list_id in lists:
+        d.close_subgraph(list_id)
+    with pytest.raises(ud.EdenUdError):
+        d.close_subgraph(0x201)
+    # a list whose operator cannot be built is refused and leaves nothing open
+    bad = ud.OperatorList(0x203, ud.MODEL_TENSORFLOW)
+    fx, fy = bad.feature_map(0, (1, 8, 6, 6), 0.1, 0), bad.feature_map(1, (1, 8, 9, 9), 0.1, 0)   # output extent does not follow from the geometry
+    bad.operator("CONV_2D", ud.OP_CONV_2D, [fx, bad.parameter(np.zeros((8, 8, 3, 3), np.uint8), 0.1, 0), bad.parameter(np.zeros(8, np.int32), 0.01, 0)], [fy])
+    with pytest.raises(ud.EdenUdError):
+        d.open_subgraph(bad)
+    with pytest.raises(ud.EdenUdError):
+        d.stats(0x203)

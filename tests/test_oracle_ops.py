@@ -371,13 +371,59 @@ def test_add_unequal_scales_against_exact_rational_arithmetic(params):
 
 
 def test_avgpool_closed_forms():
-    """parity unpinned by reference vectors: (sum + n/2) / n over the clipped window."""
+    """hand cases of (sum + n/2) / n over the clipped window (AveragepoolKernels.cpp:8-44)"""
     x = np.arange(16, dtype=np.uint8).reshape(1, 1, 4, 4)
     assert O.avgpool(x, 2, 2, stride=(2, 2)).reshape(-1).tolist() == [3, 5, 11, 13]  # 2.5->3, 4.5->5, ...
     assert O.avgpool(x, 4, 4).reshape(-1).tolist() == [8]  # 7.5 -> 8
     # padded window counts only in-image taps
     o = O.avgpool(x, 3, 3, stride=(1, 1), pad=(1, 1, 1, 1))
     assert o[0, 0, 0, 0] == (0 + 1 + 4 + 5 + 2) // 4
+
+
+@pytest.mark.parametrize("k,stride,pad", [((3, 3), (2, 2), (1, 1, 1, 1)), ((2, 2), (2, 2), (0, 0, 0, 0)), ((3, 2), (1, 2), (0, 2, 1, 0)),
+                                          ((7, 7), (1, 1), (0, 0, 0, 0)), ((4, 4), (3, 3), (2, 1, 1, 2))])
+def test_avgpool_uint8_against_exact_rational_arithmetic(k, stride, pad):
+    """No reference vector exists (the reference's averagepool_test.cpp is float only), so the uint8 pool is pinned by
+    what (sum + n / 2) / n has to be: the mean over the in-image taps of the window, rounded to nearest with ties
+    upwards, then clamped.  Checked on every output of seeded tensors in exact rational arithmetic; a version that
+    divides by the full window size on border windows, one that truncates, and one that rounds ties to even each
+    fail the same check."""
+    from fractions import Fraction
+    import math
+    rng = np.random.default_rng(31 + k[0] * 7 + k[1])
+    n, c, h, w = 2, 3, 11, 9
+    x = rng.integers(0, 256, (n, c, h, w)).astype(np.uint8)
+    x[0, 0, :4, :4] = 255   # saturated corner: the clamp's upper bound is reached
+    x[1, 2, :2, :2] = np.array([[1, 2], [3, 4]], np.uint8)  # a 2x2 window summing to 10: mean 2.5, a tie
+    lo, hi = 7, 240
+    got = O.avgpool(x, k[0], k[1], stride=stride, pad=pad, act_min=lo, act_max=hi).astype(np.int64)
+    ho = (h + pad[0] + pad[1] - k[0]) // stride[0] + 1
+    wo = (w + pad[2] + pad[3] - k[1]) // stride[1] + 1
+    assert got.shape == (n, c, ho, wo)
+    ties = 0
+    mutants = dict(full_window=0, truncating=0, ties_to_even=0)
+    for i in range(n):
+        for ch in range(c):
+            for oy in range(ho):
+                for ox in range(wo):
+                    ys = [v for v in range(oy * stride[0] - pad[0], oy * stride[0] - pad[0] + k[0]) if 0 <= v < h]
+                    xs = [v for v in range(ox * stride[1] - pad[2], ox * stride[1] - pad[2] + k[1]) if 0 <= v < w]
+                    total = int(sum(int(x[i, ch, a, b]) for a in ys for b in xs))
+                    mean = Fraction(total, len(ys) * len(xs))
+                    nearest = math.floor(mean + Fraction(1, 2))   # ties upwards
+                    ties += mean.denominator == 2
+                    assert got[i, ch, oy, ox] == min(max(nearest, lo), hi), (i, ch, oy, ox, mean)
+                    full = math.floor(Fraction(total, k[0] * k[1]) + Fraction(1, 2))
+                    mutants["full_window"] += min(max(full, lo), hi) != got[i, ch, oy, ox]
+                    mutants["truncating"] += min(max(math.floor(mean), lo), hi) != got[i, ch, oy, ox]
+                    mutants["ties_to_even"] += min(max(round(mean), lo), hi) != got[i, ch, oy, ox]
+    if k[0] * k[1] <= 9:   # large windows average the clamp's bounds away
+        assert got.min() == lo or got.max() == hi
+    if any(pad):
+        assert mutants["full_window"] > 0
+    assert mutants["truncating"] > 0
+    if k == (2, 2):
+        assert ties > 0 and mutants["ties_to_even"] > 0
 
 
 def test_avgpool_int8_rounds_half_away_from_zero():

@@ -1,4 +1,4 @@
-"""Runs the C++ operator-level tests (cl-eden-kernel_amd/host/ud_op_test.cpp): the Hip*
+"""Runs the C++ operator-level tests (tests/ud_op_test.cpp): the Hip*
 operator classes, tensors and buffer manager that mirror the reference's operator API,
 checked bit for bit against the CPU oracle inside the test program."""
 import os
@@ -7,13 +7,14 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-BIN = os.path.join(ROOT, "cl-eden-kernel_amd", "ud_op_test")
+BIN = os.path.join(ROOT, "tests", "ud_op_test")
 
 
 def _binary():
     if not os.path.exists(BIN):
         import importlib
         importlib.import_module("cl-eden-kernel_amd.build").build_all()
+        importlib.import_module("build_native").build_ud_test()
     return BIN
 
 

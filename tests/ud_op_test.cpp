@@ -16,6 +16,7 @@
 
 #include "HipOpConstructor.hpp"
 #include "HipOperators.hpp"
+#include "HipUserDriver.hpp"
 #include "eden_oracle.h"
 #include "userdriver_operator.hpp"
 
@@ -154,12 +155,28 @@ static bool conv_case(const std::shared_ptr<HipRuntime> &rt, const eo_conv_shape
 
 // ---------------------------------------------------------------- tests
 
+// One execution of a built list the way the userdriver does it: host bytes into the list's inputs, the executor,
+// the outputs back (gpu_userdriver.cc:97-103).
+static EnnReturn run_list(OperationConstructor &built, OperationExecutor &executor, const std::vector<const void *> &inputs,
+                          const std::vector<void *> &outputs) {
+    if (inputs.size() != built.in_tensors.size() || outputs.size() != built.out_tensors.size()) return ENN_RET_FAILED;
+    for (size_t i = 0; i < inputs.size(); ++i)
+        if (built.in_tensors[i]->writeData(const_cast<void *>(inputs[i]), false) != Status::SUCCESS) return ENN_RET_FAILED;
+    UDBuffers buffers;
+    BufferTable table;
+    if (executor.execute(built.operators, buffers, table) != ENN_RET_SUCCESS) return ENN_RET_FAILED;
+    for (size_t i = 0; i < outputs.size(); ++i)
+        if (built.out_tensors[i]->readData(outputs[i], true) != Status::SUCCESS) return ENN_RET_FAILED;
+    return ENN_RET_SUCCESS;
+}
+
 static int gpu_tests() {
-    auto rt = std::make_shared<HipRuntime>();
-    if (rt->initialize(0) != Status::SUCCESS || rt->initializeQueue() != Status::SUCCESS) {
+    auto lib = std::make_shared<HipComputeLibrary>(0);
+    if (!lib->valid() || lib->initialize_queue() != Status::SUCCESS) {
         std::printf("cannot initialise the GPU runtime: %s\n", eh_last_error());
         return 2;
     }
+    auto rt = lib->runtime();
     const Quant q1 = {0.02f, 0.005f, 0.05f, 128, 120, 0};
 
     run_test("Convolution.Config1_3x3_64to64_56x56_nchw_relu", [&] {
@@ -1059,15 +1076,15 @@ static int gpu_tests() {
                 eo_add_u8(t3.data(), t1.data(), t4b.data(), 16 * 64, &aq);
                 EXPECT(same(t4b, t4));  // the quantized sum does not depend on the operand order
             }
-            OperationConstructor built(rt);
+            OperationConstructor built(lib);
             built.fuse_residual_adds = fuse;
             EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
             EXPECT(built.operators && built.operators->size() == (fuse ? 5u : 6u));
             EXPECT(built.in_tensors.size() == 1 && built.out_tensors.size() == 1);
-            OperationExecutor executor(rt);
+            OperationExecutor executor(lib);
             for (int round = 0; round < 2; ++round) {  // a second execution reuses the pooled buffers
                 std::fill(got.begin(), got.end(), 0);
-                EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
+                EXPECT(run_list(built, executor, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
                 EXPECT(same(got, want));
             }
             for (auto &o : *built.operators) EXPECT(o->release() == ENN_RET_SUCCESS);
@@ -1109,10 +1126,10 @@ static int gpu_tests() {
                         {f1, param("w2", {12, 6, 2, 2}, w2.data(), TFlite::TensorType_UINT8, sw, 130),
                          param("b2", {6}, b2.data(), TFlite::TensorType_INT32, s1 * sw, 0)}, {f2}, up_opt),
             };
-            OperationConstructor built(rt);
+            OperationConstructor built(lib);
             EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
-            OperationExecutor executor(rt);
-            EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
+            OperationExecutor executor(lib);
+            EXPECT(run_list(built, executor, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
             EXPECT(same(got, want));
             EXPECT(varied(want));
         }
@@ -1137,10 +1154,10 @@ static int gpu_tests() {
         list.legacy_model = TFlite::LegacyModel_TENSORFLOW_NCHW;
         list.operators = {op_desc("CONV_2D", 1, TFlite::BuiltinOperator_CONV_2D, {f0, wt, param("b", {24}, b.data(), TFlite::TensorType_INT32, 1.0f, 0)},
                                   {f1}, std::make_shared<TFlite::Conv2DOptions>())};
-        OperationConstructor built(rt);
+        OperationConstructor built(lib);
         EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
-        OperationExecutor executor(rt);
-        EXPECT(executor.execute(built, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
+        OperationExecutor executor(lib);
+        EXPECT(run_list(built, executor, {x.data()}, {got.data()}) == ENN_RET_SUCCESS);
         EXPECT(same(std::vector<uint8_t>(got.begin(), got.end()), std::vector<uint8_t>(want.begin(), want.end())));
         EXPECT(varied(std::vector<uint8_t>(want.begin(), want.end())));
         return ok;
