@@ -126,6 +126,11 @@ public:
     // operator less than the description.  The reference builds one operator per description
     // (gpu_op_constructor.cc:63-383); set to false for that.
     bool fuse_residual_adds = true;
+    // A feature map no operator of the list writes (a list input) keeps its storage for the life of the list, so that
+    // the list can run again on data that is already on the device.  The reference hands such a buffer on to later
+    // feature maps once its last reader is built, which is safe there because every ExecuteSubGraph rewrites the
+    // inputs first (gpu_userdriver.cc:97-99); set to false for that.
+    bool keep_list_inputs = true;
 
     // ---- helpers, public because tests pin them against hand-computed cases
 
@@ -297,7 +302,9 @@ private:
             in.push_back(tensor);
             if (!edge->is_const) {
                 auto used = tensors_used_.find(edge->buffer_index);
-                if (used != tensors_used_.end() && used->second > 0 && --used->second == 0) tensor->resetInterBuffer();
+                if (used != tensors_used_.end() && used->second > 0 && --used->second == 0 &&
+                    !(keep_list_inputs && !produced_.count(edge->buffer_index)))
+                    tensor->resetInterBuffer();
             }
         }
         return true;
@@ -338,7 +345,7 @@ private:
         return finish(op, compute_library_->createConvolution(precision), in, out, p);
     }
 
-    // `add` consumes `conv`'s only output, nothing else does, both are uint8 per-tensor, and the sum is not
+    // `add` consumes `conv`'s only output, nothing else does, all four tensors are uint8, and the sum is not
     // written over one of the tensors the fused launch still reads
     bool fusable_add(const OperatorDesc &conv, const OperatorDesc &add) const {
         if (conv.code != TFlite::BuiltinOperator_CONV_2D || add.code != TFlite::BuiltinOperator_ADD) return false;
@@ -353,7 +360,6 @@ private:
         if (other->is_const) return false;
         const auto readers = tensors_used_.find(produced->buffer_index);
         if (readers == tensors_used_.end() || readers->second != 1) return false;
-        if (!conv.in_tensors[1]->per_channel_scales.empty()) return false;
         for (const auto &t : {produced, other, add.out_tensors[0], conv.in_tensors[0]})
             if (t->data_type != TFlite::TensorType_UINT8) return false;
         if (produced->shape != other->shape || produced->shape != add.out_tensors[0]->shape) return false;

@@ -260,6 +260,18 @@ public:
             desc_.weight_layout |= EH_W_SIGNED;
             desc_.layout |= EH_IO_SIGNED;
         }
+        // Weights or bias that are run-time feature maps of an operator list have no device memory until the list's
+        // pooled buffers are assigned: the plan is then made by the first execute(), which is where the reference packs
+        // such weights anyway.
+        if ((weights_as_input_ || bias_as_input_) && (weight_->getDataPtr() == nullptr || bias_->getDataPtr() == nullptr)) {
+            deferred_ = true;
+            return Status::SUCCESS;
+        }
+        return makePlan();
+    }
+
+    Status makePlan() {
+        deferred_ = false;
         eh_requant q;
         CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipConvolution::initialize: requantization parameters");
         const int rc = eh_conv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
@@ -269,6 +281,7 @@ public:
     }
 
     Status execute() {
+        if (plan_ == nullptr && deferred_) CHECK_EXPR_RETURN_FAILURE(makePlan() == Status::SUCCESS, "HipConvolution::execute: the deferred plan could not be made");
         if (plan_ == nullptr) {  // zero-sized operator
             CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipConvolution::execute before initialize");
             return Status::SUCCESS;
@@ -302,10 +315,11 @@ public:
     // From now on execute() stores add(residual, convolution) in `sum` and leaves this operator's own output tensor
     // unwritten: the quantized CLAdd that follows this convolution in an operator list, taken into its launch
     // (gpu/operators/CLAdd.cpp:159-163; the sum of the two rescaled operands does not depend on their order).  The
-    // output tensor still supplies the scale and zero point the convolution requantizes to.  UINT8, per-tensor.
+    // output tensor still supplies the scale and zero point the convolution requantizes to.  UINT8 tensors (per-tensor
+    // or per-channel weights).
     Status fuseResidualAdd(std::shared_ptr<ITensor> residual, std::shared_ptr<ITensor> sum, const ActivationInfo &add_activation) {
-        CHECK_EXPR_RETURN_FAILURE(plan_ != nullptr, "HipConvolution::fuseResidualAdd before initialize");
-        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8 && !per_channel_, "HipConvolution::fuseResidualAdd: UINT8 per-tensor only");
+        CHECK_EXPR_RETURN_FAILURE(plan_ != nullptr || deferred_, "HipConvolution::fuseResidualAdd before initialize");
+        CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8, "HipConvolution::fuseResidualAdd: UINT8 tensors only");
         auto r = std::static_pointer_cast<HipTensor>(residual), t = std::static_pointer_cast<HipTensor>(sum);
         CHECK_EXPR_RETURN_FAILURE(r && t && r->getDataType() == DataType::UINT8 && t->getDataType() == DataType::UINT8,
                                   "HipConvolution::fuseResidualAdd: expects uint8 tensors");
@@ -358,6 +372,7 @@ private:
     ActivationInfo activation_info_;
     bool weights_as_input_ = false, bias_as_input_ = false;
     eh_conv_desc desc_{};
+    bool deferred_ = false;
     eh_conv_plan *plan_ = nullptr;
 };
 
@@ -424,6 +439,18 @@ public:
             desc_.weight_layout |= EH_W_SIGNED;
             desc_.layout |= EH_IO_SIGNED;
         }
+        // Weights or bias that are run-time feature maps of an operator list have no device memory until the list's
+        // pooled buffers are assigned: the plan is then made by the first execute(), which is where the reference packs
+        // such weights anyway.
+        if (weights_as_input_ && (weight_->getDataPtr() == nullptr || bias_->getDataPtr() == nullptr)) {
+            deferred_ = true;
+            return Status::SUCCESS;
+        }
+        return makePlan();
+    }
+
+    Status makePlan() {
+        deferred_ = false;
         eh_requant q;
         CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDepthwiseConvolution::initialize: requantization parameters");
         const int rc = eh_dwconv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
@@ -433,7 +460,8 @@ public:
     }
 
     Status execute() {
-        if (plan_ == nullptr) {
+        if (plan_ == nullptr && deferred_) CHECK_EXPR_RETURN_FAILURE(makePlan() == Status::SUCCESS, "HipDepthwiseConvolution::execute: the deferred plan could not be made");
+        if (plan_ == nullptr) {  // zero-sized operator
             CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipDepthwiseConvolution::execute before initialize");
             return Status::SUCCESS;
         }
@@ -488,6 +516,7 @@ private:
     ActivationInfo activation_info_;
     bool weights_as_input_ = false;
     eh_conv_desc desc_{};
+    bool deferred_ = false;
     eh_dwconv_plan *plan_ = nullptr;
 };
 
@@ -524,14 +553,26 @@ public:
         CHECK_EXPR_RETURN_FAILURE(parameters_->androidNN || m == input_->getDim().n, "HipFullyConnected: input batch %u does not match %u rows of k = %u", input_->getDim().n, m, k);
         CHECK_EXPR_RETURN_FAILURE(output_->getTotalSizeFromDims() == m * units, "HipFullyConnected: output has %u elements, expected %u", output_->getTotalSizeFromDims(), m * units);
         m_ = (int32_t)m;
+        k_ = (int32_t)k;
+        units_ = (int32_t)units;
+        if (weights_as_input_ && (weight_->getDataPtr() == nullptr || bias_->getDataPtr() == nullptr)) {  // see HipConvolution::initialize
+            deferred_ = true;
+            return Status::SUCCESS;
+        }
+        return makePlan();
+    }
+
+    Status makePlan() {
+        deferred_ = false;
         const eh_requant q = detail::requantFromTensors(precision_, input_, weight_, bias_, output_, activation_info_);
         const int32_t flags = precision_ == PrecisionType::INT8 ? (EH_W_SIGNED | EH_IO_SIGNED) : 0;
-        const int rc = eh_fc_q8_plan(&plan_, (int32_t)m, (int32_t)k, (int32_t)units, flags, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
+        const int rc = eh_fc_q8_plan(&plan_, m_, k_, units_, flags, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
         CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipFullyConnected::initialize: %s", eh_last_error());
         return Status::SUCCESS;
     }
 
     Status execute() {
+        if (plan_ == nullptr && deferred_) CHECK_EXPR_RETURN_FAILURE(makePlan() == Status::SUCCESS, "HipFullyConnected::execute: the deferred plan could not be made");
         if (plan_ == nullptr) {
             CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipFullyConnected::execute before initialize");
             return Status::SUCCESS;
@@ -564,7 +605,8 @@ private:
     std::shared_ptr<FullyConnectedParameters> parameters_;
     ActivationInfo activation_info_;
     bool weights_as_input_ = false;
-    int32_t m_ = 0;
+    int32_t m_ = 0, k_ = 0, units_ = 0;
+    bool deferred_ = false;
     eh_fc_plan *plan_ = nullptr;
 };
 
@@ -633,6 +675,18 @@ public:
             desc_.weight_layout |= EH_W_SIGNED;
             desc_.layout |= EH_IO_SIGNED;
         }
+        // Weights or bias that are run-time feature maps of an operator list have no device memory until the list's
+        // pooled buffers are assigned: the plan is then made by the first execute(), which is where the reference packs
+        // such weights anyway.
+        if (weights_as_input_ && (weight_->getDataPtr() == nullptr || bias_->getDataPtr() == nullptr)) {
+            deferred_ = true;
+            return Status::SUCCESS;
+        }
+        return makePlan();
+    }
+
+    Status makePlan() {
+        deferred_ = false;
         eh_requant q;
         CHECK_EXPR_RETURN_FAILURE(currentRequant(&q) == Status::SUCCESS, "HipDeconvolution::initialize: requantization parameters");
         const int rc = eh_deconv2d_u8_plan(&plan_, &desc_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
@@ -642,7 +696,8 @@ public:
     }
 
     Status execute() {
-        if (plan_ == nullptr) {
+        if (plan_ == nullptr && deferred_) CHECK_EXPR_RETURN_FAILURE(makePlan() == Status::SUCCESS, "HipDeconvolution::execute: the deferred plan could not be made");
+        if (plan_ == nullptr) {  // zero-sized operator
             CHECK_EXPR_RETURN_FAILURE(weight_ && weight_->getTotalSizeFromDims() == 0, "HipDeconvolution::execute before initialize");
             return Status::SUCCESS;
         }
@@ -697,6 +752,7 @@ private:
     ActivationInfo activation_info_;
     bool weights_as_input_ = false;
     eh_conv_desc desc_{};
+    bool deferred_ = false;
     eh_deconv_plan *plan_ = nullptr;
 };
 

@@ -1163,6 +1163,168 @@ static int gpu_tests() {
         return ok;
     });
 
+
+    // ------------------------------------------------------------ compute library, executor, userdriver
+    run_test("ComputeLibrary.TensorsAndOperatorsComeFromTheLibrary", [&] {
+        bool ok = true;
+        auto t = lib->create_tensor(TFlite::TensorType_UINT8, U8, NDims{2, 3, 4, 5}, 7, BufferType::DEDICATED, false, StorageType::BUFFER, DataOrder::NCHW, 0.25f, 9);
+        EXPECT(t != nullptr);
+        if (!t) return false;
+        EXPECT(t->getDataType() == DataType::UINT8 && t->getPrecisionType() == U8 && t->getNumOfDims() == 4 && t->getTotalSizeFromDims() == 120);
+        EXPECT(t->get_buffer_index() == 7 && t->get_buffer_type() == (uint32_t)TFlite::TensorType_UINT8 && !t->is_const());
+        EXPECT(t->getScale() == 0.25f && t->getZeroPoint() == 9);
+        auto two = lib->create_tensor(TFlite::TensorType_INT32, U8, NDims{6, 10});   // rank kept, Dim4 padded with ones
+        EXPECT(two && two->getNumOfDims() == 2 && two->getDim().h == 1 && two->getDim().w == 1 && two->getNumOfBytes() == 240);
+        std::vector<int32_t> b = rand_i32(60, 501, -9999, 9999), back(60);
+        DataPtr data = b.data();
+        auto c = lib->create_and_copy_tensor(TFlite::TensorType_INT32, data, U8, NDims{60}, UNDEFINED, BufferType::DEDICATED, false, StorageType::BUFFER, DataOrder::NCHW, 0.5f, 0);
+        EXPECT(c && c->is_const() && c->getDataType() == DataType::INT32);
+        EXPECT(c && c->readData(back.data()) == Status::SUCCESS && back == b);
+        auto clone = lib->clone_tensor(t);
+        EXPECT(clone && clone->getDims() == t->getDims() && clone->getPrecisionType() == t->getPrecisionType() && clone->get_buffer_index() == 7);
+        EXPECT(clone && std::static_pointer_cast<HipTensor>(clone)->getDataPtr() != std::static_pointer_cast<HipTensor>(t)->getDataPtr());
+        EXPECT(lib->create_tensor(TFlite::TensorType_UINT8, U8, NDims{1, 1, 2, 2}, UNDEFINED, BufferType::DEDICATED, false, StorageType::TEXTURE) == nullptr);
+        EXPECT(lib->create_tensor(TFlite::TensorType_INT64, U8, NDims{4}) == nullptr);
+        EXPECT(lib->tensor_type_2_data_type(TFlite::TensorType_INT64) == DataType::SIZE && lib->tensor_type_2_data_type(TFlite::TensorType_INT8) == DataType::INT8);
+        EXPECT(lib->setPublicKernels(ANDROID_NN_API, StorageType::BUFFER) == Status::SUCCESS && lib->setPublicKernels(ANDROID_NN_API, StorageType::TEXTURE) == Status::FAILURE);
+        // an operator made by the library, on tensors made by the library
+        const eo_conv_shape s = shape(1, 16, 9, 9, 24, 3, 3, 1, 1, 1, 1, 1, 1);
+        auto x = rand_u8(16 * 81, 502), w = rand_u8(24 * 16 * 9, 503);
+        auto bias = rand_i32(24, 504, -500, 500);
+        eo_quant q;
+        eo_make_quant(0.02f, 128, 0.005f, 120, 0.02f * 0.005f, 0.05f, 3, 0, 0, &q);
+        std::vector<uint8_t> want(24 * 81), got(want.size());
+        eo_conv2d_u8(x.data(), w.data(), bias.data(), want.data(), &s, &q, nullptr);
+        DataPtr wp = w.data(), bp = bias.data();
+        auto ti = lib->create_tensor(TFlite::TensorType_UINT8, U8, NDims{1, 16, 9, 9}, 0, BufferType::DEDICATED, false, StorageType::BUFFER, DataOrder::NCHW, 0.02f, 128);
+        auto tw = lib->create_and_copy_tensor(TFlite::TensorType_UINT8, wp, U8, NDims{24, 16, 3, 3}, UNDEFINED, BufferType::DEDICATED, false, StorageType::BUFFER, DataOrder::NCHW, 0.005f, 120);
+        auto tb = lib->create_and_copy_tensor(TFlite::TensorType_INT32, bp, U8, NDims{24}, UNDEFINED, BufferType::DEDICATED, false, StorageType::BUFFER, DataOrder::NCHW, 0.02f * 0.005f, 0);
+        auto to = lib->create_tensor(TFlite::TensorType_UINT8, U8, NDims{1, 24, 9, 9}, 1, BufferType::DEDICATED, false, StorageType::BUFFER, DataOrder::NCHW, 0.05f, 3);
+        auto conv = lib->createConvolution(U8);
+        auto params = std::make_shared<ConvolutionParameters>();
+        params->padding = {1, 1, 1, 1};
+        EXPECT(conv->initialize({ti, tw, tb}, {to}, params) == Status::SUCCESS);
+        EXPECT(ti->writeData(x.data(), false) == Status::SUCCESS);
+        EXPECT(conv->execute() == Status::SUCCESS);
+        lib->flush();
+        EXPECT(to->readData(got.data(), false) == Status::SUCCESS);   // queued only ...
+        lib->synchronize();                                            // ... defined after the library has drained
+        EXPECT(same(got, want) && varied(want));
+        EXPECT(lib->createAdd(U8) && lib->createAveragepool(U8) && lib->createDeconvolution(U8) && lib->createDepthwiseConvolution(U8) && lib->createFullyConnected(U8));
+        return ok;
+    });
+
+    run_test("Executor.RecordsOnTheSecondExecutionAndLeavesWeightsAsInputListsAlone", [&] {
+        bool ok = true;
+        const eo_conv_shape s = shape(2, 8, 10, 10, 16, 3, 3, 1, 1, 1, 1, 1, 1);
+        auto x = rand_u8(2 * 8 * 100, 511), w1 = rand_u8(16 * 8 * 9, 512), w2 = rand_u8(16 * 8 * 9, 513);
+        auto bias = rand_i32(16, 514, -500, 500);
+        eo_quant q;
+        eo_make_quant(0.02f, 128, 0.005f, 120, 0.02f * 0.005f, 0.06f, 3, 0, 0, &q);
+        std::vector<uint8_t> want1(2 * 16 * 100), want2(want1.size()), got(want1.size());
+        eo_conv2d_u8(x.data(), w1.data(), bias.data(), want1.data(), &s, &q, nullptr);
+        eo_conv2d_u8(x.data(), w2.data(), bias.data(), want2.data(), &s, &q, nullptr);
+        auto conv_opt = std::make_shared<TFlite::Conv2DOptions>();
+        for (const bool const_weights : {true, false}) {
+            auto f0 = fmap("in", {2, 8, 10, 10}, 0, 0.02f, 128), f1 = fmap("out", {2, 16, 10, 10}, 1, 0.06f, 3);
+            auto wt = const_weights ? param("w", {16, 8, 3, 3}, w1.data(), TFlite::TensorType_UINT8, 0.005f, 120) : fmap("w", {16, 8, 3, 3}, 2, 0.005f, 120);
+            OperatorListDesc list;
+            list.id = const_weights ? 21 : 22;
+            list.legacy_model = TFlite::LegacyModel_TENSORFLOW;
+            list.operators = {op_desc("CONV_2D", 1, TFlite::BuiltinOperator_CONV_2D, {f0, wt, param("b", {16}, bias.data(), TFlite::TensorType_INT32, 0.02f * 0.005f, 0)}, {f1}, conv_opt)};
+            OperationConstructor built(lib);
+            EXPECT(built.open_oplist(list) == ENN_RET_SUCCESS);
+            EXPECT(built.in_tensors.size() == (const_weights ? 1u : 2u) && built.out_tensors.size() == 1);
+            OperationExecutor executor(lib);
+            for (int round = 0; round < 4; ++round) {
+                std::fill(got.begin(), got.end(), 0);
+                const auto &w = round < 2 ? w1 : w2;
+                std::vector<const void *> inputs = {x.data()};
+                if (!const_weights) inputs.push_back(w.data());
+                EXPECT(run_list(built, executor, inputs, {got.data()}) == ENN_RET_SUCCESS);
+                EXPECT(same(got, const_weights || round < 2 ? want1 : want2));
+            }
+            const auto &c = executor.counters();
+            if (const_weights)
+                EXPECT(c.direct == 1 && c.recordings == 1 && c.replays == 3);
+            else
+                EXPECT(c.direct == 4 && c.recordings == 0 && c.replays == 0);   // re-packing weights is not replayable
+            executor.forget(built.operators);
+            built.close_oplist(list.id);
+        }
+        EXPECT(varied(want1) && !same(want1, want2));
+        return ok;
+    });
+
+    run_test("UserDriver.OpenExecuteCloseThroughTheBufferTable", [&] {
+        bool ok = true;
+        HipUserDriver ud(0);
+        EXPECT(ud.Initialize() == ENN_RET_SUCCESS);
+        // conv 1x1 (24 -> 48, relu6) -> depthwise 3x3 stride 2 (relu6), channels-last androidNN model
+        const float s0 = 0.02f, sw = 0.004f, s1 = 6.0f / 255, s2 = 6.0f / 255;
+        auto x = rand_u8(2 * 12 * 12 * 24, 521), w1 = rand_u8(48 * 24, 522), wd = rand_u8(9 * 48, 523);
+        auto b1 = rand_i32(48, 524, -500, 500), bd = rand_i32(48, 525, -500, 500);
+        auto xn = nhwc_to_nchw(x, 2, 24, 12, 12);
+        std::vector<uint8_t> wdo(48 * 9);
+        for (int t = 0; t < 9; ++t)
+            for (int c = 0; c < 48; ++c) wdo[c * 9 + t] = wd[t * 48 + c];
+        eo_quant q;
+        std::vector<uint8_t> t1(2 * 48 * 144), t2(2 * 48 * 36);
+        eo_conv_shape c1 = shape(2, 24, 12, 12, 48, 1, 1);
+        eo_make_quant(s0, 128, sw, 120, s0 * sw, s1, 0, EO_ACT_RELU6, 1, &q);
+        eo_conv2d_u8(xn.data(), w1.data(), b1.data(), t1.data(), &c1, &q, nullptr);
+        eo_conv_shape c2 = shape(2, 48, 12, 12, 48, 3, 3, 2, 2, 1, 1, 1, 1, 1, 1, 1, 1);
+        c2.pad_t = 0; c2.pad_l = 0; c2.pad_b = 1; c2.pad_r = 1;   // SAME at stride 2 on an even extent: the extra row and column go last
+        eo_make_quant(s1, 0, sw, 131, s1 * sw, s2, 0, EO_ACT_RELU6, 1, &q);
+        eo_dwconv2d_u8(t1.data(), wdo.data(), bd.data(), t2.data(), &c2, &q, nullptr);
+        const auto want = nchw_to_nhwc(t2, 2, 48, 6, 6);
+        auto f0 = fmap("in", {2, 12, 12, 24}, 10, s0, 128), f1 = fmap("pw", {2, 12, 12, 48}, 11, s1, 0), f2 = fmap("dw", {2, 6, 6, 48}, 12, s2, 0);
+        auto pw_opt = std::make_shared<TFlite::Conv2DOptions>();
+        pw_opt->fused_activation_function = TFlite::ActivationFunctionType_RELU6;
+        auto dw_opt = std::make_shared<TFlite::DepthwiseConv2DOptions>();
+        dw_opt->stride_h = dw_opt->stride_w = 2;
+        dw_opt->fused_activation_function = TFlite::ActivationFunctionType_RELU6;
+        OperatorListDesc list;
+        list.id = 0xABCD;
+        list.legacy_model = TFlite::LegacyModel_ANDROID_NN;
+        list.operators = {
+            op_desc("CONV_2D", 1, TFlite::BuiltinOperator_CONV_2D,
+                    {f0, param("w1", {48, 1, 1, 24}, w1.data(), TFlite::TensorType_UINT8, sw, 120), param("b1", {48}, b1.data(), TFlite::TensorType_INT32, s0 * sw, 0)}, {f1}, pw_opt),
+            op_desc("DEPTHWISE_CONV_2D", 2, TFlite::BuiltinOperator_DEPTHWISE_CONV_2D,
+                    {f1, param("wd", {1, 3, 3, 48}, wd.data(), TFlite::TensorType_UINT8, sw, 131), param("bd", {48}, bd.data(), TFlite::TensorType_INT32, s1 * sw, 0)}, {f2}, dw_opt),
+        };
+        EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS);
+        EXPECT(ud.OpenSubGraph(list) == ENN_RET_FAILED);   // open already
+        EXPECT(ud.PrepareSubGraph(list.id) == ENN_RET_SUCCESS);
+        UDOperators ops;
+        EXPECT(ud.get_graph_for_TC(list.id, ops) == ENN_RET_SUCCESS && ops && ops->size() == 2 && (*ops)[0]->getName() == "CONV_2D");
+        std::vector<uint8_t> got(want.size());
+        for (int round = 0; round < 3; ++round) {
+            std::fill(got.begin(), got.end(), 0);
+            BufferTable table;
+            table.add(10, x.data(), x.size());
+            table.add(12, got.data(), got.size());
+            table.add(99, nullptr, 0);   // an index no tensor of the list has is ignored
+            EXPECT(ud.ExecuteSubGraph(OperatorListExecuteRequest(list.id, (uint64_t)round, table)) == ENN_RET_SUCCESS);
+            EXPECT(same(got, want));
+        }
+        EXPECT(ud.executor()->counters().direct == 1 && ud.executor()->counters().recordings == 1 && ud.executor()->counters().replays == 2);
+        {
+            BufferTable small;
+            small.add(10, x.data(), 16);   // too small for the input tensor
+            EXPECT(ud.ExecuteSubGraph(OperatorListExecuteRequest(list.id, 9, small)) == ENN_RET_FAILED);
+            BufferTable none;
+            EXPECT(ud.ExecuteSubGraph(OperatorListExecuteRequest(0x1234, 9, none)) == ENN_RET_FAILED);   // unknown list
+        }
+        EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_SUCCESS);
+        EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_FAILED);
+        EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS);   // and it can be opened again
+        EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_SUCCESS);
+        EXPECT(ud.Deinitialize() == ENN_RET_SUCCESS);
+        EXPECT(varied(want));
+        return ok;
+    });
+
     std::printf("%d of %d GPU operator tests failed\n", g_failed, g_run);
     return g_failed ? 1 : 0;
 }
