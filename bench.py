@@ -195,6 +195,28 @@ def pw_workload(eden, synth, n=32, cold=False):
                 keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 56 * 56 * 24 * 144, bytes=nbytes, bound="hbm")
 
 
+def block_workload(eden, synth, n=32, rows=0, cols=0, cold=False):
+    """BASELINE configs[2] as one launch: pointwise 24 -> 144 (ReLU6) feeding the 3x3 stride-2 depthwise convolution
+    from LDS (eh_conv_dw_block_run); algorithmic bytes = the block's input, weights and output (the 14.45 MB expanded
+    tensor is never stored)."""
+    d1 = eden.conv_desc(n, 24, 56, 56, 144, 1, 1, layout=eden.NHWC)
+    d2 = eden.conv_desc(n, 144, 56, 56, 144, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), dm=1, layout=eden.NHWC)
+    x = synth.fill_u8((n, 56, 56, 24), SEED + 51)
+    w1, b1 = synth.fill_u8((144, 24, 1, 1), SEED + 52), synth.fill_i32((144,), SEED + 53, -1000, 1000)
+    w2, b2 = synth.fill_u8((144, 1, 3, 3), SEED + 49), synth.fill_i32((144,), SEED + 50, -1000, 1000)
+    q1 = eden.make_requant(0.02, 120, 0.004, 131, 0.03, 17, eden.ACT_RELU6, True)
+    q2 = eden.make_requant(0.03, 17, 0.006, 140, 0.025, 9, eden.ACT_RELU6, True)
+    keep = [eden.DeviceBuffer(host=a) for a in (w1, b1, w2, b2)]
+    pw, dw = eden.ConvPlan(d1, keep[0], keep[1], q1), eden.DwConvPlan(d2, keep[2], keep[3], q2)
+    assert eden.conv_dw_block_applies(pw, dw)
+    nbytes = n * 56 * 56 * 24 + 144 * 24 + 576 + 144 * 9 + 576 + n * 28 * 28 * 144
+    sets = set_count(nbytes, cold)
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 28 * 28 * 144)) for _ in range(sets)]
+    return dict(name="c3block_n%d_pw24to144_dw3x3s2_56x56_nhwc%s" % (n, "_tile%dx%d" % (rows, cols) if rows or cols else ""),
+                launch=lambda s, i: eden.conv_dw_block_run(pw, dw, bufs[i][0], bufs[i][1], q1, q2, rows, cols, stream=s),
+                keep=(bufs, keep, pw, dw), sets=sets, ops=2.0 * n * (56 * 56 * 24 * 144 + 28 * 28 * 144 * 9), bytes=nbytes, bound="hbm")
+
+
 def deconv_workload(eden, synth, n=8, cold=False):
     desc = eden.conv_desc(n, 256, 32, 32, 128, 4, 4, stride=(2, 2), pad=(1, 1, 1, 1), layout=eden.NHWC,
                           weight_layout=eden.W_IOHW)
@@ -417,6 +439,7 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the oracle check of the network")
     ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2, mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, copy, tonhwc, tonchw")
+    ap.add_argument("--tile", default=None, help="with --only c3block: ROWSxCOLS output pixels per workgroup (default: chosen by the library)")
     ap.add_argument("--cold", action="store_true", help="with --only: rotate over buffer sets that together exceed the Infinity Cache")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -436,6 +459,8 @@ def main():
 
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
                     fcbig=shaped(fc_workload, m=8192, k=4096, n=4096), conv64=shaped(conv_workload, n=64),
+                    c3block=block_workload,
+                    c3blockbig=shaped(block_workload, n=256),
                     dwbig=shaped(dw_workload, n=256), pwbig=shaped(pw_workload, n=256),
                     copy=copy_workload, mbv2=mbv2_workload, mbv2narrow=shaped(mbv2_workload, weights="narrow"),
                     tonhwc=layout_workload, tonchw=shaped(layout_workload, to_nhwc=False),
@@ -454,6 +479,10 @@ def main():
                               ms_per_step=wall / steps * 1e3, us_per_step_by_events=ev / steps * 1e6, timed_region_repeats=reps,
                               images_per_s=round(64 * steps / wall, 1), executor=driver.stats(list_id))))
         return
+    if args.only and args.tile:
+        rows, cols = (int(v) for v in args.tile.split("x"))
+        families["c3block"] = shaped(block_workload, rows=rows, cols=cols)
+        families["c3blockbig"] = shaped(block_workload, n=256, rows=rows, cols=cols)
     if args.only:
         work = families[args.only](eden, synth, cold=args.cold)
         args.steps = round_steps(args.steps, work["sets"], work.get("chunk", 50))
@@ -532,7 +561,7 @@ def main():
         del net
         others = [c5]
         for make, steps, cold_too in ((conv_workload, 2000, False), (shaped(conv_workload, n=64), 300, False),
-                                      (pw_workload, 500, True), (dw_workload, 1000, True),
+                                      (pw_workload, 500, True), (dw_workload, 1000, True), (block_workload, 500, True),
                                       (shaped(pw_workload, n=256), 100, True), (shaped(dw_workload, n=256), 200, True),
                                       (deconv_workload, 500, False), (fc_workload, 500, True),
                                       (shaped(fc_workload, m=8192, k=4096, n=4096), 100, False),

@@ -73,6 +73,9 @@ EXPORTS = {
     "eh_conv2d_u8_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(AddRequant),
                                        C.c_void_p]),
     "eh_conv2d_u8_fuses_add": (C.c_int, [C.c_void_p]),
+    "eh_conv_dw_block_applies": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eh_conv_dw_block_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(Requant), C.c_int32,
+                                       C.c_int32, C.c_void_p]),
     "eh_conv2d_u8_run_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
     "eh_conv2d_u8_kernels": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_int32]),
     "eh_deconv2d_u8_kernels": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_int32]),
@@ -313,6 +316,17 @@ class PooledBuffer:
             check(lib.eh_d2h(out.ctypes.data_as(C.c_void_p), self.ptr, out.nbytes, None))
         check(lib.eh_stream_sync(None))
         return out
+
+
+def conv_dw_block_applies(pointwise, depthwise):
+    """whether a ConvPlan (1x1) and the DwConvPlan on its output can run as one launch"""
+    return bool(load().eh_conv_dw_block_applies(pointwise.handle, depthwise.handle))
+
+
+def conv_dw_block_run(pointwise, depthwise, d_in, d_out, q_pointwise, q_depthwise, rows_per_tile=0, cols_per_tile=0, stream=None):
+    """pointwise convolution + 3x3 depthwise convolution as one launch (the expanded tensor stays in LDS)"""
+    check(load().eh_conv_dw_block_run(pointwise.handle, depthwise.handle, d_in.ptr, d_out.ptr, C.byref(q_pointwise), C.byref(q_depthwise),
+                                      rows_per_tile, cols_per_tile, stream))
 
 
 class BufferPool:

@@ -363,6 +363,32 @@ struct GemmOp {
     size_t stage_out_bytes() const { return ((size_t)in_n * cout * out_hw + 256 + 255) / 256 * 256; }
     static constexpr int kInlineParts = 8;  // a run over at most this many parts allocates no host memory
 
+    // One part's kernel argument for channels-last tensors `in` / `out`, with the quantization parameters refold() left in `q`
+    GemmProblem problem(const GemmPart &g, const uint8_t *in, uint8_t *out, const uint8_t *residual, const AddDev *radd) const {
+        GemmProblem p = g.proto;
+        p.a = in;
+        p.b = g.b;
+        p.bias = g.folded;
+        p.fillbuf = fillbuf;
+        p.out = out + g.bias_base;
+        p.zw = zp_w_u8(q) - 128;
+        p.out_xor = io_signed ? 0x80808080u : 0u;
+        p.a_xor = 0x80808080u ^ p.out_xor;
+        p.fill = ((uint32_t)q.zp_in * 0x01010101u) ^ p.out_xor;
+        p.rq = make_requant_dev(q);
+        p.residual = residual ? residual + g.bias_base : nullptr;
+        if (residual) p.radd = *radd;
+        if (pc_multiplier) {
+            p.rq.pc_multiplier = pc_multiplier + g.bias_base;
+            p.rq.pc_shift = pc_shift + g.bias_base;
+            // every kernel but the register-staged one has the single-shift form per channel (the first-layer
+            // kernel for fewer than 32 channels ignores the flag)
+            const bool has_form = g.cfg.id != GEMM_STAGED;
+            p.rq.fast = (pc_fast && has_form) ? channel_fast_mode(q) : 0;
+        }
+        return p;
+    }
+
     // staging != null: a planar plan uses [staging, staging + stage_in_bytes() + stage_out_bytes()) instead of its own images
     int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream, const uint8_t *residual = nullptr,
             const AddDev *radd = nullptr, bool *fused = nullptr, uint8_t *staging = nullptr) {
@@ -386,30 +412,9 @@ struct GemmOp {
         GemmProblem *const problems = many.empty() ? inline_problems : many.data();
         int filled = 0;
         for (auto &g : parts) {
-            GemmProblem p = g.proto;
             EH_REQUIRE((reinterpret_cast<uintptr_t>(in) & (uintptr_t)(g.vec - 1)) == 0,
                        "input pointer is not aligned to %d bytes", g.vec);
-            p.a = in;
-            p.b = g.b;
-            p.bias = g.folded;
-            p.fillbuf = fillbuf;
-            p.out = out + g.bias_base;
-            p.zw = zp_w_u8(q) - 128;
-            p.out_xor = io_signed ? 0x80808080u : 0u;
-            p.a_xor = 0x80808080u ^ p.out_xor;
-            p.fill = ((uint32_t)q.zp_in * 0x01010101u) ^ p.out_xor;
-            p.rq = make_requant_dev(q);
-            p.residual = fuse ? residual + g.bias_base : nullptr;
-            if (fuse) p.radd = *radd;
-            if (pc_multiplier) {
-                p.rq.pc_multiplier = pc_multiplier + g.bias_base;
-                p.rq.pc_shift = pc_shift + g.bias_base;
-                // every kernel but the register-staged one has the single-shift form per channel (the first-layer
-                // kernel for fewer than 32 channels ignores the flag)
-                const bool has_form = g.cfg.id != GEMM_STAGED;
-                p.rq.fast = (pc_fast && has_form) ? channel_fast_mode(q) : 0;
-            }
-            problems[filled++] = p;
+            problems[filled++] = problem(g, in, out, fuse ? residual : nullptr, radd);
         }
         if ((rc = launch_igemm_batch(problems, filled, stream))) return rc;
         if (layout == EH_NCHW) {
@@ -1448,15 +1453,9 @@ int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *
     return dw_refold(plan, *q, as_stream(stream));
 }
 
-int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
-    EH_REQUIRE(plan != nullptr, "null plan");
-    int rc = check_requant(q, plan->w_signed, plan->io_signed);
-    if (rc) return rc;
+// the kernel argument of a depthwise plan whose packed arrays match plan->q (after dw_refold)
+static DwProblem dw_problem(const eh_dwconv_plan *plan, const void *input, void *output) {
     const eh_conv_desc &d = plan->d;
-    if (d.n == 0) return EH_OK;
-    EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
-    hipStream_t s = as_stream(stream);
-    if ((rc = dw_refold(plan, *q, s))) return rc;
     DwProblem p;
     p.in = static_cast<const uint8_t *>(input);
     p.w = plan->w_copy;
@@ -1494,6 +1493,19 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
         p.rq.pc_shift = plan->pc_shift;
         p.rq.fast = plan->pc_fast ? channel_fast_mode(plan->q) : 0;
     }
+    return p;
+}
+
+int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream) {
+    EH_REQUIRE(plan != nullptr, "null plan");
+    int rc = check_requant(q, plan->w_signed, plan->io_signed);
+    if (rc) return rc;
+    const eh_conv_desc &d = plan->d;
+    if (d.n == 0) return EH_OK;
+    EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
+    hipStream_t s = as_stream(stream);
+    if ((rc = dw_refold(plan, *q, s))) return rc;
+    const DwProblem p = dw_problem(plan, input, output);
     return d.layout == EH_NHWC ? launch_dwconv_nhwc(p, s) : launch_dwconv_nchw(p, s);
 }
 
@@ -1503,6 +1515,40 @@ int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan) {
         delete plan;
     }
     return EH_OK;
+}
+
+
+// ------------------------------------------------------------ pointwise + depthwise block
+
+int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise) {
+    if (pointwise == nullptr || depthwise == nullptr) return 0;
+    const GemmOp &op = pointwise->op;
+    if (op.parts.size() != 1 || op.layout != EH_NHWC || op.io_signed || op.pc_multiplier) return 0;
+    if (depthwise->d.layout != EH_NHWC || depthwise->io_signed || depthwise->pc_multiplier) return 0;
+    if (depthwise->d.n != pointwise->d.n || !(depthwise->w_trip || depthwise->w_fold)) return 0;
+    // geometry and kernel family are checked on the problems themselves; the pointers and parameters of a run do not enter
+    const GemmProblem pw = op.problem(op.parts[0], nullptr, nullptr, nullptr, nullptr);
+    const DwProblem dw = dw_problem(depthwise, nullptr, nullptr);
+    return pwdw_block_applies(pw, dw) ? 1 : 0;
+}
+
+int eh_conv_dw_block_run(eh_conv_plan *pointwise, eh_dwconv_plan *depthwise, const void *input, void *output,
+                         const eh_requant *q_pointwise, const eh_requant *q_depthwise, int32_t rows_per_tile, int32_t cols_per_tile, void *stream) {
+    EH_REQUIRE(pointwise != nullptr && depthwise != nullptr, "null plan");
+    EH_REQUIRE(eh_conv_dw_block_applies(pointwise, depthwise), "block: these two plans do not fit the fused kernel");
+    int rc = check_requant(q_pointwise, pointwise->op.w_signed, false);
+    if (rc) return rc;
+    if ((rc = check_requant(q_depthwise, depthwise->w_signed, false))) return rc;
+    EH_REQUIRE(q_pointwise->zp_out == q_depthwise->zp_in, "block: the pointwise output zero point %d is not the depthwise input zero point %d",
+               q_pointwise->zp_out, q_depthwise->zp_in);
+    if (pointwise->d.n == 0) return EH_OK;
+    EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
+    hipStream_t s = as_stream(stream);
+    if ((rc = pointwise->op.refold(*q_pointwise, s))) return rc;
+    if ((rc = dw_refold(depthwise, *q_depthwise, s))) return rc;
+    const GemmProblem pw = pointwise->op.problem(pointwise->op.parts[0], static_cast<const uint8_t *>(input), nullptr, nullptr, nullptr);
+    const DwProblem dw = dw_problem(depthwise, nullptr, output);
+    return launch_pwdw_block(pw, dw, rows_per_tile, cols_per_tile, s);
 }
 
 }  // extern "C"

@@ -494,6 +494,10 @@ int launch_dw_pack_fold(const uint8_t *w, const int32_t *bias, int32_t *w_fold, 
 int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream);
 int launch_dwconv_nchw(const DwProblem &p, hipStream_t stream);
 
+// ---------------------------------------------------------------- pointwise + depthwise in one launch (eh_block.hip)
+bool pwdw_block_applies(const GemmProblem &pw, const DwProblem &dw);
+int launch_pwdw_block(const GemmProblem &pw, const DwProblem &dw, int rows_per_tile, int cols_per_tile, hipStream_t stream);
+
 // ---------------------------------------------------------------- layout
 int launch_nchw2nhwc(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);
 int launch_nhwc2nchw(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);

@@ -335,6 +335,22 @@ int eh_dwconv2d_u8_repack(eh_dwconv_plan *plan, const void *weight, const void *
 int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, const eh_requant *q, void *stream);
 int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
 
+/* A pointwise (1x1) convolution followed by a 3x3 depthwise convolution on its output, as ONE launch: the expanded
+ * tensor between them lives in LDS only (an output tile's rows plus their halo are computed per workgroup, the halo
+ * rows twice).  Bit for bit what eh_conv2d_u8_run into a temporary followed by eh_dwconv2d_u8_run gives.  No counterpart
+ * in the reference, whose operator list runs CLConvolution and CLDepthwiseConvolution one after the other
+ * (gpu/gpu_op_executor.cc:56-103), the expanded tensor written by quantizedGemmBlocked and read back by
+ * depthwise_conv_3x3s2_pad_merge (cl_kernels/DepthwiseconvolutionKernels.cpp:1964-2083).  Takes the two operators' own
+ * plans; `_applies` says whether the pair fits (1) or has to run as two launches (0): channels-last uint8 tensors, a
+ * pointwise layer of at most 32 input channels (a multiple of 8) whose output is the depthwise input, depthwise 3x3 at
+ * stride 1 or 2 without dilation or depth multiplier on a multiple of 16 channels, per-tensor requantization in both.
+ * rows_per_tile, cols_per_tile: the tile of output pixels a workgroup owns, 0 lets the library choose.
+ * q_pointwise->zp_out must equal q_depthwise->zp_in (they describe the same tensor). */
+int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise);
+int eh_conv_dw_block_run(eh_conv_plan *pointwise, eh_dwconv_plan *depthwise, const void *input, void *output,
+                         const eh_requant *q_pointwise, const eh_requant *q_depthwise, int32_t rows_per_tile, int32_t cols_per_tile,
+                         void *stream);
+
 /* CLFullyConnected::initialize / execute / release (gpu/operators/CLFullyConnected.cpp:22-150):
  * input [m][k], weight [n][k], bias [n], output [m][n]
  * (gpu/op_test/fullyconnected_test.cpp:93-105), computed in the convolution's
