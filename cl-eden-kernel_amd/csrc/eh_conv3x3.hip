@@ -35,7 +35,6 @@ typedef __attribute__((address_space(3))) uint8_t lds_byte;
 
 namespace {
 
-constexpr int G = 4;  // 32-pixel groups a wave multiplies together
 
 __device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(uintptr_t)(lds_byte *)p; }
 
@@ -57,7 +56,11 @@ struct Conv3Launch {
 // NB: 32-channel blocks per workgroup (grid y walks the channel ranges).
 // QM: 0 two-step requantization (one pair, or one per channel), 1 / 2 the single-shift forms (2: no sign test).
 // PC: one multiplier and shift per output channel.
-template <int NB, bool ROWSUM, int QM, bool PC>
+// G: 32-pixel groups a wave multiplies together (4 where a tile has sixteen groups or more, fewer on small tiles, so
+// that no matrix instruction is spent on repeated pixels).
+// SPLIT (NB == 2 only): a wave works on ONE of the two channel blocks, the waves forming 2 x 2 over (pixel group,
+// channel block): tiles of two pixel groups then keep all four waves busy instead of two.
+template <int NB, bool ROWSUM, int QM, bool PC, int G = 4, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void conv3x3_patch_kernel(const GemmProblem p, const Conv3Launch L) {
     extern __shared__ __align__(1024) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, half = lane >> 5;
@@ -154,23 +157,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
     // Wave w takes groups w', w' + 4, w' + 8, ... in passes of up to G.  When the groups do not divide by four the
     // first of them carry one more; w' is the wave number rotated by the workgroup's round of 256, so that the two
     // workgroups that share a CU put their longer waves on different SIMDs.
+    static_assert(!SPLIT || NB == 2, "the split over channel blocks is written for two blocks");
+    constexpr int NBW = SPLIT ? 1 : NB;        // channel blocks a wave works on
+    constexpr int GW = SPLIT ? 2 : 4;          // waves side by side along the pixel groups
     const int wave_rot = (wave + (int)(blockIdx.x >> 8)) & 3;
-    for (int g0 = wave_rot; g0 < groups; g0 += 4 * G) {
-        int ng = (groups - g0 + 3) >> 2;  // groups of this pass that exist
+    const int nb_lo = SPLIT ? wave_rot >> 1 : 0;
+    for (int g0 = SPLIT ? (wave_rot & 1) : wave_rot; g0 < groups; g0 += GW * G) {
+        int ng = (groups - g0 + GW - 1) / GW;  // groups of this pass that exist
         ng = ng < G ? ng : G;
         uint32_t base[G];   // patch byte address of the lane's pixel (top-left tap)
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            int pidx = (g0 + 4 * g) * 32 + r;
+            int pidx = (g0 + GW * g) * 32 + r;
             // (groups past the tile's last one repeat its last pixel and store nothing)
             pidx = pidx < pixels ? pidx : pixels - 1;
             const int py = (int)fastdiv((uint32_t)pidx, L.div_wo), px = pidx - py * p.wo;
             base[g] = (uint32_t)((py * L.pc + px) * L.pitch);
         }
-        v16i acc[G][NB];
+        v16i acc[G][NBW];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            const int32_t *bsrc = bias_s + nb * 32 + half * 16;
+        for (int nb = 0; nb < NBW; ++nb) {
+            const int32_t *bsrc = bias_s + (nb_lo + nb) * 32 + half * 16;
             v16i b16;
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
@@ -198,7 +205,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             for (int g = 0; g < G; ++g) {
                 const int ncorr = pixel_term(g);
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
+                for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[g][nb][i] += ncorr;
             }
@@ -206,12 +213,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
 
         // The fragments of step ks + 1 are requested before step ks is multiplied: the reads fly under the matrix
         // instructions, and the SIMD's other wave (two workgroups share a CU) fills what gaps remain.
-        v4i af[2][G], bf[2][NB];
+        v4i af[2][G], bf[2][NBW];
         auto read_step = [&](int ks, auto buf_c) {
             constexpr int buf = decltype(buf_c)::value;
             const uint32_t d = (uint32_t)step_s[ks * 2 + half];
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) bf[buf][nb] = w_s[((nb < nb_count ? nb : 0) * KS + ks) * 64 + lane];
+            for (int nb = 0; nb < NBW; ++nb) bf[buf][nb] = w_s[((nb_lo + nb < nb_count ? nb_lo + nb : 0) * KS + ks) * 64 + lane];
 #pragma unroll
             for (int g = 0; g < G; ++g) af[buf][g] = *reinterpret_cast<const v4i *>(patch + base[g] + d);
         };
@@ -220,7 +227,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
 #pragma unroll
             for (int g = 0; g < G; ++g) {
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) acc[g][nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[buf][nb], af[buf][g], acc[g][nb], 0, 0, 0);
+                for (int nb = 0; nb < NBW; ++nb) acc[g][nb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[buf][nb], af[buf][g], acc[g][nb], 0, 0, 0);
             }
         };
         typedef std::integral_constant<int, 0> b0;
@@ -238,19 +245,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
         // ---- epilogue: 16 consecutive channels of one pixel per lane and channel block
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            const int pidx = (g0 + 4 * g) * 32 + r;
+            const int pidx = (g0 + GW * g) * 32 + r;
             const bool ok = g < ng && pidx < pixels;
             uint8_t *const row = p.out + out_tile + (size_t)(ok ? pidx : 0) * (size_t)p.ldc;
             int late = 0;
             if constexpr (late_corr) late = pixel_term(g);
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
+            for (int nbw = 0; nbw < NBW; ++nbw) {
+                const int nb = nb_lo + nbw;
                 const int n = (nb_first + nb) * 32 + half * 16;
                 uint32_t packed[4];
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
-                    const int32_t x0 = acc[g][nb][q4 * 4 + 0], x1 = acc[g][nb][q4 * 4 + 1];
-                    const int32_t x2 = acc[g][nb][q4 * 4 + 2], x3 = acc[g][nb][q4 * 4 + 3];
+                    const int32_t x0 = acc[g][nbw][q4 * 4 + 0], x1 = acc[g][nbw][q4 * 4 + 1];
+                    const int32_t x2 = acc[g][nbw][q4 * 4 + 2], x3 = acc[g][nbw][q4 * 4 + 3];
                     uint32_t o0, o1, o2, o3;
                     if constexpr (PC) {  // the padded per-channel arrays cover whole blocks
                         const int4 cm = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + q4 * 4);
@@ -326,14 +334,38 @@ void conv3_shape(int n_img, int ho, int wo, int cin, int cout, int *th_out, int 
     }
 }
 
+// G and SPLIT for a tile of `groups` pixel groups: four groups per pass where a wave has three or more to do, one
+// otherwise; two-group tiles with two channel blocks spread their four (group, block) pairs over the four waves.
+struct Conv3Variant {
+    int g;
+    bool split;
+};
+Conv3Variant conv3_variant(int groups, int nb) {
+    Conv3Variant v;
+    v.split = nb == 2 && groups <= 2;
+    v.g = (groups + 3) / 4 >= 3 ? 4 : 1;
+    if (v.split) v.g = 1;
+    return v;
+}
+
 template <int NB>
 int launch_nb(const GemmProblem &p, const Conv3Launch &L, size_t lds, hipStream_t stream) {
     const int n_blocks = (p.n + 31) / 32;
     const dim3 grid((unsigned)((L.tiles + 7) / 8 * 8), (unsigned)((n_blocks + NB - 1) / NB));
-    auto launch_pc = [&](auto rowsum_c, auto qm_c, auto pc_c) {
-        auto kernel = conv3x3_patch_kernel<NB, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(pc_c)::value>;
+    const int rows = L.th < p.ho ? L.th : p.ho;
+    const Conv3Variant variant = conv3_variant((rows * p.wo + 31) / 32, NB);
+    auto launch_g = [&](auto rowsum_c, auto qm_c, auto pc_c, auto g_c, auto split_c) {
+        auto kernel = conv3x3_patch_kernel<NB, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(pc_c)::value, decltype(g_c)::value,
+                                           decltype(split_c)::value>;
         hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, p, L);
         return (int)EH_OK;
+    };
+    auto launch_pc = [&](auto rowsum_c, auto qm_c, auto pc_c) {
+        if constexpr (NB == 2) {
+            if (variant.split) return launch_g(rowsum_c, qm_c, pc_c, std::integral_constant<int, 1>{}, std::true_type{});
+        }
+        if (variant.g == 1) return launch_g(rowsum_c, qm_c, pc_c, std::integral_constant<int, 1>{}, std::false_type{});
+        return launch_g(rowsum_c, qm_c, pc_c, std::integral_constant<int, 4>{}, std::false_type{});
     };
     auto launch = [&](auto rowsum_c, auto qm_c) {
         return p.rq.pc_multiplier ? launch_pc(rowsum_c, qm_c, std::true_type{}) : launch_pc(rowsum_c, qm_c, std::false_type{});
@@ -371,8 +403,17 @@ int conv3x3_patch_prepare() {
         if (e != hipSuccess && rc == EH_OK) rc = hip_fail(e, "hipFuncSetAttribute(conv3x3_patch_kernel)");
     };
     auto each_pc = [&](auto nb_c, auto rowsum_c, auto qm_c) {
-        raise(conv3x3_patch_kernel<decltype(nb_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value, false>);
-        raise(conv3x3_patch_kernel<decltype(nb_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value, true>);
+        constexpr int NB = decltype(nb_c)::value;
+        constexpr bool RS = decltype(rowsum_c)::value;
+        constexpr int QM = decltype(qm_c)::value;
+        raise(conv3x3_patch_kernel<NB, RS, QM, false, 4, false>);
+        raise(conv3x3_patch_kernel<NB, RS, QM, true, 4, false>);
+        raise(conv3x3_patch_kernel<NB, RS, QM, false, 1, false>);
+        raise(conv3x3_patch_kernel<NB, RS, QM, true, 1, false>);
+        if constexpr (NB == 2) {
+            raise(conv3x3_patch_kernel<NB, RS, QM, false, 1, true>);
+            raise(conv3x3_patch_kernel<NB, RS, QM, true, 1, true>);
+        }
     };
     auto each_qm = [&](auto nb_c, auto rowsum_c) {
         each_pc(nb_c, rowsum_c, std::integral_constant<int, 0>{});
