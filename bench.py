@@ -180,7 +180,22 @@ def dw_workload(eden, synth, n=32, cold=False):
                 keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 144 * 28 * 28 * 9, bytes=nbytes, bound="hbm")
 
 
-def pw_workload(eden, synth, n=32, cold=False):
+def pw_workload(eden, synth, n=32, cin=24, cout=144, hw=56, cold=False):
+    """pointwise (1x1) convolution, ReLU6: BASELINE configs[2]'s expansion by default; (64, 384, 14) and (384, 64, 14) are the
+    expansion and projection of MobileNetV2's 14x14 stage"""
+    if (cin, cout, hw) != (24, 144, 56):
+        desc = eden.conv_desc(n, cin, hw, hw, cout, 1, 1, layout=eden.NHWC)
+        x = synth.fill_u8((n, hw, hw, cin), SEED + 51)
+        w = synth.fill_u8_normal((cout, cin, 1, 1), SEED + 52, 128, 40)
+        b = synth.fill_i32((cout,), SEED + 53, -1000, 1000)
+        q = eden.make_requant(0.02, 120, 0.004, 131, 0.03 * (cin / 24) ** 0.5, 4, eden.ACT_RELU6, True)
+        d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+        plan = eden.ConvPlan(desc, d_w, d_b, q)
+        nbytes = n * hw * hw * cin + cout * cin + 4 * cout + n * hw * hw * cout
+        sets = set_count(nbytes, cold)
+        bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * hw * hw * cout)) for _ in range(sets)]
+        return dict(name="pw1x1_n%d_%dto%d_%dx%d_nhwc" % (n, cin, cout, hw, hw), launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                    keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * hw * hw * cin * cout, bytes=nbytes, bound="hbm")
     desc = eden.conv_desc(n, 24, 56, 56, 144, 1, 1, layout=eden.NHWC)
     x = synth.fill_u8((n, 56, 56, 24), SEED + 51)
     w = synth.fill_u8((144, 24, 1, 1), SEED + 52)
@@ -195,26 +210,38 @@ def pw_workload(eden, synth, n=32, cold=False):
                 keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 56 * 56 * 24 * 144, bytes=nbytes, bound="hbm")
 
 
-def block_workload(eden, synth, n=32, rows=0, cols=0, cold=False):
-    """BASELINE configs[2] as one launch: pointwise 24 -> 144 (ReLU6) feeding the 3x3 stride-2 depthwise convolution
-    from LDS (eh_conv_dw_block_run); algorithmic bytes = the block's input, weights and output (the 14.45 MB expanded
-    tensor is never stored)."""
-    d1 = eden.conv_desc(n, 24, 56, 56, 144, 1, 1, layout=eden.NHWC)
-    d2 = eden.conv_desc(n, 144, 56, 56, 144, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), dm=1, layout=eden.NHWC)
-    x = synth.fill_u8((n, 56, 56, 24), SEED + 51)
-    w1, b1 = synth.fill_u8((144, 24, 1, 1), SEED + 52), synth.fill_i32((144,), SEED + 53, -1000, 1000)
-    w2, b2 = synth.fill_u8((144, 1, 3, 3), SEED + 49), synth.fill_i32((144,), SEED + 50, -1000, 1000)
+def block_workload(eden, synth, n=32, rows=0, cols=0, cold=False, cin=24, c=144, hw=56, stride=2, fused=True):
+    """A pointwise expansion cin -> c (ReLU6) feeding a 3x3 depthwise convolution.  fused: one launch, the expanded
+    tensor held in LDS (eh_conv_dw_block_run); otherwise the two stand-alone launches with the expanded tensor in
+    device memory.  The default shape is BASELINE configs[2].  Algorithmic bytes = the block's input, weights and
+    output either way (the expanded tensor is an intermediate)."""
+    ho = (hw + 2 - 3) // stride + 1
+    d1 = eden.conv_desc(n, cin, hw, hw, c, 1, 1, layout=eden.NHWC)
+    d2 = eden.conv_desc(n, c, hw, hw, c, 3, 3, stride=(stride, stride), pad=(1, 1, 1, 1), dm=1, layout=eden.NHWC)
+    x = synth.fill_u8((n, hw, hw, cin), SEED + 51)
+    w1, b1 = synth.fill_u8((c, cin, 1, 1), SEED + 52), synth.fill_i32((c,), SEED + 53, -1000, 1000)
+    w2, b2 = synth.fill_u8((c, 1, 3, 3), SEED + 49), synth.fill_i32((c,), SEED + 50, -1000, 1000)
     q1 = eden.make_requant(0.02, 120, 0.004, 131, 0.03, 17, eden.ACT_RELU6, True)
     q2 = eden.make_requant(0.03, 17, 0.006, 140, 0.025, 9, eden.ACT_RELU6, True)
     keep = [eden.DeviceBuffer(host=a) for a in (w1, b1, w2, b2)]
     pw, dw = eden.ConvPlan(d1, keep[0], keep[1], q1), eden.DwConvPlan(d2, keep[2], keep[3], q2)
-    assert eden.conv_dw_block_applies(pw, dw)
-    nbytes = n * 56 * 56 * 24 + 144 * 24 + 576 + 144 * 9 + 576 + n * 28 * 28 * 144
-    sets = set_count(nbytes, cold)
-    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 28 * 28 * 144)) for _ in range(sets)]
-    return dict(name="c3block_n%d_pw24to144_dw3x3s2_56x56_nhwc%s" % (n, "_tile%dx%d" % (rows, cols) if rows or cols else ""),
-                launch=lambda s, i: eden.conv_dw_block_run(pw, dw, bufs[i][0], bufs[i][1], q1, q2, rows, cols, stream=s),
-                keep=(bufs, keep, pw, dw), sets=sets, ops=2.0 * n * (56 * 56 * 24 * 144 + 28 * 28 * 144 * 9), bytes=nbytes, bound="hbm")
+    nbytes = n * hw * hw * cin + c * cin + 4 * c + c * 9 + 4 * c + n * ho * ho * c
+    sets = set_count(nbytes + (0 if fused else 2 * n * hw * hw * c), cold)
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * ho * ho * c)) for _ in range(sets)]
+    if fused:
+        assert eden.conv_dw_block_applies(pw, dw)
+        launch = lambda s, i: eden.conv_dw_block_run(pw, dw, bufs[i][0], bufs[i][1], q1, q2, rows, cols, stream=s)
+    else:
+        mids = [eden.DeviceBuffer(nbytes=n * hw * hw * c) for _ in range(sets)]
+        keep.append(mids)
+
+        def launch(s, i):
+            pw.run(bufs[i][0], mids[i], q1, s)
+            dw.run(mids[i], bufs[i][1], q2, s)
+    shape = "c3block_n%d" % n if (cin, c, hw, stride) == (24, 144, 56, 2) else "block_n%d" % n
+    return dict(name="%s_pw%dto%d_dw3x3s%d_%dx%d_nhwc%s%s" % (shape, cin, c, stride, hw, hw, "" if fused else "_two_launches",
+                                                             "_tile%dx%d" % (rows, cols) if rows or cols else ""),
+                launch=launch, keep=(bufs, keep, pw, dw), sets=sets, ops=2.0 * n * (hw * hw * cin * c + ho * ho * c * 9), bytes=nbytes, bound="hbm")
 
 
 def deconv_workload(eden, synth, n=8, cold=False):
@@ -233,23 +260,29 @@ def deconv_workload(eden, synth, n=8, cold=False):
                 keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 1024 * 256 * 2048, bytes=nbytes, bound="mfma")
 
 
-def mbv2_workload(eden, synth, batch=64, per_channel=False, weights="minmax", cold=False):
+def mbv2_workload(eden, synth, batch=64, per_channel=False, weights="minmax", cold=False, lanes=2, fuse_blocks="auto"):
     """BASELINE.json configs[4]: MobileNetV2-1.0 uint8 at 224x224x3, batch 64, the whole operator list per step,
     its feature maps in the library's buffer pool (liveness reuse as the reference's operator constructor does it, one
     device allocation; the network input keeps its own slot, so every step reads the same images).
     weights: "minmax" = per-tensor min/max quantized random-init weights (bytes span 0 .. 255), the configuration
     BASELINE.json names; "narrow" = N(zp, 20) bytes.  per_channel: int8 weights with one scale per output channel in
-    the convolutions.  A step streams every feature map once, more than the Infinity Cache holds (working_set)."""
+    the convolutions.  A step streams every feature map once, more than the Infinity Cache holds (working_set).
+    lanes: the step's images run as that many independent chains of batch / lanes images on streams of their own
+    (parallel branches of the replayed graph; 1 = one chain of full-batch launches).  fuse_blocks: "auto" runs the
+    expansion + depthwise pairs the library's measured table prefers as one launch each, () none."""
     mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
     # residual adds inside the projection convolutions' launches
-    net = mobilenet.MobileNetV2(eden, batch, fuse_add=True, per_channel=per_channel, weights=weights, pooled=True)
+    net = mobilenet.MobileNetV2(eden, batch, fuse_add=True, per_channel=per_channel, weights=weights, pooled=True, lanes=lanes,
+                                fuse_blocks=fuse_blocks)
     net.set_input(mobilenet.network_input(batch))
-    name = "mobilenet_v2_1.0_224_u8%s%s_batch%d" % ("_perchannel_w" if per_channel else "", "" if weights == "minmax" else "_narrow_w", batch)
+    name = "mobilenet_v2_1.0_224_u8%s%s_batch%d%s%s" % ("_perchannel_w" if per_channel else "", "" if weights == "minmax" else "_narrow_w", batch,
+                                                       "_%dlanes" % net.lanes if net.lanes > 1 else "",
+                                                       "_%dfused_blocks" % len(net.fused_blocks) if net.fused_blocks else "")
     return dict(name=name, launch=lambda s, i: net.run(s), keep=net, sets=1, net=net,
                 ops=2.0 * mobilenet.macs_per_image() * batch, bytes=mobilenet.compulsory_bytes_per_image() * batch,
                 bound="hbm", images=batch, chunk=4, per_channel=per_channel, weights=weights,
-                working_set=sum(batch * t["h"] * t["w"] * t["c"] for i, t in enumerate(net.tensors) if i not in net.unwritten),
-                pool_bytes=net.pool_bytes)
+                working_set=sum(batch * t["h"] * t["w"] * t["c"] for i, t in enumerate(net.tensors) if i not in net.unwritten and i not in net.in_lds),
+                pool_bytes=net.pool_bytes, lanes=net.lanes, fused_blocks=list(net.fused_blocks))
 
 
 def mbv2_userdriver(eden, batch=64, per_channel=False, list_id=0xC5):
@@ -438,8 +471,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the oracle check of the network")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2, mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, copy, tonhwc, tonchw")
-    ap.add_argument("--tile", default=None, help="with --only c3block: ROWSxCOLS output pixels per workgroup (default: chosen by the library)")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2 (two lanes, measured pairs fused), mbv2plain / mbv2lanes / mbv2fused (neither / lanes only / fusion only), mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, copy, tonhwc, tonchw")
+    ap.add_argument("--tile", default=None, help="with --only c3block / block:...: ROWSxCOLS output pixels per workgroup (default: chosen by the library)")
     ap.add_argument("--cold", action="store_true", help="with --only: rotate over buffer sets that together exceed the Infinity Cache")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -459,12 +492,15 @@ def main():
 
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
                     fcbig=shaped(fc_workload, m=8192, k=4096, n=4096), conv64=shaped(conv_workload, n=64),
-                    c3block=block_workload,
+                    c3block=block_workload, pw14=shaped(pw_workload, n=64, cin=64, cout=384, hw=14), pj14=shaped(pw_workload, n=64, cin=384, cout=64, hw=14),
+                    pw7=shaped(pw_workload, n=64, cin=160, cout=960, hw=7), pj7=shaped(pw_workload, n=64, cin=960, cout=160, hw=7),
                     c3blockbig=shaped(block_workload, n=256),
                     dwbig=shaped(dw_workload, n=256), pwbig=shaped(pw_workload, n=256),
                     copy=copy_workload, mbv2=mbv2_workload, mbv2narrow=shaped(mbv2_workload, weights="narrow"),
                     tonhwc=layout_workload, tonchw=shaped(layout_workload, to_nhwc=False),
                     mbv2pc=shaped(mbv2_workload, per_channel=True),
+                    mbv2plain=shaped(mbv2_workload, lanes=1, fuse_blocks=()), mbv2lanes=shaped(mbv2_workload, fuse_blocks=()),
+                    mbv2fused=shaped(mbv2_workload, lanes=1),
                     stream16=stream_workload, stream16big=shaped(stream_workload, out_bytes=256 * 56 * 56 * 144),
                     stream41=shaped(stream_workload, mode=2, out_bytes=32 * 28 * 28 * 144),
                     stream41big=shaped(stream_workload, mode=2, out_bytes=256 * 28 * 28 * 144))
@@ -479,10 +515,15 @@ def main():
                               ms_per_step=wall / steps * 1e3, us_per_step_by_events=ev / steps * 1e6, timed_region_repeats=reps,
                               images_per_s=round(64 * steps / wall, 1), executor=driver.stats(list_id))))
         return
+    rows, cols = (int(v) for v in args.tile.split("x")) if args.tile else (0, 0)
     if args.only and args.tile:
-        rows, cols = (int(v) for v in args.tile.split("x"))
         families["c3block"] = shaped(block_workload, rows=rows, cols=cols)
         families["c3blockbig"] = shaped(block_workload, n=256, rows=rows, cols=cols)
+    if args.only and args.only.startswith(("block:", "twolaunch:")):
+        # block:N,CIN,C,HW,STRIDE = that expansion + 3x3 depthwise pair as one launch; twolaunch: the same as two launches
+        kind, _, spec = args.only.partition(":")
+        n, cin, c, hw, stride = (int(v) for v in spec.split(","))
+        families[args.only] = shaped(block_workload, n=n, cin=cin, c=c, hw=hw, stride=stride, rows=rows, cols=cols, fused=kind == "block")
     if args.only:
         work = families[args.only](eden, synth, cold=args.cold)
         args.steps = round_steps(args.steps, work["sets"], work.get("chunk", 50))
@@ -540,6 +581,8 @@ def main():
                   images_per_s=round(net["images"] * 40 / wall2, 1), checked_against_oracle=not args.no_cpu)
         c5["roofline"]["buffers"] = "one step streams %.0f MB of feature maps (each written once and read by the next operators) through a pool of %.0f MB" % (net["working_set"] / 1e6, net["pool_bytes"] / 1e6)
         c5["pool_bytes"] = net["pool_bytes"]
+        c5["schedule"] = ("%d lanes of %d images on streams of their own, parallel branches of one graph; expansion + depthwise pairs run as one launch "
+                          "(expanded tensor in LDS) at operators %s, chosen by eh_conv_dw_block_preferred" % (net["lanes"], net["images"] // net["lanes"], net["fused_blocks"]))
         # the same network built by OperationConstructor from an operator-list description and run by OperationExecutor
         if not use_graph:
             via_api[0].set_replay(False)

@@ -74,6 +74,7 @@ EXPORTS = {
                                        C.c_void_p]),
     "eh_conv2d_u8_fuses_add": (C.c_int, [C.c_void_p]),
     "eh_conv_dw_block_applies": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eh_conv_dw_block_preferred": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eh_conv_dw_block_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(Requant), C.c_int32,
                                        C.c_int32, C.c_void_p]),
     "eh_conv2d_u8_run_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),
@@ -135,6 +136,7 @@ EXPORTS = {
     "eh_deconv2d_u8_destroy": (C.c_int, [C.c_void_p]),
     "eh_event_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "eh_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eh_stream_wait_event": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eh_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "eh_event_destroy": (C.c_int, [C.c_void_p]),
 }
@@ -287,6 +289,21 @@ class DeviceBuffer:
             pass
 
 
+class BufferView:
+    """`base` (a DeviceBuffer or a PooledBuffer) from byte `offset` on; owns nothing."""
+
+    def __init__(self, base, offset):
+        self.base, self.offset = base, int(offset)
+
+    @property
+    def ptr(self):
+        return C.c_void_p(self.base.ptr.value + self.offset)
+
+    @property
+    def nbytes(self):
+        return self.base.nbytes - self.offset
+
+
 POOL_INTER_NEW, POOL_INTER_REUSE, POOL_INTRA = 0, 1, 2
 
 
@@ -321,6 +338,11 @@ class PooledBuffer:
 def conv_dw_block_applies(pointwise, depthwise):
     """whether a ConvPlan (1x1) and the DwConvPlan on its output can run as one launch"""
     return bool(load().eh_conv_dw_block_applies(pointwise.handle, depthwise.handle))
+
+
+def conv_dw_block_preferred(pw, dw):
+    """True when the fused launch is also the faster choice for the pair's shape (the library's measured table)."""
+    return bool(load().eh_conv_dw_block_preferred(pw.handle, dw.handle))
 
 
 def conv_dw_block_run(pointwise, depthwise, d_in, d_out, q_pointwise, q_depthwise, rows_per_tile=0, cols_per_tile=0, stream=None):
@@ -481,6 +503,10 @@ class Event:
 
     def record(self, stream=None):
         check(load().eh_event_record(self.h, stream))
+
+    def wait_on(self, stream=None):
+        """Makes later work on `stream` (a raw handle or None) wait for what this event recorded."""
+        check(load().eh_stream_wait_event(stream, self.h))
 
     def elapsed_ms_since(self, start):
         ms = C.c_float()

@@ -764,6 +764,12 @@ int eh_event_record(void *event, void *stream) {
     return EH_OK;
 }
 
+int eh_stream_wait_event(void *stream, void *event) {
+    EH_REQUIRE(event != nullptr, "null event");
+    EH_HIP(hipStreamWaitEvent(as_stream(stream), reinterpret_cast<hipEvent_t>(event), 0));
+    return EH_OK;
+}
+
 int eh_event_elapsed_ms(void *start, void *stop, float *ms) {
     EH_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(stop)));
     EH_HIP(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop)));
@@ -1530,6 +1536,14 @@ int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan
     const GemmProblem pw = op.problem(op.parts[0], nullptr, nullptr, nullptr, nullptr);
     const DwProblem dw = dw_problem(depthwise, nullptr, nullptr);
     return pwdw_block_applies(pw, dw) ? 1 : 0;
+}
+
+int eh_conv_dw_block_preferred(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise) {
+    if (!eh_conv_dw_block_applies(pointwise, depthwise)) return 0;
+    const GemmOp &op = pointwise->op;
+    const GemmProblem pw = op.problem(op.parts[0], nullptr, nullptr, nullptr, nullptr);
+    const DwProblem dw = dw_problem(depthwise, nullptr, nullptr);
+    return pwdw_block_preferred(pw, dw) ? 1 : 0;
 }
 
 int eh_conv_dw_block_run(eh_conv_plan *pointwise, eh_dwconv_plan *depthwise, const void *input, void *output,

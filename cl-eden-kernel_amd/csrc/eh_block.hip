@@ -19,6 +19,10 @@
 // The rows and columns two neighbouring workgroups both need (the halo) are computed twice; nothing else is.  Tiles are
 // cut in both directions because the halo of a stride-2 window costs (2 TH + 1)(2 TW + 1) / (4 TH TW): 1.53 for one full
 // row of 28 outputs, 1.21 for 4 x 7.
+// A depthwise channel needs only its own expanded channel, so the expanded channels are cut into ranges of whole
+// 32-channel blocks as well: a workgroup is (tile, channel range), which keeps its LDS image small (four or more
+// workgroups share a CU and overlap their stages) on layers with many channels; the input pixels are then staged once
+// per range, which costs little (they are the narrow side of an expansion).
 // Both stages produce bit for bit what the two stand-alone launches produce.
 #include <type_traits>
 
@@ -36,13 +40,16 @@ struct BlockGeom {
     int32_t tiles_y, tiles_w;  // workgroups per image, down and across
     int32_t ih, iwp;     // rows and columns of the expanded image a workgroup holds
     int32_t pixels;      // ih * iwp
-    int32_t c;           // expanded channels = bytes per pixel of the LDS image
-    int32_t nb;          // channel blocks of 32
+    int32_t c;           // expanded channels of the layer
+    int32_t nb;          // channel blocks of 32 per workgroup (grid y walks the ranges); bytes per pixel of the LDS image = 32 nb
+    int32_t ks;          // reduction steps of 32 bytes of the pointwise stage
+    int32_t cpitch;      // bytes per pixel of the LDS image
     int32_t tiles_x;     // depthwise tiles of four output columns per row of the workgroup's tile
-    int32_t units;       // th * tiles_x * (c / 4)
+    int32_t units_per_cq;  // th * tiles_x: depthwise thread-units per channel quad
     int32_t total_tiles; // n * tiles_y * tiles_w
-    int32_t a_pitch;     // LDS bytes per input pixel (the reduction bytes padded to 48: fragment reads spread over the banks)
-    FastDiv div_iwp, div_cq, div_tx, div_tiles_y, div_tiles_w, div_nb;
+    int32_t a_pitch;     // LDS bytes per input pixel: 32 ks + 16 (the slack spreads the fragment reads over the banks)
+    FastDiv div_iwp, div_tx, div_tiles_y, div_tiles_w, div_ppp;
+    FastDiv div_cq, div_cq_last;  // by the channel quads of a full range, and of the last one
     uint32_t a_off;      // byte offset of the staged input pixels
     uint32_t image_off;  // byte offset of the LDS image behind the staged weights, bias and input pixels
 };
@@ -61,13 +68,21 @@ __device__ __forceinline__ void column_words(uint32_t r0, uint32_t r1, uint32_t 
 
 // S: depthwise stride.  FOLD: the depthwise stage multiplies raw bytes (unsigned form, weights of any range) instead of
 // a - 128 against w - zp_w.  ROWSUM: the pointwise weights' zero point is not 128, so a pixel's byte sum enters.
-// QM: pointwise requantization, 0 two-step order, 1 / 2 the single-shift forms.
-template <int S, bool FOLD, bool ROWSUM, int QM>
+// QM: pointwise requantization, 0 two-step order, 1 / 2 the single-shift forms.  KS: reduction steps of the pointwise
+// stage when they are 1, 2 or 3 (a lane then keeps its pixel's operand bytes in registers across the channel blocks),
+// 0 for any number (read from LDS for every product).
+template <int S, bool FOLD, bool ROWSUM, int QM, int KS>
 __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, const DwProblem dw, const BlockGeom g) {
+    const int ksteps = KS ? KS : g.ks;
     extern __shared__ __align__(16) uint8_t lds_raw[];
-    v4i *b_s = reinterpret_cast<v4i *>(lds_raw);                              // [nb][64 lanes]: pointwise weights, fragment order
-    int32_t *bias_s = reinterpret_cast<int32_t *>(lds_raw + (size_t)g.nb * 1024);  // [nb * 32]
-    uint8_t *img_s = lds_raw + g.image_off;                                   // [ih][iwp][c] uint8 (xor 0x80 for the signed form)
+    v4i *b_s = reinterpret_cast<v4i *>(lds_raw);                              // [nb][ks][64 lanes]: pointwise weights, fragment order
+    int32_t *bias_s = reinterpret_cast<int32_t *>(lds_raw + (size_t)g.nb * ksteps * 1024);  // [nb * 32]
+    uint8_t *img_s = lds_raw + g.image_off;                                   // [ih][iwp][cpitch] uint8 (xor 0x80 for the signed form)
+    const int nb_first = blockIdx.y * g.nb;                                   // this workgroup's channel range
+    const int c_first = nb_first * 32;
+    const int c_here = g.c - c_first < g.nb * 32 ? g.c - c_first : g.nb * 32;  // channels of the range that exist (a multiple of 16)
+    const int nb_here = (c_here + 31) >> 5;
+    const int cpitch = g.cpitch;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, half = lane >> 5;
@@ -80,7 +95,7 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
     const int ty = (int)(t_row - img * (uint32_t)g.tiles_y);
     const int oy0 = ty * g.th, ox_first = txw * g.tw;
     const int iy_first = oy0 * S - dw.pad_t, ix_first = ox_first * S - dw.pad_l;  // image coordinates of the LDS image's corner
-    uint8_t *a_s = lds_raw + g.a_off;  // [pixels][a_pitch]: the input pixels' reduction bytes, 0x80-filled past the reduction length
+    uint8_t *a_s = lds_raw + g.a_off;  // [pixels][a_pitch]: the input pixels' reduction bytes as signed operands (a ^ 0x80), 0 past the reduction length
 
     // ---- stage 0: weights, bias and the tile's input pixels into LDS (8-byte pieces: pixels start on 8-byte boundaries)
     auto inside_image = [&](int q, int &iy, int &ix) {
@@ -90,19 +105,23 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
         return (unsigned)iy < (unsigned)pw.h && (unsigned)ix < (unsigned)pw.w;
     };
     {
-        const int pieces = g.pixels * 4;  // four 8-byte pieces per pixel (32 reduction bytes)
+        const int ppp = ksteps * 4;  // 8-byte pieces per pixel
+        const int pieces = g.pixels * ppp;
         for (int i = tid; i < pieces; i += 256) {
-            const int q = i >> 2, piece = i & 3;
+            const int q = KS ? i / (KS * 4) : (int)fastdiv((uint32_t)i, g.div_ppp), piece = i - q * ppp;
             int iy, ix;
-            uint2 v = make_uint2(pw.a_xor, pw.a_xor);  // bytes past the reduction length, and whole pixels outside the image, flip to 0
-            if (inside_image(q, iy, ix) && piece * 8 < pw.k)
+            uint2 v = make_uint2(0u, 0u);  // bytes past the reduction length, and whole pixels outside the image: operand 0
+            if (inside_image(q, iy, ix) && piece * 8 < pw.k) {
                 v = *reinterpret_cast<const uint2 *>(pw.a + (((img * (uint32_t)pw.h + (uint32_t)iy) * (uint32_t)pw.w + (uint32_t)ix) * (uint32_t)pw.cin +
                                                                (uint32_t)pw.a_offset + (uint32_t)piece * 8u));
+                v.x ^= pw.a_xor;
+                v.y ^= pw.a_xor;
+            }
             *reinterpret_cast<uint2 *>(a_s + q * g.a_pitch + piece * 8) = v;
         }
-        const v4i *src = reinterpret_cast<const v4i *>(pw.b);
-        for (int i = tid; i < g.nb * 64; i += 256) b_s[i] = src[i];
-        for (int i = tid; i < g.nb * 32; i += 256) bias_s[i] = pw.bias[i];
+        const v4i *src = reinterpret_cast<const v4i *>(pw.b) + (size_t)nb_first * ksteps * 64;
+        for (int i = tid; i < nb_here * ksteps * 64; i += 256) b_s[i] = src[i];
+        for (int i = tid; i < nb_here * 32; i += 256) bias_s[i] = pw.bias[c_first + i];
         __syncthreads();
     }
 
@@ -112,30 +131,35 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
     const int blocks = (g.pixels + 31) >> 5;
     const RequantDev rq = pw.rq;
     {
-        const int all = blocks * g.nb;
+        const int all = blocks * nb_here;
         const int first = (all * wave) >> 2, last = (all * (wave + 1)) >> 2;
-        int blk = (int)fastdiv((uint32_t)first, g.div_nb), nb = first - blk * g.nb;
+        int blk = first / nb_here, nb = first - blk * nb_here;
         int loaded = -1, ncorr = 0, q = 0;
         bool ok = false;
-        v4i af = {0, 0, 0, 0};
+        const uint8_t *arow = a_s;
+        v4i held[KS ? KS : 1];
         for (int u = first; u < last; ++u) {
-            if (blk != loaded) {  // this lane's pixel of the block: its fragment bytes, row-sum term and place in the image
+            if (blk != loaded) {  // this lane's pixel of the block: where its fragment bytes sit, its row-sum term, its place in the image
                 loaded = blk;
                 q = blk * 32 + r;
                 int iy, ix;
                 ok = q < g.pixels && inside_image(q, iy, ix);
-                const int qq = q < g.pixels ? q : g.pixels - 1;
-                const uint4 raw = *reinterpret_cast<const uint4 *>(a_s + qq * g.a_pitch + half * 16);
-                af.x = (int)(raw.x ^ pw.a_xor);
-                af.y = (int)(raw.y ^ pw.a_xor);
-                af.z = (int)(raw.z ^ pw.a_xor);
-                af.w = (int)(raw.w ^ pw.a_xor);
+                arow = a_s + (q < g.pixels ? q : g.pixels - 1) * g.a_pitch + half * 16;
+                if constexpr (KS != 0) {
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) held[ks] = *reinterpret_cast<const v4i *>(arow + ks * 32);
+                }
                 if constexpr (ROWSUM) {
-                    int rowsum = __builtin_amdgcn_sdot4(af.x, 0x01010101, 0, false);
-                    rowsum = __builtin_amdgcn_sdot4(af.y, 0x01010101, rowsum, false);
-                    rowsum = __builtin_amdgcn_sdot4(af.z, 0x01010101, rowsum, false);
-                    rowsum = __builtin_amdgcn_sdot4(af.w, 0x01010101, rowsum, false);
-                    rowsum += __shfl_xor(rowsum, 32);  // the other half of the pixel's reduction bytes
+                    int rowsum = 0;
+#pragma unroll
+                    for (int ks = 0; ks < ksteps; ++ks) {
+                        const v4i af = KS ? held[KS ? ks : 0] : *reinterpret_cast<const v4i *>(arow + ks * 32);
+                        rowsum = __builtin_amdgcn_sdot4(af.x, 0x01010101, rowsum, false);
+                        rowsum = __builtin_amdgcn_sdot4(af.y, 0x01010101, rowsum, false);
+                        rowsum = __builtin_amdgcn_sdot4(af.z, 0x01010101, rowsum, false);
+                        rowsum = __builtin_amdgcn_sdot4(af.w, 0x01010101, rowsum, false);
+                    }
+                    rowsum += __shfl_xor(rowsum, 32);  // the other half of every step's bytes
                     ncorr = -pw.zw * rowsum;
                 }
             }
@@ -149,7 +173,14 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
                 acc[gq * 4 + 2] = bb.z;
                 acc[gq * 4 + 3] = bb.w;
             }
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(b_s[nb * 64 + lane], af, acc, 0, 0, 0);
+            const v4i *bw = b_s + nb * ksteps * 64 + lane;
+            if constexpr (KS != 0) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bw[ks * 64], held[ks], acc, 0, 0, 0);
+            } else {
+                for (int ks = 0; ks < ksteps; ++ks)
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bw[ks * 64], *reinterpret_cast<const v4i *>(arow + ks * 32), acc, 0, 0, 0);
+            }
             uint32_t packed[4];
 #pragma unroll
             for (int gq = 0; gq < 4; ++gq) {
@@ -160,12 +191,12 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
                                             requant_u8(acc[gq * 4 + 2] + ncorr, rq), requant_u8(acc[gq * 4 + 3] + ncorr, rq));
                 }
             }
-            if (q < g.pixels && nb * 32 + half * 16 < g.c) {  // (c is a multiple of 16: a lane's sixteen channels exist or do not)
+            if (q < g.pixels && nb * 32 + half * 16 < c_here) {  // (channel counts are multiples of 16: a lane's sixteen channels exist or do not)
                 const uint4 v = ok ? make_uint4(packed[0] ^ flip_store, packed[1] ^ flip_store, packed[2] ^ flip_store, packed[3] ^ flip_store)
                                    : make_uint4(pad_word, pad_word, pad_word, pad_word);
-                *reinterpret_cast<uint4 *>(img_s + (uint32_t)q * (uint32_t)g.c + (uint32_t)(nb * 32 + half * 16)) = v;
+                *reinterpret_cast<uint4 *>(img_s + (uint32_t)q * (uint32_t)cpitch + (uint32_t)(nb * 32 + half * 16)) = v;
             }
-            if (++nb == g.nb) {
+            if (++nb == nb_here) {
                 nb = 0;
                 ++blk;
             }
@@ -175,11 +206,14 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
 
     // ---- stage 2: the depthwise outputs from the LDS image
     constexpr int TW = 4, IW = (TW - 1) * S + 3;  // a thread's four adjacent output pixels
-    const uint32_t cq_count = (uint32_t)g.c >> 2;
+    const uint32_t cq_count = (uint32_t)c_here >> 2;
+    const uint32_t units = (uint32_t)g.units_per_cq * cq_count;
+    const uint32_t cq_first = (uint32_t)c_first >> 2;
     const RequantDev drq = dw.rq;
-    for (uint32_t u = (uint32_t)tid; u < (uint32_t)g.units; u += 256u) {
-        const uint32_t t = fastdiv(u, g.div_cq);
-        const uint32_t cq = u - t * cq_count;
+    const FastDiv div_cq = blockIdx.y + 1 == gridDim.y ? g.div_cq_last : g.div_cq;
+    for (uint32_t u = (uint32_t)tid; u < units; u += 256u) {
+        const uint32_t t = fastdiv(u, div_cq);
+        const uint32_t cql = u - t * cq_count, cq = cq_first + cql;  // channel quad within the range, and in the layer
         const uint32_t row = fastdiv(t, g.div_tx);
         const int tx = (int)(t - row * (uint32_t)g.tiles_x);
         const int oy = oy0 + (int)row, lx0 = tx * TW, ox0 = ox_first + lx0;  // lx0: first column within the workgroup's tile
@@ -191,7 +225,7 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
             for (int x = 0; x < IW; ++x) {
                 int col = lx0 * S + x;
                 col = col < g.iwp ? col : g.iwp - 1;  // columns past the last window belong to outputs that are not stored
-                in[ky][x] = *reinterpret_cast<const uint32_t *>(img_s + (((int)row * S + ky) * g.iwp + col) * g.c + (int)cq * 4);
+                in[ky][x] = *reinterpret_cast<const uint32_t *>(img_s + (((int)row * S + ky) * g.iwp + col) * cpitch + (int)cql * 4);
             }
         int4 wk[3];
 #pragma unroll
@@ -245,23 +279,30 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
 
 constexpr size_t kBlockLdsMax = 150 * 1024;
 
-constexpr int kAPitch = 48;
+// Bytes per pixel of the LDS image for `nb` channel blocks of a layer of c channels: the channels of the widest range,
+// stretched where needed so that the pitch in words is an odd multiple of four (stage 1 writes sixteen bytes per lane
+// for 32 consecutive pixels; at an even multiple of four words those writes meet in a quarter of the banks).
+int block_image_pitch(int nb, int c) {
+    int words = (nb * 32 < c ? nb * 32 : c) / 4;
+    if ((words & 7) == 0) words += 4;
+    return words * 4;
+}
 
-size_t block_lds_bytes(int nb, int ih, int iwp, int c, uint32_t *a_off, uint32_t *image_off) {
-    const size_t head = ((size_t)nb * 1024 + (size_t)nb * 128 + 15) & ~(size_t)15;
-    const size_t a_bytes = ((size_t)ih * iwp * kAPitch + 15) & ~(size_t)15;
+size_t block_lds_bytes(int nb, int ks, int ih, int iwp, int c, uint32_t *a_off, uint32_t *image_off) {
+    const size_t head = ((size_t)nb * ks * 1024 + (size_t)nb * 128 + 15) & ~(size_t)15;
+    const size_t a_bytes = ((size_t)ih * iwp * (ks * 32 + 16) + 15) & ~(size_t)15;
     if (a_off) *a_off = (uint32_t)head;
     if (image_off) *image_off = (uint32_t)(head + a_bytes);
-    return head + a_bytes + (size_t)ih * iwp * c;
+    return head + a_bytes + (size_t)ih * iwp * block_image_pitch(nb, c);
 }
 
 }  // namespace
 
-// The pointwise problem is a one-tap problem of a single 32-byte reduction step on whole dense images, the depthwise
-// one a 3x3 channels-last layer of stride 1 or 2 on the pointwise output with the 8-bit dot product weights at hand;
-// uint8 tensors and one requantization pair per operator.
+// The pointwise problem is a one-tap problem of at most eight 32-byte reduction steps on whole dense images whose
+// weights are packed in fragment order, the depthwise one a 3x3 channels-last layer of stride 1 or 2 on the pointwise
+// output with the 8-bit dot product weights at hand; uint8 tensors and one requantization pair per operator.
 bool pwdw_block_applies(const GemmProblem &pw, const DwProblem &dw) {
-    if (pw.cfg.id != GEMM_THIN || pw.k_pad != 32 || pw.k > 32 || (pw.k & 7) != 0 || (pw.cin & 7) != 0) return false;
+    if (pw.cfg.id != GEMM_THIN || pw.k_pad > 256 || pw.k > pw.k_pad || (pw.k & 7) != 0 || (pw.cin & 7) != 0 || pw.k != pw.cin) return false;
     if (pw.stride_h != 1 || pw.stride_w != 1 || pw.y_base != 0 || pw.x_base != 0 || pw.ho != pw.h || pw.wo != pw.w) return false;
     if (pw.a_xor != 0x80808080u || pw.out_xor != 0u || pw.rq.pc_multiplier || pw.residual) return false;
     if (dw.kh != 3 || dw.kw != 3 || dw.dil_h != 1 || dw.dil_w != 1 || dw.stride_h != dw.stride_w || (dw.stride_h != 1 && dw.stride_h != 2)) return false;
@@ -269,7 +310,30 @@ bool pwdw_block_applies(const GemmProblem &pw, const DwProblem &dw) {
     if (dw.io_flip || dw.rq.pc_multiplier || (!dw.w_trip && !dw.w_fold)) return false;
     if (dw.pad_t < 0 || dw.pad_l < 0 || dw.pad_t > 2 || dw.pad_l > 2) return false;
     if ((size_t)dw.n * dw.h * dw.w_ * pw.cin >= (1ull << 31) || (size_t)dw.n * dw.ho * dw.wo * dw.cout >= (1ull << 31)) return false;
-    return block_lds_bytes((dw.c + 31) / 32, 3, 3 * dw.stride_w + 3, dw.c, nullptr, nullptr) <= kBlockLdsMax;  // one row of four outputs
+    return block_lds_bytes(1, pw.k_pad / 32, 3, 3 * dw.stride_w + 3, dw.c, nullptr, nullptr) <= kBlockLdsMax;  // one row of four outputs, one channel block
+}
+
+// Whether the one launch beats the two.  The fused kernel computes the expanded pixels of a tile's halo twice and
+// requantizes every expanded value on the vector ALU just as the stand-alone kernels do, so what it saves is the
+// expanded tensor's trip through memory and one launch; whether that pays depends on the shape, and the answer here
+// is a table of the shapes that were timed inside a network (MobileNetV2 at 224 x 224, 32 images per launch, each
+// pair switched to the fused kernel on its own; microseconds per network pass against 445):
+//   image  in -> expanded  stride   change        image  in -> expanded  stride   change
+//   112     16 ->  96        2      +2.1           14    64 -> 384         1      -5.5 / -3.2 / -3.7 / -1.1
+//    56     24 -> 144        1      +1.6           14    96 -> 576         1      +0.7 / +2.4
+//    56     24 -> 144        2      -7.6           14    96 -> 576         2      +0.4
+//    28     32 -> 192        1      -1.9 / -1.2     7   160 -> 960         1      +1.6 / +1.9 / +1.6
+//    28     32 -> 192        2      -3.4
+// A shape that is not in the table runs as two launches.
+bool pwdw_block_preferred(const GemmProblem &pw, const DwProblem &dw) {
+    if (!pwdw_block_applies(pw, dw) || dw.h != dw.w_ || dw.n < 8) return false;
+    struct Shape {
+        int32_t image, in, expanded, stride;
+    };
+    static const Shape faster[] = {{56, 24, 144, 2}, {28, 32, 192, 1}, {28, 32, 192, 2}, {14, 64, 384, 1}};
+    for (const Shape &s : faster)
+        if (dw.h == s.image && pw.k == s.in && dw.c == s.expanded && dw.stride_h == s.stride) return true;
+    return false;
 }
 
 // rows_per_tile / cols_per_tile: the tile a workgroup owns, 0 = chosen here
@@ -282,39 +346,52 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &caller_dw, int row
     const int S = dw.stride_h;
     BlockGeom g;
     g.c = dw.c;
-    g.nb = (dw.c + 31) / 32;
-    g.a_pitch = kAPitch;
-    auto lds_of = [&](int th, int tw) { return block_lds_bytes(g.nb, (th - 1) * S + 3, (tw - 1) * S + 3, g.c, nullptr, nullptr); };
-    // Tile shape.  A workgroup's three stages run one after the other, so the stages of different workgroups have to
-    // overlap on a CU: the shapes considered leave room for four or more workgroups in a CU's LDS (measured: tiles of
-    // twice that size take twice as long at a batch of 256, however little halo they recompute) and, where the problem
-    // is large enough, give the launch at least three workgroups per CU.  Among those the one that computes the fewest
-    // pixel slots wins, counting the slots that pixel blocks of 32 and output tiles of four leave empty.
-    int th = rows_per_tile, tw = cols_per_tile;
-    if (th <= 0 || tw <= 0) {
+    g.ks = pw.k_pad / 32;
+    g.a_pitch = g.ks * 32 + 16;
+    const int nb_all = (dw.c + 31) / 32;
+    // Tile shape and channel blocks per workgroup.  A workgroup's three stages run one after the other, so the stages
+    // of different workgroups have to overlap on a CU: the shapes considered leave room for four or more workgroups in
+    // a CU's LDS (measured: tiles of twice that size take twice as long at a batch of 256, however little halo they
+    // recompute) and, where the problem is large enough, give the launch at least three workgroups per CU.  Among those
+    // the one that computes the fewest pixel slots wins, counting the slots that pixel blocks of 32 and output tiles of
+    // four leave empty and, at a lower weight, the input bytes staged again for every channel range.
+    int th = rows_per_tile, tw = cols_per_tile, nb = nb_all;
+    {
         double best = -1;
-        int best_th = 1, best_tw = dw.wo < 4 ? dw.wo : 4;
-        for (int pass = 0; pass < 2 && best < 0; ++pass)  // second pass: any workgroup count
-            for (int ch = 1; ch <= dw.ho && ch <= 16; ++ch)
-                for (int cw = 1; cw <= dw.wo && cw <= 64; ++cw) {
-                    if (th > 0 && ch != th) continue;
-                    if (tw > 0 && cw != tw) continue;
-                    if (lds_of(ch, cw) * 4 > 144 * 1024 && !(ch == 1 && cw <= 4)) continue;
-                    const long wgs = (long)dw.n * ((dw.ho + ch - 1) / ch) * ((dw.wo + cw - 1) / cw);
-                    if (pass == 0 && wgs < 768) continue;
-                    const int px = ((ch - 1) * S + 3) * ((cw - 1) * S + 3);
-                    const double stage1 = (double)((px + 31) / 32 * 32) * wgs;                          // expanded pixels computed, block slots included
-                    const double stage2 = (double)ch * ((cw + 3) / 4 * 4) * wgs;                        // output pixels computed, tile slots included
-                    const double cost = stage1 / ((double)dw.n * dw.h * dw.w_) + 0.5 * stage2 / ((double)dw.n * dw.ho * dw.wo);
-                    if (best < 0 || cost < best) {
-                        best = cost;
-                        best_th = ch;
-                        best_tw = cw;
+        int best_th = 1, best_tw = dw.wo < 4 ? dw.wo : 4, best_nb = 1;
+        for (int pass = 0; pass < 3 && best < 0; ++pass)  // later passes: fewer workgroups, then anything that fits at all
+            for (int cn = 1; cn <= nb_all; ++cn) {
+                const int ranges = (nb_all + cn - 1) / cn;
+                if ((ranges - 1) * cn >= nb_all) continue;  // the same ranges with fewer blocks each
+                for (int ch = 1; ch <= dw.ho && ch <= 16; ++ch)
+                    for (int cw = 1; cw <= dw.wo && cw <= 64; ++cw) {
+                        if (rows_per_tile > 0 && ch != rows_per_tile) continue;
+                        if (cols_per_tile > 0 && cw != cols_per_tile) continue;
+                        const int ih = (ch - 1) * S + 3, iw = (cw - 1) * S + 3;
+                        const size_t lds = block_lds_bytes(cn, g.ks, ih, iw, dw.c, nullptr, nullptr);
+                        if (pass < 2 ? lds * 4 > 144 * 1024 : lds > kBlockLdsMax) continue;
+                        const long wgs = (long)dw.n * ((dw.ho + ch - 1) / ch) * ((dw.wo + cw - 1) / cw) * ranges;
+                        if (pass == 0 && wgs < 768) continue;
+                        const int px = ih * iw;
+                        const double tiles = (double)dw.n * ((dw.ho + ch - 1) / ch) * ((dw.wo + cw - 1) / cw);
+                        const double stage1 = (double)((px + 31) / 32 * 32) * tiles / ((double)dw.n * dw.h * dw.w_);   // pixel slots computed per real pixel
+                        const double stage2 = (double)ch * ((cw + 3) / 4 * 4) * tiles / ((double)dw.n * dw.ho * dw.wo);  // output slots per real output
+                        const double restage = (double)px * tiles * ranges * (g.ks * 32) / ((double)dw.n * dw.h * dw.w_ * dw.c);  // staged input bytes per expanded byte
+                        const double cost = stage1 + 0.5 * stage2 + 2.0 * restage;
+                        if (best < 0 || cost < best) {
+                            best = cost;
+                            best_th = ch;
+                            best_tw = cw;
+                            best_nb = cn;
+                        }
                     }
-                }
+            }
+        EH_REQUIRE(best >= 0, "block: no tile of the requested shape fits LDS");
         th = best_th;
         tw = best_tw;
+        nb = best_nb;
     }
+    g.nb = nb;
     EH_REQUIRE(th >= 1 && th <= dw.ho && tw >= 1 && tw <= dw.wo, "block: tile of %d x %d outputs", th, tw);
     g.th = th;
     g.tw = tw;
@@ -325,19 +402,22 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &caller_dw, int row
     g.tiles_y = (dw.ho + th - 1) / th;
     g.tiles_w = (dw.wo + tw - 1) / tw;
     g.total_tiles = dw.n * g.tiles_y * g.tiles_w;
-    g.units = th * g.tiles_x * (g.c >> 2);
+    g.units_per_cq = th * g.tiles_x;
     g.div_iwp = make_fastdiv((uint32_t)g.iwp);
-    g.div_cq = make_fastdiv((uint32_t)(g.c >> 2));
     g.div_tx = make_fastdiv((uint32_t)g.tiles_x);
     g.div_tiles_y = make_fastdiv((uint32_t)g.tiles_y);
     g.div_tiles_w = make_fastdiv((uint32_t)g.tiles_w);
-    g.div_nb = make_fastdiv((uint32_t)g.nb);
-    const size_t lds = block_lds_bytes(g.nb, g.ih, g.iwp, g.c, &g.a_off, &g.image_off);
+    g.div_ppp = make_fastdiv((uint32_t)(g.ks * 4));
+    const int ranges = (nb_all + g.nb - 1) / g.nb;
+    g.div_cq = make_fastdiv((uint32_t)(g.nb * 8 < g.c / 4 ? g.nb * 8 : g.c / 4));
+    g.div_cq_last = make_fastdiv((uint32_t)((g.c - (ranges - 1) * g.nb * 32) / 4));
+    g.cpitch = block_image_pitch(g.nb, g.c);
+    const size_t lds = block_lds_bytes(g.nb, g.ks, g.ih, g.iwp, g.c, &g.a_off, &g.image_off);
     EH_REQUIRE(lds <= kBlockLdsMax, "block: %zu bytes of LDS", lds);
     if (g.total_tiles <= 0) return EH_OK;
-    const dim3 grid((unsigned)((g.total_tiles + 7) / 8 * 8));
-    auto launch = [&](auto s_c, auto fold_c, auto rowsum_c, auto qm_c) {
-        auto kernel = pwdw_block_kernel<decltype(s_c)::value, decltype(fold_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value>;
+    const dim3 grid((unsigned)((g.total_tiles + 7) / 8 * 8), (unsigned)ranges);
+    auto launch = [&](auto s_c, auto fold_c, auto rowsum_c, auto qm_c, auto ks_c) {
+        auto kernel = pwdw_block_kernel<decltype(s_c)::value, decltype(fold_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(ks_c)::value>;
         if (lds > 64 * 1024) {
             // (a driver call, made per launch of the tall-tile shapes only; the default tile height stays below 64 KiB)
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlockLdsMax);
@@ -346,10 +426,16 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &caller_dw, int row
         hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, pw, dw, g);
         return (int)EH_OK;
     };
+    auto with_ks = [&](auto s_c, auto fold_c, auto rowsum_c, auto qm_c) {
+        if (g.ks == 1) return launch(s_c, fold_c, rowsum_c, qm_c, std::integral_constant<int, 1>{});
+        if (g.ks == 2) return launch(s_c, fold_c, rowsum_c, qm_c, std::integral_constant<int, 2>{});
+        if (g.ks == 3) return launch(s_c, fold_c, rowsum_c, qm_c, std::integral_constant<int, 3>{});
+        return launch(s_c, fold_c, rowsum_c, qm_c, std::integral_constant<int, 0>{});
+    };
     auto with_qm = [&](auto s_c, auto fold_c, auto rowsum_c) {
-        if (pw.rq.fast == 2) return launch(s_c, fold_c, rowsum_c, std::integral_constant<int, 2>{});
-        if (pw.rq.fast == 1) return launch(s_c, fold_c, rowsum_c, std::integral_constant<int, 1>{});
-        return launch(s_c, fold_c, rowsum_c, std::integral_constant<int, 0>{});
+        if (pw.rq.fast == 2) return with_ks(s_c, fold_c, rowsum_c, std::integral_constant<int, 2>{});
+        if (pw.rq.fast == 1) return with_ks(s_c, fold_c, rowsum_c, std::integral_constant<int, 1>{});
+        return with_ks(s_c, fold_c, rowsum_c, std::integral_constant<int, 0>{});
     };
     auto with_rowsum = [&](auto s_c, auto fold_c) {
         return pw.zw != 0 ? with_qm(s_c, fold_c, std::true_type{}) : with_qm(s_c, fold_c, std::false_type{});

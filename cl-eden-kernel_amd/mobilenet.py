@@ -257,9 +257,18 @@ class MobileNetV2:
     (gpu_op_constructor.cc:2157-2191): an operator's output is requested with INTER_SHARED_REUSE, then the inputs it
     is the last reader of are handed back, and once the list is built one device allocation holds them all
     (`pool_bytes`).  A feature map's storage is then taken over by later ones (the network input is kept), so only
-    the input and the logits can be read back after a run; without it every tensor keeps a buffer of its own (`tensor()` works for all)."""
+    the input and the logits can be read back after a run; without it every tensor keeps a buffer of its own (`tensor()` works for all).
 
-    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False, per_channel=False, weights="minmax", pooled=False):
+    lanes, lane_from, lane_to: operators lane_from .. lane_to - 1 (default: all) run as `lanes` independent chains, each
+    on its own share of the images (the batch is the outermost dimension, so a share is a contiguous slice of every
+    tensor), with its own feature maps, and on its own stream, forked from the caller's stream and joined to it again.
+    A launch ends in a tail during which most CUs idle and the next one takes a while to fill them; two chains fill
+    those gaps for one another (measured at batch 64: 490 -> 444 us per step with two lanes over the whole list, four
+    lanes of 16 images lose more in the smaller launches than they gain).  Captured in a
+    graph the chains become parallel branches.  Same plans, same kernels, same results."""
+
+    def __init__(self, eden, batch, image=224, stream=None, fuse_add=False, per_channel=False, weights="minmax", pooled=False,
+                 lanes=1, lane_from=None, lane_to=None, fuse_blocks=()):
         self.eden, self.batch, self.image = eden, batch, image
         self.tensors, self.ops = layers(image, weights)
         self.steps = []
@@ -277,48 +286,21 @@ class MobileNetV2:
                 if (op["op"] == "add" and index > 0 and self.ops[index - 1]["op"] == "conv" and self.ops[index - 1]["dst"] == op["b"]
                         and readers.get(op["b"], 0) == 1):
                     self.unwritten.add(op["b"])
-        size = lambda i: batch * self.tensors[i]["h"] * self.tensors[i]["w"] * self.tensors[i]["c"]
-        if pooled:
-            self.pool = eden.BufferPool()
-            self.buffers = [None] * len(self.tensors)
-            self.buffers[0] = self.pool.request(eden.POOL_INTER_NEW, size(0))
-            left = dict(readers)
-            left[0] += 1   # the network input keeps its storage, so that a replay reads the same image again
-            for index, op in enumerate(self.ops):
-                if op["dst"] in self.unwritten:
-                    continue   # its reads happen in the add's launch, which is where its inputs are handed back
-                self.buffers[op["dst"]] = self.pool.request(eden.POOL_INTER_REUSE, size(op["dst"]))
-                reads = [op[k] for k in ("src", "a", "b") if k in op and op[k] not in self.unwritten]
-                if op["op"] == "add" and op["b"] in self.unwritten:
-                    reads.append(self.ops[index - 1]["src"])   # the fused launch reads the projection's input
-                for t in reads:
-                    left[t] -= 1
-                    if left[t] == 0:
-                        self.pool.reset_inter(self.buffers[t])
-            self.pool_bytes = self.pool.assign()
-        else:
-            self.buffers = [eden.DeviceBuffer(nbytes=size(i)) for i in range(len(self.tensors))]
-            self.pool_bytes = None
-        for index, op in enumerate(self.ops):
+        lane_to = len(self.ops) if lane_to is None else lane_to
+        lane_from = lane_to if lanes <= 1 else (0 if lane_from is None else lane_from)
+        lanes = lanes if lane_from < lane_to else 1
+        assert batch % lanes == 0 and 0 <= lane_from <= lane_to <= len(self.ops)
+        for edge in (lane_from, lane_to):   # a fused add stays with its convolution
+            assert edge == len(self.ops) or self.ops[edge]["op"] != "add" or self.ops[edge]["b"] not in self.unwritten
+        sub = batch // lanes
+        plans = {}  # (operator index, images) -> (plan, requantization): lanes share their plans
+
+        def plan_of(index, n):
+            if (index, n) in plans:
+                return plans[(index, n)]
+            op = self.ops[index]
             kind = op["op"]
-            if kind == "add":
-                prev = self.steps[-1] if self.steps else None
-                if (fuse_add and prev and prev[0] == "plan" and self.ops[index - 1]["op"] == "conv" and
-                        self.ops[index - 1]["dst"] == op["b"] and readers.get(op["b"], 0) == 1):
-                    a, b, d = (self.tensors[op[k]] for k in ("a", "b", "dst"))
-                    q_add = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
-                    plan, src, _, q = prev[1]
-                    self.steps[-1] = ("plan_add", (plan, src, self.buffers[op["a"]], self.buffers[op["dst"]], q, q_add))
-                    continue
-                a, b, d = (self.tensors[op[k]] for k in ("a", "b", "dst"))
-                q = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
-                count = batch * d["h"] * d["w"] * d["c"]
-                self.steps.append(("add", (self.buffers[op["a"]], self.buffers[op["b"]], self.buffers[op["dst"]], count, q)))
-                continue
             s, d = self.tensors[op["src"]], self.tensors[op["dst"]]
-            if kind == "avgpool":
-                self.steps.append(("avgpool", (self.buffers[op["src"]], self.buffers[op["dst"]], s, op["k"])))
-                continue
             act = eden.ACT_RELU6 if op.get("relu6") else eden.ACT_NONE
             pairs = None
             if per_channel and kind != "fc":
@@ -333,20 +315,139 @@ class MobileNetV2:
             d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
             self._keep += [d_w, d_b]
             if kind == "fc":
-                plan = eden.FcPlan(batch, s["c"], op["cout"], d_w, d_b, q, stream)
+                plan = eden.FcPlan(n, s["c"], op["cout"], d_w, d_b, q, stream)
             else:
-                pad = (op["pad"],) * 4
-                if kind == "dw":
-                    desc = eden.conv_desc(batch, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, pad,
-                                          (1, 1), 1, 1, eden.NHWC, w_layout)
-                    plan = eden.DwConvPlan(desc, d_w, d_b, q, stream)
-                else:
-                    desc = eden.conv_desc(batch, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, pad,
-                                          (1, 1), 1, 1, eden.NHWC, w_layout)
-                    plan = eden.ConvPlan(desc, d_w, d_b, q, stream)
+                desc = eden.conv_desc(n, s["c"], s["h"], s["w"], op["cout"], op["k"], op["k"], (op["stride"],) * 2, (op["pad"],) * 4,
+                                      (1, 1), 1, 1, eden.NHWC, w_layout)
+                plan = (eden.DwConvPlan if kind == "dw" else eden.ConvPlan)(desc, d_w, d_b, q, stream)
                 if pairs:
                     plan.set_perchannel(*pairs)
-            self.steps.append(("plan", (plan, self.buffers[op["src"]], self.buffers[op["dst"]], q)))
+            plans[(index, n)] = (plan, q)
+            return plans[(index, n)]
+
+        in_lane = lambda index: lane_from <= index < lane_to
+        # An expansion (1x1 convolution, ReLU6) and the 3x3 depthwise convolution behind it as one launch, the expanded
+        # tensor in LDS only: fuse_blocks is "auto" (wherever the library's measured table prefers it for the shape and
+        # the images a launch covers) or the operator indices of the expansions to fuse.
+        self.in_lds = set()   # expanded tensors that are never stored
+        self.fused_blocks = []
+        for index in range(len(self.ops) - 1):
+            op, nxt = self.ops[index], self.ops[index + 1]
+            if not (op["op"] == "conv" and op["k"] == 1 and nxt["op"] == "dw" and nxt["src"] == op["dst"] and readers[op["dst"]] == 1
+                    and in_lane(index) == in_lane(index + 1)) or per_channel or not fuse_blocks:
+                continue
+            n = sub if in_lane(index) else batch
+            if fuse_blocks == "auto":
+                pw, dw = plan_of(index, n)[0], plan_of(index + 1, n)[0]
+                chosen = eden.conv_dw_block_preferred(pw, dw)
+            else:
+                chosen = index in fuse_blocks
+                assert not chosen or eden.conv_dw_block_applies(plan_of(index, n)[0], plan_of(index + 1, n)[0])
+            if chosen:
+                self.in_lds.add(op["dst"])
+                self.fused_blocks.append(index)
+        size = lambda i, n=batch: n * self.tensors[i]["h"] * self.tensors[i]["w"] * self.tensors[i]["c"]
+        # Tensors the full-batch operators write live in self.buffers; those the lanes write live in the lane's own
+        # buffers, sized for its share of the images (a lane's tensors must not share storage with another lane's:
+        # the lanes are at different operators at any moment).
+        # What the lanes write and an operator after them reads is one tensor again: it lives in self.buffers and every
+        # lane writes its share of it.
+        read_after = {op[k] for op in self.ops[lane_to:] for k in ("src", "a", "b") if k in op}
+        if lane_to == len(self.ops):
+            read_after.add(len(self.tensors) - 1)   # the logits
+        made_in_lane = {op["dst"] for op in self.ops[lane_from:lane_to]} - read_after
+        self.buffers = [None] * len(self.tensors)
+        self.lane_buffers = [[None] * len(self.tensors) for _ in range(lanes if lane_from < lane_to else 0)]
+        if pooled:
+            left = dict(readers)
+            left[0] += 1   # the network input keeps its storage, so that a replay reads the same image again
+
+            def place(pool, table, first_op, last_op, n, lefts):
+                for index in range(first_op, last_op):
+                    op = self.ops[index]
+                    if op["dst"] in self.unwritten or op["dst"] in self.in_lds:
+                        continue   # its reads happen in the fused launch, which is where its inputs are handed back
+                    if table is self.buffers or op["dst"] in made_in_lane:
+                        table[op["dst"]] = pool.request(eden.POOL_INTER_REUSE, size(op["dst"], n))
+                    reads = [op[k] for k in ("src", "a", "b") if k in op and op[k] not in self.unwritten and op[k] not in self.in_lds]
+                    if op["op"] == "add" and op["b"] in self.unwritten:
+                        reads.append(self.ops[index - 1]["src"])   # the fused launch reads the projection's input
+                    if op["op"] == "dw" and op["src"] in self.in_lds:
+                        reads.append(self.ops[index - 1]["src"])   # the fused launch reads the expansion's input
+                    for t in reads:
+                        lefts[t] -= 1
+                        if lefts[t] == 0 and table[t] is not None:   # (a lane hands back only what it owns)
+                            pool.reset_inter(table[t])
+
+            self.pool = eden.BufferPool()
+            self.buffers[0] = self.pool.request(eden.POOL_INTER_NEW, size(0))
+            place(self.pool, self.buffers, 0, lane_from, batch, left)
+            # the tensors that leave the lanes are placed before the lanes start and stay until their readers are done
+            for t in sorted(read_after & {op["dst"] for op in self.ops[lane_from:lane_to]}):
+                self.buffers[t] = self.pool.request(eden.POOL_INTER_REUSE, size(t))
+            self.lane_pools = []
+            after = dict(left)
+            for table in self.lane_buffers:
+                pool = eden.BufferPool()
+                after = dict(left)
+                place(pool, table, lane_from, lane_to, sub, after)
+                self.lane_pools.append(pool)
+            place(self.pool, self.buffers, lane_to, len(self.ops), batch, after)
+            self.pool_bytes = self.pool.assign() + sum(pool.assign() for pool in self.lane_pools)
+        else:
+            for i in range(len(self.tensors)):
+                if i in self.in_lds:
+                    continue
+                if i in made_in_lane:
+                    for table in self.lane_buffers:
+                        table[i] = eden.DeviceBuffer(nbytes=size(i, sub))
+                else:
+                    self.buffers[i] = eden.DeviceBuffer(nbytes=size(i))
+            self.pool_bytes = None
+        def build(first_op, last_op, lane):
+            """The steps of operators first_op .. last_op - 1; lane: None = on the whole batch, else that lane's share"""
+            n = batch if lane is None else sub
+
+            def view(t):
+                if lane is None:
+                    return self.buffers[t]
+                if t in made_in_lane:
+                    return self.lane_buffers[lane][t]
+                return eden.BufferView(self.buffers[t], size(t, lane * sub)) if lanes > 1 else self.buffers[t]
+
+            steps = []
+            for index in range(first_op, last_op):
+                op = self.ops[index]
+                kind = op["op"]
+                if kind == "add":
+                    a, b, d = (self.tensors[op[k]] for k in ("a", "b", "dst"))
+                    q_add = eden.make_add_requant(a["scale"], a["zp"], b["scale"], b["zp"], d["scale"], d["zp"])
+                    if op["b"] in self.unwritten:
+                        assert steps and steps[-1][0] == "plan", "a fused add and its convolution belong to the same lane"
+                        plan, src, _, q = steps[-1][1]
+                        steps[-1] = ("plan_add", (plan, src, view(op["a"]), view(op["dst"]), q, q_add))
+                    else:
+                        steps.append(("add", (view(op["a"]), view(op["b"]), view(op["dst"]), n * d["h"] * d["w"] * d["c"], q_add)))
+                elif kind == "avgpool":
+                    steps.append(("avgpool", (view(op["src"]), view(op["dst"]), self.tensors[op["src"]], op["k"], n)))
+                elif kind == "dw" and op["src"] in self.in_lds:
+                    dw, q_dw = plan_of(index, n)
+                    assert steps and steps[-1][0] == "plan", "an expansion and its depthwise convolution belong to the same lane"
+                    pw, src, _, q_pw = steps[-1][1]
+                    steps[-1] = ("block", (pw, dw, src, view(op["dst"]), q_pw, q_dw))
+                else:
+                    plan, q = plan_of(index, n)
+                    steps.append(("plan", (plan, view(op["src"]), None if op["dst"] in self.unwritten or op["dst"] in self.in_lds else view(op["dst"]), q)))
+            return steps
+
+        self.steps = build(0, lane_from, None)
+        self.lane_steps = [build(lane_from, lane_to, lane) for lane in range(len(self.lane_buffers))]
+        self.tail_steps = build(lane_to, len(self.ops), None)
+        self.lanes, self.lane_from, self.lane_to = len(self.lane_buffers), lane_from, lane_to
+        # lanes beyond the first run on streams of their own, forked from and joined to the caller's
+        self.lane_streams = [eden.Stream() for _ in self.lane_steps[1:]]
+        self.fork = eden.Event()
+        self.joins = [eden.Event() for _ in self.lane_streams]
         eden.sync(stream)
 
     def set_input(self, x_nhwc):
@@ -357,9 +458,25 @@ class MobileNetV2:
         self.eden.sync()
 
     def run(self, stream=None):
-        """Enqueues every operator in order on `stream` (a raw handle or None)."""
+        """Enqueues every operator in order on `stream` (a raw handle or None); the lanes fork from it and join it."""
+        self._enqueue(self.steps, stream)
+        if not self.lane_steps:
+            return self._enqueue(self.tail_steps, stream)
+        if self.lane_streams:
+            self.fork.record(stream)
+        for side in self.lane_streams:
+            self.fork.wait_on(side.h)
+        # a lane's operators in one go (captured with the lanes' operators taking turns, four lanes replay a third slower)
+        for lane, steps in enumerate(self.lane_steps):
+            self._enqueue(steps, stream if lane == 0 else self.lane_streams[lane - 1].h)
+        for side, join in zip(self.lane_streams, self.joins):
+            join.record(side.h)
+            join.wait_on(stream)
+        self._enqueue(self.tail_steps, stream)
+
+    def _enqueue(self, steps, stream):
         eden = self.eden
-        for kind, args in self.steps:
+        for kind, args in steps:
             if kind == "plan":
                 plan, src, dst, q = args
                 plan.run(src, dst, q, stream)
@@ -369,14 +486,20 @@ class MobileNetV2:
             elif kind == "add":
                 a, b, dst, count, q = args
                 eden.add_u8(a, b, dst, count, q, stream)
+            elif kind == "block":
+                pw, dw, src, dst, q_pw, q_dw = args
+                eden.conv_dw_block_run(pw, dw, src, dst, q_pw, q_dw, stream=stream)
             else:
-                src, dst, s, k = args
-                eden.avgpool_u8(src, dst, self.batch, s["c"], s["h"], s["w"], k, k, layout=eden.NHWC, stream=stream)
+                src, dst, s, k, n = args
+                eden.avgpool_u8(src, dst, n, s["c"], s["h"], s["w"], k, k, layout=eden.NHWC, stream=stream)
 
     def tensor(self, index):
         """Downloads tensor `index` as [batch, h, w, c]."""
         t = self.tensors[index]
-        return self.buffers[index].download((self.batch, t["h"], t["w"], t["c"]))
+        if self.buffers[index] is not None:
+            return self.buffers[index].download((self.batch, t["h"], t["w"], t["c"]))
+        share = self.batch // self.lanes
+        return np.concatenate([table[index].download((share, t["h"], t["w"], t["c"])) for table in self.lane_buffers])
 
     def logits(self):
         return self.tensor(len(self.tensors) - 1).reshape(self.batch, -1)

@@ -342,11 +342,15 @@ int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
  * (gpu/gpu_op_executor.cc:56-103), the expanded tensor written by quantizedGemmBlocked and read back by
  * depthwise_conv_3x3s2_pad_merge (cl_kernels/DepthwiseconvolutionKernels.cpp:1964-2083).  Takes the two operators' own
  * plans; `_applies` says whether the pair fits (1) or has to run as two launches (0): channels-last uint8 tensors, a
- * pointwise layer of at most 32 input channels (a multiple of 8) whose output is the depthwise input, depthwise 3x3 at
+ * pointwise layer of at most 256 input channels (a multiple of 8) whose output is the depthwise input, depthwise 3x3 at
  * stride 1 or 2 without dilation or depth multiplier on a multiple of 16 channels, per-tensor requantization in both.
+ * `_preferred` says whether the one launch is also the faster choice for the pair's shape (1) or the two launches
+ * are (0): a table of shapes timed inside a network, kept beside the kernel; a caller that fuses wherever
+ * `_preferred` says so never loses to the two launches on a measured shape, and unmeasured shapes stay unfused.
  * rows_per_tile, cols_per_tile: the tile of output pixels a workgroup owns, 0 lets the library choose.
  * q_pointwise->zp_out must equal q_depthwise->zp_in (they describe the same tensor). */
 int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise);
+int eh_conv_dw_block_preferred(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise);
 int eh_conv_dw_block_run(eh_conv_plan *pointwise, eh_dwconv_plan *depthwise, const void *input, void *output,
                          const eh_requant *q_pointwise, const eh_requant *q_depthwise, int32_t rows_per_tile, int32_t cols_per_tile,
                          void *stream);
@@ -386,6 +390,9 @@ int eh_deconv2d_u8_destroy(eh_deconv_plan *plan);
 int eh_event_create(void **event);
 int eh_event_record(void *event, void *stream);
 int eh_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronises on `stop` */
+/* Work enqueued on `stream` after this call waits for what `event` recorded (hipStreamWaitEvent): the way a caller
+ * forks independent work onto a second stream and joins it again, under graph capture too. */
+int eh_stream_wait_event(void *stream, void *event);
 int eh_event_destroy(void *event);
 
 #ifdef __cplusplus

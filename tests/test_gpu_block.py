@@ -68,6 +68,13 @@ CASES = [
     (2, 28, 28, 32, 192, 2, (1, 1, 1, 1), 7, False, 119),
     (1, 6, 30, 8, 160, 1, (2, 2, 2, 2), 0, False, 133),     # padding 2: two rows and columns of zero-point pixels
     (1, 7, 5, 24, 32, 1, (0, 0, 0, 0), 0, True, 128),       # no padding; output narrower than one tile of four
+    # several 32-byte reduction steps and channel ranges per workgroup: MobileNetV2's later expansions
+    (3, 14, 14, 64, 384, 1, (1, 1, 1, 1), 0, False, 122),
+    (2, 14, 14, 96, 576, 2, (1, 1, 1, 1), 0, True, 128),
+    (4, 7, 7, 160, 960, 1, (1, 1, 1, 1), 0, False, 135),
+    (1, 28, 28, 32, 192, 2, (1, 1, 1, 1), 5, False, 128),
+    (2, 9, 10, 40, 80, 1, (1, 1, 1, 1), 4, True, 119),      # a reduction that ends inside its second step; channels not a multiple of 32
+    (1, 12, 12, 256, 48, 1, (1, 1, 1, 1), 0, False, 131),   # eight reduction steps
 ]
 
 
@@ -137,15 +144,36 @@ def test_block_config3_full_size():
 
 
 def test_block_refuses_what_it_does_not_fit():
-    d_w = eden.DeviceBuffer(host=synth.fill_u8((64, 64, 1, 1), 1))
+    d_w = eden.DeviceBuffer(host=synth.fill_u8((64, 320, 1, 1), 1))
     d_b = eden.DeviceBuffer(host=synth.fill_i32((64,), 2, -10, 10))
     d_w2 = eden.DeviceBuffer(host=synth.fill_u8((64, 1, 3, 3), 3))
     q = eden.make_requant(0.02, 3, 0.004, 120, 0.03, 5)
-    wide = eden.ConvPlan(eden.conv_desc(1, 64, 8, 8, 64, 1, 1, layout=eden.NHWC), d_w, d_b, q)   # 64 input channels: two reduction steps
+    wide = eden.ConvPlan(eden.conv_desc(1, 320, 8, 8, 64, 1, 1, layout=eden.NHWC), d_w, d_b, q)   # 320 input channels: more than eight reduction steps
     dw = eden.DwConvPlan(eden.conv_desc(1, 64, 8, 8, 64, 3, 3, pad=(1, 1, 1, 1), dm=1, layout=eden.NHWC), d_w2, d_b, q)
     assert not eden.conv_dw_block_applies(wide, dw)
-    d_x, d_o = eden.DeviceBuffer(nbytes=8 * 8 * 64), eden.DeviceBuffer(nbytes=8 * 8 * 64)
+    d_x, d_o = eden.DeviceBuffer(nbytes=8 * 8 * 320), eden.DeviceBuffer(nbytes=8 * 8 * 64)
     with pytest.raises(eden.EdenHipError):
         eden.conv_dw_block_run(wide, dw, d_x, d_o, q, q)
     wide.destroy()
     dw.destroy()
+
+
+def test_block_preferred_is_a_subset_of_applies_and_holds_config3():
+    """The measured table: BASELINE configs[2]'s pair is in it, a pair of the same family that was measured slower
+    (56 x 56 at stride 1) and an unmeasured shape are not; what does not fit is never preferred."""
+    def pair(n, cin, c, hw, stride):
+        d_w = eden.DeviceBuffer(host=synth.fill_u8((c, cin, 1, 1), 1))
+        d_b = eden.DeviceBuffer(host=synth.fill_i32((c,), 2, -10, 10))
+        d_w2 = eden.DeviceBuffer(host=synth.fill_u8((c, 1, 3, 3), 3))
+        q = eden.make_requant(0.02, 3, 0.004, 120, 0.03, 5)
+        pw = eden.ConvPlan(eden.conv_desc(n, cin, hw, hw, c, 1, 1, layout=eden.NHWC), d_w, d_b, q)
+        dw = eden.DwConvPlan(eden.conv_desc(n, c, hw, hw, c, 3, 3, stride=(stride, stride), pad=(1, 1, 1, 1), dm=1, layout=eden.NHWC), d_w2, d_b, q)
+        return pw, dw, (d_w, d_b, d_w2)
+    for shape, applies, preferred in (((32, 24, 144, 56, 2), True, True), ((32, 24, 144, 56, 1), True, False),
+                                      ((32, 40, 80, 20, 1), True, False), ((32, 64, 384, 14, 1), True, True),
+                                      ((2, 24, 144, 56, 2), True, False), ((32, 320, 64, 8, 1), False, False)):
+        pw, dw, keep = pair(*shape)
+        assert eden.conv_dw_block_applies(pw, dw) == applies, shape
+        assert eden.conv_dw_block_preferred(pw, dw) == preferred, shape
+        pw.destroy()
+        dw.destroy()

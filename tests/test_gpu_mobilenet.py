@@ -111,6 +111,61 @@ def test_mobilenet_v2_on_pooled_buffers_batch_64(per_channel):
         assert np.array_equal(got, ref), (rep, np.argwhere((got != ref).any(axis=1)).ravel().tolist())
 
 
+@pytest.mark.parametrize("pooled", [False, True], ids=["own_buffers", "pooled"])
+@pytest.mark.parametrize("lanes,lane_from,lane_to", [(2, None, None), (4, None, None), (2, 13, None), (2, 6, 50), (2, 0, 39)],
+                         ids=["two_lanes", "four_lanes", "late_lanes", "middle_lanes", "early_lanes"])
+def test_mobilenet_v2_image_lanes_and_fused_blocks_match_oracle(lanes, lane_from, lane_to, pooled):
+    """The operator list as chains of image shares on streams of their own (all of it, or a range of its operators with
+    full-batch operators before and after), with every expansion + depthwise pair the fused kernel fits run as one
+    launch: every stored tensor (own buffers) or the logits (pooled, on two replays of the captured graph) against
+    the oracle, on eight distinct images."""
+    batch = DISTINCT
+    tensors, ops, want = oracle_images(False, "minmax")
+    blocks = tuple(i for i in range(len(ops) - 1) if ops[i]["op"] == "conv" and ops[i]["k"] == 1 and ops[i + 1]["op"] == "dw")
+    assert len(blocks) == 16
+    net = mobilenet.MobileNetV2(eden, batch, 224, fuse_add=True, pooled=pooled, lanes=lanes, lane_from=lane_from, lane_to=lane_to,
+                                fuse_blocks=blocks)
+    assert net.lanes == lanes and len(net.fused_blocks) == 16 and len(net.in_lds) == 16
+    net.set_input(mobilenet.network_input(DISTINCT))
+    stream = eden.Stream()
+    graph = eden.Graph(stream, lambda s: net.run(s))
+    for rep in range(2):
+        graph.launch(stream)
+        stream.sync()
+        assert np.array_equal(net.logits(), want[-1].reshape(DISTINCT, -1)), rep
+    if not pooled:
+        for op in ops:
+            i = op["dst"]
+            if i in net.unwritten or i in net.in_lds:
+                continue
+            got = net.tensor(i).transpose(0, 3, 1, 2)
+            assert np.array_equal(got, want[i]), (op["op"], i, tensors[i], int((got != want[i]).sum()))
+    # outside a graph: the lanes' streams fork from and join the caller's
+    net.set_input(mobilenet.network_input(DISTINCT)[::-1].copy())
+    net.run(stream.h)
+    stream.sync()
+    assert np.array_equal(net.logits(), want[-1].reshape(DISTINCT, -1)[::-1])
+
+
+def test_mobilenet_v2_as_the_benchmark_runs_it_batch_64():
+    """Batch 64, pooled feature maps, two lanes of 32 images, the pairs the library's table prefers fused: the logits at
+    every batch position against the oracle's for the image that sits there."""
+    batch = 64
+    tensors, ops, want = oracle_images(False, "minmax")
+    where = scattered_batch(batch, DISTINCT)
+    net = mobilenet.MobileNetV2(eden, batch, 224, fuse_add=True, pooled=True, lanes=2, fuse_blocks="auto")
+    assert net.lanes == 2 and 4 <= len(net.fused_blocks) < 16
+    net.set_input(mobilenet.network_input(DISTINCT)[where])
+    stream = eden.Stream()
+    graph = eden.Graph(stream, lambda s: net.run(s))
+    ref = want[-1].reshape(DISTINCT, -1)[where]
+    for rep in range(2):
+        graph.launch(stream)
+        stream.sync()
+        got = net.logits()
+        assert np.array_equal(got, ref), (rep, np.argwhere((got != ref).any(axis=1)).ravel().tolist())
+
+
 def test_mobilenet_v2_graph_replay_equals_eager():
     """The whole operator list captured once; every replay (with eager work between replays) gives the eager logits."""
     batch, image = 2, 96
