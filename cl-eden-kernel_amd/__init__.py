@@ -75,6 +75,7 @@ EXPORTS = {
     "eh_conv2d_u8_fuses_add": (C.c_int, [C.c_void_p]),
     "eh_conv_dw_block_applies": (C.c_int, [C.c_void_p, C.c_void_p]),
     "eh_conv_dw_block_preferred": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "eh_conv_dw_block_listed": (C.c_int, [C.c_int32] * 6),
     "eh_conv_dw_block_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.POINTER(Requant), C.c_int32,
                                        C.c_int32, C.c_void_p]),
     "eh_conv2d_u8_run_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Requant), C.c_void_p]),

@@ -1538,6 +1538,10 @@ int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan
     return pwdw_block_applies(pw, dw) ? 1 : 0;
 }
 
+int eh_conv_dw_block_listed(int32_t images, int32_t image_h, int32_t image_w, int32_t in_channels, int32_t expanded_channels, int32_t stride) {
+    return pwdw_block_listed(images, image_h, image_w, in_channels, expanded_channels, stride) ? 1 : 0;
+}
+
 int eh_conv_dw_block_preferred(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise) {
     if (!eh_conv_dw_block_applies(pointwise, depthwise)) return 0;
     const GemmOp &op = pointwise->op;

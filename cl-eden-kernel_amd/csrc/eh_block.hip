@@ -319,21 +319,26 @@ bool pwdw_block_applies(const GemmProblem &pw, const DwProblem &dw) {
 // is a table of the shapes that were timed inside a network (MobileNetV2 at 224 x 224, 32 images per launch, each
 // pair switched to the fused kernel on its own; microseconds per network pass against 445):
 //   image  in -> expanded  stride   change        image  in -> expanded  stride   change
-//   112     16 ->  96        2      +2.1           14    64 -> 384         1      -5.5 / -3.2 / -3.7 / -1.1
-//    56     24 -> 144        1      +1.6           14    96 -> 576         1      +0.7 / +2.4
-//    56     24 -> 144        2      -7.6           14    96 -> 576         2      +0.4
-//    28     32 -> 192        1      -1.9 / -1.2     7   160 -> 960         1      +1.6 / +1.9 / +1.6
-//    28     32 -> 192        2      -3.4
+//   112     16 ->  96        2      +1.9           14    64 -> 384         1      -6.1 / -5.0 / -5.4 / -3.8
+//    56     24 -> 144        1      -0.8           14    96 -> 576         1      +0.1 / -0.4
+//    56     24 -> 144        2      -6.9           14    96 -> 576         2      -1.5
+//    28     32 -> 192        1      -5.2 / -3.8     7   160 -> 960         1      +0.4 / -0.6 / -0.4
+//    28     32 -> 192        2      -6.4
+// (changes within +-1.5 are noise; the listed shapes are the ones beyond it.)
 // A shape that is not in the table runs as two launches.
-bool pwdw_block_preferred(const GemmProblem &pw, const DwProblem &dw) {
-    if (!pwdw_block_applies(pw, dw) || dw.h != dw.w_ || dw.n < 8) return false;
+bool pwdw_block_listed(int32_t images, int32_t image_h, int32_t image_w, int32_t in_channels, int32_t expanded_channels, int32_t stride) {
+    if (image_h != image_w || images < 8) return false;
     struct Shape {
         int32_t image, in, expanded, stride;
     };
     static const Shape faster[] = {{56, 24, 144, 2}, {28, 32, 192, 1}, {28, 32, 192, 2}, {14, 64, 384, 1}};
     for (const Shape &s : faster)
-        if (dw.h == s.image && pw.k == s.in && dw.c == s.expanded && dw.stride_h == s.stride) return true;
+        if (image_h == s.image && in_channels == s.in && expanded_channels == s.expanded && stride == s.stride) return true;
     return false;
+}
+
+bool pwdw_block_preferred(const GemmProblem &pw, const DwProblem &dw) {
+    return pwdw_block_applies(pw, dw) && pwdw_block_listed(dw.n, dw.h, dw.w_, pw.k, dw.c, dw.stride_h);
 }
 
 // rows_per_tile / cols_per_tile: the tile a workgroup owns, 0 = chosen here

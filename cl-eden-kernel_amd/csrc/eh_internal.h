@@ -496,6 +496,7 @@ int launch_dwconv_nchw(const DwProblem &p, hipStream_t stream);
 
 // ---------------------------------------------------------------- pointwise + depthwise in one launch (eh_block.hip)
 bool pwdw_block_applies(const GemmProblem &pw, const DwProblem &dw);
+bool pwdw_block_listed(int32_t images, int32_t image_h, int32_t image_w, int32_t in_channels, int32_t expanded_channels, int32_t stride);
 bool pwdw_block_preferred(const GemmProblem &pw, const DwProblem &dw);  // the fused launch is the faster one for this shape (measured table)
 int launch_pwdw_block(const GemmProblem &pw, const DwProblem &dw, int rows_per_tile, int cols_per_tile, hipStream_t stream);
 

@@ -191,6 +191,8 @@ struct PerChannelState {
 
 }  // namespace detail
 
+class HipDepthwiseConvolution;
+
 class HipConvolution {
 public:
     HipConvolution(const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision)
@@ -293,6 +295,7 @@ public:
             const int rc = eh_conv2d_u8_repack(plan_, weight_->getDataPtr(), bias_->getDataPtr(), &q, runtime_->stream());
             CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute (repack): %s", eh_last_error());
         }
+        if (depthwise_) return executeWithDepthwise(q);
         if (residual_) {  // output = add(residual, this convolution), as the CLAdd behind it would compute it
             eh_add_requant aq;
             eh_make_add_requant(residual_->getScale(), residual_->getZeroPoint(), output_->getScale(), output_->getZeroPoint(),
@@ -332,6 +335,14 @@ public:
         return Status::SUCCESS;
     }
 
+    // From now on execute() runs this (pointwise) convolution and the depthwise convolution that reads its output as
+    // one launch (eh_conv_dw_block_run): the convolution's own output tensor is never written and needs no storage, it
+    // still supplies the scale and zero point between the two; the depthwise operator is not executed by anyone else.
+    // The reference runs CLConvolution and CLDepthwiseConvolution one after the other (gpu/gpu_op_executor.cc:56-103).
+    // FAILURE when the pair does not fit the fused kernel; nothing is changed then.
+    Status fuseDepthwise(const std::shared_ptr<HipDepthwiseConvolution> &depthwise);
+    bool hasFusedDepthwise() const { return depthwise_ != nullptr; }
+
     Status release() {
         if (plan_) {
             (void)runtime_->synchronize();
@@ -342,6 +353,8 @@ public:
     }
 
 private:
+    Status executeWithDepthwise(const eh_requant &q);
+
     // The requantization parameters of this execution, read from the tensors now; in per-channel mode
     // also hands the plan the channel pairs when they differ from the ones it holds.
     Status currentRequant(eh_requant *q) {
@@ -367,6 +380,7 @@ private:
     PrecisionType precision_;
     std::shared_ptr<HipTensor> input_, output_, weight_, bias_;
     std::shared_ptr<HipTensor> residual_, sum_;  // set by fuseResidualAdd
+    std::shared_ptr<HipDepthwiseConvolution> depthwise_;  // set by fuseDepthwise
     ActivationInfo add_activation_;
     std::shared_ptr<ConvolutionParameters> parameters_;
     ActivationInfo activation_info_;
@@ -487,6 +501,13 @@ public:
         return Status::SUCCESS;
     }
 
+    // for the pointwise convolution that takes this operator into its launch (HipConvolution::fuseDepthwise)
+    eh_dwconv_plan *plan() const { return plan_; }
+    bool perTensorUint8() const { return !per_channel_ && precision_ == PrecisionType::UINT8 && !weights_as_input_; }
+    const std::shared_ptr<HipTensor> &inputTensor() const { return input_; }
+    const std::shared_ptr<HipTensor> &outputTensor() const { return output_; }
+    Status requantNow(eh_requant *q) { return currentRequant(q); }
+
 private:
     // The requantization parameters of this execution, read from the tensors now; in per-channel mode
     // also hands the plan the channel pairs when they differ from the ones it holds.
@@ -519,6 +540,25 @@ private:
     bool deferred_ = false;
     eh_dwconv_plan *plan_ = nullptr;
 };
+
+inline Status HipConvolution::fuseDepthwise(const std::shared_ptr<HipDepthwiseConvolution> &depthwise) {
+    CHECK_EXPR_RETURN_FAILURE(plan_ != nullptr && !deferred_ && depthwise && depthwise->plan() != nullptr, "HipConvolution::fuseDepthwise before initialize");
+    CHECK_EXPR_RETURN_FAILURE(!per_channel_ && precision_ == PrecisionType::UINT8 && launchesOnly() && !residual_ && depthwise->perTensorUint8(),
+                              "HipConvolution::fuseDepthwise: uint8 tensors, constant per-tensor quantized weights, no residual add");
+    CHECK_EXPR_RETURN_FAILURE(depthwise->inputTensor() == output_, "HipConvolution::fuseDepthwise: the depthwise convolution does not read this convolution's output");
+    if (!eh_conv_dw_block_applies(plan_, depthwise->plan())) return Status::FAILURE;  // (not an error: the caller runs the two operators apart)
+    depthwise_ = depthwise;
+    return Status::SUCCESS;
+}
+
+inline Status HipConvolution::executeWithDepthwise(const eh_requant &q) {
+    eh_requant q_dw;
+    CHECK_EXPR_RETURN_FAILURE(depthwise_->requantNow(&q_dw) == Status::SUCCESS, "HipConvolution::execute: the depthwise stage's requantization parameters");
+    const int rc = eh_conv_dw_block_run(plan_, depthwise_->plan(), input_->getDataPtr(), depthwise_->outputTensor()->getDataPtr(), &q, &q_dw, 0, 0,
+                                        runtime_->stream());
+    CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipConvolution::execute (with the depthwise stage): %s", eh_last_error());
+    return Status::SUCCESS;
+}
 
 class HipFullyConnected {
 public:

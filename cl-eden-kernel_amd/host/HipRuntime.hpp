@@ -30,17 +30,20 @@ namespace hip {
 // A device allocation that may not exist yet (pooled buffers materialise in assignBufferPool).
 class HipBuffer {
 public:
-    explicit HipBuffer(size_t byte, int32_t pool_slot = -1) : byte_(byte), buffer_(nullptr), pool_slot_(pool_slot) {}
+    explicit HipBuffer(size_t byte, int32_t pool_slot = -1, int32_t arena = 0)
+        : byte_(byte), buffer_(nullptr), pool_slot_(pool_slot), arena_(arena) {}
     void assignBuffer(void *buffer) { buffer_ = buffer; }
     void setBytes(size_t byte) { byte_ = byte; }
     size_t getBytes() { return byte_; }
     void *getDataPtr() { return buffer_; }
-    int32_t poolSlot() const { return pool_slot_; }  // >= 0: lives in the runtime's pooled allocation
+    int32_t poolSlot() const { return pool_slot_; }  // >= 0: lives in one of the runtime's pooled allocations
+    int32_t arena() const { return arena_; }         // which one
 
 private:
     size_t byte_;
     void *buffer_;
     int32_t pool_slot_;
+    int32_t arena_;
 };
 
 class HipRuntime {
@@ -48,7 +51,10 @@ public:
     HipRuntime() = default;
     ~HipRuntime() {
         for (auto &kv : allocations_) eh_free(kv.second);
-        if (pool_) eh_pool_destroy(pool_);
+        for (auto &a : arenas_)
+            if (a.pool) eh_pool_destroy(a.pool);
+        for (void *e : events_) eh_event_destroy(e);
+        for (void *s : lane_streams_) eh_stream_destroy(s);
         if (stream_) eh_stream_destroy(stream_);
     }
     HipRuntime(const HipRuntime &) = delete;
@@ -62,7 +68,40 @@ public:
         if (!stream_) CHECK_EXPR_RETURN_FAILURE(eh_stream_create(&stream_) == EH_OK, "stream: %s", eh_last_error());
         return Status::SUCCESS;
     }
-    void *stream() { return stream_; }
+    // The stream operators launch on: the runtime's own, unless the list executor has pointed the launches of a lane
+    // at that lane's stream for the moment (launchOn).
+    void *stream() { return launch_stream_ ? launch_stream_ : stream_; }
+    void *mainStream() { return stream_; }
+    void launchOn(void *stream) { launch_stream_ = stream; }
+
+    // Streams for the lanes of an operator list beyond the first (default priority, made on first use), and events to
+    // fork them from the main stream and join them to it.
+    void *laneStream(size_t lane) {
+        while (lane_streams_.size() <= lane) {
+            void *s = nullptr;
+            if (eh_stream_create(&s) != EH_OK) return nullptr;
+            lane_streams_.push_back(s);
+        }
+        return lane_streams_[lane];
+    }
+    void *event(size_t index) {
+        while (events_.size() <= index) {
+            void *e = nullptr;
+            if (eh_event_create(&e) != EH_OK) return nullptr;
+            events_.push_back(e);
+        }
+        return events_[index];
+    }
+
+    // Pooled buffers are requested from the arena selected at the time.  Arenas are separate pools, each laid out in
+    // an allocation of its own: a buffer never takes over storage from another arena's buffers, which is what the
+    // lanes of an operator list need (they are at different operators at any moment, so one lane's liveness says
+    // nothing about when another lane's buffer is free).
+    void selectArena(int32_t arena) {
+        if (arena < 0) arena = 0;
+        if ((size_t)arena >= arenas_.size()) arenas_.resize((size_t)arena + 1);
+        arena_ = arena;
+    }
 
     // BufferType protocol, as CLRuntime::getBuffer.
     std::shared_ptr<HipBuffer> getBuffer(const PrecisionType &precision, const DataType &data_type, const Dim4 &dims,
@@ -90,18 +129,21 @@ public:
     // Materialises every pooled buffer at its final size, all of them in ONE device allocation (the reference
     // allocates each: CLRuntime.cpp:120-137), then forgets the pools.
     Status assignBufferPool() {
-        if (!pool_) return Status::SUCCESS;
-        size_t arena = 0;
-        CHECK_EXPR_RETURN_FAILURE(eh_pool_assign(pool_, &arena) == EH_OK, "assignBufferPool: %s", eh_last_error());
-        last_arena_bytes_ = arena;
-        for (auto &kv : pending_) {
-            void *ptr = nullptr;
-            size_t bytes = 0;
-            CHECK_EXPR_RETURN_FAILURE(eh_pool_slot(pool_, kv.first, &ptr, &bytes) == EH_OK, "assignBufferPool: %s", eh_last_error());
-            kv.second.first->setBytes(bytes);
-            kv.second.first->assignBuffer(bytes ? ptr : nullptr);
+        last_arena_bytes_ = 0;
+        for (auto &a : arenas_) {
+            if (!a.pool) continue;
+            size_t arena = 0;
+            CHECK_EXPR_RETURN_FAILURE(eh_pool_assign(a.pool, &arena) == EH_OK, "assignBufferPool: %s", eh_last_error());
+            last_arena_bytes_ += arena;
+            for (auto &kv : a.pending) {
+                void *ptr = nullptr;
+                size_t bytes = 0;
+                CHECK_EXPR_RETURN_FAILURE(eh_pool_slot(a.pool, kv.first, &ptr, &bytes) == EH_OK, "assignBufferPool: %s", eh_last_error());
+                kv.second.first->setBytes(bytes);
+                kv.second.first->assignBuffer(bytes ? ptr : nullptr);
+            }
+            a.pending.clear();
         }
-        pending_.clear();
         return Status::SUCCESS;
     }
 
@@ -109,28 +151,32 @@ public:
     // they take no part in the next assignment and get no memory.
     Status abandonPendingBuffers() {
         Status st = Status::SUCCESS;
-        for (auto &kv : pending_)
-            if (pool_ && eh_pool_release(pool_, kv.first) != EH_OK) st = Status::FAILURE;
-        pending_.clear();
+        for (auto &a : arenas_) {
+            for (auto &kv : a.pending)
+                if (a.pool && eh_pool_release(a.pool, kv.first) != EH_OK) st = Status::FAILURE;
+            a.pending.clear();
+        }
         return st;
     }
 
     Status resetIntraBuffer() {
-        if (pool_) CHECK_EXPR_RETURN_FAILURE(eh_pool_reset_intra(pool_) == EH_OK, "resetIntraBuffer: %s", eh_last_error());
+        Arena &a = arenas_[(size_t)arena_];
+        if (a.pool) CHECK_EXPR_RETURN_FAILURE(eh_pool_reset_intra(a.pool) == EH_OK, "resetIntraBuffer: %s", eh_last_error());
         return Status::SUCCESS;
     }
 
     Status resetInterBuffer(const std::shared_ptr<HipBuffer> buffer) {
-        auto it = buffer ? pending_.find(buffer->poolSlot()) : pending_.end();
-        if (it == pending_.end() || it->second.first != buffer || it->second.second == EH_POOL_INTRA || !pool_ ||
-            eh_pool_reset_inter(pool_, it->first) != EH_OK) {
+        Arena *a = buffer && buffer->arena() >= 0 && (size_t)buffer->arena() < arenas_.size() ? &arenas_[(size_t)buffer->arena()] : nullptr;
+        auto it = a ? a->pending.find(buffer->poolSlot()) : std::map<int32_t, std::pair<std::shared_ptr<HipBuffer>, int>>::iterator();
+        if (!a || it == a->pending.end() || it->second.first != buffer || it->second.second == EH_POOL_INTRA || !a->pool ||
+            eh_pool_reset_inter(a->pool, it->first) != EH_OK) {
             ERROR_PRINT("HipRuntime::resetInterBuffer: buffer not found\n");
             return Status::FAILURE;
         }
         return Status::SUCCESS;
     }
 
-    // bytes of the single allocation the last assignBufferPool() made for its pooled buffers
+    // bytes of the allocations (one per arena in use) the last assignBufferPool() made for its pooled buffers
     size_t lastPoolAllocationBytes() const { return last_arena_bytes_; }
 
     size_t interPoolSize() const { return countPending(false); }
@@ -157,9 +203,10 @@ public:
     Status releaseBuffer(std::shared_ptr<HipBuffer> buffer) {
         std::lock_guard<std::mutex> lock(mutex_);
         if (buffer->poolSlot() >= 0) {  // a pooled buffer: its allocation goes when the last buffer in it is released
-            CHECK_EXPR_RETURN_FAILURE(pool_ != nullptr, "HipRuntime::releaseBuffer: no pool");
+            eh_pool *pool = buffer->arena() >= 0 && (size_t)buffer->arena() < arenas_.size() ? arenas_[(size_t)buffer->arena()].pool : nullptr;
+            CHECK_EXPR_RETURN_FAILURE(pool != nullptr, "HipRuntime::releaseBuffer: no pool");
             synchronizeLocked();
-            const int rc = eh_pool_release(pool_, buffer->poolSlot());
+            const int rc = eh_pool_release(pool, buffer->poolSlot());
             buffer->assignBuffer(nullptr);
             return rc == EH_OK ? Status::SUCCESS : Status::CL_FAILURE;
         }
@@ -224,34 +271,42 @@ private:
     // to be in the end); a slot that is taken over keeps its HipBuffer object, as the reference hands back the same
     // CLBuffer.
     std::shared_ptr<HipBuffer> pooled(int kind, size_t bytes) {
-        if (!pool_ && eh_pool_create(&pool_) != EH_OK) {
+        Arena &a = arenas_[(size_t)arena_];
+        if (!a.pool && eh_pool_create(&a.pool) != EH_OK) {
             ERROR_PRINT("HipRuntime::getBuffer: %s\n", eh_last_error());
             return nullptr;
         }
         int32_t slot = -1;
-        if (eh_pool_request(pool_, kind, bytes, &slot) != EH_OK) {
+        if (eh_pool_request(a.pool, kind, bytes, &slot) != EH_OK) {
             ERROR_PRINT("HipRuntime::getBuffer: %s\n", eh_last_error());
             return nullptr;
         }
         size_t final_bytes = bytes;
-        (void)eh_pool_slot(pool_, slot, nullptr, &final_bytes);
-        auto it = pending_.find(slot);
-        if (it != pending_.end()) {
+        (void)eh_pool_slot(a.pool, slot, nullptr, &final_bytes);
+        auto it = a.pending.find(slot);
+        if (it != a.pending.end()) {
             it->second.first->setBytes(final_bytes);
             return it->second.first;
         }
-        auto buffer = std::make_shared<HipBuffer>(final_bytes, slot);
-        pending_[slot] = std::make_pair(buffer, kind);
+        auto buffer = std::make_shared<HipBuffer>(final_bytes, slot, arena_);
+        a.pending[slot] = std::make_pair(buffer, kind);
         return buffer;
     }
     size_t countPending(bool intra) const {
         size_t n = 0;
-        for (auto &kv : pending_) n += (kv.second.second == EH_POOL_INTRA) == intra ? 1 : 0;
+        for (auto &a : arenas_)
+            for (auto &kv : a.pending) n += (kv.second.second == EH_POOL_INTRA) == intra ? 1 : 0;
         return n;
     }
 
-    eh_pool *pool_ = nullptr;
-    std::map<int32_t, std::pair<std::shared_ptr<HipBuffer>, int>> pending_;  // slots requested since the last assignment
+    struct Arena {
+        eh_pool *pool = nullptr;
+        std::map<int32_t, std::pair<std::shared_ptr<HipBuffer>, int>> pending;  // slots requested since the last assignment
+    };
+    std::vector<Arena> arenas_ = std::vector<Arena>(1);
+    int32_t arena_ = 0;
+    std::vector<void *> lane_streams_, events_;
+    void *launch_stream_ = nullptr;
     size_t last_arena_bytes_ = 0;
     std::map<void *, void *> allocations_;  // user pointer -> hipMalloc base
     std::mutex mutex_;

@@ -78,6 +78,36 @@ public:
         vdims_ = ndim;
     }
 
+    // A tensor that is never stored: shape and quantization parameters of a value that only exists inside a fused
+    // launch (the operators on either side of it still read its scale and zero point).  No device memory, no pool
+    // request; reconfigureDimsAndBuffer() gives it a buffer of its own should it have to be stored after all.
+    struct NoStorage {};
+    HipTensor(NoStorage, const std::shared_ptr<HipRuntime> runtime, const PrecisionType &precision, const DataType &data_type,
+              const NDims &ndim, const DataOrder &data_order, const float &scale, const int32_t &zero_point, const uint32_t buffer_data_type,
+              const int32_t buffer_index)
+        : runtime_(runtime), precision_(precision), data_type_(data_type), dims_(extendToDim4(ndim)), vdims_(ndim), order_(data_order),
+          scale_(scale), zero_point_(zero_point), buffer_type_(BufferType::DEDICATED), storage_type_(StorageType::BUFFER),
+          buffer_data_type_(buffer_data_type), buffer_index_(buffer_index), is_const_(false) {}
+    bool hasStorage() { return whole_ ? whole_->hasStorage() : (buf_ != nullptr); }
+
+    // A view: `images` of the leading dimension of `whole`, starting at `first_image`, as a tensor of its own shape.
+    // It owns no storage (its address follows the whole tensor's, also when that is assigned or moved later) and
+    // reads scale and zero point from the whole tensor, which is the one the owner of the list talks to.  The lanes of
+    // an operator list see their share of the list's inputs and outputs through such views.  No counterpart in the
+    // reference, whose operators always work on whole tensors.
+    HipTensor(const std::shared_ptr<HipTensor> &whole, uint32_t first_image, uint32_t images)
+        : runtime_(whole->runtime_), precision_(whole->precision_), data_type_(whole->data_type_), dims_(whole->dims_),
+          vdims_(whole->vdims_), order_(whole->order_), scale_(whole->scale_), zero_point_(whole->zero_point_),
+          buffer_type_(whole->buffer_type_), storage_type_(whole->storage_type_), buffer_data_type_(whole->buffer_data_type_),
+          buffer_index_(whole->buffer_index_), is_const_(whole->is_const_), whole_(whole) {
+        const uint32_t all = vdims_.empty() ? 1 : vdims_[0];
+        const size_t per_image = all ? whole->getNumOfBytes() / all : 0;
+        view_offset_ = per_image * first_image;
+        if (!vdims_.empty()) vdims_[0] = images;
+        dims_ = extendToDim4(vdims_);
+    }
+    bool isView() const { return whole_ != nullptr; }
+
     ~HipTensor() override {
         if (buf_ && buf_.use_count() == 1 && buf_->getDataPtr() != nullptr) (void)runtime_->releaseBuffer(buf_);
     }
@@ -91,10 +121,16 @@ public:
     uint32_t getNumOfDims() override { return (uint32_t)vdims_.size(); }
     uint32_t getTotalSizeFromDims() override { return getTensorSizeFromDims(vdims_); }
     DataOrder getDataOrder() override { return order_; }
-    float getScale() override { return scale_; }
-    int32_t getZeroPoint() override { return zero_point_; }
-    void setZeroPoint(int32_t zero_point) override { zero_point_ = zero_point; }
-    void setScale(float scale) override { scale_ = scale; }
+    float getScale() override { return whole_ ? whole_->getScale() : scale_; }
+    int32_t getZeroPoint() override { return whole_ ? whole_->getZeroPoint() : zero_point_; }
+    void setZeroPoint(int32_t zero_point) override {
+        if (whole_) return whole_->setZeroPoint(zero_point);
+        zero_point_ = zero_point;
+    }
+    void setScale(float scale) override {
+        if (whole_) return whole_->setScale(scale);
+        scale_ = scale;
+    }
     void set_buffer_index(int32_t index) override { buffer_index_ = index; }
     int32_t get_buffer_index() override { return buffer_index_; }
     void set_buffer_type(uint32_t type) override { buffer_data_type_ = type; }
@@ -102,7 +138,13 @@ public:
     void set_buffer_ptr(void *addr) override { raw_buffer = addr; }
     bool is_const() override { return is_const_; }
 
-    void *getDataPtr() { return buf_ ? buf_->getDataPtr() : nullptr; }
+    void *getDataPtr() {
+        if (whole_) {
+            void *base = whole_->getDataPtr();
+            return base ? static_cast<char *>(base) + view_offset_ : nullptr;
+        }
+        return buf_ ? buf_->getDataPtr() : nullptr;
+    }
     std::shared_ptr<HipBuffer> getBuffer() { return buf_; }
     BufferType getBufferType() const { return buffer_type_; }
 
@@ -203,10 +245,11 @@ public:
             std::fclose(f);
         }
     }
-    Status resetInterBuffer() override { return runtime_->resetInterBuffer(buf_); }
+    Status resetInterBuffer() override { return whole_ || !buf_ ? Status::SUCCESS : runtime_->resetInterBuffer(buf_); }
 
 private:
     Status growBuffer() {
+        CHECK_EXPR_RETURN_FAILURE(!whole_, "HipTensor: a view cannot be given storage of its own");
         if (buf_ && buf_->getDataPtr() && buf_->getBytes() >= getNumOfBytes()) return Status::SUCCESS;
         if (buf_ && buf_->getDataPtr()) (void)runtime_->releaseBuffer(buf_);
         buf_ = std::make_shared<HipBuffer>(getNumOfBytes());
@@ -228,6 +271,8 @@ private:
     int32_t buffer_index_;
     bool is_const_;
     std::shared_ptr<HipBuffer> buf_;
+    std::shared_ptr<HipTensor> whole_;  // views only
+    size_t view_offset_ = 0;
 };
 
 }  // namespace hip

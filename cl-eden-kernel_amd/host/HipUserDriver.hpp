@@ -131,8 +131,7 @@ public:
         if (get_ud_operators(operator_list_id, operators, in_tensors, out_tensors) != ENN_RET_SUCCESS) return ENN_RET_FAILED;
         UDBuffers buffer;
         BufferTable none;
-        for (int i = 0; i < times; ++i)
-            if (op_executor->execute(operators, buffer, none) != ENN_RET_SUCCESS) return ENN_RET_FAILED;
+        if (op_executor->execute_times(operators, buffer, none, times) != ENN_RET_SUCCESS) return ENN_RET_FAILED;
         compute_library->flush();
         return ENN_RET_SUCCESS;
     }

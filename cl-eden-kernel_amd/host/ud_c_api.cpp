@@ -281,6 +281,22 @@ int eud_set_replay(eud_driver *driver, int32_t replay) {
     return 0;
 }
 
+int eud_set_image_lanes(eud_driver *driver, int32_t lanes, int32_t min_lane_images) {
+    if (driver == nullptr || driver->ud.constructor() == nullptr) return fail("eud_set_image_lanes: no driver");
+    if (lanes < 1 || min_lane_images < 1) return fail("eud_set_image_lanes: lanes and min_lane_images start at 1");
+    driver->ud.constructor()->image_lanes = lanes;
+    driver->ud.constructor()->min_lane_images = min_lane_images;
+    return 0;
+}
+
+int eud_set_fuse_expansions(eud_driver *driver, int32_t mode) {
+    if (driver == nullptr || driver->ud.constructor() == nullptr) return fail("eud_set_fuse_expansions: no driver");
+    if (mode < 0 || mode > 2) return fail("eud_set_fuse_expansions: mode is 0, 1 or 2");
+    driver->ud.constructor()->fuse_expansions = mode != 0;
+    driver->ud.constructor()->fuse_unlisted_expansions = mode == 2;
+    return 0;
+}
+
 int eud_synchronize(eud_driver *driver) {
     if (driver == nullptr || !driver->ud.computeLibrary()) return fail("eud_synchronize: no driver");
     return driver->ud.computeLibrary()->runtime()->synchronize() == Status::SUCCESS ? 0 : fail_below("eud_synchronize");

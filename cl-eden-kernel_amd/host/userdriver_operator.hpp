@@ -38,16 +38,25 @@ public:
     // device addresses, scales and zero points): such an execution can be recorded once and replayed.  Not part of the
     // reference's UDOperator; the list executor of this backend asks it.
     virtual bool replayable() const { return false; }
+    // The lane of its list this operator belongs to (0 unless the constructor cut the list's images into lanes, each
+    // with operators of its own that share nothing with the other lanes' but read-only parameters).  Not part of the
+    // reference's UDOperator either.
+    int lane() const { return lane_; }
+    void setLane(int lane) { lane_ = lane; }
     std::string getName() { return name_; }
     uint64_t getId() { return id_; }
     std::vector<std::shared_ptr<ITensor>> getInTensors() { return in_; }
     std::vector<std::shared_ptr<ITensor>> getOutTensors() { return out_; }
     std::vector<std::shared_ptr<ITensor>> getDataTensors() { return data_; }
+    // the same lists without a copy, for the executor's per-execution walk over every tensor of every operator
+    const std::vector<std::shared_ptr<ITensor>> &inTensors() const { return in_; }
+    const std::vector<std::shared_ptr<ITensor>> &outTensors() const { return out_; }
 
 protected:
     std::string name_;
     uint64_t id_;
     std::vector<std::shared_ptr<ITensor>> in_, out_, data_;
+    int lane_ = 0;
 };
 
 // The reference stamps execute() per operator type with a macro; the operators of

@@ -54,6 +54,8 @@ EXPORTS = {
     "eud_close_subgraph": (C.c_int, [C.c_void_p, C.c_uint64]),
     "eud_execute_operators": (C.c_int, [C.c_void_p, C.c_uint64, C.c_int32]),
     "eud_set_replay": (C.c_int, [C.c_void_p, C.c_int32]),
+    "eud_set_image_lanes": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32]),
+    "eud_set_fuse_expansions": (C.c_int, [C.c_void_p, C.c_int32]),
     "eud_synchronize": (C.c_int, [C.c_void_p]),
     "eud_stream": (C.c_void_p, [C.c_void_p]),
     "eud_stats": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_int32), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
@@ -156,6 +158,14 @@ class UserDriver:
 
     def set_replay(self, on):
         check(load().eud_set_replay(self.h, int(on)))
+
+    def set_image_lanes(self, lanes, min_lane_images=16):
+        """Lists opened from now on run as `lanes` chains of images side by side when a chain gets min_lane_images or more."""
+        check(load().eud_set_image_lanes(self.h, lanes, min_lane_images), "set_image_lanes")
+
+    def set_fuse_expansions(self, mode):
+        """0: never; 1: where the library's measured table prefers the one launch (default); 2: wherever the kernel fits"""
+        check(load().eud_set_fuse_expansions(self.h, mode), "set_fuse_expansions")
 
     def synchronize(self):
         check(load().eud_synchronize(self.h), "synchronize")

@@ -351,6 +351,10 @@ int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
  * q_pointwise->zp_out must equal q_depthwise->zp_in (they describe the same tensor). */
 int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise);
 int eh_conv_dw_block_preferred(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise);
+/* The table alone, for a caller that has to decide before the plans exist (an operator constructor that does not
+ * give the expanded tensor any storage): images per launch, the square image's extent, pointwise input channels,
+ * expanded channels, depthwise stride.  `_preferred` is `_applies` and this. */
+int eh_conv_dw_block_listed(int32_t images, int32_t image_h, int32_t image_w, int32_t in_channels, int32_t expanded_channels, int32_t stride);
 int eh_conv_dw_block_run(eh_conv_plan *pointwise, eh_dwconv_plan *depthwise, const void *input, void *output,
                          const eh_requant *q_pointwise, const eh_requant *q_depthwise, int32_t rows_per_tile, int32_t cols_per_tile,
                          void *stream);

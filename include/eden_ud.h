@@ -93,6 +93,16 @@ int eud_close_subgraph(eud_driver *driver, uint64_t list_id);
 int eud_execute_operators(eud_driver *driver, uint64_t list_id, int32_t times);
 /* replay = 0: every execution runs operator by operator, as the reference's executor does */
 int eud_set_replay(eud_driver *driver, int32_t replay);
+/* Lists opened from now on whose feature maps all carry the same number of images are built `lanes` times over, each
+ * on 1 / lanes of the images, and the lanes run side by side on streams of their own (parallel branches of the recorded
+ * graph), when a share holds at least min_lane_images images.  Default 2 lanes from 16 images per lane; lanes = 1 builds
+ * one operator per description as the reference does.  Results do not depend on it. */
+int eud_set_image_lanes(eud_driver *driver, int32_t lanes, int32_t min_lane_images);
+/* Lists opened from now on: a uint8 1x1 CONV_2D whose only reader is a 3x3 DEPTHWISE_CONV_2D runs with it as one launch
+ * (eh_conv_dw_block_run; the tensor between them gets no storage) for mode 1 where the library lists the shape as
+ * faster that way (the default), for mode 2 wherever the kernel fits, for mode 0 never (one operator per description,
+ * as the reference builds the list).  Results do not depend on it. */
+int eud_set_fuse_expansions(eud_driver *driver, int32_t mode);
 int eud_synchronize(eud_driver *driver);         /* IComputeLibrary::synchronize */
 void *eud_stream(eud_driver *driver);            /* the hipStream_t the operators are enqueued on */
 /* operators built for the list, and what the executor has done so far (over all lists) */

@@ -64,7 +64,8 @@ def test_mobilenet_v2_batch_64_through_the_userdriver_on_scattered_images():
     ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch)
     d.open_subgraph(ol)
     s = d.stats(list_id)
-    assert 0 < s["pool_bytes"] < 0.45 * sum(batch * t["h"] * t["w"] * t["c"] for t in tensors)   # liveness reuse, one allocation
+    assert s["operators"] == 2 * (54 - 8)   # two lanes of 32 images, each with the whole list (adds fused, eight listed expansions fused)
+    assert 0 < s["pool_bytes"] < 0.45 * sum(batch * t["h"] * t["w"] * t["c"] for t in tensors)   # liveness reuse within each lane
     x = np.ascontiguousarray(mobilenet.network_input(8)[where])
     ref = want[-1].reshape(8, -1)[where]
     for rep in range(3):
@@ -77,6 +78,71 @@ def test_mobilenet_v2_batch_64_through_the_userdriver_on_scattered_images():
     d.synchronize()
     assert np.array_equal(d.read_output(list_id, 0, shape), ref)
     d.close_subgraph(list_id)
+
+
+@pytest.mark.parametrize("lanes,batch,replay", [(2, 4, True), (4, 8, True), (2, 6, False), (3, 6, True)],
+                         ids=["two_lanes", "four_lanes", "two_lanes_operator_by_operator", "three_lanes"])
+def test_image_lanes_give_the_same_logits(lanes, batch, replay):
+    """The list built once per lane on a share of the images, lanes on streams of their own (recorded as parallel
+    branches, or enqueued operator by operator): logits equal to the oracle's through ExecuteSubGraph on whole host
+    buffers, on several executions, and after the input changed."""
+    d = driver()
+    image, list_id = 96, 0x7000 + lanes * 64 + batch
+    d.set_image_lanes(lanes, 1)
+    d.set_replay(replay)
+    try:
+        ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image)
+        d.open_subgraph(ol)
+        assert d.stats(list_id)["operators"] == lanes * 54
+        x = mobilenet.network_input(batch, image)
+        _, _, want = oracle_images(batch, image, False)
+        ref = want[-1].reshape(batch, -1)
+        for rep in range(3):
+            got = np.zeros(shape, np.uint8)
+            d.execute_subgraph(list_id, {in_index: x, out_index: got})
+            assert np.array_equal(got, ref), (rep, np.argwhere((got != ref).any(axis=1)).ravel().tolist())
+        got = np.zeros(shape, np.uint8)
+        d.execute_subgraph(list_id, {in_index: np.ascontiguousarray(x[::-1]), out_index: got})
+        assert np.array_equal(got, ref[::-1])
+        d.close_subgraph(list_id)
+        # a batch the lanes do not divide runs as one chain
+        if batch % 4:
+            d.set_image_lanes(4, 1)
+            ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id + 1, batch, image)
+            d.open_subgraph(ol)
+            assert d.stats(list_id + 1)["operators"] == 54
+            got = np.zeros(shape, np.uint8)
+            d.execute_subgraph(list_id + 1, {in_index: x, out_index: got})
+            assert np.array_equal(got, ref)
+            d.close_subgraph(list_id + 1)
+    finally:
+        d.set_image_lanes(2, 16)
+        d.set_replay(True)
+
+
+def test_every_fitting_expansion_fused_with_its_depthwise_convolution():
+    """All sixteen expansion + depthwise pairs of the network as one launch each (mode 2), in two lanes: 38 operators
+    per lane, logits equal to the oracle's; then mode 0 builds one operator per description again."""
+    d = driver()
+    batch, image, list_id = 4, 224, 0x7F00
+    _, _, want = oracle_images(batch, image, False)
+    ref = want[-1].reshape(batch, -1)
+    x = mobilenet.network_input(batch, image)
+    try:
+        for mode, lanes, operators in ((2, 2, 2 * 38), (2, 1, 38), (0, 1, 54), (1, 1, 54)):   # (mode 1: four images are below the table's floor)
+            d.set_fuse_expansions(mode)
+            d.set_image_lanes(lanes, 1)
+            ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image)
+            d.open_subgraph(ol)
+            assert d.stats(list_id)["operators"] == operators, (mode, lanes)
+            for rep in range(3):
+                got = np.zeros(shape, np.uint8)
+                d.execute_subgraph(list_id, {in_index: x, out_index: got})
+                assert np.array_equal(got, ref), (mode, lanes, rep, np.argwhere((got != ref).any(axis=1)).ravel().tolist())
+            d.close_subgraph(list_id)
+    finally:
+        d.set_fuse_expansions(1)
+        d.set_image_lanes(2, 16)
 
 
 def test_quantization_parameters_changed_between_executions_are_honoured():

@@ -22,7 +22,7 @@ def test_host_side_buffer_pool_and_types():
     r = subprocess.run([_binary(), "--host-only"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
     print(r.stdout)
     assert r.returncode == 0, r.stdout
-    assert "0 of 4 host-only tests failed" in r.stdout
+    assert "0 of 5 host-only tests failed" in r.stdout
 
 
 @pytest.mark.gpu

@@ -1249,6 +1249,22 @@ static int gpu_tests() {
                 EXPECT(c.direct == 1 && c.recordings == 1 && c.replays == 3);
             else
                 EXPECT(c.direct == 4 && c.recordings == 0 && c.replays == 0);   // re-packing weights is not replayable
+            if (const_weights) {
+                // eleven executions in a row on the resident tensors: two bursts of four out of a graph of their own, three single replays
+                UDBuffers none;
+                BufferTable table;
+                std::vector<uint8_t> zeros(got.size(), 0);
+                EXPECT(built.out_tensors[0]->writeData(zeros.data()) == Status::SUCCESS);
+                EXPECT(executor.execute_times(built.operators, none, table, 11) == ENN_RET_SUCCESS);
+                EXPECT(c.direct == 1 && c.recordings == 1 && c.replays == 14);
+                EXPECT(built.out_tensors[0]->readData(got.data()) == Status::SUCCESS && same(got, want1));
+                // a fresh executor asked for a burst straight away still runs its first execution directly and records at the second
+                OperationExecutor second(lib);
+                EXPECT(second.execute_times(built.operators, none, table, 6) == ENN_RET_SUCCESS);
+                EXPECT(second.counters().direct == 1 && second.counters().recordings == 1 && second.counters().replays == 5);
+                EXPECT(built.out_tensors[0]->readData(got.data()) == Status::SUCCESS && same(got, want1));
+                second.forget(built.operators);
+            }
             executor.forget(built.operators);
             built.close_oplist(list.id);
         }
@@ -1320,6 +1336,64 @@ static int gpu_tests() {
         EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_FAILED);
         EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS);   // and it can be opened again
         EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_SUCCESS);
+        // the same list as two lanes of one image each: the list built twice, each lane's operators on its share of the
+        // whole input and output tensors, recorded as two branches; then operator by operator on the lanes' streams
+        ud.constructor()->image_lanes = 2;
+        ud.constructor()->min_lane_images = 1;
+        EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS);
+        EXPECT(ud.constructor()->lanes() == 2);
+        EXPECT(ud.get_graph_for_TC(list.id, ops) == ENN_RET_SUCCESS && ops && ops->size() == 4);
+        if (ops && ops->size() == 4) {
+            EXPECT((*ops)[0]->lane() == 0 && (*ops)[1]->lane() == 0 && (*ops)[2]->lane() == 1 && (*ops)[3]->lane() == 1);
+            auto in0 = std::static_pointer_cast<HipTensor>((*ops)[0]->getInTensors()[0]), in1 = std::static_pointer_cast<HipTensor>((*ops)[2]->getInTensors()[0]);
+            EXPECT(in0->isView() && in1->isView() && in0->getDim().n == 1 && in0->getNumOfBytes() == x.size() / 2);
+            EXPECT(static_cast<char *>(in1->getDataPtr()) == static_cast<char *>(in0->getDataPtr()) + x.size() / 2);
+            // the lanes' feature maps are different tensors, and the parameters are shared
+            EXPECT((*ops)[0]->getOutTensors()[0] != (*ops)[2]->getOutTensors()[0]);
+            EXPECT((*ops)[0]->getInTensors()[1] == (*ops)[2]->getInTensors()[1]);
+        }
+        const auto before = ud.executor()->counters();
+        for (int round = 0; round < 5; ++round) {
+            if (round == 3) ud.executor()->replay = false;
+            std::fill(got.begin(), got.end(), 0);
+            BufferTable table;
+            table.add(10, x.data(), x.size());
+            table.add(12, got.data(), got.size());
+            EXPECT(ud.ExecuteSubGraph(OperatorListExecuteRequest(list.id, (uint64_t)round, table)) == ENN_RET_SUCCESS);
+            EXPECT(same(got, want));
+        }
+        ud.executor()->replay = true;
+        EXPECT(ud.executor()->counters().direct == before.direct + 3 && ud.executor()->counters().recordings == before.recordings + 1 &&
+               ud.executor()->counters().replays == before.replays + 2);
+        EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_SUCCESS);
+        // three lanes do not divide two images: one chain
+        ud.constructor()->image_lanes = 3;
+        EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS && ud.constructor()->lanes() == 1);
+        EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_SUCCESS);
+        // the pair as one launch (the shape is not in the library's table, so only on request), alone and in two lanes:
+        // one operator per lane, the expanded tensor without storage, results unchanged
+        ud.constructor()->fuse_unlisted_expansions = true;
+        for (const int lanes : {1, 2}) {
+            ud.constructor()->image_lanes = lanes;
+            EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS);
+            EXPECT(ud.get_graph_for_TC(list.id, ops) == ENN_RET_SUCCESS && ops && ops->size() == (size_t)lanes);
+            if (ops && ops->size() == (size_t)lanes) {
+                auto fused = std::dynamic_pointer_cast<EnnUDOperator<HipConvolution>>((*ops)[0]);
+                EXPECT(fused && fused->getOp()->hasFusedDepthwise());
+                auto expanded = std::static_pointer_cast<HipTensor>((*ops)[0]->getOutTensors()[0]);
+                EXPECT(!expanded->hasStorage() && expanded->getDataPtr() == nullptr && expanded->getDim().c == 12);
+                EXPECT((*ops)[0]->getOutTensors().size() == 2 && (*ops)[0]->getInTensors().size() == 5);
+            }
+            for (int round = 0; round < 3; ++round) {
+                std::fill(got.begin(), got.end(), 0);
+                BufferTable table;
+                table.add(10, x.data(), x.size());
+                table.add(12, got.data(), got.size());
+                EXPECT(ud.ExecuteSubGraph(OperatorListExecuteRequest(list.id, (uint64_t)round, table)) == ENN_RET_SUCCESS);
+                EXPECT(same(got, want));
+            }
+            EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_SUCCESS);
+        }
         EXPECT(ud.Deinitialize() == ENN_RET_SUCCESS);
         EXPECT(varied(want));
         return ok;
@@ -1344,6 +1418,24 @@ static int host_tests() {
         EXPECT(d != a && d != b && rt->interPoolSize() == 3);
         EXPECT(rt->resetInterBuffer(std::make_shared<HipBuffer>(4)) == Status::FAILURE);
         EXPECT(a->getDataPtr() == nullptr);  // deferred until assignBufferPool
+        return ok;
+    });
+    run_test("BufferPool.ArenasDoNotTakeOverOneAnothersBuffers", [&] {
+        bool ok = true;
+        auto own = std::make_shared<HipRuntime>();
+        auto a = own->getBuffer(U8, DataType::UINT8, Dim4{1, 8, 8, 8}, BufferType::INTER_SHARED_NEW);
+        EXPECT(own->resetInterBuffer(a) == Status::SUCCESS);   // free for the next request of its arena
+        own->selectArena(1);
+        auto b = own->getBuffer(U8, DataType::UINT8, Dim4{1, 8, 4, 4}, BufferType::INTER_SHARED_REUSE);
+        EXPECT(b != a && b->arena() == 1 && a->arena() == 0 && own->interPoolSize() == 2);   // another arena: a new buffer
+        EXPECT(own->resetInterBuffer(b) == Status::SUCCESS);
+        own->selectArena(0);
+        auto c = own->getBuffer(U8, DataType::UINT8, Dim4{1, 8, 4, 4}, BufferType::INTER_SHARED_REUSE);
+        EXPECT(c == a);                                        // its own arena's free buffer
+        own->selectArena(1);
+        auto d = own->getBuffer(U8, DataType::UINT8, Dim4{1, 8, 2, 2}, BufferType::INTER_SHARED_REUSE);
+        EXPECT(d == b);
+        EXPECT(own->abandonPendingBuffers() == Status::SUCCESS && own->interPoolSize() == 0);
         return ok;
     });
     run_test("BufferPool.IntraSharedIsSizedToTheLargestRequest", [&] {
