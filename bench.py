@@ -165,19 +165,22 @@ def conv_workload(eden, synth, n=1, cold=False):
                 keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 56 * 56 * 64 * 576, bytes=nbytes, bound="mfma")
 
 
-def dw_workload(eden, synth, n=32, cold=False):
-    desc = eden.conv_desc(n, 144, 56, 56, 144, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), dm=1, layout=eden.NHWC)
-    x = synth.fill_u8((n, 56, 56, 144), SEED + 48)
-    w = synth.fill_u8((144, 1, 3, 3), SEED + 49)
-    b = synth.fill_i32((144,), SEED + 50, -1000, 1000)
-    q = eden.make_requant(0.03, 17, 0.006, 140, 0.025, 9, eden.ACT_RELU6, True)
+def dw_workload(eden, synth, n=32, cold=False, c=144, hw=56, stride=2, k=3):
+    """depthwise k x k convolution, ReLU6, channels-last: BASELINE configs[2]'s stride-2 3x3 layer by default"""
+    pad = k // 2
+    ho = (hw + 2 * pad - k) // stride + 1
+    desc = eden.conv_desc(n, c, hw, hw, c, k, k, stride=(stride, stride), pad=(pad,) * 4, dm=1, layout=eden.NHWC)
+    x = synth.fill_u8((n, hw, hw, c), SEED + 48)
+    w = synth.fill_u8((c, 1, k, k), SEED + 49)
+    b = synth.fill_i32((c,), SEED + 50, -1000, 1000)
+    q = eden.make_requant(0.03, 17, 0.006, 140, 0.025 * k / 3, 9, eden.ACT_RELU6, True)
     d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
     plan = eden.DwConvPlan(desc, d_w, d_b, q)
-    nbytes = n * 144 * 56 * 56 + 144 * 9 + 144 * 4 + n * 144 * 28 * 28
+    nbytes = n * c * hw * hw + c * k * k + c * 4 + n * c * ho * ho
     sets = set_count(nbytes, cold)
-    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 28 * 28 * 144)) for _ in range(sets)]
-    return dict(name="dw3x3s2_n%d_c144_56x56_nhwc" % n, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
-                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 144 * 28 * 28 * 9, bytes=nbytes, bound="hbm")
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * ho * ho * c)) for _ in range(sets)]
+    return dict(name="dw%dx%ds%d_n%d_c%d_%dx%d_nhwc" % (k, k, stride, n, c, hw, hw), launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * c * ho * ho * k * k, bytes=nbytes, bound="hbm")
 
 
 def pw_workload(eden, synth, n=32, cin=24, cout=144, hw=56, cold=False):
@@ -471,7 +474,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the oracle check of the network")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2 (two lanes, measured pairs fused), mbv2plain / mbv2lanes / mbv2fused (neither / lanes only / fusion only), mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, copy, tonhwc, tonchw")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2 (two lanes, measured pairs fused), mbv2plain / mbv2lanes / mbv2fused (neither / lanes only / fusion only), mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, copy, tonhwc, tonchw, feedprobe (what a CU's matrix pipe can be fed with, per tile shape)")
     ap.add_argument("--tile", default=None, help="with --only c3block / block:...: ROWSxCOLS output pixels per workgroup (default: chosen by the library)")
     ap.add_argument("--cold", action="store_true", help="with --only: rotate over buffer sets that together exceed the Infinity Cache")
     args = ap.parse_args()
@@ -504,6 +507,11 @@ def main():
                     stream16=stream_workload, stream16big=shaped(stream_workload, out_bytes=256 * 56 * 56 * 144),
                     stream41=shaped(stream_workload, mode=2, out_bytes=32 * 28 * 28 * 144),
                     stream41big=shaped(stream_workload, mode=2, out_bytes=256 * 28 * 28 * 144))
+    if args.only == "feedprobe":
+        # the yardsticks the GEMM tiles' inner loops are set against: one JSON line per mix
+        for mix in range(len(eden.FEED_MIXES)):
+            print(json.dumps(eden.probe_feed(mix, 256, 4000)), flush=True)
+        return
     if args.only in ("mbv2ud", "mbv2udpc"):
         mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
         driver, list_id, _ = mbv2_userdriver(eden, per_channel=args.only == "mbv2udpc")
@@ -519,6 +527,12 @@ def main():
     if args.only and args.tile:
         families["c3block"] = shaped(block_workload, rows=rows, cols=cols)
         families["c3blockbig"] = shaped(block_workload, n=256, rows=rows, cols=cols)
+    if args.only and args.only.startswith("pw:"):      # pw:N,CIN,COUT,HW = that pointwise convolution
+        n, cin, cout, hw = (int(v) for v in args.only[3:].split(","))
+        families[args.only] = shaped(pw_workload, n=n, cin=cin, cout=cout, hw=hw)
+    if args.only and args.only.startswith("dw:"):      # dw:N,C,HW,STRIDE[,K] = that depthwise convolution
+        v = [int(t) for t in args.only[3:].split(",")]
+        families[args.only] = shaped(dw_workload, n=v[0], c=v[1], hw=v[2], stride=v[3], k=v[4] if len(v) > 4 else 3)
     if args.only and args.only.startswith(("block:", "twolaunch:")):
         # block:N,CIN,C,HW,STRIDE = that expansion + 3x3 depthwise pair as one launch; twolaunch: the same as two launches
         kind, _, spec = args.only.partition(":")

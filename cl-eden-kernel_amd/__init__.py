@@ -67,6 +67,7 @@ EXPORTS = {
     "eh_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(AddRequant), C.c_void_p]),
     "eh_avgpool_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PoolDesc), C.c_void_p]),
     "eh_probe_mfma_i8": (C.c_int, [C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
+    "eh_probe_feed": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_int32)]),
     "eh_probe_stream": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]),
     "eh_make_requant_perchannel": (None, [C.c_float, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32, C.c_int, C.c_int,
                                           C.POINTER(Requant), C.c_void_p, C.c_void_p]),
@@ -212,6 +213,25 @@ def avgpool_u8(src, dst, n, c, h, w, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), la
 
 def _addr(x):
     return x.ptr if hasattr(x, "ptr") else x
+
+
+FEED_MIXES = ("dma_alone", "lds_reads_alone", "mfma_alone", "tile_128x128", "tile_64x64_splitk", "tile_256x128", "tile_256x256",
+              "tile_128x128_weights_to_registers", "tile_256x256_weights_to_registers")
+
+
+def probe_feed(mix, workgroups=256, iterations=4000):
+    """One feed-probe mix: ns per iteration and what an iteration holds per wave, as rates per CU and as a fraction of
+    the 5 POP/s matrix peak.  A workgroup takes a CU's LDS, so 256 workgroups are one per CU and more run in rounds."""
+    ns, per = C.c_double(0), (C.c_int32 * 4)()
+    check(load().eh_probe_feed(mix, workgroups, iterations, C.byref(ns), per))
+    rounds = -(-workgroups // 256)
+    ns.value /= rounds
+    per_cu = 4   # waves per CU
+    mfma, reads, dma, regs = per
+    return dict(mix=FEED_MIXES[mix], workgroups=workgroups, ns_per_iteration=round(ns.value, 2), per_wave_iteration=dict(mfma=mfma, lds_reads=reads, dma_1k=dma, register_loads_1k=regs),
+                mfma_frac_of_5_pops=round(min(workgroups, 256) * 4 * mfma * 65536 / ns.value / 5e6, 4) if mfma else None,
+                lds_read_bytes_per_ns_per_cu=round(per_cu * reads * 1024 / ns.value, 1), dma_bytes_per_ns_per_cu=round(per_cu * dma * 1024 / ns.value, 1),
+                register_load_bytes_per_ns_per_cu=round(per_cu * regs * 1024 / ns.value, 1))
 
 
 def probe_mfma_i8(iterations=100000, toggling_operands=True):

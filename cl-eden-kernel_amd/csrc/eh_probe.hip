@@ -4,6 +4,8 @@
 // clock under this load is lower than with constant operands, so both are
 // reported.  And what plain streaming kernels reach on the byte ratios of the HBM-bound layers.
 // Measurement utilities: they have no counterpart in the reference.
+#include <utility>
+
 #include "eh_internal.h"
 
 namespace eh {
@@ -47,10 +49,158 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(const uint4 *__restri
     }
 }
 
+// What the matrix pipe of a CU can be fed with.  A workgroup of four waves (one per SIMD, as in the GEMM kernels) repeats
+// an iteration of NM matrix instructions, NR 16-byte-per-lane LDS fragment reads, ND direct-to-LDS loads of 1 KiB
+// (global_load_lds_dwordx4 from a region that stays in the XCD's L2) and NV ordinary 1 KiB loads into registers that
+// SHARE waves request alike (an operand kept out of LDS), DEPTH iterations in flight, a barrier every SYNC iterations
+// (0: none).  The proportions are those of the GEMM tiles' inner loops; the times say how far below the matrix
+// instructions' own rate the feeding alone puts a tile shape, before any epilogue.
+typedef __attribute__((address_space(3))) uint8_t lds_byte;
+
+__device__ __forceinline__ void probe_dma16(const void *base_uniform, uint32_t lane_offset, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base_uniform), "s"(lds_base_uniform) : "memory");
+}
+__device__ __forceinline__ v4i probe_dsread(uint32_t a) {
+    v4i r;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(a) : "memory");
+    return r;
+}
+template <int N>
+__device__ __forceinline__ void probe_wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+template <int... I, class F>
+__device__ __forceinline__ void probe_for_impl(std::integer_sequence<int, I...>, F &&f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void probe_for(F &&f) {
+    probe_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+constexpr uint32_t kFeedRegion = 1u << 20;  // bytes of source per XCD: stays in its 4 MiB L2
+
+template <int NM, int NR, int ND, int NV, int SHARE, int SYNC>
+__global__ __launch_bounds__(256) void feed_probe_kernel(const uint8_t *src, const int iters, int *sink) {
+    constexpr int DEPTH = 4;
+    constexpr uint32_t region_mask = kFeedRegion - 1;
+    __shared__ __align__(1024) uint8_t lds[128 * 1024];  // fragment reads in the lower half, DMA destinations in the upper
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    for (int i = tid; i < 128 * 256; i += 256) reinterpret_cast<int *>(lds)[i] = (int)(i * 2654435761u);
+    __syncthreads();
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_byte *)lds;
+    const uint8_t *base = src + (size_t)(blockIdx.x & 7) * kFeedRegion;
+    uint32_t goff = ((blockIdx.x >> 3) * 65536u + wave * 1024u + lane * 16u) & region_mask;
+    uint32_t voff = ((blockIdx.x >> 3) * 65536u + 32768u + (wave / SHARE) * 1024u + lane * 16u) & region_mask;
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const uint32_t raddr = lds0 + wave * 16384 + frow * 128 + ((fhalf ^ (frow & 7)) << 4);
+    v16i acc[4];
+    for (int q = 0; q < 4; ++q)
+        for (int r = 0; r < 16; ++r) acc[q][r] = 0;
+    const v4i fa = {tid, tid * 3, tid * 7, tid * 11};
+    v4i fr[NR > 0 ? NR : 1];
+    v4i vg[DEPTH][NV > 0 ? NV : 1];
+    for (int d = 0; d < DEPTH; ++d)
+        for (int j = 0; j < (NV > 0 ? NV : 1); ++j) vg[d][j] = fa;
+    for (int j = 0; j < (NR > 0 ? NR : 1); ++j) fr[j] = fa;
+    uint32_t ring = 0;
+    for (int it = 0; it < iters; it += DEPTH) {
+        probe_for<DEPTH>([&](auto d_c) {
+            constexpr int d = decltype(d_c)::value;
+            // this iteration's memory operations are consumed DEPTH - 1 iterations later
+            probe_for<ND>([&](auto) {
+                probe_dma16(base, goff, lds0 + 65536 + ((ring + wave * 1024) & 0xFFFF));
+                ring += 4096;
+                goff = (goff + 4096u) & region_mask;
+            });
+            constexpr int slot = (d + DEPTH - 1) % DEPTH;
+            // (ordinary loads: the compiler tracks their registers and waits)
+            probe_for<NV>([&](auto j_c) {
+                vg[slot][decltype(j_c)::value] = *reinterpret_cast<const v4i *>(base + voff);
+                voff = (voff + 4096u) & region_mask;
+            });
+            probe_for<NM>([&](auto q_c) {
+                constexpr int q = decltype(q_c)::value;
+                const v4i b = NV > 0 ? vg[d][q % (NV > 0 ? NV : 1)] : fa;
+                const v4i a = NR > 0 ? fr[q % (NR > 0 ? NR : 1)] : fa;
+                acc[q & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[q & 3], 0, 0, 0);
+                if constexpr (NR > 0 && q < NR) fr[q] = probe_dsread(raddr);
+            });
+            if constexpr (NM == 0) probe_for<NR>([&](auto q_c) { fr[decltype(q_c)::value] = probe_dsread(raddr); });
+            if constexpr (NR > 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if constexpr (ND + NV > 0) probe_wait_vmcnt<(DEPTH - 1) * (ND + NV)>();
+            if constexpr (SYNC > 0) {
+                if constexpr (d % SYNC == SYNC - 1) __syncthreads();
+            }
+        });
+    }
+    probe_wait_vmcnt<0>();
+    int s = acc[0][0] + acc[1][1] + acc[2][2] + acc[3][3] + fa.x + lds[65536 + tid];
+    for (int d = 0; d < DEPTH; ++d) s += vg[d][0].x;
+    for (int j = 0; j < (NR > 0 ? NR : 1); ++j) s += fr[j].x;
+    sink[blockIdx.x * 256 + tid] = s;
+}
+
+struct FeedMix {
+    int mfma, lds_reads, dma, reg_loads;
+    void (*kernel)(const uint8_t *, int, int *);
+};
+const FeedMix kFeedMixes[] = {
+    {0, 0, 4, 0, feed_probe_kernel<0, 0, 4, 0, 1, 0>},    // 0: direct-to-LDS loads alone
+    {0, 8, 0, 0, feed_probe_kernel<0, 8, 0, 0, 1, 0>},    // 1: fragment reads alone
+    {4, 0, 0, 0, feed_probe_kernel<4, 0, 0, 0, 1, 0>},    // 2: matrix instructions alone
+    {4, 4, 2, 0, feed_probe_kernel<4, 4, 2, 0, 1, 4>},    // 3: 128 x 128 tile, 128-byte slabs
+    {4, 4, 4, 0, feed_probe_kernel<4, 4, 4, 0, 1, 2>},    // 4: 64 x 64 tile with the reduction split over the waves, 256-byte slabs
+    {8, 6, 3, 0, feed_probe_kernel<8, 6, 3, 0, 1, 4>},    // 5: 256 x 128 tile
+    {16, 8, 4, 0, feed_probe_kernel<16, 8, 4, 0, 1, 4>},  // 6: 256 x 256 tile
+    {4, 2, 1, 2, feed_probe_kernel<4, 2, 1, 2, 2, 4>},    // 7: 128 x 128 with the weight operand straight into registers
+    {16, 4, 2, 4, feed_probe_kernel<16, 4, 2, 4, 2, 4>},  // 8: 256 x 256 likewise
+};
+
 }  // namespace
 }  // namespace eh
 
 using namespace eh;
+
+extern "C" int eh_probe_feed(int32_t mix, int32_t workgroups, int32_t iterations, double *ns_per_iteration, int32_t *per_iteration) {
+    constexpr int MIXES = (int)(sizeof(kFeedMixes) / sizeof(kFeedMixes[0]));
+    EH_REQUIRE(mix >= 0 && mix < MIXES && ns_per_iteration != nullptr, "feed probe: mix 0 .. %d", MIXES - 1);
+    EH_REQUIRE(workgroups >= 1 && workgroups <= 4096 && iterations >= 4 && iterations <= (1 << 20) && iterations % 4 == 0,
+               "feed probe: 1 .. 4096 workgroups, a multiple of four iterations up to 2^20");
+    const FeedMix &m = kFeedMixes[mix];
+    if (per_iteration) {
+        per_iteration[0] = m.mfma;
+        per_iteration[1] = m.lds_reads;
+        per_iteration[2] = m.dma;
+        per_iteration[3] = m.reg_loads;
+    }
+    uint8_t *src = nullptr;
+    int *sink = nullptr;
+    EH_HIP(hipMalloc(reinterpret_cast<void **>(&src), 8ull * kFeedRegion + 65536));
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&sink), (size_t)workgroups * 256 * sizeof(int));
+    if (e != hipSuccess) {
+        (void)hipFree(src);
+        return hip_fail(e, "hipMalloc(feed probe sink)");
+    }
+    (void)hipMemset(src, 1, 8ull * kFeedRegion + 65536);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    hipLaunchKernelGGL(m.kernel, dim3(workgroups), dim3(256), 0, 0, src, 64, sink);  // warm-up: the region is in L2 afterwards
+    (void)hipEventRecord(e0, 0);
+    hipLaunchKernelGGL(m.kernel, dim3(workgroups), dim3(256), 0, 0, src, iterations, sink);
+    (void)hipEventRecord(e1, 0);
+    e = hipEventSynchronize(e1);
+    float ms = 0;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    (void)hipFree(src);
+    if (e != hipSuccess) return hip_fail(e, "feed probe");
+    *ns_per_iteration = (double)ms * 1e6 / iterations;
+    return EH_OK;
+}
 
 extern "C" int eh_probe_stream(const void *src, void *dst, int64_t out_bytes, int32_t mode, void *stream) {
     EH_REQUIRE(src && dst && out_bytes > 0 && (out_bytes & 15) == 0 && out_bytes < (1ll << 35), "stream probe: %lld bytes", (long long)out_bytes);

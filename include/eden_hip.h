@@ -215,6 +215,14 @@ int eh_graph_destroy(void *graph);
  * ceiling the benchmark prints beside the published peak; no counterpart in the
  * reference.  Synchronous; allocates and frees a small device buffer. */
 int eh_probe_mfma_i8(int32_t iterations, int32_t toggling_operands, double *tops);
+/* What a CU's matrix pipe can be fed with: `workgroups` workgroups of four waves repeat an iteration of so many matrix
+ * instructions, 16-byte-per-lane LDS fragment reads, 1 KiB direct-to-LDS loads from an L2-resident region and 1 KiB
+ * loads into registers per wave (returned in per_iteration[0..3], may be NULL), in the proportions of a GEMM tile's
+ * inner loop.  mix: 0 direct-to-LDS loads alone, 1 fragment reads alone, 2 matrix instructions alone, 3 the 128x128
+ * tile, 4 the 64x64 split-reduction tile, 5 256x128, 6 256x256, 7 / 8 the 128x128 / 256x256 tile with the weight
+ * operand loaded straight into registers.  Returns the nanoseconds one iteration takes (all workgroups in parallel).
+ * A yardstick like eh_probe_mfma_i8; no counterpart in the reference.  Synchronous; allocates and frees 8 MiB. */
+int eh_probe_feed(int32_t mix, int32_t workgroups, int32_t iterations, double *ns_per_iteration, int32_t *per_iteration);
 /* A kernel that only moves bytes (16 per lane, whole lines per wave), launched on `stream`:
  * the yardstick beside the HBM-bound kernels' figures.  mode 0 copies out_bytes; mode 1
  * writes every 16-byte source chunk six times (reads out_bytes / 6: the ratio of a 24 -> 144
