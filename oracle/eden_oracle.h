@@ -30,8 +30,13 @@
  *                            pinned by reduction: the result + 128 equals the uint8 function above on every byte,
  *                                    zero point and clamp bound + 128; no reference vector exists for them
  *   eo_nchw2nhwc_u8 / eo_nhwc2nchw_u8  pinned: round trip + index closed form
- *   eo_add_u8 / eo_avgpool_u8 / eo_avgpool_s8
- *                            parity unpinned by reference vectors (closed-form checks only)
+ *   eo_add_u8 / eo_avgpool_u8
+ *                            no reference vector exists (the reference's add and average-pool tests are float only);
+ *                                    pinned by mathematics: every output against exact rational arithmetic over all byte
+ *                                    pairs (add) or a sweep of windows, strides and paddings (pool), with mutants of
+ *                                    the plausible mistakes (swapped multipliers, a shift off by one; a divisor that
+ *                                    counts padded taps, truncation, ties to even) failing the same checks
+ *   eo_avgpool_s8            parity unpinned by reference vectors (closed forms and exact rational arithmetic only)
  */
 #ifndef EDEN_ORACLE_H_
 #define EDEN_ORACLE_H_
