@@ -150,19 +150,24 @@ def fc_workload(eden, synth, m=256, k=4096, n=4096, cold=False):
                 host=(a, w, b, q), out=per_set[0][1], out_shape=(m, n))
 
 
-def conv_workload(eden, synth, n=1, cold=False):
-    desc = eden.conv_desc(n, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=eden.NHWC)
-    x = synth.fill_u8((n, 56, 56, 64), SEED + 16)
-    w = synth.fill_u8((64, 64, 3, 3), SEED + 17)
-    b = synth.fill_i32((64,), SEED + 18, -1000, 1000)
-    q = eden.make_requant(0.02, 128, 0.005, 120, 0.05, 0, eden.ACT_RELU, True)
+def conv_workload(eden, synth, n=1, cold=False, cin=64, cout=64, hw=56, k=3, stride=1):
+    """k x k convolution, ReLU, channels-last: BASELINE configs[0] (3x3, 64 -> 64 channels at 56 x 56) by default"""
+    pad = k // 2
+    ho = (hw + 2 * pad - k) // stride + 1
+    desc = eden.conv_desc(n, cin, hw, hw, cout, k, k, stride=(stride, stride), pad=(pad,) * 4, layout=eden.NHWC)
+    x = synth.fill_u8((n, hw, hw, cin), SEED + 16)
+    w = synth.fill_u8((cout, cin, k, k), SEED + 17)
+    b = synth.fill_i32((cout,), SEED + 18, -1000, 1000)
+    q = eden.make_requant(0.02, 128, 0.005, 120, 0.05 * (cin * k * k / 576.0) ** 0.5, 0, eden.ACT_RELU, True)
     d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
     plan = eden.ConvPlan(desc, d_w, d_b, q)
-    nbytes = 2 * n * 56 * 56 * 64 + 64 * 576 + 256
+    nbytes = n * hw * hw * cin + n * ho * ho * cout + cout * cin * k * k + 4 * cout
     sets = set_count(nbytes, cold)
-    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 56 * 56 * 64)) for _ in range(sets)]
-    return dict(name="conv3x3_n%d_c64_56x56_nhwc" % n, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
-                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 56 * 56 * 64 * 576, bytes=nbytes, bound="mfma")
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * ho * ho * cout)) for _ in range(sets)]
+    name = "conv3x3_n%d_c64_56x56_nhwc" % n if (cin, cout, hw, k, stride) == (64, 64, 56, 3, 1) else \
+        "conv%dx%ds%d_n%d_%dto%d_%dx%d_nhwc" % (k, k, stride, n, cin, cout, hw, hw)
+    return dict(name=name, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * ho * ho * cout * cin * k * k, bytes=nbytes, bound="mfma")
 
 
 def dw_workload(eden, synth, n=32, cold=False, c=144, hw=56, stride=2, k=3):
@@ -530,6 +535,9 @@ def main():
     if args.only and args.only.startswith("pw:"):      # pw:N,CIN,COUT,HW = that pointwise convolution
         n, cin, cout, hw = (int(v) for v in args.only[3:].split(","))
         families[args.only] = shaped(pw_workload, n=n, cin=cin, cout=cout, hw=hw)
+    if args.only and args.only.startswith("conv:"):    # conv:N,CIN,COUT,HW,K,STRIDE = that convolution
+        n, cin, cout, hw, k, stride = (int(v) for v in args.only[5:].split(","))
+        families[args.only] = shaped(conv_workload, n=n, cin=cin, cout=cout, hw=hw, k=k, stride=stride)
     if args.only and args.only.startswith("dw:"):      # dw:N,C,HW,STRIDE[,K] = that depthwise convolution
         v = [int(t) for t in args.only[3:].split(",")]
         families[args.only] = shaped(dw_workload, n=v[0], c=v[1], hw=v[2], stride=v[3], k=v[4] if len(v) > 4 else 3)

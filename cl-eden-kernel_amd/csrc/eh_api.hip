@@ -471,6 +471,9 @@ struct eh_dwconv_plan {
     int32_t *w_trip = nullptr, *bias_trip = nullptr;
     int32_t *w_fold = nullptr, *bias_fold = nullptr;  // the unsigned form of the same plans, for weights of any range
     bool fold_valid = false;
+    // 5x5 / 7x7 channels-last plans: the unsigned form with two words per kernel column
+    int32_t *w_foldk = nullptr, *bias_foldk = nullptr;
+    bool foldk_valid = false;
     bool range_known = false;   // w_lo / w_hi hold the extremes of the weight bytes (in the caller's own domain)
     int32_t w_lo = 0, w_hi = 0;
     bool trip_valid = false;    // w_trip / bias_trip match the current zero points
@@ -1310,6 +1313,8 @@ static void dw_release(eh_dwconv_plan *pl) {
     dev_free(pl->bias_trip);
     dev_free(pl->w_fold);
     dev_free(pl->bias_fold);
+    dev_free(pl->w_foldk);
+    dev_free(pl->bias_foldk);
 }
 
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
@@ -1347,6 +1352,13 @@ static int dw_refold(eh_dwconv_plan *pl, const eh_requant &caller_q, hipStream_t
                                      q.zp_w + (pl->w_signed ? 128 : 0), pl->w_signed ? 1 : 0, stream);
             if (rc) return rc;
             pl->fold_valid = true;
+        }
+        pl->foldk_valid = false;
+        if (pl->w_foldk) {
+            rc = launch_dw_pack_foldk(pl->w_copy, pl->has_bias ? pl->bias_copy : nullptr, pl->w_foldk, pl->bias_foldk, pl->cout, pl->d.kh, q.zp_in,
+                                      q.zp_w + (pl->w_signed ? 128 : 0), pl->w_signed ? 1 : 0, stream);
+            if (rc) return rc;
+            pl->foldk_valid = true;
         }
         pl->packed_valid = true;
     }
@@ -1398,6 +1410,12 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
         if (!rc) rc = dev_alloc(&pl->bias_trip, (size_t)pl->cout + 4);
         if (!rc) rc = dev_alloc(&pl->w_fold, (size_t)3 * pl->cout);
         if (!rc) rc = dev_alloc(&pl->bias_fold, (size_t)pl->cout + 4);
+    }
+    const bool tile_form_k = pl->d.layout == EH_NHWC && pl->d.kh == pl->d.kw && (pl->d.kh == 5 || pl->d.kh == 7) && pl->d.depth_multiplier == 1 &&
+                             pl->d.dil_h == 1 && pl->d.dil_w == 1;
+    if (!rc && tile_form_k) {
+        rc = dev_alloc(&pl->w_foldk, (size_t)pl->d.kw * 2 * pl->cout);
+        if (!rc) rc = dev_alloc(&pl->bias_foldk, (size_t)pl->cout + 4);
     }
     if (!rc) rc = dw_set_weights(pl, weight, bias, s);
     if (!rc && tile_form && pl->cout > 0) {
@@ -1492,6 +1510,8 @@ static DwProblem dw_problem(const eh_dwconv_plan *plan, const void *input, void 
     p.bias_trip = plan->bias_trip;
     p.w_fold = plan->fold_valid ? plan->w_fold : nullptr;
     p.bias_fold = plan->bias_fold;
+    p.w_foldk = plan->foldk_valid ? plan->w_foldk : nullptr;
+    p.bias_foldk = plan->bias_foldk;
     p.io_flip = plan->io_signed ? 0x80808080u : 0u;
     p.rq = make_requant_dev(plan->q);
     if (plan->pc_multiplier) {

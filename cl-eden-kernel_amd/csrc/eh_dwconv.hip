@@ -336,6 +336,137 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
     }
 }
 
+// 5x5 and 7x7 kernels with the same tile (four adjacent channels of four horizontally adjacent output pixels per thread)
+// and the unsigned dot-product form.  The tile's input columns are walked one at a time: a column's K words (one per
+// row, four channels each) are turned into two words per channel holding its vertical taps 0..3 and 4..K-1, whose dot
+// products with the kernel column kx = x - j S go to every output j of the tile that the column lies under, and whose
+// byte sum goes to those outputs' zero-point term.  A kernel column's two weight words are read when the walk first
+// needs them and are used by four consecutive (stride 2: every other) input columns.  Replaces the one-pixel kernel's
+// K*K 16-bit multiply-adds per output by 2 K dot products shared between the tile's pixels.
+template <int K, int S, bool FLIP>
+__global__ __launch_bounds__(256) void dwkxk_nhwc_tile4_kernel(const DwProblem p, const uint32_t total, const int tiles_x, const FastDiv div_cq,
+                                                               const FastDiv div_tiles, const FastDiv div_ho) {
+    static_assert(K == 5 || K == 7, "two words per kernel column: four taps and the other one or three");
+    constexpr int TW = 4, IW = (TW - 1) * S + K;
+    const uint32_t idx = xcd_contiguous_block() * 256u + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t cq_count = (uint32_t)p.c >> 2;
+    uint32_t r = fastdiv(idx, div_cq);
+    const uint32_t cq = idx - r * cq_count;
+    const uint32_t r2 = fastdiv(r, div_tiles);
+    const int tx = (int)(r - r2 * (uint32_t)tiles_x);
+    const uint32_t img = fastdiv(r2, div_ho);
+    const int oy = (int)(r2 - img * (uint32_t)p.ho);
+    const int ox0 = tx * TW;
+    const int iy0 = oy * S - p.pad_t, ix0 = ox0 * S - p.pad_l;
+    const uint32_t fill = (uint32_t)p.zp_in * 0x01010101u;
+    const uint32_t flip_word = FLIP ? 0x80808080u : 0u;  // int8 tensors: the bytes as uint8 values
+    const uint32_t base = img * (uint32_t)(p.h * p.w_ * p.c) + cq * 4u;
+    const int row_pitch = p.w_ * p.c;
+    const bool inside = iy0 >= 0 && iy0 + K - 1 < p.h && ix0 >= 0 && ix0 + IW - 1 < p.w_;
+    const bool all_inside = __builtin_amdgcn_ballot_w64(!inside) == 0;
+    const uint8_t *src = p.in + (base + (uint32_t)__mul24(iy0 < 0 ? 0 : iy0, row_pitch) + (uint32_t)__mul24(ix0 < 0 ? 0 : ix0, p.c));
+    uint32_t row_off[K];
+    bool row_ok[K];
+#pragma unroll
+    for (int ky = 0; ky < K; ++ky) {
+        const int iy = iy0 + ky;
+        row_ok[ky] = (unsigned)iy < (unsigned)p.h;
+        const int iyc = iy < 0 ? 0 : (iy >= p.h ? p.h - 1 : iy);
+        row_off[ky] = base + (uint32_t)__mul24(iyc, row_pitch);
+    }
+    const int4 b4 = *reinterpret_cast<const int4 *>(p.bias_foldk + cq * 4u);
+    int acc[TW][4], csum[TW][4];
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        acc[j][0] = b4.x;
+        acc[j][1] = b4.y;
+        acc[j][2] = b4.z;
+        acc[j][3] = b4.w;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) csum[j][c] = 0;
+    }
+    auto load_column = [&](int x, uint32_t (&rows)[K]) {
+        if (all_inside) {
+#pragma unroll
+            for (int ky = 0; ky < K; ++ky) rows[ky] = *reinterpret_cast<const uint32_t *>(src + (uint32_t)(ky * row_pitch + x * p.c)) ^ flip_word;
+        } else {
+            const int ix = ix0 + x;
+            const bool col_ok = (unsigned)ix < (unsigned)p.w_;
+            const uint32_t col_off = (uint32_t)__mul24(ix < 0 ? 0 : (ix >= p.w_ ? p.w_ - 1 : ix), p.c);
+#pragma unroll
+            for (int ky = 0; ky < K; ++ky) {
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in + (row_off[ky] + col_off)) ^ flip_word;
+                rows[ky] = row_ok[ky] && col_ok ? v : fill;
+            }
+        }
+    };
+    // The walk is fenced column by column: left alone the compiler requests every column and every weight word at the
+    // top (170 registers for 7x7, two waves per SIMD); fenced, a column's words and the weights of the kernel column
+    // that enters with it are requested one column ahead.
+    int4 wk[K][2];
+    auto load_weights = [&](int kx) {
+        wk[kx][0] = *reinterpret_cast<const int4 *>(p.w_foldk + ((uint32_t)(kx * 2) * (uint32_t)p.cout + cq * 4u));
+        wk[kx][1] = *reinterpret_cast<const int4 *>(p.w_foldk + ((uint32_t)(kx * 2 + 1) * (uint32_t)p.cout + cq * 4u));
+    };
+    uint32_t ahead[K];
+    load_column(0, ahead);
+    load_weights(0);
+#pragma unroll
+    for (int x = 0; x < IW; ++x) {
+        uint32_t rows[K];
+#pragma unroll
+        for (int ky = 0; ky < K; ++ky) rows[ky] = ahead[ky];
+        if (x + 1 < K) load_weights(x + 1);  // the kernel column that enters the walk at the next input column
+        if (x + 1 < IW) load_column(x + 1, ahead);
+        __builtin_amdgcn_sched_barrier(0);
+        // rows 0..3: a 4 x 4 byte transpose; the rest: the three-row gather of the 3x3 kernel, or single bytes
+        uint32_t lo[4], hi[4];
+        {
+            const uint32_t t0 = __builtin_amdgcn_perm(rows[1], rows[0], 0x05010400u), t1 = __builtin_amdgcn_perm(rows[1], rows[0], 0x07030602u);
+            const uint32_t u0 = __builtin_amdgcn_perm(rows[3], rows[2], 0x05010400u), u1 = __builtin_amdgcn_perm(rows[3], rows[2], 0x07030602u);
+            lo[0] = __builtin_amdgcn_perm(u0, t0, 0x05040100u);
+            lo[1] = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
+            lo[2] = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
+            lo[3] = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
+        }
+        if constexpr (K == 7) {
+            column_words(rows[4], rows[5], rows[6], hi);
+        } else {
+            hi[0] = rows[4] & 0xFFu;
+            hi[1] = (rows[4] >> 8) & 0xFFu;
+            hi[2] = (rows[4] >> 16) & 0xFFu;
+            hi[3] = rows[4] >> 24;
+        }
+        int cs[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) cs[c] = udot4(hi[c], 0x01010101u, udot4(lo[c], 0x01010101u, 0));
+#pragma unroll
+        for (int j = 0; j < TW; ++j) {
+            const int kx = x - j * S;
+            if (kx < 0 || kx >= K) continue;
+            acc[j][0] = udot4(hi[0], (uint32_t)wk[kx][1].x, udot4(lo[0], (uint32_t)wk[kx][0].x, acc[j][0]));
+            acc[j][1] = udot4(hi[1], (uint32_t)wk[kx][1].y, udot4(lo[1], (uint32_t)wk[kx][0].y, acc[j][1]));
+            acc[j][2] = udot4(hi[2], (uint32_t)wk[kx][1].z, udot4(lo[2], (uint32_t)wk[kx][0].z, acc[j][2]));
+            acc[j][3] = udot4(hi[3], (uint32_t)wk[kx][1].w, udot4(lo[3], (uint32_t)wk[kx][0].w, acc[j][3]));
+#pragma unroll
+            for (int c = 0; c < 4; ++c) csum[j][c] += cs[c];
+        }
+    }
+    uint8_t *dst = p.out + (((img * (uint32_t)p.ho + (uint32_t)oy) * (uint32_t)p.wo + (uint32_t)ox0) * (uint32_t)p.cout + cq * 4u);
+    const RequantDev rq = p.rq;
+    const ChannelQuad quad{};
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+        // (K * K bytes times a zero point of at most 383: a 24-bit multiply-add)
+        const int a0 = acc[j][0] + __mul24(-p.zp_w, csum[j][0]), a1 = acc[j][1] + __mul24(-p.zp_w, csum[j][1]);
+        const int a2 = acc[j][2] + __mul24(-p.zp_w, csum[j][2]), a3 = acc[j][3] + __mul24(-p.zp_w, csum[j][3]);
+        uint32_t o = requant4<false>(a0, a1, a2, a3, rq, quad);
+        if (FLIP) o ^= 0x80808080u;
+        if (ox0 + j < p.wo) *reinterpret_cast<uint32_t *>(dst + (uint32_t)j * (uint32_t)p.cout) = o;
+    }
+}
+
 // One output element per thread; any depth multiplier, dilation, channel count.
 // NHWC = true: channel fastest.  NHWC = false: planar NCHW, x fastest.
 template <bool NHWC>
@@ -438,7 +569,36 @@ __global__ void dw_pack_fold_kernel(const uint8_t *w, const int32_t *bias, int32
     bias_fold[oc] = (bias ? bias[oc] : 0) - zp_in * sum + 9 * zp_in * zp_w;
 }
 
+// K x K weights [cout][K*K] -> w_foldk[kx][2][cout]: the vertical taps 0..3 and 4..K-1 of column kx as uint8 bytes (int8
+// weights: byte + 128, `zp_w` being their zero point + 128); bias_foldk[c] = bias - zp_in * sum w + K K zp_in zp_w
+__global__ void dw_pack_foldk_kernel(const uint8_t *w, const int32_t *bias, int32_t *w_foldk, int32_t *bias_foldk, int32_t cout, int32_t k,
+                                     int32_t zp_in, int32_t zp_w, int32_t w_signed) {
+    const int oc = blockIdx.x * blockDim.x + threadIdx.x;
+    if (oc >= cout) return;
+    int32_t sum = 0;
+    for (int kx = 0; kx < k; ++kx) {
+        uint32_t word[2] = {0, 0};
+        for (int ky = 0; ky < k; ++ky) {
+            const uint32_t v = (uint32_t)w[(size_t)oc * k * k + ky * k + kx] ^ (w_signed ? 0x80u : 0u);
+            sum += (int32_t)v;
+            word[ky >> 2] |= v << (8 * (ky & 3));
+        }
+        w_foldk[(size_t)(kx * 2) * cout + oc] = (int32_t)word[0];
+        w_foldk[(size_t)(kx * 2 + 1) * cout + oc] = (int32_t)word[1];
+    }
+    bias_foldk[oc] = (bias ? bias[oc] : 0) - zp_in * sum + k * k * zp_in * zp_w;
+}
+
 }  // namespace
+
+int launch_dw_pack_foldk(const uint8_t *w, const int32_t *bias, int32_t *w_foldk, int32_t *bias_foldk, int32_t cout, int32_t k,
+                         int32_t zp_in, int32_t zp_w_u8, int32_t w_signed, hipStream_t stream) {
+    if (cout <= 0) return EH_OK;
+    hipLaunchKernelGGL(dw_pack_foldk_kernel, dim3((cout + 127) / 128), dim3(128), 0, stream, w, bias, w_foldk, bias_foldk, cout, k, zp_in,
+                       zp_w_u8, w_signed);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
 
 int launch_dw_pack_fold(const uint8_t *w, const int32_t *bias, int32_t *w_fold, int32_t *bias_fold, int32_t cout, int32_t zp_in,
                         int32_t zp_w_u8, int32_t w_signed, hipStream_t stream) {
@@ -479,6 +639,31 @@ int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
     const bool tile3x3 = vec && p.kh == 3 && p.kw == 3 && p.dil_h == 1 && p.dil_w == 1 && p.stride_h == p.stride_w &&
                          (p.stride_h == 1 || p.stride_h == 2) && (size_t)p.n * p.h * p.w_ * p.c < (1ull << 31) &&
                          (size_t)p.n * p.ho * p.wo * p.cout < (1ull << 31);
+    const bool tile_kxk = vec && p.w_foldk != nullptr && p.kh == p.kw && (p.kh == 5 || p.kh == 7) && p.dil_h == 1 && p.dil_w == 1 && p.dm == 1 &&
+                          (p.c & 3) == 0 && p.stride_h == p.stride_w && (p.stride_h == 1 || p.stride_h == 2) && p.rq.pc_multiplier == nullptr &&
+                          p.pad_t >= 0 && p.pad_l >= 0 && (size_t)p.n * p.h * p.w_ * p.c < (1ull << 31) &&
+                          (size_t)p.n * p.ho * p.wo * p.cout < (1ull << 31) && (long)p.w_ * p.c < (1l << 23) && p.h < (1 << 23);
+    if (tile_kxk) {
+        DwProblem q = p;
+        q.zp_w += q.w_signed ? 128 : 0;  // zero point of the uint8 values the unsigned form multiplies
+        const int tiles_x = (q.wo + 3) / 4;
+        const long total = (long)q.n * q.ho * tiles_x * (q.c >> 2);
+        EH_REQUIRE(total < (1l << 31), "depthwise: grid too large");
+        const long blocks = (total + 255) / 256;
+        const FastDiv d_cq = make_fastdiv((uint32_t)(q.c >> 2)), d_t = make_fastdiv((uint32_t)tiles_x), d_ho = make_fastdiv((uint32_t)q.ho);
+        const bool flip = q.io_flip != 0;
+        auto pick = [&](auto k_c, auto s_c) {
+            constexpr int K = decltype(k_c)::value, S = decltype(s_c)::value;
+            return flip ? dwkxk_nhwc_tile4_kernel<K, S, true> : dwkxk_nhwc_tile4_kernel<K, S, false>;
+        };
+        using one = std::integral_constant<int, 1>;
+        using two = std::integral_constant<int, 2>;
+        auto kernel = q.kh == 5 ? (q.stride_h == 1 ? pick(std::integral_constant<int, 5>{}, one{}) : pick(std::integral_constant<int, 5>{}, two{}))
+                                : (q.stride_h == 1 ? pick(std::integral_constant<int, 7>{}, one{}) : pick(std::integral_constant<int, 7>{}, two{}));
+        hipLaunchKernelGGL(kernel, dim3((unsigned)((blocks + 7) / 8 * 8)), dim3(256), 0, stream, q, (uint32_t)total, tiles_x, d_cq, d_t, d_ho);
+        EH_HIP(hipGetLastError());
+        return EH_OK;
+    }
     if (tile3x3) {
         const int tiles_x = (p.wo + 3) / 4;
         const long total = (long)p.n * p.ho * tiles_x * (p.c >> 2);

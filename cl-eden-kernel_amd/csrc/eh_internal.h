@@ -476,6 +476,10 @@ struct DwProblem {
     // weight bytes (int8 weights: byte + 128), and the bias with -zp_in * sum w + 9 zp_in zp_w folded in
     const int32_t *w_fold;
     const int32_t *bias_fold;
+    // 5x5 and 7x7 weights of any range for the same form (else null): [kw columns][2][cout] words of a column's
+    // vertical taps 0..3 and 4..kh-1 as uint8 bytes, and the bias with -zp_in * sum w + kh kw zp_in zp_w folded in
+    const int32_t *w_foldk;
+    const int32_t *bias_foldk;
     uint8_t *out;
     int32_t n, c, h, w_, cout, dm;
     int32_t kh, kw, stride_h, stride_w, pad_t, pad_l, dil_h, dil_w;
@@ -491,6 +495,8 @@ int launch_dw_pack_trip(const uint8_t *w, const int32_t *bias, int32_t *w_trip, 
                         int32_t zp_w, int32_t w_signed, hipStream_t stream);
 int launch_dw_pack_fold(const uint8_t *w, const int32_t *bias, int32_t *w_fold, int32_t *bias_fold, int32_t cout, int32_t zp_in,
                         int32_t zp_w_u8, int32_t w_signed, hipStream_t stream);
+int launch_dw_pack_foldk(const uint8_t *w, const int32_t *bias, int32_t *w_foldk, int32_t *bias_foldk, int32_t cout, int32_t k,
+                         int32_t zp_in, int32_t zp_w_u8, int32_t w_signed, hipStream_t stream);
 int launch_dwconv_nhwc(const DwProblem &p, hipStream_t stream);
 int launch_dwconv_nchw(const DwProblem &p, hipStream_t stream);
 

@@ -85,6 +85,7 @@ DW_CASES = [
     dict(n=2, c=32, h=15, w=14, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),
     dict(n=2, c=24, h=15, w=17, cout=24, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),
     dict(n=1, c=16, h=12, w=12, cout=16, kh=5, kw=5, stride=(1, 1), pad=(2, 2, 2, 2)),
+    dict(n=2, c=8, h=17, w=15, cout=8, kh=7, kw=7, stride=(2, 2), pad=(3, 3, 3, 3)),
     dict(n=2, c=5, h=9, w=8, cout=10, kh=3, kw=3, stride=(2, 1), pad=(1, 0, 1, 1), dm=2),
 ]
 

@@ -422,6 +422,15 @@ DW_CASES = [
     dict(n=1, c=12, h=3, w=1, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1)),
     dict(n=1, c=6, h=12, w=10, cout=12, kh=3, kw=2, stride=(2, 1), pad=(2, 2, 1, 1), dil=(2, 3), dm=2),   # dilation, stride and depth multiplier
     dict(n=2, c=32, h=16, w=16, cout=32, kh=3, kw=3, stride=(2, 2), pad=(2, 2, 2, 2), dil=(2, 2)),
+    # 5x5 and 7x7 tiles of four output pixels (two words per kernel column): both strides, ragged widths, every border,
+    # an image smaller than the kernel
+    dict(n=2, c=16, h=13, w=11, cout=16, kh=5, kw=5, pad=(2, 2, 2, 2)),
+    dict(n=1, c=24, h=14, w=14, cout=24, kh=5, kw=5, stride=(2, 2), pad=(2, 2, 2, 2)),
+    dict(n=2, c=8, h=15, w=17, cout=8, kh=7, kw=7, pad=(3, 3, 3, 3)),
+    dict(n=1, c=32, h=20, w=18, cout=32, kh=7, kw=7, stride=(2, 2), pad=(3, 2, 3, 2)),
+    dict(n=1, c=12, h=4, w=3, cout=12, kh=5, kw=5, pad=(2, 2, 2, 2)),
+    dict(n=3, c=144, h=28, w=28, cout=144, kh=5, kw=5, pad=(2, 2, 2, 2)),
+    dict(n=1, c=4, h=9, w=9, cout=4, kh=7, kw=7),
 ]
 
 
