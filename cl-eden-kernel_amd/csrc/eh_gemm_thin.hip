@@ -107,13 +107,17 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
 
     const RequantDev rq = p.rq;
     const bool wide = (p.ldc & 3) == 0 && ((reinterpret_cast<uintptr_t>(p.out) & 3) == 0);  // dword-aligned rows: vector stores
-    const int rb_stride = gridDim.x * 4;
+    // XCD x (workgroups x, x + 8, ...: gridDim.x is a multiple of 8) owns the x-th contiguous eighth of the row blocks
+    const int rb_per_xcd = (row_blocks + 7) >> 3;
+    const int rb_first = (int)(blockIdx.x & 7u) * rb_per_xcd + (int)(blockIdx.x >> 3) * 4 + wave;
+    const int rb_end = ((int)(blockIdx.x & 7u) + 1) * rb_per_xcd < row_blocks ? ((int)(blockIdx.x & 7u) + 1) * rb_per_xcd : row_blocks;
+    const int rb_stride = (int)(gridDim.x >> 3) * 4;
     constexpr bool SINGLE = KU < 4;  // the whole reduction is one group of KU steps (the launcher guarantees ksteps <= KU)
 
     // where the lane's pixel of row block `rb` reads and writes
     auto locate = [&](int rb, bool &ok, size_t &in_off, size_t &out_off) {
         const int m = rb * 32 + r;
-        ok = rb < row_blocks && m < p.m;
+        ok = rb < rb_end && m < p.m;
         in_off = 0;
         out_off = 0;
         if (ok && stage.linear) {
@@ -269,12 +273,12 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         bool ok, ok_next;
         size_t in_off, out_off, in_next, out_next;
         uint2 lo[KU], hi[KU], lo_next[KU], hi_next[KU];
-        int rb = blockIdx.x * 4 + wave;
+        int rb = rb_first;
         locate(rb, ok, in_off, out_off);
 #pragma unroll
         for (int t = 0; t < KU; ++t) load_a(ok, in_off, t, lo[t], hi[t]);
         stage_weights();  // after the first activation loads are on their way: the two latencies overlap
-        for (; rb < row_blocks; rb += rb_stride) {
+        for (; rb < rb_end; rb += rb_stride) {
             locate(rb + rb_stride, ok_next, in_next, out_next);
 #pragma unroll
             for (int t = 0; t < KU; ++t) load_a(ok_next, in_next, t, lo_next[t], hi_next[t]);
@@ -319,7 +323,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
         }
     } else {
         stage_weights();
-        for (int rb = blockIdx.x * 4 + wave; rb < row_blocks; rb += rb_stride) {
+        for (int rb = rb_first; rb < rb_end; rb += rb_stride) {
             bool ok;
             size_t in_off, out_off;
             locate(rb, ok, in_off, out_off);
@@ -415,8 +419,8 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
             per_cu = n < 4 ? 4 : (n > 8 ? 8 : n);
             resident[slot].store(per_cu, std::memory_order_relaxed);
         }
-        int row_wgs = (row_blocks + 3) / 4;
-        const int wg_target = 256 * per_cu / ranges > 0 ? 256 * per_cu / ranges : 1;
+        int row_wgs = ((row_blocks + 7) / 8 + 3) / 4 * 8;   // a multiple of 8: every XCD walks its own eighth of the row blocks
+        const int wg_target = 256 * per_cu / ranges > 8 ? 256 * per_cu / ranges / 8 * 8 : 8;
         if (row_wgs > wg_target) row_wgs = wg_target;
         hipLaunchKernelGGL(kernel, dim3(row_wgs, ranges), dim3(256), lds_all, stream, p, n_blocks, ksteps, nbw, row_blocks, stage);
     };
