@@ -504,6 +504,7 @@ def main():
                     pw7=shaped(pw_workload, n=64, cin=160, cout=960, hw=7), pj7=shaped(pw_workload, n=64, cin=960, cout=160, hw=7),
                     c3blockbig=shaped(block_workload, n=256),
                     dwbig=shaped(dw_workload, n=256), pwbig=shaped(pw_workload, n=256),
+                    dw5x5=shaped(dw_workload, n=64, c=144, hw=56, stride=1, k=5), dw7x7=shaped(dw_workload, n=64, c=144, hw=56, stride=1, k=7),
                     copy=copy_workload, mbv2=mbv2_workload, mbv2narrow=shaped(mbv2_workload, weights="narrow"),
                     tonhwc=layout_workload, tonchw=shaped(layout_workload, to_nhwc=False),
                     mbv2pc=shaped(mbv2_workload, per_channel=True),
@@ -628,6 +629,8 @@ def main():
         for make, steps, cold_too in ((conv_workload, 2000, False), (shaped(conv_workload, n=64), 300, False),
                                       (pw_workload, 500, True), (dw_workload, 1000, True), (block_workload, 500, True),
                                       (shaped(pw_workload, n=256), 100, True), (shaped(dw_workload, n=256), 200, True),
+                                      (shaped(dw_workload, n=64, c=144, hw=56, stride=1, k=5), 200, False),
+                                      (shaped(dw_workload, n=64, c=144, hw=56, stride=1, k=7), 200, False),
                                       (deconv_workload, 500, False), (fc_workload, 500, True),
                                       (shaped(fc_workload, m=8192, k=4096, n=4096), 100, False),
                                       (layout_workload, 200, True), (shaped(layout_workload, to_nhwc=False), 200, True),
