@@ -24,7 +24,7 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-W
 # MFMA results straight into ordinary registers for the kernels whose epilogue is the bottleneck (no AGPR -> VGPR
 # copy per output); the big-tile GEMM keeps its accumulators in the AGPR half of the register file
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
-PER_FILE_FLAGS = {"eh_gemm_thin.hip": VGPR_FORM, "eh_block.hip": VGPR_FORM, "eh_conv_c3.hip": VGPR_FORM}
+PER_FILE_FLAGS = {"eh_gemm_thin.hip": VGPR_FORM, "eh_block.hip": VGPR_FORM, "eh_conv_c3.hip": VGPR_FORM, "eh_conv_rows.hip": VGPR_FORM}
 
 RESOURCES = os.path.join(OBJ, "kernel_resources.txt")
 

@@ -151,6 +151,18 @@ static bool units_are_3x3(const std::vector<KUnit> &units, int per_tap) {
     return true;
 }
 
+// Whether the load units describe kh x kw taps at dilation 1, row by row, `per_tap` units each; kw = the taps of row 0.
+static bool units_are_rows(const std::vector<KUnit> &units, int per_tap, int taps, int &kh, int &kw) {
+    if (per_tap <= 0 || taps <= 0 || units.size() != (size_t)taps * per_tap) return false;
+    kw = 0;
+    while (kw < taps && units[(size_t)kw * per_tap].dy == 0) ++kw;
+    if (kw == 0 || taps % kw != 0) return false;
+    kh = taps / kw;
+    for (int t = 0; t < taps; ++t)
+        if (units[(size_t)t * per_tap].dy != t / kw || units[(size_t)t * per_tap].dx != t % kw) return false;
+    return true;
+}
+
 // Allocates a part's device arrays and uploads its tables.  `units` holds one
 // KUnit per `vec` bytes of the real reduction length; padding units are added here.
 int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream,
@@ -170,6 +182,14 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         // three channels, 3x3 taps, dilation 1: the first layer of image networks
         g.cfg.id = GEMM_C3K3;
         g.cfg.slab = 32;
+    } else if (int kh = 0, kw = 0; g.cin >= 1 && g.cin <= 4 && g.taps > 1 && g.k == g.taps * g.cin && !units.empty() && units[0].offset == 0 &&
+                                   units_are_rows(units, g.cin / g.vec, g.taps, kh, kw) && conv_rows_applies(g.cin, g.proto.cin, kh, kw) &&
+                                   (long)g.proto.h * g.proto.w * g.cin >= 16) {
+        // one to four input channels, a kernel row within 32 bytes: first layers on RGB(A) or grey images beyond 3x3 RGB
+        g.cfg.id = GEMM_ROWS;
+        g.cfg.slab = 32;
+        g.proto.rows_kh = kh;
+        g.proto.rows_kw = kw;
     } else if (g.vec == 16 && g.taps == 9 && g.k == 9 * g.cin && units.size() == (size_t)g.k / 16 && g.proto.stride_h == 1 &&
                g.proto.stride_w == 1 && g.proto.out_sy == 1 && g.proto.out_sx == 1 && g.proto.out_y0 == 0 && g.proto.out_x0 == 0 &&
                g.proto.out_h == g.proto.ho && g.proto.out_w == g.proto.wo && units_are_3x3(units, g.cin / 16) &&
@@ -179,7 +199,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         g.cfg.slab = 32;
     } else if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
         g.cfg = igemm_dma_select(g.proto.m, g.n, g.k, siblings);
-    g.k_pad = round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
+    g.k_pad = g.cfg.id == GEMM_ROWS ? g.proto.rows_kh * 32 : round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
     g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
     KUnit pad;
     pad.offset = 0;
@@ -232,6 +252,7 @@ int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t str
     pp.taps = g.taps;
     pp.k = g.k;
     pp.k_pad = g.k_pad;
+    pp.row_bytes = g.cfg.id == GEMM_ROWS ? g.proto.rows_kw * g.cin : 0;
     pp.so = g.so;
     pp.sc = g.sc;
     pp.tap_off = g.tap_off;

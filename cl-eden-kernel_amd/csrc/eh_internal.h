@@ -365,6 +365,7 @@ enum GemmConfigId {
     GEMM_THIN = 6,              // one-tap problems short of work for tiles; weights in MFMA fragment order
     GEMM_C3K3 = 7,              // 3 input channels, 3x3 taps (first layers); weights row-major [n_pad][32]
     GEMM_CONV3X3 = 8,           // 3x3 taps, stride 1, input patch staged in LDS once; weights in MFMA fragment order
+    GEMM_ROWS = 9,              // 1 - 4 input channels, kernel rows of at most 32 bytes; weights row-major [n_pad][32 per kernel row]
 };
 struct GemmConfig {
     int32_t id = GEMM_STAGED;
@@ -397,6 +398,7 @@ struct GemmProblem {
     // int8 tensors (PrecisionType::INT8) run as their uint8 equivalents (value + 128, zero points + 128):
     uint32_t a_xor;    // turns four stored activation bytes into int8 MFMA operands: 0x80808080 for uint8 data, 0 for int8
     uint32_t out_xor;  // turns four uint8 results into the stored bytes: 0 for uint8 data, 0x80808080 for int8
+    int32_t rows_kh, rows_kw;  // GEMM_ROWS: the kernel's extent (other kernels find their taps in ktab)
     // fused residual add (one-tap and split-reduction kernels only): out = add(residual, result) with `radd`;
     // `residual` is addressed like `out`.  Null: plain convolution.
     const uint8_t *residual;
@@ -418,6 +420,9 @@ inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
 int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream);
+// few input channels, a kernel row per reduction step (eh_conv_rows.hip)
+bool conv_rows_applies(int32_t cin_group, int32_t pixel_stride, int32_t kh, int32_t kw);
+int launch_conv_rows(const GemmProblem &p, hipStream_t stream);
 int conv3x3_patch_prepare();  // per device, from eh_init
 bool conv3x3_patch_applies(int32_t cin_group, int32_t pixel_stride, int32_t wo, int32_t ho);
 bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, int32_t channel_offset, int32_t y_base,
@@ -429,7 +434,7 @@ bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, i
 // 16h + 4g + t sits in row 8g + 4h + t): a lane of the 32x32x32 MFMA holds result
 // rows 8g + 4h + t (h = lane / 32), which this way are 16 consecutive channels.
 __host__ __device__ inline size_t packed_b_offset(const GemmConfig &cfg, int n, int kc16, int k_pad) {
-    if (cfg.id == GEMM_STAGED || cfg.id == GEMM_C3K3) return (size_t)n * k_pad + (size_t)kc16 * 16;
+    if (cfg.id == GEMM_STAGED || cfg.id == GEMM_C3K3 || cfg.id == GEMM_ROWS) return (size_t)n * k_pad + (size_t)kc16 * 16;
     const int ch = n & 31;
     n = (n & ~31) | (((ch & 15) >> 2) << 3) | ((ch >> 4) << 2) | (ch & 3);
     // fragment order: [32-channel block][32-byte step][lane = 32 * (chunk & 1) + row][16 bytes]
@@ -451,6 +456,7 @@ struct PackProblem {
     int32_t *colsum;       // [n_pad]  sum_k (w - 128)
     GemmConfig cfg;
     int32_t n, n_pad, cin, taps, k, k_pad;
+    int32_t row_bytes;     // GEMM_ROWS: kw * cin, the bytes of a kernel row, which starts every 32 packed bytes; else 0
     // source index of (out channel o, in channel c, tap t) = o*so + c*sc + tap_off[t]
     int64_t so, sc;
     const int32_t *tap_off;  // device [taps]

@@ -19,8 +19,10 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
     int32_t sum = 0;
     for (int k = threadIdx.x; k < p.k_pad; k += 256) {
         int32_t v = 0;
-        if (o < p.n && k < p.k) {
-            const int t = k / p.cin, c = k - t * p.cin;
+        // source position in (tap, channel) order: k itself, or with one kernel row per 32 packed bytes, row * row_bytes + byte
+        const int kk = p.row_bytes ? ((k & 31) < p.row_bytes ? (k >> 5) * p.row_bytes + (k & 31) : p.k) : k;
+        if (o < p.n && kk < p.k) {
+            const int t = kk / p.cin, c = kk - t * p.cin;
             const uint8_t raw = p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]];
             v = p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw - 128;
         }

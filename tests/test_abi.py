@@ -188,6 +188,19 @@ def test_3x3_stride_1_convolutions_take_the_patch_kernel():
         assert "conv3x3_patch" not in eden.conv_kernels(d)
 
 
+def test_few_channel_convolutions_take_the_kernel_row_kernel():
+    nhwc = eden.NHWC
+    assert eden.conv_kernels(eden.conv_desc(64, 3, 224, 224, 64, 7, 7, stride=(2, 2), pad=(3, 3, 3, 3), layout=nhwc)) == ["few_channel_rows"]
+    assert eden.conv_kernels(eden.conv_desc(1, 1, 64, 64, 56, 9, 9, pad=(4, 4, 4, 4), layout=nhwc)) == ["few_channel_rows"]
+    assert eden.conv_kernels(eden.conv_desc(1, 4, 64, 64, 16, 5, 5, layout=nhwc)) == ["few_channel_rows"]
+    assert eden.conv_kernels(eden.conv_desc(1, 1, 64, 64, 16, 3, 3, layout=nhwc)) == ["few_channel_rows"]
+    # RGB 3x3 keeps its own kernel; rows beyond 32 bytes, an even number of rows, dilation, more channels: the implicit GEMM
+    assert eden.conv_kernels(eden.conv_desc(1, 3, 64, 64, 32, 3, 3, layout=nhwc)) == ["c3k3"]
+    for d in (eden.conv_desc(1, 3, 64, 64, 32, 11, 11, layout=nhwc), eden.conv_desc(1, 3, 64, 64, 32, 4, 4, layout=nhwc),
+              eden.conv_desc(1, 3, 64, 64, 32, 5, 5, dil=(2, 2), layout=nhwc), eden.conv_desc(1, 8, 64, 64, 32, 7, 7, layout=nhwc)):
+        assert "few_channel_rows" not in eden.conv_kernels(d)
+
+
 def test_buffer_pool_protocol_without_a_gpu():
     """request / reset / layout are host bookkeeping (CLRuntime.cpp:34-118, 147-157): a REUSE request takes over the
     first feature map handed back and grows it, intra-operator scratch is sized to the largest request per slot, and

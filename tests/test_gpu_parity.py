@@ -221,6 +221,17 @@ CONV_CASES = [
     dict(n=5, c=64, h=33, w=12, cout=64, kh=3, kw=3),
     dict(n=2, c=64, h=14, w=70, cout=32, kh=3, kw=3, pad=(2, 2, 2, 2)),
     dict(n=9, c=64, h=56, w=56, cout=16, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    # one to four input channels, 3 - 11 kernel rows of at most 32 bytes: a kernel row per matrix-instruction step, read
+    # straight from the image (channels-last; the NCHW runs of these cases keep the implicit-GEMM kernel's coverage of them)
+    dict(n=2, c=3, h=37, w=41, cout=64, kh=7, kw=7, stride=(2, 2), pad=(3, 3, 3, 3)),       # an image network's 7x7 stride-2 stem
+    dict(n=1, c=1, h=20, w=33, cout=56, kh=9, kw=9, pad=(4, 4, 4, 4)),                      # grey image, 9x9
+    dict(n=2, c=4, h=18, w=18, cout=24, kh=5, kw=5, stride=(1, 2), pad=(2, 2, 2, 2)),       # 20-byte rows: both fragment halves
+    dict(n=3, c=3, h=9, w=7, cout=16, kh=5, kw=5, pad=(4, 4, 4, 4)),                        # windows mostly in the padding, some wholly
+    dict(n=1, c=2, h=12, w=40, cout=40, kh=3, kw=11, pad=(1, 1, 5, 5)),                     # two channels, wide kernel rows
+    dict(n=1, c=3, h=30, w=30, cout=33, kh=11, kw=10, stride=(3, 3)),                       # 30-byte rows, eleven of them; 33 channels
+    dict(n=2, c=1, h=64, w=64, cout=32, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=70, c=3, h=24, w=24, cout=96, kh=7, kw=7, stride=(2, 2), pad=(3, 3, 3, 3)),      # many workgroups, three channel blocks
+    dict(n=1, c=3, h=10, w=10, cout=8, kh=4, kw=4),                                         # an even number of rows: not that kernel
 ]
 
 
