@@ -10,8 +10,8 @@
 // for the reference's direct3x3 kernels, which likewise read an input pixel once per output-channel group and reuse
 // it over the taps (gpu/operators/cl_kernels/DirectConvolutionKernel.cpp:4324-4869).
 //
-// LDS patch layout: pixel q = row * (W_out + 2) + column at byte q * (C + 16): the 16 bytes of slack per pixel make
-// the pitch an odd number of 16-byte chunks (C is a multiple of 32), so the sixteen lanes that read one chunk
+// LDS patch layout: pixel q = row * (W_out + 2) + column at byte q * pitch, pitch = C + 16 (C a multiple of 32) or
+// C + 32 (C = 16 mod 32): the slack makes the pitch an odd number of 16-byte chunks, so the sixteen lanes that read one chunk
 // position of sixteen consecutive pixels fall on sixteen distinct bank groups, and the fragment address of tap
 // (ky, kx), channel offset c is the lane's base address plus one per-step constant.  The slack chunks are never
 // fetched (their lanes are masked off) and never read.
@@ -47,8 +47,8 @@ struct Conv3Launch {
     int32_t th;               // output rows per tile
     int32_t tiles_per_image;  // ceil(ho / th)
     int32_t tiles;            // n * tiles_per_image
-    int32_t ksteps;           // 9 * cin / 32
-    int32_t pitch;            // LDS bytes per patch pixel: cin + 16
+    int32_t ksteps;           // ceil(9 * cin / 32)
+    int32_t pitch;            // LDS bytes per patch pixel: cin + 16 or + 32 (conv3_pitch)
     int32_t pc;               // patch columns: wo + 2
     FastDiv div_pch, div_pc, div_wo, div_tiles;
 };
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
         const uint8_t *wsrc = reinterpret_cast<const uint8_t *>(p.b) + (size_t)nb_first * KS * 1024;
         const int w_instr = nb_count * KS;  // 1 KiB each
         for (int i = wave; i < w_instr; i += 4) dma16(wsrc + (size_t)i * 1024 + lane * 16, lds_offset(lds) + (uint32_t)i * 1024u);
-        const int pch = L.pitch >> 4, cpp = pch - 1;  // chunks per pixel with and without the slack chunk
+        const int pch = L.pitch >> 4, cpp = p.cin >> 4;  // chunks per pixel with and without the slack
         const int patch_pixels = (rows + 2) * L.pc;
         const int chunks = patch_pixels * pch;
         const int iy0 = oy0 + p.y_base, ix0 = p.x_base;
@@ -111,7 +111,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
             const int koff = tid * 16;
             const int tap = koff / p.cin, c0 = koff - tap * p.cin;
             const int ky = tap / 3, kx = tap - ky * 3;
-            step_s[tid] = (ky * L.pc + kx) * L.pitch + c0;
+            // (the half step past the ninth tap of a 16 (mod 32) channel count multiplies zero weights: any bytes will do)
+            step_s[tid] = tap < 9 ? (ky * L.pc + kx) * L.pitch + c0 : 0;
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -295,10 +296,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
 
 constexpr size_t kLdsTwoPerCu = 80 * 1024, kLdsMax = 160 * 1024;
 
+// LDS bytes per patch pixel: the channels and one or two chunks of slack, an odd number of 16-byte chunks in all
+int conv3_pitch(int cin) { return cin + ((cin & 16) ? 32 : 16); }
+
 size_t conv3_lds_bytes(int nb, int cin, int wo, int th) {
-    const size_t ks = (size_t)9 * cin / 32;
+    const size_t ks = ((size_t)9 * cin + 31) / 32;
     const size_t head = ((size_t)nb * ks * 1024 + (size_t)nb * 128 + ks * 8 + 1023) & ~(size_t)1023;
-    return head + (size_t)(th + 2) * (wo + 2) * (cin + 16);
+    return head + (size_t)(th + 2) * (wo + 2) * conv3_pitch(cin);
 }
 
 // Tile height and channel blocks per workgroup for a problem.  Two workgroups per CU hide each other's staging and
@@ -383,10 +387,10 @@ int launch_nb(const GemmProblem &p, const Conv3Launch &L, size_t lds, hipStream_
 
 }  // namespace
 
-// 3x3 taps at dilation 1 and stride 1 over all of the input's channels, which come in whole 32-byte steps, on an
+// 3x3 taps at dilation 1 and stride 1 over all of the input's channels, which come in whole 16-byte chunks, on an
 // output wide enough that a tile of rows fills the waves, and a patch of three rows that fits LDS beside the weights.
 bool conv3x3_patch_applies(int32_t cin_group, int32_t pixel_stride, int32_t wo, int32_t ho) {
-    if (cin_group != pixel_stride || (cin_group & 31) != 0 || cin_group > 128) return false;
+    if (cin_group != pixel_stride || (cin_group & 15) != 0 || cin_group > 128) return false;
     if (wo < 8 || (long)wo * ho < 128) return false;
     return conv3_lds_bytes(1, cin_group, wo, 1) <= kLdsMax;
 }
@@ -431,7 +435,7 @@ int conv3x3_patch_prepare() {
 }
 
 int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream) {
-    EH_REQUIRE(p.k == 9 * p.cin && (p.cin & 31) == 0 && p.k_pad == p.k && p.stride_h == 1 && p.stride_w == 1,
+    EH_REQUIRE(p.k == 9 * p.cin && (p.cin & 15) == 0 && p.k_pad == (p.k + 31) / 32 * 32 && p.stride_h == 1 && p.stride_w == 1,
                "conv3x3: unsupported problem (k %d, cin %d)", p.k, p.cin);
     // the kernel addresses the output as one dense image per input image: no window, offset or stride on the output side
     EH_REQUIRE(p.out_sy == 1 && p.out_sx == 1 && p.out_y0 == 0 && p.out_x0 == 0 && p.out_h == p.ho && p.out_w == p.wo,
@@ -445,8 +449,8 @@ int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream) {
     L.th = th;
     L.tiles_per_image = (p.ho + th - 1) / th;
     L.tiles = n_img * L.tiles_per_image;
-    L.ksteps = p.k / 32;
-    L.pitch = p.cin + 16;
+    L.ksteps = p.k_pad / 32;
+    L.pitch = conv3_pitch(p.cin);
     L.pc = p.wo + 2;
     L.div_pch = make_fastdiv((uint32_t)(L.pitch >> 4));
     L.div_pc = make_fastdiv((uint32_t)L.pc);

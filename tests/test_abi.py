@@ -179,11 +179,13 @@ def test_3x3_stride_1_convolutions_take_the_patch_kernel():
     assert eden.conv_kernels(eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
     assert eden.conv_kernels(eden.conv_desc(64, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
     assert eden.conv_kernels(eden.conv_desc(2, 128, 16, 16, 100, 3, 3, layout=eden.NCHW)) == ["conv3x3_patch"]
-    # stride 2, dilation 2, groups, 16-byte channel counts, tiny images: the implicit-GEMM kernels
+    assert eden.conv_kernels(eden.conv_desc(1, 48, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    assert eden.conv_kernels(eden.conv_desc(1, 16, 112, 112, 32, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    # stride 2, dilation 2, groups, 8-byte channel counts, tiny images: the implicit-GEMM kernels
     for d in (eden.conv_desc(1, 64, 56, 56, 64, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), layout=nhwc),
               eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(2, 2, 2, 2), dil=(2, 2), layout=nhwc),
               eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), groups=2, layout=nhwc),
-              eden.conv_desc(1, 48, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc),
+              eden.conv_desc(1, 24, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc),
               eden.conv_desc(4, 64, 7, 7, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)):
         assert "conv3x3_patch" not in eden.conv_kernels(d)
 

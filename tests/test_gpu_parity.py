@@ -221,6 +221,11 @@ CONV_CASES = [
     dict(n=5, c=64, h=33, w=12, cout=64, kh=3, kw=3),
     dict(n=2, c=64, h=14, w=70, cout=32, kh=3, kw=3, pad=(2, 2, 2, 2)),
     dict(n=9, c=64, h=56, w=56, cout=16, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    # ... and over channel counts of 16 (mod 32): the reduction ends in half a step of zero weights
+    dict(n=2, c=16, h=23, w=40, cout=32, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=3, c=48, h=14, w=19, cout=80, kh=3, kw=3, pad=(1, 0, 2, 1)),
+    dict(n=1, c=112, h=12, w=12, cout=40, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=6, c=16, h=64, w=64, cout=16, kh=3, kw=3),
     # one to four input channels, 3 - 11 kernel rows of at most 32 bytes: a kernel row per matrix-instruction step, read
     # straight from the image (channels-last; the NCHW runs of these cases keep the implicit-GEMM kernel's coverage of them)
     dict(n=2, c=3, h=37, w=41, cout=64, kh=7, kw=7, stride=(2, 2), pad=(3, 3, 3, 3)),       # an image network's 7x7 stride-2 stem

@@ -55,6 +55,7 @@ PC_CASES = [
     dict(n=2, c=64, h=14, w=14, cout=96, kh=3, kw=3, pad=(1, 1, 1, 1)),                 # direct-to-LDS tiles, k-table
     dict(n=1, c=3, h=20, w=20, cout=32, kh=3, kw=3, stride=(2, 2), pad=(1, 1, 1, 1)),    # first-layer kernel
     dict(n=2, c=3, h=21, w=20, cout=40, kh=7, kw=7, stride=(2, 2), pad=(3, 3, 3, 3)),    # few-channel kernel-row kernel
+    dict(n=2, c=48, h=16, w=16, cout=40, kh=3, kw=3, pad=(1, 1, 1, 1)),                  # patch kernel, channels 16 (mod 32)
     dict(n=2, c=24, h=9, w=9, cout=40, kh=1, kw=1),                                      # one-tap kernel, ragged channel blocks
     dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, groups=2),                            # register-staged kernel, groups
     dict(n=4, c=264, h=28, w=28, cout=256, kh=1, kw=1),                                  # few tiles: reduction split over waves
