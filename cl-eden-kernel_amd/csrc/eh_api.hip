@@ -193,7 +193,10 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     } else if (g.vec == 16 && g.taps == 9 && g.k == 9 * g.cin && units.size() == (size_t)g.k / 16 && g.proto.stride_h == 1 &&
                g.proto.stride_w == 1 && g.proto.out_sy == 1 && g.proto.out_sx == 1 && g.proto.out_y0 == 0 && g.proto.out_x0 == 0 &&
                g.proto.out_h == g.proto.ho && g.proto.out_w == g.proto.wo && units_are_3x3(units, g.cin / 16) &&
-               conv3x3_patch_applies(g.cin, g.proto.cin, g.proto.wo, g.proto.ho)) {
+               conv3x3_patch_applies(g.cin, g.proto.cin, g.proto.wo, g.proto.ho) &&
+               // (128 channels and a full round of 128 x 128 tiles or more: the implicit GEMM is the faster one, measured 15.0
+               // against 20.6 us at 28 x 28 and 59.5 against 81.9 us at 56 x 56, batch 64, 128 output channels)
+               !(g.cin >= 128 && (long)((g.proto.m + 127) / 128) * ((g.n + 127) / 128) >= 240)) {
         // 3x3 taps at dilation 1 and stride 1 over all input channels: the patch-in-LDS kernel
         g.cfg.id = GEMM_CONV3X3;
         g.cfg.slab = 32;

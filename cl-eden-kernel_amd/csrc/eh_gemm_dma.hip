@@ -741,7 +741,7 @@ GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k, int32_t siblings) {
     } else if (n > 64 && t256 >= 240) {
         c.id = GEMM_DMA_256x128;
         c.slab = 128;
-    } else if (n > 64 && t128 >= 200) {
+    } else if (n > 64 && t128 >= 160) {  // (from 5/8 of the CUs on, one round of these beats three of the split-reduction tiles)
         c.id = GEMM_DMA_128x128;
         c.slab = 128;
     } else if (n <= 64 && t128x64 >= 200) {

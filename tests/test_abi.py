@@ -179,6 +179,10 @@ def test_3x3_stride_1_convolutions_take_the_patch_kernel():
     assert eden.conv_kernels(eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
     assert eden.conv_kernels(eden.conv_desc(64, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
     assert eden.conv_kernels(eden.conv_desc(2, 128, 16, 16, 100, 3, 3, layout=eden.NCHW)) == ["conv3x3_patch"]
+    # 128 channels over a full round of 128 x 128 tiles and more: the implicit GEMM again
+    assert eden.conv_kernels(eden.conv_desc(16, 128, 28, 28, 128, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    assert eden.conv_kernels(eden.conv_desc(64, 128, 28, 28, 128, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["dma_128x128"]
+    assert eden.conv_kernels(eden.conv_desc(64, 256, 14, 14, 256, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["dma_128x128"]
     assert eden.conv_kernels(eden.conv_desc(1, 48, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
     assert eden.conv_kernels(eden.conv_desc(1, 16, 112, 112, 32, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
     # stride 2, dilation 2, groups, 8-byte channel counts, tiny images: the implicit-GEMM kernels
