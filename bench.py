@@ -146,7 +146,9 @@ def fc_workload(eden, synth, m=256, k=4096, n=4096, cold=False):
             d_w.free()   # the plan keeps its own packed copy; the raw weights are not read again
         per_set.append((d_a, d_o, plan))
     return dict(name="fc_m%d_k%d_n%d" % (m, k, n), launch=lambda s, i: per_set[i][2].run(per_set[i][0], per_set[i][1], q, s),
-                keep=(per_set, d_b), sets=sets, ops=2.0 * m * k * n, bytes=nbytes, bound="mfma",
+                keep=(per_set, d_b), sets=sets, ops=2.0 * m * k * n, bytes=nbytes,
+                # (few rows: the weights' trip from HBM is the lower roof; the published peaks meet at 625 operations per byte)
+                bound="mfma" if m >= 256 or 2.0 * m * k * n / nbytes >= 625 else "hbm",
                 host=(a, w, b, q), out=per_set[0][1], out_shape=(m, n))
 
 
@@ -501,7 +503,7 @@ def main():
         return lambda e, s, cold=False: fn(e, s, cold=cold, **fixed)
 
     families = dict(fc=fc_workload, conv=conv_workload, dw=dw_workload, pw=pw_workload, deconv=deconv_workload,
-                    fcbig=shaped(fc_workload, m=8192, k=4096, n=4096), conv64=shaped(conv_workload, n=64),
+                    fcbig=shaped(fc_workload, m=8192, k=4096, n=4096), fc1=shaped(fc_workload, m=1, k=4096, n=4096), conv64=shaped(conv_workload, n=64),
                     c3block=block_workload, pw14=shaped(pw_workload, n=64, cin=64, cout=384, hw=14), pj14=shaped(pw_workload, n=64, cin=384, cout=64, hw=14),
                     pw7=shaped(pw_workload, n=64, cin=160, cout=960, hw=7), pj7=shaped(pw_workload, n=64, cin=960, cout=160, hw=7),
                     c3blockbig=shaped(block_workload, n=256),
@@ -539,6 +541,9 @@ def main():
     if args.only and args.only.startswith("pw:"):      # pw:N,CIN,COUT,HW = that pointwise convolution
         n, cin, cout, hw = (int(v) for v in args.only[3:].split(","))
         families[args.only] = shaped(pw_workload, n=n, cin=cin, cout=cout, hw=hw)
+    if args.only and args.only.startswith("fc:"):      # fc:M,K,N = that fully connected layer
+        m, k, n = (int(v) for v in args.only[3:].split(","))
+        families[args.only] = shaped(fc_workload, m=m, k=k, n=n)
     if args.only and args.only.startswith("conv:"):    # conv:N,CIN,COUT,HW,K,STRIDE = that convolution
         n, cin, cout, hw, k, stride = (int(v) for v in args.only[5:].split(","))
         families[args.only] = shaped(conv_workload, n=n, cin=cin, cout=cout, hw=hw, k=k, stride=stride)
@@ -637,6 +642,7 @@ def main():
                                       (shaped(dw_workload, n=64, c=144, hw=56, stride=1, k=7), 200, False),
                                       (deconv_workload, 500, False), (fc_workload, 500, True),
                                       (shaped(fc_workload, m=8192, k=4096, n=4096), 100, False),
+                                      (shaped(fc_workload, m=1, k=4096, n=4096), 500, True),
                                       (layout_workload, 200, True), (shaped(layout_workload, to_nhwc=False), 200, True),
                                       (copy_workload, 200, True),
                                       (stream_workload, 500, True), (shaped(stream_workload, out_bytes=256 * 56 * 56 * 144), 100, True),

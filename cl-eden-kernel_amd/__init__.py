@@ -260,7 +260,7 @@ def conv_desc(n, c, h, w, cout, kh, kw, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1,
                     dil[0], dil[1], groups, dm, layout, weight_layout)
 
 
-KERNEL_NAMES = ("staged", "dma_256x128", "dma_128x128", "dma_128x64", "dma_64x64_splitk", "dma_256x256", "one_tap", "c3k3", "conv3x3_patch", "few_channel_rows")
+KERNEL_NAMES = ("staged", "dma_256x128", "dma_128x128", "dma_128x64", "dma_64x64_splitk", "dma_256x256", "one_tap", "c3k3", "conv3x3_patch", "few_channel_rows", "skinny")
 
 
 def conv_kernels(desc, deconv=False):

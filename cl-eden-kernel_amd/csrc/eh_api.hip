@@ -177,6 +177,13 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         (g.proto.ho - 1) * g.proto.stride_h < g.proto.h && (g.proto.wo - 1) * g.proto.stride_w < g.proto.w) {
         g.cfg.id = GEMM_THIN;
         g.cfg.slab = 32;
+    } else if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 && g.vec == 16 && g.k == g.cin &&
+               gemm_skinny_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.m, g.n) && g.proto.stride_h == 1 && g.proto.stride_w == 1 &&
+               g.proto.y_base == 0 && g.proto.x_base == 0 && g.proto.h == g.proto.ho && g.proto.w == g.proto.wo && g.proto.out_sy == 1 &&
+               g.proto.out_sx == 1 && g.proto.out_y0 == 0 && g.proto.out_x0 == 0 && g.proto.out_h == g.proto.ho && g.proto.out_w == g.proto.wo) {
+        // a classifier head at batch 1 .. 64: the launch is the weights' one trip from memory
+        g.cfg.id = GEMM_SKINNY;
+        g.cfg.slab = 32;
     } else if (g.cin == 3 && g.proto.cin == 3 && g.taps == 9 && g.k == 27 && units.size() == 27 && units[26].dy == 2 &&
                units[26].dx == 2 && units[12].dy == 1 && units[12].dx == 1 && units[0].offset == 0) {
         // three channels, 3x3 taps, dilation 1: the first layer of image networks

@@ -293,6 +293,7 @@ int launch_igemm(const GemmProblem &p, hipStream_t stream) {
     if (p.cfg.id == GEMM_C3K3) return launch_conv_c3k3(p, stream);
     if (p.cfg.id == GEMM_CONV3X3) return launch_conv3x3_patch(p, stream);
     if (p.cfg.id == GEMM_ROWS) return launch_conv_rows(p, stream);
+    if (p.cfg.id == GEMM_SKINNY) return launch_gemm_skinny(p, stream);
     EH_REQUIRE(p.k_pad % BK == 0 && p.k_pad > 0, "igemm: padded reduction length %d is not a multiple of %d", p.k_pad, BK);
     EH_REQUIRE(p.vec == 16 || p.vec == 4 || p.vec == 1, "igemm: bad load unit %d", p.vec);
     if (p.cfg.id != GEMM_STAGED) return launch_igemm_dma(&p, 1, stream);
@@ -311,7 +312,7 @@ int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream) {
     while (i < count) {
         const GemmProblem &p = ps[i];
         int run = 1;
-        const bool dma = p.cfg.id != GEMM_STAGED && p.cfg.id != GEMM_THIN && p.cfg.id != GEMM_C3K3 && p.cfg.id != GEMM_CONV3X3 && p.cfg.id != GEMM_ROWS && p.m > 0 && p.n > 0;
+        const bool dma = p.cfg.id != GEMM_STAGED && p.cfg.id != GEMM_THIN && p.cfg.id != GEMM_C3K3 && p.cfg.id != GEMM_CONV3X3 && p.cfg.id != GEMM_ROWS && p.cfg.id != GEMM_SKINNY && p.m > 0 && p.n > 0;
         if (dma)
             while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == p.cfg.id && ps[i + run].m == p.m &&
                    ps[i + run].n == p.n && ps[i + run].k_pad == p.k_pad && ps[i + run].dense == p.dense && ps[i + run].zw == p.zw)

@@ -365,6 +365,7 @@ enum GemmConfigId {
     GEMM_THIN = 6,              // one-tap problems short of work for tiles; weights in MFMA fragment order
     GEMM_C3K3 = 7,              // 3 input channels, 3x3 taps (first layers); weights row-major [n_pad][32]
     GEMM_CONV3X3 = 8,           // 3x3 taps, stride 1, input patch staged in LDS once; weights in MFMA fragment order
+    GEMM_SKINNY = 10,           // one tap, at most 64 output pixels, long reductions; weights in MFMA fragment order
     GEMM_ROWS = 9,              // 1 - 4 input channels, kernel rows of at most 32 bytes; weights row-major [n_pad][32 per kernel row]
 };
 struct GemmConfig {
@@ -420,6 +421,9 @@ inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
 int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream);
+// one tap, few output pixels, long reductions: cut along the weights (eh_gemm_skinny.hip)
+bool gemm_skinny_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, int32_t channel_offset, int64_t m, int64_t n);
+int launch_gemm_skinny(const GemmProblem &p, hipStream_t stream);
 // few input channels, a kernel row per reduction step (eh_conv_rows.hip)
 bool conv_rows_applies(int32_t cin_group, int32_t pixel_stride, int32_t kh, int32_t kw);
 int launch_conv_rows(const GemmProblem &p, hipStream_t stream);
@@ -438,7 +442,7 @@ __host__ __device__ inline size_t packed_b_offset(const GemmConfig &cfg, int n, 
     const int ch = n & 31;
     n = (n & ~31) | (((ch & 15) >> 2) << 3) | ((ch >> 4) << 2) | (ch & 3);
     // fragment order: [32-channel block][32-byte step][lane = 32 * (chunk & 1) + row][16 bytes]
-    if (cfg.id == GEMM_THIN || cfg.id == GEMM_CONV3X3) return ((((size_t)(n >> 5) * (k_pad / 32) + (kc16 >> 1)) * 2 + (kc16 & 1)) * 32 + (n & 31)) * 16;
+    if (cfg.id == GEMM_THIN || cfg.id == GEMM_CONV3X3 || cfg.id == GEMM_SKINNY) return ((((size_t)(n >> 5) * (k_pad / 32) + (kc16 >> 1)) * 2 + (kc16 & 1)) * 32 + (n & 31)) * 16;
     const int cpr = cfg.slab / 16, rpb = 1024 / cfg.slab;
     const int c = kc16 % cpr;
     return ((size_t)(n / rpb) * (k_pad / cfg.slab) + kc16 / cpr) * 1024 + (size_t)(n % rpb) * cfg.slab +

@@ -293,7 +293,8 @@ typedef enum eh_kernel_id {
     EH_KERNEL_ONE_TAP = 6,        /* 1x1 problems with short reductions or few pixels               */
     EH_KERNEL_C3K3 = 7,           /* 3x3 on three input channels (first layers)                     */
     EH_KERNEL_CONV3X3_PATCH = 8,  /* 3x3, stride 1: input patch staged in LDS once                  */
-    EH_KERNEL_FEW_CHANNEL_ROWS = 9 /* 1 - 4 input channels, 3 - 11 kernel rows of at most 32 bytes   */
+    EH_KERNEL_FEW_CHANNEL_ROWS = 9, /* 1 - 4 input channels, 3 - 11 kernel rows of at most 32 bytes  */
+    EH_KERNEL_SKINNY = 10         /* one tap, at most 64 output pixels, reductions beyond 256 bytes */
 } eh_kernel_id;
 int eh_conv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_t cap);
 int eh_deconv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_t cap);

@@ -207,6 +207,19 @@ def test_few_channel_convolutions_take_the_kernel_row_kernel():
         assert "few_channel_rows" not in eden.conv_kernels(d)
 
 
+def test_classifier_heads_take_the_kernel_cut_along_the_weights():
+    nhwc = eden.NHWC
+    assert eden.conv_kernels(eden.conv_desc(1, 1280, 1, 1, 1000, 1, 1, layout=nhwc)) == ["skinny"]
+    assert eden.conv_kernels(eden.conv_desc(32, 4096, 1, 1, 4096, 1, 1, layout=nhwc)) == ["skinny"]
+    assert eden.conv_kernels(eden.conv_desc(64, 1280, 1, 1, 1000, 1, 1, layout=nhwc)) == ["skinny"]
+    assert "skinny" not in eden.conv_kernels(eden.conv_desc(64, 4096, 1, 1, 4096, 1, 1, layout=nhwc))
+    assert eden.conv_kernels(eden.conv_desc(2, 512, 5, 5, 48, 1, 1, layout=nhwc)) == ["skinny"]
+    # more than 64 pixels, a reduction within the one-tap kernel's, a stride: the other kernels
+    assert "skinny" not in eden.conv_kernels(eden.conv_desc(65, 1280, 1, 1, 1000, 1, 1, layout=nhwc))
+    assert eden.conv_kernels(eden.conv_desc(1, 256, 1, 1, 1000, 1, 1, layout=nhwc)) == ["one_tap"]
+    assert "skinny" not in eden.conv_kernels(eden.conv_desc(1, 512, 9, 9, 48, 1, 1, stride=(2, 2), layout=nhwc))
+
+
 def test_buffer_pool_protocol_without_a_gpu():
     """request / reset / layout are host bookkeeping (CLRuntime.cpp:34-118, 147-157): a REUSE request takes over the
     first feature map handed back and grows it, intra-operator scratch is sized to the largest request per slot, and

@@ -181,7 +181,7 @@ def test_int8_deconv_matches_oracle(case, layout):
     assert want.std() > 4
 
 
-@pytest.mark.parametrize("m,k,n", [(64, 512, 256), (5, 100, 33), (256, 4096, 512)])
+@pytest.mark.parametrize("m,k,n", [(64, 512, 256), (5, 100, 33), (256, 4096, 512), (3, 1024, 200)])
 def test_int8_fc_matches_oracle(m, k, n):
     print("int8 fc", m, k, n, flush=True)
     a, w = s8((m, k), SEED + 71), s8((n, k), SEED + 72)

@@ -63,6 +63,14 @@ FC_CASES = [
     (130, 272, 200, 77, 201),
     (64, 1296, 130, 3, 128),
     (200, 528, 64, 131, 120),
+    # at most 64 rows and a reduction beyond 256 bytes: the kernel that is cut along the weights (one and two groups of
+    # 32 rows, no row-sum term, a reduction that ends inside its last step, fewer steps than waves + 1, eight channels)
+    (1, 4096, 1000, 3, 128),
+    (1, 1280, 1000, 10, 20),
+    (32, 272, 40, 77, 201),
+    (33, 2048, 72, 131, 120),
+    (64, 9216, 64, 0, 255),
+    (17, 304, 8, 5, 100),
 ]
 
 
@@ -237,6 +245,9 @@ CONV_CASES = [
     dict(n=2, c=1, h=64, w=64, cout=32, kh=3, kw=3, pad=(1, 1, 1, 1)),
     dict(n=70, c=3, h=24, w=24, cout=96, kh=7, kw=7, stride=(2, 2), pad=(3, 3, 3, 3)),      # many workgroups, three channel blocks
     dict(n=1, c=3, h=10, w=10, cout=8, kh=4, kw=4),                                         # an even number of rows: not that kernel
+    # 1x1 on at most 64 pixels with a long reduction: cut along the weights
+    dict(n=8, c=1280, h=1, w=1, cout=100, kh=1, kw=1),
+    dict(n=2, c=512, h=5, w=5, cout=48, kh=1, kw=1),
 ]
 
 
