@@ -297,17 +297,19 @@ def mbv2_workload(eden, synth, batch=64, per_channel=False, weights="minmax", co
                 pool_bytes=net.pool_bytes, lanes=net.lanes, fused_blocks=list(net.fused_blocks))
 
 
-def mbv2_userdriver(eden, batch=64, per_channel=False, list_id=0xC5):
+def mbv2_userdriver(eden, batch=64, per_channel=False, list_id=0xC5, planar=False):
     """The same network through the operator API the reference binds: described as an operator list, opened by the C++
     OperationConstructor on a HipComputeLibrary (HipConvolution ... operators, pooled feature maps), executed by the
     OperationExecutor, which records the list into a HIP graph on its second execution and replays it.  Returns
-    (driver, list id, logits shape); the input tensor holds network_input(batch)."""
+    (driver, list id, logits shape); the input tensor holds network_input(batch).  planar: the model as a planar list
+    (feature maps [n, c, h, w]), whose feature maps the constructor stores channels-last behind one layout operator."""
     mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
     ud = importlib.import_module("cl-eden-kernel_amd.userdriver")
     driver = ud.UserDriver(0)
-    ol, _, _, shape = mobilenet.operator_list(ud, list_id, batch, per_channel=per_channel)
+    ol, _, _, shape = mobilenet.operator_list(ud, list_id, batch, per_channel=per_channel, nchw=planar)
     driver.open_subgraph(ol)
-    driver.write_input(list_id, 0, mobilenet.network_input(batch))
+    x = mobilenet.network_input(batch)
+    driver.write_input(list_id, 0, np.ascontiguousarray(x.transpose(0, 3, 1, 2)) if planar else x)
     return driver, list_id, shape
 
 
@@ -523,9 +525,9 @@ def main():
         for mix in range(len(eden.FEED_MIXES)):
             print(json.dumps(eden.probe_feed(mix, 256, 4000)), flush=True)
         return
-    if args.only in ("mbv2ud", "mbv2udpc"):
+    if args.only in ("mbv2ud", "mbv2udpc", "mbv2udplanar"):
         mobilenet = importlib.import_module("cl-eden-kernel_amd.mobilenet")
-        driver, list_id, _ = mbv2_userdriver(eden, per_channel=args.only == "mbv2udpc")
+        driver, list_id, _ = mbv2_userdriver(eden, per_channel=args.only == "mbv2udpc", planar=args.only == "mbv2udplanar")
         if args.no_graph:
             driver.set_replay(False)
         steps = min(args.steps, 200)
@@ -632,6 +634,13 @@ def main():
                                                      "userdriver classes (OperationConstructor / OperationExecutor), ms per batch %.4f" % (wall2 / 40 * 1e3, wall3 / 40 * 1e3))
         via_api[0].close()
         del via_api
+        # ... and as a planar list (feature maps [n, c, h, w], as Caffe-style models come): stored channels-last inside
+        planar = mbv2_userdriver(eden, list_id=0xC6, planar=True)
+        wall4, ev4, _ = time_userdriver(eden, planar[0], planar[1], 40, 4)
+        c5["operator_api"]["planar_list"] = dict(images_per_s=round(net["images"] * 40 / wall4, 1), us_per_batch_by_events=round(ev4 / 40 * 1e6, 1),
+                                                  executor=planar[0].stats(planar[1]))
+        planar[0].close()
+        del planar
         del net
         others = [c5]
         for make, steps, cold_too in ((conv_workload, 2000, False), (shaped(conv_workload, n=64), 300, False),

@@ -193,9 +193,62 @@ __global__ __launch_bounds__(256) void transpose_u8_wide_kernel(const uint8_t *_
     }
 }
 
+// Two to four rows (an RGB image's planes to interleaved pixels) or two to four columns (the way back), the long
+// extent a multiple of 4: a thread moves four positions of the long axis, one dword per plane on the planar side and
+// C consecutive dwords on the interleaved side, so both sides are whole, coalesced dword accesses.  (The tiled kernels
+// would leave nine tenths of a tile empty.)
+template <int C, bool INTERLEAVE>
+__global__ __launch_bounds__(256) void transpose_u8_few_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int32_t L) {
+    const int i = blockIdx.x * 256 + threadIdx.x;  // positions 4 i .. 4 i + 3 of the long axis
+    if (4 * i >= L) return;
+    const size_t batch_off = (size_t)blockIdx.z * C * L;
+    const uint8_t *plane_side = (INTERLEAVE ? src : dst) + batch_off + 4 * (size_t)i;
+    const uint8_t *pixel_side = (INTERLEAVE ? dst : src) + batch_off + 4 * (size_t)i * C;
+    uint32_t planes[C], pixels[C];
+    if constexpr (INTERLEAVE) {
+#pragma unroll
+        for (int c = 0; c < C; ++c) planes[c] = *reinterpret_cast<const uint32_t *>(plane_side + (size_t)c * L);
+#pragma unroll
+        for (int d = 0; d < C; ++d) pixels[d] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int c = 0; c < C; ++c) pixels[(j * C + c) >> 2] |= ((planes[c] >> (8 * j)) & 255u) << (8 * ((j * C + c) & 3));
+#pragma unroll
+        for (int d = 0; d < C; ++d) *reinterpret_cast<uint32_t *>(const_cast<uint8_t *>(pixel_side) + 4 * d) = pixels[d];
+    } else {
+#pragma unroll
+        for (int d = 0; d < C; ++d) pixels[d] = *reinterpret_cast<const uint32_t *>(pixel_side + 4 * d);
+#pragma unroll
+        for (int c = 0; c < C; ++c) planes[c] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int c = 0; c < C; ++c) planes[c] |= ((pixels[(j * C + c) >> 2] >> (8 * ((j * C + c) & 3))) & 255u) << (8 * j);
+#pragma unroll
+        for (int c = 0; c < C; ++c) *reinterpret_cast<uint32_t *>(const_cast<uint8_t *>(plane_side) + (size_t)c * L) = planes[c];
+    }
+}
+
+template <bool INTERLEAVE>
+int launch_transpose_few(const uint8_t *src, uint8_t *dst, int32_t batch, int32_t c, int32_t L, hipStream_t stream) {
+    const dim3 grid((unsigned)((L / 4 + 255) / 256), 1, (unsigned)batch);
+    if (c == 2)
+        hipLaunchKernelGGL((transpose_u8_few_kernel<2, INTERLEAVE>), grid, dim3(256), 0, stream, src, dst, L);
+    else if (c == 3)
+        hipLaunchKernelGGL((transpose_u8_few_kernel<3, INTERLEAVE>), grid, dim3(256), 0, stream, src, dst, L);
+    else
+        hipLaunchKernelGGL((transpose_u8_few_kernel<4, INTERLEAVE>), grid, dim3(256), 0, stream, src, dst, L);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
+
 int launch_transpose(const uint8_t *src, uint8_t *dst, int32_t batch, int32_t R, int32_t S, hipStream_t stream) {
     if (batch <= 0 || R <= 0 || S <= 0) return EH_OK;
     EH_REQUIRE(batch <= 65535, "transpose: batch %d exceeds the grid limit", batch);
+    const bool dwords = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 3) == 0;
+    if (dwords && R >= 2 && R <= 4 && S % 4 == 0 && S >= 64) return launch_transpose_few<true>(src, dst, batch, R, S, stream);
+    if (dwords && S >= 2 && S <= 4 && R % 4 == 0 && R >= 64) return launch_transpose_few<false>(src, dst, batch, S, R, stream);
     if (R % 4 == 0 && S % 4 == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 3) == 0) {
         if (S <= 32 && (R + 511) / 512 <= 65535) {
             hipLaunchKernelGGL((transpose_u8_wide_kernel<512, 32>), dim3(1, (R + 511) / 512, batch), dim3(256), 0, stream, src, dst, R, S);

@@ -67,6 +67,8 @@ public:
             for (const auto &t : op.in_tensors)
                 if (!t->is_const) consumed_[t->buffer_index] = true;
         }
+        channels_last_ = store_channels_last && planar_list_can_be_stored_channels_last(list);
+        pending_layout_ops_.clear();
         lanes_ = lanes_for(list);
         const auto runtime = compute_library_->runtime();
         for (lane_ = 0; lane_ < lanes_; ++lane_) {
@@ -85,6 +87,7 @@ public:
                         return abandon();
                     }
                     ++index;  // the Add went into the convolution's launch
+                    append_pending_layout_changes();
                     continue;
                 }
                 if (fuse_expansions && index + 1 < list.operators.size() && fusable_expansion(op, list.operators[index + 1])) {
@@ -93,12 +96,14 @@ public:
                         return abandon();
                     }
                     ++index;  // the depthwise convolution went into the pointwise convolution's launch
+                    append_pending_layout_changes();
                     continue;
                 }
                 if (create_ud_operator(op) != ENN_RET_SUCCESS) {
                     ERROR_PRINT("OperationConstructor: building %s failed\n", op.name.c_str());
                     return abandon();
                 }
+                append_pending_layout_changes();
             }
             for (size_t i = first_operator; i < operators->size(); ++i) (*operators)[i]->setLane(lane_);
         }
@@ -117,6 +122,58 @@ public:
                 return ENN_RET_FAILED;
             }
         return ENN_RET_SUCCESS;
+    }
+
+    // Whether every operator of the list is a planar one this constructor can run on channels-last storage: the six
+    // operator kinds, all in planar mode, constant parameters, byte feature maps, and no fully connected layer that
+    // flattens more than one pixel per image (its weights are ordered for the planar flattening).
+    bool planar_list_can_be_stored_channels_last(const OperatorListDesc &list) const {
+        if (list.operators.empty()) return false;
+        for (const auto &op : list.operators) {
+            bool android = false, nchw = true;
+            switch (op.code) {
+                case TFlite::BuiltinOperator_CONV_2D:
+                    if (!op.option) return false;
+                    layout_of(*options_of<TFlite::Conv2DOptions>(op), &android, &nchw);
+                    break;
+                case TFlite::BuiltinOperator_DEPTHWISE_CONV_2D:
+                    if (!op.option) return false;
+                    layout_of(*options_of<TFlite::DepthwiseConv2DOptions>(op), &android, &nchw);
+                    break;
+                case TFlite::BuiltinOperator_TRANSPOSE_CONV:
+                    if (!op.option) return false;
+                    layout_of(*options_of<TFlite::TransposeConvOptions>(op), &android, &nchw);
+                    break;
+                case TFlite::BuiltinOperator_AVERAGE_POOL_2D:
+                    if (!op.option) return false;
+                    layout_of(*options_of<TFlite::Pool2DOptions>(op), &android, &nchw);
+                    break;
+                case TFlite::BuiltinOperator_FULLY_CONNECTED:
+                    if (op.in_tensors.empty()) return false;
+                    if (!op.in_tensors[0]->is_const && op.in_tensors[0]->shape.size() == 4 &&
+                        (uint64_t)op.in_tensors[0]->shape[2] * op.in_tensors[0]->shape[3] > 1)
+                        return false;
+                    break;
+                case TFlite::BuiltinOperator_ADD: break;
+                default: return false;
+            }
+            if (!nchw) return false;
+            // weights and bias that are run-time feature maps have shapes of their own kind: such a list stays as it is
+            if (op.code != TFlite::BuiltinOperator_ADD && op.code != TFlite::BuiltinOperator_AVERAGE_POOL_2D)
+                for (size_t i = 1; i < op.in_tensors.size(); ++i)
+                    if (!op.in_tensors[i]->is_const) return false;
+            for (const auto *edges : {&op.in_tensors, &op.out_tensors})
+                for (const auto &t : *edges)
+                    if (!t->is_const && t->shape.size() == 4 && t->data_type != TFlite::TensorType_UINT8 && t->data_type != TFlite::TensorType_INT8)
+                        return false;
+        }
+        return true;
+    }
+
+    // the layout operators that follow the operator built last (those of the list's outputs it writes)
+    void append_pending_layout_changes() {
+        for (auto &op : pending_layout_ops_) operators->push_back(op);
+        pending_layout_ops_.clear();
     }
 
     // How many lanes the list's images are cut into (1: none).  A list qualifies when every feature map carries the
@@ -191,6 +248,14 @@ public:
     // description, as the reference builds the list.
     bool fuse_expansions = true;
     bool fuse_unlisted_expansions = false;  // fuse every pair the kernel fits, measured faster or not (tests, experiments)
+    // The feature maps inside a PLANAR operator list (a Caffe-style model, or an androidNN one with use_nchw) are stored
+    // channels-last: the kernels of this backend work on channels-last data, and a planar tensor costs every operator a
+    // transposition on either side (MobileNetV2 at 64 images as a planar list: 1872 us per execution with planar
+    // storage).  The list's inputs and outputs stay planar for its owner; one layout operator behind each input and in
+    // front of each output is added to the list.  Shapes, parameters and results are those of the planar list.
+    // false = every tensor stored as its shape reads, as the reference does.
+    bool store_channels_last = true;
+    bool stores_channels_last() const { return channels_last_; }  // of the list opened last
     int lanes() const { return lanes_; }  // of the list opened last
 
     // ---- helpers, public because tests pin them against hand-computed cases
@@ -309,6 +374,55 @@ private:
         }
     }
 
+    // The feature map of `edge` as its shape reads: one pooled tensor per buffer index and lane, or, for an input or output
+    // of a list that is cut into lanes, one whole tensor and this lane's view of its share.
+    std::shared_ptr<ITensor> allocate_feature_map(const std::shared_ptr<TensorDesc> &edge, const PrecisionType &precision, const BufferType &buffer_type,
+                                                  const DataOrder &data_order, const NDims &dims, bool list_io) {
+        auto &made = alloc_tensors_map_[operator_list_id_];
+        if (lanes_ > 1 && list_io) {
+            // an input or output of the list: one whole tensor in an arena no lane takes storage from, and this
+            // lane's view of its share
+            std::shared_ptr<ITensor> &whole = made[edge->buffer_index];
+            if (whole == nullptr) {
+                compute_library_->runtime()->selectArena(lanes_);
+                whole = compute_library_->create_tensor(edge->data_type, precision, dims, edge->buffer_index, BufferType::INTER_SHARED_NEW,
+                                                        false, StorageType::BUFFER, data_order, edge->scale, edge->zero_point);
+                compute_library_->runtime()->selectArena(lane_);
+                if (whole == nullptr) {
+                    made.erase(edge->buffer_index);
+                    ERROR_PRINT("OperationConstructor: feature map %s could not be made\n", edge->name.c_str());
+                    return nullptr;
+                }
+                (produced_.count(edge->buffer_index) ? out_tensors : in_tensors).push_back(whole);
+            }
+            std::shared_ptr<ITensor> &view = made[lane_key(edge->buffer_index)];
+            if (view == nullptr) {
+                const uint32_t share = dims[0] / (uint32_t)lanes_;
+                view = std::make_shared<HipTensor>(std::static_pointer_cast<HipTensor>(whole), share * (uint32_t)lane_, share);
+            }
+            return view;
+        }
+        auto found = made.find(lane_key(edge->buffer_index));
+        if (found != made.end()) return found->second;
+        NDims lane_dims = dims;
+        lane_dims[0] /= (uint32_t)lanes_;
+        std::shared_ptr<ITensor> tensor = compute_library_->create_tensor(edge->data_type, precision, lane_dims, edge->buffer_index, buffer_type,
+                                                                          false, StorageType::BUFFER, data_order, edge->scale,
+                                                                          edge->zero_point);
+        if (tensor == nullptr) {
+            ERROR_PRINT("OperationConstructor: feature map %s could not be made\n", edge->name.c_str());
+            return nullptr;
+        }
+        made[lane_key(edge->buffer_index)] = tensor;
+        if (lanes_ == 1) {
+            if (!produced_.count(edge->buffer_index))
+                in_tensors.push_back(tensor);
+            else if (!consumed_.count(edge->buffer_index))
+                out_tensors.push_back(tensor);
+        }
+        return tensor;
+    }
+
     // A feature map becomes a pooled run-time tensor, made once per buffer index of the list; a parameter becomes a
     // constant tensor uploaded at once (gpu_op_constructor.cc:2062-2155).
     std::shared_ptr<ITensor> allocate_tensor(const std::shared_ptr<TensorDesc> &edge, const PrecisionType &precision,
@@ -323,48 +437,42 @@ private:
         if (!edge->is_const) {
             auto &made = alloc_tensors_map_[operator_list_id_];
             const bool list_io = !produced_.count(edge->buffer_index) || !consumed_.count(edge->buffer_index);
-            if (lanes_ > 1 && list_io) {
-                // an input or output of the list: one whole tensor in an arena no lane takes storage from, and this
-                // lane's view of its share
-                std::shared_ptr<ITensor> &whole = made[edge->buffer_index];
-                if (whole == nullptr) {
-                    compute_library_->runtime()->selectArena(lanes_);
-                    whole = compute_library_->create_tensor(edge->data_type, precision, dims, edge->buffer_index, BufferType::INTER_SHARED_NEW,
-                                                            false, StorageType::BUFFER, data_order, edge->scale, edge->zero_point);
-                    compute_library_->runtime()->selectArena(lane_);
-                    if (whole == nullptr) {
-                        made.erase(edge->buffer_index);
-                        ERROR_PRINT("OperationConstructor: feature map %s could not be made\n", edge->name.c_str());
-                        return nullptr;
-                    }
-                    (produced_.count(edge->buffer_index) ? out_tensors : in_tensors).push_back(whole);
-                }
-                std::shared_ptr<ITensor> &view = made[lane_key(edge->buffer_index)];
-                if (view == nullptr) {
-                    const uint32_t share = dims[0] / (uint32_t)lanes_;
-                    view = std::make_shared<HipTensor>(std::static_pointer_cast<HipTensor>(whole), share * (uint32_t)lane_, share);
-                }
-                return view;
+            // stored channels-last inside a planar list (a tensor of one pixel per image, or of one channel, is both orders at once)
+            const bool channels_last = channels_last_ && edge->shape.size() == 4 && (uint64_t)d4.h * d4.w > 1 && d4.c > 1;
+            if (!(channels_last && list_io)) {
+                auto tensor = allocate_feature_map(edge, precision, buffer_type, data_order, dims, list_io);
+                if (tensor != nullptr && channels_last) std::static_pointer_cast<HipTensor>(tensor)->storeChannelsLast(true);
+                return tensor;
             }
-            auto found = made.find(lane_key(edge->buffer_index));
+            // An input or output of such a list: its owner reads and writes the planar tensor; the operators see a
+            // channels-last twin (this lane's share of it), and a layout operator carries the data across.
+            const int32_t twin_key = lane_key(edge->buffer_index) + kTwinKeyOffset;
+            auto found = made.find(twin_key);
             if (found != made.end()) return found->second;
+            auto planar = allocate_feature_map(edge, precision, buffer_type, data_order, dims, list_io);
+            if (planar == nullptr) return nullptr;
             NDims lane_dims = dims;
             lane_dims[0] /= (uint32_t)lanes_;
-            std::shared_ptr<ITensor> tensor = compute_library_->create_tensor(edge->data_type, precision, lane_dims, edge->buffer_index, buffer_type,
-                                                                              false, StorageType::BUFFER, data_order, edge->scale,
-                                                                              edge->zero_point);
-            if (tensor == nullptr) {
-                ERROR_PRINT("OperationConstructor: feature map %s could not be made\n", edge->name.c_str());
+            const bool is_input = !produced_.count(edge->buffer_index);
+            std::shared_ptr<ITensor> twin = compute_library_->create_tensor(edge->data_type, precision, lane_dims, edge->buffer_index,
+                                                                            is_input ? BufferType::INTER_SHARED_NEW : buffer_type, false,
+                                                                            StorageType::BUFFER, data_order, edge->scale, edge->zero_point);
+            if (twin == nullptr) {
+                ERROR_PRINT("OperationConstructor: the channels-last twin of feature map %s could not be made\n", edge->name.c_str());
                 return nullptr;
             }
-            made[lane_key(edge->buffer_index)] = tensor;
-            if (lanes_ == 1) {
-                if (!produced_.count(edge->buffer_index))
-                    in_tensors.push_back(tensor);
-                else if (!consumed_.count(edge->buffer_index))
-                    out_tensors.push_back(tensor);
-            }
-            return tensor;
+            std::static_pointer_cast<HipTensor>(twin)->storeChannelsLast(true);
+            auto change = std::make_shared<HipLayoutChange>(compute_library_->runtime(), is_input);
+            const UDTensors from = {is_input ? planar : twin}, to = {is_input ? twin : planar};
+            if (change->initialize(from, to) != Status::SUCCESS) return nullptr;
+            auto wrapped = std::make_shared<EnnUDOperator<HipLayoutChange>>((is_input ? "TO_CHANNELS_LAST_" : "TO_PLANAR_") + std::to_string(edge->buffer_index),
+                                                                           0, from, to, UDTensors(), change);
+            if (is_input)
+                operators->push_back(wrapped);  // in front of the operator that is being built, the input's first reader
+            else
+                pending_layout_ops_.push_back(wrapped);  // behind it, the output's writer
+            made[twin_key] = twin;
+            return twin;
         }
         // a parameter is uploaded once and read by every lane's operator
         auto shared = const_tensors_.find(edge.get());
@@ -388,6 +496,7 @@ private:
         return lane_ == 0 && !whole_tensor_has_the_index ? buffer_index : buffer_index + (lane_ + 1) * kLaneKeyStride;
     }
     static constexpr int32_t kLaneKeyStride = 1 << 24;
+    static constexpr int32_t kTwinKeyOffset = 1 << 29;  // the channels-last twins of a planar list's inputs and outputs
 
     // outputs first (they may take over storage released by earlier operators), then inputs; an input
     // whose last reader this operator is gives its storage back (gpu_op_constructor.cc:2157-2191)
@@ -531,17 +640,22 @@ private:
         bool android = false, nchw = true, dw_nchw = true;
         layout_of(*co, &android, &nchw);
         layout_of(*dwo, &android, &dw_nchw);
-        if (nchw || dw_nchw) return false;
+        // channels-last data: the list's own, or a planar list whose feature maps are stored that way
+        if (nchw != dw_nchw || (nchw && !channels_last_)) return false;
+        // shapes read (n, c, h, w) in a planar list, (n, h, w, c) otherwise; filters (out, kh, kw, in) / (1, kh, kw, c) in
+        // androidNN models, (out, in, kh, kw) / (c, 1, kh, kw) otherwise
+        const int hi = nchw ? 2 : 1, wi = nchw ? 3 : 2, ci = nchw ? 1 : 3, ki = android ? 1 : 2;
         const auto &cw = conv.in_tensors[1]->shape, &dww = dw.in_tensors[1]->shape;
-        if (cw.size() != 4 || cw[1] != 1 || cw[2] != 1 || co->stride_h != 1 || co->stride_w != 1 || co->dilation_h_factor != 1 || co->dilation_w_factor != 1)
+        if (cw.size() != 4 || cw[ki] != 1 || cw[ki + 1] != 1 || co->stride_h != 1 || co->stride_w != 1 || co->dilation_h_factor != 1 ||
+            co->dilation_w_factor != 1)
             return false;
-        if (dww.size() != 4 || dww[1] != 3 || dww[2] != 3 || dwo->stride_h != dwo->stride_w || dwo->dilation_h_factor != 1 || dwo->dilation_w_factor != 1 ||
-            dwo->depth_multiplier != 1)
+        if (dww.size() != 4 || dww[ki] != 3 || dww[ki + 1] != 3 || dwo->stride_h != dwo->stride_w || dwo->dilation_h_factor != 1 ||
+            dwo->dilation_w_factor != 1 || dwo->depth_multiplier != 1)
             return false;
-        if (x->shape[1] != e->shape[1] || x->shape[2] != e->shape[2] || x->shape[0] != e->shape[0]) return false;
+        if (x->shape[hi] != e->shape[hi] || x->shape[wi] != e->shape[wi] || x->shape[0] != e->shape[0]) return false;
         return fuse_unlisted_expansions ||
-               eh_conv_dw_block_listed((int32_t)(e->shape[0] / (uint32_t)lanes_), (int32_t)e->shape[1], (int32_t)e->shape[2], (int32_t)x->shape[3],
-                                       (int32_t)e->shape[3], dwo->stride_h) != 0;
+               eh_conv_dw_block_listed((int32_t)(e->shape[0] / (uint32_t)lanes_), (int32_t)e->shape[hi], (int32_t)e->shape[wi], (int32_t)x->shape[ci],
+                                       (int32_t)e->shape[ci], dwo->stride_h) != 0;
     }
 
     // The depthwise convolution's tensors are made first: its output then cannot be given the storage of the feature
@@ -557,6 +671,7 @@ private:
         auto expanded = std::make_shared<HipTensor>(HipTensor::NoStorage{}, compute_library_->runtime(), precision,
                                                     compute_library_->tensor_type_2_data_type(edge->data_type), dims, DataOrder::NCHW, edge->scale,
                                                     edge->zero_point, static_cast<uint32_t>(edge->data_type), edge->buffer_index);
+        expanded->storeChannelsLast(channels_last_);  // (a fused pair's tensors have more than one pixel per image)
         alloc_tensors_map_[operator_list_id_][lane_key(edge->buffer_index)] = expanded;
         UDTensors dw_in, dw_out;
         if (!convert_to_tensors(dw, precision, dw_in, dw_out)) return ENN_RET_FAILED;
@@ -643,6 +758,8 @@ private:
     std::map<int32_t, bool> produced_, consumed_;
     std::map<const TensorDesc *, std::shared_ptr<ITensor>> const_tensors_;  // parameters of the list being built, shared by its lanes
     int lanes_ = 1, lane_ = 0;
+    bool channels_last_ = false;  // the list being opened stores its feature maps channels-last
+    std::vector<std::shared_ptr<UDOperator>> pending_layout_ops_;
 };
 
 // Runs a built list: every operator in order on the compute library's stream (gpu_op_executor.cc:56-103).  Moving host

@@ -115,6 +115,17 @@ struct Pool2DParameters : public Parameters {
 
 namespace detail {
 
+// How the plan of an operator on planar-shaped (n, c, h, w) tensors addresses them: EH_NCHW when both are stored planar,
+// EH_NHWC when they are stored channels-last (HipTensor::storedChannelsLast; a tensor of one pixel per image is both at
+// once, and so is one of a single channel), -1 when the two disagree.
+inline int planarOperatorLayout(const std::shared_ptr<HipTensor> &a, const std::shared_ptr<HipTensor> &b) {
+    const bool al = a->storedChannelsLast(), bl = b->storedChannelsLast();
+    if (!al && !bl) return EH_NCHW;
+    const Dim4 ad = a->getDim(), bd = b->getDim();
+    const bool a_flat = (uint64_t)ad.h * ad.w <= 1 || ad.c <= 1, b_flat = (uint64_t)bd.h * bd.w <= 1 || bd.c <= 1;
+    return (al || a_flat) && (bl || b_flat) ? EH_NHWC : -1;
+}
+
 inline int toEhActivation(const ActivationInfo &a) {
     switch (a.activation()) {
         case ActivationInfo::ActivationType::RELU: return EH_ACT_RELU;
@@ -246,7 +257,8 @@ public:
         d.dil_w = (int32_t)parameters_->dilation.w;
         d.groups = (int32_t)groups;
         d.depth_multiplier = 1;
-        d.layout = parameters_->isNCHW ? EH_NCHW : EH_NHWC;
+        d.layout = parameters_->isNCHW ? detail::planarOperatorLayout(input_, output_) : EH_NHWC;
+        CHECK_EXPR_RETURN_FAILURE(d.layout >= 0, "HipConvolution: input and output are stored in different element orders");
         d.weight_layout = ohwi ? EH_W_OHWI : EH_W_OIHW;
         desc_ = d;
         const int32_t ho = eh_conv_out_dim(d.h, d.pad_t, d.pad_b, d.kh, d.dil_h, d.stride_h);
@@ -441,7 +453,8 @@ public:
         d.dil_w = (int32_t)parameters_->dilation.w;
         d.groups = 1;
         d.depth_multiplier = (int32_t)parameters_->depth_multiplier;
-        d.layout = parameters_->isNCHW ? EH_NCHW : EH_NHWC;
+        d.layout = parameters_->isNCHW ? detail::planarOperatorLayout(input_, output_) : EH_NHWC;
+        CHECK_EXPR_RETURN_FAILURE(d.layout >= 0, "HipDepthwiseConvolution: input and output are stored in different element orders");
         d.weight_layout = hwo ? EH_W_OHWI : EH_W_OIHW;
         CHECK_EXPR_RETURN_FAILURE(wd.n == (uint32_t)d.cout && wd.c == 1, "HipDepthwiseConvolution: weight shape [%u %u %u %u] is not [C*dm][1][kh][kw]", wd.n, wd.c, wd.h, wd.w);
         desc_ = d;
@@ -584,7 +597,10 @@ public:
         CHECK_EXPR_RETURN_FAILURE(parameters_->storage_type == StorageType::BUFFER, "HipFullyConnected: no texture storage");
         CHECK_EXPR_RETURN_FAILURE(detail::tensorTypesMatch(precision_, false, input_, weight_, bias_, output_),
                                   "HipFullyConnected: expects uint8 (INT8 precision: int8) input/weight/output and int32 bias");
-        // weight [units][k]; the input is flattened to [size / k][k]
+        // weight [units][k]; the input is flattened to [size / k][k] (in the order its shape reads: a tensor stored
+        // channels-last must be one pixel per image)
+        CHECK_EXPR_RETURN_FAILURE(!input_->storedChannelsLast() || (uint64_t)input_->getDim().h * input_->getDim().w <= 1,
+                                  "HipFullyConnected: the input is stored channels-last and has more than one pixel per image");
         // (CLFullyConnected.cpp:46-57: in androidNN mode the batch is whatever the element count gives)
         const Dim4 wd = weight_->getDim();
         const uint32_t units = wd.n, k = wd.c * wd.h * wd.w;
@@ -698,7 +714,8 @@ public:
         d.dil_w = 1;
         d.groups = (int32_t)groups;
         d.depth_multiplier = 1;
-        d.layout = parameters_->isNCHW ? EH_NCHW : EH_NHWC;
+        d.layout = parameters_->isNCHW ? detail::planarOperatorLayout(input_, output_) : EH_NHWC;
+        CHECK_EXPR_RETURN_FAILURE(d.layout >= 0, "HipDeconvolution: input and output are stored in different element orders");
         d.weight_layout = nn ? EH_W_OHWI : EH_W_IOHW;
         CHECK_EXPR_RETURN_FAILURE((nn ? wd.w : wd.n) == in.c, "HipDeconvolution: weight input channels %u do not match the input's %u", nn ? wd.w : wd.n, in.c);
         desc_ = d;
@@ -820,6 +837,9 @@ public:
                                       output_->getDataType() == DataType::UINT8, "HipAdd: expects uint8 tensors");
         CHECK_EXPR_RETURN_FAILURE(a_->getTotalSizeFromDims() == b_->getTotalSizeFromDims() &&
                                       a_->getTotalSizeFromDims() == output_->getTotalSizeFromDims(), "HipAdd: shapes differ (no broadcast)");
+        // element by element: any element order, as long as it is the same one
+        CHECK_EXPR_RETURN_FAILURE(a_->storedChannelsLast() == b_->storedChannelsLast() && a_->storedChannelsLast() == output_->storedChannelsLast(),
+                                  "HipAdd: the tensors are stored in different element orders");
         ready_ = true;
         return Status::SUCCESS;
     }
@@ -881,7 +901,9 @@ public:
         d_.pad_b = (int32_t)parameters_->padding.b;
         d_.pad_l = (int32_t)parameters_->padding.l;
         d_.pad_r = (int32_t)parameters_->padding.r;
-        d_.layout = (nchw ? EH_NCHW : EH_NHWC) | (precision_ == PrecisionType::INT8 ? EH_IO_SIGNED : 0);
+        const int order = nchw ? detail::planarOperatorLayout(input_, output_) : EH_NHWC;
+        CHECK_EXPR_RETURN_FAILURE(order >= 0, "HipAveragepool: input and output are stored in different element orders");
+        d_.layout = order | (precision_ == PrecisionType::INT8 ? EH_IO_SIGNED : 0);
         CHECK_EXPR_RETURN_FAILURE(d_.kh > 0 && d_.kw > 0 && d_.stride_h > 0 && d_.stride_w > 0, "HipAveragepool: bad window or stride");
         const int32_t ho = (d_.h + d_.pad_t + d_.pad_b - d_.kh) / d_.stride_h + 1, wo = (d_.w + d_.pad_l + d_.pad_r - d_.kw) / d_.stride_w + 1;
         CHECK_EXPR_RETURN_FAILURE((uint64_t)output_->getTotalSizeFromDims() == (uint64_t)d_.n * d_.c * ho * wo,
@@ -911,6 +933,47 @@ private:
     std::shared_ptr<HipTensor> input_, output_;
     std::shared_ptr<Pool2DParameters> parameters_;
     eh_pool_desc d_{};
+    bool ready_ = false;
+};
+
+// Planar <-> channels-last storage of one byte tensor whose shape reads (n, c, h, w): the operator constructor puts one
+// behind every input and in front of every output of a planar operator list whose feature maps it stores channels-last
+// (nchw2nhwc_uint8 / nhwc2nchw_uint8, cl_kernels/NormalizationKernels and CLTensor.cpp:181-225, as operators of the list).
+class HipLayoutChange {
+public:
+    HipLayoutChange(const std::shared_ptr<HipRuntime> runtime, bool to_channels_last) : runtime_(runtime), to_channels_last_(to_channels_last) {}
+
+    Status initialize(const std::vector<std::shared_ptr<ITensor>> &input_tensors, const std::vector<std::shared_ptr<ITensor>> &output_tensors,
+                      const std::shared_ptr<Parameters> = nullptr) {
+        CHECK_EXPR_RETURN_FAILURE(input_tensors.size() == 1 && output_tensors.size() == 1, "HipLayoutChange: needs one input and one output");
+        input_ = std::static_pointer_cast<HipTensor>(input_tensors.at(0));
+        output_ = std::static_pointer_cast<HipTensor>(output_tensors.at(0));
+        CHECK_EXPR_RETURN_FAILURE(input_->getNumOfBytes() == input_->getTotalSizeFromDims() && output_->getNumOfBytes() == input_->getNumOfBytes(),
+                                  "HipLayoutChange: byte tensors of one size");
+        CHECK_EXPR_RETURN_FAILURE(input_->storedChannelsLast() != to_channels_last_ && output_->storedChannelsLast() == to_channels_last_,
+                                  "HipLayoutChange: the tensors' element orders do not fit the direction");
+        ready_ = true;
+        return Status::SUCCESS;
+    }
+
+    Status execute() {
+        CHECK_EXPR_RETURN_FAILURE(ready_, "HipLayoutChange::execute before initialize");
+        if (input_->getTotalSizeFromDims() == 0) return Status::SUCCESS;
+        const Dim4 d = input_->getDim();
+        const int rc = (to_channels_last_ ? eh_transpose_u8_nchw2nhwc : eh_transpose_u8_nhwc2nchw)(input_->getDataPtr(), output_->getDataPtr(), (int32_t)d.n,
+                                                                                                  (int32_t)d.c, (int32_t)d.h, (int32_t)d.w,
+                                                                                                  runtime_->stream());
+        CHECK_EXPR_RETURN_FAILURE(rc == EH_OK, "HipLayoutChange::execute: %s", eh_last_error());
+        return Status::SUCCESS;
+    }
+
+    bool launchesOnly() const { return true; }
+    Status release() { return Status::SUCCESS; }
+
+private:
+    std::shared_ptr<HipRuntime> runtime_;
+    bool to_channels_last_;
+    std::shared_ptr<HipTensor> input_, output_;
     bool ready_ = false;
 };
 

@@ -108,6 +108,14 @@ public:
     }
     bool isView() const { return whole_ != nullptr; }
 
+    // The device bytes of this tensor, whose shape reads (n, c, h, w), are stored channels-last ([n][h][w][c]).  The
+    // operator constructor stores the feature maps inside a planar operator list that way: the kernels of this backend
+    // work on channels-last data, and a planar tensor costs every operator a transposition on either side.  Operators
+    // ask the tensors they are given; what the owner of the list reads and writes (its inputs and outputs) stays
+    // planar.  No counterpart in the reference, whose kernels are planar.
+    void storeChannelsLast(bool on) { channels_last_ = on; }
+    bool storedChannelsLast() const { return whole_ ? whole_->storedChannelsLast() : channels_last_; }
+
     ~HipTensor() override {
         if (buf_ && buf_.use_count() == 1 && buf_->getDataPtr() != nullptr) (void)runtime_->releaseBuffer(buf_);
     }
@@ -270,6 +278,7 @@ private:
     uint32_t buffer_data_type_;
     int32_t buffer_index_;
     bool is_const_;
+    bool channels_last_ = false;
     std::shared_ptr<HipBuffer> buf_;
     std::shared_ptr<HipTensor> whole_;  // views only
     size_t view_offset_ = 0;

@@ -297,6 +297,12 @@ int eud_set_fuse_expansions(eud_driver *driver, int32_t mode) {
     return 0;
 }
 
+int eud_set_store_channels_last(eud_driver *driver, int32_t on) {
+    if (driver == nullptr || driver->ud.constructor() == nullptr) return fail("eud_set_store_channels_last: no driver");
+    driver->ud.constructor()->store_channels_last = on != 0;
+    return 0;
+}
+
 int eud_synchronize(eud_driver *driver) {
     if (driver == nullptr || !driver->ud.computeLibrary()) return fail("eud_synchronize: no driver");
     return driver->ud.computeLibrary()->runtime()->synchronize() == Status::SUCCESS ? 0 : fail_below("eud_synchronize");

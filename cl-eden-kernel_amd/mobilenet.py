@@ -189,11 +189,12 @@ def compulsory_bytes_per_image(image=224):
     return total
 
 
-def operator_list(ud, list_id, batch, image=224, per_channel=False, weights="minmax"):
+def operator_list(ud, list_id, batch, image=224, per_channel=False, weights="minmax", nchw=False):
     """The same network as a description for the userdriver (`ud` = the userdriver module): an androidNN model with
     channels-last data (use_nchw false), i.e. feature maps [batch, h, w, c], convolution filters [out, kh, kw, in] and
     depthwise filters [1, kh, kw, c] as TFLite stores them, and the explicit padding values of layers() (its
-    symmetric padding is not what SAME gives a stride-2 layer).  Returns (OperatorList, input buffer index, output
+    symmetric padding is not what SAME gives a stride-2 layer).  nchw: the same model with planar data (use_nchw true:
+    feature maps [batch, c, h, w]; the filters stay as they are).  Returns (OperatorList, input buffer index, output
     buffer index, logits shape).  Buffer index i is tensor i of layers()."""
     tensors, ops = layers(image, weights)
     ol = ud.OperatorList(list_id, ud.MODEL_ANDROID_NN)
@@ -202,7 +203,7 @@ def operator_list(ud, list_id, batch, image=224, per_channel=False, weights="min
     def feature_map(i):
         if i not in fm:
             t = tensors[i]
-            shape = (batch, t["h"], t["w"], t["c"])
+            shape = (batch, t["c"], t["h"], t["w"]) if nchw else (batch, t["h"], t["w"], t["c"])
             fm[i] = ol.feature_map(i, shape, t["scale"], t["zp"])
         return fm[i]
 
@@ -214,7 +215,7 @@ def operator_list(ud, list_id, batch, image=224, per_channel=False, weights="min
         s = tensors[op["src"]]
         if kind == "avgpool":
             ol.operator("AVERAGE_POOL_2D_%d" % n, ud.OP_AVERAGE_POOL_2D, [feature_map(op["src"])], [feature_map(op["dst"])],
-                        ud.options(padding=ud.PADDING_VALID, stride=(1, 1), filter=(op["k"], op["k"])))
+                        ud.options(padding=ud.PADDING_VALID, stride=(1, 1), filter=(op["k"], op["k"]), use_nchw=nchw))
             continue
         act = ud.ACT_RELU6 if op.get("relu6") else ud.ACT_NONE
         bias_scale = float(np.float32(s["scale"]) * np.float32(op["w_scale"]))
@@ -236,7 +237,7 @@ def operator_list(ud, list_id, batch, image=224, per_channel=False, weights="min
         wt = ol.parameter(w, 0.0 if per_channel else op["w_scale"], 0 if per_channel else op["w_zp"], per_channel_scales=w_scales)
         bt = ol.parameter(b, 1.0 if per_channel else bias_scale, 0)
         pad = op["pad"]
-        opts = ud.options(padding=ud.PADDING_VALID, stride=(op["stride"],) * 2, activation=act, padding_value=(pad,) * 4)
+        opts = ud.options(padding=ud.PADDING_VALID, stride=(op["stride"],) * 2, activation=act, padding_value=(pad,) * 4, use_nchw=nchw)
         code, name = (ud.OP_DEPTHWISE_CONV_2D, "DEPTHWISE_CONV_2D_%d") if kind == "dw" else (ud.OP_CONV_2D, "CONV_2D_%d")
         ol.operator(name % n, code, [feature_map(op["src"]), wt, bt], [feature_map(op["dst"])], opts)
     last = len(tensors) - 1

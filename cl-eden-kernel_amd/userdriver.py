@@ -56,6 +56,7 @@ EXPORTS = {
     "eud_set_replay": (C.c_int, [C.c_void_p, C.c_int32]),
     "eud_set_image_lanes": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32]),
     "eud_set_fuse_expansions": (C.c_int, [C.c_void_p, C.c_int32]),
+    "eud_set_store_channels_last": (C.c_int, [C.c_void_p, C.c_int32]),
     "eud_synchronize": (C.c_int, [C.c_void_p]),
     "eud_stream": (C.c_void_p, [C.c_void_p]),
     "eud_stats": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_int32), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
@@ -166,6 +167,10 @@ class UserDriver:
     def set_fuse_expansions(self, mode):
         """0: never; 1: where the library's measured table prefers the one launch (default); 2: wherever the kernel fits"""
         check(load().eud_set_fuse_expansions(self.h, mode), "set_fuse_expansions")
+
+    def set_store_channels_last(self, on):
+        """Lists opened from now on: feature maps inside a planar list are stored channels-last (default) or as their shapes read."""
+        check(load().eud_set_store_channels_last(self.h, int(on)), "set_store_channels_last")
 
     def synchronize(self):
         check(load().eud_synchronize(self.h), "synchronize")

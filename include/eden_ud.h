@@ -103,6 +103,12 @@ int eud_set_image_lanes(eud_driver *driver, int32_t lanes, int32_t min_lane_imag
  * faster that way (the default), for mode 2 wherever the kernel fits, for mode 0 never (one operator per description,
  * as the reference builds the list).  Results do not depend on it. */
 int eud_set_fuse_expansions(eud_driver *driver, int32_t mode);
+/* Lists opened from now on: the feature maps inside a PLANAR list (a Caffe-style model, or an androidNN one whose
+ * operators say use_nchw) are stored channels-last, the order the kernels work in, instead of being transposed on either
+ * side of every operator; the list's inputs and outputs stay planar, and one layout operator behind each input and in
+ * front of each output joins the list (on: the default).  off: every tensor is stored as its shape reads, as the
+ * reference does.  Results do not depend on it. */
+int eud_set_store_channels_last(eud_driver *driver, int32_t on);
 int eud_synchronize(eud_driver *driver);         /* IComputeLibrary::synchronize */
 void *eud_stream(eud_driver *driver);            /* the hipStream_t the operators are enqueued on */
 /* operators built for the list, and what the executor has done so far (over all lists) */

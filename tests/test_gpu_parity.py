@@ -616,7 +616,9 @@ def test_deconv_config4_full_size():
                                    (2, 96, 16, 24), (3, 32, 20, 20), (2, 16, 8, 10), (1, 144, 28, 28), (2, 48, 4, 4),
                                    (1, 256, 32, 16), (2, 32, 33, 32), (1, 1280, 4, 4),
                                    # multiples of 4 only: rows finished with single dwords, 16-row groups with single row quads
-                                   (2, 24, 14, 14), (1, 1000, 2, 2), (2, 40, 6, 6), (1, 36, 5, 4), (3, 20, 2, 2), (1, 4, 1, 4)])
+                                   (2, 24, 14, 14), (1, 1000, 2, 2), (2, 40, 6, 6), (1, 36, 5, 4), (3, 20, 2, 2), (1, 4, 1, 4),
+                                   # two to four channels over many pixels (images): a dword per plane, C dwords of pixels
+                                   (2, 3, 32, 40), (3, 2, 16, 16), (1, 4, 9, 28), (5, 3, 224, 224), (2, 3, 7, 9)])
 def test_layout_conversion(shape):
     n, c, h, w = shape
     x = synth.fill_u8(shape, SEED + 70)

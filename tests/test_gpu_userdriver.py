@@ -227,3 +227,83 @@ def test_two_lists_open_at_once_and_error_paths():
         d.open_subgraph(bad)
     with pytest.raises(ud.EdenUdError):
         d.stats(0x203)
+
+
+@pytest.mark.parametrize("batch,lanes", [(2, 1), (4, 2)], ids=["one_chain", "two_lanes"])
+def test_planar_list_stored_channels_last_gives_the_planar_results(batch, lanes):
+    """MobileNetV2 as a PLANAR operator list (feature maps [n, c, h, w], use_nchw): by default the constructor stores the
+    feature maps channels-last and adds one layout operator behind the list's input (per lane); with the switch off
+    every operator transposes on either side, as a planar tensor demands.  The owner of the list writes a planar image
+    either way, and the logits equal the oracle's."""
+    d = driver()
+    image = 96
+    x = np.ascontiguousarray(mobilenet.network_input(batch, image).transpose(0, 3, 1, 2))
+    _, _, want = oracle_images(batch, image, False)
+    ref = want[-1].reshape(batch, -1)
+    d.set_image_lanes(lanes, 1)
+    try:
+        for stored, extra in ((True, lanes), (False, 0)):
+            list_id = 0xA000 + batch * 4 + (1 if stored else 0)
+            d.set_store_channels_last(stored)
+            ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image, nchw=True)
+            d.open_subgraph(ol)
+            assert d.stats(list_id)["operators"] == lanes * 54 + extra
+            for rep in range(3):
+                got = np.zeros(shape, np.uint8)
+                d.execute_subgraph(list_id, {in_index: x, out_index: got})
+                assert np.array_equal(got, ref), (stored, rep, int((got != ref).sum()))
+            d.close_subgraph(list_id)
+    finally:
+        d.set_store_channels_last(True)
+        d.set_image_lanes(2, 16)
+
+
+def test_planar_list_with_planar_outputs_of_many_pixels():
+    """A planar list whose output is a feature map of many pixels (a convolution, a depthwise convolution behind it, and
+    their residual sum): the owner reads a planar tensor although the operators worked on channels-last tensors, the
+    layout operator in front of the output included."""
+    d = driver()
+    n, c, h, w, cout = 3, 8, 13, 18, 16
+    x = O.fill_u8((n, c, h, w), 901)
+    w1 = O.fill_u8((cout, c, 3, 3), 902)
+    b1 = O.fill_i32((cout,), 903, -500, 500)
+    w2 = O.fill_u8((cout, 1, 3, 3), 904)
+    b2 = O.fill_i32((cout,), 905, -500, 500)
+    s_in, z_in, s_w, z_w = 0.02, 120, 0.005, 131
+    s1 = float(0.02 * 0.005 * 74.0 * 74.0 * np.sqrt(9 * c) / 40.0)
+    s2 = float(s1 * 0.005 * 74.0 * 74.0 * 3 / 40.0)
+    q1 = O.make_quant(s_in, z_in, s_w, z_w, s1, 128, O.ACT_NONE, False)
+    q2 = O.make_quant(s1, 128, s_w, z_w, s2, 128, O.ACT_RELU, True)
+    qa = O.make_add_quant(s1, 128, s2, 128, s1, 100, O.ACT_NONE, False)
+    y1 = O.conv2d(x, w1, b1, O.conv_shape(n, c, h, w, cout, 3, 3, pad=(1, 1, 1, 1)), q1)
+    y2 = O.dwconv2d(y1, w2, b2, O.conv_shape(n, cout, h, w, cout, 3, 3, pad=(1, 1, 1, 1), groups=cout), q2)
+    y3 = O.add(y1, y2, qa)
+    for stored in (True, False):
+        list_id = 0xB000 + (1 if stored else 0)
+        d.set_store_channels_last(stored)
+        d.set_image_lanes(1, 16)
+        try:
+            ol = ud.OperatorList(list_id, ud.MODEL_ANDROID_NN)
+            t0 = ol.feature_map(0, (n, c, h, w), s_in, z_in)
+            t1 = ol.feature_map(1, (n, cout, h, w), s1, 128)
+            t2 = ol.feature_map(2, (n, cout, h, w), s2, 128)
+            t3 = ol.feature_map(3, (n, cout, h, w), s1, 100)
+            pad = ud.options(padding=ud.PADDING_VALID, padding_value=(1, 1, 1, 1), use_nchw=True)
+            relu = ud.options(padding=ud.PADDING_VALID, padding_value=(1, 1, 1, 1), use_nchw=True, activation=ud.ACT_RELU)
+            ol.operator("CONV", ud.OP_CONV_2D, [t0, ol.parameter(np.ascontiguousarray(w1.transpose(0, 2, 3, 1)), s_w, z_w),
+                                               ol.parameter(b1, s_in * s_w, 0)], [t1], pad)
+            ol.operator("DW", ud.OP_DEPTHWISE_CONV_2D, [t1, ol.parameter(np.ascontiguousarray(w2.transpose(1, 2, 3, 0)), s_w, z_w),
+                                                        ol.parameter(b2, s1 * s_w, 0)], [t2], relu)
+            ol.operator("ADD", ud.OP_ADD, [t1, t2], [t3])
+            d.open_subgraph(ol)
+            assert d.stats(list_id)["operators"] == (5 if stored else 3)   # + one layout operator per list input and output
+            got = np.zeros((n, cout, h, w), np.uint8)
+            for rep in range(3):
+                got[:] = 0
+                d.execute_subgraph(list_id, {0: x, 3: got})
+                assert np.array_equal(got, y3), (stored, rep, int((got != y3).sum()))
+            d.close_subgraph(list_id)
+        finally:
+            d.set_store_channels_last(True)
+            d.set_image_lanes(2, 16)
+    assert y3.std() > 5 and y2.std() > 5
