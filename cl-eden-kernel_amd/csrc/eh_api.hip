@@ -1580,8 +1580,9 @@ int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan) {
 int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise) {
     if (pointwise == nullptr || depthwise == nullptr) return 0;
     const GemmOp &op = pointwise->op;
-    if (op.parts.size() != 1 || op.layout != EH_NHWC || op.io_signed || op.pc_multiplier) return 0;
-    if (depthwise->d.layout != EH_NHWC || depthwise->io_signed || depthwise->pc_multiplier) return 0;
+    if (op.parts.size() != 1 || op.layout != EH_NHWC || op.io_signed) return 0;
+    if (depthwise->d.layout != EH_NHWC || depthwise->io_signed) return 0;
+    if ((op.pc_multiplier != nullptr) != (depthwise->pc_multiplier != nullptr)) return 0;  // one pair per operator, or one per channel in both
     if (depthwise->d.n != pointwise->d.n || !(depthwise->w_trip || depthwise->w_fold)) return 0;
     // geometry and kernel family are checked on the problems themselves; the pointers and parameters of a run do not enter
     const GemmProblem pw = op.problem(op.parts[0], nullptr, nullptr, nullptr, nullptr);

@@ -71,12 +71,15 @@ __device__ __forceinline__ void column_words(uint32_t r0, uint32_t r1, uint32_t 
 // QM: pointwise requantization, 0 two-step order, 1 / 2 the single-shift forms.  KS: reduction steps of the pointwise
 // stage when they are 1, 2 or 3 (a lane then keeps its pixel's operand bytes in registers across the channel blocks),
 // 0 for any number (read from LDS for every product).
-template <int S, bool FOLD, bool ROWSUM, int QM, int KS>
+template <int S, bool FOLD, bool ROWSUM, int QM, int KS, bool PC>
 __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, const DwProblem dw, const BlockGeom g) {
     const int ksteps = KS ? KS : g.ks;
     extern __shared__ __align__(16) uint8_t lds_raw[];
     v4i *b_s = reinterpret_cast<v4i *>(lds_raw);                              // [nb][ks][64 lanes]: pointwise weights, fragment order
     int32_t *bias_s = reinterpret_cast<int32_t *>(lds_raw + (size_t)g.nb * ksteps * 1024);  // [nb * 32]
+    // PC (one multiplier and shift per channel in both operators): the pointwise stage's pairs beside the bias, as the
+    // single-shift form's table (multiplier, right shift - 1, high word of the rounding term) or, two-step, as they are
+    int32_t *pcm_s = bias_s + g.nb * 32, *pcf_s = pcm_s + g.nb * 32, *pch_s = pcf_s + g.nb * 32;
     uint8_t *img_s = lds_raw + g.image_off;                                   // [ih][iwp][cpitch] uint8 (xor 0x80 for the signed form)
     const int nb_first = blockIdx.y * g.nb;                                   // this workgroup's channel range
     const int c_first = nb_first * 32;
@@ -122,6 +125,14 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
         const v4i *src = reinterpret_cast<const v4i *>(pw.b) + (size_t)nb_first * ksteps * 64;
         for (int i = tid; i < nb_here * ksteps * 64; i += 256) b_s[i] = src[i];
         for (int i = tid; i < nb_here * 32; i += 256) bias_s[i] = pw.bias[c_first + i];
+        if constexpr (PC) {  // (the per-channel arrays are padded to whole channel blocks)
+            for (int i = tid; i < nb_here * 32; i += 256) {
+                const int32_t m = pw.rq.pc_multiplier[c_first + i], sh = pw.rq.pc_shift[c_first + i];
+                pcm_s[i] = m;
+                pcf_s[i] = QM != 0 ? -sh - 1 : sh;
+                pch_s[i] = QM != 0 ? channel_table_pos_hi(pw.rq.zp_out, -sh) : 0;
+            }
+        }
         __syncthreads();
     }
 
@@ -184,7 +195,25 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
             uint32_t packed[4];
 #pragma unroll
             for (int gq = 0; gq < 4; ++gq) {
-                if constexpr (QM != 0) {
+                if constexpr (PC) {
+                    const int tab = nb * 32 + half * 16 + gq * 4;
+                    const int4 cm = *reinterpret_cast<const int4 *>(pcm_s + tab);
+                    const int4 cf = *reinterpret_cast<const int4 *>(pcf_s + tab);
+                    uint32_t o0, o1, o2, o3;
+                    if constexpr (QM != 0) {
+                        const int4 ch = *reinterpret_cast<const int4 *>(pch_s + tab);
+                        o0 = requant_u8_channel_table<QM>(acc[gq * 4 + 0] + ncorr, cm.x, cf.x, ch.x, rq);
+                        o1 = requant_u8_channel_table<QM>(acc[gq * 4 + 1] + ncorr, cm.y, cf.y, ch.y, rq);
+                        o2 = requant_u8_channel_table<QM>(acc[gq * 4 + 2] + ncorr, cm.z, cf.z, ch.z, rq);
+                        o3 = requant_u8_channel_table<QM>(acc[gq * 4 + 3] + ncorr, cm.w, cf.w, ch.w, rq);
+                    } else {
+                        o0 = requant_u8_channel(acc[gq * 4 + 0] + ncorr, cm.x, cf.x, rq);
+                        o1 = requant_u8_channel(acc[gq * 4 + 1] + ncorr, cm.y, cf.y, rq);
+                        o2 = requant_u8_channel(acc[gq * 4 + 2] + ncorr, cm.z, cf.z, rq);
+                        o3 = requant_u8_channel(acc[gq * 4 + 3] + ncorr, cm.w, cf.w, rq);
+                    }
+                    packed[gq] = pack_bytes(o0, o1, o2, o3);
+                } else if constexpr (QM != 0) {
                     packed[gq] = requant4_fast<QM>(acc[gq * 4 + 0], acc[gq * 4 + 1], acc[gq * 4 + 2], acc[gq * 4 + 3], ncorr, rq);
                 } else {
                     packed[gq] = pack_bytes(requant_u8(acc[gq * 4 + 0] + ncorr, rq), requant_u8(acc[gq * 4 + 1] + ncorr, rq),
@@ -231,6 +260,11 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
 #pragma unroll
         for (int kx = 0; kx < 3; ++kx) wk[kx] = *reinterpret_cast<const int4 *>((FOLD ? dw.w_fold : dw.w_trip) + ((uint32_t)kx * (uint32_t)dw.cout + cq * 4u));
         const int4 b4 = *reinterpret_cast<const int4 *>((FOLD ? dw.bias_fold : dw.bias_trip) + cq * 4u);
+        int4 dm = make_int4(0, 0, 0, 0), ds = dm;  // PC: the depthwise stage's four pairs
+        if constexpr (PC) {
+            dm = *reinterpret_cast<const int4 *>(drq.pc_multiplier + cq * 4u);
+            ds = *reinterpret_cast<const int4 *>(drq.pc_shift + cq * 4u);
+        }
         uint32_t colw[IW][4];
         int cs[FOLD ? IW : 1][4];
 #pragma unroll
@@ -266,7 +300,17 @@ __global__ __launch_bounds__(256) void pwdw_block_kernel(const GemmProblem pw, c
                 acc3 += __mul24(-dw.zp_w, cs[j * S][3] + cs[j * S + 1][3] + cs[j * S + 2][3]);
             }
             uint32_t o;
-            if (drq.fast == 2)
+            if constexpr (PC) {
+                if (drq.fast == 2)
+                    o = pack_bytes(requant_u8_channel_fast<2>(acc0, dm.x, ds.x, drq), requant_u8_channel_fast<2>(acc1, dm.y, ds.y, drq),
+                                   requant_u8_channel_fast<2>(acc2, dm.z, ds.z, drq), requant_u8_channel_fast<2>(acc3, dm.w, ds.w, drq));
+                else if (drq.fast)
+                    o = pack_bytes(requant_u8_channel_fast<1>(acc0, dm.x, ds.x, drq), requant_u8_channel_fast<1>(acc1, dm.y, ds.y, drq),
+                                   requant_u8_channel_fast<1>(acc2, dm.z, ds.z, drq), requant_u8_channel_fast<1>(acc3, dm.w, ds.w, drq));
+                else
+                    o = pack_bytes(requant_u8_channel(acc0, dm.x, ds.x, drq), requant_u8_channel(acc1, dm.y, ds.y, drq),
+                                   requant_u8_channel(acc2, dm.z, ds.z, drq), requant_u8_channel(acc3, dm.w, ds.w, drq));
+            } else if (drq.fast == 2)
                 o = requant4_fast<2>(acc0, acc1, acc2, acc3, 0, drq);
             else if (drq.fast)
                 o = requant4_fast<1>(acc0, acc1, acc2, acc3, 0, drq);
@@ -289,7 +333,7 @@ int block_image_pitch(int nb, int c) {
 }
 
 size_t block_lds_bytes(int nb, int ks, int ih, int iwp, int c, uint32_t *a_off, uint32_t *image_off) {
-    const size_t head = ((size_t)nb * ks * 1024 + (size_t)nb * 128 + 15) & ~(size_t)15;
+    const size_t head = ((size_t)nb * ks * 1024 + (size_t)nb * 512 + 15) & ~(size_t)15;  // weights, bias, three per-channel tables
     const size_t a_bytes = ((size_t)ih * iwp * (ks * 32 + 16) + 15) & ~(size_t)15;
     if (a_off) *a_off = (uint32_t)head;
     if (image_off) *image_off = (uint32_t)(head + a_bytes);
@@ -300,14 +344,16 @@ size_t block_lds_bytes(int nb, int ks, int ih, int iwp, int c, uint32_t *a_off, 
 
 // The pointwise problem is a one-tap problem of at most eight 32-byte reduction steps on whole dense images whose
 // weights are packed in fragment order, the depthwise one a 3x3 channels-last layer of stride 1 or 2 on the pointwise
-// output with the 8-bit dot product weights at hand; uint8 tensors and one requantization pair per operator.
+// output with the 8-bit dot product weights at hand; uint8 tensors; one requantization pair per operator, or one pair per
+// channel in both.
 bool pwdw_block_applies(const GemmProblem &pw, const DwProblem &dw) {
     if (pw.cfg.id != GEMM_THIN || pw.k_pad > 256 || pw.k > pw.k_pad || (pw.k & 7) != 0 || (pw.cin & 7) != 0 || pw.k != pw.cin) return false;
     if (pw.stride_h != 1 || pw.stride_w != 1 || pw.y_base != 0 || pw.x_base != 0 || pw.ho != pw.h || pw.wo != pw.w) return false;
-    if (pw.a_xor != 0x80808080u || pw.out_xor != 0u || pw.rq.pc_multiplier || pw.residual) return false;
+    if (pw.a_xor != 0x80808080u || pw.out_xor != 0u || pw.residual) return false;
+    if ((pw.rq.pc_multiplier != nullptr) != (dw.rq.pc_multiplier != nullptr)) return false;
     if (dw.kh != 3 || dw.kw != 3 || dw.dil_h != 1 || dw.dil_w != 1 || dw.stride_h != dw.stride_w || (dw.stride_h != 1 && dw.stride_h != 2)) return false;
     if (dw.dm != 1 || dw.c != dw.cout || dw.c != pw.n || (dw.c & 15) != 0 || dw.h != pw.h || dw.w_ != pw.w) return false;
-    if (dw.io_flip || dw.rq.pc_multiplier || (!dw.w_trip && !dw.w_fold)) return false;
+    if (dw.io_flip || (!dw.w_trip && !dw.w_fold)) return false;
     if (dw.pad_t < 0 || dw.pad_l < 0 || dw.pad_t > 2 || dw.pad_l > 2) return false;
     if ((size_t)dw.n * dw.h * dw.w_ * pw.cin >= (1ull << 31) || (size_t)dw.n * dw.ho * dw.wo * dw.cout >= (1ull << 31)) return false;
     return block_lds_bytes(1, pw.k_pad / 32, 3, 3 * dw.stride_w + 3, dw.c, nullptr, nullptr) <= kBlockLdsMax;  // one row of four outputs, one channel block
@@ -421,8 +467,9 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &caller_dw, int row
     EH_REQUIRE(lds <= kBlockLdsMax, "block: %zu bytes of LDS", lds);
     if (g.total_tiles <= 0) return EH_OK;
     const dim3 grid((unsigned)((g.total_tiles + 7) / 8 * 8), (unsigned)ranges);
-    auto launch = [&](auto s_c, auto fold_c, auto rowsum_c, auto qm_c, auto ks_c) {
-        auto kernel = pwdw_block_kernel<decltype(s_c)::value, decltype(fold_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(ks_c)::value>;
+    auto launch_pc = [&](auto s_c, auto fold_c, auto rowsum_c, auto qm_c, auto ks_c, auto pc_c) {
+        auto kernel = pwdw_block_kernel<decltype(s_c)::value, decltype(fold_c)::value, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(ks_c)::value,
+                                        decltype(pc_c)::value>;
         if (lds > 64 * 1024) {
             // (a driver call, made per launch of the tall-tile shapes only; the default tile height stays below 64 KiB)
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBlockLdsMax);
@@ -430,6 +477,9 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &caller_dw, int row
         }
         hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, pw, dw, g);
         return (int)EH_OK;
+    };
+    auto launch = [&](auto s_c, auto fold_c, auto rowsum_c, auto qm_c, auto ks_c) {
+        return pw.rq.pc_multiplier ? launch_pc(s_c, fold_c, rowsum_c, qm_c, ks_c, std::true_type{}) : launch_pc(s_c, fold_c, rowsum_c, qm_c, ks_c, std::false_type{});
     };
     auto with_ks = [&](auto s_c, auto fold_c, auto rowsum_c, auto qm_c) {
         if (g.ks == 1) return launch(s_c, fold_c, rowsum_c, qm_c, std::integral_constant<int, 1>{});

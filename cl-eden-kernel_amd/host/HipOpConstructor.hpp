@@ -629,9 +629,13 @@ private:
         if (dw.in_tensors[0]->is_const || dw.in_tensors[0]->buffer_index != e->buffer_index) return false;
         const auto readers = tensors_used_.find(e->buffer_index);
         if (readers == tensors_used_.end() || readers->second != 1) return false;
+        // weights quantized per tensor in both operators (uint8), or per channel in both (int8)
+        const bool per_channel = !conv.in_tensors[1]->per_channel_scales.empty();
         for (const auto *op : {&conv, &dw}) {
-            if (!op->in_tensors[1]->is_const || !op->in_tensors[2]->is_const || !op->in_tensors[1]->per_channel_scales.empty()) return false;
-            if (op->in_tensors[1]->data_type != TFlite::TensorType_UINT8 || op->in_tensors[2]->data_type != TFlite::TensorType_INT32) return false;
+            if (!op->in_tensors[1]->is_const || !op->in_tensors[2]->is_const || op->in_tensors[1]->per_channel_scales.empty() == per_channel) return false;
+            if (op->in_tensors[1]->data_type != (per_channel ? TFlite::TensorType_INT8 : TFlite::TensorType_UINT8) ||
+                op->in_tensors[2]->data_type != TFlite::TensorType_INT32)
+                return false;
         }
         for (const auto &t : {x, e, d})
             if (t->is_const || t->data_type != TFlite::TensorType_UINT8 || t->shape.size() != 4) return false;

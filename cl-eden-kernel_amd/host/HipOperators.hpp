@@ -517,6 +517,7 @@ public:
     // for the pointwise convolution that takes this operator into its launch (HipConvolution::fuseDepthwise)
     eh_dwconv_plan *plan() const { return plan_; }
     bool perTensorUint8() const { return !per_channel_ && precision_ == PrecisionType::UINT8 && !weights_as_input_; }
+    bool perChannelUint8() const { return per_channel_ && precision_ == PrecisionType::UINT8 && !weights_as_input_; }
     const std::shared_ptr<HipTensor> &inputTensor() const { return input_; }
     const std::shared_ptr<HipTensor> &outputTensor() const { return output_; }
     Status requantNow(eh_requant *q) { return currentRequant(q); }
@@ -556,8 +557,9 @@ private:
 
 inline Status HipConvolution::fuseDepthwise(const std::shared_ptr<HipDepthwiseConvolution> &depthwise) {
     CHECK_EXPR_RETURN_FAILURE(plan_ != nullptr && !deferred_ && depthwise && depthwise->plan() != nullptr, "HipConvolution::fuseDepthwise before initialize");
-    CHECK_EXPR_RETURN_FAILURE(!per_channel_ && precision_ == PrecisionType::UINT8 && launchesOnly() && !residual_ && depthwise->perTensorUint8(),
-                              "HipConvolution::fuseDepthwise: uint8 tensors, constant per-tensor quantized weights, no residual add");
+    CHECK_EXPR_RETURN_FAILURE(precision_ == PrecisionType::UINT8 && launchesOnly() && !residual_ &&
+                                  (per_channel_ ? depthwise->perChannelUint8() : depthwise->perTensorUint8()),
+                              "HipConvolution::fuseDepthwise: uint8 tensors, constant weights quantized per tensor in both operators or per channel in both, no residual add");
     CHECK_EXPR_RETURN_FAILURE(depthwise->inputTensor() == output_, "HipConvolution::fuseDepthwise: the depthwise convolution does not read this convolution's output");
     if (!eh_conv_dw_block_applies(plan_, depthwise->plan())) return Status::FAILURE;  // (not an error: the caller runs the two operators apart)
     depthwise_ = depthwise;

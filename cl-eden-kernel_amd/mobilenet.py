@@ -335,7 +335,7 @@ class MobileNetV2:
         for index in range(len(self.ops) - 1):
             op, nxt = self.ops[index], self.ops[index + 1]
             if not (op["op"] == "conv" and op["k"] == 1 and nxt["op"] == "dw" and nxt["src"] == op["dst"] and readers[op["dst"]] == 1
-                    and in_lane(index) == in_lane(index + 1)) or per_channel or not fuse_blocks:
+                    and in_lane(index) == in_lane(index + 1)) or not fuse_blocks:
                 continue
             n = sub if in_lane(index) else batch
             if fuse_blocks == "auto":

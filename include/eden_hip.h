@@ -353,7 +353,7 @@ int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
  * depthwise_conv_3x3s2_pad_merge (cl_kernels/DepthwiseconvolutionKernels.cpp:1964-2083).  Takes the two operators' own
  * plans; `_applies` says whether the pair fits (1) or has to run as two launches (0): channels-last uint8 tensors, a
  * pointwise layer of at most 256 input channels (a multiple of 8) whose output is the depthwise input, depthwise 3x3 at
- * stride 1 or 2 without dilation or depth multiplier on a multiple of 16 channels, per-tensor requantization in both.
+ * stride 1 or 2 without dilation or depth multiplier on a multiple of 16 channels, requantization per tensor in both or per channel in both.
  * `_preferred` says whether the one launch is also the faster choice for the pair's shape (1) or the two launches
  * are (0): a table of shapes timed inside a network, kept beside the kernel; a caller that fuses wherever
  * `_preferred` says so never loses to the two launches on a measured shape, and unmeasured shapes stay unfused.

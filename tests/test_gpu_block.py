@@ -177,3 +177,74 @@ def test_block_preferred_is_a_subset_of_applies_and_holds_config3():
         assert eden.conv_dw_block_preferred(pw, dw) == preferred, shape
         pw.destroy()
         dw.destroy()
+
+
+PC_BLOCK_CASES = [
+    # n, h, w, cin, c, stride, rows
+    (2, 56, 56, 24, 144, 2, 0),
+    (2, 28, 28, 32, 192, 1, 4),
+    (3, 14, 14, 64, 384, 1, 0),
+    (1, 13, 11, 16, 48, 1, 3),
+    (1, 9, 10, 40, 80, 2, 0),      # a reduction that ends inside its second step; channels not a multiple of 32
+]
+
+
+@pytest.mark.parametrize("case", PC_BLOCK_CASES, ids=lambda c: "x".join(str(v) for v in c))
+def test_block_with_one_pair_per_channel_in_both_operators(case):
+    """int8 weights with one multiplier and shift per channel in the pointwise and in the depthwise operator: the fused
+    launch against the oracle's per-channel chain and the two stand-alone launches; the single-shift forms with and
+    without the sign test, the two-step order once a channel's shift leaves the range, a weight zero point other than 0
+    (row-sum term in the pointwise stage, the unsigned dot-product form in the depthwise stage)."""
+    n, h, w, cin, c, stride, rows = case
+    print("per-channel block", case, flush=True)
+    x = synth.fill_u8((n, h, w, cin), SEED + 5000 + c)
+    w1 = (synth.fill_u8((c, cin, 1, 1), SEED + 5001).astype(np.int16) - 128).astype(np.int8)
+    b1 = synth.fill_i32((c,), SEED + 5002, -500, 500)
+    w2 = (synth.fill_u8((c, 1, 3, 3), SEED + 5003).astype(np.int16) - 128).astype(np.int8)
+    b2 = synth.fill_i32((c,), SEED + 5004, -500, 500)
+    ws1 = (0.002 * (1.0 + 29.0 * synth.fill_u8((c,), SEED + 5005) / 255.0)).astype(np.float32)
+    ws2 = (0.002 * (1.0 + 29.0 * synth.fill_u8((c,), SEED + 5006) / 255.0)).astype(np.float32)
+    s_mid = float(0.02 * float(ws1.max()) * 74.0 * 74.0 * np.sqrt(cin) / 60.0)
+    s_out = float(s_mid * float(ws2.max()) * 74.0 * 74.0 * 3.0 / 60.0)
+    pad = (1, 1, 1, 1)
+    ho, wo = (h + 2 - 3) // stride + 1, (w + 2 - 3) // stride + 1
+    xp = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    s1 = O.conv_shape(n, cin, h, w, c, 1, 1)
+    s2 = O.conv_shape(n, c, h, w, c, 3, 3, stride=(stride, stride), pad=pad, groups=c)
+    d1 = eden.conv_desc(n, cin, h, w, c, 1, 1, layout=eden.NHWC, weight_layout=eden.W_OIHW | eden.W_SIGNED)
+    d2 = eden.conv_desc(n, c, h, w, c, 3, 3, stride=(stride, stride), pad=pad, dm=1, layout=eden.NHWC, weight_layout=eden.W_OIHW | eden.W_SIGNED)
+    keep = [eden.DeviceBuffer(host=a) for a in (w1, b1, w2, b2)]
+    d_x, d_o, d_mid, d_o2 = (eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * ho * wo * c), eden.DeviceBuffer(nbytes=n * h * w * c),
+                             eden.DeviceBuffer(nbytes=n * ho * wo * c))
+    variants = 0
+    for act_floor, zp_w, odd in ((0, 0, False), (128, 0, False), (0, 0, True), (0, -9, False)):
+        q1, m1, sh1 = eden.make_requant_perchannel(0.02, 117, ws1, s_mid, 128, eden.ACT_NONE, False)
+        q2, m2, sh2 = eden.make_requant_perchannel(s_mid, 128, ws2, s_out, 128, eden.ACT_NONE, False)
+        q1.act_min = q2.act_min = act_floor
+        q1.zp_w = q2.zp_w = zp_w
+        if odd:   # one channel of each operator outside the single-shift form's range
+            sh1, sh2 = sh1.copy(), sh2.copy()
+            sh1[c // 3] = 0
+            sh2[c // 2] = -21
+        oq1 = O.raw_quant(zp_in=117, zp_w=zp_w, zp_out=128, act_min=act_floor)
+        oq2 = O.raw_quant(zp_in=128, zp_w=zp_w, zp_out=128, act_min=act_floor)
+        mid = O.conv2d_perchannel(xp, w1, b1, s1, oq1, m1, sh1)
+        want = np.ascontiguousarray(O.dwconv2d_perchannel(mid, w2, b2, s2, oq2, m2, sh2).transpose(0, 2, 3, 1))
+        pw = eden.ConvPlan(d1, keep[0], keep[1], q1)
+        dw = eden.DwConvPlan(d2, keep[2], keep[3], q2)
+        pw.set_perchannel(m1, sh1)
+        assert not eden.conv_dw_block_applies(pw, dw)   # one operator per channel, the other per tensor
+        dw.set_perchannel(m2, sh2)
+        assert eden.conv_dw_block_applies(pw, dw)
+        eden.conv_dw_block_run(pw, dw, d_x, d_o, q1, q2, rows)
+        fused = d_o.download((n, ho, wo, c))
+        pw.run(d_x, d_mid, q1)
+        dw.run(d_mid, d_o2, q2)
+        apart = d_o2.download((n, ho, wo, c))
+        pw.destroy()
+        dw.destroy()
+        assert np.array_equal(apart, want), (act_floor, zp_w, odd, diff_report(apart, want))
+        assert np.array_equal(fused, want), (act_floor, zp_w, odd, diff_report(fused, want))
+        assert want.std() > 4 and mid.std() > 4
+        variants += 1
+    assert variants == 4
