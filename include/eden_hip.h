@@ -314,7 +314,8 @@ int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const 
  * (n*c*h*w + n*cout*ho*wo bytes, each rounded up to 256 plus 256) exceeds the array or the plan has more than
  * 8 groups.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
  * threads) race; calls ordered on one stream do not.  Results are bit for bit those of eh_conv2d_u8_run.  The first
- * launch of a one-tap kernel variant at a given LDS size asks the driver once how many of its workgroups a CU holds
+ * launch of a persistent-grid kernel variant (the one-tap and the few-channel first-layer kernels) at a given LDS size
+ * asks the driver once how many of its workgroups a CU holds
  * (an occupancy query: no allocation, no stream operation, legal under capture); every later launch reads the cached
  * answer. */
 #define EH_STATIC_SCRATCH_BYTES (32u << 20)
