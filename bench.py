@@ -256,20 +256,25 @@ def block_workload(eden, synth, n=32, rows=0, cols=0, cold=False, cin=24, c=144,
                 launch=launch, keep=(bufs, keep, pw, dw), sets=sets, ops=2.0 * n * (hw * hw * cin * c + ho * ho * c * 9), bytes=nbytes, bound="hbm")
 
 
-def deconv_workload(eden, synth, n=8, cold=False):
-    desc = eden.conv_desc(n, 256, 32, 32, 128, 4, 4, stride=(2, 2), pad=(1, 1, 1, 1), layout=eden.NHWC,
+def deconv_workload(eden, synth, n=8, cold=False, cin=256, cout=128, hw=32, k=4, stride=2):
+    """transposed convolution, channels-last: BASELINE configs[3] (4x4 stride 2, 256 -> 128 channels at 32 x 32) by default"""
+    pad = (k - stride) // 2 if k >= stride else 0
+    ho = (hw - 1) * stride + k - 2 * pad
+    desc = eden.conv_desc(n, cin, hw, hw, cout, k, k, stride=(stride, stride), pad=(pad,) * 4, layout=eden.NHWC,
                           weight_layout=eden.W_IOHW)
-    x = synth.fill_u8((n, 32, 32, 256), SEED + 64)
-    w = synth.fill_u8((256, 128, 4, 4), SEED + 65)
-    b = synth.fill_i32((128,), SEED + 66, -1000, 1000)
-    q = eden.make_requant(0.02, 121, 0.005, 133, 0.35, 128)
+    x = synth.fill_u8((n, hw, hw, cin), SEED + 64)
+    w = synth.fill_u8((cin, cout, k, k), SEED + 65)
+    b = synth.fill_i32((cout,), SEED + 66, -1000, 1000)
+    q = eden.make_requant(0.02, 121, 0.005, 133, 0.35 * (cin * k * k / 4096.0) ** 0.5, 128)
     d_w, d_b = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
     plan = eden.DeconvPlan(desc, d_w, d_b, q)
-    nbytes = n * 256 * 1024 + 256 * 128 * 16 + 512 + n * 128 * 4096
+    nbytes = n * cin * hw * hw + cin * cout * k * k + 4 * cout + n * cout * ho * ho
     sets = set_count(nbytes, cold)
-    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * 64 * 64 * 128)) for _ in range(sets)]
-    return dict(name="deconv4x4s2_n%d_256to128_32x32_nhwc" % n, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
-                keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * 1024 * 256 * 2048, bytes=nbytes, bound="mfma")
+    bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * ho * ho * cout)) for _ in range(sets)]
+    ops = 2.0 * n * hw * hw * cin * cout * k * k   # every input pixel meets every tap once
+    return dict(name="deconv%dx%ds%d_n%d_%dto%d_%dx%d_nhwc" % (k, k, stride, n, cin, cout, hw, hw), launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+                keep=(bufs, d_w, d_b, plan), sets=sets, ops=ops, bytes=nbytes,
+                bound="mfma" if (cin, cout, hw, k, stride) == (256, 128, 32, 4, 2) or ops / nbytes >= 625 else "hbm")
 
 
 def mbv2_workload(eden, synth, batch=64, per_channel=False, weights="minmax", cold=False, lanes=2, fuse_blocks="auto"):
@@ -546,6 +551,9 @@ def main():
     if args.only and args.only.startswith("fc:"):      # fc:M,K,N = that fully connected layer
         m, k, n = (int(v) for v in args.only[3:].split(","))
         families[args.only] = shaped(fc_workload, m=m, k=k, n=n)
+    if args.only and args.only.startswith("deconv:"):  # deconv:N,CIN,COUT,HW,K,STRIDE = that transposed convolution
+        n, cin, cout, hw, k, stride = (int(v) for v in args.only[7:].split(","))
+        families[args.only] = shaped(deconv_workload, n=n, cin=cin, cout=cout, hw=hw, k=k, stride=stride)
     if args.only and args.only.startswith("conv:"):    # conv:N,CIN,COUT,HW,K,STRIDE = that convolution
         n, cin, cout, hw, k, stride = (int(v) for v in args.only[5:].split(","))
         families[args.only] = shaped(conv_workload, n=n, cin=cin, cout=cout, hw=hw, k=k, stride=stride)

@@ -289,7 +289,7 @@ int igemm_n_tile(int32_t, int32_t, int32_t) { return 256; }
 
 int launch_igemm(const GemmProblem &p, hipStream_t stream) {
     if (p.m <= 0 || p.n <= 0) return EH_OK;
-    if (p.cfg.id == GEMM_THIN) return launch_igemm_thin(p, stream);
+    if (p.cfg.id == GEMM_THIN) return launch_igemm_thin(&p, 1, stream);
     if (p.cfg.id == GEMM_C3K3) return launch_conv_c3k3(p, stream);
     if (p.cfg.id == GEMM_CONV3X3) return launch_conv3x3_patch(p, stream);
     if (p.cfg.id == GEMM_ROWS) return launch_conv_rows(p, stream);
@@ -317,8 +317,21 @@ int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream) {
             while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == p.cfg.id && ps[i + run].m == p.m &&
                    ps[i + run].n == p.n && ps[i + run].k_pad == p.k_pad && ps[i + run].dense == p.dense && ps[i + run].zw == p.zw)
                 ++run;
+        // ... and so do equally shaped one-tap problems (the phases of a transposed convolution whose kernel is its stride)
+        const bool thin = p.cfg.id == GEMM_THIN && p.m > 0 && p.n > 0 && p.residual == nullptr;
+        if (thin)
+            while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == GEMM_THIN && ps[i + run].residual == nullptr &&
+                   ps[i + run].m == p.m && ps[i + run].n == p.n && ps[i + run].k == p.k && ps[i + run].k_pad == p.k_pad && ps[i + run].cin == p.cin &&
+                   ps[i + run].ldc == p.ldc && ps[i + run].zw == p.zw && ps[i + run].ho == p.ho && ps[i + run].wo == p.wo && ps[i + run].h == p.h &&
+                   ps[i + run].w == p.w && ps[i + run].stride_h == p.stride_h && ps[i + run].stride_w == p.stride_w && ps[i + run].out_sy == p.out_sy &&
+                   ps[i + run].out_sx == p.out_sx && ps[i + run].out_h == p.out_h && ps[i + run].out_w == p.out_w &&
+                   ps[i + run].y_base == p.y_base && ps[i + run].x_base == p.x_base && ps[i + run].a_offset == p.a_offset &&
+                   ps[i + run].rq.fast == p.rq.fast && (ps[i + run].rq.pc_multiplier != nullptr) == (p.rq.pc_multiplier != nullptr))
+                ++run;
         int rc;
-        if (dma && run > 1) {
+        if (thin && run > 1) {
+            rc = launch_igemm_thin(ps + i, run, stream);
+        } else if (dma && run > 1) {
             EH_REQUIRE(p.k_pad % 64 == 0 && p.k_pad > 0, "igemm: padded reduction length %d", p.k_pad);
             rc = launch_igemm_dma(ps + i, run, stream);
         } else {

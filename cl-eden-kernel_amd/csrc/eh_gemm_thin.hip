@@ -52,9 +52,17 @@ struct ThinStage {
     int32_t linear;
 };
 
-template <int NBU, int KU, bool ROWSUM, int QM, bool RES>
-__global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, const int n_blocks, const int ksteps, const int nbw,
-                                                          const int row_blocks, const ThinStage stage) {
+// one problem, or (BATCHED) up to four equally shaped ones along grid z
+__device__ __forceinline__ const GemmProblem &problem_of(const GemmProblem &one) { return one; }
+__device__ __forceinline__ const GemmProblem &problem_of(const GemmBatch &batch) { return batch.p[blockIdx.z]; }
+
+template <int NBU, int KU, bool ROWSUM, int QM, bool RES, bool BATCHED = false>
+__global__ __launch_bounds__(256) void direct_gemm_kernel(const std::conditional_t<BATCHED, GemmBatch, GemmProblem> arg, const int n_blocks,
+                                                          const int ksteps, const int nbw, const int row_blocks, const ThinStage stage) {
+    // BATCHED: equally shaped problems of one operator (the output phases of a transposed convolution whose kernel is its
+    // stride) that differ in their weights and in where their outputs go.  (A kernel of its own: indexing the argument
+    // costs the single problem 2 - 3 %.)
+    const GemmProblem &p = problem_of(arg);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, half = lane >> 5;
     const int plane = p.ho * p.wo;
@@ -367,7 +375,10 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const GemmProblem p, c
 }
 
 template <int NBU, int KU>
-int launch_nbu(const GemmProblem &p, hipStream_t stream) {
+int launch_nbu(const GemmProblem *ps, int count, hipStream_t stream) {
+    const GemmProblem &p = ps[0];
+    GemmBatch batch;
+    for (int i = 0; i < count; ++i) batch.p[i] = ps[i];
     const int n_blocks = (p.n + 31) / 32, ksteps = p.k_pad / 32;
     const int row_blocks = (p.m + 31) / 32;
     // Channel ranges: as few as the LDS budget for the weights allows (32 KiB, so that several workgroups share a CU),
@@ -406,7 +417,10 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
     // row sums, the single-shift requantization and the fused residual add are compile-time variants: a launch pays for
     // none of the code it does not use
     auto launch = [&](auto rowsum_c, auto qm_c, auto res_c) {
-        auto kernel = direct_gemm_kernel<NBU, KU, decltype(rowsum_c)::value, decltype(qm_c)::value, decltype(res_c)::value>;
+        constexpr bool RS = decltype(rowsum_c)::value, RES = decltype(res_c)::value;
+        constexpr int QM = decltype(qm_c)::value;
+        const void *kernel = count > 1 ? reinterpret_cast<const void *>(direct_gemm_kernel<NBU, KU, RS, QM, false, true>)
+                                       : reinterpret_cast<const void *>(direct_gemm_kernel<NBU, KU, RS, QM, RES, false>);
         // The grid is persistent: as many workgroups as the device holds at once with this variant's registers and
         // this launch's LDS (a wave has one pixel block in flight, so the bytes in flight grow with the waves), and
         // at least four per CU.  The answer is kept per KiB of LDS.
@@ -420,9 +434,14 @@ int launch_nbu(const GemmProblem &p, hipStream_t stream) {
             resident[slot].store(per_cu, std::memory_order_relaxed);
         }
         int row_wgs = ((row_blocks + 7) / 8 + 3) / 4 * 8;   // a multiple of 8: every XCD walks its own eighth of the row blocks
-        const int wg_target = 256 * per_cu / ranges > 8 ? 256 * per_cu / ranges / 8 * 8 : 8;
+        const int wg_target = 256 * per_cu / (ranges * count) > 8 ? 256 * per_cu / (ranges * count) / 8 * 8 : 8;
         if (row_wgs > wg_target) row_wgs = wg_target;
-        hipLaunchKernelGGL(kernel, dim3(row_wgs, ranges), dim3(256), lds_all, stream, p, n_blocks, ksteps, nbw, row_blocks, stage);
+        if (count > 1)
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, RS, QM, false, true>), dim3(row_wgs, ranges, count), dim3(256), lds_all, stream, batch, n_blocks,
+                               ksteps, nbw, row_blocks, stage);
+        else
+            hipLaunchKernelGGL((direct_gemm_kernel<NBU, KU, RS, QM, RES, false>), dim3(row_wgs, ranges), dim3(256), lds_all, stream, p, n_blocks, ksteps, nbw,
+                               row_blocks, stage);
     };
     auto with_res = [&](auto rowsum_c, auto qm_c) {
         if (p.residual)
@@ -460,27 +479,36 @@ bool igemm_thin_applies(int32_t taps, int32_t cin_group, int32_t pixel_stride, i
     return cin_group <= 64 || (cin_group <= 256 && m * n * cin_group <= 1500000000ll);
 }
 
-int launch_igemm_thin(const GemmProblem &p, hipStream_t stream) {
+int launch_igemm_thin(const GemmProblem *ps, int count, hipStream_t stream) {
+    const GemmProblem &p = ps[0];
+    EH_REQUIRE(count >= 1 && count <= GemmBatch::MAX, "igemm_thin: batch of %d", count);
+    for (int i = 1; i < count; ++i)
+        EH_REQUIRE(ps[i].m == p.m && ps[i].n == p.n && ps[i].k == p.k && ps[i].k_pad == p.k_pad && ps[i].cin == p.cin && ps[i].ldc == p.ldc && ps[i].zw == p.zw &&
+                       ps[i].residual == nullptr && p.residual == nullptr && ps[i].rq.fast == p.rq.fast &&
+                       (ps[i].rq.pc_multiplier != nullptr) == (p.rq.pc_multiplier != nullptr) && ps[i].h == p.h && ps[i].w == p.w && ps[i].ho == p.ho &&
+                       ps[i].wo == p.wo && ps[i].stride_h == p.stride_h && ps[i].stride_w == p.stride_w && ps[i].out_sy == p.out_sy && ps[i].out_sx == p.out_sx &&
+                       ps[i].out_h == p.out_h && ps[i].out_w == p.out_w,
+                   "igemm_thin: a batch must hold equally shaped problems");
     EH_REQUIRE(p.k_pad % 32 == 0 && p.k_pad >= p.k, "igemm_thin: padded reduction length %d", p.k_pad);
     EH_REQUIRE((p.k & 7) == 0 && (p.cin & 7) == 0 && (reinterpret_cast<uintptr_t>(p.a) & 7) == 0,
                "igemm_thin: rows must start on 8-byte boundaries");
     const int n_blocks = (p.n + 31) / 32;
     if (p.k_pad == 32) {
-        if (n_blocks == 1) return launch_nbu<1, 1>(p, stream);
-        if (n_blocks == 2) return launch_nbu<2, 1>(p, stream);
-        return launch_nbu<4, 1>(p, stream);
+        if (n_blocks == 1) return launch_nbu<1, 1>(ps, count, stream);
+        if (n_blocks == 2) return launch_nbu<2, 1>(ps, count, stream);
+        return launch_nbu<4, 1>(ps, count, stream);
     }
     if (p.k_pad == 64) {
-        if (n_blocks == 1) return launch_nbu<1, 2>(p, stream);
-        if (n_blocks == 2) return launch_nbu<2, 2>(p, stream);
-        return launch_nbu<4, 2>(p, stream);
+        if (n_blocks == 1) return launch_nbu<1, 2>(ps, count, stream);
+        if (n_blocks == 2) return launch_nbu<2, 2>(ps, count, stream);
+        return launch_nbu<4, 2>(ps, count, stream);
     }
     if (p.k_pad <= 192) {  // one group of six steps: a row block's loads leave together
-        if (n_blocks == 1) return launch_nbu<1, 6>(p, stream);
-        return launch_nbu<2, 6>(p, stream);
+        if (n_blocks == 1) return launch_nbu<1, 6>(ps, count, stream);
+        return launch_nbu<2, 6>(ps, count, stream);
     }
-    if (n_blocks == 1) return launch_nbu<1, 4>(p, stream);
-    return launch_nbu<2, 4>(p, stream);
+    if (n_blocks == 1) return launch_nbu<1, 4>(ps, count, stream);
+    return launch_nbu<2, 4>(ps, count, stream);
 }
 
 }  // namespace eh

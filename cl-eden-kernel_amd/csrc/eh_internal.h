@@ -418,7 +418,7 @@ int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream);
 int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream);  // vec == 16 and a k-table that fits LDS
 GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k, int32_t siblings);
 inline size_t igemm_dma_ktab_limit() { return 12288; }
-int launch_igemm_thin(const GemmProblem &p, hipStream_t stream);
+int launch_igemm_thin(const GemmProblem *ps, int count, hipStream_t stream);  // `count` equally shaped problems as one launch
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
 int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream);
 // one tap, few output pixels, long reductions: cut along the weights (eh_gemm_skinny.hip)

@@ -564,6 +564,9 @@ DECONV_CASES = [
     # kernel <= stride (every phase is one tap) with a negative tail padding: phases larger than the input
     dict(n=2, c=16, h=6, w=6, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, -2, 0, -2)),
     dict(n=2, c=16, h=6, w=6, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, 0, 0, 0)),
+    # nine one-tap phases of equal shape: launches of four, four and one problems of the one-tap kernel
+    dict(n=2, c=32, h=9, w=7, cout=48, kh=3, kw=3, stride=(3, 3), pad=(0, 0, 0, 0)),
+    dict(n=3, c=64, h=20, w=20, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, 0, 0, 0)),
 ]
 
 
