@@ -317,7 +317,8 @@ int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream) {
             while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == p.cfg.id && ps[i + run].m == p.m &&
                    ps[i + run].n == p.n && ps[i + run].k_pad == p.k_pad && ps[i + run].dense == p.dense && ps[i + run].zw == p.zw)
                 ++run;
-        // ... and so do equally shaped one-tap problems (the phases of a transposed convolution whose kernel is its stride)
+        // ... and so do equally shaped one-tap problems (the phases of a transposed convolution whose kernel is its stride,
+        // the groups of a grouped 1x1 convolution)
         const bool thin = p.cfg.id == GEMM_THIN && p.m > 0 && p.n > 0 && p.residual == nullptr;
         if (thin)
             while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == GEMM_THIN && ps[i + run].residual == nullptr &&
@@ -325,7 +326,7 @@ int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream) {
                    ps[i + run].ldc == p.ldc && ps[i + run].zw == p.zw && ps[i + run].ho == p.ho && ps[i + run].wo == p.wo && ps[i + run].h == p.h &&
                    ps[i + run].w == p.w && ps[i + run].stride_h == p.stride_h && ps[i + run].stride_w == p.stride_w && ps[i + run].out_sy == p.out_sy &&
                    ps[i + run].out_sx == p.out_sx && ps[i + run].out_h == p.out_h && ps[i + run].out_w == p.out_w &&
-                   ps[i + run].y_base == p.y_base && ps[i + run].x_base == p.x_base && ps[i + run].a_offset == p.a_offset &&
+                   ps[i + run].y_base == p.y_base && ps[i + run].x_base == p.x_base &&
                    ps[i + run].rq.fast == p.rq.fast && (ps[i + run].rq.pc_multiplier != nullptr) == (p.rq.pc_multiplier != nullptr))
                 ++run;
         int rc;

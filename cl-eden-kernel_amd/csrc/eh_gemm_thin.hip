@@ -409,7 +409,8 @@ int launch_nbu(const GemmProblem *ps, int count, hipStream_t stream) {
     }
     const size_t lds_all = stage.pitch ? (size_t)stage.offset + 4u * 32u * stage.pitch : lds;
     {
-        const long reach_in = (long)p.m * p.cin + p.a_offset + 16, reach_out = (long)p.m * p.ldc;
+        // (a batch's problems may start at different channels of the pixel: none starts beyond its end)
+        const long reach_in = (long)p.m * p.cin + p.cin + 16, reach_out = (long)p.m * p.ldc;
         stage.linear = dense_out && p.stride_h == 1 && p.stride_w == 1 && p.y_base == 0 && p.x_base == 0 && p.h == p.ho && p.w == p.wo &&
                        p.a_offset >= 0 && p.m < (1 << 24) && p.cin < (1 << 24) && p.ldc < (1 << 24) && reach_in < (1l << 32) &&
                        reach_out < (1l << 32);

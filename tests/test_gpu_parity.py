@@ -198,6 +198,7 @@ CONV_CASES = [
     dict(n=2, c=40, h=13, w=13, cout=240, kh=1, kw=1, stride=(2, 2)),                       # two steps, strided rows
     dict(n=2, c=64, h=12, w=12, cout=32, kh=1, kw=1),
     dict(n=1, c=48, h=10, w=10, cout=96, kh=1, kw=1, groups=2),                             # 24-byte rows inside 48-byte pixels
+    dict(n=2, c=240, h=14, w=14, cout=120, kh=1, kw=1, groups=6),                            # six groups: launches of four and two problems
     dict(n=5, c=16, h=33, w=5, cout=96, kh=1, kw=1, stride=(1, 2)),
     # ... whose output leaves through the per-wave LDS image: one 16-byte chunk per pixel, the widest pixel (256 bytes),
     # a last pixel block of three pixels
