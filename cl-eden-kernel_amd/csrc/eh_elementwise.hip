@@ -36,6 +36,7 @@ __global__ __launch_bounds__(256) void add_u8_kernel(const uint8_t *__restrict__
 struct PoolDev {
     int32_t n, c, h, w, ho, wo, kh, kw, stride_h, stride_w, pad_t, pad_l, act_min, act_max;
     uint32_t flip;  // 0x80808080 for int8 tensors: stored byte ^ 0x80 = value + 128
+    FastDiv div_cq, div_wo, div_ho, div_full;  // by c / 4, wo, ho and kh * kw (launches of fewer than 2^31 threads)
 };
 
 // Window sum over (value + 128 for int8 tensors) to the stored output byte.  uint8: (sum + n/2) / n.  int8: the sum of
@@ -112,6 +113,73 @@ __global__ __launch_bounds__(256) void avgpool_nhwc_vec4_kernel(const uint8_t *_
     if (live && part == 0)
         *reinterpret_cast<uint32_t *>(out + idx * 4) = pool_finish(s0, cnt, p) | (pool_finish(s1, cnt, p) << 8) |
                                                        (pool_finish(s2, cnt, p) << 16) | (pool_finish(s3, cnt, p) << 24);
+}
+
+// The same for launches of fewer than 2^31 threads, which is all but absurd ones: 32-bit indices decoded with
+// multiplications (the 64-bit divisions of the kernel above cost more than a small window's loads and sums together:
+// a 2x2 stride-2 pool of 64 x 112 x 112 x 64 took 34 us for 64 MB), the division by the window size as a multiplication
+// wherever the window lies wholly inside the image, and a window row fetched four pixels at a time.
+template <int ROWS>
+__global__ __launch_bounds__(256) void avgpool_nhwc_vec4_small_index_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                                            const PoolDev p, const uint32_t total) {
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t idx = tid / ROWS;
+    const int part = (int)(tid % ROWS);
+    const bool live = idx < total;  // whole groups of ROWS lanes are live or not; all lanes reach the shuffles
+    const uint32_t cq = (uint32_t)p.c >> 2;
+    uint32_t r = live ? fastdiv(idx, p.div_cq) : 0u;
+    const uint32_t c4 = live ? idx - r * cq : 0u;
+    const uint32_t r1 = fastdiv(r, p.div_wo);
+    const int ox = (int)(r - r1 * (uint32_t)p.wo);
+    const uint32_t img = fastdiv(r1, p.div_ho);
+    const int oy = (int)(r1 - img * (uint32_t)p.ho);
+    int y0 = oy * p.stride_h - p.pad_t, x0 = ox * p.stride_w - p.pad_l;
+    const int y1 = y0 + p.kh < p.h ? y0 + p.kh : p.h, x1 = x0 + p.kw < p.w ? x0 + p.kw : p.w;
+    y0 = y0 < 0 ? 0 : y0;
+    x0 = x0 < 0 ? 0 : x0;
+    const int cnt = (y1 - y0) * (x1 - x0);
+    int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    auto take = [&](uint32_t v) {
+        v ^= p.flip;
+        s0 += v & 255u;
+        s1 += (v >> 8) & 255u;
+        s2 += (v >> 16) & 255u;
+        s3 += v >> 24;
+    };
+    const size_t row_bytes = (size_t)p.w * p.c;
+    for (int y = y0 + part; y < y1 && live; y += ROWS) {
+        const uint8_t *row = in + ((size_t)img * p.h + y) * row_bytes + c4 * 4;
+        for (int x = x0; x < x1; x += 4) {  // four window pixels are requested before the first is summed
+            uint32_t v[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) v[t] = x + t < x1 ? *reinterpret_cast<const uint32_t *>(row + (size_t)(x + t) * p.c) : p.flip;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) take(v[t]);
+        }
+    }
+#pragma unroll
+    for (int step = 1; step < ROWS; step <<= 1) {
+        s0 += __shfl_xor(s0, step);
+        s1 += __shfl_xor(s1, step);
+        s2 += __shfl_xor(s2, step);
+        s3 += __shfl_xor(s3, step);
+    }
+    if (live && part == 0) {
+        uint32_t o;
+        if (cnt == p.kh * p.kw && !p.flip) {  // the whole window, uint8 rule: (sum + n / 2) / n with the division as a multiplication
+            const uint32_t half = (uint32_t)cnt >> 1;
+            auto fin = [&](int sum) {
+                int v = (int)fastdiv((uint32_t)sum + half, p.div_full);
+                v = v < p.act_min ? p.act_min : v;
+                v = v > p.act_max ? p.act_max : v;
+                return (uint32_t)v & 255u;
+            };
+            o = fin(s0) | (fin(s1) << 8) | (fin(s2) << 16) | (fin(s3) << 24);
+        } else {
+            o = pool_finish(s0, cnt, p) | (pool_finish(s1, cnt, p) << 8) | (pool_finish(s2, cnt, p) << 16) | (pool_finish(s3, cnt, p) << 24);
+        }
+        *reinterpret_cast<uint32_t *>(out + (size_t)idx * 4) = o;
+    }
 }
 
 // one output element per thread, either layout
@@ -245,6 +313,20 @@ int eh_avgpool_u8(const void *in, void *out, const eh_pool_desc *desc, void *str
     const bool split_rows = vec4 && total < 256 * 1024 && d.kh >= 4;  // few threads, tall windows: eight lanes per output
     const int64_t blocks = ((split_rows ? total * 8 : total) + 255) / 256;
     EH_REQUIRE(blocks < (1ll << 31), "avgpool: tensor too large");
+    if (vec4 && blocks * 256 < (1ll << 31) && p.ho > 0 && p.wo > 0 && total > 0) {
+        p.div_cq = make_fastdiv((uint32_t)(d.c >> 2));
+        p.div_wo = make_fastdiv((uint32_t)p.wo);
+        p.div_ho = make_fastdiv((uint32_t)p.ho);
+        p.div_full = make_fastdiv((uint32_t)(d.kh * d.kw));
+        if (split_rows)
+            hipLaunchKernelGGL(avgpool_nhwc_vec4_small_index_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint8_t *>(in),
+                               static_cast<uint8_t *>(out), p, (uint32_t)total);
+        else
+            hipLaunchKernelGGL(avgpool_nhwc_vec4_small_index_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint8_t *>(in),
+                               static_cast<uint8_t *>(out), p, (uint32_t)total);
+        EH_HIP(hipGetLastError());
+        return EH_OK;
+    }
     if (split_rows)
         hipLaunchKernelGGL(avgpool_nhwc_vec4_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint8_t *>(in),
                            static_cast<uint8_t *>(out), p, total);
