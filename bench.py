@@ -174,11 +174,11 @@ def conv_workload(eden, synth, n=1, cold=False, cin=64, cout=64, hw=56, k=3, str
                 bound="mfma" if (cin, cout, hw, k, stride) == (64, 64, 56, 3, 1) or 2.0 * n * ho * ho * cout * cin * k * k / nbytes >= 625 else "hbm")
 
 
-def dw_workload(eden, synth, n=32, cold=False, c=144, hw=56, stride=2, k=3):
+def dw_workload(eden, synth, n=32, cold=False, c=144, hw=56, stride=2, k=3, dil=1):
     """depthwise k x k convolution, ReLU6, channels-last: BASELINE configs[2]'s stride-2 3x3 layer by default"""
-    pad = k // 2
-    ho = (hw + 2 * pad - k) // stride + 1
-    desc = eden.conv_desc(n, c, hw, hw, c, k, k, stride=(stride, stride), pad=(pad,) * 4, dm=1, layout=eden.NHWC)
+    pad = dil * (k - 1) // 2
+    ho = (hw + 2 * pad - dil * (k - 1) - 1) // stride + 1
+    desc = eden.conv_desc(n, c, hw, hw, c, k, k, stride=(stride, stride), pad=(pad,) * 4, dil=(dil, dil), dm=1, layout=eden.NHWC)
     x = synth.fill_u8((n, hw, hw, c), SEED + 48)
     w = synth.fill_u8((c, 1, k, k), SEED + 49)
     b = synth.fill_i32((c,), SEED + 50, -1000, 1000)
@@ -188,7 +188,7 @@ def dw_workload(eden, synth, n=32, cold=False, c=144, hw=56, stride=2, k=3):
     nbytes = n * c * hw * hw + c * k * k + c * 4 + n * c * ho * ho
     sets = set_count(nbytes, cold)
     bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * ho * ho * c)) for _ in range(sets)]
-    return dict(name="dw%dx%ds%d_n%d_c%d_%dx%d_nhwc" % (k, k, stride, n, c, hw, hw), launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
+    return dict(name="dw%dx%ds%d%s_n%d_c%d_%dx%d_nhwc" % (k, k, stride, "" if dil == 1 else "d%d" % dil, n, c, hw, hw), launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
                 keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * c * ho * ho * k * k, bytes=nbytes, bound="hbm")
 
 
@@ -557,9 +557,9 @@ def main():
     if args.only and args.only.startswith("conv:"):    # conv:N,CIN,COUT,HW,K,STRIDE = that convolution
         n, cin, cout, hw, k, stride = (int(v) for v in args.only[5:].split(","))
         families[args.only] = shaped(conv_workload, n=n, cin=cin, cout=cout, hw=hw, k=k, stride=stride)
-    if args.only and args.only.startswith("dw:"):      # dw:N,C,HW,STRIDE[,K] = that depthwise convolution
+    if args.only and args.only.startswith("dw:"):      # dw:N,C,HW,STRIDE[,K[,DILATION]] = that depthwise convolution
         v = [int(t) for t in args.only[3:].split(",")]
-        families[args.only] = shaped(dw_workload, n=v[0], c=v[1], hw=v[2], stride=v[3], k=v[4] if len(v) > 4 else 3)
+        families[args.only] = shaped(dw_workload, n=v[0], c=v[1], hw=v[2], stride=v[3], k=v[4] if len(v) > 4 else 3, dil=v[5] if len(v) > 5 else 1)
     if args.only and args.only.startswith(("block:", "twolaunch:")):
         # block:N,CIN,C,HW,STRIDE = that expansion + 3x3 depthwise pair as one launch; twolaunch: the same as two launches
         kind, _, spec = args.only.partition(":")

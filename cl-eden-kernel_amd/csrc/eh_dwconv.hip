@@ -72,54 +72,84 @@ __device__ __forceinline__ uint32_t requant4_channel_fast(int acc0, int acc1, in
 // multiples of 8): a shared input row is then fetched from HBM into one L2 instead of two or three.
 __device__ __forceinline__ uint32_t xcd_contiguous_block() { return (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3); }
 
-template <int KH, int KW>
-__global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, const long total) {
+// One output pixel's four adjacent channels per thread, any kernel size, stride and dilation (KH = 0: sizes from the
+// problem).  SMALL: both tensors below 2^31 bytes, so the index is decoded with 32-bit multiplications and the taps'
+// offsets are 32-bit (64-bit divisions and multiply-adds cost several times the rest of a small kernel's arithmetic).
+template <int KH, int KW, bool SMALL>
+__global__ __launch_bounds__(256) void dw_nhwc_vec4_kernel(const DwProblem p, const long total, const FastDiv div_cq, const FastDiv div_wo,
+                                                           const FastDiv div_ho) {
+    using Offset = std::conditional_t<SMALL, uint32_t, size_t>;
     const long idx = (long)xcd_contiguous_block() * 256 + threadIdx.x;
     if (idx >= total) return;
     const int cq_count = p.c >> 2;
-    const int cq = (int)(idx % cq_count);
-    const long pix = idx / cq_count;
-    const int ox = (int)(pix % p.wo);
-    const long t0 = pix / p.wo;
-    const int oy = (int)(t0 % p.ho), img = (int)(t0 / p.ho);
+    int cq, ox, oy, img;
+    Offset pix;
+    if constexpr (SMALL) {
+        const uint32_t i = (uint32_t)idx, px = fastdiv(i, div_cq), t0 = fastdiv(px, div_wo), im = fastdiv(t0, div_ho);
+        cq = (int)(i - px * (uint32_t)cq_count);
+        ox = (int)(px - t0 * (uint32_t)p.wo);
+        oy = (int)(t0 - im * (uint32_t)p.ho);
+        img = (int)im;
+        pix = px;
+    } else {
+        cq = (int)(idx % cq_count);
+        const long px = idx / cq_count;
+        ox = (int)(px % p.wo);
+        const long t0 = px / p.wo;
+        oy = (int)(t0 % p.ho), img = (int)(t0 / p.ho);
+        pix = (Offset)px;
+    }
     const int kh = KH ? KH : p.kh, kw = KW ? KW : p.kw;
     const int taps = kh * kw, pairs = (taps + 1) >> 1;
     const int iy0 = oy * p.stride_h - p.pad_t, ix0 = ox * p.stride_w - p.pad_l;
-    const uint8_t *src = p.in + (size_t)img * p.h * p.w_ * p.c + cq * 4;
+    const uint8_t *src = p.in + ((Offset)img * (Offset)(p.h * p.w_) * (Offset)p.c + (Offset)(cq * 4));
     const uint32_t fill = (uint32_t)p.zp_in * 0x01010101u;
 
-    auto tap = [&](int t) -> uint32_t {
-        if (t >= taps) return 0u;
-        const int ky = t / kw, kx = t - ky * kw;
+    auto tap_at = [&](int ky, int kx) -> uint32_t {
+        // loaded from a clamped address whatever the tap, so that the loads of several taps can be in flight together
         const int iy = iy0 + ky * p.dil_h, ix = ix0 + kx * p.dil_w;
-        if ((unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w_)
-            return *reinterpret_cast<const uint32_t *>(src + ((size_t)iy * p.w_ + ix) * p.c) ^ p.io_flip;
-        return fill;
+        const int iyc = iy < 0 ? 0 : (iy >= p.h ? p.h - 1 : iy), ixc = ix < 0 ? 0 : (ix >= p.w_ ? p.w_ - 1 : ix);
+        const uint32_t v = *reinterpret_cast<const uint32_t *>(src + ((Offset)iyc * (Offset)p.w_ + (Offset)ixc) * (Offset)p.c) ^ p.io_flip;
+        return (unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)p.w_ ? v : fill;
     };
-
     const int4 b4 = *reinterpret_cast<const int4 *>(p.bias_folded + cq * 4);
     int acc0 = b4.x, acc1 = b4.y, acc2 = b4.z, acc3 = b4.w;
-#pragma unroll
-    for (int pr = 0; pr < (KH ? (KH * KW + 1) / 2 : 1); ++pr) {
-        if constexpr (KH == 0) break;
-        const uint32_t lo = tap(2 * pr), hi = tap(2 * pr + 1);
-        const int4 w4 = *reinterpret_cast<const int4 *>(p.w_pair + (size_t)pr * p.cout + cq * 4);
+    auto accumulate = [&](int pr, uint32_t lo, uint32_t hi) {
+        const int4 w4 = *reinterpret_cast<const int4 *>(p.w_pair + ((Offset)pr * (Offset)p.cout + (Offset)(cq * 4)));
         acc0 = dot2(pair_bytes<0>(lo, hi), w4.x, acc0);
         acc1 = dot2(pair_bytes<1>(lo, hi), w4.y, acc1);
         acc2 = dot2(pair_bytes<2>(lo, hi), w4.z, acc2);
         acc3 = dot2(pair_bytes<3>(lo, hi), w4.w, acc3);
-    }
-    if constexpr (KH == 0) {
-        for (int pr = 0; pr < pairs; ++pr) {
-            const uint32_t lo = tap(2 * pr), hi = tap(2 * pr + 1);
-            const int4 w4 = *reinterpret_cast<const int4 *>(p.w_pair + (size_t)pr * p.cout + cq * 4);
-            acc0 = dot2(pair_bytes<0>(lo, hi), w4.x, acc0);
-            acc1 = dot2(pair_bytes<1>(lo, hi), w4.y, acc1);
-            acc2 = dot2(pair_bytes<2>(lo, hi), w4.z, acc2);
-            acc3 = dot2(pair_bytes<3>(lo, hi), w4.w, acc3);
+    };
+    if constexpr (KH != 0) {
+#pragma unroll
+        for (int pr = 0; pr < (KH * KW + 1) / 2; ++pr) {
+            constexpr int kw_c = KW ? KW : 1;
+            const int t = 2 * pr;
+            accumulate(pr, tap_at(t / kw_c, t % kw_c), t + 1 < KH * KW ? tap_at((t + 1) / kw_c, (t + 1) % kw_c) : 0u);
+        }
+    } else {
+        // taps in row-major order, two per step; (ky, kx) walk along without a division per tap
+        int ky = 0, kx = 0;
+        auto next = [&]() -> uint32_t {
+            const uint32_t v = ky < kh ? tap_at(ky, kx) : 0u;
+            if (++kx == kw) kx = 0, ++ky;
+            return v;
+        };
+        int pr = 0;
+        for (; pr + 4 <= pairs; pr += 4) {  // eight taps requested before the first is used
+            uint32_t v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = next();
+#pragma unroll
+            for (int i = 0; i < 4; ++i) accumulate(pr + i, v[2 * i], v[2 * i + 1]);
+        }
+        for (; pr < pairs; ++pr) {
+            const uint32_t lo = next(), hi = next();
+            accumulate(pr, lo, hi);
         }
     }
-    *reinterpret_cast<uint32_t *>(p.out + (size_t)pix * p.cout + cq * 4) =
+    *reinterpret_cast<uint32_t *>(p.out + (pix * (Offset)p.cout + (Offset)(cq * 4))) =
         requant4(acc0, acc1, acc2, acc3, p.rq, load_channel_quad<true>(p.rq, (uint32_t)cq * 4u)) ^ p.io_flip;
 }
 
@@ -227,12 +257,21 @@ __device__ __forceinline__ void column_words(uint32_t r0, uint32_t r1, uint32_t 
 // with the last two terms folded into the bias and sum a (nine taps, those outside the image reading za) taken from
 // per-column sums that neighbouring outputs share: one more dot product per column and channel.  p.zp_w is then the
 // zero point of the uint8 values being multiplied (int8 weights: + 128).
+// D: the dilation (stride 1 only).  2 or 4: the tile's outputs j and j + D share input columns, so it reads
+// TW + 2 D columns.  0: any dilation, read from the problem; no column is shared then and the tile reads three groups of
+// TW adjacent columns, one per kernel column (what remains shared is the index arithmetic, the weights and the
+// border tests).
 __device__ __forceinline__ int udot4(uint32_t a, uint32_t b, int acc) { return (int)__builtin_amdgcn_udot4(a, b, (uint32_t)acc, false); }
 
-template <int S, bool FLIP, int TW = 4, bool PC = false, bool FOLD = false>
+template <int S, bool FLIP, int TW = 4, bool PC = false, bool FOLD = false, int D = 1>
 __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProblem p, const uint32_t total, const int tiles_x,
                                                                     const FastDiv div_cq, const FastDiv div_tiles, const FastDiv div_ho) {
-    constexpr int IW = (TW - 1) * S + 3;
+    static_assert(D == 1 || S == 1, "dilated tiles are stride 1");
+    constexpr int IW = D ? (TW - 1) * S + 2 * D + 1 : 3 * TW;
+    const int dil = D ? D : p.dil_w;
+    // tile column x lies this many pixels right of the tile's first input column; output j's tap kx reads tile column col_of(j, kx)
+    auto x_offset = [&](int x) { return D ? x : (x / TW) * dil + (x % TW); };
+    auto col_of = [](int j, int kx) { return D ? j * S + kx * D : kx * TW + j; };
     const uint32_t idx = xcd_contiguous_block() * 256u + threadIdx.x;
     if (idx >= total) return;
     const uint32_t cq_count = (uint32_t)p.c >> 2;
@@ -254,7 +293,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
     // 32-bit ones at a quarter of it)
     const int row_pitch = p.w_ * p.c;
     uint32_t in[3][IW];
-    const bool inside = iy0 >= 0 && iy0 + 2 < p.h && ix0 >= 0 && ix0 + IW - 1 < p.w_;
+    const bool inside = iy0 >= 0 && iy0 + 2 * dil < p.h && ix0 >= 0 && ix0 + x_offset(IW - 1) < p.w_;
     if (__builtin_amdgcn_ballot_w64(!inside) == 0) {
         // every window of the wave lies inside the image (most waves): no clamps, no selects, offsets that differ
         // between the loads by wave-uniform amounts; a wave with one window on the border takes the general path whole
@@ -263,7 +302,7 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
         for (int ky = 0; ky < 3; ++ky)
 #pragma unroll
             for (int x = 0; x < IW; ++x) {
-                const uint32_t v = *reinterpret_cast<const uint32_t *>(src + (uint32_t)(ky * row_pitch + x * p.c));
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(src + (uint32_t)(ky * dil * row_pitch + x_offset(x) * p.c));
                 in[ky][x] = flip_loaded ? v ^ 0x80808080u : v;
             }
     } else {
@@ -271,14 +310,14 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
         bool col_ok[IW];
 #pragma unroll
         for (int x = 0; x < IW; ++x) {
-            const int ix = ix0 + x;
+            const int ix = ix0 + x_offset(x);
             col_ok[x] = (unsigned)ix < (unsigned)p.w_;
             const int ixc = ix < 0 ? 0 : (ix >= p.w_ ? p.w_ - 1 : ix);
             col_off[x] = base + (uint32_t)__mul24(ixc, p.c);
         }
 #pragma unroll
         for (int ky = 0; ky < 3; ++ky) {
-            const int iy = iy0 + ky;
+            const int iy = iy0 + ky * dil;
             const bool row_ok = (unsigned)iy < (unsigned)p.h;
             const int iyc = iy < 0 ? 0 : (iy >= p.h ? p.h - 1 : iy);
             const uint32_t row_off = (uint32_t)__mul24(iyc, row_pitch);
@@ -312,23 +351,23 @@ __global__ __launch_bounds__(256) void dw3x3_nhwc_tile4_dot4_kernel(const DwProb
 #pragma unroll
         for (int kx = 0; kx < 3; ++kx) {
             if constexpr (FOLD) {
-                acc0 = udot4(col[j * S + kx][0], (uint32_t)wk[kx].x, acc0);
-                acc1 = udot4(col[j * S + kx][1], (uint32_t)wk[kx].y, acc1);
-                acc2 = udot4(col[j * S + kx][2], (uint32_t)wk[kx].z, acc2);
-                acc3 = udot4(col[j * S + kx][3], (uint32_t)wk[kx].w, acc3);
+                acc0 = udot4(col[col_of(j, kx)][0], (uint32_t)wk[kx].x, acc0);
+                acc1 = udot4(col[col_of(j, kx)][1], (uint32_t)wk[kx].y, acc1);
+                acc2 = udot4(col[col_of(j, kx)][2], (uint32_t)wk[kx].z, acc2);
+                acc3 = udot4(col[col_of(j, kx)][3], (uint32_t)wk[kx].w, acc3);
             } else {
-                acc0 = __builtin_amdgcn_sdot4((int)col[j * S + kx][0], wk[kx].x, acc0, false);
-                acc1 = __builtin_amdgcn_sdot4((int)col[j * S + kx][1], wk[kx].y, acc1, false);
-                acc2 = __builtin_amdgcn_sdot4((int)col[j * S + kx][2], wk[kx].z, acc2, false);
-                acc3 = __builtin_amdgcn_sdot4((int)col[j * S + kx][3], wk[kx].w, acc3, false);
+                acc0 = __builtin_amdgcn_sdot4((int)col[col_of(j, kx)][0], wk[kx].x, acc0, false);
+                acc1 = __builtin_amdgcn_sdot4((int)col[col_of(j, kx)][1], wk[kx].y, acc1, false);
+                acc2 = __builtin_amdgcn_sdot4((int)col[col_of(j, kx)][2], wk[kx].z, acc2, false);
+                acc3 = __builtin_amdgcn_sdot4((int)col[col_of(j, kx)][3], wk[kx].w, acc3, false);
             }
         }
         if constexpr (FOLD) {
             // (nine bytes times a zero point of at most 383: a 24-bit multiply-add)
-            acc0 += __mul24(-p.zp_w, cs[j * S][0] + cs[j * S + 1][0] + cs[j * S + 2][0]);
-            acc1 += __mul24(-p.zp_w, cs[j * S][1] + cs[j * S + 1][1] + cs[j * S + 2][1]);
-            acc2 += __mul24(-p.zp_w, cs[j * S][2] + cs[j * S + 1][2] + cs[j * S + 2][2]);
-            acc3 += __mul24(-p.zp_w, cs[j * S][3] + cs[j * S + 1][3] + cs[j * S + 2][3]);
+            acc0 += __mul24(-p.zp_w, cs[col_of(j, 0)][0] + cs[col_of(j, 1)][0] + cs[col_of(j, 2)][0]);
+            acc1 += __mul24(-p.zp_w, cs[col_of(j, 0)][1] + cs[col_of(j, 1)][1] + cs[col_of(j, 2)][1]);
+            acc2 += __mul24(-p.zp_w, cs[col_of(j, 0)][2] + cs[col_of(j, 1)][2] + cs[col_of(j, 2)][2]);
+            acc3 += __mul24(-p.zp_w, cs[col_of(j, 0)][3] + cs[col_of(j, 1)][3] + cs[col_of(j, 2)][3]);
         }
         uint32_t o = PC ? requant4_channel_fast(acc0, acc1, acc2, acc3, rq, quad) : requant4<false>(acc0, acc1, acc2, acc3, rq, quad);
         if (FLIP) o ^= 0x80808080u;
@@ -474,7 +513,17 @@ __global__ __launch_bounds__(256) void dw_scalar_kernel(const DwProblem p, const
     const long idx = (long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     int oc, ox, oy, img;
-    if (NHWC) {
+    if (total < (1l << 31)) {  // (uniform) 32-bit divisions: a fraction of the 64-bit ones' instructions
+        const uint32_t i = (uint32_t)idx, d0 = (uint32_t)(NHWC ? p.cout : p.wo), d2 = (uint32_t)(NHWC ? p.ho : p.cout);
+        const uint32_t d1 = (uint32_t)(NHWC ? p.wo : p.ho);
+        const uint32_t r0 = i / d0, r1 = r0 / d1, r2 = r1 / d2;
+        const int f0 = (int)(i - r0 * d0), f1 = (int)(r0 - r1 * d1), f2 = (int)(r1 - r2 * d2);
+        img = (int)r2;
+        if (NHWC)
+            oc = f0, ox = f1, oy = f2;
+        else
+            ox = f0, oy = f1, oc = f2;
+    } else if (NHWC) {
         oc = (int)(idx % p.cout);
         long r = idx / p.cout;
         ox = (int)(r % p.wo);
@@ -627,6 +676,8 @@ int launch_dw_pack_trip(const uint8_t *w, const int32_t *bias, int32_t *w_trip, 
     return EH_OK;
 }
 
+static long pairs_of(const DwProblem &p) { return ((long)p.kh * p.kw + 1) / 2; }
+
 int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
     DwProblem p = caller_p;
     const bool pc_two_step = p.rq.pc_multiplier != nullptr && !p.rq.fast;
@@ -636,7 +687,10 @@ int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
     if (outs <= 0) return EH_OK;
     const bool vec = p.dm == 1 && (p.c & 3) == 0 && (reinterpret_cast<uintptr_t>(p.in) & 3) == 0 &&
                      (reinterpret_cast<uintptr_t>(p.out) & 3) == 0;
-    const bool tile3x3 = vec && p.kh == 3 && p.kw == 3 && p.dil_h == 1 && p.dil_w == 1 && p.stride_h == p.stride_w &&
+    // (the dot product kernels index rows and pixels with 24-bit multiplies)
+    const bool dot4_form = (p.w_trip || p.w_fold) && (p.rq.pc_multiplier == nullptr || p.rq.fast) && (long)p.w_ * p.c < (1l << 23) && p.h < (1 << 23);
+    const bool dilated = p.dil_h > 1 && p.dil_h == p.dil_w && p.stride_h == 1 && dot4_form && (long)p.dil_h * p.w_ * p.c < (1l << 22);
+    const bool tile3x3 = vec && p.kh == 3 && p.kw == 3 && ((p.dil_h == 1 && p.dil_w == 1) || dilated) && p.stride_h == p.stride_w &&
                          (p.stride_h == 1 || p.stride_h == 2) && (size_t)p.n * p.h * p.w_ * p.c < (1ull << 31) &&
                          (size_t)p.n * p.ho * p.wo * p.cout < (1ull << 31);
     const bool tile_kxk = vec && p.w_foldk != nullptr && p.kh == p.kw && (p.kh == 5 || p.kh == 7) && p.dil_h == 1 && p.dil_w == 1 && p.dm == 1 &&
@@ -689,11 +743,23 @@ int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
                       : (flip ? dw3x3_nhwc_tile4_dot4_kernel<S, true, TW, false> : dw3x3_nhwc_tile4_dot4_kernel<S, false, TW, false>);
         };
         using tw4 = std::integral_constant<int, 4>;
-        // (the dot product kernels index rows and pixels with 24-bit multiplies)
-        const bool dot4 = (p.w_trip || p.w_fold) && (!pc || p.rq.fast) && (long)p.w_ * p.c < (1l << 23) && p.h < (1 << 23);
-        if (dot4)
+        const bool dot4 = dot4_form;
+        if (p.dil_h > 1) {
+            // dilated, stride 1: the tiles that share columns for dilations 2 and 4, the three-group tile for the rest
+            auto pick_dilated = [&](auto d_tag) {
+                constexpr int D = decltype(d_tag)::value;
+                if (fold)
+                    return pc ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true, 4, true, true, D> : dw3x3_nhwc_tile4_dot4_kernel<1, false, 4, true, true, D>)
+                              : (flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true, 4, false, true, D> : dw3x3_nhwc_tile4_dot4_kernel<1, false, 4, false, true, D>);
+                return pc ? (flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true, 4, true, false, D> : dw3x3_nhwc_tile4_dot4_kernel<1, false, 4, true, false, D>)
+                          : (flip ? dw3x3_nhwc_tile4_dot4_kernel<1, true, 4, false, false, D> : dw3x3_nhwc_tile4_dot4_kernel<1, false, 4, false, false, D>);
+            };
+            kernel = p.dil_h == 2   ? pick_dilated(std::integral_constant<int, 2>{})
+                     : p.dil_h == 4 ? pick_dilated(std::integral_constant<int, 4>{})
+                                    : pick_dilated(std::integral_constant<int, 0>{});
+        } else if (dot4)
             kernel = p.stride_h == 1 ? pick_dot4(std::integral_constant<int, 1>{}, tw4{}) : pick_dot4(std::integral_constant<int, 2>{}, tw4{});
-        if (dot4 && p.stride_h == 1 && (p.wo & 7) == 0 && total >= (1l << 20)) {
+        if (dot4 && p.dil_h == 1 && p.stride_h == 1 && (p.wo & 7) == 0 && total >= (1l << 20)) {
             // large stride-1 layers with rows of whole eight-pixel tiles: eight outputs per thread
             const int tiles8 = p.wo / 8;
             const long total8 = (long)p.n * p.ho * tiles8 * (p.c >> 2);
@@ -709,10 +775,12 @@ int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
         const long total = outs / 4;
         const long blocks = (total + 255) / 256;
         EH_REQUIRE(blocks < (1l << 31), "depthwise: grid too large");
-        if (p.kh == 3 && p.kw == 3)
-            hipLaunchKernelGGL((dw_nhwc_vec4_kernel<3, 3>), dim3((unsigned)((blocks + 7) / 8 * 8)), dim3(256), 0, stream, p, total);
-        else
-            hipLaunchKernelGGL((dw_nhwc_vec4_kernel<0, 0>), dim3((unsigned)((blocks + 7) / 8 * 8)), dim3(256), 0, stream, p, total);
+        const bool small = (size_t)p.n * p.h * p.w_ * p.c < (1ull << 31) && outs < (1l << 31) && (size_t)pairs_of(p) * p.cout < (1ull << 30);
+        const FastDiv d_cq = make_fastdiv((uint32_t)(p.c >> 2)), d_wo = make_fastdiv((uint32_t)p.wo), d_ho = make_fastdiv((uint32_t)p.ho);
+        const bool k3 = p.kh == 3 && p.kw == 3;
+        auto kernel = k3 ? (small ? dw_nhwc_vec4_kernel<3, 3, true> : dw_nhwc_vec4_kernel<3, 3, false>)
+                         : (small ? dw_nhwc_vec4_kernel<0, 0, true> : dw_nhwc_vec4_kernel<0, 0, false>);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)((blocks + 7) / 8 * 8)), dim3(256), 0, stream, p, total, d_cq, d_wo, d_ho);
     } else {
         const long blocks = (outs + 255) / 256;
         EH_REQUIRE(blocks < (1l << 31), "depthwise: grid too large");

@@ -459,6 +459,16 @@ DW_CASES = [
     dict(n=1, c=12, h=4, w=3, cout=12, kh=5, kw=5, pad=(2, 2, 2, 2)),
     dict(n=3, c=144, h=28, w=28, cout=144, kh=5, kw=5, pad=(2, 2, 2, 2)),
     dict(n=1, c=4, h=9, w=9, cout=4, kh=7, kw=7),
+    # dilated 3x3 tiles at stride 1: the column-sharing tiles of dilations 2 and 4, the three-group tile of any other
+    # dilation; ragged widths, every border, windows wider than the image, uneven padding
+    dict(n=2, c=24, h=19, w=21, cout=24, kh=3, kw=3, pad=(2, 2, 2, 2), dil=(2, 2)),
+    dict(n=1, c=8, h=17, w=18, cout=8, kh=3, kw=3, pad=(4, 4, 4, 4), dil=(4, 4)),
+    dict(n=2, c=16, h=15, w=14, cout=16, kh=3, kw=3, pad=(3, 3, 3, 3), dil=(3, 3)),
+    dict(n=1, c=32, h=33, w=33, cout=32, kh=3, kw=3, pad=(6, 6, 6, 6), dil=(6, 6)),
+    dict(n=1, c=8, h=5, w=6, cout=8, kh=3, kw=3, pad=(4, 4, 4, 4), dil=(4, 4)),
+    dict(n=1, c=12, h=9, w=30, cout=12, kh=3, kw=3, pad=(0, 3, 1, 0), dil=(2, 2)),
+    dict(n=1, c=4, h=40, w=41, cout=4, kh=3, kw=3, pad=(12, 12, 12, 12), dil=(12, 12)),
+    dict(n=3, c=384, h=33, w=33, cout=384, kh=3, kw=3, pad=(2, 2, 2, 2), dil=(2, 2)),
 ]
 
 
@@ -478,7 +488,7 @@ def test_depthwise_matches_oracle(case, layout):
     assert want.std() > 10
 
 
-DW_INT8_RANGE_CASES = [c for c in DW_CASES if c["kh"] == 3 and c.get("dm", 1) == 1 and c.get("dil", (1, 1)) == (1, 1)] + [
+DW_INT8_RANGE_CASES = [c for c in DW_CASES if c["kh"] == 3 and c["kw"] == 3 and c.get("dm", 1) == 1] + [
     # large stride-1 layers whose rows are whole eight-pixel tiles: eight outputs per thread
     dict(n=44, c=32, h=112, w=112, cout=32, kh=3, kw=3, pad=(1, 1, 1, 1)),
     dict(n=70, c=16, h=37, w=112, cout=16, kh=3, kw=3, pad=(0, 1, 2, 0)),
@@ -501,7 +511,7 @@ def test_depthwise_3x3_weights_within_int8_of_their_zero_point(case):
         _, acc = O.dwconv2d(x, w, b, s, O.raw_quant(zp_in=37, zp_w=z), want_acc=True)
         quants.append(centred_quant(acc, 37, z, act_min=5, act_max=250))
     ho, wo = O.conv_out_hw(s)
-    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, 3, 3, (s.stride_h, s.stride_w), (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (1, 1), 1, 1,
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, 3, 3, (s.stride_h, s.stride_w), (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), 1, 1,
                           eden.NHWC, eden.W_OIHW)
     d_x = eden.DeviceBuffer(host=np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
     d_w, d_b, d_o = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b), eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
