@@ -18,6 +18,7 @@ NCHW, NHWC = 0, 1
 W_OIHW, W_OHWI, W_IOHW = 0, 1, 2
 W_SIGNED = 0x100  # or-ed into a convolution's weight layout: int8 weight bytes
 IO_SIGNED = 0x200  # or-ed into a convolution's tensor layout: int8 input and output (zero points and range in [-128, 127])
+EXACT_CHANNELS = 0x400  # or-ed into a convolution's tensor layout or a fully connected plan's flags: no channel-padded staging copy
 
 
 class EdenHipError(RuntimeError):
@@ -508,7 +509,7 @@ class FcPlan(_Plan):
     _kind = "fc"
 
     def __init__(self, m, k, n, d_w, d_b, q, stream=None, flags=0):
-        """flags: any of W_SIGNED | IO_SIGNED"""
+        """flags: any of W_SIGNED | IO_SIGNED | EXACT_CHANNELS"""
         super().__init__()
         self.m, self.k, self.n = m, k, n
         if flags:

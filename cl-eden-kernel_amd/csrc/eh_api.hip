@@ -122,6 +122,7 @@ struct GemmPart {
     KUnit *ktab = nullptr;
     int32_t *tap_off = nullptr;
     int32_t n = 0, n_pad = 0, k = 0, k_pad = 0, vec = 1, taps = 0, cin = 0;
+    int32_t cin_real = 0;     // channels per tap in the source weights when `cin` includes padding channels; 0 = cin
     GemmConfig cfg;
     int64_t so = 0, sc = 0;   // source weight strides (out channel, in channel)
     int64_t w_base = 0;       // element offset of this part in the source weights
@@ -263,6 +264,7 @@ int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t str
     pp.k = g.k;
     pp.k_pad = g.k_pad;
     pp.row_bytes = g.cfg.id == GEMM_ROWS ? g.proto.rows_kw * g.cin : 0;
+    pp.cin_real = g.cin_real;
     pp.so = g.so;
     pp.sc = g.sc;
     pp.tap_off = g.tap_off;
@@ -310,6 +312,14 @@ struct GemmOp {
     int32_t layout = EH_NHWC;
     int32_t in_n = 0, in_c = 0, in_hw = 0, out_hw = 0;
     size_t in_bytes = 0;
+    // Channel padding.  Channel counts (per group) that are no multiple of 16 would leave the byte-gathering kernel as
+    // the only choice; instead the kernels then read a copy of the input in which every group's `pad_cg` channels are
+    // followed by bytes holding the input zero point up to `pad_cg_to` channels, a multiple of 16.  Such a byte
+    // contributes (zp_in - zp_in) * (w - zp_w) = 0 whatever weight it meets (the packed weights hold 0 there), so the
+    // padded problem is the caller's problem exactly.
+    int32_t pad_groups = 0, pad_cg = 0, pad_cg_to = 0;
+    bool exact_channels = false;  // the caller asked for no padded copy
+    uint8_t *stage_pad = nullptr;
     // int8 weights (value = byte as signed; zp_w is then an int8 zero point) and one multiplier / shift per
     // output channel instead of the requant's single pair
     bool has_bias = true;
@@ -343,6 +353,7 @@ struct GemmOp {
         dev_free(bias_copy);
         dev_free(stage_in);
         dev_free(stage_out);
+        dev_free(stage_pad);
         dev_free(fillbuf);
         dev_free(pc_multiplier);
         dev_free(pc_shift);
@@ -392,6 +403,18 @@ struct GemmOp {
     // bytes of the two channels-last staging images of a planar plan (each with the slack the kernels' wide loads need)
     size_t stage_in_bytes() const { return ((size_t)in_n * in_c * in_hw + 256 + 255) / 256 * 256; }
     size_t stage_out_bytes() const { return ((size_t)in_n * cout * out_hw + 256 + 255) / 256 * 256; }
+    size_t stage_pad_bytes() const { return ((size_t)in_n * in_hw * pad_groups * pad_cg_to + 256 + 255) / 256 * 256; }
+    // what a run that brings its own staging memory needs: the planar plan's two images, then the padded input
+    size_t staging_bytes() const { return (layout == EH_NCHW ? stage_in_bytes() + stage_out_bytes() : 0) + (pad_cg_to ? stage_pad_bytes() : 0); }
+    int alloc_staging() {
+        int rc = EH_OK;
+        if (layout == EH_NCHW) {
+            if ((rc = dev_alloc(&stage_in, stage_in_bytes()))) return rc;
+            if ((rc = dev_alloc(&stage_out, stage_out_bytes()))) return rc;
+        }
+        if (pad_cg_to) rc = dev_alloc(&stage_pad, stage_pad_bytes());
+        return rc;
+    }
     static constexpr int kInlineParts = 8;  // a run over at most this many parts allocates no host memory
 
     // One part's kernel argument for channels-last tensors `in` / `out`, with the quantization parameters refold() left in `q`
@@ -420,7 +443,7 @@ struct GemmOp {
         return p;
     }
 
-    // staging != null: a planar plan uses [staging, staging + stage_in_bytes() + stage_out_bytes()) instead of its own images
+    // staging != null: the plan uses [staging, staging + staging_bytes()) instead of its own images
     int run(const void *input, void *output, const eh_requant *nq, hipStream_t stream, const uint8_t *residual = nullptr,
             const AddDev *radd = nullptr, bool *fused = nullptr, uint8_t *staging = nullptr) {
         EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
@@ -436,6 +459,14 @@ struct GemmOp {
             if ((rc = launch_nchw2nhwc(in, st_in, in_n, in_c, in_hw, stream))) return rc;
             in = st_in;
             out = st_out;
+        }
+        if (pad_cg_to) {
+            uint8_t *const st_pad = staging ? staging + (layout == EH_NCHW ? stage_in_bytes() + stage_out_bytes() : 0) : stage_pad;
+            // (q holds the uint8-equivalent input zero point after refold(); int8 tensors store it minus 128)
+            if ((rc = launch_pad_channels(in, st_pad, (int64_t)in_n * in_hw, pad_groups, pad_cg, pad_cg_to,
+                                          (uint32_t)(q.zp_in & 0xFF) ^ (io_signed ? 0x80u : 0u), stream)))
+                return rc;
+            in = st_pad;
         }
         GemmProblem inline_problems[kInlineParts];
         std::vector<GemmProblem> many;
@@ -833,11 +864,30 @@ int eh_transpose_u8_nhwc2nchw(const void *src, void *dst, int32_t n, int32_t c, 
     return launch_nhwc2nchw(static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), n, c, h * w, as_stream(stream));
 }
 
+// Whether a plan just built on the caller's channel count should be built again on padded channels: some part fell to
+// the byte-gathering kernel.  Sets the padding up and drops the parts if so.
+static bool wants_channel_padding(GemmOp &op, int groups, int channels_per_group) {
+    if (op.exact_channels || op.pad_cg_to != 0 || (channels_per_group & 15) == 0) return false;
+    bool staged = false;
+    for (const GemmPart &g : op.parts) staged = staged || (g.cfg.id == GEMM_STAGED && g.k > 0);
+    if (!staged) return false;
+    const int64_t padded = (int64_t)op.in_n * op.in_hw * groups * round_up(channels_per_group, 16);
+    if (padded >= (1ll << 31)) return false;
+    for (auto &g : op.parts) g.release();
+    op.parts.clear();
+    dev_free(op.bias_copy);
+    op.pad_groups = groups;
+    op.pad_cg = channels_per_group;
+    op.pad_cg_to = round_up(channels_per_group, 16);
+    return true;
+}
+
 // ------------------------------------------------------------ convolution
 
 static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t stream) {
     GemmOp &op = pl->op;
-    const int G = d->groups, cig = d->c / G, cog = d->cout / G;
+    const int G = d->groups, cog = d->cout / G;
+    int cig = d->c / G;
     const int ho = eh_conv_out_dim(d->h, d->pad_t, d->pad_b, d->kh, d->dil_h, d->stride_h);
     const int wo = eh_conv_out_dim(d->w, d->pad_l, d->pad_r, d->kw, d->dil_w, d->stride_w);
     EH_REQUIRE(ho > 0 && wo > 0, "convolution output is empty (%d x %d)", ho, wo);
@@ -851,30 +901,33 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
     op.out_hw = ho * wo;
     int rc;
     if ((rc = dev_alloc(&op.bias_copy, (size_t)d->cout))) return rc;
-    if (d->layout == EH_NCHW) {
-        if ((rc = dev_alloc(&op.stage_in, op.stage_in_bytes()))) return rc;
-        if ((rc = dev_alloc(&op.stage_out, op.stage_out_bytes()))) return rc;
-    }
     const int taps = d->kh * d->kw;
+    // built on the caller's channel count first; when that leaves a group to the byte-gathering kernel, built again on
+    // channels padded to a multiple of 16
+    const int cig_real = cig;
+    const bool padded = op.pad_cg_to != 0;
+    if (padded) cig = op.pad_cg_to;
+    const int pixel_c = padded ? G * cig : d->c;
     op.parts.resize(G);
     for (int g = 0; g < G; ++g) {
         GemmPart &part = op.parts[g];
         part.n = cog;
         part.cin = cig;
+        part.cin_real = padded ? cig_real : 0;
         part.taps = taps;
         part.k = taps * cig;
-        part.vec = pick_vec(cig, d->c);
+        part.vec = pick_vec(cig, pixel_c);
         part.bias_base = g * cog;
         if (d->weight_layout == EH_W_OIHW) {
-            part.so = (int64_t)cig * taps;
+            part.so = (int64_t)cig_real * taps;
             part.sc = taps;
         } else {
-            part.so = (int64_t)taps * cig;
+            part.so = (int64_t)taps * cig_real;
             part.sc = 1;
         }
         part.w_base = (int64_t)g * cog * part.so;
         std::vector<int32_t> tap_off(taps);
-        for (int t = 0; t < taps; ++t) tap_off[t] = d->weight_layout == EH_W_OIHW ? t : t * cig;
+        for (int t = 0; t < taps; ++t) tap_off[t] = d->weight_layout == EH_W_OIHW ? t : t * cig_real;
         std::vector<KUnit> units;
         for (int k = 0; k < part.k; k += part.vec) {
             const int t = k / cig, c = k - t * cig;
@@ -882,14 +935,14 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
             KUnit u;
             u.dy = (int16_t)(ky * d->dil_h);
             u.dx = (int16_t)(kx * d->dil_w);
-            u.offset = (u.dy * d->w + u.dx) * d->c + g * cig + c;
+            u.offset = (u.dy * d->w + u.dx) * pixel_c + g * cig + c;
             units.push_back(u);
         }
         GemmProblem &p = part.proto;
         p.m = d->n * ho * wo;
         p.h = d->h;
         p.w = d->w;
-        p.cin = d->c;
+        p.cin = pixel_c;
         p.ho = ho;
         p.wo = wo;
         p.stride_h = d->stride_h;
@@ -905,7 +958,8 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
         p.ldc = d->cout;
         if ((rc = finish_part(part, units, tap_off, stream, std::min(G, (int)GemmBatch::MAX)))) return rc;
     }
-    return EH_OK;
+    if (wants_channel_padding(op, G, cig_real)) return conv_plan_build(pl, d, stream);
+    return op.alloc_staging();
 }
 
 // `desc` with the two flag bits taken out, checked
@@ -913,7 +967,7 @@ static int conv_desc_checked(const eh_conv_desc *desc, eh_conv_desc *plain) {
     EH_REQUIRE(desc != nullptr, "descriptor is null");
     *plain = *desc;
     plain->weight_layout &= ~EH_W_SIGNED;
-    plain->layout &= ~EH_IO_SIGNED;
+    plain->layout &= ~(EH_IO_SIGNED | EH_EXACT_CHANNELS);
     desc = plain;
     int rc = check_desc_common(desc);
     if (rc) return rc;
@@ -939,6 +993,7 @@ int eh_conv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_t 
     if (rc) return rc;
     if (plain.n == 0) return 0;
     eh_conv_plan pl;
+    pl.op.exact_channels = (desc->layout & EH_EXACT_CHANNELS) != 0;
     g_dry_run = true;
     rc = conv_plan_build(&pl, &plain, nullptr);
     g_dry_run = false;
@@ -951,6 +1006,7 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
     *plan = nullptr;
     EH_REQUIRE(desc != nullptr, "descriptor is null");
     const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
+    const bool exact_channels = (desc->layout & EH_EXACT_CHANNELS) != 0;
     eh_conv_desc plain;
     int rc = conv_desc_checked(desc, &plain);
     if (rc) return rc;
@@ -961,6 +1017,7 @@ int eh_conv2d_u8_plan(eh_conv_plan **plan, const eh_conv_desc *desc, const void 
     pl->d = *desc;
     pl->op.w_signed = w_signed;
     pl->op.io_signed = io_signed;
+    pl->op.exact_channels = exact_channels;
     if (desc->n > 0) {
         rc = conv_plan_build(pl, desc, as_stream(stream));
         if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
@@ -1004,10 +1061,9 @@ int eh_conv2d_u8_run_static(eh_conv_plan *plan, const void *input, void *output,
     EH_REQUIRE(op.parts.size() <= (size_t)GemmOp::kInlineParts, "run_static: %zu convolution groups, at most %d are supported",
                op.parts.size(), GemmOp::kInlineParts);
     uint8_t *staging = nullptr;
-    if (op.layout == EH_NCHW) {
-        const size_t need = op.stage_in_bytes() + op.stage_out_bytes();
+    if (const size_t need = op.staging_bytes(); need != 0) {
         EH_REQUIRE(need <= (size_t)EH_STATIC_SCRATCH_BYTES,
-                   "run_static: the channels-last staging of this plan takes %zu bytes, the static scratch holds %zu", need,
+                   "run_static: the staging images of this plan (channels-last, channel-padded) take %zu bytes, the static scratch holds %zu", need,
                    (size_t)EH_STATIC_SCRATCH_BYTES);
         int rc = static_scratch(&staging);
         if (rc) return rc;
@@ -1059,7 +1115,7 @@ int eh_fc_q8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, int32_t fl
     *plan = nullptr;
     EH_REQUIRE(m >= 0 && k > 0 && n > 0, "bad extents m=%d k=%d n=%d", m, k, n);
     EH_REQUIRE((int64_t)m * k < (1ll << 31), "input larger than 2 GiB is not supported");
-    EH_REQUIRE((flags & ~(EH_W_SIGNED | EH_IO_SIGNED)) == 0, "unknown flags 0x%x", flags);
+    EH_REQUIRE((flags & ~(EH_W_SIGNED | EH_IO_SIGNED | EH_EXACT_CHANNELS)) == 0, "unknown flags 0x%x", flags);
     const bool w_signed = (flags & EH_W_SIGNED) != 0, io_signed = (flags & EH_IO_SIGNED) != 0;
     int rc = check_requant(q, w_signed, io_signed);
     if (rc) return rc;
@@ -1071,19 +1127,32 @@ int eh_fc_q8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, int32_t fl
     GemmOp &op = pl->op;
     op.w_signed = w_signed;
     op.io_signed = io_signed;
+    op.exact_channels = (flags & EH_EXACT_CHANNELS) != 0;
     op.cout = n;
     op.layout = EH_NHWC;
+    op.in_n = m;
+    op.in_c = k;
+    op.in_hw = 1;
+    op.out_hw = 1;
     hipStream_t s = as_stream(stream);
-    rc = dev_alloc(&op.bias_copy, (size_t)n);
-    if (!rc) {
+    // (a second pass on a row length padded to a multiple of 16 when the first leaves the byte-gathering kernel)
+    const int k_real = k;
+    for (int pass = 0; pass < 2 && !rc; ++pass) {
+        if (pass == 1) {
+            if (!wants_channel_padding(op, 1, k_real)) break;
+            k = op.pad_cg_to;
+        }
+        rc = dev_alloc(&op.bias_copy, (size_t)n);
+        if (rc) break;
         op.parts.resize(1);
         GemmPart &part = op.parts[0];
         part.n = n;
         part.cin = k;
+        part.cin_real = pass == 1 ? k_real : 0;
         part.taps = 1;
         part.k = k;
         part.vec = pick_vec(k, k);
-        part.so = k;
+        part.so = k_real;
         part.sc = 1;
         std::vector<int32_t> tap_off(1, 0);
         std::vector<KUnit> units;
@@ -1114,6 +1183,7 @@ int eh_fc_q8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, int32_t fl
         p.ldc = n;
         rc = finish_part(part, units, tap_off, s);
     }
+    if (!rc) rc = op.alloc_staging();
     if (!rc) rc = op.set_weights(weight, bias, s);
     if (!rc) rc = op.refold(*q, s);
     if (rc) {
@@ -1157,7 +1227,8 @@ int eh_fc_u8_destroy(eh_fc_plan *plan) {
 
 static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStream_t stream) {
     GemmOp &op = pl->op;
-    const int G = d->groups, cig = d->c / G, cog = d->cout / G;
+    const int G = d->groups, cog = d->cout / G;
+    int cig = d->c / G;
     const int oh = eh_deconv_out_dim(d->h, d->pad_t, d->pad_b, d->kh, d->stride_h);
     const int ow = eh_deconv_out_dim(d->w, d->pad_l, d->pad_r, d->kw, d->stride_w);
     EH_REQUIRE(oh > 0 && ow > 0, "deconvolution output is empty (%d x %d)", oh, ow);
@@ -1170,10 +1241,11 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
     op.out_hw = oh * ow;
     int rc;
     if ((rc = dev_alloc(&op.bias_copy, (size_t)d->cout))) return rc;
-    if (d->layout == EH_NCHW) {
-        if ((rc = dev_alloc(&op.stage_in, op.stage_in_bytes()))) return rc;
-        if ((rc = dev_alloc(&op.stage_out, op.stage_out_bytes()))) return rc;
-    }
+    // (built a second time on channels padded to a multiple of 16 when a phase is left to the byte-gathering kernel)
+    const int cig_real = cig;
+    const bool padded = op.pad_cg_to != 0;
+    if (padded) cig = op.pad_cg_to;
+    const int pixel_c = padded ? G * cig : d->c;
     const int sh = d->stride_h, sw = d->stride_w;
     for (int g = 0; g < G; ++g)
         for (int py = 0; py < sh; ++py)
@@ -1188,15 +1260,16 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                 GemmPart &part = op.parts.back();
                 part.n = cog;
                 part.cin = cig;
+                part.cin_real = padded ? cig_real : 0;
                 part.taps = nty * ntx;
                 part.k = part.taps * cig;
-                part.vec = pick_vec(cig, d->c);
+                part.vec = pick_vec(cig, pixel_c);
                 part.bias_base = g * cog;
                 std::vector<int32_t> tap_off(part.taps > 0 ? part.taps : 0);
                 if (d->weight_layout == EH_W_IOHW) {
                     part.so = (int64_t)d->kh * d->kw;
                     part.sc = (int64_t)cog * d->kh * d->kw;
-                    part.w_base = (int64_t)g * cig * cog * d->kh * d->kw;
+                    part.w_base = (int64_t)g * cig_real * cog * d->kh * d->kw;
                 } else {  // OHWI, groups == 1
                     part.so = (int64_t)d->kh * d->kw * d->c;
                     part.sc = 1;
@@ -1214,14 +1287,14 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                     KUnit u;
                     u.dy = (int16_t)(by - ty);
                     u.dx = (int16_t)(bx - tx);
-                    u.offset = (u.dy * d->w + u.dx) * d->c + g * cig + c;
+                    u.offset = (u.dy * d->w + u.dx) * pixel_c + g * cig + c;
                     units.push_back(u);
                 }
                 GemmProblem &p = part.proto;
                 p.m = d->n * ho_p * wo_p;
                 p.h = d->h;
                 p.w = d->w;
-                p.cin = d->c;
+                p.cin = pixel_c;
                 p.ho = ho_p;
                 p.wo = wo_p;
                 p.stride_h = 1;
@@ -1239,14 +1312,15 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                 const int siblings = (d->kh % sh == 0 && d->kw % sw == 0) ? std::min(G * sh * sw, (int)GemmBatch::MAX) : 1;
                 if ((rc = finish_part(part, units, tap_off, stream, siblings))) return rc;
             }
-    return EH_OK;
+    if (wants_channel_padding(op, G, cig_real)) return deconv_plan_build(pl, d, stream);
+    return op.alloc_staging();
 }
 
 static int deconv_desc_checked(const eh_conv_desc *desc, eh_conv_desc *plain) {
     EH_REQUIRE(desc != nullptr, "descriptor is null");
     *plain = *desc;
     plain->weight_layout &= ~EH_W_SIGNED;
-    plain->layout &= ~EH_IO_SIGNED;
+    plain->layout &= ~(EH_IO_SIGNED | EH_EXACT_CHANNELS);
     desc = plain;
     int rc = check_desc_common(desc, true);
     if (rc) return rc;
@@ -1265,6 +1339,7 @@ int eh_deconv2d_u8_kernels(const eh_conv_desc *desc, int32_t *kernel_ids, int32_
     if (rc) return rc;
     if (plain.n == 0) return 0;
     eh_deconv_plan pl;
+    pl.op.exact_channels = (desc->layout & EH_EXACT_CHANNELS) != 0;
     g_dry_run = true;
     rc = deconv_plan_build(&pl, &plain, nullptr);
     g_dry_run = false;
@@ -1277,6 +1352,7 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
     *plan = nullptr;
     EH_REQUIRE(desc != nullptr, "descriptor is null");
     const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
+    const bool exact_channels = (desc->layout & EH_EXACT_CHANNELS) != 0;
     eh_conv_desc plain;
     int rc = deconv_desc_checked(desc, &plain);
     if (rc) return rc;
@@ -1287,6 +1363,7 @@ int eh_deconv2d_u8_plan(eh_deconv_plan **plan, const eh_conv_desc *desc, const v
     pl->d = *desc;
     pl->op.w_signed = w_signed;
     pl->op.io_signed = io_signed;
+    pl->op.exact_channels = exact_channels;
     if (desc->n > 0) {
         rc = deconv_plan_build(pl, desc, as_stream(stream));
         if (!rc) rc = pl->op.set_weights(weight, bias, as_stream(stream));
@@ -1405,7 +1482,7 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
     eh_conv_desc plain = *desc;
     plain.weight_layout &= ~EH_W_SIGNED;
-    plain.layout &= ~EH_IO_SIGNED;
+    plain.layout &= ~(EH_IO_SIGNED | EH_EXACT_CHANNELS);  // (the second flag has no meaning for a depthwise plan)
     desc = &plain;
     int rc = check_desc_common(desc);
     if (rc) return rc;

@@ -461,6 +461,7 @@ struct PackProblem {
     GemmConfig cfg;
     int32_t n, n_pad, cin, taps, k, k_pad;
     int32_t row_bytes;     // GEMM_ROWS: kw * cin, the bytes of a kernel row, which starts every 32 packed bytes; else 0
+    int32_t cin_real;      // channels the source weights hold per tap when `cin` counts padding channels behind them (those pack as 0); 0 = cin
     // source index of (out channel o, in channel c, tap t) = o*so + c*sc + tap_off[t]
     int64_t so, sc;
     const int32_t *tap_off;  // device [taps]
@@ -518,6 +519,9 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &dw, int rows_per_t
 
 // ---------------------------------------------------------------- layout
 int launch_nchw2nhwc(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);
+// dst[pixel][g][0 .. cg_to) = src[pixel][g][0 .. cg) followed by cg_to - cg bytes `fill`, for `groups` channel groups per pixel
+int launch_pad_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t groups, int32_t cg, int32_t cg_to, uint32_t fill,
+                        hipStream_t stream);
 int launch_nhwc2nchw(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);
 
 }  // namespace eh

@@ -23,8 +23,10 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
         const int kk = p.row_bytes ? ((k & 31) < p.row_bytes ? (k >> 5) * p.row_bytes + (k & 31) : p.k) : k;
         if (o < p.n && kk < p.k) {
             const int t = kk / p.cin, c = kk - t * p.cin;
-            const uint8_t raw = p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]];
-            v = p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw - 128;
+            if (p.cin_real == 0 || c < p.cin_real) {
+                const uint8_t raw = p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]];
+                v = p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw - 128;
+            }
         }
         p.b[packed_b_offset(p.cfg, o, k >> 4, p.k_pad) + (k & 15)] = (int8_t)v;
         sum += v;
@@ -47,6 +49,28 @@ __global__ void fold_bias_kernel(const int32_t *bias, const int32_t *colsum, int
     int32_t v = 0;
     if (i < n) v = (bias ? bias[i] : 0) - za * colsum[i] + k * za * zw;
     folded[i] = v;
+}
+
+// Channel padding: rows of `cg` bytes (a pixel's channels, or one group's) copied to rows of `cg_to` bytes, the tail set
+// to `fill`.  Stands in for the reference's pad-and-align passes over activations (PadConvertKernels.cpp:25-167 pads the
+// reduction length of the im2col matrix to a multiple of 16).  One thread per destination dword; source dwords
+// are read at byte addresses.
+typedef uint32_t u32_a1 __attribute__((aligned(1)));
+__global__ __launch_bounds__(256) void pad_channels_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, const uint32_t total,
+                                                           const FastDiv div_quads, const int32_t cg, const int32_t cg_to, const uint32_t fill) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t row = fastdiv(idx, div_quads), quad = idx - row * (uint32_t)(cg_to >> 2);
+    const int c = (int)quad * 4;
+    const uint8_t *s = src + ((size_t)row * (size_t)cg + (size_t)c);
+    uint32_t v;
+    if (c + 4 <= cg) {
+        v = *reinterpret_cast<const u32_a1 *>(s);
+    } else {
+        v = fill * 0x01010101u;
+        for (int b = 0; c + b < cg; ++b) v = (v & ~(0xFFu << (8 * b))) | ((uint32_t)s[b] << (8 * b));
+    }
+    reinterpret_cast<uint32_t *>(dst)[idx] = v;
 }
 
 // Byte-matrix transpose per batch: src [batch][R][S] -> dst [batch][S][R].
@@ -273,6 +297,18 @@ int launch_transpose(const uint8_t *src, uint8_t *dst, int32_t batch, int32_t R,
 }
 
 }  // namespace
+
+int launch_pad_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t groups, int32_t cg, int32_t cg_to, uint32_t fill,
+                        hipStream_t stream) {
+    EH_REQUIRE(groups > 0 && cg > 0 && cg_to >= cg && (cg_to & 3) == 0, "pad_channels: bad extents %d x %d -> %d", groups, cg, cg_to);
+    const int64_t total = pixels * groups * (cg_to >> 2);
+    if (total <= 0) return EH_OK;
+    EH_REQUIRE(total < (1ll << 31) && pixels * groups * cg < (1ll << 31), "pad_channels: tensor too large");
+    hipLaunchKernelGGL(pad_channels_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, dst, (uint32_t)total,
+                       make_fastdiv((uint32_t)(cg_to >> 2)), cg, cg_to, fill & 0xFFu);
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
 
 int launch_pack_weights(const PackProblem &p, hipStream_t stream) {
     if (p.n_pad <= 0) return EH_OK;

@@ -56,6 +56,14 @@ typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh
  * eh_requant.zp_in, zp_out, act_min and act_max are then int8 values in [-128, 127].  The reference pairs this
  * precision with int8 weights (EH_W_SIGNED); the two flags are independent here. */
 #define EH_IO_SIGNED 0x200
+/* Or-ed into eh_conv_desc.layout (convolution, deconvolution) or into eh_fc_q8_plan's flags: keep the plan from staging
+ * a channel-padded copy of its input.  Without the flag, a plan whose channels per group (a fully connected layer's row
+ * length) are no multiple of 16 and fit none of the kernels for few channels copies the input, on every run, into an
+ * image of its own with each group padded to the next multiple of 16 (the role of the reference's pad-and-align pass,
+ * gpu/operators/cl_kernels/PadConvertKernels.cpp:25-167) and runs the wide-load kernels on that; with it, the
+ * byte-gathering kernel reads the caller's tensor directly: several times slower, no staging memory.  Results are
+ * the same bytes either way. */
+#define EH_EXACT_CHANNELS 0x400
 
 /* Integer requantization parameters of one operator execution: what
  * CLGEMMConvolutionQuantized::execute derives from its tensors

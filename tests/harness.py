@@ -30,10 +30,12 @@ def assert_same_host_quant(args, kwargs):
 
 
 def gpu_conv(x_nchw, w, bias, s, q, layout=eden.NCHW, weight_layout=eden.W_OIHW, runs=1):
-    """x_nchw: uint8 NCHW array; w in OIHW; returns NCHW uint8 output of the GPU path."""
+    """x_nchw: uint8 NCHW array; w in OIHW; returns NCHW uint8 output of the GPU path.  `layout` may carry plan flags
+    (eden.EXACT_CHANNELS) beside the tensor order."""
+    flags, layout = layout & ~0xFF, layout & 0xFF
     ho, wo = O.conv_out_hw(s)
     desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, (s.stride_h, s.stride_w),
-                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), s.groups, 1, layout, weight_layout)
+                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), s.groups, 1, layout | flags, weight_layout)
     x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
     w_dev = w if weight_layout == eden.W_OIHW else w.transpose(0, 2, 3, 1)
     d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), (eden.DeviceBuffer(host=bias) if bias is not None else None)
@@ -68,9 +70,10 @@ def gpu_dwconv(x_nchw, w, bias, s, q, layout=eden.NCHW):
 
 
 def gpu_deconv(x_nchw, w_iohw, bias, s, q, layout=eden.NCHW, weight_layout=eden.W_IOHW):
+    flags, layout = layout & ~0xFF, layout & 0xFF
     ho, wo = O.deconv_out_hw(s)
     desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, (s.stride_h, s.stride_w),
-                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (1, 1), s.groups, 1, layout, weight_layout)
+                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (1, 1), s.groups, 1, layout | flags, weight_layout)
     x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
     w_dev = w_iohw if weight_layout == eden.W_IOHW else w_iohw.transpose(1, 2, 3, 0)
     d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w_dev), (eden.DeviceBuffer(host=bias) if bias is not None else None)
@@ -85,12 +88,12 @@ def gpu_deconv(x_nchw, w_iohw, bias, s, q, layout=eden.NCHW, weight_layout=eden.
     return np.ascontiguousarray(out)
 
 
-def gpu_fc(a, w, bias, q):
+def gpu_fc(a, w, bias, q, flags=0):
     m, k = a.shape
     n = w.shape[0]
     d_a, d_w, d_b = eden.DeviceBuffer(host=a), eden.DeviceBuffer(host=w), (eden.DeviceBuffer(host=bias) if bias is not None else None)
     d_o = eden.DeviceBuffer(nbytes=m * n)
-    plan = eden.FcPlan(m, k, n, d_w, d_b, q)
+    plan = eden.FcPlan(m, k, n, d_w, d_b, q, flags=flags)
     plan.run(d_a, d_o, q)
     out = d_o.download((m, n))
     plan.destroy()

@@ -185,11 +185,10 @@ def test_3x3_stride_1_convolutions_take_the_patch_kernel():
     assert eden.conv_kernels(eden.conv_desc(64, 256, 14, 14, 256, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["dma_128x128"]
     assert eden.conv_kernels(eden.conv_desc(1, 48, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
     assert eden.conv_kernels(eden.conv_desc(1, 16, 112, 112, 32, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
-    # stride 2, dilation 2, groups, 8-byte channel counts, tiny images: the implicit-GEMM kernels
+    # stride 2, dilation 2, groups, tiny images: the implicit-GEMM kernels
     for d in (eden.conv_desc(1, 64, 56, 56, 64, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), layout=nhwc),
               eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(2, 2, 2, 2), dil=(2, 2), layout=nhwc),
               eden.conv_desc(1, 64, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), groups=2, layout=nhwc),
-              eden.conv_desc(1, 24, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc),
               eden.conv_desc(4, 64, 7, 7, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)):
         assert "conv3x3_patch" not in eden.conv_kernels(d)
 
@@ -205,6 +204,23 @@ def test_few_channel_convolutions_take_the_kernel_row_kernel():
     for d in (eden.conv_desc(1, 3, 64, 64, 32, 11, 11, layout=nhwc), eden.conv_desc(1, 3, 64, 64, 32, 4, 4, layout=nhwc),
               eden.conv_desc(1, 3, 64, 64, 32, 5, 5, dil=(2, 2), layout=nhwc), eden.conv_desc(1, 8, 64, 64, 32, 7, 7, layout=nhwc)):
         assert "few_channel_rows" not in eden.conv_kernels(d)
+
+
+def test_ragged_channel_counts_run_on_a_padded_copy_unless_told_otherwise():
+    """Channels per group that are no multiple of 16 and fit none of the few-channel kernels: the plan is built on
+    channels padded to the next multiple of 16 (the wide-load kernels); EXACT_CHANNELS keeps the byte-gathering kernel."""
+    nhwc, exact = eden.NHWC, eden.NHWC | eden.EXACT_CHANNELS
+    assert eden.conv_kernels(eden.conv_desc(8, 21, 64, 64, 21, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    assert eden.conv_kernels(eden.conv_desc(8, 21, 64, 64, 21, 3, 3, pad=(1, 1, 1, 1), layout=exact)) == ["staged"]
+    assert eden.conv_kernels(eden.conv_desc(8, 100, 32, 32, 100, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    assert eden.conv_kernels(eden.conv_desc(1, 24, 56, 56, 64, 3, 3, pad=(1, 1, 1, 1), layout=nhwc)) == ["conv3x3_patch"]
+    assert eden.conv_kernels(eden.conv_desc(8, 6, 112, 112, 16, 5, 5, layout=nhwc))[0].startswith("dma_")
+    assert eden.conv_kernels(eden.conv_desc(1, 20, 8, 8, 12, 3, 3, groups=2, layout=exact)) == ["staged", "staged"]
+    assert "staged" not in eden.conv_kernels(eden.conv_desc(1, 20, 8, 8, 12, 3, 3, groups=2, layout=nhwc))
+    assert "staged" not in eden.conv_kernels(eden.conv_desc(8, 21, 64, 64, 21, 16, 16, stride=(8, 8), pad=(4, 4, 4, 4), layout=nhwc, weight_layout=eden.W_IOHW), deconv=True)
+    # channel counts the one-tap and few-channel kernels take as they are keep them
+    assert eden.conv_kernels(eden.conv_desc(32, 24, 56, 56, 144, 1, 1, layout=nhwc)) == ["one_tap"]
+    assert eden.conv_kernels(eden.conv_desc(1, 3, 64, 64, 32, 3, 3, layout=nhwc)) == ["c3k3"]
 
 
 def test_classifier_heads_take_the_kernel_cut_along_the_weights():

@@ -112,7 +112,9 @@ RUN_ADD_CASES = [
     dict(n=4, c=384, h=14, w=14, cout=64, kh=1, kw=1, fused=True),
     dict(n=2, c=576, h=7, w=7, cout=96, kh=1, kw=1, fused=True),
     dict(n=32, c=264, h=28, w=28, cout=256, kh=1, kw=1, fused=False),
-    dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2, fused=False),
+    dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2, fused=False, exact=True),
+    # the same on its channel-padded copy: split-reduction tiles (fused)
+    dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2, fused=True),
 ]
 
 
@@ -122,6 +124,7 @@ def test_conv_with_residual_add_equals_conv_then_add(case, layout):
     print("conv + add", case, layout, flush=True)
     case = dict(case)
     fused = case.pop("fused")
+    flags = eden.EXACT_CHANNELS if case.pop("exact", False) else 0
     s = O.conv_shape(**case)
     ho, wo = O.conv_out_hw(s)
     x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 500 + s.c)
@@ -136,7 +139,7 @@ def test_conv_with_residual_add_equals_conv_then_add(case, layout):
         want = O.add(res, O.conv2d(x, w, b, s, q), aq)
         nhwc = layout == "nhwc"
         desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, s.kh, s.kw, (s.stride_h, s.stride_w), (s.pad_t, s.pad_b, s.pad_l, s.pad_r),
-                              (1, 1), s.groups, 1, eden.NHWC if nhwc else eden.NCHW, eden.W_OIHW)
+                              (1, 1), s.groups, 1, (eden.NHWC if nhwc else eden.NCHW) | flags, eden.W_OIHW)
         to_dev = (lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))) if nhwc else (lambda a: a)
         d_x, d_w, d_b = eden.DeviceBuffer(host=to_dev(x)), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
         d_r, d_o = eden.DeviceBuffer(host=to_dev(res)), eden.DeviceBuffer(nbytes=want.size)

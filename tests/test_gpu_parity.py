@@ -71,19 +71,29 @@ FC_CASES = [
     (33, 2048, 72, 131, 120),
     (64, 9216, 64, 0, 255),
     (17, 304, 8, 5, 100),
+    # row lengths that are no multiple of 16 beyond the one-tap kernel's reach: the channel-padded copy of the input
+    (1, 1001, 1001, 3, 128),
+    (64, 1001, 77, 131, 120),
+    (8, 300, 10, 200, 9),
+    (300, 90, 40, 17, 250),
+    (2, 70, 130, 255, 0),
 ]
 
 
+@pytest.mark.parametrize("exact_channels", [False, True], ids=["", "exact_channels"])
 @pytest.mark.parametrize("m,k,n,zp_a,zp_w", FC_CASES)
-def test_fc_matches_oracle(m, k, n, zp_a, zp_w):
-    print("fc", m, k, n, zp_a, zp_w, flush=True)
+def test_fc_matches_oracle(m, k, n, zp_a, zp_w, exact_channels):
+    """exact_channels: the plan may not stage a padded copy of its input, which keeps the byte-gathering kernel covered"""
+    if exact_channels and k % 16 == 0:
+        pytest.skip("the flag changes nothing for whole 16-byte rows")
+    print("fc", m, k, n, zp_a, zp_w, exact_channels, flush=True)
     a = synth.fill_u8((m, k), SEED + m)
     w = synth.fill_u8((n, k), SEED + k)
     b = synth.fill_i32((n,), SEED + n, -1000, 1000)
     _, acc = O.fc(a, w, b, O.raw_quant(zp_in=zp_a, zp_w=zp_w), want_acc=True)
     q = centred_quant(acc, zp_a, zp_w)
     want = O.fc(a, w, b, q)
-    got = gpu_fc(a, w, b, to_eh_requant(q))
+    got = gpu_fc(a, w, b, to_eh_requant(q), flags=eden.EXACT_CHANNELS if exact_channels else 0)
     assert np.array_equal(got, want), diff_report(got, want)
     assert want.std() > 10  # the case exercises the requant range, not a saturated constant
 
@@ -249,12 +259,23 @@ CONV_CASES = [
     # 1x1 on at most 64 pixels with a long reduction: cut along the weights
     dict(n=8, c=1280, h=1, w=1, cout=100, kh=1, kw=1),
     dict(n=2, c=512, h=5, w=5, cout=48, kh=1, kw=1),
+    # channels per group that are no multiple of 16 and fit no few-channel kernel: the channel-padded copy of the input
+    # (NCHW: after the transposition); with EXACT_CHANNELS the byte-gathering kernel
+    dict(n=2, c=21, h=17, w=15, cout=21, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=6, h=20, w=20, cout=16, kh=5, kw=5),
+    dict(n=3, c=68, h=9, w=11, cout=68, kh=1, kw=1, pad=(0, 1, 0, 1)),
+    dict(n=2, c=100, h=12, w=12, cout=100, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=42, h=14, w=9, cout=30, kh=3, kw=2, stride=(2, 1), pad=(1, 0, 1, 1), dil=(1, 2), groups=2),
+    dict(n=2, c=30, h=8, w=8, cout=45, kh=1, kw=1, groups=3, stride=(2, 2)),
+    dict(n=1, c=17, h=1, w=1, cout=9, kh=1, kw=1),
 ]
 
 
-@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC, eden.NHWC | eden.EXACT_CHANNELS], ids=["nchw", "nhwc", "nhwc_exact_channels"])
 @pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
 def test_conv_matches_oracle(case, layout):
+    if layout & eden.EXACT_CHANNELS and (case["c"] // case.get("groups", 1)) % 16 == 0:
+        pytest.skip("the flag changes nothing for whole 16-byte channel groups")
     print("conv", case, layout, flush=True)
     s = O.conv_shape(**case)
     x, w, b = conv_tensors(s, SEED + s.c + s.cout)
@@ -578,12 +599,20 @@ DECONV_CASES = [
     # nine one-tap phases of equal shape: launches of four, four and one problems of the one-tap kernel
     dict(n=2, c=32, h=9, w=7, cout=48, kh=3, kw=3, stride=(3, 3), pad=(0, 0, 0, 0)),
     dict(n=3, c=64, h=20, w=20, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, 0, 0, 0)),
+    # channels per group that are no multiple of 16, several taps per phase: the channel-padded copy of the input
+    # (an upsampling layer over 21 class scores, kernel twice the stride; groups; a kernel that is no multiple of the stride)
+    dict(n=2, c=21, h=9, w=8, cout=21, kh=4, kw=4, stride=(2, 2), pad=(1, 1, 1, 1)),
+    dict(n=1, c=21, h=5, w=6, cout=21, kh=16, kw=16, stride=(8, 8), pad=(4, 4, 4, 4)),
+    dict(n=1, c=40, h=7, w=7, cout=12, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0), groups=2),
+    dict(n=2, c=5, h=6, w=6, cout=7, kh=5, kw=5, stride=(2, 2), pad=(2, 2, 2, 2)),
 ]
 
 
-@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC, eden.NHWC | eden.EXACT_CHANNELS], ids=["nchw", "nhwc", "nhwc_exact_channels"])
 @pytest.mark.parametrize("case", DECONV_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
 def test_deconv_matches_oracle(case, layout):
+    if layout & eden.EXACT_CHANNELS and (case["c"] // case.get("groups", 1)) % 16 == 0:
+        pytest.skip("the flag changes nothing for whole 16-byte channel groups")
     print("deconv", case, layout, flush=True)
     s = O.conv_shape(**case)
     x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 60)
@@ -595,6 +624,29 @@ def test_deconv_matches_oracle(case, layout):
     got = gpu_deconv(x, w, b, s, to_eh_requant(q), layout=layout)
     assert np.array_equal(got, want), diff_report(got, want)
     assert want.std() > 10
+
+
+def test_channel_padded_plan_follows_the_input_zero_point():
+    """The padding bytes of the staged copy hold the input zero point of the run that reads them: one plan, run with
+    two zero points, int8 tensors included."""
+    s = O.conv_shape(2, 21, 11, 9, 24, 3, 3, pad=(1, 1, 1, 1))
+    x, w, b = conv_tensors(s, SEED + 777)
+    ho, wo = O.conv_out_hw(s)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, 1, eden.NHWC, eden.W_OIHW)
+    assert eden.conv_kernels(desc) != ["staged"]
+    d_x = eden.DeviceBuffer(host=np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+    d_w, d_b, d_o = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b), eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
+    quants = []
+    for zp_in in (131, 7, 255):
+        _, acc = O.conv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=120), want_acc=True)
+        quants.append(centred_quant(acc, zp_in, 120))
+    plan = eden.ConvPlan(desc, d_w, d_b, to_eh_requant(quants[0]))
+    for q in quants:
+        plan.run(d_x, d_o, to_eh_requant(q))
+        got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+        want = O.conv2d(x, w, b, s, q)
+        assert np.array_equal(got, want), diff_report(got, want)
+    plan.destroy()
 
 
 def test_deconv_ohwi_weights():

@@ -35,7 +35,9 @@ def test_static_scratch_entry_point_equals_the_allocating_one_on_two_calls_in_a_
     big = planar_conv(dict(n=3, c=64, h=40, w=36, cout=96, kh=3, kw=3, pad=(1, 1, 1, 1)), SEED)
     small = planar_conv(dict(n=1, c=16, h=9, w=11, cout=24, kh=3, kw=3, stride=(2, 1), pad=(1, 0, 0, 1)), SEED + 10)
     grouped = planar_conv(dict(n=2, c=32, h=10, w=10, cout=48, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2), SEED + 20)
-    for case in (big, small, grouped, big):   # the second call is smaller and finds the first one's bytes in the scratch
+    # 21 channels: the plan also stages a channel-padded copy of the transposed input, behind the two planar images
+    ragged = planar_conv(dict(n=2, c=21, h=17, w=15, cout=21, kh=3, kw=3, pad=(1, 1, 1, 1)), SEED + 25)
+    for case in (big, small, grouped, ragged, big, ragged):   # the second call is smaller and finds the first one's bytes in the scratch
         count = int(np.prod(case["shape"]))
         d_ref, d_got = eden.DeviceBuffer(nbytes=count), eden.DeviceBuffer(nbytes=count)
         case["plan"].run(case["d_x"], d_ref, case["q"])
