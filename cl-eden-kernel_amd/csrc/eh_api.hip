@@ -123,6 +123,11 @@ struct GemmPart {
     int32_t *tap_off = nullptr;
     int32_t n = 0, n_pad = 0, k = 0, k_pad = 0, vec = 1, taps = 0, cin = 0;
     int32_t cin_real = 0;     // channels per tap in the source weights when `cin` includes padding channels; 0 = cin
+    // Several kernel columns of a transposed convolution as one problem (their outputs are neighbouring pixels): column
+    // o of the problem is output channel o % n_period of kernel column o / n_period, `period_step` weight elements on.
+    int32_t n_period = 0;
+    int64_t period_step = 0;
+    int32_t *pc_multiplier_rep = nullptr, *pc_shift_rep = nullptr;  // the operator's per-channel pairs, repeated per kernel column
     GemmConfig cfg;
     int64_t so = 0, sc = 0;   // source weight strides (out channel, in channel)
     int64_t w_base = 0;       // element offset of this part in the source weights
@@ -135,6 +140,8 @@ struct GemmPart {
         dev_free(folded);
         dev_free(ktab);
         dev_free(tap_off);
+        dev_free(pc_multiplier_rep);
+        dev_free(pc_shift_rep);
     }
 };
 
@@ -265,6 +272,8 @@ int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t str
     pp.k_pad = g.k_pad;
     pp.row_bytes = g.cfg.id == GEMM_ROWS ? g.proto.rows_kw * g.cin : 0;
     pp.cin_real = g.cin_real;
+    pp.n_period = g.n_period;
+    pp.period_step = g.period_step;
     pp.so = g.so;
     pp.sc = g.sc;
     pp.tap_off = g.tap_off;
@@ -335,6 +344,10 @@ struct GemmOp {
             EH_HIP(hipStreamSynchronize(stream));
             dev_free(pc_multiplier);
             dev_free(pc_shift);
+            for (auto &g : parts) {
+                dev_free(g.pc_multiplier_rep);
+                dev_free(g.pc_shift_rep);
+            }
             return EH_OK;
         }
         EH_REQUIRE(multipliers != nullptr && shifts != nullptr && count == cout, "per-channel arrays must hold %d entries (got %d)", cout, count);
@@ -344,7 +357,19 @@ struct GemmOp {
         if (!pc_multiplier && (rc = dev_alloc(&pc_multiplier, (size_t)cout + 512))) return rc;
         if (!pc_shift && (rc = dev_alloc(&pc_shift, (size_t)cout + 512))) return rc;
         pc_fast = all_pairs_fast(multipliers, shifts, cout, -2);  // the table form's rounding term needs rs >= 2
-        return upload_padded_pairs(pc_multiplier, pc_shift, multipliers, shifts, cout, 512, stream);
+        if ((rc = upload_padded_pairs(pc_multiplier, pc_shift, multipliers, shifts, cout, 512, stream))) return rc;
+        for (auto &g : parts) {
+            if (g.n_period == 0) continue;
+            std::vector<int32_t> m_rep((size_t)g.n), s_rep((size_t)g.n);
+            for (int i = 0; i < g.n; ++i) {
+                m_rep[i] = multipliers[g.bias_base + i % g.n_period];
+                s_rep[i] = shifts[g.bias_base + i % g.n_period];
+            }
+            if (!g.pc_multiplier_rep && (rc = dev_alloc(&g.pc_multiplier_rep, (size_t)g.n + 512))) return rc;
+            if (!g.pc_shift_rep && (rc = dev_alloc(&g.pc_shift_rep, (size_t)g.n + 512))) return rc;
+            if ((rc = upload_padded_pairs(g.pc_multiplier_rep, g.pc_shift_rep, m_rep.data(), s_rep.data(), g.n, 512, stream))) return rc;
+        }
+        return EH_OK;
     }
 
     void release() {
@@ -384,7 +409,7 @@ struct GemmOp {
         }
         for (auto &g : parts) {
             int rc = launch_fold_bias(has_bias ? bias_copy + g.bias_base : nullptr, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, zp_w_u8(nq),
-                                      fillbuf, io_signed ? 0x80 : 0, stream);
+                                      fillbuf, io_signed ? 0x80 : 0, stream, g.n_period);
             if (rc) return rc;
         }
         q = nq;
@@ -433,8 +458,8 @@ struct GemmOp {
         p.residual = residual ? residual + g.bias_base : nullptr;
         if (residual) p.radd = *radd;
         if (pc_multiplier) {
-            p.rq.pc_multiplier = pc_multiplier + g.bias_base;
-            p.rq.pc_shift = pc_shift + g.bias_base;
+            p.rq.pc_multiplier = g.n_period ? g.pc_multiplier_rep : pc_multiplier + g.bias_base;
+            p.rq.pc_shift = g.n_period ? g.pc_shift_rep : pc_shift + g.bias_base;
             // every kernel but the register-staged one has the single-shift form per channel (the first-layer
             // kernel for fewer than 32 channels ignores the flag)
             const bool has_form = g.cfg.id != GEMM_STAGED;
@@ -1247,18 +1272,45 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
     if (padded) cig = op.pad_cg_to;
     const int pixel_c = padded ? G * cig : d->c;
     const int sh = d->stride_h, sw = d->stride_w;
+    // Output columns ox0, ox0 + 1, ... whose phases read the same input columns (their kernel columns px, px + 1, ...
+    // differ, their taps' positions do not) and cover equally many positions go out as ONE problem whose columns are
+    // (kernel column, output channel): a row of the problem then writes neighbouring output pixels, count * cout
+    // contiguous bytes, and the launches shrink by that count.  Needs one group (a pixel holds the problem's channels
+    // alone) and more than one tap (the one-tap kernel has its own batching).
+    struct XPhase {
+        int px, ox0, wo_p, ntx, bx;
+    };
     for (int g = 0; g < G; ++g)
-        for (int py = 0; py < sh; ++py)
+        for (int py = 0; py < sh; ++py) {
+            const int oy0 = ((py - d->pad_t) % sh + sh) % sh;
+            if (oy0 >= oh) continue;
+            const int ho_p = (oh - oy0 + sh - 1) / sh;
+            const int nty = py < d->kh ? (d->kh - py + sh - 1) / sh : 0;
+            const int by = (oy0 + d->pad_t - py) / sh;
+            std::vector<XPhase> xs;
             for (int px = 0; px < sw; ++px) {
-                const int oy0 = ((py - d->pad_t) % sh + sh) % sh, ox0 = ((px - d->pad_l) % sw + sw) % sw;
-                if (oy0 >= oh || ox0 >= ow) continue;
-                const int ho_p = (oh - oy0 + sh - 1) / sh, wo_p = (ow - ox0 + sw - 1) / sw;
-                const int nty = py < d->kh ? (d->kh - py + sh - 1) / sh : 0;
-                const int ntx = px < d->kw ? (d->kw - px + sw - 1) / sw : 0;
-                const int by = (oy0 + d->pad_t - py) / sh, bx = (ox0 + d->pad_l - px) / sw;
+                XPhase x;
+                x.px = px;
+                x.ox0 = ((px - d->pad_l) % sw + sw) % sw;
+                if (x.ox0 >= ow) continue;
+                x.wo_p = (ow - x.ox0 + sw - 1) / sw;
+                x.ntx = px < d->kw ? (d->kw - px + sw - 1) / sw : 0;
+                x.bx = (x.ox0 + d->pad_l - px) / sw;
+                xs.push_back(x);
+            }
+            std::sort(xs.begin(), xs.end(), [](const XPhase &a, const XPhase &b) { return a.ox0 < b.ox0; });
+            for (size_t first = 0; first < xs.size();) {
+                const XPhase &x0 = xs[first];
+                size_t last = first + 1;
+                while (G == 1 && nty * x0.ntx > 1 && last < xs.size() && xs[last].ox0 == xs[last - 1].ox0 + 1 &&
+                       xs[last].px == xs[last - 1].px + 1 && xs[last].bx == x0.bx && xs[last].wo_p == x0.wo_p && xs[last].ntx == x0.ntx)
+                    ++last;
+                const int count = (int)(last - first);
+                first = last;
+                const int px = x0.px, ox0 = x0.ox0, wo_p = x0.wo_p, ntx = x0.ntx, bx = x0.bx;
                 op.parts.emplace_back();
                 GemmPart &part = op.parts.back();
-                part.n = cog;
+                part.n = cog * count;
                 part.cin = cig;
                 part.cin_real = padded ? cig_real : 0;
                 part.taps = nty * ntx;
@@ -1270,11 +1322,14 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                     part.so = (int64_t)d->kh * d->kw;
                     part.sc = (int64_t)cog * d->kh * d->kw;
                     part.w_base = (int64_t)g * cig_real * cog * d->kh * d->kw;
+                    part.period_step = 1;
                 } else {  // OHWI, groups == 1
                     part.so = (int64_t)d->kh * d->kw * d->c;
                     part.sc = 1;
                     part.w_base = 0;
+                    part.period_step = d->c;
                 }
+                part.n_period = count > 1 ? cog : 0;
                 for (int ty = 0; ty < nty; ++ty)
                     for (int tx = 0; tx < ntx; ++tx) {
                         const int ky = py + sh * ty, kx = px + sw * tx;
@@ -1309,9 +1364,10 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                 p.out_x0 = ox0;
                 p.ldc = d->cout;
                 // phases (and groups) of equal shape share launches: choose the tile shape for the joint tile count
-                const int siblings = (d->kh % sh == 0 && d->kw % sw == 0) ? std::min(G * sh * sw, (int)GemmBatch::MAX) : 1;
+                const int siblings = (d->kh % sh == 0 && d->kw % sw == 0) ? std::min(G * sh * sw / count, (int)GemmBatch::MAX) : 1;
                 if ((rc = finish_part(part, units, tap_off, stream, siblings))) return rc;
             }
+        }
     if (wants_channel_padding(op, G, cig_real)) return deconv_plan_build(pl, d, stream);
     return op.alloc_staging();
 }

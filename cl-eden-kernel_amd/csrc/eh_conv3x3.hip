@@ -285,8 +285,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void c
                     if (wide && n + 16 <= p.n) {
                         *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
                     } else {
-                        const int cnt = p.n - n < 16 ? p.n - n : 16;
-                        for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+                        store_bytes_any_alignment(dst, packed, p.n - n < 16 ? p.n - n : 16);
                     }
                 }
             }

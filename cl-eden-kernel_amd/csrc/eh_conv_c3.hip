@@ -184,8 +184,7 @@ __global__ __launch_bounds__(256) void conv_c3k3_mfma_kernel(const GemmProblem p
                 if (cnt >= 16 && (p.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 3) == 0) {
                     *reinterpret_cast<u32x4_a4 *>(dst) = u32x4_a4{packed[0], packed[1], packed[2], packed[3]};
                 } else {
-                    const int c = cnt < 16 ? cnt : 16;
-                    for (int t = 0; t < c; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+                    store_bytes_any_alignment(dst, packed, cnt < 16 ? cnt : 16);
                 }
             }
         }
@@ -284,8 +283,7 @@ __global__ __launch_bounds__(256) void conv_c3k3_kernel(const GemmProblem p, con
     if (aligned16 && n0 + 16 <= p.n) {
         *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     } else {
-        const int cnt = p.n - n0 < 16 ? p.n - n0 : 16;
-        for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+        store_bytes_any_alignment(dst, packed, p.n - n0 < 16 ? p.n - n0 : 16);
     }
 }
 

@@ -263,8 +263,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_u8_kernel(const GemmProbl
         if (wide && n + 16 <= p.n) {
             *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
         } else {
-            const int cnt = p.n - n < 16 ? p.n - n : 16;
-            for (int t = 0; t < cnt; ++t) dst[t] = src[t];
+            const uint4 v = *reinterpret_cast<const uint4 *>(src);
+            const uint32_t packed[4] = {v.x, v.y, v.z, v.w};
+            store_bytes_any_alignment(dst, packed, p.n - n < 16 ? p.n - n : 16);
         }
     }
 }

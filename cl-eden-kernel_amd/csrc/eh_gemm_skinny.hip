@@ -154,8 +154,7 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_gemm_kernel(const GemmProb
         if (cnt >= 16 && (p.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 3) == 0) {
             *reinterpret_cast<u32x4_a4 *>(dst) = u32x4_a4{packed[0], packed[1], packed[2], packed[3]};
         } else {
-            const int c = cnt < 16 ? cnt : 16;
-            for (int t = 0; t < c; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+            store_bytes_any_alignment(dst, packed, cnt < 16 ? cnt : 16);
         }
     }
 }

@@ -257,8 +257,7 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const std::conditional
         } else if (wide && cnt == 8) {
             *reinterpret_cast<u32x2_a4 *>(dst) = u32x2_a4{packed[0], packed[1]};
         } else {
-            const int c = cnt < 16 ? cnt : 16;
-            for (int t = 0; t < c; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+            store_bytes_any_alignment(dst, packed, cnt < 16 ? cnt : 16);
         }
     };
 

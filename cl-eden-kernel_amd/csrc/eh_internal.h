@@ -227,6 +227,23 @@ __host__ __device__ __forceinline__ uint32_t pack_bytes(uint32_t b0, uint32_t b1
 #endif
 }
 
+// The first `cnt` (1 .. 16) of sixteen result bytes to a destination of any alignment: whole dwords at byte addresses
+// (global memory takes them), single bytes for the last one to three.  The fallback of every epilogue whose rows do
+// not start on 16-byte boundaries (an odd channel count) or end inside a 16-byte chunk.
+typedef uint32_t u32_any_alignment __attribute__((aligned(1)));
+__device__ __forceinline__ void store_bytes_any_alignment(uint8_t *dst, const uint32_t (&packed)[4], int cnt) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        if (cnt >= 4 * g + 4) {
+            *reinterpret_cast<u32_any_alignment *>(dst + 4 * g) = packed[g];
+        } else {
+#pragma unroll
+            for (int t = 0; t < 3; ++t)
+                if (4 * g + t < cnt) dst[4 * g + t] = (uint8_t)(packed[g] >> (8 * t));
+        }
+    }
+}
+
 template <int MODE>
 __host__ __device__ __forceinline__ uint32_t requant_u8_as(int32_t acc, const RequantDev &r) {
     if constexpr (MODE == 2)
@@ -464,13 +481,17 @@ struct PackProblem {
     int32_t cin_real;      // channels the source weights hold per tap when `cin` counts padding channels behind them (those pack as 0); 0 = cin
     // source index of (out channel o, in channel c, tap t) = o*so + c*sc + tap_off[t]
     int64_t so, sc;
+    // n_period != 0: packed row o is output channel o % n_period of the (o / n_period)-th of several kernel columns
+    // that share a launch, and its source index is (o % n_period)*so + (o / n_period)*period_step + c*sc + tap_off[t]
+    int32_t n_period;
+    int64_t period_step;
     const int32_t *tap_off;  // device [taps]
 };
 int launch_pack_weights(const PackProblem &p, hipStream_t stream);
-// folded[n] = bias[n] - za * colsum[n] + k * za * zw   (za = zp_in - 128, zw = zp_w - 128)
+// folded[n] = bias[n] - za * colsum[n] + k * za * zw   (za = zp_in - 128, zw = zp_w - 128); bias_period != 0: bias[n % bias_period]
 // also refreshes the 32-byte fill constant when `fillbuf` is not null
 int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad,
-                     int32_t k, int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, int32_t io_flip, hipStream_t stream);
+                     int32_t k, int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, int32_t io_flip, hipStream_t stream, int32_t bias_period = 0);
 
 // ---------------------------------------------------------------- depthwise
 struct DwProblem {

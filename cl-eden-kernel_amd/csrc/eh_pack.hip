@@ -24,7 +24,8 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
         if (o < p.n && kk < p.k) {
             const int t = kk / p.cin, c = kk - t * p.cin;
             if (p.cin_real == 0 || c < p.cin_real) {
-                const uint8_t raw = p.w[(int64_t)o * p.so + (int64_t)c * p.sc + p.tap_off[t]];
+                const int64_t row = p.n_period ? (int64_t)(o % p.n_period) * p.so + (int64_t)(o / p.n_period) * p.period_step : (int64_t)o * p.so;
+                const uint8_t raw = p.w[row + (int64_t)c * p.sc + p.tap_off[t]];
                 v = p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw - 128;
             }
         }
@@ -41,13 +42,13 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
 }
 
 __global__ void fold_bias_kernel(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad,
-                                 int32_t k, int32_t za, int32_t zw, uint8_t *fillbuf, int32_t io_flip) {
+                                 int32_t k, int32_t za, int32_t zw, uint8_t *fillbuf, int32_t io_flip, int32_t bias_period) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     // bytes as the input tensor stores them: int8 tensors (io_flip = 0x80) hold value - 128
     if (fillbuf && i < 32) fillbuf[i] = (uint8_t)((i < 16 ? za + 128 : 0x80) ^ io_flip);
     if (i >= n_pad) return;
     int32_t v = 0;
-    if (i < n) v = (bias ? bias[i] : 0) - za * colsum[i] + k * za * zw;
+    if (i < n) v = (bias ? bias[bias_period ? i % bias_period : i] : 0) - za * colsum[i] + k * za * zw;
     folded[i] = v;
 }
 
@@ -318,10 +319,10 @@ int launch_pack_weights(const PackProblem &p, hipStream_t stream) {
 }
 
 int launch_fold_bias(const int32_t *bias, const int32_t *colsum, int32_t *folded, int32_t n, int32_t n_pad, int32_t k,
-                     int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, int32_t io_flip, hipStream_t stream) {
+                     int32_t zp_in, int32_t zp_w, uint8_t *fillbuf, int32_t io_flip, hipStream_t stream, int32_t bias_period) {
     if (n_pad <= 0) return EH_OK;
     hipLaunchKernelGGL(fold_bias_kernel, dim3((n_pad + 255) / 256), dim3(256), 0, stream, bias, colsum, folded, n, n_pad,
-                       k, zp_in - 128, zp_w - 128, fillbuf, io_flip);
+                       k, zp_in - 128, zp_w - 128, fillbuf, io_flip, bias_period);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }

@@ -169,6 +169,7 @@ DECONV_CASES = [
     dict(n=2, c=64, h=14, w=14, cout=32, kh=2, kw=2, stride=(2, 2)),
     dict(n=1, c=24, h=7, w=9, cout=40, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),
     dict(n=2, c=12, h=6, w=5, cout=8, kh=4, kw=4, stride=(2, 2), pad=(1, 1, 1, 1), groups=2),
+    dict(n=1, c=21, h=6, w=6, cout=21, kh=8, kw=8, stride=(4, 4), pad=(2, 2, 2, 2)),       # merged kernel columns on a channel-padded copy
 ]
 
 

@@ -605,6 +605,15 @@ DECONV_CASES = [
     dict(n=1, c=21, h=5, w=6, cout=21, kh=16, kw=16, stride=(8, 8), pad=(4, 4, 4, 4)),
     dict(n=1, c=40, h=7, w=7, cout=12, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0), groups=2),
     dict(n=2, c=5, h=6, w=6, cout=7, kh=5, kw=5, stride=(2, 2), pad=(2, 2, 2, 2)),
+    # output columns whose phases read the same input columns leave as one problem (kernel a multiple of the stride,
+    # several taps): three kernel columns in one, two classes of two, a ragged last column group (kept apart), a padding
+    # beyond the stride, a kernel three times the stride
+    dict(n=2, c=16, h=7, w=6, cout=24, kh=6, kw=6, stride=(3, 3), pad=(0, 0, 0, 0)),
+    dict(n=1, c=32, h=9, w=9, cout=20, kh=8, kw=8, stride=(4, 4), pad=(2, 2, 2, 2)),
+    dict(n=2, c=16, h=6, w=7, cout=16, kh=6, kw=6, stride=(3, 3), pad=(1, 2, 1, 3)),
+    dict(n=1, c=16, h=5, w=8, cout=40, kh=4, kw=8, stride=(2, 4), pad=(1, 1, 5, 5)),
+    dict(n=1, c=16, h=6, w=6, cout=8, kh=3, kw=9, stride=(1, 3), pad=(1, 1, 3, 3)),
+    dict(n=3, c=48, h=12, w=12, cout=21, kh=16, kw=16, stride=(8, 8), pad=(4, 4, 4, 4)),
 ]
 
 
@@ -649,15 +658,17 @@ def test_channel_padded_plan_follows_the_input_zero_point():
     plan.destroy()
 
 
-def test_deconv_ohwi_weights():
-    s = O.conv_shape(1, 16, 5, 5, 12, 4, 4, stride=(2, 2), pad=(1, 1, 1, 1))
+@pytest.mark.parametrize("k,stride,pad", [(4, 2, 1), (8, 4, 2), (6, 3, 0)], ids=["k4s2", "k8s4_merged_columns", "k6s3_merged_columns"])
+def test_deconv_ohwi_weights(k, stride, pad):
+    s = O.conv_shape(1, 16, 5, 5, 12, k, k, stride=(stride, stride), pad=(pad,) * 4)
     x = synth.fill_u8((1, 16, 5, 5), SEED + 63)
-    w = synth.fill_u8((16, 12, 4, 4), SEED + 64)
+    w = synth.fill_u8((16, 12, k, k), SEED + 64)
     b = synth.fill_i32((12,), SEED + 65, -100, 100)
     q = quant(0.03, 131, 0.01, 77, 0.3, 5)
     want = O.deconv2d(x, w, b, s, q)
     got = gpu_deconv(x, w, b, s, to_eh_requant(q), layout=eden.NHWC, weight_layout=eden.W_OHWI)
     assert np.array_equal(got, want), diff_report(got, want)
+    assert want.std() > 10
 
 
 def test_deconv_config4_full_size():

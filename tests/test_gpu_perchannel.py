@@ -233,6 +233,8 @@ DECONV_PC_CASES = [
     dict(n=1, c=24, h=7, w=9, cout=40, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),       # unequal phases
     dict(n=2, c=12, h=6, w=5, cout=8, kh=4, kw=4, stride=(2, 2), pad=(1, 1, 1, 1), groups=2),
     dict(n=1, c=16, h=8, w=8, cout=16, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),
+    dict(n=2, c=16, h=7, w=6, cout=24, kh=6, kw=6, stride=(3, 3)),                         # three kernel columns per problem: the pairs repeat per column
+    dict(n=1, c=21, h=6, w=6, cout=21, kh=8, kw=8, stride=(4, 4), pad=(2, 2, 2, 2)),       # ... on a channel-padded copy, two classes of two columns
 ]
 
 
