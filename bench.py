@@ -152,11 +152,11 @@ def fc_workload(eden, synth, m=256, k=4096, n=4096, cold=False):
                 host=(a, w, b, q), out=per_set[0][1], out_shape=(m, n))
 
 
-def conv_workload(eden, synth, n=1, cold=False, cin=64, cout=64, hw=56, k=3, stride=1):
+def conv_workload(eden, synth, n=1, cold=False, cin=64, cout=64, hw=56, k=3, stride=1, dil=1):
     """k x k convolution, ReLU, channels-last: BASELINE configs[0] (3x3, 64 -> 64 channels at 56 x 56) by default"""
-    pad = k // 2
-    ho = (hw + 2 * pad - k) // stride + 1
-    desc = eden.conv_desc(n, cin, hw, hw, cout, k, k, stride=(stride, stride), pad=(pad,) * 4, layout=eden.NHWC)
+    pad = dil * (k - 1) // 2
+    ho = (hw + 2 * pad - dil * (k - 1) - 1) // stride + 1
+    desc = eden.conv_desc(n, cin, hw, hw, cout, k, k, stride=(stride, stride), pad=(pad,) * 4, dil=(dil, dil), layout=eden.NHWC)
     x = synth.fill_u8((n, hw, hw, cin), SEED + 16)
     w = synth.fill_u8((cout, cin, k, k), SEED + 17)
     b = synth.fill_i32((cout,), SEED + 18, -1000, 1000)
@@ -167,7 +167,7 @@ def conv_workload(eden, synth, n=1, cold=False, cin=64, cout=64, hw=56, k=3, str
     sets = set_count(nbytes, cold)
     bufs = [(eden.DeviceBuffer(host=x), eden.DeviceBuffer(nbytes=n * ho * ho * cout)) for _ in range(sets)]
     name = "conv3x3_n%d_c64_56x56_nhwc" % n if (cin, cout, hw, k, stride) == (64, 64, 56, 3, 1) else \
-        "conv%dx%ds%d_n%d_%dto%d_%dx%d_nhwc" % (k, k, stride, n, cin, cout, hw, hw)
+        "conv%dx%ds%d%s_n%d_%dto%d_%dx%d_nhwc" % (k, k, stride, "" if dil == 1 else "d%d" % dil, n, cin, cout, hw, hw)
     return dict(name=name, launch=lambda s, i: plan.run(bufs[i][0], bufs[i][1], q, s),
                 keep=(bufs, d_w, d_b, plan), sets=sets, ops=2.0 * n * ho * ho * cout * cin * k * k, bytes=nbytes,
                 # (which roof is the lower one: the published peaks meet at 5000 / 8 = 625 operations per byte)
@@ -554,9 +554,9 @@ def main():
     if args.only and args.only.startswith("deconv:"):  # deconv:N,CIN,COUT,HW,K,STRIDE = that transposed convolution
         n, cin, cout, hw, k, stride = (int(v) for v in args.only[7:].split(","))
         families[args.only] = shaped(deconv_workload, n=n, cin=cin, cout=cout, hw=hw, k=k, stride=stride)
-    if args.only and args.only.startswith("conv:"):    # conv:N,CIN,COUT,HW,K,STRIDE = that convolution
-        n, cin, cout, hw, k, stride = (int(v) for v in args.only[5:].split(","))
-        families[args.only] = shaped(conv_workload, n=n, cin=cin, cout=cout, hw=hw, k=k, stride=stride)
+    if args.only and args.only.startswith("conv:"):    # conv:N,CIN,COUT,HW,K,STRIDE[,DILATION] = that convolution
+        v = [int(t) for t in args.only[5:].split(",")]
+        families[args.only] = shaped(conv_workload, n=v[0], cin=v[1], cout=v[2], hw=v[3], k=v[4], stride=v[5], dil=v[6] if len(v) > 6 else 1)
     if args.only and args.only.startswith("dw:"):      # dw:N,C,HW,STRIDE[,K[,DILATION]] = that depthwise convolution
         v = [int(t) for t in args.only[3:].split(",")]
         families[args.only] = shaped(dw_workload, n=v[0], c=v[1], hw=v[2], stride=v[3], k=v[4] if len(v) > 4 else 3, dil=v[5] if len(v) > 5 else 1)
