@@ -128,6 +128,10 @@ struct GemmPart {
     int32_t n_period = 0;
     int64_t period_step = 0;
     int32_t *pc_multiplier_rep = nullptr, *pc_shift_rep = nullptr;  // the operator's per-channel pairs, repeated per kernel column
+    // Few output tiles under a long reduction: `slices` workgroups share each tile's reduction (equal runs of slabs) and
+    // leave int32 sums in `partial` [slices][m][n_pad], which a second small launch adds up and requantizes.
+    int32_t slices = 0;
+    int32_t *partial = nullptr;
     GemmConfig cfg;
     int64_t so = 0, sc = 0;   // source weight strides (out channel, in channel)
     int64_t w_base = 0;       // element offset of this part in the source weights
@@ -142,6 +146,7 @@ struct GemmPart {
         dev_free(tap_off);
         dev_free(pc_multiplier_rep);
         dev_free(pc_shift_rep);
+        dev_free(partial);
     }
 };
 
@@ -219,6 +224,22 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         g.cfg = igemm_dma_select(g.proto.m, g.n, g.k, siblings);
     g.k_pad = g.cfg.id == GEMM_ROWS ? g.proto.rows_kh * 32 : round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
     g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
+    g.slices = 0;
+    if (g.cfg.id == GEMM_DMA_64x64_SPLITK && siblings == 1 && g.n_period == 0) {
+        // A launch of at most 64 tiles leaves three quarters of the CUs idle while each tile walks its whole reduction:
+        // from 24 slabs on (6 KiB of reduction), up to four workgroups share a tile's reduction (at least 6 slabs each,
+        // at most about 200 workgroups in all).  The second launch and the trip of the sums through memory cost about
+        // 4 us, which shorter reductions do not win back (18 slabs, 3x3 on 512 channels at 7 x 7, batch 8: 12.0 us
+        // either way; 45 slabs, 3x3 on 1280 channels at 10 x 10: 23.6 -> 14.1 us).
+        const long tiles = (long)((g.proto.m + 63) / 64) * ((g.n + 63) / 64);
+        const int slabs = g.k_pad / g.cfg.slab;
+        int s = 4;
+        while (s > 1 && (slabs < 6 * s || tiles * s > 208)) --s;
+        if (tiles <= 64 && slabs >= 24 && s >= 2) {
+            g.slices = s;
+            g.k_pad = round_up(g.k_pad, g.cfg.slab * s);
+        }
+    }
     KUnit pad;
     pad.offset = 0;
     pad.dy = INT16_MIN;
@@ -230,6 +251,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     if ((rc = dev_alloc(&g.folded, (size_t)g.n_pad))) return rc;
     if ((rc = dev_alloc(&g.ktab, units.size()))) return rc;
     if ((rc = dev_alloc(&g.tap_off, tap_off.size()))) return rc;
+    if (g.slices && (rc = dev_alloc(&g.partial, (size_t)g.slices * g.proto.m * g.n_pad))) return rc;
     if (!g_dry_run) {
         EH_HIP(hipMemcpyAsync(g.ktab, units.data(), units.size() * sizeof(KUnit), hipMemcpyHostToDevice, stream));
         if (!tap_off.empty())
@@ -253,6 +275,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
                      g.cin == g.proto.cin && !units.empty() && units[0].dy == 0 && units[0].dx == 0 && units[0].offset == 0)
                         ? 1
                         : 0;
+    if (g.slices) g.proto.dense = 0;  // slices are cut out of the k-table
     return EH_OK;
 }
 
@@ -495,15 +518,37 @@ struct GemmOp {
         }
         GemmProblem inline_problems[kInlineParts];
         std::vector<GemmProblem> many;
-        if (parts.size() > (size_t)kInlineParts) many.resize(parts.size());
+        size_t launches = 0;
+        for (auto &g : parts) launches += g.slices ? (size_t)g.slices : 1;
+        if (launches > (size_t)kInlineParts) many.resize(launches);
         GemmProblem *const problems = many.empty() ? inline_problems : many.data();
         int filled = 0;
         for (auto &g : parts) {
             EH_REQUIRE((reinterpret_cast<uintptr_t>(in) & (uintptr_t)(g.vec - 1)) == 0,
                        "input pointer is not aligned to %d bytes", g.vec);
-            problems[filled++] = problem(g, in, out, fuse ? residual : nullptr, radd);
+            const GemmProblem whole = problem(g, in, out, fuse ? residual : nullptr, radd);
+            if (g.slices == 0) {
+                problems[filled++] = whole;
+                continue;
+            }
+            // equal runs of slabs, one problem each: its part of the k-table and of every packed row block
+            const int slabs = g.k_pad / g.cfg.slab, run = slabs / g.slices;
+            for (int s = 0; s < g.slices; ++s) {
+                GemmProblem slice = whole;
+                slice.ktab = whole.ktab + (size_t)s * run * (g.cfg.slab / 16);
+                slice.b = whole.b + (size_t)s * run * 1024;
+                slice.b_slabs = slabs;
+                slice.k_pad = run * g.cfg.slab;
+                slice.k = slice.k_pad;
+                slice.partial = g.partial + (size_t)s * whole.m * g.n_pad;
+                slice.partial_ld = g.n_pad;
+                slice.residual = nullptr;
+                problems[filled++] = slice;
+            }
         }
         if ((rc = launch_igemm_batch(problems, filled, stream))) return rc;
+        for (auto &g : parts)
+            if (g.slices && (rc = launch_splitk_finish(problem(g, in, out, fuse ? residual : nullptr, radd), g.partial, g.n_pad, g.slices, stream))) return rc;
         if (layout == EH_NCHW) {
             if ((rc = launch_nhwc2nchw(st_out, static_cast<uint8_t *>(output), in_n, cout, out_hw, stream))) return rc;
         }

@@ -256,8 +256,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
         return ku;
     };
     const int8_t *b_base[B_LOADS];  // uniform: the packed 1 KiB blocks of this wave's weight rows, slab 0
+    // (only the split-reduction tile runs slices of a reduction, whose row blocks lie a whole reduction apart)
+    const int b_block_slabs = (WGK != 1 && p.b_slabs) ? p.b_slabs : k_slabs;
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) b_base[i] = p.b + ((size_t)(n0 / RPB + i * 4 + wave) * k_slabs) * 1024;
+    for (int i = 0; i < B_LOADS; ++i) b_base[i] = p.b + ((size_t)(n0 / RPB + i * 4 + wave) * b_block_slabs) * 1024;
     uint32_t b_voff = lane * 16;    // advances by one block per issued stage
     const uint32_t wave_lds = lds_offset(stages) + (wave << 10);
 
@@ -511,7 +513,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
                         if (aligned16 && n + 16 <= p.n) {
                             *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
                         } else {
-                            store_bytes_any_alignment(dst, packed, p.n - n < 16 ? p.n - n : 16);
+                            if constexpr (BM == 256 && BN == 256) {  // (no registers to spare for the dword form's copies)
+                                const int cnt = p.n - n < 16 ? p.n - n : 16;
+                                for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+                            } else {
+                                store_bytes_any_alignment(dst, packed, p.n - n < 16 ? p.n - n : 16);
+                            }
                         }
                         __builtin_amdgcn_sched_barrier(0);
                     }
@@ -565,6 +572,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
             corr *= p.zw;
         }
         const int32_t *pr = reinterpret_cast<const int32_t *>(stages) + ml * PART_ROW + nl;
+        if (p.partial) {  // a slice of a reduction shared between workgroups: the sums leave as they are
+            int32_t *dst = p.partial + ((size_t)m * (size_t)p.partial_ld + (size_t)n);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                int4 s4 = *reinterpret_cast<const int4 *>(pr + g * 4);
+#pragma unroll
+                for (int w = 1; w < WGK; ++w) {
+                    const int4 t = *reinterpret_cast<const int4 *>(pr + g * 4 + w * BM * PART_ROW);
+                    s4.x += t.x;
+                    s4.y += t.y;
+                    s4.z += t.z;
+                    s4.w += t.w;
+                }
+                *reinterpret_cast<int4 *>(dst + g * 4) = make_int4(s4.x - corr, s4.y - corr, s4.z - corr, s4.w - corr);
+            }
+            return;
+        }
         uint32_t packed[4];
         auto reduce = [&](auto fast_c) {
             constexpr int fast = decltype(fast_c)::value;
@@ -721,7 +745,67 @@ int launch_cfg(const GemmProblem *ps, int count, hipStream_t stream) {
     return EH_OK;
 }
 
+// Adds up the slices of a reduction that several workgroups shared and finishes the outputs: bias, requantization in
+// the reference's own order (the single-shift forms the epilogues use are its equivalents), the residual add, the store.
+// One thread per output pixel and sixteen channels.
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const GemmProblem p, const int32_t *__restrict__ partial, const int partial_ld,
+                                                            const int slices, const int chunks, const FastDiv div_chunks) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    const int m = (int)fastdiv(idx, div_chunks), n = ((int)idx - m * chunks) * 16;
+    if (m >= p.m) return;
+    const size_t slice_stride = (size_t)p.m * (size_t)partial_ld;
+    const int32_t *src = partial + ((size_t)m * (size_t)partial_ld + (size_t)n);
+    const RequantDev rq = p.rq;
+    uint32_t packed[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        int4 v = *reinterpret_cast<const int4 *>(p.bias + n + g * 4);
+        for (int s = 0; s < slices; ++s) {
+            const int4 t = *reinterpret_cast<const int4 *>(src + s * slice_stride + g * 4);
+            v.x += t.x;
+            v.y += t.y;
+            v.z += t.z;
+            v.w += t.w;
+        }
+        uint32_t o0, o1, o2, o3;
+        if (rq.pc_multiplier) {
+            const int4 cm = *reinterpret_cast<const int4 *>(rq.pc_multiplier + n + g * 4), cs = *reinterpret_cast<const int4 *>(rq.pc_shift + n + g * 4);
+            o0 = requant_u8_channel(v.x, cm.x, cs.x, rq), o1 = requant_u8_channel(v.y, cm.y, cs.y, rq);
+            o2 = requant_u8_channel(v.z, cm.z, cs.z, rq), o3 = requant_u8_channel(v.w, cm.w, cs.w, rq);
+        } else {
+            o0 = requant_u8(v.x, rq), o1 = requant_u8(v.y, rq), o2 = requant_u8(v.z, rq), o3 = requant_u8(v.w, rq);
+        }
+        packed[g] = pack_bytes(o0, o1, o2, o3) ^ p.out_xor;
+    }
+    const int cnt = p.n - n < 16 ? p.n - n : 16;
+    const size_t out_off = out_pixel_offset(p, m, p.ho * p.wo) + (size_t)n;
+    if (p.residual) {
+        const uint8_t *res = p.residual + out_off;
+        for (int t = 0; t < cnt; ++t) {
+            const uint32_t v = add_one(res[t], (packed[t >> 2] >> (8 * (t & 3))) & 255u, p.radd);
+            packed[t >> 2] = (packed[t >> 2] & ~(255u << (8 * (t & 3)))) | (v << (8 * (t & 3)));
+        }
+    }
+    uint8_t *dst = p.out + out_off;
+    if (cnt == 16 && (p.ldc & 15) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0)
+        *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    else
+        store_bytes_any_alignment(dst, packed, cnt);
+}
+
 }  // namespace
+
+int launch_splitk_finish(const GemmProblem &p, const int32_t *partial, int32_t partial_ld, int32_t slices, hipStream_t stream) {
+    EH_REQUIRE(partial != nullptr && slices >= 1 && partial_ld >= (p.n + 15) / 16 * 16 && (partial_ld & 3) == 0, "splitk_finish: bad partial image");
+    const int chunks = (p.n + 15) / 16;
+    const long total = (long)p.m * chunks;
+    if (total <= 0) return EH_OK;
+    EH_REQUIRE(total < (1l << 31), "splitk_finish: too many outputs");
+    hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p, partial, partial_ld, slices, chunks,
+                       make_fastdiv((uint32_t)chunks));
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
 
 // Which kernel shape serves an (m, n, k) problem whose activations come in
 // 16-byte channel units.  The packed weight layout depends on the slab, so the

@@ -422,6 +422,13 @@ struct GemmProblem {
     const uint8_t *residual;
     AddDev radd;
     RequantDev rq;
+    // A slice of a reduction that several workgroups share (64 x 64 split-reduction tiles, table-driven): `ktab`, `b`
+    // and `k_pad` describe the slice, `b_slabs` is the whole reduction's slab count (the distance between the packed
+    // weights' row blocks; 0: k_pad / slab), and the tile's int32 sums minus its activation-sum term go to
+    // partial[m * partial_ld + n] instead of being requantized (launch_splitk_finish adds the slices up and does that).
+    int32_t *partial;
+    int32_t partial_ld;
+    int32_t b_slabs;
 };
 
 // Equally shaped problems of one operator that go out as one launch (kernel argument).
@@ -436,6 +443,8 @@ int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream);  // 
 GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k, int32_t siblings);
 inline size_t igemm_dma_ktab_limit() { return 12288; }
 int launch_igemm_thin(const GemmProblem *ps, int count, hipStream_t stream);  // `count` equally shaped problems as one launch
+// p: the whole problem (bias, requantization, output addressing, residual); partial: [slices][p.m][partial_ld] int32
+int launch_splitk_finish(const GemmProblem &p, const int32_t *partial, int32_t partial_ld, int32_t slices, hipStream_t stream);
 int launch_conv_c3k3(const GemmProblem &p, hipStream_t stream);
 int launch_conv3x3_patch(const GemmProblem &p, hipStream_t stream);
 // one tap, few output pixels, long reductions: cut along the weights (eh_gemm_skinny.hip)

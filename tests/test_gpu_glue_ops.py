@@ -113,6 +113,8 @@ RUN_ADD_CASES = [
     dict(n=2, c=576, h=7, w=7, cout=96, kh=1, kw=1, fused=True),
     dict(n=32, c=264, h=28, w=28, cout=256, kh=1, kw=1, fused=False),
     dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2, fused=False, exact=True),
+    # a reduction sliced over workgroups: the launch that adds the slices up adds the residual
+    dict(n=2, c=768, h=7, w=7, cout=72, kh=3, kw=3, pad=(1, 1, 1, 1), fused=True),
     # the same on its channel-padded copy: split-reduction tiles (fused)
     dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2, fused=True),
 ]

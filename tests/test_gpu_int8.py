@@ -48,6 +48,7 @@ CONV_CASES = [
     dict(n=2, c=24, h=9, w=9, cout=40, kh=1, kw=1),                                      # one-tap kernel
     dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, pad=(1, 1, 1, 1), groups=2),          # channel-padded copy (EXACT_CHANNELS: register-staged kernel)
     dict(n=2, c=21, h=9, w=10, cout=21, kh=3, kw=3, pad=(1, 1, 1, 1)),                   # channel-padded copy: int8 padding bytes
+    dict(n=2, c=768, h=7, w=7, cout=200, kh=3, kw=3, pad=(1, 1, 1, 1)),                  # reduction sliced over workgroups
     dict(n=32, c=264, h=28, w=28, cout=256, kh=1, kw=1),                                 # 128 x 128 tiles, no row sums needed? (zp_w != 0: needed)
     dict(n=1, c=200, h=6, w=6, cout=64, kh=3, kw=3, pad=(1, 1, 1, 1)),                   # reduction not a multiple of the slab
 ]
@@ -70,7 +71,7 @@ def test_int8_conv_matches_oracle(case, layout):
         want = O.conv2d_s8(x, w, b, s, oq)
         got = run_conv(eden.ConvPlan, None, x, w, b, s, q, (s.n, s.cout, ho, wo), layout, eden.W_OIHW)
         assert np.array_equal(got, want), int((got != want).sum())
-        assert want.std() > 4
+        assert want.std() > 3   # (the long reductions leave ReLU6 about eight output steps)
 
 
 def test_int8_conv_perchannel_and_symmetric_weights():

@@ -77,6 +77,10 @@ FC_CASES = [
     (8, 300, 10, 200, 9),
     (300, 90, 40, 17, 250),
     (2, 70, 130, 255, 0),
+    # more than 64 rows, few tiles, a long reduction: slices of the reduction on separate workgroups
+    (100, 6400, 200, 77, 201),
+    (70, 6200, 64, 3, 128),
+    (129, 9216, 40, 131, 120),
 ]
 
 
@@ -268,6 +272,13 @@ CONV_CASES = [
     dict(n=1, c=42, h=14, w=9, cout=30, kh=3, kw=2, stride=(2, 1), pad=(1, 0, 1, 1), dil=(1, 2), groups=2),
     dict(n=2, c=30, h=8, w=8, cout=45, kh=1, kw=1, groups=3, stride=(2, 2)),
     dict(n=1, c=17, h=1, w=1, cout=9, kh=1, kw=1),
+    # few 64 x 64 tiles under a reduction of 24 slabs or more: two to four workgroups share each tile's reduction and
+    # a second launch adds their sums up (45 slabs padded to 48 for four slices and 24 channels; 27 slabs and 28 tiles; a
+    # stride and three slices; just below the bound: one workgroup per tile)
+    dict(n=3, c=1280, h=5, w=5, cout=24, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=2, c=768, h=7, w=7, cout=400, kh=3, kw=3, pad=(1, 1, 1, 1)),
+    dict(n=1, c=1024, h=14, w=14, cout=200, kh=3, kw=2, stride=(2, 2), pad=(1, 1, 1, 0)),
+    dict(n=2, c=512, h=7, w=7, cout=512, kh=3, kw=3, pad=(1, 1, 1, 1)),
 ]
 
 
