@@ -257,7 +257,14 @@ __global__ __launch_bounds__(256) void direct_gemm_kernel(const std::conditional
         } else if (wide && cnt == 8) {
             *reinterpret_cast<u32x2_a4 *>(dst) = u32x2_a4{packed[0], packed[1]};
         } else {
-            store_bytes_any_alignment(dst, packed, cnt < 16 ? cnt : 16);
+            // (whole chunks of rows that start at odd addresses: dwords at byte addresses; written out here because the
+            // shared helper's per-dword tests cost the aligned path 2.5 % through register allocation)
+            if (cnt >= 16) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) *reinterpret_cast<u32_any_alignment *>(dst + 4 * g) = packed[g];
+            } else {
+                for (int t = 0; t < cnt; ++t) dst[t] = (uint8_t)(packed[t >> 2] >> (8 * (t & 3)));
+            }
         }
     };
 
