@@ -52,7 +52,7 @@ struct ThinStage {
     int32_t linear;
 };
 
-// one problem, or (BATCHED) up to four equally shaped ones along grid z
+// one problem, or (BATCHED) up to eight equally shaped ones along grid z
 __device__ __forceinline__ const GemmProblem &problem_of(const GemmProblem &one) { return one; }
 __device__ __forceinline__ const GemmProblem &problem_of(const GemmBatch &batch) { return batch.p[blockIdx.z]; }
 

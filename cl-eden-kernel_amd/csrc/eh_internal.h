@@ -433,7 +433,7 @@ struct GemmProblem {
 
 // Equally shaped problems of one operator that go out as one launch (kernel argument).
 struct GemmBatch {
-    static constexpr int MAX = 4;
+    static constexpr int MAX = 8;
     GemmProblem p[MAX];
 };
 int launch_igemm(const GemmProblem &p, hipStream_t stream);

@@ -212,7 +212,7 @@ CONV_CASES = [
     dict(n=2, c=40, h=13, w=13, cout=240, kh=1, kw=1, stride=(2, 2)),                       # two steps, strided rows
     dict(n=2, c=64, h=12, w=12, cout=32, kh=1, kw=1),
     dict(n=1, c=48, h=10, w=10, cout=96, kh=1, kw=1, groups=2),                             # 24-byte rows inside 48-byte pixels
-    dict(n=2, c=240, h=14, w=14, cout=120, kh=1, kw=1, groups=6),                            # six groups: launches of four and two problems
+    dict(n=2, c=240, h=14, w=14, cout=120, kh=1, kw=1, groups=6),                            # six groups: one launch of six problems
     dict(n=5, c=16, h=33, w=5, cout=96, kh=1, kw=1, stride=(1, 2)),
     # ... whose output leaves through the per-wave LDS image: one 16-byte chunk per pixel, the widest pixel (256 bytes),
     # a last pixel block of three pixels
@@ -607,7 +607,7 @@ DECONV_CASES = [
     # kernel <= stride (every phase is one tap) with a negative tail padding: phases larger than the input
     dict(n=2, c=16, h=6, w=6, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, -2, 0, -2)),
     dict(n=2, c=16, h=6, w=6, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, 0, 0, 0)),
-    # nine one-tap phases of equal shape: launches of four, four and one problems of the one-tap kernel
+    # nine one-tap phases of equal shape: launches of eight problems and of one problem of the one-tap kernel
     dict(n=2, c=32, h=9, w=7, cout=48, kh=3, kw=3, stride=(3, 3), pad=(0, 0, 0, 0)),
     dict(n=3, c=64, h=20, w=20, cout=32, kh=2, kw=2, stride=(2, 2), pad=(0, 0, 0, 0)),
     # channels per group that are no multiple of 16, several taps per phase: the channel-padded copy of the input
