@@ -1759,6 +1759,8 @@ int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan
     if (pointwise == nullptr || depthwise == nullptr) return 0;
     const GemmOp &op = pointwise->op;
     if (op.parts.size() != 1 || op.layout != EH_NHWC || op.io_signed) return 0;
+    // (a plan that reads a channel-padded copy of its input, or shares its reduction between workgroups, runs as itself)
+    if (op.pad_cg_to != 0 || op.parts[0].slices != 0) return 0;
     if (depthwise->d.layout != EH_NHWC || depthwise->io_signed) return 0;
     if ((op.pc_multiplier != nullptr) != (depthwise->pc_multiplier != nullptr)) return 0;  // one pair per operator, or one per channel in both
     if (depthwise->d.n != pointwise->d.n || !(depthwise->w_trip || depthwise->w_fold)) return 0;

@@ -155,6 +155,14 @@ def test_block_refuses_what_it_does_not_fit():
     with pytest.raises(eden.EdenHipError):
         eden.conv_dw_block_run(wide, dw, d_x, d_o, q, q)
     wide.destroy()
+    # 21 input channels: that plan runs the one-tap kernel too, but on a channel-padded copy of its input, which the
+    # fused kernel would not read
+    d_w3 = eden.DeviceBuffer(host=synth.fill_u8((64, 21, 1, 1), 4))
+    desc = eden.conv_desc(1, 21, 8, 8, 64, 1, 1, layout=eden.NHWC)
+    assert eden.conv_kernels(desc) == ["one_tap"]
+    ragged = eden.ConvPlan(desc, d_w3, d_b, q)
+    assert not eden.conv_dw_block_applies(ragged, dw)
+    ragged.destroy()
     dw.destroy()
 
 
