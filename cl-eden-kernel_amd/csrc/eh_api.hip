@@ -132,6 +132,10 @@ struct GemmPart {
     // leave int32 sums in `partial` [slices][m][n_pad], which a second small launch adds up and requantizes.
     int32_t slices = 0;
     int32_t *partial = nullptr;
+    // Several convolution groups as one block-diagonal problem (channels per group below 16): `block_cin` input and
+    // `block_n` output channels per group; the entries off the blocks hold the weight zero point, so they are packed
+    // again from the operator's copy of the weights whenever that changes.
+    int32_t block_cin = 0, block_n = 0;
     GemmConfig cfg;
     int64_t so = 0, sc = 0;   // source weight strides (out channel, in channel)
     int64_t w_base = 0;       // element offset of this part in the source weights
@@ -279,7 +283,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     return EH_OK;
 }
 
-int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t stream) {
+int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t stream, int32_t off_block = 0) {
     PackProblem pp;
     pp.w = weight + g.w_base;
     pp.w_signed = w_signed ? 1 : 0;
@@ -297,6 +301,9 @@ int pack_part(GemmPart &g, const uint8_t *weight, bool w_signed, hipStream_t str
     pp.cin_real = g.cin_real;
     pp.n_period = g.n_period;
     pp.period_step = g.period_step;
+    pp.block_cin = g.block_cin;
+    pp.block_n = g.block_n;
+    pp.off_block = off_block;
     pp.so = g.so;
     pp.sc = g.sc;
     pp.tap_off = g.tap_off;
@@ -351,6 +358,10 @@ struct GemmOp {
     // padded problem is the caller's problem exactly.
     int32_t pad_groups = 0, pad_cg = 0, pad_cg_to = 0;
     bool exact_channels = false;  // the caller asked for no padded copy
+    // block-diagonal bundles of groups: the operator's copy of the weights and the zero point they were last packed with
+    uint8_t *w_keep = nullptr;
+    size_t w_keep_bytes = 0;
+    int32_t packed_zp_w = INT32_MIN;
     uint8_t *stage_pad = nullptr;
     // int8 weights (value = byte as signed; zp_w is then an int8 zero point) and one multiplier / shift per
     // output channel instead of the requant's single pair
@@ -402,6 +413,7 @@ struct GemmOp {
         dev_free(stage_in);
         dev_free(stage_out);
         dev_free(stage_pad);
+        dev_free(w_keep);
         dev_free(fillbuf);
         dev_free(pc_multiplier);
         dev_free(pc_shift);
@@ -413,9 +425,18 @@ struct GemmOp {
             int rc = dev_alloc(&fillbuf, 256);
             if (rc) return rc;
         }
-        for (auto &g : parts) {
-            int rc = pack_part(g, static_cast<const uint8_t *>(weight), w_signed, stream);
-            if (rc) return rc;
+        if (w_keep_bytes) {  // packed by refold(), which knows the zero point
+            if (!w_keep) {
+                int rc = dev_alloc(&w_keep, w_keep_bytes);
+                if (rc) return rc;
+            }
+            EH_HIP(hipMemcpyAsync(w_keep, weight, w_keep_bytes, hipMemcpyDeviceToDevice, stream));
+            packed_zp_w = INT32_MIN;
+        } else {
+            for (auto &g : parts) {
+                int rc = pack_part(g, static_cast<const uint8_t *>(weight), w_signed, stream);
+                if (rc) return rc;
+            }
         }
         has_bias = bias != nullptr;  // no bias: the fold kernel takes zeros (no memset, so that a caller may capture this)
         if (bias) EH_HIP(hipMemcpyAsync(bias_copy, bias, (size_t)cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
@@ -429,6 +450,14 @@ struct GemmOp {
         if (folded_valid && nq.zp_in == q.zp_in && nq.zp_w == q.zp_w) {  // (w_signed and io_signed are fixed per plan)
             q = nq;
             return EH_OK;
+        }
+        if (w_keep_bytes && packed_zp_w != zp_w_u8(nq)) {
+            EH_REQUIRE(w_keep != nullptr, "weights were never set");
+            for (auto &g : parts) {
+                int rc = pack_part(g, w_keep, w_signed, stream, zp_w_u8(nq) - 128);
+                if (rc) return rc;
+            }
+            packed_zp_w = zp_w_u8(nq);
         }
         for (auto &g : parts) {
             int rc = launch_fold_bias(has_bias ? bias_copy + g.bias_base : nullptr, g.colsum, g.folded, g.n, g.n_pad, g.k, nq.zp_in, zp_w_u8(nq),
@@ -956,8 +985,8 @@ static bool wants_channel_padding(GemmOp &op, int groups, int channels_per_group
 
 static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t stream) {
     GemmOp &op = pl->op;
-    const int G = d->groups, cog = d->cout / G;
-    int cig = d->c / G;
+    const int G = d->groups;
+    int cig = d->c / G, cog = d->cout / G;
     const int ho = eh_conv_out_dim(d->h, d->pad_t, d->pad_b, d->kh, d->dil_h, d->stride_h);
     const int wo = eh_conv_out_dim(d->w, d->pad_l, d->pad_r, d->kw, d->dil_w, d->stride_w);
     EH_REQUIRE(ho > 0 && wo > 0, "convolution output is empty (%d x %d)", ho, wo);
@@ -978,12 +1007,25 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
     const bool padded = op.pad_cg_to != 0;
     if (padded) cig = op.pad_cg_to;
     const int pixel_c = padded ? G * cig : d->c;
-    op.parts.resize(G);
-    for (int g = 0; g < G; ++g) {
+    // Groups of fewer than 16 channels each (ResNeXt-style 3x3 layers): `bundle` neighbouring groups run as one
+    // block-diagonal problem over their 16 .. 64 adjacent channels, read in 16-byte units straight from the tensor,
+    // instead of one small problem per group on a padded copy.
+    int bundle = 1;
+    if (G > 1 && !padded && !op.exact_channels && (cig & 15) != 0 && d->weight_layout == EH_W_OIHW)
+        for (int b = G; b >= 2 && bundle == 1; --b)
+            if (G % b == 0 && b * cig <= 64 && ((b * cig) & 15) == 0) bundle = b;
+    op.w_keep_bytes = bundle > 1 ? (size_t)d->cout * cig * taps : 0;
+    const int parts_n = G / bundle;
+    cig *= bundle;
+    cog *= bundle;
+    op.parts.resize(parts_n);
+    for (int g = 0; g < parts_n; ++g) {
         GemmPart &part = op.parts[g];
         part.n = cog;
         part.cin = cig;
         part.cin_real = padded ? cig_real : 0;
+        part.block_cin = bundle > 1 ? cig / bundle : 0;
+        part.block_n = bundle > 1 ? cog / bundle : 0;
         part.taps = taps;
         part.k = taps * cig;
         part.vec = pick_vec(cig, pixel_c);
@@ -1026,7 +1068,7 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
         p.out_y0 = 0;
         p.out_x0 = 0;
         p.ldc = d->cout;
-        if ((rc = finish_part(part, units, tap_off, stream, std::min(G, (int)GemmBatch::MAX)))) return rc;
+        if ((rc = finish_part(part, units, tap_off, stream, std::min(parts_n, (int)GemmBatch::MAX)))) return rc;
     }
     if (wants_channel_padding(op, G, cig_real)) return conv_plan_build(pl, d, stream);
     return op.alloc_staging();

@@ -494,6 +494,11 @@ struct PackProblem {
     // that share a launch, and its source index is (o % n_period)*so + (o / n_period)*period_step + c*sc + tap_off[t]
     int32_t n_period;
     int64_t period_step;
+    // block_cin != 0: several convolution groups as one block-diagonal problem.  Packed row o belongs to group
+    // o / block_n of the bundle and reduction channel c to group c / block_cin; where the two differ the row holds
+    // `off_block` (the weight zero point minus 128, so that the product with any activation is zero), elsewhere
+    // source channel c % block_cin.
+    int32_t block_cin, block_n, off_block;
     const int32_t *tap_off;  // device [taps]
 };
 int launch_pack_weights(const PackProblem &p, hipStream_t stream);

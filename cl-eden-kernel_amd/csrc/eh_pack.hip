@@ -23,7 +23,14 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const PackProblem p) 
         const int kk = p.row_bytes ? ((k & 31) < p.row_bytes ? (k >> 5) * p.row_bytes + (k & 31) : p.k) : k;
         if (o < p.n && kk < p.k) {
             const int t = kk / p.cin, c = kk - t * p.cin;
-            if (p.cin_real == 0 || c < p.cin_real) {
+            if (p.block_cin) {
+                if (c / p.block_cin == o / p.block_n) {
+                    const uint8_t raw = p.w[(int64_t)o * p.so + (int64_t)(c % p.block_cin) * p.sc + p.tap_off[t]];
+                    v = p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw - 128;
+                } else {
+                    v = p.off_block;
+                }
+            } else if (p.cin_real == 0 || c < p.cin_real) {
                 const int64_t row = p.n_period ? (int64_t)(o % p.n_period) * p.so + (int64_t)(o / p.n_period) * p.period_step : (int64_t)o * p.so;
                 const uint8_t raw = p.w[row + (int64_t)c * p.sc + p.tap_off[t]];
                 v = p.w_signed ? (int32_t)(int8_t)raw : (int32_t)raw - 128;

@@ -223,6 +223,17 @@ def test_ragged_channel_counts_run_on_a_padded_copy_unless_told_otherwise():
     assert eden.conv_kernels(eden.conv_desc(1, 3, 64, 64, 32, 3, 3, layout=nhwc)) == ["c3k3"]
 
 
+def test_small_groups_are_bundled_into_block_diagonal_problems():
+    nhwc = eden.NHWC
+    # 32 groups of 4 channels: two problems over 64 adjacent channels each; 8 groups of 8: one; EXACT_CHANNELS: one per group
+    assert len(eden.conv_kernels(eden.conv_desc(8, 128, 56, 56, 128, 3, 3, pad=(1, 1, 1, 1), groups=32, layout=nhwc))) == 2
+    assert len(eden.conv_kernels(eden.conv_desc(8, 64, 28, 28, 64, 3, 3, pad=(1, 1, 1, 1), groups=8, layout=nhwc))) == 1
+    assert len(eden.conv_kernels(eden.conv_desc(8, 128, 56, 56, 128, 3, 3, pad=(1, 1, 1, 1), groups=32, layout=nhwc | eden.EXACT_CHANNELS))) == 32
+    # groups of 16 channels or more run one problem each, as before
+    assert len(eden.conv_kernels(eden.conv_desc(8, 512, 14, 14, 512, 3, 3, pad=(1, 1, 1, 1), groups=32, layout=nhwc))) == 32
+    assert "staged" not in eden.conv_kernels(eden.conv_desc(8, 128, 56, 56, 128, 3, 3, pad=(1, 1, 1, 1), groups=32, layout=nhwc))
+
+
 def test_classifier_heads_take_the_kernel_cut_along_the_weights():
     nhwc = eden.NHWC
     assert eden.conv_kernels(eden.conv_desc(1, 1280, 1, 1, 1000, 1, 1, layout=nhwc)) == ["skinny"]

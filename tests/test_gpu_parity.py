@@ -272,6 +272,14 @@ CONV_CASES = [
     dict(n=1, c=42, h=14, w=9, cout=30, kh=3, kw=2, stride=(2, 1), pad=(1, 0, 1, 1), dil=(1, 2), groups=2),
     dict(n=2, c=30, h=8, w=8, cout=45, kh=1, kw=1, groups=3, stride=(2, 2)),
     dict(n=1, c=17, h=1, w=1, cout=9, kh=1, kw=1),
+    # groups of fewer than 16 channels: neighbouring groups as block-diagonal problems over 16 .. 64 adjacent channels
+    # (32 groups of 4 -> two bundles of 16; 8 of 8 -> one bundle; 6 groups of 8 -> three bundles of 2; 12 of 4 with a
+    # stride and dilation; 1x1 with 4 channels per group and 3 outputs per group)
+    dict(n=2, c=128, h=14, w=14, cout=128, kh=3, kw=3, pad=(1, 1, 1, 1), groups=32),
+    dict(n=1, c=64, h=9, w=11, cout=96, kh=3, kw=3, pad=(1, 1, 1, 1), groups=8),
+    dict(n=2, c=48, h=10, w=10, cout=24, kh=3, kw=3, pad=(1, 0, 0, 1), groups=6),
+    dict(n=1, c=48, h=13, w=12, cout=48, kh=3, kw=2, stride=(2, 1), pad=(2, 2, 1, 1), dil=(2, 1), groups=12),
+    dict(n=3, c=32, h=6, w=6, cout=24, kh=1, kw=1, groups=8),
     # few 64 x 64 tiles under a reduction of 24 slabs or more: two to four workgroups share each tile's reduction and
     # a second launch adds their sums up (45 slabs padded to 48 for four slices and 24 channels; 27 slabs and 28 tiles; a
     # stride and three slices; just below the bound: one workgroup per tile)
@@ -666,6 +674,38 @@ def test_channel_padded_plan_follows_the_input_zero_point():
         got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
         want = O.conv2d(x, w, b, s, q)
         assert np.array_equal(got, want), diff_report(got, want)
+    plan.destroy()
+
+
+def test_bundled_groups_follow_the_weight_zero_point():
+    """Groups bundled into block-diagonal problems hold the weight zero point off their blocks: one plan, run with
+    three weight zero points (packed again each time), and once more after its weights were replaced."""
+    s = O.conv_shape(2, 64, 12, 10, 64, 3, 3, pad=(1, 1, 1, 1), groups=16)
+    x, w, b = conv_tensors(s, SEED + 888)
+    ho, wo = O.conv_out_hw(s)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 16, 1, eden.NHWC, eden.W_OIHW)
+    assert len(eden.conv_kernels(desc)) == 1   # sixteen groups, one problem
+    d_x = eden.DeviceBuffer(host=np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+    d_w, d_b, d_o = eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b), eden.DeviceBuffer(nbytes=s.n * s.cout * ho * wo)
+
+    def q_for(weights, zp_w):
+        _, acc = O.conv2d(x, weights, b, s, O.raw_quant(zp_in=131, zp_w=zp_w), want_acc=True)
+        return centred_quant(acc, 131, zp_w)
+    plan = eden.ConvPlan(desc, d_w, d_b, to_eh_requant(q_for(w, 120)))
+    for zp_w in (120, 7, 255, 120):
+        q = q_for(w, zp_w)
+        plan.run(d_x, d_o, to_eh_requant(q))
+        got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+        want = O.conv2d(x, w, b, s, q)
+        assert np.array_equal(got, want), (zp_w, diff_report(got, want))
+        assert want.std() > 10
+    w2 = synth.fill_u8(w.shape, SEED + 889)
+    d_w2 = eden.DeviceBuffer(host=w2)
+    q = q_for(w2, 33)
+    plan.repack(d_w2, d_b, to_eh_requant(q))
+    plan.run(d_x, d_o, to_eh_requant(q))
+    got = d_o.download((s.n, ho, wo, s.cout)).transpose(0, 3, 1, 2)
+    assert np.array_equal(got, O.conv2d(x, w2, b, s, q))
     plan.destroy()
 
 

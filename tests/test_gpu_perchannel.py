@@ -61,6 +61,7 @@ PC_CASES = [
     dict(n=1, c=20, h=8, w=8, cout=12, kh=3, kw=3, groups=2),                            # channel-padded copy (EXACT_CHANNELS: register-staged kernel), groups
     dict(n=2, c=21, h=9, w=10, cout=21, kh=3, kw=3, pad=(1, 1, 1, 1)),                   # channel-padded copy, patch kernel
     dict(n=2, c=768, h=7, w=7, cout=200, kh=3, kw=3, pad=(1, 1, 1, 1)),                  # reduction sliced over workgroups
+    dict(n=2, c=64, h=10, w=10, cout=64, kh=3, kw=3, pad=(1, 1, 1, 1), groups=16),       # block-diagonal bundle of 16 groups
     dict(n=4, c=264, h=28, w=28, cout=256, kh=1, kw=1),                                  # few tiles: reduction split over waves
     dict(n=32, c=264, h=28, w=28, cout=256, kh=1, kw=1),                                 # 128 x 128 tiles
     dict(n=33, c=68, h=28, w=28, cout=64, kh=1, kw=1),                                   # 128 x 64 tiles
