@@ -61,8 +61,10 @@ typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh
  * length) are no multiple of 16 and fit none of the kernels for few channels copies the input, on every run, into an
  * image of its own with each group padded to the next multiple of 16 (the role of the reference's pad-and-align pass,
  * gpu/operators/cl_kernels/PadConvertKernels.cpp:25-167) and runs the wide-load kernels on that; with it, the
- * byte-gathering kernel reads the caller's tensor directly: several times slower, no staging memory.  Results are
- * the same bytes either way. */
+ * byte-gathering kernel reads the caller's tensor directly: several times slower, no staging memory.  The flag also
+ * keeps convolution groups of fewer than 16 channels as one problem per group; without it neighbouring groups run in
+ * bundles as block-diagonal problems over 16 to 64 adjacent channels, for which the plan keeps a copy of the
+ * weights (it packs them again when a run brings another weight zero point).  Results are the same bytes either way. */
 #define EH_EXACT_CHANNELS 0x400
 
 /* Integer requantization parameters of one operator execution: what
