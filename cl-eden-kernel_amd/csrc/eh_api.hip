@@ -638,6 +638,13 @@ struct eh_dwconv_plan {
     bool range_known = false;   // w_lo / w_hi hold the extremes of the weight bytes (in the caller's own domain)
     int32_t w_lo = 0, w_hi = 0;
     bool trip_valid = false;    // w_trip / bias_trip match the current zero points
+    // Staging.  `d` describes what the kernels run: channels-last tensors with depth multiplier 1.  A caller's depth
+    // multiplier m > 1 (channels-last) is met by a copy of the input with every channel m times in a row, so that
+    // output channel j reads channel j of the copy; a caller's planar tensors (multiplier 1) by the two transpositions
+    // the convolution plans use.  Both only where the output channels are a multiple of 4 (the four-channel kernels).
+    int32_t rep_c = 0, rep_dm = 0;  // the caller's channel count and depth multiplier when the input is replicated
+    bool planar = false;            // the caller's tensors are NCHW
+    uint8_t *stage_in = nullptr, *stage_out = nullptr;
 };
 
 extern "C" {
@@ -1566,6 +1573,8 @@ static void dw_release(eh_dwconv_plan *pl) {
     dev_free(pl->bias_fold);
     dev_free(pl->w_foldk);
     dev_free(pl->bias_foldk);
+    dev_free(pl->stage_in);
+    dev_free(pl->stage_out);
 }
 
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
@@ -1623,9 +1632,10 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     *plan = nullptr;
     EH_REQUIRE(desc != nullptr, "descriptor is null");
     const bool w_signed = (desc->weight_layout & EH_W_SIGNED) != 0, io_signed = (desc->layout & EH_IO_SIGNED) != 0;
+    const bool no_staging = (desc->layout & EH_EXACT_CHANNELS) != 0;
     eh_conv_desc plain = *desc;
     plain.weight_layout &= ~EH_W_SIGNED;
-    plain.layout &= ~(EH_IO_SIGNED | EH_EXACT_CHANNELS);  // (the second flag has no meaning for a depthwise plan)
+    plain.layout &= ~(EH_IO_SIGNED | EH_EXACT_CHANNELS);
     desc = &plain;
     int rc = check_desc_common(desc);
     if (rc) return rc;
@@ -1639,6 +1649,18 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     eh_dwconv_plan *pl = new (std::nothrow) eh_dwconv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
+    if (!no_staging && (desc->cout & 3) == 0 && desc->n > 0) {
+        if (desc->layout == EH_NHWC && desc->depth_multiplier > 1) {
+            pl->rep_c = desc->c;
+            pl->rep_dm = desc->depth_multiplier;
+            pl->d.c = desc->cout;
+            pl->d.depth_multiplier = 1;
+        } else if (desc->layout == EH_NCHW && desc->depth_multiplier == 1) {
+            pl->planar = true;
+            pl->d.layout = EH_NHWC;
+        }
+    }
+    desc = &pl->d;
     pl->w_signed = w_signed;
     pl->io_signed = io_signed;
     pl->ho = eh_conv_out_dim(desc->h, desc->pad_t, desc->pad_b, desc->kh, desc->dil_h, desc->stride_h);
@@ -1652,6 +1674,8 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     }
     hipStream_t s = as_stream(stream);
     rc = dev_alloc(&pl->w_copy, (size_t)pl->cout * pl->taps);
+    if (!rc && (pl->rep_dm || pl->planar)) rc = dev_alloc(&pl->stage_in, (size_t)desc->n * desc->h * desc->w * pl->cout + 256);
+    if (!rc && pl->planar) rc = dev_alloc(&pl->stage_out, (size_t)desc->n * pl->ho * pl->wo * pl->cout + 256);
     if (!rc) rc = dev_alloc(&pl->bias_copy, (size_t)pl->cout);
     if (!rc) rc = dev_alloc(&pl->w_pair, (size_t)((pl->taps + 1) / 2) * pl->cout);
     if (!rc) rc = dev_alloc(&pl->bias_folded, (size_t)pl->cout + 4);
@@ -1782,6 +1806,14 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     EH_REQUIRE(input != nullptr && output != nullptr, "input/output pointer is null");
     hipStream_t s = as_stream(stream);
     if ((rc = dw_refold(plan, *q, s))) return rc;
+    if (plan->rep_dm) {
+        if ((rc = launch_replicate_channels(static_cast<const uint8_t *>(input), plan->stage_in, (int64_t)d.n * d.h * d.w, plan->rep_c, plan->rep_dm, s))) return rc;
+        input = plan->stage_in;
+    } else if (plan->planar) {
+        if ((rc = launch_nchw2nhwc(static_cast<const uint8_t *>(input), plan->stage_in, d.n, d.c, d.h * d.w, s))) return rc;
+        if ((rc = launch_dwconv_nhwc(dw_problem(plan, plan->stage_in, plan->stage_out), s))) return rc;
+        return launch_nhwc2nchw(plan->stage_out, static_cast<uint8_t *>(output), d.n, plan->cout, plan->ho * plan->wo, s);
+    }
     const DwProblem p = dw_problem(plan, input, output);
     return d.layout == EH_NHWC ? launch_dwconv_nhwc(p, s) : launch_dwconv_nchw(p, s);
 }
@@ -1803,7 +1835,7 @@ int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan
     if (op.parts.size() != 1 || op.layout != EH_NHWC || op.io_signed) return 0;
     // (a plan that reads a channel-padded copy of its input, or shares its reduction between workgroups, runs as itself)
     if (op.pad_cg_to != 0 || op.parts[0].slices != 0) return 0;
-    if (depthwise->d.layout != EH_NHWC || depthwise->io_signed) return 0;
+    if (depthwise->d.layout != EH_NHWC || depthwise->io_signed || depthwise->rep_dm || depthwise->planar) return 0;
     if ((op.pc_multiplier != nullptr) != (depthwise->pc_multiplier != nullptr)) return 0;  // one pair per operator, or one per channel in both
     if (depthwise->d.n != pointwise->d.n || !(depthwise->w_trip || depthwise->w_fold)) return 0;
     // geometry and kernel family are checked on the problems themselves; the pointers and parameters of a run do not enter

@@ -554,6 +554,8 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &dw, int rows_per_t
 
 // ---------------------------------------------------------------- layout
 int launch_nchw2nhwc(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);
+// dst[pixel][c * times + d] = src[pixel][c] for d < times (c * times a multiple of 4)
+int launch_replicate_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c, int32_t times, hipStream_t stream);
 // dst[pixel][g][0 .. cg_to) = src[pixel][g][0 .. cg) followed by cg_to - cg bytes `fill`, for `groups` channel groups per pixel
 int launch_pad_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t groups, int32_t cg, int32_t cg_to, uint32_t fill,
                         hipStream_t stream);

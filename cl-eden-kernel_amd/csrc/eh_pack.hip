@@ -81,6 +81,22 @@ __global__ __launch_bounds__(256) void pad_channels_kernel(const uint8_t *__rest
     reinterpret_cast<uint32_t *>(dst)[idx] = v;
 }
 
+// Every channel `times` times in a row: what a depthwise convolution with a depth multiplier reads, laid out so that
+// output channel j reads input channel j of the copy (DepthwiseconvolutionKernels.cpp:1242-1321 indexes the input by
+// out_channel / depth_multiplier instead).  One thread per destination dword.
+__global__ __launch_bounds__(256) void replicate_channels_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, const uint32_t total,
+                                                                 const uint32_t quads_per_pixel, const FastDiv div_quads, const int32_t c,
+                                                                 const FastDiv div_times) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t pixel = fastdiv(idx, div_quads), quad = idx - pixel * quads_per_pixel;
+    const uint8_t *s = src + (size_t)pixel * (size_t)c;
+    uint32_t v = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) v |= (uint32_t)s[fastdiv(quad * 4u + (uint32_t)b, div_times)] << (8 * b);
+    reinterpret_cast<uint32_t *>(dst)[idx] = v;
+}
+
 // Byte-matrix transpose per batch: src [batch][R][S] -> dst [batch][S][R].
 // 64x64 tiles through LDS; 4-byte global accesses when the extents allow.
 constexpr int TT = 64;
@@ -305,6 +321,17 @@ int launch_transpose(const uint8_t *src, uint8_t *dst, int32_t batch, int32_t R,
 }
 
 }  // namespace
+
+int launch_replicate_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c, int32_t times, hipStream_t stream) {
+    EH_REQUIRE(c > 0 && times > 0 && ((c * times) & 3) == 0, "replicate_channels: bad extents %d x %d", c, times);
+    const int64_t total = pixels * (c * times >> 2);
+    if (total <= 0) return EH_OK;
+    EH_REQUIRE(total < (1ll << 31), "replicate_channels: tensor too large");
+    hipLaunchKernelGGL(replicate_channels_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, dst, (uint32_t)total,
+                       (uint32_t)(c * times >> 2), make_fastdiv((uint32_t)(c * times >> 2)), c, make_fastdiv((uint32_t)times));
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
 
 int launch_pad_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t groups, int32_t cg, int32_t cg_to, uint32_t fill,
                         hipStream_t stream) {

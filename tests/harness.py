@@ -52,10 +52,11 @@ def gpu_conv(x_nchw, w, bias, s, q, layout=eden.NCHW, weight_layout=eden.W_OIHW,
 
 
 def gpu_dwconv(x_nchw, w, bias, s, q, layout=eden.NCHW):
+    flags, layout = layout & ~0xFF, layout & 0xFF   # (eden.EXACT_CHANNELS: no staging images)
     ho, wo = O.conv_out_hw(s)
     cout = s.c * max(s.dm, 1)
     desc = eden.conv_desc(s.n, s.c, s.h, s.w, cout, s.kh, s.kw, (s.stride_h, s.stride_w),
-                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), 1, max(s.dm, 1), layout, eden.W_OIHW)
+                          (s.pad_t, s.pad_b, s.pad_l, s.pad_r), (s.dil_h, s.dil_w), 1, max(s.dm, 1), layout | flags, eden.W_OIHW)
     x_dev = x_nchw if layout == eden.NCHW else x_nchw.transpose(0, 2, 3, 1)
     d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), (eden.DeviceBuffer(host=bias) if bias is not None else None)
     d_o = eden.DeviceBuffer(nbytes=s.n * cout * ho * wo)

@@ -509,12 +509,26 @@ DW_CASES = [
     dict(n=1, c=12, h=9, w=30, cout=12, kh=3, kw=3, pad=(0, 3, 1, 0), dil=(2, 2)),
     dict(n=1, c=4, h=40, w=41, cout=4, kh=3, kw=3, pad=(12, 12, 12, 12), dil=(12, 12)),
     dict(n=3, c=384, h=33, w=33, cout=384, kh=3, kw=3, pad=(2, 2, 2, 2), dil=(2, 2)),
+    # depth multipliers on a copy of the input with every channel repeated (channels-last, outputs a multiple of 4)
+    dict(n=2, c=16, h=14, w=13, cout=32, kh=3, kw=3, pad=(1, 1, 1, 1), dm=2),
+    dict(n=1, c=3, h=21, w=20, cout=24, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1), dm=8),
+    dict(n=2, c=5, h=9, w=9, cout=20, kh=5, kw=5, pad=(2, 2, 2, 2), dm=4),
+    dict(n=1, c=6, h=8, w=8, cout=18, kh=3, kw=3, pad=(1, 1, 1, 1), dm=3),                  # 18 outputs: no multiple of 4, one output per thread
 ]
 
 
-@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("layout", [eden.NCHW, eden.NHWC, eden.NCHW | eden.EXACT_CHANNELS, eden.NHWC | eden.EXACT_CHANNELS],
+                         ids=["nchw", "nhwc", "nchw_unstaged", "nhwc_unstaged"])
 @pytest.mark.parametrize("case", DW_CASES, ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
 def test_depthwise_matches_oracle(case, layout):
+    """Planar tensors run between two transpositions and depth multipliers on a channel-replicated copy of the input;
+    EXACT_CHANNELS keeps both on the one-output-per-thread kernels (the `unstaged` runs, where that differs)."""
+    if layout & eden.EXACT_CHANNELS and case["cout"] % 4 != 0:
+        pytest.skip("no staging either way")
+    if layout == (eden.NHWC | eden.EXACT_CHANNELS) and case.get("dm", 1) == 1:
+        pytest.skip("no staging either way")
+    if layout == (eden.NCHW | eden.EXACT_CHANNELS) and case.get("dm", 1) != 1:
+        pytest.skip("no staging either way")
     print("dw", case, layout, flush=True)
     s = O.conv_shape(**case)
     x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 40)
