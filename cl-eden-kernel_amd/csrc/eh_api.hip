@@ -186,6 +186,11 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
                 int siblings = 1) {
     // the kernel shape is fixed here because the packed weight layout depends on it
     g.cfg = GemmConfig();
+    // a plain matrix: one tap at the pixel itself, unit stride, no padding (the tiled kernels then need no k-table)
+    const bool plain_matrix = g.taps == 1 && g.proto.stride_h == 1 && g.proto.stride_w == 1 && g.proto.y_base == 0 && g.proto.x_base == 0 &&
+                              g.proto.ho == g.proto.h && g.proto.wo == g.proto.w && g.vec == 16 && g.cin == g.proto.cin && !units.empty() &&
+                              units[0].dy == 0 && units[0].dx == 0 && units[0].offset == 0;
+    const bool ktab_fits = (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit();
     if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 &&
         igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base, g.proto.m, g.n) &&
         // the one-tap kernel does not test its pixel against the image: every output pixel's tap must lie inside
@@ -224,8 +229,18 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         // 3x3 taps at dilation 1 and stride 1 over all input channels: the patch-in-LDS kernel
         g.cfg.id = GEMM_CONV3X3;
         g.cfg.slab = 32;
-    } else if (g.vec == 16 && (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit())
+    } else if (g.vec == 16 && (ktab_fits || (plain_matrix && g.k % 256 == 0)))
+        // (a reduction too long for its k-table to fit LDS still runs as a plain matrix of whole slabs: a fully
+        // connected layer on 25088 inputs)
         g.cfg = igemm_dma_select(g.proto.m, g.n, g.k, siblings);
+    bool must_slice = false;
+    if (g.cfg.id == GEMM_STAGED && g.vec == 16 && !ktab_fits && siblings == 1 && g.n_period == 0) {
+        // table-driven and too long for one k-table (a 7x7 convolution over 512 channels): the split-reduction tiles
+        // with the reduction sliced, each slice under its own part of the table -- if few enough slices do it (below)
+        g.cfg.id = GEMM_DMA_64x64_SPLITK;
+        g.cfg.slab = 256;
+        must_slice = true;
+    }
     g.k_pad = g.cfg.id == GEMM_ROWS ? g.proto.rows_kh * 32 : round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
     g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
     g.slices = 0;
@@ -237,9 +252,26 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         // either way; 45 slabs, 3x3 on 1280 channels at 10 x 10: 23.6 -> 14.1 us).
         const long tiles = (long)((g.proto.m + 63) / 64) * ((g.n + 63) / 64);
         const int slabs = g.k_pad / g.cfg.slab;
+        // (a slice is table-driven: its part of the k-table has to fit)
+        auto table_fits = [&](int n_slices) {
+            return (size_t)(round_up(slabs, n_slices) / n_slices) * (g.cfg.slab / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit();
+        };
         int s = 4;
-        while (s > 1 && (slabs < 6 * s || tiles * s > 208)) --s;
-        if (tiles <= 64 && slabs >= 24 && s >= 2) {
+        if (must_slice) {
+            // as few slices as fit their tables and a launch batch; the sums of all slices within 256 MiB
+            s = 2;
+            while (s <= GemmBatch::MAX && !table_fits(s)) ++s;
+            if (s > GemmBatch::MAX || (size_t)s * g.proto.m * g.n_pad * 4 > ((size_t)256 << 20)) {
+                s = 0;
+                g.cfg = GemmConfig();  // the register-staged kernel after all
+                g.k_pad = round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
+                g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
+            }
+        } else {
+            while (s > 1 && (slabs < 6 * s || tiles * s > 208)) --s;
+            if (!(tiles <= 64 && slabs >= 24 && s >= 2 && table_fits(s))) s = 0;
+        }
+        if (s >= 2) {
             g.slices = s;
             g.k_pad = round_up(g.k_pad, g.cfg.slab * s);
         }
@@ -274,11 +306,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     g.proto.div_wo = make_fastdiv((uint32_t)g.proto.wo);
     // a plain matrix: one tap at the pixel itself, unit stride, no padding, whole slabs
     // (a reduction that ends inside its last slab is handled by the kernel: the chunks past the end read a constant)
-    g.proto.dense = (g.taps == 1 && g.proto.stride_h == 1 && g.proto.stride_w == 1 && g.proto.y_base == 0 &&
-                     g.proto.x_base == 0 && g.proto.ho == g.proto.h && g.proto.wo == g.proto.w && g.vec == 16 &&
-                     g.cin == g.proto.cin && !units.empty() && units[0].dy == 0 && units[0].dx == 0 && units[0].offset == 0)
-                        ? 1
-                        : 0;
+    g.proto.dense = plain_matrix ? 1 : 0;
     if (g.slices) g.proto.dense = 0;  // slices are cut out of the k-table
     return EH_OK;
 }

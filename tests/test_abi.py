@@ -234,6 +234,12 @@ def test_small_groups_are_bundled_into_block_diagonal_problems():
     assert "staged" not in eden.conv_kernels(eden.conv_desc(8, 128, 56, 56, 128, 3, 3, pad=(1, 1, 1, 1), groups=32, layout=nhwc))
 
 
+def test_reductions_beyond_one_k_table_stay_on_the_tiled_kernels():
+    nhwc = eden.NHWC
+    assert eden.conv_kernels(eden.conv_desc(8, 512, 7, 7, 4096, 7, 7, layout=nhwc)) == ["dma_64x64_splitk"]     # sliced
+    assert eden.conv_kernels(eden.conv_desc(64, 25088, 1, 1, 4096, 1, 1, layout=nhwc))[0].startswith("dma_")   # a plain matrix needs no table
+
+
 def test_classifier_heads_take_the_kernel_cut_along_the_weights():
     nhwc = eden.NHWC
     assert eden.conv_kernels(eden.conv_desc(1, 1280, 1, 1, 1000, 1, 1, layout=nhwc)) == ["skinny"]

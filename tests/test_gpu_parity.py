@@ -81,6 +81,12 @@ FC_CASES = [
     (100, 6400, 200, 77, 201),
     (70, 6200, 64, 3, 128),
     (129, 9216, 40, 131, 120),
+    # a reduction whose k-table would not fit LDS: as a plain matrix of whole slabs (and sliced, each slice with its
+    # part of the table); as a table-driven problem it cannot run on the tiled kernels (the last case: ragged length)
+    (40, 25088, 72, 131, 120),
+    (70, 25088, 130, 3, 128),
+    (300, 25088, 64, 77, 201),
+    (66, 25000, 40, 5, 100),
 ]
 
 
@@ -280,6 +286,10 @@ CONV_CASES = [
     dict(n=2, c=48, h=10, w=10, cout=24, kh=3, kw=3, pad=(1, 0, 0, 1), groups=6),
     dict(n=1, c=48, h=13, w=12, cout=48, kh=3, kw=2, stride=(2, 1), pad=(2, 2, 1, 1), dil=(2, 1), groups=12),
     dict(n=3, c=32, h=6, w=6, cout=24, kh=1, kw=1, groups=8),
+    # a table-driven reduction too long for one k-table (7x7 over 512 channels: a fully connected layer written as a
+    # convolution): sliced, each slice under its part of the table
+    dict(n=2, c=512, h=7, w=7, cout=72, kh=7, kw=7),
+    dict(n=1, c=512, h=9, w=8, cout=40, kh=7, kw=7, pad=(1, 0, 0, 1)),
     # few 64 x 64 tiles under a reduction of 24 slabs or more: two to four workgroups share each tile's reduction and
     # a second launch adds their sums up (45 slabs padded to 48 for four slices and 24 channels; 27 slabs and 28 tiles; a
     # stride and three slices; just below the bound: one workgroup per tile)
