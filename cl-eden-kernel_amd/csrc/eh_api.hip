@@ -182,16 +182,21 @@ static bool units_are_rows(const std::vector<KUnit> &units, int per_tap, int tap
 
 // Allocates a part's device arrays and uploads its tables.  `units` holds one
 // KUnit per `vec` bytes of the real reduction length; padding units are added here.
+// k_floor > 0: the part is one of several whose reductions differ in length and that should share a launch: its
+// reduction is padded to k_floor (the padding units read a constant that multiplies to zero) and only the tiled
+// kernels are considered, so that every sibling gets the same configuration.
 int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream,
-                int siblings = 1) {
+                int siblings = 1, int k_floor = 0) {
     // the kernel shape is fixed here because the packed weight layout depends on it
     g.cfg = GemmConfig();
+    const bool equalize = k_floor > 0;
+    const int k_len = g.k > k_floor ? g.k : k_floor;
     // a plain matrix: one tap at the pixel itself, unit stride, no padding (the tiled kernels then need no k-table)
     const bool plain_matrix = g.taps == 1 && g.proto.stride_h == 1 && g.proto.stride_w == 1 && g.proto.y_base == 0 && g.proto.x_base == 0 &&
                               g.proto.ho == g.proto.h && g.proto.wo == g.proto.w && g.vec == 16 && g.cin == g.proto.cin && !units.empty() &&
                               units[0].dy == 0 && units[0].dx == 0 && units[0].offset == 0;
-    const bool ktab_fits = (size_t)(round_up(g.k > 0 ? g.k : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit();
-    if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 &&
+    const bool ktab_fits = (size_t)(round_up(k_len > 0 ? k_len : 1, 256) / 16) * sizeof(KUnit) <= igemm_dma_ktab_limit();
+    if (!equalize && !units.empty() && units[0].dy == 0 && units[0].dx == 0 &&
         igemm_thin_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.y_base, g.proto.x_base, g.proto.m, g.n) &&
         // the one-tap kernel does not test its pixel against the image: every output pixel's tap must lie inside
         // (bottom / right padding of a 1x1 convolution, or a deconvolution phase enlarged by a negative tail padding,
@@ -199,19 +204,19 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         (g.proto.ho - 1) * g.proto.stride_h < g.proto.h && (g.proto.wo - 1) * g.proto.stride_w < g.proto.w) {
         g.cfg.id = GEMM_THIN;
         g.cfg.slab = 32;
-    } else if (!units.empty() && units[0].dy == 0 && units[0].dx == 0 && g.vec == 16 && g.k == g.cin &&
+    } else if (!equalize && !units.empty() && units[0].dy == 0 && units[0].dx == 0 && g.vec == 16 && g.k == g.cin &&
                gemm_skinny_applies(g.taps, g.cin, g.proto.cin, units[0].offset, g.proto.m, g.n) && g.proto.stride_h == 1 && g.proto.stride_w == 1 &&
                g.proto.y_base == 0 && g.proto.x_base == 0 && g.proto.h == g.proto.ho && g.proto.w == g.proto.wo && g.proto.out_sy == 1 &&
                g.proto.out_sx == 1 && g.proto.out_y0 == 0 && g.proto.out_x0 == 0 && g.proto.out_h == g.proto.ho && g.proto.out_w == g.proto.wo) {
         // a classifier head at batch 1 .. 64: the launch is the weights' one trip from memory
         g.cfg.id = GEMM_SKINNY;
         g.cfg.slab = 32;
-    } else if (g.cin == 3 && g.proto.cin == 3 && g.taps == 9 && g.k == 27 && units.size() == 27 && units[26].dy == 2 &&
+    } else if (!equalize && g.cin == 3 && g.proto.cin == 3 && g.taps == 9 && g.k == 27 && units.size() == 27 && units[26].dy == 2 &&
                units[26].dx == 2 && units[12].dy == 1 && units[12].dx == 1 && units[0].offset == 0) {
         // three channels, 3x3 taps, dilation 1: the first layer of image networks
         g.cfg.id = GEMM_C3K3;
         g.cfg.slab = 32;
-    } else if (int kh = 0, kw = 0; g.cin >= 1 && g.cin <= 4 && g.taps > 1 && g.k == g.taps * g.cin && !units.empty() && units[0].offset == 0 &&
+    } else if (int kh = 0, kw = 0; !equalize && g.cin >= 1 && g.cin <= 4 && g.taps > 1 && g.k == g.taps * g.cin && !units.empty() && units[0].offset == 0 &&
                                    units_are_rows(units, g.cin / g.vec, g.taps, kh, kw) && conv_rows_applies(g.cin, g.proto.cin, kh, kw) &&
                                    (long)g.proto.h * g.proto.w * g.cin >= 16) {
         // one to four input channels, a kernel row within 32 bytes: first layers on RGB(A) or grey images beyond 3x3 RGB
@@ -219,7 +224,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         g.cfg.slab = 32;
         g.proto.rows_kh = kh;
         g.proto.rows_kw = kw;
-    } else if (g.vec == 16 && g.taps == 9 && g.k == 9 * g.cin && units.size() == (size_t)g.k / 16 && g.proto.stride_h == 1 &&
+    } else if (!equalize && g.vec == 16 && g.taps == 9 && g.k == 9 * g.cin && units.size() == (size_t)g.k / 16 && g.proto.stride_h == 1 &&
                g.proto.stride_w == 1 && g.proto.out_sy == 1 && g.proto.out_sx == 1 && g.proto.out_y0 == 0 && g.proto.out_x0 == 0 &&
                g.proto.out_h == g.proto.ho && g.proto.out_w == g.proto.wo && units_are_3x3(units, g.cin / 16) &&
                conv3x3_patch_applies(g.cin, g.proto.cin, g.proto.wo, g.proto.ho) &&
@@ -241,7 +246,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
         g.cfg.slab = 256;
         must_slice = true;
     }
-    g.k_pad = g.cfg.id == GEMM_ROWS ? g.proto.rows_kh * 32 : round_up(g.k > 0 ? g.k : 1, g.cfg.slab);
+    g.k_pad = g.cfg.id == GEMM_ROWS ? g.proto.rows_kh * 32 : round_up(k_len > 0 ? k_len : 1, g.cfg.slab);
     g.n_pad = round_up(g.n, igemm_n_tile(0, g.n, g.k));
     g.slices = 0;
     if (g.cfg.id == GEMM_DMA_64x64_SPLITK && siblings == 1 && g.n_period == 0) {
@@ -307,7 +312,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     // a plain matrix: one tap at the pixel itself, unit stride, no padding, whole slabs
     // (a reduction that ends inside its last slab is handled by the kernel: the chunks past the end read a constant)
     g.proto.dense = plain_matrix ? 1 : 0;
-    if (g.slices) g.proto.dense = 0;  // slices are cut out of the k-table
+    if (g.slices || equalize) g.proto.dense = 0;  // slices are cut out of the k-table; siblings of one launch all run table-driven
     return EH_OK;
 }
 
@@ -1402,6 +1407,28 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
     struct XPhase {
         int px, ox0, wo_p, ntx, bx;
     };
+    // A kernel that is no multiple of the stride (3x3 at stride 2) gives phases with 4, 2, 2 and 1 taps.  When they
+    // cover equally many output pixels (even output extents), padding every phase's reduction to the longest puts them
+    // into one launch of equally shaped problems instead of one launch each; accepted up to twice the multiply-adds.
+    int k_floor = 0;
+    if (G == 1 && (cig & 15) == 0 && (d->kh % sh != 0 || d->kw % sw != 0) && sh * sw <= GemmBatch::MAX) {
+        long m_first = -1, taps_max = 0, taps_sum = 0;
+        int phases = 0;
+        bool equal_m = true;
+        for (int py = 0; py < sh; ++py)
+            for (int px = 0; px < sw; ++px) {
+                const int oy0 = ((py - d->pad_t) % sh + sh) % sh, ox0 = ((px - d->pad_l) % sw + sw) % sw;
+                if (oy0 >= oh || ox0 >= ow) continue;
+                const long m_p = (long)((oh - oy0 + sh - 1) / sh) * ((ow - ox0 + sw - 1) / sw);
+                const long taps_p = (long)(py < d->kh ? (d->kh - py + sh - 1) / sh : 0) * (px < d->kw ? (d->kw - px + sw - 1) / sw : 0);
+                if (m_first < 0) m_first = m_p;
+                equal_m = equal_m && m_p == m_first;
+                taps_max = std::max(taps_max, taps_p);
+                taps_sum += taps_p;
+                ++phases;
+            }
+        if (phases >= 2 && equal_m && taps_max * phases <= 2 * taps_sum && taps_max * phases > taps_sum) k_floor = (int)taps_max * cig;
+    }
     for (int g = 0; g < G; ++g)
         for (int py = 0; py < sh; ++py) {
             const int oy0 = ((py - d->pad_t) % sh + sh) % sh;
@@ -1486,8 +1513,8 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                 p.out_x0 = ox0;
                 p.ldc = d->cout;
                 // phases (and groups) of equal shape share launches: choose the tile shape for the joint tile count
-                const int siblings = (d->kh % sh == 0 && d->kw % sw == 0) ? std::min(G * sh * sw / count, (int)GemmBatch::MAX) : 1;
-                if ((rc = finish_part(part, units, tap_off, stream, siblings))) return rc;
+                const int siblings = (k_floor > 0 || (d->kh % sh == 0 && d->kw % sw == 0)) ? std::min(G * sh * sw / count, (int)GemmBatch::MAX) : 1;
+                if ((rc = finish_part(part, units, tap_off, stream, siblings, k_floor))) return rc;
             }
         }
     if (wants_channel_padding(op, G, cig_real)) return deconv_plan_build(pl, d, stream);

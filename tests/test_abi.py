@@ -240,6 +240,16 @@ def test_reductions_beyond_one_k_table_stay_on_the_tiled_kernels():
     assert eden.conv_kernels(eden.conv_desc(64, 25088, 1, 1, 4096, 1, 1, layout=nhwc))[0].startswith("dma_")   # a plain matrix needs no table
 
 
+def test_unequal_deconvolution_phases_share_one_configuration():
+    """3x3 at stride 2 over even output extents: the four phases (4, 2, 2, 1 taps) are padded to one reduction length and
+    take one tiled configuration, the one-tap phase included; odd extents keep each phase's own choice."""
+    even = eden.conv_desc(8, 256, 16, 16, 256, 3, 3, stride=(2, 2), pad=(1, 0, 1, 0), layout=eden.NHWC, weight_layout=eden.W_IOHW)
+    kernels = eden.conv_kernels(even, deconv=True)
+    assert len(kernels) == 4 and len(set(kernels)) == 1 and kernels[0].startswith("dma_")
+    odd = eden.conv_desc(8, 256, 16, 16, 256, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), layout=eden.NHWC, weight_layout=eden.W_IOHW)
+    assert "one_tap" in eden.conv_kernels(odd, deconv=True)
+
+
 def test_classifier_heads_take_the_kernel_cut_along_the_weights():
     nhwc = eden.NHWC
     assert eden.conv_kernels(eden.conv_desc(1, 1280, 1, 1, 1000, 1, 1, layout=nhwc)) == ["skinny"]

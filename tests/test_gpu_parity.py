@@ -657,6 +657,13 @@ DECONV_CASES = [
     dict(n=1, c=16, h=5, w=8, cout=40, kh=4, kw=8, stride=(2, 4), pad=(1, 1, 5, 5)),
     dict(n=1, c=16, h=6, w=6, cout=8, kh=3, kw=9, stride=(1, 3), pad=(1, 1, 3, 3)),
     dict(n=3, c=48, h=12, w=12, cout=21, kh=16, kw=16, stride=(8, 8), pad=(4, 4, 4, 4)),
+    # kernels that are no multiple of the stride over even output extents: phases of 4, 2, 2 and 1 taps (5x5: 9, 6, 6, 4)
+    # padded to one length and launched together; 21 channels on their padded copy; odd extents keep a launch per phase
+    dict(n=2, c=32, h=6, w=7, cout=24, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),
+    dict(n=1, c=64, h=9, w=8, cout=72, kh=5, kw=5, stride=(2, 2), pad=(2, 1, 2, 1)),
+    dict(n=2, c=21, h=8, w=8, cout=21, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),
+    dict(n=1, c=16, h=7, w=7, cout=16, kh=3, kw=3, stride=(2, 2), pad=(1, 1, 1, 1)),
+    dict(n=8, c=256, h=16, w=16, cout=256, kh=3, kw=3, stride=(2, 2), pad=(1, 0, 1, 0)),
 ]
 
 
