@@ -1210,8 +1210,10 @@ int eh_conv2d_u8_run_static(eh_conv_plan *plan, const void *input, void *output,
     EH_REQUIRE(plan != nullptr, "null plan");
     if (plan->d.n == 0) return check_requant(q, plan->op.w_signed, plan->op.io_signed);
     const GemmOp &op = plan->op;
-    EH_REQUIRE(op.parts.size() <= (size_t)GemmOp::kInlineParts, "run_static: %zu convolution groups, at most %d are supported",
-               op.parts.size(), GemmOp::kInlineParts);
+    size_t problems = 0;  // (beyond the inline array a run would allocate host memory)
+    for (const GemmPart &g : op.parts) problems += g.slices ? (size_t)g.slices : 1;
+    EH_REQUIRE(problems <= (size_t)GemmOp::kInlineParts, "run_static: the plan runs as %zu problems (groups, slices), at most %d are supported",
+               problems, GemmOp::kInlineParts);
     uint8_t *staging = nullptr;
     if (const size_t need = op.staging_bytes(); need != 0) {
         EH_REQUIRE(need <= (size_t)EH_STATIC_SCRATCH_BYTES,

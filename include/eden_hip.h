@@ -322,10 +322,12 @@ int eh_conv2d_u8_run(eh_conv_plan *plan, const void *input, void *output, const 
  * that forbid it): no counterpart in the reference.  Calls no hipMalloc / hipFree and allocates no host memory.  A
  * planar (EH_NCHW) plan computes channels-last between two layout conversions; here the two channels-last staging
  * images live in a static device array of EH_STATIC_SCRATCH_BYTES that each GPU holds from the moment the library
- * is loaded on it, instead of in the plan's own buffers (an EH_NHWC plan needs no staging and runs as
- * eh_conv2d_u8_run does).  Fails with EH_INVALID_PARAMS, launching nothing, when the staging
- * (n*c*h*w + n*cout*ho*wo bytes, each rounded up to 256 plus 256) exceeds the array or the plan has more than
- * 8 groups.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * is loaded on it, instead of in the plan's own buffers; so does the channel-padded copy of the input that a plan
+ * with a channel count off the multiples of 16 reads (see EH_EXACT_CHANNELS).  Any other EH_NHWC plan needs no staging
+ * and runs as eh_conv2d_u8_run does.  Fails with EH_INVALID_PARAMS, launching nothing, when the staging
+ * (planar: n*c*h*w + n*cout*ho*wo bytes; padded: n*h*w*groups*ceil16(c/groups); each rounded up to 256 plus 256)
+ * exceeds the array or the plan runs as more than 8 problems (groups, slices of a long reduction).  What a plan
+ * allocated when it was made (packed weights, the int32 image of a sliced reduction) stays the plan's.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two
  * threads) race; calls ordered on one stream do not.  Results are bit for bit those of eh_conv2d_u8_run.  The first
  * launch of a persistent-grid kernel variant (the one-tap and the few-channel first-layer kernels) at a given LDS size
  * asks the driver once how many of its workgroups a CU holds

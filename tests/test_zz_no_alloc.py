@@ -75,6 +75,19 @@ def test_static_scratch_entry_point_on_a_stream_and_channels_last():
     eden.sync()
     got = d_o.download((s.n, a["shape"][2], a["shape"][3], s.cout)).transpose(0, 3, 1, 2)
     assert np.array_equal(got, a["want"])
+    # channels-last with 21 channels: the channel-padded copy of the input is the one staging image, in the scratch too
+    r = planar_conv(dict(n=2, c=21, h=13, w=12, cout=24, kh=3, kw=3, pad=(1, 1, 1, 1)), SEED + 50)
+    s = r["s"]
+    x = synth.fill_u8((s.n, s.c, s.h, s.w), SEED + 50)
+    desc = eden.conv_desc(s.n, s.c, s.h, s.w, s.cout, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1, 1, eden.NHWC, eden.W_OIHW)
+    d_x = eden.DeviceBuffer(host=np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+    plan = eden.ConvPlan(desc, r["keep"][0], r["keep"][1], r["q"])
+    for _ in range(2):
+        d_o = eden.DeviceBuffer(nbytes=r["want"].size)
+        plan.run_static(d_x, d_o, r["q"])
+        eden.sync()
+        got = d_o.download((s.n, r["shape"][2], r["shape"][3], s.cout)).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, r["want"])
 
 
 def test_static_scratch_entry_point_refuses_what_does_not_fit():
