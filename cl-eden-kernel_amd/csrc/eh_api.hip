@@ -186,7 +186,7 @@ static bool units_are_rows(const std::vector<KUnit> &units, int per_tap, int tap
 // reduction is padded to k_floor (the padding units read a constant that multiplies to zero) and only the tiled
 // kernels are considered, so that every sibling gets the same configuration.
 int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_t> &tap_off, hipStream_t stream,
-                int siblings = 1, int k_floor = 0) {
+                int siblings = 1, int k_floor = 0, int m_floor = 0) {
     // the kernel shape is fixed here because the packed weight layout depends on it
     g.cfg = GemmConfig();
     const bool equalize = k_floor > 0;
@@ -237,7 +237,7 @@ int finish_part(GemmPart &g, std::vector<KUnit> &units, const std::vector<int32_
     } else if (g.vec == 16 && (ktab_fits || (plain_matrix && g.k % 256 == 0)))
         // (a reduction too long for its k-table to fit LDS still runs as a plain matrix of whole slabs: a fully
         // connected layer on 25088 inputs)
-        g.cfg = igemm_dma_select(g.proto.m, g.n, g.k, siblings);
+        g.cfg = igemm_dma_select(g.proto.m > m_floor ? g.proto.m : m_floor, g.n, g.k, siblings);  // (m_floor: the siblings' largest row count)
     bool must_slice = false;
     if (g.cfg.id == GEMM_STAGED && g.vec == 16 && !ktab_fits && siblings == 1 && g.n_period == 0) {
         // table-driven and too long for one k-table (a 7x7 convolution over 512 channels): the split-reduction tiles
@@ -1409,27 +1409,26 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
     struct XPhase {
         int px, ox0, wo_p, ntx, bx;
     };
-    // A kernel that is no multiple of the stride (3x3 at stride 2) gives phases with 4, 2, 2 and 1 taps.  When they
-    // cover equally many output pixels (even output extents), padding every phase's reduction to the longest puts them
-    // into one launch of equally shaped problems instead of one launch each; accepted up to twice the multiply-adds.
-    int k_floor = 0;
+    // A kernel that is no multiple of the stride (3x3 at stride 2) gives phases with 4, 2, 2 and 1 taps.  Padding every
+    // phase's reduction to the longest and choosing the tile shape for the largest phase puts them into one launch
+    // instead of one launch each (the phases' pixel counts may differ by a row or a column: every problem of a launch
+    // tests rows against its own count); accepted up to twice the multiply-adds.
+    int k_floor = 0, m_floor = 0;
     if (G == 1 && (cig & 15) == 0 && (d->kh % sh != 0 || d->kw % sw != 0) && sh * sw <= GemmBatch::MAX) {
-        long m_first = -1, taps_max = 0, taps_sum = 0;
+        long taps_max = 0, taps_sum = 0;
         int phases = 0;
-        bool equal_m = true;
         for (int py = 0; py < sh; ++py)
             for (int px = 0; px < sw; ++px) {
                 const int oy0 = ((py - d->pad_t) % sh + sh) % sh, ox0 = ((px - d->pad_l) % sw + sw) % sw;
                 if (oy0 >= oh || ox0 >= ow) continue;
                 const long m_p = (long)((oh - oy0 + sh - 1) / sh) * ((ow - ox0 + sw - 1) / sw);
                 const long taps_p = (long)(py < d->kh ? (d->kh - py + sh - 1) / sh : 0) * (px < d->kw ? (d->kw - px + sw - 1) / sw : 0);
-                if (m_first < 0) m_first = m_p;
-                equal_m = equal_m && m_p == m_first;
+                m_floor = (int)std::max((long)m_floor, (long)d->n * m_p);
                 taps_max = std::max(taps_max, taps_p);
                 taps_sum += taps_p;
                 ++phases;
             }
-        if (phases >= 2 && equal_m && taps_max * phases <= 2 * taps_sum && taps_max * phases > taps_sum) k_floor = (int)taps_max * cig;
+        if (phases >= 2 && taps_max * phases <= 2 * taps_sum && taps_max * phases > taps_sum) k_floor = (int)taps_max * cig;
     }
     for (int g = 0; g < G; ++g)
         for (int py = 0; py < sh; ++py) {
@@ -1516,7 +1515,7 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
                 p.ldc = d->cout;
                 // phases (and groups) of equal shape share launches: choose the tile shape for the joint tile count
                 const int siblings = (k_floor > 0 || (d->kh % sh == 0 && d->kw % sw == 0)) ? std::min(G * sh * sw / count, (int)GemmBatch::MAX) : 1;
-                if ((rc = finish_part(part, units, tap_off, stream, siblings, k_floor))) return rc;
+                if ((rc = finish_part(part, units, tap_off, stream, siblings, k_floor, k_floor ? m_floor : 0))) return rc;
             }
         }
     if (wants_channel_padding(op, G, cig_real)) return deconv_plan_build(pl, d, stream);

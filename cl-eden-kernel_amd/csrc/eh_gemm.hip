@@ -315,7 +315,8 @@ int launch_igemm_batch(const GemmProblem *ps, int count, hipStream_t stream) {
         int run = 1;
         const bool dma = p.cfg.id != GEMM_STAGED && p.cfg.id != GEMM_THIN && p.cfg.id != GEMM_C3K3 && p.cfg.id != GEMM_CONV3X3 && p.cfg.id != GEMM_ROWS && p.cfg.id != GEMM_SKINNY && p.m > 0 && p.n > 0;
         if (dma)
-            while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == p.cfg.id && ps[i + run].m == p.m &&
+            // (row counts may differ where nothing depends on them: table-driven problems; the launch covers the largest)
+            while (i + run < count && run < GemmBatch::MAX && ps[i + run].cfg.id == p.cfg.id && (ps[i + run].m == p.m || (!p.dense && !p.partial)) &&
                    ps[i + run].n == p.n && ps[i + run].k_pad == p.k_pad && ps[i + run].dense == p.dense && ps[i + run].zw == p.zw)
                 ++run;
         // ... and so do equally shaped one-tap problems (the phases of a transposed convolution whose kernel is its stride,

@@ -683,7 +683,9 @@ int launch_cfg(const GemmProblem *ps, int count, hipStream_t stream) {
     GemmBatch batch;
     for (int i = 0; i < count; ++i) batch.p[i] = ps[i];
     static_assert(STAGES * (BM + BN) * SLAB + WGK * 2 * BM * 4 + BN * 4 <= 160 * 1024 - 12288, "LDS budget with the largest k-table");
-    const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    int m_max = p.m;  // (table-driven problems of one launch may differ in their row counts: every kernel tests rows against its own problem's)
+    for (int i = 1; i < count; ++i) m_max = ps[i].m > m_max ? ps[i].m : m_max;
+    const int tiles_m = (m_max + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     // group size: 32 tiles, or fewer (a power of two) when that is needed to give each of the 8 XCDs a group
     int gs = 32;
     while (gs > 1 && (long)tiles_m * tiles_n * count < 8l * gs) gs >>= 1;
@@ -842,7 +844,7 @@ int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream) {
     EH_REQUIRE(count >= 1 && count <= GemmBatch::MAX, "igemm_dma: batch of %d", count);
     for (int i = 0; i < count; ++i) {
         EH_REQUIRE(ps[i].vec == 16 && ps[i].k_pad % ps[i].cfg.slab == 0, "igemm_dma: unsupported problem");
-        EH_REQUIRE(ps[i].cfg.id == p.cfg.id && ps[i].m == p.m && ps[i].n == p.n && ps[i].k_pad == p.k_pad &&
+        EH_REQUIRE(ps[i].cfg.id == p.cfg.id && (ps[i].m == p.m || (!p.dense && !p.partial)) && ps[i].n == p.n && ps[i].k_pad == p.k_pad &&
                        ps[i].dense == p.dense && ps[i].zw == p.zw,
                    "igemm_dma: a batch must hold equally shaped problems");
     }
@@ -855,7 +857,9 @@ int launch_igemm_dma(const GemmProblem *ps, int count, hipStream_t stream) {
             // Two stages take half the LDS, so two workgroups share a CU: for reductions of one or two slabs (deeper
             // staging has nothing to prefetch) and for launches with more tiles than CUs (the second workgroup's
             // prologue and epilogue hide behind the first one's loop instead of forming a second round).
-            const long tiles = (long)((p.m + 63) / 64) * ((p.n + 63) / 64) * count;
+            int m_max = p.m;
+            for (int i = 1; i < count; ++i) m_max = ps[i].m > m_max ? ps[i].m : m_max;
+            const long tiles = (long)((m_max + 63) / 64) * ((p.n + 63) / 64) * count;
             if (p.k_pad / 256 <= 2 || tiles > 256) return launch_cfg<64, 64, 1, 1, 4, 256, 2>(ps, count, stream);
             return launch_cfg<64, 64, 1, 1, 4, 256, 4>(ps, count, stream);
         }

@@ -241,13 +241,17 @@ def test_reductions_beyond_one_k_table_stay_on_the_tiled_kernels():
 
 
 def test_unequal_deconvolution_phases_share_one_configuration():
-    """3x3 at stride 2 over even output extents: the four phases (4, 2, 2, 1 taps) are padded to one reduction length and
-    take one tiled configuration, the one-tap phase included; odd extents keep each phase's own choice."""
-    even = eden.conv_desc(8, 256, 16, 16, 256, 3, 3, stride=(2, 2), pad=(1, 0, 1, 0), layout=eden.NHWC, weight_layout=eden.W_IOHW)
-    kernels = eden.conv_kernels(even, deconv=True)
-    assert len(kernels) == 4 and len(set(kernels)) == 1 and kernels[0].startswith("dma_")
-    odd = eden.conv_desc(8, 256, 16, 16, 256, 3, 3, stride=(2, 2), pad=(1, 1, 1, 1), layout=eden.NHWC, weight_layout=eden.W_IOHW)
-    assert "one_tap" in eden.conv_kernels(odd, deconv=True)
+    """3x3 at stride 2: the four phases (4, 2, 2, 1 taps) are padded to one reduction length and take one tiled
+    configuration, the one-tap phase included, over even output extents and over odd ones (phases of 16x16, 16x15,
+    15x16 and 15x15 pixels); 24 channels likewise on their padded copy; EXACT_CHANNELS there keeps the byte gathers."""
+    for pad in ((1, 0, 1, 0), (1, 1, 1, 1)):
+        desc = eden.conv_desc(8, 256, 16, 16, 256, 3, 3, stride=(2, 2), pad=pad, layout=eden.NHWC, weight_layout=eden.W_IOHW)
+        kernels = eden.conv_kernels(desc, deconv=True)
+        assert len(kernels) == 4 and len(set(kernels)) == 1 and kernels[0].startswith("dma_"), (pad, kernels)
+    ragged = eden.conv_desc(8, 24, 16, 16, 24, 3, 3, stride=(2, 2), pad=(1, 0, 1, 0), layout=eden.NHWC, weight_layout=eden.W_IOHW)
+    assert len(set(eden.conv_kernels(ragged, deconv=True))) == 1
+    ragged.layout |= eden.EXACT_CHANNELS
+    assert "staged" in eden.conv_kernels(ragged, deconv=True)
 
 
 def test_classifier_heads_take_the_kernel_cut_along_the_weights():
