@@ -825,7 +825,10 @@ GemmConfig igemm_dma_select(int32_t m, int32_t n, int32_t k, int32_t siblings) {
     } else if (n > 64 && t256 >= 240) {
         c.id = GEMM_DMA_256x128;
         c.slab = 128;
-    } else if (n > 64 && t128 >= 160) {  // (from 5/8 of the CUs on, one round of these beats three of the split-reduction tiles)
+    } else if (n > 64 && t128 > 128) {
+        // (more than 128 of these are more than 512 split-reduction tiles, i.e. three of those per CU on some CUs: from there
+        // on one round of 128 x 128 tiles is as fast or faster at every reduction length measured, 1.5x at 18 KiB; up to
+        // 128 the split-reduction tiles win, 17.9 against 26.0 us at 100 tiles and a 4.5 KiB reduction)
         c.id = GEMM_DMA_128x128;
         c.slab = 128;
     } else if (n <= 64 && t128x64 >= 200) {
