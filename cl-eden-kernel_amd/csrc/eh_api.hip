@@ -676,6 +676,10 @@ struct eh_dwconv_plan {
     // output channel j reads channel j of the copy; a caller's planar tensors (multiplier 1) by the two transpositions
     // the convolution plans use.  Both only where the output channels are a multiple of 4 (the four-channel kernels).
     int32_t rep_c = 0, rep_dm = 0;  // the caller's channel count and depth multiplier when the input is replicated
+    // ... and output channels that are no multiple of 4 (channels-last) by rounding them up: the copy of the input ends
+    // every pixel with repeats of its last channel, the weights of the extra channels are zero, and the result is
+    // computed into an image of the padded width, from which the caller's channels are copied out.
+    int32_t cout_caller = 0;        // `cout` counts the padded channels; this is what the caller's tensors hold
     bool planar = false;            // the caller's tensors are NCHW
     uint8_t *stage_in = nullptr, *stage_out = nullptr;
 };
@@ -1636,13 +1640,13 @@ static void dw_release(eh_dwconv_plan *pl) {
 static int dw_set_weights(eh_dwconv_plan *pl, const void *weight, const void *bias, hipStream_t stream) {
     EH_REQUIRE(weight != nullptr, "weight pointer is null");
     if (pl->d.weight_layout == EH_W_OHWI) {  // [taps][cout] -> [cout][taps]
-        int rc = launch_nhwc2nchw(static_cast<const uint8_t *>(weight), pl->w_copy, 1, pl->cout, pl->taps, stream);
+        int rc = launch_nhwc2nchw(static_cast<const uint8_t *>(weight), pl->w_copy, 1, pl->cout_caller, pl->taps, stream);
         if (rc) return rc;
     } else {
-        EH_HIP(hipMemcpyAsync(pl->w_copy, weight, (size_t)pl->cout * pl->taps, hipMemcpyDeviceToDevice, stream));
+        EH_HIP(hipMemcpyAsync(pl->w_copy, weight, (size_t)pl->cout_caller * pl->taps, hipMemcpyDeviceToDevice, stream));
     }
     pl->has_bias = bias != nullptr;
-    if (bias) EH_HIP(hipMemcpyAsync(pl->bias_copy, bias, (size_t)pl->cout * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
+    if (bias) EH_HIP(hipMemcpyAsync(pl->bias_copy, bias, (size_t)pl->cout_caller * sizeof(int32_t), hipMemcpyDeviceToDevice, stream));
     pl->packed_valid = false;
     pl->range_known = false;  // the plan call looks at the bytes once; weights replaced later keep the 16-bit form
     pl->trip_valid = false;
@@ -1705,13 +1709,17 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     eh_dwconv_plan *pl = new (std::nothrow) eh_dwconv_plan();
     EH_REQUIRE(pl != nullptr, "out of host memory");
     pl->d = *desc;
-    if (!no_staging && (desc->cout & 3) == 0 && desc->n > 0) {
-        if (desc->layout == EH_NHWC && desc->depth_multiplier > 1) {
+    pl->cout_caller = desc->cout;
+    if (!no_staging && desc->n > 0) {
+        const int32_t cout4 = (desc->cout + 3) & ~3;
+        if (desc->layout == EH_NHWC && (desc->depth_multiplier > 1 || cout4 != desc->cout) &&
+            (int64_t)desc->n * desc->h * desc->w * cout4 < (1ll << 31)) {
             pl->rep_c = desc->c;
             pl->rep_dm = desc->depth_multiplier;
-            pl->d.c = desc->cout;
+            pl->d.c = cout4;
+            pl->d.cout = cout4;
             pl->d.depth_multiplier = 1;
-        } else if (desc->layout == EH_NCHW && desc->depth_multiplier == 1) {
+        } else if (desc->layout == EH_NCHW && desc->depth_multiplier == 1 && cout4 == desc->cout) {
             pl->planar = true;
             pl->d.layout = EH_NHWC;
         }
@@ -1731,8 +1739,12 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     hipStream_t s = as_stream(stream);
     rc = dev_alloc(&pl->w_copy, (size_t)pl->cout * pl->taps);
     if (!rc && (pl->rep_dm || pl->planar)) rc = dev_alloc(&pl->stage_in, (size_t)desc->n * desc->h * desc->w * pl->cout + 256);
-    if (!rc && pl->planar) rc = dev_alloc(&pl->stage_out, (size_t)desc->n * pl->ho * pl->wo * pl->cout + 256);
+    if (!rc && (pl->planar || pl->cout != pl->cout_caller)) rc = dev_alloc(&pl->stage_out, (size_t)desc->n * pl->ho * pl->wo * pl->cout + 256);
     if (!rc) rc = dev_alloc(&pl->bias_copy, (size_t)pl->cout);
+    if (!rc && pl->cout != pl->cout_caller && !g_dry_run) {  // the extra channels: zero weights, zero bias
+        EH_HIP(hipMemsetAsync(pl->w_copy, 0, (size_t)pl->cout * pl->taps, s));
+        EH_HIP(hipMemsetAsync(pl->bias_copy, 0, (size_t)pl->cout * sizeof(int32_t), s));
+    }
     if (!rc) rc = dev_alloc(&pl->w_pair, (size_t)((pl->taps + 1) / 2) * pl->cout);
     if (!rc) rc = dev_alloc(&pl->bias_folded, (size_t)pl->cout + 4);
     const bool tile_form = pl->d.layout == EH_NHWC && pl->d.kh == 3 && pl->d.kw == 3 && pl->d.depth_multiplier == 1;
@@ -1751,7 +1763,7 @@ int eh_dwconv2d_u8_plan(eh_dwconv_plan **plan, const eh_conv_desc *desc, const v
     if (!rc) rc = dw_set_weights(pl, weight, bias, s);
     if (!rc && tile_form && pl->cout > 0) {
         // the extremes of the weight bytes decide, per zero point, whether the 8-bit dot product form applies
-        std::vector<uint8_t> host((size_t)pl->cout * 9);
+        std::vector<uint8_t> host((size_t)pl->cout_caller * 9);
         hipError_t e = hipMemcpyAsync(host.data(), pl->w_copy, host.size(), hipMemcpyDeviceToHost, s);
         if (e == hipSuccess) e = hipStreamSynchronize(s);
         if (e != hipSuccess) {
@@ -1789,7 +1801,7 @@ int eh_dwconv2d_u8_set_perchannel(eh_dwconv_plan *plan, const int32_t *multiplie
         plan->pc_multiplier = plan->pc_shift = nullptr;
         return EH_OK;
     }
-    EH_REQUIRE(count == plan->cout, "per-channel: %d pairs for %d output channels", count, plan->cout);
+    EH_REQUIRE(count == plan->cout_caller, "per-channel: %d pairs for %d output channels", count, plan->cout_caller);
     int rc = check_perchannel(multipliers, shifts, count);
     if (rc) return rc;
     hipStream_t s = as_stream(stream);
@@ -1863,7 +1875,16 @@ int eh_dwconv2d_u8_run(eh_dwconv_plan *plan, const void *input, void *output, co
     hipStream_t s = as_stream(stream);
     if ((rc = dw_refold(plan, *q, s))) return rc;
     if (plan->rep_dm) {
-        if ((rc = launch_replicate_channels(static_cast<const uint8_t *>(input), plan->stage_in, (int64_t)d.n * d.h * d.w, plan->rep_c, plan->rep_dm, s))) return rc;
+        // (multiplier 1: only the rows' tails are new, and the copy reads whole dwords)
+        rc = plan->rep_dm == 1 ? launch_pad_channels(static_cast<const uint8_t *>(input), plan->stage_in, (int64_t)d.n * d.h * d.w, 1, plan->rep_c, plan->cout, 0, s)
+                               : launch_replicate_channels(static_cast<const uint8_t *>(input), plan->stage_in, (int64_t)d.n * d.h * d.w, plan->rep_c,
+                                                           plan->rep_dm, plan->cout, s);
+        if (rc) return rc;
+        if (plan->cout != plan->cout_caller) {
+            if ((rc = launch_dwconv_nhwc(dw_problem(plan, plan->stage_in, plan->stage_out), s))) return rc;
+            return launch_keep_channels(plan->stage_out, static_cast<uint8_t *>(output), (int64_t)d.n * plan->ho * plan->wo, plan->cout,
+                                        plan->cout_caller, s);
+        }
         input = plan->stage_in;
     } else if (plan->planar) {
         if ((rc = launch_nchw2nhwc(static_cast<const uint8_t *>(input), plan->stage_in, d.n, d.c, d.h * d.w, s))) return rc;

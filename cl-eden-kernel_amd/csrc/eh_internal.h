@@ -554,8 +554,11 @@ int launch_pwdw_block(const GemmProblem &pw, const DwProblem &dw, int rows_per_t
 
 // ---------------------------------------------------------------- layout
 int launch_nchw2nhwc(const uint8_t *src, uint8_t *dst, int32_t n, int32_t c, int32_t hw, hipStream_t stream);
-// dst[pixel][c * times + d] = src[pixel][c] for d < times (c * times a multiple of 4)
-int launch_replicate_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c, int32_t times, hipStream_t stream);
+// dst[pixel][c * times + d] = src[pixel][c] for d < times; rows of c_to >= c * times bytes (a multiple of 4), the tail
+// filled with repeats of the pixel's last channel
+int launch_replicate_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c, int32_t times, int32_t c_to, hipStream_t stream);
+// dst[pixel][0 .. c_keep) = src[pixel][0 .. c_keep) from rows of c_from bytes (a multiple of 4)
+int launch_keep_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c_from, int32_t c_keep, hipStream_t stream);
 // dst[pixel][g][0 .. cg_to) = src[pixel][g][0 .. cg) followed by cg_to - cg bytes `fill`, for `groups` channel groups per pixel
 int launch_pad_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t groups, int32_t cg, int32_t cg_to, uint32_t fill,
                         hipStream_t stream);

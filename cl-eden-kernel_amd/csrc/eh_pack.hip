@@ -93,8 +93,28 @@ __global__ __launch_bounds__(256) void replicate_channels_kernel(const uint8_t *
     const uint8_t *s = src + (size_t)pixel * (size_t)c;
     uint32_t v = 0;
 #pragma unroll
-    for (int b = 0; b < 4; ++b) v |= (uint32_t)s[fastdiv(quad * 4u + (uint32_t)b, div_times)] << (8 * b);
+    for (int b = 0; b < 4; ++b) {
+        const uint32_t ch = fastdiv(quad * 4u + (uint32_t)b, div_times);  // (past the last channel in a row's padding tail)
+        v |= (uint32_t)s[ch < (uint32_t)c ? ch : (uint32_t)c - 1u] << (8 * b);
+    }
     reinterpret_cast<uint32_t *>(dst)[idx] = v;
+}
+
+// The first c_keep bytes of every row of c_from bytes: the caller's channels out of an image computed on a channel count
+// rounded up to a multiple of 4.  One thread per source dword; whole dwords leave at byte addresses.
+__global__ __launch_bounds__(256) void keep_channels_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, const uint32_t total,
+                                                            const uint32_t quads_per_pixel, const FastDiv div_quads, const int32_t c_keep) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t pixel = fastdiv(idx, div_quads), quad = idx - pixel * quads_per_pixel;
+    const uint32_t v = reinterpret_cast<const uint32_t *>(src)[idx];
+    const int left = c_keep - (int)quad * 4;
+    uint8_t *d = dst + ((size_t)pixel * (size_t)c_keep + (size_t)quad * 4u);
+    if (left >= 4) {
+        *reinterpret_cast<u32_a1 *>(d) = v;
+    } else {
+        for (int b = 0; b < left; ++b) d[b] = (uint8_t)(v >> (8 * b));
+    }
 }
 
 // Byte-matrix transpose per batch: src [batch][R][S] -> dst [batch][S][R].
@@ -322,13 +342,24 @@ int launch_transpose(const uint8_t *src, uint8_t *dst, int32_t batch, int32_t R,
 
 }  // namespace
 
-int launch_replicate_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c, int32_t times, hipStream_t stream) {
-    EH_REQUIRE(c > 0 && times > 0 && ((c * times) & 3) == 0, "replicate_channels: bad extents %d x %d", c, times);
-    const int64_t total = pixels * (c * times >> 2);
+int launch_replicate_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c, int32_t times, int32_t c_to, hipStream_t stream) {
+    EH_REQUIRE(c > 0 && times > 0 && c_to >= c * times && (c_to & 3) == 0, "replicate_channels: bad extents %d x %d -> %d", c, times, c_to);
+    const int64_t total = pixels * (c_to >> 2);
     if (total <= 0) return EH_OK;
     EH_REQUIRE(total < (1ll << 31), "replicate_channels: tensor too large");
     hipLaunchKernelGGL(replicate_channels_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, dst, (uint32_t)total,
-                       (uint32_t)(c * times >> 2), make_fastdiv((uint32_t)(c * times >> 2)), c, make_fastdiv((uint32_t)times));
+                       (uint32_t)(c_to >> 2), make_fastdiv((uint32_t)(c_to >> 2)), c, make_fastdiv((uint32_t)times));
+    EH_HIP(hipGetLastError());
+    return EH_OK;
+}
+
+int launch_keep_channels(const uint8_t *src, uint8_t *dst, int64_t pixels, int32_t c_from, int32_t c_keep, hipStream_t stream) {
+    EH_REQUIRE(c_keep > 0 && c_from >= c_keep && (c_from & 3) == 0, "keep_channels: bad extents %d of %d", c_keep, c_from);
+    const int64_t total = pixels * (c_from >> 2);
+    if (total <= 0) return EH_OK;
+    EH_REQUIRE(total < (1ll << 31), "keep_channels: tensor too large");
+    hipLaunchKernelGGL(keep_channels_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, dst, (uint32_t)total,
+                       (uint32_t)(c_from >> 2), make_fastdiv((uint32_t)(c_from >> 2)), c_keep);
     EH_HIP(hipGetLastError());
     return EH_OK;
 }

@@ -65,9 +65,10 @@ typedef enum eh_weight_layout { EH_W_OIHW = 0, EH_W_OHWI = 1, EH_W_IOHW = 2 } eh
  * keeps convolution groups of fewer than 16 channels as one problem per group; without it neighbouring groups run in
  * bundles as block-diagonal problems over 16 to 64 adjacent channels, for which the plan keeps a copy of the
  * weights (it packs them again when a run brings another weight zero point).  A depthwise plan with a depth
- * multiplier (channels-last) or planar tensors (multiplier 1) whose output channels are a multiple of 4 likewise owns
- * a staging image (the input with every channel repeated; the two transposed tensors) unless the flag is set, which
- * keeps it on the one-output-per-thread kernel.  Results are the same bytes either way. */
+ * multiplier or output channels off the multiples of 4 (channels-last), or planar tensors (multiplier 1, channels a
+ * multiple of 4), likewise owns staging images (the input with every channel repeated and the pixels' tails padded, the
+ * result at the padded width; the two transposed tensors) unless the flag is set, which keeps it on the
+ * one-output-per-thread kernel.  Results are the same bytes either way. */
 #define EH_EXACT_CHANNELS 0x400
 
 /* Integer requantization parameters of one operator execution: what

@@ -98,6 +98,7 @@ DW_CASES = [
     dict(n=2, c=16, h=17, w=14, cout=16, kh=3, kw=3, stride=(1, 1), pad=(2, 2, 2, 2), dil=(2, 2)),   # dilated 3x3 tiles
     dict(n=1, c=8, h=13, w=19, cout=8, kh=3, kw=3, stride=(1, 1), pad=(4, 4, 4, 4), dil=(4, 4)),
     dict(n=1, c=12, h=16, w=15, cout=12, kh=3, kw=3, stride=(1, 1), pad=(5, 5, 5, 5), dil=(5, 5)),
+    dict(n=2, c=30, h=11, w=10, cout=30, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),             # 30 channels computed as 32
 ]
 
 
@@ -121,7 +122,7 @@ def test_int8_depthwise_matches_oracle(case, layout):
         assert want.std() > 4
 
 
-@pytest.mark.parametrize("case", DW_CASES[:2] + DW_CASES[-3:] + [dict(n=40, c=64, h=64, w=64, cout=64, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1))],
+@pytest.mark.parametrize("case", DW_CASES[:2] + DW_CASES[-4:] + [dict(n=40, c=64, h=64, w=64, cout=64, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1))],
                          ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
 def test_int8_depthwise_weights_within_int8_of_their_zero_point(case):
     """channels-last 3x3 with every w - zp_w inside int8: the 8-bit dot product kernel on int8 tensors"""
@@ -140,7 +141,7 @@ def test_int8_depthwise_weights_within_int8_of_their_zero_point(case):
         assert want.std() > 4
 
 
-DW_PC_S8_CASES = DW_CASES[-3:] + [
+DW_PC_S8_CASES = DW_CASES[-4:] + [
     dict(n=2, c=32, h=15, w=14, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),     # four outputs per thread, stride 1
     dict(n=2, c=24, h=15, w=17, cout=24, kh=3, kw=3, stride=(2, 2), pad=(0, 1, 0, 1)),     # four outputs per thread, stride 2
     dict(n=44, c=32, h=112, w=112, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),  # eight outputs per thread

@@ -179,7 +179,8 @@ DW_PC_CASES = [
     dict(n=2, c=8, h=14, w=17, cout=8, kh=3, kw=3, stride=(1, 1), pad=(4, 4, 4, 4), dil=(4, 4)),    # 3x3 dilated tile, columns shared
     dict(n=1, c=24, h=13, w=11, cout=24, kh=3, kw=3, stride=(1, 1), pad=(3, 3, 3, 3), dil=(3, 3)),  # 3x3 dilated tile, three column groups
     dict(n=1, c=16, h=12, w=12, cout=16, kh=3, kw=3, stride=(2, 2), pad=(2, 2, 2, 2), dil=(2, 2)),  # four-channel kernel: dilated with stride 2
-    dict(n=2, c=5, h=9, w=8, cout=10, kh=3, kw=3, stride=(2, 1), pad=(1, 0, 1, 1), dm=2),           # one output per thread
+    dict(n=2, c=5, h=9, w=8, cout=10, kh=3, kw=3, stride=(2, 1), pad=(1, 0, 1, 1), dm=2),           # ten outputs: computed as twelve (planar: one output per thread)
+    dict(n=2, c=30, h=11, w=10, cout=30, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),              # 30 channels computed as 32
     dict(n=44, c=32, h=112, w=112, cout=32, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1)),           # 3x3 tile kernel, eight outputs per thread
 ]
 
