@@ -29,31 +29,35 @@ def test_random_operator_instances_match_the_oracle(seed):
         zp_in, zp_w = int(rng.integers(0, 256)), int(rng.choice([128, int(rng.integers(0, 256))]))
         lo = int(rng.choice([0, 0, int(rng.integers(0, 100))])); hi = int(rng.choice([255, 255, int(rng.integers(150, 256))]))
         layout = eden.NHWC if rng.random() < 0.7 else eden.NCHW
+        if rng.random() < 0.2:
+            layout |= eden.EXACT_CHANNELS   # no staged copies, no bundled groups: the kernels that read the caller's tensors as they are
         tseed = int(rng.integers(1, 1 << 30))
         try:
             if kind == "fc":
-                m, k, n = int(rng.integers(1, 300)), int(rng.choice([8, 16, 24, 40, 64, 100, 128, 192, 256, 260, 512, 1000])), int(rng.integers(1, 300))
+                m, k, n = int(rng.integers(1, 300)), int(rng.choice([8, 16, 24, 37, 40, 64, 100, 128, 192, 256, 260, 512, 1000, 1001, 6200])), int(rng.integers(1, 300))
                 a = synth.fill_u8((m, k), tseed); w = synth.fill_u8((n, k), tseed + 1); b = synth.fill_i32((n,), tseed + 2, -1000, 1000)
                 _, acc = O.fc(a, w, b, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
                 q = centred(acc, zp_in, zp_w, lo, hi)
-                want = O.fc(a, w, b, q); got = gpu_fc(a, w, b, to_eh_requant(q)); desc = (kind, m, k, n)
+                want = O.fc(a, w, b, q); got = gpu_fc(a, w, b, to_eh_requant(q), flags=layout & eden.EXACT_CHANNELS); desc = (kind, m, k, n, layout)
             else:
                 n = int(rng.integers(1, 5))
                 if kind == "dw":
-                    c = int(rng.choice([4, 8, 12, 16, 32, 36, 144, 20, 7])); h, w_ = int(rng.integers(3, 30)), int(rng.integers(3, 30))
-                    k = int(rng.choice([3, 3, 3, 5, 2])); st = int(rng.choice([1, 2])); pads = tuple(int(v) for v in rng.integers(0, k, 4))
-                    s = O.conv_shape(n, c, h, w_, c, k, k, stride=(st, st), pad=pads, groups=c)
+                    c = int(rng.choice([4, 8, 12, 16, 32, 36, 144, 20, 7, 5, 30])); h, w_ = int(rng.integers(3, 30)), int(rng.integers(3, 30))
+                    k = int(rng.choice([3, 3, 3, 5, 2, 7])); st = int(rng.choice([1, 1, 2])); dil = int(rng.choice([1, 1, 1, 2, 3, 4])); dm = int(rng.choice([1, 1, 1, 2, 3]))
+                    pads = tuple(int(v) for v in rng.integers(0, dil * (k - 1) + 1, 4))
+                    s = O.conv_shape(n, c, h, w_, c * dm, k, k, stride=(st, st), pad=pads, dil=(dil, dil), dm=dm)
                     if min(O.conv_out_hw(s)) < 1: continue
-                    x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((c, 1, k, k), tseed + 1); b = synth.fill_i32((c,), tseed + 2, -1000, 1000)
+                    x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((c * dm, 1, k, k), tseed + 1); b = synth.fill_i32((c * dm,), tseed + 2, -1000, 1000)
                     _, acc = O.dwconv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
                     q = centred(acc, zp_in, zp_w, lo, hi)
                     want = O.dwconv2d(x, w, b, s, q); got = gpu_dwconv(x, w, b, s, to_eh_requant(q), layout=layout); desc = (kind, s, layout)
                 elif kind == "deconv":
-                    c = int(rng.choice([8, 16, 32, 24])); cout = int(rng.choice([8, 16, 20, 32, 64])); h, w_ = int(rng.integers(2, 12)), int(rng.integers(2, 12))
-                    k = int(rng.choice([2, 3, 4])); st = int(rng.choice([1, 2])); pad = int(rng.integers(0, k))
-                    s = O.conv_shape(n, c, h, w_, cout, k, k, stride=(st, st), pad=(pad, pad, pad, pad))
+                    groups = int(rng.choice([1, 1, 1, 2]))
+                    c = groups * int(rng.choice([8, 16, 32, 24, 21, 5])); cout = groups * int(rng.choice([8, 16, 20, 32, 21])); h, w_ = int(rng.integers(2, 12)), int(rng.integers(2, 12))
+                    k = int(rng.choice([2, 3, 4, 5, 6, 8])); st = int(rng.choice([1, 2, 2, 3, 4])); pads = tuple(int(v) for v in rng.integers(0, k, 4))
+                    s = O.conv_shape(n, c, h, w_, cout, k, k, stride=(st, st), pad=pads, groups=groups)
                     if min(O.deconv_out_hw(s)) < 1: continue
-                    x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((c, cout, k, k), tseed + 1); b = synth.fill_i32((cout,), tseed + 2, -1000, 1000)
+                    x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((c, cout // groups, k, k), tseed + 1); b = synth.fill_i32((cout,), tseed + 2, -1000, 1000)
                     _, acc = O.deconv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
                     q = centred(acc, zp_in, zp_w, lo, hi)
                     want = O.deconv2d(x, w, b, s, q); got = gpu_deconv(x, w, b, s, to_eh_requant(q), layout=layout); desc = (kind, s, layout)
@@ -65,8 +69,8 @@ def test_random_operator_instances_match_the_oracle(seed):
                         c = int(rng.choice([32, 64, 96, 128])); cout = int(rng.choice([16, 32, 40, 64, 100])); k = 3
                         h, w_ = int(rng.integers(6, 24)), int(rng.integers(8, 40)); st = 1; pads = tuple(int(v) for v in rng.integers(0, 3, 4)); groups = 1; dil = 1
                     else:
-                        groups = int(rng.choice([1, 1, 1, 2, 4])); c = groups * int(rng.choice([1, 3, 4, 8, 16, 20])); cout = groups * int(rng.choice([1, 4, 8, 10, 16]))
-                        k = int(rng.choice([1, 2, 3, 5])); h, w_ = int(rng.integers(k, 20)), int(rng.integers(k, 20)); st = int(rng.choice([1, 2, 3])); pads = tuple(int(v) for v in rng.integers(0, k + 1, 4)); dil = int(rng.choice([1, 1, 2]))
+                        groups = int(rng.choice([1, 1, 1, 2, 4, 8, 16])); c = groups * int(rng.choice([1, 2, 3, 4, 8, 16, 20, 21])); cout = groups * int(rng.choice([1, 3, 4, 8, 10, 16]))
+                        k = int(rng.choice([1, 2, 3, 5, 7])); h, w_ = int(rng.integers(k, 20)), int(rng.integers(k, 20)); st = int(rng.choice([1, 2, 3])); pads = tuple(int(v) for v in rng.integers(0, k + 1, 4)); dil = int(rng.choice([1, 1, 2]))
                     s = O.conv_shape(n, c, h, w_, cout, k, k, stride=(st, st), pad=pads, dil=(dil, dil), groups=groups)
                     if min(O.conv_out_hw(s)) < 1: continue
                     x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((cout, c // groups, k, k), tseed + 1); b = synth.fill_i32((cout,), tseed + 2, -1000, 1000)
