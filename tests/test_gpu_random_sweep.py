@@ -85,3 +85,70 @@ def test_random_operator_instances_match_the_oracle(seed):
             print("MISMATCH", it, desc, q.as_tuple(), diff_report(got, want), flush=True)
     assert bad == 0, "%d of %d random instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
     assert sum(ran.values()) > 300 and all(ran.get(k, 0) > 10 for k in ("conv", "conv1x1", "conv3x3", "dw", "fc", "deconv")), ran
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_perchannel_instances_match_the_oracle(seed):
+    """The same idea for int8 weights with one multiplier and shift per output channel (uint8 tensors): convolution,
+    depthwise convolution and deconvolution over random shapes, channel counts off the multiples of 16 and 4, groups,
+    depth multipliers, both layouts and EXACT_CHANNELS on a fifth of the instances."""
+    eden.init(0)
+    print("random per-channel sweep, seed", seed, flush=True)
+    rng = np.random.default_rng(seed)
+    plans = {"conv": eden.ConvPlan, "dw": eden.DwConvPlan, "deconv": eden.DeconvPlan}
+    ran, bad = {}, 0
+    for it in range(240):
+        kind = str(rng.choice(["conv", "dw", "deconv"]))
+        layout = eden.NHWC if rng.random() < 0.7 else eden.NCHW
+        flags = eden.EXACT_CHANNELS if rng.random() < 0.2 else 0
+        tseed = int(rng.integers(1, 1 << 30))
+        n = int(rng.integers(1, 4))
+        h, w_ = int(rng.integers(3, 16)), int(rng.integers(3, 16))
+        dm = 1
+        if kind == "conv":
+            groups = int(rng.choice([1, 1, 1, 2, 8])); cig = int(rng.choice([3, 4, 8, 16, 21, 32, 64])); cog = int(rng.choice([3, 8, 16, 24]))
+            k = int(rng.choice([1, 1, 3, 3, 5])); st = int(rng.choice([1, 1, 2])); dil = int(rng.choice([1, 1, 2]))
+            pads = tuple(int(v) for v in rng.integers(0, dil * (k - 1) + 1, 4))
+            s = O.conv_shape(n, groups * cig, h, w_, groups * cog, k, k, stride=(st, st), pad=pads, dil=(dil, dil), groups=groups)
+            out_hw, wshape, cout, fan = O.conv_out_hw(s), (groups * cog, cig, k, k), groups * cog, cig * k * k
+        elif kind == "dw":
+            c = int(rng.choice([4, 8, 16, 30, 7, 32])); dm = int(rng.choice([1, 1, 2])); k = int(rng.choice([3, 3, 5])); st = int(rng.choice([1, 2])); dil = int(rng.choice([1, 1, 2]))
+            pads = tuple(int(v) for v in rng.integers(0, dil * (k - 1) + 1, 4))
+            s = O.conv_shape(n, c, h, w_, c * dm, k, k, stride=(st, st), pad=pads, dil=(dil, dil), dm=dm)
+            out_hw, wshape, cout, fan = O.conv_out_hw(s), (c * dm, 1, k, k), c * dm, k * k
+        else:
+            c = int(rng.choice([8, 16, 21, 32])); cout = int(rng.choice([8, 16, 21])); k = int(rng.choice([2, 3, 4, 6])); st = int(rng.choice([1, 2, 3]))
+            pads = tuple(int(v) for v in rng.integers(0, k, 4))
+            s = O.conv_shape(n, c, h // 2 + 1, w_ // 2 + 1, cout, k, k, stride=(st, st), pad=pads)
+            out_hw, wshape, fan = O.deconv_out_hw(s), (c, cout, k, k), c * max(1, (k // st) ** 2)
+        if min(out_hw) < 1:
+            continue
+        x = synth.fill_u8((s.n, s.c, s.h, s.w), tseed)
+        w = (synth.fill_u8(wshape, tseed + 1).astype(np.int16) - 128).astype(np.int8)
+        b = synth.fill_i32((cout,), tseed + 2, -500, 500)
+        w_scales = (0.002 * (1.0 + 29.0 * synth.fill_u8((cout,), tseed + 3) / 255.0)).astype(np.float32)
+        s_out = float(0.02 * float(w_scales.max()) * 74.0 * 74.0 * np.sqrt(fan) / 60.0)
+        zp_in, zp_out = int(rng.integers(0, 256)), int(rng.integers(0, 256))
+        q, mults, shifts = eden.make_requant_perchannel(0.02, zp_in, w_scales, s_out, zp_out, eden.ACT_NONE, False)
+        oq = O.raw_quant(zp_in=zp_in, zp_w=0, zp_out=zp_out)
+        want = {"conv": O.conv2d_perchannel, "dw": O.dwconv2d_perchannel, "deconv": O.deconv2d_perchannel}[kind](x, w, b, s, oq, mults, shifts)
+        weight_layout = (eden.W_IOHW if kind == "deconv" else eden.W_OIHW) | eden.W_SIGNED
+        desc = eden.conv_desc(s.n, s.c, s.h, s.w, cout, s.kh, s.kw, (s.stride_h, s.stride_w), (s.pad_t, s.pad_b, s.pad_l, s.pad_r),
+                              (s.dil_h, s.dil_w), 1 if kind == "dw" else s.groups, dm, layout | flags, weight_layout)
+        x_dev = x if layout == eden.NCHW else x.transpose(0, 2, 3, 1)
+        d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+        d_o = eden.DeviceBuffer(nbytes=want.size)
+        try:
+            plan = plans[kind](desc, d_w, d_b, q)
+            plan.set_perchannel(mults, shifts)
+            plan.run(d_x, d_o, q)
+            got = d_o.download(want.shape) if layout == eden.NCHW else d_o.download((s.n, out_hw[0], out_hw[1], cout)).transpose(0, 3, 1, 2)
+            plan.destroy()
+        except Exception as e:
+            raise AssertionError(("error", seed, it, kind, s, layout, flags, repr(e)[:300]))
+        ran[kind] = ran.get(kind, 0) + 1
+        if not np.array_equal(got, want):
+            bad += 1
+            print("MISMATCH", it, kind, s, layout, flags, diff_report(np.ascontiguousarray(got), want), flush=True)
+    assert bad == 0, "%d of %d random per-channel instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
+    assert all(ran.get(k, 0) > 40 for k in plans), ran
