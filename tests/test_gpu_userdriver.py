@@ -307,3 +307,58 @@ def test_planar_list_with_planar_outputs_of_many_pixels():
             d.set_store_channels_last(True)
             d.set_image_lanes(2, 16)
     assert y3.std() > 5 and y2.std() > 5
+
+
+def test_segmentation_head_with_21_classes_through_the_userdriver():
+    """Channel counts off the multiples of 16 all the way: a 1x1 convolution to 21 class scores, a 3x3 convolution on
+    them and a transposed convolution (4x4, stride 2) that doubles their resolution, as a planar list stored
+    channels-last and stored as it is.  The plans stage channel-padded copies of their inputs; the owner sees none of it."""
+    d = driver()
+    n, c, h, w, classes = 2, 32, 12, 10, 21
+    x = O.fill_u8((n, c, h, w), 911)
+    w1 = O.fill_u8((classes, c, 1, 1), 912)
+    b1 = O.fill_i32((classes,), 913, -500, 500)
+    w2 = O.fill_u8((classes, classes, 3, 3), 914)
+    b2 = O.fill_i32((classes,), 915, -500, 500)
+    w3 = O.fill_u8((classes, classes, 4, 4), 916)      # [cin][cout][kh][kw]
+    b3 = O.fill_i32((classes,), 917, -500, 500)
+    s_in, z_in, s_w, z_w = 0.02, 120, 0.005, 131
+    s1 = float(0.02 * 0.005 * 74.0 * 74.0 * np.sqrt(c) / 40.0)
+    s2 = float(s1 * 0.005 * 74.0 * 74.0 * np.sqrt(9 * classes) / 40.0)
+    s3 = float(s2 * 0.005 * 74.0 * 74.0 * np.sqrt(4 * classes) / 40.0)
+    q1 = O.make_quant(s_in, z_in, s_w, z_w, s1, 128, O.ACT_NONE, False)
+    q2 = O.make_quant(s1, 128, s_w, z_w, s2, 128, O.ACT_NONE, False)
+    q3 = O.make_quant(s2, 128, s_w, z_w, s3, 128, O.ACT_NONE, False)
+    y1 = O.conv2d(x, w1, b1, O.conv_shape(n, c, h, w, classes, 1, 1), q1)
+    y2 = O.conv2d(y1, w2, b2, O.conv_shape(n, classes, h, w, classes, 3, 3, pad=(1, 1, 1, 1)), q2)
+    y3 = O.deconv2d(y2, w3, b3, O.conv_shape(n, classes, h, w, classes, 4, 4, stride=(2, 2), pad=(1, 1, 1, 1)), q3)
+    assert y3.shape == (n, classes, 2 * h, 2 * w) and y3.std() > 5
+    for stored in (True, False):
+        list_id = 0xB100 + (1 if stored else 0)
+        d.set_store_channels_last(stored)
+        d.set_image_lanes(1, 16)
+        try:
+            ol = ud.OperatorList(list_id, ud.MODEL_ANDROID_NN)
+            t0 = ol.feature_map(0, (n, c, h, w), s_in, z_in)
+            t1 = ol.feature_map(1, (n, classes, h, w), s1, 128)
+            t2 = ol.feature_map(2, (n, classes, h, w), s2, 128)
+            t3 = ol.feature_map(3, (n, classes, 2 * h, 2 * w), s3, 128)
+            valid = ud.options(padding=ud.PADDING_VALID, use_nchw=True)
+            pad1 = ud.options(padding=ud.PADDING_VALID, padding_value=(1, 1, 1, 1), use_nchw=True)
+            up = ud.options(padding=ud.PADDING_VALID, padding_value=(1, 1, 1, 1), stride=(2, 2), use_nchw=True)
+            ol.operator("SCORE", ud.OP_CONV_2D, [t0, ol.parameter(np.ascontiguousarray(w1.transpose(0, 2, 3, 1)), s_w, z_w),
+                                                ol.parameter(b1, s_in * s_w, 0)], [t1], valid)
+            ol.operator("REFINE", ud.OP_CONV_2D, [t1, ol.parameter(np.ascontiguousarray(w2.transpose(0, 2, 3, 1)), s_w, z_w),
+                                                 ol.parameter(b2, s1 * s_w, 0)], [t2], pad1)
+            ol.operator("UPSAMPLE", ud.OP_TRANSPOSE_CONV, [t2, ol.parameter(np.ascontiguousarray(w3.transpose(1, 2, 3, 0)), s_w, z_w),
+                                                          ol.parameter(b3, s2 * s_w, 0)], [t3], up)
+            d.open_subgraph(ol)
+            got = np.zeros((n, classes, 2 * h, 2 * w), np.uint8)
+            for rep in range(3):
+                got[:] = 0
+                d.execute_subgraph(list_id, {0: x, 3: got})
+                assert np.array_equal(got, y3), (stored, rep, int((got != y3).sum()))
+            d.close_subgraph(list_id)
+        finally:
+            d.set_store_channels_last(True)
+            d.set_image_lanes(2, 16)
