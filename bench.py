@@ -490,7 +490,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--no-others", action="store_true", help="time the headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the oracle check of the network")
-    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2 (two lanes, measured pairs fused), mbv2plain / mbv2lanes / mbv2fused (neither / lanes only / fusion only), mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, dwdil2, conv21, deconv21 (an atrous depthwise layer and a 21-class segmentation head), copy, tonhwc, tonchw, feedprobe (what a CU's matrix pipe can be fed with, per tile shape)")
+    ap.add_argument("--only", default=None, help="time one named workload family only: fc, fcbig, conv, conv64, dw, dwbig, pw, pwbig, deconv, mbv2 (two lanes, measured pairs fused), mbv2plain / mbv2lanes / mbv2fused (neither / lanes only / fusion only), mbv2ud (the same through the operator API), mbv2narrow, mbv2pc, mbv2udpc, mbv2b1 / mbv2b8 (the network at batch 1 and 8, one chain: latency), dwdil2, conv21, deconv21 (an atrous depthwise layer and a 21-class segmentation head), copy, tonhwc, tonchw, feedprobe (what a CU's matrix pipe can be fed with, per tile shape)")
     ap.add_argument("--tile", default=None, help="with --only c3block / block:...: ROWSxCOLS output pixels per workgroup (default: chosen by the library)")
     ap.add_argument("--cold", action="store_true", help="with --only: rotate over buffer sets that together exceed the Infinity Cache")
     args = ap.parse_args()
@@ -520,6 +520,7 @@ def main():
                     dwdil2=shaped(dw_workload, n=64, c=144, hw=56, stride=1, k=3, dil=2), conv21=shaped(conv_workload, n=8, cin=21, cout=21, hw=64, k=3, stride=1),
                     deconv21=shaped(deconv_workload, n=1, cin=21, cout=21, hw=64, k=16, stride=8),
                     copy=copy_workload, mbv2=mbv2_workload, mbv2narrow=shaped(mbv2_workload, weights="narrow"),
+                    mbv2b1=shaped(mbv2_workload, batch=1, lanes=1), mbv2b8=shaped(mbv2_workload, batch=8, lanes=1),
                     tonhwc=layout_workload, tonchw=shaped(layout_workload, to_nhwc=False),
                     mbv2pc=shaped(mbv2_workload, per_channel=True),
                     mbv2plain=shaped(mbv2_workload, lanes=1, fuse_blocks=()), mbv2lanes=shaped(mbv2_workload, fuse_blocks=()),

@@ -372,15 +372,18 @@ int eh_dwconv2d_u8_destroy(eh_dwconv_plan *plan);
  * pointwise layer of at most 256 input channels (a multiple of 8) whose output is the depthwise input, depthwise 3x3 at
  * stride 1 or 2 without dilation or depth multiplier on a multiple of 16 channels, requantization per tensor in both or per channel in both.
  * `_preferred` says whether the one launch is also the faster choice for the pair's shape (1) or the two launches
- * are (0): a table of shapes timed inside a network, kept beside the kernel; a caller that fuses wherever
- * `_preferred` says so never loses to the two launches on a measured shape, and unmeasured shapes stay unfused.
+ * are (0): below 32 images per launch every fitting pair (a launch is mostly latency there, and a whole network
+ * measured faster with all of them fused at every batch from 1 to 24); from 32 images on a table of shapes timed
+ * inside a network, kept beside the kernel: a caller that fuses wherever `_preferred` says so never loses to the
+ * two launches on a measured shape, and unmeasured shapes stay unfused.
  * rows_per_tile, cols_per_tile: the tile of output pixels a workgroup owns, 0 lets the library choose.
  * q_pointwise->zp_out must equal q_depthwise->zp_in (they describe the same tensor). */
 int eh_conv_dw_block_applies(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise);
 int eh_conv_dw_block_preferred(const eh_conv_plan *pointwise, const eh_dwconv_plan *depthwise);
 /* The table alone, for a caller that has to decide before the plans exist (an operator constructor that does not
  * give the expanded tensor any storage): images per launch, the square image's extent, pointwise input channels,
- * expanded channels, depthwise stride.  `_preferred` is `_applies` and this. */
+ * expanded channels, depthwise stride.  `_preferred` is `_applies` and this (below 32 images it is 1 for every
+ * shape: whether the pair fits is `_applies`' business). */
 int eh_conv_dw_block_listed(int32_t images, int32_t image_h, int32_t image_w, int32_t in_channels, int32_t expanded_channels, int32_t stride);
 int eh_conv_dw_block_run(eh_conv_plan *pointwise, eh_dwconv_plan *depthwise, const void *input, void *output,
                          const eh_requant *q_pointwise, const eh_requant *q_depthwise, int32_t rows_per_tile, int32_t cols_per_tile,

@@ -179,7 +179,9 @@ def test_block_preferred_is_a_subset_of_applies_and_holds_config3():
         return pw, dw, (d_w, d_b, d_w2)
     for shape, applies, preferred in (((32, 24, 144, 56, 2), True, True), ((32, 24, 144, 56, 1), True, False),
                                       ((32, 40, 80, 20, 1), True, False), ((32, 64, 384, 14, 1), True, True),
-                                      ((2, 24, 144, 56, 2), True, False), ((32, 320, 64, 8, 1), False, False)):
+                                      # below 32 images per launch every fitting pair is preferred (latency), none that does not fit
+                                      ((2, 24, 144, 56, 2), True, True), ((8, 40, 80, 20, 1), True, True), ((24, 24, 144, 56, 1), True, True),
+                                      ((4, 320, 64, 8, 1), False, False), ((32, 320, 64, 8, 1), False, False)):
         pw, dw, keep = pair(*shape)
         assert eden.conv_dw_block_applies(pw, dw) == applies, shape
         assert eden.conv_dw_block_preferred(pw, dw) == preferred, shape

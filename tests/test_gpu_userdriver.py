@@ -37,7 +37,8 @@ def test_mobilenet_v2_through_open_execute_close(batch, image, per_channel, fuse
     ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image, per_channel=per_channel)
     d.open_subgraph(ol, fuse_residual_adds=fuse)
     before = d.stats(list_id)
-    assert before["operators"] == (54 if fuse else 64)   # ten residual adds ride in their convolutions' launches
+    # ten residual adds ride in their convolutions' launches; below 32 images all sixteen expansion + depthwise pairs are one launch each
+    assert before["operators"] == (54 if fuse else 64) - 16
     x = mobilenet.network_input(batch, image)
     _, _, want = oracle_images(batch, image, per_channel)
     ref = want[-1].reshape(batch, -1)
@@ -93,7 +94,7 @@ def test_image_lanes_give_the_same_logits(lanes, batch, replay):
     try:
         ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image)
         d.open_subgraph(ol)
-        assert d.stats(list_id)["operators"] == lanes * 54
+        assert d.stats(list_id)["operators"] == lanes * 38
         x = mobilenet.network_input(batch, image)
         _, _, want = oracle_images(batch, image, False)
         ref = want[-1].reshape(batch, -1)
@@ -110,7 +111,7 @@ def test_image_lanes_give_the_same_logits(lanes, batch, replay):
             d.set_image_lanes(4, 1)
             ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id + 1, batch, image)
             d.open_subgraph(ol)
-            assert d.stats(list_id + 1)["operators"] == 54
+            assert d.stats(list_id + 1)["operators"] == 38
             got = np.zeros(shape, np.uint8)
             d.execute_subgraph(list_id + 1, {in_index: x, out_index: got})
             assert np.array_equal(got, ref)
@@ -129,7 +130,7 @@ def test_every_fitting_expansion_fused_with_its_depthwise_convolution():
     ref = want[-1].reshape(batch, -1)
     x = mobilenet.network_input(batch, image)
     try:
-        for mode, lanes, operators in ((2, 2, 2 * 38), (2, 1, 38), (0, 1, 54), (1, 1, 54)):   # (mode 1: four images are below the table's floor)
+        for mode, lanes, operators in ((2, 2, 2 * 38), (2, 1, 38), (0, 1, 54), (1, 1, 38)):   # (mode 1: below 32 images every fitting pair is preferred)
             d.set_fuse_expansions(mode)
             d.set_image_lanes(lanes, 1)
             ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image)
@@ -247,7 +248,8 @@ def test_planar_list_stored_channels_last_gives_the_planar_results(batch, lanes)
             d.set_store_channels_last(stored)
             ol, in_index, out_index, shape = mobilenet.operator_list(ud, list_id, batch, image, nchw=True)
             d.open_subgraph(ol)
-            assert d.stats(list_id)["operators"] == lanes * 54 + extra
+            # (planar operators stay one per description: the fused launch works on channels-last tensors)
+            assert d.stats(list_id)["operators"] == lanes * (38 if stored else 54) + extra
             for rep in range(3):
                 got = np.zeros(shape, np.uint8)
                 d.execute_subgraph(list_id, {in_index: x, out_index: got})

@@ -1309,6 +1309,7 @@ static int gpu_tests() {
             op_desc("DEPTHWISE_CONV_2D", 2, TFlite::BuiltinOperator_DEPTHWISE_CONV_2D,
                     {f1, param("wd", {1, 3, 3, 48}, wd.data(), TFlite::TensorType_UINT8, sw, 131), param("bd", {48}, bd.data(), TFlite::TensorType_INT32, s1 * sw, 0)}, {f2}, dw_opt),
         };
+        ud.constructor()->fuse_expansions = false;   // this test counts operators: one per description (two images would fuse the pair)
         EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS);
         EXPECT(ud.OpenSubGraph(list) == ENN_RET_FAILED);   // open already
         EXPECT(ud.PrepareSubGraph(list.id) == ENN_RET_SUCCESS);
@@ -1370,8 +1371,9 @@ static int gpu_tests() {
         ud.constructor()->image_lanes = 3;
         EXPECT(ud.OpenSubGraph(list) == ENN_RET_SUCCESS && ud.constructor()->lanes() == 1);
         EXPECT(ud.CloseSubGraph(list.id) == ENN_RET_SUCCESS);
-        // the pair as one launch (the shape is not in the library's table, so only on request), alone and in two lanes:
-        // one operator per lane, the expanded tensor without storage, results unchanged
+        // the pair as one launch, alone and in two lanes: one operator per lane, the expanded tensor without storage,
+        // results unchanged
+        ud.constructor()->fuse_expansions = true;
         ud.constructor()->fuse_unlisted_expansions = true;
         for (const int lanes : {1, 2}) {
             ud.constructor()->image_lanes = lanes;
