@@ -502,10 +502,10 @@ struct GemmOp {
         return EH_OK;
     }
 
-    // the one-tap kernel and the split-reduction epilogue of the tiled kernel can add a residual tensor
+    // the one-tap kernel, the split-reduction epilogue of the tiled kernel and the kernel for few rows can add a residual tensor
     bool fuses_add() const {
         bool fuse = layout == EH_NHWC && !io_signed && !parts.empty();
-        for (auto &g : parts) fuse = fuse && (g.cfg.id == GEMM_THIN || g.cfg.id == GEMM_DMA_64x64_SPLITK);
+        for (auto &g : parts) fuse = fuse && (g.cfg.id == GEMM_THIN || g.cfg.id == GEMM_DMA_64x64_SPLITK || g.cfg.id == GEMM_SKINNY);
         return fuse;
     }
 

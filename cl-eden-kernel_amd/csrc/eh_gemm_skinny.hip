@@ -96,6 +96,11 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_gemm_kernel(const GemmProb
     if (wave >= G) return;
     const int g = wave;  // wave 0 finishes rows 0 .. 31, wave 1 rows 32 .. 63
     const int n = nb * 32 + half * 16;  // this lane's sixteen consecutive channels
+    // the sixteen residual bytes these outputs are added to, requested before the requantization that hides their way
+    u32x4_a4 res4 = u32x4_a4{0, 0, 0, 0};
+    const bool res_vec = p.residual != nullptr && g * 32 + r < p.m && n + 16 <= p.n && (p.ldc & 3) == 0 &&
+                         (reinterpret_cast<uintptr_t>(p.residual) & 3) == 0;
+    if (res_vec) res4 = *reinterpret_cast<const u32x4_a4 *>(p.residual + (size_t)(g * 32 + r) * (size_t)p.ldc + n);
     int ncorr = 0;
     if constexpr (ROWSUM) {
         int rs = part_s[g][16][lane];
@@ -151,6 +156,18 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_gemm_kernel(const GemmProb
     if (row < p.m && n < p.n) {
         uint8_t *dst = p.out + (size_t)row * (size_t)p.ldc + n;
         const int cnt = p.n - n;
+        if (p.residual) {  // out = add(residual, result)
+            if (res_vec) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) packed[q4] = add_word(res4[q4], packed[q4], p.radd);
+            } else {
+                const uint8_t *res = p.residual + (size_t)row * (size_t)p.ldc + n;
+                for (int t = 0; t < (cnt < 16 ? cnt : 16); ++t) {
+                    const uint32_t v = add_one(res[t], (packed[t >> 2] >> (8 * (t & 3))) & 255u, p.radd);
+                    packed[t >> 2] = (packed[t >> 2] & ~(255u << (8 * (t & 3)))) | (v << (8 * (t & 3)));
+                }
+            }
+        }
         if (cnt >= 16 && (p.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 3) == 0) {
             *reinterpret_cast<u32x4_a4 *>(dst) = u32x4_a4{packed[0], packed[1], packed[2], packed[3]};
         } else {
@@ -175,7 +192,6 @@ int launch_gemm_skinny(const GemmProblem &p, hipStream_t stream) {
     EH_REQUIRE(p.m >= 1 && p.m <= 64 && p.k_pad % 32 == 0 && p.k_pad >= p.k && (p.k & 15) == 0 && (p.cin & 15) == 0 && (p.a_offset & 15) == 0,
                "gemm_skinny: %d rows, reduction %d (padded %d), row stride %d", p.m, p.k, p.k_pad, p.cin);
     EH_REQUIRE((reinterpret_cast<uintptr_t>(p.a) & 15) == 0, "gemm_skinny: the activations must start on a 16-byte boundary");
-    EH_REQUIRE(p.residual == nullptr, "gemm_skinny: no fused residual add");
     // pixel m of the problem is row m of a matrix: stride 1, no offsets, dense output
     EH_REQUIRE(p.stride_h == 1 && p.stride_w == 1 && p.y_base == 0 && p.x_base == 0 && p.h == p.ho && p.w == p.wo && p.out_sy == 1 && p.out_sx == 1 &&
                    p.out_y0 == 0 && p.out_x0 == 0 && p.out_h == p.ho && p.out_w == p.wo,

@@ -109,6 +109,9 @@ RUN_ADD_CASES = [
     # one-tap kernel (fused), split-reduction tiles (fused), 128 x 128 tiles and the register-staged kernel (second launch)
     dict(n=2, c=144, h=14, w=14, cout=24, kh=1, kw=1, fused=True),
     dict(n=2, c=32, h=9, w=9, cout=40, kh=1, kw=1, fused=True),
+    # at most 64 pixels under a long reduction (the 7 x 7 stage of an image network at batch 1): the kernel cut along the weights adds the residual too
+    dict(n=1, c=960, h=7, w=7, cout=160, kh=1, kw=1, fused=True),
+    dict(n=2, c=512, h=5, w=5, cout=50, kh=1, kw=1, fused=True),
     dict(n=4, c=384, h=14, w=14, cout=64, kh=1, kw=1, fused=True),
     dict(n=2, c=576, h=7, w=7, cout=96, kh=1, kw=1, fused=True),
     dict(n=32, c=264, h=28, w=28, cout=256, kh=1, kw=1, fused=False),
