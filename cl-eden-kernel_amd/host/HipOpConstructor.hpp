@@ -241,7 +241,10 @@ public:
     // (MobileNetV2 at 64 images: 490 -> 444 us per execution; four lanes of 16 images lose more in their smaller
     // launches than they gain).  1 = one operator per description, as the reference builds the list.
     int image_lanes = 2;
-    int min_lane_images = 16;
+    // (from 12 images per lane on two lanes win: MobileNetV2 at batch 24 309 against 327 us, at 32 338 against 352;
+    // at batch 16 they tie and below that the lanes' launches no longer overlap and two lanes cost 282 against 248 us at
+    // batch 8, 271 against 195 at batch 2)
+    int min_lane_images = 12;
     // A uint8 1x1 CONV_2D whose only reader is a 3x3 DEPTHWISE_CONV_2D (an inverted-residual block's expansion) runs
     // with it as one launch where the library's table of measured shapes says that is the faster way
     // (eh_conv_dw_block_listed); the tensor between them then has no storage at all.  false = one operator per

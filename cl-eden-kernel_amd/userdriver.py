@@ -160,7 +160,7 @@ class UserDriver:
     def set_replay(self, on):
         check(load().eud_set_replay(self.h, int(on)))
 
-    def set_image_lanes(self, lanes, min_lane_images=16):
+    def set_image_lanes(self, lanes, min_lane_images=12):
         """Lists opened from now on run as `lanes` chains of images side by side when a chain gets min_lane_images or more."""
         check(load().eud_set_image_lanes(self.h, lanes, min_lane_images), "set_image_lanes")
 

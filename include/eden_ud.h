@@ -95,7 +95,7 @@ int eud_execute_operators(eud_driver *driver, uint64_t list_id, int32_t times);
 int eud_set_replay(eud_driver *driver, int32_t replay);
 /* Lists opened from now on whose feature maps all carry the same number of images are built `lanes` times over, each
  * on 1 / lanes of the images, and the lanes run side by side on streams of their own (parallel branches of the recorded
- * graph), when a share holds at least min_lane_images images.  Default 2 lanes from 16 images per lane; lanes = 1 builds
+ * graph), when a share holds at least min_lane_images images.  Default 2 lanes from 12 images per lane; lanes = 1 builds
  * one operator per description as the reference does.  Results do not depend on it. */
 int eud_set_image_lanes(eud_driver *driver, int32_t lanes, int32_t min_lane_images);
 /* Lists opened from now on: a uint8 1x1 CONV_2D whose only reader is a 3x3 DEPTHWISE_CONV_2D runs with it as one launch

@@ -117,7 +117,7 @@ def test_image_lanes_give_the_same_logits(lanes, batch, replay):
             assert np.array_equal(got, ref)
             d.close_subgraph(list_id + 1)
     finally:
-        d.set_image_lanes(2, 16)
+        d.set_image_lanes(2, 12)
         d.set_replay(True)
 
 
@@ -143,7 +143,7 @@ def test_every_fitting_expansion_fused_with_its_depthwise_convolution():
             d.close_subgraph(list_id)
     finally:
         d.set_fuse_expansions(1)
-        d.set_image_lanes(2, 16)
+        d.set_image_lanes(2, 12)
 
 
 def test_quantization_parameters_changed_between_executions_are_honoured():
@@ -257,7 +257,7 @@ def test_planar_list_stored_channels_last_gives_the_planar_results(batch, lanes)
             d.close_subgraph(list_id)
     finally:
         d.set_store_channels_last(True)
-        d.set_image_lanes(2, 16)
+        d.set_image_lanes(2, 12)
 
 
 def test_planar_list_with_planar_outputs_of_many_pixels():
@@ -307,7 +307,7 @@ def test_planar_list_with_planar_outputs_of_many_pixels():
             d.close_subgraph(list_id)
         finally:
             d.set_store_channels_last(True)
-            d.set_image_lanes(2, 16)
+            d.set_image_lanes(2, 12)
     assert y3.std() > 5 and y2.std() > 5
 
 
@@ -363,4 +363,4 @@ def test_segmentation_head_with_21_classes_through_the_userdriver():
             d.close_subgraph(list_id)
         finally:
             d.set_store_channels_last(True)
-            d.set_image_lanes(2, 16)
+            d.set_image_lanes(2, 12)
