@@ -673,6 +673,8 @@ def main():
                                       (stream_workload, 500, True), (shaped(stream_workload, out_bytes=256 * 56 * 56 * 144), 100, True),
                                       (shaped(stream_workload, mode=2, out_bytes=32 * 28 * 28 * 144), 500, True),
                                       (shaped(stream_workload, mode=2, out_bytes=256 * 28 * 28 * 144), 100, True),
+                                      # the network's latency: one image, and eight, as one chain
+                                      (shaped(mbv2_workload, batch=1, lanes=1), 200, False), (shaped(mbv2_workload, batch=8, lanes=1), 200, False),
                                       (shaped(mbv2_workload, weights="narrow"), 40, False),
                                       (shaped(mbv2_workload, per_channel=True), 40, False)):
             others.append(measure(eden, synth, stream, make, steps, max(4, steps // 10), use_graph, cold_too))
