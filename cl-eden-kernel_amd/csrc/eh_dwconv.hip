@@ -682,7 +682,6 @@ int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
     DwProblem p = caller_p;
     const bool pc_two_step = p.rq.pc_multiplier != nullptr && !p.rq.fast;
     if (p.w_trip || pc_two_step) p.w_fold = nullptr;  // the signed form where it applies; per-channel pairs outside the single-shift range use the 16-bit kernel
-    if (p.w_fold) p.zp_w += p.w_signed ? 128 : 0;     // zero point of the uint8 values the unsigned form multiplies
     const long outs = (long)p.n * p.ho * p.wo * p.cout;
     if (outs <= 0) return EH_OK;
     const bool vec = p.dm == 1 && (p.c & 3) == 0 && (reinterpret_cast<uintptr_t>(p.in) & 3) == 0 &&
@@ -719,6 +718,9 @@ int launch_dwconv_nhwc(const DwProblem &caller_p, hipStream_t stream) {
         return EH_OK;
     }
     if (tile3x3) {
+        // zero point of the uint8 values the unsigned form multiplies (only here: the one-output-per-thread kernel reads
+        // the weights as the caller quantized them)
+        if (p.w_fold) p.zp_w += p.w_signed ? 128 : 0;
         const int tiles_x = (p.wo + 3) / 4;
         const long total = (long)p.n * p.ho * tiles_x * (p.c >> 2);
         const long blocks = (total + 255) / 256;

@@ -122,6 +122,26 @@ def test_int8_depthwise_matches_oracle(case, layout):
         assert want.std() > 4
 
 
+@pytest.mark.parametrize("case", [DW_CASES[-1],
+                                  dict(n=3, c=7, h=14, w=11, cout=7, kh=3, kw=3, stride=(2, 2), pad=(1, 2, 0, 0)),
+                                  dict(n=3, c=7, h=9, w=4, cout=7, kh=3, kw=3, stride=(2, 2), pad=(4, 1, 2, 0), dil=(2, 2))],
+                         ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
+def test_int8_depthwise_on_ragged_channels_without_staging(case):
+    """Channels-last 3x3 with a channel count that is no multiple of four and the plan told not to stage: the kernel
+    with one output per thread runs, and reads the weights about the zero point the caller gave (the plan also holds
+    the dot-product form of the weights, whose zero point is shifted by 128 for int8 weights)."""
+    print("int8 depthwise, ragged channels unstaged", case, flush=True)
+    s = O.conv_shape(**case)
+    x, w = s8((s.n, s.c, s.h, s.w), SEED + 61), s8((s.c, 1, s.kh, s.kw), SEED + 62)
+    b = synth.fill_i32((s.c,), SEED + 63, -500, 500)
+    ho, wo = O.conv_out_hw(s)
+    q, oq = quant_pair(s.kh * s.kw, eden.ACT_NONE, False, zp_out=-3)
+    want = O.dwconv2d_s8(x, w, b, s, oq)
+    got = run_conv(eden.DwConvPlan, None, x, w, b, s, q, (s.n, s.c, ho, wo), eden.NHWC | eden.EXACT_CHANNELS, eden.W_OIHW)
+    assert np.array_equal(got, want), int((got != want).sum())
+    assert want.std() > 4
+
+
 @pytest.mark.parametrize("case", DW_CASES[:2] + DW_CASES[-4:] + [dict(n=40, c=64, h=64, w=64, cout=64, kh=3, kw=3, stride=(1, 1), pad=(1, 1, 1, 1))],
                          ids=lambda c: "x".join(str(v) for v in list(c.values())[:7]))
 def test_int8_depthwise_weights_within_int8_of_their_zero_point(case):

@@ -152,3 +152,87 @@ def test_random_perchannel_instances_match_the_oracle(seed):
             print("MISMATCH", it, kind, s, layout, flags, diff_report(np.ascontiguousarray(got), want), flush=True)
     assert bad == 0, "%d of %d random per-channel instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
     assert all(ran.get(k, 0) > 40 for k in plans), ran
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_int8_instances_match_the_oracle(seed):
+    """And for INT8 precision (int8 tensors and weights, zero points in [-128, 127]): the same kernels behind a sign flip
+    on the way in and out, so what has to hold is that every staged copy, padding byte and zero-point constant is
+    flipped too.  Convolution, depthwise convolution, deconvolution and fully connected layers over random shapes."""
+    eden.init(0)
+    print("random int8 sweep, seed", seed, flush=True)
+    rng = np.random.default_rng(seed)
+    s8 = lambda shape, sd: (synth.fill_u8(shape, sd).astype(np.int16) - 128).astype(np.int8)
+    plans = {"conv": eden.ConvPlan, "dw": eden.DwConvPlan, "deconv": eden.DeconvPlan}
+    oracles = {"conv": O.conv2d_s8, "dw": O.dwconv2d_s8, "deconv": O.deconv2d_s8}
+    ran, bad = {}, 0
+    for it in range(240):
+        kind = str(rng.choice(["conv", "dw", "deconv", "fc"]))
+        layout = eden.NHWC if rng.random() < 0.7 else eden.NCHW
+        flags = eden.EXACT_CHANNELS if rng.random() < 0.2 else 0
+        tseed = int(rng.integers(1, 1 << 30))
+        zp_in, zp_w, zp_out = int(rng.integers(-128, 128)), int(rng.integers(-20, 21)), int(rng.integers(-128, 128))
+        act, enabled = (eden.ACT_RELU6, True) if rng.random() < 0.3 else (eden.ACT_NONE, False)
+        s_in, s_w = 0.02, 0.005
+        if kind == "fc":
+            m, k, n = int(rng.integers(1, 200)), int(rng.choice([16, 37, 64, 100, 256, 1001])), int(rng.integers(1, 200))
+            s_out = float(s_in * s_w * 74.0 * 74.0 * np.sqrt(k) / 50.0)
+            q = eden.make_requant_s8(s_in, zp_in, s_w, zp_w, s_out, zp_out, act, enabled)
+            oq = O.make_quant_s8(s_in, zp_in, s_w, zp_w, s_out, zp_out, act, enabled)
+            a, w, b = s8((m, k), tseed), s8((n, k), tseed + 1), synth.fill_i32((n,), tseed + 2, -500, 500)
+            want = O.fc_s8(a, w, b, oq)
+            d_a, d_w, d_b, d_o = eden.DeviceBuffer(host=a), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b), eden.DeviceBuffer(nbytes=m * n)
+            plan = eden.FcPlan(m, k, n, d_w, d_b, q, flags=eden.W_SIGNED | eden.IO_SIGNED | flags)
+            plan.run(d_a, d_o, q)
+            got = d_o.download((m, n)).view(np.int8)
+            plan.destroy()
+            desc_txt = (m, k, n)
+        else:
+            n = int(rng.integers(1, 4))
+            h, w_ = int(rng.integers(3, 16)), int(rng.integers(3, 16))
+            dm = 1
+            if kind == "conv":
+                groups = int(rng.choice([1, 1, 1, 2, 8])); cig = int(rng.choice([3, 4, 8, 16, 21, 32, 64])); cog = int(rng.choice([3, 8, 16, 24]))
+                k = int(rng.choice([1, 1, 3, 3, 5])); st = int(rng.choice([1, 1, 2])); dil = int(rng.choice([1, 1, 2]))
+                pads = tuple(int(v) for v in rng.integers(0, dil * (k - 1) + 1, 4))
+                s = O.conv_shape(n, groups * cig, h, w_, groups * cog, k, k, stride=(st, st), pad=pads, dil=(dil, dil), groups=groups)
+                out_hw, wshape, cout, fan = O.conv_out_hw(s), (groups * cog, cig, k, k), groups * cog, cig * k * k
+            elif kind == "dw":
+                c = int(rng.choice([4, 8, 16, 30, 7, 32])); dm = int(rng.choice([1, 1, 2])); k = int(rng.choice([3, 3, 5])); st = int(rng.choice([1, 2])); dil = int(rng.choice([1, 1, 2]))
+                pads = tuple(int(v) for v in rng.integers(0, dil * (k - 1) + 1, 4))
+                s = O.conv_shape(n, c, h, w_, c * dm, k, k, stride=(st, st), pad=pads, dil=(dil, dil), dm=dm)
+                out_hw, wshape, cout, fan = O.conv_out_hw(s), (c * dm, 1, k, k), c * dm, k * k
+            else:
+                c = int(rng.choice([8, 16, 21, 32])); cout = int(rng.choice([8, 16, 21])); k = int(rng.choice([2, 3, 4, 6])); st = int(rng.choice([1, 2, 3]))
+                pads = tuple(int(v) for v in rng.integers(0, k, 4))
+                s = O.conv_shape(n, c, h // 2 + 1, w_ // 2 + 1, cout, k, k, stride=(st, st), pad=pads)
+                out_hw, wshape, fan = O.deconv_out_hw(s), (c, cout, k, k), c * max(1, (k // st) ** 2)
+            if min(out_hw) < 1:
+                continue
+            s_out = float(s_in * s_w * 74.0 * 74.0 * np.sqrt(fan) / 50.0)
+            q = eden.make_requant_s8(s_in, zp_in, s_w, zp_w, s_out, zp_out, act, enabled)
+            oq = O.make_quant_s8(s_in, zp_in, s_w, zp_w, s_out, zp_out, act, enabled)
+            x, w, b = s8((s.n, s.c, s.h, s.w), tseed), s8(wshape, tseed + 1), synth.fill_i32((cout,), tseed + 2, -500, 500)
+            want = oracles[kind](x, w, b, s, oq)
+            weight_layout = (eden.W_IOHW if kind == "deconv" else eden.W_OIHW) | eden.W_SIGNED
+            desc = eden.conv_desc(s.n, s.c, s.h, s.w, cout, s.kh, s.kw, (s.stride_h, s.stride_w), (s.pad_t, s.pad_b, s.pad_l, s.pad_r),
+                                  (s.dil_h, s.dil_w), 1 if kind == "dw" else s.groups, dm, layout | flags | eden.IO_SIGNED, weight_layout)
+            x_dev = x if layout == eden.NCHW else x.transpose(0, 2, 3, 1)
+            d_x, d_w, d_b = eden.DeviceBuffer(host=x_dev), eden.DeviceBuffer(host=w), eden.DeviceBuffer(host=b)
+            d_o = eden.DeviceBuffer(nbytes=want.size)
+            try:
+                plan = plans[kind](desc, d_w, d_b, q)
+                plan.run(d_x, d_o, q)
+                raw = d_o.download(want.shape) if layout == eden.NCHW else d_o.download((s.n, out_hw[0], out_hw[1], cout)).transpose(0, 3, 1, 2)
+                plan.destroy()
+            except Exception as e:
+                raise AssertionError(("error", seed, it, kind, s, layout, flags, repr(e)[:300]))
+            got = np.ascontiguousarray(raw).view(np.int8)
+            desc_txt = (dict(n=s.n, c=s.c, h=s.h, w=s.w, cout=cout, k=s.kh, stride=s.stride_h, pad=(s.pad_t, s.pad_b, s.pad_l, s.pad_r), dil=s.dil_h, groups=s.groups, dm=dm),
+                        layout, flags, (zp_in, zp_w, zp_out), act)
+        ran[kind] = ran.get(kind, 0) + 1
+        if not np.array_equal(got, want):
+            bad += 1
+            print("MISMATCH", it, kind, desc_txt, int((got != want).sum()), flush=True)
+    assert bad == 0, "%d of %d random int8 instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
+    assert all(ran.get(k, 0) > 30 for k in ("conv", "dw", "deconv", "fc")), ran
