@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from harness import diff_report, eden, gpu_conv, gpu_deconv, gpu_dwconv, gpu_fc, synth, to_eh_requant
+from harness import diff_report, eden, gpu_conv, gpu_deconv, gpu_dwconv, gpu_fc, synth, to_eh_add, to_eh_requant
 
 pytestmark = pytest.mark.gpu
 
@@ -236,3 +236,128 @@ def test_random_int8_instances_match_the_oracle(seed):
             print("MISMATCH", it, kind, desc_txt, int((got != want).sum()), flush=True)
     assert bad == 0, "%d of %d random int8 instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
     assert all(ran.get(k, 0) > 30 for k in ("conv", "dw", "deconv", "fc")), ran
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_random_network_sized_instances_match_the_oracle(seed):
+    """The sweeps above keep to small tensors, which the small tiles serve.  This one draws layer shapes of the sizes image
+    networks have (up to 1280 channels, 112 x 112 pixels, batch 32, reductions up to 9216 long), so that every tile
+    size, the sliced reductions, the one-tap and patch kernels and the wide depthwise tiles are chosen by the same
+    selection code that serves a real model; weight layouts vary too, and a convolution is run in one of four ways: as
+    planned, with requantization parameters that differ from the ones it was planned with, with a residual added, or
+    through the entry point that allocates nothing."""
+    eden.init(0)
+    print("random network-sized sweep, seed", seed, flush=True)
+    rng = np.random.default_rng(seed)
+    pick = lambda *v: v[int(rng.integers(0, len(v)))]
+    jitter = lambda v: max(1, v + int(rng.integers(-1, 2)))
+    def centred(acc, zp_in, zp_w):
+        sd = float(acc.std()) or 1.0
+        qm, sh = O.quantize_multiplier(float(pick(20.0, 40.0, 80.0)) / sd)
+        zp_out = int(np.clip(128 - round(float(acc.mean()) * 40.0 / sd), 0, 255))
+        return O.raw_quant(zp_in=zp_in, zp_w=zp_w, zp_out=zp_out, multiplier=qm, shift=sh, act_min=pick(0, 0, 30), act_max=pick(255, 255, 200))
+    ran, kernels, modes, bad = {}, set(), {}, 0
+    for it in range(110):
+        kind = pick("pw", "pw", "conv3x3", "conv3x3", "convk", "grouped", "dw", "dw", "deconv", "fc")
+        zp_in, zp_w = int(rng.integers(0, 256)), int(pick(128, int(rng.integers(100, 160))))
+        layout = eden.NHWC if rng.random() < 0.8 else eden.NCHW
+        flags = eden.EXACT_CHANNELS if rng.random() < 0.15 else 0
+        tseed = int(rng.integers(1, 1 << 30))
+        mode = "run"
+        if kind == "fc":
+            m, k, n = pick(1, 2, 8, 32, 64, 128, 256), pick(256, 1001, 1024, 1280, 2048, 4096, 9216), pick(10, 100, 1000, 1001, 4096)
+            a, w, b = synth.fill_u8((m, k), tseed), synth.fill_u8_normal((n, k), tseed + 1, zp_w, 20), synth.fill_i32((n,), tseed + 2, -1000, 1000)
+            _, acc = O.fc(a, w, b, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+            q = centred(acc, zp_in, zp_w)
+            want, got, desc_txt = O.fc(a, w, b, q), gpu_fc(a, w, b, to_eh_requant(q), flags=flags), (m, k, n, flags)
+        else:
+            n = pick(1, 2, 8, 16, 32)
+            hw = pick(7, 14, 28, 56, 112)
+            groups, dm, dil, st = 1, 1, 1, pick(1, 1, 2)
+            if kind == "pw":
+                c, cout, k = pick(16, 24, 32, 64, 96, 144, 192, 256, 320, 384, 576, 960, 1280), pick(16, 21, 24, 32, 64, 96, 160, 256, 320, 512, 1001, 1280), 1
+            elif kind == "conv3x3":
+                c, cout, k, dil = pick(3, 16, 32, 64, 128, 256, 512), pick(16, 32, 64, 128, 256), 3, pick(1, 1, 1, 2)
+            elif kind == "convk":
+                c, cout, k = pick(3, 16, 64), pick(32, 64, 96), pick(5, 7)
+            elif kind == "grouped":
+                groups = pick(2, 4, 32); c, cout, k = groups * pick(4, 8, 16, 32), groups * pick(4, 8, 16, 32), pick(1, 3)
+            elif kind == "dw":
+                c = pick(32, 96, 144, 192, 384, 576, 960); cout, k, dil = c, pick(3, 3, 5), pick(1, 1, 2)
+            else:
+                c, cout, k = pick(21, 32, 64, 128, 256), pick(21, 32, 64, 128), pick(2, 3, 4, 8, 16)
+                st = pick(*[v for v in (1, 2, 4, 8) if v <= k]); hw = pick(4, 7, 14, 28)
+            h, w_ = jitter(hw), jitter(hw)
+            same = dil * (k - 1)
+            pads = (same // 2, same - same // 2, same // 2, same - same // 2) if rng.random() < 0.7 else tuple(int(v) for v in rng.integers(0, same + 1, 4))
+            if kind == "deconv":
+                pads = tuple(int(v) for v in rng.integers(0, max(1, k - st + 1), 4))
+            s = O.conv_shape(n, c, h, w_, cout, k, k, stride=(st, st), pad=pads, dil=(dil, dil), groups=groups, dm=1)
+            out_hw = O.deconv_out_hw(s) if kind == "deconv" else O.conv_out_hw(s)
+            if min(out_hw) < 1:
+                continue
+            def work(nn):   # multiply-accumulates and bytes of the instance at batch nn
+                px = nn * (s.h * s.w if kind == "deconv" else out_hw[0] * out_hw[1])
+                red = k * k if kind == "dw" else (c // groups) * k * k
+                return px * (cout if kind != "dw" else c) * red, nn * (c * h * w_ + cout * out_hw[0] * out_hw[1])
+            cap = 8e9 if rng.random() < 0.2 else 1.2e9   # (one in five large enough for the 256-row tiles)
+            while n > 1 and (work(n)[0] > cap or work(n)[1] > 0.04 * cap):
+                n //= 2
+            if work(n)[0] > 2 * cap:
+                continue
+            s = O.conv_shape(n, c, h, w_, cout, k, k, stride=(st, st), pad=pads, dil=(dil, dil), groups=groups, dm=1)
+            x, b = synth.fill_u8((n, c, h, w_), tseed), synth.fill_i32((cout,), tseed + 2, -1000, 1000)
+            if kind == "dw":
+                w = synth.fill_u8((c, 1, k, k), tseed + 1)
+                _, acc = O.dwconv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+                q = centred(acc, zp_in, zp_w)
+                want, got = O.dwconv2d(x, w, b, s, q), gpu_dwconv(x, w, b, s, to_eh_requant(q), layout=layout | flags)
+            elif kind == "deconv":
+                w = synth.fill_u8_normal((c, cout, k, k), tseed + 1, zp_w, 20)
+                wl = pick(eden.W_IOHW, eden.W_OHWI)
+                _, acc = O.deconv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+                q = centred(acc, zp_in, zp_w)
+                want, got = O.deconv2d(x, w, b, s, q), gpu_deconv(x, w, b, s, to_eh_requant(q), layout=layout | flags, weight_layout=wl)
+                kernels.update(eden.conv_kernels(eden.conv_desc(n, c, h, w_, cout, k, k, (st, st), pads, (1, 1), 1, 1, layout | flags, wl), deconv=True))
+            else:
+                w = synth.fill_u8_normal((cout, c // groups, k, k), tseed + 1, zp_w, 20)
+                wl = pick(eden.W_OIHW, eden.W_OHWI) if groups == 1 else eden.W_OIHW   # (OHWI weights are taken for ungrouped layers only)
+                _, acc = O.conv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
+                q = centred(acc, zp_in, zp_w)
+                want = O.conv2d(x, w, b, s, q)
+                mode = pick("run", "run", "other parameters", "residual", "static")
+                desc = eden.conv_desc(n, c, h, w_, cout, k, k, (st, st), pads, (dil, dil), groups, 1, layout | flags, wl)
+                kernels.update(eden.conv_kernels(desc))
+                nhwc = layout == eden.NHWC
+                to_dev = (lambda t: np.ascontiguousarray(t.transpose(0, 2, 3, 1))) if nhwc else (lambda t: t)
+                d_x, d_w, d_b = eden.DeviceBuffer(host=to_dev(x)), eden.DeviceBuffer(host=w if wl == eden.W_OIHW else w.transpose(0, 2, 3, 1)), eden.DeviceBuffer(host=b)
+                d_o = eden.DeviceBuffer(nbytes=want.size)
+                planned = q
+                if mode == "other parameters":
+                    planned = O.raw_quant(zp_in=(zp_in + 77) % 256, zp_w=(zp_w + 9) % 256, zp_out=17, multiplier=q.multiplier // 2 + (1 << 29), shift=q.shift, act_min=0, act_max=255)
+                plan = eden.ConvPlan(desc, d_w, d_b, to_eh_requant(planned))
+                if mode == "residual":
+                    res = synth.fill_u8(want.shape, tseed + 3)
+                    aq = O.make_add_quant(0.031, 120, 0.043, q.zp_out, 0.05, 125, O.ACT_NONE, False)
+                    want = O.add(res, want, aq)
+                    d_r = eden.DeviceBuffer(host=to_dev(res))
+                    plan.run_add(d_x, d_r, d_o, to_eh_requant(q), to_eh_add(aq))
+                elif mode == "static" and x.size + 2 * want.size < (8 << 20):
+                    try:
+                        plan.run_static(d_x, d_o, to_eh_requant(q))
+                    except eden.EdenHipError as e:   # (its stated limit: the problems of one launch list)
+                        assert "at most" in str(e), e
+                        plan.run(d_x, d_o, to_eh_requant(q))
+                else:
+                    plan.run(d_x, d_o, to_eh_requant(q))
+                got = d_o.download((n, out_hw[0], out_hw[1], cout)).transpose(0, 3, 1, 2) if nhwc else d_o.download(want.shape)
+                plan.destroy()
+            desc_txt = (dict(n=n, c=c, h=h, w=w_, cout=cout, k=k, stride=st, pad=pads, dil=dil, groups=groups), layout, flags, mode)
+        ran[kind] = ran.get(kind, 0) + 1
+        modes[mode] = modes.get(mode, 0) + 1
+        if not np.array_equal(got, want):
+            bad += 1
+            print("MISMATCH", it, kind, desc_txt, q.as_tuple(), diff_report(got, want), flush=True)
+    print("kernels chosen:", sorted(kernels), "modes:", modes, "kinds:", ran, flush=True)
+    assert bad == 0, "%d of %d network-sized instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
+    assert sum(ran.values()) > 80 and len(kernels) >= 7, (ran, kernels)
