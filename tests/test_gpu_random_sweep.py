@@ -361,3 +361,58 @@ def test_random_network_sized_instances_match_the_oracle(seed):
     print("kernels chosen:", sorted(kernels), "modes:", modes, "kinds:", ran, flush=True)
     assert bad == 0, "%d of %d network-sized instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
     assert sum(ran.values()) > 80 and len(kernels) >= 7, (ran, kernels)
+
+
+@pytest.mark.parametrize("seed", [51])
+def test_random_add_and_average_pool_instances_match_the_oracle(seed):
+    """The two operators between the convolutions: element-wise Add over random lengths, pointer offsets and
+    quantization parameters, AveragePool over random windows, strides, paddings, both tensor orders and both
+    precisions."""
+    eden.init(0)
+    print("random add / average pool sweep, seed", seed, flush=True)
+    rng = np.random.default_rng(seed)
+    bad = 0
+    for it in range(150):
+        tseed = int(rng.integers(1, 1 << 30))
+        count, off = int(rng.choice([1, 7, 16, 63, 1000, 4097, 70001, int(rng.integers(1, 200000))])), int(rng.choice([0, 0, 1, 3, 8]))
+        s_a, s_b, s_o = (float(v) for v in rng.uniform(0.002, 0.3, 3))
+        zps = [int(v) for v in rng.integers(0, 256, 3)]
+        act, en = (O.ACT_NONE, False) if rng.random() < 0.6 else (int(rng.choice([O.ACT_RELU, O.ACT_RELU6])), True)
+        q = O.make_add_quant(s_a, zps[0], s_b, zps[1], s_o, zps[2], act, en)
+        a, b = synth.fill_u8((count,), tseed), synth.fill_u8((count,), tseed + 1)
+        pad = np.zeros(off, np.uint8)
+        d_a, d_b = eden.DeviceBuffer(host=np.concatenate([pad, a])), eden.DeviceBuffer(host=np.concatenate([pad, b]))
+        d_o = eden.DeviceBuffer(nbytes=count + off + 16)
+        eden.add_u8(d_a.ptr.value + off, d_b.ptr.value + off, d_o.ptr.value + off, count, to_eh_add(q))
+        if not np.array_equal(d_o.download((count + off,))[off:], O.add(a, b, q)):
+            bad += 1
+            print("MISMATCH add", it, count, off, (s_a, s_b, s_o), zps, act, flush=True)
+    for it in range(150):
+        tseed = int(rng.integers(1, 1 << 30))
+        n, c = int(rng.integers(1, 5)), int(rng.choice([1, 3, 4, 5, 8, 16, 24, 30, 64, 100, 320]))
+        h, w = int(rng.integers(1, 24)), int(rng.integers(1, 24))
+        kh, kw = int(rng.integers(1, min(h, 8) + 1)), int(rng.integers(1, min(w, 8) + 1))
+        if rng.random() < 0.2:
+            kh, kw = h, w   # a global pool
+        stride = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        pad = (int(rng.integers(0, kh)), int(rng.integers(0, kh)), int(rng.integers(0, kw)), int(rng.integers(0, kw)))
+        lo, hi = int(rng.choice([0, 0, 20])), int(rng.choice([255, 255, 180]))
+        nhwc, signed = rng.random() < 0.6, rng.random() < 0.4
+        x = synth.fill_u8((n, c, h, w), tseed)
+        if signed:
+            x = (x.astype(np.int16) - 128).astype(np.int8)
+            want = O.avgpool_s8(x, kh, kw, stride, pad, lo - 128, hi - 128)
+        else:
+            want = O.avgpool(x, kh, kw, stride, pad, lo, hi)
+        if want.size == 0:
+            continue
+        d_in = eden.DeviceBuffer(host=np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if nhwc else x)
+        d_out = eden.DeviceBuffer(nbytes=want.size)
+        eden.avgpool_u8(d_in, d_out, n, c, h, w, kh, kw, stride, pad, (eden.NHWC if nhwc else eden.NCHW) | (eden.IO_SIGNED if signed else 0),
+                        lo - 128 if signed else lo, hi - 128 if signed else hi)
+        ho, wo = want.shape[2:]
+        got = d_out.download((n, ho, wo, c)).transpose(0, 3, 1, 2) if nhwc else d_out.download(want.shape)
+        if not np.array_equal(np.ascontiguousarray(got).view(want.dtype), want):
+            bad += 1
+            print("MISMATCH avgpool", it, (n, c, h, w), (kh, kw), stride, pad, (lo, hi), "nhwc" if nhwc else "nchw", "int8" if signed else "uint8", flush=True)
+    assert bad == 0, "%d random add / average pool instances differ from the oracle (MISMATCH lines above)" % bad
