@@ -1055,7 +1055,7 @@ static int conv_plan_build(eh_conv_plan *pl, const eh_conv_desc *d, hipStream_t 
     // block-diagonal problem over their 16 .. 64 adjacent channels, read in 16-byte units straight from the tensor,
     // instead of one small problem per group on a padded copy.
     int bundle = 1;
-    if (G > 1 && !padded && !op.exact_channels && (cig & 15) != 0 && d->weight_layout == EH_W_OIHW)
+    if (G > 1 && !padded && !op.exact_channels && (cig & 15) != 0)
         for (int b = G; b >= 2 && bundle == 1; --b)
             if (G % b == 0 && b * cig <= 64 && ((b * cig) & 15) == 0) bundle = b;
     op.w_keep_bytes = bundle > 1 ? (size_t)d->cout * cig * taps : 0;
@@ -1132,7 +1132,6 @@ static int conv_desc_checked(const eh_conv_desc *desc, eh_conv_desc *plain) {
                "groups %d do not divide channels (%d, %d)", desc->groups, desc->c, desc->cout);
     EH_REQUIRE(desc->weight_layout == EH_W_OIHW || desc->weight_layout == EH_W_OHWI, "bad convolution weight layout %d",
                desc->weight_layout);
-    EH_REQUIRE(desc->weight_layout == EH_W_OIHW || desc->groups == 1, "OHWI weights support groups == 1 only");
     EH_REQUIRE(desc->kh * desc->dil_h < 32000 && desc->kw * desc->dil_w < 32000, "kernel extent too large");
     return EH_OK;
 }

@@ -40,7 +40,7 @@ typedef enum eh_activation { EH_ACT_NONE = 0, EH_ACT_RELU = 1, EH_ACT_RELU1 = 2,
 typedef enum eh_layout { EH_NCHW = 0, EH_NHWC = 1 } eh_layout;
 
 /* Weight element order.  OIHW is the reference's default [Cout][Cin/g][kh][kw];
- * OHWI is its androidNN order [Cout][kh][kw][Cin]
+ * OHWI is its androidNN order [Cout][kh][kw][Cin/g] (deconvolution: groups == 1 only)
  * (gpu/operators/cl_optimized_impls/CLDeconvolutionQuantized.cpp:39-46), for a depthwise
  * convolution [1][kh][kw][C*dm] (gpu/operators/CLDepthwiseConvolution.cpp:128-131,146);
  * IOHW is the deconvolution order [Cin][Cout/g][kh][kw] (gpu/op_test/deconv_guard.h:53-69). */

@@ -330,8 +330,10 @@ def test_conv_config1_exact_and_fastpath_census():
     assert O.count_fastpath_overflow(acc, q) == 0
 
 
-def test_conv_ohwi_weights_equal_oihw():
-    s = O.conv_shape(2, 16, 9, 9, 32, 3, 3, pad=(1, 1, 1, 1))
+@pytest.mark.parametrize("groups,cig,cog", [(1, 16, 32), (2, 16, 8), (8, 4, 4), (4, 5, 3)], ids=["ungrouped", "two_groups", "bundled_groups", "ragged_groups"])
+def test_conv_ohwi_weights_equal_oihw(groups, cig, cog):
+    """[Cout][kh][kw][Cin / groups] weights give what the same weights in [Cout][Cin / groups][kh][kw] give."""
+    s = O.conv_shape(2, groups * cig, 9, 9, groups * cog, 3, 3, pad=(1, 1, 1, 1), groups=groups)
     x, w, b = conv_tensors(s, SEED + 5)
     q = quant(0.02, 100, 0.005, 90, 0.04, 10)
     want = O.conv2d(x, w, b, s, q)

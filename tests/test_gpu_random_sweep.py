@@ -76,7 +76,8 @@ def test_random_operator_instances_match_the_oracle(seed):
                     x = synth.fill_u8((n, c, h, w_), tseed); w = synth.fill_u8((cout, c // groups, k, k), tseed + 1); b = synth.fill_i32((cout,), tseed + 2, -1000, 1000)
                     _, acc = O.conv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
                     q = centred(acc, zp_in, zp_w, lo, hi)
-                    want = O.conv2d(x, w, b, s, q); got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=layout); desc = (kind, s, layout)
+                    wl = eden.W_OHWI if tseed % 3 == 0 else eden.W_OIHW
+                    want = O.conv2d(x, w, b, s, q); got = gpu_conv(x, w, b, s, to_eh_requant(q), layout=layout, weight_layout=wl); desc = (kind, s, layout, wl)
         except Exception as e:
             raise AssertionError(("error", seed, it, kind, repr(e)[:300]))
         ran[kind] = ran.get(kind, 0) + 1
@@ -321,7 +322,7 @@ def test_random_network_sized_instances_match_the_oracle(seed):
                 kernels.update(eden.conv_kernels(eden.conv_desc(n, c, h, w_, cout, k, k, (st, st), pads, (1, 1), 1, 1, layout | flags, wl), deconv=True))
             else:
                 w = synth.fill_u8_normal((cout, c // groups, k, k), tseed + 1, zp_w, 20)
-                wl = pick(eden.W_OIHW, eden.W_OHWI) if groups == 1 else eden.W_OIHW   # (OHWI weights are taken for ungrouped layers only)
+                wl = pick(eden.W_OIHW, eden.W_OHWI)
                 _, acc = O.conv2d(x, w, b, s, O.raw_quant(zp_in=zp_in, zp_w=zp_w), want_acc=True)
                 q = centred(acc, zp_in, zp_w)
                 want = O.conv2d(x, w, b, s, q)
