@@ -35,6 +35,9 @@ int hip_fail(hipError_t e, const char *what) {
 // current, and every later use (kernel arguments, copies) goes through the address it keeps.
 static __device__ __align__(256) uint8_t scratch[EH_STATIC_SCRATCH_BYTES];
 static constexpr int kMaxDevices = 64;
+// longest reduction (channels x kernel taps, or the columns of a fully connected layer) a plan is built for:
+// the per-plan tables grow with it, and no layer of the networks this serves comes near it
+static constexpr int EH_MAX_REDUCTION = 1 << 24;
 static uint8_t *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until asked
 
 static int static_scratch(uint8_t **ptr) {
@@ -1133,6 +1136,8 @@ static int conv_desc_checked(const eh_conv_desc *desc, eh_conv_desc *plain) {
     EH_REQUIRE(desc->weight_layout == EH_W_OIHW || desc->weight_layout == EH_W_OHWI, "bad convolution weight layout %d",
                desc->weight_layout);
     EH_REQUIRE(desc->kh * desc->dil_h < 32000 && desc->kw * desc->dil_w < 32000, "kernel extent too large");
+    EH_REQUIRE((int64_t)desc->c * desc->kh * desc->kw <= EH_MAX_REDUCTION,
+               "reductions over %lld terms (all groups) are not supported (at most %d)", (long long)desc->c * desc->kh * desc->kw, EH_MAX_REDUCTION);
     return EH_OK;
 }
 
@@ -1272,6 +1277,7 @@ int eh_fc_q8_plan(eh_fc_plan **plan, int32_t m, int32_t k, int32_t n, int32_t fl
     *plan = nullptr;
     EH_REQUIRE(m >= 0 && k > 0 && n > 0, "bad extents m=%d k=%d n=%d", m, k, n);
     EH_REQUIRE((int64_t)m * k < (1ll << 31), "input larger than 2 GiB is not supported");
+    EH_REQUIRE(k <= EH_MAX_REDUCTION, "a reduction over %d terms is not supported (at most %d)", k, EH_MAX_REDUCTION);
     EH_REQUIRE((flags & ~(EH_W_SIGNED | EH_IO_SIGNED | EH_EXACT_CHANNELS)) == 0, "unknown flags 0x%x", flags);
     const bool w_signed = (flags & EH_W_SIGNED) != 0, io_signed = (flags & EH_IO_SIGNED) != 0;
     int rc = check_requant(q, w_signed, io_signed);
@@ -1538,6 +1544,10 @@ static int deconv_desc_checked(const eh_conv_desc *desc, eh_conv_desc *plain) {
     EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->weight_layout == EH_W_OHWI, "bad deconvolution weight layout %d",
                desc->weight_layout);
     EH_REQUIRE(desc->weight_layout == EH_W_IOHW || desc->groups == 1, "OHWI weights support groups == 1 only");
+    EH_REQUIRE((int64_t)desc->groups * desc->stride_h * desc->stride_w <= 65536, "%lld output phases (groups x strides) are not supported (at most 65536)",
+               (long long)desc->groups * desc->stride_h * desc->stride_w);
+    EH_REQUIRE((int64_t)desc->c * desc->kh * desc->kw <= EH_MAX_REDUCTION,
+               "reductions over %lld terms (all groups) are not supported (at most %d)", (long long)desc->c * desc->kh * desc->kw, EH_MAX_REDUCTION);
     return EH_OK;
 }
 

@@ -110,7 +110,9 @@ typedef struct eh_pool_desc {
  * the memory order; `layout` says how input and output bytes are ordered.
  * Mirrors ConvolutionParameters / DepthwiseConvolutionParameters /
  * DeconvolutionParameters (gpu/operators/CLConvolution.hpp:31-44,
- * CLDepthwiseConvolution.hpp:18-29, CLDeconvolution.hpp:20-31). */
+ * CLDepthwiseConvolution.hpp:18-29, CLDeconvolution.hpp:20-31).
+ * Limits the plan calls check (EH_ERR_UNSUPPORTED beyond them): every tensor below 2 GiB, kernel extents times
+ * dilation below 32000, and reductions (c * kh * kw; k of a fully connected layer) of at most 2^24 terms. */
 typedef struct eh_conv_desc {
     int32_t n, c, h, w;
     int32_t cout;

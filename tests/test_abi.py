@@ -267,6 +267,44 @@ def test_classifier_heads_take_the_kernel_cut_along_the_weights():
     assert "skinny" not in eden.conv_kernels(eden.conv_desc(1, 512, 9, 9, 48, 1, 1, stride=(2, 2), layout=nhwc))
 
 
+def test_descriptor_queries_answer_or_refuse_whatever_the_descriptor():
+    """Descriptors drawn from edge values (zero, negative, 2^31 - 1, unknown layouts): the kernel query, which runs the
+    plan builder's host side, either answers or refuses with a status, and does so quickly; the stated limits (a
+    reduction of 2^24 terms, 65536 deconvolution phases) keep absurd descriptors from building tables of that size."""
+    import time
+    rng = np.random.default_rng(5)
+    edge = [0, 1, 2, 3, 7, 16, 17, 64, 255, 1001, 4096, 65536, 1 << 24, (1 << 31) - 1, -1]
+    small = [0, 1, 2, 3, 5, 7, 16, 64, -1]
+    answered = refused = 0
+    start = time.time()
+    for it in range(6000):
+        p = lambda: int(edge[int(rng.integers(0, len(edge)))]) if rng.random() < 0.4 else int(rng.integers(1, 70))
+        k = lambda: int(small[int(rng.integers(0, len(small)))]) if rng.random() < 0.5 else int(rng.integers(1, 8))
+        groups = int(rng.choice([1, 1, 1, 2, 4, 32, 1000, 0]))
+        c, cout = p(), p()
+        if groups > 0 and rng.random() < 0.7:
+            c, cout = max(groups, abs(c) // groups * groups), max(groups, abs(cout) // groups * groups)
+        kh, kw = k(), k()
+        desc = eden.conv_desc(p(), c, p(), p(), cout, kh, kw, (k(), k()), (max(kh, 0) // 2, max(kh, 0) // 2, max(kw, 0) // 2, max(kw, 0) // 2),
+                              (int(rng.choice([1, 1, 2, 1000, 0])),) * 2, groups, int(rng.choice([1, 1, 2, 0])),
+                              int(rng.choice([0, 1, 1, 0x401, 0x201, 2, 77])), int(rng.choice([0, 0, 1, 2, 0x100, 9])))
+        for deconv in (False, True):
+            if deconv and desc.weight_layout & 0xFF == 0:
+                desc.weight_layout |= eden.W_IOHW
+            try:
+                assert len(eden.conv_kernels(desc, deconv=deconv)) >= 0
+                answered += 1
+            except eden.EdenHipError:
+                refused += 1
+    assert answered > 500 and refused > 500, (answered, refused)
+    assert time.time() - start < 60
+    for absurd in (eden.conv_desc(1, 1 << 24, 8, 8, 16, 3, 3), eden.conv_desc(1, 4096, 8, 8, 16, 64, 65)):
+        with pytest.raises(eden.EdenHipError, match="reductions over"):
+            eden.conv_kernels(absurd)
+    with pytest.raises(eden.EdenHipError, match="output phases"):
+        eden.conv_kernels(eden.conv_desc(1, 1024, 8, 8, 1024, 64, 64, stride=(64, 64), groups=1024, weight_layout=eden.W_IOHW), deconv=True)
+
+
 def test_buffer_pool_protocol_without_a_gpu():
     """request / reset / layout are host bookkeeping (CLRuntime.cpp:34-118, 147-157): a REUSE request takes over the
     first feature map handed back and grows it, intra-operator scratch is sized to the largest request per slot, and
