@@ -428,3 +428,60 @@ def test_random_add_and_average_pool_instances_match_the_oracle(seed):
             bad += 1
             print("MISMATCH avgpool", it, (n, c, h, w), (kh, kw), stride, pad, (lo, hi), "nhwc" if nhwc else "nchw", "int8" if signed else "uint8", flush=True)
     assert bad == 0, "%d random add / average pool instances differ from the oracle (MISMATCH lines above)" % bad
+
+
+@pytest.mark.parametrize("seed", [61, 62])
+def test_random_rectangular_instances_match_the_oracle(seed):
+    """Kernels, strides and dilations that differ between rows and columns (the 1 x 7 and 7 x 1 layers of Inception-style
+    networks and their like): convolution, depthwise convolution and deconvolution over random shapes, at channel
+    counts that reach the patch, row, one-tap and tiled kernels."""
+    eden.init(0)
+    print("random rectangular sweep, seed", seed, flush=True)
+    rng = np.random.default_rng(seed)
+    pick = lambda *v: v[int(rng.integers(0, len(v)))]
+    ran, bad = {}, 0
+    for it in range(300):
+        kind = pick("conv", "conv", "dw", "deconv")
+        zp_in, zp_w = int(rng.integers(0, 256)), int(pick(128, int(rng.integers(0, 256))))
+        layout = (eden.NHWC if rng.random() < 0.7 else eden.NCHW) | (eden.EXACT_CHANNELS if rng.random() < 0.15 else 0)
+        tseed = int(rng.integers(1, 1 << 30))
+        n, h, w_ = int(rng.integers(1, 4)), int(rng.integers(4, 24)), int(rng.integers(4, 24))
+        kh, kw = pick(1, 1, 2, 3, 5, 7), pick(1, 1, 2, 3, 5, 7)
+        sh, sw = pick(1, 1, 2, 3), pick(1, 1, 2, 3)
+        dh, dw_ = pick(1, 1, 2, 3), pick(1, 1, 2, 3)
+        raw = lambda: O.raw_quant(zp_in=zp_in, zp_w=zp_w)
+        def centred(acc):
+            sd = float(acc.std()) or 1.0
+            qm, sh_ = O.quantize_multiplier(float(pick(10.0, 40.0, 120.0)) / sd)
+            return O.raw_quant(zp_in=zp_in, zp_w=zp_w, zp_out=int(np.clip(128 - round(float(acc.mean()) * 40.0 / sd), 0, 255)), multiplier=qm, shift=sh_, act_min=0, act_max=255)
+        if kind == "deconv":
+            c, cout = pick(8, 16, 21, 32, 64), pick(8, 16, 21, 32)
+            pads = (int(rng.integers(0, kh)), int(rng.integers(0, kh)), int(rng.integers(0, kw)), int(rng.integers(0, kw)))
+            s = O.conv_shape(n, c, h // 2 + 1, w_ // 2 + 1, cout, kh, kw, stride=(sh, sw), pad=pads)
+            if min(O.deconv_out_hw(s)) < 1: continue
+            x, w, b = synth.fill_u8((n, c, s.h, s.w), tseed), synth.fill_u8((c, cout, kh, kw), tseed + 1), synth.fill_i32((cout,), tseed + 2, -1000, 1000)
+            q = centred(O.deconv2d(x, w, b, s, raw(), want_acc=True)[1])
+            want, got = O.deconv2d(x, w, b, s, q), gpu_deconv(x, w, b, s, to_eh_requant(q), layout=layout, weight_layout=pick(eden.W_IOHW, eden.W_OHWI))
+        else:
+            pads = (int(rng.integers(0, dh * (kh - 1) + 1)), int(rng.integers(0, dh * (kh - 1) + 1)), int(rng.integers(0, dw_ * (kw - 1) + 1)), int(rng.integers(0, dw_ * (kw - 1) + 1)))
+            if kind == "dw":
+                c, dm = pick(4, 8, 16, 30, 32, 7, 144), pick(1, 1, 1, 2)
+                s = O.conv_shape(n, c, h, w_, c * dm, kh, kw, stride=(sh, sw), pad=pads, dil=(dh, dw_), dm=dm)
+                if min(O.conv_out_hw(s)) < 1: continue
+                x, w, b = synth.fill_u8((n, c, h, w_), tseed), synth.fill_u8((c * dm, 1, kh, kw), tseed + 1), synth.fill_i32((c * dm,), tseed + 2, -1000, 1000)
+                q = centred(O.dwconv2d(x, w, b, s, raw(), want_acc=True)[1])
+                want, got = O.dwconv2d(x, w, b, s, q), gpu_dwconv(x, w, b, s, to_eh_requant(q), layout=layout)
+            else:
+                groups = pick(1, 1, 1, 2, 8)
+                c, cout = groups * pick(1, 3, 4, 8, 16, 21, 32, 64, 128, 192), groups * pick(3, 8, 16, 24, 64, 100)
+                s = O.conv_shape(n, c, h, w_, cout, kh, kw, stride=(sh, sw), pad=pads, dil=(dh, dw_), groups=groups)
+                if min(O.conv_out_hw(s)) < 1: continue
+                x, w, b = synth.fill_u8((n, c, h, w_), tseed), synth.fill_u8((cout, c // groups, kh, kw), tseed + 1), synth.fill_i32((cout,), tseed + 2, -1000, 1000)
+                q = centred(O.conv2d(x, w, b, s, raw(), want_acc=True)[1])
+                want, got = O.conv2d(x, w, b, s, q), gpu_conv(x, w, b, s, to_eh_requant(q), layout=layout, weight_layout=pick(eden.W_OIHW, eden.W_OHWI))
+        ran[kind] = ran.get(kind, 0) + 1
+        if not np.array_equal(got, want):
+            bad += 1
+            print("MISMATCH", it, kind, s, layout, q.as_tuple(), diff_report(got, want), flush=True)
+    assert bad == 0, "%d of %d rectangular instances differ from the oracle (MISMATCH lines above)" % (bad, sum(ran.values()))
+    assert all(ran.get(k, 0) > 40 for k in ("conv", "dw", "deconv")), ran
