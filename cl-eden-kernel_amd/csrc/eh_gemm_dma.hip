@@ -464,6 +464,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 const int nl = wn * WTN + j * 32 + fhalf * 16, n = n0 + nl;  // this lane's 16 consecutive channels
+                if constexpr (checked) {
+                    if (n >= p.n) continue;  // past the last channel: nothing to requantize
+                }
                 int4 bb[4];
 #pragma unroll
                 for (int g = 0; g < 4; ++g) bb[g] = *reinterpret_cast<const int4 *>(bias_s + nl + g * 4);
@@ -509,7 +512,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
                         *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
                         __builtin_amdgcn_sched_barrier(0);  // one fragment at a time: keeps the accumulators where they are
                     } else {
-                        if (!row_ok[i] || n >= p.n) continue;
+                        if (!row_ok[i]) continue;
                         if (aligned16 && n + 16 <= p.n) {
                             *reinterpret_cast<uint4 *>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
                         } else {
@@ -540,6 +543,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 128 &
                 emit(std::false_type{}, std::integral_constant<int, 2>{}, std::false_type{});
             else
                 emit(std::false_type{}, std::integral_constant<int, 1>{}, std::false_type{});
+        } else if (rq.fast == 2) {  // edge tiles (and layers narrower than the tile) keep the short requantization forms
+            emit(std::true_type{}, std::integral_constant<int, 2>{}, std::false_type{});
+        } else if (rq.fast == 1) {
+            emit(std::true_type{}, std::integral_constant<int, 1>{}, std::false_type{});
         } else {
             emit(std::true_type{}, std::integral_constant<int, 0>{}, std::false_type{});
         }
