@@ -1414,7 +1414,8 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
     // differ, their taps' positions do not) and cover equally many positions go out as ONE problem whose columns are
     // (kernel column, output channel): a row of the problem then writes neighbouring output pixels, count * cout
     // contiguous bytes, and the launches shrink by that count.  Needs one group (a pixel holds the problem's channels
-    // alone) and more than one tap (the one-tap kernel has its own batching).
+    // alone) and more than one tap (the one-tap kernel has its own batching) or an output channel count that is no
+    // multiple of 16 (a phase alone would store rows of that many bytes at unaligned addresses).
     struct XPhase {
         int px, ox0, wo_p, ntx, bx;
     };
@@ -1461,7 +1462,7 @@ static int deconv_plan_build(eh_deconv_plan *pl, const eh_conv_desc *d, hipStrea
             for (size_t first = 0; first < xs.size();) {
                 const XPhase &x0 = xs[first];
                 size_t last = first + 1;
-                while (G == 1 && nty * x0.ntx > 1 && last < xs.size() && xs[last].ox0 == xs[last - 1].ox0 + 1 &&
+                while (G == 1 && (nty * x0.ntx > 1 || (cog & 15) != 0) && last < xs.size() && xs[last].ox0 == xs[last - 1].ox0 + 1 &&
                        xs[last].px == xs[last - 1].px + 1 && xs[last].bx == x0.bx && xs[last].wo_p == x0.wo_p && xs[last].ntx == x0.ntx)
                     ++last;
                 const int count = (int)(last - first);
